@@ -1,0 +1,89 @@
+/* splash_ops.h -- flat C entry points of the verify step's C++ operators (splash::ops::*), for
+ * hosts that bind through an FFI (the Python tests and bench of this repository, a cgo/JNI stub).
+ * Each function wraps one method of an operator that keeps the reference's name and argument
+ * meaning; the reference method is cited beside it. A std::invalid_argument of an operator comes
+ * back as SP_INVALID_ARGUMENT with its message in sp_last_error(), thrown -- as in the reference --
+ * before any dispatch is added to the graph.
+ */
+#ifndef SPLASH_OPS_H
+#define SPLASH_OPS_H
+
+#include "splash_hip.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct spo_graph spo_graph;           /* metal::CommandGraph (runtime/metal/CommandGraph.hpp:26) */
+typedef struct spo_projection spo_projection; /* ops::Projection (runtime/ops/Weights.hpp:170) */
+typedef struct spo_linear spo_linear;         /* ops::Linear (runtime/ops/Linear.hpp:289) */
+
+/* ---- CommandGraph ---- */
+sp_status spo_graph_create(spo_graph **out);
+void spo_graph_destroy(spo_graph *graph);
+uint32_t spo_graph_size(const spo_graph *graph);
+/* The kernel name of dispatch `index`; returns the bytes needed. */
+size_t spo_graph_kernel(const spo_graph *graph, uint32_t index, char *out, size_t capacity);
+/* CommandGraph::add (CommandGraph.hpp:44-54): a raw dispatch with a parameter struct. */
+sp_status spo_graph_add(spo_graph *graph, const char *kernel, sp_buffer *const *buffers, uint32_t buffer_count,
+                        const void *params, uint32_t params_bytes, const uint32_t grid[3], const uint32_t block[3]);
+/* MetalBackend::submitCommandAsync(graph.dispatches()) (MetalBackend.hpp:490-491). */
+sp_status spo_graph_submit(sp_backend *backend, const spo_graph *graph, sp_ticket **out);
+/* The graph recorded for replay (sp_command_create). */
+sp_status spo_graph_record(sp_backend *backend, const spo_graph *graph, sp_command **out);
+
+/* ---- weight image (load-time repack: runtime/model/GgufPreparation.cpp, gguf_repack.metal) ---- */
+uint64_t spo_gguf_image_bytes(uint32_t format, uint32_t rows, uint32_t input_size);
+uint64_t spo_gguf_table_bytes(uint32_t input_size, uint32_t rows);
+sp_status spo_gguf_pack_image(uint32_t format, const uint8_t *native, uint32_t rows, uint32_t input_size, uint8_t *image);
+sp_status spo_gguf_unpack_image(uint32_t format, const uint8_t *image, uint32_t rows, uint32_t input_size, uint8_t *native);
+/* The image's fp32 values [rows][input_size] (the reference's gguf_dequant_test.metal kernel). */
+sp_status spo_gguf_add_dequant(spo_graph *graph, uint32_t format, sp_buffer *image, sp_buffer *out, uint32_t rows,
+                               uint32_t input_size);
+
+/* ---- Projection (Weights.hpp:170-186): segments tile the leading output columns in order ---- */
+sp_status spo_projection_create(uint32_t segments, const uint32_t *formats, const uint32_t *output_sizes,
+                                uint32_t input_size, sp_buffer *const *images, int float32_destination,
+                                spo_projection **out);
+void spo_projection_destroy(spo_projection *projection);
+uint64_t spo_projection_weight_bytes(const spo_projection *projection);
+
+/* ---- Linear ---- */
+/* ops::Linear::Linear(device, ...) (Linear.hpp:291): plans follow the device the backend opened. */
+sp_status spo_linear_create(sp_backend *backend, spo_linear **out);
+/* A Linear of a given calibration (KernelCalibration), for CPU tests and sweeps. */
+sp_status spo_linear_create_calibrated(uint32_t compute_units, uint32_t waves_per_unit, uint32_t minimum_blocks_per_wave,
+                                       spo_linear **out);
+void spo_linear_destroy(spo_linear *linear);
+/* LinearEpilogue (Linear.hpp:77): 0 None, 1 Residual, 2 GateUp. */
+typedef struct spo_linear_plan {
+  uint32_t rows, epilogue;
+  uint32_t splits, k_waves; /* LinearConfig */
+  uint32_t storage_rows;    /* LinearPlan::storageRows */
+  uint32_t float32;         /* LinearPlan::destination */
+  uint64_t scratch_input, scratch_partials, scratch_counters; /* LinearPlan::scratchSize */
+} spo_linear_plan;
+/* Linear::plan(projection, rows, epilogue) (Linear.hpp:307-309): the device's plan. */
+sp_status spo_linear_plan_for(const spo_linear *linear, const spo_projection *projection, uint32_t rows, uint32_t epilogue,
+                              spo_linear_plan *out);
+/* Linear::plan(workload, config, destination) (Linear.hpp:327-328): the plan of a given configuration;
+ * fills storage_rows and scratch sizes from rows, epilogue, splits, k_waves, float32. */
+sp_status spo_linear_plan_with(const spo_projection *projection, spo_linear_plan *plan);
+/* Linear::add (Linear.hpp:330-332). table/partials/counters are the LinearScratch; `prepared`
+ * nonzero says the table already holds `input` (PreparedInput). gate only for a GateUp plan. */
+sp_status spo_linear_add(const spo_linear *linear, spo_graph *graph, const spo_projection *projection,
+                         const spo_projection *gate, const spo_linear_plan *plan, sp_buffer *input, sp_buffer *output,
+                         sp_buffer *residual, sp_buffer *table, sp_buffer *partials, sp_buffer *counters, int prepared);
+/* Linear::addSwiGlu (Linear.hpp:352-354): output = residual + down(silu(gate x) * up x). */
+sp_status spo_linear_add_swiglu(const spo_linear *linear, spo_graph *graph, const spo_projection *gate,
+                                const spo_projection *up, const spo_projection *down, sp_buffer *normalized,
+                                sp_buffer *intermediate, sp_buffer *residual, sp_buffer *output, uint32_t rows,
+                                sp_buffer *table, sp_buffer *partials, sp_buffer *counters);
+/* Linear::scratchSize (Linear.hpp:319): of every plan of up to `rows` rows of the matrix. */
+sp_status spo_linear_scratch_size(const spo_linear *linear, uint32_t output_size, uint32_t input_size, uint32_t rows,
+                                  uint64_t *table, uint64_t *partials, uint64_t *counters);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SPLASH_OPS_H */

@@ -1,0 +1,136 @@
+// CPU oracle of the speculative-decoding verify step: TEST INFRASTRUCTURE ONLY.
+//
+// A plain C++ restatement of the arithmetic rules of the reference (incoai/splash): its test
+// references (dev/tests/engine/*Reference.hpp, the fp64 references inside the kernel tests) and
+// the operation order of its kernels. Only tests/, __graft_entry__.smoke() and bench.py's
+// cpu_baseline leg may load this library, and only as the checker or the reported CPU baseline.
+// Nothing under splash_amd/ links, loads or calls it.
+//
+// Pin status of each group of functions (what fixes it besides its own formula):
+//   orc_dequant_rows (Q4_K, Q6_K)   pinned: SHA-256 goldens of upstream GGML over the 256x1024
+//                                   fixture (dev/tests/fixtures/weight-goldens/goldens.json:3,7)
+//                                   and the compiled reference header (oracle/_ref).
+//   orc_fixture                     pinned by the same goldens (a wrong byte order changes the hash).
+//   orc_quantize_q4k / q6k          PARITY UNPINNED: the K-quantizer lives in llama.cpp/ggml
+//                                   (goldens cite commit 7ab4ee7), absent from the reference tree.
+//                                   Oracle and GPU consume the same bytes, so verify parity does not
+//                                   depend on it; tests bound its round-trip error only.
+//   orc_gemm_*                      pinned by fp64 dot + projectionBound interval, and invariants.
+//   orc_kv_quantize                 pinned: closed form, compiled reference header (oracle/_ref).
+//   orc_attention_*                 pinned by dense-softmax special cases and invariants.
+//   orc_gdn_*                       pinned by 1-row closed form and fold/rollback invariants.
+//   orc_argmax / orc_accept_tree    pinned by brute force on tiny vocabularies.
+//   orc_rejection_*                 pinned by enumeration: selection law equals target to 1e-12.
+#pragma once
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+// Format ids follow the reference's GGUF_FMT_* numbering (runtime/metal/abi/QuantFormat.h:138-154).
+enum { ORC_FMT_Q4K = 0, ORC_FMT_Q6K = 4 };
+
+// ---- half / bfloat16 scalar conversions (round to nearest even) ----
+uint16_t orc_f2h(float f);
+float orc_h2f(uint16_t h);
+uint16_t orc_f2bf(float f);
+float orc_bf2f(uint16_t b);
+
+// ---- GGUF K-quants ----
+// Bytes of one native row of K values (K a multiple of 256). 0 for an unknown format.
+uint64_t orc_row_bytes(uint32_t fmt, uint32_t K);
+// dev/tests/engine/GgufFixtures.hpp:148-165 fixture(f, rows, K, seed): random bytes, finite half scales.
+int orc_fixture(uint32_t fmt, uint32_t rows, uint32_t K, uint32_t seed, uint8_t *native);
+// dev/tests/engine/GgufFormatReference.hpp:195-219,295-323 makeNative with realistic scales.
+int orc_make_native(uint32_t fmt, uint32_t rows, uint32_t K, uint32_t seed, uint8_t *native);
+// llama.cpp dequantize_row_q4_K / q6_K semantics (GgufFormatReference.hpp:370-381, :418-432).
+int orc_dequant_rows(uint32_t fmt, const uint8_t *native, uint32_t rows, uint32_t K, float *out);
+// llama.cpp-style quantize_row_q4_K_ref / q6_K_ref (parity unpinned, see header).
+int orc_quantize_rows(uint32_t fmt, const float *values, uint32_t rows, uint32_t K, uint8_t *native);
+
+// Projection out[m][n] = sum_k x[m][k] W[n][k], x bf16 [M][K], W native rows [N].
+// exact:  fp64 dot product.  bound: projectionBound(register tile) (GgufFormatReference.hpp:739-742).
+// chain:  the register rule in fp32 (linear_gguf_sgmatrix.metal:140-151, :199-288).
+// Any of the three outputs may be NULL. threads <= 0 uses every core.
+int orc_gemm(uint32_t fmt, const uint8_t *native, const uint16_t *x, uint32_t M, uint32_t K, uint32_t N,
+             double *exact, double *bound, float *chain, int threads);
+// Epilogues on fp32 sums (kernels/common/gguf_tile.h:10-16, gguf_linear.metal:34-71).
+uint16_t orc_epilogue_plain(float v);
+uint16_t orc_epilogue_residual(float v, uint16_t residual);
+uint16_t orc_epilogue_swiglu(float gate, float up);
+float orc_silu(float x);
+
+// ---- glue ----
+// bf16((x * rsqrt(sum x^2 / W + 1e-6)) * w) per row (normalization.metal:59-99).
+void orc_rms_norm(const uint16_t *x, const uint16_t *w, uint32_t rows, uint32_t width, uint16_t *out);
+// Token gather from native rows: bf16(decode(table[token][dim])), token >= vocab -> 0 (embedding.metal:10-18).
+int orc_embed(uint32_t fmt, const uint8_t *table, uint32_t vocab, uint32_t hidden, const uint32_t *tokens,
+              uint32_t rows, uint16_t *out);
+// cos/sin of (anchor + depth[row]) * invfreq[pair], fp32 (rope.metal:51-80).
+void orc_rope_tables(uint32_t anchor, const uint32_t *depth, uint32_t rows, const float *invfreq, uint32_t pairs,
+                     float *cosv, float *sinv);
+
+// ---- INT8 KV ----
+// Per (token, head) over D values: scale = max|v| / 127, code = clamp(rint(v * 127 / max), -127, 127)
+// (Q8PageFormatReference.hpp:107-122, attention_store.h:52-85). The stored scale is fp16 when
+// half_scale is nonzero (rounded after the codes are computed), else fp32; *scale_out holds its value.
+void orc_kv_quantize(const float *v, uint32_t D, int half_scale, int8_t *codes, float *scale_out);
+
+struct OrcAttention {
+  uint32_t q_heads, kv_heads, head_dim;
+  uint32_t rows;        // query rows of the block
+  uint32_t committed;   // tokens in the cache before the block; row r sits at slot committed + r
+  uint32_t page_tokens; // tokens per page
+  uint32_t splits;      // history splits merged in split order (1 = none)
+  uint32_t pages_per_split;
+  uint32_t half_scale;  // scales are fp16 values (already rounded) -- informational
+};
+// q/k per-head RMS norm + partial RoPE + staging (attention_qkv_prepare.h:28-91).
+// qkv bf16 [rows][(q_heads + 2 kv_heads) * D]; qw/kw bf16 [D] norm weights (NULL = no norm);
+// cos/sin fp32 [rows][pairs]; pairs*2 <= D rotated as (i, i + pairs).
+// q_out bf16 [rows][q_heads][D]; k_out/v_out fp32 [rows][kv_heads][D] are the values to quantize.
+void orc_attention_prepare(const struct OrcAttention *a, const uint16_t *qkv, const uint16_t *qw, const uint16_t *kw,
+                           const float *cosv, const float *sinv, uint32_t pairs, uint16_t *q_out, float *k_out,
+                           float *v_out);
+// Block-causal attention over paged INT8 KV, page by page with the online softmax of
+// paged_attention_tile.h:179-285 and the ordered split merge of :499-535.
+// pages: page_table[p] names the physical page of logical page p. A physical page holds
+// keys int8 [kv_heads][page_tokens][D], values int8 [kv_heads][page_tokens][D] and scales
+// float [kv_heads][page_tokens] each (already the stored, possibly fp16-rounded, values).
+// ancestors[r]: bit j set when block row j is visible to row r (chain: (2 << r) - 1).
+// out bf16 [rows][q_heads * D]. out64 (optional) is the fp64 dense-softmax reference
+// (q8_flash_attention_metal_test.mm:485-536), unrounded.
+void orc_attention(const struct OrcAttention *a, const uint16_t *q, const int8_t *kcodes, const float *kscales,
+                   const int8_t *vcodes, const float *vscales, const uint32_t *page_table,
+                   const uint32_t *ancestors, uint16_t *out, double *out64, int threads);
+
+// ---- acceptance ----
+#define ORC_NO_TOKEN 0xFFFFFFFFu
+// Largest finite logit, ties to the lowest id; NaN and -inf skipped (sampling.metal:1896-1997).
+uint32_t orc_argmax(const float *logits, uint32_t vocab);
+struct OrcTreeRow { uint32_t ancestors; uint16_t parent; uint16_t depth; };
+// sampling.metal:2044-2083 decode_accept_tree for one lane.
+// tokens[r]: input token of row r; selected[r]: the target's selection at row r.
+// Returns kept count; out_tokens[0..kept), *accepted, *retained_rows (ancestor mask of the last kept row).
+uint32_t orc_accept_tree(const struct OrcTreeRow *tree, const uint32_t *tokens, const uint32_t *selected,
+                         uint32_t rows, uint32_t remaining, const uint32_t *stop_tokens, uint32_t stops,
+                         uint32_t *out_tokens, uint32_t *accepted, uint32_t *retained_rows);
+// One sampled verify row under the textbook full-vocabulary rule in the reference's order of
+// operations (sampling.metal:713-885): weight_t = exp((logit_t - max) / T); p = weight / total;
+// accept the drafted token iff u_child * q[draft] < p[draft]; else draw from max(p - q, 0)
+// renormalised by an id-ordered prefix walk at u_row. q NULL: plain draw at u_row * total.
+uint32_t orc_rejection_row(const float *logits, uint32_t vocab, float temperature, const float *q,
+                           uint32_t draft_token, float u_child, float u_row, int *accepted_draft);
+
+// ---- Gated DeltaNet ----
+struct OrcGdn { uint32_t key_heads, value_heads, head_dim /*128*/, conv_taps /*4*/; };
+// One token step on one value head's state S [D v][D k] fp32 (gdn.metal:270-298):
+// S *= d; mem = S k; delta = beta (v - mem); S += delta k^T. o (optional) = S q after the update.
+void orc_gdn_step(float *S, uint32_t D, const float *k, const float *v, float decay, float beta, const float *q,
+                  float *o);
+
+#ifdef __cplusplus
+}
+#endif

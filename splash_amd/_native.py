@@ -1,0 +1,142 @@
+"""ctypes loader of libsplash_hip.so. Fails loudly when the library is missing."""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+def library_path():
+    return os.path.join(_HERE, "lib", "libsplash_hip.so")
+
+
+class SplashError(RuntimeError):
+    """A failed C ABI call; .status is the sp_status code."""
+
+    def __init__(self, status, message):
+        super().__init__(f"sp_status {status}: {message}")
+        self.status = status
+        self.message = message
+
+
+class InvalidArgument(SplashError, ValueError):
+    """SP_INVALID_ARGUMENT / SP_UNKNOWN_KERNEL: the operators' std::invalid_argument."""
+
+
+def _load():
+    path = library_path()
+    if not os.path.exists(path):
+        raise ImportError(
+            f"{path} is missing: build it with `python -c 'import __graft_entry__ as g; g.build()'` "
+            "(or `make -C splash_amd/csrc`); there is no fallback path")
+    return ctypes.CDLL(path, mode=ctypes.RTLD_GLOBAL)
+
+
+lib = _load()
+
+SP_OK, SP_INVALID_ARGUMENT, SP_BACKEND_ERROR, SP_UNHEALTHY, SP_BUSY, SP_OUT_OF_MEMORY, SP_UNKNOWN_KERNEL, SP_TIMEOUT = range(8)
+
+lib.sp_last_error.restype = ctypes.c_char_p
+
+
+def check(status):
+    if status == SP_OK:
+        return
+    message = lib.sp_last_error().decode("utf-8", "replace")
+    if status in (SP_INVALID_ARGUMENT, SP_UNKNOWN_KERNEL):
+        raise InvalidArgument(status, message)
+    raise SplashError(status, message)
+
+
+c_u32, c_u64, c_p, c_int, c_double, c_size = (ctypes.c_uint32, ctypes.c_uint64, ctypes.c_void_p, ctypes.c_int,
+                                              ctypes.c_double, ctypes.c_size_t)
+P = ctypes.POINTER
+
+
+class DeviceInfo(ctypes.Structure):
+    _fields_ = [("name", ctypes.c_char * 64), ("arch", ctypes.c_char * 32), ("compute_units", c_u32),
+                ("wavefront_size", c_u32), ("lds_bytes_per_cu", c_u32), ("l2_bytes", c_u32), ("hbm_bytes", c_u64),
+                ("clock_khz", c_u32), ("memory_clock_khz", c_u32), ("memory_bus_bits", c_u32)]
+
+
+class Dispatch(ctypes.Structure):
+    _fields_ = [("kernel", ctypes.c_char_p), ("buffer_count", c_u32), ("buffers", P(c_p)), ("params", c_p),
+                ("params_bytes", c_u32), ("grid", c_u32 * 3), ("block", c_u32 * 3), ("indirect", c_p),
+                ("indirect_offset", c_u64)]
+
+
+class MemoryStats(ctypes.Structure):
+    _fields_ = [("allocated_bytes", c_u64), ("peak_allocated_bytes", c_u64), ("device_current_allocated_bytes", c_u64),
+                ("device_peak_allocated_bytes", c_u64)]
+
+
+class LinearPlan(ctypes.Structure):
+    _fields_ = [("rows", c_u32), ("epilogue", c_u32), ("splits", c_u32), ("k_waves", c_u32), ("storage_rows", c_u32),
+                ("float32", c_u32), ("scratch_input", c_u64), ("scratch_partials", c_u64), ("scratch_counters", c_u64)]
+
+
+def _sig(name, restype, *argtypes):
+    fn = getattr(lib, name)
+    fn.restype = restype
+    fn.argtypes = list(argtypes)
+    return fn
+
+
+_sig("sp_backend_create", c_int, c_int, c_double, P(c_p))
+_sig("sp_backend_destroy", None, c_p)
+_sig("sp_backend_stop", None, c_p)
+_sig("sp_backend_device_info", c_int, c_p, P(DeviceInfo))
+_sig("sp_buffer_alloc", c_int, c_p, c_u64, c_int, ctypes.c_char_p, P(c_p))
+_sig("sp_buffer_view", c_int, c_p, c_u64, c_u64, P(c_p))
+_sig("sp_buffer_retain", None, c_p)
+_sig("sp_buffer_release", None, c_p)
+_sig("sp_buffer_size", c_u64, c_p)
+_sig("sp_buffer_allocated", c_u64, c_p)
+_sig("sp_buffer_storage", c_int, c_p)
+_sig("sp_buffer_contents", c_p, c_p)
+_sig("sp_buffer_gpu_address", c_u64, c_p)
+_sig("sp_buffer_same_view", c_int, c_p, c_p)
+_sig("sp_buffer_upload", c_int, c_p, c_u64, c_p, c_u64)
+_sig("sp_buffer_download", c_int, c_p, c_u64, c_p, c_u64)
+_sig("sp_buffer_fill", c_int, c_p, c_u64, c_int, c_u64)
+_sig("sp_kernel_exists", c_int, ctypes.c_char_p)
+_sig("sp_kernel_names", c_size, ctypes.c_char_p, c_size)
+_sig("sp_submit", c_int, c_p, P(Dispatch), c_u32, c_p, c_p, P(c_p))
+_sig("sp_ticket_ready", c_int, c_p)
+_sig("sp_ticket_wait", c_int, c_p, P(c_double), P(c_double))
+_sig("sp_ticket_release", None, c_p)
+_sig("sp_backend_set_dispatch_profiling", None, c_p, c_int)
+_sig("sp_ticket_wait_profiled", c_int, c_p, P(c_double), P(c_double), P(c_double), c_u32)
+_sig("sp_command_create", c_int, c_p, P(Dispatch), c_u32, P(c_p))
+_sig("sp_command_submit", c_int, c_p, c_p, c_p, P(c_p))
+_sig("sp_command_release", None, c_p)
+_sig("sp_command_in_flight", c_int, c_p)
+_sig("sp_backend_healthy", c_int, c_p)
+_sig("sp_backend_check_health", c_int, c_p)
+_sig("sp_backend_unhealthy_reason", c_size, c_p, ctypes.c_char_p, c_size)
+_sig("sp_memory_stats", c_int, c_p, P(MemoryStats))
+_sig("sp_restart_peaks", None, c_p)
+_sig("sp_backend_stream", c_p, c_p)
+
+_sig("spo_graph_create", c_int, P(c_p))
+_sig("spo_graph_destroy", None, c_p)
+_sig("spo_graph_size", c_u32, c_p)
+_sig("spo_graph_kernel", c_size, c_p, c_u32, ctypes.c_char_p, c_size)
+_sig("spo_graph_add", c_int, c_p, ctypes.c_char_p, P(c_p), c_u32, c_p, c_u32, P(c_u32), P(c_u32))
+_sig("spo_graph_submit", c_int, c_p, c_p, P(c_p))
+_sig("spo_graph_record", c_int, c_p, c_p, P(c_p))
+_sig("spo_gguf_image_bytes", c_u64, c_u32, c_u32, c_u32)
+_sig("spo_gguf_table_bytes", c_u64, c_u32, c_u32)
+_sig("spo_gguf_pack_image", c_int, c_u32, c_p, c_u32, c_u32, c_p)
+_sig("spo_gguf_unpack_image", c_int, c_u32, c_p, c_u32, c_u32, c_p)
+_sig("spo_gguf_add_dequant", c_int, c_p, c_u32, c_p, c_p, c_u32, c_u32)
+_sig("spo_projection_create", c_int, c_u32, P(c_u32), P(c_u32), c_u32, P(c_p), c_int, P(c_p))
+_sig("spo_projection_destroy", None, c_p)
+_sig("spo_projection_weight_bytes", c_u64, c_p)
+_sig("spo_linear_create", c_int, c_p, P(c_p))
+_sig("spo_linear_create_calibrated", c_int, c_u32, c_u32, c_u32, P(c_p))
+_sig("spo_linear_destroy", None, c_p)
+_sig("spo_linear_plan_for", c_int, c_p, c_p, c_u32, c_u32, P(LinearPlan))
+_sig("spo_linear_plan_with", c_int, c_p, P(LinearPlan))
+_sig("spo_linear_add", c_int, c_p, c_p, c_p, c_p, P(LinearPlan), c_p, c_p, c_p, c_p, c_p, c_p, c_int)
+_sig("spo_linear_add_swiglu", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_u32, c_p, c_p, c_p)
+_sig("spo_linear_scratch_size", c_int, c_p, c_u32, c_u32, c_u32, P(c_u64), P(c_u64), P(c_u64))

@@ -1,0 +1,143 @@
+// Quantized projection ABI shared by the host operators and the HIP kernels: the weight image a
+// K-quant tensor is re-tiled into at load time, the activation table a projection reads, and the
+// parameter structs of the kernels. The counterpart of the reference's runtime/metal/abi/Gguf.h and
+// QuantFormat.h, laid out for 64-lane wavefronts and 16x16 MFMA tiles instead of 32-lane
+// simdgroups.
+//
+// Vocabulary: a group is 32 inputs, a super-block 256 (one native K-quant block); a column tile is
+// 16 output columns (one MFMA tile); a record is one column tile's bytes of one super-block.
+//
+// WEIGHT IMAGE  [N / 16][K / 256] records, K fastest, so a wave that walks K reads one contiguous
+// stream. Lane l of a wave owns column c = l % 16 and input quarter kq = l / 16 of the tile.
+//
+//   Q4_K record, 2304 B (16 native blocks of 144 B, byte for byte re-ordered):
+//     [   0, 2048)  nibbles: two 1024-B halves h; in half h lane l owns 16 B at 1024 h + 16 l =
+//                   native qs bytes  [64 h + 4 kq, +4) [64 h + 16 + 4 kq, +4)
+//                                    [64 h + 32 + 4 kq, +4) [64 h + 48 + 4 kq, +4)
+//                   i.e. words w0, w1 hold inputs 4 kq + 0..3 and 16 + 4 kq + 0..3 of groups 4 h
+//                   (low nibbles) and 4 h + 1 (high nibbles), w2, w3 those of groups 4 h + 2, 4 h + 3.
+//     [2048, 2304)  meta: column c's native d, dmin and 12 scale bytes at 2048 + 16 c.
+//
+//   Q6_K record, 3360 B (16 native blocks of 210 B):
+//     [   0, 2048)  low nibbles, arranged exactly as Q4_K's nibbles (code & 15 of the same inputs).
+//     [2048, 3072)  high bits: lane l owns 16 B at 2048 + 16 l: word i covers groups 2 i, 2 i + 1;
+//                   the 2-bit field of pair v (0..7: operand register v % 4 of group 2 i + v / 4)
+//                   sits at bits 2 v (low half's code) and 16 + 2 v (high half's code).
+//     [3072, 3328)  scales: column c's 16 int8 scales at 3072 + 16 c.
+//     [3328, 3360)  d: column c's fp16 d at 3328 + 2 c.
+//
+// Within a group, lane (c, kq) holds eight codes as four registers of two bf16 operands
+// 128 + code: register j (0..3) holds inputs 16 (j / 2) + 4 kq + (j % 2) [low half] and that + 2
+// [high half]. Element e = 2 j + half of the lane's MFMA operand is therefore input
+//     gguf_operand_input(kq, e) = 16 (e / 4) + 4 kq + {0, 2, 1, 3}[e % 4]
+// of the group, and the activation table stores x in that order.
+//
+// ACTIVATION TABLE of `tiles` row tiles (16 rows each, rows past the live ones zero) and G = K / 32
+// groups: values bf16 [tiles][G][64 lanes][8]: lane (r = l % 16, kq = l / 16) holds inputs
+// gguf_operand_input(kq, 0..7) of row 16 t + r; then sums32 fp32 [tiles][G][16 rows] and sums16
+// fp32 [tiles][2 G][16 rows], the fp32 sums of each row's 32 and 16 inputs in input order.
+#pragma once
+#include <stdint.h>
+
+#define GGUF_FMT_Q4K 0u
+#define GGUF_FMT_Q6K 4u
+#define GGUF_FMT_COUNT 26u
+
+#define GGUF_BLOCK 256u
+#define GGUF_TILE_COLUMNS 16u
+#define GGUF_Q4K_NATIVE 144u
+#define GGUF_Q6K_NATIVE 210u
+#define GGUF_Q4K_RECORD (GGUF_TILE_COLUMNS * GGUF_Q4K_NATIVE)  // 2304
+#define GGUF_Q6K_RECORD (GGUF_TILE_COLUMNS * GGUF_Q6K_NATIVE)  // 3360
+#define GGUF_Q6K_HIGH 2048u
+#define GGUF_Q6K_SCALES 3072u
+#define GGUF_Q6K_D 3328u
+#define GGUF_ROW_TILE 16u
+// The most rows one projection dispatch takes: four lanes of sixteen verify rows.
+#define GGUF_MAXIMUM_ROWS 64u
+#define GGUF_MAXIMUM_SEGMENTS 3u
+#define GGUF_MAXIMUM_SPLITS 16u
+
+#if defined(__HIPCC__) || defined(__cplusplus)
+#define GGUF_INLINE inline
+#if defined(__HIPCC__)
+#undef GGUF_INLINE
+#define GGUF_INLINE __host__ __device__ inline
+#endif
+
+GGUF_INLINE uint32_t gguf_record_bytes(uint32_t format) {
+  return format == GGUF_FMT_Q4K ? GGUF_Q4K_RECORD : format == GGUF_FMT_Q6K ? GGUF_Q6K_RECORD : 0u;
+}
+GGUF_INLINE uint32_t gguf_native_bytes(uint32_t format) {
+  return format == GGUF_FMT_Q4K ? GGUF_Q4K_NATIVE : format == GGUF_FMT_Q6K ? GGUF_Q6K_NATIVE : 0u;
+}
+// Bytes of the image of an [N, K] tensor (N a multiple of 16, K of 256): those of its native rows.
+GGUF_INLINE uint64_t gguf_image_bytes(uint32_t format, uint32_t n, uint32_t k) {
+  return uint64_t(n / GGUF_TILE_COLUMNS) * (k / GGUF_BLOCK) * gguf_record_bytes(format);
+}
+GGUF_INLINE uint32_t gguf_operand_input(uint32_t kq, uint32_t e) {
+  return 16u * (e >> 2) + 4u * kq + (((e & 1u) << 1) | ((e >> 1) & 1u));
+}
+GGUF_INLINE uint32_t gguf_row_tiles(uint32_t rows) { return (rows + GGUF_ROW_TILE - 1) / GGUF_ROW_TILE; }
+// Activation table geometry, in bytes from the table's start.
+GGUF_INLINE uint64_t gguf_table_values_bytes(uint32_t k, uint32_t tiles) { return uint64_t(tiles) * k * 16u * 2u; }
+GGUF_INLINE uint64_t gguf_table_sums32_offset(uint32_t k, uint32_t tiles) { return gguf_table_values_bytes(k, tiles); }
+GGUF_INLINE uint64_t gguf_table_sums16_offset(uint32_t k, uint32_t tiles) {
+  return gguf_table_sums32_offset(k, tiles) + uint64_t(tiles) * (k / 32u) * 16u * 4u;
+}
+GGUF_INLINE uint64_t gguf_table_bytes(uint32_t k, uint32_t tiles) {
+  return gguf_table_sums16_offset(k, tiles) + uint64_t(tiles) * (k / 16u) * 16u * 4u;
+}
+#endif
+
+// gguf_prepare_table: bf16 rows [rows][input_size] -> the activation table of `tiles` row tiles.
+// Grid (K / 32, tiles), 64 threads.
+struct GgufPrepareParams {
+  uint32_t input_size;
+  uint32_t rows;
+  uint32_t tiles;
+  uint32_t row_stride;  // elements between input rows
+};
+
+// Epilogues of a decode projection (the reference's LinearEpilogue, runtime/ops/Linear.hpp:77).
+#define GGUF_EPILOGUE_PLAIN 0u     // out = bf16(v)         kernel suffix _a
+#define GGUF_EPILOGUE_PLAIN_F32 1u // out = v               kernel suffix _a_f32
+#define GGUF_EPILOGUE_RESIDUAL 2u  // out = bf16(v + res)   kernel suffix _r
+#define GGUF_EPILOGUE_GATE_UP 3u   // out = bf16(bf16(up) * silu(bf16(gate)))   kernel suffix _g
+
+// gguf_decode_<fmt>_m<16|32|64>_<a|a_f32|r|g>: up to three column segments of one format in one
+// dispatch (the reference's GgufDecodeFusedParams, runtime/metal/abi/Gguf.h:168-178), tiles in
+// segment order; a single tensor is one segment. A gate/up pair binds gate as segment 0 and up as
+// segment 1, both of cols[0] columns. Grid (units / waves-across-tiles, splits), 256 threads.
+struct GgufDecodeParams {
+  uint32_t input_size;  // K
+  uint32_t rows;        // live rows
+  uint32_t splits;      // K partitions across workgroups (grid.y); 1 = no cross-workgroup reduction
+  uint32_t k_waves;     // waves of a workgroup that share its tiles and split its K partition: 1, 2 or 4
+  uint32_t out_stride;  // columns of a destination row
+  uint32_t cols[3];     // columns per segment (multiples of 16); 0 past the last
+  uint32_t offset[3];   // first destination column per segment
+  uint32_t units;       // wave work units: each GGUF_DECODE_UNIT_TILES column tiles (gate/up: pairs)
+};
+
+// gguf_dequant_<fmt>: the image's fp32 values [N][K], for the bit-exactness test
+// (the reference's gguf_dequant_test.metal). Grid (K / 256, N / 16), 64 threads.
+struct GgufDequantParams {
+  uint32_t input_size;
+  uint32_t output_size;
+};
+
+// gguf_embed_<fmt>: out[r][:] = bf16(decode(table row tokens[r])) from NATIVE rows; a token at or
+// past the vocabulary gives zeros (the reference's GgufEmbedParams, abi/Gguf.h:180-185).
+struct GgufEmbedParams {
+  uint32_t rows;
+  uint32_t vocabulary;
+  uint32_t hidden;
+};
+
+#ifdef __cplusplus
+static_assert(sizeof(GgufPrepareParams) == 16, "prepare parameters are 16 bytes on both sides");
+static_assert(sizeof(GgufDecodeParams) == 48, "decode parameters are 48 bytes on both sides");
+static_assert(sizeof(GgufDequantParams) == 8, "dequant parameters are 8 bytes on both sides");
+static_assert(sizeof(GgufEmbedParams) == 12, "embedding parameters are 12 bytes on both sides");
+#endif

@@ -1,0 +1,58 @@
+// Device-side decode of the Q4_K / Q6_K weight image (abi/Gguf.h): every kernel that reads the
+// image -- the projection tiles, the value dump of the bit-exactness test -- unpacks it through
+// these functions, so the test of one covers the others.
+#pragma once
+#include "abi/Gguf.h"
+#include "kernels/device_common.hpp"
+
+namespace splash::kernels {
+
+// The 6-bit scales and mins of a Q4_K super-block (llama.cpp get_scale_min_k4; the reference's
+// quant_formats.h:105-118), four per word as bytes: scales of groups 0..3 and 4..7, mins likewise.
+struct Q4KScales {
+  uint32_t sc_lo, sc_hi, mn_lo, mn_hi;
+  float d, dmin;
+};
+__device__ __forceinline__ Q4KScales q4k_scales(uint4 meta) {
+  Q4KScales s;
+  s.d = half_bits_to_float(meta.x & 0xFFFFu);
+  s.dmin = half_bits_to_float(meta.x >> 16);
+  s.sc_lo = meta.y & 0x3F3F3F3Fu;
+  s.mn_lo = meta.z & 0x3F3F3F3Fu;
+  s.sc_hi = (meta.w & 0x0F0F0F0Fu) | ((meta.y >> 2) & 0x30303030u);
+  s.mn_hi = ((meta.w >> 4) & 0x0F0F0F0Fu) | ((meta.z >> 2) & 0x30303030u);
+  return s;
+}
+__device__ __forceinline__ float byte_of(uint32_t word, uint32_t index) { return float((word >> (8u * index)) & 0xFFu); }
+
+// Register j (0..3) of a group's bf16 operands 128 + code, from the two words that hold the
+// lane's eight codes of that group in their low (high = false) or high nibbles.
+template <bool High> __device__ __forceinline__ uint4 q4_operands(uint32_t wa, uint32_t wb) {
+  constexpr uint32_t kMask = 0x000F000Fu, kBase = 0x43004300u;  // bf16 0x4300 = 128, ulp 1
+  constexpr uint32_t s = High ? 4u : 0u;
+  uint4 r;
+  r.x = ((wa >> s) & kMask) | kBase;
+  r.y = ((wa >> (s + 8u)) & kMask) | kBase;
+  r.z = ((wb >> s) & kMask) | kBase;
+  r.w = ((wb >> (s + 8u)) & kMask) | kBase;
+  return r;
+}
+// The same for Q6_K: the low nibbles as Q4_K's, then the 2-bit high fields of pair v0..v0+3 of
+// the high-bits word (abi/Gguf.h) at bits 4..5 of each half.
+template <bool High, uint32_t V0> __device__ __forceinline__ uint4 q6_operands(uint32_t wa, uint32_t wb, uint32_t hw) {
+  constexpr uint32_t kHigh = 0x00300030u;
+  uint4 r = q4_operands<High>(wa, wb);
+  auto field = [&](uint32_t v) -> uint32_t {
+    return (2u * v >= 4u ? hw >> (2u * v - 4u) : hw << (4u - 2u * v)) & kHigh;
+  };
+  r.x |= field(V0);
+  r.y |= field(V0 + 1);
+  r.z |= field(V0 + 2);
+  r.w |= field(V0 + 3);
+  return r;
+}
+
+// The code (0..15, or 0..63 for Q6_K) in half `half` of operand register `reg`.
+__device__ __forceinline__ uint32_t operand_code(uint32_t reg, uint32_t half) { return (reg >> (16u * half)) & 0x7Fu; }
+
+} // namespace splash::kernels

@@ -1,0 +1,147 @@
+#include "ops/GgufImage.hpp"
+
+#include <cstring>
+#include <stdexcept>
+#include <string>
+#include <thread>
+
+namespace splash::ops {
+
+namespace {
+
+void requireShape(uint32_t formatId, uint32_t rows, uint32_t inputSize) {
+  if (!gguf_record_bytes(formatId)) throw std::invalid_argument("no weight image for format " + std::to_string(formatId));
+  if (!rows || rows % GGUF_TILE_COLUMNS) throw std::invalid_argument("a weight image holds whole tiles of 16 rows");
+  if (!inputSize || inputSize % GGUF_BLOCK) throw std::invalid_argument("a weight image holds whole super-blocks of 256 inputs");
+}
+
+// Q6_K: the 6-bit code of input k (0..255) of a native block (llama.cpp dequantize_row_q6_K order).
+inline uint32_t q6Code(const uint8_t *blk, uint32_t k) {
+  const uint32_t n = k / 128, r = (k % 128) / 32, e = k % 32;
+  const uint32_t l4 = (blk[64 * n + e + 32 * (r & 1)] >> (4 * (r >> 1))) & 15u;
+  const uint32_t h2 = (blk[128 + 32 * n + e] >> (2 * r)) & 3u;
+  return l4 | (h2 << 4);
+}
+inline void q6SetCode(uint8_t *blk, uint32_t k, uint32_t code) {
+  const uint32_t n = k / 128, r = (k % 128) / 32, e = k % 32;
+  uint8_t &low = blk[64 * n + e + 32 * (r & 1)];
+  low = uint8_t((low & ~(0xFu << (4 * (r >> 1)))) | ((code & 15u) << (4 * (r >> 1))));
+  uint8_t &high = blk[128 + 32 * n + e];
+  high = uint8_t((high & ~(0x3u << (2 * r))) | ((code >> 4) << (2 * r)));
+}
+
+template <class Body> void forTiles(uint32_t tiles, Body body) {
+  const uint32_t workers = std::min<uint32_t>(std::max(1u, std::thread::hardware_concurrency()), std::max(1u, tiles / 8));
+  if (workers <= 1) { for (uint32_t t = 0; t < tiles; ++t) body(t); return; }
+  std::vector<std::thread> pool;
+  for (uint32_t w = 0; w < workers; ++w)
+    pool.emplace_back([=] { for (uint32_t t = w; t < tiles; t += workers) body(t); });
+  for (auto &th : pool) th.join();
+}
+
+// The nibble part of a record: lane (c, kq), half h, word w (0..3) holds, in its low nibbles, the
+// codes of group 4 h + 2 (w / 2) and, in its high nibbles, of group 4 h + 2 (w / 2) + 1, for inputs
+// 16 (w % 2) + 4 kq + 0..3 of each group, one byte per input.
+inline uint32_t nibbleOffset(uint32_t c, uint32_t kq, uint32_t h, uint32_t w) { return 1024 * h + 16 * (kq * 16 + c) + 4 * w; }
+
+} // namespace
+
+void packGgufImage(uint32_t formatId, const uint8_t *native, uint32_t rows, uint32_t inputSize, uint8_t *image) {
+  requireShape(formatId, rows, inputSize);
+  const uint32_t blocks = inputSize / GGUF_BLOCK, nb = gguf_native_bytes(formatId), rb = gguf_record_bytes(formatId);
+  const size_t rowBytes = size_t(blocks) * nb;
+  forTiles(rows / GGUF_TILE_COLUMNS, [&](uint32_t tile) {
+    for (uint32_t b = 0; b < blocks; ++b) {
+      uint8_t *rec = image + (size_t(tile) * blocks + b) * rb;
+      std::memset(rec, 0, rb);
+      for (uint32_t c = 0; c < 16; ++c) {
+        const uint8_t *blk = native + size_t(16 * tile + c) * rowBytes + size_t(b) * nb;
+        if (formatId == GGUF_FMT_Q4K) {
+          // Native qs byte 32 p + i holds input i of groups 2 p (low) and 2 p + 1 (high): the
+          // record's words are native words, moved.
+          const uint8_t *qs = blk + 16;
+          for (uint32_t kq = 0; kq < 4; ++kq)
+            for (uint32_t h = 0; h < 2; ++h)
+              for (uint32_t w = 0; w < 4; ++w)
+                std::memcpy(rec + nibbleOffset(c, kq, h, w), qs + 64 * h + 32 * (w / 2) + 16 * (w % 2) + 4 * kq, 4);
+          std::memcpy(rec + 2048 + 16 * c, blk, 16);
+        } else {
+          for (uint32_t kq = 0; kq < 4; ++kq) {
+            for (uint32_t h = 0; h < 2; ++h)
+              for (uint32_t w = 0; w < 4; ++w)
+                for (uint32_t i = 0; i < 4; ++i) {
+                  const uint32_t group = 4 * h + 2 * (w / 2), input = 16 * (w % 2) + 4 * kq + i;
+                  const uint32_t low = q6Code(blk, 32 * group + input) & 15u, high = q6Code(blk, 32 * (group + 1) + input) & 15u;
+                  rec[nibbleOffset(c, kq, h, w) + i] = uint8_t(low | (high << 4));
+                }
+            // High bits: word i covers groups 2 i, 2 i + 1; pair v = register v % 4 of group
+            // 2 i + v / 4; element e = 2 (v % 4) + half; fields at bits 2 v and 16 + 2 v.
+            for (uint32_t i = 0; i < 4; ++i) {
+              uint32_t word = 0;
+              for (uint32_t v = 0; v < 8; ++v)
+                for (uint32_t half = 0; half < 2; ++half) {
+                  const uint32_t group = 2 * i + v / 4, e = 2 * (v % 4) + half;
+                  const uint32_t code = q6Code(blk, 32 * group + gguf_operand_input(kq, e));
+                  word |= (code >> 4) << (2 * v + 16 * half);
+                }
+              std::memcpy(rec + GGUF_Q6K_HIGH + 16 * (kq * 16 + c) + 4 * i, &word, 4);
+            }
+          }
+          std::memcpy(rec + GGUF_Q6K_SCALES + 16 * c, blk + 192, 16);
+          std::memcpy(rec + GGUF_Q6K_D + 2 * c, blk + 208, 2);
+        }
+      }
+    }
+  });
+}
+
+std::vector<uint8_t> packGgufImage(uint32_t formatId, const std::vector<uint8_t> &native, uint32_t rows, uint32_t inputSize) {
+  requireShape(formatId, rows, inputSize);
+  if (native.size() != gguf_image_bytes(formatId, rows, inputSize))
+    throw std::invalid_argument("native rows do not match the tensor's shape");
+  std::vector<uint8_t> image(native.size());
+  packGgufImage(formatId, native.data(), rows, inputSize, image.data());
+  return image;
+}
+
+void unpackGgufImage(uint32_t formatId, const uint8_t *image, uint32_t rows, uint32_t inputSize, uint8_t *native) {
+  requireShape(formatId, rows, inputSize);
+  const uint32_t blocks = inputSize / GGUF_BLOCK, nb = gguf_native_bytes(formatId), rb = gguf_record_bytes(formatId);
+  const size_t rowBytes = size_t(blocks) * nb;
+  forTiles(rows / GGUF_TILE_COLUMNS, [&](uint32_t tile) {
+    for (uint32_t b = 0; b < blocks; ++b) {
+      const uint8_t *rec = image + (size_t(tile) * blocks + b) * rb;
+      for (uint32_t c = 0; c < 16; ++c) {
+        uint8_t *blk = native + size_t(16 * tile + c) * rowBytes + size_t(b) * nb;
+        std::memset(blk, 0, nb);
+        if (formatId == GGUF_FMT_Q4K) {
+          for (uint32_t kq = 0; kq < 4; ++kq)
+            for (uint32_t h = 0; h < 2; ++h)
+              for (uint32_t w = 0; w < 4; ++w)
+                std::memcpy(blk + 16 + 64 * h + 32 * (w / 2) + 16 * (w % 2) + 4 * kq, rec + nibbleOffset(c, kq, h, w), 4);
+          std::memcpy(blk, rec + 2048 + 16 * c, 16);
+        } else {
+          for (uint32_t kq = 0; kq < 4; ++kq) {
+            uint32_t highWords[4];
+            std::memcpy(highWords, rec + GGUF_Q6K_HIGH + 16 * (kq * 16 + c), 16);
+            for (uint32_t group = 0; group < 8; ++group)
+              for (uint32_t e = 0; e < 8; ++e) {
+                const uint32_t input = gguf_operand_input(kq, e);
+                // low nibble: word w = 2 ((group % 4) / 2) + input / 16 of half group / 4, byte input % 4 ... of lane kq
+                const uint32_t h = group / 4, w = 2 * ((group % 4) / 2) + input / 16, i = input % 4;
+                const uint8_t byte = rec[nibbleOffset(c, kq, h, w) + i];
+                const uint32_t low = group % 2 ? byte >> 4 : byte & 15u;
+                const uint32_t v = 4 * (group % 2) + e / 2, half = e % 2;
+                const uint32_t high = (highWords[group / 2] >> (2 * v + 16 * half)) & 3u;
+                q6SetCode(blk, 32 * group + input, low | (high << 4));
+              }
+          }
+          std::memcpy(blk + 192, rec + GGUF_Q6K_SCALES + 16 * c, 16);
+          std::memcpy(blk + 208, rec + GGUF_Q6K_D + 2 * c, 2);
+        }
+      }
+    }
+  });
+}
+
+} // namespace splash::ops

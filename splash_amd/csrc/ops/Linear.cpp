@@ -1,0 +1,235 @@
+#include "ops/Linear.hpp"
+
+#include <array>
+#include <stdexcept>
+
+namespace splash::ops {
+
+void requireBytes(const hip::Buffer &buffer, uint64_t bytes, const char *what) {
+  if (!buffer) throw std::invalid_argument(std::string(what) + " buffer is missing");
+  if (buffer.sizeBytes() < bytes) throw std::invalid_argument(std::string(what) + " buffer is too small");
+}
+
+namespace {
+
+const char *epilogueSuffix(LinearEpilogue epilogue, FloatOutput destination) {
+  switch (epilogue) {
+  case LinearEpilogue::None: return destination == FloatOutput::Float32 ? "_a_f32" : "_a";
+  case LinearEpilogue::Residual: return "_r";
+  case LinearEpilogue::GateUp: return "_g";
+  }
+  return "_a";
+}
+
+// Wave work units of a dispatch: two column tiles each; a gate/up pair's unit is one tile of each.
+uint32_t unitsOf(uint32_t columns, LinearEpilogue epilogue) {
+  const uint32_t tiles = columns / GGUF_TILE_COLUMNS;
+  return epilogue == LinearEpilogue::GateUp ? tiles : (tiles + 1) / 2;
+}
+
+void requireSegments(const Projection &p, LinearMatrix matrix) {
+  if (p.outputSize != matrix.outputSize || p.inputSize != matrix.inputSize)
+    throw std::invalid_argument("block projection does not match its plan's matrix");
+  const std::vector<QuantizedSegment> &segments = p.blocks().segments;
+  if (segments.empty() || segments.size() > GGUF_MAXIMUM_SEGMENTS)
+    throw std::invalid_argument("a block projection dispatch takes one to three segments");
+  for (const QuantizedSegment &s : segments) {
+    if (s.formatId != segments.front().formatId)
+      throw std::invalid_argument("the segments of one block dispatch share a format");
+    if (s.outputSize % GGUF_TILE_COLUMNS || s.inputSize % GGUF_BLOCK)
+      throw std::invalid_argument("block segments hold whole 16-column tiles of whole 256-input super-blocks");
+    requireBytes(s.image, gguf_image_bytes(s.formatId, s.outputSize, s.inputSize), "block weight image");
+  }
+}
+
+} // namespace
+
+LinearPlan::LinearPlan(LinearWorkload workload, LinearConfig config, FloatOutput destination)
+    : workload_(workload), config_(config), destination_(destination) {
+  requireConfiguration();
+}
+
+void LinearPlan::requireConfiguration() const {
+  const auto [n, k] = workload_.matrix;
+  if (!workload_.rows || workload_.rows > kMaximumDecodeTileRows)
+    throw std::invalid_argument("the block tile runs plans of 1 to 64 rows");
+  if (!n || n % GGUF_TILE_COLUMNS || !k || k % GGUF_BLOCK)
+    throw std::invalid_argument("block projections take whole 16-column tiles and 256-input super-blocks");
+  const LinearConfig &c = config_;
+  if (c.kWaves != 1 && c.kWaves != 2 && c.kWaves != 4)
+    throw std::invalid_argument("a block workgroup splits K over 1, 2 or 4 waves");
+  if (!c.validSplits() || uint64_t{c.splits} * c.kWaves > k / GGUF_BLOCK)
+    throw std::invalid_argument("block splits take at least one super-block each");
+  if (destination_ == FloatOutput::Float32 && workload_.epilogue != LinearEpilogue::None)
+    throw std::invalid_argument("only a plain block plan writes fp32");
+}
+
+LinearScratchSize LinearPlan::scratchSize() const noexcept {
+  const auto [n, k] = workload_.matrix;
+  const uint32_t tiles = gguf_row_tiles(workload_.rows);
+  LinearScratchSize size;
+  size.input = gguf_table_bytes(k, tiles);
+  if (config_.splits > 1) {
+    // [split][row][column] fp32 partials over the tile's rows, a gate/up pair's of both tensors,
+    // and one counter per workgroup.
+    const uint64_t columns = workload_.epilogue == LinearEpilogue::GateUp ? 2 * uint64_t{n} : n;
+    const uint32_t across = 4 / config_.kWaves;
+    size.partials = uint64_t{config_.splits} * tiles * GGUF_ROW_TILE * columns * sizeof(float);
+    size.counters = uint64_t{(unitsOf(n, workload_.epilogue) + across - 1) / across} * sizeof(uint32_t);
+  }
+  return size;
+}
+
+Linear::Linear(const sp_device_info &device) noexcept {
+  if (device.compute_units) calibration_.computeUnits = device.compute_units;
+}
+
+LinearPlan Linear::plan(LinearWorkload workload, LinearConfig config, FloatOutput destination) {
+  return LinearPlan(workload, config, destination);
+}
+
+LinearPlan Linear::plan(LinearWorkload w, FloatOutput destination) const {
+  // Fill the device: partition K, first over the waves of a workgroup (summed through LDS, no
+  // memory traffic), then across workgroups (fp32 partials), until the dispatch holds
+  // wavesPerUnit waves per compute unit or a wave's range is down to minimumBlocksPerWave.
+  const uint32_t blocks = w.matrix.inputSize / GGUF_BLOCK;
+  const uint32_t units = std::max(1u, unitsOf(w.matrix.outputSize, w.epilogue));
+  const uint64_t wanted = uint64_t{calibration_.computeUnits} * calibration_.wavesPerUnit;
+  LinearConfig config;
+  auto parts = [&] { return config.splits * config.kWaves; };
+  auto mayDouble = [&] { return uint64_t{units} * parts() < wanted && blocks / (2 * parts()) >= calibration_.minimumBlocksPerWave; };
+  while (config.kWaves < 4 && mayDouble()) config.kWaves *= 2;
+  while (config.splits < LinearConfig::kMaximumSplits && mayDouble()) config.splits *= 2;
+  return LinearPlan(w, config, destination);
+}
+
+LinearPlan Linear::plan(const Projection &projection, uint32_t rows, LinearEpilogue epilogue) const {
+  return plan(LinearWorkload{{projection.outputSize, projection.inputSize}, rows, epilogue},
+              epilogue == LinearEpilogue::None ? projection.destination : FloatOutput::BFloat16);
+}
+
+LinearScratchSize Linear::scratchSize(LinearMatrix matrix, uint32_t rows) const {
+  LinearScratchSize size;
+  for (LinearEpilogue e : {LinearEpilogue::None, LinearEpilogue::Residual, LinearEpilogue::GateUp})
+    size.include(plan(LinearWorkload{matrix, rows, e}).scratchSize());
+  return size;
+}
+
+void Linear::addPrepare(hip::CommandGraph &graph, const hip::Buffer &input, const LinearScratch &scratch, uint32_t width,
+                        uint32_t rows) {
+  if (!rows || rows > kMaximumDecodeTileRows) throw std::invalid_argument("the block tile runs plans of 1 to 64 rows");
+  if (!width || width % GGUF_BLOCK) throw std::invalid_argument("block projections take whole 256-input super-blocks");
+  const uint32_t tiles = gguf_row_tiles(rows);
+  requireBytes(input, uint64_t{rows} * width * 2, "projection input");
+  requireBytes(scratch.input, gguf_table_bytes(width, tiles), "projection table");
+  graph.add("gguf_prepare_table", {input, scratch.input}, GgufPrepareParams{width, rows, tiles, width},
+            {width / 32, tiles, 1}, {64, 1, 1});
+}
+
+PreparedInput Linear::add(hip::CommandGraph &graph, LinearBuffers b, const Projection &p, const LinearPlan &plan,
+                          const Projection *gate) const {
+  const LinearWorkload w = plan.workload();
+  const LinearConfig c = plan.configuration();
+  const auto [n, k] = w.matrix;
+  // Everything is checked before anything is added.
+  requireSegments(p, w.matrix);
+  const bool gateUp = w.epilogue == LinearEpilogue::GateUp;
+  if (gateUp != (gate != nullptr)) throw std::invalid_argument("a block gate/up plan takes a gate projection, no other does");
+  if (gate) {
+    requireSegments(*gate, w.matrix);
+    if (p.blocks().segments.size() != 1 || gate->blocks().segments.size() != 1 ||
+        gate->blocks().segments.front().formatId != p.blocks().segments.front().formatId)
+      throw std::invalid_argument("a one-pass block gate/up takes single tensors of one format");
+  }
+  const uint32_t tiles = gguf_row_tiles(w.rows);
+  const uint64_t outBytes = plan.destination() == FloatOutput::Float32 ? 4 : 2;
+  requireBytes(b.output, uint64_t{w.rows} * n * outBytes, "projection output");
+  if (w.epilogue == LinearEpilogue::Residual) requireBytes(b.residual, uint64_t{w.rows} * n * 2, "projection residual");
+  const LinearScratchSize need = plan.scratchSize();
+  requireBytes(b.scratch.input, need.input, "projection table");
+  if (c.splits > 1) {
+    requireBytes(b.scratch.partials, need.partials, "projection partials");
+    requireBytes(b.scratch.counters, need.counters, "projection counters");
+  }
+  const bool prepared = b.prepared.layout == LinearInput::Table16 && b.prepared.source && b.input &&
+                        b.prepared.source.sameView(b.input);
+  if (!prepared) requireBytes(b.input, uint64_t{w.rows} * k * 2, "projection input");
+
+  if (!prepared) addPrepare(graph, b.input, b.scratch, k, w.rows);
+
+  GgufDecodeParams params{};
+  params.input_size = k;
+  params.rows = w.rows;
+  params.splits = c.splits;
+  params.k_waves = c.kWaves;
+  params.out_stride = n;
+  std::array<hip::Buffer, 3> images;
+  const std::vector<QuantizedSegment> &segments = p.blocks().segments;
+  if (gateUp) {
+    images = {gate->blocks().segments.front().image, segments.front().image, segments.front().image};
+    params.cols[0] = n;
+    params.offset[0] = 0;
+  } else {
+    for (size_t s = 0; s < 3; ++s) {
+      const QuantizedSegment &segment = segments[std::min(s, segments.size() - 1)];
+      images[s] = segment.image;
+      if (s < segments.size()) {
+        params.cols[s] = segment.outputSize;
+        params.offset[s] = segment.columnOffset;
+      }
+    }
+  }
+  params.units = unitsOf(n, w.epilogue);
+  // Unused bindings still name a buffer: the table stands in for them.
+  const hip::Buffer &spare = b.scratch.input;
+  const uint32_t across = 4 / c.kWaves;
+  const std::string name = std::string("gguf_decode_") + segments.front().name() + "_m" + std::to_string(plan.storageRows()) +
+                           epilogueSuffix(w.epilogue, plan.destination());
+  graph.add(name,
+            {images[0], images[1], images[2], b.scratch.input, b.output,
+             w.epilogue == LinearEpilogue::Residual ? b.residual : spare, c.splits > 1 ? b.scratch.partials : spare,
+             c.splits > 1 ? b.scratch.counters : spare},
+            params, {(params.units + across - 1) / across, c.splits, 1}, {256, 1, 1});
+  (void)tiles;
+  return {b.input, LinearInput::Table16};
+}
+
+void Linear::addProjection(hip::CommandGraph &graph, hip::Buffer input, const Projection &projection, hip::Buffer output,
+                           uint32_t rows, LinearScratch scratch) const {
+  LinearBuffers buffers;
+  buffers.input = std::move(input);
+  buffers.output = std::move(output);
+  buffers.scratch = std::move(scratch);
+  add(graph, std::move(buffers), projection, plan(projection, rows));
+}
+
+void Linear::addResidualProjection(hip::CommandGraph &graph, hip::Buffer input, const Projection &projection,
+                                   hip::Buffer residual, hip::Buffer output, uint32_t rows, LinearScratch scratch) const {
+  LinearBuffers buffers;
+  buffers.input = std::move(input);
+  buffers.output = std::move(output);
+  buffers.residual = std::move(residual);
+  buffers.scratch = std::move(scratch);
+  add(graph, std::move(buffers), projection, plan(projection, rows, LinearEpilogue::Residual));
+}
+
+void Linear::addSwiGlu(hip::CommandGraph &graph, const SwiGluProjections &ffn, const FfnBuffers &b, hip::Buffer residual,
+                       hip::Buffer output, uint32_t rows, PreparedInput normalized) const {
+  if (!ffn.gate || !ffn.up || !ffn.down) throw std::invalid_argument("a SwiGLU takes gate, up and down projections");
+  LinearBuffers pair;
+  pair.input = b.normalized;
+  pair.output = b.intermediate;
+  pair.scratch = b.scratch;
+  pair.prepared = std::move(normalized);
+  const LinearPlan pairPlan = plan(*ffn.up, rows, LinearEpilogue::GateUp);
+  LinearBuffers down;
+  down.input = b.intermediate;
+  down.output = std::move(output);
+  down.residual = std::move(residual);
+  down.scratch = b.scratch;
+  const LinearPlan downPlan = plan(*ffn.down, rows, LinearEpilogue::Residual);
+  add(graph, std::move(pair), *ffn.up, pairPlan, ffn.gate);
+  add(graph, std::move(down), *ffn.down, downPlan);
+}
+
+} // namespace splash::ops

@@ -1,0 +1,163 @@
+// Quantized projection planner and dispatcher for the verify step's 1..64-row blocks: the
+// counterpart of the reference's ops::Linear (runtime/ops/Linear.hpp:138-376, LinearGguf.cpp) over
+// the gfx950 MFMA tile (kernels/gguf_linear.hip). Same roles: a LinearPlan fixes tile height, K
+// partitions and scratch; Linear::add validates every buffer and throws std::invalid_argument
+// before any dispatch is added; producers and consumers hand the prepared activation table along
+// as PreparedInput.
+#pragma once
+#include "abi/Gguf.h"
+#include "hip/Backend.hpp"
+#include "ops/Weights.hpp"
+
+#include <algorithm>
+#include <compare>
+#include <cstdint>
+#include <string>
+
+namespace splash::ops {
+
+struct LinearMatrix final {
+  uint32_t outputSize = 0;
+  uint32_t inputSize = 0;
+  auto operator<=>(const LinearMatrix &) const = default;
+};
+
+// Linear.hpp:77 in the reference; UpWithGate (its two-pass gate/up) has no use here: the MFMA tile
+// runs every gate/up pair in one pass.
+enum class LinearEpilogue : uint8_t { None, Residual, GateUp };
+// One tile: 16-column MFMA tiles, two per wave, 16/32/64 rows.
+enum class LinearTile : uint8_t { GgufMfma };
+inline constexpr uint32_t kMaximumDecodeTileRows = GGUF_MAXIMUM_ROWS;
+
+// The tile height that holds `rows` rows (the reference's stagedTileRows, Linear.hpp:118-120).
+[[nodiscard]] constexpr uint32_t mfmaTileRows(uint32_t rows) noexcept { return rows <= 16 ? 16 : rows <= 32 ? 32 : 64; }
+
+struct LinearWorkload final {
+  LinearMatrix matrix;
+  uint32_t rows = 0;
+  LinearEpilogue epilogue = LinearEpilogue::None;
+  auto operator<=>(const LinearWorkload &) const = default;
+};
+
+struct LinearConfig final {
+  LinearTile tile = LinearTile::GgufMfma;
+  // Cross-workgroup K partitions, a power of two up to kMaximumSplits.
+  uint32_t splits = 1;
+  static constexpr uint32_t kMaximumSplits = GGUF_MAXIMUM_SPLITS;
+  // Waves of a workgroup that share its column tiles and split its K partition: 1, 2 or 4.
+  uint32_t kWaves = 1;
+  [[nodiscard]] constexpr bool validSplits() const noexcept {
+    return splits && splits <= kMaximumSplits && !(splits & (splits - 1));
+  }
+  bool operator==(const LinearConfig &) const = default;
+};
+
+// Reused serially within one command stream; counters are zeroed at allocation and restored by
+// each completed split dispatch (Linear.hpp:183-196 in the reference).
+struct LinearScratch final {
+  hip::Buffer input;     // the activation table (values and sums, abi/Gguf.h)
+  hip::Buffer partials;
+  hip::Buffer counters;
+};
+struct LinearScratchSize final {
+  uint64_t input = 0, partials = 0, counters = 0;
+  LinearScratchSize &include(const LinearScratchSize &other) noexcept {
+    input = std::max(input, other.input);
+    partials = std::max(partials, other.partials);
+    counters = std::max(counters, other.counters);
+    return *this;
+  }
+};
+struct SwiGluProjections final {
+  const Projection *gate = nullptr;
+  const Projection *up = nullptr;
+  const Projection *down = nullptr;
+};
+// A block's buffers of its dense FFN: the intermediate rows and the linear scratch.
+struct FfnBuffers final {
+  hip::Buffer normalized, intermediate;
+  LinearScratch scratch;
+};
+
+enum class LinearInput : uint8_t {
+  Plain,    // bf16 [rows][K]
+  Table16,  // the activation table of abi/Gguf.h
+};
+// The scratch table currently holds `source` in `layout` (Linear.hpp:250-256 in the reference).
+struct PreparedInput final {
+  hip::Buffer source;
+  LinearInput layout = LinearInput::Plain;
+};
+
+class LinearPlan final {
+public:
+  [[nodiscard]] LinearWorkload workload() const noexcept { return workload_; }
+  [[nodiscard]] LinearConfig configuration() const noexcept { return config_; }
+  [[nodiscard]] FloatOutput destination() const noexcept { return destination_; }
+  [[nodiscard]] uint32_t storageRows() const noexcept { return mfmaTileRows(workload_.rows); }
+  [[nodiscard]] LinearInput input() const noexcept { return LinearInput::Table16; }
+  [[nodiscard]] LinearScratchSize scratchSize() const noexcept;
+
+private:
+  friend class Linear;
+  LinearPlan(LinearWorkload workload, LinearConfig config, FloatOutput destination = FloatOutput::BFloat16);
+  void requireConfiguration() const;
+  LinearWorkload workload_;
+  LinearConfig config_;
+  FloatOutput destination_;
+};
+
+struct LinearBuffers final {
+  hip::Buffer input;
+  hip::Buffer output;
+  hip::Buffer residual;
+  LinearScratch scratch{};
+  PreparedInput prepared{};
+};
+
+// What the plans read of the device (the reference's KernelCalibration, ops/KernelCalibration.hpp):
+// measured on MI355X, overridable for sweeps.
+struct KernelCalibration final {
+  uint32_t computeUnits = 256;
+  // Waves a projection should put in flight per compute unit before it stops partitioning K.
+  uint32_t wavesPerUnit = 8;
+  // Fewest super-blocks a wave's K range keeps.
+  uint32_t minimumBlocksPerWave = 2;
+};
+
+class Linear final {
+public:
+  explicit Linear(const sp_device_info &device) noexcept;
+  explicit Linear(KernelCalibration calibration) noexcept : calibration_(calibration) {}
+  [[nodiscard]] const KernelCalibration &calibration() const noexcept { return calibration_; }
+
+  [[nodiscard]] LinearPlan plan(LinearWorkload workload, FloatOutput destination = FloatOutput::BFloat16) const;
+  [[nodiscard]] LinearPlan plan(const Projection &projection, uint32_t rows,
+                                LinearEpilogue epilogue = LinearEpilogue::None) const;
+  [[nodiscard]] static LinearPlan plan(LinearWorkload workload, LinearConfig config, FloatOutput destination);
+  [[nodiscard]] uint32_t storageRows(uint32_t rows) const noexcept { return mfmaTileRows(rows); }
+  // The scratch of every plan of up to `rows` rows of a projection of `matrix`, every epilogue.
+  [[nodiscard]] LinearScratchSize scratchSize(LinearMatrix matrix, uint32_t rows) const;
+
+  // Writes the activation table of `rows` rows of `input` into scratch.input.
+  static void addPrepare(hip::CommandGraph &graph, const hip::Buffer &input, const LinearScratch &scratch, uint32_t width,
+                         uint32_t rows);
+  // Returns what the scratch table describes after the dispatch.
+  PreparedInput add(hip::CommandGraph &graph, LinearBuffers buffers, const Projection &projection,
+                    const LinearPlan &plan, const Projection *gate = nullptr) const;
+  void addProjection(hip::CommandGraph &graph, hip::Buffer input, const Projection &projection, hip::Buffer output,
+                     uint32_t rows, LinearScratch scratch) const;
+  void addResidualProjection(hip::CommandGraph &graph, hip::Buffer input, const Projection &projection,
+                             hip::Buffer residual, hip::Buffer output, uint32_t rows, LinearScratch scratch) const;
+  // output = residual + down(silu(gate x) * up x) of `rows` normalized rows.
+  void addSwiGlu(hip::CommandGraph &graph, const SwiGluProjections &ffn, const FfnBuffers &buffers, hip::Buffer residual,
+                 hip::Buffer output, uint32_t rows, PreparedInput normalized = {}) const;
+
+private:
+  KernelCalibration calibration_;
+};
+
+// Throws std::invalid_argument unless `buffer` holds `bytes` bytes ("<what> buffer is too small").
+void requireBytes(const hip::Buffer &buffer, uint64_t bytes, const char *what);
+
+} // namespace splash::ops

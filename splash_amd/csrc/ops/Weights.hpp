@@ -1,0 +1,74 @@
+// Quantized projection weights as the operators see them (the reference's runtime/ops/Weights.hpp:
+// QuantizedSegment :108-160, BlockWeights :162-164, Projection :170-225): a projection is a list of
+// column segments, each one tensor's weight image in HBM (abi/Gguf.h).
+#pragma once
+#include "abi/Gguf.h"
+#include "hip/Backend.hpp"
+
+#include <cstdint>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+namespace splash::ops {
+
+enum class FloatOutput : uint8_t { BFloat16, Float32 };
+
+struct QuantizedSegment final {
+  // The image of an [outputSize, inputSize] tensor of formatId (gguf_image_bytes).
+  [[nodiscard]] static QuantizedSegment ofImage(uint32_t formatId, uint32_t outputSize, uint32_t inputSize,
+                                              hip::Buffer image, uint32_t columnOffset = 0) {
+    if (!gguf_record_bytes(formatId)) throw std::invalid_argument("no weight image for format " + std::to_string(formatId));
+    QuantizedSegment s;
+    s.image = std::move(image);
+    s.outputSize = outputSize;
+    s.inputSize = inputSize;
+    s.columnOffset = columnOffset;
+    s.formatId = formatId;
+    return s;
+  }
+  hip::Buffer image;
+  uint32_t outputSize = 0;
+  uint32_t inputSize = 0;
+  uint32_t columnOffset = 0;
+  uint32_t formatId = GGUF_FMT_Q4K;
+  // The kernel name token of its format (the reference's kQuantFormats[].name).
+  [[nodiscard]] const char *name() const noexcept { return formatId == GGUF_FMT_Q6K ? "q6k" : "q4k"; }
+};
+
+struct BlockWeights final {
+  std::vector<QuantizedSegment> segments;
+};
+
+// A projection of outputSize x inputSize whose segments tile its leading output columns in order
+// (Weights.hpp:170-186 in the reference, same checks).
+class Projection final {
+public:
+  Projection() = default;
+  Projection(uint32_t output, uint32_t input, BlockWeights weights)
+      : outputSize(output), inputSize(input), weights_(std::move(weights)) {
+    if (weights_.segments.empty()) throw std::invalid_argument("block projection has no segments");
+    uint32_t covered = 0;
+    for (const QuantizedSegment &s : weights_.segments) {
+      if (s.inputSize != input || s.columnOffset != covered || !s.outputSize || s.outputSize > output - covered)
+        throw std::invalid_argument("block segments do not tile the projection");
+      covered += s.outputSize;
+    }
+  }
+  [[nodiscard]] const BlockWeights &blocks() const noexcept { return weights_; }
+  // Native bytes of its weights: what one pass over it streams from HBM.
+  [[nodiscard]] uint64_t weightBytes() const noexcept {
+    uint64_t bytes = 0;
+    for (const QuantizedSegment &s : weights_.segments) bytes += gguf_image_bytes(s.formatId, s.outputSize, s.inputSize);
+    return bytes;
+  }
+  uint32_t outputSize = 0;
+  uint32_t inputSize = 0;
+  // fp32 only for plain plans (the LM head's logits).
+  FloatOutput destination = FloatOutput::BFloat16;
+
+private:
+  BlockWeights weights_;
+};
+
+} // namespace splash::ops

@@ -1,0 +1,141 @@
+"""ctypes bindings of the CPU oracle (oracle/liboracle.so) and, where it was built, of the
+reference's own header-only CPU references (oracle/_ref/libref.so). Test infrastructure only."""
+import ctypes
+import os
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+FMT_Q4K, FMT_Q6K = 0, 4
+NO_TOKEN = 0xFFFFFFFF
+
+_path = os.path.join(ROOT, "oracle", "liboracle.so")
+if not os.path.exists(_path):
+    raise ImportError(f"{_path} is missing: run `make -C oracle` (or __graft_entry__.build())")
+lib = ctypes.CDLL(_path)
+_ref_path = os.path.join(ROOT, "oracle", "_ref", "libref.so")
+ref = ctypes.CDLL(_ref_path) if os.path.exists(_ref_path) else None
+
+u8p, u16p, u32p, f32p, f64p, i8p = (ctypes.POINTER(t) for t in (ctypes.c_uint8, ctypes.c_uint16, ctypes.c_uint32,
+                                                             ctypes.c_float, ctypes.c_double, ctypes.c_int8))
+c_u32, c_int, c_f = ctypes.c_uint32, ctypes.c_int, ctypes.c_float
+
+
+def _p(a, t):
+    return a.ctypes.data_as(t) if a is not None else None
+
+
+lib.orc_f2h.restype = ctypes.c_uint16
+lib.orc_f2h.argtypes = [c_f]
+lib.orc_h2f.restype = c_f
+lib.orc_h2f.argtypes = [ctypes.c_uint16]
+lib.orc_f2bf.restype = ctypes.c_uint16
+lib.orc_f2bf.argtypes = [c_f]
+lib.orc_bf2f.restype = c_f
+lib.orc_bf2f.argtypes = [ctypes.c_uint16]
+lib.orc_row_bytes.restype = ctypes.c_uint64
+lib.orc_row_bytes.argtypes = [c_u32, c_u32]
+lib.orc_silu.restype = c_f
+lib.orc_silu.argtypes = [c_f]
+lib.orc_epilogue_swiglu.restype = ctypes.c_uint16
+lib.orc_epilogue_swiglu.argtypes = [c_f, c_f]
+lib.orc_epilogue_residual.restype = ctypes.c_uint16
+lib.orc_epilogue_residual.argtypes = [c_f, ctypes.c_uint16]
+
+
+def bf16_to_f32(bits):
+    return (np.asarray(bits, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+def f32_to_bf16(values):
+    """Round to nearest even, as the kernels and the oracle do."""
+    u = np.ascontiguousarray(values, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    r = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+    nan = (u & 0x7FFFFFFF) > 0x7F800000
+    r[nan] = ((u[nan] >> 16) | 0x40).astype(np.uint16)
+    return r
+
+
+def row_bytes(fmt, K):
+    return lib.orc_row_bytes(fmt, K)
+
+
+def fixture(fmt, rows, K, seed, library=None):
+    out = np.empty(rows * row_bytes(fmt, K), dtype=np.uint8)
+    fn = (library or lib).orc_fixture if library is None else library.ref_fixture
+    assert fn(c_u32(fmt), c_u32(rows), c_u32(K), c_u32(seed), _p(out, u8p)) == 0
+    return out
+
+
+def make_native(fmt, rows, K, seed, library=None):
+    out = np.empty(rows * row_bytes(fmt, K), dtype=np.uint8)
+    fn = lib.orc_make_native if library is None else library.ref_make_native
+    assert fn(c_u32(fmt), c_u32(rows), c_u32(K), c_u32(seed), _p(out, u8p)) == 0
+    return out
+
+
+def dequant_rows(fmt, native, rows, K, library=None):
+    out = np.empty((rows, K), dtype=np.float32)
+    fn = lib.orc_dequant_rows if library is None else library.ref_dequant_rows
+    assert fn(c_u32(fmt), _p(native, u8p), c_u32(rows), c_u32(K), _p(out, f32p)) == 0
+    return out
+
+
+def quantize_rows(fmt, values):
+    values = np.ascontiguousarray(values, dtype=np.float32)
+    rows, K = values.shape
+    out = np.empty(rows * row_bytes(fmt, K), dtype=np.uint8)
+    assert lib.orc_quantize_rows(c_u32(fmt), _p(values, f32p), c_u32(rows), c_u32(K), _p(out, u8p)) == 0
+    return out
+
+
+def gemm(fmt, native, x_bf16, N, want=("exact", "bound", "chain"), threads=0):
+    """x_bf16: uint16 [M][K]. Returns dict of exact (f64), bound (f64), chain (f32), each [M][N]."""
+    x = np.ascontiguousarray(x_bf16, dtype=np.uint16)
+    M, K = x.shape
+    out = {}
+    exact = np.empty((M, N), dtype=np.float64) if "exact" in want else None
+    bound = np.empty((M, N), dtype=np.float64) if "bound" in want else None
+    chain = np.empty((M, N), dtype=np.float32) if "chain" in want else None
+    assert lib.orc_gemm(c_u32(fmt), _p(native, u8p), _p(x, u16p), c_u32(M), c_u32(K), c_u32(N), _p(exact, f64p),
+                        _p(bound, f64p), _p(chain, f32p), c_int(threads)) == 0
+    if exact is not None:
+        out["exact"] = exact
+    if bound is not None:
+        out["bound"] = bound
+    if chain is not None:
+        out["chain"] = chain
+    return out
+
+
+def rms_norm(x_bf16, w_bf16):
+    x = np.ascontiguousarray(x_bf16, dtype=np.uint16)
+    w = np.ascontiguousarray(w_bf16, dtype=np.uint16)
+    out = np.empty_like(x)
+    lib.orc_rms_norm(_p(x, u16p), _p(w, u16p), c_u32(x.shape[0]), c_u32(x.shape[1]), _p(out, u16p))
+    return out
+
+
+def embed(fmt, table, vocab, hidden, tokens):
+    tokens = np.ascontiguousarray(tokens, dtype=np.uint32)
+    out = np.empty((len(tokens), hidden), dtype=np.uint16)
+    assert lib.orc_embed(c_u32(fmt), _p(table, u8p), c_u32(vocab), c_u32(hidden), _p(tokens, u32p), c_u32(len(tokens)),
+                         _p(out, u16p)) == 0
+    return out
+
+
+def swiglu(gate_f32, up_f32):
+    g = np.ascontiguousarray(gate_f32, dtype=np.float32).ravel()
+    u = np.ascontiguousarray(up_f32, dtype=np.float32).ravel()
+    out = np.empty(g.size, dtype=np.uint16)
+    for i in range(g.size):
+        out[i] = lib.orc_epilogue_swiglu(float(g[i]), float(u[i]))
+    return out.reshape(np.shape(gate_f32))
+
+
+def projection_interval(exact, bound):
+    """[bf16(lo), bf16(hi)] of the reference's projection check (gguf_projection_test.mm:217-237)."""
+    lo = bf16_to_f32(f32_to_bf16((exact - bound).astype(np.float32)))
+    hi = bf16_to_f32(f32_to_bf16((exact + bound).astype(np.float32)))
+    # float32 rounding of lo/hi before bf16 can move them inward by an fp32 ulp: widen by it.
+    return np.nextafter(lo, -np.inf), np.nextafter(hi, np.inf)

@@ -1,0 +1,75 @@
+"""The C-ABI library loads without a GPU and exports every symbol include/*.h declares (CPU)."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+import splash_amd
+from splash_amd import ops
+from tests import oracle as orc
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    names = set()
+    for header in ("splash_hip.h", "splash_ops.h"):
+        text = open(os.path.join(ROOT, "include", header)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        names.update(re.findall(r"\b(spo?_[a-z0-9_]+)\s*\(", text))
+    names.discard("sp_completion")
+    return sorted(names)
+
+
+def test_library_exports_every_declared_symbol():
+    symbols = declared_symbols()
+    assert len(symbols) > 50
+    missing = [s for s in symbols if not hasattr(splash_amd.lib, s)]
+    assert not missing, missing
+
+
+def test_kernels_are_registered_by_name():
+    for name in ("gguf_prepare_table", "gguf_dequant_q4k", "gguf_dequant_q6k", "gguf_decode_q4k_m16_a",
+                 "gguf_decode_q6k_m16_a_f32", "gguf_decode_q4k_m32_g", "gguf_decode_q6k_m64_r"):
+        assert splash_amd.lib.sp_kernel_exists(name.encode()), name
+    assert not splash_amd.lib.sp_kernel_exists(b"no_such_kernel")
+
+
+@pytest.mark.parametrize("fmt", [ops.FMT_Q4K, ops.FMT_Q6K])
+def test_image_is_a_permutation_of_the_native_rows(fmt):
+    """decode(retile(native)) == decode(native) follows from unpack(pack(native)) == native."""
+    native = orc.fixture(fmt, 48, 768, 5)
+    image = ops.pack_gguf_image(fmt, native, 48, 768)
+    assert image.size == native.size == ops.gguf_image_bytes(fmt, 48, 768)
+    assert np.array_equal(ops.unpack_gguf_image(fmt, image, 48, 768), native)
+    if fmt == ops.FMT_Q4K:  # byte-for-byte re-ordering
+        assert np.array_equal(np.sort(image), np.sort(native))
+
+
+def test_pack_rejects_partial_tiles():
+    native = np.zeros(144 * 3 * 10, dtype=np.uint8)
+    with pytest.raises(ValueError):
+        ops.pack_gguf_image(ops.FMT_Q4K, native, 10, 768)
+    with pytest.raises(ValueError):
+        ops.pack_gguf_image(7, native, 16, 768)
+
+
+def test_linear_plans_without_a_device():
+    """Linear::plan partitions K to fill the device; LinearPlan rejects what no tile runs."""
+    linear = ops.Linear(calibration=(256, 8, 2))
+
+    class FakeProjection:
+        pass
+    # plans need only shapes: build a projection handle over no memory is not possible, so check
+    # the scratch sizing entry point, which plans every epilogue
+    table, partials, counters = linear.scratch_size(5120, 25600, 16)
+    assert table == ops.gguf_table_bytes(25600, 16)
+    assert partials > 0 and counters > 0   # a 5120-column projection of K 25600 splits across workgroups
+    table, partials, counters = linear.scratch_size(151936, 5120, 16)
+    assert partials == 0                    # the LM head fills the device without splitting
+    with pytest.raises(ValueError):
+        linear.scratch_size(5120, 25600, 65)
+    with pytest.raises(ValueError):
+        linear.scratch_size(5121, 25600, 16)

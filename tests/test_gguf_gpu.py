@@ -1,0 +1,202 @@
+"""GPU parity of the GGUF weight image and the dequant-GEMM against the oracle, through the C ABI."""
+import hashlib
+import json
+import os
+
+import numpy as np
+import pytest
+
+import splash_amd
+from splash_amd import ops
+from tests import oracle as orc
+
+pytestmark = pytest.mark.gpu
+HERE = os.path.dirname(os.path.abspath(__file__))
+GOLDENS = json.load(open(os.path.join(HERE, "golden", "gguf_dequantization.json")))
+
+
+def dequant_on_gpu(backend, fmt, native, rows, K):
+    image = backend.from_array(ops.pack_gguf_image(fmt, native, rows, K), label="image")
+    out = backend.allocate_buffer(rows * K * 4, label="values")
+    graph = splash_amd.CommandGraph()
+    ops.add_dequant(graph, fmt, image, out, rows, K)
+    backend.run(graph)
+    return out.download(np.float32).reshape(rows, K)
+
+
+@pytest.mark.parametrize("name,fmt", [("q4k", ops.FMT_Q4K), ("q6k", ops.FMT_Q6K)])
+def test_image_dequantization_matches_ggml_golden_hash(backend, name, fmt):
+    """gguf_reference_test.mm:23-30 + gguf_dequant_test.mm:44-58: the kernels' unpacking of the
+    re-tiled image gives GGML's fp32 values bit for bit."""
+    print(f"case dequant golden {name}", flush=True)
+    native = orc.fixture(fmt, 256, 1024, 7 + fmt)
+    values = dequant_on_gpu(backend, fmt, native, 256, 1024)
+    assert hashlib.sha256(values.tobytes()).hexdigest() == GOLDENS[name]
+
+
+@pytest.mark.parametrize("fmt", [ops.FMT_Q4K, ops.FMT_Q6K])
+def test_image_dequantization_of_quantized_weights(backend, fmt):
+    print(f"case dequant quantized fmt={fmt}", flush=True)
+    rng = np.random.default_rng(5)
+    w = (rng.standard_normal((64, 2048)) * 0.02).astype(np.float32)
+    native = orc.quantize_rows(fmt, w)
+    values = dequant_on_gpu(backend, fmt, native, 64, 2048)
+    assert values.tobytes() == orc.dequant_rows(fmt, native, 64, 2048).tobytes()
+
+
+def run_projection(backend, linear, fmt, native_segments, K, x_bits, epilogue=ops.EPILOGUE_NONE, float32=False,
+                   residual_bits=None, gate_native=None, splits=None, k_waves=None):
+    M = x_bits.shape[0]
+    proj = ops.Projection.from_native(backend, [(fmt, n, nat) for n, nat in native_segments], K, float32=float32)
+    gate = ops.Projection.from_native(backend, [(fmt, native_segments[0][0], gate_native)], K) if gate_native is not None else None
+    N = proj.output_size
+    plan = linear.plan(proj, M, epilogue, splits=splits, k_waves=k_waves)
+    scratch = linear.scratch_for(backend, [plan])
+    x = backend.from_array(x_bits, label="x")
+    out = backend.allocate_buffer(M * N * (4 if float32 else 2), label="out")
+    res = backend.from_array(residual_bits, label="residual") if residual_bits is not None else None
+    graph = splash_amd.CommandGraph()
+    linear.add(graph, proj, plan, x, out, scratch, residual=res, gate=gate)
+    backend.run(graph)
+    got = out.download(np.float32 if float32 else np.uint16).reshape(M, N)
+    return got, plan, scratch
+
+
+def check_interval(got_f32, oracle_result):
+    lo, hi = orc.projection_interval(oracle_result["exact"], oracle_result["bound"])
+    bad = ~((got_f32 >= lo) & (got_f32 <= hi))
+    assert not bad.any(), (int(bad.sum()), got_f32[bad][:4], lo[bad][:4], hi[bad][:4])
+
+
+@pytest.mark.parametrize("fmt", [ops.FMT_Q4K, ops.FMT_Q6K])
+@pytest.mark.parametrize("M", [1, 4, 8, 16, 32, 64])
+def test_projection_lies_in_the_reference_interval(backend, fmt, M):
+    """gguf_projection_test.mm:217-237: the bf16 result lies in [bf16(lo), bf16(hi)] of the fp64 dot
+    +- projectionBound; fp32 logits lie within the bound itself."""
+    print(f"case projection fmt={fmt} M={M}", flush=True)
+    rng = np.random.default_rng(100 + M)
+    N, K = 192, 2048
+    native = orc.make_native(fmt, N, K, 40 + M)
+    x = orc.f32_to_bf16(rng.standard_normal((M, K)).astype(np.float32))
+    linear = ops.Linear(backend)
+    want = orc.gemm(fmt, native, x, N)
+    got, plan, _ = run_projection(backend, linear, fmt, [(N, native)], K, x)
+    check_interval(orc.bf16_to_f32(got), want)
+    got32, _, _ = run_projection(backend, linear, fmt, [(N, native)], K, x, float32=True)
+    assert np.all(np.abs(got32.astype(np.float64) - want["exact"]) <= want["bound"])
+
+
+@pytest.mark.parametrize("fmt", [ops.FMT_Q4K, ops.FMT_Q6K])
+def test_rows_do_not_depend_on_the_block_or_the_partition(backend, fmt):
+    """Tested invariants of the reference (gguf_projection_test.mm): a row's result is bitwise the same
+    alone or in a taller block, and splits sum in split order so a re-run is bit-identical."""
+    print(f"case projection invariants fmt={fmt}", flush=True)
+    rng = np.random.default_rng(7)
+    N, K = 128, 4096
+    native = orc.make_native(fmt, N, K, 3)
+    x = orc.f32_to_bf16(rng.standard_normal((32, K)).astype(np.float32))
+    linear = ops.Linear(backend)
+    full, _, _ = run_projection(backend, linear, fmt, [(N, native)], K, x, float32=True, splits=1, k_waves=1)
+    for rows in (1, 5, 16):
+        part, _, _ = run_projection(backend, linear, fmt, [(N, native)], K, x[:rows], float32=True, splits=1, k_waves=1)
+        assert part.tobytes() == full[:rows].tobytes()
+    want = orc.gemm(fmt, native, x, N)
+    for splits, k_waves in ((1, 4), (2, 2), (4, 4), (16, 1)):
+        a, _, _ = run_projection(backend, linear, fmt, [(N, native)], K, x, float32=True, splits=splits, k_waves=k_waves)
+        b, _, _ = run_projection(backend, linear, fmt, [(N, native)], K, x, float32=True, splits=splits, k_waves=k_waves)
+        assert a.tobytes() == b.tobytes()
+        assert np.all(np.abs(a.astype(np.float64) - want["exact"]) <= want["bound"])
+
+
+def test_fused_segments_equal_each_alone(backend):
+    """A fused q|k|v dispatch gives each segment the bits it gets alone (LinearGguf.cpp:78-96)."""
+    print("case fused segments", flush=True)
+    rng = np.random.default_rng(9)
+    K, sizes = 1024, (160, 32, 48)
+    natives = [orc.make_native(ops.FMT_Q4K, n, K, 60 + i) for i, n in enumerate(sizes)]
+    x = orc.f32_to_bf16(rng.standard_normal((16, K)).astype(np.float32))
+    linear = ops.Linear(backend)
+    fused, _, _ = run_projection(backend, linear, ops.FMT_Q4K, list(zip(sizes, natives)), K, x, splits=1, k_waves=2)
+    at = 0
+    for n, native in zip(sizes, natives):
+        alone, _, _ = run_projection(backend, linear, ops.FMT_Q4K, [(n, native)], K, x, splits=1, k_waves=2)
+        assert np.array_equal(fused[:, at:at + n], alone)
+        at += n
+
+
+@pytest.mark.parametrize("fmt", [ops.FMT_Q4K, ops.FMT_Q6K])
+def test_residual_and_gate_up_epilogues(backend, fmt):
+    """gguf_tile.h:10-16, gguf_linear.metal:34-71: bf16(v + res) and bf16(bf16(up) silu(bf16(gate)));
+    the one-pass pair equals the two projections' fp32 sums put through the oracle's epilogue."""
+    print(f"case epilogues fmt={fmt}", flush=True)
+    rng = np.random.default_rng(13)
+    N, K, M = 96, 1024, 16
+    up_native = orc.make_native(fmt, N, K, 70)
+    gate_native = orc.make_native(fmt, N, K, 71)
+    x = orc.f32_to_bf16(rng.standard_normal((M, K)).astype(np.float32))
+    res = orc.f32_to_bf16(rng.standard_normal((M, N)).astype(np.float32))
+    linear = ops.Linear(backend)
+    kw = dict(splits=2, k_waves=2)
+    up32, _, _ = run_projection(backend, linear, fmt, [(N, up_native)], K, x, float32=True, **kw)
+    gate32, _, _ = run_projection(backend, linear, fmt, [(N, gate_native)], K, x, float32=True, **kw)
+    got, _, _ = run_projection(backend, linear, fmt, [(N, up_native)], K, x, epilogue=ops.EPILOGUE_RESIDUAL,
+                               residual_bits=res, **kw)
+    want = orc.f32_to_bf16(up32 + orc.bf16_to_f32(res))
+    assert np.array_equal(got, want)
+    pair, _, _ = run_projection(backend, linear, fmt, [(N, up_native)], K, x, epilogue=ops.EPILOGUE_GATE_UP,
+                                gate_native=gate_native, **kw)
+    want = orc.swiglu(gate32, up32)
+    # exp2 differs in its last bits between the CPU and the GPU: allow one bf16 step on a few values
+    diff = np.abs(pair.astype(np.int32) - want.astype(np.int32))
+    assert diff.max() <= 1 and (diff > 0).mean() < 0.02, (diff.max(), (diff > 0).mean())
+
+
+def test_linear_rejects_bad_buffers_before_adding_anything(backend):
+    """Operators throw std::invalid_argument before any dispatch is added (LinearGguf.cpp:126-163)."""
+    native = orc.make_native(ops.FMT_Q4K, 32, 512, 1)
+    proj = ops.Projection.from_native(backend, [(ops.FMT_Q4K, 32, native)], 512)
+    linear = ops.Linear(backend)
+    plan = linear.plan(proj, 16)
+    scratch = linear.scratch_for(backend, [plan])
+    x = backend.allocate_buffer(16 * 512 * 2)
+    small = backend.allocate_buffer(16)
+    graph = splash_amd.CommandGraph()
+    with pytest.raises(ValueError, match="too small"):
+        linear.add(graph, proj, plan, x, small, scratch)
+    with pytest.raises(ValueError, match="too small"):
+        linear.add(graph, proj, plan, small, x, scratch)
+    with pytest.raises(ValueError):
+        linear.plan(proj, 65)
+    with pytest.raises(ValueError):
+        linear.plan(proj, 16, splits=3)
+    assert len(graph) == 0
+
+
+def test_backend_one_command_in_flight_and_unknown_kernel(backend):
+    """MetalBackend.hpp:474-476: a second command is refused until the first ticket is consumed."""
+    import ctypes
+    a = backend.allocate_buffer(4096)
+    graph = splash_amd.CommandGraph()
+
+    class P(ctypes.Structure):
+        _fields_ = [("x", ctypes.c_uint32)]
+    graph.add("no_such_kernel", [a], P(1), (1, 1, 1))
+    with pytest.raises(ValueError, match="no kernel"):
+        backend.submit_command_async(graph)
+    native = orc.make_native(ops.FMT_Q4K, 16, 256, 1)
+    image = backend.from_array(ops.pack_gguf_image(ops.FMT_Q4K, native, 16, 256))
+    out = backend.allocate_buffer(16 * 256 * 4)
+    g2 = splash_amd.CommandGraph()
+    ops.add_dequant(g2, ops.FMT_Q4K, image, out, 16, 256)
+    t1 = backend.submit_command_async(g2)
+    with pytest.raises(splash_amd.SplashError) as e:
+        backend.submit_command_async(g2)
+    assert e.value.status == 4  # SP_BUSY
+    gpu, wall = t1.wait()
+    assert gpu >= 0 and wall > 0 and backend.healthy() and not backend.command_in_flight()
+    # a recorded command replays to the same bytes
+    first = out.download(np.float32).copy()
+    out.fill(0)
+    rec = backend.record(g2)
+    rec.submit().wait()
+    assert np.array_equal(out.download(np.float32), first)
