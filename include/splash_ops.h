@@ -83,6 +83,42 @@ sp_status spo_linear_add_swiglu(const spo_linear *linear, spo_graph *graph, cons
 sp_status spo_linear_scratch_size(const spo_linear *linear, uint32_t output_size, uint32_t input_size, uint32_t rows,
                                   uint64_t *table, uint64_t *partials, uint64_t *counters);
 
+/* ---- PagedAttention (runtime/ops/PagedAttention.hpp:259-366) ---- */
+typedef struct spo_attention_plan spo_attention_plan; /* ops::AttentionPlan (PagedAttention.hpp:179-234) */
+typedef struct spo_attention_geometry {
+  uint32_t q_heads, kv_heads, head_dim;
+  uint32_t rotary_pairs; /* RoPE pairs (i, i + pairs) */
+  uint32_t normalize;    /* RMS-norm q and k heads */
+} spo_attention_geometry;
+typedef struct spo_attention_rows { /* one sequence: ops::AttentionRows / AttentionHistory */
+  uint32_t first_row, rows, committed, table_first;
+} spo_attention_rows;
+/* kv::Layout::bytesPerLayerPage (runtime/ops/PagedKv.hpp:155-260) at 256-token pages, fp16 scales. */
+uint64_t spo_kv_page_bytes(uint32_t kv_heads, uint32_t head_dim);
+/* Element offsets of the page layout, for hosts that fill or read pages (abi/KvExtent.h:23-111). */
+uint64_t spo_kv_key_index(uint32_t head, uint32_t token, uint32_t dim, uint32_t head_dim);
+uint64_t spo_kv_value_index(uint32_t head, uint32_t token, uint32_t dim, uint32_t head_dim);
+/* PagedAttention::plan (PagedAttention.cpp:351-389). */
+sp_status spo_attention_plan_create(const spo_attention_geometry *geometry, const spo_attention_rows *sequences,
+                                    uint32_t count, spo_attention_plan **out);
+void spo_attention_plan_destroy(spo_attention_plan *plan);
+uint32_t spo_attention_plan_splits(const spo_attention_plan *plan);
+/* PagedAttention::workspace: bytes of the staged queries, their sums, the split partials, their sums. */
+sp_status spo_attention_workspace(const spo_attention_plan *plan, uint64_t sizes[4]);
+/* PagedAttention::addProjection (PagedAttention.cpp:441-464). */
+sp_status spo_attention_add_projection(spo_graph *graph, const spo_attention_plan *plan, sp_buffer *qkv,
+                                       sp_buffer *query_norm, sp_buffer *key_norm, sp_buffer *rope_cos,
+                                       sp_buffer *rope_sin, sp_buffer *queries, sp_buffer *query_sums,
+                                       sp_buffer *page_table, sp_buffer *pool, uint64_t page_bytes);
+/* PagedAttention::addAttention (PagedAttention.cpp:466-607): split, then ordered reduce. */
+sp_status spo_attention_add_attention(spo_graph *graph, const spo_attention_plan *plan, sp_buffer *queries,
+                                      sp_buffer *query_sums, sp_buffer *partials, sp_buffer *partial_sums,
+                                      sp_buffer *tree_rows, sp_buffer *page_table, sp_buffer *pool, uint64_t page_bytes,
+                                      sp_buffer *output);
+/* PagedAttention::addPathCommit (PagedAttention.cpp:647-667). */
+sp_status spo_attention_add_path_commit(spo_graph *graph, const spo_attention_plan *plan, sp_buffer *retained,
+                                        sp_buffer *page_table, sp_buffer *pool, uint64_t page_bytes);
+
 #ifdef __cplusplus
 }
 #endif

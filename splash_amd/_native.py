@@ -74,6 +74,14 @@ class LinearPlan(ctypes.Structure):
                 ("float32", c_u32), ("scratch_input", c_u64), ("scratch_partials", c_u64), ("scratch_counters", c_u64)]
 
 
+class AttentionGeometry(ctypes.Structure):
+    _fields_ = [("q_heads", c_u32), ("kv_heads", c_u32), ("head_dim", c_u32), ("rotary_pairs", c_u32), ("normalize", c_u32)]
+
+
+class AttentionRows(ctypes.Structure):
+    _fields_ = [("first_row", c_u32), ("rows", c_u32), ("committed", c_u32), ("table_first", c_u32)]
+
+
 def _sig(name, restype, *argtypes):
     fn = getattr(lib, name)
     fn.restype = restype
@@ -140,3 +148,14 @@ _sig("spo_linear_plan_with", c_int, c_p, P(LinearPlan))
 _sig("spo_linear_add", c_int, c_p, c_p, c_p, c_p, P(LinearPlan), c_p, c_p, c_p, c_p, c_p, c_p, c_int)
 _sig("spo_linear_add_swiglu", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_u32, c_p, c_p, c_p)
 _sig("spo_linear_scratch_size", c_int, c_p, c_u32, c_u32, c_u32, P(c_u64), P(c_u64), P(c_u64))
+
+_sig("spo_kv_page_bytes", c_u64, c_u32, c_u32)
+_sig("spo_kv_key_index", c_u64, c_u32, c_u32, c_u32, c_u32)
+_sig("spo_kv_value_index", c_u64, c_u32, c_u32, c_u32, c_u32)
+_sig("spo_attention_plan_create", c_int, P(AttentionGeometry), P(AttentionRows), c_u32, P(c_p))
+_sig("spo_attention_plan_destroy", None, c_p)
+_sig("spo_attention_plan_splits", c_u32, c_p)
+_sig("spo_attention_workspace", c_int, c_p, P(c_u64))
+_sig("spo_attention_add_projection", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_u64)
+_sig("spo_attention_add_attention", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_u64, c_p)
+_sig("spo_attention_add_path_commit", c_int, c_p, c_p, c_p, c_p, c_p, c_u64)

@@ -113,7 +113,7 @@ struct GgufDecodeParams {
   uint32_t input_size;  // K
   uint32_t rows;        // live rows
   uint32_t splits;      // K partitions across workgroups (grid.y); 1 = no cross-workgroup reduction
-  uint32_t k_waves;     // waves of a workgroup that share its tiles and split its K partition: 1, 2 or 4
+  uint32_t k_waves;     // waves of a workgroup that split its K partition between them: 1
   uint32_t out_stride;  // columns of a destination row
   uint32_t cols[3];     // columns per segment (multiples of 16); 0 past the last
   uint32_t offset[3];   // first destination column per segment

@@ -2,6 +2,7 @@
 #include "splash_ops.h"
 #include "backend/Internal.hpp"
 #include "capi/Guard.hpp"
+#include "capi/Handles.hpp"
 #include "ops/GgufImage.hpp"
 #include "ops/Linear.hpp"
 
@@ -9,7 +10,7 @@
 
 using namespace splash;
 
-struct spo_graph { hip::CommandGraph graph; };
+
 struct spo_projection { ops::Projection projection; };
 struct spo_linear { ops::Linear linear; };
 

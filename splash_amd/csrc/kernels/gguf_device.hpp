@@ -27,14 +27,21 @@ __device__ __forceinline__ float byte_of(uint32_t word, uint32_t index) { return
 
 // Register j (0..3) of a group's bf16 operands 128 + code, from the two words that hold the
 // lane's eight codes of that group in their low (high = false) or high nibbles.
+// (a & mask) | base in one instruction: the mask rides the scalar bus, the base a register (on
+// this ISA a three-operand vector instruction takes no literal, so the compiler would emit two).
+__device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t mask, uint32_t base) {
+  uint32_t r;
+  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "s"(mask), "v"(base));
+  return r;
+}
 template <bool High> __device__ __forceinline__ uint4 q4_operands(uint32_t wa, uint32_t wb) {
   constexpr uint32_t kMask = 0x000F000Fu, kBase = 0x43004300u;  // bf16 0x4300 = 128, ulp 1
   constexpr uint32_t s = High ? 4u : 0u;
   uint4 r;
-  r.x = ((wa >> s) & kMask) | kBase;
-  r.y = ((wa >> (s + 8u)) & kMask) | kBase;
-  r.z = ((wb >> s) & kMask) | kBase;
-  r.w = ((wb >> (s + 8u)) & kMask) | kBase;
+  r.x = and_or(s ? wa >> s : wa, kMask, kBase);
+  r.y = and_or(wa >> (s + 8u), kMask, kBase);
+  r.z = and_or(s ? wb >> s : wb, kMask, kBase);
+  r.w = and_or(wb >> (s + 8u), kMask, kBase);
   return r;
 }
 // The same for Q6_K: the low nibbles as Q4_K's, then the 2-bit high fields of pair v0..v0+3 of
@@ -42,13 +49,13 @@ template <bool High> __device__ __forceinline__ uint4 q4_operands(uint32_t wa, u
 template <bool High, uint32_t V0> __device__ __forceinline__ uint4 q6_operands(uint32_t wa, uint32_t wb, uint32_t hw) {
   constexpr uint32_t kHigh = 0x00300030u;
   uint4 r = q4_operands<High>(wa, wb);
-  auto field = [&](uint32_t v) -> uint32_t {
-    return (2u * v >= 4u ? hw >> (2u * v - 4u) : hw << (4u - 2u * v)) & kHigh;
+  auto with = [&](uint32_t v, uint32_t low) -> uint32_t {
+    return and_or(2u * v > 4u ? hw >> (2u * v - 4u) : 2u * v < 4u ? hw << (4u - 2u * v) : hw, kHigh, low);
   };
-  r.x |= field(V0);
-  r.y |= field(V0 + 1);
-  r.z |= field(V0 + 2);
-  r.w |= field(V0 + 3);
+  r.x = with(V0, r.x);
+  r.y = with(V0 + 1, r.y);
+  r.z = with(V0 + 2, r.z);
+  r.w = with(V0 + 3, r.w);
   return r;
 }
 

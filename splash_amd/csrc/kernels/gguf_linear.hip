@@ -72,26 +72,48 @@ SP_REGISTER_KERNEL("gguf_prepare_table", &gguf_prepare_table);
 // ---------------------------------------------------------------------------------------------
 // Records in registers.
 // ---------------------------------------------------------------------------------------------
+// A wave's cursors into one column tile's record stream: its lane's 16 bytes of each 1024-byte
+// part, and its column's scale fields. They advance one record per super-block.
+template <uint32_t FMT> struct Cursor {
+  const uint4 *mine = nullptr;
+  const uint4 *column = nullptr;
+  const uint16_t *d = nullptr;  // Q6_K only
+  __device__ __forceinline__ void open(const uint8_t *record, uint32_t lane) {
+    const uint4 *p = reinterpret_cast<const uint4 *>(record);
+    mine = p + lane;
+    if constexpr (FMT == GGUF_FMT_Q4K) {
+      column = p + 128 + (lane & 15u);
+    } else {
+      column = p + 192 + (lane & 15u);
+      d = reinterpret_cast<const uint16_t *>(record + GGUF_Q6K_D) + (lane & 15u);
+    }
+  }
+  __device__ __forceinline__ void advance() {
+    constexpr uint32_t kVectors = (FMT == GGUF_FMT_Q4K ? GGUF_Q4K_RECORD : GGUF_Q6K_RECORD) / 16u;
+    mine += kVectors;
+    column += kVectors;
+    if constexpr (FMT == GGUF_FMT_Q6K) d += kVectors * 8u;
+  }
+};
+
 template <uint32_t FMT> struct Record;
 template <> struct Record<GGUF_FMT_Q4K> {
   uint4 n0, n1, meta;
-  __device__ __forceinline__ void load(const uint8_t *rec, uint32_t lane) {
-    const uint4 *p = reinterpret_cast<const uint4 *>(rec);
-    n0 = load_stream(p + lane);
-    n1 = load_stream(p + 64 + lane);
-    meta = load_stream(p + 128 + (lane & 15u));
+  __device__ __forceinline__ void load(const Cursor<GGUF_FMT_Q4K> &at) {
+    n0 = load_stream(at.mine);
+    n1 = load_stream(at.mine + 64);
+    meta = load_stream(at.column);
   }
 };
 template <> struct Record<GGUF_FMT_Q6K> {
   uint4 n0, n1, high, scales;
   uint32_t d;
-  __device__ __forceinline__ void load(const uint8_t *rec, uint32_t lane) {
-    const uint4 *p = reinterpret_cast<const uint4 *>(rec);
-    n0 = load_stream(p + lane);
-    n1 = load_stream(p + 64 + lane);
-    high = load_stream(p + 128 + lane);
-    scales = load_stream(p + 192 + (lane & 15u));
-    d = __builtin_nontemporal_load(reinterpret_cast<const uint16_t *>(rec + GGUF_Q6K_D) + (lane & 15u));
+  __device__ __forceinline__ void load(const Cursor<GGUF_FMT_Q6K> &at) {
+    n0 = load_stream(at.mine);
+    n1 = load_stream(at.mine + 64);
+    high = load_stream(at.mine + 128);
+    scales = load_stream(at.column);
+    d = __builtin_nontemporal_load(at.d);
   }
 };
 
@@ -130,7 +152,9 @@ template <uint32_t FMT> __global__ __launch_bounds__(64) void gguf_dequant(const
   const uint32_t b = blockIdx.x, tile = blockIdx.y, lane = threadIdx.x, c = lane & 15u, kq = lane >> 4;
   const uint32_t blocks = p.input_size / GGUF_BLOCK;
   Record<FMT> rec;
-  rec.load(image + (size_t(tile) * blocks + b) * gguf_record_bytes(FMT), lane);
+  Cursor<FMT> cursor;
+  cursor.open(image + (size_t(tile) * blocks + b) * gguf_record_bytes(FMT), lane);
+  rec.load(cursor);
   uint4 ops[8];
   record_operands(rec, ops);
   float *row = out + size_t(16u * tile + c) * p.input_size + size_t(b) * GGUF_BLOCK;
@@ -193,14 +217,19 @@ __device__ __forceinline__ TileRef find_tile(uint32_t index, const uint8_t *cons
   return ref;
 }
 
+// One record's contribution to a wave's sums. `a` and `sums` are the workgroup's staged
+// activations of the record's super-block in LDS: a[t][g][lane] the MFMA operand of row tile t,
+// group g; sums[t][j][lane] the row sums of the j-th K = 4 MFMA.
 template <uint32_t FMT, int RT>
-__device__ __forceinline__ void accumulate_record(const Record<FMT> &rec, const uint4 (&a)[RT][8], const float (&sums)[RT][4],
-                                                  f32x4 (&acc)[RT], uint32_t kq) {
+__device__ __forceinline__ void accumulate_record(const Record<FMT> &rec, const uint4 (*a)[8][64], const float (*sums)[4][64],
+                                                  f32x4 (&acc)[RT], uint32_t lane, uint32_t kq, float keep) {
   uint4 ops[8];
   record_operands(rec, ops);
   const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
   if constexpr (FMT == GGUF_FMT_Q4K) {
-    const Q4KScales sc = q4k_scales(rec.meta);
+    Q4KScales sc = q4k_scales(rec.meta);
+    sc.d *= keep;
+    sc.dmin *= keep;
     float s[8];
 #pragma unroll
     for (uint32_t g = 0; g < 8; ++g) s[g] = sc.d * byte_of(g < 4 ? sc.sc_lo : sc.sc_hi, g & 3u);
@@ -210,40 +239,41 @@ __device__ __forceinline__ void accumulate_record(const Record<FMT> &rec, const 
     const float c_hi = __fmaf_rn(-128.f, s_hi, -(sc.dmin * byte_of(sc.mn_hi, kq)));
 #pragma unroll
     for (int t = 0; t < RT; ++t) {
-      acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(sums[t][0], c_lo, acc[t], 0, 0, 0);
-      acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(sums[t][1], c_hi, acc[t], 0, 0, 0);
+      acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(sums[t][0][lane], c_lo, acc[t], 0, 0, 0);
+      acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(sums[t][1][lane], c_hi, acc[t], 0, 0, 0);
     }
 #pragma unroll
     for (uint32_t g = 0; g < 8; ++g) {
       const bf16x8 b = as_bf16x8(ops[g]);
 #pragma unroll
       for (int t = 0; t < RT; ++t) {
-        const f32x4 dot = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a[t][g]), b, zero, 0, 0, 0);
+        const f32x4 dot = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a[t][g][lane]), b, zero, 0, 0, 0);
 #pragma unroll
         for (int i = 0; i < 4; ++i) acc[t][i] = __fmaf_rn(dot[i], s[g], acc[t][i]);
       }
     }
   } else {
-    const float d = half_bits_to_float(rec.d);
+    const float d = half_bits_to_float(rec.d) * keep;
     // Constant terms of 16-input blocks 4 j + kq: -160 d sc (operand 128 + q, value q - 32).
 #pragma unroll
     for (uint32_t j = 0; j < 4; ++j) {
       const uint32_t word = j == 0 ? rec.scales.x : j == 1 ? rec.scales.y : j == 2 ? rec.scales.z : rec.scales.w;
       const float coef = -160.f * (d * float(int(int8_t((word >> (8u * kq)) & 0xFFu))));
 #pragma unroll
-      for (int t = 0; t < RT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(sums[t][j], coef, acc[t], 0, 0, 0);
+      for (int t = 0; t < RT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(sums[t][j][lane], coef, acc[t], 0, 0, 0);
     }
 #pragma unroll
     for (uint32_t g = 0; g < 8; ++g) {
 #pragma unroll
-      for (uint32_t h = 0; h < 2; ++h) {
-        const float s = d * q6_scale(rec.scales, 2u * g + h);
-        const uint2 bw = h ? make_uint2(ops[g].z, ops[g].w) : make_uint2(ops[g].x, ops[g].y);
-        const s16x4 b = __builtin_bit_cast(s16x4, bw);
+      for (int t = 0; t < RT; ++t) {
+        const uint4 av = a[t][g][lane];
 #pragma unroll
-        for (int t = 0; t < RT; ++t) {
-          const uint2 aw = h ? make_uint2(a[t][g].z, a[t][g].w) : make_uint2(a[t][g].x, a[t][g].y);
-          const f32x4 dot = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4, aw), b, zero, 0, 0, 0);
+        for (uint32_t h = 0; h < 2; ++h) {
+          const float s = d * q6_scale(rec.scales, 2u * g + h);
+          const uint2 bw = h ? make_uint2(ops[g].z, ops[g].w) : make_uint2(ops[g].x, ops[g].y);
+          const uint2 aw = h ? make_uint2(av.z, av.w) : make_uint2(av.x, av.y);
+          const f32x4 dot = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4, aw),
+                                                                      __builtin_bit_cast(s16x4, bw), zero, 0, 0, 0);
 #pragma unroll
           for (int i = 0; i < 4; ++i) acc[t][i] = __fmaf_rn(dot[i], s, acc[t][i]);
         }
@@ -260,34 +290,44 @@ __global__ __launch_bounds__(256) void gguf_decode(const uint8_t *__restrict__ s
                                                    GgufDecodeParams p) {
   constexpr uint32_t kRecord = FMT == GGUF_FMT_Q4K ? GGUF_Q4K_RECORD : GGUF_Q6K_RECORD;
   constexpr uint32_t kSumsPerBlock = FMT == GGUF_FMT_Q4K ? 2 : 4;  // K = 4 MFMAs of row sums per super-block
-  __shared__ float reduce[3][kUnitTiles][RT][4][64];
+  // The workgroup's four waves walk one K range in step and own different column tiles; the
+  // range's activations pass through LDS one super-block at a time (two buffers, one barrier per
+  // super-block), each wave fetching a quarter of them, so a wave's vector-memory queue holds
+  // almost only weights and the MFMA operands arrive on the LDS counter instead.
+  __shared__ uint4 ldsA[2][RT][8][64];
+  __shared__ float ldsSums[2][RT][4][64];
   __shared__ uint32_t arrived;
 
   const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6, c = lane & 15u, kq = lane >> 4;
-  const uint32_t kw = p.k_waves, ks = wave % kw, across = 4u / kw;
-  const uint32_t unit = blockIdx.x * across + wave / kw;
+  const uint32_t unit = blockIdx.x * 4u + wave;
   const uint32_t split = blockIdx.y;
   const uint32_t blocks = p.input_size / GGUF_BLOCK, G = p.input_size / 32u;
   const uint32_t tiles = gguf_row_tiles(p.rows);
   const uint8_t *const seg[3] = {seg0, seg1, seg2};
+  const uint32_t ks = 0;
 
+  // Every wave streams real records, so the main loop has no divergent control flow: a wave past
+  // the dispatch's last unit, or a tile past its last tile, re-reads the first tile and stores nothing.
   TileRef tile[kUnitTiles];
-  if (unit < p.units) {
+  bool live[kUnitTiles];
+  {
+    const uint32_t mine = unit < p.units ? unit : 0u;
     if constexpr (EP == GGUF_EPILOGUE_GATE_UP) {
-      tile[0] = {seg0 + size_t(unit) * blocks * kRecord, p.offset[0] + unit * GGUF_TILE_COLUMNS};
-      tile[1] = {seg1 + size_t(unit) * blocks * kRecord, p.offset[0] + unit * GGUF_TILE_COLUMNS};
+      tile[0] = {seg0 + size_t(mine) * blocks * kRecord, p.offset[0] + mine * GGUF_TILE_COLUMNS};
+      tile[1] = {seg1 + size_t(mine) * blocks * kRecord, p.offset[0] + mine * GGUF_TILE_COLUMNS};
+      live[0] = live[1] = unit < p.units;
     } else {
 #pragma unroll
-      for (int i = 0; i < kUnitTiles; ++i) tile[i] = find_tile(unit * kUnitTiles + i, seg, p, kRecord);
+      for (int i = 0; i < kUnitTiles; ++i) {
+        tile[i] = find_tile(mine * kUnitTiles + i, seg, p, kRecord);
+        live[i] = unit < p.units && tile[i].image != nullptr;
+        if (!tile[i].image) tile[i] = {seg0, p.offset[0]};
+      }
     }
-  } else {
-#pragma unroll
-    for (int i = 0; i < kUnitTiles; ++i) tile[i] = {nullptr, 0};
   }
 
-  // This wave's super-blocks: part ks of its workgroup's part `split`.
-  const uint32_t parts = p.splits * kw, part = split * kw + ks;
-  const uint32_t b0 = uint32_t(uint64_t(blocks) * part / parts), b1 = uint32_t(uint64_t(blocks) * (part + 1) / parts);
+  // The workgroup's super-blocks: part `split` of K.
+  const uint32_t b0 = uint32_t(uint64_t(blocks) * split / p.splits), b1 = uint32_t(uint64_t(blocks) * (split + 1) / p.splits);
 
   f32x4 acc[kUnitTiles][RT];
 #pragma unroll
@@ -300,58 +340,84 @@ __global__ __launch_bounds__(256) void gguf_decode(const uint8_t *__restrict__ s
       table + (FMT == GGUF_FMT_Q4K ? gguf_table_sums32_offset(p.input_size, tiles) : gguf_table_sums16_offset(p.input_size, tiles)));
   const uint32_t sumGroups = FMT == GGUF_FMT_Q4K ? G : 2u * G;  // row-sum entries per row tile
 
-  if (tile[0].image && b0 < b1) {
-    Record<FMT> cur[kUnitTiles], next[kUnitTiles];
+  {
+    // A software pipeline of kStages super-blocks in registers: the loads of super-block
+    // b + kStages - 1 are issued before the MFMAs of super-block b, so kStages - 1 super-blocks of
+    // weights per wave stay in flight (loads return in issue order, so waiting for b's never
+    // waits for a later one's). The loop body is one straight block: the range is walked in
+    // rounds of kStages, loads past its end re-read its last super-block (the cursors stop
+    // there) and the super-blocks past its end are multiplied by a zero scale.
+    constexpr int kStages = RT > 1 ? 2 : FMT == GGUF_FMT_Q4K ? 4 : 3;
+    constexpr uint32_t kSumFloats = RT * kSumsPerBlock * 64u;  // staged row sums per super-block
+    constexpr int kSumShare = (kSumFloats + 255u) / 256u;
+    struct Stage {
+      Record<FMT> rec[kUnitTiles];
+      uint4 a[2 * RT];       // this thread's share of the super-block's RT * 8 * 64 operand vectors
+      float sum[kSumShare];  // and of its row sums
+    };
+    Stage stage[kStages];
+    Cursor<FMT> cursor[kUnitTiles];
 #pragma unroll
-    for (int i = 0; i < kUnitTiles; ++i)
-      if (tile[i].image) cur[i].load(tile[i].image + size_t(b0) * kRecord, lane);
-    for (uint32_t b = b0; b < b1; ++b) {
-      // Activations of this super-block first, then the next one's weights: the loads return in
-      // order, so the weights may stay in flight while the MFMAs wait for the activations only.
-      uint4 a[RT][8];
-      float sums[RT][4];
+    for (int i = 0; i < kUnitTiles; ++i) cursor[i].open(tile[i].image + size_t(b0) * kRecord, lane);
+    const uint4 *share[2 * RT];
 #pragma unroll
-      for (int t = 0; t < RT; ++t) {
+    for (int j = 0; j < 2 * RT; ++j) {
+      const uint32_t at = threadIdx.x + 256u * j, t = at / 512u, g = (at / 64u) % 8u, l = at % 64u;
+      share[j] = values + (size_t(t) * G + 8u * b0 + g) * 64u + l;
+    }
+    // Threads past the staged sums repeat an earlier thread's (same value to the same slot).
+    const float *sumShare[kSumShare];
+    uint32_t sumSlot[kSumShare];
 #pragma unroll
-        for (uint32_t g = 0; g < 8; ++g) a[t][g] = values[(size_t(t) * G + 8u * b + g) * 64u + lane];
+    for (int q = 0; q < kSumShare; ++q) {
+      const uint32_t at = (threadIdx.x + 256u * q) % kSumFloats;
+      const uint32_t t = at / (kSumsPerBlock * 64u), j = (at / 64u) % kSumsPerBlock, l = at % 64u;
+      sumShare[q] = sumsBase + (size_t(t) * sumGroups + kSumsPerBlock * 4u * b0 + 4u * j + (l >> 4)) * 16u + (l & 15u);
+      sumSlot[q] = (t * 4u + j) * 64u + l;
+    }
+    uint32_t issued = b0;  // the next super-block to issue; stops at b1 - 1
+    auto issue = [&](Stage &st) {
 #pragma unroll
-        for (uint32_t j = 0; j < kSumsPerBlock; ++j)
-          sums[t][j] = sumsBase[(size_t(t) * sumGroups + kSumsPerBlock * 4u * b + 4u * j + kq) * 16u + c];
+      for (int j = 0; j < 2 * RT; ++j) st.a[j] = *share[j];
+#pragma unroll
+      for (int q = 0; q < kSumShare; ++q) st.sum[q] = *sumShare[q];
+#pragma unroll
+      for (int i = 0; i < kUnitTiles; ++i) st.rec[i].load(cursor[i]);
+      if (issued + 1 < b1) {  // uniform: scalar branch over a few pointer bumps
+        ++issued;
+#pragma unroll
+        for (int j = 0; j < 2 * RT; ++j) share[j] += 8u * 64u;
+#pragma unroll
+        for (int q = 0; q < kSumShare; ++q) sumShare[q] += kSumsPerBlock * 4u * 16u;
+#pragma unroll
+        for (int i = 0; i < kUnitTiles; ++i) cursor[i].advance();
       }
-      if (b + 1 < b1) {
+    };
+#pragma unroll
+    for (int s = 0; s < kStages - 1; ++s) issue(stage[s]);
+    const uint32_t count = b1 - b0, rounds = (count + kStages - 1) / kStages;
+    uint32_t now = 0;
+    for (uint32_t round = 0; round < rounds; ++round) {
+#pragma unroll
+      for (int u = 0; u < kStages; ++u, ++now) {
+        const uint32_t buffer = now & 1u;
+#pragma unroll
+        for (int j = 0; j < 2 * RT; ++j) (&ldsA[buffer][0][0][0])[threadIdx.x + 256u * j] = stage[u].a[j];
+#pragma unroll
+        for (int q = 0; q < kSumShare; ++q) (&ldsSums[buffer][0][0][0])[sumSlot[q]] = stage[u].sum[q];
+        __syncthreads();
+        issue(stage[(u + kStages - 1) % kStages]);
+        const float keep = now < count ? 1.0f : 0.0f;
 #pragma unroll
         for (int i = 0; i < kUnitTiles; ++i)
-          if (tile[i].image) next[i].load(tile[i].image + size_t(b + 1) * kRecord, lane);
+          accumulate_record<FMT, RT>(stage[u].rec[i], ldsA[buffer], ldsSums[buffer], acc[i], lane, kq, keep);
       }
-#pragma unroll
-      for (int i = 0; i < kUnitTiles; ++i)
-        if (tile[i].image) accumulate_record<FMT, RT>(cur[i], a, sums, acc[i], kq);
-#pragma unroll
-      for (int i = 0; i < kUnitTiles; ++i) cur[i] = next[i];
     }
   }
 
-  // Waves that share tiles: wave ks = 0 adds the others' sums in wave order.
-  if (kw > 1) {
-    if (ks > 0) {
+  tile[0].image = live[0] ? tile[0].image : nullptr;
 #pragma unroll
-      for (int i = 0; i < kUnitTiles; ++i)
-#pragma unroll
-        for (int t = 0; t < RT; ++t)
-#pragma unroll
-          for (int v = 0; v < 4; ++v) reduce[wave - 1][i][t][v][lane] = acc[i][t][v];
-    }
-    __syncthreads();
-    if (ks == 0) {
-      for (uint32_t other = 1; other < kw; ++other)
-#pragma unroll
-        for (int i = 0; i < kUnitTiles; ++i)
-#pragma unroll
-          for (int t = 0; t < RT; ++t)
-#pragma unroll
-            for (int v = 0; v < 4; ++v) acc[i][t][v] += reduce[wave + other - 1][i][t][v][lane];
-    }
-  }
+  for (int i = 1; i < kUnitTiles; ++i) tile[i].image = live[i] ? tile[i].image : nullptr;
 
   // Element (i, t, v) of this lane is row 16 t + 4 kq + v, column tile[i].column + c.
   const uint32_t paddedRows = tiles * GGUF_ROW_TILE;
@@ -367,15 +433,19 @@ __global__ __launch_bounds__(256) void gguf_decode(const uint8_t *__restrict__ s
         for (int t = 0; t < RT; ++t)
 #pragma unroll
           for (int v = 0; v < 4; ++v)
-            partials[(size_t(split) * paddedRows + 16u * t + 4u * kq + v) * width + column] = acc[i][t][v];
+            __hip_atomic_store(&partials[(size_t(split) * paddedRows + 16u * t + 4u * kq + v) * width + column], acc[i][t][v],
+                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
     }
-    __threadfence();
+    // The partials are written and read with agent-scope atomics, which go to the coherence
+    // point instead of a compute die's own L2, so no cache write-back or invalidate is needed: the
+    // workgroup only waits for its stores to complete before it counts itself in.
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
-    if (threadIdx.x == 0) arrived = atomicAdd(&counters[blockIdx.x], 1u);
+    if (threadIdx.x == 0) arrived = __hip_atomic_fetch_add(&counters[blockIdx.x], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
     if (arrived != p.splits - 1) return;
-    __threadfence();
     if (finish) {
 #pragma unroll
       for (int i = 0; i < kUnitTiles; ++i) {
@@ -388,12 +458,13 @@ __global__ __launch_bounds__(256) void gguf_decode(const uint8_t *__restrict__ s
           for (int v = 0; v < 4; ++v) {
             float sum = 0.f;
             for (uint32_t s = 0; s < p.splits; ++s)
-              sum += partials[(size_t(s) * paddedRows + 16u * t + 4u * kq + v) * width + column];
+              sum += __hip_atomic_load(&partials[(size_t(s) * paddedRows + 16u * t + 4u * kq + v) * width + column],
+                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             acc[i][t][v] = sum;
           }
       }
     }
-    if (threadIdx.x == 0) counters[blockIdx.x] = 0;
+    if (threadIdx.x == 0) __hip_atomic_store(&counters[blockIdx.x], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
   if (!finish) return;
 

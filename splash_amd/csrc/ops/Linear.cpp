@@ -56,8 +56,7 @@ void LinearPlan::requireConfiguration() const {
   if (!n || n % GGUF_TILE_COLUMNS || !k || k % GGUF_BLOCK)
     throw std::invalid_argument("block projections take whole 16-column tiles and 256-input super-blocks");
   const LinearConfig &c = config_;
-  if (c.kWaves != 1 && c.kWaves != 2 && c.kWaves != 4)
-    throw std::invalid_argument("a block workgroup splits K over 1, 2 or 4 waves");
+  if (c.kWaves != 1) throw std::invalid_argument("the waves of a block workgroup walk one K range");
   if (!c.validSplits() || uint64_t{c.splits} * c.kWaves > k / GGUF_BLOCK)
     throw std::invalid_argument("block splits take at least one super-block each");
   if (destination_ == FloatOutput::Float32 && workload_.epilogue != LinearEpilogue::None)
@@ -73,7 +72,7 @@ LinearScratchSize LinearPlan::scratchSize() const noexcept {
     // [split][row][column] fp32 partials over the tile's rows, a gate/up pair's of both tensors,
     // and one counter per workgroup.
     const uint64_t columns = workload_.epilogue == LinearEpilogue::GateUp ? 2 * uint64_t{n} : n;
-    const uint32_t across = 4 / config_.kWaves;
+    const uint32_t across = 4;
     size.partials = uint64_t{config_.splits} * tiles * GGUF_ROW_TILE * columns * sizeof(float);
     size.counters = uint64_t{(unitsOf(n, workload_.epilogue) + across - 1) / across} * sizeof(uint32_t);
   }
@@ -89,16 +88,15 @@ LinearPlan Linear::plan(LinearWorkload workload, LinearConfig config, FloatOutpu
 }
 
 LinearPlan Linear::plan(LinearWorkload w, FloatOutput destination) const {
-  // Fill the device: partition K, first over the waves of a workgroup (summed through LDS, no
-  // memory traffic), then across workgroups (fp32 partials), until the dispatch holds
-  // wavesPerUnit waves per compute unit or a wave's range is down to minimumBlocksPerWave.
+  // Fill the device: partition K across workgroups (fp32 partials, summed in split order by the
+  // last arriver) until the dispatch holds wavesPerUnit waves per compute unit or a wave's range
+  // is down to minimumBlocksPerWave.
   const uint32_t blocks = w.matrix.inputSize / GGUF_BLOCK;
   const uint32_t units = std::max(1u, unitsOf(w.matrix.outputSize, w.epilogue));
   const uint64_t wanted = uint64_t{calibration_.computeUnits} * calibration_.wavesPerUnit;
   LinearConfig config;
   auto parts = [&] { return config.splits * config.kWaves; };
   auto mayDouble = [&] { return uint64_t{units} * parts() < wanted && blocks / (2 * parts()) >= calibration_.minimumBlocksPerWave; };
-  while (config.kWaves < 4 && mayDouble()) config.kWaves *= 2;
   while (config.splits < LinearConfig::kMaximumSplits && mayDouble()) config.splits *= 2;
   return LinearPlan(w, config, destination);
 }
@@ -182,7 +180,7 @@ PreparedInput Linear::add(hip::CommandGraph &graph, LinearBuffers b, const Proje
   params.units = unitsOf(n, w.epilogue);
   // Unused bindings still name a buffer: the table stands in for them.
   const hip::Buffer &spare = b.scratch.input;
-  const uint32_t across = 4 / c.kWaves;
+  const uint32_t across = 4;
   const std::string name = std::string("gguf_decode_") + segments.front().name() + "_m" + std::to_string(plan.storageRows()) +
                            epilogueSuffix(w.epilogue, plan.destination());
   graph.add(name,

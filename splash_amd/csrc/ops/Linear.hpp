@@ -44,7 +44,8 @@ struct LinearConfig final {
   // Cross-workgroup K partitions, a power of two up to kMaximumSplits.
   uint32_t splits = 1;
   static constexpr uint32_t kMaximumSplits = GGUF_MAXIMUM_SPLITS;
-  // Waves of a workgroup that share its column tiles and split its K partition: 1, 2 or 4.
+  // Waves of a workgroup that split its K partition between them: 1 (its four waves walk the
+  // partition in step, each over its own column tiles).
   uint32_t kWaves = 1;
   [[nodiscard]] constexpr bool validSplits() const noexcept {
     return splits && splits <= kMaximumSplits && !(splits & (splits - 1));

@@ -1,0 +1,150 @@
+#include "ops/PagedAttention.hpp"
+#include "ops/Linear.hpp"  // requireBytes
+
+#include <algorithm>
+#include <stdexcept>
+#include <string>
+
+namespace splash::ops {
+
+AttentionSplits attentionSplits(uint64_t tokens) noexcept {
+  // About 64 splits of a long history, whole pages each: with 8 KV heads that is two workgroups
+  // per compute unit; a split never holds less than one page.
+  const uint32_t pages = std::max(1u, kv::Layout::pagesFor(tokens));
+  AttentionSplits s;
+  s.pagesPerSplit = std::max(1u, (pages + 63) / 64);
+  s.splits = (pages + s.pagesPerSplit - 1) / s.pagesPerSplit;
+  return s;
+}
+
+namespace {
+std::string kernelSuffix(const AttentionGeometry &g) { return "_d" + std::to_string(g.headDimension); }
+bool compiled(const AttentionGeometry &g) {
+  return (g.headDimension == 128 && (g.group() == 8 || g.group() == 4)) || (g.headDimension == 64 && g.group() == 2);
+}
+uint32_t totalRows(const std::vector<AttentionRows> &sequences) {
+  uint32_t rows = 0;
+  for (const AttentionRows &s : sequences) rows = std::max(rows, s.firstRow + s.rows);
+  return rows;
+}
+void requirePages(const AttentionPlan &plan, const KvPages &pages) {
+  const uint64_t need = plan.geometry().layout().bytesPerLayerPage();
+  if (pages.pageBytes < need || pages.pageBytes % 16) throw std::invalid_argument("KV page stride is smaller than a page or unaligned");
+  if (!pages.pool || pages.pool.sizeBytes() < pages.pageBytes) throw std::invalid_argument("KV pool buffer is too small");
+  uint64_t entries = 0;
+  for (const AttentionRows &s : plan.sequences())
+    entries = std::max<uint64_t>(entries, uint64_t{s.tableFirst} + kv::Layout::pagesFor(uint64_t{s.committed} + s.rows));
+  requireBytes(pages.pageTable, entries * 8, "KV page table");
+}
+} // namespace
+
+AttentionWorkspaceSize AttentionPlan::workspace() const noexcept {
+  const uint64_t fused = uint64_t{sequences_.size()} * geometry_.kvHeads * geometry_.group() * 16;
+  AttentionWorkspaceSize size;
+  size.queries = fused * geometry_.headDimension * 2;
+  size.querySums = fused * 4;
+  size.partials = fused * splits_ * geometry_.headDimension * 4;
+  size.partialSums = fused * splits_ * 8;
+  return size;
+}
+
+AttentionParams AttentionPlan::params(uint64_t pageBytes) const noexcept {
+  AttentionParams p{};
+  p.q_heads = geometry_.qHeads;
+  p.kv_heads = geometry_.kvHeads;
+  p.head_dim = geometry_.headDimension;
+  p.rotary_pairs = geometry_.rotaryPairs;
+  p.normalize = geometry_.normalize;
+  p.qkv_stride = geometry_.packedWidth();
+  p.splits = splits_;
+  p.sequences = uint32_t(sequences_.size());
+  p.page_bytes = pageBytes;
+  for (size_t i = 0; i < sequences_.size(); ++i)
+    p.sequence[i] = {sequences_[i].firstRow, sequences_[i].committed, sequences_[i].tableFirst, uint16_t(sequences_[i].rows),
+                     uint16_t(partition_[i].pagesPerSplit)};
+  return p;
+}
+
+AttentionPlan PagedAttention::plan(const AttentionGeometry &geometry, std::vector<AttentionRows> sequences) {
+  if (!geometry.kvHeads || geometry.qHeads % geometry.kvHeads || !compiled(geometry))
+    throw std::invalid_argument("no attention kernel for this head geometry");
+  if (2 * geometry.rotaryPairs > geometry.headDimension) throw std::invalid_argument("the rotated pairs are dimensions of the head");
+  if (sequences.empty() || sequences.size() > ATTENTION_MAXIMUM_SEQUENCES)
+    throw std::invalid_argument("an attention dispatch takes 1 to 8 sequences");
+  AttentionPlan plan;
+  plan.geometry_ = geometry;
+  for (const AttentionRows &s : sequences) {
+    if (!s.rows || s.rows > ATTENTION_MAXIMUM_ROWS) throw std::invalid_argument("a sequence's verify block holds 1 to 16 rows");
+    const AttentionSplits part = attentionSplits(uint64_t{s.committed} + s.rows);
+    if (part.splits > ATTENTION_MAXIMUM_SPLITS || part.pagesPerSplit > 0xFFFF)
+      throw std::invalid_argument("the sequence is longer than the attention kernels split");
+    plan.partition_.push_back(part);
+    plan.splits_ = std::max(plan.splits_, part.splits);
+  }
+  plan.sequences_ = std::move(sequences);
+  return plan;
+}
+
+void PagedAttention::addProjection(hip::CommandGraph &graph, const AttentionPlan &plan, const AttentionProjectionBuffers &b,
+                                   const AttentionWorkspace &w, const KvPages &pages) {
+  const AttentionGeometry &g = plan.geometry();
+  const uint32_t rows = totalRows(plan.sequences());
+  requireBytes(b.qkv, uint64_t{rows} * g.packedWidth() * 2, "attention qkv");
+  if (g.normalize) {
+    requireBytes(b.queryNorm, g.headDimension * 2, "query norm weight");
+    requireBytes(b.keyNorm, g.headDimension * 2, "key norm weight");
+  }
+  if (g.rotaryPairs) {
+    requireBytes(b.ropeCos, uint64_t{rows} * g.rotaryPairs * 4, "RoPE cosine table");
+    requireBytes(b.ropeSin, uint64_t{rows} * g.rotaryPairs * 4, "RoPE sine table");
+  }
+  const AttentionWorkspaceSize need = plan.workspace();
+  requireBytes(w.queries, need.queries, "staged queries");
+  requireBytes(w.querySums, need.querySums, "staged query sums");
+  requirePages(plan, pages);
+  // Unused bindings still name a buffer.
+  const hip::Buffer &spare = b.qkv;
+  graph.add("attention_q8_qkv" + kernelSuffix(g),
+            {b.qkv, g.normalize ? b.queryNorm : spare, g.normalize ? b.keyNorm : spare, g.rotaryPairs ? b.ropeCos : spare,
+             g.rotaryPairs ? b.ropeSin : spare, w.queries, w.querySums, pages.pageTable, pages.pool},
+            plan.params(pages.pageBytes), {g.qHeads + g.kvHeads, ATTENTION_MAXIMUM_ROWS, plan.sequences().size()},
+            {g.headDimension, 1, 1});
+}
+
+void PagedAttention::addAttention(hip::CommandGraph &graph, const AttentionPlan &plan, const AttentionWorkspace &w,
+                                  const hip::Buffer &treeRows, const KvPages &pages, const hip::Buffer &output) {
+  const AttentionGeometry &g = plan.geometry();
+  const uint32_t rows = totalRows(plan.sequences());
+  const AttentionWorkspaceSize need = plan.workspace();
+  requireBytes(w.queries, need.queries, "staged queries");
+  requireBytes(w.querySums, need.querySums, "staged query sums");
+  requireBytes(w.partials, need.partials, "attention partials");
+  requireBytes(w.partialSums, need.partialSums, "attention partial sums");
+  requireBytes(treeRows, uint64_t{rows} * sizeof(AttentionTreeRow), "verify tree rows");
+  requireBytes(output, uint64_t{rows} * g.qHeads * g.headDimension * 2, "attention output");
+  requirePages(plan, pages);
+  const AttentionParams params = plan.params(pages.pageBytes);
+  graph.add("attention_q8_split" + kernelSuffix(g) + "_g" + std::to_string(g.group()),
+            {w.queries, w.querySums, treeRows, pages.pageTable, pages.pool, w.partials, w.partialSums}, params,
+            {g.kvHeads, plan.splits(), plan.sequences().size()}, {256, 1, 1});
+  graph.add("attention_reduce" + kernelSuffix(g), {w.partials, w.partialSums, output}, params,
+            {g.qHeads, ATTENTION_MAXIMUM_ROWS, plan.sequences().size()}, {g.headDimension, 1, 1});
+}
+
+void PagedAttention::addPathCommit(hip::CommandGraph &graph, const AttentionPlan &plan, const hip::Buffer &retained,
+                                   const KvPages &pages) {
+  const AttentionGeometry &g = plan.geometry();
+  requireBytes(retained, plan.sequences().size() * 4, "retained rows");
+  requirePages(plan, pages);
+  const AttentionParams full = plan.params(pages.pageBytes);
+  AttentionCommitParams params{};
+  params.kv_heads = g.kvHeads;
+  params.head_dim = g.headDimension;
+  params.sequences = full.sequences;
+  params.page_bytes = pages.pageBytes;
+  for (uint32_t i = 0; i < full.sequences; ++i) params.sequence[i] = full.sequence[i];
+  graph.add("attention_q8_commit" + kernelSuffix(g), {retained, pages.pageTable, pages.pool}, params,
+            {g.kvHeads, plan.sequences().size(), 1}, {g.headDimension, 1, 1});
+}
+
+} // namespace splash::ops

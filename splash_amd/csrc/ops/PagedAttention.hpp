@@ -1,0 +1,106 @@
+// Paged INT8-KV attention of a verify block: the counterpart of the reference's
+// ops::PagedAttention (runtime/ops/PagedAttention.hpp:179-366, PagedAttention.cpp:125-146,
+// :351-389, :441-667) and kv::Layout (runtime/ops/PagedKv.hpp:155-260) over the gfx950 kernels of
+// kernels/paged_attention.hip. Every add* validates its buffers and throws std::invalid_argument
+// before it adds a dispatch.
+#pragma once
+#include "abi/PagedAttention.h"
+#include "hip/Backend.hpp"
+
+#include <cstdint>
+#include <vector>
+
+namespace splash::ops {
+
+namespace kv {
+// A layer's page geometry (PagedKv.hpp:155-260 in the reference; 256-token pages, fp16 scales here).
+struct Layout final {
+  uint32_t kvHeads = 0;
+  uint32_t headDimension = 0;
+  static constexpr uint32_t kPageTokens = ATTENTION_PAGE_TOKENS;
+  [[nodiscard]] uint64_t bytesPerLayerPage() const noexcept { return attention_page_bytes(kvHeads, headDimension); }
+  [[nodiscard]] uint64_t bytesPerToken() const noexcept { return bytesPerLayerPage() / kPageTokens; }
+  [[nodiscard]] static uint32_t pagesFor(uint64_t tokens) noexcept { return uint32_t((tokens + kPageTokens - 1) / kPageTokens); }
+};
+} // namespace kv
+
+struct AttentionGeometry final {
+  uint32_t qHeads = 0, kvHeads = 0, headDimension = 0;
+  uint32_t rotaryPairs = 0;  // pairs (i, i + pairs) RoPE rotates
+  bool normalize = false;    // RMS-norm q and k heads (q_norm, k_norm weights)
+  [[nodiscard]] uint32_t group() const noexcept { return kvHeads ? qHeads / kvHeads : 0; }
+  [[nodiscard]] uint32_t packedWidth() const noexcept { return (qHeads + 2 * kvHeads) * headDimension; }
+  [[nodiscard]] kv::Layout layout() const noexcept { return {kvHeads, headDimension}; }
+};
+
+// One sequence's rows of a dispatch (the reference's AttentionRows / AttentionHistory).
+struct AttentionRows final {
+  uint32_t firstRow = 0;    // first packed row
+  uint32_t rows = 0;        // 1..16
+  uint32_t committed = 0;   // tokens cached before the block
+  uint32_t tableFirst = 0;  // first page-table entry of the sequence
+};
+
+// History splits of a sequence of `tokens` tokens (committed + rows): a split holds
+// pagesPerSplit logical pages; the partition follows the sequence alone
+// (PagedAttention.cpp:125-146 in the reference states the same rule for its geometry).
+struct AttentionSplits final {
+  uint32_t splits = 1;
+  uint32_t pagesPerSplit = 1;
+};
+[[nodiscard]] AttentionSplits attentionSplits(uint64_t tokens) noexcept;
+
+struct AttentionWorkspaceSize final {
+  uint64_t queries = 0, querySums = 0, partials = 0, partialSums = 0;
+};
+struct AttentionWorkspace final {
+  hip::Buffer queries;      // staged fp16 query rows
+  hip::Buffer querySums;    // their fp32 sums
+  hip::Buffer partials;     // fp32 split outputs
+  hip::Buffer partialSums;  // fp32 (max, sum) per split and fused row
+};
+
+class AttentionPlan final {
+public:
+  [[nodiscard]] const AttentionGeometry &geometry() const noexcept { return geometry_; }
+  [[nodiscard]] const std::vector<AttentionRows> &sequences() const noexcept { return sequences_; }
+  [[nodiscard]] uint32_t splits() const noexcept { return splits_; }
+  [[nodiscard]] AttentionWorkspaceSize workspace() const noexcept;
+  [[nodiscard]] AttentionParams params(uint64_t pageBytes) const noexcept;
+
+private:
+  friend class PagedAttention;
+  AttentionGeometry geometry_;
+  std::vector<AttentionRows> sequences_;
+  std::vector<AttentionSplits> partition_;
+  uint32_t splits_ = 1;
+};
+
+struct AttentionProjectionBuffers final {
+  hip::Buffer qkv;             // bf16 [packed rows][(q + 2 kv) heads * D]
+  hip::Buffer queryNorm, keyNorm;  // bf16 [D]; used when geometry.normalize
+  hip::Buffer ropeCos, ropeSin;    // fp32 [packed rows][rotaryPairs]; used when rotaryPairs
+};
+struct KvPages final {
+  hip::Buffer pageTable;  // uint64 physical page per logical page
+  hip::Buffer pool;       // the layer's physical pages
+  uint64_t pageBytes = 0; // bytes between pages (>= layout.bytesPerLayerPage())
+};
+
+class PagedAttention final {
+public:
+  // Throws for a geometry no kernel is compiled for, no or too many sequences, or rows outside 1..16.
+  [[nodiscard]] static AttentionPlan plan(const AttentionGeometry &geometry, std::vector<AttentionRows> sequences);
+  // q/k norm + RoPE + query staging + INT8 store of the block's K and V (PagedAttention.cpp:441-464).
+  static void addProjection(hip::CommandGraph &graph, const AttentionPlan &plan, const AttentionProjectionBuffers &buffers,
+                            const AttentionWorkspace &workspace, const KvPages &pages);
+  // Split + reduce (PagedAttention.cpp:466-607): output bf16 [packed rows][q heads * D].
+  static void addAttention(hip::CommandGraph &graph, const AttentionPlan &plan, const AttentionWorkspace &workspace,
+                           const hip::Buffer &treeRows, const KvPages &pages, const hip::Buffer &output);
+  // Moves the retained path's slots to their depths (PagedAttention.cpp:647-667); retained is a
+  // uint32 mask per sequence.
+  static void addPathCommit(hip::CommandGraph &graph, const AttentionPlan &plan, const hip::Buffer &retained,
+                            const KvPages &pages);
+};
+
+} // namespace splash::ops

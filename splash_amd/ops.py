@@ -137,3 +137,132 @@ class Linear:
         check(lib.spo_linear_scratch_size(self.handle, output_size, input_size, rows, ctypes.byref(t), ctypes.byref(s),
                                           ctypes.byref(c)))
         return t.value, s.value, c.value
+
+
+# ---------------------------------------------------------------------------------------------
+# PagedAttention (runtime/ops/PagedAttention.hpp in the reference)
+# ---------------------------------------------------------------------------------------------
+PAGE_TOKENS = 256
+VALUE_BLOCK = 64
+
+
+def kv_page_bytes(kv_heads, head_dim):
+    return lib.spo_kv_page_bytes(kv_heads, head_dim)
+
+
+class KvPages:
+    """One layer's KV pool: physical pages, and the page table (uint64 physical page per logical page)."""
+
+    def __init__(self, backend, kv_heads, head_dim, physical_pages, page_table):
+        self.kv_heads, self.head_dim = kv_heads, head_dim
+        self.page_bytes = kv_page_bytes(kv_heads, head_dim)
+        self.physical_pages = physical_pages
+        self.pool = backend.allocate_buffer(self.page_bytes * physical_pages, STORAGE_PRIVATE, "kv pool")
+        self.table = backend.from_array(np.asarray(page_table, dtype=np.uint64), STORAGE_PRIVATE, "page table")
+
+    # Host-side (de)serialisation of pages from logical arrays, for tests and synthetic contexts.
+    def pack_pages(self, kcodes, kscales, vcodes, vscales):
+        """Logical arrays [pages][kv_heads][256][D] int8 and [pages][kv_heads][256] float -> page bytes."""
+        pages, H, T, D = kcodes.shape
+        out = np.zeros((pages, self.page_bytes), dtype=np.uint8)
+        kb = H * T * D
+        out[:, :kb] = kcodes.reshape(pages, kb).view(np.uint8)
+        # values: [H][T/64][D][64]
+        v = vcodes.reshape(pages, H, T // VALUE_BLOCK, VALUE_BLOCK, D).transpose(0, 1, 2, 4, 3)
+        out[:, kb:2 * kb] = np.ascontiguousarray(v).reshape(pages, kb).view(np.uint8)
+        sb = H * T * 2
+        out[:, 2 * kb:2 * kb + sb] = kscales.astype(np.float16).reshape(pages, H * T).view(np.uint8)
+        out[:, 2 * kb + sb:2 * kb + 2 * sb] = vscales.astype(np.float16).reshape(pages, H * T).view(np.uint8)
+        return out
+
+    def unpack_pages(self, raw):
+        pages = raw.shape[0]
+        H, T, D = self.kv_heads, PAGE_TOKENS, self.head_dim
+        kb, sb = H * T * D, H * T * 2
+        kcodes = raw[:, :kb].view(np.int8).reshape(pages, H, T, D)
+        v = raw[:, kb:2 * kb].view(np.int8).reshape(pages, H, T // VALUE_BLOCK, D, VALUE_BLOCK).transpose(0, 1, 2, 4, 3)
+        vcodes = np.ascontiguousarray(v).reshape(pages, H, T, D)
+        kscales = raw[:, 2 * kb:2 * kb + sb].copy().view(np.float16).reshape(pages, H, T).astype(np.float32)
+        vscales = raw[:, 2 * kb + sb:2 * kb + 2 * sb].copy().view(np.float16).reshape(pages, H, T).astype(np.float32)
+        return kcodes, kscales, vcodes, vscales
+
+    def upload(self, page_bytes_array, first_page=0):
+        self.pool.upload(page_bytes_array, first_page * self.page_bytes)
+
+    def download(self):
+        return self.pool.download(np.uint8).reshape(self.physical_pages, self.page_bytes)
+
+
+class AttentionPlan:
+    """ops::AttentionPlan: geometry + sequences + history splits."""
+
+    def __init__(self, q_heads, kv_heads, head_dim, sequences, rotary_pairs=0, normalize=False):
+        """sequences: [(first_row, rows, committed, table_first)]"""
+        g = nat.AttentionGeometry(q_heads, kv_heads, head_dim, rotary_pairs, int(normalize))
+        rows = (nat.AttentionRows * len(sequences))(*[nat.AttentionRows(*s) for s in sequences])
+        h = ctypes.c_void_p()
+        check(lib.spo_attention_plan_create(ctypes.byref(g), rows, len(sequences), ctypes.byref(h)))
+        self.handle = h
+        self.geometry = g
+        self.sequences = sequences
+
+    @property
+    def splits(self):
+        return lib.spo_attention_plan_splits(self.handle)
+
+    def workspace_sizes(self):
+        sizes = (ctypes.c_uint64 * 4)()
+        check(lib.spo_attention_workspace(self.handle, sizes))
+        return list(sizes)
+
+    def __del__(self):
+        try:
+            lib.spo_attention_plan_destroy(self.handle)
+        except Exception:
+            pass
+
+
+class AttentionWorkspace:
+    def __init__(self, backend, plan):
+        q, qs, po, ps = plan.workspace_sizes()
+        self.queries = backend.allocate_buffer(q, STORAGE_PRIVATE, "staged queries")
+        self.query_sums = backend.allocate_buffer(qs, STORAGE_PRIVATE, "query sums")
+        self.partials = backend.allocate_buffer(po, STORAGE_PRIVATE, "attention partials")
+        self.partial_sums = backend.allocate_buffer(ps, STORAGE_PRIVATE, "attention partial sums")
+
+
+class PagedAttention:
+    """ops::PagedAttention: addProjection, addAttention, addPathCommit."""
+
+    @staticmethod
+    def add_projection(graph, plan, qkv, workspace, pages, query_norm=None, key_norm=None, rope_cos=None, rope_sin=None):
+        h = lambda b: b.handle if b is not None else None
+        check(lib.spo_attention_add_projection(graph.handle, plan.handle, qkv.handle, h(query_norm), h(key_norm), h(rope_cos),
+                                               h(rope_sin), workspace.queries.handle, workspace.query_sums.handle,
+                                               pages.table.handle, pages.pool.handle, pages.page_bytes))
+        graph._keep.extend([plan, qkv, workspace, pages, query_norm, key_norm, rope_cos, rope_sin])
+
+    @staticmethod
+    def add_attention(graph, plan, workspace, tree_rows, pages, output):
+        check(lib.spo_attention_add_attention(graph.handle, plan.handle, workspace.queries.handle, workspace.query_sums.handle,
+                                              workspace.partials.handle, workspace.partial_sums.handle, tree_rows.handle,
+                                              pages.table.handle, pages.pool.handle, pages.page_bytes, output.handle))
+        graph._keep.extend([plan, workspace, tree_rows, pages, output])
+
+    @staticmethod
+    def add_path_commit(graph, plan, retained, pages):
+        check(lib.spo_attention_add_path_commit(graph.handle, plan.handle, retained.handle, pages.table.handle,
+                                                pages.pool.handle, pages.page_bytes))
+        graph._keep.extend([plan, retained, pages])
+
+
+def chain_tree_rows(rows_per_sequence):
+    """SplashTreeRow of chains: ancestors (2 << r) - 1, parent r - 1, depth r, packed per sequence."""
+    out = []
+    for rows in rows_per_sequence:
+        for r in range(rows):
+            out.append(((2 << r) - 1, max(r - 1, 0) if r else 0xFFFF, r))
+    arr = np.zeros(len(out), dtype=np.dtype([("ancestors", "<u4"), ("parent", "<u2"), ("depth", "<u2")]))
+    for i, (a, p, d) in enumerate(out):
+        arr[i] = (a, p, d)
+    return arr

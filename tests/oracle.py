@@ -139,3 +139,51 @@ def projection_interval(exact, bound):
     hi = bf16_to_f32(f32_to_bf16((exact + bound).astype(np.float32)))
     # float32 rounding of lo/hi before bf16 can move them inward by an fp32 ulp: widen by it.
     return np.nextafter(lo, -np.inf), np.nextafter(hi, np.inf)
+
+
+class OrcAttention(ctypes.Structure):
+    _fields_ = [("q_heads", c_u32), ("kv_heads", c_u32), ("head_dim", c_u32), ("rows", c_u32), ("committed", c_u32),
+                ("page_tokens", c_u32), ("splits", c_u32), ("pages_per_split", c_u32), ("half_scale", c_u32)]
+
+
+def kv_quantize(values, half_scale=True):
+    """values float32 [..., D] -> (codes int8 [..., D], scales float32 [...]) by the reference's store rule."""
+    v = np.ascontiguousarray(values, dtype=np.float32)
+    flat = v.reshape(-1, v.shape[-1])
+    codes = np.empty(flat.shape, dtype=np.int8)
+    scales = np.empty(flat.shape[0], dtype=np.float32)
+    s = c_f()
+    for i in range(flat.shape[0]):
+        lib.orc_kv_quantize(_p(flat[i], f32p), c_u32(flat.shape[1]), c_int(int(half_scale)), _p(codes[i], i8p), ctypes.byref(s))
+        scales[i] = s.value
+    return codes.reshape(v.shape), scales.reshape(v.shape[:-1])
+
+
+def attention_prepare(q_heads, kv_heads, head_dim, qkv_bits, qw, kw, cosv, sinv, pairs):
+    rows = qkv_bits.shape[0]
+    a = OrcAttention(q_heads, kv_heads, head_dim, rows, 0, 256, 1, 1, 1)
+    q = np.empty((rows, q_heads, head_dim), dtype=np.uint16)
+    k = np.empty((rows, kv_heads, head_dim), dtype=np.float32)
+    v = np.empty((rows, kv_heads, head_dim), dtype=np.float32)
+    qkv_bits = np.ascontiguousarray(qkv_bits, dtype=np.uint16)
+    lib.orc_attention_prepare(ctypes.byref(a), _p(qkv_bits, u16p), _p(qw, u16p), _p(kw, u16p), _p(cosv, f32p), _p(sinv, f32p),
+                              c_u32(pairs), _p(q, u16p), _p(k, f32p), _p(v, f32p))
+    return q, k, v
+
+
+def attention(q_bits, kcodes, kscales, vcodes, vscales, page_table, ancestors, committed, splits=1, pages_per_split=1 << 20,
+              want64=True, threads=0):
+    """q_bits uint16 [rows][q_heads][D]; K/V logical pages [phys][kv_heads][256][D] int8, scales [phys][kv_heads][256]."""
+    rows, q_heads, D = q_bits.shape
+    kv_heads, PT = kcodes.shape[1], kcodes.shape[2]
+    a = OrcAttention(q_heads, kv_heads, D, rows, committed, PT, splits, pages_per_split, 1)
+    out = np.empty((rows, q_heads, D), dtype=np.uint16)
+    out64 = np.empty((rows, q_heads, D), dtype=np.float64) if want64 else None
+    q_bits = np.ascontiguousarray(q_bits, dtype=np.uint16)
+    kcodes, vcodes = np.ascontiguousarray(kcodes, dtype=np.int8), np.ascontiguousarray(vcodes, dtype=np.int8)
+    kscales, vscales = np.ascontiguousarray(kscales, dtype=np.float32), np.ascontiguousarray(vscales, dtype=np.float32)
+    pt = np.ascontiguousarray(page_table, dtype=np.uint32)
+    anc = np.ascontiguousarray(ancestors, dtype=np.uint32)
+    lib.orc_attention(ctypes.byref(a), _p(q_bits, u16p), _p(kcodes, i8p), _p(kscales, f32p), _p(vcodes, i8p), _p(vscales, f32p),
+                      _p(pt, u32p), _p(anc, u32p), _p(out, u16p), _p(out64, f64p), c_int(threads))
+    return out, out64
