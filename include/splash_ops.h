@@ -119,6 +119,74 @@ sp_status spo_attention_add_attention(spo_graph *graph, const spo_attention_plan
 sp_status spo_attention_add_path_commit(spo_graph *graph, const spo_attention_plan *plan, sp_buffer *retained,
                                         sp_buffer *page_table, sp_buffer *pool, uint64_t page_bytes);
 
+/* ---- Normalization, Embedding, RoPE (runtime/ops/Normalization.cpp:16-40, Embedding.cpp:20-47, RoPE.hpp:33-37) ---- */
+sp_status spo_norm_add_rms(spo_graph *graph, sp_buffer *input, sp_buffer *weight, sp_buffer *output, uint32_t width,
+                           uint32_t rows);
+/* The norm that also writes the projection activation table of its rows (norm_rms_table16_decode). */
+sp_status spo_norm_add_rms_table(spo_graph *graph, sp_buffer *input, sp_buffer *weight, sp_buffer *output,
+                                 sp_buffer *table, uint32_t width, uint32_t rows);
+sp_status spo_embedding_add(spo_graph *graph, uint32_t format, sp_buffer *native_rows, uint32_t vocabulary,
+                            uint32_t hidden, sp_buffer *tokens, sp_buffer *output, uint32_t rows);
+typedef struct spo_rope_sequence { uint32_t first_row, rows, anchor; } spo_rope_sequence;
+sp_status spo_rope_add_tree_tables(spo_graph *graph, sp_buffer *inverse_frequency, sp_buffer *depth, sp_buffer *cosines,
+                                   sp_buffer *sines, uint32_t pairs, const spo_rope_sequence *sequences, uint32_t count);
+
+/* ---- Sampling (runtime/ops/Sampling.hpp:64-254, Sampling.cpp:283-357) ---- */
+typedef struct spo_lane_rows { uint32_t first, rows; } spo_lane_rows; /* SplashLaneRows */
+/* Sampling::workspace: bytes of the argmax partial values and indices, the masses, ranges, decisions. */
+sp_status spo_sampling_workspace(uint32_t rows, uint64_t sizes[5]);
+typedef struct spo_sampling_buffers {
+  sp_buffer *logits, *tokens, *partial_values, *partial_indices;
+  sp_buffer *draft_probabilities, *uniforms, *masses, *ranges, *decisions, *input_tokens, *tree_rows; /* sampled lanes */
+} spo_sampling_buffers;
+/* Sampling::addVerify (Sampling.cpp:283-328): temperature 0 is greedy. */
+sp_status spo_sampling_add_verify(spo_graph *graph, const spo_sampling_buffers *buffers, uint32_t vocabulary,
+                                  uint32_t logits_stride, const spo_lane_rows *lanes, const float *temperatures,
+                                  uint32_t count);
+/* Sampling::addAcceptance (Sampling.cpp:330-357). */
+sp_status spo_sampling_add_acceptance(spo_graph *graph, sp_buffer *input_tokens, sp_buffer *tree_rows, sp_buffer *tokens,
+                                      sp_buffer *retained, sp_buffer *accepted_count, sp_buffer *retained_rows,
+                                      const spo_lane_rows *lanes, const uint32_t *remaining, uint32_t count,
+                                      const uint32_t stop_tokens[4]);
+
+/* ---- The dense verify step (the reference's model layer: QwenTarget.cpp:206-395, :457-496;
+ *      Runtime.cpp:2677-2717, :2883-2892) ---- */
+typedef struct spo_dense_verify spo_dense_verify;
+typedef struct spo_dense_dimensions {
+  uint32_t hidden, q_heads, kv_heads, head_dim, ffn, vocabulary, layers, rotary_pairs, normalize_heads;
+  float rope_theta;
+} spo_dense_dimensions;
+typedef struct spo_verify_lane {
+  uint32_t rows, committed, table_first;
+  float temperature;  /* 0: greedy */
+  uint32_t remaining; /* tokens the lane may still keep */
+} spo_verify_lane;
+sp_status spo_dense_verify_create(sp_backend *backend, const spo_dense_dimensions *dimensions, uint32_t max_lanes,
+                                  uint32_t physical_pages, uint32_t page_table_entries, spo_dense_verify **out);
+void spo_dense_verify_destroy(spo_dense_verify *verify);
+sp_status spo_dense_verify_set_layer(spo_dense_verify *verify, uint32_t layer, const spo_projection *qkv,
+                                     const spo_projection *output, const spo_projection *gate, const spo_projection *up,
+                                     const spo_projection *down, sp_buffer *input_norm, sp_buffer *post_norm,
+                                     sp_buffer *query_norm, sp_buffer *key_norm);
+sp_status spo_dense_verify_set_head(spo_dense_verify *verify, uint32_t embedding_format, sp_buffer *embedding_rows,
+                                    sp_buffer *final_norm, const spo_projection *head);
+/* The step's buffers; each call returns a new reference (release it). `index` is the layer for KV pools. */
+typedef enum spo_verify_buffer {
+  SPO_VERIFY_INPUT_TOKENS = 0, SPO_VERIFY_TREE_ROWS, SPO_VERIFY_DEPTHS, SPO_VERIFY_UNIFORMS, SPO_VERIFY_TOKENS,
+  SPO_VERIFY_RETAINED, SPO_VERIFY_ACCEPTED, SPO_VERIFY_RETAINED_ROWS, SPO_VERIFY_PAGE_TABLE, SPO_VERIFY_KV_POOL,
+  SPO_VERIFY_LOGITS, SPO_VERIFY_DRAFT_PROBABILITIES, SPO_VERIFY_HIDDEN
+} spo_verify_buffer;
+sp_status spo_dense_verify_buffer(spo_dense_verify *verify, spo_verify_buffer which, uint32_t index, sp_buffer **out);
+uint64_t spo_dense_verify_page_bytes(const spo_dense_verify *verify);
+/* Algorithmic HBM bytes of one step: weights once, each lane's KV, logits written and read. */
+uint64_t spo_dense_verify_step_bytes(const spo_dense_verify *verify, const spo_verify_lane *lanes, uint32_t count);
+/* Appends the whole target part of a cycle (Runtime.cpp:3985-3993) to the graph. */
+sp_status spo_dense_verify_encode(spo_dense_verify *verify, spo_graph *graph, const spo_verify_lane *lanes, uint32_t count,
+                                  int commit);
+/* One part of it, for per-part timing: 0 embedding, 1 one layer (index), 2 final norm + head. */
+sp_status spo_dense_verify_encode_part(spo_dense_verify *verify, spo_graph *graph, uint32_t part, uint32_t index,
+                                       const spo_verify_lane *lanes, uint32_t count);
+
 #ifdef __cplusplus
 }
 #endif

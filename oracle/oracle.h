@@ -121,8 +121,14 @@ uint32_t orc_accept_tree(const struct OrcTreeRow *tree, const uint32_t *tokens, 
 // operations (sampling.metal:713-885): weight_t = exp((logit_t - max) / T); p = weight / total;
 // accept the drafted token iff u_child * q[draft] < p[draft]; else draw from max(p - q, 0)
 // renormalised by an id-ordered prefix walk at u_row. q NULL: plain draw at u_row * total.
+// closeness (optional): the smallest relative distance of a decisive comparison from its threshold;
+// tests treat a row below 1e-5 as "close", as target_sampling_metal_test.mm:2645-2709 does.
 uint32_t orc_rejection_row(const float *logits, uint32_t vocab, float temperature, const float *q,
-                           uint32_t draft_token, float u_child, float u_row, int *accepted_draft);
+                           uint32_t draft_token, float u_child, float u_row, int *accepted_draft, double *closeness);
+// The selection law of one sampled row in fp64, for the enumeration check
+// (target_sampling_metal_test.mm:2602-2631): out[t] = P(row selects t) when the draft proposes its
+// child from q and the row tests and redraws as above. It must equal softmax(logits / T).
+void orc_rejection_law(const float *logits, uint32_t vocab, float temperature, const float *q, double *out);
 
 // ---- Gated DeltaNet ----
 struct OrcGdn { uint32_t key_heads, value_heads, head_dim /*128*/, conv_taps /*4*/; };

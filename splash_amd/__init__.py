@@ -7,3 +7,4 @@ this package only binds it with ctypes. There is no CPU fallback: importing work
 from ._native import lib, library_path, SplashError, check  # noqa: F401
 from .backend import Backend, Buffer, CommandGraph, STORAGE_PRIVATE, STORAGE_SHARED  # noqa: F401
 from . import ops  # noqa: F401
+from . import verify  # noqa: F401

@@ -82,6 +82,29 @@ class AttentionRows(ctypes.Structure):
     _fields_ = [("first_row", c_u32), ("rows", c_u32), ("committed", c_u32), ("table_first", c_u32)]
 
 
+class RopeSequence(ctypes.Structure):
+    _fields_ = [("first_row", c_u32), ("rows", c_u32), ("anchor", c_u32)]
+
+
+class LaneRows(ctypes.Structure):
+    _fields_ = [("first", c_u32), ("rows", c_u32)]
+
+
+class SamplingBuffers(ctypes.Structure):
+    _fields_ = [(n, c_p) for n in ("logits", "tokens", "partial_values", "partial_indices", "draft_probabilities", "uniforms",
+                                   "masses", "ranges", "decisions", "input_tokens", "tree_rows")]
+
+
+class DenseDimensions(ctypes.Structure):
+    _fields_ = [(n, c_u32) for n in ("hidden", "q_heads", "kv_heads", "head_dim", "ffn", "vocabulary", "layers", "rotary_pairs",
+                                     "normalize_heads")] + [("rope_theta", ctypes.c_float)]
+
+
+class VerifyLane(ctypes.Structure):
+    _fields_ = [("rows", c_u32), ("committed", c_u32), ("table_first", c_u32), ("temperature", ctypes.c_float),
+                ("remaining", c_u32)]
+
+
 def _sig(name, restype, *argtypes):
     fn = getattr(lib, name)
     fn.restype = restype
@@ -159,3 +182,20 @@ _sig("spo_attention_workspace", c_int, c_p, P(c_u64))
 _sig("spo_attention_add_projection", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_u64)
 _sig("spo_attention_add_attention", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_u64, c_p)
 _sig("spo_attention_add_path_commit", c_int, c_p, c_p, c_p, c_p, c_p, c_u64)
+
+_sig("spo_norm_add_rms", c_int, c_p, c_p, c_p, c_p, c_u32, c_u32)
+_sig("spo_norm_add_rms_table", c_int, c_p, c_p, c_p, c_p, c_p, c_u32, c_u32)
+_sig("spo_embedding_add", c_int, c_p, c_u32, c_p, c_u32, c_u32, c_p, c_p, c_u32)
+_sig("spo_rope_add_tree_tables", c_int, c_p, c_p, c_p, c_p, c_p, c_u32, P(RopeSequence), c_u32)
+_sig("spo_sampling_workspace", c_int, c_u32, P(c_u64))
+_sig("spo_sampling_add_verify", c_int, c_p, P(SamplingBuffers), c_u32, c_u32, P(LaneRows), P(ctypes.c_float), c_u32)
+_sig("spo_sampling_add_acceptance", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, P(LaneRows), P(c_u32), c_u32, P(c_u32))
+_sig("spo_dense_verify_create", c_int, c_p, P(DenseDimensions), c_u32, c_u32, c_u32, P(c_p))
+_sig("spo_dense_verify_destroy", None, c_p)
+_sig("spo_dense_verify_set_layer", c_int, c_p, c_u32, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p)
+_sig("spo_dense_verify_set_head", c_int, c_p, c_u32, c_p, c_p, c_p)
+_sig("spo_dense_verify_buffer", c_int, c_p, c_int, c_u32, P(c_p))
+_sig("spo_dense_verify_page_bytes", c_u64, c_p)
+_sig("spo_dense_verify_step_bytes", c_u64, c_p, P(VerifyLane), c_u32)
+_sig("spo_dense_verify_encode", c_int, c_p, c_p, P(VerifyLane), c_u32, c_int)
+_sig("spo_dense_verify_encode_part", c_int, c_p, c_p, c_u32, c_u32, P(VerifyLane), c_u32)

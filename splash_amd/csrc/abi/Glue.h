@@ -1,0 +1,33 @@
+// Parameters of the glue kernels on the verify path: RMS norm, RoPE tables, token embedding
+// (the reference's abi/RoPE.h, abi/Embedding.h and the `uint width` of its norm kernels).
+#pragma once
+#include <stdint.h>
+
+#define SPLASH_RMS_EPSILON 1e-6f
+
+// norm_rms / norm_rms_table16: one workgroup of 256 threads per row. norm_rms_table16 also writes
+// the projection activation table of the normalized rows (abi/Gguf.h), as the reference's
+// norm_rms_table16_decode does for its register tile.
+struct NormParams {
+  uint32_t width;
+  uint32_t rows;
+  uint32_t tiles;  // row tiles of the table (norm_rms_table16)
+  uint32_t reserved;
+};
+
+// rope_build_tree_tables: cos and sin of (anchor[sequence] + depth[row]) * inverse_frequency[pair]
+// per packed row (the reference's RopeTreeParams, abi/RoPE.h). Grid (rows), `pairs` threads.
+struct RopeTreeParams {
+  uint32_t pairs;
+  uint32_t rows;
+  uint32_t sequences;
+  uint32_t reserved;
+  uint32_t first_row[8];  // per sequence
+  uint32_t row_count[8];
+  uint32_t anchor[8];     // position of the sequence's row 0
+};
+
+#ifdef __cplusplus
+static_assert(sizeof(NormParams) == 16, "norm parameters are 16 bytes on both sides");
+static_assert(sizeof(RopeTreeParams) == 112, "RoPE tree parameters are 112 bytes on both sides");
+#endif

@@ -90,8 +90,9 @@ struct AttentionParams {
 struct AttentionCommitParams {
   uint32_t kv_heads, head_dim;
   uint32_t sequences;
-  uint32_t reserved;
+  uint32_t layers;         // grid.z: the layers' pools lie layer_bytes apart from the bound pool
   uint64_t page_bytes;
+  uint64_t layer_bytes;
   struct AttentionSequence sequence[ATTENTION_MAXIMUM_SEQUENCES];
 };
 
@@ -99,5 +100,5 @@ struct AttentionCommitParams {
 static_assert(sizeof(AttentionTreeRow) == 8, "a tree row is 8 bytes on both sides");
 static_assert(sizeof(AttentionSequence) == 16, "an attention sequence is 16 bytes on both sides");
 static_assert(sizeof(AttentionParams) == 48 + 16 * ATTENTION_MAXIMUM_SEQUENCES, "attention parameters are 176 bytes on both sides");
-static_assert(sizeof(AttentionCommitParams) == 24 + 16 * ATTENTION_MAXIMUM_SEQUENCES, "commit parameters are 152 bytes on both sides");
+static_assert(sizeof(AttentionCommitParams) == 32 + 16 * ATTENTION_MAXIMUM_SEQUENCES, "commit parameters are 160 bytes on both sides");
 #endif

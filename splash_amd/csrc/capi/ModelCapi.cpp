@@ -1,0 +1,187 @@
+// C entry points of the glue operators, ops::Sampling and model::DenseVerify (include/splash_ops.h).
+#include "splash_ops.h"
+#include "capi/Guard.hpp"
+#include "capi/Handles.hpp"
+#include "model/DenseVerify.hpp"
+#include "ops/Glue.hpp"
+#include "ops/Sampling.hpp"
+
+#include <memory>
+
+using namespace splash;
+
+struct spo_dense_verify {
+  std::unique_ptr<hip::Backend> backend;  // a borrowed wrapper of the caller's backend
+  std::unique_ptr<model::DenseVerify> verify;
+};
+
+namespace {
+hip::Buffer B(sp_buffer *b) { return hip::Buffer::share(b); }
+std::vector<model::VerifyLane> lanesOf(const spo_verify_lane *lanes, uint32_t count) {
+  capi::require(lanes && count, "lanes");
+  std::vector<model::VerifyLane> out;
+  for (uint32_t i = 0; i < count; ++i)
+    out.push_back({lanes[i].rows, lanes[i].committed, lanes[i].table_first, ops::SamplingPolicy{lanes[i].temperature}, lanes[i].remaining});
+  return out;
+}
+ops::AttentionPlan planOf(const model::DenseVerify &v, const std::vector<model::VerifyLane> &lanes) {
+  const model::DenseDimensions &d = v.dimensions();
+  std::vector<ops::AttentionRows> sequences;
+  uint32_t rows = 0;
+  for (const model::VerifyLane &l : lanes) { sequences.push_back({rows, l.rows, l.committed, l.tableFirst}); rows += l.rows; }
+  return ops::PagedAttention::plan({d.qHeads, d.kvHeads, d.headDimension, d.rotaryPairs, d.normalizeHeads}, sequences);
+}
+} // namespace
+
+extern "C" {
+
+sp_status spo_norm_add_rms(spo_graph *graph, sp_buffer *input, sp_buffer *weight, sp_buffer *output, uint32_t width, uint32_t rows) {
+  return capi::guard([&] { capi::require(graph, "graph"); ops::Normalization::addRms(capi::graphOf(graph), B(input), B(weight), B(output), width, rows); });
+}
+sp_status spo_norm_add_rms_table(spo_graph *graph, sp_buffer *input, sp_buffer *weight, sp_buffer *output, sp_buffer *table,
+                                 uint32_t width, uint32_t rows) {
+  return capi::guard([&] {
+    capi::require(graph, "graph");
+    ops::LinearScratch scratch{B(table), {}, {}};
+    ops::Normalization::addRmsTable(capi::graphOf(graph), B(input), B(weight), B(output), scratch, width, rows);
+  });
+}
+sp_status spo_embedding_add(spo_graph *graph, uint32_t format, sp_buffer *native_rows, uint32_t vocabulary, uint32_t hidden,
+                            sp_buffer *tokens, sp_buffer *output, uint32_t rows) {
+  return capi::guard([&] {
+    capi::require(graph, "graph");
+    ops::Embedding::add(capi::graphOf(graph), {B(native_rows), format, vocabulary, hidden}, B(tokens), B(output), rows);
+  });
+}
+sp_status spo_rope_add_tree_tables(spo_graph *graph, sp_buffer *inverse_frequency, sp_buffer *depth, sp_buffer *cosines,
+                                   sp_buffer *sines, uint32_t pairs, const spo_rope_sequence *sequences, uint32_t count) {
+  return capi::guard([&] {
+    capi::require(graph && sequences, "graph or sequences");
+    std::vector<ops::RopeSequence> list;
+    for (uint32_t i = 0; i < count; ++i) list.push_back({sequences[i].first_row, sequences[i].rows, sequences[i].anchor});
+    ops::RoPE::addTreeTables(capi::graphOf(graph), B(inverse_frequency), B(depth), B(cosines), B(sines), pairs, list);
+  });
+}
+
+sp_status spo_sampling_workspace(uint32_t rows, uint64_t sizes[5]) {
+  return capi::guard([&] {
+    capi::require(sizes, "result");
+    const ops::SamplingWorkspaceSize s = ops::Sampling::workspace(rows);
+    sizes[0] = s.partialValues; sizes[1] = s.partialIndices; sizes[2] = s.masses; sizes[3] = s.ranges; sizes[4] = s.decisions;
+  });
+}
+sp_status spo_sampling_add_verify(spo_graph *graph, const spo_sampling_buffers *b, uint32_t vocabulary, uint32_t logits_stride,
+                                  const spo_lane_rows *lanes, const float *temperatures, uint32_t count) {
+  return capi::guard([&] {
+    capi::require(graph && b && lanes && temperatures, "graph, buffers, lanes or temperatures");
+    ops::SamplingBuffers buffers{B(b->logits), B(b->tokens), B(b->partial_values), B(b->partial_indices), B(b->draft_probabilities),
+                                 B(b->uniforms), B(b->masses), B(b->ranges), B(b->decisions), B(b->input_tokens), B(b->tree_rows)};
+    std::vector<ops::LaneRows> rows;
+    std::vector<ops::SamplingPolicy> policies;
+    for (uint32_t i = 0; i < count; ++i) { rows.push_back({lanes[i].first, lanes[i].rows}); policies.push_back({temperatures[i]}); }
+    ops::Sampling::addVerify(capi::graphOf(graph), buffers, vocabulary, logits_stride, rows, policies);
+  });
+}
+sp_status spo_sampling_add_acceptance(spo_graph *graph, sp_buffer *input_tokens, sp_buffer *tree_rows, sp_buffer *tokens,
+                                      sp_buffer *retained, sp_buffer *accepted_count, sp_buffer *retained_rows,
+                                      const spo_lane_rows *lanes, const uint32_t *remaining, uint32_t count,
+                                      const uint32_t stop_tokens[4]) {
+  return capi::guard([&] {
+    capi::require(graph && lanes && remaining && stop_tokens, "graph, lanes, remaining or stop tokens");
+    std::vector<ops::LaneRows> rows;
+    std::vector<uint32_t> left;
+    for (uint32_t i = 0; i < count; ++i) { rows.push_back({lanes[i].first, lanes[i].rows}); left.push_back(remaining[i]); }
+    ops::Sampling::addAcceptance(capi::graphOf(graph), {B(input_tokens), B(tree_rows), B(tokens), B(retained), B(accepted_count), B(retained_rows)},
+                                 rows, left, {stop_tokens[0], stop_tokens[1], stop_tokens[2], stop_tokens[3]});
+  });
+}
+
+sp_status spo_dense_verify_create(sp_backend *backend, const spo_dense_dimensions *d, uint32_t max_lanes, uint32_t physical_pages,
+                                  uint32_t page_table_entries, spo_dense_verify **out) {
+  return capi::guard([&] {
+    capi::require(backend && d && out, "backend, dimensions or result");
+    auto holder = std::make_unique<spo_dense_verify>();
+    holder->backend = std::make_unique<hip::Backend>(backend);
+    model::DenseDimensions dims{d->hidden, d->q_heads, d->kv_heads, d->head_dim, d->ffn, d->vocabulary, d->layers,
+                                d->rotary_pairs, d->normalize_heads != 0, d->rope_theta};
+    holder->verify = std::make_unique<model::DenseVerify>(*holder->backend, dims, max_lanes, physical_pages, page_table_entries);
+    *out = holder.release();
+  });
+}
+void spo_dense_verify_destroy(spo_dense_verify *verify) { delete verify; }
+
+sp_status spo_dense_verify_set_layer(spo_dense_verify *verify, uint32_t layer, const spo_projection *qkv, const spo_projection *output,
+                                     const spo_projection *gate, const spo_projection *up, const spo_projection *down,
+                                     sp_buffer *input_norm, sp_buffer *post_norm, sp_buffer *query_norm, sp_buffer *key_norm) {
+  return capi::guard([&] {
+    capi::require(verify && qkv && output && gate && up && down, "verify or projections");
+    model::DenseWeights &w = verify->verify->weights();
+    if (layer >= w.layers.size()) throw std::invalid_argument("no such layer");
+    w.layers[layer] = {capi::projectionOf(qkv), capi::projectionOf(output), capi::projectionOf(gate), capi::projectionOf(up),
+                       capi::projectionOf(down), B(input_norm), B(post_norm), B(query_norm), B(key_norm)};
+  });
+}
+sp_status spo_dense_verify_set_head(spo_dense_verify *verify, uint32_t embedding_format, sp_buffer *embedding_rows,
+                                    sp_buffer *final_norm, const spo_projection *head) {
+  return capi::guard([&] {
+    capi::require(verify && head, "verify or head");
+    model::DenseWeights &w = verify->verify->weights();
+    const model::DenseDimensions &d = verify->verify->dimensions();
+    w.embedding = {B(embedding_rows), embedding_format, d.vocabulary, d.hidden};
+    w.finalNorm = B(final_norm);
+    w.head = capi::projectionOf(head);
+    w.head.destination = ops::FloatOutput::Float32;
+  });
+}
+sp_status spo_dense_verify_buffer(spo_dense_verify *verify, spo_verify_buffer which, uint32_t index, sp_buffer **out) {
+  return capi::guard([&] {
+    capi::require(verify && out, "verify or result");
+    model::DenseVerify &v = *verify->verify;
+    hip::Buffer b;
+    switch (which) {
+    case SPO_VERIFY_INPUT_TOKENS: b = v.inputTokens(); break;
+    case SPO_VERIFY_TREE_ROWS: b = v.treeRows(); break;
+    case SPO_VERIFY_DEPTHS: b = v.depths(); break;
+    case SPO_VERIFY_UNIFORMS: b = v.uniforms(); break;
+    case SPO_VERIFY_TOKENS: b = v.tokens(); break;
+    case SPO_VERIFY_RETAINED: b = v.retained(); break;
+    case SPO_VERIFY_ACCEPTED: b = v.acceptedCount(); break;
+    case SPO_VERIFY_RETAINED_ROWS: b = v.retainedRows(); break;
+    case SPO_VERIFY_PAGE_TABLE: b = v.pageTable(); break;
+    case SPO_VERIFY_KV_POOL: b = v.kvPool(index); break;
+    case SPO_VERIFY_LOGITS: b = v.logits(); break;
+    case SPO_VERIFY_DRAFT_PROBABILITIES: b = v.draftProbabilities(); break;
+    case SPO_VERIFY_HIDDEN: b = v.hidden(index); break;
+    default: throw std::invalid_argument("no such verify buffer");
+    }
+    sp_buffer_retain(b.handle());
+    *out = b.handle();
+  });
+}
+uint64_t spo_dense_verify_page_bytes(const spo_dense_verify *verify) { return verify ? verify->verify->pageBytes() : 0; }
+uint64_t spo_dense_verify_step_bytes(const spo_dense_verify *verify, const spo_verify_lane *lanes, uint32_t count) {
+  uint64_t bytes = 0;
+  capi::guard([&] { capi::require(verify, "verify"); bytes = verify->verify->stepBytes(lanesOf(lanes, count)); });
+  return bytes;
+}
+sp_status spo_dense_verify_encode(spo_dense_verify *verify, spo_graph *graph, const spo_verify_lane *lanes, uint32_t count, int commit) {
+  return capi::guard([&] {
+    capi::require(verify && graph, "verify or graph");
+    verify->verify->encode(capi::graphOf(graph), lanesOf(lanes, count), commit != 0);
+  });
+}
+sp_status spo_dense_verify_encode_part(spo_dense_verify *verify, spo_graph *graph, uint32_t part, uint32_t index,
+                                       const spo_verify_lane *lanes, uint32_t count) {
+  return capi::guard([&] {
+    capi::require(verify && graph, "verify or graph");
+    const std::vector<model::VerifyLane> list = lanesOf(lanes, count);
+    uint32_t rows = 0;
+    for (const model::VerifyLane &l : list) rows += l.rows;
+    if (part == 0) verify->verify->encodeEmbedding(capi::graphOf(graph), rows);
+    else if (part == 1) verify->verify->encodeLayer(capi::graphOf(graph), index, planOf(*verify->verify, list), rows);
+    else if (part == 2) verify->verify->encodeHead(capi::graphOf(graph), rows);
+    else throw std::invalid_argument("no such part of the step");
+  });
+}
+
+} // extern "C"

@@ -11,8 +11,6 @@
 using namespace splash;
 
 
-struct spo_projection { ops::Projection projection; };
-struct spo_linear { ops::Linear linear; };
 
 namespace {
 ops::LinearPlan toPlan(const ops::Projection &projection, const spo_linear_plan &p) {

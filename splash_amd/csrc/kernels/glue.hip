@@ -1,0 +1,138 @@
+// Glue kernels of the verify path: RMS norm (with the projection's activation table fused in),
+// RoPE tables per packed row, token embedding from native K-quant rows (the reference's
+// kernels/shared/normalization.metal, rope.metal, embedding.metal).
+#include "abi/Glue.h"
+#include "abi/Gguf.h"
+#include "backend/KernelRegistry.hpp"
+#include "kernels/device_common.hpp"
+
+namespace splash::kernels {
+
+// The row's inverse RMS: 256 threads sum the squares of columns tid, tid + 256, ... in column
+// order; a wavefront sums its lanes by butterfly, the four wavefronts' sums are added in order
+// (normalization.metal:59-99 and common/rms_inverse.h:15-33, on 64-lane wavefronts).
+__device__ __forceinline__ float rms_inverse(const uint16_t *row, uint32_t width, float *scratch) {
+  float sum = 0.f;
+  for (uint32_t c = threadIdx.x; c < width; c += 256) {
+    const float v = bf16_bits_to_float(row[c]);
+    sum += v * v;
+  }
+  sum = wave_sum(sum);
+  if ((threadIdx.x & 63u) == 0) scratch[threadIdx.x >> 6] = sum;
+  __syncthreads();
+  const float total = ((scratch[0] + scratch[1]) + scratch[2]) + scratch[3];
+  return 1.0f / sqrtf(total / float(width) + SPLASH_RMS_EPSILON);
+}
+
+__global__ __launch_bounds__(256) void norm_rms(const uint16_t *__restrict__ input, const uint16_t *__restrict__ weight,
+                                                uint16_t *__restrict__ output, NormParams p) {
+  __shared__ float scratch[4];
+  const uint32_t row = blockIdx.x;
+  const uint16_t *x = input + size_t(row) * p.width;
+  const float inverse = rms_inverse(x, p.width, scratch);
+  for (uint32_t c = threadIdx.x; c < p.width; c += 256)
+    output[size_t(row) * p.width + c] = uint16_t(float_to_bf16_bits((bf16_bits_to_float(x[c]) * inverse) * bf16_bits_to_float(weight[c])));
+}
+SP_REGISTER_KERNEL("norm_rms", &norm_rms);
+
+// The same, and the activation table of the normalized rows: grid (tiles * 16) so that the rows
+// past the live ones are written as zeros. Each thread normalizes runs of four inputs
+// (4 kq .. 4 kq + 3 of a group's half), which are one 8-byte piece of a table entry.
+__global__ __launch_bounds__(256) void norm_rms_table16(const uint16_t *__restrict__ input, const uint16_t *__restrict__ weight,
+                                                        uint16_t *__restrict__ output, uint8_t *__restrict__ table, NormParams p) {
+  __shared__ float scratch[4];
+  const uint32_t row = blockIdx.x, tile = row / 16u, r = row % 16u, G = p.width / 32u;
+  const bool live = row < p.rows;
+  const uint16_t *x = input + size_t(live ? row : 0) * p.width;
+  const float inverse = live ? rms_inverse(x, p.width, scratch) : 0.f;
+  uint2 *values = reinterpret_cast<uint2 *>(table);
+  float *sums32 = reinterpret_cast<float *>(table + gguf_table_sums32_offset(p.width, p.tiles));
+  float *sums16 = reinterpret_cast<float *>(table + gguf_table_sums16_offset(p.width, p.tiles));
+  // run q covers inputs 4 q .. 4 q + 3: group g = q / 8, half = (q / 4) % 2, kq = q % 4
+  for (uint32_t q = threadIdx.x; q < p.width / 4u; q += 256) {
+    uint32_t bits[4] = {0, 0, 0, 0};
+    float v[4] = {0.f, 0.f, 0.f, 0.f};
+    if (live) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const uint32_t c = 4u * q + i;
+        bits[i] = float_to_bf16_bits((bf16_bits_to_float(x[c]) * inverse) * bf16_bits_to_float(weight[c]));
+        v[i] = bf16_bits_to_float(bits[i]);
+        output[size_t(row) * p.width + c] = uint16_t(bits[i]);
+      }
+    }
+    const uint32_t g = q / 8u, half = (q / 4u) % 2u, kq = q % 4u;
+    // operand elements 4 half + {0,1,2,3} are inputs 4 kq + {0,2,1,3} of the half
+    const uint2 piece = make_uint2(bits[0] | (bits[2] << 16), bits[1] | (bits[3] << 16));
+    values[((size_t(tile) * G + g) * 64u + kq * 16u + r) * 2u + half] = piece;
+    // sums of 16 inputs in input order: the four runs of a half sit in four consecutive lanes
+    float s = (v[0] + v[1]) + (v[2] + v[3]);
+    const float s1 = __shfl_down(s, 1, 64), s2 = __shfl_down(s, 2, 64), s3 = __shfl_down(s, 3, 64);
+    s = ((s + s1) + s2) + s3;
+    const float other = __shfl_down(s, 4, 64);
+    if (kq == 0) {
+      sums16[(size_t(tile) * 2u * G + 2u * g + half) * 16u + r] = s;
+      if (half == 0) sums32[(size_t(tile) * G + g) * 16u + r] = s + other;
+    }
+  }
+}
+SP_REGISTER_KERNEL("norm_rms_table16", &norm_rms_table16);
+
+__global__ void rope_build_tree_tables(const float *__restrict__ inverse_frequency, const uint32_t *__restrict__ depth,
+                                       float *__restrict__ cosines, float *__restrict__ sines, RopeTreeParams p) {
+  const uint32_t row = blockIdx.x, pair = threadIdx.x;
+  if (row >= p.rows || pair >= p.pairs) return;
+  uint32_t anchor = 0;
+  for (uint32_t s = 0; s < p.sequences; ++s)
+    if (row >= p.first_row[s] && row < p.first_row[s] + p.row_count[s]) anchor = p.anchor[s];
+  const float angle = float(anchor + depth[row]) * inverse_frequency[pair];
+  cosines[size_t(row) * p.pairs + pair] = cosf(angle);
+  sines[size_t(row) * p.pairs + pair] = sinf(angle);
+}
+SP_REGISTER_KERNEL("rope_build_tree_tables", &rope_build_tree_tables);
+
+// gguf_embed_<fmt>: out[r][:] = bf16(decode(native row tokens[r])); a token at or past the
+// vocabulary gives zeros (embedding.metal:10-18). Grid (rows, hidden / 256), 64 threads: a thread
+// decodes four values of a super-block.
+template <uint32_t FMT>
+__global__ __launch_bounds__(64) void gguf_embed(const uint8_t *__restrict__ table, const uint32_t *__restrict__ tokens,
+                                                 uint16_t *__restrict__ out, GgufEmbedParams p) {
+  const uint32_t row = blockIdx.x, block = blockIdx.y, tid = threadIdx.x;
+  const uint32_t token = tokens[row];
+  uint16_t *o = out + size_t(row) * p.hidden + size_t(block) * 256u;
+  if (token >= p.vocabulary) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[tid + 64 * i] = 0;
+    return;
+  }
+  const uint32_t blocks = p.hidden / 256u;
+  if constexpr (FMT == GGUF_FMT_Q4K) {
+    const uint8_t *blk = table + (size_t(token) * blocks + block) * GGUF_Q4K_NATIVE;
+    const float d = half_bits_to_float(blk[0] | (blk[1] << 8)), dmin = half_bits_to_float(blk[2] | (blk[3] << 8));
+    const uint8_t *sc = blk + 4, *qs = blk + 16;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t k = tid + 64u * i, j = k / 32u, e = k % 32u;
+      uint32_t s, m;
+      if (j < 4) { s = sc[j] & 63u; m = sc[j + 4] & 63u; }
+      else { s = (sc[j + 4] & 0xFu) | ((sc[j - 4] >> 6) << 4); m = (sc[j + 4] >> 4) | ((sc[j] >> 6) << 4); }
+      const uint32_t code = (qs[32u * (j / 2u) + e] >> (4u * (j % 2u))) & 15u;
+      o[k] = uint16_t(float_to_bf16_bits(__fmaf_rn(d * float(s), float(code), -(dmin * float(m)))));
+    }
+  } else {
+    const uint8_t *blk = table + (size_t(token) * blocks + block) * GGUF_Q6K_NATIVE;
+    const float d = half_bits_to_float(blk[208] | (blk[209] << 8));
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t k = tid + 64u * i, n = k / 128u, r = (k % 128u) / 32u, e = k % 32u;
+      const uint32_t l4 = (blk[64u * n + e + 32u * (r & 1u)] >> (4u * (r >> 1))) & 15u, h2 = (blk[128u + 32u * n + e] >> (2u * r)) & 3u;
+      const int q = int(l4 | (h2 << 4)) - 32;
+      const float scale = float(int(int8_t(blk[192u + 8u * n + 2u * r + e / 16u])));
+      o[k] = uint16_t(float_to_bf16_bits(d * scale * float(q)));
+    }
+  }
+}
+SP_REGISTER_KERNEL("gguf_embed_q4k", &gguf_embed<GGUF_FMT_Q4K>);
+SP_REGISTER_KERNEL("gguf_embed_q6k", &gguf_embed<GGUF_FMT_Q6K>);
+
+} // namespace splash::kernels

@@ -394,7 +394,7 @@ SP_REGISTER_KERNEL("attention_reduce_d128", &attention_reduce<128>);
 SP_REGISTER_KERNEL("attention_reduce_d64", &attention_reduce<64>);
 
 // ---------------------------------------------------------------------------------------------
-// attention_q8_commit: grid (kv_heads, sequences), D threads. retained[z] is the mask of the block
+// attention_q8_commit: grid (kv_heads, sequences, layers), D threads. retained[z] is the mask of the block
 // rows on the accepted path; its k-th set bit (row r) moves from slot committed + r to committed + k.
 // ---------------------------------------------------------------------------------------------
 template <int D>
@@ -403,6 +403,7 @@ __global__ __launch_bounds__(D) void attention_q8_commit(const uint32_t *__restr
                                                          AttentionCommitParams p) {
   const uint32_t tid = threadIdx.x, h = blockIdx.x, z = blockIdx.y;
   const AttentionSequence seq = p.sequence[z];
+  pool += uint64_t(blockIdx.z) * p.layer_bytes;
   uint32_t mask = retained[z];
   uint32_t depth = 0;
   while (mask) {

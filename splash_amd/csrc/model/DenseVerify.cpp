@@ -1,0 +1,174 @@
+#include "model/DenseVerify.hpp"
+
+#include <algorithm>
+#include <cmath>
+#include <stdexcept>
+
+namespace splash::model {
+
+using hip::BufferStorage;
+
+DenseVerify::DenseVerify(hip::Backend &backend, DenseDimensions d, uint32_t maxLanes, uint32_t physicalPages,
+                         uint32_t pageTableEntries)
+    : backend_(backend), dims_(d), linear_(backend.deviceInfo()), maxLanes_(maxLanes) {
+  if (!d.hidden || !d.layers || !d.vocabulary || !d.ffn || !maxLanes || maxLanes > 4)
+    throw std::invalid_argument("a dense verify step takes a model and 1 to 4 lanes");
+  if (d.hidden % GGUF_BLOCK || d.ffn % GGUF_BLOCK || d.attentionWidth() % GGUF_BLOCK || d.vocabulary % GGUF_TILE_COLUMNS)
+    throw std::invalid_argument("the model's widths hold whole super-blocks and its vocabulary whole column tiles");
+  maxRows_ = maxLanes * ATTENTION_MAXIMUM_ROWS;
+  weights_.layers.resize(d.layers);
+  const ops::kv::Layout layout{d.kvHeads, d.headDimension};
+  pageBytes_ = layout.bytesPerLayerPage();
+  auto device = [&](uint64_t bytes, const char *label) { return backend.allocateBuffer(std::max<uint64_t>(bytes, 16), BufferStorage::Private, label); };
+  auto shared = [&](uint64_t bytes, const char *label) { return backend.allocateBuffer(std::max<uint64_t>(bytes, 16), BufferStorage::Shared, label); };
+  const uint64_t R = maxRows_;
+  hidden_[0] = device(R * d.hidden * 2, "hidden 0");
+  hidden_[1] = device(R * d.hidden * 2, "hidden 1");
+  normalized_ = device(R * d.hidden * 2, "normalized");
+  qkv_ = device(R * d.qkvWidth() * 2, "qkv");
+  attention_ = device(R * d.attentionWidth() * 2, "attention output");
+  intermediate_ = device(R * d.ffn * 2, "ffn intermediate");
+  logits_ = device(R * d.vocabulary * 4, "logits");
+  ropeCos_ = device(R * std::max(1u, d.rotaryPairs) * 4, "rope cos");
+  ropeSin_ = device(R * std::max(1u, d.rotaryPairs) * 4, "rope sin");
+  inverseFrequency_ = device(std::max(1u, d.rotaryPairs) * 4, "rope inverse frequency");
+  if (d.rotaryPairs) {
+    std::vector<float> inv(d.rotaryPairs);
+    for (uint32_t i = 0; i < d.rotaryPairs; ++i) inv[i] = float(std::pow(double(d.ropeTheta), -double(i) / d.rotaryPairs));
+    inverseFrequency_.upload(inv.data(), inv.size() * 4);
+  }
+  inputTokens_ = shared(R * 4, "input tokens");
+  treeRows_ = shared(R * sizeof(AttentionTreeRow), "tree rows");
+  depths_ = shared(R * 4, "row depths");
+  uniforms_ = shared(R * 8, "uniforms");
+  tokens_ = shared(R * 4, "selected tokens");
+  retained_ = shared(maxLanes * 4, "retained");
+  acceptedCount_ = shared(maxLanes * 4, "accepted");
+  retainedRows_ = shared(maxLanes * 4, "retained rows");
+  pageTable_ = device(uint64_t{pageTableEntries} * 8, "page table");
+  // One allocation holds every layer's pool, layerBytes_ apart, so one dispatch commits them all.
+  layerBytes_ = pageBytes_ * physicalPages;
+  kvAll_ = device(layerBytes_ * d.layers, "kv pools");
+  kvPools_.reserve(d.layers);
+  for (uint32_t l = 0; l < d.layers; ++l) kvPools_.push_back(backend.view(kvAll_, layerBytes_ * l, layerBytes_));
+  // Scratch of every projection of the step at its most rows.
+  ops::LinearScratchSize size;
+  for (ops::LinearMatrix m : {ops::LinearMatrix{d.qkvWidth(), d.hidden}, ops::LinearMatrix{d.hidden, d.attentionWidth()},
+                              ops::LinearMatrix{d.ffn, d.hidden}, ops::LinearMatrix{d.hidden, d.ffn},
+                              ops::LinearMatrix{d.vocabulary, d.hidden}})
+    size.include(linear_.scratchSize(m, maxRows_));
+  scratch_.input = device(size.input, "linear table");
+  scratch_.partials = device(size.partials, "linear partials");
+  scratch_.counters = device(std::max<uint64_t>(size.counters, 4), "linear counters");
+  // Attention workspace for the most splits any sequence may take.
+  const uint64_t fused = uint64_t{maxLanes} * d.kvHeads * (d.qHeads / d.kvHeads) * 16;
+  maxSplits_ = ATTENTION_MAXIMUM_SPLITS;
+  attentionWorkspace_.queries = device(fused * d.headDimension * 2, "staged queries");
+  attentionWorkspace_.querySums = device(fused * 4, "query sums");
+  attentionWorkspace_.partials = device(fused * maxSplits_ * d.headDimension * 4, "attention partials");
+  attentionWorkspace_.partialSums = device(fused * maxSplits_ * 8, "attention partial sums");
+  const ops::SamplingWorkspaceSize s = ops::Sampling::workspace(maxRows_);
+  sampling_.logits = logits_;
+  sampling_.tokens = tokens_;
+  sampling_.partialValues = device(s.partialValues, "argmax values");
+  sampling_.partialIndices = device(s.partialIndices, "argmax indices");
+  sampling_.masses = device(s.masses, "sampling masses");
+  sampling_.ranges = device(s.ranges, "sampling ranges");
+  sampling_.decisions = device(s.decisions, "sampling decisions");
+  sampling_.uniforms = uniforms_;
+  sampling_.inputTokens = inputTokens_;
+  sampling_.treeRows = treeRows_;
+}
+
+const hip::Buffer &DenseVerify::draftProbabilities() {
+  if (!draft_) {
+    draft_ = backend_.allocateBuffer(uint64_t{maxRows_} * dims_.vocabulary * 4, BufferStorage::Private, "draft probabilities");
+    sampling_.draftProbabilities = draft_;
+  }
+  return draft_;
+}
+
+uint64_t DenseVerify::stepBytes(const std::vector<VerifyLane> &lanes) const {
+  uint64_t bytes = weights_.head.weightBytes();
+  for (const DenseLayer &l : weights_.layers)
+    bytes += l.qkv.weightBytes() + l.output.weightBytes() + l.gate.weightBytes() + l.up.weightBytes() + l.down.weightBytes();
+  uint32_t rows = 0;
+  for (const VerifyLane &lane : lanes) {
+    bytes += uint64_t{dims_.layers} * (uint64_t{lane.committed} + lane.rows) * (pageBytes_ / ATTENTION_PAGE_TOKENS);
+    rows += lane.rows;
+  }
+  return bytes + 2ull * rows * dims_.vocabulary * 4;  // logits written, then read by acceptance
+}
+
+void DenseVerify::encodeEmbedding(hip::CommandGraph &graph, uint32_t rows) {
+  ops::Embedding::add(graph, weights_.embedding, inputTokens_, hidden_[0], rows);
+}
+
+void DenseVerify::encodeLayer(hip::CommandGraph &graph, uint32_t layer, const ops::AttentionPlan &plan, uint32_t rows) {
+  const DenseLayer &w = weights_.layers.at(layer);
+  const hip::Buffer &residual = hidden_[0], &next = hidden_[1];
+  // Attention block: hidden[1] = hidden[0] + o(attention(qkv(norm(hidden[0])))).
+  ops::PreparedInput prepared = ops::Normalization::addRmsTable(graph, residual, w.inputNorm, normalized_, scratch_, dims_.hidden, rows);
+  ops::LinearBuffers qkv;
+  qkv.input = normalized_;
+  qkv.output = qkv_;
+  qkv.scratch = scratch_;
+  qkv.prepared = prepared;
+  linear_.add(graph, qkv, w.qkv, linear_.plan(w.qkv, rows));
+  const ops::KvPages pages{pageTable_, kvPools_.at(layer), pageBytes_};
+  ops::AttentionProjectionBuffers projection{qkv_, w.queryNorm, w.keyNorm, ropeCos_, ropeSin_};
+  ops::PagedAttention::addProjection(graph, plan, projection, attentionWorkspace_, pages);
+  ops::PagedAttention::addAttention(graph, plan, attentionWorkspace_, treeRows_, pages, attention_);
+  linear_.addResidualProjection(graph, attention_, w.output, residual, next, rows, scratch_);
+  // FFN block: hidden[0] = hidden[1] + down(silu(gate n) * up n), n = norm(hidden[1]).
+  prepared = ops::Normalization::addRmsTable(graph, next, w.postNorm, normalized_, scratch_, dims_.hidden, rows);
+  const ops::FfnBuffers ffn{normalized_, intermediate_, scratch_};
+  linear_.addSwiGlu(graph, {&w.gate, &w.up, &w.down}, ffn, next, residual, rows, prepared);
+}
+
+void DenseVerify::encodeHead(hip::CommandGraph &graph, uint32_t rows) {
+  const ops::PreparedInput prepared =
+      ops::Normalization::addRmsTable(graph, hidden_[0], weights_.finalNorm, normalized_, scratch_, dims_.hidden, rows);
+  ops::LinearBuffers head;
+  head.input = normalized_;
+  head.output = logits_;
+  head.scratch = scratch_;
+  head.prepared = prepared;
+  linear_.add(graph, head, weights_.head, linear_.plan(weights_.head, rows));
+}
+
+void DenseVerify::encode(hip::CommandGraph &graph, const std::vector<VerifyLane> &lanes, bool commit) {
+  if (lanes.empty() || lanes.size() > maxLanes_) throw std::invalid_argument("the step takes 1 to its most lanes");
+  std::vector<ops::AttentionRows> sequences;
+  std::vector<ops::LaneRows> laneRows;
+  std::vector<ops::RopeSequence> rope;
+  std::vector<ops::SamplingPolicy> policies;
+  std::vector<uint32_t> remaining;
+  uint32_t rows = 0;
+  bool samples = false;
+  for (const VerifyLane &lane : lanes) {
+    sequences.push_back({rows, lane.rows, lane.committed, lane.tableFirst});
+    laneRows.push_back({rows, lane.rows});
+    rope.push_back({rows, lane.rows, lane.committed});
+    policies.push_back(lane.policy);
+    remaining.push_back(lane.remaining);
+    samples = samples || lane.policy.samples();
+    rows += lane.rows;
+  }
+  const ops::AttentionGeometry geometry{dims_.qHeads, dims_.kvHeads, dims_.headDimension, dims_.rotaryPairs, dims_.normalizeHeads};
+  const ops::AttentionPlan plan = ops::PagedAttention::plan(geometry, sequences);
+  if (samples) (void)draftProbabilities();
+  if (dims_.rotaryPairs)
+    ops::RoPE::addTreeTables(graph, inverseFrequency_, depths_, ropeCos_, ropeSin_, dims_.rotaryPairs, rope);
+  encodeEmbedding(graph, rows);
+  for (uint32_t layer = 0; layer < dims_.layers; ++layer) encodeLayer(graph, layer, plan, rows);
+  encodeHead(graph, rows);
+  ops::Sampling::addVerify(graph, sampling_, dims_.vocabulary, dims_.vocabulary, laneRows, policies);
+  const ops::AcceptanceBuffers acceptance{inputTokens_, treeRows_, tokens_, retained_, acceptedCount_, retainedRows_};
+  ops::Sampling::addAcceptance(graph, acceptance, laneRows, remaining,
+                               {SAMPLING_NO_TOKEN, SAMPLING_NO_TOKEN, SAMPLING_NO_TOKEN, SAMPLING_NO_TOKEN});
+  if (commit)
+    ops::PagedAttention::addPathCommit(graph, plan, retainedRows_, {pageTable_, kvAll_, pageBytes_}, dims_.layers, layerBytes_);
+}
+
+} // namespace splash::model

@@ -1,0 +1,104 @@
+// The target part of one speculative-decoding cycle for a dense decoder: embedding -> N x
+// {RMSNorm -> fused q|k|v -> q/k norm + RoPE + INT8 KV store -> paged attention -> o-proj + residual
+// -> RMSNorm -> one-pass gate/up SwiGLU -> down + residual} -> final norm -> LM head (fp32 logits)
+// -> verify (argmax or rejection sampling) -> acceptance -> KV path commit. It strings the operators
+// together as the reference's model layer does (runtime/model/QwenTarget.cpp:206-395, :457-496 layer
+// recipe; Runtime.cpp:2677-2717 encodeTargetDecodeForward, :2883-2892 encodeVerifyCommit) and owns
+// the step's buffers; the residual stream ping-pongs between two hidden buffers.
+#pragma once
+#include "hip/Backend.hpp"
+#include "ops/Glue.hpp"
+#include "ops/Linear.hpp"
+#include "ops/PagedAttention.hpp"
+#include "ops/Sampling.hpp"
+
+#include <array>
+#include <cstdint>
+#include <vector>
+
+namespace splash::model {
+
+struct DenseDimensions final {
+  uint32_t hidden = 0, qHeads = 0, kvHeads = 0, headDimension = 0, ffn = 0, vocabulary = 0, layers = 0;
+  uint32_t rotaryPairs = 0;
+  bool normalizeHeads = true;   // per-head q/k RMS norm
+  float ropeTheta = 1000000.0f;
+  [[nodiscard]] uint32_t qkvWidth() const noexcept { return (qHeads + 2 * kvHeads) * headDimension; }
+  [[nodiscard]] uint32_t attentionWidth() const noexcept { return qHeads * headDimension; }
+};
+
+struct DenseLayer final {
+  ops::Projection qkv, output, gate, up, down;
+  hip::Buffer inputNorm, postNorm, queryNorm, keyNorm;  // bf16 weights
+};
+
+struct DenseWeights final {
+  ops::EmbeddingTable embedding;
+  std::vector<DenseLayer> layers;
+  hip::Buffer finalNorm;
+  ops::Projection head;  // destination Float32
+};
+
+// One lane (request) of a step.
+struct VerifyLane final {
+  uint32_t rows = 0;        // rows of its verify block
+  uint32_t committed = 0;   // tokens cached before the block
+  uint32_t tableFirst = 0;  // its first page-table entry
+  ops::SamplingPolicy policy;
+  uint32_t remaining = 0xFFFFFFFFu;
+};
+
+class DenseVerify final {
+public:
+  // maxLanes x 16 rows at most; the KV pool holds `physicalPages` pages per layer.
+  DenseVerify(hip::Backend &backend, DenseDimensions dimensions, uint32_t maxLanes, uint32_t physicalPages,
+              uint32_t pageTableEntries);
+
+  [[nodiscard]] const DenseDimensions &dimensions() const noexcept { return dims_; }
+  DenseWeights &weights() noexcept { return weights_; }
+  // Host-visible step inputs and results (Shared storage).
+  [[nodiscard]] const hip::Buffer &inputTokens() const noexcept { return inputTokens_; }
+  [[nodiscard]] const hip::Buffer &treeRows() const noexcept { return treeRows_; }
+  [[nodiscard]] const hip::Buffer &depths() const noexcept { return depths_; }
+  [[nodiscard]] const hip::Buffer &uniforms() const noexcept { return uniforms_; }
+  [[nodiscard]] const hip::Buffer &tokens() const noexcept { return tokens_; }
+  [[nodiscard]] const hip::Buffer &retained() const noexcept { return retained_; }
+  [[nodiscard]] const hip::Buffer &acceptedCount() const noexcept { return acceptedCount_; }
+  [[nodiscard]] const hip::Buffer &retainedRows() const noexcept { return retainedRows_; }
+  // Device buffers a host fills or inspects.
+  [[nodiscard]] const hip::Buffer &pageTable() const noexcept { return pageTable_; }
+  [[nodiscard]] const hip::Buffer &kvPool(uint32_t layer) const { return kvPools_.at(layer); }
+  [[nodiscard]] const hip::Buffer &logits() const noexcept { return logits_; }
+  [[nodiscard]] const hip::Buffer &draftProbabilities();  // allocated on first use
+  [[nodiscard]] const hip::Buffer &hidden(uint32_t index) const noexcept { return hidden_[index & 1]; }
+  [[nodiscard]] uint64_t pageBytes() const noexcept { return pageBytes_; }
+  // Algorithmic bytes one step of `lanes` streams from HBM: weights once, each lane's KV, logits.
+  [[nodiscard]] uint64_t stepBytes(const std::vector<VerifyLane> &lanes) const;
+
+  // Appends the whole target part of a cycle to `graph`. `commit` adds the KV path commit.
+  void encode(hip::CommandGraph &graph, const std::vector<VerifyLane> &lanes, bool commit = true);
+  // Its parts, for per-kernel timing and tests.
+  void encodeEmbedding(hip::CommandGraph &graph, uint32_t rows);
+  void encodeLayer(hip::CommandGraph &graph, uint32_t layer, const ops::AttentionPlan &plan, uint32_t rows);
+  void encodeHead(hip::CommandGraph &graph, uint32_t rows);
+
+private:
+  hip::Backend &backend_;
+  DenseDimensions dims_;
+  DenseWeights weights_;
+  ops::Linear linear_;
+  uint32_t maxRows_ = 0, maxLanes_ = 0;
+  uint64_t pageBytes_ = 0, layerBytes_ = 0;
+  hip::Buffer kvAll_;
+  hip::Buffer hidden_[2], normalized_, qkv_, attention_, intermediate_, logits_, draft_;
+  hip::Buffer inverseFrequency_, ropeCos_, ropeSin_;
+  hip::Buffer inputTokens_, treeRows_, depths_, uniforms_, tokens_, retained_, acceptedCount_, retainedRows_;
+  hip::Buffer pageTable_;
+  std::vector<hip::Buffer> kvPools_;
+  ops::LinearScratch scratch_;
+  ops::AttentionWorkspace attentionWorkspace_;
+  ops::SamplingBuffers sampling_;
+  uint32_t maxSplits_ = 0;
+};
+
+} // namespace splash::model

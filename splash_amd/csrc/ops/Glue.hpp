@@ -1,0 +1,49 @@
+// Glue operators of the verify path: ops::Normalization (runtime/ops/Normalization.cpp:16-40),
+// ops::Embedding (runtime/ops/Embedding.cpp:20-47) and ops::RoPE (runtime/ops/RoPE.hpp:33-37) of the
+// reference, over kernels/glue.hip. Each validates its buffers and throws std::invalid_argument
+// before it adds a dispatch.
+#pragma once
+#include "abi/Glue.h"
+#include "hip/Backend.hpp"
+#include "ops/Linear.hpp"
+
+#include <vector>
+
+namespace splash::ops {
+
+class Normalization final {
+public:
+  // output = bf16((x * rsqrt(mean x^2 + 1e-6)) * weight) over `rows` rows of `width`.
+  static void addRms(hip::CommandGraph &graph, const hip::Buffer &input, const hip::Buffer &weight, const hip::Buffer &output,
+                     uint32_t width, uint32_t rows);
+  // The same, and the projection activation table of the normalized rows in scratch.input; returns
+  // what the table then describes (the reference's norm_rms_table16_decode producer).
+  static PreparedInput addRmsTable(hip::CommandGraph &graph, const hip::Buffer &input, const hip::Buffer &weight,
+                                   const hip::Buffer &output, const LinearScratch &scratch, uint32_t width, uint32_t rows);
+};
+
+// A token table's rows as stored: native K-quant blocks, gathered, never multiplied (Weights.hpp:227-260).
+struct EmbeddingTable final {
+  hip::Buffer rows;
+  uint32_t formatId = GGUF_FMT_Q4K;
+  uint32_t vocabulary = 0;
+  uint32_t hidden = 0;
+};
+class Embedding final {
+public:
+  static void add(hip::CommandGraph &graph, const EmbeddingTable &table, const hip::Buffer &tokens, const hip::Buffer &output,
+                  uint32_t rows);
+};
+
+struct RopeSequence final {
+  uint32_t firstRow = 0, rows = 0, anchor = 0;
+};
+class RoPE final {
+public:
+  // cos/sin of (anchor + depth[row]) * inverseFrequency[pair] per packed row.
+  static void addTreeTables(hip::CommandGraph &graph, const hip::Buffer &inverseFrequency, const hip::Buffer &depth,
+                            const hip::Buffer &cosines, const hip::Buffer &sines, uint32_t pairs,
+                            const std::vector<RopeSequence> &sequences);
+};
+
+} // namespace splash::ops

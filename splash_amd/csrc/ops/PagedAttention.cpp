@@ -132,19 +132,23 @@ void PagedAttention::addAttention(hip::CommandGraph &graph, const AttentionPlan 
 }
 
 void PagedAttention::addPathCommit(hip::CommandGraph &graph, const AttentionPlan &plan, const hip::Buffer &retained,
-                                   const KvPages &pages) {
+                                   const KvPages &pages, uint32_t layers, uint64_t layerBytes) {
   const AttentionGeometry &g = plan.geometry();
   requireBytes(retained, plan.sequences().size() * 4, "retained rows");
   requirePages(plan, pages);
+  if (!layers || (layers > 1 && (layerBytes < pages.pageBytes || pages.pool.sizeBytes() < layerBytes * layers)))
+    throw std::invalid_argument("KV pool buffer does not hold the layers' pools");
   const AttentionParams full = plan.params(pages.pageBytes);
   AttentionCommitParams params{};
   params.kv_heads = g.kvHeads;
   params.head_dim = g.headDimension;
   params.sequences = full.sequences;
+  params.layers = layers;
   params.page_bytes = pages.pageBytes;
+  params.layer_bytes = layerBytes;
   for (uint32_t i = 0; i < full.sequences; ++i) params.sequence[i] = full.sequence[i];
   graph.add("attention_q8_commit" + kernelSuffix(g), {retained, pages.pageTable, pages.pool}, params,
-            {g.kvHeads, plan.sequences().size(), 1}, {g.headDimension, 1, 1});
+            {g.kvHeads, plan.sequences().size(), layers}, {g.headDimension, 1, 1});
 }
 
 } // namespace splash::ops

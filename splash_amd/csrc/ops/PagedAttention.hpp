@@ -99,8 +99,10 @@ public:
                            const hip::Buffer &treeRows, const KvPages &pages, const hip::Buffer &output);
   // Moves the retained path's slots to their depths (PagedAttention.cpp:647-667); retained is a
   // uint32 mask per sequence.
+  // `layers` pools lie layerBytes apart from pages.pool (one dispatch commits them all, as the
+  // reference's grid of layers x KV heads does).
   static void addPathCommit(hip::CommandGraph &graph, const AttentionPlan &plan, const hip::Buffer &retained,
-                            const KvPages &pages);
+                            const KvPages &pages, uint32_t layers = 1, uint64_t layerBytes = 0);
 };
 
 } // namespace splash::ops

@@ -1,0 +1,95 @@
+#include "ops/Sampling.hpp"
+#include "abi/PagedAttention.h"
+#include "ops/Linear.hpp"  // requireBytes
+
+#include <algorithm>
+#include <stdexcept>
+
+namespace splash::ops {
+
+namespace {
+uint32_t packedRows(const std::vector<LaneRows> &lanes) {
+  if (lanes.empty() || lanes.size() > SAMPLING_MAXIMUM_LANES) throw std::invalid_argument("acceptance takes 1 to 8 lanes");
+  uint32_t rows = 0;
+  for (const LaneRows &l : lanes) {
+    if (!l.rows || l.rows > SAMPLING_MAXIMUM_ROWS) throw std::invalid_argument("a lane's verify block holds 1 to 16 rows");
+    rows = std::max(rows, l.first + l.rows);
+  }
+  return rows;
+}
+} // namespace
+
+SamplingWorkspaceSize Sampling::workspace(uint32_t rows) noexcept {
+  SamplingWorkspaceSize size;
+  size.partialValues = uint64_t{rows} * SAMPLING_SHARDS * 4;
+  size.partialIndices = uint64_t{rows} * SAMPLING_SHARDS * 4;
+  size.masses = uint64_t{rows} * SAMPLING_SHARDS * 8;
+  size.ranges = uint64_t{rows} * SAMPLING_RANGES * 4;
+  size.decisions = uint64_t{rows} * 8;
+  return size;
+}
+
+void Sampling::addVerify(hip::CommandGraph &graph, const SamplingBuffers &b, uint32_t vocabulary, uint32_t logitsStride,
+                         const std::vector<LaneRows> &lanes, const std::vector<SamplingPolicy> &policies) {
+  const uint32_t rows = packedRows(lanes);
+  if (policies.size() != lanes.size()) throw std::invalid_argument("acceptance takes one policy per lane");
+  if (!vocabulary || logitsStride < vocabulary) throw std::invalid_argument("logits rows hold the vocabulary");
+  TargetSamplingParams params{};
+  params.vocabulary = vocabulary;
+  params.rows = rows;
+  params.lanes = uint32_t(lanes.size());
+  params.logits_stride = logitsStride;
+  for (size_t l = 0; l < lanes.size(); ++l) {
+    params.lane[l] = {lanes[l].first, lanes[l].rows};
+    params.temperature[l] = policies[l].samples() ? policies[l].temperature : 1.0f;
+    if (policies[l].samples()) params.sampling_mask |= 1u << l;
+  }
+  const SamplingWorkspaceSize need = workspace(rows);
+  requireBytes(b.logits, (uint64_t{rows - 1} * logitsStride + vocabulary) * 4, "logits");
+  requireBytes(b.tokens, uint64_t{rows} * 4, "selected tokens");
+  requireBytes(b.partialValues, need.partialValues, "argmax partial values");
+  requireBytes(b.partialIndices, need.partialIndices, "argmax partial indices");
+  if (params.sampling_mask) {
+    requireBytes(b.draftProbabilities, (uint64_t{rows - 1} * logitsStride + vocabulary) * 4, "draft probabilities");
+    requireBytes(b.uniforms, uint64_t{rows} * 8, "sampling uniforms");
+    requireBytes(b.masses, need.masses, "sampling masses");
+    requireBytes(b.ranges, need.ranges, "sampling ranges");
+    requireBytes(b.decisions, need.decisions, "sampling decisions");
+    requireBytes(b.inputTokens, uint64_t{rows} * 4, "input tokens");
+    requireBytes(b.treeRows, uint64_t{rows} * sizeof(AttentionTreeRow), "verify tree rows");
+  }
+  // Every row gets its argmax; the sampled lanes' rows are then overwritten by their draw.
+  graph.add("decode_sample_argmax_sharded", {b.logits, b.partialValues, b.partialIndices}, params, {rows * SAMPLING_SHARDS, 1, 1},
+            {SAMPLING_THREADS, 1, 1});
+  graph.add("decode_sample_argmax_reduce", {b.partialValues, b.partialIndices, b.tokens}, params, {rows, 1, 1}, {64, 1, 1});
+  if (!params.sampling_mask) return;
+  graph.add("decode_sample_mass_sharded", {b.logits, b.masses}, params, {rows * SAMPLING_SHARDS, 1, 1}, {SAMPLING_THREADS, 1, 1});
+  graph.add("decode_sample_residual_ranges",
+            {b.logits, b.draftProbabilities, b.masses, b.uniforms, b.treeRows, b.inputTokens, b.ranges, b.decisions}, params,
+            {rows * (SAMPLING_RANGES / 4), 1, 1}, {256, 1, 1});
+  graph.add("decode_sample_draw", {b.logits, b.draftProbabilities, b.masses, b.uniforms, b.ranges, b.decisions, b.tokens}, params,
+            {rows, 1, 1}, {64, 1, 1});
+}
+
+void Sampling::addAcceptance(hip::CommandGraph &graph, const AcceptanceBuffers &b, const std::vector<LaneRows> &lanes,
+                             const std::vector<uint32_t> &remaining, const std::array<uint32_t, SAMPLING_STOP_TOKENS> &stopTokens) {
+  const uint32_t rows = packedRows(lanes);
+  if (remaining.size() != lanes.size()) throw std::invalid_argument("acceptance takes one remaining count per lane");
+  AcceptBatchParams params{};
+  params.lanes = uint32_t(lanes.size());
+  for (size_t l = 0; l < lanes.size(); ++l) {
+    params.lane[l] = {lanes[l].first, lanes[l].rows};
+    params.remaining[l] = remaining[l];
+  }
+  for (size_t s = 0; s < stopTokens.size(); ++s) params.stop_tokens[s] = stopTokens[s];
+  requireBytes(b.inputTokens, uint64_t{rows} * 4, "input tokens");
+  requireBytes(b.treeRows, uint64_t{rows} * sizeof(AttentionTreeRow), "verify tree rows");
+  requireBytes(b.tokens, uint64_t{rows} * 4, "selected tokens");
+  requireBytes(b.retained, lanes.size() * 4, "retained counts");
+  requireBytes(b.acceptedCount, lanes.size() * 4, "accepted counts");
+  requireBytes(b.retainedRows, lanes.size() * 4, "retained rows");
+  graph.add("decode_accept_tree", {b.inputTokens, b.treeRows, b.tokens, b.retained, b.acceptedCount, b.retainedRows}, params,
+            {lanes.size(), 1, 1}, {64, 1, 1});
+}
+
+} // namespace splash::ops

@@ -1,0 +1,57 @@
+// Acceptance of a verify block: ops::Sampling (runtime/ops/Sampling.hpp:64-254, Sampling.cpp:283-357
+// in the reference) over kernels/sampling.hip. addVerify selects each row's token (argmax, or
+// rejection sampling over the row's drafted child at temperature > 0); addAcceptance walks each
+// lane's block from its first row and writes the retained tokens, counts and retained-row mask.
+#pragma once
+#include "abi/Sampling.h"
+#include "hip/Backend.hpp"
+
+#include <array>
+#include <vector>
+
+namespace splash::ops {
+
+// Sampling.hpp:64-110 in the reference, reduced to what the verify configurations use.
+struct SamplingPolicy final {
+  float temperature = 0.0f;
+  // Sampling.cpp:78-89: a policy samples iff temperature > 0.
+  [[nodiscard]] bool samples() const noexcept { return temperature > 0.0f; }
+};
+
+struct LaneRows final {
+  uint32_t first = 0, rows = 0;
+};
+
+struct SamplingWorkspaceSize final {
+  uint64_t partialValues = 0, partialIndices = 0, masses = 0, ranges = 0, decisions = 0;
+};
+struct SamplingBuffers final {
+  hip::Buffer logits;         // fp32 [rows][stride]
+  hip::Buffer tokens;         // uint32 [rows]: each row's selection
+  hip::Buffer partialValues, partialIndices;  // greedy shards
+  // sampled rows only:
+  hip::Buffer draftProbabilities;  // fp32 [rows][stride]: the distribution each row's child was drawn from
+  hip::Buffer uniforms;            // fp32 [rows][2]: the row's draw, its child's test
+  hip::Buffer masses, ranges, decisions;
+  hip::Buffer inputTokens, treeRows;  // the block's input tokens and SplashTreeRow rows
+};
+struct AcceptanceBuffers final {
+  hip::Buffer inputTokens;    // uint32 [rows]
+  hip::Buffer treeRows;       // AttentionTreeRow [rows]
+  hip::Buffer tokens;         // in: selections; out: each lane's retained tokens from its first row
+  hip::Buffer retained;       // uint32 [lanes]: retained token count
+  hip::Buffer acceptedCount;  // uint32 [lanes]
+  hip::Buffer retainedRows;   // uint32 [lanes]: mask of the block rows retained
+};
+
+class Sampling final {
+public:
+  [[nodiscard]] static SamplingWorkspaceSize workspace(uint32_t rows) noexcept;
+  // One policy per lane. Throws for no or too many lanes, rows outside 1..16, or missing buffers.
+  static void addVerify(hip::CommandGraph &graph, const SamplingBuffers &buffers, uint32_t vocabulary, uint32_t logitsStride,
+                        const std::vector<LaneRows> &lanes, const std::vector<SamplingPolicy> &policies);
+  static void addAcceptance(hip::CommandGraph &graph, const AcceptanceBuffers &buffers, const std::vector<LaneRows> &lanes,
+                            const std::vector<uint32_t> &remaining, const std::array<uint32_t, SAMPLING_STOP_TOKENS> &stopTokens);
+};
+
+} // namespace splash::ops

@@ -266,3 +266,67 @@ def chain_tree_rows(rows_per_sequence):
     for i, (a, p, d) in enumerate(out):
         arr[i] = (a, p, d)
     return arr
+
+
+# ---------------------------------------------------------------------------------------------
+# Normalization, Embedding, RoPE, Sampling
+# ---------------------------------------------------------------------------------------------
+class Normalization:
+    @staticmethod
+    def add_rms(graph, input, weight, output, width, rows):
+        check(lib.spo_norm_add_rms(graph.handle, input.handle, weight.handle, output.handle, width, rows))
+        graph._keep.extend([input, weight, output])
+
+    @staticmethod
+    def add_rms_table(graph, input, weight, output, table, width, rows):
+        check(lib.spo_norm_add_rms_table(graph.handle, input.handle, weight.handle, output.handle, table.handle, width, rows))
+        graph._keep.extend([input, weight, output, table])
+
+
+class Embedding:
+    @staticmethod
+    def add(graph, fmt, native_rows, vocabulary, hidden, tokens, output, rows):
+        check(lib.spo_embedding_add(graph.handle, fmt, native_rows.handle, vocabulary, hidden, tokens.handle, output.handle, rows))
+        graph._keep.extend([native_rows, tokens, output])
+
+
+class RoPE:
+    @staticmethod
+    def add_tree_tables(graph, inverse_frequency, depth, cosines, sines, pairs, sequences):
+        """sequences: [(first_row, rows, anchor)]"""
+        arr = (nat.RopeSequence * len(sequences))(*[nat.RopeSequence(*s) for s in sequences])
+        check(lib.spo_rope_add_tree_tables(graph.handle, inverse_frequency.handle, depth.handle, cosines.handle, sines.handle,
+                                           pairs, arr, len(sequences)))
+        graph._keep.extend([inverse_frequency, depth, cosines, sines])
+
+
+NO_TOKEN = 0xFFFFFFFF
+
+
+class Sampling:
+    """ops::Sampling: addVerify (argmax or rejection sampling per row), addAcceptance (tree walk)."""
+
+    @staticmethod
+    def workspace(rows):
+        sizes = (ctypes.c_uint64 * 5)()
+        check(lib.spo_sampling_workspace(rows, sizes))
+        return list(sizes)
+
+    @staticmethod
+    def add_verify(graph, buffers, vocabulary, stride, lanes, temperatures):
+        """buffers: dict of Buffer by the names of spo_sampling_buffers; lanes: [(first, rows)]."""
+        b = nat.SamplingBuffers(**{k: (v.handle if v is not None else None) for k, v in buffers.items()})
+        arr = (nat.LaneRows * len(lanes))(*[nat.LaneRows(*l) for l in lanes])
+        temps = (ctypes.c_float * len(lanes))(*temperatures)
+        check(lib.spo_sampling_add_verify(graph.handle, ctypes.byref(b), vocabulary, stride, arr, temps, len(lanes)))
+        graph._keep.extend(list(buffers.values()))
+
+    @staticmethod
+    def add_acceptance(graph, input_tokens, tree_rows, tokens, retained, accepted, retained_rows, lanes, remaining,
+                       stop_tokens=(NO_TOKEN,) * 4):
+        arr = (nat.LaneRows * len(lanes))(*[nat.LaneRows(*l) for l in lanes])
+        rem = (ctypes.c_uint32 * len(lanes))(*remaining)
+        stops = (ctypes.c_uint32 * 4)(*stop_tokens)
+        check(lib.spo_sampling_add_acceptance(graph.handle, input_tokens.handle, tree_rows.handle, tokens.handle, retained.handle,
+                                              accepted.handle, retained_rows.handle, arr, rem, len(lanes), stops))
+        graph._keep.extend([input_tokens, tree_rows, tokens, retained, accepted, retained_rows])

@@ -187,3 +187,49 @@ def attention(q_bits, kcodes, kscales, vcodes, vscales, page_table, ancestors, c
     lib.orc_attention(ctypes.byref(a), _p(q_bits, u16p), _p(kcodes, i8p), _p(kscales, f32p), _p(vcodes, i8p), _p(vscales, f32p),
                       _p(pt, u32p), _p(anc, u32p), _p(out, u16p), _p(out64, f64p), c_int(threads))
     return out, out64
+
+
+class OrcTreeRow(ctypes.Structure):
+    _fields_ = [("ancestors", c_u32), ("parent", ctypes.c_uint16), ("depth", ctypes.c_uint16)]
+
+
+lib.orc_argmax.restype = c_u32
+
+
+def argmax(logits):
+    x = np.ascontiguousarray(logits, dtype=np.float32)
+    return lib.orc_argmax(_p(x, f32p), c_u32(x.size))
+
+
+def accept_tree(tree, tokens, selected, remaining=0xFFFFFFFF, stop_tokens=()):
+    """tree: structured array (ancestors, parent, depth). Returns (kept tokens, accepted, retained_rows)."""
+    rows = len(tree)
+    nodes = (OrcTreeRow * rows)(*[OrcTreeRow(int(t["ancestors"]), int(t["parent"]), int(t["depth"])) for t in tree])
+    tok = np.ascontiguousarray(tokens, dtype=np.uint32)
+    sel = np.ascontiguousarray(selected, dtype=np.uint32)
+    stops = np.ascontiguousarray(list(stop_tokens) or [NO_TOKEN], dtype=np.uint32)
+    out = np.zeros(rows, dtype=np.uint32)
+    acc, ret = c_u32(), c_u32()
+    lib.orc_accept_tree.restype = c_u32
+    kept = lib.orc_accept_tree(nodes, _p(tok, u32p), _p(sel, u32p), c_u32(rows), c_u32(remaining), _p(stops, u32p), c_u32(len(stops)),
+                               _p(out, u32p), ctypes.byref(acc), ctypes.byref(ret))
+    return out[:kept].copy(), acc.value, ret.value
+
+
+def rejection_row(logits, temperature, q, draft_token, u_child, u_row):
+    """Returns (token, accepted_draft, closeness)."""
+    x = np.ascontiguousarray(logits, dtype=np.float32)
+    qq = np.ascontiguousarray(q, dtype=np.float32) if q is not None else None
+    acc, close = c_int(), ctypes.c_double()
+    lib.orc_rejection_row.restype = c_u32
+    tok = lib.orc_rejection_row(_p(x, f32p), c_u32(x.size), c_f(temperature), _p(qq, f32p), c_u32(draft_token), c_f(u_child),
+                                c_f(u_row), ctypes.byref(acc), ctypes.byref(close))
+    return tok, bool(acc.value), close.value
+
+
+def rejection_law(logits, temperature, q):
+    x = np.ascontiguousarray(logits, dtype=np.float32)
+    qq = np.ascontiguousarray(q, dtype=np.float32)
+    out = np.empty(x.size, dtype=np.float64)
+    lib.orc_rejection_law(_p(x, f32p), c_u32(x.size), c_f(temperature), _p(qq, f32p), _p(out, f64p))
+    return out

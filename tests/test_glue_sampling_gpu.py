@@ -1,0 +1,173 @@
+"""GPU parity of the glue kernels and the acceptance kernels against the oracle, through the C ABI."""
+import numpy as np
+import pytest
+
+import splash_amd
+from splash_amd import ops
+from tests import oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("rows,width", [(1, 1024), (16, 5120), (33, 2048)])
+def test_rms_norm_and_its_activation_table(backend, rows, width):
+    """normalization.metal:59-99; the fused table equals gguf_prepare_table of the normalized rows bit for bit."""
+    print(f"case norm rows={rows} width={width}", flush=True)
+    rng = np.random.default_rng(rows)
+    x = orc.f32_to_bf16((rng.standard_normal((rows, width)) * 3).astype(np.float32))
+    w = orc.f32_to_bf16((1 + 0.2 * rng.standard_normal(width)).astype(np.float32))
+    xb, wb = backend.from_array(x), backend.from_array(w)
+    plain, fused = backend.allocate_buffer(rows * width * 2), backend.allocate_buffer(rows * width * 2)
+    nbytes = ops.gguf_table_bytes(width, rows)
+    table, table2 = backend.allocate_buffer(nbytes), backend.allocate_buffer(nbytes)
+    g = splash_amd.CommandGraph()
+    ops.Normalization.add_rms(g, xb, wb, plain, width, rows)
+    ops.Normalization.add_rms_table(g, xb, wb, fused, table, width, rows)
+    import ctypes
+
+    class Prepare(ctypes.Structure):
+        _fields_ = [("input_size", ctypes.c_uint32), ("rows", ctypes.c_uint32), ("tiles", ctypes.c_uint32), ("row_stride", ctypes.c_uint32)]
+    tiles = (rows + 15) // 16
+    g.add("gguf_prepare_table", [plain, table2], Prepare(width, rows, tiles, width), (width // 32, tiles, 1), (64, 1, 1))
+    backend.run(g)
+    got = plain.download(np.uint16).reshape(rows, width)
+    want = orc.rms_norm(x, w)
+    assert np.array_equal(fused.download(np.uint16).reshape(rows, width), got)
+    # the reduction tree of a 64-lane wavefront differs from the oracle's 32-lane one: bf16 ulp at most
+    diff = np.abs(got.astype(np.int32) - want.astype(np.int32))
+    assert diff.max() <= 1 and (diff > 0).mean() < 0.01, (diff.max(), (diff > 0).mean())
+    assert np.array_equal(table.download(), table2.download())
+
+
+@pytest.mark.parametrize("fmt", [ops.FMT_Q4K, ops.FMT_Q6K])
+def test_embedding_gathers_native_rows(backend, fmt):
+    """embedding.metal:10-18: bf16(decode(row)); a token past the vocabulary gives zeros."""
+    vocab, hidden = 500, 1024
+    native = orc.make_native(fmt, vocab, hidden, 3)
+    tokens = np.array([0, 499, 17, 500, 4_000_000_000, 17], dtype=np.uint32)
+    out = backend.allocate_buffer(len(tokens) * hidden * 2)
+    g = splash_amd.CommandGraph()
+    ops.Embedding.add(g, fmt, backend.from_array(native), vocab, hidden, backend.from_array(tokens), out, len(tokens))
+    backend.run(g)
+    assert np.array_equal(out.download(np.uint16).reshape(len(tokens), hidden), orc.embed(fmt, native, vocab, hidden, tokens))
+
+
+def test_rope_tree_tables(backend):
+    """rope.metal:51-80: cos/sin of (anchor + depth) * inverse frequency per packed row."""
+    pairs = 64
+    inv = (1e6 ** (-np.arange(pairs) / pairs)).astype(np.float32)
+    depth = np.array([0, 1, 2, 2, 3, 0, 1], dtype=np.uint32)
+    seqs = [(0, 5, 32752), (5, 2, 7)]
+    cos, sin = backend.allocate_buffer(7 * pairs * 4), backend.allocate_buffer(7 * pairs * 4)
+    g = splash_amd.CommandGraph()
+    ops.RoPE.add_tree_tables(g, backend.from_array(inv), backend.from_array(depth), cos, sin, pairs, seqs)
+    backend.run(g)
+    pos = np.array([32752 + d for d in depth[:5]] + [7 + d for d in depth[5:]], dtype=np.float32)
+    angle = (pos[:, None] * inv[None, :]).astype(np.float32).astype(np.float64)
+    assert np.abs(cos.download(np.float32).reshape(7, pairs) - np.cos(angle)).max() < 2e-6
+    assert np.abs(sin.download(np.float32).reshape(7, pairs) - np.sin(angle)).max() < 2e-6
+
+
+def sampling_buffers(backend, rows, V, logits, draft=None, uniforms=None, tokens=None, tree=None):
+    sizes = ops.Sampling.workspace(rows)
+    b = dict(logits=backend.from_array(logits.astype(np.float32)), tokens=backend.allocate_buffer(rows * 4),
+             partial_values=backend.allocate_buffer(sizes[0]), partial_indices=backend.allocate_buffer(sizes[1]),
+             draft_probabilities=backend.from_array(draft.astype(np.float32)) if draft is not None else None,
+             uniforms=backend.from_array(uniforms.astype(np.float32)) if uniforms is not None else None,
+             masses=backend.allocate_buffer(sizes[2]), ranges=backend.allocate_buffer(sizes[3]),
+             decisions=backend.allocate_buffer(sizes[4]),
+             input_tokens=backend.from_array(tokens) if tokens is not None else None,
+             tree_rows=backend.from_array(tree) if tree is not None else None)
+    return b
+
+
+def test_greedy_argmax_ties_sentinel_and_large_vocabulary(backend):
+    """sampling.metal:1896-1997: ties to the lowest id, NaN/-inf skipped, no selectable logit -> sentinel."""
+    print("case argmax", flush=True)
+    rng = np.random.default_rng(5)
+    rows, V = 16, 151936
+    logits = rng.standard_normal((rows, V)).astype(np.float32)
+    logits[1, [7, 90000, 151935]] = 9.0                      # a three-way tie
+    logits[2, :] = -np.inf
+    logits[3, :] = np.nan
+    logits[4, 151935] = 50.0                                 # the last token
+    logits[5, rng.random(V) < 0.5] = np.nan
+    logits[6, :] = 1.0                                       # all equal: id 0
+    b = sampling_buffers(backend, rows, V, logits)
+    g = splash_amd.CommandGraph()
+    ops.Sampling.add_verify(g, b, V, V, [(0, rows)], [0.0])
+    backend.run(g)
+    got = b["tokens"].download(np.uint32)
+    want = np.array([orc.argmax(logits[r]) for r in range(rows)], dtype=np.uint32)
+    assert np.array_equal(got, want)
+    assert got[1] == 7 and got[2] == ops.NO_TOKEN and got[3] == ops.NO_TOKEN and got[4] == 151935 and got[6] == 0
+
+
+def test_acceptance_walk_matches_oracle_on_trees(backend):
+    """sampling.metal:2044-2083 decode_accept_tree over chains and trees, several lanes, caps and stop tokens."""
+    print("case accept tree", flush=True)
+    from tests.test_oracle_sampling import random_tree
+    rng = np.random.default_rng(6)
+    for trial in range(20):
+        lanes, first = [], 0
+        trees, toks, sels = [], [], []
+        for _ in range(int(rng.integers(1, 5))):
+            rows = int(rng.integers(1, 17))
+            lanes.append((first, rows)); first += rows
+            trees.append(random_tree(rng, rows) if trial % 2 else ops.chain_tree_rows([rows]))
+            toks.append(rng.integers(0, 3, rows).astype(np.uint32)); sels.append(rng.integers(0, 3, rows).astype(np.uint32))
+        tree, tokens, selected = np.concatenate(trees), np.concatenate(toks), np.concatenate(sels)
+        remaining = [int(rng.integers(1, 20)) for _ in lanes]
+        stops = (2, ops.NO_TOKEN, ops.NO_TOKEN, ops.NO_TOKEN) if trial % 3 == 0 else (ops.NO_TOKEN,) * 4
+        tb = backend.from_array(selected)
+        ret, acc, mask = (backend.allocate_buffer(len(lanes) * 4) for _ in range(3))
+        g = splash_amd.CommandGraph()
+        ops.Sampling.add_acceptance(g, backend.from_array(tokens), backend.from_array(tree), tb, ret, acc, mask, lanes, remaining, stops)
+        backend.run(g)
+        out, retained, accepted, masks = tb.download(np.uint32), ret.download(np.uint32), acc.download(np.uint32), mask.download(np.uint32)
+        for i, (f, rows) in enumerate(lanes):
+            kept, a, m = orc.accept_tree(tree[f:f + rows], tokens[f:f + rows], selected[f:f + rows], remaining[i],
+                                         [s for s in stops if s != ops.NO_TOKEN])
+            assert retained[i] == len(kept) and accepted[i] == a and masks[i] == m
+            assert np.array_equal(out[f:f + len(kept)], kept)
+
+
+def test_rejection_sampling_rows_match_oracle(backend):
+    """sampling.metal:713-885 at a full-vocabulary draft distribution: the drafted child is accepted iff
+    u q < p, else the row draws from max(p - q, 0); ids equal the oracle's except where a comparison
+    lies within 1e-5 of its threshold (target_sampling_metal_test.mm:2645-2709)."""
+    print("case rejection sampling", flush=True)
+    rng = np.random.default_rng(7)
+    rows, V, T = 16, 32000, 0.7
+    logits = (rng.standard_normal((rows, V)) * 2.5).astype(np.float32)
+    logits[3, rng.random(V) < 0.01] = -np.inf
+    dl = rng.standard_normal((rows, V)) * 2
+    draft = np.exp(dl - dl.max(axis=1, keepdims=True)); draft = (draft / draft.sum(axis=1, keepdims=True)).astype(np.float32)
+    p = np.exp((logits.astype(np.float64) - np.nanmax(np.where(np.isfinite(logits), logits, -1e30), axis=1, keepdims=True)) / T)
+    p = np.where(np.isfinite(logits), p, 0); p /= p.sum(axis=1, keepdims=True)
+    tokens = np.zeros(rows, dtype=np.uint32)
+    for r in range(1, rows):   # row r's token is the child drawn at row r - 1: mix likely-accepted and likely-rejected ones
+        tokens[r] = int(np.argmax(p[r - 1])) if r % 2 else int(rng.choice(V, p=draft[r - 1].astype(np.float64) / draft[r - 1].sum()))
+    uniforms = rng.random((rows, 2)).astype(np.float32)
+    tree = ops.chain_tree_rows([rows])
+    b = sampling_buffers(backend, rows, V, logits, draft, uniforms, tokens, tree)
+    g = splash_amd.CommandGraph()
+    ops.Sampling.add_verify(g, b, V, V, [(0, rows)], [T])
+    backend.run(g)
+    got = b["tokens"].download(np.uint32)
+    checked = accepted_rows = 0
+    for r in range(rows):
+        child = int(tokens[r + 1]) if r + 1 < rows else orc.NO_TOKEN
+        want, accepted, close = orc.rejection_row(logits[r], T, draft[r] if child != orc.NO_TOKEN else None, child,
+                                                  float(uniforms[r, 1]), float(uniforms[r, 0]))
+        if close > 1e-5:
+            assert got[r] == want, (r, got[r], want, accepted)
+            checked += 1
+            accepted_rows += accepted
+    assert checked >= rows - 2 and 0 < accepted_rows < rows
+    # a greedy lane beside a sampled one keeps its argmax
+    g = splash_amd.CommandGraph()
+    ops.Sampling.add_verify(g, b, V, V, [(0, 8), (8, 8)], [0.0, T])
+    backend.run(g)
+    mixed = b["tokens"].download(np.uint32)
+    assert all(mixed[r] == orc.argmax(logits[r]) for r in range(8))

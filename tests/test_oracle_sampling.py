@@ -1,0 +1,127 @@
+"""The oracle's acceptance functions against brute force, the enumerated selection law and statistics (CPU)."""
+import numpy as np
+import pytest
+
+from tests import oracle as orc
+
+
+def test_argmax_brute_force_ties_and_unselectable():
+    rng = np.random.default_rng(0)
+    for _ in range(200):
+        n = int(rng.integers(1, 40))
+        x = rng.integers(-3, 4, n).astype(np.float32)           # many ties
+        x[rng.random(n) < 0.2] = -np.inf
+        x[rng.random(n) < 0.1] = np.nan
+        ok = np.isfinite(x)
+        want = orc.NO_TOKEN if not ok.any() else int(np.flatnonzero(ok & (x == x[ok].max()))[0])   # lowest id of the max
+        assert orc.argmax(x) == want
+    assert orc.argmax(np.array([np.inf, 1.0], dtype=np.float32)) == 0    # +inf is selectable
+
+
+def walk(tree, tokens, selected, remaining, stops):
+    """An independent restatement of the acceptance walk, recursive on children."""
+    rows = len(tree)
+    path = [0]
+    while True:
+        row = path[-1]
+        nxt = [c for c in range(row + 1, rows) if tree[c]["parent"] == row and tokens[c] == selected[row]]
+        if not nxt:
+            break
+        path.append(nxt[0])
+    accepted = len(path) - 1
+    kept = min(accepted + 1, max(remaining, 1))
+    out = []
+    for i in range(kept):
+        out.append(int(selected[path[i]]))
+        if out[-1] in stops:
+            kept = i + 1
+            break
+    return out[:kept], min(accepted, kept), int(tree[path[kept - 1]]["ancestors"])
+
+
+def random_tree(rng, rows):
+    tree = np.zeros(rows, dtype=np.dtype([("ancestors", "<u4"), ("parent", "<u2"), ("depth", "<u2")]))
+    tree[0] = (1, 0xFFFF, 0)
+    for r in range(1, rows):
+        parent = int(rng.integers(0, r))
+        tree[r] = (int(tree[parent]["ancestors"]) | (1 << r), parent, int(tree[parent]["depth"]) + 1)
+    return tree
+
+
+def test_accept_tree_fuzz_against_independent_walk():
+    rng = np.random.default_rng(1)
+    for _ in range(500):
+        rows = int(rng.integers(1, 17))
+        tree = random_tree(rng, rows)
+        tokens = rng.integers(0, 4, rows).astype(np.uint32)
+        selected = rng.integers(0, 4, rows).astype(np.uint32)
+        remaining = int(rng.integers(1, 20))
+        stops = [3] if rng.random() < 0.3 else []
+        got = orc.accept_tree(tree, tokens, selected, remaining, stops)
+        want = walk(tree, tokens, selected, remaining, stops)
+        assert list(got[0]) == want[0] and got[1] == want[1] and got[2] == want[2]
+
+
+def test_chain_acceptance_closed_form():
+    """A chain keeps the longest prefix whose drafted tokens equal the selections, plus the bonus token."""
+    rows = 16
+    tree = np.zeros(rows, dtype=np.dtype([("ancestors", "<u4"), ("parent", "<u2"), ("depth", "<u2")]))
+    for r in range(rows):
+        tree[r] = ((2 << r) - 1, r - 1 if r else 0xFFFF, r)
+    selected = np.arange(100, 100 + rows, dtype=np.uint32)
+    for match in range(rows):
+        tokens = np.zeros(rows, dtype=np.uint32)
+        tokens[1:match + 1] = selected[:match]          # rows 1..match were drafted right
+        tokens[match + 1:] = 7
+        kept, accepted, mask = orc.accept_tree(tree, tokens, selected)
+        assert accepted == match and list(kept) == list(selected[:match + 1]) and mask == (2 << match) - 1
+
+
+def test_rejection_rule_enumerated_law_equals_target():
+    """target_sampling_metal_test.mm:2602-2631: the selection law of test-then-residual equals softmax(logits / T)."""
+    rng = np.random.default_rng(2)
+    for V in (3, 17, 300):
+        x = (rng.standard_normal(V) * 3).astype(np.float32)
+        x[rng.random(V) < 0.1] = -np.inf
+        if not np.isfinite(x).any():
+            x[0] = 0
+        q = np.exp(rng.standard_normal(V) * 2); q = (q / q.sum()).astype(np.float32)
+        T = float(np.float32(0.7))    # the temperature the fp32 interface carries
+        p = np.where(np.isfinite(x), np.exp((x.astype(np.float64) - x[np.isfinite(x)].max()) / T), 0); p /= p.sum()
+        law = orc.rejection_law(x, T, q)
+        assert np.abs(law - p).max() < 1e-12 and abs(law.sum() - 1) < 1e-9
+
+
+def test_rejection_row_follows_the_target_distribution():
+    """target_sampling_metal_test.mm:3019 followsDistribution: chi-square of the row's selections over seeds."""
+    rng = np.random.default_rng(3)
+    V, T, draws = 12, 0.7, 20000
+    x = (rng.standard_normal(V) * 2).astype(np.float32)
+    q = np.exp(rng.standard_normal(V)); q = (q / q.sum()).astype(np.float32)
+    p = np.exp((x.astype(np.float64) - x.max()) / T); p /= p.sum()
+    counts = np.zeros(V)
+    children = rng.choice(V, size=draws, p=q / q.sum())
+    u = rng.random((draws, 2)).astype(np.float32)
+    for i in range(draws):
+        tok, accepted, _ = orc.rejection_row(x, T, q, int(children[i]), float(u[i, 0]), float(u[i, 1]))
+        counts[tok] += 1
+    chi2 = ((counts - draws * p) ** 2 / (draws * p)).sum()
+    assert chi2 < 40, chi2      # 11 degrees of freedom: P(chi2 > 40) < 1e-4
+    # without a child the row is a plain draw from p
+    counts = np.zeros(V)
+    for i in range(draws):
+        tok, _, _ = orc.rejection_row(x, T, None, orc.NO_TOKEN, 0.0, float(u[i, 1]))
+        counts[tok] += 1
+    assert ((counts - draws * p) ** 2 / (draws * p)).sum() < 40
+
+
+def test_rejection_row_accepts_iff_uq_below_p():
+    x = np.array([0.0, 1.0, 2.0, -1.0], dtype=np.float32)
+    q = np.array([0.1, 0.2, 0.3, 0.4], dtype=np.float32)
+    p = np.exp(x.astype(np.float64) / 0.7); p /= p.sum()
+    for child in range(4):
+        for u in (0.01, 0.3, 0.6, 0.99):
+            tok, accepted, close = orc.rejection_row(x, 0.7, q, child, u, 0.5)
+            if close > 1e-5:
+                assert accepted == (u * q[child] < p[child])
+                assert (tok == child) if accepted else (p[tok] > q[tok])   # a redraw comes from max(p - q, 0)

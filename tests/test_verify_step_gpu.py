@@ -1,0 +1,107 @@
+"""End-to-end parity of the dense verify step (BASELINE config 1) against the oracle, through the C ABI."""
+import numpy as np
+import pytest
+
+import splash_amd
+from splash_amd import ops, verify
+from tests import oracle as orc
+from tests.dense_reference import DenseModel
+
+pytestmark = pytest.mark.gpu
+
+
+def top2_gap(logits):
+    part = np.partition(logits, -2, axis=1)
+    return part[:, -1] - part[:, -2]
+
+
+def close_bf16(got_bits, want_bits):
+    """Two bf16 tensors agree: cosine >= 0.9999 and every element within max(2e-2, two bf16 steps of it)."""
+    g, w = orc.bf16_to_f32(got_bits).astype(np.float64), orc.bf16_to_f32(want_bits).astype(np.float64)
+    cos = (g * w).sum() / np.sqrt((g * g).sum() * (w * w).sum())
+    allowed = np.maximum(2e-2, 2 * np.abs(w) * 2.0 ** -8)
+    return cos >= 0.9999 and bool((np.abs(g - w) <= allowed).all()), (cos, np.abs(g - w).max())
+
+
+@pytest.mark.parametrize("rows,context", [(16, 512), (5, 37)])
+def test_config1_verify_step(backend, rows, context):
+    """2-layer dense decoder (hidden 1024, 16 q / 8 kv heads x 64, SwiGLU 3072, vocab 32000), N(0, 0.02)
+    weights quantized to Q4_K (Q6_K head), INT8 KV context, a block of uniform-random draft tokens, greedy.
+    Layer by layer from the GPU's own layer input: hidden rows within the bf16 tolerance of the oracle's;
+    logits from the GPU's final hidden rows within max-abs 2e-2 and cosine >= 0.9999; accepted ids bit-exact.
+    The whole chain against the oracle's own chain: cosine >= 0.9999 and max-abs 5e-2 -- a bf16 pipeline is
+    chaotic at that level: the oracle with fp32 instead of fp64 projection sums moves its own logits by 2.2e-2."""
+    print(f"case config 1 rows={rows} context={context}", flush=True)
+    model = DenseModel(seed=11, hidden=1024, q_heads=16, kv_heads=8, head_dim=64, ffn=3072, vocabulary=32000, layers=2)
+    rng = np.random.default_rng(rows)
+    tokens = rng.integers(0, 32000, rows).astype(np.uint32)
+    gpu = model.build_gpu(backend, max_lanes=1, context_tokens=context + 16)
+    model.seed_context(gpu, context, rng)
+    lane = verify.Lane(rows, context)
+    gpu.set_block([lane], tokens)
+    # the whole step in one command
+    backend.run(gpu.encode([lane], commit=True))
+    chain_logits = gpu.buffer(verify.LOGITS).download(np.float32, rows * 32000).reshape(rows, 32000)
+    selected, retained, accepted, mask = gpu.results([lane])
+    # the same step part by part, teacher-forcing the oracle with the GPU's hidden rows
+    hidden_of = lambda: gpu.buffer(verify.HIDDEN, 0).download(np.uint16, rows * 1024).reshape(rows, 1024)
+    full = gpu.encode([lane], commit=False)      # RoPE tables of the block (first dispatch of a step)
+    backend.run(gpu.encode_part(0, 0, [lane]))
+    assert np.array_equal(hidden_of(), model.oracle_embedding(tokens))
+    for layer in range(2):
+        before = hidden_of()
+        backend.run(gpu.encode_part(1, layer, [lane]))
+        ok, detail = close_bf16(hidden_of(), model.oracle_layer(before, layer, context))
+        assert ok, (layer, detail)
+    final = hidden_of()
+    backend.run(gpu.encode_part(2, 0, [lane]))
+    got_logits = gpu.buffer(verify.LOGITS).download(np.float32, rows * 32000).reshape(rows, 32000)
+    assert np.array_equal(got_logits, chain_logits)     # parts and whole are the same dispatches: bit-identical
+    want_logits = model.oracle_head(final)
+    cos = (got_logits.astype(np.float64) * want_logits).sum() / np.sqrt((got_logits.astype(np.float64) ** 2).sum() * (want_logits ** 2).sum())
+    err = np.abs(got_logits - want_logits).max()
+    assert cos >= 0.9999 and err <= 2e-2, (cos, err)
+    # greedy acceptance of the GPU's logits is bit-exact
+    gpu_argmax = np.array([orc.argmax(got_logits[r]) for r in range(rows)], dtype=np.uint32)
+    kept, acc, m = orc.accept_tree(ops.chain_tree_rows([rows]), tokens, gpu_argmax)
+    assert retained[0] == len(kept) and accepted[0] == acc and mask[0] == m and np.array_equal(selected[:len(kept)], kept)
+    # the whole chain against the oracle's own chain
+    model.seed_context(gpu, context, np.random.default_rng(rows + 1000))   # fresh context arrays for the oracle's stores
+    del full
+    rng = np.random.default_rng(rows); rng.integers(0, 32000, rows)
+    model.seed_context(gpu, context, rng)
+    want = model.oracle_step(tokens, context)
+    cos = (chain_logits.astype(np.float64) * want["logits"]).sum() / np.sqrt((chain_logits.astype(np.float64) ** 2).sum() * (want["logits"] ** 2).sum())
+    err = np.abs(chain_logits - want["logits"]).max()
+    assert cos >= 0.9999 and err <= 5e-2, (cos, err)
+    sure = top2_gap(want["logits"]) > 1e-1
+    assert np.array_equal(gpu_argmax[sure], want["selected"][sure])
+    # where the oracle's top two are closer than that, the GPU's choice is still one of the oracle's near-ties
+    picked = want["logits"][np.arange(rows), gpu_argmax]
+    assert (picked >= want["logits"].max(axis=1) - 1e-1).all()
+    if sure.all():
+        assert np.array_equal(selected[:retained[0]], want["kept"]) and accepted[0] == want["accepted"] and mask[0] == want["retained_rows"]
+
+
+def test_config1_accepts_a_self_consistent_draft(backend):
+    """A draft block that continues the target's own greedy choices is accepted up to the first planted mismatch."""
+    print("case config 1 accepted draft", flush=True)
+    rows, context = 8, 100
+    model = DenseModel(seed=12, hidden=1024, q_heads=16, kv_heads=8, head_dim=64, ffn=3072, vocabulary=32000, layers=2)
+    rng = np.random.default_rng(3)
+    gpu = model.build_gpu(backend, max_lanes=1, context_tokens=context + 16)
+    model.seed_context(gpu, context, rng)
+    tokens = np.zeros(rows, dtype=np.uint32)
+    tokens[0] = 1234
+    lane = verify.Lane(rows, context)
+    for r in range(1, rows):     # grow the block row by row with the target's own selection
+        gpu.set_block([lane], tokens)
+        backend.run(gpu.encode([lane], commit=False))
+        tokens[r] = gpu.buffer(verify.LOGITS).download(np.float32, rows * 32000).reshape(rows, 32000)[r - 1].argmax()
+    planted = tokens.copy()
+    planted[5] = (planted[5] + 1) % 32000
+    gpu.set_block([lane], planted)
+    backend.run(gpu.encode([lane], commit=True))
+    selected, retained, accepted, mask = gpu.results([lane])
+    assert accepted[0] == 4 and retained[0] == 5 and mask[0] == 0b11111
+    assert np.array_equal(selected[:4], planted[1:5]) and selected[4] == tokens[5]
