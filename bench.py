@@ -1,0 +1,228 @@
+#!/usr/bin/env python3
+"""Benchmark of the speculative-decoding verify step on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c4|c1] [--lanes B]
+
+A step is one verify of a 16-token draft block by the 27B-shaped dense target (64 layers, hidden 5120,
+64 q / 8 kv heads x 128, SwiGLU 25600, vocabulary 151936, Q4_K weights with Q6_K down-projection and
+LM head) over a 32K-token INT8 KV context, greedy acceptance, batch 1: BASELINE.json's headline
+configuration. Weights and context are synthetic and resident in HBM before the timed region. One JSON
+line goes to stdout; progress goes to stderr.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0   # MI355X published HBM3E bandwidth
+
+WORKLOADS = {
+    # hidden, q heads, kv heads, head dim, ffn, vocabulary, layers, context, rows
+    "c4": dict(hidden=5120, q_heads=64, kv_heads=8, head_dim=128, ffn=25600, vocabulary=151936, layers=64, context=32768, rows=16,
+               name="27B-shaped dense verify step, Q4_K (Q6_K down-proj and lm_head), 16-token draft, 32K INT8 context"),
+    "c1": dict(hidden=1024, q_heads=16, kv_heads=8, head_dim=64, ffn=3072, vocabulary=32000, layers=2, context=512, rows=16,
+               name="2-layer dense verify step (reference plumbing config), Q4_K, 16-token draft, 512-token INT8 context"),
+}
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def device_copy(backend, source, destination, nbytes):
+    """destination <- source on the device (copy_bytes kernel)."""
+    import ctypes
+    import splash_amd
+
+    class P(ctypes.Structure):
+        _fields_ = [("vectors", ctypes.c_uint64)]
+    g = splash_amd.CommandGraph()
+    g.add("copy_bytes", [source, destination], P(nbytes // 16), (2048, 1, 1), (256, 1, 1))
+    backend.run(g)
+
+
+def build_model(backend, w, lanes):
+    """The synthetic model: one layer's tensors are generated and re-tiled on the host, every other
+    layer holds its own copy in HBM (distinct addresses, so nothing is served from a cache)."""
+    import splash_amd
+    from splash_amd import ops, synthetic, verify
+    rng = np.random.default_rng(20260101)
+    H, D, F, V = w["hidden"], w["head_dim"], w["ffn"], w["vocabulary"]
+    QW, KW = w["q_heads"] * D, w["kv_heads"] * D
+    context_pages = (w["context"] + ops.PAGE_TOKENS - 1) // ops.PAGE_TOKENS
+    physical = context_pages * lanes + 1
+    gpu = verify.DenseVerify(backend, H, w["q_heads"], w["kv_heads"], D, F, V, w["layers"], max_lanes=lanes,
+                             physical_pages=physical, page_table_entries=context_pages * lanes)
+    table = rng.permutation(physical)[:context_pages * lanes].astype(np.uint64)
+    gpu.buffer(verify.PAGE_TABLE).upload(table)
+
+    def image(fmt, n, k):
+        t0 = time.time()
+        img = ops.pack_gguf_image(fmt, synthetic.native(rng, fmt, n, k), n, k)
+        log(f"  tensor {n}x{k} fmt {fmt}: {img.nbytes / 1e6:.1f} MB in {time.time() - t0:.1f}s")
+        return img
+    tensors = dict(q=(ops.FMT_Q4K, QW, H), k=(ops.FMT_Q4K, KW, H), v=(ops.FMT_Q4K, KW, H), o=(ops.FMT_Q4K, H, QW),
+                   gate=(ops.FMT_Q4K, F, H), up=(ops.FMT_Q4K, F, H), down=(ops.FMT_Q6K, H, F))
+    first = {name: backend.from_array(image(*shape), label=name) for name, shape in tensors.items()}
+    norm = lambda n: backend.from_array(((1 + 0.05 * rng.standard_normal(n)).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16))
+    norms = dict(input=norm(H), post=norm(H), q=norm(D), k=norm(D), final=norm(H))
+    for layer in range(w["layers"]):
+        bufs = first if layer == 0 else {}
+        if layer:
+            for name in tensors:
+                bufs[name] = backend.allocate_buffer(first[name].size_bytes, label=name)
+                device_copy(backend, first[name], bufs[name], first[name].size_bytes)
+        P = lambda segs, k: ops.Projection([(tensors[n][0], tensors[n][1], bufs[n]) for n in segs], k)
+        gpu.set_layer(layer, P(["q", "k", "v"], H), P(["o"], QW), P(["gate"], H), P(["up"], H), P(["down"], F),
+                      norms["input"], norms["post"], norms["q"], norms["k"])
+        if layer % 16 == 15:
+            log(f"  layer {layer + 1}/{w['layers']} resident")
+    embedding = backend.from_array(synthetic.native(rng, ops.FMT_Q4K, V, H), label="embedding")
+    head = ops.Projection([(ops.FMT_Q6K, V, backend.from_array(image(ops.FMT_Q6K, V, H), label="head"))], H, float32=True)
+    gpu.set_head(ops.FMT_Q4K, embedding, norms["final"], head)
+    # the INT8 context: one layer's pages from the host, the others copied on the device
+    pages = synthetic.kv_pages(rng, w["kv_heads"], D, physical)
+    pool0 = gpu.buffer(verify.KV_POOL, 0)
+    pool0.upload(pages)
+    for layer in range(1, w["layers"]):
+        device_copy(backend, pool0, gpu.buffer(verify.KV_POOL, layer), pages.nbytes)
+    return gpu
+
+
+def cpu_baseline(w):
+    """The CPU oracle (a port of the reference's test references) timed on this host's cores on a bounded
+    sample of the same step: one layer's projections at reduced width and one layer's attention at reduced
+    context, scaled to the whole step by algorithmic bytes."""
+    from tests import oracle as orc
+    from splash_amd import synthetic
+    cores = os.cpu_count() or 1
+    rng = np.random.default_rng(5)
+    rows, H, F = w["rows"], w["hidden"], w["ffn"]
+    x = orc.f32_to_bf16(rng.standard_normal((rows, H)).astype(np.float32))
+    PASSES = 10
+    sample_n = F      # the whole gate projection, and a quarter of the down projection's columns
+    t0 = time.time()
+    bytes_done = 0
+    for fmt, n, k, xin in ((orc.FMT_Q4K, sample_n, H, x), (orc.FMT_Q6K, max(16, H // 4), F, None)):
+        nat = synthetic.native(rng, fmt, n, k)
+        xi = xin if xin is not None else orc.f32_to_bf16(rng.standard_normal((rows, k)).astype(np.float32))
+        t1 = time.time()
+        for _ in range(PASSES):
+            orc.gemm(fmt, nat, xi, n, want=("chain",), threads=0)
+            bytes_done += nat.nbytes
+        log(f"  cpu gemm fmt {fmt} {n}x{k} x{PASSES}: {time.time() - t1:.2f}s")
+    gemm_seconds = time.time() - t0
+    # attention sample: all heads, reduced context
+    ctx = min(w["context"], 16384)
+    D, KH, QH = w["head_dim"], w["kv_heads"], w["q_heads"]
+    pages = (ctx + rows + 255) // 256
+    kc = rng.integers(-127, 128, (pages, KH, 256, D)).astype(np.int8)
+    vc = rng.integers(-127, 128, (pages, KH, 256, D)).astype(np.int8)
+    ks = np.full((pages, KH, 256), 0.03, dtype=np.float32)
+    q = orc.f32_to_bf16(rng.standard_normal((rows, QH, D)).astype(np.float32))
+    anc = np.array([(2 << r) - 1 for r in range(rows)], dtype=np.uint32)
+    t1 = time.time()
+    orc.attention(q, kc, ks, vc, ks, np.arange(pages, dtype=np.uint32), anc, ctx, want64=False, threads=0)
+    attention_seconds = time.time() - t1
+    log(f"  cpu attention ctx {ctx}: {attention_seconds:.2f}s")
+    weight_bytes = w["layers"] * ((w["q_heads"] + 2 * KH) * D * H * 0.5625 + H * QH * D * 0.5625 + 2 * F * H * 0.5625 + H * F * 0.8203125) \
+        + w["vocabulary"] * H * 0.8203125
+    kv_bytes = w["layers"] * w["context"] * KH * (2 * D + 4)
+    step_seconds = gemm_seconds * weight_bytes / bytes_done + attention_seconds * (w["context"] / ctx) * w["layers"]
+    return {"value": round(step_seconds * 1e3, 1), "unit": "ms", "cores": cores, "kind": "port",
+            "sample": f"oracle register-rule GEMM of {sample_n}x{H} Q4_K and {max(16, H // 4)}x{F} Q6_K at {rows} rows ({PASSES} passes each), oracle paged "
+                      f"attention of one layer at {ctx}-token context; scaled to the step by weight bytes and context length "
+                      f"({gemm_seconds + attention_seconds:.1f}s of CPU work on {cores} threads)"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="c4", choices=sorted(WORKLOADS))
+    ap.add_argument("--lanes", type=int, default=1)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        log("bench.py measures one GPU: this build runs the verify step on a single MI355X (no collectives); use --gpus 1")
+        sys.exit(2)
+    import splash_amd
+    from splash_amd import ops, verify
+    w = WORKLOADS[args.workload]
+    backend = splash_amd.Backend(0)
+    info = backend.device_info()
+    log(f"device {info.name.decode()} {info.arch.decode()} CUs {info.compute_units}")
+    t0 = time.time()
+    gpu = build_model(backend, w, args.lanes)
+    log(f"model resident in {time.time() - t0:.1f}s; allocated {backend.memory_stats().allocated_bytes / 1e9:.2f} GB")
+    context_pages = (w["context"] + ops.PAGE_TOKENS - 1) // ops.PAGE_TOKENS
+    lanes = [verify.Lane(w["rows"], w["context"] - w["rows"], table_first=i * context_pages) for i in range(args.lanes)]
+    rows = w["rows"] * args.lanes
+    rng = np.random.default_rng(1)
+    gpu.set_block(lanes, rng.integers(0, w["vocabulary"], rows).astype(np.uint32))
+    graph = gpu.encode(lanes, commit=True)
+    kernels = graph.kernels()
+    step_bytes = gpu.step_bytes(lanes)
+    log(f"step: {len(kernels)} dispatches, {step_bytes / 1e9:.3f} GB algorithmic")
+    command = backend.record(graph)
+    for _ in range(args.warmup):
+        command.submit().wait()
+    # K steps, one HIP graph launch each, back to back on the command stream; each ticket's GPU time
+    # is the step's first kernel start to its last kernel end.
+    wall0 = time.time()
+    gpu_seconds = 0.0
+    for _ in range(args.steps):
+        gpu_seconds += command.submit().wait()[0]
+    wall = time.time() - wall0
+    ms = gpu_seconds / args.steps * 1e3
+    wall_ms = wall / args.steps * 1e3
+    selected, retained, accepted, mask = gpu.results(lanes)
+    log(f"{ms:.3f} ms/step on the GPU clock, {wall_ms:.3f} ms/step wall; retained {retained.tolist()} accepted {accepted.tolist()}")
+    # The dominant kernel (one-pass gate/up projection), measured live: one more step with an event
+    # pair around every dispatch on the command stream.
+    backend.set_dispatch_profiling(True)
+    _, _, per = backend.run(graph, profiled=True)
+    backend.set_dispatch_profiling(False)
+    by_kernel = {}
+    for name, seconds in zip(kernels, per):
+        by_kernel.setdefault(name, []).append(seconds)
+    totals = sorted(((sum(v), k) for k, v in by_kernel.items()), reverse=True)
+    for total, name in totals[:8]:
+        log(f"  {name:36s} x{len(by_kernel[name]):3d}  avg {total / len(by_kernel[name]) * 1e6:8.2f} us  total {total * 1e3:7.3f} ms")
+    dominant = totals[0][1]
+    gate_up = [k for k in by_kernel if k.endswith("_g")][0]
+    avg = sum(by_kernel[gate_up]) / len(by_kernel[gate_up])
+    H, F = w["hidden"], w["ffn"]
+    gate_up_bytes = 2 * F * H * 0.5625 + rows * H * 2 + rows * F * 2     # both tensors once + bf16 rows in and out
+    achieved = gate_up_bytes / avg / 1e9
+    result = {
+        "metric": "verify-step ms + % HBM roofline, 27B-shape Q4_K, 16-tok draft, 32K ctx" if args.workload == "c4" else "verify-step ms (config 1)",
+        "value": round(ms, 4), "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16 x int4/int6 codes -> fp32 (MFMA); int8 KV",
+        "data": "synthetic: native Q4_K/Q6_K blocks with uniform codes and model-like scales (every layer a copy in its own HBM), "
+                "uniform INT8 KV codes, uniform-random draft tokens, random page table",
+        "config": {"workload": w["name"], "lanes": args.lanes, "rows_per_lane": w["rows"], "context_tokens": w["context"],
+                   "layers": w["layers"], "dispatches": len(kernels), "acceptance": "greedy"},
+        "step_hbm": {"algorithmic_gb": round(step_bytes / 1e9, 3), "achieved_gbs": round(step_bytes / (ms * 1e-3) / 1e9, 1),
+                     "frac_of_peak": round(step_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "wall_ms_per_step": round(wall_ms, 4)},
+        "roofline": {"bound": "hbm", "kernel": gate_up, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None, "launches": len(by_kernel[gate_up]),
+                     "avg_us": round(avg * 1e6, 2), "algorithmic_bytes": int(gate_up_bytes), "largest_total": dominant},
+    }
+    if not args.no_cpu_baseline:
+        log("cpu baseline (oracle on the host cores)...")
+        result["cpu_baseline"] = cpu_baseline(w)
+    else:
+        result["cpu_baseline"] = None
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

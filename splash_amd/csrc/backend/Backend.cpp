@@ -81,6 +81,10 @@ struct sp_backend {
   uint64_t allocated = 0, peak = 0, deviceCurrent = 0, devicePeak = 0;
   uint64_t deviceBaseline = 0;  // bytes in use on the device before this backend allocated
   std::atomic<int> liveBuffers{0};
+  // The backend's memory outlives sp_backend_destroy while buffers, tickets or commands still name it.
+  std::atomic<int> refs{1};
+  void retain() { ++refs; }
+  void release() { if (--refs == 0) delete this; }
 
   void markUnhealthy(const std::string &why) {
     std::lock_guard<std::mutex> lock(mutex);
@@ -300,9 +304,10 @@ void sp_backend_destroy(sp_backend *backend) {
   (void)hipSetDevice(backend->device);
   (void)hipStreamSynchronize(backend->stream);
   (void)hipStreamDestroy(backend->stream);
-  if (backend->liveBuffers.load() > 0)
-    std::fprintf(stderr, "splash_hip: backend destroyed with %d live buffers (leaked)\n", backend->liveBuffers.load());
-  delete backend;
+  backend->stream = nullptr;
+  backend->stopped = true;
+  // Buffers still alive keep the backend's bookkeeping; their memory is freed as they are released.
+  backend->release();
 }
 
 void sp_backend_stop(sp_backend *backend) { if (backend) backend->stopped = true; }
@@ -358,6 +363,7 @@ sp_status sp_buffer_alloc(sp_backend *backend, uint64_t bytes, sp_storage storag
   buffer->size = buffer->allocated = bytes;
   buffer->storage = storage;
   buffer->label = label ? label : "";
+  backend->retain();
   ++backend->liveBuffers;
   {
     std::lock_guard<std::mutex> lock(backend->mutex);
@@ -407,6 +413,7 @@ void sp_buffer_release(sp_buffer *buffer) {
   }
   --backend->liveBuffers;
   delete buffer;
+  backend->release();
 }
 
 uint64_t sp_buffer_size(const sp_buffer *buffer) { return buffer ? buffer->size : 0; }
@@ -424,6 +431,7 @@ sp_status sp_buffer_upload(sp_buffer *buffer, uint64_t offset_bytes, const void 
     return fail(SP_INVALID_ARGUMENT, "upload outside " + buffer->label);
   if (!bytes) return SP_OK;
   sp_backend *backend = buffer->backend;
+  if (!backend->stream) return fail(SP_BACKEND_ERROR, "the backend is destroyed");
   (void)hipSetDevice(backend->device);
   hipError_t e = hipMemcpyAsync(buffer->device + offset_bytes, source, bytes, hipMemcpyHostToDevice, backend->stream);
   if (e == hipSuccess) e = hipStreamSynchronize(backend->stream);
@@ -436,6 +444,7 @@ sp_status sp_buffer_download(const sp_buffer *buffer, uint64_t offset_bytes, voi
     return fail(SP_INVALID_ARGUMENT, "download outside " + buffer->label);
   if (!bytes) return SP_OK;
   sp_backend *backend = buffer->backend;
+  if (!backend->stream) return fail(SP_BACKEND_ERROR, "the backend is destroyed");
   (void)hipSetDevice(backend->device);
   hipError_t e = hipMemcpyAsync(destination, buffer->device + offset_bytes, bytes, hipMemcpyDeviceToHost, backend->stream);
   if (e == hipSuccess) e = hipStreamSynchronize(backend->stream);
@@ -448,6 +457,7 @@ sp_status sp_buffer_fill(sp_buffer *buffer, uint64_t offset_bytes, int byte_valu
     return fail(SP_INVALID_ARGUMENT, "fill outside " + buffer->label);
   if (!bytes) return SP_OK;
   sp_backend *backend = buffer->backend;
+  if (!backend->stream) return fail(SP_BACKEND_ERROR, "the backend is destroyed");
   (void)hipSetDevice(backend->device);
   hipError_t e = hipMemsetAsync(buffer->device + offset_bytes, byte_value, bytes, backend->stream);
   if (e == hipSuccess) e = hipStreamSynchronize(backend->stream);
