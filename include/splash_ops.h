@@ -52,7 +52,7 @@ uint64_t spo_projection_weight_bytes(const spo_projection *projection);
 /* ops::Linear::Linear(device, ...) (Linear.hpp:291): plans follow the device the backend opened. */
 sp_status spo_linear_create(sp_backend *backend, spo_linear **out);
 /* A Linear of a given calibration (KernelCalibration), for CPU tests and sweeps. */
-sp_status spo_linear_create_calibrated(uint32_t compute_units, uint32_t waves_per_unit, uint32_t minimum_blocks_per_wave,
+sp_status spo_linear_create_calibrated(uint32_t compute_units, uint32_t groups_per_unit, uint32_t minimum_blocks_per_wave,
                                        spo_linear **out);
 void spo_linear_destroy(spo_linear *linear);
 /* LinearEpilogue (Linear.hpp:77): 0 None, 1 Residual, 2 GateUp. */

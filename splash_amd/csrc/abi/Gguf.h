@@ -108,7 +108,7 @@ struct GgufPrepareParams {
 // gguf_decode_<fmt>_m<16|32|64>_<a|a_f32|r|g>: up to three column segments of one format in one
 // dispatch (the reference's GgufDecodeFusedParams, runtime/metal/abi/Gguf.h:168-178), tiles in
 // segment order; a single tensor is one segment. A gate/up pair binds gate as segment 0 and up as
-// segment 1, both of cols[0] columns. Grid (units / waves-across-tiles, splits), 256 threads.
+// segment 1, both of cols[0] columns. Grid (units / 4, splits), 256 threads: a wave per unit.
 struct GgufDecodeParams {
   uint32_t input_size;  // K
   uint32_t rows;        // live rows
@@ -117,7 +117,7 @@ struct GgufDecodeParams {
   uint32_t out_stride;  // columns of a destination row
   uint32_t cols[3];     // columns per segment (multiples of 16); 0 past the last
   uint32_t offset[3];   // first destination column per segment
-  uint32_t units;       // wave work units: each GGUF_DECODE_UNIT_TILES column tiles (gate/up: pairs)
+  uint32_t units;       // wave work units: one column tile each (gate/up: gate tile j is unit 2 j, up tile j unit 2 j + 1)
 };
 
 // gguf_dequant_<fmt>: the image's fp32 values [N][K], for the bit-exactness test

@@ -135,12 +135,12 @@ sp_status spo_linear_create(sp_backend *backend, spo_linear **out) {
     *out = new spo_linear{ops::Linear(info)};
   });
 }
-sp_status spo_linear_create_calibrated(uint32_t compute_units, uint32_t waves_per_unit, uint32_t minimum_blocks_per_wave,
+sp_status spo_linear_create_calibrated(uint32_t compute_units, uint32_t groups_per_unit, uint32_t minimum_blocks_per_wave,
                                        spo_linear **out) {
   return capi::guard([&] {
     capi::require(out, "result");
-    if (!compute_units || !waves_per_unit || !minimum_blocks_per_wave) throw std::invalid_argument("a calibration has no zero entry");
-    *out = new spo_linear{ops::Linear(ops::KernelCalibration{compute_units, waves_per_unit, minimum_blocks_per_wave})};
+    if (!compute_units || !groups_per_unit || !minimum_blocks_per_wave) throw std::invalid_argument("a calibration has no zero entry");
+    *out = new spo_linear{ops::Linear(ops::KernelCalibration{compute_units, groups_per_unit, minimum_blocks_per_wave})};
   });
 }
 void spo_linear_destroy(spo_linear *linear) { delete linear; }

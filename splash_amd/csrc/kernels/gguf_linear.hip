@@ -192,6 +192,41 @@ SP_REGISTER_KERNEL("gguf_dequant_q6k", &gguf_dequant<GGUF_FMT_Q6K>);
 // ---------------------------------------------------------------------------------------------
 // The decode projection.
 // ---------------------------------------------------------------------------------------------
+// Streams are read through buffer resources: a load past the end of its range returns zeros and
+// moves no memory, so the software pipeline below needs no branch around a load and no
+// special case at the end of a range, and its address arithmetic is one 32-bit add per stream.
+using Resource = __amdgpu_buffer_rsrc_t;
+__device__ __forceinline__ Resource make_resource(const void *base, uint32_t bytes) {
+  // The base must be wave-uniform (it lives in scalar registers).
+  const uint64_t v = reinterpret_cast<uint64_t>(base);
+  // readfirstlane returns a signed int: widen each half as unsigned.
+  const uint32_t hi = uint32_t(__builtin_amdgcn_readfirstlane(int(uint32_t(v >> 32))));
+  const uint32_t lo = uint32_t(__builtin_amdgcn_readfirstlane(int(uint32_t(v))));
+  const uint64_t u = (uint64_t(hi) << 32) | uint64_t(lo);
+  return __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void *>(u), 0, __builtin_amdgcn_readfirstlane(int(bytes)), 0x00020000);
+}
+constexpr int kStreamOnce = 2;  // non-temporal: weights are read once
+template <int Aux> __device__ __forceinline__ uint4 load128(Resource r, uint32_t offset) {
+  const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(r, int(offset), 0, Aux);
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+// `mine` is the lane's 16 bytes of the record's first 1024-byte part, `column` its column's scale
+// field, both as byte offsets into the resource.
+__device__ __forceinline__ void load_record(Record<GGUF_FMT_Q4K> &rec, Resource r, uint32_t mine, uint32_t column) {
+  rec.n0 = load128<kStreamOnce>(r, mine);
+  rec.n1 = load128<kStreamOnce>(r, mine + 1024u);
+  rec.meta = load128<kStreamOnce>(r, column);
+}
+__device__ __forceinline__ void load_record(Record<GGUF_FMT_Q6K> &rec, Resource r, uint32_t mine, uint32_t column) {
+  rec.n0 = load128<kStreamOnce>(r, mine);
+  rec.n1 = load128<kStreamOnce>(r, mine + 1024u);
+  rec.high = load128<kStreamOnce>(r, mine + 2048u);
+  rec.scales = load128<kStreamOnce>(r, column);
+  // The lane's 16 l and the column's 16 c locate the record and c: d sits at record + 3328 + 2 c.
+  const uint32_t lane = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+  rec.d = __builtin_amdgcn_raw_buffer_load_b16(r, int(mine - 16u * lane + GGUF_Q6K_D + 2u * (lane & 15u)), 0, kStreamOnce);
+}
+
 struct TileRef {
   const uint8_t *image;  // the tile's first record; null for a tile past the dispatch's last
   uint32_t column;       // its first destination column
@@ -222,14 +257,12 @@ __device__ __forceinline__ TileRef find_tile(uint32_t index, const uint8_t *cons
 // group g; sums[t][j][lane] the row sums of the j-th K = 4 MFMA.
 template <uint32_t FMT, int RT>
 __device__ __forceinline__ void accumulate_record(const Record<FMT> &rec, const uint4 (*a)[8][64], const float (*sums)[4][64],
-                                                  f32x4 (&acc)[RT], uint32_t lane, uint32_t kq, float keep) {
+                                                  f32x4 (&acc)[RT], uint32_t lane, uint32_t kq) {
   uint4 ops[8];
   record_operands(rec, ops);
   const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
   if constexpr (FMT == GGUF_FMT_Q4K) {
-    Q4KScales sc = q4k_scales(rec.meta);
-    sc.d *= keep;
-    sc.dmin *= keep;
+    const Q4KScales sc = q4k_scales(rec.meta);
     float s[8];
 #pragma unroll
     for (uint32_t g = 0; g < 8; ++g) s[g] = sc.d * byte_of(g < 4 ? sc.sc_lo : sc.sc_hi, g & 3u);
@@ -253,7 +286,7 @@ __device__ __forceinline__ void accumulate_record(const Record<FMT> &rec, const 
       }
     }
   } else {
-    const float d = half_bits_to_float(rec.d) * keep;
+    const float d = half_bits_to_float(rec.d);
     // Constant terms of 16-input blocks 4 j + kq: -160 d sc (operand 128 + q, value q - 32).
 #pragma unroll
     for (uint32_t j = 0; j < 4; ++j) {
@@ -282,6 +315,10 @@ __device__ __forceinline__ void accumulate_record(const Record<FMT> &rec, const 
   }
 }
 
+// Work split: a wave owns one column tile over the workgroup's K range; the four waves of a
+// workgroup walk that range in step and share its activations through LDS. Unit u of a dispatch
+// is tile u of its concatenated segments; of a gate/up pair, unit 2 j is gate tile j and unit
+// 2 j + 1 up tile j, so the two halves of a pair sit in neighbouring waves of one workgroup.
 template <uint32_t FMT, int RT, uint32_t EP>
 __global__ __launch_bounds__(256) void gguf_decode(const uint8_t *__restrict__ seg0, const uint8_t *__restrict__ seg1,
                                                    const uint8_t *__restrict__ seg2, const uint8_t *__restrict__ table,
@@ -289,10 +326,10 @@ __global__ __launch_bounds__(256) void gguf_decode(const uint8_t *__restrict__ s
                                                    float *__restrict__ partials, uint32_t *__restrict__ counters,
                                                    GgufDecodeParams p) {
   constexpr uint32_t kRecord = FMT == GGUF_FMT_Q4K ? GGUF_Q4K_RECORD : GGUF_Q6K_RECORD;
+  constexpr uint32_t kColumnPart = FMT == GGUF_FMT_Q4K ? 2048u : GGUF_Q6K_SCALES;
   constexpr uint32_t kSumsPerBlock = FMT == GGUF_FMT_Q4K ? 2 : 4;  // K = 4 MFMAs of row sums per super-block
-  // The workgroup's four waves walk one K range in step and own different column tiles; the
-  // range's activations pass through LDS one super-block at a time (two buffers, one barrier per
-  // super-block), each wave fetching a quarter of them, so a wave's vector-memory queue holds
+  // The range's activations pass through LDS one super-block at a time (two buffers, one barrier
+  // per super-block), each wave fetching a quarter of them, so a wave's vector-memory queue holds
   // almost only weights and the MFMA operands arrive on the LDS counter instead.
   __shared__ uint4 ldsA[2][RT][8][64];
   __shared__ float ldsSums[2][RT][4][64];
@@ -303,99 +340,86 @@ __global__ __launch_bounds__(256) void gguf_decode(const uint8_t *__restrict__ s
   const uint32_t split = blockIdx.y;
   const uint32_t blocks = p.input_size / GGUF_BLOCK, G = p.input_size / 32u;
   const uint32_t tiles = gguf_row_tiles(p.rows);
-  const uint8_t *const seg[3] = {seg0, seg1, seg2};
-  const uint32_t ks = 0;
+  const bool live = unit < p.units;
 
-  // Every wave streams real records, so the main loop has no divergent control flow: a wave past
-  // the dispatch's last unit, or a tile past its last tile, re-reads the first tile and stores nothing.
-  TileRef tile[kUnitTiles];
-  bool live[kUnitTiles];
-  {
-    const uint32_t mine = unit < p.units ? unit : 0u;
+  TileRef tile{nullptr, 0};
+  if (live) {
     if constexpr (EP == GGUF_EPILOGUE_GATE_UP) {
-      tile[0] = {seg0 + size_t(mine) * blocks * kRecord, p.offset[0] + mine * GGUF_TILE_COLUMNS};
-      tile[1] = {seg1 + size_t(mine) * blocks * kRecord, p.offset[0] + mine * GGUF_TILE_COLUMNS};
-      live[0] = live[1] = unit < p.units;
+      tile = {(unit & 1u ? seg1 : seg0) + size_t(unit >> 1) * blocks * kRecord, p.offset[0] + (unit >> 1) * GGUF_TILE_COLUMNS};
     } else {
-#pragma unroll
-      for (int i = 0; i < kUnitTiles; ++i) {
-        tile[i] = find_tile(mine * kUnitTiles + i, seg, p, kRecord);
-        live[i] = unit < p.units && tile[i].image != nullptr;
-        if (!tile[i].image) tile[i] = {seg0, p.offset[0]};
-      }
+      const uint8_t *const seg[3] = {seg0, seg1, seg2};
+      tile = find_tile(unit, seg, p, kRecord);
     }
   }
 
   // The workgroup's super-blocks: part `split` of K.
-  const uint32_t b0 = uint32_t(uint64_t(blocks) * split / p.splits), b1 = uint32_t(uint64_t(blocks) * (split + 1) / p.splits);
+  // (blocks <= 2^16 and splits <= 16, so the products fit 32 bits; the quotients are wave-uniform.)
+  const uint32_t b0 = uint32_t(__builtin_amdgcn_readfirstlane(int(blocks * split / p.splits)));
+  const uint32_t b1 = uint32_t(__builtin_amdgcn_readfirstlane(int(blocks * (split + 1u) / p.splits)));
+  const uint32_t count = b1 - b0;
 
-  f32x4 acc[kUnitTiles][RT];
+  f32x4 acc[RT];
 #pragma unroll
-  for (int i = 0; i < kUnitTiles; ++i)
-#pragma unroll
-    for (int t = 0; t < RT; ++t) acc[i][t] = f32x4{0.f, 0.f, 0.f, 0.f};
-
-  const uint4 *values = reinterpret_cast<const uint4 *>(table);
-  const float *sumsBase = reinterpret_cast<const float *>(
-      table + (FMT == GGUF_FMT_Q4K ? gguf_table_sums32_offset(p.input_size, tiles) : gguf_table_sums16_offset(p.input_size, tiles)));
-  const uint32_t sumGroups = FMT == GGUF_FMT_Q4K ? G : 2u * G;  // row-sum entries per row tile
+  for (int t = 0; t < RT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   {
     // A software pipeline of kStages super-blocks in registers: the loads of super-block
     // b + kStages - 1 are issued before the MFMAs of super-block b, so kStages - 1 super-blocks of
     // weights per wave stay in flight (loads return in issue order, so waiting for b's never
-    // waits for a later one's). The loop body is one straight block: the range is walked in
-    // rounds of kStages, loads past its end re-read its last super-block (the cursors stop
-    // there) and the super-blocks past its end are multiplied by a zero scale.
-    constexpr int kStages = RT > 1 ? 2 : FMT == GGUF_FMT_Q4K ? 4 : 3;
+    // waits for a later one's). Loads past the range return zeros without touching memory.
+    constexpr int kStages = RT > 2 ? 2 : 3;
     constexpr uint32_t kSumFloats = RT * kSumsPerBlock * 64u;  // staged row sums per super-block
     constexpr int kSumShare = (kSumFloats + 255u) / 256u;
     struct Stage {
-      Record<FMT> rec[kUnitTiles];
+      Record<FMT> rec;
       uint4 a[2 * RT];       // this thread's share of the super-block's RT * 8 * 64 operand vectors
       float sum[kSumShare];  // and of its row sums
     };
     Stage stage[kStages];
-    Cursor<FMT> cursor[kUnitTiles];
+    // A wave without a tile reads an empty range.
+    const Resource weights = make_resource(tile.image ? tile.image + size_t(b0) * kRecord : seg0, tile.image ? count * kRecord : 0u);
+    uint32_t mine = 16u * lane, column = kColumnPart + 16u * c;
+    // The table's values of row tile t, super-blocks b0..b1: one resource per row tile.
+    Resource values[RT];
 #pragma unroll
-    for (int i = 0; i < kUnitTiles; ++i) cursor[i].open(tile[i].image + size_t(b0) * kRecord, lane);
-    const uint4 *share[2 * RT];
+    for (int t = 0; t < RT; ++t) values[t] = make_resource(table + (size_t(t) * G + 8u * b0) * 1024u, count * 8192u);
+    uint32_t share[2];  // vector j of a row tile's super-block: byte offset of this thread's
 #pragma unroll
-    for (int j = 0; j < 2 * RT; ++j) {
-      const uint32_t at = threadIdx.x + 256u * j, t = at / 512u, g = (at / 64u) % 8u, l = at % 64u;
-      share[j] = values + (size_t(t) * G + 8u * b0 + g) * 64u + l;
-    }
+    for (int j = 0; j < 2; ++j) share[j] = (threadIdx.x + 256u * j) * 16u;
+    const uint32_t sumsAt = FMT == GGUF_FMT_Q4K ? gguf_table_sums32_offset(p.input_size, tiles) : gguf_table_sums16_offset(p.input_size, tiles);
+    const uint32_t sumGroups = FMT == GGUF_FMT_Q4K ? G : 2u * G;  // row-sum entries per row tile
+    const Resource sums = make_resource(table + sumsAt, tiles * sumGroups * 64u);
     // Threads past the staged sums repeat an earlier thread's (same value to the same slot).
-    const float *sumShare[kSumShare];
-    uint32_t sumSlot[kSumShare];
+    uint32_t sumShare[kSumShare], sumSlot[kSumShare];
 #pragma unroll
     for (int q = 0; q < kSumShare; ++q) {
       const uint32_t at = (threadIdx.x + 256u * q) % kSumFloats;
       const uint32_t t = at / (kSumsPerBlock * 64u), j = (at / 64u) % kSumsPerBlock, l = at % 64u;
-      sumShare[q] = sumsBase + (size_t(t) * sumGroups + kSumsPerBlock * 4u * b0 + 4u * j + (l >> 4)) * 16u + (l & 15u);
+      sumShare[q] = ((t * sumGroups + kSumsPerBlock * 4u * b0 + 4u * j + (l >> 4)) * 16u + (l & 15u)) * 4u;
       sumSlot[q] = (t * 4u + j) * 64u + l;
     }
-    uint32_t issued = b0;  // the next super-block to issue; stops at b1 - 1
     auto issue = [&](Stage &st) {
 #pragma unroll
-      for (int j = 0; j < 2 * RT; ++j) st.a[j] = *share[j];
+      for (int j = 0; j < 2 * RT; ++j) st.a[j] = load128<0>(values[j / 2], share[j % 2]);
 #pragma unroll
-      for (int q = 0; q < kSumShare; ++q) st.sum[q] = *sumShare[q];
+      for (int q = 0; q < kSumShare; ++q)
+        st.sum[q] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(sums, int(sumShare[q]), 0, 0));
+      load_record(st.rec, weights, mine, column);
+      mine += kRecord;
+      column += kRecord;
 #pragma unroll
-      for (int i = 0; i < kUnitTiles; ++i) st.rec[i].load(cursor[i]);
-      if (issued + 1 < b1) {  // uniform: scalar branch over a few pointer bumps
-        ++issued;
+      for (int j = 0; j < 2; ++j) share[j] += 8192u;
+      // Sums past the range are the next range's or, past the table, zeros: staged and never used.
 #pragma unroll
-        for (int j = 0; j < 2 * RT; ++j) share[j] += 8u * 64u;
-#pragma unroll
-        for (int q = 0; q < kSumShare; ++q) sumShare[q] += kSumsPerBlock * 4u * 16u;
-#pragma unroll
-        for (int i = 0; i < kUnitTiles; ++i) cursor[i].advance();
-      }
+      for (int q = 0; q < kSumShare; ++q) sumShare[q] += kSumsPerBlock * 4u * 16u * 4u;
     };
 #pragma unroll
-    for (int s = 0; s < kStages - 1; ++s) issue(stage[s]);
-    const uint32_t count = b1 - b0, rounds = (count + kStages - 1) / kStages;
+    for (int s = 0; s < kStages - 1; ++s) {
+      issue(stage[s]);
+      // Keep the stages' loads in issue order: the loop's counted waits assume it on entry too.
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    const uint32_t rounds = (count + kStages - 1) / kStages;
     uint32_t now = 0;
     for (uint32_t round = 0; round < rounds; ++round) {
 #pragma unroll
@@ -407,35 +431,22 @@ __global__ __launch_bounds__(256) void gguf_decode(const uint8_t *__restrict__ s
         for (int q = 0; q < kSumShare; ++q) (&ldsSums[buffer][0][0][0])[sumSlot[q]] = stage[u].sum[q];
         __syncthreads();
         issue(stage[(u + kStages - 1) % kStages]);
-        const float keep = now < count ? 1.0f : 0.0f;
-#pragma unroll
-        for (int i = 0; i < kUnitTiles; ++i)
-          accumulate_record<FMT, RT>(stage[u].rec[i], ldsA[buffer], ldsSums[buffer], acc[i], lane, kq, keep);
+        if (now < count) accumulate_record<FMT, RT>(stage[u].rec, ldsA[buffer], ldsSums[buffer], acc, lane, kq);
       }
     }
   }
 
-  tile[0].image = live[0] ? tile[0].image : nullptr;
-#pragma unroll
-  for (int i = 1; i < kUnitTiles; ++i) tile[i].image = live[i] ? tile[i].image : nullptr;
-
-  // Element (i, t, v) of this lane is row 16 t + 4 kq + v, column tile[i].column + c.
-  const uint32_t paddedRows = tiles * GGUF_ROW_TILE;
-  bool finish = ks == 0 && tile[0].image;
+  // Element (t, v) of this lane is row 16 t + 4 kq + v, column tile.column + c.
   if (p.splits > 1) {
-    if (finish) {
+    // Partials [split][unit][t][v][lane]: whole-wave contiguous stores and loads.
+    const size_t stride = size_t(gridDim.x) * 4u * RT * 256u;
+    float *mineAt = partials + (size_t(unit) * RT * 4u) * 64u + lane;
+    if (live) {
 #pragma unroll
-      for (int i = 0; i < kUnitTiles; ++i) {
-        if (!tile[i].image) continue;
-        const uint32_t column = (EP == GGUF_EPILOGUE_GATE_UP ? uint32_t(i) * p.out_stride : 0u) + tile[i].column + c;
-        const uint32_t width = EP == GGUF_EPILOGUE_GATE_UP ? 2u * p.out_stride : p.out_stride;
+      for (int t = 0; t < RT; ++t)
 #pragma unroll
-        for (int t = 0; t < RT; ++t)
-#pragma unroll
-          for (int v = 0; v < 4; ++v)
-            __hip_atomic_store(&partials[(size_t(split) * paddedRows + 16u * t + 4u * kq + v) * width + column], acc[i][t][v],
-                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      }
+        for (int v = 0; v < 4; ++v)
+          __hip_atomic_store(mineAt + size_t(split) * stride + (t * 4 + v) * 64, acc[t][v], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     // The partials are written and read with agent-scope atomics, which go to the coherence
     // point instead of a compute die's own L2, so no cache write-back or invalidate is needed: the
@@ -446,29 +457,44 @@ __global__ __launch_bounds__(256) void gguf_decode(const uint8_t *__restrict__ s
     if (threadIdx.x == 0) arrived = __hip_atomic_fetch_add(&counters[blockIdx.x], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
     if (arrived != p.splits - 1) return;
-    if (finish) {
+    // The last arriver sums the splits in split order; the loads of a round of eight are in flight together.
 #pragma unroll
-      for (int i = 0; i < kUnitTiles; ++i) {
-        if (!tile[i].image) continue;
-        const uint32_t column = (EP == GGUF_EPILOGUE_GATE_UP ? uint32_t(i) * p.out_stride : 0u) + tile[i].column + c;
-        const uint32_t width = EP == GGUF_EPILOGUE_GATE_UP ? 2u * p.out_stride : p.out_stride;
+    for (int t = 0; t < RT; ++t)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) acc[t][v] = 0.f;
+    for (uint32_t s0 = 0; s0 < p.splits; s0 += 4u) {
+      float part[4][RT][4];
+#pragma unroll
+      for (uint32_t s = 0; s < 4u; ++s)
 #pragma unroll
         for (int t = 0; t < RT; ++t)
 #pragma unroll
           for (int v = 0; v < 4; ++v) {
-            float sum = 0.f;
-            for (uint32_t s = 0; s < p.splits; ++s)
-              sum += __hip_atomic_load(&partials[(size_t(s) * paddedRows + 16u * t + 4u * kq + v) * width + column],
-                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            acc[i][t][v] = sum;
+            const uint32_t from = s0 + s < p.splits ? s0 + s : s0;
+            part[s][t][v] = __hip_atomic_load(mineAt + size_t(from) * stride + (t * 4 + v) * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           }
-      }
+#pragma unroll
+      for (uint32_t s = 0; s < 4u; ++s)
+#pragma unroll
+        for (int t = 0; t < RT; ++t)
+#pragma unroll
+          for (int v = 0; v < 4; ++v) acc[t][v] += s0 + s < p.splits ? part[s][t][v] : 0.f;
     }
     if (threadIdx.x == 0) __hip_atomic_store(&counters[blockIdx.x], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
-  if (!finish) return;
 
   if constexpr (EP == GGUF_EPILOGUE_GATE_UP) {
+    // The up wave hands its sums to the gate wave beside it through LDS (the staging buffers are free).
+    float *exchange = reinterpret_cast<float *>(&ldsA[0][0][0][0]);
+    __syncthreads();
+    if (wave & 1u) {
+#pragma unroll
+      for (int t = 0; t < RT; ++t)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) exchange[((wave >> 1) * RT * 4u + t * 4 + v) * 64u + lane] = acc[t][v];
+    }
+    __syncthreads();
+    if ((wave & 1u) || !live) return;
     uint16_t *o = static_cast<uint16_t *>(out);
 #pragma unroll
     for (int t = 0; t < RT; ++t)
@@ -476,26 +502,23 @@ __global__ __launch_bounds__(256) void gguf_decode(const uint8_t *__restrict__ s
       for (int v = 0; v < 4; ++v) {
         const uint32_t row = 16u * t + 4u * kq + v;
         if (row >= p.rows) continue;
-        const float gate = round_bf16(acc[0][t][v]), up = round_bf16(acc[1][t][v]);
-        o[size_t(row) * p.out_stride + tile[0].column + c] = uint16_t(float_to_bf16_bits(up * silu(gate)));
+        const float gate = round_bf16(acc[t][v]), up = round_bf16(exchange[((wave >> 1) * RT * 4u + t * 4 + v) * 64u + lane]);
+        o[size_t(row) * p.out_stride + tile.column + c] = uint16_t(float_to_bf16_bits(up * silu(gate)));
       }
   } else {
+    if (!live || !tile.image) return;
 #pragma unroll
-    for (int i = 0; i < kUnitTiles; ++i) {
-      if (!tile[i].image) continue;
+    for (int t = 0; t < RT; ++t)
 #pragma unroll
-      for (int t = 0; t < RT; ++t)
-#pragma unroll
-        for (int v = 0; v < 4; ++v) {
-          const uint32_t row = 16u * t + 4u * kq + v;
-          if (row >= p.rows) continue;
-          const size_t at = size_t(row) * p.out_stride + tile[i].column + c;
-          if constexpr (EP == GGUF_EPILOGUE_PLAIN_F32) static_cast<float *>(out)[at] = acc[i][t][v];
-          else if constexpr (EP == GGUF_EPILOGUE_RESIDUAL)
-            static_cast<uint16_t *>(out)[at] = uint16_t(float_to_bf16_bits(acc[i][t][v] + bf16_bits_to_float(residual[at])));
-          else static_cast<uint16_t *>(out)[at] = uint16_t(float_to_bf16_bits(acc[i][t][v]));
-        }
-    }
+      for (int v = 0; v < 4; ++v) {
+        const uint32_t row = 16u * t + 4u * kq + v;
+        if (row >= p.rows) continue;
+        const size_t at = size_t(row) * p.out_stride + tile.column + c;
+        if constexpr (EP == GGUF_EPILOGUE_PLAIN_F32) static_cast<float *>(out)[at] = acc[t][v];
+        else if constexpr (EP == GGUF_EPILOGUE_RESIDUAL)
+          static_cast<uint16_t *>(out)[at] = uint16_t(float_to_bf16_bits(acc[t][v] + bf16_bits_to_float(residual[at])));
+        else static_cast<uint16_t *>(out)[at] = uint16_t(float_to_bf16_bits(acc[t][v]));
+      }
   }
 }
 

@@ -1,5 +1,6 @@
 #include "ops/Linear.hpp"
 
+#include <algorithm>
 #include <array>
 #include <stdexcept>
 
@@ -21,11 +22,13 @@ const char *epilogueSuffix(LinearEpilogue epilogue, FloatOutput destination) {
   return "_a";
 }
 
-// Wave work units of a dispatch: two column tiles each; a gate/up pair's unit is one tile of each.
+// Wave work units of a dispatch: one column tile each; a gate/up pair holds the tiles of both tensors.
 uint32_t unitsOf(uint32_t columns, LinearEpilogue epilogue) {
   const uint32_t tiles = columns / GGUF_TILE_COLUMNS;
-  return epilogue == LinearEpilogue::GateUp ? tiles : (tiles + 1) / 2;
+  return epilogue == LinearEpilogue::GateUp ? 2 * tiles : tiles;
 }
+constexpr uint32_t kWavesAcross = 4;  // waves, and so units, of a workgroup
+uint32_t groupsOf(uint32_t columns, LinearEpilogue epilogue) { return (unitsOf(columns, epilogue) + kWavesAcross - 1) / kWavesAcross; }
 
 void requireSegments(const Projection &p, LinearMatrix matrix) {
   if (p.outputSize != matrix.outputSize || p.inputSize != matrix.inputSize)
@@ -69,12 +72,10 @@ LinearScratchSize LinearPlan::scratchSize() const noexcept {
   LinearScratchSize size;
   size.input = gguf_table_bytes(k, tiles);
   if (config_.splits > 1) {
-    // [split][row][column] fp32 partials over the tile's rows, a gate/up pair's of both tensors,
-    // and one counter per workgroup.
-    const uint64_t columns = workload_.epilogue == LinearEpilogue::GateUp ? 2 * uint64_t{n} : n;
-    const uint32_t across = 4;
-    size.partials = uint64_t{config_.splits} * tiles * GGUF_ROW_TILE * columns * sizeof(float);
-    size.counters = uint64_t{(unitsOf(n, workload_.epilogue) + across - 1) / across} * sizeof(uint32_t);
+    // [split][unit][row tile][4][64 lanes] fp32 partials over whole workgroups, and one counter per workgroup.
+    const uint64_t groups = groupsOf(n, workload_.epilogue);
+    size.partials = uint64_t{config_.splits} * groups * kWavesAcross * tiles * 256u * sizeof(float);
+    size.counters = groups * sizeof(uint32_t);
   }
   return size;
 }
@@ -89,15 +90,14 @@ LinearPlan Linear::plan(LinearWorkload workload, LinearConfig config, FloatOutpu
 
 LinearPlan Linear::plan(LinearWorkload w, FloatOutput destination) const {
   // Fill the device: partition K across workgroups (fp32 partials, summed in split order by the
-  // last arriver) until the dispatch holds wavesPerUnit waves per compute unit or a wave's range
-  // is down to minimumBlocksPerWave.
+  // last arriver) until the dispatch holds groupsPerUnit workgroups per compute unit or a
+  // workgroup's range is down to minimumBlocksPerWave super-blocks.
   const uint32_t blocks = w.matrix.inputSize / GGUF_BLOCK;
-  const uint32_t units = std::max(1u, unitsOf(w.matrix.outputSize, w.epilogue));
-  const uint64_t wanted = uint64_t{calibration_.computeUnits} * calibration_.wavesPerUnit;
+  const uint32_t groups = std::max(1u, groupsOf(w.matrix.outputSize, w.epilogue));
+  const uint32_t wanted = calibration_.computeUnits * calibration_.groupsPerUnit;
   LinearConfig config;
-  auto parts = [&] { return config.splits * config.kWaves; };
-  auto mayDouble = [&] { return uint64_t{units} * parts() < wanted && blocks / (2 * parts()) >= calibration_.minimumBlocksPerWave; };
-  while (config.splits < LinearConfig::kMaximumSplits && mayDouble()) config.splits *= 2;
+  config.splits = std::clamp((wanted + groups / 2) / groups, 1u,
+                             std::min(LinearConfig::kMaximumSplits, std::max(1u, blocks / calibration_.minimumBlocksPerWave)));
   return LinearPlan(w, config, destination);
 }
 
@@ -180,14 +180,13 @@ PreparedInput Linear::add(hip::CommandGraph &graph, LinearBuffers b, const Proje
   params.units = unitsOf(n, w.epilogue);
   // Unused bindings still name a buffer: the table stands in for them.
   const hip::Buffer &spare = b.scratch.input;
-  const uint32_t across = 4;
   const std::string name = std::string("gguf_decode_") + segments.front().name() + "_m" + std::to_string(plan.storageRows()) +
                            epilogueSuffix(w.epilogue, plan.destination());
   graph.add(name,
             {images[0], images[1], images[2], b.scratch.input, b.output,
              w.epilogue == LinearEpilogue::Residual ? b.residual : spare, c.splits > 1 ? b.scratch.partials : spare,
              c.splits > 1 ? b.scratch.counters : spare},
-            params, {(params.units + across - 1) / across, c.splits, 1}, {256, 1, 1});
+            params, {groupsOf(n, w.epilogue), c.splits, 1}, {256, 1, 1});
   (void)tiles;
   return {b.input, LinearInput::Table16};
 }

@@ -41,14 +41,14 @@ struct LinearWorkload final {
 
 struct LinearConfig final {
   LinearTile tile = LinearTile::GgufMfma;
-  // Cross-workgroup K partitions, a power of two up to kMaximumSplits.
+  // Cross-workgroup K partitions, 1 to kMaximumSplits.
   uint32_t splits = 1;
   static constexpr uint32_t kMaximumSplits = GGUF_MAXIMUM_SPLITS;
   // Waves of a workgroup that split its K partition between them: 1 (its four waves walk the
   // partition in step, each over its own column tiles).
   uint32_t kWaves = 1;
   [[nodiscard]] constexpr bool validSplits() const noexcept {
-    return splits && splits <= kMaximumSplits && !(splits & (splits - 1));
+    return splits && splits <= kMaximumSplits;
   }
   bool operator==(const LinearConfig &) const = default;
 };
@@ -120,10 +120,10 @@ struct LinearBuffers final {
 // measured on MI355X, overridable for sweeps.
 struct KernelCalibration final {
   uint32_t computeUnits = 256;
-  // Waves a projection should put in flight per compute unit before it stops partitioning K.
-  uint32_t wavesPerUnit = 8;
-  // Fewest super-blocks a wave's K range keeps.
-  uint32_t minimumBlocksPerWave = 2;
+  // Workgroups a projection should hold per compute unit before it stops partitioning K.
+  uint32_t groupsPerUnit = 4;
+  // Fewest super-blocks a workgroup's K range keeps.
+  uint32_t minimumBlocksPerWave = 5;
 };
 
 class Linear final {
