@@ -8,6 +8,26 @@
 
 namespace splash::kernels {
 
+// Rows of up to kStagedWidth columns are staged in LDS with every global load in flight at once
+// (a row's columns are read twice, in an order no vector load gives directly).
+constexpr uint32_t kStagedWidth = 8192;
+
+// Copies `width` bf16 values (a multiple of 8, 16-byte aligned) to LDS; no barrier.
+__device__ __forceinline__ void stage_row(const uint16_t *__restrict__ source, uint32_t width, uint16_t *lds) {
+  const uint32_t vectors = width / 8u;
+  uint4 held[kStagedWidth / 8u / 256u];
+#pragma unroll
+  for (uint32_t i = 0; i < kStagedWidth / 8u / 256u; ++i) {
+    const uint32_t v = threadIdx.x + 256u * i;
+    if (v < vectors) held[i] = reinterpret_cast<const uint4 *>(source)[v];
+  }
+#pragma unroll
+  for (uint32_t i = 0; i < kStagedWidth / 8u / 256u; ++i) {
+    const uint32_t v = threadIdx.x + 256u * i;
+    if (v < vectors) reinterpret_cast<uint4 *>(lds)[v] = held[i];
+  }
+}
+
 // The row's inverse RMS: 256 threads sum the squares of columns tid, tid + 256, ... in column
 // order; a wavefront sums its lanes by butterfly, the four wavefronts' sums are added in order
 // (normalization.metal:59-99 and common/rms_inverse.h:15-33, on 64-lane wavefronts).
@@ -27,11 +47,19 @@ __device__ __forceinline__ float rms_inverse(const uint16_t *row, uint32_t width
 __global__ __launch_bounds__(256) void norm_rms(const uint16_t *__restrict__ input, const uint16_t *__restrict__ weight,
                                                 uint16_t *__restrict__ output, NormParams p) {
   __shared__ float scratch[4];
+  __shared__ __align__(16) uint16_t rowX[kStagedWidth], rowW[kStagedWidth];
   const uint32_t row = blockIdx.x;
-  const uint16_t *x = input + size_t(row) * p.width;
+  const uint16_t *x = input + size_t(row) * p.width, *w = weight;
+  if (p.width <= kStagedWidth && p.width % 8u == 0) {
+    stage_row(x, p.width, rowX);
+    stage_row(w, p.width, rowW);
+    __syncthreads();
+    x = rowX;
+    w = rowW;
+  }
   const float inverse = rms_inverse(x, p.width, scratch);
   for (uint32_t c = threadIdx.x; c < p.width; c += 256)
-    output[size_t(row) * p.width + c] = uint16_t(float_to_bf16_bits((bf16_bits_to_float(x[c]) * inverse) * bf16_bits_to_float(weight[c])));
+    output[size_t(row) * p.width + c] = uint16_t(float_to_bf16_bits((bf16_bits_to_float(x[c]) * inverse) * bf16_bits_to_float(w[c])));
 }
 SP_REGISTER_KERNEL("norm_rms", &norm_rms);
 
@@ -41,9 +69,17 @@ SP_REGISTER_KERNEL("norm_rms", &norm_rms);
 __global__ __launch_bounds__(256) void norm_rms_table16(const uint16_t *__restrict__ input, const uint16_t *__restrict__ weight,
                                                         uint16_t *__restrict__ output, uint8_t *__restrict__ table, NormParams p) {
   __shared__ float scratch[4];
+  __shared__ __align__(16) uint16_t rowX[kStagedWidth], rowW[kStagedWidth];
   const uint32_t row = blockIdx.x, tile = row / 16u, r = row % 16u, G = p.width / 32u;
   const bool live = row < p.rows;
-  const uint16_t *x = input + size_t(live ? row : 0) * p.width;
+  const uint16_t *x = input + size_t(live ? row : 0) * p.width, *w = weight;
+  if (live && p.width <= kStagedWidth) {  // the width is a multiple of 256
+    stage_row(x, p.width, rowX);
+    stage_row(w, p.width, rowW);
+    __syncthreads();
+    x = rowX;
+    w = rowW;
+  }
   const float inverse = live ? rms_inverse(x, p.width, scratch) : 0.f;
   uint2 *values = reinterpret_cast<uint2 *>(table);
   float *sums32 = reinterpret_cast<float *>(table + gguf_table_sums32_offset(p.width, p.tiles));
@@ -53,13 +89,15 @@ __global__ __launch_bounds__(256) void norm_rms_table16(const uint16_t *__restri
     uint32_t bits[4] = {0, 0, 0, 0};
     float v[4] = {0.f, 0.f, 0.f, 0.f};
     if (live) {
+      const uint2 xs = *reinterpret_cast<const uint2 *>(x + 4u * q), ws = *reinterpret_cast<const uint2 *>(w + 4u * q);
+      const uint32_t xb[4] = {xs.x & 0xFFFFu, xs.x >> 16, xs.y & 0xFFFFu, xs.y >> 16};
+      const uint32_t wb[4] = {ws.x & 0xFFFFu, ws.x >> 16, ws.y & 0xFFFFu, ws.y >> 16};
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const uint32_t c = 4u * q + i;
-        bits[i] = float_to_bf16_bits((bf16_bits_to_float(x[c]) * inverse) * bf16_bits_to_float(weight[c]));
+        bits[i] = float_to_bf16_bits((bf16_bits_to_float(xb[i]) * inverse) * bf16_bits_to_float(wb[i]));
         v[i] = bf16_bits_to_float(bits[i]);
-        output[size_t(row) * p.width + c] = uint16_t(bits[i]);
       }
+      *reinterpret_cast<uint2 *>(output + size_t(row) * p.width + 4u * q) = make_uint2(bits[0] | (bits[1] << 16), bits[2] | (bits[3] << 16));
     }
     const uint32_t g = q / 8u, half = (q / 4u) % 2u, kq = q % 4u;
     // operand elements 4 half + {0,1,2,3} are inputs 4 kq + {0,2,1,3} of the half

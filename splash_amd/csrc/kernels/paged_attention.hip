@@ -21,6 +21,7 @@
 #include "abi/PagedAttention.h"
 #include "backend/KernelRegistry.hpp"
 #include "kernels/device_common.hpp"
+#include <type_traits>
 
 namespace splash::kernels {
 
@@ -154,7 +155,7 @@ SP_REGISTER_KERNEL("attention_q8_qkv_d64", &attention_q8_qkv<64>);
 // [sequence][kv head][split][16 G]; the max is in the log2 domain of the scaled scores.
 // ---------------------------------------------------------------------------------------------
 template <int D, int G>
-__global__ __launch_bounds__(256) void attention_q8_split(const _Float16 *__restrict__ queries, const float *__restrict__ qsums,
+__global__ __launch_bounds__(256, 2) void attention_q8_split(const _Float16 *__restrict__ queries, const float *__restrict__ qsums,
                                                           const AttentionTreeRow *__restrict__ tree,
                                                           const uint64_t *__restrict__ page_table, uint8_t *__restrict__ pool,
                                                           float *__restrict__ partialO, float *__restrict__ partialML,
@@ -165,7 +166,7 @@ __global__ __launch_bounds__(256) void attention_q8_split(const _Float16 *__rest
   static_assert(kKeyVectors >= 1, "a step's keys fill the workgroup's loads");
   __shared__ __align__(16) _Float16 ldsK[2][kStep][D + 8];
   __shared__ __align__(16) _Float16 ldsV[2][D][kStep + 8];
-  __shared__ float ldsKS[2][kStep], ldsVS[2][kStep];
+  __shared__ __align__(16) float ldsKS[2][kStep], ldsVS[2][kStep];
 
   const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, row = lane & 15u, kq = lane >> 4;
   const uint32_t h = blockIdx.x, split = blockIdx.y, z = blockIdx.z;
@@ -188,7 +189,7 @@ __global__ __launch_bounds__(256) void attention_q8_split(const _Float16 *__rest
     const size_t at = ((size_t(z) * p.kv_heads + h) * G + (owns[k] ? g : 0u)) * 16u + row;
 #pragma unroll
     for (int j = 0; j < JD; ++j) q[k][j] = *reinterpret_cast<const f16x8 *>(queries + at * D + 32 * j + 8 * kq);
-    qsum[k] = qsums[at] * kCodeOffset;
+    qsum[k] = -(qsums[at] * kCodeOffset);
   }
   const uint32_t ancestors = row < seq.rows ? tree[seq.first_row + row].ancestors : 0u;
 
@@ -205,9 +206,20 @@ __global__ __launch_bounds__(256) void attention_q8_split(const _Float16 *__rest
   // A step's loads of this thread: kKeyVectors 16-byte vectors of keys, as many of values, a scale.
   uint4 keyLoad[kKeyVectors], valueLoad[kValueVectors];
   uint32_t scaleLoad = 0;
+  // The page table is read one page ahead of the page loop, so that a step's loads never wait
+  // for a table entry first (all of this is wave-uniform).
+  const uint64_t *entries = page_table + seq.table_first;
+  const uint32_t lastPage = total ? (total - 1u) / ATTENTION_PAGE_TOKENS : 0u;
+  uint32_t heldPage = min(first / ATTENTION_PAGE_TOKENS, lastPage);
+  uint64_t heldEntry = entries[heldPage], nextEntry = entries[min(heldPage + 1u, lastPage)];
   auto load = [&](uint32_t step) {
     const uint32_t token0 = first + step * kStep;
-    uint8_t *page = page_of(pool, page_table, seq, p.page_bytes, token0 / ATTENTION_PAGE_TOKENS);
+    if (token0 / ATTENTION_PAGE_TOKENS != heldPage) {
+      heldPage = token0 / ATTENTION_PAGE_TOKENS;
+      heldEntry = nextEntry;
+      nextEntry = entries[min(heldPage + 1u, lastPage)];
+    }
+    uint8_t *page = pool + heldEntry * p.page_bytes;
     const uint32_t inPage = token0 % ATTENTION_PAGE_TOKENS;
     const uint4 *keys = reinterpret_cast<const uint4 *>(page + attention_key_index(h, inPage, 0, D));
     const uint4 *values = reinterpret_cast<const uint4 *>(page + attention_page_values_offset(p.kv_heads, D) +
@@ -244,7 +256,8 @@ __global__ __launch_bounds__(256) void attention_q8_split(const _Float16 *__rest
       for (uint32_t quarter = 0; quarter < 4; ++quarter)
         *reinterpret_cast<uint2 *>(&ldsV[buffer][d][((tt >> 1) * 4u + quarter) * 8u + 4u * (tt & 1u)]) = bytes_to_f16(words[quarter]);
     }
-    if (tid < 2 * kStep) (tid < kStep ? ldsKS[buffer] : ldsVS[buffer])[tid & (kStep - 1)] = half_bits_to_float(scaleLoad);
+    // Key scales carry the softmax scale (log2 domain), value scales the 2^10 of P.
+    if (tid < 2 * kStep) (tid < kStep ? ldsKS[buffer] : ldsVS[buffer])[tid & (kStep - 1)] = half_bits_to_float(scaleLoad) * (tid < kStep ? scale2 : kPScale);
   };
 
   if (steps) {
@@ -253,11 +266,12 @@ __global__ __launch_bounds__(256) void attention_q8_split(const _Float16 *__rest
   }
   __syncthreads();
   const f16x8 ones = {_Float16(1.f), _Float16(1.f), _Float16(1.f), _Float16(1.f), _Float16(1.f), _Float16(1.f), _Float16(1.f), _Float16(1.f)};
-  for (uint32_t step = 0; step < steps; ++step) {
-    const uint32_t buffer = step & 1u, token0 = first + step * kStep;
-    if (step + 1 < steps) load(step + 1);
-
+  // One 64-token step. Masked steps (those that reach the block's own rows or the end of the
+  // sequence) test every score's visibility; the steps before them, all of the history, do not.
+  auto compute = [&](uint32_t buffer, uint32_t token0, auto maskedTag) {
+    constexpr bool kMasked = decltype(maskedTag)::value;
     // Scores, transposed: tile tt holds tokens 16 tt + 4 kq + i of the step for fused row `row`.
+    // The accumulator starts at -1152 sum(q), which takes the code offset out of the product.
     f32x4 s[kTiles][4];
 #pragma unroll
     for (int tt = 0; tt < 4; ++tt) {
@@ -266,13 +280,18 @@ __global__ __launch_bounds__(256) void attention_q8_split(const _Float16 *__rest
       for (int j = 0; j < JD; ++j) key[j] = *reinterpret_cast<const f16x8 *>(&ldsK[buffer][16 * tt + row][32 * j + 8 * kq]);
 #pragma unroll
       for (int k = 0; k < kTiles; ++k) {
-        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+        f32x4 acc = {qsum[k], qsum[k], qsum[k], qsum[k]};
 #pragma unroll
         for (int j = 0; j < JD; ++j) acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(key[j], q[k][j], acc, 0, 0, 0);
         s[k][tt] = acc;
       }
     }
-    const bool masked = token0 + kStep > seq.committed;  // the step reaches the block's own rows or the end
+    f32x4 keyScale[4], valueScale[4];
+#pragma unroll
+    for (int tt = 0; tt < 4; ++tt) {
+      keyScale[tt] = *reinterpret_cast<const f32x4 *>(&ldsKS[buffer][16 * tt + 4 * kq]);
+      valueScale[tt] = *reinterpret_cast<const f32x4 *>(&ldsVS[buffer][16 * tt + 4 * kq]);
+    }
     f16x8 pOperand[kTiles][2];
 #pragma unroll
     for (int k = 0; k < kTiles; ++k) {
@@ -281,9 +300,9 @@ __global__ __launch_bounds__(256) void attention_q8_split(const _Float16 *__rest
       for (int tt = 0; tt < 4; ++tt)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const uint32_t local = 16u * tt + 4u * kq + i, token = token0 + local;
-          float score = (s[k][tt][i] - qsum[k]) * (ldsKS[buffer][local] * scale2);
-          if (masked) {
+          float score = s[k][tt][i] * keyScale[tt][i];
+          if constexpr (kMasked) {
+            const uint32_t token = token0 + 16u * tt + 4u * kq + i;
             const bool visible = token < seq.committed || (token < total && ((ancestors >> (token - seq.committed)) & 1u));
             score = visible ? score : -INFINITY;
           }
@@ -296,15 +315,16 @@ __global__ __launch_bounds__(256) void attention_q8_split(const _Float16 *__rest
       const float alpha = __builtin_amdgcn_exp2f(m[k] - safeMax);
       m[k] = newMax;
       float sum = 0.f;
-      _Float16 weights[16];
+      float folded[16];
 #pragma unroll
       for (int tt = 0; tt < 4; ++tt)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const float pr = __builtin_amdgcn_exp2f(s[k][tt][i] - safeMax);
           sum += pr;
-          const float folded = pr * (ldsVS[buffer][16 * tt + 4 * kq + i] * kPScale);
-          weights[4 * tt + i] = _Float16(pr > 0.f ? folded : 0.f);
+          const float f = pr * valueScale[tt][i];
+          // A slot past the sequence's end may hold any scale: its weight is zero whatever it is.
+          folded[4 * tt + i] = kMasked ? (pr > 0.f ? f : 0.f) : f;
         }
       l[k] = l[k] * alpha + sum;
       // rescale the running output only when some row's maximum grew (paged_attention_tile.h:450-458)
@@ -316,8 +336,14 @@ __global__ __launch_bounds__(256) void attention_q8_split(const _Float16 *__rest
       }
 #pragma unroll
       for (int pair = 0; pair < 2; ++pair)
-        pOperand[k][pair] = f16x8{weights[8 * pair], weights[8 * pair + 1], weights[8 * pair + 2], weights[8 * pair + 3],
-                                  weights[8 * pair + 4], weights[8 * pair + 5], weights[8 * pair + 6], weights[8 * pair + 7]};
+#pragma unroll
+        for (int e = 0; e < 8; e += 2) {
+          typedef __attribute__((ext_vector_type(2))) float f32x2;
+          typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
+          const f16x2 two = __builtin_convertvector(f32x2{folded[8 * pair + e], folded[8 * pair + e + 1]}, f16x2);
+          pOperand[k][pair][e] = two[0];
+          pOperand[k][pair][e + 1] = two[1];
+        }
     }
     // Outputs, transposed: o[dt] holds dimensions 16 dt + 4 kq + i of fused row `row`.
 #pragma unroll
@@ -331,6 +357,21 @@ __global__ __launch_bounds__(256) void attention_q8_split(const _Float16 *__rest
 #pragma unroll
       for (int k = 0; k < kTiles; ++k) o[k][DT] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ones, pOperand[k][pair], o[k][DT], 0, 0, 0);
     }
+  };
+  // Steps wholly inside the committed history come first, in a loop of their own.
+  const uint32_t plain = first < seq.committed ? min(steps, (seq.committed - first) / kStep) : 0u;
+  uint32_t step = 0;
+  for (; step < plain; ++step) {
+    const uint32_t buffer = step & 1u;
+    if (step + 1 < steps) load(step + 1);
+    compute(buffer, first + step * kStep, std::false_type{});
+    if (step + 1 < steps) stage(buffer ^ 1u);
+    __syncthreads();
+  }
+  for (; step < steps; ++step) {
+    const uint32_t buffer = step & 1u;
+    if (step + 1 < steps) load(step + 1);
+    compute(buffer, first + step * kStep, std::true_type{});
     if (step + 1 < steps) stage(buffer ^ 1u);
     __syncthreads();
   }
@@ -365,30 +406,68 @@ SP_REGISTER_KERNEL("attention_q8_split_d128_g4", &attention_q8_split<128, 4>);
 SP_REGISTER_KERNEL("attention_q8_split_d64_g2", &attention_q8_split<64, 2>);
 
 // ---------------------------------------------------------------------------------------------
-// attention_reduce: grid (q_heads, 16, sequences), D threads. Merges the splits in split order
-// (paged_attention_tile.h:499-535) and writes bf16 [packed row][q_heads * D].
+// attention_reduce: grid (q_heads, 16, sequences), 256 threads. Merges the splits of one (head,
+// row) in a fixed order (paged_attention_tile.h:499-535) and writes bf16 [packed row][q_heads * D].
+// Thread (part, quad) sums splits part, part + P, ... of dimensions 4 quad .. 4 quad + 3, all its
+// loads in flight together; the P parts are then added in part order.
 // ---------------------------------------------------------------------------------------------
 template <int D>
-__global__ __launch_bounds__(D) void attention_reduce(const float *__restrict__ partialO, const float *__restrict__ partialML,
-                                                      uint16_t *__restrict__ out, AttentionParams p) {
+__global__ __launch_bounds__(256) void attention_reduce(const float *__restrict__ partialO, const float *__restrict__ partialML,
+                                                        uint16_t *__restrict__ out, AttentionParams p) {
+  constexpr uint32_t kQuads = D / 4, kParts = 256 / kQuads;
+  __shared__ float weights[ATTENTION_MAXIMUM_SPLITS];
+  __shared__ float scratch[4];
+  __shared__ __align__(16) float4 sums[kParts][kQuads];
   const uint32_t tid = threadIdx.x, head = blockIdx.x, row = blockIdx.y, z = blockIdx.z;
   const AttentionSequence seq = p.sequence[z];
   if (row >= seq.rows) return;
   const uint32_t group = p.q_heads / p.kv_heads, h = head / group, g = head % group, fusedRows = 16u * group;
   const size_t base = (size_t(z) * p.kv_heads + h) * p.splits;
-  float maximum = -INFINITY;
-  for (uint32_t s = 0; s < p.splits; ++s) maximum = fmaxf(maximum, partialML[2 * ((base + s) * fusedRows + 16u * g + row)]);
-  float numerator = 0.f, denominator = 0.f;
-  for (uint32_t s = 0; s < p.splits; ++s) {
-    const size_t fused = (base + s) * fusedRows + 16u * g + row;
-    const float ms = partialML[2 * fused];
-    if (ms == -INFINITY) continue;
-    const float weight = __builtin_amdgcn_exp2f(ms - maximum);
-    numerator += weight * partialO[fused * D + tid];
-    denominator += weight * partialML[2 * fused + 1];
+  auto fusedOf = [&](uint32_t s) { return (base + s) * fusedRows + 16u * g + row; };
+
+  // Split tid's maximum and sum; the block's maximum; the split's weight and its share of the denominator.
+  float ms = -INFINITY, ls = 0.f;
+  if (tid < p.splits) {
+    const float2 ml = *reinterpret_cast<const float2 *>(partialML + 2 * fusedOf(tid));
+    ms = ml.x;
+    ls = ml.y;
   }
-  const float value = denominator > 0.f ? numerator / denominator : 0.f;
-  out[(size_t(seq.first_row) + row) * (p.q_heads * D) + head * D + tid] = uint16_t(float_to_bf16_bits(value));
+  const float maximum = block_max<256>(ms, scratch, tid);
+  const float weight = ms == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ms - maximum);
+  if (tid < ATTENTION_MAXIMUM_SPLITS) weights[tid] = weight;
+  const float denominator = block_sum<256>(weight * ls, scratch, tid);  // block_sum's barriers publish the weights too
+
+  const uint32_t part = tid / kQuads, quad = tid % kQuads;
+  float4 total = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (uint32_t s0 = part; s0 < p.splits; s0 += 4u * kParts) {
+    float4 held[4];
+#pragma unroll
+    for (uint32_t i = 0; i < 4u; ++i) {
+      const uint32_t s = s0 + i * kParts;
+      held[i] = s < p.splits ? reinterpret_cast<const float4 *>(partialO + fusedOf(s) * D)[quad] : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+#pragma unroll
+    for (uint32_t i = 0; i < 4u; ++i) {
+      const uint32_t s = s0 + i * kParts;
+      const float w = s < p.splits ? weights[s] : 0.f;
+      if (w != 0.f) {  // a split without a visible token may hold anything
+        total.x += w * held[i].x;
+        total.y += w * held[i].y;
+        total.z += w * held[i].z;
+        total.w += w * held[i].w;
+      }
+    }
+  }
+  sums[part][quad] = total;
+  __syncthreads();
+  if (tid < D) {
+    const float *flat = reinterpret_cast<const float *>(&sums[0][0]);
+    float numerator = 0.f;
+#pragma unroll
+    for (uint32_t q = 0; q < kParts; ++q) numerator += flat[q * D + tid];
+    const float value = denominator > 0.f ? numerator / denominator : 0.f;
+    out[(size_t(seq.first_row) + row) * (p.q_heads * D) + head * D + tid] = uint16_t(float_to_bf16_bits(value));
+  }
 }
 SP_REGISTER_KERNEL("attention_reduce_d128", &attention_reduce<128>);
 SP_REGISTER_KERNEL("attention_reduce_d64", &attention_reduce<64>);

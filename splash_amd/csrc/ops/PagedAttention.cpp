@@ -128,7 +128,7 @@ void PagedAttention::addAttention(hip::CommandGraph &graph, const AttentionPlan 
             {w.queries, w.querySums, treeRows, pages.pageTable, pages.pool, w.partials, w.partialSums}, params,
             {g.kvHeads, plan.splits(), plan.sequences().size()}, {256, 1, 1});
   graph.add("attention_reduce" + kernelSuffix(g), {w.partials, w.partialSums, output}, params,
-            {g.qHeads, ATTENTION_MAXIMUM_ROWS, plan.sequences().size()}, {g.headDimension, 1, 1});
+            {g.qHeads, ATTENTION_MAXIMUM_ROWS, plan.sequences().size()}, {256, 1, 1});
 }
 
 void PagedAttention::addPathCommit(hip::CommandGraph &graph, const AttentionPlan &plan, const hip::Buffer &retained,
