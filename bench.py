@@ -197,7 +197,7 @@ def main():
     for total, name in totals[:8]:
         log(f"  {name:36s} x{len(by_kernel[name]):3d}  avg {total / len(by_kernel[name]) * 1e6:8.2f} us  total {total * 1e3:7.3f} ms")
     dominant = totals[0][1]
-    gate_up = [k for k in by_kernel if k.endswith("_g")][0]
+    gate_up = [k for k in by_kernel if k.endswith("_g") or k.endswith("_gt")][0]
     avg = sum(by_kernel[gate_up]) / len(by_kernel[gate_up])
     H, F = w["hidden"], w["ffn"]
     gate_up_bytes = 2 * F * H * 0.5625 + rows * H * 2 + rows * F * 2     # both tensors once + bf16 rows in and out

@@ -74,11 +74,14 @@ sp_status spo_linear_plan_with(const spo_projection *projection, spo_linear_plan
 sp_status spo_linear_add(const spo_linear *linear, spo_graph *graph, const spo_projection *projection,
                          const spo_projection *gate, const spo_linear_plan *plan, sp_buffer *input, sp_buffer *output,
                          sp_buffer *residual, sp_buffer *table, sp_buffer *partials, sp_buffer *counters, int prepared);
-/* Linear::addSwiGlu (Linear.hpp:352-354): output = residual + down(silu(gate x) * up x). */
+/* Linear::addSwiGlu (Linear.hpp:352-354): output = residual + down(silu(gate x) * up x).
+ * next_table (optional, spo_gguf_table_bytes(ffn, rows) bytes, not `table`): the gate/up pass
+ * then writes the down projection's activation table from its epilogue and no separate table
+ * pass is recorded; results are bit-identical either way. */
 sp_status spo_linear_add_swiglu(const spo_linear *linear, spo_graph *graph, const spo_projection *gate,
                                 const spo_projection *up, const spo_projection *down, sp_buffer *normalized,
                                 sp_buffer *intermediate, sp_buffer *residual, sp_buffer *output, uint32_t rows,
-                                sp_buffer *table, sp_buffer *partials, sp_buffer *counters);
+                                sp_buffer *table, sp_buffer *partials, sp_buffer *counters, sp_buffer *next_table);
 /* Linear::scratchSize (Linear.hpp:319): of every plan of up to `rows` rows of the matrix. */
 sp_status spo_linear_scratch_size(const spo_linear *linear, uint32_t output_size, uint32_t input_size, uint32_t rows,
                                   uint64_t *table, uint64_t *partials, uint64_t *counters);
@@ -110,11 +113,13 @@ sp_status spo_attention_add_projection(spo_graph *graph, const spo_attention_pla
                                        sp_buffer *query_norm, sp_buffer *key_norm, sp_buffer *rope_cos,
                                        sp_buffer *rope_sin, sp_buffer *queries, sp_buffer *query_sums,
                                        sp_buffer *page_table, sp_buffer *pool, uint64_t page_bytes);
-/* PagedAttention::addAttention (PagedAttention.cpp:466-607): split, then ordered reduce. */
+/* PagedAttention::addAttention (PagedAttention.cpp:466-607): split, then ordered reduce.
+ * output_table (optional, spo_gguf_table_bytes(q_heads * head_dim, rows) bytes): the reduce also
+ * writes the rows as the activation table of the projection that follows. */
 sp_status spo_attention_add_attention(spo_graph *graph, const spo_attention_plan *plan, sp_buffer *queries,
                                       sp_buffer *query_sums, sp_buffer *partials, sp_buffer *partial_sums,
                                       sp_buffer *tree_rows, sp_buffer *page_table, sp_buffer *pool, uint64_t page_bytes,
-                                      sp_buffer *output);
+                                      sp_buffer *output, sp_buffer *output_table);
 /* PagedAttention::addPathCommit (PagedAttention.cpp:647-667). */
 sp_status spo_attention_add_path_commit(spo_graph *graph, const spo_attention_plan *plan, sp_buffer *retained,
                                         sp_buffer *page_table, sp_buffer *pool, uint64_t page_bytes);

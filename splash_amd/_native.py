@@ -169,7 +169,7 @@ _sig("spo_linear_destroy", None, c_p)
 _sig("spo_linear_plan_for", c_int, c_p, c_p, c_u32, c_u32, P(LinearPlan))
 _sig("spo_linear_plan_with", c_int, c_p, P(LinearPlan))
 _sig("spo_linear_add", c_int, c_p, c_p, c_p, c_p, P(LinearPlan), c_p, c_p, c_p, c_p, c_p, c_p, c_int)
-_sig("spo_linear_add_swiglu", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_u32, c_p, c_p, c_p)
+_sig("spo_linear_add_swiglu", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_u32, c_p, c_p, c_p, c_p)
 _sig("spo_linear_scratch_size", c_int, c_p, c_u32, c_u32, c_u32, P(c_u64), P(c_u64), P(c_u64))
 
 _sig("spo_kv_page_bytes", c_u64, c_u32, c_u32)
@@ -180,7 +180,7 @@ _sig("spo_attention_plan_destroy", None, c_p)
 _sig("spo_attention_plan_splits", c_u32, c_p)
 _sig("spo_attention_workspace", c_int, c_p, P(c_u64))
 _sig("spo_attention_add_projection", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_u64)
-_sig("spo_attention_add_attention", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_u64, c_p)
+_sig("spo_attention_add_attention", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_u64, c_p, c_p)
 _sig("spo_attention_add_path_commit", c_int, c_p, c_p, c_p, c_p, c_p, c_u64)
 
 _sig("spo_norm_add_rms", c_int, c_p, c_p, c_p, c_p, c_u32, c_u32)

@@ -104,6 +104,9 @@ struct GgufPrepareParams {
 #define GGUF_EPILOGUE_PLAIN_F32 1u // out = v               kernel suffix _a_f32
 #define GGUF_EPILOGUE_RESIDUAL 2u  // out = bf16(v + res)   kernel suffix _r
 #define GGUF_EPILOGUE_GATE_UP 3u   // out = bf16(bf16(up) * silu(bf16(gate)))   kernel suffix _g
+// The same, and `out` also leaves as the next projection's activation table, written to the buffer
+// bound in the residual's place (columns a multiple of 256): kernel suffix _gt.
+#define GGUF_EPILOGUE_GATE_UP_TABLE 4u
 
 // gguf_decode_<fmt>_m<16|32|64>_<a|a_f32|r|g>: up to three column segments of one format in one
 // dispatch (the reference's GgufDecodeFusedParams, runtime/metal/abi/Gguf.h:168-178), tiles in

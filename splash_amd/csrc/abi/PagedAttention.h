@@ -80,7 +80,8 @@ struct AttentionParams {
   uint32_t qkv_stride;       // elements of a packed qkv row: (q_heads + 2 kv_heads) * head_dim
   uint32_t splits;           // grid.y of the split kernel: the most splits of any sequence
   uint32_t sequences;
-  uint32_t reserved[2];
+  uint32_t table_tiles;      // attention_reduce_*_t: row tiles of the activation table it writes
+  uint32_t reserved;
   uint64_t page_bytes;       // bytes between physical pages of the layer's pool
   struct AttentionSequence sequence[ATTENTION_MAXIMUM_SEQUENCES];
 };

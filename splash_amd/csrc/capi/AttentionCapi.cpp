@@ -58,13 +58,14 @@ sp_status spo_attention_add_projection(spo_graph *graph, const spo_attention_pla
 }
 sp_status spo_attention_add_attention(spo_graph *graph, const spo_attention_plan *plan, sp_buffer *queries, sp_buffer *query_sums,
                                       sp_buffer *partials, sp_buffer *partial_sums, sp_buffer *tree_rows, sp_buffer *page_table,
-                                      sp_buffer *pool, uint64_t page_bytes, sp_buffer *output) {
+                                      sp_buffer *pool, uint64_t page_bytes, sp_buffer *output, sp_buffer *output_table) {
   return capi::guard([&] {
     capi::require(graph && plan, "graph or plan");
     ops::AttentionWorkspace w{hip::Buffer::share(queries), hip::Buffer::share(query_sums), hip::Buffer::share(partials),
                               hip::Buffer::share(partial_sums)};
     ops::PagedAttention::addAttention(capi::graphOf(graph), plan->plan, w, hip::Buffer::share(tree_rows),
-                                      pagesOf(page_table, pool, page_bytes), hip::Buffer::share(output));
+                                      pagesOf(page_table, pool, page_bytes), hip::Buffer::share(output),
+                                      hip::Buffer::share(output_table));
   });
 }
 sp_status spo_attention_add_path_commit(spo_graph *graph, const spo_attention_plan *plan, sp_buffer *retained,

@@ -177,10 +177,11 @@ sp_status spo_linear_add(const spo_linear *linear, spo_graph *graph, const spo_p
 sp_status spo_linear_add_swiglu(const spo_linear *linear, spo_graph *graph, const spo_projection *gate,
                                 const spo_projection *up, const spo_projection *down, sp_buffer *normalized,
                                 sp_buffer *intermediate, sp_buffer *residual, sp_buffer *output, uint32_t rows,
-                                sp_buffer *table, sp_buffer *partials, sp_buffer *counters) {
+                                sp_buffer *table, sp_buffer *partials, sp_buffer *counters, sp_buffer *next_table) {
   return capi::guard([&] {
     capi::require(linear && graph && gate && up && down, "linear, graph or projections");
-    ops::FfnBuffers buffers{hip::Buffer::share(normalized), hip::Buffer::share(intermediate), scratchOf(table, partials, counters)};
+    ops::FfnBuffers buffers{hip::Buffer::share(normalized), hip::Buffer::share(intermediate), scratchOf(table, partials, counters),
+                            hip::Buffer::share(next_table)};
     linear->linear.addSwiGlu(graph->graph, {&gate->projection, &up->projection, &down->projection}, buffers,
                              hip::Buffer::share(residual), hip::Buffer::share(output), rows);
   });

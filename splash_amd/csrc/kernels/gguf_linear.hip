@@ -326,6 +326,7 @@ __global__ __launch_bounds__(256) void gguf_decode(const uint8_t *__restrict__ s
                                                    float *__restrict__ partials, uint32_t *__restrict__ counters,
                                                    GgufDecodeParams p) {
   constexpr uint32_t kRecord = FMT == GGUF_FMT_Q4K ? GGUF_Q4K_RECORD : GGUF_Q6K_RECORD;
+  constexpr bool kTable = EP == GGUF_EPILOGUE_GATE_UP_TABLE, kGateUp = EP == GGUF_EPILOGUE_GATE_UP || kTable;
   constexpr uint32_t kColumnPart = FMT == GGUF_FMT_Q4K ? 2048u : GGUF_Q6K_SCALES;
   constexpr uint32_t kSumsPerBlock = FMT == GGUF_FMT_Q4K ? 2 : 4;  // K = 4 MFMAs of row sums per super-block
   // The range's activations pass through LDS one super-block at a time (two buffers, one barrier
@@ -344,7 +345,7 @@ __global__ __launch_bounds__(256) void gguf_decode(const uint8_t *__restrict__ s
 
   TileRef tile{nullptr, 0};
   if (live) {
-    if constexpr (EP == GGUF_EPILOGUE_GATE_UP) {
+    if constexpr (kGateUp) {
       tile = {(unit & 1u ? seg1 : seg0) + size_t(unit >> 1) * blocks * kRecord, p.offset[0] + (unit >> 1) * GGUF_TILE_COLUMNS};
     } else {
       const uint8_t *const seg[3] = {seg0, seg1, seg2};
@@ -382,7 +383,8 @@ __global__ __launch_bounds__(256) void gguf_decode(const uint8_t *__restrict__ s
     // The table's values of row tile t, super-blocks b0..b1: one resource per row tile.
     Resource values[RT];
 #pragma unroll
-    for (int t = 0; t < RT; ++t) values[t] = make_resource(table + (size_t(t) * G + 8u * b0) * 1024u, count * 8192u);
+    for (int t = 0; t < RT; ++t)  // a row tile past the table's reads as zeros
+      values[t] = make_resource(table + (size_t(uint32_t(t) < tiles ? t : 0) * G + 8u * b0) * 1024u, uint32_t(t) < tiles ? count * 8192u : 0u);
     uint32_t share[2];  // vector j of a row tile's super-block: byte offset of this thread's
 #pragma unroll
     for (int j = 0; j < 2; ++j) share[j] = (threadIdx.x + 256u * j) * 16u;
@@ -483,7 +485,7 @@ __global__ __launch_bounds__(256) void gguf_decode(const uint8_t *__restrict__ s
     if (threadIdx.x == 0) __hip_atomic_store(&counters[blockIdx.x], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 
-  if constexpr (EP == GGUF_EPILOGUE_GATE_UP) {
+  if constexpr (kGateUp) {
     // The up wave hands its sums to the gate wave beside it through LDS (the staging buffers are free).
     float *exchange = reinterpret_cast<float *>(&ldsA[0][0][0][0]);
     __syncthreads();
@@ -494,17 +496,57 @@ __global__ __launch_bounds__(256) void gguf_decode(const uint8_t *__restrict__ s
         for (int v = 0; v < 4; ++v) exchange[((wave >> 1) * RT * 4u + t * 4 + v) * 64u + lane] = acc[t][v];
     }
     __syncthreads();
-    if ((wave & 1u) || !live) return;
-    uint16_t *o = static_cast<uint16_t *>(out);
+    // With the table epilogue the workgroup's 32 columns, one group of the next projection's
+    // inputs, also leave as that projection's activation table (abi/Gguf.h), as gguf_prepare_table
+    // would write them: tileOut[half][row tile][row][column] collects the bf16 results.
+    uint16_t *tileOut = reinterpret_cast<uint16_t *>(exchange + 2u * RT * 256u);
+    float *halfSums = reinterpret_cast<float *>(tileOut + 2u * RT * 256u);
+    const uint32_t half = wave >> 1;
+    if (!(wave & 1u)) {
+      uint16_t *o = static_cast<uint16_t *>(out);
 #pragma unroll
-    for (int t = 0; t < RT; ++t)
+      for (int t = 0; t < RT; ++t)
 #pragma unroll
-      for (int v = 0; v < 4; ++v) {
-        const uint32_t row = 16u * t + 4u * kq + v;
-        if (row >= p.rows) continue;
-        const float gate = round_bf16(acc[t][v]), up = round_bf16(exchange[((wave >> 1) * RT * 4u + t * 4 + v) * 64u + lane]);
-        o[size_t(row) * p.out_stride + tile.column + c] = uint16_t(float_to_bf16_bits(up * silu(gate)));
+        for (int v = 0; v < 4; ++v) {
+          const uint32_t row = 16u * t + 4u * kq + v;
+          uint32_t bits = 0;
+          if (live && row < p.rows) {
+            const float gate = round_bf16(acc[t][v]), up = round_bf16(exchange[(half * RT * 4u + t * 4 + v) * 64u + lane]);
+            bits = float_to_bf16_bits(up * silu(gate));
+            o[size_t(row) * p.out_stride + tile.column + c] = uint16_t(bits);
+          }
+          if constexpr (kTable) tileOut[((half * RT + t) * 16u + 4u * kq + v) * 16u + c] = uint16_t(bits);
+        }
+    }
+    if constexpr (kTable) {
+      __syncthreads();
+      uint8_t *next = reinterpret_cast<uint8_t *>(const_cast<uint16_t *>(residual));
+      const uint32_t G2 = p.out_stride / 32u, g = blockIdx.x;
+      uint2 *values = reinterpret_cast<uint2 *>(next);
+      float *sums32 = reinterpret_cast<float *>(next + gguf_table_sums32_offset(p.out_stride, tiles));
+      float *sums16 = reinterpret_cast<float *>(next + gguf_table_sums16_offset(p.out_stride, tiles));
+      // Piece (t, half, kq, r): inputs 16 half + 4 kq .. + 3 of row 16 t + r; a wave holds one (t, half).
+      for (uint32_t piece = threadIdx.x; piece < 2u * RT * 64u; piece += 256u) {
+        const uint32_t r = piece & 15u, q4 = (piece >> 4) & 3u, h2 = (piece >> 6) & 1u, t2 = piece >> 7;
+        if (t2 >= tiles) continue;  // a whole wave: the kernel's row tiles past the table's
+        const uint2 raw = *reinterpret_cast<const uint2 *>(&tileOut[((h2 * RT + t2) * 16u + r) * 16u + 4u * q4]);
+        const uint32_t x0 = raw.x & 0xFFFFu, x1 = raw.x >> 16, x2 = raw.y & 0xFFFFu, x3 = raw.y >> 16;
+        values[((size_t(t2) * G2 + g) * 64u + q4 * 16u + r) * 2u + h2] = make_uint2(x0 | (x2 << 16), x1 | (x3 << 16));
+        const float run = (bf16_bits_to_float(x0) + bf16_bits_to_float(x1)) + (bf16_bits_to_float(x2) + bf16_bits_to_float(x3));
+        const float r0 = __shfl(run, int(r), 64), r1 = __shfl(run, int(r) + 16, 64), r2 = __shfl(run, int(r) + 32, 64),
+                    r3 = __shfl(run, int(r) + 48, 64);
+        const float sum = ((r0 + r1) + r2) + r3;
+        if (q4 == 0) {
+          sums16[(size_t(t2) * 2u * G2 + 2u * g + h2) * 16u + r] = sum;
+          halfSums[(t2 * 2u + h2) * 16u + r] = sum;
+        }
       }
+      __syncthreads();
+      if (threadIdx.x < tiles * 16u) {
+        const uint32_t t2 = threadIdx.x >> 4, r = threadIdx.x & 15u;
+        sums32[(size_t(t2) * G2 + g) * 16u + r] = halfSums[(t2 * 2u) * 16u + r] + halfSums[(t2 * 2u + 1u) * 16u + r];
+      }
+    }
   } else {
     if (!live || !tile.image) return;
 #pragma unroll
@@ -526,7 +568,8 @@ __global__ __launch_bounds__(256) void gguf_decode(const uint8_t *__restrict__ s
   SP_REGISTER_KERNEL("gguf_decode_" fmt "_m" #rows "_a", &gguf_decode<FMT, RT, GGUF_EPILOGUE_PLAIN>);   \
   SP_REGISTER_KERNEL("gguf_decode_" fmt "_m" #rows "_a_f32", &gguf_decode<FMT, RT, GGUF_EPILOGUE_PLAIN_F32>); \
   SP_REGISTER_KERNEL("gguf_decode_" fmt "_m" #rows "_r", &gguf_decode<FMT, RT, GGUF_EPILOGUE_RESIDUAL>); \
-  SP_REGISTER_KERNEL("gguf_decode_" fmt "_m" #rows "_g", &gguf_decode<FMT, RT, GGUF_EPILOGUE_GATE_UP>)
+  SP_REGISTER_KERNEL("gguf_decode_" fmt "_m" #rows "_g", &gguf_decode<FMT, RT, GGUF_EPILOGUE_GATE_UP>);  \
+  SP_REGISTER_KERNEL("gguf_decode_" fmt "_m" #rows "_gt", &gguf_decode<FMT, RT, GGUF_EPILOGUE_GATE_UP_TABLE>)
 SP_GGUF_DECODE("q4k", GGUF_FMT_Q4K, 16, 1);
 SP_GGUF_DECODE("q4k", GGUF_FMT_Q4K, 32, 2);
 SP_GGUF_DECODE("q4k", GGUF_FMT_Q4K, 64, 4);

@@ -18,6 +18,7 @@
 // from one more MFMA against a tile of ones. Scores are kept transposed (tokens x rows) so that a
 // lane owns one fused row from the first MFMA to the last: row maxima, sums and rescales never
 // cross lanes except over the four lanes that share a row.
+#include "abi/Gguf.h"
 #include "abi/PagedAttention.h"
 #include "backend/KernelRegistry.hpp"
 #include "kernels/device_common.hpp"
@@ -411,13 +412,17 @@ SP_REGISTER_KERNEL("attention_q8_split_d64_g2", &attention_q8_split<64, 2>);
 // Thread (part, quad) sums splits part, part + P, ... of dimensions 4 quad .. 4 quad + 3, all its
 // loads in flight together; the P parts are then added in part order.
 // ---------------------------------------------------------------------------------------------
-template <int D>
+// The _t variant also writes the rows as the activation table (abi/Gguf.h) of the projection that
+// follows, as gguf_prepare_table would from `out`; p.table_tiles is the table's row tiles. Rows of
+// a tile past the packed rows keep what the table held.
+template <int D, bool Table>
 __global__ __launch_bounds__(256) void attention_reduce(const float *__restrict__ partialO, const float *__restrict__ partialML,
-                                                        uint16_t *__restrict__ out, AttentionParams p) {
+                                                        uint16_t *__restrict__ out, uint8_t *__restrict__ table, AttentionParams p) {
   constexpr uint32_t kQuads = D / 4, kParts = 256 / kQuads;
   __shared__ float weights[ATTENTION_MAXIMUM_SPLITS];
   __shared__ float scratch[4];
   __shared__ __align__(16) float4 sums[kParts][kQuads];
+  __shared__ uint16_t staged[D];
   const uint32_t tid = threadIdx.x, head = blockIdx.x, row = blockIdx.y, z = blockIdx.z;
   const AttentionSequence seq = p.sequence[z];
   if (row >= seq.rows) return;
@@ -466,11 +471,36 @@ __global__ __launch_bounds__(256) void attention_reduce(const float *__restrict_
 #pragma unroll
     for (uint32_t q = 0; q < kParts; ++q) numerator += flat[q * D + tid];
     const float value = denominator > 0.f ? numerator / denominator : 0.f;
-    out[(size_t(seq.first_row) + row) * (p.q_heads * D) + head * D + tid] = uint16_t(float_to_bf16_bits(value));
+    const uint32_t bits = float_to_bf16_bits(value);
+    out[(size_t(seq.first_row) + row) * (p.q_heads * D) + head * D + tid] = uint16_t(bits);
+    if constexpr (Table) staged[tid] = uint16_t(bits);
+  }
+  if constexpr (Table) {
+    __syncthreads();
+    if (tid < D / 4u) {
+      // Run q: inputs 4 q .. 4 q + 3 of the packed row (norm_rms_table16 writes the same pieces).
+      const uint32_t width = p.q_heads * D, G = width / 32u, q = head * (D / 4u) + tid;
+      const uint32_t packed = seq.first_row + row, tile = packed / 16u, r = packed % 16u;
+      const uint32_t x0 = staged[4 * tid], x1 = staged[4 * tid + 1], x2 = staged[4 * tid + 2], x3 = staged[4 * tid + 3];
+      const uint32_t g = q / 8u, half = (q / 4u) % 2u, kq = q % 4u;
+      reinterpret_cast<uint2 *>(table)[((size_t(tile) * G + g) * 64u + kq * 16u + r) * 2u + half] = make_uint2(x0 | (x2 << 16), x1 | (x3 << 16));
+      float s = (bf16_bits_to_float(x0) + bf16_bits_to_float(x1)) + (bf16_bits_to_float(x2) + bf16_bits_to_float(x3));
+      const float s1 = __shfl_down(s, 1, 64), s2 = __shfl_down(s, 2, 64), s3 = __shfl_down(s, 3, 64);
+      s = ((s + s1) + s2) + s3;
+      const float other = __shfl_down(s, 4, 64);
+      if (kq == 0) {
+        float *sums32 = reinterpret_cast<float *>(table + gguf_table_sums32_offset(width, p.table_tiles));
+        float *sums16 = reinterpret_cast<float *>(table + gguf_table_sums16_offset(width, p.table_tiles));
+        sums16[(size_t(tile) * 2u * G + 2u * g + half) * 16u + r] = s;
+        if (half == 0) sums32[(size_t(tile) * G + g) * 16u + r] = s + other;
+      }
+    }
   }
 }
-SP_REGISTER_KERNEL("attention_reduce_d128", &attention_reduce<128>);
-SP_REGISTER_KERNEL("attention_reduce_d64", &attention_reduce<64>);
+SP_REGISTER_KERNEL("attention_reduce_d128", &attention_reduce<128, false>);
+SP_REGISTER_KERNEL("attention_reduce_d64", &attention_reduce<64, false>);
+SP_REGISTER_KERNEL("attention_reduce_d128_t", &attention_reduce<128, true>);
+SP_REGISTER_KERNEL("attention_reduce_d64_t", &attention_reduce<64, true>);
 
 // ---------------------------------------------------------------------------------------------
 // attention_q8_commit: grid (kv_heads, sequences, layers), D threads. retained[z] is the mask of the block

@@ -60,6 +60,8 @@ DenseVerify::DenseVerify(hip::Backend &backend, DenseDimensions d, uint32_t maxL
   scratch_.input = device(size.input, "linear table");
   scratch_.partials = device(size.partials, "linear partials");
   scratch_.counters = device(std::max<uint64_t>(size.counters, 4), "linear counters");
+  // The attention merge and the gate/up pass write the table of the projection after them here.
+  nextTable_ = device(gguf_table_bytes(std::max(d.attentionWidth(), d.ffn), gguf_row_tiles(maxRows_)), "linear table 2");
   // Attention workspace for the most splits any sequence may take.
   const uint64_t fused = uint64_t{maxLanes} * d.kvHeads * (d.qHeads / d.kvHeads) * 16;
   maxSplits_ = ATTENTION_MAXIMUM_SPLITS;
@@ -118,11 +120,18 @@ void DenseVerify::encodeLayer(hip::CommandGraph &graph, uint32_t layer, const op
   const ops::KvPages pages{pageTable_, kvPools_.at(layer), pageBytes_};
   ops::AttentionProjectionBuffers projection{qkv_, w.queryNorm, w.keyNorm, ropeCos_, ropeSin_};
   ops::PagedAttention::addProjection(graph, plan, projection, attentionWorkspace_, pages);
-  ops::PagedAttention::addAttention(graph, plan, attentionWorkspace_, treeRows_, pages, attention_);
-  linear_.addResidualProjection(graph, attention_, w.output, residual, next, rows, scratch_);
+  ops::PagedAttention::addAttention(graph, plan, attentionWorkspace_, treeRows_, pages, attention_, nextTable_);
+  ops::LinearBuffers output;
+  output.input = attention_;
+  output.output = next;
+  output.residual = residual;
+  output.scratch = scratch_;
+  output.scratch.input = nextTable_;
+  output.prepared = {attention_, ops::LinearInput::Table16};
+  linear_.add(graph, output, w.output, linear_.plan(w.output, rows, ops::LinearEpilogue::Residual));
   // FFN block: hidden[0] = hidden[1] + down(silu(gate n) * up n), n = norm(hidden[1]).
   prepared = ops::Normalization::addRmsTable(graph, next, w.postNorm, normalized_, scratch_, dims_.hidden, rows);
-  const ops::FfnBuffers ffn{normalized_, intermediate_, scratch_};
+  const ops::FfnBuffers ffn{normalized_, intermediate_, scratch_, nextTable_};
   linear_.addSwiGlu(graph, {&w.gate, &w.up, &w.down}, ffn, next, residual, rows, prepared);
 }
 

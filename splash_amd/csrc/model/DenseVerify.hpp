@@ -96,6 +96,7 @@ private:
   hip::Buffer pageTable_;
   std::vector<hip::Buffer> kvPools_;
   ops::LinearScratch scratch_;
+  hip::Buffer nextTable_;
   ops::AttentionWorkspace attentionWorkspace_;
   ops::SamplingBuffers sampling_;
   uint32_t maxSplits_ = 0;

@@ -13,7 +13,8 @@ void requireBytes(const hip::Buffer &buffer, uint64_t bytes, const char *what) {
 
 namespace {
 
-const char *epilogueSuffix(LinearEpilogue epilogue, FloatOutput destination) {
+const char *epilogueSuffix(LinearEpilogue epilogue, FloatOutput destination, bool table = false) {
+  if (epilogue == LinearEpilogue::GateUp && table) return "_gt";
   switch (epilogue) {
   case LinearEpilogue::None: return destination == FloatOutput::Float32 ? "_a_f32" : "_a";
   case LinearEpilogue::Residual: return "_r";
@@ -149,6 +150,13 @@ PreparedInput Linear::add(hip::CommandGraph &graph, LinearBuffers b, const Proje
     requireBytes(b.scratch.partials, need.partials, "projection partials");
     requireBytes(b.scratch.counters, need.counters, "projection counters");
   }
+  const bool writesTable = gateUp && bool(b.nextTable);
+  if (b.nextTable && !gateUp) throw std::invalid_argument("only a block gate/up plan writes the next projection's table");
+  if (writesTable) {
+    if (n % GGUF_BLOCK) throw std::invalid_argument("a table epilogue takes whole super-blocks of output columns");
+    requireBytes(b.nextTable, gguf_table_bytes(n, tiles), "next projection table");
+    if (b.nextTable.sameView(b.scratch.input)) throw std::invalid_argument("the next projection's table is not the plan's own");
+  }
   const bool prepared = b.prepared.layout == LinearInput::Table16 && b.prepared.source && b.input &&
                         b.prepared.source.sameView(b.input);
   if (!prepared) requireBytes(b.input, uint64_t{w.rows} * k * 2, "projection input");
@@ -181,10 +189,11 @@ PreparedInput Linear::add(hip::CommandGraph &graph, LinearBuffers b, const Proje
   // Unused bindings still name a buffer: the table stands in for them.
   const hip::Buffer &spare = b.scratch.input;
   const std::string name = std::string("gguf_decode_") + segments.front().name() + "_m" + std::to_string(plan.storageRows()) +
-                           epilogueSuffix(w.epilogue, plan.destination());
+                           epilogueSuffix(w.epilogue, plan.destination(), writesTable);
   graph.add(name,
             {images[0], images[1], images[2], b.scratch.input, b.output,
-             w.epilogue == LinearEpilogue::Residual ? b.residual : spare, c.splits > 1 ? b.scratch.partials : spare,
+             w.epilogue == LinearEpilogue::Residual ? b.residual : writesTable ? b.nextTable : spare,
+             c.splits > 1 ? b.scratch.partials : spare,
              c.splits > 1 ? b.scratch.counters : spare},
             params, {groupsOf(n, w.epilogue), c.splits, 1}, {256, 1, 1});
   (void)tiles;
@@ -224,6 +233,11 @@ void Linear::addSwiGlu(hip::CommandGraph &graph, const SwiGluProjections &ffn, c
   down.output = std::move(output);
   down.residual = std::move(residual);
   down.scratch = b.scratch;
+  if (b.nextTable) {
+    pair.nextTable = b.nextTable;
+    down.scratch.input = b.nextTable;
+    down.prepared = {b.intermediate, LinearInput::Table16};
+  }
   const LinearPlan downPlan = plan(*ffn.down, rows, LinearEpilogue::Residual);
   add(graph, std::move(pair), *ffn.up, pairPlan, ffn.gate);
   add(graph, std::move(down), *ffn.down, downPlan);

@@ -78,6 +78,9 @@ struct SwiGluProjections final {
 struct FfnBuffers final {
   hip::Buffer normalized, intermediate;
   LinearScratch scratch;
+  // Optional second activation table: the gate/up pass then writes the down projection's table
+  // from its epilogue and the separate table pass is dropped.
+  hip::Buffer nextTable{};
 };
 
 enum class LinearInput : uint8_t {
@@ -114,6 +117,8 @@ struct LinearBuffers final {
   hip::Buffer residual;
   LinearScratch scratch{};
   PreparedInput prepared{};
+  // Gate/up plans only: where the epilogue also writes `output` as an activation table.
+  hip::Buffer nextTable{};
 };
 
 // What the plans read of the device (the reference's KernelCalibration, ops/KernelCalibration.hpp):

@@ -112,7 +112,8 @@ void PagedAttention::addProjection(hip::CommandGraph &graph, const AttentionPlan
 }
 
 void PagedAttention::addAttention(hip::CommandGraph &graph, const AttentionPlan &plan, const AttentionWorkspace &w,
-                                  const hip::Buffer &treeRows, const KvPages &pages, const hip::Buffer &output) {
+                                  const hip::Buffer &treeRows, const KvPages &pages, const hip::Buffer &output,
+                                  const hip::Buffer &outputTable) {
   const AttentionGeometry &g = plan.geometry();
   const uint32_t rows = totalRows(plan.sequences());
   const AttentionWorkspaceSize need = plan.workspace();
@@ -123,11 +124,18 @@ void PagedAttention::addAttention(hip::CommandGraph &graph, const AttentionPlan 
   requireBytes(treeRows, uint64_t{rows} * sizeof(AttentionTreeRow), "verify tree rows");
   requireBytes(output, uint64_t{rows} * g.qHeads * g.headDimension * 2, "attention output");
   requirePages(plan, pages);
-  const AttentionParams params = plan.params(pages.pageBytes);
+  AttentionParams params = plan.params(pages.pageBytes);
+  const uint32_t width = g.qHeads * g.headDimension;
+  if (outputTable) {
+    if (width % GGUF_BLOCK) throw std::invalid_argument("an attention output table holds whole super-blocks");
+    params.table_tiles = gguf_row_tiles(rows);
+    requireBytes(outputTable, gguf_table_bytes(width, params.table_tiles), "attention output table");
+  }
   graph.add("attention_q8_split" + kernelSuffix(g) + "_g" + std::to_string(g.group()),
             {w.queries, w.querySums, treeRows, pages.pageTable, pages.pool, w.partials, w.partialSums}, params,
             {g.kvHeads, plan.splits(), plan.sequences().size()}, {256, 1, 1});
-  graph.add("attention_reduce" + kernelSuffix(g), {w.partials, w.partialSums, output}, params,
+  graph.add("attention_reduce" + kernelSuffix(g) + (outputTable ? "_t" : ""),
+            {w.partials, w.partialSums, output, outputTable ? outputTable : output}, params,
             {g.qHeads, ATTENTION_MAXIMUM_ROWS, plan.sequences().size()}, {256, 1, 1});
 }
 

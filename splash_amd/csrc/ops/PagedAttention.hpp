@@ -95,8 +95,11 @@ public:
   static void addProjection(hip::CommandGraph &graph, const AttentionPlan &plan, const AttentionProjectionBuffers &buffers,
                             const AttentionWorkspace &workspace, const KvPages &pages);
   // Split + reduce (PagedAttention.cpp:466-607): output bf16 [packed rows][q heads * D].
+  // outputTable (optional): the reduce also writes the rows as the activation table of the
+  // projection that follows (gguf_table_bytes(q heads * D, rows)), which then needs no table pass.
   static void addAttention(hip::CommandGraph &graph, const AttentionPlan &plan, const AttentionWorkspace &workspace,
-                           const hip::Buffer &treeRows, const KvPages &pages, const hip::Buffer &output);
+                           const hip::Buffer &treeRows, const KvPages &pages, const hip::Buffer &output,
+                           const hip::Buffer &outputTable = {});
   // Moves the retained path's slots to their depths (PagedAttention.cpp:647-667); retained is a
   // uint32 mask per sequence.
   // `layers` pools lie layerBytes apart from pages.pool (one dispatch commits them all, as the

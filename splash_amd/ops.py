@@ -126,11 +126,14 @@ class Linear:
                                  scratch.counters.handle, int(prepared)))
         graph._keep.extend([projection, gate, input, output, residual, scratch])
 
-    def add_swiglu(self, graph, gate, up, down, normalized, intermediate, residual, output, rows, scratch):
+    def add_swiglu(self, graph, gate, up, down, normalized, intermediate, residual, output, rows, scratch, next_table=None):
+        """next_table: a second activation table (gguf_table_bytes(ffn, rows)); the gate/up pass then writes
+        the down projection's table itself."""
         check(lib.spo_linear_add_swiglu(self.handle, graph.handle, gate.handle, up.handle, down.handle, normalized.handle,
                                         intermediate.handle, residual.handle, output.handle, rows, scratch.table.handle,
-                                        scratch.partials.handle, scratch.counters.handle))
-        graph._keep.extend([gate, up, down, normalized, intermediate, residual, output, scratch])
+                                        scratch.partials.handle, scratch.counters.handle,
+                                        next_table.handle if next_table is not None else None))
+        graph._keep.extend([gate, up, down, normalized, intermediate, residual, output, scratch, next_table])
 
     def scratch_size(self, output_size, input_size, rows):
         t, s, c = ctypes.c_uint64(), ctypes.c_uint64(), ctypes.c_uint64()
@@ -243,11 +246,12 @@ class PagedAttention:
         graph._keep.extend([plan, qkv, workspace, pages, query_norm, key_norm, rope_cos, rope_sin])
 
     @staticmethod
-    def add_attention(graph, plan, workspace, tree_rows, pages, output):
+    def add_attention(graph, plan, workspace, tree_rows, pages, output, output_table=None):
         check(lib.spo_attention_add_attention(graph.handle, plan.handle, workspace.queries.handle, workspace.query_sums.handle,
                                               workspace.partials.handle, workspace.partial_sums.handle, tree_rows.handle,
-                                              pages.table.handle, pages.pool.handle, pages.page_bytes, output.handle))
-        graph._keep.extend([plan, workspace, tree_rows, pages, output])
+                                              pages.table.handle, pages.pool.handle, pages.page_bytes, output.handle,
+                                              output_table.handle if output_table is not None else None))
+        graph._keep.extend([plan, workspace, tree_rows, pages, output, output_table])
 
     @staticmethod
     def add_path_commit(graph, plan, retained, pages):

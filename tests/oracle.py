@@ -233,3 +233,39 @@ def rejection_law(logits, temperature, q):
     out = np.empty(x.size, dtype=np.float64)
     lib.orc_rejection_law(_p(x, f32p), c_u32(x.size), c_f(temperature), _p(qq, f32p), _p(out, f64p))
     return out
+
+
+def activation_table(x_bits, tiles=None):
+    """The activation table of bf16 rows [M][K] (K a multiple of 32) as the projection kernels read it:
+    values uint16 [tiles][K/32][64][8] (lane kq*16 + r holds inputs 16 (e//4) + 4 kq + (0,2,1,3)[e%4] of
+    the group for row 16 t + r), fp32 sums of each row's 32 inputs [tiles][K/32][16] and 16 inputs
+    [tiles][K/16][16], added in input order: runs of four as (x0 + x1) + (x2 + x3), the four runs of a
+    half in order, then the two halves. Rows past M are zero. Returns (values, sums32, sums16)."""
+    M, K = x_bits.shape
+    tiles = tiles or (M + 15) // 16
+    G = K // 32
+    x = np.zeros((tiles * 16, K), dtype=np.uint16)
+    x[:M] = x_bits
+    order = np.array([0, 2, 1, 3])
+    e = np.arange(8)
+    kq = np.arange(4)
+    inputs = 16 * (e[None, :] // 4) + 4 * kq[:, None] + order[e[None, :] % 4]      # [kq][e]
+    grouped = x.reshape(tiles, 16, G, 32)                                          # [t][r][g][i]
+    values = grouped[:, :, :, inputs]                                              # [t][r][g][kq][e]
+    values = np.ascontiguousarray(values.transpose(0, 2, 3, 1, 4)).reshape(tiles, G, 64, 8)
+    f = bf16_to_f32(x).reshape(tiles, 16, 2 * G, 4, 4)                             # [t][r][half block][run][i]
+    runs = (f[..., 0] + f[..., 1]) + (f[..., 2] + f[..., 3])
+    s16 = ((runs[..., 0] + runs[..., 1]) + runs[..., 2]) + runs[..., 3]            # [t][r][2G]
+    s32 = s16[..., 0::2] + s16[..., 1::2]
+    return values, np.ascontiguousarray(s32.transpose(0, 2, 1)), np.ascontiguousarray(s16.transpose(0, 2, 1))
+
+
+def split_activation_table(raw_bytes, K, tiles):
+    """(values, sums32, sums16) views of a table downloaded as bytes."""
+    G = K // 32
+    nv = tiles * K * 16 * 2
+    n32 = tiles * G * 16 * 4
+    values = raw_bytes[:nv].view(np.uint16).reshape(tiles, G, 64, 8)
+    s32 = raw_bytes[nv:nv + n32].view(np.float32).reshape(tiles, G, 16)
+    s16 = raw_bytes[nv + n32:nv + 3 * n32].view(np.float32).reshape(tiles, 2 * G, 16)
+    return values, s32, s16

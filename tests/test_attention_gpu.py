@@ -165,6 +165,36 @@ def test_batched_sequences_equal_each_alone(backend):
         assert np.array_equal(together[s[0]:s[0] + s[1]], alone[s[0]:s[0] + s[1]])
 
 
+@pytest.mark.parametrize("rows,committed", [(16, 300), (5, 1000)])
+def test_attention_output_table(backend, rows, committed):
+    """The split merge may also write its rows as the next projection's activation table: the rows are
+    unchanged and the table is the one they define."""
+    print(f"case attention output table rows={rows}", flush=True)
+    rng = np.random.default_rng(77)
+    q_heads, kv_heads, D = 16, 8, 64
+    kv, _, _ = build_context(rng, backend, q_heads, kv_heads, D, rows, committed)
+    qkv = backend.from_array(orc.f32_to_bf16(rng.standard_normal((rows, (q_heads + 2 * kv_heads) * D)).astype(np.float32)))
+    plan = ops.AttentionPlan(q_heads, kv_heads, D, [(0, rows, committed, 0)])
+    ws = ops.AttentionWorkspace(backend, plan)
+    tree = backend.from_array(ops.chain_tree_rows([rows]))
+    width = q_heads * D
+    outs = []
+    for fused in (False, True):
+        out = backend.allocate_buffer(rows * width * 2)
+        table = backend.allocate_buffer(ops.gguf_table_bytes(width, rows)) if fused else None
+        graph = splash_amd.CommandGraph()
+        ops.PagedAttention.add_projection(graph, plan, qkv, ws, kv)
+        ops.PagedAttention.add_attention(graph, plan, ws, tree, kv, out, output_table=table)
+        backend.run(graph)
+        outs.append(out.download(np.uint16).reshape(rows, width))
+    assert np.array_equal(outs[0], outs[1])
+    values, s32, s16 = orc.split_activation_table(table.download(np.uint8), width, 1)
+    wv, w32, w16 = orc.activation_table(outs[1])
+    live = np.arange(64) % 16 < rows   # rows of the tile past the block keep what the table held (zeros here)
+    assert np.array_equal(values[:, :, live], wv[:, :, live])
+    assert s32[..., :rows].tobytes() == w32[..., :rows].tobytes() and s16[..., :rows].tobytes() == w16[..., :rows].tobytes()
+
+
 def test_path_commit_moves_the_retained_rows(backend):
     """kv_path_commit.metal:21-48: the k-th retained row's slot moves to depth k; a chain is a no-op."""
     print("case attention commit", flush=True)

@@ -151,6 +151,43 @@ def test_residual_and_gate_up_epilogues(backend, fmt):
     assert diff.max() <= 1 and (diff > 0).mean() < 0.02, (diff.max(), (diff > 0).mean())
 
 
+@pytest.mark.parametrize("M", [16, 5, 40])
+def test_gate_up_table_epilogue_equals_the_table_pass(backend, M):
+    """The one-pass gate/up may write the down projection's activation table from its epilogue: table,
+    intermediate rows and the block's output are bit-identical to the path with a separate table pass,
+    and the table is the one the rows define."""
+    print(f"case swiglu table epilogue M={M}", flush=True)
+    rng = np.random.default_rng(31 + M)
+    hidden, ffn = 1024, 768
+    linear = ops.Linear(backend)
+    gate = ops.Projection.from_native(backend, [(ops.FMT_Q4K, ffn, orc.make_native(ops.FMT_Q4K, ffn, hidden, 5))], hidden)
+    up = ops.Projection.from_native(backend, [(ops.FMT_Q4K, ffn, orc.make_native(ops.FMT_Q4K, ffn, hidden, 6))], hidden)
+    down = ops.Projection.from_native(backend, [(ops.FMT_Q6K, hidden, orc.make_native(ops.FMT_Q6K, hidden, ffn, 7))], ffn)
+    x = backend.from_array(orc.f32_to_bf16(rng.standard_normal((M, hidden)).astype(np.float32)))
+    res = backend.from_array(orc.f32_to_bf16(rng.standard_normal((M, hidden)).astype(np.float32)))
+    tiles = (M + 15) // 16
+    results = []
+    for fused in (False, True):
+        sizes = [linear.scratch_size(ffn, hidden, M), linear.scratch_size(hidden, ffn, M)]
+        scratch = ops.LinearScratch(backend, *[max(s[i] for s in sizes) for i in range(3)])
+        table2 = backend.allocate_buffer(ops.gguf_table_bytes(ffn, M)) if fused else None
+        mid = backend.allocate_buffer(M * ffn * 2)
+        out = backend.allocate_buffer(M * hidden * 2)
+        graph = splash_amd.CommandGraph()
+        linear.add_swiglu(graph, gate, up, down, x, mid, res, out, M, scratch, next_table=table2)
+        assert len(graph) == (3 if fused else 4)
+        backend.run(graph)
+        table = (table2 if fused else scratch.table).download(np.uint8)[:ops.gguf_table_bytes(ffn, M)]
+        results.append((mid.download(np.uint16).reshape(M, ffn), out.download(np.uint16), table))
+    assert np.array_equal(results[0][0], results[1][0])
+    assert np.array_equal(results[0][1], results[1][1])
+    for mid, _, table in results:
+        values, s32, s16 = orc.split_activation_table(table, ffn, tiles)
+        wv, w32, w16 = orc.activation_table(mid)
+        assert np.array_equal(values, wv)
+        assert s32.tobytes() == w32.tobytes() and s16.tobytes() == w16.tobytes()
+
+
 def test_linear_rejects_bad_buffers_before_adding_anything(backend):
     """Operators throw std::invalid_argument before any dispatch is added (LinearGguf.cpp:126-163)."""
     native = orc.make_native(ops.FMT_Q4K, 32, 512, 1)
