@@ -58,7 +58,7 @@ void spo_linear_destroy(spo_linear *linear);
 /* LinearEpilogue (Linear.hpp:77): 0 None, 1 Residual, 2 GateUp. */
 typedef struct spo_linear_plan {
   uint32_t rows, epilogue;
-  uint32_t splits, k_waves; /* LinearConfig */
+  uint32_t splits, whole_groups; /* LinearConfig: K partitions, and the leading workgroups that take K whole */
   uint32_t storage_rows;    /* LinearPlan::storageRows */
   uint32_t float32;         /* LinearPlan::destination */
   uint64_t scratch_input, scratch_partials, scratch_counters; /* LinearPlan::scratchSize */
@@ -67,7 +67,7 @@ typedef struct spo_linear_plan {
 sp_status spo_linear_plan_for(const spo_linear *linear, const spo_projection *projection, uint32_t rows, uint32_t epilogue,
                               spo_linear_plan *out);
 /* Linear::plan(workload, config, destination) (Linear.hpp:327-328): the plan of a given configuration;
- * fills storage_rows and scratch sizes from rows, epilogue, splits, k_waves, float32. */
+ * fills storage_rows and scratch sizes from rows, epilogue, splits, whole_groups, float32. */
 sp_status spo_linear_plan_with(const spo_projection *projection, spo_linear_plan *plan);
 /* Linear::add (Linear.hpp:330-332). table/partials/counters are the LinearScratch; `prepared`
  * nonzero says the table already holds `input` (PreparedInput). gate only for a GateUp plan. */

@@ -111,12 +111,12 @@ struct GgufPrepareParams {
 // gguf_decode_<fmt>_m<16|32|64>_<a|a_f32|r|g>: up to three column segments of one format in one
 // dispatch (the reference's GgufDecodeFusedParams, runtime/metal/abi/Gguf.h:168-178), tiles in
 // segment order; a single tensor is one segment. A gate/up pair binds gate as segment 0 and up as
-// segment 1, both of cols[0] columns. Grid (units / 4, splits), 256 threads: a wave per unit.
+// segment 1, both of cols[0] columns. Grid (whole_groups + (groups - whole_groups) * splits), 256 threads: a wave per unit.
 struct GgufDecodeParams {
   uint32_t input_size;  // K
   uint32_t rows;        // live rows
-  uint32_t splits;      // K partitions across workgroups (grid.y); 1 = no cross-workgroup reduction
-  uint32_t k_waves;     // waves of a workgroup that split its K partition between them: 1
+  uint32_t splits;      // K partitions of the workgroups past the whole ones; 1 = no cross-workgroup reduction
+  uint32_t whole_groups;  // leading workgroups (four units each) that walk all of K; the others take one of `splits` parts
   uint32_t out_stride;  // columns of a destination row
   uint32_t cols[3];     // columns per segment (multiples of 16); 0 past the last
   uint32_t offset[3];   // first destination column per segment

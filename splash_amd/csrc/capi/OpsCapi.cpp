@@ -17,7 +17,7 @@ ops::LinearPlan toPlan(const ops::Projection &projection, const spo_linear_plan 
   if (p.epilogue > 2) throw std::invalid_argument("unknown linear epilogue");
   ops::LinearConfig config;
   config.splits = p.splits;
-  config.kWaves = p.k_waves;
+  config.wholeGroups = p.whole_groups;
   return ops::Linear::plan(ops::LinearWorkload{{projection.outputSize, projection.inputSize}, p.rows,
                                                static_cast<ops::LinearEpilogue>(p.epilogue)},
                            config, p.float32 ? ops::FloatOutput::Float32 : ops::FloatOutput::BFloat16);
@@ -27,7 +27,7 @@ void fromPlan(const ops::LinearPlan &plan, spo_linear_plan *out) {
   out->rows = plan.workload().rows;
   out->epilogue = uint32_t(plan.workload().epilogue);
   out->splits = plan.configuration().splits;
-  out->k_waves = plan.configuration().kWaves;
+  out->whole_groups = plan.configuration().wholeGroups;
   out->storage_rows = plan.storageRows();
   out->float32 = plan.destination() == ops::FloatOutput::Float32;
   out->scratch_input = size.input;

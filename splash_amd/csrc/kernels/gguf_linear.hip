@@ -337,8 +337,15 @@ __global__ __launch_bounds__(256) void gguf_decode(const uint8_t *__restrict__ s
   __shared__ uint32_t arrived;
 
   const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6, c = lane & 15u, kq = lane >> 4;
-  const uint32_t unit = blockIdx.x * 4u + wave;
-  const uint32_t split = blockIdx.y;
+  // Workgroup items: the whole groups first, then the partitioned ones part by part.
+  uint32_t group = blockIdx.x, split = 0, splits = 1;
+  if (blockIdx.x >= p.whole_groups && p.splits > 1) {
+    const uint32_t past = blockIdx.x - p.whole_groups;
+    group = p.whole_groups + uint32_t(__builtin_amdgcn_readfirstlane(int(past / p.splits)));
+    split = uint32_t(__builtin_amdgcn_readfirstlane(int(past % p.splits)));
+    splits = p.splits;
+  }
+  const uint32_t unit = group * 4u + wave;
   const uint32_t blocks = p.input_size / GGUF_BLOCK, G = p.input_size / 32u;
   const uint32_t tiles = gguf_row_tiles(p.rows);
   const bool live = unit < p.units;
@@ -355,8 +362,8 @@ __global__ __launch_bounds__(256) void gguf_decode(const uint8_t *__restrict__ s
 
   // The workgroup's super-blocks: part `split` of K.
   // (blocks <= 2^16 and splits <= 16, so the products fit 32 bits; the quotients are wave-uniform.)
-  const uint32_t b0 = uint32_t(__builtin_amdgcn_readfirstlane(int(blocks * split / p.splits)));
-  const uint32_t b1 = uint32_t(__builtin_amdgcn_readfirstlane(int(blocks * (split + 1u) / p.splits)));
+  const uint32_t b0 = uint32_t(__builtin_amdgcn_readfirstlane(int(blocks * split / splits)));
+  const uint32_t b1 = uint32_t(__builtin_amdgcn_readfirstlane(int(blocks * (split + 1u) / splits)));
   const uint32_t count = b1 - b0;
 
   f32x4 acc[RT];
@@ -439,10 +446,12 @@ __global__ __launch_bounds__(256) void gguf_decode(const uint8_t *__restrict__ s
   }
 
   // Element (t, v) of this lane is row 16 t + 4 kq + v, column tile.column + c.
-  if (p.splits > 1) {
-    // Partials [split][unit][t][v][lane]: whole-wave contiguous stores and loads.
-    const size_t stride = size_t(gridDim.x) * 4u * RT * 256u;
-    float *mineAt = partials + (size_t(unit) * RT * 4u) * 64u + lane;
+  if (splits > 1) {
+    // Partials [split][partitioned unit][t][v][lane]: whole-wave contiguous stores and loads.
+    const uint32_t partitioned = (p.units + 3u) / 4u - p.whole_groups;  // workgroups
+    const size_t stride = size_t(partitioned) * 4u * RT * 256u;
+    float *mineAt = partials + (size_t(unit - 4u * p.whole_groups) * RT * 4u) * 64u + lane;
+    uint32_t *counter = counters + (group - p.whole_groups);
     if (live) {
 #pragma unroll
       for (int t = 0; t < RT; ++t)
@@ -456,15 +465,15 @@ __global__ __launch_bounds__(256) void gguf_decode(const uint8_t *__restrict__ s
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
-    if (threadIdx.x == 0) arrived = __hip_atomic_fetch_add(&counters[blockIdx.x], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (threadIdx.x == 0) arrived = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
-    if (arrived != p.splits - 1) return;
+    if (arrived != splits - 1) return;
     // The last arriver sums the splits in split order; the loads of a round of eight are in flight together.
 #pragma unroll
     for (int t = 0; t < RT; ++t)
 #pragma unroll
       for (int v = 0; v < 4; ++v) acc[t][v] = 0.f;
-    for (uint32_t s0 = 0; s0 < p.splits; s0 += 4u) {
+    for (uint32_t s0 = 0; s0 < splits; s0 += 4u) {
       float part[4][RT][4];
 #pragma unroll
       for (uint32_t s = 0; s < 4u; ++s)
@@ -472,7 +481,7 @@ __global__ __launch_bounds__(256) void gguf_decode(const uint8_t *__restrict__ s
         for (int t = 0; t < RT; ++t)
 #pragma unroll
           for (int v = 0; v < 4; ++v) {
-            const uint32_t from = s0 + s < p.splits ? s0 + s : s0;
+            const uint32_t from = s0 + s < splits ? s0 + s : s0;
             part[s][t][v] = __hip_atomic_load(mineAt + size_t(from) * stride + (t * 4 + v) * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           }
 #pragma unroll
@@ -480,9 +489,9 @@ __global__ __launch_bounds__(256) void gguf_decode(const uint8_t *__restrict__ s
 #pragma unroll
         for (int t = 0; t < RT; ++t)
 #pragma unroll
-          for (int v = 0; v < 4; ++v) acc[t][v] += s0 + s < p.splits ? part[s][t][v] : 0.f;
+          for (int v = 0; v < 4; ++v) acc[t][v] += s0 + s < splits ? part[s][t][v] : 0.f;
     }
-    if (threadIdx.x == 0) __hip_atomic_store(&counters[blockIdx.x], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (threadIdx.x == 0) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 
   if constexpr (kGateUp) {
@@ -521,7 +530,7 @@ __global__ __launch_bounds__(256) void gguf_decode(const uint8_t *__restrict__ s
     if constexpr (kTable) {
       __syncthreads();
       uint8_t *next = reinterpret_cast<uint8_t *>(const_cast<uint16_t *>(residual));
-      const uint32_t G2 = p.out_stride / 32u, g = blockIdx.x;
+      const uint32_t G2 = p.out_stride / 32u, g = group;
       uint2 *values = reinterpret_cast<uint2 *>(next);
       float *sums32 = reinterpret_cast<float *>(next + gguf_table_sums32_offset(p.out_stride, tiles));
       float *sums16 = reinterpret_cast<float *>(next + gguf_table_sums16_offset(p.out_stride, tiles));

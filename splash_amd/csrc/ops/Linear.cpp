@@ -60,9 +60,9 @@ void LinearPlan::requireConfiguration() const {
   if (!n || n % GGUF_TILE_COLUMNS || !k || k % GGUF_BLOCK)
     throw std::invalid_argument("block projections take whole 16-column tiles and 256-input super-blocks");
   const LinearConfig &c = config_;
-  if (c.kWaves != 1) throw std::invalid_argument("the waves of a block workgroup walk one K range");
-  if (!c.validSplits() || uint64_t{c.splits} * c.kWaves > k / GGUF_BLOCK)
+  if (!c.validSplits() || c.splits > k / GGUF_BLOCK)
     throw std::invalid_argument("block splits take at least one super-block each");
+  if (c.wholeGroups > groupsOf(n, workload_.epilogue)) throw std::invalid_argument("more whole workgroups than the projection has");
   if (destination_ == FloatOutput::Float32 && workload_.epilogue != LinearEpilogue::None)
     throw std::invalid_argument("only a plain block plan writes fp32");
 }
@@ -74,7 +74,8 @@ LinearScratchSize LinearPlan::scratchSize() const noexcept {
   size.input = gguf_table_bytes(k, tiles);
   if (config_.splits > 1) {
     // [split][unit][row tile][4][64 lanes] fp32 partials over whole workgroups, and one counter per workgroup.
-    const uint64_t groups = groupsOf(n, workload_.epilogue);
+    // of the partitioned workgroups only
+    const uint64_t groups = std::max<uint64_t>(1, groupsOf(n, workload_.epilogue) - config_.wholeGroups);
     size.partials = uint64_t{config_.splits} * groups * kWavesAcross * tiles * 256u * sizeof(float);
     size.counters = groups * sizeof(uint32_t);
   }
@@ -96,9 +97,19 @@ LinearPlan Linear::plan(LinearWorkload w, FloatOutput destination) const {
   const uint32_t blocks = w.matrix.inputSize / GGUF_BLOCK;
   const uint32_t groups = std::max(1u, groupsOf(w.matrix.outputSize, w.epilogue));
   const uint32_t wanted = calibration_.computeUnits * calibration_.groupsPerUnit;
+  const uint32_t most = std::min(LinearConfig::kMaximumSplits, std::max(1u, blocks / calibration_.minimumBlocksPerWave));
   LinearConfig config;
-  config.splits = std::clamp((wanted + groups / 2) / groups, 1u,
-                             std::min(LinearConfig::kMaximumSplits, std::max(1u, blocks / calibration_.minimumBlocksPerWave)));
+  const uint32_t units = calibration_.computeUnits;
+  if (groups >= 2 * units && groups % units) {
+    // Enough workgroups to fill the device without partitioning, but a remainder that would leave
+    // most units idle at the end: the whole rounds run unsplit and the remainder is partitioned
+    // into about one piece per unit, dispatched last.
+    config.wholeGroups = groups - groups % units;
+    config.splits = std::clamp((units + (groups % units) / 2) / (groups % units), 1u, most);
+    if (config.splits == 1) config.wholeGroups = 0;
+  } else {
+    config.splits = std::clamp((wanted + groups / 2) / groups, 1u, most);
+  }
   return LinearPlan(w, config, destination);
 }
 
@@ -167,7 +178,7 @@ PreparedInput Linear::add(hip::CommandGraph &graph, LinearBuffers b, const Proje
   params.input_size = k;
   params.rows = w.rows;
   params.splits = c.splits;
-  params.k_waves = c.kWaves;
+  params.whole_groups = c.wholeGroups;
   params.out_stride = n;
   std::array<hip::Buffer, 3> images;
   const std::vector<QuantizedSegment> &segments = p.blocks().segments;
@@ -195,7 +206,7 @@ PreparedInput Linear::add(hip::CommandGraph &graph, LinearBuffers b, const Proje
              w.epilogue == LinearEpilogue::Residual ? b.residual : writesTable ? b.nextTable : spare,
              c.splits > 1 ? b.scratch.partials : spare,
              c.splits > 1 ? b.scratch.counters : spare},
-            params, {groupsOf(n, w.epilogue), c.splits, 1}, {256, 1, 1});
+            params, {c.wholeGroups + (groupsOf(n, w.epilogue) - c.wholeGroups) * c.splits, 1, 1}, {256, 1, 1});
   (void)tiles;
   return {b.input, LinearInput::Table16};
 }

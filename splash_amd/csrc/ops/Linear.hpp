@@ -44,9 +44,10 @@ struct LinearConfig final {
   // Cross-workgroup K partitions, 1 to kMaximumSplits.
   uint32_t splits = 1;
   static constexpr uint32_t kMaximumSplits = GGUF_MAXIMUM_SPLITS;
-  // Waves of a workgroup that split its K partition between them: 1 (its four waves walk the
-  // partition in step, each over its own column tiles).
-  uint32_t kWaves = 1;
+  // Leading workgroups (four column tiles each) that walk all of K themselves; only the
+  // workgroups past them are partitioned. With G workgroups on C compute units, G - G % C whole
+  // ones and the remainder partitioned C / (G % C) ways leaves every unit the same work.
+  uint32_t wholeGroups = 0;
   [[nodiscard]] constexpr bool validSplits() const noexcept {
     return splits && splits <= kMaximumSplits;
   }

@@ -102,14 +102,14 @@ class Linear:
         except Exception:
             pass
 
-    def plan(self, projection, rows, epilogue=EPILOGUE_NONE, splits=None, k_waves=None):
+    def plan(self, projection, rows, epilogue=EPILOGUE_NONE, splits=None, whole_groups=None):
         p = nat.LinearPlan()
         check(lib.spo_linear_plan_for(self.handle, projection.handle, rows, epilogue, ctypes.byref(p)))
-        if splits is not None or k_waves is not None:
+        if splits is not None or whole_groups is not None:
             if splits is not None:
                 p.splits = splits
-            if k_waves is not None:
-                p.k_waves = k_waves
+            if whole_groups is not None:
+                p.whole_groups = whole_groups
             check(lib.spo_linear_plan_with(projection.handle, ctypes.byref(p)))
         return p
 

@@ -68,7 +68,8 @@ def test_linear_plans_without_a_device():
     assert table == ops.gguf_table_bytes(25600, 16)
     assert partials > 0 and counters > 0   # a 5120-column projection of K 25600 splits across workgroups
     table, partials, counters = linear.scratch_size(151936, 5120, 16)
-    assert partials == 0                    # the LM head fills the device without splitting
+    # the LM head fills the device in whole rounds; only the workgroups of the last, partial round split
+    assert partials <= 16 * 255 * 4 * 256 * 4
     with pytest.raises(ValueError):
         linear.scratch_size(5120, 25600, 65)
     with pytest.raises(ValueError):

@@ -45,12 +45,12 @@ def test_image_dequantization_of_quantized_weights(backend, fmt):
 
 
 def run_projection(backend, linear, fmt, native_segments, K, x_bits, epilogue=ops.EPILOGUE_NONE, float32=False,
-                   residual_bits=None, gate_native=None, splits=None, k_waves=None):
+                   residual_bits=None, gate_native=None, splits=None, whole_groups=None):
     M = x_bits.shape[0]
     proj = ops.Projection.from_native(backend, [(fmt, n, nat) for n, nat in native_segments], K, float32=float32)
     gate = ops.Projection.from_native(backend, [(fmt, native_segments[0][0], gate_native)], K) if gate_native is not None else None
     N = proj.output_size
-    plan = linear.plan(proj, M, epilogue, splits=splits, k_waves=k_waves)
+    plan = linear.plan(proj, M, epilogue, splits=splits, whole_groups=whole_groups)
     scratch = linear.scratch_for(backend, [plan])
     x = backend.from_array(x_bits, label="x")
     out = backend.allocate_buffer(M * N * (4 if float32 else 2), label="out")
@@ -92,18 +92,18 @@ def test_rows_do_not_depend_on_the_block_or_the_partition(backend, fmt):
     alone or in a taller block, and splits sum in split order so a re-run is bit-identical."""
     print(f"case projection invariants fmt={fmt}", flush=True)
     rng = np.random.default_rng(7)
-    N, K = 128, 4096
+    N, K = 256, 4096
     native = orc.make_native(fmt, N, K, 3)
     x = orc.f32_to_bf16(rng.standard_normal((32, K)).astype(np.float32))
     linear = ops.Linear(backend)
-    full, _, _ = run_projection(backend, linear, fmt, [(N, native)], K, x, float32=True, splits=1, k_waves=1)
+    full, _, _ = run_projection(backend, linear, fmt, [(N, native)], K, x, float32=True, splits=1, whole_groups=0)
     for rows in (1, 5, 16):
-        part, _, _ = run_projection(backend, linear, fmt, [(N, native)], K, x[:rows], float32=True, splits=1, k_waves=1)
+        part, _, _ = run_projection(backend, linear, fmt, [(N, native)], K, x[:rows], float32=True, splits=1, whole_groups=0)
         assert part.tobytes() == full[:rows].tobytes()
     want = orc.gemm(fmt, native, x, N)
-    for splits, k_waves in ((1, 1), (2, 1), (4, 1), (16, 1)):
-        a, _, _ = run_projection(backend, linear, fmt, [(N, native)], K, x, float32=True, splits=splits, k_waves=k_waves)
-        b, _, _ = run_projection(backend, linear, fmt, [(N, native)], K, x, float32=True, splits=splits, k_waves=k_waves)
+    for splits, whole_groups in ((1, 0), (2, 0), (4, 0), (16, 0), (4, 1), (3, 2), (2, 3), (2, 4)):
+        a, _, _ = run_projection(backend, linear, fmt, [(N, native)], K, x, float32=True, splits=splits, whole_groups=whole_groups)
+        b, _, _ = run_projection(backend, linear, fmt, [(N, native)], K, x, float32=True, splits=splits, whole_groups=whole_groups)
         assert a.tobytes() == b.tobytes()
         assert np.all(np.abs(a.astype(np.float64) - want["exact"]) <= want["bound"])
 
@@ -116,10 +116,10 @@ def test_fused_segments_equal_each_alone(backend):
     natives = [orc.make_native(ops.FMT_Q4K, n, K, 60 + i) for i, n in enumerate(sizes)]
     x = orc.f32_to_bf16(rng.standard_normal((16, K)).astype(np.float32))
     linear = ops.Linear(backend)
-    fused, _, _ = run_projection(backend, linear, ops.FMT_Q4K, list(zip(sizes, natives)), K, x, splits=1, k_waves=1)
+    fused, _, _ = run_projection(backend, linear, ops.FMT_Q4K, list(zip(sizes, natives)), K, x, splits=1, whole_groups=0)
     at = 0
     for n, native in zip(sizes, natives):
-        alone, _, _ = run_projection(backend, linear, ops.FMT_Q4K, [(n, native)], K, x, splits=1, k_waves=1)
+        alone, _, _ = run_projection(backend, linear, ops.FMT_Q4K, [(n, native)], K, x, splits=1, whole_groups=0)
         assert np.array_equal(fused[:, at:at + n], alone)
         at += n
 
@@ -136,7 +136,7 @@ def test_residual_and_gate_up_epilogues(backend, fmt):
     x = orc.f32_to_bf16(rng.standard_normal((M, K)).astype(np.float32))
     res = orc.f32_to_bf16(rng.standard_normal((M, N)).astype(np.float32))
     linear = ops.Linear(backend)
-    kw = dict(splits=2, k_waves=1)
+    kw = dict(splits=2, whole_groups=1)
     up32, _, _ = run_projection(backend, linear, fmt, [(N, up_native)], K, x, float32=True, **kw)
     gate32, _, _ = run_projection(backend, linear, fmt, [(N, gate_native)], K, x, float32=True, **kw)
     got, _, _ = run_projection(backend, linear, fmt, [(N, up_native)], K, x, epilogue=ops.EPILOGUE_RESIDUAL,
