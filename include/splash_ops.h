@@ -136,6 +136,44 @@ typedef struct spo_rope_sequence { uint32_t first_row, rows, anchor; } spo_rope_
 sp_status spo_rope_add_tree_tables(spo_graph *graph, sp_buffer *inverse_frequency, sp_buffer *depth, sp_buffer *cosines,
                                    sp_buffer *sines, uint32_t pairs, const spo_rope_sequence *sequences, uint32_t count);
 
+/* ---- GDN (runtime/ops/GDN.hpp:16-203, GDN.cpp:225-330): the verify step of Gated DeltaNet layers ---- */
+typedef struct spo_gdn_shape { /* ops::GdnShape (GDN.hpp:16-36); head dimension 128 */
+  uint32_t key_heads, value_heads;
+  uint32_t convolution_dimension; /* (2 key_heads + value_heads) * 128 */
+  uint32_t packed_width;          /* [q | k | v | z | b | a] */
+  uint32_t sigmoid_gate;
+} spo_gdn_shape;
+typedef struct spo_gdn_state_strides { /* ops::GdnStateStrides (GDN.hpp:63-73), fp32 recurrent states */
+  uint64_t convolution_layer_bytes, recurrent_layer_bytes, convolution_state_bytes;
+} spo_gdn_state_strides;
+/* The strides and size of a state cell of `layers` layers, and one layer's tape bytes of one lane's
+ * step (gdnTapeLayerBytes, GDN.hpp:120). Any of the results may be NULL. */
+sp_status spo_gdn_layout(const spo_gdn_shape *shape, uint32_t layers, spo_gdn_state_strides *strides, uint64_t *cell_bytes,
+                         uint64_t *tape_layer_bytes);
+typedef struct spo_gdn_lane { /* ops::GdnTapeLane + SplashLaneRows + the lane's cells */
+  uint32_t first_row, rows;
+  uint32_t pending_path; /* rows of the lane's previous step it accepted and its state does not hold yet */
+  uint32_t reserved;
+  uint64_t pending_tape, step_tape;   /* byte offsets of this layer's tapes in the tape buffer */
+  uint64_t current_cell, next_cell;   /* byte offsets of the lane's cells in the states buffer */
+} spo_gdn_lane;
+typedef struct spo_gdn_decode_buffers { /* ops::GdnDecodeBuffers (GDN.hpp:122-152) */
+  sp_buffer *packed, *convolution_weights, *states, *tape, *decay_weights, *time_bias, *mixer_norm, *hidden;
+  uint32_t float_norm; /* the output norm's weights are fp32 */
+} spo_gdn_decode_buffers;
+/* GDN::addDecode (GDN.hpp:184): the step of 1 to 8 lanes of one layer. The state a step writes is
+ * the one BEFORE its rows (the lane's pending path folded in); its rows go to the lane's tape.
+ * chains: every lane's block is a chain; 0 (a tree block) is SP_INVALID_ARGUMENT. */
+sp_status spo_gdn_add_decode(spo_graph *graph, const spo_gdn_decode_buffers *buffers, const spo_gdn_shape *shape, uint32_t layer,
+                             const spo_gdn_state_strides *state, uint32_t tiled_heads, const spo_gdn_lane *lanes, uint32_t count,
+                             int chains);
+/* GDN::addFold (GDN.hpp:198): the state after the first `rows` rows of the path a lane retained of a
+ * step (retained_rows[0]), every layer, written to fold_cell exactly as the lane's next step would
+ * hold it; nothing when the path holds fewer rows. */
+sp_status spo_gdn_add_fold(spo_graph *graph, sp_buffer *states, sp_buffer *tape, sp_buffer *retained_rows, uint64_t step_tape,
+                           uint64_t state_cell, uint64_t fold_cell, const spo_gdn_shape *shape, uint32_t layers, uint32_t rows,
+                           const spo_gdn_state_strides *state);
+
 /* ---- Sampling (runtime/ops/Sampling.hpp:64-254, Sampling.cpp:283-357) ---- */
 typedef struct spo_lane_rows { uint32_t first, rows; } spo_lane_rows; /* SplashLaneRows */
 /* Sampling::workspace: bytes of the argmax partial values and indices, the masses, ranges, decisions. */

@@ -1,0 +1,327 @@
+// CPU oracle, Gated DeltaNet verify step (test infrastructure only; see oracle.h).
+//
+// A restatement of the reference's decode step for one lane and one layer
+// (runtime/metal/kernels/decode/gdn.metal:139-526, common/gdn_primitives.h:20-99) in its order of
+// operations: short convolution + SiLU, q/k RMS norms, gates, the fold of the pending (previously
+// accepted) rows into the state, the block rows' outputs, the gated output norm, the step's tape.
+// Sums over a head's 128 channels or a state row's 128 columns are four (resp. one) butterfly
+// sums over 32 lanes, as the kernels compute them.
+#include "oracle.h"
+#include "common.hpp"
+
+#include <cmath>
+#include <vector>
+
+using namespace orc;
+
+namespace {
+
+constexpr uint32_t kTaps = 4, kDim = 128, kRowsMax = 16;
+constexpr float kEps = 1e-6f;
+
+float butterfly32(float *lane) {
+  for (int step = 16; step; step >>= 1)
+    for (int l = 0; l < step; ++l) lane[l] += lane[l + step];
+  return lane[0];
+}
+// sum of 128 squares: four 32-channel groups, added in channel order
+float sumSquares128(const float *v) {
+  float total = 0.f;
+  for (int g = 0; g < 4; ++g) {
+    float lane[32];
+    for (int l = 0; l < 32; ++l) lane[l] = v[32 * g + l] * v[32 * g + l];
+    total += butterfly32(lane);
+  }
+  return total;
+}
+float silu(float x) { return x / (1.0f + std::exp2(-1.44269504089f * x)); }
+float sigmoid(float x) { return 1.0f / (1.0f + std::exp2(-1.44269504089f * x)); }
+
+uint32_t pathRow(uint32_t path, uint32_t depth) {
+  for (uint32_t i = 0; i < depth; ++i) path &= path - 1;
+  return uint32_t(__builtin_ctz(path));
+}
+
+struct Tape {
+  uint16_t *inputs, *kv;
+  float *decay;
+  uint16_t *beta;
+};
+Tape tapeOf(uint8_t *base, const OrcGdnShape &s) {
+  const uint32_t kvWidth = (s.key_heads + s.value_heads) * kDim;
+  uint8_t *p = base;
+  Tape t;
+  t.inputs = reinterpret_cast<uint16_t *>(p);
+  p += size_t(kRowsMax) * s.conv_dim * 2;
+  t.kv = reinterpret_cast<uint16_t *>(p);
+  p += size_t(kRowsMax) * kvWidth * 2;
+  t.decay = reinterpret_cast<float *>(p);
+  p += size_t(kRowsMax) * s.value_heads * 4;
+  t.beta = reinterpret_cast<uint16_t *>(p);
+  return t;
+}
+
+// The three rows of convolution inputs before a command's first row, after `consumed` rows of
+// the pending path (gdn_primitives.h:20-35).
+void history(const uint16_t *carried, const Tape *pending, uint32_t convDim, uint32_t consumed, uint32_t path,
+             const uint16_t *rows[3]) {
+  for (uint32_t r = 0; r < 3; ++r) {
+    const uint32_t source = consumed + r;
+    rows[r] = source < 3 ? carried + size_t(source) * convDim : pending->inputs + size_t(pathRow(path, source - 3)) * convDim;
+  }
+}
+
+// delta-rule update of one state row over `count` tokens (gdn.metal:270-298); with q, also the outputs.
+void foldRow(float *state /*[128]*/, uint32_t valueDim, uint32_t count, const uint16_t *keys /*[count][128]*/,
+             const uint16_t *values, const float *decay, const uint16_t *beta, const uint16_t *queries, uint16_t *out /*[count][128]*/) {
+  for (uint32_t t = 0; t < count; ++t) {
+    const float d = decay[t], b = bf2f(beta[t]);
+    float lane[32];
+    for (int l = 0; l < 32; ++l) {
+      float memory = 0.f;
+      for (int i = 0; i < 4; ++i) {
+        state[4 * l + i] *= d;
+        memory += state[4 * l + i] * bf2f(keys[t * kDim + 4 * l + i]);
+      }
+      lane[l] = memory;
+    }
+    const float memory = butterfly32(lane);
+    const float delta = (bf2f(values[t * kDim + valueDim]) - memory) * b;
+    for (int l = 0; l < 32; ++l) {
+      float result = 0.f;
+      for (int i = 0; i < 4; ++i) {
+        state[4 * l + i] += bf2f(keys[t * kDim + 4 * l + i]) * delta;
+        if (queries) result += state[4 * l + i] * bf2f(queries[t * kDim + 4 * l + i]);
+      }
+      lane[l] = result;
+    }
+    if (queries) out[t * kDim + valueDim] = f2bf(butterfly32(lane));
+  }
+}
+
+} // namespace
+
+extern "C" {
+
+uint64_t orc_gdn_tape_bytes(const OrcGdnShape *s) {
+  const uint32_t kvWidth = (s->key_heads + s->value_heads) * kDim;
+  return (uint64_t(kRowsMax) * (uint64_t(s->conv_dim) * 2 + uint64_t(kvWidth) * 2 + uint64_t(s->value_heads) * 6) + 15) / 16 * 16;
+}
+
+void orc_gdn_step(float *S, uint32_t D, const float *k, const float *v, float decay, float beta, const float *q, float *o) {
+  // fp32 textbook form of one token on S [D v][D k]: S *= d; mem = S k; delta = beta (v - mem); S += delta k^T; o = S q.
+  for (uint32_t r = 0; r < D; ++r) {
+    double memory = 0;
+    for (uint32_t c = 0; c < D; ++c) { S[r * D + c] *= decay; memory += double(S[r * D + c]) * k[c]; }
+    const float delta = float((double(v[r]) - memory) * beta);
+    double result = 0;
+    for (uint32_t c = 0; c < D; ++c) { S[r * D + c] += k[c] * delta; result += double(S[r * D + c]) * (q ? q[c] : 0.f); }
+    if (o) o[r] = float(result);
+  }
+}
+
+int orc_gdn_decode(const OrcGdnShape *s, const uint16_t *packed, uint32_t rows, const uint16_t *conv_weights, const float *a_scale,
+                   const uint16_t *dt_bias, const void *norm_weight, const uint16_t *conv_in, const float *state_in,
+                   uint8_t *pending_tape, uint32_t pending_path, uint16_t *conv_out, float *state_out, uint8_t *step_tape,
+                   uint16_t *hidden) {
+  if (!rows || rows > kRowsMax || s->conv_dim != (2 * s->key_heads + s->value_heads) * kDim) return -1;
+  const uint32_t KH = s->key_heads, VH = s->value_heads, C = s->conv_dim, P = s->packed_width, perKey = VH / KH;
+  const uint32_t keyWidth = KH * kDim, kvWidth = keyWidth + VH * kDim;
+  const uint32_t zOffset = C, bOffset = C + VH * kDim, aOffset = bOffset + VH;
+  const uint32_t pending = uint32_t(__builtin_popcount(pending_path));
+  Tape pend{}, step = tapeOf(step_tape, *s);
+  if (pending) pend = tapeOf(pending_tape, *s);
+  const uint16_t *hist[3];
+  history(conv_in, &pend, C, pending, pending_path, hist);
+  // conv carry the pending path leaves
+  std::vector<uint16_t> carry(3 * size_t(C));
+  for (uint32_t r = 0; r < 3; ++r) std::copy(hist[r], hist[r] + C, carry.begin() + size_t(r) * C);
+
+  // conv + SiLU of every conv channel of every row (a chain: row t's taps are rows t-3..t)
+  std::vector<uint16_t> conv(size_t(rows) * C);
+  for (uint32_t t = 0; t < rows; ++t)
+    for (uint32_t c = 0; c < C; ++c) {
+      float value = 0.f;
+      for (uint32_t tap = 0; tap < kTaps; ++tap) {
+        const int position = int(t) + int(tap) - 3;  // block row, or history row position + 3
+        const uint16_t *row = position < 0 ? carry.data() + size_t(position + 3) * C : packed + size_t(position) * P;
+        value += bf2f(row[c]) * bf2f(conv_weights[size_t(c) * kTaps + tap]);
+      }
+      value = bf2f(f2bf(value));
+      conv[size_t(t) * C + c] = f2bf(silu(value));
+    }
+  // per key head: normalized q and k rows; per value head: gates
+  std::vector<uint16_t> queries(size_t(KH) * rows * kDim), keys(size_t(KH) * rows * kDim);
+  for (uint32_t kh = 0; kh < KH; ++kh)
+    for (uint32_t t = 0; t < rows; ++t) {
+      float q[kDim], k[kDim];
+      for (uint32_t d = 0; d < kDim; ++d) {
+        q[d] = bf2f(conv[size_t(t) * C + kh * kDim + d]);
+        k[d] = bf2f(conv[size_t(t) * C + keyWidth + kh * kDim + d]);
+      }
+      const float qs = 1.0f / std::sqrt(sumSquares128(q) / float(kDim) + kEps), ks = 1.0f / std::sqrt(sumSquares128(k) / float(kDim) + kEps);
+      for (uint32_t d = 0; d < kDim; ++d) {
+        queries[(size_t(kh) * rows + t) * kDim + d] = f2bf(bf2f(f2bf(q[d] * qs)) * 0.0078125f);
+        keys[(size_t(kh) * rows + t) * kDim + d] = f2bf(bf2f(f2bf(k[d] * ks)) * 0.08838834765f);
+      }
+    }
+  // tape: inputs, k, v, gates
+  for (uint32_t t = 0; t < rows; ++t) {
+    std::copy(packed + size_t(t) * P, packed + size_t(t) * P + C, step.inputs + size_t(t) * C);
+    for (uint32_t kh = 0; kh < KH; ++kh)
+      std::copy(keys.begin() + (size_t(kh) * rows + t) * kDim, keys.begin() + (size_t(kh) * rows + t + 1) * kDim,
+                step.kv + size_t(t) * kvWidth + kh * kDim);
+    for (uint32_t c = 0; c < VH * kDim; ++c) step.kv[size_t(t) * kvWidth + keyWidth + c] = conv[size_t(t) * C + 2 * keyWidth + c];
+    for (uint32_t h = 0; h < VH; ++h) {
+      const float b = bf2f(packed[size_t(t) * P + bOffset + h]);
+      step.beta[t * VH + h] = f2bf(sigmoid(b));
+      const float x = bf2f(f2bf(bf2f(packed[size_t(t) * P + aOffset + h]) + bf2f(dt_bias[h])));
+      const float softplus = bf2f(f2bf(std::max(x, 0.0f) + std::log2(1.0f + std::exp2(-1.44269504089f * std::fabs(x))) * 0.69314718056f));
+      step.decay[t * VH + h] = std::exp(a_scale[h] * softplus);
+    }
+  }
+  std::copy(carry.begin(), carry.end(), conv_out);
+
+  // per value head: fold the pending rows -> state_out; then the block rows for their outputs
+  for (uint32_t h = 0; h < VH; ++h) {
+    const uint32_t kh = h / perKey;
+    uint16_t pk[kRowsMax * kDim], pv[kRowsMax * kDim], pb[kRowsMax];
+    float pd[kRowsMax];
+    for (uint32_t t = 0; t < pending; ++t) {
+      const uint32_t row = pathRow(pending_path, t);
+      std::copy(pend.kv + size_t(row) * kvWidth + kh * kDim, pend.kv + size_t(row) * kvWidth + (kh + 1) * kDim, pk + t * kDim);
+      std::copy(pend.kv + size_t(row) * kvWidth + keyWidth + h * kDim, pend.kv + size_t(row) * kvWidth + keyWidth + (h + 1) * kDim, pv + t * kDim);
+      pd[t] = pend.decay[row * VH + h];
+      pb[t] = pend.beta[row * VH + h];
+    }
+    uint16_t bv[kRowsMax * kDim], bb[kRowsMax], out[kRowsMax * kDim];
+    float bd[kRowsMax];
+    for (uint32_t t = 0; t < rows; ++t) {
+      std::copy(step.kv + size_t(t) * kvWidth + keyWidth + h * kDim, step.kv + size_t(t) * kvWidth + keyWidth + (h + 1) * kDim, bv + t * kDim);
+      bd[t] = step.decay[t * VH + h];
+      bb[t] = step.beta[t * VH + h];
+    }
+    for (uint32_t r = 0; r < kDim; ++r) {
+      float state[kDim];
+      const size_t base = (size_t(h) * kDim + r) * kDim;
+      std::copy(state_in + base, state_in + base + kDim, state);
+      foldRow(state, r, pending, pk, pv, pd, pb, nullptr, nullptr);
+      std::copy(state, state + kDim, state_out + base);
+      foldRow(state, r, rows, keys.data() + size_t(kh) * rows * kDim, bv, bd, bb, queries.data() + size_t(kh) * rows * kDim, out);
+    }
+    // gated output norm (gdn.metal:489-526)
+    const uint32_t outHead = (s->flags & 1u) ? (h % perKey) * KH + h / perKey : h;
+    for (uint32_t t = 0; t < rows; ++t) {
+      float value[kDim];
+      for (uint32_t d = 0; d < kDim; ++d) value[d] = bf2f(out[t * kDim + d]);
+      const float inverse = 1.0f / std::sqrt(sumSquares128(value) / float(kDim) + kEps);
+      for (uint32_t d = 0; d < kDim; ++d) {
+        const float w = (s->flags & 4u) ? static_cast<const float *>(norm_weight)[d] : bf2f(static_cast<const uint16_t *>(norm_weight)[d]);
+        const float normalized = bf2f(f2bf((value[d] * inverse) * w));
+        const float z = bf2f(packed[size_t(t) * P + zOffset + h * kDim + d]);
+        hidden[(size_t(t) * VH + outHead) * kDim + d] = f2bf((normalized * ((s->flags & 2u) ? 1.0f : z)) / (1.0f + std::exp2(-1.44269504089f * z)));
+      }
+    }
+  }
+  return 0;
+}
+
+int orc_gdn_fold(const OrcGdnShape *s, const uint16_t *conv_in, const float *state_in, uint8_t *step_tape, uint32_t path, uint32_t rows,
+                 uint16_t *conv_out, float *state_out) {
+  if (uint32_t(__builtin_popcount(path)) < rows) return 1;
+  const uint32_t KH = s->key_heads, VH = s->value_heads, C = s->conv_dim, perKey = VH / KH, keyWidth = KH * kDim, kvWidth = keyWidth + VH * kDim;
+  Tape step = tapeOf(step_tape, *s);
+  const uint16_t *hist[3];
+  history(conv_in, &step, C, rows, path, hist);
+  std::vector<uint16_t> carry(3 * size_t(C));
+  for (uint32_t r = 0; r < 3; ++r) std::copy(hist[r], hist[r] + C, carry.begin() + size_t(r) * C);
+  std::copy(carry.begin(), carry.end(), conv_out);
+  for (uint32_t h = 0; h < VH; ++h) {
+    const uint32_t kh = h / perKey;
+    uint16_t pk[kRowsMax * kDim], pv[kRowsMax * kDim], pb[kRowsMax];
+    float pd[kRowsMax];
+    for (uint32_t t = 0; t < rows; ++t) {
+      const uint32_t row = pathRow(path, t);
+      std::copy(step.kv + size_t(row) * kvWidth + kh * kDim, step.kv + size_t(row) * kvWidth + (kh + 1) * kDim, pk + t * kDim);
+      std::copy(step.kv + size_t(row) * kvWidth + keyWidth + h * kDim, step.kv + size_t(row) * kvWidth + keyWidth + (h + 1) * kDim, pv + t * kDim);
+      pd[t] = step.decay[row * VH + h];
+      pb[t] = step.beta[row * VH + h];
+    }
+    for (uint32_t r = 0; r < kDim; ++r) {
+      float state[kDim];
+      const size_t base = (size_t(h) * kDim + r) * kDim;
+      std::copy(state_in + base, state_in + base + kDim, state);
+      foldRow(state, r, rows, pk, pv, pd, pb, nullptr, nullptr);
+      std::copy(state, state + kDim, state_out + base);
+    }
+  }
+  return 0;
+}
+
+// The reference's own check of a decode step (gdn_decode_metal_test.mm:373-522): convolution + SiLU,
+// normalized heads, gates and the recurrence in fp64 from the same packed rows, no intermediate
+// rounding but the stored bf16 inputs. Outputs: k and v rows [rows][kv_width], beta and decay
+// [rows][vh], the state after `rows` rows and the un-normed recurrent outputs [rows][vh][128].
+int orc_gdn_reference(const OrcGdnShape *s, const uint16_t *packed, uint32_t rows, const uint16_t *conv_weights, const float *a_scale,
+                      const uint16_t *dt_bias, const uint16_t *conv_in, const float *state_in, double *kv, double *beta, double *decay,
+                      double *state_out, double *outputs) {
+  const uint32_t KH = s->key_heads, VH = s->value_heads, C = s->conv_dim, P = s->packed_width, perKey = VH / KH;
+  const uint32_t keyWidth = KH * kDim, kvWidth = keyWidth + VH * kDim, bOffset = C + VH * kDim, aOffset = bOffset + VH;
+  std::vector<double> conv(size_t(rows) * C);
+  for (uint32_t t = 0; t < rows; ++t)
+    for (uint32_t c = 0; c < C; ++c) {
+      double value = 0;
+      for (uint32_t tap = 0; tap < kTaps; ++tap) {
+        const int position = int(t) + int(tap) - 3;
+        const uint16_t *row = position < 0 ? conv_in + size_t(position + 3) * C : packed + size_t(position) * P;
+        value += double(bf2f(row[c])) * double(bf2f(conv_weights[size_t(c) * kTaps + tap]));
+      }
+      conv[size_t(t) * C + c] = value / (1.0 + std::exp(-value));
+    }
+  std::vector<double> q(size_t(rows) * keyWidth);
+  for (uint32_t t = 0; t < rows; ++t) {
+    for (uint32_t kh = 0; kh < KH; ++kh) {
+      double qs = 0, ks = 0;
+      for (uint32_t d = 0; d < kDim; ++d) {
+        qs += conv[size_t(t) * C + kh * kDim + d] * conv[size_t(t) * C + kh * kDim + d];
+        ks += conv[size_t(t) * C + keyWidth + kh * kDim + d] * conv[size_t(t) * C + keyWidth + kh * kDim + d];
+      }
+      qs = 1.0 / std::sqrt(qs / kDim + 1e-6);
+      ks = 1.0 / std::sqrt(ks / kDim + 1e-6);
+      for (uint32_t d = 0; d < kDim; ++d) {
+        q[size_t(t) * keyWidth + kh * kDim + d] = conv[size_t(t) * C + kh * kDim + d] * qs / 128.0;
+        kv[size_t(t) * kvWidth + kh * kDim + d] = conv[size_t(t) * C + keyWidth + kh * kDim + d] * ks / std::sqrt(128.0);
+      }
+    }
+    for (uint32_t c = 0; c < VH * kDim; ++c) kv[size_t(t) * kvWidth + keyWidth + c] = conv[size_t(t) * C + 2 * keyWidth + c];
+    for (uint32_t h = 0; h < VH; ++h) {
+      beta[t * VH + h] = 1.0 / (1.0 + std::exp(-double(bf2f(packed[size_t(t) * P + bOffset + h]))));
+      const double x = double(bf2f(packed[size_t(t) * P + aOffset + h])) + double(bf2f(dt_bias[h]));
+      decay[t * VH + h] = std::exp(double(a_scale[h]) * (std::max(x, 0.0) + std::log1p(std::exp(-std::fabs(x)))));
+    }
+  }
+  for (uint32_t h = 0; h < VH; ++h) {
+    const uint32_t kh = h / perKey;
+    for (uint32_t r = 0; r < kDim; ++r) {
+      double state[kDim];
+      const size_t base = (size_t(h) * kDim + r) * kDim;
+      for (uint32_t c = 0; c < kDim; ++c) state[c] = state_in[base + c];
+      for (uint32_t t = 0; t < rows; ++t) {
+        const double d = decay[t * VH + h], b = beta[t * VH + h];
+        double memory = 0;
+        for (uint32_t c = 0; c < kDim; ++c) { state[c] *= d; memory += state[c] * kv[size_t(t) * kvWidth + kh * kDim + c]; }
+        const double delta = (kv[size_t(t) * kvWidth + keyWidth + h * kDim + r] - memory) * b;
+        double result = 0;
+        for (uint32_t c = 0; c < kDim; ++c) {
+          state[c] += kv[size_t(t) * kvWidth + kh * kDim + c] * delta;
+          result += state[c] * q[size_t(t) * keyWidth + kh * kDim + c];
+        }
+        outputs[(size_t(t) * VH + h) * kDim + r] = result;
+      }
+      for (uint32_t c = 0; c < kDim; ++c) state_out[base + c] = state[c];
+    }
+  }
+  return 0;
+}
+
+} // extern "C"

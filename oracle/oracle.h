@@ -18,7 +18,8 @@
 //   orc_gemm_*                      pinned by fp64 dot + projectionBound interval, and invariants.
 //   orc_kv_quantize                 pinned: closed form, compiled reference header (oracle/_ref).
 //   orc_attention_*                 pinned by dense-softmax special cases and invariants.
-//   orc_gdn_*                       pinned by 1-row closed form and fold/rollback invariants.
+//   orc_gdn_*                       pinned by the fp64 textbook recurrence (orc_gdn_reference, the check
+//                                   the reference's own test makes) and fold/rollback invariants.
 //   orc_argmax / orc_accept_tree    pinned by brute force on tiny vocabularies.
 //   orc_rejection_*                 pinned by enumeration: selection law equals target to 1e-12.
 #pragma once
@@ -131,11 +132,34 @@ uint32_t orc_rejection_row(const float *logits, uint32_t vocab, float temperatur
 void orc_rejection_law(const float *logits, uint32_t vocab, float temperature, const float *q, double *out);
 
 // ---- Gated DeltaNet ----
-struct OrcGdn { uint32_t key_heads, value_heads, head_dim /*128*/, conv_taps /*4*/; };
-// One token step on one value head's state S [D v][D k] fp32 (gdn.metal:270-298):
-// S *= d; mem = S k; delta = beta (v - mem); S += delta k^T. o (optional) = S q after the update.
+// Shapes of a layer: packed row = [q (kh 128) | k (kh 128) | v (vh 128) | z (vh 128) | b (vh) | a (vh)],
+// conv_dim = (2 kh + vh) 128; flags: 1 tiled output heads, 2 sigmoid gate, 4 fp32 output-norm weights.
+struct OrcGdnShape { uint32_t key_heads, value_heads, conv_dim, packed_width, flags; };
+// Bytes of one layer's tape of one lane's step (abi/GDN.h:44-67 in the reference): room for 16 rows of
+// convolution inputs, k then v rows, decay fp32 and beta bf16.
+uint64_t orc_gdn_tape_bytes(const struct OrcGdnShape *s);
+// One token on one value head's state S [D v][D k] in the textbook form, sums in fp64 (the
+// closed form the restatement below is pinned against): S *= d; mem = S k; delta = beta (v - mem);
+// S += delta k^T; o (optional) = S q after the update.
 void orc_gdn_step(float *S, uint32_t D, const float *k, const float *v, float decay, float beta, const float *q,
                   float *o);
+// One decode step of one lane and one layer over a chain of `rows` rows (gdn.metal:139-526): folds
+// the pending path of the previous step's tape into the state and writes THAT as state_out (the
+// state before this step's rows) with the convolution carry it leaves; writes this step's tape;
+// hidden bf16 [rows][vh * 128] are the gated, normed outputs of the block rows.
+// conv_in/out bf16 [3][conv_dim]; state fp32 [vh][128][128]; pending_tape may be NULL when the path is 0.
+int orc_gdn_decode(const struct OrcGdnShape *s, const uint16_t *packed, uint32_t rows, const uint16_t *conv_weights,
+                   const float *a_scale, const uint16_t *dt_bias, const void *norm_weight, const uint16_t *conv_in,
+                   const float *state_in, uint8_t *pending_tape, uint32_t pending_path, uint16_t *conv_out,
+                   float *state_out, uint8_t *step_tape, uint16_t *hidden);
+// The state after the first `rows` rows of `path` of a step's tape, as the lane's next step would
+// hold it (gdn.metal:630-698, exact cells). Returns 1 and writes nothing when the path is shorter.
+int orc_gdn_fold(const struct OrcGdnShape *s, const uint16_t *conv_in, const float *state_in, uint8_t *step_tape,
+                 uint32_t path, uint32_t rows, uint16_t *conv_out, float *state_out);
+// The fp64 check of a step the reference's test makes (gdn_decode_metal_test.mm:373-522).
+int orc_gdn_reference(const struct OrcGdnShape *s, const uint16_t *packed, uint32_t rows, const uint16_t *conv_weights,
+                      const float *a_scale, const uint16_t *dt_bias, const uint16_t *conv_in, const float *state_in,
+                      double *kv, double *beta, double *decay, double *state_out, double *outputs);
 
 #ifdef __cplusplus
 }

@@ -90,6 +90,25 @@ class LaneRows(ctypes.Structure):
     _fields_ = [("first", c_u32), ("rows", c_u32)]
 
 
+class GdnShape(ctypes.Structure):
+    _fields_ = [("key_heads", c_u32), ("value_heads", c_u32), ("convolution_dimension", c_u32), ("packed_width", c_u32),
+                ("sigmoid_gate", c_u32)]
+
+
+class GdnStateStrides(ctypes.Structure):
+    _fields_ = [("convolution_layer_bytes", c_u64), ("recurrent_layer_bytes", c_u64), ("convolution_state_bytes", c_u64)]
+
+
+class GdnLane(ctypes.Structure):
+    _fields_ = [("first_row", c_u32), ("rows", c_u32), ("pending_path", c_u32), ("reserved", c_u32), ("pending_tape", c_u64),
+                ("step_tape", c_u64), ("current_cell", c_u64), ("next_cell", c_u64)]
+
+
+class GdnDecodeBuffers(ctypes.Structure):
+    _fields_ = [(n, c_p) for n in ("packed", "convolution_weights", "states", "tape", "decay_weights", "time_bias", "mixer_norm",
+                                   "hidden")] + [("float_norm", c_u32)]
+
+
 class SamplingBuffers(ctypes.Structure):
     _fields_ = [(n, c_p) for n in ("logits", "tokens", "partial_values", "partial_indices", "draft_probabilities", "uniforms",
                                    "masses", "ranges", "decisions", "input_tokens", "tree_rows")]
@@ -187,6 +206,9 @@ _sig("spo_norm_add_rms", c_int, c_p, c_p, c_p, c_p, c_u32, c_u32)
 _sig("spo_norm_add_rms_table", c_int, c_p, c_p, c_p, c_p, c_p, c_u32, c_u32)
 _sig("spo_embedding_add", c_int, c_p, c_u32, c_p, c_u32, c_u32, c_p, c_p, c_u32)
 _sig("spo_rope_add_tree_tables", c_int, c_p, c_p, c_p, c_p, c_p, c_u32, P(RopeSequence), c_u32)
+_sig("spo_gdn_layout", c_int, P(GdnShape), c_u32, P(GdnStateStrides), P(c_u64), P(c_u64))
+_sig("spo_gdn_add_decode", c_int, c_p, P(GdnDecodeBuffers), P(GdnShape), c_u32, P(GdnStateStrides), c_u32, P(GdnLane), c_u32, c_int)
+_sig("spo_gdn_add_fold", c_int, c_p, c_p, c_p, c_p, c_u64, c_u64, c_u64, P(GdnShape), c_u32, c_u32, P(GdnStateStrides))
 _sig("spo_sampling_workspace", c_int, c_u32, P(c_u64))
 _sig("spo_sampling_add_verify", c_int, c_p, P(SamplingBuffers), c_u32, c_u32, P(LaneRows), P(ctypes.c_float), c_u32)
 _sig("spo_sampling_add_acceptance", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, P(LaneRows), P(c_u32), c_u32, P(c_u32))

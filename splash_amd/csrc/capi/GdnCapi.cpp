@@ -1,0 +1,66 @@
+// C shim of ops::GDN (include/splash_ops.h).
+#include "capi/Guard.hpp"
+#include "capi/Handles.hpp"
+#include "ops/Gdn.hpp"
+#include "splash_ops.h"
+
+using namespace splash;
+
+namespace {
+hip::Buffer B(sp_buffer *b) { return hip::Buffer::share(b); }
+ops::GdnShape shapeOf(const spo_gdn_shape &s) {
+  ops::GdnShape shape;
+  shape.keyHeads = s.key_heads;
+  shape.valueHeads = s.value_heads;
+  shape.convolutionDimension = s.convolution_dimension;
+  shape.packedWidth = s.packed_width;
+  shape.sigmoidGate = s.sigmoid_gate != 0;
+  return shape;
+}
+ops::GdnStateStrides stridesOf(const spo_gdn_state_strides &s) {
+  return {s.convolution_layer_bytes, s.recurrent_layer_bytes, s.convolution_state_bytes};
+}
+} // namespace
+
+extern "C" {
+
+sp_status spo_gdn_layout(const spo_gdn_shape *shape, uint32_t layers, spo_gdn_state_strides *strides, uint64_t *cell_bytes,
+                         uint64_t *tape_layer_bytes) {
+  return capi::guard([&] {
+    capi::require(shape, "shape");
+    const ops::GdnShape s = shapeOf(*shape);
+    if (!s.valid() || !layers) throw std::invalid_argument("invalid GDN shape");
+    const ops::GdnStateStrides st = ops::GdnStateStrides::of(s, layers);
+    if (strides) *strides = {st.convolutionLayerBytes, st.recurrentLayerBytes, st.convolutionStateBytes};
+    if (cell_bytes) *cell_bytes = st.cellBytes(layers);
+    if (tape_layer_bytes) *tape_layer_bytes = ops::gdnTapeLayerBytes(s);
+  });
+}
+
+sp_status spo_gdn_add_decode(spo_graph *graph, const spo_gdn_decode_buffers *b, const spo_gdn_shape *shape, uint32_t layer,
+                             const spo_gdn_state_strides *state, uint32_t tiled_heads, const spo_gdn_lane *lanes, uint32_t count,
+                             int chains) {
+  return capi::guard([&] {
+    capi::require(graph && b && shape && state && lanes, "graph, buffers, shape, strides or lanes");
+    ops::GdnDecodeBuffers buffers{B(b->packed), B(b->convolution_weights), B(b->states), B(b->tape), B(b->decay_weights),
+                                  B(b->time_bias), B(b->mixer_norm), b->float_norm != 0, B(b->hidden)};
+    std::vector<ops::GdnLaneStep> list;
+    for (uint32_t i = 0; i < count; ++i)
+      list.push_back({lanes[i].first_row, lanes[i].rows, lanes[i].pending_path, lanes[i].pending_tape, lanes[i].step_tape,
+                      lanes[i].current_cell, lanes[i].next_cell});
+    ops::GDN::addDecode(capi::graphOf(graph), buffers, shapeOf(*shape), layer, stridesOf(*state),
+                        tiled_heads ? ops::GdnHeadOrder::Tiled : ops::GdnHeadOrder::Grouped, list, chains != 0);
+  });
+}
+
+sp_status spo_gdn_add_fold(spo_graph *graph, sp_buffer *states, sp_buffer *tape, sp_buffer *retained_rows, uint64_t step_tape,
+                           uint64_t state_cell, uint64_t fold_cell, const spo_gdn_shape *shape, uint32_t layers, uint32_t rows,
+                           const spo_gdn_state_strides *state) {
+  return capi::guard([&] {
+    capi::require(graph && shape && state, "graph, shape or strides");
+    ops::GdnFoldBuffers buffers{B(states), B(tape), B(retained_rows), step_tape, state_cell, fold_cell};
+    ops::GDN::addFold(capi::graphOf(graph), buffers, shapeOf(*shape), layers, rows, stridesOf(*state));
+  });
+}
+
+} // extern "C"

@@ -1,0 +1,92 @@
+#include "ops/Gdn.hpp"
+#include "ops/Linear.hpp"  // requireBytes
+
+#include <algorithm>
+#include <stdexcept>
+
+namespace splash::ops {
+
+GdnStateStrides GdnStateStrides::of(const GdnShape &shape, uint32_t layers) noexcept {
+  GdnStateStrides s;
+  s.convolutionLayerBytes = uint64_t{GDN_CONVOLUTION_TAPS - 1} * shape.convolutionDimension * 2;
+  s.recurrentLayerBytes = uint64_t{shape.valueHeads} * GDN_HEAD_DIMENSION * GDN_HEAD_DIMENSION * 4;
+  s.convolutionStateBytes = (s.convolutionLayerBytes * layers + 255) / 256 * 256;
+  return s;
+}
+
+uint64_t gdnTapeLayerBytes(const GdnShape &shape) noexcept {
+  return gdn_tape_layer_bytes(shape.convolutionDimension, shape.kvWidth(), shape.valueHeads);
+}
+
+void GDN::addDecode(hip::CommandGraph &graph, const GdnDecodeBuffers &b, const GdnShape &shape, uint32_t layer,
+                    const GdnStateStrides &state, GdnHeadOrder order, const std::vector<GdnLaneStep> &lanes, bool chains) {
+  if (!shape.valid()) throw std::invalid_argument("invalid GDN shape");
+  if (!state.valid()) throw std::invalid_argument("invalid GDN state strides");
+  if (lanes.empty() || lanes.size() > GDN_MAXIMUM_LANES) throw std::invalid_argument("a GDN step takes 1 to 8 lanes");
+  if (!chains) throw std::invalid_argument("GDN tree blocks are not built: a lane's rows are a chain");
+  const uint64_t tapeBytes = gdnTapeLayerBytes(shape);
+  const uint64_t cellNeed = state.convolutionStateBytes + uint64_t{layer + 1} * state.recurrentLayerBytes;
+  if (uint64_t{layer + 1} * state.convolutionLayerBytes > state.convolutionStateBytes)
+    throw std::invalid_argument("the layer's convolution rows lie past the cell's convolution part");
+  uint32_t rows = 0;
+  GdnDecodeParams params{};
+  params.shape = shape.params();
+  params.flags = (order == GdnHeadOrder::Tiled ? GDN_TILED_HEADS : 0u) | (shape.sigmoidGate ? GDN_SIGMOID_GATE : 0u) |
+                 (b.floatNorm ? GDN_FLOAT_NORM : 0u);
+  params.layer = layer;
+  params.lanes = uint32_t(lanes.size());
+  params.conv_layer_bytes = state.convolutionLayerBytes;
+  params.recurrent_layer_bytes = state.recurrentLayerBytes;
+  params.convolution_state_bytes = state.convolutionStateBytes;
+  for (size_t i = 0; i < lanes.size(); ++i) {
+    const GdnLaneStep &l = lanes[i];
+    if (!l.rows || l.rows > GDN_MAXIMUM_ROWS) throw std::invalid_argument("a lane's block holds 1 to 16 rows");
+    if (l.firstRow < rows) throw std::invalid_argument("the lanes' blocks ascend and do not overlap");
+    rows = l.firstRow + l.rows;
+    if (l.pendingPath >> GDN_MAXIMUM_ROWS) throw std::invalid_argument("a pending path names rows of a 16-row block");
+    if (l.stepTape % 16 || l.pendingTape % 16) throw std::invalid_argument("tape slots are 16-byte aligned");
+    if (l.stepTape + tapeBytes > b.tape.sizeBytes() || (l.pendingPath && l.pendingTape + tapeBytes > b.tape.sizeBytes()))
+      throw std::invalid_argument("a tape slot lies past the tape buffer");
+    if (l.pendingPath && l.pendingTape < l.stepTape + tapeBytes && l.stepTape < l.pendingTape + tapeBytes)
+      throw std::invalid_argument("a lane's pending and step tapes overlap");
+    if (l.currentCell % 16 || l.nextCell % 16) throw std::invalid_argument("state cells are 16-byte aligned");
+    if (l.currentCell + cellNeed > b.states.sizeBytes() || l.nextCell + cellNeed > b.states.sizeBytes())
+      throw std::invalid_argument("a state cell lies past the states buffer");
+    if (l.currentCell == l.nextCell) throw std::invalid_argument("a step reads and writes different cells");
+    params.lane[i] = {l.firstRow, l.rows, l.pendingPath, 0, l.pendingTape, l.stepTape, l.currentCell, l.nextCell};
+  }
+  requireBytes(b.packed, uint64_t{rows} * shape.packedWidth * 2, "GDN packed rows");
+  requireBytes(b.convolutionWeights, uint64_t{shape.convolutionDimension} * GDN_CONVOLUTION_TAPS * 2, "GDN convolution weights");
+  requireBytes(b.decayWeights, uint64_t{shape.valueHeads} * 4, "GDN decay weights");
+  requireBytes(b.timeBias, uint64_t{shape.valueHeads} * 2, "GDN time bias");
+  requireBytes(b.mixerNorm, uint64_t{GDN_HEAD_DIMENSION} * (b.floatNorm ? 4 : 2), "GDN output norm");
+  requireBytes(b.hidden, uint64_t{rows} * shape.valueHeads * GDN_HEAD_DIMENSION * 2, "GDN hidden rows");
+  graph.add("gdn_decode", {b.packed, b.convolutionWeights, b.states, b.tape, b.decayWeights, b.timeBias, b.mixerNorm, b.hidden}, params,
+            {shape.valueHeads, uint32_t(lanes.size()), 1}, {256, 1, 1});
+}
+
+void GDN::addFold(hip::CommandGraph &graph, const GdnFoldBuffers &b, const GdnShape &shape, uint32_t layers, uint32_t rows,
+                  const GdnStateStrides &state) {
+  if (!shape.valid()) throw std::invalid_argument("invalid GDN shape");
+  if (!state.valid() || !layers) throw std::invalid_argument("invalid GDN state strides");
+  if (!rows || rows > GDN_MAXIMUM_ROWS) throw std::invalid_argument("a fold takes 1 to 16 rows");
+  const uint64_t tapeBytes = gdnTapeLayerBytes(shape), cell = state.cellBytes(layers);
+  if (b.stepTape % 16 || b.stepTape + tapeBytes * layers > b.tape.sizeBytes()) throw std::invalid_argument("the step's tapes lie past the tape buffer");
+  if (b.stateCell % 16 || b.foldCell % 16 || b.stateCell + cell > b.states.sizeBytes() || b.foldCell + cell > b.states.sizeBytes())
+    throw std::invalid_argument("a state cell lies past the states buffer");
+  if (b.stateCell == b.foldCell) throw std::invalid_argument("a fold reads and writes different cells");
+  requireBytes(b.retainedRows, 4, "retained rows");
+  GdnFoldParams params{};
+  params.shape = shape.params();
+  params.rows = rows;
+  params.conv_layer_bytes = state.convolutionLayerBytes;
+  params.recurrent_layer_bytes = state.recurrentLayerBytes;
+  params.convolution_state_bytes = state.convolutionStateBytes;
+  params.step_tape = b.stepTape;
+  params.tape_layer_bytes = tapeBytes;
+  params.state_cell = b.stateCell;
+  params.fold_cell = b.foldCell;
+  graph.add("gdn_fold", {b.states, b.tape, b.retainedRows}, params, {shape.valueHeads, layers, 1}, {256, 1, 1});
+}
+
+} // namespace splash::ops

@@ -1,0 +1,79 @@
+// ops::GDN of the reference (runtime/ops/GDN.hpp:16-203, GDN.cpp:225-330) for the verify step: the
+// decode step of up to eight lanes with its tape, and the fold of a step's accepted rows alone,
+// over kernels/gdn.hip. Prefill and the cached states' codes are not part of the verify step.
+#pragma once
+#include "abi/Gdn.h"
+#include "hip/Backend.hpp"
+
+#include <vector>
+
+namespace splash::ops {
+
+struct GdnShape final {
+  uint32_t keyHeads = 0, valueHeads = 0;
+  uint32_t headDimension = GDN_HEAD_DIMENSION;
+  uint32_t convolutionDimension = 0;
+  uint32_t packedWidth = 0;
+  bool sigmoidGate = false;
+  [[nodiscard]] bool valid() const noexcept {
+    return keyHeads && valueHeads && valueHeads % keyHeads == 0 && headDimension == GDN_HEAD_DIMENSION &&
+           convolutionDimension == (2ull * keyHeads + valueHeads) * headDimension &&
+           packedWidth >= convolutionDimension + uint64_t{valueHeads} * headDimension + 2ull * valueHeads;
+  }
+  [[nodiscard]] uint32_t kvWidth() const noexcept { return (keyHeads + valueHeads) * headDimension; }
+  [[nodiscard]] GdnShapeParams params() const noexcept { return {keyHeads, valueHeads, convolutionDimension, packedWidth}; }
+};
+enum class GdnHeadOrder : uint8_t { Grouped, Tiled };
+
+// A state cell's strides (GDN.hpp:63-73): fp32 recurrent states only.
+struct GdnStateStrides final {
+  uint64_t convolutionLayerBytes = 0, recurrentLayerBytes = 0, convolutionStateBytes = 0;
+  [[nodiscard]] bool valid() const noexcept { return convolutionLayerBytes && recurrentLayerBytes && convolutionStateBytes; }
+  // The strides of a cell of `layers` layers, and its size.
+  static GdnStateStrides of(const GdnShape &shape, uint32_t layers) noexcept;
+  [[nodiscard]] uint64_t cellBytes(uint32_t layers) const noexcept { return convolutionStateBytes + layers * recurrentLayerBytes; }
+};
+[[nodiscard]] uint64_t gdnTapeLayerBytes(const GdnShape &shape) noexcept;
+
+// One lane of a step: its block of the step's rows, its tape slots (byte offsets of this layer's
+// tapes in the tape buffer), the path of its previous step's rows its state does not hold yet, and
+// its cells (byte offsets in the states buffer).
+struct GdnLaneStep final {
+  uint32_t firstRow = 0, rows = 0;
+  uint32_t pendingPath = 0;
+  uint64_t pendingTape = 0, stepTape = 0;
+  uint64_t currentCell = 0, nextCell = 0;
+};
+
+struct GdnDecodeBuffers final {
+  hip::Buffer packed;              // bf16 [rows][packedWidth]
+  hip::Buffer convolutionWeights;  // bf16 [convolutionDimension][4]
+  hip::Buffer states;              // the lanes' cells
+  hip::Buffer tape;
+  hip::Buffer decayWeights;        // fp32 [valueHeads]: a_scale
+  hip::Buffer timeBias;            // bf16 [valueHeads]: dt_bias
+  hip::Buffer mixerNorm;           // bf16 or fp32 [128]
+  bool floatNorm = false;
+  hip::Buffer hidden;              // bf16 [rows][valueHeads * 128]
+};
+struct GdnFoldBuffers final {
+  hip::Buffer states;
+  hip::Buffer tape;
+  hip::Buffer retainedRows;  // uint32: the row mask the step's acceptance wrote
+  uint64_t stepTape = 0;     // the step's first layer's tape
+  uint64_t stateCell = 0;    // the cell the step wrote
+  uint64_t foldCell = 0;     // the cell the fold writes
+};
+
+class GDN final {
+public:
+  // The step of 1 to 8 lanes of one layer. `chains`: every lane's block is a chain (row r follows
+  // row r - 1); a tree block is refused (the kernel does not transform tree rows).
+  static void addDecode(hip::CommandGraph &graph, const GdnDecodeBuffers &buffers, const GdnShape &shape, uint32_t layer,
+                        const GdnStateStrides &state, GdnHeadOrder order, const std::vector<GdnLaneStep> &lanes, bool chains = true);
+  // The state after the first `rows` rows of the path a lane retained of a step, in each of `layers` layers.
+  static void addFold(hip::CommandGraph &graph, const GdnFoldBuffers &buffers, const GdnShape &shape, uint32_t layers, uint32_t rows,
+                      const GdnStateStrides &state);
+};
+
+} // namespace splash::ops

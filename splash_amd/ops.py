@@ -304,6 +304,35 @@ class RoPE:
         graph._keep.extend([inverse_frequency, depth, cosines, sines])
 
 
+class GDN:
+    """ops::GDN: the verify step of Gated DeltaNet layers (addDecode) and the fold of a step's accepted rows (addFold)."""
+
+    def __init__(self, key_heads, value_heads, packed_width=None, sigmoid_gate=False, layers=1):
+        conv = (2 * key_heads + value_heads) * 128
+        packed_width = packed_width or conv + value_heads * 128 + 2 * value_heads
+        self.shape = nat.GdnShape(key_heads, value_heads, conv, packed_width, int(sigmoid_gate))
+        self.layers = layers
+        self.strides = nat.GdnStateStrides()
+        cell, tape = ctypes.c_uint64(), ctypes.c_uint64()
+        check(lib.spo_gdn_layout(ctypes.byref(self.shape), layers, ctypes.byref(self.strides), ctypes.byref(cell), ctypes.byref(tape)))
+        self.cell_bytes, self.tape_layer_bytes = cell.value, tape.value
+
+    def add_decode(self, graph, buffers, layer, lanes, tiled_heads=False, float_norm=False, chains=True):
+        """buffers: dict of Buffer by the names of spo_gdn_decode_buffers; lanes: [dict(first_row, rows, pending_path,
+        pending_tape, step_tape, current_cell, next_cell)]."""
+        b = nat.GdnDecodeBuffers(**{k: v.handle for k, v in buffers.items()}, float_norm=int(float_norm))
+        arr = (nat.GdnLane * len(lanes))(*[nat.GdnLane(l["first_row"], l["rows"], l.get("pending_path", 0), 0, l.get("pending_tape", 0),
+                                                       l["step_tape"], l["current_cell"], l["next_cell"]) for l in lanes])
+        check(lib.spo_gdn_add_decode(graph.handle, ctypes.byref(b), ctypes.byref(self.shape), layer, ctypes.byref(self.strides),
+                                     int(tiled_heads), arr, len(lanes), int(chains)))
+        graph._keep.extend(list(buffers.values()))
+
+    def add_fold(self, graph, states, tape, retained_rows, step_tape, state_cell, fold_cell, rows):
+        check(lib.spo_gdn_add_fold(graph.handle, states.handle, tape.handle, retained_rows.handle, step_tape, state_cell, fold_cell,
+                                   ctypes.byref(self.shape), self.layers, rows, ctypes.byref(self.strides)))
+        graph._keep.extend([states, tape, retained_rows])
+
+
 NO_TOKEN = 0xFFFFFFFF
 
 

@@ -269,3 +269,93 @@ def split_activation_table(raw_bytes, K, tiles):
     s32 = raw_bytes[nv:nv + n32].view(np.float32).reshape(tiles, G, 16)
     s16 = raw_bytes[nv + n32:nv + 3 * n32].view(np.float32).reshape(tiles, 2 * G, 16)
     return values, s32, s16
+
+
+# ---- Gated DeltaNet ----
+class GdnShape(ctypes.Structure):
+    _fields_ = [("key_heads", c_u32), ("value_heads", c_u32), ("conv_dim", c_u32), ("packed_width", c_u32), ("flags", c_u32)]
+
+
+lib.orc_gdn_tape_bytes.restype = ctypes.c_uint64
+lib.orc_gdn_tape_bytes.argtypes = [ctypes.POINTER(GdnShape)]
+lib.orc_gdn_step.restype = None
+lib.orc_gdn_step.argtypes = [f32p, c_u32, f32p, f32p, c_f, c_f, f32p, f32p]
+
+
+def gdn_shape(key_heads, value_heads, flags=0, packed_width=None):
+    conv = (2 * key_heads + value_heads) * 128
+    return GdnShape(key_heads, value_heads, conv, packed_width or conv + value_heads * 128 + 2 * value_heads, flags)
+
+
+def gdn_tape_bytes(shape):
+    return int(lib.orc_gdn_tape_bytes(ctypes.byref(shape)))
+
+
+def gdn_split_tape(shape, tape):
+    """(inputs [16][conv], kv [16][kv width], decay [16][vh] f32, beta [16][vh]) views of one layer's tape bytes."""
+    kvw = (shape.key_heads + shape.value_heads) * 128
+    a = 16 * shape.conv_dim * 2
+    b = a + 16 * kvw * 2
+    c = b + 16 * shape.value_heads * 4
+    d = c + 16 * shape.value_heads * 2
+    return (tape[:a].view(np.uint16).reshape(16, shape.conv_dim), tape[a:b].view(np.uint16).reshape(16, kvw),
+            tape[b:c].view(np.float32).reshape(16, shape.value_heads), tape[c:d].view(np.uint16).reshape(16, shape.value_heads))
+
+
+def gdn_decode(shape, packed, conv_weights, a_scale, dt_bias, norm_weight, conv_in, state_in, pending_tape=None, pending_path=0):
+    """One lane, one layer, a chain of packed.shape[0] rows. Returns (conv_out, state_out, step_tape bytes, hidden)."""
+    rows = packed.shape[0]
+    vh = shape.value_heads
+    conv_out = np.zeros((3, shape.conv_dim), np.uint16)
+    state_out = np.zeros((vh, 128, 128), np.float32)
+    tape = np.zeros(gdn_tape_bytes(shape), np.uint8)
+    hidden = np.zeros((rows, vh * 128), np.uint16)
+    packed, conv_weights, a_scale, dt_bias, norm_weight, conv_in, state_in = (np.ascontiguousarray(x) for x in (
+        packed, conv_weights, a_scale, dt_bias, norm_weight, conv_in, state_in))
+    rc = lib.orc_gdn_decode(ctypes.byref(shape), _p(packed, u16p), rows, _p(conv_weights, u16p), _p(a_scale, f32p), _p(dt_bias, u16p),
+                            norm_weight.ctypes.data_as(ctypes.c_void_p), _p(conv_in, u16p), _p(state_in, f32p),
+                            _p(pending_tape, u8p), pending_path, _p(conv_out, u16p), _p(state_out, f32p), _p(tape, u8p), _p(hidden, u16p))
+    assert rc == 0
+    return conv_out, state_out, tape, hidden
+
+
+lib.orc_gdn_decode.restype = c_int
+lib.orc_gdn_decode.argtypes = [ctypes.POINTER(GdnShape), u16p, c_u32, u16p, f32p, u16p, ctypes.c_void_p, u16p, f32p, u8p, c_u32, u16p,
+                               f32p, u8p, u16p]
+lib.orc_gdn_fold.restype = c_int
+lib.orc_gdn_fold.argtypes = [ctypes.POINTER(GdnShape), u16p, f32p, u8p, c_u32, c_u32, u16p, f32p]
+lib.orc_gdn_reference.restype = c_int
+lib.orc_gdn_reference.argtypes = [ctypes.POINTER(GdnShape), u16p, c_u32, u16p, f32p, u16p, u16p, f32p, f64p, f64p, f64p, f64p, f64p]
+
+
+def gdn_fold(shape, conv_in, state_in, step_tape, path, rows):
+    conv_out = np.zeros((3, shape.conv_dim), np.uint16)
+    state_out = np.zeros_like(state_in)
+    conv_in, state_in = np.ascontiguousarray(conv_in), np.ascontiguousarray(state_in)
+    rc = lib.orc_gdn_fold(ctypes.byref(shape), _p(conv_in, u16p), _p(state_in, f32p), _p(step_tape, u8p), path, rows,
+                          _p(conv_out, u16p), _p(state_out, f32p))
+    return rc, conv_out, state_out
+
+
+def gdn_reference(shape, packed, conv_weights, a_scale, dt_bias, conv_in, state_in):
+    """fp64: (kv rows [rows][kv width], beta, decay [rows][vh], state after the rows, outputs [rows][vh][128])."""
+    rows, vh = packed.shape[0], shape.value_heads
+    kvw = (shape.key_heads + vh) * 128
+    kv = np.zeros((rows, kvw)); beta = np.zeros((rows, vh)); decay = np.zeros((rows, vh))
+    state = np.zeros((vh, 128, 128)); out = np.zeros((rows, vh, 128))
+    packed, conv_weights, a_scale, dt_bias, conv_in, state_in = (np.ascontiguousarray(x) for x in (
+        packed, conv_weights, a_scale, dt_bias, conv_in, state_in))
+    rc = lib.orc_gdn_reference(ctypes.byref(shape), _p(packed, u16p), rows, _p(conv_weights, u16p), _p(a_scale, f32p), _p(dt_bias, u16p),
+                               _p(conv_in, u16p), _p(state_in, f32p), _p(kv, f64p), _p(beta, f64p), _p(decay, f64p), _p(state, f64p),
+                               _p(out, f64p))
+    assert rc == 0
+    return kv, beta, decay, state, out
+
+
+def gdn_step(S, k, v, decay, beta, q=None):
+    S = np.ascontiguousarray(S, np.float32).copy()
+    o = np.zeros(S.shape[0], np.float32)
+    k, v = np.ascontiguousarray(k, np.float32), np.ascontiguousarray(v, np.float32)
+    qq = np.ascontiguousarray(q, np.float32) if q is not None else None
+    lib.orc_gdn_step(_p(S, f32p), S.shape[0], _p(k, f32p), _p(v, f32p), decay, beta, _p(qq, f32p), _p(o, f32p) if q is not None else None)
+    return S, o

@@ -1,0 +1,104 @@
+"""The GDN oracle against the fp64 textbook recurrence (the check the reference's own test makes,
+gdn_decode_metal_test.mm:373-598, with its tolerances) and against the invariants of the tape
+protocol: a fold equals what the next step holds, a rejected suffix never reaches the state."""
+import numpy as np
+import pytest
+
+from tests import oracle as orc
+from tests.gdn_case import make_layer, make_rows, make_state, ulps
+
+
+def test_step_matches_the_fp64_recurrence():
+    rng = np.random.default_rng(3)
+    shape, conv_w, a_scale, dt_bias, norm = make_layer(rng, 2, 4)
+    rows = 16
+    packed = make_rows(rng, shape, rows)
+    conv_in, state_in = make_state(rng, shape)
+    _, state0, tape, hidden = orc.gdn_decode(shape, packed, conv_w, a_scale, dt_bias, norm, conv_in, state_in)
+    assert np.array_equal(state0, state_in)          # nothing pending: the state before the rows is the state
+    inputs, kv, decay, beta = orc.gdn_split_tape(shape, tape)
+    kv64, beta64, decay64, state64, out64 = orc.gdn_reference(shape, packed, conv_w, a_scale, dt_bias, conv_in, state_in)
+    assert np.array_equal(inputs[:rows], packed[:, :shape.conv_dim])
+    # k/v rows within 3 bf16 steps (:425-429), beta within 2 (:451), decay 1e-4 relative with one bf16 step on the softplus (:457-468)
+    assert ulps(kv[:rows], orc.f32_to_bf16(kv64.astype(np.float32))).max() <= 3
+    assert ulps(beta[:rows], orc.f32_to_bf16(beta64.astype(np.float32))).max() <= 2
+    vh = shape.value_heads
+    x = (orc.bf16_to_f32(packed[:, shape.conv_dim + vh * 128 + vh:shape.conv_dim + vh * 128 + 2 * vh]).astype(np.float64)
+         + orc.bf16_to_f32(dt_bias).astype(np.float64)[None, :])
+    softplus = np.maximum(x, 0) + np.log1p(np.exp(-np.abs(x)))
+    # bf16(a + dt_bias) and bf16(softplus) each move the exponent by up to half a bf16 step
+    assert np.all(np.abs(decay[:rows] - decay64) <= decay64 * (1e-4 + np.abs(a_scale)[None, :] * (np.abs(x) + softplus) * 2.0 ** -8))
+    # the state after the rows, through the next step's fold: 1e-4 relative to the state's scale (:531)
+    _, state1, _, _ = orc.gdn_decode(shape, make_rows(rng, shape, 1), conv_w, a_scale, dt_bias, norm, conv_in, state_in,
+                                     pending_tape=tape, pending_path=(1 << rows) - 1)
+    # the fp64 reference ran on unrounded k, v and gates: bound by the rounding of those (bf16 inputs, 16 rows)
+    assert np.abs(state1 - state64).max() <= 2e-2 * np.abs(state64).max()
+    # hidden rows: gate the fp64 outputs the same way; a few bf16 steps, nearly all exact or one step
+    z = orc.bf16_to_f32(packed[:, shape.conv_dim:shape.conv_dim + vh * 128]).astype(np.float64).reshape(rows, vh, 128)
+    w = orc.bf16_to_f32(norm).astype(np.float64)
+    normed = out64 / np.sqrt((out64 ** 2).mean(axis=2, keepdims=True) + 1e-6) * w
+    want = orc.f32_to_bf16((normed * z / (1 + np.exp(-z))).astype(np.float32)).reshape(rows, vh * 128)
+    # q, k and v enter the recurrence rounded to bf16 (2^-9 each), so an output carries a few bf16 steps of
+    # its own size plus a cancellation term of its row's size (:590-598)
+    got, ref = orc.bf16_to_f32(hidden).astype(np.float64), orc.bf16_to_f32(want).astype(np.float64)
+    scale = np.abs(ref).reshape(rows, vh, 128).max(axis=2, keepdims=True).repeat(128, axis=2).reshape(rows, vh * 128)
+    error = np.abs(got - ref)
+    assert np.all(error <= 2.0 ** -5 * np.abs(ref) + 2.0 ** -6 * scale)
+    assert (error <= 2.0 ** -7 * np.abs(ref) + 2.0 ** -9 * scale).mean() >= 0.9
+
+
+def test_one_row_is_the_closed_form():
+    """S' = d S + beta (v - d S k) k^T and o = S' q, in fp64 sums, from the tape's own k, v and gates."""
+    rng = np.random.default_rng(4)
+    shape, conv_w, a_scale, dt_bias, norm = make_layer(rng, 1, 2)
+    packed = make_rows(rng, shape, 1)
+    conv_in, state_in = make_state(rng, shape)
+    _, _, tape, _ = orc.gdn_decode(shape, packed, conv_w, a_scale, dt_bias, norm, conv_in, state_in)
+    _, kv, decay, beta = orc.gdn_split_tape(shape, tape)
+    _, state1, _, _ = orc.gdn_decode(shape, make_rows(rng, shape, 2), conv_w, a_scale, dt_bias, norm, conv_in, state_in,
+                                     pending_tape=tape, pending_path=1)
+    for h in range(2):
+        k = orc.bf16_to_f32(kv[0, :128]).astype(np.float64)
+        v = orc.bf16_to_f32(kv[0, 128 + 128 * h:256 + 128 * h]).astype(np.float64)
+        d, b = float(decay[0, h]), float(orc.bf16_to_f32(beta[0, h:h + 1])[0])
+        S = state_in[h].astype(np.float64) * d
+        want = S + b * np.outer(v - S @ k, k)
+        assert np.abs(state1[h] - want).max() <= 1e-5 * np.abs(want).max()
+        got, _ = orc.gdn_step(state_in[h], k, v, d, b)
+        assert np.abs(got - want).max() <= 1e-5 * np.abs(want).max()
+
+
+@pytest.mark.parametrize("accepted", [0, 1, 5, 16])
+def test_fold_and_rollback(accepted):
+    """The state a step writes holds exactly the accepted rows of the step before (a rejected suffix
+    never reaches it), the fold of those rows alone is that state bit for bit, and the block's outputs
+    are those of the same tokens run as one chain."""
+    rng = np.random.default_rng(10 + accepted)
+    shape, conv_w, a_scale, dt_bias, norm = make_layer(rng, 2, 4)
+    conv_in, state_in = make_state(rng, shape)
+    first = make_rows(rng, shape, 16)
+    second = make_rows(rng, shape, 7)
+    conv0, state0, tape0, hidden_first = orc.gdn_decode(shape, first, conv_w, a_scale, dt_bias, norm, conv_in, state_in)
+    path = (1 << accepted) - 1
+    conv1, state1, tape1, hidden1 = orc.gdn_decode(shape, second, conv_w, a_scale, dt_bias, norm, conv0, state0,
+                                                   pending_tape=tape0 if accepted else None, pending_path=path)
+    # the same tokens as one history: the accepted rows, then the second block
+    if accepted:
+        rc, conv_f, state_f = orc.gdn_fold(shape, conv0, state0, tape0, path, accepted)
+        assert rc == 0
+        assert np.array_equal(conv_f, conv1) and state_f.tobytes() == state1.tobytes()
+        # a step of only the accepted rows, wholly accepted, leaves the same state: rejection costs nothing
+        convA, stateA, tapeA, hiddenA = orc.gdn_decode(shape, first[:accepted], conv_w, a_scale, dt_bias, norm, conv_in, state_in)
+        assert np.array_equal(hiddenA, hidden_first[:accepted])
+        convB, stateB, _, hiddenB = orc.gdn_decode(shape, second, conv_w, a_scale, dt_bias, norm, convA, stateA,
+                                                   pending_tape=tapeA, pending_path=path)
+        assert np.array_equal(convB, conv1) and stateB.tobytes() == state1.tobytes() and np.array_equal(hiddenB, hidden1)
+        if accepted + 7 <= 16:
+            # and one chain of accepted + 7 rows gives the second block's outputs bit for bit
+            _, _, _, hidden_chain = orc.gdn_decode(shape, np.concatenate([first[:accepted], second]), conv_w, a_scale, dt_bias, norm,
+                                                   conv_in, state_in)
+            assert np.array_equal(hidden_chain[accepted:], hidden1)
+        rc, _, _ = orc.gdn_fold(shape, conv0, state0, tape0, path, accepted + 1)
+        assert rc == 1                                   # a path shorter than the rows asked for folds nothing
+    else:
+        assert np.array_equal(conv1, conv_in) and state1.tobytes() == state_in.tobytes()
