@@ -174,6 +174,26 @@ sp_status spo_gdn_add_fold(spo_graph *graph, sp_buffer *states, sp_buffer *tape,
                            uint64_t state_cell, uint64_t fold_cell, const spo_gdn_shape *shape, uint32_t layers, uint32_t rows,
                            const spo_gdn_state_strides *state);
 
+/* ---- MoE (runtime/ops/MoE.hpp:403-410, MoE.cpp:143-287; runtime/metal/abi/MoE.h:23-245) ---- */
+typedef struct spo_moe_shape { uint32_t hidden, ffn, experts, top_k; } spo_moe_shape;
+typedef struct spo_moe_workspace { /* in the order of spo_moe_workspace_sizes */
+  sp_buffer *selected, *weights, *route_slot, *slot_row, *tile_expert, *tile_rows, *tile_total, *tables, *next_tables,
+      *intermediate, *expert_output;
+} spo_moe_workspace;
+/* Bytes of each workspace buffer for a step of `rows` rows (1..256). */
+sp_status spo_moe_workspace_sizes(const spo_moe_shape *shape, uint32_t rows, uint64_t sizes[11]);
+/* MoE::addRouting (MoE.cpp:143-206): from fp32 router scores [rows][score_stride], each row's top_k
+ * experts by (score descending, id ascending) in selected, their weights exp2((s_r - s_0) log2 e) / sum
+ * in rank order, and the routes grouped by expert into tiles of up to 16 rows. */
+sp_status spo_moe_add_routing(spo_graph *graph, sp_buffer *scores, uint32_t score_stride, const spo_moe_workspace *workspace,
+                              const spo_moe_shape *shape, uint32_t rows);
+/* MoE::addRouted (MoE.cpp:242-287): output = bf16(residual + sum over a row's routes, in rank order, of
+ * weight * down_e(silu(gate_e x) * up_e x)). *_images hold every expert's re-tiled image of the tensor,
+ * expert e at e * spo_gguf_image_bytes(format, rows of the tensor, its inputs). */
+sp_status spo_moe_add_routed(spo_graph *graph, sp_buffer *normalized, sp_buffer *residual, sp_buffer *output, sp_buffer *gate_images,
+                             sp_buffer *up_images, sp_buffer *down_images, uint32_t format, uint32_t down_format,
+                             const spo_moe_workspace *workspace, const spo_moe_shape *shape, uint32_t rows);
+
 /* ---- Sampling (runtime/ops/Sampling.hpp:64-254, Sampling.cpp:283-357) ---- */
 typedef struct spo_lane_rows { uint32_t first, rows; } spo_lane_rows; /* SplashLaneRows */
 /* Sampling::workspace: bytes of the argmax partial values and indices, the masses, ranges, decisions. */

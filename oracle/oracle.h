@@ -22,6 +22,8 @@
 //                                   the reference's own test makes) and fold/rollback invariants.
 //   orc_argmax / orc_accept_tree    pinned by brute force on tiny vocabularies.
 //   orc_rejection_*                 pinned by enumeration: selection law equals target to 1e-12.
+//   orc_moe_*                       pinned by a stable sort and softmax closed form; the layer by the dense FFN it
+//                                   reduces to when every expert is the same.
 #pragma once
 #include <stddef.h>
 #include <stdint.h>
@@ -160,6 +162,16 @@ int orc_gdn_fold(const struct OrcGdnShape *s, const uint16_t *conv_in, const flo
 int orc_gdn_reference(const struct OrcGdnShape *s, const uint16_t *packed, uint32_t rows, const uint16_t *conv_weights,
                       const float *a_scale, const uint16_t *dt_bias, const uint16_t *conv_in, const float *state_in,
                       double *kv, double *beta, double *decay, double *state_out, double *outputs);
+
+// ---- mixture of experts ----
+// kernels/shared/moe.metal:23-113: each row's top_k experts ranked by (score descending, id ascending)
+// and their weights exp2((s_r - s_0) log2 e) / sum, the sum in rank order.
+void orc_moe_route(const float *scores, uint32_t rows, uint32_t experts, uint32_t stride, uint32_t top_k, uint32_t *selected,
+                   float *weights);
+// kernels/shared/moe.metal:367-392: out = bf16(residual + sum over ranks of w y) in fp32, rank order;
+// y bf16 [rows][top_k][hidden] the expert outputs of the routes.
+void orc_moe_combine(const uint16_t *y, const float *weights, const uint16_t *residual, uint32_t rows, uint32_t top_k,
+                     uint32_t hidden, uint16_t *out);
 
 #ifdef __cplusplus
 }

@@ -109,6 +109,18 @@ class GdnDecodeBuffers(ctypes.Structure):
                                    "hidden")] + [("float_norm", c_u32)]
 
 
+class MoeShape(ctypes.Structure):
+    _fields_ = [("hidden", c_u32), ("ffn", c_u32), ("experts", c_u32), ("top_k", c_u32)]
+
+
+MOE_WORKSPACE_FIELDS = ("selected", "weights", "route_slot", "slot_row", "tile_expert", "tile_rows", "tile_total", "tables", "next_tables",
+                        "intermediate", "expert_output")
+
+
+class MoeWorkspace(ctypes.Structure):
+    _fields_ = [(n, c_p) for n in MOE_WORKSPACE_FIELDS]
+
+
 class SamplingBuffers(ctypes.Structure):
     _fields_ = [(n, c_p) for n in ("logits", "tokens", "partial_values", "partial_indices", "draft_probabilities", "uniforms",
                                    "masses", "ranges", "decisions", "input_tokens", "tree_rows")]
@@ -209,6 +221,9 @@ _sig("spo_rope_add_tree_tables", c_int, c_p, c_p, c_p, c_p, c_p, c_u32, P(RopeSe
 _sig("spo_gdn_layout", c_int, P(GdnShape), c_u32, P(GdnStateStrides), P(c_u64), P(c_u64))
 _sig("spo_gdn_add_decode", c_int, c_p, P(GdnDecodeBuffers), P(GdnShape), c_u32, P(GdnStateStrides), c_u32, P(GdnLane), c_u32, c_int)
 _sig("spo_gdn_add_fold", c_int, c_p, c_p, c_p, c_p, c_u64, c_u64, c_u64, P(GdnShape), c_u32, c_u32, P(GdnStateStrides))
+_sig("spo_moe_workspace_sizes", c_int, P(MoeShape), c_u32, P(c_u64))
+_sig("spo_moe_add_routing", c_int, c_p, c_p, c_u32, P(MoeWorkspace), P(MoeShape), c_u32)
+_sig("spo_moe_add_routed", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_u32, c_u32, P(MoeWorkspace), P(MoeShape), c_u32)
 _sig("spo_sampling_workspace", c_int, c_u32, P(c_u64))
 _sig("spo_sampling_add_verify", c_int, c_p, P(SamplingBuffers), c_u32, c_u32, P(LaneRows), P(ctypes.c_float), c_u32)
 _sig("spo_sampling_add_acceptance", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, P(LaneRows), P(c_u32), c_u32, P(c_u32))

@@ -1,0 +1,65 @@
+// Mixture-of-experts routing of a verify block: parameters shared by the host operator (ops/Moe)
+// and the HIP kernels. The counterpart of the reference's runtime/metal/abi/MoE.h:23-245.
+//
+// A row's router scores (fp32, one per expert) select top_k experts, ranked by (score descending,
+// expert id ascending); route (row, rank) carries the weight exp2((s_rank - s_0) log2 e) / sum over
+// the k selected, summed in rank order. Routes are grouped by expert into tiles of up to 16 rows (one
+// MFMA row tile): tile t serves expert tile_expert[t] with tile_rows[t] rows in grouped slots
+// 16 t .. 16 t + tile_rows[t] - 1; route_slot[route] names a route's slot and slot_row[slot] the
+// row a slot gathers (0xFFFFFFFF for an empty slot). An expert's routes keep their route order.
+#pragma once
+#include <stdint.h>
+#include "abi/Gguf.h"
+
+#define MOE_MAXIMUM_EXPERTS 256u
+#define MOE_MAXIMUM_TOP 16u
+#define MOE_TILE_ROWS 16u
+#define MOE_NO_ROW 0xFFFFFFFFu
+
+// The most tiles `routes` routes over `experts` experts can take.
+#if defined(__HIPCC__)
+__host__ __device__
+#endif
+inline uint32_t moe_maximum_tiles(uint32_t routes, uint32_t experts) {
+  const uint32_t full = routes / MOE_TILE_ROWS, partial = experts < routes ? experts : routes;
+  return full + partial;
+}
+
+// moe_route_select: grid (rows), 64 threads.
+struct MoeRouteParams {
+  uint32_t rows, experts, top_k;
+  uint32_t score_stride;  // floats between rows of scores
+};
+// moe_group_routes: one workgroup of 256 threads.
+struct MoeGroupParams {
+  uint32_t routes;  // rows * top_k
+  uint32_t experts, top_k;
+  uint32_t maximum_tiles;
+};
+// moe_gather_table: grid (hidden / 32, maximum tiles), 64 threads: a tile's rows as its activation table.
+struct MoeGatherParams {
+  uint32_t hidden;
+  uint32_t maximum_tiles;
+  uint64_t table_bytes;  // between tiles' tables
+};
+// moe_combine: grid (rows, hidden / 256), 256 threads: out = bf16(residual + sum_rank w y[slot]) in rank order.
+struct MoeCombineParams {
+  uint32_t rows, hidden, top_k;
+  uint32_t reserved;
+};
+
+// gguf_moe_decode_<fmt>_<a|gt>: grid (workgroups of one expert projection, maximum tiles), 256 threads.
+struct GgufMoeParams {
+  struct GgufDecodeParams decode;  // rows is the tile's, from tile_rows; splits 1
+  uint64_t expert_bytes;           // between experts' images of a tensor
+  uint64_t table_bytes;            // between tiles' activation tables
+  uint64_t next_table_bytes;       // between tiles' next tables (table epilogue)
+  uint32_t out_row_bytes;          // bytes of an output row
+  uint32_t reserved;
+};
+
+#ifdef __cplusplus
+static_assert(sizeof(MoeRouteParams) == 16 && sizeof(MoeGroupParams) == 16 && sizeof(MoeGatherParams) == 16 &&
+                  sizeof(MoeCombineParams) == 16 && sizeof(GgufMoeParams) == 80,
+              "MoE parameters have the same size on both sides");
+#endif

@@ -15,6 +15,7 @@
 // (grid.y) sum theirs through fp32 partials in split order, the last arriver applying the
 // epilogue (the reference's split_reduce.h:28-54), so a result never depends on arrival order.
 #include "abi/Gguf.h"
+#include "abi/Moe.h"
 #include "backend/KernelRegistry.hpp"
 #include "kernels/gguf_device.hpp"
 
@@ -319,12 +320,13 @@ __device__ __forceinline__ void accumulate_record(const Record<FMT> &rec, const 
 // workgroup walk that range in step and share its activations through LDS. Unit u of a dispatch
 // is tile u of its concatenated segments; of a gate/up pair, unit 2 j is gate tile j and unit
 // 2 j + 1 up tile j, so the two halves of a pair sit in neighbouring waves of one workgroup.
+// `item` is the workgroup's place in the dispatch (blockIdx.x of gguf_decode).
 template <uint32_t FMT, int RT, uint32_t EP>
-__global__ __launch_bounds__(256) void gguf_decode(const uint8_t *__restrict__ seg0, const uint8_t *__restrict__ seg1,
-                                                   const uint8_t *__restrict__ seg2, const uint8_t *__restrict__ table,
-                                                   void *__restrict__ out, const uint16_t *__restrict__ residual,
-                                                   float *__restrict__ partials, uint32_t *__restrict__ counters,
-                                                   GgufDecodeParams p) {
+__device__ __forceinline__ void decode_workgroup(const uint8_t *__restrict__ seg0, const uint8_t *__restrict__ seg1,
+                                                 const uint8_t *__restrict__ seg2, const uint8_t *__restrict__ table,
+                                                 void *__restrict__ out, const uint16_t *__restrict__ residual,
+                                                 float *__restrict__ partials, uint32_t *__restrict__ counters,
+                                                 const GgufDecodeParams &p, const uint32_t item) {
   constexpr uint32_t kRecord = FMT == GGUF_FMT_Q4K ? GGUF_Q4K_RECORD : GGUF_Q6K_RECORD;
   constexpr bool kTable = EP == GGUF_EPILOGUE_GATE_UP_TABLE, kGateUp = EP == GGUF_EPILOGUE_GATE_UP || kTable;
   constexpr uint32_t kColumnPart = FMT == GGUF_FMT_Q4K ? 2048u : GGUF_Q6K_SCALES;
@@ -338,9 +340,9 @@ __global__ __launch_bounds__(256) void gguf_decode(const uint8_t *__restrict__ s
 
   const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6, c = lane & 15u, kq = lane >> 4;
   // Workgroup items: the whole groups first, then the partitioned ones part by part.
-  uint32_t group = blockIdx.x, split = 0, splits = 1;
-  if (blockIdx.x >= p.whole_groups && p.splits > 1) {
-    const uint32_t past = blockIdx.x - p.whole_groups;
+  uint32_t group = item, split = 0, splits = 1;
+  if (item >= p.whole_groups && p.splits > 1) {
+    const uint32_t past = item - p.whole_groups;
     group = p.whole_groups + uint32_t(__builtin_amdgcn_readfirstlane(int(past / p.splits)));
     split = uint32_t(__builtin_amdgcn_readfirstlane(int(past % p.splits)));
     splits = p.splits;
@@ -572,6 +574,40 @@ __global__ __launch_bounds__(256) void gguf_decode(const uint8_t *__restrict__ s
       }
   }
 }
+
+template <uint32_t FMT, int RT, uint32_t EP>
+__global__ __launch_bounds__(256) void gguf_decode(const uint8_t *__restrict__ seg0, const uint8_t *__restrict__ seg1,
+                                                   const uint8_t *__restrict__ seg2, const uint8_t *__restrict__ table,
+                                                   void *__restrict__ out, const uint16_t *__restrict__ residual,
+                                                   float *__restrict__ partials, uint32_t *__restrict__ counters,
+                                                   GgufDecodeParams p) {
+  decode_workgroup<FMT, RT, EP>(seg0, seg1, seg2, table, out, residual, partials, counters, p, blockIdx.x);
+}
+
+// The routed experts of a mixture-of-experts layer (the reference's moe_expert_gguf_*, abi/MoE.h):
+// grid (workgroups of one expert projection, tile slots). Tile t holds up to 16 rows routed to
+// expert tile_expert[t]; it reads that expert's image (expert_bytes apart in each bound tensor), its
+// own activation table (table_bytes apart) and writes its own 16 output rows (and, with the table
+// epilogue, its own next table). Slots at or past tile_total[0] are empty.
+template <uint32_t FMT, uint32_t EP>
+__global__ __launch_bounds__(256) void gguf_moe_decode(const uint8_t *__restrict__ seg0, const uint8_t *__restrict__ seg1,
+                                                       const uint8_t *__restrict__ tables, uint8_t *__restrict__ out,
+                                                       uint8_t *__restrict__ next_tables, const uint32_t *__restrict__ tile_expert,
+                                                       const uint32_t *__restrict__ tile_rows, const uint32_t *__restrict__ tile_total,
+                                                       GgufMoeParams m) {
+  const uint32_t tile = blockIdx.y;
+  if (tile >= tile_total[0]) return;
+  const uint32_t expert = tile_expert[tile];
+  GgufDecodeParams p = m.decode;
+  p.rows = tile_rows[tile];
+  decode_workgroup<FMT, 1, EP>(seg0 + expert * m.expert_bytes, seg1 + expert * m.expert_bytes, seg0 + expert * m.expert_bytes,
+                               tables + tile * m.table_bytes, out + size_t(tile) * 16u * m.out_row_bytes,
+                               reinterpret_cast<const uint16_t *>(next_tables + tile * m.next_table_bytes), nullptr, nullptr, p,
+                               blockIdx.x);
+}
+SP_REGISTER_KERNEL("gguf_moe_decode_q4k_gt", (&gguf_moe_decode<GGUF_FMT_Q4K, GGUF_EPILOGUE_GATE_UP_TABLE>));
+SP_REGISTER_KERNEL("gguf_moe_decode_q4k_a", (&gguf_moe_decode<GGUF_FMT_Q4K, GGUF_EPILOGUE_PLAIN>));
+SP_REGISTER_KERNEL("gguf_moe_decode_q6k_a", (&gguf_moe_decode<GGUF_FMT_Q6K, GGUF_EPILOGUE_PLAIN>));
 
 #define SP_GGUF_DECODE(fmt, FMT, rows, RT)                                                              \
   SP_REGISTER_KERNEL("gguf_decode_" fmt "_m" #rows "_a", &gguf_decode<FMT, RT, GGUF_EPILOGUE_PLAIN>);   \

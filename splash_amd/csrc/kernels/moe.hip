@@ -1,0 +1,152 @@
+// Mixture-of-experts routing around the grouped expert projections (kernels/gguf_linear.hip):
+// top-k selection, grouping of routes by expert, the tiles' activation tables, the weighted sum
+// (the reference's kernels/shared/moe.metal).
+#include "abi/Moe.h"
+#include "backend/KernelRegistry.hpp"
+#include "kernels/device_common.hpp"
+
+namespace splash::kernels {
+
+// moe_route_select (moe.metal:23-113): one wave per row; lane l holds experts l, l + 64, ... Each
+// rank takes the highest remaining score and, among equals, the lowest expert id.
+__global__ __launch_bounds__(64) void moe_route_select(const float *__restrict__ scores, uint32_t *__restrict__ selected,
+                                                       float *__restrict__ weights, MoeRouteParams p) {
+  constexpr uint32_t kPerLane = MOE_MAXIMUM_EXPERTS / 64u;
+  __shared__ float ordered[MOE_MAXIMUM_TOP];
+  const uint32_t row = blockIdx.x, lane = threadIdx.x;
+  float mine[kPerLane];
+#pragma unroll
+  for (uint32_t slot = 0; slot < kPerLane; ++slot) {
+    const uint32_t expert = lane + 64u * slot;
+    mine[slot] = expert < p.experts ? scores[size_t(row) * p.score_stride + expert] : -INFINITY;
+  }
+  for (uint32_t rank = 0; rank < p.top_k; ++rank) {
+    float best = -INFINITY;
+    uint32_t bestSlot = 0;
+#pragma unroll
+    for (uint32_t slot = 0; slot < kPerLane; ++slot)
+      if (mine[slot] > best) {
+        best = mine[slot];
+        bestSlot = slot;
+      }
+    const float rowBest = wave_max(best);
+    uint32_t candidate = best == rowBest ? lane + 64u * bestSlot : 0xFFFFFFFFu;
+    uint32_t winner = candidate;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) winner = min(winner, uint32_t(__shfl_xor(int(winner), o, 64)));
+    if (candidate == winner) {
+#pragma unroll
+      for (uint32_t slot = 0; slot < kPerLane; ++slot)
+        if (slot == bestSlot) mine[slot] = -INFINITY;
+    }
+    if (lane == 0) {
+      ordered[rank] = rowBest;
+      selected[size_t(row) * p.top_k + rank] = winner;
+    }
+  }
+  __syncthreads();
+  if (lane < p.top_k) {
+    float denominator = 0.f;
+    for (uint32_t other = 0; other < p.top_k; ++other) denominator += __builtin_amdgcn_exp2f((ordered[other] - ordered[0]) * 1.44269504089f);
+    weights[size_t(row) * p.top_k + lane] = __builtin_amdgcn_exp2f((ordered[lane] - ordered[0]) * 1.44269504089f) / denominator;
+  }
+}
+SP_REGISTER_KERNEL("moe_route_select", &moe_route_select);
+
+// moe_group_routes: thread e walks the routes in order and gives expert e's their slots, so an
+// expert's routes keep their route order and the grouping never depends on timing.
+__global__ __launch_bounds__(256) void moe_group_routes(const uint32_t *__restrict__ selected, uint32_t *__restrict__ route_slot,
+                                                        uint32_t *__restrict__ slot_row, uint32_t *__restrict__ tile_expert,
+                                                        uint32_t *__restrict__ tile_rows, uint32_t *__restrict__ tile_total,
+                                                        MoeGroupParams p) {
+  __shared__ uint32_t counts[MOE_MAXIMUM_EXPERTS], firstTile[MOE_MAXIMUM_EXPERTS];
+  const uint32_t e = threadIdx.x;
+  for (uint32_t slot = e; slot < p.maximum_tiles * MOE_TILE_ROWS; slot += 256u) slot_row[slot] = MOE_NO_ROW;
+  uint32_t count = 0;
+  if (e < p.experts)
+    for (uint32_t route = 0; route < p.routes; ++route) count += selected[route] == e ? 1u : 0u;
+  counts[e] = e < p.experts ? count : 0u;
+  __syncthreads();
+  if (e == 0) {
+    uint32_t tiles = 0;
+    for (uint32_t x = 0; x < p.experts; ++x) {
+      firstTile[x] = tiles;
+      tiles += (counts[x] + MOE_TILE_ROWS - 1) / MOE_TILE_ROWS;
+    }
+    tile_total[0] = tiles;
+  }
+  __syncthreads();
+  if (e >= p.experts || !count) return;
+  const uint32_t first = firstTile[e], tiles = (count + MOE_TILE_ROWS - 1) / MOE_TILE_ROWS;
+  for (uint32_t t = 0; t < tiles; ++t) {
+    tile_expert[first + t] = e;
+    tile_rows[first + t] = min(MOE_TILE_ROWS, count - t * MOE_TILE_ROWS);
+  }
+  uint32_t placed = 0;
+  for (uint32_t route = 0; route < p.routes; ++route)
+    if (selected[route] == e) {
+      const uint32_t slot = (first + placed / MOE_TILE_ROWS) * MOE_TILE_ROWS + placed % MOE_TILE_ROWS;
+      route_slot[route] = slot;
+      slot_row[slot] = route / p.top_k;
+      ++placed;
+    }
+}
+SP_REGISTER_KERNEL("moe_group_routes", &moe_group_routes);
+
+// moe_gather_table: the activation table (abi/Gguf.h) of each tile's gathered rows, as
+// gguf_prepare_table writes a block's; empty slots are zero rows.
+__global__ __launch_bounds__(64) void moe_gather_table(const uint16_t *__restrict__ input, const uint32_t *__restrict__ slot_row,
+                                                       const uint32_t *__restrict__ tile_total, uint8_t *__restrict__ tables,
+                                                       MoeGatherParams p) {
+  const uint32_t g = blockIdx.x, tile = blockIdx.y, lane = threadIdx.x, r = lane & 15u, kq = lane >> 4;
+  if (tile >= tile_total[0]) return;
+  const uint32_t G = p.hidden / 32u, row = slot_row[tile * MOE_TILE_ROWS + r];
+  uint8_t *table = tables + tile * p.table_bytes;
+  float v[8];
+  uint32_t bits[8] = {};
+#pragma unroll
+  for (uint32_t e = 0; e < 8; ++e) v[e] = 0.f;
+  if (row != MOE_NO_ROW) {
+    const uint16_t *x = input + size_t(row) * p.hidden + 32u * g;
+#pragma unroll
+    for (uint32_t e = 0; e < 8; ++e) {
+      bits[e] = x[gguf_operand_input(kq, e)];
+      v[e] = bf16_bits_to_float(bits[e]);
+    }
+  }
+  reinterpret_cast<uint4 *>(table)[size_t(g) * 64u + lane] =
+      make_uint4(bits[0] | (bits[1] << 16), bits[2] | (bits[3] << 16), bits[4] | (bits[5] << 16), bits[6] | (bits[7] << 16));
+  const float half0 = (v[0] + v[2]) + (v[1] + v[3]), half1 = (v[4] + v[6]) + (v[5] + v[7]);
+  float h0[4], h1[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    h0[q] = __shfl(half0, int(r) + 16 * q, 64);
+    h1[q] = __shfl(half1, int(r) + 16 * q, 64);
+  }
+  const float s0 = ((h0[0] + h0[1]) + h0[2]) + h0[3], s1 = ((h1[0] + h1[1]) + h1[2]) + h1[3];
+  if (kq == 0) {
+    float *sums32 = reinterpret_cast<float *>(table + gguf_table_sums32_offset(p.hidden, 1));
+    float *sums16 = reinterpret_cast<float *>(table + gguf_table_sums16_offset(p.hidden, 1));
+    sums32[size_t(g) * 16u + r] = s0 + s1;
+    sums16[(2u * size_t(g)) * 16u + r] = s0;
+    sums16[(2u * size_t(g) + 1u) * 16u + r] = s1;
+  }
+}
+SP_REGISTER_KERNEL("moe_gather_table", &moe_gather_table);
+
+// moe_combine (moe.metal:367-392): out = bf16(residual + sum over the row's routes of w y) in rank order, fp32.
+__global__ __launch_bounds__(256) void moe_combine(const uint16_t *__restrict__ expert_output, const uint32_t *__restrict__ route_slot,
+                                                   const float *__restrict__ weights, const uint16_t *__restrict__ residual,
+                                                   uint16_t *__restrict__ output, MoeCombineParams p) {
+  const uint32_t row = blockIdx.x, d = blockIdx.y * 256u + threadIdx.x;
+  if (d >= p.hidden) return;
+  float value = bf16_bits_to_float(residual[size_t(row) * p.hidden + d]);
+  for (uint32_t rank = 0; rank < p.top_k; ++rank) {
+    const size_t route = size_t(row) * p.top_k + rank;
+    value += weights[route] * bf16_bits_to_float(expert_output[size_t(route_slot[route]) * p.hidden + d]);
+  }
+  output[size_t(row) * p.hidden + d] = uint16_t(float_to_bf16_bits(value));
+}
+SP_REGISTER_KERNEL("moe_combine", &moe_combine);
+
+} // namespace splash::kernels

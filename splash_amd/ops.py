@@ -333,6 +333,30 @@ class GDN:
         graph._keep.extend([states, tape, retained_rows])
 
 
+class MoE:
+    """ops::MoE: routing (addRouting) and the routed experts with their weighted sum (addRouted)."""
+
+    def __init__(self, backend, hidden, ffn, experts, top_k, rows):
+        self.shape = nat.MoeShape(hidden, ffn, experts, top_k)
+        self.rows = rows
+        sizes = (ctypes.c_uint64 * 11)()
+        check(lib.spo_moe_workspace_sizes(ctypes.byref(self.shape), rows, sizes))
+        self.buffers = {n: backend.allocate_buffer(max(int(b), 16), STORAGE_PRIVATE, "moe " + n) for n, b in zip(nat.MOE_WORKSPACE_FIELDS, sizes)}
+        self.workspace = nat.MoeWorkspace(**{n: b.handle for n, b in self.buffers.items()})
+
+    def add_routing(self, graph, scores, rows=None, score_stride=None):
+        check(lib.spo_moe_add_routing(graph.handle, scores.handle, score_stride or self.shape.experts, ctypes.byref(self.workspace),
+                                      ctypes.byref(self.shape), rows or self.rows))
+        graph._keep.extend([scores, self])
+
+    def add_routed(self, graph, normalized, residual, output, gate_images, up_images, down_images, rows=None, fmt=FMT_Q4K,
+                   down_fmt=FMT_Q4K):
+        check(lib.spo_moe_add_routed(graph.handle, normalized.handle, residual.handle, output.handle, gate_images.handle, up_images.handle,
+                                     down_images.handle, fmt, down_fmt, ctypes.byref(self.workspace), ctypes.byref(self.shape),
+                                     rows or self.rows))
+        graph._keep.extend([normalized, residual, output, gate_images, up_images, down_images, self])
+
+
 NO_TOKEN = 0xFFFFFFFF
 
 

@@ -359,3 +359,44 @@ def gdn_step(S, k, v, decay, beta, q=None):
     qq = np.ascontiguousarray(q, np.float32) if q is not None else None
     lib.orc_gdn_step(_p(S, f32p), S.shape[0], _p(k, f32p), _p(v, f32p), decay, beta, _p(qq, f32p), _p(o, f32p) if q is not None else None)
     return S, o
+
+
+# ---- mixture of experts ----
+lib.orc_moe_route.restype = None
+lib.orc_moe_route.argtypes = [f32p, c_u32, c_u32, c_u32, c_u32, u32p, f32p]
+lib.orc_moe_combine.restype = None
+lib.orc_moe_combine.argtypes = [u16p, f32p, u16p, c_u32, c_u32, c_u32, u16p]
+
+
+def moe_route(scores, top_k):
+    scores = np.ascontiguousarray(scores, np.float32)
+    rows, experts = scores.shape
+    selected = np.zeros((rows, top_k), np.uint32)
+    weights = np.zeros((rows, top_k), np.float32)
+    lib.orc_moe_route(_p(scores, f32p), rows, experts, experts, top_k, _p(selected, u32p), _p(weights, f32p))
+    return selected, weights
+
+
+def moe_combine(y_bits, weights, residual_bits):
+    rows, top_k, hidden = y_bits.shape
+    out = np.zeros((rows, hidden), np.uint16)
+    y_bits, weights, residual_bits = (np.ascontiguousarray(a) for a in (y_bits, weights, residual_bits))
+    lib.orc_moe_combine(_p(y_bits, u16p), _p(weights, f32p), _p(residual_bits, u16p), rows, top_k, hidden, _p(out, u16p))
+    return out
+
+
+def moe_layer(x_bits, residual_bits, scores, top_k, gate_native, up_native, down_native, ffn, fmt=FMT_Q4K, down_fmt=FMT_Q4K):
+    """The routed experts of a layer: x bf16 [rows][hidden] (normalized), natives per expert. Each expert's
+    rows go through the oracle's projections together; a row's result does not depend on the rows beside it."""
+    rows, hidden = x_bits.shape
+    selected, weights = moe_route(scores, top_k)
+    y = np.zeros((rows, top_k, hidden), np.uint16)
+    for e in np.unique(selected):
+        r, k = np.nonzero(selected == e)
+        xe = np.ascontiguousarray(x_bits[r])
+        gate = gemm(fmt, gate_native[e], xe, ffn, want=("chain",))["chain"]
+        up = gemm(fmt, up_native[e], xe, ffn, want=("chain",))["chain"]
+        mid = swiglu(gate, up).reshape(len(r), ffn)
+        down = gemm(down_fmt, down_native[e], mid, hidden, want=("chain",))["chain"]
+        y[r, k] = f32_to_bf16(down)
+    return selected, weights, y, moe_combine(y, weights, residual_bits)

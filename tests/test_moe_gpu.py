@@ -1,0 +1,95 @@
+"""Mixture-of-experts routing, grouped expert projections and combine on the GPU against the oracle."""
+import numpy as np
+import pytest
+
+import splash_amd
+from splash_amd import ops
+from tests import oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+
+def run_layer(backend, rng, hidden, ffn, experts, top_k, rows, down_fmt=ops.FMT_Q4K):
+    gate = [orc.make_native(ops.FMT_Q4K, ffn, hidden, 100 + e) for e in range(experts)]
+    up = [orc.make_native(ops.FMT_Q4K, ffn, hidden, 300 + e) for e in range(experts)]
+    down = [orc.make_native(down_fmt, hidden, ffn, 500 + e) for e in range(experts)]
+    images = [backend.from_array(np.concatenate([ops.pack_gguf_image(f, n, r, k) for n in natives]))
+              for natives, f, r, k in ((gate, ops.FMT_Q4K, ffn, hidden), (up, ops.FMT_Q4K, ffn, hidden), (down, down_fmt, hidden, ffn))]
+    x = orc.f32_to_bf16(rng.standard_normal((rows, hidden)).astype(np.float32))
+    res = orc.f32_to_bf16(rng.standard_normal((rows, hidden)).astype(np.float32))
+    scores = rng.standard_normal((rows, experts)).astype(np.float32)
+    scores[0, :] = 0.5                                 # a row of ties: experts 0..top_k-1 in id order
+    moe = ops.MoE(backend, hidden, ffn, experts, top_k, rows)
+    out = backend.allocate_buffer(rows * hidden * 2)
+    graph = splash_amd.CommandGraph()
+    moe.add_routing(graph, backend.from_array(scores))
+    moe.add_routed(graph, backend.from_array(x), backend.from_array(res), out, *images, down_fmt=down_fmt)
+    assert len(graph) == 6
+    backend.run(graph)
+    got = out.download(np.uint16).reshape(rows, hidden)
+    want = orc.moe_layer(x, res, scores, top_k, gate, up, down, ffn, down_fmt=down_fmt)
+    return moe, got, want
+
+
+def check_layer(moe, got, want, rows, experts, top_k):
+    selected, weights, y, out = want
+    b = moe.buffers
+    got_selected = b["selected"].download(np.uint32)[:rows * top_k].reshape(rows, top_k)
+    assert np.array_equal(got_selected, selected)                        # routing is exact, ties by id
+    got_weights = b["weights"].download(np.float32)[:rows * top_k].reshape(rows, top_k)
+    assert np.abs(got_weights - weights).max() <= 1e-6
+    # grouping: every route has its own slot, in a tile of its expert, routes of an expert in route order
+    tiles = int(b["tile_total"].download(np.uint32)[0])
+    tile_expert = b["tile_expert"].download(np.uint32)[:tiles]
+    tile_rows = b["tile_rows"].download(np.uint32)[:tiles]
+    slot = b["route_slot"].download(np.uint32)[:rows * top_k]
+    slot_row = b["slot_row"].download(np.uint32)
+    assert len(set(slot.tolist())) == rows * top_k
+    flat = selected.ravel()
+    assert np.array_equal(tile_expert[slot // 16], flat)
+    assert np.array_equal(slot_row[slot], np.arange(rows * top_k) // top_k)
+    assert int(tile_rows.sum()) == rows * top_k and np.all(np.diff(tile_expert.astype(np.int64)) >= 0)
+    assert tiles == sum((np.count_nonzero(flat == e) + 15) // 16 for e in range(experts))
+    for e in np.unique(flat):
+        assert np.all(np.diff(slot[flat == e].astype(np.int64)) > 0)
+    # expert outputs of the routes, then the combined rows: exp2 and the SwiGLU's exp2 differ in their
+    # last bits between host and GPU, which moves a few values by one bf16 step
+    # (a step of an intermediate value moves a down-projection sum by its weight, however small the sum: the
+    # error is bounded against the row's size, not the element's)
+    def close(got_bits, want_bits):
+        g, w = orc.bf16_to_f32(got_bits).astype(np.float64), orc.bf16_to_f32(want_bits).astype(np.float64)
+        scale = np.abs(w).max(axis=-1, keepdims=True)
+        assert np.all(np.abs(g - w) <= 2.0 ** -7 * np.abs(w) + 2.0 ** -8 * scale), np.abs(g - w).max()
+        assert (got_bits != want_bits).mean() < 0.03
+    got_y = b["expert_output"].download(np.uint16).reshape(-1, y.shape[2])[slot].reshape(y.shape)
+    close(got_y, y)
+    close(got, out)
+
+
+@pytest.mark.parametrize("config", [(512, 256, 8, 2, 20), (256, 256, 5, 5, 3), (1024, 512, 64, 4, 48)])
+def test_moe_layer_matches_the_oracle(backend, config):
+    print(f"case moe {config}", flush=True)
+    hidden, ffn, experts, top_k, rows = config
+    rng = np.random.default_rng(experts)
+    moe, got, want = run_layer(backend, rng, hidden, ffn, experts, top_k, rows)
+    check_layer(moe, got, want, rows, experts, top_k)
+
+
+def test_moe_layer_at_the_35b_shape(backend):
+    """Hidden 2048, 128 experts of FFN 768, top-8, eight lanes of sixteen rows (BASELINE config 5's MoE layer)."""
+    print("case moe 35B shape", flush=True)
+    rng = np.random.default_rng(9)
+    moe, got, want = run_layer(backend, rng, 2048, 768, 128, 8, 128)
+    check_layer(moe, got, want, 128, 128, 8)
+
+
+def test_moe_rejects_bad_arguments(backend):
+    with pytest.raises(ValueError):
+        ops.MoE(backend, 2048, 768, 128, 8, 300)
+    with pytest.raises(ValueError):
+        ops.MoE(backend, 2048, 700, 128, 8, 16)
+    moe = ops.MoE(backend, 512, 256, 8, 2, 4)
+    graph = splash_amd.CommandGraph()
+    with pytest.raises(ValueError):
+        moe.add_routing(graph, backend.allocate_buffer(16))
+    assert len(graph) == 0
