@@ -4,8 +4,8 @@
 // (runtime/metal/kernels/decode/gdn.metal:139-526, common/gdn_primitives.h:20-99) in its order of
 // operations: short convolution + SiLU, q/k RMS norms, gates, the fold of the pending (previously
 // accepted) rows into the state, the block rows' outputs, the gated output norm, the step's tape.
-// Sums over a head's 128 channels or a state row's 128 columns are four (resp. one) butterfly
-// sums over 32 lanes, as the kernels compute them.
+// Sums over a head's 128 channels or a state row's 128 columns are four (resp. one) tree sums
+// over 32 lanes (neighbouring pairs first), as the kernels compute them.
 #include "oracle.h"
 #include "common.hpp"
 
@@ -19,9 +19,10 @@ namespace {
 constexpr uint32_t kTaps = 4, kDim = 128, kRowsMax = 16;
 constexpr float kEps = 1e-6f;
 
+// a binary tree over neighbours: pairs, quads, eights, sixteens, then the two sixteens
 float butterfly32(float *lane) {
-  for (int step = 16; step; step >>= 1)
-    for (int l = 0; l < step; ++l) lane[l] += lane[l + step];
+  for (int step = 1; step < 32; step <<= 1)
+    for (int l = 0; l < 32; l += 2 * step) lane[l] += lane[l + step];
   return lane[0];
 }
 // sum of 128 squares: four 32-channel groups, added in channel order

@@ -68,7 +68,7 @@ struct GdnLane {
   uint64_t next_cell;     // and the one it writes: the state before this step's rows
 };
 
-// gdn_decode: grid (value_heads, lanes), 256 threads.
+// gdn_decode: grid (value_heads, lanes), 1024 threads.
 struct GdnDecodeParams {
   struct GdnShapeParams shape;
   uint32_t flags;
@@ -81,7 +81,7 @@ struct GdnDecodeParams {
   struct GdnLane lane[GDN_MAXIMUM_LANES];
 };
 
-// gdn_fold: grid (value_heads, layers), 256 threads: folds the first `rows` rows of the path a lane
+// gdn_fold: grid (value_heads, layers), 1024 threads: folds the first `rows` rows of the path a lane
 // retained of a step (retained[0], the mask its acceptance wrote) into the state before them, every
 // layer's tape tape_layer_bytes after `step_tape`, and writes the cell a next step would hold to
 // `fold_cell` (the reference's GDNFoldParams with exact cached states). Nothing when the path

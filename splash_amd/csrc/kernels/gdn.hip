@@ -4,11 +4,11 @@
 // into the head's 128 x 128 fp32 state, writes THAT state (the one before the block's rows, so a
 // rejected row never has to be undone), runs the block's rows for their outputs and gates them.
 //
-// Four waves. In the prologue and the gate a wave takes a row: lane l holds channels l and 64 + l,
-// and a sum over the head's 128 channels is four butterfly sums over 32 lanes added in channel
+// Sixteen waves. In the prologue and the gate a wave takes a row: lane l holds channels l and 64 + l,
+// and a sum over the head's 128 channels is four tree sums over 32 lanes added in channel
 // order, the reference's simdgroup sums (gdn.metal:215-222). In the recurrence a wave advances
 // two state rows at once, one per half-wave, lane j of a half holding key columns 4 j .. 4 j + 3;
-// the row's products with k and q are butterfly sums over the half's 32 lanes, and each token keeps
+// the row's products with k and q are tree sums over the half's 32 lanes, and each token keeps
 // the decay, memory, delta, update, output order of gdn.metal:270-298.
 #include "abi/Gdn.h"
 #include "abi/PagedAttention.h"  // AttentionTreeRow
@@ -22,10 +22,18 @@ namespace {
 constexpr uint32_t kDim = GDN_HEAD_DIMENSION, kTaps = GDN_CONVOLUTION_TAPS, kRows = GDN_MAXIMUM_ROWS;
 constexpr float kLog2e = 1.44269504089f;
 
-// The sum over each half-wave's 32 lanes (lanes 0..31 and 32..63 apart), in every lane of the half.
+// The sum over each half-wave's 32 lanes (lanes 0..31 and 32..63 apart), in every lane of the half: a
+// binary tree over neighbours (pairs, quads, eights, sixteens, the two rows of sixteen), four of its
+// levels as row-local DPP operands of the add itself.
+template <int Control> __device__ __forceinline__ float dpp_of(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), Control, 0xF, 0xF, false));
+}
 __device__ __forceinline__ float half_sum(float v) {
-#pragma unroll
-  for (int o = 16; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  v += dpp_of<0xB1>(v);   // quad_perm [1, 0, 3, 2]
+  v += dpp_of<0x4E>(v);   // quad_perm [2, 3, 0, 1]
+  v += dpp_of<0x141>(v);  // row_half_mirror: the other quad of the eight
+  v += dpp_of<0x140>(v);  // row_mirror: the other eight of the row
+  v += __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x401F));  // lane ^ 16
   return v;
 }
 // The sum of a head's 128 values, lane l holding a = value[l] and b = value[64 + l]: the four
@@ -138,13 +146,14 @@ __device__ __forceinline__ void advance(float (&state)[R][4], const uint16_t *ke
   }
 }
 
-constexpr int kInFlight = 2;  // row pairs a wave advances together, to overlap their reductions
+constexpr int kInFlight = 4;  // row pairs a wave advances together, to overlap their reductions
+constexpr uint32_t kWaves = 16;  // of a workgroup: with four pairs each they hold the head's 128 state rows at once
 
 } // namespace
 
-// gdn_decode: grid (value_heads, lanes), 256 threads. Chains only: a block whose rows are not a
+// gdn_decode: grid (value_heads, lanes), 1024 threads. Chains only: a block whose rows are not a
 // chain is rejected by the host operator.
-__global__ __launch_bounds__(256) void gdn_decode(const uint16_t *__restrict__ packed, const uint16_t *__restrict__ conv_weights,
+__global__ __launch_bounds__(64 * kWaves) void gdn_decode(const uint16_t *__restrict__ packed, const uint16_t *__restrict__ conv_weights,
                                                   uint8_t *__restrict__ states, uint8_t *__restrict__ tape,
                                                   const float *__restrict__ a_scale, const uint16_t *__restrict__ dt_bias,
                                                   const void *__restrict__ norm_weight, uint16_t *__restrict__ hidden,
@@ -189,9 +198,9 @@ __global__ __launch_bounds__(256) void gdn_decode(const uint16_t *__restrict__ p
       }
     }
   }
-  for (uint32_t token = wave; token < pendingRows; token += 4u)
+  for (uint32_t token = wave; token < pendingRows; token += kWaves)
     load_pending(pendingTape, pending, token, path_row(L.pending_path, token), head, s, lane);
-  for (uint32_t token = wave; token < rows; token += 4u) {
+  for (uint32_t token = wave; token < rows; token += kWaves) {
     const uint16_t *taps[kTaps];
 #pragma unroll
     for (uint32_t tap = 0; tap < kTaps; ++tap) {
@@ -262,12 +271,12 @@ __global__ __launch_bounds__(256) void gdn_decode(const uint16_t *__restrict__ p
   // ---- recurrence ----
   {
     const uint32_t half = lane >> 5, column = 4u * (lane & 31u);
-    for (uint32_t batch = 0; batch < kDim / 8u; batch += kInFlight) {
+    for (uint32_t batch = 0; batch < kDim / (2u * kWaves); batch += kInFlight) {
       uint32_t valueDim[kInFlight];
       float state[kInFlight][4], result[kInFlight];
 #pragma unroll
       for (int r = 0; r < kInFlight; ++r) {
-        valueDim[r] = (batch + r) * 8u + wave * 2u + half;
+        valueDim[r] = (batch + r) * 2u * kWaves + wave * 2u + half;
         const float4 loaded = *reinterpret_cast<const float4 *>(stateIn + (size_t(head) * kDim + valueDim[r]) * kDim + column);
         state[r][0] = loaded.x;
         state[r][1] = loaded.y;
@@ -295,7 +304,7 @@ __global__ __launch_bounds__(256) void gdn_decode(const uint16_t *__restrict__ p
 
   // ---- gated output norm (gdn.metal:489-526) ----
   const uint32_t outHead = (p.flags & GDN_TILED_HEADS) ? (head % perKey) * s.key_heads + head / perKey : head;
-  for (uint32_t token = wave; token < rows; token += 4u) {
+  for (uint32_t token = wave; token < rows; token += kWaves) {
     float value[2];
 #pragma unroll
     for (uint32_t part = 0; part < 2; ++part) value[part] = bf16_bits_to_float(outputs[token][lane + 64u * part]);
@@ -314,8 +323,8 @@ __global__ __launch_bounds__(256) void gdn_decode(const uint16_t *__restrict__ p
 }
 SP_REGISTER_KERNEL("gdn_decode", &gdn_decode);
 
-// gdn_fold: grid (value_heads, layers), 256 threads (gdn.metal:630-698, exact cells).
-__global__ __launch_bounds__(256) void gdn_fold(uint8_t *__restrict__ states, uint8_t *__restrict__ tape,
+// gdn_fold: grid (value_heads, layers), 1024 threads (gdn.metal:630-698, exact cells).
+__global__ __launch_bounds__(64 * kWaves) void gdn_fold(uint8_t *__restrict__ states, uint8_t *__restrict__ tape,
                                                 const uint32_t *__restrict__ retained, GdnFoldParams p) {
   __shared__ __align__(16) Pending pending;
   const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, head = blockIdx.x, layer = blockIdx.y;
@@ -326,7 +335,7 @@ __global__ __launch_bounds__(256) void gdn_fold(uint8_t *__restrict__ states, ui
   const Tape step = tape_at(tape, p.step_tape + uint64_t(layer) * p.tape_layer_bytes, s);
   const uint8_t *cell = states + p.state_cell;
   uint8_t *fold = states + p.fold_cell;
-  for (uint32_t token = wave; token < rows; token += 4u) load_pending(step, pending, token, path_row(path, token), head, s, lane);
+  for (uint32_t token = wave; token < rows; token += kWaves) load_pending(step, pending, token, path_row(path, token), head, s, lane);
   if (wave < kTaps - 1) {
     const History history = history_of(reinterpret_cast<const uint16_t *>(cell + uint64_t(layer) * p.conv_layer_bytes), step.inputs, C, rows, path);
     uint16_t *carried = reinterpret_cast<uint16_t *>(fold + uint64_t(layer) * p.conv_layer_bytes) + size_t(wave) * C;
@@ -345,12 +354,12 @@ __global__ __launch_bounds__(256) void gdn_fold(uint8_t *__restrict__ states, ui
   const float *stateIn = reinterpret_cast<const float *>(cell + p.convolution_state_bytes + uint64_t(layer) * p.recurrent_layer_bytes);
   float *stateOut = reinterpret_cast<float *>(fold + p.convolution_state_bytes + uint64_t(layer) * p.recurrent_layer_bytes);
   const uint32_t half = lane >> 5, column = 4u * (lane & 31u);
-  for (uint32_t batch = 0; batch < kDim / 8u; batch += kInFlight) {
+  for (uint32_t batch = 0; batch < kDim / (2u * kWaves); batch += kInFlight) {
     uint32_t valueDim[kInFlight];
     float state[kInFlight][4], result[kInFlight];
 #pragma unroll
     for (int r = 0; r < kInFlight; ++r) {
-      valueDim[r] = (batch + r) * 8u + wave * 2u + half;
+      valueDim[r] = (batch + r) * 2u * kWaves + wave * 2u + half;
       const float4 loaded = *reinterpret_cast<const float4 *>(stateIn + (size_t(head) * kDim + valueDim[r]) * kDim + column);
       state[r][0] = loaded.x;
       state[r][1] = loaded.y;

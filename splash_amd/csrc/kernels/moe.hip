@@ -59,12 +59,29 @@ __global__ __launch_bounds__(256) void moe_group_routes(const uint32_t *__restri
                                                         uint32_t *__restrict__ slot_row, uint32_t *__restrict__ tile_expert,
                                                         uint32_t *__restrict__ tile_rows, uint32_t *__restrict__ tile_total,
                                                         MoeGroupParams p) {
+  constexpr uint32_t kStaged = 256u * MOE_MAXIMUM_TOP;  // routes of a step: 256 rows of up to 16
   __shared__ uint32_t counts[MOE_MAXIMUM_EXPERTS], firstTile[MOE_MAXIMUM_EXPERTS];
+  __shared__ __align__(16) uint8_t staged[kStaged];  // expert ids fit a byte
   const uint32_t e = threadIdx.x;
   for (uint32_t slot = e; slot < p.maximum_tiles * MOE_TILE_ROWS; slot += 256u) slot_row[slot] = MOE_NO_ROW;
+  for (uint32_t route = e; route < p.routes; route += 256u) staged[route] = uint8_t(selected[route]);
+  __syncthreads();
+  // Sixteen routes per LDS read (a broadcast: every thread reads the same address).
+  const uint32_t vectors = (p.routes + 15u) / 16u;
+  auto matches = [&](uint32_t vector) -> uint32_t {  // bit i: route 16 vector + i is expert e's
+    const uint4 ids = reinterpret_cast<const uint4 *>(staged)[vector];
+    const uint32_t words[4] = {ids.x, ids.y, ids.z, ids.w};
+    uint32_t mask = 0;
+#pragma unroll
+    for (uint32_t i = 0; i < 16; ++i) mask |= (((words[i >> 2] >> (8u * (i & 3u))) & 0xFFu) == e ? 1u : 0u) << i;
+    const uint32_t live = p.routes - 16u * vector;
+    return live >= 16u ? mask : mask & ((1u << live) - 1u);
+  };
   uint32_t count = 0;
-  if (e < p.experts)
-    for (uint32_t route = 0; route < p.routes; ++route) count += selected[route] == e ? 1u : 0u;
+  if (e < p.experts) {
+#pragma unroll 4
+    for (uint32_t vector = 0; vector < vectors; ++vector) count += uint32_t(__builtin_popcount(matches(vector)));
+  }
   counts[e] = e < p.experts ? count : 0u;
   __syncthreads();
   if (e == 0) {
@@ -83,13 +100,18 @@ __global__ __launch_bounds__(256) void moe_group_routes(const uint32_t *__restri
     tile_rows[first + t] = min(MOE_TILE_ROWS, count - t * MOE_TILE_ROWS);
   }
   uint32_t placed = 0;
-  for (uint32_t route = 0; route < p.routes; ++route)
-    if (selected[route] == e) {
+#pragma unroll 4
+  for (uint32_t vector = 0; vector < vectors; ++vector) {
+    uint32_t mask = matches(vector);
+    while (mask) {
+      const uint32_t route = 16u * vector + uint32_t(__builtin_ctz(mask));
+      mask &= mask - 1u;
       const uint32_t slot = (first + placed / MOE_TILE_ROWS) * MOE_TILE_ROWS + placed % MOE_TILE_ROWS;
       route_slot[route] = slot;
       slot_row[slot] = route / p.top_k;
       ++placed;
     }
+  }
 }
 SP_REGISTER_KERNEL("moe_group_routes", &moe_group_routes);
 

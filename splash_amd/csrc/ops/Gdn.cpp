@@ -62,7 +62,7 @@ void GDN::addDecode(hip::CommandGraph &graph, const GdnDecodeBuffers &b, const G
   requireBytes(b.mixerNorm, uint64_t{GDN_HEAD_DIMENSION} * (b.floatNorm ? 4 : 2), "GDN output norm");
   requireBytes(b.hidden, uint64_t{rows} * shape.valueHeads * GDN_HEAD_DIMENSION * 2, "GDN hidden rows");
   graph.add("gdn_decode", {b.packed, b.convolutionWeights, b.states, b.tape, b.decayWeights, b.timeBias, b.mixerNorm, b.hidden}, params,
-            {shape.valueHeads, uint32_t(lanes.size()), 1}, {256, 1, 1});
+            {shape.valueHeads, uint32_t(lanes.size()), 1}, {1024, 1, 1});
 }
 
 void GDN::addFold(hip::CommandGraph &graph, const GdnFoldBuffers &b, const GdnShape &shape, uint32_t layers, uint32_t rows,
@@ -86,7 +86,7 @@ void GDN::addFold(hip::CommandGraph &graph, const GdnFoldBuffers &b, const GdnSh
   params.tape_layer_bytes = tapeBytes;
   params.state_cell = b.stateCell;
   params.fold_cell = b.foldCell;
-  graph.add("gdn_fold", {b.states, b.tape, b.retainedRows}, params, {shape.valueHeads, layers, 1}, {256, 1, 1});
+  graph.add("gdn_fold", {b.states, b.tape, b.retainedRows}, params, {shape.valueHeads, layers, 1}, {1024, 1, 1});
 }
 
 } // namespace splash::ops
