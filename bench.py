@@ -21,6 +21,10 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0   # MI355X published HBM3E bandwidth
+# HBM bytes per launch of the one-pass gate/up projection, by (hidden, ffn, rows): FETCH_SIZE + WRITE_SIZE of
+# rocprofv3 --pmc runs of this file, each scaled by what the counter reads for the copy kernel's known bytes
+# (profiles/verify_step_c4_hbm_traffic.md). Counters cannot be read from inside the run.
+GATE_UP_TRAFFIC_BYTES = {(5120, 25600, 16): 124.1e6}
 
 WORKLOADS = {
     # hidden, q heads, kv heads, head dim, ffn, vocabulary, layers, context, rows
@@ -141,6 +145,63 @@ def cpu_baseline(w):
                       f"({gemm_seconds + attention_seconds:.1f}s of CPU work on {cores} threads)"}
 
 
+def time_c5_ops(backend):
+    """Per-dispatch GPU time (HIP events around each dispatch) of the Gated DeltaNet step and the MoE layer at the
+    35B-A3B shape of BASELINE config 5, batch 8 of 16-row blocks; weights and states in rings past the caches.
+    Prints one JSON line; not the headline metric (that is the dense step)."""
+    import splash_amd
+    from splash_amd import ops
+    rng = np.random.default_rng(0)
+    bf = lambda a: (np.ascontiguousarray(a, np.float32).view(np.uint32) >> 16).astype(np.uint16)
+    KH, VH, lanes, rows, copies = 16, 32, 8, 16, 6
+    gdn = ops.GDN(KH, VH, layers=copies)
+    shape = gdn.shape
+    bufs = dict(packed=backend.from_array(bf(rng.standard_normal((lanes * rows, shape.packed_width)))),
+                convolution_weights=backend.from_array(bf(rng.standard_normal((shape.convolution_dimension, 4)) * 0.4)),
+                states=backend.allocate_buffer(gdn.cell_bytes * 2 * lanes), tape=backend.allocate_buffer(gdn.tape_layer_bytes * copies * 2 * lanes),
+                decay_weights=backend.from_array(-np.ones(VH, np.float32)), time_bias=backend.from_array(bf(np.zeros(VH))),
+                mixer_norm=backend.from_array(bf(np.ones(128))), hidden=backend.allocate_buffer(lanes * rows * VH * 128 * 2))
+
+    def lane_list(layer, parity, path):
+        return [dict(first_row=l * rows, rows=rows, pending_path=path,
+                     pending_tape=((l * 2 + (parity ^ 1)) * copies + layer) * gdn.tape_layer_bytes,
+                     step_tape=((l * 2 + parity) * copies + layer) * gdn.tape_layer_bytes,
+                     current_cell=(l * 2 + parity) * gdn.cell_bytes, next_cell=(l * 2 + (parity ^ 1)) * gdn.cell_bytes) for l in range(lanes)]
+    graph = splash_amd.CommandGraph()
+    for layer in range(copies):
+        gdn.add_decode(graph, bufs, layer, lane_list(layer, 0, 0))
+    for _ in range(3):
+        for layer in range(copies):
+            gdn.add_decode(graph, bufs, layer, lane_list(layer, 1, 0xFFFF))   # folds 16 pending rows, runs 16
+    backend.set_dispatch_profiling(True)
+    _, _, per = backend.run(graph, profiled=True)
+    gdn_us = float(np.median(np.array(per[copies:]) * 1e6))
+    state_bytes = lanes * VH * 128 * 128 * 4 * 2
+    H, F, E, K, R = 2048, 768, 128, 8, 128
+    image = lambda n, k: backend.from_array(rng.integers(0, 256, ops.gguf_image_bytes(ops.FMT_Q4K, n, k) * E, dtype=np.uint8))
+    sets = [(image(F, H), image(F, H), image(H, F)) for _ in range(3)]
+    moe = ops.MoE(backend, H, F, E, K, R)
+    x, res = backend.from_array(bf(rng.standard_normal((R, H)))), backend.from_array(bf(rng.standard_normal((R, H))))
+    scores, out = backend.from_array(rng.standard_normal((R, E)).astype(np.float32)), backend.allocate_buffer(R * H * 2)
+    graph = splash_amd.CommandGraph()
+    for _ in range(4):
+        for s in sets:
+            moe.add_routing(graph, scores)
+            moe.add_routed(graph, x, res, out, *s)
+    _, _, per = backend.run(graph, profiled=True)
+    backend.set_dispatch_profiling(False)
+    med = np.median(np.array(per).reshape(-1, 6)[3:] * 1e6, axis=0)
+    names = ["moe_route_select", "moe_group_routes", "moe_gather_table", "gguf_moe_decode_q4k_gt", "gguf_moe_decode_q4k_a", "moe_combine"]
+    weights = E * 3 * F * H * 0.5625
+    print(json.dumps({
+        "ops": "c5", "n_gpus": 1, "data": "synthetic",
+        "gdn_decode": {"workload": "32 value heads x 8 lanes, 16 pending + 16 rows", "us": round(gdn_us, 1),
+                       "state_bytes": state_bytes, "achieved_gbs": round(state_bytes / gdn_us / 1e3, 1)},
+        "moe_layer": {"workload": "hidden 2048, 128 experts top-8, FFN 768, 128 rows", "us": {n: round(float(m), 1) for n, m in zip(names, med)},
+                      "total_us": round(float(med.sum()), 1), "expert_weight_bytes": int(weights),
+                      "expert_gbs": round(weights / float(med[3] + med[4]) / 1e3, 1)}}), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -149,6 +210,7 @@ def main():
     ap.add_argument("--workload", default="c4", choices=sorted(WORKLOADS))
     ap.add_argument("--lanes", type=int, default=1)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--ops", choices=["c5"], help="time the GDN step and the MoE layer of config 5 instead of the dense step")
     args = ap.parse_args()
     if args.gpus != 1:
         log("bench.py measures one GPU: this build runs the verify step on a single MI355X (no collectives); use --gpus 1")
@@ -157,6 +219,9 @@ def main():
     from splash_amd import ops, verify
     w = WORKLOADS[args.workload]
     backend = splash_amd.Backend(0)
+    if args.ops == "c5":
+        time_c5_ops(backend)
+        return
     info = backend.device_info()
     log(f"device {info.name.decode()} {info.arch.decode()} CUs {info.compute_units}")
     t0 = time.time()
@@ -213,7 +278,7 @@ def main():
         "step_hbm": {"algorithmic_gb": round(step_bytes / 1e9, 3), "achieved_gbs": round(step_bytes / (ms * 1e-3) / 1e9, 1),
                      "frac_of_peak": round(step_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "wall_ms_per_step": round(wall_ms, 4)},
         "roofline": {"bound": "hbm", "kernel": gate_up, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None, "launches": len(by_kernel[gate_up]),
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": GATE_UP_TRAFFIC_BYTES.get((w["hidden"], w["ffn"], rows)), "launches": len(by_kernel[gate_up]),
                      "avg_us": round(avg * 1e6, 2), "algorithmic_bytes": int(gate_up_bytes), "largest_total": dominant},
     }
     if not args.no_cpu_baseline:
