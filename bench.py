@@ -160,7 +160,10 @@ def time_c5_ops(backend):
                 convolution_weights=backend.from_array(bf(rng.standard_normal((shape.convolution_dimension, 4)) * 0.4)),
                 states=backend.allocate_buffer(gdn.cell_bytes * 2 * lanes), tape=backend.allocate_buffer(gdn.tape_layer_bytes * copies * 2 * lanes),
                 decay_weights=backend.from_array(-np.ones(VH, np.float32)), time_bias=backend.from_array(bf(np.zeros(VH))),
-                mixer_norm=backend.from_array(bf(np.ones(128))), hidden=backend.allocate_buffer(lanes * rows * VH * 128 * 2))
+                mixer_norm=backend.from_array(bf(np.ones(128))), hidden=backend.allocate_buffer(lanes * rows * VH * 128 * 2),
+                # chain blocks: row r of a block follows row r - 1 (ancestors (2 << r) - 1, parent r - 1, depth r)
+                tree_rows=backend.from_array(np.array([[(2 << r) - 1, ((r - 1) & 0xFFFF) | (r << 16)] for _ in range(lanes)
+                                                       for r in range(rows)], np.uint32)))
 
     def lane_list(layer, parity, path):
         return [dict(first_row=l * rows, rows=rows, pending_path=path,

@@ -6,6 +6,10 @@
 // accepted) rows into the state, the block rows' outputs, the gated output norm, the step's tape.
 // Sums over a head's 128 channels or a state row's 128 columns are four (resp. one) tree sums
 // over 32 lanes (neighbouring pairs first), as the kernels compute them.
+//
+// A block that is not a chain (gdn.metal:417-478): every row's convolution taps follow its path,
+// and its output comes from the committed state through its transformed query and its path's
+// coefficients, S_-1 z_-1 + sum_j c_j v_j.
 #include "oracle.h"
 #include "common.hpp"
 
@@ -121,11 +125,18 @@ void orc_gdn_step(float *S, uint32_t D, const float *k, const float *v, float de
   }
 }
 
-int orc_gdn_decode(const OrcGdnShape *s, const uint16_t *packed, uint32_t rows, const uint16_t *conv_weights, const float *a_scale,
-                   const uint16_t *dt_bias, const void *norm_weight, const uint16_t *conv_in, const float *state_in,
+int orc_gdn_decode(const OrcGdnShape *s, const uint16_t *packed, uint32_t rows, const uint32_t *ancestors, const uint16_t *conv_weights,
+                   const float *a_scale, const uint16_t *dt_bias, const void *norm_weight, const uint16_t *conv_in, const float *state_in,
                    uint8_t *pending_tape, uint32_t pending_path, uint16_t *conv_out, float *state_out, uint8_t *step_tape,
                    uint16_t *hidden) {
   if (!rows || rows > kRowsMax || s->conv_dim != (2 * s->key_heads + s->value_heads) * kDim) return -1;
+  // each row's path within the block, itself the last; without tree rows, a chain
+  uint32_t paths[kRowsMax];
+  bool chain = true;
+  for (uint32_t t = 0; t < rows; ++t) {
+    paths[t] = ancestors ? (ancestors[t] & ((1u << t) - 1u)) | (1u << t) : (2u << t) - 1u;
+    chain = chain && paths[t] == (2u << t) - 1u;
+  }
   const uint32_t KH = s->key_heads, VH = s->value_heads, C = s->conv_dim, P = s->packed_width, perKey = VH / KH;
   const uint32_t keyWidth = KH * kDim, kvWidth = keyWidth + VH * kDim;
   const uint32_t zOffset = C, bOffset = C + VH * kDim, aOffset = bOffset + VH;
@@ -138,19 +149,24 @@ int orc_gdn_decode(const OrcGdnShape *s, const uint16_t *packed, uint32_t rows, 
   std::vector<uint16_t> carry(3 * size_t(C));
   for (uint32_t r = 0; r < 3; ++r) std::copy(hist[r], hist[r] + C, carry.begin() + size_t(r) * C);
 
-  // conv + SiLU of every conv channel of every row (a chain: row t's taps are rows t-3..t)
+  // conv + SiLU of every conv channel of every row: the taps are the last four tokens of the
+  // row's path, those before the block from the history (gdn_primitives.h:37-50, gdn.metal:198-206)
   std::vector<uint16_t> conv(size_t(rows) * C);
-  for (uint32_t t = 0; t < rows; ++t)
+  for (uint32_t t = 0; t < rows; ++t) {
+    const uint32_t depth = uint32_t(__builtin_popcount(paths[t])) - 1;
+    const uint16_t *taps[kTaps];
+    for (uint32_t tap = kTaps, up = paths[t]; tap-- > 0;) {
+      const uint32_t row = up ? 31u - uint32_t(__builtin_clz(up)) : 0u;
+      up &= ~(1u << row);
+      taps[tap] = depth + tap < 3 ? carry.data() + size_t(depth + tap) * C : packed + size_t(row) * P;
+    }
     for (uint32_t c = 0; c < C; ++c) {
       float value = 0.f;
-      for (uint32_t tap = 0; tap < kTaps; ++tap) {
-        const int position = int(t) + int(tap) - 3;  // block row, or history row position + 3
-        const uint16_t *row = position < 0 ? carry.data() + size_t(position + 3) * C : packed + size_t(position) * P;
-        value += bf2f(row[c]) * bf2f(conv_weights[size_t(c) * kTaps + tap]);
-      }
+      for (uint32_t tap = 0; tap < kTaps; ++tap) value += bf2f(taps[tap][c]) * bf2f(conv_weights[size_t(c) * kTaps + tap]);
       value = bf2f(f2bf(value));
       conv[size_t(t) * C + c] = f2bf(silu(value));
     }
+  }
   // per key head: normalized q and k rows; per value head: gates
   std::vector<uint16_t> queries(size_t(KH) * rows * kDim), keys(size_t(KH) * rows * kDim);
   for (uint32_t kh = 0; kh < KH; ++kh)
@@ -202,13 +218,47 @@ int orc_gdn_decode(const OrcGdnShape *s, const uint16_t *packed, uint32_t rows, 
       bd[t] = step.decay[t * VH + h];
       bb[t] = step.beta[t * VH + h];
     }
+    // tree rows: the transformed query z_-1 and the path's coefficients (gdn.metal:435-478)
+    float transformed[kRowsMax][kDim], coefficient[kRowsMax][kRowsMax] = {};
+    if (!chain)
+      for (uint32_t t = 0; t < rows; ++t) {
+        float *z = transformed[t];
+        for (uint32_t d = 0; d < kDim; ++d) z[d] = bf2f(queries[(size_t(kh) * rows + t) * kDim + d]);
+        for (uint32_t up = paths[t]; up;) {
+          const uint32_t row = 31u - uint32_t(__builtin_clz(up));
+          up &= ~(1u << row);
+          const uint16_t *key = keys.data() + (size_t(kh) * rows + row) * kDim;
+          float lane[32];
+          for (int l = 0; l < 32; ++l) {
+            float product = 0.f;
+            for (int i = 0; i < 4; ++i) product += bf2f(key[4 * l + i]) * z[4 * l + i];
+            lane[l] = product;
+          }
+          const float c = bf2f(bb[row]) * butterfly32(lane), d = bd[row];
+          for (uint32_t i = 0; i < kDim; ++i) z[i] = d * (z[i] - c * bf2f(key[i]));
+          coefficient[t][row] = c;
+        }
+      }
     for (uint32_t r = 0; r < kDim; ++r) {
       float state[kDim];
       const size_t base = (size_t(h) * kDim + r) * kDim;
       std::copy(state_in + base, state_in + base + kDim, state);
       foldRow(state, r, pending, pk, pv, pd, pb, nullptr, nullptr);
       std::copy(state, state + kDim, state_out + base);
-      foldRow(state, r, rows, keys.data() + size_t(kh) * rows * kDim, bv, bd, bb, queries.data() + size_t(kh) * rows * kDim, out);
+      if (chain) {
+        foldRow(state, r, rows, keys.data() + size_t(kh) * rows * kDim, bv, bd, bb, queries.data() + size_t(kh) * rows * kDim, out);
+        continue;
+      }
+      // a lane per block row carries the path's term beside its four columns' products (gdn.metal:363-377)
+      for (uint32_t t = 0; t < rows; ++t) {
+        float lane[32];
+        for (uint32_t l = 0; l < 32; ++l) {
+          float result = l < kRowsMax && ((paths[t] >> l) & 1u) ? coefficient[t][l] * bf2f(bv[l * kDim + r]) : 0.0f;
+          for (int i = 0; i < 4; ++i) result += state[4 * l + i] * transformed[t][4 * l + i];
+          lane[l] = result;
+        }
+        out[t * kDim + r] = f2bf(butterfly32(lane));
+      }
     }
     // gated output norm (gdn.metal:489-526)
     const uint32_t outHead = (s->flags & 1u) ? (h % perKey) * KH + h / perKey : h;

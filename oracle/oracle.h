@@ -145,15 +145,19 @@ uint64_t orc_gdn_tape_bytes(const struct OrcGdnShape *s);
 // S += delta k^T; o (optional) = S q after the update.
 void orc_gdn_step(float *S, uint32_t D, const float *k, const float *v, float decay, float beta, const float *q,
                   float *o);
-// One decode step of one lane and one layer over a chain of `rows` rows (gdn.metal:139-526): folds
+// One decode step of one lane and one layer over a block of `rows` rows (gdn.metal:139-526): folds
 // the pending path of the previous step's tape into the state and writes THAT as state_out (the
 // state before this step's rows) with the convolution carry it leaves; writes this step's tape;
 // hidden bf16 [rows][vh * 128] are the gated, normed outputs of the block rows.
 // conv_in/out bf16 [3][conv_dim]; state fp32 [vh][128][128]; pending_tape may be NULL when the path is 0.
-int orc_gdn_decode(const struct OrcGdnShape *s, const uint16_t *packed, uint32_t rows, const uint16_t *conv_weights,
-                   const float *a_scale, const uint16_t *dt_bias, const void *norm_weight, const uint16_t *conv_in,
-                   const float *state_in, uint8_t *pending_tape, uint32_t pending_path, uint16_t *conv_out,
-                   float *state_out, uint8_t *step_tape, uint16_t *hidden);
+// ancestors[r]: the block rows on row r's path (bit j: row j; NULL: a chain, (2 << r) - 1). A chain's
+// rows run the recurrence in order; any other tree's rows read the state before the block along
+// their paths (gdn.metal:417-478). Pinned by the fp64 check below on chains, and for trees by the
+// same check along each row's path (the tree form is algebraically the chain of the path).
+int orc_gdn_decode(const struct OrcGdnShape *s, const uint16_t *packed, uint32_t rows, const uint32_t *ancestors,
+                   const uint16_t *conv_weights, const float *a_scale, const uint16_t *dt_bias, const void *norm_weight,
+                   const uint16_t *conv_in, const float *state_in, uint8_t *pending_tape, uint32_t pending_path,
+                   uint16_t *conv_out, float *state_out, uint8_t *step_tape, uint16_t *hidden);
 // The state after the first `rows` rows of `path` of a step's tape, as the lane's next step would
 // hold it (gdn.metal:630-698, exact cells). Returns 1 and writes nothing when the path is shorter.
 int orc_gdn_fold(const struct OrcGdnShape *s, const uint16_t *conv_in, const float *state_in, uint8_t *step_tape,

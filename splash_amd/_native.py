@@ -106,7 +106,7 @@ class GdnLane(ctypes.Structure):
 
 class GdnDecodeBuffers(ctypes.Structure):
     _fields_ = [(n, c_p) for n in ("packed", "convolution_weights", "states", "tape", "decay_weights", "time_bias", "mixer_norm",
-                                   "hidden")] + [("float_norm", c_u32)]
+                                   "hidden")] + [("float_norm", c_u32), ("tree_rows", c_p)]
 
 
 class MoeShape(ctypes.Structure):
@@ -219,7 +219,7 @@ _sig("spo_norm_add_rms_table", c_int, c_p, c_p, c_p, c_p, c_p, c_u32, c_u32)
 _sig("spo_embedding_add", c_int, c_p, c_u32, c_p, c_u32, c_u32, c_p, c_p, c_u32)
 _sig("spo_rope_add_tree_tables", c_int, c_p, c_p, c_p, c_p, c_p, c_u32, P(RopeSequence), c_u32)
 _sig("spo_gdn_layout", c_int, P(GdnShape), c_u32, P(GdnStateStrides), P(c_u64), P(c_u64))
-_sig("spo_gdn_add_decode", c_int, c_p, P(GdnDecodeBuffers), P(GdnShape), c_u32, P(GdnStateStrides), c_u32, P(GdnLane), c_u32, c_int)
+_sig("spo_gdn_add_decode", c_int, c_p, P(GdnDecodeBuffers), P(GdnShape), c_u32, P(GdnStateStrides), c_u32, P(GdnLane), c_u32)
 _sig("spo_gdn_add_fold", c_int, c_p, c_p, c_p, c_p, c_u64, c_u64, c_u64, P(GdnShape), c_u32, c_u32, P(GdnStateStrides))
 _sig("spo_moe_workspace_sizes", c_int, P(MoeShape), c_u32, P(c_u64))
 _sig("spo_moe_add_routing", c_int, c_p, c_p, c_u32, P(MoeWorkspace), P(MoeShape), c_u32)

@@ -38,18 +38,17 @@ sp_status spo_gdn_layout(const spo_gdn_shape *shape, uint32_t layers, spo_gdn_st
 }
 
 sp_status spo_gdn_add_decode(spo_graph *graph, const spo_gdn_decode_buffers *b, const spo_gdn_shape *shape, uint32_t layer,
-                             const spo_gdn_state_strides *state, uint32_t tiled_heads, const spo_gdn_lane *lanes, uint32_t count,
-                             int chains) {
+                             const spo_gdn_state_strides *state, uint32_t tiled_heads, const spo_gdn_lane *lanes, uint32_t count) {
   return capi::guard([&] {
     capi::require(graph && b && shape && state && lanes, "graph, buffers, shape, strides or lanes");
     ops::GdnDecodeBuffers buffers{B(b->packed), B(b->convolution_weights), B(b->states), B(b->tape), B(b->decay_weights),
-                                  B(b->time_bias), B(b->mixer_norm), b->float_norm != 0, B(b->hidden)};
+                                  B(b->time_bias), B(b->mixer_norm), b->float_norm != 0, B(b->hidden), B(b->tree_rows)};
     std::vector<ops::GdnLaneStep> list;
     for (uint32_t i = 0; i < count; ++i)
       list.push_back({lanes[i].first_row, lanes[i].rows, lanes[i].pending_path, lanes[i].pending_tape, lanes[i].step_tape,
                       lanes[i].current_cell, lanes[i].next_cell});
     ops::GDN::addDecode(capi::graphOf(graph), buffers, shapeOf(*shape), layer, stridesOf(*state),
-                        tiled_heads ? ops::GdnHeadOrder::Tiled : ops::GdnHeadOrder::Grouped, list, chains != 0);
+                        tiled_heads ? ops::GdnHeadOrder::Tiled : ops::GdnHeadOrder::Grouped, list);
   });
 }
 

@@ -140,7 +140,9 @@ sp_status spo_linear_create_calibrated(uint32_t compute_units, uint32_t groups_p
   return capi::guard([&] {
     capi::require(out, "result");
     if (!compute_units || !groups_per_unit || !minimum_blocks_per_wave) throw std::invalid_argument("a calibration has no zero entry");
-    *out = new spo_linear{ops::Linear(ops::KernelCalibration{compute_units, groups_per_unit, minimum_blocks_per_wave})};
+    ops::KernelCalibration calibration{compute_units, groups_per_unit, minimum_blocks_per_wave};
+    calibration.groupsPerUnitQ6K = std::min(calibration.groupsPerUnitQ6K, groups_per_unit);
+    *out = new spo_linear{ops::Linear(calibration)};
   });
 }
 void spo_linear_destroy(spo_linear *linear) { delete linear; }

@@ -10,6 +10,12 @@
 // two state rows at once, one per half-wave, lane j of a half holding key columns 4 j .. 4 j + 3;
 // the row's products with k and q are tree sums over the half's 32 lanes, and each token keeps
 // the decay, memory, delta, update, output order of gdn.metal:270-298.
+//
+// A block whose rows are not a chain (some row's parent is not the row before it) takes its rows'
+// outputs from the committed state instead (gdn.metal:417-478): with S_j the state after the j-th
+// token of a row's path, S_j z = S_j-1 (d_j (z - c k_j)) + c v_j for c = beta_j (k_j . z), so the
+// row's output is S_-1 z_-1 + sum_j c_j v_j; a wave per row walks its path upward for z_-1 and the
+// coefficients, and the recurrence's waves add the path terms to the state's product with z_-1.
 #include "abi/Gdn.h"
 #include "abi/PagedAttention.h"  // AttentionTreeRow
 #include "backend/KernelRegistry.hpp"
@@ -151,16 +157,19 @@ constexpr uint32_t kWaves = 16;  // of a workgroup: with four pairs each they ho
 
 } // namespace
 
-// gdn_decode: grid (value_heads, lanes), 1024 threads. Chains only: a block whose rows are not a
-// chain is rejected by the host operator.
+// gdn_decode: grid (value_heads, lanes), 1024 threads. `tree` holds the step's rows' places in their
+// blocks (bit j of a row's ancestors: row j of its block is on its path, itself included).
 __global__ __launch_bounds__(64 * kWaves) void gdn_decode(const uint16_t *__restrict__ packed, const uint16_t *__restrict__ conv_weights,
                                                   uint8_t *__restrict__ states, uint8_t *__restrict__ tape,
                                                   const float *__restrict__ a_scale, const uint16_t *__restrict__ dt_bias,
                                                   const void *__restrict__ norm_weight, uint16_t *__restrict__ hidden,
-                                                  GdnDecodeParams p) {
+                                                  const AttentionTreeRow *__restrict__ tree, GdnDecodeParams p) {
   __shared__ __align__(16) uint16_t queries[kRows][kDim], keys[kRows][kDim], values[kRows][kDim], outputs[kRows][kDim];
+  __shared__ __align__(16) float transformed[kRows][kDim];
+  __shared__ float coefficients[kRows][kRows];
   __shared__ float decays[kRows];
   __shared__ uint16_t betas[kRows];
+  __shared__ uint32_t paths[kRows];
   __shared__ __align__(16) Pending pending;
 
   const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, head = blockIdx.x;
@@ -201,11 +210,19 @@ __global__ __launch_bounds__(64 * kWaves) void gdn_decode(const uint16_t *__rest
   for (uint32_t token = wave; token < pendingRows; token += kWaves)
     load_pending(pendingTape, pending, token, path_row(L.pending_path, token), head, s, lane);
   for (uint32_t token = wave; token < rows; token += kWaves) {
+    // The row's path within the block (its own row the last), its depth, and the block rows of its
+    // last four path tokens; taps before the block's first row read the history (gdn.metal:198-206).
+    const uint32_t path = (tree[L.first_row + token].ancestors & ((1u << token) - 1u)) | (1u << token);
+    const uint32_t depth = uint32_t(__builtin_popcount(path)) - 1u;
     const uint16_t *taps[kTaps];
+    {
+      uint32_t up = path;
 #pragma unroll
-    for (uint32_t tap = 0; tap < kTaps; ++tap) {
-      const int position = int(token) + int(tap) - int(kTaps - 1);
-      taps[tap] = position < 0 ? history.row[position + int(kTaps - 1)] : rowsIn + size_t(position) * P;
+      for (uint32_t tap = kTaps; tap-- > 0;) {
+        const uint32_t row = up ? 31u - uint32_t(__builtin_clz(up)) : 0u;
+        up &= ~(1u << row);
+        taps[tap] = depth + tap < kTaps - 1 ? history.row[depth + tap] : rowsIn + size_t(row) * P;
+      }
     }
     auto conv = [&](uint32_t channel) -> float {
       float value = 0.f;
@@ -253,6 +270,7 @@ __global__ __launch_bounds__(64 * kWaves) void gdn_decode(const uint16_t *__rest
       stepTape.decay[token * s.value_heads + head] = decay;
       betas[token] = uint16_t(beta);
       decays[token] = decay;
+      paths[token] = path;
     }
   }
   if (wave < kTaps - 1) {
@@ -267,6 +285,40 @@ __global__ __launch_bounds__(64 * kWaves) void gdn_decode(const uint16_t *__rest
     }
   }
   __syncthreads();
+
+  // Every thread reads the same paths, so the branch on them is uniform.
+  bool chain = true;
+  for (uint32_t token = 0; token < rows; ++token) chain = chain && paths[token] == (2u << token) - 1u;
+  if (!chain) {
+    // ---- tree rows: transformed queries and path coefficients, a wave per row ----
+    const uint32_t j = lane & 31u, column = 4u * j;
+    for (uint32_t token = wave; token < rows; token += kWaves) {
+      const uint2 qb = *reinterpret_cast<const uint2 *>(&queries[token][column]);
+      float z[4] = {bf16_bits_to_float(qb.x & 0xFFFFu), bf16_bits_to_float(qb.x >> 16), bf16_bits_to_float(qb.y & 0xFFFFu),
+                    bf16_bits_to_float(qb.y >> 16)};
+      float coefficient = 0.f;
+      for (uint32_t up = paths[token]; up;) {
+        const uint32_t row = 31u - uint32_t(__builtin_clz(up));
+        up &= ~(1u << row);
+        const uint2 kb = *reinterpret_cast<const uint2 *>(&keys[row][column]);
+        const float k[4] = {bf16_bits_to_float(kb.x & 0xFFFFu), bf16_bits_to_float(kb.x >> 16), bf16_bits_to_float(kb.y & 0xFFFFu),
+                            bf16_bits_to_float(kb.y >> 16)};
+        float product = 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) product += k[i] * z[i];
+        const float c = bf16_bits_to_float(betas[row]) * half_sum(product);
+        const float d = decays[row];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) z[i] = d * (z[i] - c * k[i]);
+        if (j == row) coefficient = c;
+      }
+      if (lane < 32u) {
+        *reinterpret_cast<float4 *>(&transformed[token][column]) = make_float4(z[0], z[1], z[2], z[3]);
+        if (j < kRows) coefficients[token][j] = coefficient;
+      }
+    }
+    __syncthreads();
+  }
 
   // ---- recurrence ----
   {
@@ -291,8 +343,26 @@ __global__ __launch_bounds__(64 * kWaves) void gdn_decode(const uint16_t *__rest
         *reinterpret_cast<float4 *>(stateOut + (size_t(head) * kDim + valueDim[r]) * kDim + column) =
             make_float4(state[r][0], state[r][1], state[r][2], state[r][3]);
       for (uint32_t token = 0; token < rows; ++token) {
-        advance<kInFlight, true>(state, keys[token], values[token], valueDim, decays[token], bf16_bits_to_float(betas[token]),
-                                 queries[token], result, column);
+        if (chain) {
+          advance<kInFlight, true>(state, keys[token], values[token], valueDim, decays[token], bf16_bits_to_float(betas[token]),
+                                   queries[token], result, column);
+        } else {
+          // The path's terms, a lane per block row, beside the committed state's product with the
+          // transformed query (gdn.metal:363-377).
+          const uint32_t j = lane & 31u, pathRowIndex = j & (kRows - 1u);
+          const bool onPath = j < kRows && ((paths[token] >> j) & 1u);
+          const float coefficient = coefficients[token][pathRowIndex];
+          const float4 zq = *reinterpret_cast<const float4 *>(&transformed[token][column]);
+#pragma unroll
+          for (int r = 0; r < kInFlight; ++r) {
+            result[r] = onPath ? coefficient * bf16_bits_to_float(values[pathRowIndex][valueDim[r]]) : 0.0f;
+            result[r] += state[r][0] * zq.x;
+            result[r] += state[r][1] * zq.y;
+            result[r] += state[r][2] * zq.z;
+            result[r] += state[r][3] * zq.w;
+            result[r] = half_sum(result[r]);
+          }
+        }
         if ((lane & 31u) == 0) {
 #pragma unroll
           for (int r = 0; r < kInFlight; ++r) outputs[token][valueDim[r]] = uint16_t(float_to_bf16_bits(result[r]));

@@ -1,4 +1,5 @@
 #include "ops/Gdn.hpp"
+#include "abi/PagedAttention.h"  // AttentionTreeRow
 #include "ops/Linear.hpp"  // requireBytes
 
 #include <algorithm>
@@ -19,11 +20,10 @@ uint64_t gdnTapeLayerBytes(const GdnShape &shape) noexcept {
 }
 
 void GDN::addDecode(hip::CommandGraph &graph, const GdnDecodeBuffers &b, const GdnShape &shape, uint32_t layer,
-                    const GdnStateStrides &state, GdnHeadOrder order, const std::vector<GdnLaneStep> &lanes, bool chains) {
+                    const GdnStateStrides &state, GdnHeadOrder order, const std::vector<GdnLaneStep> &lanes) {
   if (!shape.valid()) throw std::invalid_argument("invalid GDN shape");
   if (!state.valid()) throw std::invalid_argument("invalid GDN state strides");
   if (lanes.empty() || lanes.size() > GDN_MAXIMUM_LANES) throw std::invalid_argument("a GDN step takes 1 to 8 lanes");
-  if (!chains) throw std::invalid_argument("GDN tree blocks are not built: a lane's rows are a chain");
   const uint64_t tapeBytes = gdnTapeLayerBytes(shape);
   const uint64_t cellNeed = state.convolutionStateBytes + uint64_t{layer + 1} * state.recurrentLayerBytes;
   if (uint64_t{layer + 1} * state.convolutionLayerBytes > state.convolutionStateBytes)
@@ -61,7 +61,9 @@ void GDN::addDecode(hip::CommandGraph &graph, const GdnDecodeBuffers &b, const G
   requireBytes(b.timeBias, uint64_t{shape.valueHeads} * 2, "GDN time bias");
   requireBytes(b.mixerNorm, uint64_t{GDN_HEAD_DIMENSION} * (b.floatNorm ? 4 : 2), "GDN output norm");
   requireBytes(b.hidden, uint64_t{rows} * shape.valueHeads * GDN_HEAD_DIMENSION * 2, "GDN hidden rows");
-  graph.add("gdn_decode", {b.packed, b.convolutionWeights, b.states, b.tape, b.decayWeights, b.timeBias, b.mixerNorm, b.hidden}, params,
+  requireBytes(b.tree, uint64_t{rows} * sizeof(AttentionTreeRow), "GDN tree rows");
+  graph.add("gdn_decode", {b.packed, b.convolutionWeights, b.states, b.tape, b.decayWeights, b.timeBias, b.mixerNorm, b.hidden, b.tree},
+            params,
             {shape.valueHeads, uint32_t(lanes.size()), 1}, {1024, 1, 1});
 }
 

@@ -55,6 +55,10 @@ struct GdnDecodeBuffers final {
   hip::Buffer mixerNorm;           // bf16 or fp32 [128]
   bool floatNorm = false;
   hip::Buffer hidden;              // bf16 [rows][valueHeads * 128]
+  // The step's rows' places in their blocks' trees (AttentionTreeRow, a row each): a chain's rows
+  // run the sequential recurrence, another tree's rows each read the state before the block along
+  // their own path, and every row's convolution reads its path's tokens (GDN.hpp:143-147).
+  hip::Buffer tree;
 };
 struct GdnFoldBuffers final {
   hip::Buffer states;
@@ -67,10 +71,9 @@ struct GdnFoldBuffers final {
 
 class GDN final {
 public:
-  // The step of 1 to 8 lanes of one layer. `chains`: every lane's block is a chain (row r follows
-  // row r - 1); a tree block is refused (the kernel does not transform tree rows).
+  // The step of 1 to 8 lanes of one layer.
   static void addDecode(hip::CommandGraph &graph, const GdnDecodeBuffers &buffers, const GdnShape &shape, uint32_t layer,
-                        const GdnStateStrides &state, GdnHeadOrder order, const std::vector<GdnLaneStep> &lanes, bool chains = true);
+                        const GdnStateStrides &state, GdnHeadOrder order, const std::vector<GdnLaneStep> &lanes);
   // The state after the first `rows` rows of the path a lane retained of a step, in each of `layers` layers.
   static void addFold(hip::CommandGraph &graph, const GdnFoldBuffers &buffers, const GdnShape &shape, uint32_t layers, uint32_t rows,
                       const GdnStateStrides &state);

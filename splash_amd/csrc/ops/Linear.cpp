@@ -96,7 +96,8 @@ LinearPlan Linear::plan(LinearWorkload w, FloatOutput destination) const {
   // workgroup's range is down to minimumBlocksPerWave super-blocks.
   const uint32_t blocks = w.matrix.inputSize / GGUF_BLOCK;
   const uint32_t groups = std::max(1u, groupsOf(w.matrix.outputSize, w.epilogue));
-  const uint32_t wanted = calibration_.computeUnits * calibration_.groupsPerUnit;
+  const uint32_t wanted =
+      calibration_.computeUnits * (w.formatId == GGUF_FMT_Q6K ? calibration_.groupsPerUnitQ6K : calibration_.groupsPerUnit);
   const uint32_t most = std::min(LinearConfig::kMaximumSplits, std::max(1u, blocks / calibration_.minimumBlocksPerWave));
   LinearConfig config;
   const uint32_t units = calibration_.computeUnits;
@@ -108,13 +109,17 @@ LinearPlan Linear::plan(LinearWorkload w, FloatOutput destination) const {
     config.splits = std::clamp((units + (groups % units) / 2) / (groups % units), 1u, most);
     if (config.splits == 1) config.wholeGroups = 0;
   } else {
-    config.splits = std::clamp((wanted + groups / 2) / groups, 1u, most);
+    // Rounded down: one workgroup past a full round costs a second round.
+    config.splits = std::clamp(wanted / groups, 1u, most);
   }
   return LinearPlan(w, config, destination);
 }
 
 LinearPlan Linear::plan(const Projection &projection, uint32_t rows, LinearEpilogue epilogue) const {
-  return plan(LinearWorkload{{projection.outputSize, projection.inputSize}, rows, epilogue},
+  uint32_t format = GGUF_FMT_Q4K;
+  for (const QuantizedSegment &segment : projection.blocks().segments)
+    if (segment.formatId == GGUF_FMT_Q6K) format = GGUF_FMT_Q6K;
+  return plan(LinearWorkload{{projection.outputSize, projection.inputSize}, rows, epilogue, format},
               epilogue == LinearEpilogue::None ? projection.destination : FloatOutput::BFloat16);
 }
 

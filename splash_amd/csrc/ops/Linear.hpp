@@ -36,6 +36,9 @@ struct LinearWorkload final {
   LinearMatrix matrix;
   uint32_t rows = 0;
   LinearEpilogue epilogue = LinearEpilogue::None;
+  // The widest record format among the projection's segments: it sets how many workgroups a
+  // compute unit holds at once.
+  uint32_t formatId = GGUF_FMT_Q4K;
   auto operator<=>(const LinearWorkload &) const = default;
 };
 
@@ -126,10 +129,13 @@ struct LinearBuffers final {
 // measured on MI355X, overridable for sweeps.
 struct KernelCalibration final {
   uint32_t computeUnits = 256;
-  // Workgroups a projection should hold per compute unit before it stops partitioning K.
+  // Workgroups a compute unit holds at once (what the kernel's registers allow): a projection
+  // partitions K until one round of them fills the device, and no further. Q6_K records keep more
+  // registers live than Q4_K ones.
   uint32_t groupsPerUnit = 4;
   // Fewest super-blocks a workgroup's K range keeps.
   uint32_t minimumBlocksPerWave = 5;
+  uint32_t groupsPerUnitQ6K = 3;
 };
 
 class Linear final {

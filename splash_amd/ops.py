@@ -317,14 +317,15 @@ class GDN:
         check(lib.spo_gdn_layout(ctypes.byref(self.shape), layers, ctypes.byref(self.strides), ctypes.byref(cell), ctypes.byref(tape)))
         self.cell_bytes, self.tape_layer_bytes = cell.value, tape.value
 
-    def add_decode(self, graph, buffers, layer, lanes, tiled_heads=False, float_norm=False, chains=True):
-        """buffers: dict of Buffer by the names of spo_gdn_decode_buffers; lanes: [dict(first_row, rows, pending_path,
-        pending_tape, step_tape, current_cell, next_cell)]."""
+    def add_decode(self, graph, buffers, layer, lanes, tiled_heads=False, float_norm=False):
+        """buffers: dict of Buffer by the names of spo_gdn_decode_buffers (tree_rows among them: 8 bytes a row, uint32
+        ancestors, uint16 parent, uint16 depth); lanes: [dict(first_row, rows, pending_path, pending_tape, step_tape,
+        current_cell, next_cell)]."""
         b = nat.GdnDecodeBuffers(**{k: v.handle for k, v in buffers.items()}, float_norm=int(float_norm))
         arr = (nat.GdnLane * len(lanes))(*[nat.GdnLane(l["first_row"], l["rows"], l.get("pending_path", 0), 0, l.get("pending_tape", 0),
                                                        l["step_tape"], l["current_cell"], l["next_cell"]) for l in lanes])
         check(lib.spo_gdn_add_decode(graph.handle, ctypes.byref(b), ctypes.byref(self.shape), layer, ctypes.byref(self.strides),
-                                     int(tiled_heads), arr, len(lanes), int(chains)))
+                                     int(tiled_heads), arr, len(lanes)))
         graph._keep.extend(list(buffers.values()))
 
     def add_fold(self, graph, states, tape, retained_rows, step_tape, state_cell, fold_cell, rows):

@@ -30,3 +30,27 @@ def ulps(a_bits, b_bits):
         x = x.astype(np.int32)
         return np.where(x & 0x8000, 0x8000 - x, x)
     return np.abs(key(np.asarray(a_bits)) - key(np.asarray(b_bits)))
+
+
+def make_tree(rng, rows):
+    """A random tree over `rows` block rows, row 0 its root: each row's parent is an earlier row. Returns the
+    rows' path masks (bit j: row j is on the row's path, itself included)."""
+    masks = np.zeros(rows, np.uint32)
+    masks[0] = 1
+    for r in range(1, rows):
+        masks[r] = masks[int(rng.integers(0, r))] | np.uint32(1 << r)
+    return masks
+
+
+def path_rows(mask):
+    return [j for j in range(32) if (int(mask) >> j) & 1]
+
+
+def tree_rows_array(masks):
+    """The 8-byte tree rows (uint32 ancestors, uint16 parent, uint16 depth) of path masks."""
+    out = np.zeros((len(masks), 2), np.uint32)
+    for r, m in enumerate(masks):
+        path = path_rows(m)
+        parent = path[-2] if len(path) > 1 else 0xFFFF
+        out[r] = (int(m), parent | ((len(path) - 1) << 16))
+    return out

@@ -302,8 +302,10 @@ def gdn_split_tape(shape, tape):
             tape[b:c].view(np.float32).reshape(16, shape.value_heads), tape[c:d].view(np.uint16).reshape(16, shape.value_heads))
 
 
-def gdn_decode(shape, packed, conv_weights, a_scale, dt_bias, norm_weight, conv_in, state_in, pending_tape=None, pending_path=0):
-    """One lane, one layer, a chain of packed.shape[0] rows. Returns (conv_out, state_out, step_tape bytes, hidden)."""
+def gdn_decode(shape, packed, conv_weights, a_scale, dt_bias, norm_weight, conv_in, state_in, pending_tape=None, pending_path=0,
+               ancestors=None):
+    """One lane, one layer, a block of packed.shape[0] rows (a chain without `ancestors`, the rows' path masks).
+    Returns (conv_out, state_out, step_tape bytes, hidden)."""
     rows = packed.shape[0]
     vh = shape.value_heads
     conv_out = np.zeros((3, shape.conv_dim), np.uint16)
@@ -312,7 +314,8 @@ def gdn_decode(shape, packed, conv_weights, a_scale, dt_bias, norm_weight, conv_
     hidden = np.zeros((rows, vh * 128), np.uint16)
     packed, conv_weights, a_scale, dt_bias, norm_weight, conv_in, state_in = (np.ascontiguousarray(x) for x in (
         packed, conv_weights, a_scale, dt_bias, norm_weight, conv_in, state_in))
-    rc = lib.orc_gdn_decode(ctypes.byref(shape), _p(packed, u16p), rows, _p(conv_weights, u16p), _p(a_scale, f32p), _p(dt_bias, u16p),
+    masks = None if ancestors is None else np.ascontiguousarray(ancestors, np.uint32)
+    rc = lib.orc_gdn_decode(ctypes.byref(shape), _p(packed, u16p), rows, _p(masks, u32p), _p(conv_weights, u16p), _p(a_scale, f32p), _p(dt_bias, u16p),
                             norm_weight.ctypes.data_as(ctypes.c_void_p), _p(conv_in, u16p), _p(state_in, f32p),
                             _p(pending_tape, u8p), pending_path, _p(conv_out, u16p), _p(state_out, f32p), _p(tape, u8p), _p(hidden, u16p))
     assert rc == 0
@@ -320,7 +323,7 @@ def gdn_decode(shape, packed, conv_weights, a_scale, dt_bias, norm_weight, conv_
 
 
 lib.orc_gdn_decode.restype = c_int
-lib.orc_gdn_decode.argtypes = [ctypes.POINTER(GdnShape), u16p, c_u32, u16p, f32p, u16p, ctypes.c_void_p, u16p, f32p, u8p, c_u32, u16p,
+lib.orc_gdn_decode.argtypes = [ctypes.POINTER(GdnShape), u16p, c_u32, u32p, u16p, f32p, u16p, ctypes.c_void_p, u16p, f32p, u8p, c_u32, u16p,
                                f32p, u8p, u16p]
 lib.orc_gdn_fold.restype = c_int
 lib.orc_gdn_fold.argtypes = [ctypes.POINTER(GdnShape), u16p, f32p, u8p, c_u32, c_u32, u16p, f32p]

@@ -6,7 +6,7 @@ import pytest
 import splash_amd
 from splash_amd import ops
 from tests import oracle as orc
-from tests.gdn_case import make_layer, make_rows, make_state, ulps
+from tests.gdn_case import make_layer, make_rows, make_state, make_tree, path_rows, tree_rows_array, ulps
 
 pytestmark = pytest.mark.gpu
 
@@ -50,17 +50,20 @@ class Layer:
         return raw[self.slot(lane, parity, layer):][:self.gdn.tape_layer_bytes].copy()
 
     def step(self, blocks, layer=0):
-        """blocks: [(lane, packed rows, pending_path, parity, current cell, next cell)]; returns hidden rows per block."""
+        """blocks: [(lane, packed rows, pending_path, parity, current cell, next cell[, path masks])]; a block without
+        masks is a chain. Returns hidden rows per block."""
         packed = np.concatenate([b[1] for b in blocks])
         rows = packed.shape[0]
         hidden = self.backend.allocate_buffer(rows * self.shape.value_heads * 128 * 2)
+        tree = np.concatenate([tree_rows_array(b[6] if len(b) > 6 else [(2 << r) - 1 for r in range(b[1].shape[0])]) for b in blocks])
         lanes, first = [], 0
-        for lane, block, path, parity, cur, nxt in blocks:
+        for lane, block, path, parity, cur, nxt in (b[:6] for b in blocks):
             lanes.append(dict(first_row=first, rows=block.shape[0], pending_path=path, pending_tape=self.slot(lane, parity ^ 1, layer),
                               step_tape=self.slot(lane, parity, layer), current_cell=self.cell(lane, cur), next_cell=self.cell(lane, nxt)))
             first += block.shape[0]
         graph = splash_amd.CommandGraph()
-        buffers = dict(packed=self.backend.from_array(packed), states=self.states, tape=self.tape, hidden=hidden, **self.weights)
+        buffers = dict(packed=self.backend.from_array(packed), states=self.states, tape=self.tape, hidden=hidden,
+                       tree_rows=self.backend.from_array(tree), **self.weights)
         self.gdn.add_decode(graph, buffers, layer, lanes, float_norm=self.float_norm)
         self.backend.run(graph)
         out = hidden.download(np.uint16).reshape(rows, self.shape.value_heads * 128)
@@ -188,6 +191,70 @@ def test_full_size_step_keeps_the_invariants(backend):
         assert np.array_equal(conv, fconv) and state.tobytes() == fstate.tobytes()
 
 
+@pytest.mark.parametrize("heads", [(2, 4), (16, 32)])
+def test_tree_blocks(backend, heads):
+    """A block that is not a chain: against the oracle's tree form (same order of operations: a bf16 step where the
+    GPU's exp2 differs), every row's tape entries bit for bit those of its path run as a chain on the GPU, its
+    output the chain's up to the reordering of the path form; a chain lane beside a tree lane in one dispatch is
+    unchanged; and the step after folds an accepted path of the tree to the state its chain leaves, bit for bit."""
+    print(f"case gdn tree heads={heads}", flush=True)
+    rng = np.random.default_rng(25)
+    layer = Layer(backend, rng, *heads, lanes=2, cells=4)
+    shape, vh = layer.shape, layer.shape.value_heads
+    rows = 16
+    cells = [make_state(rng, shape) for _ in range(2)]
+    blocks = [make_rows(rng, shape, rows), make_rows(rng, shape, 7)]
+    previous = make_rows(rng, shape, 6)
+    pending = 0b101101
+    masks = make_tree(rng, rows)
+    for lane in range(2):
+        layer.write_cell(lane, 0, *cells[lane])
+    layer.step([(0, previous, 0, 0, 0, 1), (1, previous, 0, 0, 0, 1)])
+    hidden_tree, hidden_chain = layer.step([(0, blocks[0], pending, 1, 1, 2, masks), (1, blocks[1], pending, 1, 1, 2)])
+    conv_b, state_b = layer.read_cell(0, 1)
+    want = orc.gdn_decode(shape, blocks[0], layer.conv_w, layer.a_scale, layer.dt_bias, layer.norm, conv_b, state_b,
+                          pending_tape=layer.read_tape(0, 0), pending_path=pending, ancestors=masks)
+    got_conv, got_state = layer.read_cell(0, 2)
+    assert np.array_equal(got_conv, want[0])
+    assert np.abs(got_state - want[1]).max() <= 1e-4 * np.abs(want[1]).max()
+
+    def close(got_bits, want_bits, relative=2.0 ** -6, of_row=2.0 ** -7):
+        g, w = orc.bf16_to_f32(got_bits).astype(np.float64), orc.bf16_to_f32(want_bits).astype(np.float64)
+        scale = np.abs(w).reshape(-1, vh, 128).max(axis=2, keepdims=True).repeat(128, axis=2).reshape(w.shape)
+        assert np.all(np.abs(g - w) <= relative * np.abs(w) + of_row * scale), np.abs(g - w).max()
+    close(hidden_tree, want[3])
+    assert (ulps(hidden_tree, want[3]) <= 1).mean() >= 0.97
+    # the chain lane beside it equals the chain lane alone
+    solo = Layer(backend, np.random.default_rng(25), *heads, lanes=2, cells=4)
+    solo.write_cell(1, 0, *cells[1])
+    solo.step([(1, previous, 0, 0, 0, 1)])
+    (alone,) = solo.step([(1, blocks[1], pending, 1, 1, 2)])
+    assert np.array_equal(alone, hidden_chain)
+    # each tree row against its path run as a chain on the GPU
+    tape_tree = orc.gdn_split_tape(shape, layer.read_tape(0, 1))
+    deepest = max(range(rows), key=lambda r: bin(int(masks[r])).count("1"))
+    for r in sorted({deepest, rows - 1, 1}):
+        path = path_rows(masks[r])
+        chain = Layer(backend, np.random.default_rng(25), *heads, lanes=1, cells=4)
+        chain.write_cell(0, 0, *cells[0])
+        chain.step([(0, previous, 0, 0, 0, 1)])
+        (hc,) = chain.step([(0, blocks[0][path], pending, 1, 1, 2)])
+        tape_chain = orc.gdn_split_tape(shape, chain.read_tape(0, 1))
+        last = len(path) - 1
+        for part in range(4):
+            assert np.array_equal(tape_tree[part][r], tape_chain[part][last]), (r, part)
+        close(hidden_tree[r:r + 1], hc[last:last + 1], of_row=2.0 ** -8)
+        if r != deepest:
+            continue
+        # accept the deepest row's path: the next step's cell and outputs are those after the chain
+        nxt = make_rows(rng, shape, 4)
+        (ha,) = layer.step([(0, nxt, int(masks[r]), 0, 2, 3)])
+        (hb,) = chain.step([(0, nxt, (1 << len(path)) - 1, 0, 2, 3)])
+        conv_a, state_a = layer.read_cell(0, 3)
+        conv_c, state_c = chain.read_cell(0, 3)
+        assert np.array_equal(conv_a, conv_c) and state_a.tobytes() == state_c.tobytes() and np.array_equal(ha, hb)
+
+
 def test_gdn_rejects_bad_arguments(backend):
     rng = np.random.default_rng(24)
     layer = Layer(backend, rng, 2, 4, lanes=1)
@@ -198,10 +265,11 @@ def test_gdn_rejects_bad_arguments(backend):
         layer.step([(0, make_rows(rng, layer.shape, 17), 0, 0, 0, 1)])
     graph = splash_amd.CommandGraph()
     buffers = dict(packed=backend.from_array(rows), states=layer.states, tape=layer.tape,
-                   hidden=backend.allocate_buffer(4 * layer.shape.value_heads * 256), **layer.weights)
+                   hidden=backend.allocate_buffer(4 * layer.shape.value_heads * 256),
+                   tree_rows=backend.from_array(tree_rows_array([1, 3, 7])), **layer.weights)
     lane = dict(first_row=0, rows=4, step_tape=0, current_cell=0, next_cell=layer.gdn.cell_bytes)
-    with pytest.raises(ValueError, match="tree"):
-        layer.gdn.add_decode(graph, buffers, 0, [lane], chains=False)
+    with pytest.raises(ValueError, match="tree rows"):
+        layer.gdn.add_decode(graph, buffers, 0, [lane])        # three tree rows for a block of four
     with pytest.raises(ValueError):
         ops.GDN(3, 4)
     assert len(graph) == 0

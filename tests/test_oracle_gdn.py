@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 
 from tests import oracle as orc
-from tests.gdn_case import make_layer, make_rows, make_state, ulps
+from tests.gdn_case import make_layer, make_rows, make_state, make_tree, path_rows, ulps
 
 
 def test_step_matches_the_fp64_recurrence():
@@ -102,3 +102,75 @@ def test_fold_and_rollback(accepted):
         assert rc == 1                                   # a path shorter than the rows asked for folds nothing
     else:
         assert np.array_equal(conv1, conv_in) and state1.tobytes() == state_in.tobytes()
+
+
+def test_tree_rows_are_the_chains_of_their_paths():
+    """A tree block (gdn.metal:417-478): every row's tape entries are bit for bit those of its path run as a chain
+    (the convolution follows the path), its output is the chain's up to the fp32 reordering of the path form
+    S_-1 z_-1 + sum c_j v_j, and within the fp64 recurrence's bounds along the path; a tree whose rows happen to
+    be a chain is the chain bit for bit; the state the step writes does not depend on the tree."""
+    rng = np.random.default_rng(31)
+    shape, conv_w, a_scale, dt_bias, norm = make_layer(rng, 2, 4)
+    rows, vh = 12, shape.value_heads
+    packed = make_rows(rng, shape, rows)
+    conv_in, state_in = make_state(rng, shape)
+    previous = make_rows(rng, shape, 5)
+    conv0, state0, tape0, _ = orc.gdn_decode(shape, previous, conv_w, a_scale, dt_bias, norm, conv_in, state_in)
+    pending = 0b10011      # rows 0, 1, 4 of the previous step were accepted
+    args = (conv_w, a_scale, dt_bias, norm, conv0, state0)
+    chain = orc.gdn_decode(shape, packed, *args, pending_tape=tape0, pending_path=pending)
+    as_tree = orc.gdn_decode(shape, packed, *args, pending_tape=tape0, pending_path=pending,
+                             ancestors=[(2 << r) - 1 for r in range(rows)])
+    for a, b in zip(chain, as_tree):
+        assert np.array_equal(a, b)
+    masks = make_tree(rng, rows)
+    assert any(int(m) != (2 << r) - 1 for r, m in enumerate(masks))
+    conv1, state1, tape1, hidden = orc.gdn_decode(shape, packed, *args, pending_tape=tape0, pending_path=pending, ancestors=masks)
+    assert np.array_equal(conv1, chain[0]) and state1.tobytes() == chain[1].tobytes()
+    inputs, kv, decay, beta = orc.gdn_split_tape(shape, tape1)
+    assert np.array_equal(inputs[:rows], packed[:, :shape.conv_dim])
+    # the fp64 check starts from the state after the pending rows (state1) and the convolution carry they leave
+    for r in range(rows):
+        path = path_rows(masks[r])
+        along = packed[path]
+        _, _, tape_c, hidden_c = orc.gdn_decode(shape, along, *args, pending_tape=tape0, pending_path=pending)
+        ci, ckv, cdecay, cbeta = orc.gdn_split_tape(shape, tape_c)
+        last = len(path) - 1
+        assert np.array_equal(kv[r], ckv[last]) and np.array_equal(beta[r], cbeta[last]) and np.array_equal(decay[r], cdecay[last])
+        got = orc.bf16_to_f32(hidden[r]).astype(np.float64)
+        want = orc.bf16_to_f32(hidden_c[last]).astype(np.float64)
+        scale = np.abs(want).reshape(vh, 128).max(axis=1, keepdims=True).repeat(128, axis=1).reshape(-1)
+        # the two forms round differently before the output norm: a bf16 step of the value, a fraction of one of the row
+        assert np.all(np.abs(got - want) <= 2.0 ** -6 * np.abs(want) + 2.0 ** -8 * scale), (r, np.abs(got - want).max())
+        assert (ulps(hidden[r], hidden_c[last]) <= 1).mean() >= 0.95
+        kv64, beta64, decay64, state64, out64 = orc.gdn_reference(shape, along, conv_w, a_scale, dt_bias, conv1, state1)
+        z = orc.bf16_to_f32(packed[r, shape.conv_dim:shape.conv_dim + vh * 128]).astype(np.float64).reshape(vh, 128)
+        w = orc.bf16_to_f32(norm).astype(np.float64)
+        o = out64[last]
+        normed = o / np.sqrt((o ** 2).mean(axis=1, keepdims=True) + 1e-6) * w
+        ref = orc.bf16_to_f32(orc.f32_to_bf16((normed * z / (1 + np.exp(-z))).astype(np.float32))).astype(np.float64).reshape(-1)
+        rscale = np.abs(ref).reshape(vh, 128).max(axis=1, keepdims=True).repeat(128, axis=1).reshape(-1)
+        assert np.all(np.abs(got - ref) <= 2.0 ** -5 * np.abs(ref) + 2.0 ** -6 * rscale)
+
+
+def test_a_tree_path_folds_like_its_chain():
+    """Accepting a path of a tree step: the next step's state is bit for bit the state after the path's rows run
+    as a chain, and the fold of the path alone is that state."""
+    rng = np.random.default_rng(32)
+    shape, conv_w, a_scale, dt_bias, norm = make_layer(rng, 1, 2)
+    rows = 9
+    packed = make_rows(rng, shape, rows)
+    conv_in, state_in = make_state(rng, shape)
+    masks = make_tree(rng, rows)
+    leaf = max(range(rows), key=lambda r: bin(int(masks[r])).count("1"))
+    path = int(masks[leaf])
+    args = (conv_w, a_scale, dt_bias, norm)
+    conv0, state0, tape0, _ = orc.gdn_decode(shape, packed, *args, conv_in, state_in, ancestors=masks)
+    nxt = make_rows(rng, shape, 3)
+    conv1, state1, _, hidden1 = orc.gdn_decode(shape, nxt, *args, conv0, state0, pending_tape=tape0, pending_path=path)
+    along = packed[path_rows(path)]
+    convc, statec, tapec, _ = orc.gdn_decode(shape, along, *args, conv_in, state_in)
+    conv2, state2, _, hidden2 = orc.gdn_decode(shape, nxt, *args, convc, statec, pending_tape=tapec, pending_path=(1 << len(along)) - 1)
+    assert np.array_equal(conv1, conv2) and state1.tobytes() == state2.tobytes() and np.array_equal(hidden1, hidden2)
+    rc, convf, statef = orc.gdn_fold(shape, conv0, state0, tape0, path, len(along))
+    assert rc == 0 and np.array_equal(convf, conv1) and statef.tobytes() == state1.tobytes()
