@@ -252,6 +252,54 @@ sp_status spo_dense_verify_encode(spo_dense_verify *verify, spo_graph *graph, co
 sp_status spo_dense_verify_encode_part(spo_dense_verify *verify, spo_graph *graph, uint32_t part, uint32_t index,
                                        const spo_verify_lane *lanes, uint32_t count);
 
+/* ---- The hybrid mixture-of-experts verify step (the reference's Qwen3.5 target with Gated
+ *      DeltaNet mixers: QwenTarget.cpp:206-255 the GDN mixer, :263-347 the attention mixer, :372-395
+ *      the MoE routing, :457-496 the layer recipe; Runtime.cpp:2701-2707 tape parity and pending
+ *      path). Layer l attends when (l + 1) % attention_interval == 0; the others run GDN. ---- */
+typedef struct spo_hybrid_verify spo_hybrid_verify;
+typedef struct spo_hybrid_dimensions {
+  uint32_t hidden, vocabulary, layers, attention_interval;
+  uint32_t q_heads, kv_heads, head_dim, rotary_pairs, normalize_heads;
+  float rope_theta;
+  uint32_t gdn_key_heads, gdn_value_heads, gdn_packed_width; /* packed row [q|k|v|z|b|a], whole column tiles */
+  uint32_t experts, top_k, expert_ffn;
+} spo_hybrid_dimensions;
+typedef struct spo_hybrid_lane {
+  spo_verify_lane block;
+  uint32_t pending_path; /* rows of the lane's previous step it accepted: that step's retained-rows mask */
+  uint32_t parity;       /* the step reads the lane's cell `parity` and writes the other; the next step flips it */
+} spo_hybrid_lane;
+typedef struct spo_hybrid_layer {
+  const spo_projection *mixer_input, *mixer_output; /* q|k|v and o, or the packed GDN row and its output projection */
+  sp_buffer *input_norm, *post_norm;
+  sp_buffer *query_norm, *key_norm;                                   /* attention layers */
+  sp_buffer *convolution_weights, *decay_weights, *time_bias, *mixer_norm; /* GDN layers; mixer_norm bf16 [128] */
+  const spo_projection *router;                                       /* hidden -> experts, fp32 scores */
+  sp_buffer *gate_images, *up_images, *down_images;                   /* every expert's image of each tensor */
+  uint32_t expert_format, expert_down_format;
+} spo_hybrid_layer;
+sp_status spo_hybrid_verify_create(sp_backend *backend, const spo_hybrid_dimensions *dimensions, uint32_t max_lanes,
+                                   uint32_t physical_pages, uint32_t page_table_entries, spo_hybrid_verify **out);
+void spo_hybrid_verify_destroy(spo_hybrid_verify *verify);
+sp_status spo_hybrid_verify_set_layer(spo_hybrid_verify *verify, uint32_t layer, const spo_hybrid_layer *weights);
+sp_status spo_hybrid_verify_set_head(spo_hybrid_verify *verify, uint32_t embedding_format, sp_buffer *embedding_rows,
+                                     sp_buffer *final_norm, const spo_projection *head);
+/* The step's buffers, as spo_dense_verify_buffer; `index` is the attention layer for KV pools. */
+#define SPO_VERIFY_GDN_STATES 13
+#define SPO_VERIFY_GDN_TAPE 14
+sp_status spo_hybrid_verify_buffer(spo_hybrid_verify *verify, uint32_t which, uint32_t index, sp_buffer **out);
+/* Where the recurrent state lives: a lane's cell of a parity at (lane * 2 + parity) * cell_bytes in the
+ * states buffer (strides as spo_gdn_layout gives them for the model's GDN layers), GDN layer g's tape of
+ * a lane's step of a parity at ((lane * 2 + parity) * gdn_layers + g) * tape_layer_bytes in the tape buffer. */
+sp_status spo_hybrid_verify_layout(const spo_hybrid_verify *verify, uint64_t *page_bytes, uint64_t *cell_bytes,
+                                   uint64_t *tape_layer_bytes, spo_gdn_state_strides *strides);
+uint64_t spo_hybrid_verify_step_bytes(const spo_hybrid_verify *verify, const spo_hybrid_lane *lanes, uint32_t count);
+sp_status spo_hybrid_verify_encode(spo_hybrid_verify *verify, spo_graph *graph, const spo_hybrid_lane *lanes, uint32_t count,
+                                   int commit);
+/* One part of it: 0 embedding, 1 one layer (index), 2 final norm + head. */
+sp_status spo_hybrid_verify_encode_part(spo_hybrid_verify *verify, spo_graph *graph, uint32_t part, uint32_t index,
+                                        const spo_hybrid_lane *lanes, uint32_t count);
+
 #ifdef __cplusplus
 }
 #endif

@@ -136,6 +136,22 @@ class VerifyLane(ctypes.Structure):
                 ("remaining", c_u32)]
 
 
+class HybridDimensions(ctypes.Structure):
+    _fields_ = [(n, c_u32) for n in ("hidden", "vocabulary", "layers", "attention_interval", "q_heads", "kv_heads", "head_dim",
+                                     "rotary_pairs", "normalize_heads")] + [("rope_theta", ctypes.c_float)] + [
+        (n, c_u32) for n in ("gdn_key_heads", "gdn_value_heads", "gdn_packed_width", "experts", "top_k", "expert_ffn")]
+
+
+class HybridLane(ctypes.Structure):
+    _fields_ = [("block", VerifyLane), ("pending_path", c_u32), ("parity", c_u32)]
+
+
+class HybridLayer(ctypes.Structure):
+    _fields_ = [(n, c_p) for n in ("mixer_input", "mixer_output", "input_norm", "post_norm", "query_norm", "key_norm",
+                                   "convolution_weights", "decay_weights", "time_bias", "mixer_norm", "router", "gate_images",
+                                   "up_images", "down_images")] + [("expert_format", c_u32), ("expert_down_format", c_u32)]
+
+
 def _sig(name, restype, *argtypes):
     fn = getattr(lib, name)
     fn.restype = restype
@@ -236,3 +252,12 @@ _sig("spo_dense_verify_page_bytes", c_u64, c_p)
 _sig("spo_dense_verify_step_bytes", c_u64, c_p, P(VerifyLane), c_u32)
 _sig("spo_dense_verify_encode", c_int, c_p, c_p, P(VerifyLane), c_u32, c_int)
 _sig("spo_dense_verify_encode_part", c_int, c_p, c_p, c_u32, c_u32, P(VerifyLane), c_u32)
+_sig("spo_hybrid_verify_create", c_int, c_p, P(HybridDimensions), c_u32, c_u32, c_u32, P(c_p))
+_sig("spo_hybrid_verify_destroy", None, c_p)
+_sig("spo_hybrid_verify_set_layer", c_int, c_p, c_u32, P(HybridLayer))
+_sig("spo_hybrid_verify_set_head", c_int, c_p, c_u32, c_p, c_p, c_p)
+_sig("spo_hybrid_verify_buffer", c_int, c_p, c_u32, c_u32, P(c_p))
+_sig("spo_hybrid_verify_layout", c_int, c_p, P(c_u64), P(c_u64), P(c_u64), P(GdnStateStrides))
+_sig("spo_hybrid_verify_step_bytes", c_u64, c_p, P(HybridLane), c_u32)
+_sig("spo_hybrid_verify_encode", c_int, c_p, c_p, P(HybridLane), c_u32, c_int)
+_sig("spo_hybrid_verify_encode_part", c_int, c_p, c_p, c_u32, c_u32, P(HybridLane), c_u32)

@@ -1,0 +1,158 @@
+// C entry points of model::HybridVerify (include/splash_ops.h).
+#include "splash_ops.h"
+#include "capi/Guard.hpp"
+#include "capi/Handles.hpp"
+#include "model/HybridVerify.hpp"
+
+#include <memory>
+
+using namespace splash;
+
+struct spo_hybrid_verify {
+  std::unique_ptr<hip::Backend> backend;  // a borrowed wrapper of the caller's backend
+  std::unique_ptr<model::HybridVerify> verify;
+};
+
+namespace {
+hip::Buffer B(sp_buffer *b) { return hip::Buffer::share(b); }
+std::vector<model::HybridLane> lanesOf(const spo_hybrid_lane *lanes, uint32_t count) {
+  capi::require(lanes && count, "lanes");
+  std::vector<model::HybridLane> out;
+  for (uint32_t i = 0; i < count; ++i) {
+    const spo_verify_lane &b = lanes[i].block;
+    out.push_back({{b.rows, b.committed, b.table_first, ops::SamplingPolicy{b.temperature}, b.remaining}, lanes[i].pending_path,
+                   lanes[i].parity});
+  }
+  return out;
+}
+} // namespace
+
+extern "C" {
+
+sp_status spo_hybrid_verify_create(sp_backend *backend, const spo_hybrid_dimensions *d, uint32_t max_lanes, uint32_t physical_pages,
+                                   uint32_t page_table_entries, spo_hybrid_verify **out) {
+  return capi::guard([&] {
+    capi::require(backend && d && out, "backend, dimensions or result");
+    auto holder = std::make_unique<spo_hybrid_verify>();
+    holder->backend = std::make_unique<hip::Backend>(backend);
+    model::HybridDimensions dims;
+    dims.hidden = d->hidden;
+    dims.vocabulary = d->vocabulary;
+    dims.layers = d->layers;
+    dims.attentionInterval = d->attention_interval;
+    dims.qHeads = d->q_heads;
+    dims.kvHeads = d->kv_heads;
+    dims.headDimension = d->head_dim;
+    dims.rotaryPairs = d->rotary_pairs;
+    dims.normalizeHeads = d->normalize_heads != 0;
+    dims.ropeTheta = d->rope_theta;
+    dims.gdnKeyHeads = d->gdn_key_heads;
+    dims.gdnValueHeads = d->gdn_value_heads;
+    dims.gdnPackedWidth = d->gdn_packed_width;
+    dims.experts = d->experts;
+    dims.topK = d->top_k;
+    dims.expertFfn = d->expert_ffn;
+    holder->verify = std::make_unique<model::HybridVerify>(*holder->backend, dims, max_lanes, physical_pages, page_table_entries);
+    *out = holder.release();
+  });
+}
+void spo_hybrid_verify_destroy(spo_hybrid_verify *verify) { delete verify; }
+
+sp_status spo_hybrid_verify_set_layer(spo_hybrid_verify *verify, uint32_t layer, const spo_hybrid_layer *l) {
+  return capi::guard([&] {
+    capi::require(verify && l && l->mixer_input && l->mixer_output && l->router, "verify, layer or projections");
+    model::HybridWeights &w = verify->verify->weights();
+    if (layer >= w.layers.size()) throw std::invalid_argument("no such layer");
+    model::HybridLayer out;
+    out.mixerInput = capi::projectionOf(l->mixer_input);
+    out.mixerOutput = capi::projectionOf(l->mixer_output);
+    out.inputNorm = B(l->input_norm);
+    out.postNorm = B(l->post_norm);
+    out.queryNorm = B(l->query_norm);
+    out.keyNorm = B(l->key_norm);
+    out.convolutionWeights = B(l->convolution_weights);
+    out.decay = B(l->decay_weights);
+    out.timeBias = B(l->time_bias);
+    out.mixerNorm = B(l->mixer_norm);
+    out.router = capi::projectionOf(l->router);
+    out.router.destination = ops::FloatOutput::Float32;
+    out.experts = {B(l->gate_images), B(l->up_images), B(l->down_images), l->expert_format, l->expert_down_format};
+    w.layers[layer] = std::move(out);
+  });
+}
+sp_status spo_hybrid_verify_set_head(spo_hybrid_verify *verify, uint32_t embedding_format, sp_buffer *embedding_rows, sp_buffer *final_norm,
+                                     const spo_projection *head) {
+  return capi::guard([&] {
+    capi::require(verify && head, "verify or head");
+    model::HybridWeights &w = verify->verify->weights();
+    const model::HybridDimensions &d = verify->verify->dimensions();
+    w.embedding = {B(embedding_rows), embedding_format, d.vocabulary, d.hidden};
+    w.finalNorm = B(final_norm);
+    w.head = capi::projectionOf(head);
+    w.head.destination = ops::FloatOutput::Float32;
+  });
+}
+sp_status spo_hybrid_verify_buffer(spo_hybrid_verify *verify, uint32_t which, uint32_t index, sp_buffer **out) {
+  return capi::guard([&] {
+    capi::require(verify && out, "verify or result");
+    model::HybridVerify &v = *verify->verify;
+    hip::Buffer b;
+    switch (which) {
+    case SPO_VERIFY_INPUT_TOKENS: b = v.inputTokens(); break;
+    case SPO_VERIFY_TREE_ROWS: b = v.treeRows(); break;
+    case SPO_VERIFY_DEPTHS: b = v.depths(); break;
+    case SPO_VERIFY_UNIFORMS: b = v.uniforms(); break;
+    case SPO_VERIFY_TOKENS: b = v.tokens(); break;
+    case SPO_VERIFY_RETAINED: b = v.retained(); break;
+    case SPO_VERIFY_ACCEPTED: b = v.acceptedCount(); break;
+    case SPO_VERIFY_RETAINED_ROWS: b = v.retainedRows(); break;
+    case SPO_VERIFY_PAGE_TABLE: b = v.pageTable(); break;
+    case SPO_VERIFY_KV_POOL: b = v.kvPool(index); break;
+    case SPO_VERIFY_LOGITS: b = v.logits(); break;
+    case SPO_VERIFY_DRAFT_PROBABILITIES: b = v.draftProbabilities(); break;
+    case SPO_VERIFY_HIDDEN: b = v.hidden(index); break;
+    case SPO_VERIFY_GDN_STATES: b = v.gdnStates(); break;
+    case SPO_VERIFY_GDN_TAPE: b = v.gdnTape(); break;
+    default: throw std::invalid_argument("no such verify buffer");
+    }
+    sp_buffer_retain(b.handle());
+    *out = b.handle();
+  });
+}
+sp_status spo_hybrid_verify_layout(const spo_hybrid_verify *verify, uint64_t *page_bytes, uint64_t *cell_bytes, uint64_t *tape_layer_bytes,
+                                   spo_gdn_state_strides *strides) {
+  return capi::guard([&] {
+    capi::require(verify, "verify");
+    const model::HybridVerify &v = *verify->verify;
+    if (page_bytes) *page_bytes = v.pageBytes();
+    if (cell_bytes) *cell_bytes = v.gdnCellBytes();
+    if (tape_layer_bytes) *tape_layer_bytes = v.gdnTapeLayerBytes();
+    if (strides) *strides = {v.gdnStrides().convolutionLayerBytes, v.gdnStrides().recurrentLayerBytes, v.gdnStrides().convolutionStateBytes};
+  });
+}
+uint64_t spo_hybrid_verify_step_bytes(const spo_hybrid_verify *verify, const spo_hybrid_lane *lanes, uint32_t count) {
+  uint64_t bytes = 0;
+  capi::guard([&] { capi::require(verify, "verify"); bytes = verify->verify->stepBytes(lanesOf(lanes, count)); });
+  return bytes;
+}
+sp_status spo_hybrid_verify_encode(spo_hybrid_verify *verify, spo_graph *graph, const spo_hybrid_lane *lanes, uint32_t count, int commit) {
+  return capi::guard([&] {
+    capi::require(verify && graph, "verify or graph");
+    verify->verify->encode(capi::graphOf(graph), lanesOf(lanes, count), commit != 0);
+  });
+}
+sp_status spo_hybrid_verify_encode_part(spo_hybrid_verify *verify, spo_graph *graph, uint32_t part, uint32_t index,
+                                        const spo_hybrid_lane *lanes, uint32_t count) {
+  return capi::guard([&] {
+    capi::require(verify && graph, "verify or graph");
+    const std::vector<model::HybridLane> list = lanesOf(lanes, count);
+    uint32_t rows = 0;
+    for (const model::HybridLane &l : list) rows += l.block.rows;
+    if (part == 0) verify->verify->encodeEmbedding(capi::graphOf(graph), rows);
+    else if (part == 1) verify->verify->encodeLayer(capi::graphOf(graph), index, list);
+    else if (part == 2) verify->verify->encodeHead(capi::graphOf(graph), rows);
+    else throw std::invalid_argument("no such part of the step");
+  });
+}
+
+} // extern "C"

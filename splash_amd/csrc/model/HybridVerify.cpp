@@ -1,0 +1,254 @@
+#include "model/HybridVerify.hpp"
+
+#include <algorithm>
+#include <cmath>
+#include <stdexcept>
+
+namespace splash::model {
+
+using hip::BufferStorage;
+
+namespace {
+// Rows one projection dispatch takes: a longer step runs its dense projections in pieces.
+constexpr uint32_t kProjectionRows = ops::kMaximumDecodeTileRows;
+template <class F> void forRowPieces(uint32_t rows, F &&piece) {
+  for (uint32_t first = 0; first < rows; first += kProjectionRows) piece(first, std::min(kProjectionRows, rows - first));
+}
+} // namespace
+
+HybridVerify::HybridVerify(hip::Backend &backend, HybridDimensions d, uint32_t maxLanes, uint32_t physicalPages,
+                           uint32_t pageTableEntries)
+    : backend_(backend), dims_(d), linear_(backend.deviceInfo()), maxLanes_(maxLanes) {
+  if (!d.hidden || !d.layers || !d.vocabulary || !maxLanes || maxLanes > GDN_MAXIMUM_LANES)
+    throw std::invalid_argument("a hybrid verify step takes a model and 1 to 8 lanes");
+  if (!d.attentionInterval || d.layers % d.attentionInterval)
+    throw std::invalid_argument("the layers hold whole groups of recurrent layers and one attention layer");
+  if (d.hidden % GGUF_BLOCK || d.attentionWidth() % GGUF_BLOCK || d.gdnWidth() % GGUF_BLOCK || d.vocabulary % GGUF_TILE_COLUMNS ||
+      d.gdnPackedWidth % GGUF_TILE_COLUMNS || d.experts % GGUF_TILE_COLUMNS)
+    throw std::invalid_argument("the model's widths hold whole super-blocks and its projections whole column tiles");
+  if (!d.gdnShape().valid()) throw std::invalid_argument("invalid GDN shape");
+  if (!d.moeShape().valid()) throw std::invalid_argument("invalid MoE shape");
+  maxRows_ = maxLanes * ATTENTION_MAXIMUM_ROWS;
+  weights_.layers.resize(d.layers);
+  const ops::kv::Layout layout{d.kvHeads, d.headDimension};
+  pageBytes_ = layout.bytesPerLayerPage();
+  auto device = [&](uint64_t bytes, const char *label) { return backend.allocateBuffer(std::max<uint64_t>(bytes, 16), BufferStorage::Private, label); };
+  auto shared = [&](uint64_t bytes, const char *label) { return backend.allocateBuffer(std::max<uint64_t>(bytes, 16), BufferStorage::Shared, label); };
+  const uint64_t R = maxRows_;
+  hidden_[0] = device(R * d.hidden * 2, "hidden 0");
+  hidden_[1] = device(R * d.hidden * 2, "hidden 1");
+  normalized_ = device(R * d.hidden * 2, "normalized");
+  packed_ = device(R * std::max(d.qkvWidth(), d.gdnPackedWidth) * 2, "mixer input rows");
+  mixed_ = device(R * std::max(d.attentionWidth(), d.gdnWidth()) * 2, "mixer output rows");
+  scores_ = device(R * d.experts * 4, "router scores");
+  logits_ = device(R * d.vocabulary * 4, "logits");
+  ropeCos_ = device(R * std::max(1u, d.rotaryPairs) * 4, "rope cos");
+  ropeSin_ = device(R * std::max(1u, d.rotaryPairs) * 4, "rope sin");
+  inverseFrequency_ = device(std::max(1u, d.rotaryPairs) * 4, "rope inverse frequency");
+  if (d.rotaryPairs) {
+    std::vector<float> inv(d.rotaryPairs);
+    for (uint32_t i = 0; i < d.rotaryPairs; ++i) inv[i] = float(std::pow(double(d.ropeTheta), -double(i) / d.rotaryPairs));
+    inverseFrequency_.upload(inv.data(), inv.size() * 4);
+  }
+  inputTokens_ = shared(R * 4, "input tokens");
+  treeRows_ = shared(R * sizeof(AttentionTreeRow), "tree rows");
+  depths_ = shared(R * 4, "row depths");
+  uniforms_ = shared(R * 8, "uniforms");
+  tokens_ = shared(R * 4, "selected tokens");
+  retained_ = shared(maxLanes * 4, "retained");
+  acceptedCount_ = shared(maxLanes * 4, "accepted");
+  retainedRows_ = shared(maxLanes * 4, "retained rows");
+  pageTable_ = device(uint64_t{pageTableEntries} * 8, "page table");
+  layerBytes_ = pageBytes_ * physicalPages;
+  kvAll_ = device(layerBytes_ * d.attentionLayers(), "kv pools");
+  for (uint32_t l = 0; l < d.attentionLayers(); ++l) kvPools_.push_back(backend.view(kvAll_, layerBytes_ * l, layerBytes_));
+  // Recurrent state: two cells and two tapes a lane.
+  const ops::GdnShape gdn = d.gdnShape();
+  strides_ = ops::GdnStateStrides::of(gdn, d.gdnLayers());
+  cellBytes_ = strides_.cellBytes(d.gdnLayers());
+  tapeLayerBytes_ = ops::gdnTapeLayerBytes(gdn);
+  states_ = device(cellBytes_ * 2 * maxLanes, "GDN state cells");
+  tape_ = device(tapeLayerBytes_ * d.gdnLayers() * 2 * maxLanes, "GDN tapes");
+  // Scratch of every dense projection at a piece's most rows.
+  const uint32_t pieceRows = std::min(maxRows_, kProjectionRows);
+  ops::LinearScratchSize size;
+  for (ops::LinearMatrix m : {ops::LinearMatrix{d.qkvWidth(), d.hidden}, ops::LinearMatrix{d.hidden, d.attentionWidth()},
+                              ops::LinearMatrix{d.gdnPackedWidth, d.hidden}, ops::LinearMatrix{d.hidden, d.gdnWidth()},
+                              ops::LinearMatrix{d.experts, d.hidden}, ops::LinearMatrix{d.vocabulary, d.hidden}})
+    size.include(linear_.scratchSize(m, pieceRows));
+  scratch_.input = device(size.input, "linear table");
+  scratch_.partials = device(size.partials, "linear partials");
+  scratch_.counters = device(std::max<uint64_t>(size.counters, 4), "linear counters");
+  const uint64_t fused = uint64_t{maxLanes} * d.kvHeads * (d.qHeads / std::max(1u, d.kvHeads)) * 16;
+  attentionWorkspace_.queries = device(fused * d.headDimension * 2, "staged queries");
+  attentionWorkspace_.querySums = device(fused * 4, "query sums");
+  attentionWorkspace_.partials = device(fused * ATTENTION_MAXIMUM_SPLITS * d.headDimension * 4, "attention partials");
+  attentionWorkspace_.partialSums = device(fused * ATTENTION_MAXIMUM_SPLITS * 8, "attention partial sums");
+  const ops::MoeWorkspaceSize moe = ops::MoE::workspace(d.moeShape(), maxRows_);
+  moeWorkspace_ = {device(moe.selected, "moe selected"),    device(moe.weights, "moe weights"),     device(moe.routeSlot, "moe route slots"),
+                   device(moe.slotRow, "moe slot rows"),    device(moe.tileExpert, "moe tile experts"), device(moe.tileRows, "moe tile rows"),
+                   device(moe.tileTotal, "moe tile count"), device(moe.tables, "moe tables"),       device(moe.nextTables, "moe SwiGLU tables"),
+                   device(moe.intermediate, "moe SwiGLU rows"), device(moe.expertOutput, "moe expert outputs")};
+  const ops::SamplingWorkspaceSize s = ops::Sampling::workspace(maxRows_);
+  sampling_.logits = logits_;
+  sampling_.tokens = tokens_;
+  sampling_.partialValues = device(s.partialValues, "argmax values");
+  sampling_.partialIndices = device(s.partialIndices, "argmax indices");
+  sampling_.masses = device(s.masses, "sampling masses");
+  sampling_.ranges = device(s.ranges, "sampling ranges");
+  sampling_.decisions = device(s.decisions, "sampling decisions");
+  sampling_.uniforms = uniforms_;
+  sampling_.inputTokens = inputTokens_;
+  sampling_.treeRows = treeRows_;
+}
+
+const hip::Buffer &HybridVerify::draftProbabilities() {
+  if (!draft_) {
+    draft_ = backend_.allocateBuffer(uint64_t{maxRows_} * dims_.vocabulary * 4, BufferStorage::Private, "draft probabilities");
+    sampling_.draftProbabilities = draft_;
+  }
+  return draft_;
+}
+
+uint64_t HybridVerify::stepBytes(const std::vector<HybridLane> &lanes) const {
+  const ops::MoeShape moe = dims_.moeShape();
+  uint64_t bytes = weights_.head.weightBytes();
+  for (const HybridLayer &l : weights_.layers) {
+    bytes += l.mixerInput.weightBytes() + l.mixerOutput.weightBytes() + l.router.weightBytes();
+    bytes += uint64_t{moe.experts} * (2 * gguf_image_bytes(l.experts.format, moe.ffn, moe.hidden) +
+                                      gguf_image_bytes(l.experts.downFormat, moe.hidden, moe.ffn));
+  }
+  uint32_t rows = 0;
+  for (const HybridLane &lane : lanes) {
+    bytes += uint64_t{dims_.attentionLayers()} * (uint64_t{lane.block.committed} + lane.block.rows) * (pageBytes_ / ATTENTION_PAGE_TOKENS);
+    bytes += 2ull * dims_.gdnLayers() * strides_.recurrentLayerBytes;  // each state read, and written
+    rows += lane.block.rows;
+  }
+  return bytes + 2ull * rows * dims_.vocabulary * 4;
+}
+
+ops::AttentionPlan HybridVerify::planOf(const std::vector<HybridLane> &lanes) const {
+  std::vector<ops::AttentionRows> sequences;
+  uint32_t rows = 0;
+  for (const HybridLane &lane : lanes) {
+    sequences.push_back({rows, lane.block.rows, lane.block.committed, lane.block.tableFirst});
+    rows += lane.block.rows;
+  }
+  return ops::PagedAttention::plan({dims_.qHeads, dims_.kvHeads, dims_.headDimension, dims_.rotaryPairs, dims_.normalizeHeads}, sequences);
+}
+
+void HybridVerify::encodeEmbedding(hip::CommandGraph &graph, uint32_t rows) {
+  ops::Embedding::add(graph, weights_.embedding, inputTokens_, hidden_[0], rows);
+}
+
+void HybridVerify::encodeLayer(hip::CommandGraph &graph, uint32_t layer, const std::vector<HybridLane> &lanes) {
+  if (lanes.empty() || lanes.size() > maxLanes_) throw std::invalid_argument("the step takes 1 to its most lanes");
+  const HybridLayer &w = weights_.layers.at(layer);
+  const bool attends = dims_.attends(layer);
+  const uint32_t index = dims_.mixerIndex(layer);
+  uint32_t rows = 0;
+  for (const HybridLane &lane : lanes) rows += lane.block.rows;
+  if (rows > maxRows_) throw std::invalid_argument("more rows than the step's buffers hold");
+  const hip::Buffer &residual = hidden_[0], &next = hidden_[1];
+  const uint64_t hiddenBytes = uint64_t{dims_.hidden} * 2;
+  const uint32_t inputWidth = w.mixerInput.outputSize, mixedWidth = w.mixerOutput.inputSize;
+  if (inputWidth != (attends ? dims_.qkvWidth() : dims_.gdnPackedWidth) || mixedWidth != (attends ? dims_.attentionWidth() : dims_.gdnWidth()) ||
+      w.mixerInput.inputSize != dims_.hidden || w.mixerOutput.outputSize != dims_.hidden || w.router.outputSize != dims_.experts ||
+      w.router.inputSize != dims_.hidden)
+    throw std::invalid_argument("the layer's projections do not fit the model");
+
+  // Mixer: hidden[1] = hidden[0] + out(mixer(in(norm(hidden[0])))).
+  forRowPieces(rows, [&](uint32_t first, uint32_t count) {
+    const hip::Buffer normalized = rowsOf(normalized_, first, count, hiddenBytes);
+    ops::LinearBuffers in;
+    in.input = normalized;
+    in.output = rowsOf(packed_, first, count, uint64_t{inputWidth} * 2);
+    in.scratch = scratch_;
+    in.prepared = ops::Normalization::addRmsTable(graph, rowsOf(residual, first, count, hiddenBytes), w.inputNorm, normalized, scratch_,
+                                                  dims_.hidden, count);
+    linear_.add(graph, in, w.mixerInput, linear_.plan(w.mixerInput, count));
+  });
+  if (attends) {
+    const ops::AttentionPlan plan = planOf(lanes);
+    const ops::KvPages pages{pageTable_, kvPools_.at(index), pageBytes_};
+    ops::PagedAttention::addProjection(graph, plan, {packed_, w.queryNorm, w.keyNorm, ropeCos_, ropeSin_}, attentionWorkspace_, pages);
+    ops::PagedAttention::addAttention(graph, plan, attentionWorkspace_, treeRows_, pages, mixed_, {});
+  } else {
+    std::vector<ops::GdnLaneStep> steps;
+    uint32_t firstRow = 0;
+    for (size_t i = 0; i < lanes.size(); ++i) {
+      const HybridLane &lane = lanes[i];
+      steps.push_back({firstRow, lane.block.rows, lane.pendingPath, tapeOffset(uint32_t(i), lane.parity ^ 1u, index),
+                       tapeOffset(uint32_t(i), lane.parity, index), cellOffset(uint32_t(i), lane.parity), cellOffset(uint32_t(i), lane.parity ^ 1u)});
+      firstRow += lane.block.rows;
+    }
+    ops::GdnDecodeBuffers buffers{packed_, w.convolutionWeights, states_, tape_, w.decay, w.timeBias, w.mixerNorm, false, mixed_, treeRows_};
+    ops::GDN::addDecode(graph, buffers, dims_.gdnShape(), index, strides_, ops::GdnHeadOrder::Grouped, steps);
+  }
+  forRowPieces(rows, [&](uint32_t first, uint32_t count) {
+    linear_.addResidualProjection(graph, rowsOf(mixed_, first, count, uint64_t{mixedWidth} * 2), w.mixerOutput,
+                                  rowsOf(residual, first, count, hiddenBytes), rowsOf(next, first, count, hiddenBytes), count, scratch_);
+  });
+
+  // FFN: hidden[0] = hidden[1] + sum over a row's experts of weight * expert(norm(hidden[1])).
+  forRowPieces(rows, [&](uint32_t first, uint32_t count) {
+    const hip::Buffer normalized = rowsOf(normalized_, first, count, hiddenBytes);
+    ops::LinearBuffers router;
+    router.input = normalized;
+    router.output = rowsOf(scores_, first, count, uint64_t{dims_.experts} * 4);
+    router.scratch = scratch_;
+    router.prepared = ops::Normalization::addRmsTable(graph, rowsOf(next, first, count, hiddenBytes), w.postNorm, normalized, scratch_,
+                                                      dims_.hidden, count);
+    linear_.add(graph, router, w.router, linear_.plan(w.router, count));
+  });
+  const ops::MoeShape moe = dims_.moeShape();
+  ops::MoE::addRouting(graph, scores_, dims_.experts, moeWorkspace_, moe, rows);
+  ops::MoE::addRouted(graph, normalized_, next, residual, w.experts, moeWorkspace_, moe, rows);
+}
+
+void HybridVerify::encodeHead(hip::CommandGraph &graph, uint32_t rows) {
+  const uint64_t hiddenBytes = uint64_t{dims_.hidden} * 2;
+  forRowPieces(rows, [&](uint32_t first, uint32_t count) {
+    const hip::Buffer normalized = rowsOf(normalized_, first, count, hiddenBytes);
+    ops::LinearBuffers head;
+    head.input = normalized;
+    head.output = rowsOf(logits_, first, count, uint64_t{dims_.vocabulary} * 4);
+    head.scratch = scratch_;
+    head.prepared = ops::Normalization::addRmsTable(graph, rowsOf(hidden_[0], first, count, hiddenBytes), weights_.finalNorm, normalized,
+                                                    scratch_, dims_.hidden, count);
+    linear_.add(graph, head, weights_.head, linear_.plan(weights_.head, count));
+  });
+}
+
+void HybridVerify::encode(hip::CommandGraph &graph, const std::vector<HybridLane> &lanes, bool commit) {
+  if (lanes.empty() || lanes.size() > maxLanes_) throw std::invalid_argument("the step takes 1 to its most lanes");
+  std::vector<ops::LaneRows> laneRows;
+  std::vector<ops::RopeSequence> rope;
+  std::vector<ops::SamplingPolicy> policies;
+  std::vector<uint32_t> remaining;
+  uint32_t rows = 0;
+  bool samples = false;
+  for (const HybridLane &lane : lanes) {
+    laneRows.push_back({rows, lane.block.rows});
+    rope.push_back({rows, lane.block.rows, lane.block.committed});
+    policies.push_back(lane.block.policy);
+    remaining.push_back(lane.block.remaining);
+    samples = samples || lane.block.policy.samples();
+    rows += lane.block.rows;
+  }
+  if (samples) (void)draftProbabilities();
+  if (dims_.rotaryPairs)
+    ops::RoPE::addTreeTables(graph, inverseFrequency_, depths_, ropeCos_, ropeSin_, dims_.rotaryPairs, rope);
+  encodeEmbedding(graph, rows);
+  for (uint32_t layer = 0; layer < dims_.layers; ++layer) encodeLayer(graph, layer, lanes);
+  encodeHead(graph, rows);
+  ops::Sampling::addVerify(graph, sampling_, dims_.vocabulary, dims_.vocabulary, laneRows, policies);
+  const ops::AcceptanceBuffers acceptance{inputTokens_, treeRows_, tokens_, retained_, acceptedCount_, retainedRows_};
+  ops::Sampling::addAcceptance(graph, acceptance, laneRows, remaining,
+                               {SAMPLING_NO_TOKEN, SAMPLING_NO_TOKEN, SAMPLING_NO_TOKEN, SAMPLING_NO_TOKEN});
+  if (commit && dims_.attentionLayers())
+    ops::PagedAttention::addPathCommit(graph, planOf(lanes), retainedRows_, {pageTable_, kvAll_, pageBytes_}, dims_.attentionLayers(),
+                                       layerBytes_);
+}
+
+} // namespace splash::model

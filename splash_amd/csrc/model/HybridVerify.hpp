@@ -1,0 +1,154 @@
+// The target part of one speculative-decoding cycle for a hybrid mixture-of-experts decoder
+// (the reference's Qwen3.5 family with Gated DeltaNet mixers and a MoE FFN, model/QwenTarget.cpp:
+// 206-255 the GDN mixer, :263-347 the attention mixer, :372-395 the MoE routing, :457-496 the layer
+// recipe; Runtime.cpp:2701-2707 the tape parity and pending path): embedding -> N x {RMSNorm ->
+// mixer input projection -> [GDN decode | q/k norm + RoPE + INT8 store + paged attention] ->
+// output projection + residual -> RMSNorm -> router -> top-k routing -> routed experts + combine}
+// -> final norm -> LM head -> verify -> acceptance -> KV path commit. Every fourth layer attends,
+// the others run Gated DeltaNet.
+//
+// A lane's recurrent state is never rolled back: a step writes the state BEFORE its rows and leaves
+// its rows on the lane's tape, and the lane's next step folds the accepted path (the acceptance's
+// retained-rows mask, which its caller hands back as `pendingPath`) first. Cells and tapes are
+// double-buffered by the lane's step parity.
+#pragma once
+#include "hip/Backend.hpp"
+#include "model/DenseVerify.hpp"
+#include "ops/Gdn.hpp"
+#include "ops/Glue.hpp"
+#include "ops/Linear.hpp"
+#include "ops/Moe.hpp"
+#include "ops/PagedAttention.hpp"
+#include "ops/Sampling.hpp"
+
+#include <cstdint>
+#include <vector>
+
+namespace splash::model {
+
+struct HybridDimensions final {
+  uint32_t hidden = 0, vocabulary = 0, layers = 0;
+  uint32_t attentionInterval = 4;  // layer l attends when (l + 1) % attentionInterval == 0
+  uint32_t qHeads = 0, kvHeads = 0, headDimension = 0, rotaryPairs = 0;
+  bool normalizeHeads = true;
+  float ropeTheta = 1000000.0f;
+  uint32_t gdnKeyHeads = 0, gdnValueHeads = 0;
+  uint32_t gdnPackedWidth = 0;  // the GDN input projection's width (whole column tiles)
+  uint32_t experts = 0, topK = 0, expertFfn = 0;
+
+  [[nodiscard]] bool attends(uint32_t layer) const noexcept { return (layer + 1) % attentionInterval == 0; }
+  [[nodiscard]] uint32_t attentionLayers() const noexcept { return layers / attentionInterval; }
+  [[nodiscard]] uint32_t gdnLayers() const noexcept { return layers - attentionLayers(); }
+  // The layer's place among the layers of its kind.
+  [[nodiscard]] uint32_t mixerIndex(uint32_t layer) const noexcept {
+    const uint32_t before = layer / attentionInterval;  // attention layers before it
+    return attends(layer) ? before : layer - before;
+  }
+  [[nodiscard]] uint32_t qkvWidth() const noexcept { return (qHeads + 2 * kvHeads) * headDimension; }
+  [[nodiscard]] uint32_t attentionWidth() const noexcept { return qHeads * headDimension; }
+  [[nodiscard]] uint32_t gdnWidth() const noexcept { return gdnValueHeads * GDN_HEAD_DIMENSION; }
+  [[nodiscard]] ops::GdnShape gdnShape() const noexcept {
+    ops::GdnShape s;
+    s.keyHeads = gdnKeyHeads;
+    s.valueHeads = gdnValueHeads;
+    s.convolutionDimension = (2 * gdnKeyHeads + gdnValueHeads) * GDN_HEAD_DIMENSION;
+    s.packedWidth = gdnPackedWidth;
+    return s;
+  }
+  [[nodiscard]] ops::MoeShape moeShape() const noexcept { return {hidden, expertFfn, experts, topK}; }
+};
+
+struct HybridLayer final {
+  // q|k|v -> o of an attention layer; the packed row [q|k|v|z|b|a] -> out of a GDN layer
+  ops::Projection mixerInput, mixerOutput;
+  hip::Buffer inputNorm, postNorm;                                  // bf16 [hidden]
+  hip::Buffer queryNorm, keyNorm;                                   // attention layers: bf16 [head dimension]
+  hip::Buffer convolutionWeights, decay, timeBias, mixerNorm;       // GDN layers (mixerNorm bf16 [128])
+  ops::Projection router;                                           // hidden -> experts, fp32 scores
+  ops::MoeExperts experts;
+};
+
+struct HybridWeights final {
+  ops::EmbeddingTable embedding;
+  std::vector<HybridLayer> layers;
+  hip::Buffer finalNorm;
+  ops::Projection head;
+};
+
+// One lane of a step: its verify block, and what its previous step left.
+struct HybridLane final {
+  VerifyLane block;
+  uint32_t pendingPath = 0;  // rows of its previous step it accepted (that step's retained-rows mask)
+  // A step of parity p reads the lane's cell p and writes cell p ^ 1; its rows go to tape p and its
+  // pending rows are on tape p ^ 1. The lane's next step has parity p ^ 1.
+  uint32_t parity = 0;
+};
+
+class HybridVerify final {
+public:
+  HybridVerify(hip::Backend &backend, HybridDimensions dimensions, uint32_t maxLanes, uint32_t physicalPages,
+               uint32_t pageTableEntries);
+
+  [[nodiscard]] const HybridDimensions &dimensions() const noexcept { return dims_; }
+  HybridWeights &weights() noexcept { return weights_; }
+  [[nodiscard]] const hip::Buffer &inputTokens() const noexcept { return inputTokens_; }
+  [[nodiscard]] const hip::Buffer &treeRows() const noexcept { return treeRows_; }
+  [[nodiscard]] const hip::Buffer &depths() const noexcept { return depths_; }
+  [[nodiscard]] const hip::Buffer &uniforms() const noexcept { return uniforms_; }
+  [[nodiscard]] const hip::Buffer &tokens() const noexcept { return tokens_; }
+  [[nodiscard]] const hip::Buffer &retained() const noexcept { return retained_; }
+  [[nodiscard]] const hip::Buffer &acceptedCount() const noexcept { return acceptedCount_; }
+  [[nodiscard]] const hip::Buffer &retainedRows() const noexcept { return retainedRows_; }
+  [[nodiscard]] const hip::Buffer &pageTable() const noexcept { return pageTable_; }
+  [[nodiscard]] const hip::Buffer &kvPool(uint32_t attentionLayer) const { return kvPools_.at(attentionLayer); }
+  [[nodiscard]] const hip::Buffer &logits() const noexcept { return logits_; }
+  [[nodiscard]] const hip::Buffer &draftProbabilities();
+  [[nodiscard]] const hip::Buffer &hidden(uint32_t index) const noexcept { return hidden_[index & 1]; }
+  [[nodiscard]] const hip::Buffer &gdnStates() const noexcept { return states_; }
+  [[nodiscard]] const hip::Buffer &gdnTape() const noexcept { return tape_; }
+  [[nodiscard]] uint64_t pageBytes() const noexcept { return pageBytes_; }
+  [[nodiscard]] const ops::GdnStateStrides &gdnStrides() const noexcept { return strides_; }
+  [[nodiscard]] uint64_t gdnCellBytes() const noexcept { return cellBytes_; }
+  [[nodiscard]] uint64_t gdnTapeLayerBytes() const noexcept { return tapeLayerBytes_; }
+  // Where lane `lane` keeps the cell and the tapes of a step of parity `parity`: the step reads the
+  // cell of its parity and writes the other one; its tape is its parity's, its pending tape the other's.
+  [[nodiscard]] uint64_t cellOffset(uint32_t lane, uint32_t parity) const noexcept { return (uint64_t{lane} * 2 + (parity & 1)) * cellBytes_; }
+  [[nodiscard]] uint64_t tapeOffset(uint32_t lane, uint32_t parity, uint32_t gdnLayer) const noexcept {
+    return ((uint64_t{lane} * 2 + (parity & 1)) * dims_.gdnLayers() + gdnLayer) * tapeLayerBytes_;
+  }
+  // Algorithmic bytes one step streams from HBM: dense weights once, every expert of every layer
+  // once (a batch of 8 x 16 rows routes to all of them), each lane's KV and recurrent states
+  // (read and written), the logits.
+  [[nodiscard]] uint64_t stepBytes(const std::vector<HybridLane> &lanes) const;
+
+  void encode(hip::CommandGraph &graph, const std::vector<HybridLane> &lanes, bool commit = true);
+  void encodeEmbedding(hip::CommandGraph &graph, uint32_t rows);
+  void encodeLayer(hip::CommandGraph &graph, uint32_t layer, const std::vector<HybridLane> &lanes);
+  void encodeHead(hip::CommandGraph &graph, uint32_t rows);
+
+private:
+  [[nodiscard]] ops::AttentionPlan planOf(const std::vector<HybridLane> &lanes) const;
+  [[nodiscard]] hip::Buffer rowsOf(const hip::Buffer &buffer, uint32_t first, uint32_t count, uint64_t rowBytes) const {
+    return backend_.view(buffer, first * rowBytes, count * rowBytes);
+  }
+
+  hip::Backend &backend_;
+  HybridDimensions dims_;
+  HybridWeights weights_;
+  ops::Linear linear_;
+  uint32_t maxRows_ = 0, maxLanes_ = 0;
+  uint64_t pageBytes_ = 0, layerBytes_ = 0, cellBytes_ = 0, tapeLayerBytes_ = 0;
+  ops::GdnStateStrides strides_;
+  hip::Buffer kvAll_, states_, tape_;
+  hip::Buffer hidden_[2], normalized_, packed_, mixed_, scores_, logits_, draft_;
+  hip::Buffer inverseFrequency_, ropeCos_, ropeSin_;
+  hip::Buffer inputTokens_, treeRows_, depths_, uniforms_, tokens_, retained_, acceptedCount_, retainedRows_;
+  hip::Buffer pageTable_;
+  std::vector<hip::Buffer> kvPools_;
+  ops::LinearScratch scratch_;
+  ops::AttentionWorkspace attentionWorkspace_;
+  ops::MoeWorkspace moeWorkspace_;
+  ops::SamplingBuffers sampling_;
+};
+
+} // namespace splash::model

@@ -1,5 +1,5 @@
-"""The dense verify step (model::DenseVerify), bound through include/splash_ops.h: the target part of
-one speculative-decoding cycle, as the reference's Runtime::decodeAsync encodes it
+"""The verify step's drivers (model::DenseVerify, model::HybridVerify), bound through include/splash_ops.h: the
+target part of one speculative-decoding cycle, as the reference's Runtime::decodeAsync encodes it
 (runtime/model/Runtime.cpp:3985-3993)."""
 import ctypes
 
@@ -11,7 +11,7 @@ from .backend import Buffer, CommandGraph, STORAGE_PRIVATE
 from . import ops
 
 (INPUT_TOKENS, TREE_ROWS, DEPTHS, UNIFORMS, TOKENS, RETAINED, ACCEPTED, RETAINED_ROWS, PAGE_TABLE, KV_POOL, LOGITS,
- DRAFT_PROBABILITIES, HIDDEN) = range(13)
+ DRAFT_PROBABILITIES, HIDDEN, GDN_STATES, GDN_TAPE) = range(15)
 
 
 class Lane:
@@ -96,3 +96,101 @@ class DenseVerify:
         n = len(lanes)
         rd = lambda which, count: self.buffer(which).contents()[:count * 4].view(np.uint32).copy()
         return rd(TOKENS, rows), rd(RETAINED, n), rd(ACCEPTED, n), rd(RETAINED_ROWS, n)
+
+
+class HybridLane(Lane):
+    """A lane of a hybrid step: its block, the rows of its previous step it accepted, and the step's parity (a step
+    reads the lane's state cell `parity` and writes the other; the lane's next step flips it)."""
+
+    def __init__(self, rows, committed, table_first=0, temperature=0.0, remaining=0xFFFFFFFF, pending_path=0, parity=0):
+        super().__init__(rows, committed, table_first, temperature, remaining)
+        self.pending_path, self.parity = pending_path, parity
+
+    def struct(self):
+        return nat.HybridLane(super().struct(), self.pending_path, self.parity)
+
+
+class HybridVerify:
+    """model::HybridVerify: Gated DeltaNet and attention mixers (every `attention_interval`-th layer attends) over a
+    mixture-of-experts FFN."""
+
+    def __init__(self, backend, hidden, vocabulary, layers, q_heads, kv_heads, head_dim, gdn_key_heads, gdn_value_heads, experts, top_k,
+                 expert_ffn, attention_interval=4, rotary_pairs=None, normalize_heads=True, rope_theta=1e6, gdn_packed_width=None,
+                 max_lanes=1, physical_pages=2, page_table_entries=None):
+        self.backend = backend
+        pairs = head_dim // 2 if rotary_pairs is None else rotary_pairs
+        conv = (2 * gdn_key_heads + gdn_value_heads) * 128
+        packed = gdn_packed_width or (conv + gdn_value_heads * 128 + 2 * gdn_value_heads + 15) // 16 * 16
+        self.dims = nat.HybridDimensions(hidden, vocabulary, layers, attention_interval, q_heads, kv_heads, head_dim, pairs,
+                                         int(normalize_heads), rope_theta, gdn_key_heads, gdn_value_heads, packed, experts, top_k, expert_ffn)
+        h = ctypes.c_void_p()
+        entries = page_table_entries if page_table_entries is not None else physical_pages
+        check(lib.spo_hybrid_verify_create(backend.handle, ctypes.byref(self.dims), max_lanes, physical_pages, entries, ctypes.byref(h)))
+        self.handle = h
+        self.physical_pages = physical_pages
+        page, cell, tape = ctypes.c_uint64(), ctypes.c_uint64(), ctypes.c_uint64()
+        self.strides = nat.GdnStateStrides()
+        check(lib.spo_hybrid_verify_layout(h, ctypes.byref(page), ctypes.byref(cell), ctypes.byref(tape), ctypes.byref(self.strides)))
+        self.page_bytes, self.cell_bytes, self.tape_layer_bytes = page.value, cell.value, tape.value
+        self.gdn_layers = layers - layers // attention_interval
+        self._keep = []
+
+    def __del__(self):
+        try:
+            lib.spo_hybrid_verify_destroy(self.handle)
+        except Exception:
+            pass
+
+    def attends(self, layer):
+        return (layer + 1) % self.dims.attention_interval == 0
+
+    def mixer_index(self, layer):
+        before = layer // self.dims.attention_interval
+        return before if self.attends(layer) else layer - before
+
+    def cell_offset(self, lane, parity):
+        return (lane * 2 + (parity & 1)) * self.cell_bytes
+
+    def tape_offset(self, lane, parity, gdn_layer):
+        return ((lane * 2 + (parity & 1)) * self.gdn_layers + gdn_layer) * self.tape_layer_bytes
+
+    def buffer(self, which, index=0):
+        out = ctypes.c_void_p()
+        check(lib.spo_hybrid_verify_buffer(self.handle, which, index, ctypes.byref(out)))
+        return Buffer(out.value)
+
+    def set_layer(self, layer, mixer_input, mixer_output, input_norm, post_norm, router, gate_images, up_images, down_images,
+                  query_norm=None, key_norm=None, convolution_weights=None, decay_weights=None, time_bias=None, mixer_norm=None,
+                  expert_format=ops.FMT_Q4K, expert_down_format=ops.FMT_Q4K):
+        handle = lambda b: b.handle if b is not None else None
+        w = nat.HybridLayer(mixer_input.handle, mixer_output.handle, handle(input_norm), handle(post_norm), handle(query_norm),
+                            handle(key_norm), handle(convolution_weights), handle(decay_weights), handle(time_bias), handle(mixer_norm),
+                            router.handle, handle(gate_images), handle(up_images), handle(down_images), expert_format, expert_down_format)
+        check(lib.spo_hybrid_verify_set_layer(self.handle, layer, ctypes.byref(w)))
+        self._keep.extend([mixer_input, mixer_output, input_norm, post_norm, router, gate_images, up_images, down_images, query_norm,
+                           key_norm, convolution_weights, decay_weights, time_bias, mixer_norm])
+
+    def set_head(self, embedding_format, embedding_rows, final_norm, head):
+        check(lib.spo_hybrid_verify_set_head(self.handle, embedding_format, embedding_rows.handle, final_norm.handle, head.handle))
+        self._keep.extend([embedding_rows, final_norm, head])
+
+    def _lanes(self, lanes):
+        return (nat.HybridLane * len(lanes))(*[l.struct() for l in lanes])
+
+    def step_bytes(self, lanes):
+        return lib.spo_hybrid_verify_step_bytes(self.handle, self._lanes(lanes), len(lanes))
+
+    def encode(self, lanes, commit=True, graph=None):
+        graph = graph or CommandGraph()
+        check(lib.spo_hybrid_verify_encode(self.handle, graph.handle, self._lanes(lanes), len(lanes), int(commit)))
+        graph._keep.append(self)
+        return graph
+
+    def encode_part(self, part, index, lanes, graph=None):
+        graph = graph or CommandGraph()
+        check(lib.spo_hybrid_verify_encode_part(self.handle, graph.handle, part, index, self._lanes(lanes), len(lanes)))
+        graph._keep.append(self)
+        return graph
+
+    set_block = DenseVerify.set_block
+    results = DenseVerify.results

@@ -1,0 +1,198 @@
+"""A random-init hybrid decoder (Gated DeltaNet and attention mixers over a mixture-of-experts FFN) for the
+parity tests: its weights, the GPU model built from them, and the oracle's evaluation of each layer.
+Test infrastructure only."""
+import numpy as np
+
+from splash_amd import ops, verify
+from tests import oracle as orc
+
+
+class HybridModel:
+    def __init__(self, seed, hidden, vocabulary, layers, q_heads, kv_heads, head_dim, gdn_key_heads, gdn_value_heads, experts, top_k,
+                 expert_ffn, attention_interval=4, rope_theta=1e6):
+        self.dims = dict(hidden=hidden, vocabulary=vocabulary, layers=layers, q_heads=q_heads, kv_heads=kv_heads, head_dim=head_dim,
+                         gdn_key_heads=gdn_key_heads, gdn_value_heads=gdn_value_heads, experts=experts, top_k=top_k, expert_ffn=expert_ffn,
+                         attention_interval=attention_interval)
+        self.rope_theta = rope_theta
+        rng = np.random.default_rng(seed)
+        self.rng = rng
+        D = head_dim
+        conv = (2 * gdn_key_heads + gdn_value_heads) * 128
+        self.packed_width = (conv + gdn_value_heads * 128 + 2 * gdn_value_heads + 15) // 16 * 16
+        self.gdn_shape = orc.gdn_shape(gdn_key_heads, gdn_value_heads, packed_width=self.packed_width)
+
+        def quant(n, k, fmt=orc.FMT_Q4K, scale=0.02):
+            return orc.quantize_rows(fmt, (rng.standard_normal((n, k)) * scale).astype(np.float32))
+
+        def norm(n):
+            return orc.f32_to_bf16((1 + 0.1 * rng.standard_normal(n)).astype(np.float32))
+        self.layers = []
+        for l in range(layers):
+            w = dict(input_norm=norm(hidden), post_norm=norm(hidden), router=quant(experts, hidden, orc.FMT_Q6K, 0.05),
+                     gate=[quant(expert_ffn, hidden) for _ in range(experts)], up=[quant(expert_ffn, hidden) for _ in range(experts)],
+                     down=[quant(hidden, expert_ffn) for _ in range(experts)])
+            if self.attends(l):
+                w.update(q=quant(q_heads * D, hidden), k=quant(kv_heads * D, hidden), v=quant(kv_heads * D, hidden),
+                         o=quant(hidden, q_heads * D), q_norm=norm(D), k_norm=norm(D))
+            else:
+                # a wider spread than a dense projection's, so that the recurrence's inputs are of order one
+                w.update(mixer_in=quant(self.packed_width, hidden, scale=0.06), mixer_out=quant(hidden, gdn_value_heads * 128),
+                         conv_w=orc.f32_to_bf16((rng.standard_normal((conv, 4)) * 0.4).astype(np.float32)),
+                         a_scale=(-np.exp(rng.uniform(-1.0, 1.0, gdn_value_heads))).astype(np.float32),
+                         dt_bias=orc.f32_to_bf16(rng.uniform(-1.0, 1.0, gdn_value_heads).astype(np.float32)), mixer_norm=norm(128))
+            self.layers.append(w)
+        self.embedding = quant(vocabulary, hidden)
+        self.final_norm = norm(hidden)
+        self.head = quant(vocabulary, hidden, orc.FMT_Q6K)
+
+    def attends(self, layer):
+        return (layer + 1) % self.dims["attention_interval"] == 0
+
+    # ------------------------------------------------------------------ GPU side
+    def build_gpu(self, backend, max_lanes, pages_per_lane):
+        d = self.dims
+        self.pages_per_lane = pages_per_lane
+        self.physical_pages = max_lanes * pages_per_lane + 1
+        gpu = verify.HybridVerify(backend, d["hidden"], d["vocabulary"], d["layers"], d["q_heads"], d["kv_heads"], d["head_dim"],
+                                  d["gdn_key_heads"], d["gdn_value_heads"], d["experts"], d["top_k"], d["expert_ffn"],
+                                  attention_interval=d["attention_interval"], rope_theta=self.rope_theta, max_lanes=max_lanes,
+                                  physical_pages=self.physical_pages, page_table_entries=max_lanes * pages_per_lane)
+        assert gpu.dims.gdn_packed_width == self.packed_width
+        self.table = np.random.default_rng(99).permutation(self.physical_pages)[:max_lanes * pages_per_lane].astype(np.uint64)
+        gpu.buffer(verify.PAGE_TABLE).upload(self.table)
+        D, H, F = d["head_dim"], d["hidden"], d["expert_ffn"]
+        P = lambda segs, k, f32=False: ops.Projection.from_native(backend, segs, k, float32=f32)
+        images = lambda fmt, natives, n, k: backend.from_array(np.concatenate([ops.pack_gguf_image(fmt, x, n, k) for x in natives]))
+        for i, w in enumerate(self.layers):
+            common = dict(input_norm=backend.from_array(w["input_norm"]), post_norm=backend.from_array(w["post_norm"]),
+                          router=P([(orc.FMT_Q6K, d["experts"], w["router"])], H, True), gate_images=images(orc.FMT_Q4K, w["gate"], F, H),
+                          up_images=images(orc.FMT_Q4K, w["up"], F, H), down_images=images(orc.FMT_Q4K, w["down"], H, F))
+            if self.attends(i):
+                gpu.set_layer(i, P([(orc.FMT_Q4K, d["q_heads"] * D, w["q"]), (orc.FMT_Q4K, d["kv_heads"] * D, w["k"]),
+                                    (orc.FMT_Q4K, d["kv_heads"] * D, w["v"])], H), P([(orc.FMT_Q4K, H, w["o"])], d["q_heads"] * D),
+                              query_norm=backend.from_array(w["q_norm"]), key_norm=backend.from_array(w["k_norm"]), **common)
+            else:
+                gpu.set_layer(i, P([(orc.FMT_Q4K, self.packed_width, w["mixer_in"])], H),
+                              P([(orc.FMT_Q4K, H, w["mixer_out"])], d["gdn_value_heads"] * 128),
+                              convolution_weights=backend.from_array(w["conv_w"]), decay_weights=backend.from_array(w["a_scale"]),
+                              time_bias=backend.from_array(w["dt_bias"]), mixer_norm=backend.from_array(w["mixer_norm"]), **common)
+        gpu.set_head(orc.FMT_Q4K, backend.from_array(self.embedding), backend.from_array(self.final_norm),
+                     P([(orc.FMT_Q6K, d["vocabulary"], self.head)], H, True))
+        self.gpu = gpu
+        return gpu
+
+    def seed_context(self, rng):
+        """A seeded INT8 context in every physical page of every attention layer."""
+        d, gpu = self.dims, self.gpu
+        H, D, PT = d["kv_heads"], d["head_dim"], ops.PAGE_TOKENS
+        helper = ops.KvPages.__new__(ops.KvPages)
+        helper.kv_heads, helper.head_dim, helper.page_bytes = H, D, gpu.page_bytes
+        self.context = []
+        for layer in range(d["layers"] // d["attention_interval"]):
+            def quant(x):
+                mx = np.abs(x).max(axis=-1, keepdims=True)
+                codes = np.clip(np.rint(x * np.float32(127.0) / mx), -127, 127).astype(np.int8)
+                return codes, (mx[..., 0] / np.float32(127.0)).astype(np.float16).astype(np.float32)
+            (kc, ks), (vc, vs) = (quant(rng.standard_normal((self.physical_pages, H, PT, D)).astype(np.float32)) for _ in range(2))
+            self.context.append([kc, ks, vc, vs])
+            gpu.buffer(verify.KV_POOL, layer).upload(helper.pack_pages(kc, ks, vc, vs))
+
+    def seed_states(self, rng, lanes, parity=0):
+        """Random recurrent states and convolution carries in every lane's cell of `parity`."""
+        gpu, shape = self.gpu, self.gdn_shape
+        states = gpu.buffer(verify.GDN_STATES)
+        for lane in range(lanes):
+            for g in range(gpu.gdn_layers):
+                conv = orc.f32_to_bf16(rng.standard_normal((3, shape.conv_dim)).astype(np.float32))
+                state = (rng.standard_normal((shape.value_heads, 128, 128)) * 0.05).astype(np.float32)
+                base = gpu.cell_offset(lane, parity)
+                states.upload(conv, base + g * gpu.strides.convolution_layer_bytes)
+                states.upload(state, base + gpu.strides.convolution_state_bytes + g * gpu.strides.recurrent_layer_bytes)
+
+    def read_cell(self, lane, parity, gdn_layer):
+        gpu, shape = self.gpu, self.gdn_shape
+        st = gpu.strides
+        raw = gpu.buffer(verify.GDN_STATES).download(np.uint8)
+        base = gpu.cell_offset(lane, parity)
+        conv = raw[base + gdn_layer * st.convolution_layer_bytes:][:3 * shape.conv_dim * 2].view(np.uint16).reshape(3, shape.conv_dim)
+        at = base + st.convolution_state_bytes + gdn_layer * st.recurrent_layer_bytes
+        return conv.copy(), raw[at:at + st.recurrent_layer_bytes].view(np.float32).reshape(shape.value_heads, 128, 128).copy()
+
+    def read_tape(self, lane, parity, gdn_layer):
+        gpu = self.gpu
+        raw = gpu.buffer(verify.GDN_TAPE).download(np.uint8)
+        return raw[gpu.tape_offset(lane, parity, gdn_layer):][:gpu.tape_layer_bytes].copy()
+
+    # ------------------------------------------------------------------ oracle side
+    def _project(self, fmt, native, x_bits, n):
+        return orc.gemm(fmt, native, x_bits, n, want=("exact",))["exact"]
+
+    def oracle_embedding(self, tokens):
+        return orc.embed(orc.FMT_Q4K, self.embedding, self.dims["vocabulary"], self.dims["hidden"], tokens)
+
+    def oracle_mixer_input(self, hidden, li):
+        w, d = self.layers[li], self.dims
+        n = orc.rms_norm(hidden, w["input_norm"])
+        if self.attends(li):
+            D = d["head_dim"]
+            out = np.concatenate([self._project(orc.FMT_Q4K, w[name], n, width) for name, width in
+                                  (("q", d["q_heads"] * D), ("k", d["kv_heads"] * D), ("v", d["kv_heads"] * D))], axis=1)
+        else:
+            out = self._project(orc.FMT_Q4K, w["mixer_in"], n, self.packed_width)
+        return orc.f32_to_bf16(out.astype(np.float32))
+
+    def oracle_attention(self, packed, li, lanes):
+        """Every lane's attention rows; stores the blocks' K/V into the layer's context arrays."""
+        d, w = self.dims, self.layers[li]
+        D, pairs = d["head_dim"], d["head_dim"] // 2
+        kc, ks, vc, vs = self.context[li // d["attention_interval"]]
+        inv = np.array([self.rope_theta ** (-i / pairs) for i in range(pairs)]).astype(np.float32)
+        out, first = [], 0
+        for lane in lanes:
+            rows, committed = lane.rows, lane.committed
+            table = self.table[lane.table_first:lane.table_first + self.pages_per_lane].astype(np.uint32)
+            pos = (committed + np.arange(rows)).astype(np.float32)
+            angle = (pos[:, None] * inv[None, :]).astype(np.float32)
+            cosv, sinv = np.cos(angle.astype(np.float64)).astype(np.float32), np.sin(angle.astype(np.float64)).astype(np.float32)
+            q, kf, vf = orc.attention_prepare(d["q_heads"], d["kv_heads"], D, packed[first:first + rows], w["q_norm"], w["k_norm"], cosv, sinv, pairs)
+            kcod, kscl = orc.kv_quantize(kf)
+            vcod, vscl = orc.kv_quantize(vf)
+            for r in range(rows):
+                t = committed + r
+                p, s = table[t // ops.PAGE_TOKENS], t % ops.PAGE_TOKENS
+                kc[p, :, s], ks[p, :, s], vc[p, :, s], vs[p, :, s] = kcod[r], kscl[r], vcod[r], vscl[r]
+            anc = np.array([(2 << r) - 1 for r in range(rows)], dtype=np.uint32)
+            attn, _ = orc.attention(q, kc, ks, vc, vs, table, anc, committed, want64=False)
+            out.append(attn.reshape(rows, d["q_heads"] * D))
+            first += rows
+        return np.concatenate(out)
+
+    def oracle_gdn(self, packed, li, lanes, cells, tapes):
+        """Every lane's GDN rows from its cell (conv, state) and pending tape; returns (rows, [(conv, state, tape)] it leaves)."""
+        w = self.layers[li]
+        out, left, first = [], [], 0
+        for lane, (conv_in, state_in), tape in zip(lanes, cells, tapes):
+            conv, state, step_tape, hidden = orc.gdn_decode(self.gdn_shape, packed[first:first + lane.rows], w["conv_w"], w["a_scale"], w["dt_bias"],
+                                                            w["mixer_norm"], conv_in, state_in, pending_tape=tape if lane.pending_path else None,
+                                                            pending_path=lane.pending_path)
+            out.append(hidden)
+            left.append((conv, state, step_tape))
+            first += lane.rows
+        return np.concatenate(out), left
+
+    def oracle_mixer_output(self, mixed, hidden, li):
+        w = self.layers[li]
+        o = self._project(orc.FMT_Q4K, w["o"] if self.attends(li) else w["mixer_out"], mixed, self.dims["hidden"])
+        return orc.f32_to_bf16((o + orc.bf16_to_f32(hidden)).astype(np.float32))
+
+    def oracle_ffn(self, hidden1, li):
+        """(router scores, output rows) of the layer's mixture of experts."""
+        w, d = self.layers[li], self.dims
+        n = orc.rms_norm(hidden1, w["post_norm"])
+        scores = self._project(orc.FMT_Q6K, w["router"], n, d["experts"]).astype(np.float32)
+        _, _, _, out = orc.moe_layer(n, hidden1, scores, d["top_k"], w["gate"], w["up"], w["down"], d["expert_ffn"])
+        return scores, out
+
+    def oracle_head(self, hidden):
+        n = orc.rms_norm(hidden, self.final_norm)
+        return self._project(orc.FMT_Q6K, self.head, n, self.dims["vocabulary"])

@@ -1,0 +1,140 @@
+"""End-to-end parity of the hybrid mixture-of-experts verify step (BASELINE config 5 at a small shape: three Gated
+DeltaNet layers and one attention layer, 16 experts top-2) against the oracle, through the C ABI: every layer
+teacher-forced from the GPU's own layer input, the step's parts bitwise the whole step, greedy acceptance exact,
+and the state rollback across two steps of two lanes (the accepted path of the first step is what the second folds)."""
+import numpy as np
+import pytest
+
+from splash_amd import ops, verify
+from tests import oracle as orc
+from tests.hybrid_reference import HybridModel
+from tests.test_verify_step_gpu import close_bf16
+
+pytestmark = pytest.mark.gpu
+
+SHAPE = dict(hidden=256, vocabulary=1024, layers=4, q_heads=8, kv_heads=2, head_dim=128, gdn_key_heads=2, gdn_value_heads=4,
+             experts=16, top_k=2, expert_ffn=256)
+
+
+def sure_routes(scores, top_k):
+    """Rows whose k-th and (k + 1)-th scores are far enough apart that a last-bit difference cannot reroute them."""
+    ordered = -np.sort(-scores, axis=1)
+    return (ordered[:, top_k - 1] - ordered[:, top_k]) > 1e-3 * np.abs(scores).max()
+
+
+def check_step(backend, model, gpu, lanes, tokens):
+    """Runs the step whole, then part by part, each layer against the oracle from the GPU's own input rows, cells
+    and tapes. Returns the step's results."""
+    d = model.dims
+    H, V = d["hidden"], d["vocabulary"]
+    rows = sum(l.rows for l in lanes)
+    gpu.set_block(lanes, tokens)
+    backend.run(gpu.encode(lanes, commit=True))
+    whole_logits = gpu.buffer(verify.LOGITS).download(np.float32, rows * V).reshape(rows, V)
+    results = gpu.results(lanes)
+    hidden_of = lambda i=0: gpu.buffer(verify.HIDDEN, i).download(np.uint16, rows * H).reshape(rows, H)
+    backend.run(gpu.encode_part(0, 0, lanes))
+    assert np.array_equal(hidden_of(), model.oracle_embedding(tokens))
+    for layer in range(d["layers"]):
+        before = hidden_of()
+        g = gpu.mixer_index(layer)
+        if not model.attends(layer):
+            cells = [model.read_cell(i, l.parity, g) for i, l in enumerate(lanes)]
+            tapes = [model.read_tape(i, l.parity ^ 1, g) for i, l in enumerate(lanes)]
+        backend.run(gpu.encode_part(1, layer, lanes))
+        packed = model.oracle_mixer_input(before, layer)
+        if model.attends(layer):
+            mixed = model.oracle_attention(packed, layer, lanes)
+        else:
+            mixed, left = model.oracle_gdn(packed, layer, lanes, cells, tapes)
+            for i, l in enumerate(lanes):
+                conv, state = model.read_cell(i, l.parity ^ 1, g)
+                assert np.array_equal(conv, left[i][0]), (layer, i)
+                assert np.abs(state - left[i][1]).max() <= 1e-4 * np.abs(left[i][1]).max(), (layer, i)
+        hidden1 = model.oracle_mixer_output(mixed, before, layer)
+        ok, detail = close_bf16(hidden_of(1), hidden1)
+        assert ok, ("mixer", layer, detail)
+        # the FFN from the GPU's own mixer output
+        scores, want = model.oracle_ffn(hidden_of(1), layer)
+        sure = sure_routes(scores, d["top_k"])
+        assert sure.mean() >= 0.9
+        ok, detail = close_bf16(hidden_of()[sure], want[sure])
+        assert ok, ("ffn", layer, detail)
+    final = hidden_of()
+    backend.run(gpu.encode_part(2, 0, lanes))
+    logits = gpu.buffer(verify.LOGITS).download(np.float32, rows * V).reshape(rows, V)
+    assert np.array_equal(logits, whole_logits)        # parts and whole are the same dispatches
+    want_logits = model.oracle_head(final)
+    cos = (logits.astype(np.float64) * want_logits).sum() / np.sqrt((logits.astype(np.float64) ** 2).sum() * (want_logits ** 2).sum())
+    assert cos >= 0.9999 and np.abs(logits - want_logits).max() <= 2e-2, (cos, np.abs(logits - want_logits).max())
+    # greedy acceptance of the GPU's own logits, lane by lane, is exact
+    selected, retained, accepted, masks = results
+    first = 0
+    for i, l in enumerate(lanes):
+        picks = np.array([orc.argmax(logits[first + r]) for r in range(l.rows)], dtype=np.uint32)
+        kept, acc, mask = orc.accept_tree(ops.chain_tree_rows([l.rows]), tokens[first:first + l.rows], picks)
+        assert retained[i] == len(kept) and accepted[i] == acc and masks[i] == mask
+        assert np.array_equal(selected[first:first + len(kept)], kept)
+        first += l.rows
+    return logits, results
+
+
+def test_config5_two_steps_with_rollback(backend):
+    print("case config 5 hybrid two steps", flush=True)
+    model = HybridModel(seed=41, **SHAPE)
+    gpu = model.build_gpu(backend, max_lanes=2, pages_per_lane=2)
+    rng = np.random.default_rng(5)
+    model.seed_context(rng)
+    model.seed_states(rng, lanes=2)
+    V = SHAPE["vocabulary"]
+    committed = [70, 300]
+    rows = [6, 16]
+    lanes = [verify.HybridLane(rows[i], committed[i], table_first=i * model.pages_per_lane) for i in range(2)]
+    # lane 0's draft continues the target's own choices for three rows and then departs; lane 1's is random
+    tokens = rng.integers(0, V, sum(rows)).astype(np.uint32)
+    for r in range(1, 4):
+        gpu.set_block(lanes, tokens)
+        backend.run(gpu.encode(lanes, commit=False))
+        tokens[r] = gpu.buffer(verify.LOGITS).download(np.float32, sum(rows) * V).reshape(-1, V)[r - 1].argmax()
+    logits, (selected, retained, accepted, masks) = check_step(backend, model, gpu, lanes, tokens)
+    assert accepted[0] >= 3 and masks[0] & 0b1111 == 0b1111 and retained[1] >= 1 and masks[1] & 1
+    # what the step left: each GDN layer's tape of parity 0 and the cell of parity 1 (the state BEFORE the block)
+    before = [[model.read_cell(i, 1, g) for g in range(gpu.gdn_layers)] for i in range(2)]
+    # second step: every lane folds the path it retained, at the other parity, after its kept tokens
+    lanes2 = [verify.HybridLane(rows2, committed[i] + int(retained[i]), table_first=i * model.pages_per_lane, pending_path=int(masks[i]), parity=1)
+              for i, rows2 in enumerate((16, 3))]
+    tokens2 = rng.integers(0, V, 19).astype(np.uint32)
+    check_step(backend, model, gpu, lanes2, tokens2)
+    # the cell the second step wrote holds exactly the accepted rows of the first: the fold of the first step's
+    # tape along the retained path, bit for bit (identical arithmetic), and nothing of the rejected rows
+    for i in range(2):
+        count = bin(int(masks[i])).count("1")
+        for g in range(gpu.gdn_layers):
+            rc, conv, state = orc.gdn_fold(model.gdn_shape, before[i][g][0], before[i][g][1], model.read_tape(i, 0, g), int(masks[i]), count)
+            got_conv, got_state = model.read_cell(i, 0, g)
+            assert rc == 0 and np.array_equal(conv, got_conv) and state.tobytes() == got_state.tobytes(), (i, g)
+
+
+def test_config5_more_rows_than_one_projection_takes(backend):
+    """Five lanes of sixteen rows: the dense projections run in pieces of at most 64 rows, the mixers, the routed
+    experts and the acceptance over all 80 at once."""
+    print("case config 5 hybrid 80 rows", flush=True)
+    model = HybridModel(seed=42, **SHAPE)
+    gpu = model.build_gpu(backend, max_lanes=5, pages_per_lane=1)
+    rng = np.random.default_rng(6)
+    model.seed_context(rng)
+    model.seed_states(rng, lanes=5)
+    lanes = [verify.HybridLane(16, 20 + 30 * i, table_first=i) for i in range(5)]
+    check_step(backend, model, gpu, lanes, rng.integers(0, SHAPE["vocabulary"], 80).astype(np.uint32))
+
+
+def test_hybrid_rejects_bad_arguments(backend):
+    with pytest.raises(ValueError):
+        verify.HybridVerify(backend, **{**SHAPE, "layers": 5})            # not whole groups of four layers
+    with pytest.raises(ValueError):
+        verify.HybridVerify(backend, **{**SHAPE, "experts": 12})          # the router writes whole column tiles
+    with pytest.raises(ValueError):
+        verify.HybridVerify(backend, **SHAPE, max_lanes=9)
+    gpu = verify.HybridVerify(backend, **SHAPE, max_lanes=1)
+    with pytest.raises(ValueError):
+        gpu.encode([verify.HybridLane(4, 0), verify.HybridLane(4, 0)])    # more lanes than it was built for
