@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the speculative-decoding verify step on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c4|c1] [--lanes B]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c4|c1|c5] [--lanes B]
 
 A step is one verify of a 16-token draft block by the 27B-shaped dense target (64 layers, hidden 5120,
 64 q / 8 kv heads x 128, SwiGLU 25600, vocabulary 151936, Q4_K weights with Q6_K down-projection and
@@ -205,12 +205,114 @@ def time_c5_ops(backend):
                       "expert_gbs": round(weights / float(med[3] + med[4]) / 1e3, 1)}}), flush=True)
 
 
+C5 = dict(hidden=2048, vocabulary=151936, layers=48, q_heads=32, kv_heads=4, head_dim=128, gdn_key_heads=16, gdn_value_heads=32,
+          experts=128, top_k=8, expert_ffn=768, context=16384, rows=16, lanes=8,
+          name="35B-A3B-shaped hybrid MoE verify step: 36 GDN + 12 attention layers, 128 experts top-8 (Q4_K), 16-token draft, "
+               "16K INT8 context, batch 8")
+
+
+def bench_c5(backend, args):
+    """BASELINE config 5 at full size: a step of 8 lanes x 16 rows that folds the 16 rows each lane accepted of the
+    step before (the worst case of the rollback protocol) and runs 16 new ones. Not the headline metric."""
+    import splash_amd
+    from splash_amd import ops, synthetic, verify
+    w = C5
+    lanes_n = args.lanes if args.lanes > 1 else w["lanes"]
+    rng = np.random.default_rng(20260105)
+    H, D, F, V, E = w["hidden"], w["head_dim"], w["expert_ffn"], w["vocabulary"], w["experts"]
+    context_pages = (w["context"] + ops.PAGE_TOKENS - 1) // ops.PAGE_TOKENS
+    physical = context_pages * lanes_n + 1
+    t0 = time.time()
+    gpu = verify.HybridVerify(backend, H, V, w["layers"], w["q_heads"], w["kv_heads"], D, w["gdn_key_heads"], w["gdn_value_heads"], E,
+                              w["top_k"], F, max_lanes=lanes_n, physical_pages=physical, page_table_entries=context_pages * lanes_n)
+    gpu.buffer(verify.PAGE_TABLE).upload(rng.permutation(physical)[:context_pages * lanes_n].astype(np.uint64))
+    packed, QKV, QW, GW = gpu.dims.gdn_packed_width, (w["q_heads"] + 2 * w["kv_heads"]) * D, w["q_heads"] * D, w["gdn_value_heads"] * 128
+    image = lambda fmt, n, k: ops.pack_gguf_image(fmt, synthetic.native(rng, fmt, n, k), n, k)
+    experts = lambda n, k: np.concatenate([image(ops.FMT_Q4K, n, k) for _ in range(8)] * (E // 8))   # eight distinct experts, tiled
+    tensors = dict(gdn_in=image(ops.FMT_Q4K, packed, H), gdn_out=image(ops.FMT_Q4K, H, GW), qkv=image(ops.FMT_Q4K, QKV, H),
+                   o=image(ops.FMT_Q4K, H, QW), router=image(ops.FMT_Q6K, E, H), gate=experts(F, H), up=experts(F, H), down=experts(H, F))
+    first = {name: backend.from_array(t, label=name) for name, t in tensors.items()}
+    bf = lambda a: (np.ascontiguousarray(a, np.float32).view(np.uint32) >> 16).astype(np.uint16)
+    norm = lambda n: backend.from_array(bf(1 + 0.05 * rng.standard_normal(n)))
+    shared = dict(input_norm=norm(H), post_norm=norm(H))
+    conv_dim = (2 * w["gdn_key_heads"] + w["gdn_value_heads"]) * 128
+    gdn_small = dict(convolution_weights=backend.from_array(bf(rng.standard_normal((conv_dim, 4)) * 0.4)),
+                     decay_weights=backend.from_array((-np.exp(rng.uniform(-1, 1, w["gdn_value_heads"]))).astype(np.float32)),
+                     time_bias=backend.from_array(bf(rng.uniform(-1, 1, w["gdn_value_heads"]))), mixer_norm=norm(128))
+    attention_small = dict(query_norm=norm(D), key_norm=norm(D))
+
+    for layer in range(w["layers"]):
+        attends = gpu.attends(layer)
+        names = ("qkv", "o") if attends else ("gdn_in", "gdn_out")
+        fresh = lambda name: first[name] if layer == (3 if attends else 0) or (name in ("gate", "up", "down", "router") and layer == 0) else None
+        buf = {}
+        for name in names + ("router", "gate", "up", "down"):
+            buf[name] = fresh(name)
+            if buf[name] is None:
+                buf[name] = backend.allocate_buffer(first[name].size_bytes, label=name)
+                device_copy(backend, first[name], buf[name], first[name].size_bytes)
+        widths = dict(qkv=(QKV, H), o=(H, QW), gdn_in=(packed, H), gdn_out=(H, GW))
+        P = lambda name: ops.Projection([(ops.FMT_Q4K, widths[name][0], buf[name])], widths[name][1])
+        gpu.set_layer(layer, P(names[0]), P(names[1]), router=ops.Projection([(ops.FMT_Q6K, E, buf["router"])], H, float32=True),
+                      gate_images=buf["gate"], up_images=buf["up"], down_images=buf["down"], **shared,
+                      **(attention_small if attends else gdn_small))
+        if layer % 12 == 11:
+            log(f"  layer {layer + 1}/{w['layers']} resident")
+    gpu.set_head(ops.FMT_Q4K, backend.from_array(synthetic.native(rng, ops.FMT_Q4K, V, H), label="embedding"), norm(H),
+                 ops.Projection([(ops.FMT_Q6K, V, backend.from_array(image(ops.FMT_Q6K, V, H), label="head"))], H, float32=True))
+    pages = synthetic.kv_pages(rng, w["kv_heads"], D, physical)
+    pool0 = gpu.buffer(verify.KV_POOL, 0)
+    pool0.upload(pages)
+    for layer in range(1, w["layers"] // 4):
+        device_copy(backend, pool0, gpu.buffer(verify.KV_POOL, layer), pages.nbytes)
+    log(f"model resident in {time.time() - t0:.1f}s; allocated {backend.memory_stats().allocated_bytes / 1e9:.2f} GB")
+    rows = w["rows"] * lanes_n
+    lane = lambda i, parity, path: verify.HybridLane(w["rows"], w["context"] - w["rows"], table_first=i * context_pages,
+                                                     pending_path=path, parity=parity)
+    gpu.set_block([lane(i, 1, 0) for i in range(lanes_n)], rng.integers(0, V, rows).astype(np.uint32))
+    backend.run(gpu.encode([lane(i, 1, 0) for i in range(lanes_n)], commit=False))      # the step before: fills the tapes
+    lanes = [lane(i, 0, 0xFFFF) for i in range(lanes_n)]
+    graph = gpu.encode(lanes, commit=True)
+    kernels = graph.kernels()
+    step_bytes = gpu.step_bytes(lanes)
+    log(f"step: {len(kernels)} dispatches, {step_bytes / 1e9:.3f} GB algorithmic")
+    command = backend.record(graph)
+    for _ in range(args.warmup):
+        command.submit().wait()
+    gpu_seconds = 0.0
+    wall0 = time.time()
+    for _ in range(args.steps):
+        gpu_seconds += command.submit().wait()[0]
+    wall_ms = (time.time() - wall0) / args.steps * 1e3
+    ms = gpu_seconds / args.steps * 1e3
+    selected, retained, accepted, mask = gpu.results(lanes)
+    log(f"{ms:.3f} ms/step on the GPU clock, {wall_ms:.3f} ms/step wall; retained {retained.tolist()}")
+    backend.set_dispatch_profiling(True)
+    _, _, per = backend.run(graph, profiled=True)
+    backend.set_dispatch_profiling(False)
+    by_kernel = {}
+    for name, seconds in zip(kernels, per):
+        by_kernel.setdefault(name, []).append(seconds)
+    totals = sorted(((sum(v), k) for k, v in by_kernel.items()), reverse=True)
+    for total, name in totals[:14]:
+        log(f"  {name:36s} x{len(by_kernel[name]):4d}  avg {total / len(by_kernel[name]) * 1e6:8.2f} us  total {total * 1e3:7.3f} ms")
+    print(json.dumps({
+        "metric": "verify-step ms (config 5: hybrid MoE, batch 8)", "value": round(ms, 4), "unit": "ms", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16 x int4/int6 codes -> fp32 (MFMA); fp32 recurrent state; int8 KV", "data": "synthetic",
+        "config": {"workload": w["name"], "lanes": lanes_n, "rows_per_lane": w["rows"], "context_tokens": w["context"],
+                   "layers": w["layers"], "dispatches": len(kernels), "acceptance": "greedy", "pending_rows_folded": 16},
+        "step_hbm": {"algorithmic_gb": round(step_bytes / 1e9, 3), "achieved_gbs": round(step_bytes / (ms * 1e-3) / 1e9, 1),
+                     "frac_of_peak": round(step_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "wall_ms_per_step": round(wall_ms, 4)},
+        "kernels_ms": {name: round(total * 1e3, 3) for total, name in totals[:14]}, "cpu_baseline": None}), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="c4", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="c4", choices=sorted(WORKLOADS) + ["c5"])
     ap.add_argument("--lanes", type=int, default=1)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--ops", choices=["c5"], help="time the GDN step and the MoE layer of config 5 instead of the dense step")
@@ -220,11 +322,14 @@ def main():
         sys.exit(2)
     import splash_amd
     from splash_amd import ops, verify
-    w = WORKLOADS[args.workload]
     backend = splash_amd.Backend(0)
     if args.ops == "c5":
         time_c5_ops(backend)
         return
+    if args.workload == "c5":
+        bench_c5(backend, args)
+        return
+    w = WORKLOADS[args.workload]
     info = backend.device_info()
     log(f"device {info.name.decode()} {info.arch.decode()} CUs {info.compute_units}")
     t0 = time.time()

@@ -98,7 +98,10 @@ LinearPlan Linear::plan(LinearWorkload w, FloatOutput destination) const {
   const uint32_t groups = std::max(1u, groupsOf(w.matrix.outputSize, w.epilogue));
   const uint32_t wanted =
       calibration_.computeUnits * (w.formatId == GGUF_FMT_Q6K ? calibration_.groupsPerUnitQ6K : calibration_.groupsPerUnit);
-  const uint32_t most = std::min(LinearConfig::kMaximumSplits, std::max(1u, blocks / calibration_.minimumBlocksPerWave));
+  uint32_t most = std::min(LinearConfig::kMaximumSplits, std::max(1u, blocks / calibration_.minimumBlocksPerWave));
+  // A projection of a few column tiles (a router) leaves most of the device idle however short its
+  // ranges: it partitions K down to single super-blocks.
+  if (groups * most * 4 < calibration_.computeUnits) most = std::min(LinearConfig::kMaximumSplits, blocks);
   LinearConfig config;
   const uint32_t units = calibration_.computeUnits;
   if (groups >= 2 * units && groups % units) {

@@ -53,7 +53,7 @@ void MoE::addRouting(hip::CommandGraph &graph, const hip::Buffer &scores, uint32
   graph.add("moe_route_select", {scores, w.selected, w.weights}, MoeRouteParams{rows, shape.experts, shape.topK, scoreStride}, {rows, 1, 1},
             {64, 1, 1});
   graph.add("moe_group_routes", {w.selected, w.routeSlot, w.slotRow, w.tileExpert, w.tileRows, w.tileTotal},
-            MoeGroupParams{routes, shape.experts, shape.topK, moe_maximum_tiles(routes, shape.experts)}, {1, 1, 1}, {256, 1, 1});
+            MoeGroupParams{routes, shape.experts, shape.topK, moe_maximum_tiles(routes, shape.experts)}, {1, 1, 1}, {1024, 1, 1});
 }
 
 void MoE::addRouted(hip::CommandGraph &graph, const hip::Buffer &normalized, const hip::Buffer &residual, const hip::Buffer &output,
