@@ -92,6 +92,8 @@ typedef struct spo_attention_geometry {
   uint32_t q_heads, kv_heads, head_dim;
   uint32_t rotary_pairs; /* RoPE pairs (i, i + pairs) */
   uint32_t normalize;    /* RMS-norm q and k heads */
+  uint32_t gated;        /* the projection row holds each query head's queries, then its gate; the output rows
+                            are multiplied by the gates' sigmoids (kernels/common/attention_gate.h:19-44) */
 } spo_attention_geometry;
 typedef struct spo_attention_rows { /* one sequence: ops::AttentionRows / AttentionHistory */
   uint32_t first_row, rows, committed, table_first;
@@ -115,11 +117,12 @@ sp_status spo_attention_add_projection(spo_graph *graph, const spo_attention_pla
                                        sp_buffer *page_table, sp_buffer *pool, uint64_t page_bytes);
 /* PagedAttention::addAttention (PagedAttention.cpp:466-607): split, then ordered reduce.
  * output_table (optional, spo_gguf_table_bytes(q_heads * head_dim, rows) bytes): the reduce also
- * writes the rows as the activation table of the projection that follows. */
+ * writes the rows as the activation table of the projection that follows. packed_qkv: the rows'
+ * projection, which holds the gates of a gated geometry (NULL otherwise). */
 sp_status spo_attention_add_attention(spo_graph *graph, const spo_attention_plan *plan, sp_buffer *queries,
                                       sp_buffer *query_sums, sp_buffer *partials, sp_buffer *partial_sums,
                                       sp_buffer *tree_rows, sp_buffer *page_table, sp_buffer *pool, uint64_t page_bytes,
-                                      sp_buffer *output, sp_buffer *output_table);
+                                      sp_buffer *output, sp_buffer *output_table, sp_buffer *packed_qkv);
 /* PagedAttention::addPathCommit (PagedAttention.cpp:647-667). */
 sp_status spo_attention_add_path_commit(spo_graph *graph, const spo_attention_plan *plan, sp_buffer *retained,
                                         sp_buffer *page_table, sp_buffer *pool, uint64_t page_bytes);
@@ -260,6 +263,7 @@ typedef struct spo_hybrid_verify spo_hybrid_verify;
 typedef struct spo_hybrid_dimensions {
   uint32_t hidden, vocabulary, layers, attention_interval;
   uint32_t q_heads, kv_heads, head_dim, rotary_pairs, normalize_heads;
+  uint32_t gated_attention; /* the attention layers' rows carry output gates (the reference's Qwen3.5 attention) */
   float rope_theta;
   uint32_t gdn_key_heads, gdn_value_heads, gdn_packed_width; /* packed row [q|k|v|z|b|a], whole column tiles */
   uint32_t experts, top_k, expert_ffn;

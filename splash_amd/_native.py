@@ -75,7 +75,7 @@ class LinearPlan(ctypes.Structure):
 
 
 class AttentionGeometry(ctypes.Structure):
-    _fields_ = [("q_heads", c_u32), ("kv_heads", c_u32), ("head_dim", c_u32), ("rotary_pairs", c_u32), ("normalize", c_u32)]
+    _fields_ = [("q_heads", c_u32), ("kv_heads", c_u32), ("head_dim", c_u32), ("rotary_pairs", c_u32), ("normalize", c_u32), ("gated", c_u32)]
 
 
 class AttentionRows(ctypes.Structure):
@@ -138,7 +138,7 @@ class VerifyLane(ctypes.Structure):
 
 class HybridDimensions(ctypes.Structure):
     _fields_ = [(n, c_u32) for n in ("hidden", "vocabulary", "layers", "attention_interval", "q_heads", "kv_heads", "head_dim",
-                                     "rotary_pairs", "normalize_heads")] + [("rope_theta", ctypes.c_float)] + [
+                                     "rotary_pairs", "normalize_heads", "gated_attention")] + [("rope_theta", ctypes.c_float)] + [
         (n, c_u32) for n in ("gdn_key_heads", "gdn_value_heads", "gdn_packed_width", "experts", "top_k", "expert_ffn")]
 
 
@@ -227,7 +227,7 @@ _sig("spo_attention_plan_destroy", None, c_p)
 _sig("spo_attention_plan_splits", c_u32, c_p)
 _sig("spo_attention_workspace", c_int, c_p, P(c_u64))
 _sig("spo_attention_add_projection", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_u64)
-_sig("spo_attention_add_attention", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_u64, c_p, c_p)
+_sig("spo_attention_add_attention", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_u64, c_p, c_p, c_p)
 _sig("spo_attention_add_path_commit", c_int, c_p, c_p, c_p, c_p, c_p, c_u64)
 
 _sig("spo_norm_add_rms", c_int, c_p, c_p, c_p, c_p, c_u32, c_u32)

@@ -77,11 +77,12 @@ struct AttentionParams {
   uint32_t q_heads, kv_heads, head_dim;
   uint32_t rotary_pairs;     // pairs (i, i + pairs) rotated by RoPE; 0 for none
   uint32_t normalize;        // 1: q and k heads are RMS-normed with the bound weights first
-  uint32_t qkv_stride;       // elements of a packed qkv row: (q_heads + 2 kv_heads) * head_dim
+  uint32_t qkv_stride;       // elements of a packed qkv row: (q_heads + 2 kv_heads) * head_dim, or with gates
+                             // (2 q_heads + 2 kv_heads) * head_dim: each query head's queries, then its gate
   uint32_t splits;           // grid.y of the split kernel: the most splits of any sequence
   uint32_t sequences;
   uint32_t table_tiles;      // attention_reduce_*_t: row tiles of the activation table it writes
-  uint32_t reserved;
+  uint32_t gated;            // 1: the output rows are multiplied by the sigmoid of their heads' gates (attention_gate.h:19-44)
   uint64_t page_bytes;       // bytes between physical pages of the layer's pool
   struct AttentionSequence sequence[ATTENTION_MAXIMUM_SEQUENCES];
 };

@@ -32,7 +32,7 @@ sp_status spo_attention_plan_create(const spo_attention_geometry *geometry, cons
     for (uint32_t i = 0; i < count; ++i)
       rows.push_back({sequences[i].first_row, sequences[i].rows, sequences[i].committed, sequences[i].table_first});
     const ops::AttentionGeometry g{geometry->q_heads, geometry->kv_heads, geometry->head_dim, geometry->rotary_pairs,
-                                   geometry->normalize != 0};
+                                   geometry->normalize != 0, geometry->gated != 0};
     *out = new spo_attention_plan{ops::PagedAttention::plan(g, std::move(rows))};
   });
 }
@@ -58,14 +58,15 @@ sp_status spo_attention_add_projection(spo_graph *graph, const spo_attention_pla
 }
 sp_status spo_attention_add_attention(spo_graph *graph, const spo_attention_plan *plan, sp_buffer *queries, sp_buffer *query_sums,
                                       sp_buffer *partials, sp_buffer *partial_sums, sp_buffer *tree_rows, sp_buffer *page_table,
-                                      sp_buffer *pool, uint64_t page_bytes, sp_buffer *output, sp_buffer *output_table) {
+                                      sp_buffer *pool, uint64_t page_bytes, sp_buffer *output, sp_buffer *output_table,
+                                      sp_buffer *packed_qkv) {
   return capi::guard([&] {
     capi::require(graph && plan, "graph or plan");
     ops::AttentionWorkspace w{hip::Buffer::share(queries), hip::Buffer::share(query_sums), hip::Buffer::share(partials),
                               hip::Buffer::share(partial_sums)};
     ops::PagedAttention::addAttention(capi::graphOf(graph), plan->plan, w, hip::Buffer::share(tree_rows),
                                       pagesOf(page_table, pool, page_bytes), hip::Buffer::share(output),
-                                      hip::Buffer::share(output_table));
+                                      hip::Buffer::share(output_table), hip::Buffer::share(packed_qkv));
   });
 }
 sp_status spo_attention_add_path_commit(spo_graph *graph, const spo_attention_plan *plan, sp_buffer *retained,

@@ -45,6 +45,7 @@ sp_status spo_hybrid_verify_create(sp_backend *backend, const spo_hybrid_dimensi
     dims.headDimension = d->head_dim;
     dims.rotaryPairs = d->rotary_pairs;
     dims.normalizeHeads = d->normalize_heads != 0;
+    dims.gatedAttention = d->gated_attention != 0;
     dims.ropeTheta = d->rope_theta;
     dims.gdnKeyHeads = d->gdn_key_heads;
     dims.gdnValueHeads = d->gdn_value_heads;

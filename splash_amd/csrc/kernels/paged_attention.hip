@@ -99,7 +99,9 @@ __global__ __launch_bounds__(D) void attention_q8_qkv(const uint16_t *__restrict
   }
   const uint32_t index = query ? head : head - p.q_heads;
   const size_t packed = size_t(seq.first_row) + row;
-  const uint16_t *source = qkv + packed * p.qkv_stride + (query ? index * D : p.q_heads * D + index * D);
+  // A gated layer's row holds each query head's queries, then its gate (attention_gate.h:27-31).
+  const uint32_t queryStride = p.gated ? 2u * D : uint32_t(D);
+  const uint16_t *source = qkv + packed * p.qkv_stride + (query ? index * queryStride : p.q_heads * queryStride + index * D);
   const float element = bf16_bits_to_float(source[tid]);
   float result = element;
   if (p.normalize) {
@@ -417,7 +419,8 @@ SP_REGISTER_KERNEL("attention_q8_split_d64_g2", &attention_q8_split<64, 2>);
 // a tile past the packed rows keep what the table held.
 template <int D, bool Table>
 __global__ __launch_bounds__(256) void attention_reduce(const float *__restrict__ partialO, const float *__restrict__ partialML,
-                                                        uint16_t *__restrict__ out, uint8_t *__restrict__ table, AttentionParams p) {
+                                                        uint16_t *__restrict__ out, uint8_t *__restrict__ table,
+                                                        const uint16_t *__restrict__ qkv, AttentionParams p) {
   constexpr uint32_t kQuads = D / 4, kParts = 256 / kQuads;
   __shared__ float weights[ATTENTION_MAXIMUM_SPLITS];
   __shared__ float scratch[4];
@@ -471,7 +474,12 @@ __global__ __launch_bounds__(256) void attention_reduce(const float *__restrict_
 #pragma unroll
     for (uint32_t q = 0; q < kParts; ++q) numerator += flat[q * D + tid];
     const float value = denominator > 0.f ? numerator / denominator : 0.f;
-    const uint32_t bits = float_to_bf16_bits(value);
+    uint32_t bits = float_to_bf16_bits(value);
+    if (p.gated) {
+      // attention_gate.h:27-31: bf16(value) times the sigmoid of the head's gate in the row's packed projection.
+      const float gate = bf16_bits_to_float(qkv[(size_t(seq.first_row) + row) * p.qkv_stride + head * 2u * D + D + tid]);
+      bits = float_to_bf16_bits(bf16_bits_to_float(bits) * (1.0f / (1.0f + __builtin_amdgcn_exp2f(-kLog2e * gate))));
+    }
     out[(size_t(seq.first_row) + row) * (p.q_heads * D) + head * D + tid] = uint16_t(bits);
     if constexpr (Table) staged[tid] = uint16_t(bits);
   }

@@ -134,7 +134,9 @@ ops::AttentionPlan HybridVerify::planOf(const std::vector<HybridLane> &lanes) co
     sequences.push_back({rows, lane.block.rows, lane.block.committed, lane.block.tableFirst});
     rows += lane.block.rows;
   }
-  return ops::PagedAttention::plan({dims_.qHeads, dims_.kvHeads, dims_.headDimension, dims_.rotaryPairs, dims_.normalizeHeads}, sequences);
+  return ops::PagedAttention::plan({dims_.qHeads, dims_.kvHeads, dims_.headDimension, dims_.rotaryPairs, dims_.normalizeHeads,
+                                    dims_.gatedAttention},
+                                   sequences);
 }
 
 void HybridVerify::encodeEmbedding(hip::CommandGraph &graph, uint32_t rows) {
@@ -172,7 +174,7 @@ void HybridVerify::encodeLayer(hip::CommandGraph &graph, uint32_t layer, const s
     const ops::AttentionPlan plan = planOf(lanes);
     const ops::KvPages pages{pageTable_, kvPools_.at(index), pageBytes_};
     ops::PagedAttention::addProjection(graph, plan, {packed_, w.queryNorm, w.keyNorm, ropeCos_, ropeSin_}, attentionWorkspace_, pages);
-    ops::PagedAttention::addAttention(graph, plan, attentionWorkspace_, treeRows_, pages, mixed_, {});
+    ops::PagedAttention::addAttention(graph, plan, attentionWorkspace_, treeRows_, pages, mixed_, {}, packed_);
   } else {
     std::vector<ops::GdnLaneStep> steps;
     uint32_t firstRow = 0;

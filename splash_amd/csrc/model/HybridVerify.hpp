@@ -31,6 +31,7 @@ struct HybridDimensions final {
   uint32_t attentionInterval = 4;  // layer l attends when (l + 1) % attentionInterval == 0
   uint32_t qHeads = 0, kvHeads = 0, headDimension = 0, rotaryPairs = 0;
   bool normalizeHeads = true;
+  bool gatedAttention = false;  // the attention layers' rows carry output gates
   float ropeTheta = 1000000.0f;
   uint32_t gdnKeyHeads = 0, gdnValueHeads = 0;
   uint32_t gdnPackedWidth = 0;  // the GDN input projection's width (whole column tiles)
@@ -44,7 +45,7 @@ struct HybridDimensions final {
     const uint32_t before = layer / attentionInterval;  // attention layers before it
     return attends(layer) ? before : layer - before;
   }
-  [[nodiscard]] uint32_t qkvWidth() const noexcept { return (qHeads + 2 * kvHeads) * headDimension; }
+  [[nodiscard]] uint32_t qkvWidth() const noexcept { return ((gatedAttention ? 2 : 1) * qHeads + 2 * kvHeads) * headDimension; }
   [[nodiscard]] uint32_t attentionWidth() const noexcept { return qHeads * headDimension; }
   [[nodiscard]] uint32_t gdnWidth() const noexcept { return gdnValueHeads * GDN_HEAD_DIMENSION; }
   [[nodiscard]] ops::GdnShape gdnShape() const noexcept {

@@ -56,6 +56,7 @@ AttentionParams AttentionPlan::params(uint64_t pageBytes) const noexcept {
   p.rotary_pairs = geometry_.rotaryPairs;
   p.normalize = geometry_.normalize;
   p.qkv_stride = geometry_.packedWidth();
+  p.gated = geometry_.gated;
   p.splits = splits_;
   p.sequences = uint32_t(sequences_.size());
   p.page_bytes = pageBytes;
@@ -113,7 +114,7 @@ void PagedAttention::addProjection(hip::CommandGraph &graph, const AttentionPlan
 
 void PagedAttention::addAttention(hip::CommandGraph &graph, const AttentionPlan &plan, const AttentionWorkspace &w,
                                   const hip::Buffer &treeRows, const KvPages &pages, const hip::Buffer &output,
-                                  const hip::Buffer &outputTable) {
+                                  const hip::Buffer &outputTable, const hip::Buffer &packed) {
   const AttentionGeometry &g = plan.geometry();
   const uint32_t rows = totalRows(plan.sequences());
   const AttentionWorkspaceSize need = plan.workspace();
@@ -123,6 +124,7 @@ void PagedAttention::addAttention(hip::CommandGraph &graph, const AttentionPlan 
   requireBytes(w.partialSums, need.partialSums, "attention partial sums");
   requireBytes(treeRows, uint64_t{rows} * sizeof(AttentionTreeRow), "verify tree rows");
   requireBytes(output, uint64_t{rows} * g.qHeads * g.headDimension * 2, "attention output");
+  if (g.gated) requireBytes(packed, uint64_t{rows} * g.packedWidth() * 2, "attention qkv (the gates)");
   requirePages(plan, pages);
   AttentionParams params = plan.params(pages.pageBytes);
   const uint32_t width = g.qHeads * g.headDimension;
@@ -135,7 +137,7 @@ void PagedAttention::addAttention(hip::CommandGraph &graph, const AttentionPlan 
             {w.queries, w.querySums, treeRows, pages.pageTable, pages.pool, w.partials, w.partialSums}, params,
             {g.kvHeads, plan.splits(), plan.sequences().size()}, {256, 1, 1});
   graph.add("attention_reduce" + kernelSuffix(g) + (outputTable ? "_t" : ""),
-            {w.partials, w.partialSums, output, outputTable ? outputTable : output}, params,
+            {w.partials, w.partialSums, output, outputTable ? outputTable : output, g.gated ? packed : output}, params,
             {g.qHeads, ATTENTION_MAXIMUM_ROWS, plan.sequences().size()}, {256, 1, 1});
 }
 

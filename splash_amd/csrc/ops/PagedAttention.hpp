@@ -28,8 +28,11 @@ struct AttentionGeometry final {
   uint32_t qHeads = 0, kvHeads = 0, headDimension = 0;
   uint32_t rotaryPairs = 0;  // pairs (i, i + pairs) RoPE rotates
   bool normalize = false;    // RMS-norm q and k heads (q_norm, k_norm weights)
+  // The projection row holds each query head's queries, then its gate, and the output rows are
+  // multiplied by the gates' sigmoids (the reference's Gated geometries, attention_gate.h:19-44).
+  bool gated = false;
   [[nodiscard]] uint32_t group() const noexcept { return kvHeads ? qHeads / kvHeads : 0; }
-  [[nodiscard]] uint32_t packedWidth() const noexcept { return (qHeads + 2 * kvHeads) * headDimension; }
+  [[nodiscard]] uint32_t packedWidth() const noexcept { return ((gated ? 2 : 1) * qHeads + 2 * kvHeads) * headDimension; }
   [[nodiscard]] kv::Layout layout() const noexcept { return {kvHeads, headDimension}; }
 };
 
@@ -99,7 +102,7 @@ public:
   // projection that follows (gguf_table_bytes(q heads * D, rows)), which then needs no table pass.
   static void addAttention(hip::CommandGraph &graph, const AttentionPlan &plan, const AttentionWorkspace &workspace,
                            const hip::Buffer &treeRows, const KvPages &pages, const hip::Buffer &output,
-                           const hip::Buffer &outputTable = {});
+                           const hip::Buffer &outputTable = {}, const hip::Buffer &packed = {});
   // Moves the retained path's slots to their depths (PagedAttention.cpp:647-667); retained is a
   // uint32 mask per sequence.
   // `layers` pools lie layerBytes apart from pages.pool (one dispatch commits them all, as the

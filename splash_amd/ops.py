@@ -199,9 +199,10 @@ class KvPages:
 class AttentionPlan:
     """ops::AttentionPlan: geometry + sequences + history splits."""
 
-    def __init__(self, q_heads, kv_heads, head_dim, sequences, rotary_pairs=0, normalize=False):
-        """sequences: [(first_row, rows, committed, table_first)]"""
-        g = nat.AttentionGeometry(q_heads, kv_heads, head_dim, rotary_pairs, int(normalize))
+    def __init__(self, q_heads, kv_heads, head_dim, sequences, rotary_pairs=0, normalize=False, gated=False):
+        """sequences: [(first_row, rows, committed, table_first)]; gated: a projection row holds each query head's
+        queries, then its gate, and the output rows are multiplied by the gates' sigmoids."""
+        g = nat.AttentionGeometry(q_heads, kv_heads, head_dim, rotary_pairs, int(normalize), int(gated))
         rows = (nat.AttentionRows * len(sequences))(*[nat.AttentionRows(*s) for s in sequences])
         h = ctypes.c_void_p()
         check(lib.spo_attention_plan_create(ctypes.byref(g), rows, len(sequences), ctypes.byref(h)))
@@ -246,12 +247,13 @@ class PagedAttention:
         graph._keep.extend([plan, qkv, workspace, pages, query_norm, key_norm, rope_cos, rope_sin])
 
     @staticmethod
-    def add_attention(graph, plan, workspace, tree_rows, pages, output, output_table=None):
+    def add_attention(graph, plan, workspace, tree_rows, pages, output, output_table=None, packed_qkv=None):
         check(lib.spo_attention_add_attention(graph.handle, plan.handle, workspace.queries.handle, workspace.query_sums.handle,
                                               workspace.partials.handle, workspace.partial_sums.handle, tree_rows.handle,
                                               pages.table.handle, pages.pool.handle, pages.page_bytes, output.handle,
-                                              output_table.handle if output_table is not None else None))
-        graph._keep.extend([plan, workspace, tree_rows, pages, output, output_table])
+                                              output_table.handle if output_table is not None else None,
+                                              packed_qkv.handle if packed_qkv is not None else None))
+        graph._keep.extend([plan, workspace, tree_rows, pages, output, output_table, packed_qkv])
 
     @staticmethod
     def add_path_commit(graph, plan, retained, pages):

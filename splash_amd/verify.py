@@ -116,13 +116,13 @@ class HybridVerify:
 
     def __init__(self, backend, hidden, vocabulary, layers, q_heads, kv_heads, head_dim, gdn_key_heads, gdn_value_heads, experts, top_k,
                  expert_ffn, attention_interval=4, rotary_pairs=None, normalize_heads=True, rope_theta=1e6, gdn_packed_width=None,
-                 max_lanes=1, physical_pages=2, page_table_entries=None):
+                 max_lanes=1, physical_pages=2, page_table_entries=None, gated_attention=False):
         self.backend = backend
         pairs = head_dim // 2 if rotary_pairs is None else rotary_pairs
         conv = (2 * gdn_key_heads + gdn_value_heads) * 128
         packed = gdn_packed_width or (conv + gdn_value_heads * 128 + 2 * gdn_value_heads + 15) // 16 * 16
         self.dims = nat.HybridDimensions(hidden, vocabulary, layers, attention_interval, q_heads, kv_heads, head_dim, pairs,
-                                         int(normalize_heads), rope_theta, gdn_key_heads, gdn_value_heads, packed, experts, top_k, expert_ffn)
+                                         int(normalize_heads), int(gated_attention), rope_theta, gdn_key_heads, gdn_value_heads, packed, experts, top_k, expert_ffn)
         h = ctypes.c_void_p()
         entries = page_table_entries if page_table_entries is not None else physical_pages
         check(lib.spo_hybrid_verify_create(backend.handle, ctypes.byref(self.dims), max_lanes, physical_pages, entries, ctypes.byref(h)))

@@ -9,11 +9,12 @@ from tests import oracle as orc
 
 class HybridModel:
     def __init__(self, seed, hidden, vocabulary, layers, q_heads, kv_heads, head_dim, gdn_key_heads, gdn_value_heads, experts, top_k,
-                 expert_ffn, attention_interval=4, rope_theta=1e6):
+                 expert_ffn, attention_interval=4, rope_theta=1e6, gated_attention=False):
         self.dims = dict(hidden=hidden, vocabulary=vocabulary, layers=layers, q_heads=q_heads, kv_heads=kv_heads, head_dim=head_dim,
                          gdn_key_heads=gdn_key_heads, gdn_value_heads=gdn_value_heads, experts=experts, top_k=top_k, expert_ffn=expert_ffn,
                          attention_interval=attention_interval)
         self.rope_theta = rope_theta
+        self.gated = gated_attention       # a query head's rows of the projection: its queries, then its gate
         rng = np.random.default_rng(seed)
         self.rng = rng
         D = head_dim
@@ -32,7 +33,7 @@ class HybridModel:
                      gate=[quant(expert_ffn, hidden) for _ in range(experts)], up=[quant(expert_ffn, hidden) for _ in range(experts)],
                      down=[quant(hidden, expert_ffn) for _ in range(experts)])
             if self.attends(l):
-                w.update(q=quant(q_heads * D, hidden), k=quant(kv_heads * D, hidden), v=quant(kv_heads * D, hidden),
+                w.update(q=quant(q_heads * D * (2 if self.gated else 1), hidden), k=quant(kv_heads * D, hidden), v=quant(kv_heads * D, hidden),
                          o=quant(hidden, q_heads * D), q_norm=norm(D), k_norm=norm(D))
             else:
                 # a wider spread than a dense projection's, so that the recurrence's inputs are of order one
@@ -56,6 +57,7 @@ class HybridModel:
         gpu = verify.HybridVerify(backend, d["hidden"], d["vocabulary"], d["layers"], d["q_heads"], d["kv_heads"], d["head_dim"],
                                   d["gdn_key_heads"], d["gdn_value_heads"], d["experts"], d["top_k"], d["expert_ffn"],
                                   attention_interval=d["attention_interval"], rope_theta=self.rope_theta, max_lanes=max_lanes,
+                                  gated_attention=self.gated,
                                   physical_pages=self.physical_pages, page_table_entries=max_lanes * pages_per_lane)
         assert gpu.dims.gdn_packed_width == self.packed_width
         self.table = np.random.default_rng(99).permutation(self.physical_pages)[:max_lanes * pages_per_lane].astype(np.uint64)
@@ -68,7 +70,7 @@ class HybridModel:
                           router=P([(orc.FMT_Q6K, d["experts"], w["router"])], H, True), gate_images=images(orc.FMT_Q4K, w["gate"], F, H),
                           up_images=images(orc.FMT_Q4K, w["up"], F, H), down_images=images(orc.FMT_Q4K, w["down"], H, F))
             if self.attends(i):
-                gpu.set_layer(i, P([(orc.FMT_Q4K, d["q_heads"] * D, w["q"]), (orc.FMT_Q4K, d["kv_heads"] * D, w["k"]),
+                gpu.set_layer(i, P([(orc.FMT_Q4K, d["q_heads"] * D * (2 if self.gated else 1), w["q"]), (orc.FMT_Q4K, d["kv_heads"] * D, w["k"]),
                                     (orc.FMT_Q4K, d["kv_heads"] * D, w["v"])], H), P([(orc.FMT_Q4K, H, w["o"])], d["q_heads"] * D),
                               query_norm=backend.from_array(w["q_norm"]), key_norm=backend.from_array(w["k_norm"]), **common)
             else:
@@ -136,7 +138,7 @@ class HybridModel:
         if self.attends(li):
             D = d["head_dim"]
             out = np.concatenate([self._project(orc.FMT_Q4K, w[name], n, width) for name, width in
-                                  (("q", d["q_heads"] * D), ("k", d["kv_heads"] * D), ("v", d["kv_heads"] * D))], axis=1)
+                                  (("q", d["q_heads"] * D * (2 if self.gated else 1)), ("k", d["kv_heads"] * D), ("v", d["kv_heads"] * D))], axis=1)
         else:
             out = self._project(orc.FMT_Q4K, w["mixer_in"], n, self.packed_width)
         return orc.f32_to_bf16(out.astype(np.float32))
@@ -147,6 +149,11 @@ class HybridModel:
         D, pairs = d["head_dim"], d["head_dim"] // 2
         kc, ks, vc, vs = self.context[li // d["attention_interval"]]
         inv = np.array([self.rope_theta ** (-i / pairs) for i in range(pairs)]).astype(np.float32)
+        gates = None
+        if self.gated:
+            heads = packed[:, :d["q_heads"] * 2 * D].reshape(-1, d["q_heads"], 2, D)
+            gates = orc.bf16_to_f32(heads[:, :, 1]).reshape(-1, d["q_heads"] * D)
+            packed = np.concatenate([heads[:, :, 0].reshape(-1, d["q_heads"] * D), packed[:, d["q_heads"] * 2 * D:]], axis=1)
         out, first = [], 0
         for lane in lanes:
             rows, committed = lane.rows, lane.committed
@@ -165,7 +172,11 @@ class HybridModel:
             attn, _ = orc.attention(q, kc, ks, vc, vs, table, anc, committed, want64=False)
             out.append(attn.reshape(rows, d["q_heads"] * D))
             first += rows
-        return np.concatenate(out)
+        out = np.concatenate(out)
+        if self.gated:      # attention_gate.h:27-31: bf16(bf16(value) * sigmoid(gate))
+            sigmoid = np.float32(1) / (np.float32(1) + np.exp2(np.float32(-1.44269504089) * gates))
+            out = orc.f32_to_bf16((orc.bf16_to_f32(out) * sigmoid).astype(np.float32))
+        return out
 
     def oracle_gdn(self, packed, li, lanes, cells, tapes):
         """Every lane's GDN rows from its cell (conv, state) and pending tape; returns (rows, [(conv, state, tape)] it leaves)."""

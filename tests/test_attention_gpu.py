@@ -195,6 +195,55 @@ def test_attention_output_table(backend, rows, committed):
     assert s32[..., :rows].tobytes() == w32[..., :rows].tobytes() and s16[..., :rows].tobytes() == w16[..., :rows].tobytes()
 
 
+@pytest.mark.parametrize("geometry", [(32, 4, 128), (16, 8, 64)])
+def test_gated_output(backend, geometry):
+    """A gated geometry (attention_gate.h:19-44): the projection row holds each query head's queries, then its gate,
+    and a row's output is bf16(bf16(value) * sigmoid(gate)). Against the ungated run of the same queries, keys
+    and values on the GPU: the stored pages are identical and every output is the ungated one times the sigmoid,
+    to the bf16 step the GPU's exp2 may move it."""
+    print(f"case attention gated {geometry}", flush=True)
+    q_heads, kv_heads, D = geometry
+    rows, committed, pairs = 11, 700, D // 2
+    rng = np.random.default_rng(77)
+    kv_plain, _, table = build_context(rng, backend, q_heads, kv_heads, D, rows, committed)
+    kv_gated = ops.KvPages(backend, kv_heads, D, kv_plain.physical_pages, table)
+    kv_gated.upload(kv_plain.download())
+    q = orc.f32_to_bf16(rng.standard_normal((rows, q_heads, D)).astype(np.float32))
+    gates = orc.f32_to_bf16((rng.standard_normal((rows, q_heads, D)) * 2).astype(np.float32))
+    kvrows = orc.f32_to_bf16(rng.standard_normal((rows, 2 * kv_heads * D)).astype(np.float32))
+    plain = np.concatenate([q.reshape(rows, -1), kvrows], axis=1)
+    gated = np.concatenate([np.concatenate([q, gates], axis=2).reshape(rows, -1), kvrows], axis=1)
+    qw = orc.f32_to_bf16((1 + 0.1 * rng.standard_normal(D)).astype(np.float32))
+    kw = orc.f32_to_bf16((1 + 0.1 * rng.standard_normal(D)).astype(np.float32))
+    angles = rng.uniform(0, 6.28, (rows, pairs)).astype(np.float32)
+    cosv, sinv = backend.from_array(np.cos(angles).astype(np.float32)), backend.from_array(np.sin(angles).astype(np.float32))
+    tree = backend.from_array(ops.chain_tree_rows([rows]))
+    outs = []
+    for packed, kv, is_gated in ((plain, kv_plain, False), (gated, kv_gated, True)):
+        plan = ops.AttentionPlan(q_heads, kv_heads, D, [(0, rows, committed, 0)], rotary_pairs=pairs, normalize=True, gated=is_gated)
+        ws = ops.AttentionWorkspace(backend, plan)
+        out = backend.allocate_buffer(rows * q_heads * D * 2)
+        rows_buffer = backend.from_array(packed)
+        graph = splash_amd.CommandGraph()
+        ops.PagedAttention.add_projection(graph, plan, rows_buffer, ws, kv, query_norm=backend.from_array(qw), key_norm=backend.from_array(kw),
+                                          rope_cos=cosv, rope_sin=sinv)
+        ops.PagedAttention.add_attention(graph, plan, ws, tree, kv, out, packed_qkv=rows_buffer if is_gated else None)
+        backend.run(graph)
+        outs.append(out.download(np.uint16).reshape(rows, q_heads, D))
+    assert np.array_equal(kv_plain.download(), kv_gated.download())
+    value, gate = orc.bf16_to_f32(outs[0]), orc.bf16_to_f32(gates)
+    want = orc.f32_to_bf16((value * (np.float32(1) / (np.float32(1) + np.exp2(np.float32(-1.44269504089) * gate)))).astype(np.float32))
+    def key(x):
+        x = x.astype(np.int32)
+        return np.where(x & 0x8000, 0x8000 - x, x)
+    steps = np.abs(key(outs[1]) - key(want))
+    assert steps.max() <= 1 and (steps > 0).mean() < 0.01
+    with pytest.raises(ValueError, match="gates"):
+        plan = ops.AttentionPlan(q_heads, kv_heads, D, [(0, rows, committed, 0)], gated=True)
+        ops.PagedAttention.add_attention(splash_amd.CommandGraph(), plan, ops.AttentionWorkspace(backend, plan), tree, kv_gated,
+                                         backend.allocate_buffer(rows * q_heads * D * 2))
+
+
 def test_path_commit_moves_the_retained_rows(backend):
     """kv_path_commit.metal:21-48: the k-th retained row's slot moves to depth k; a chain is a no-op."""
     print("case attention commit", flush=True)

@@ -115,11 +115,13 @@ def test_config5_two_steps_with_rollback(backend):
             assert rc == 0 and np.array_equal(conv, got_conv) and state.tobytes() == got_state.tobytes(), (i, g)
 
 
-def test_config5_more_rows_than_one_projection_takes(backend):
+@pytest.mark.parametrize("gated", [False, True])
+def test_config5_more_rows_than_one_projection_takes(backend, gated):
     """Five lanes of sixteen rows: the dense projections run in pieces of at most 64 rows, the mixers, the routed
-    experts and the acceptance over all 80 at once."""
-    print("case config 5 hybrid 80 rows", flush=True)
-    model = HybridModel(seed=42, **SHAPE)
+    experts and the acceptance over all 80 at once. Gated: the attention layer's rows carry output gates, as the
+    reference's Qwen3.5 attention layers do."""
+    print(f"case config 5 hybrid 80 rows gated={gated}", flush=True)
+    model = HybridModel(seed=42, gated_attention=gated, **SHAPE)
     gpu = model.build_gpu(backend, max_lanes=5, pages_per_lane=1)
     rng = np.random.default_rng(6)
     model.seed_context(rng)
