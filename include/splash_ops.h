@@ -207,9 +207,17 @@ typedef struct spo_sampling_buffers {
   sp_buffer *logits, *tokens, *partial_values, *partial_indices;
   sp_buffer *draft_probabilities, *uniforms, *masses, *ranges, *decisions, *input_tokens, *tree_rows; /* sampled lanes */
 } spo_sampling_buffers;
-/* Sampling::addVerify (Sampling.cpp:283-328): temperature 0 is greedy. */
+/* ops::SamplingPolicy (Sampling.hpp:56-83): temperature 0 is greedy; a sampling lane keeps the tokens that
+ * weigh at least min_p of its heaviest (0: all), then the top_k most likely of those (0: all), then their
+ * top_p nucleus (1: all). */
+typedef struct spo_sampling_policy {
+  float temperature, min_p;
+  uint32_t top_k;
+  float top_p;
+} spo_sampling_policy;
+/* Sampling::addVerify (Sampling.cpp:283-328). */
 sp_status spo_sampling_add_verify(spo_graph *graph, const spo_sampling_buffers *buffers, uint32_t vocabulary,
-                                  uint32_t logits_stride, const spo_lane_rows *lanes, const float *temperatures,
+                                  uint32_t logits_stride, const spo_lane_rows *lanes, const spo_sampling_policy *policies,
                                   uint32_t count);
 /* Sampling::addAcceptance (Sampling.cpp:330-357). */
 sp_status spo_sampling_add_acceptance(spo_graph *graph, sp_buffer *input_tokens, sp_buffer *tree_rows, sp_buffer *tokens,
@@ -228,6 +236,9 @@ typedef struct spo_verify_lane {
   uint32_t rows, committed, table_first;
   float temperature;  /* 0: greedy */
   uint32_t remaining; /* tokens the lane may still keep */
+  float min_p;        /* as spo_sampling_policy; all zero keeps every token */
+  uint32_t top_k;
+  float top_p;        /* 0 is read as 1 */
 } spo_verify_lane;
 sp_status spo_dense_verify_create(sp_backend *backend, const spo_dense_dimensions *dimensions, uint32_t max_lanes,
                                   uint32_t physical_pages, uint32_t page_table_entries, spo_dense_verify **out);

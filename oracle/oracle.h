@@ -128,6 +128,20 @@ uint32_t orc_accept_tree(const struct OrcTreeRow *tree, const uint32_t *tokens, 
 // tests treat a row below 1e-5 as "close", as target_sampling_metal_test.mm:2645-2709 does.
 uint32_t orc_rejection_row(const float *logits, uint32_t vocab, float temperature, const float *q,
                            uint32_t draft_token, float u_child, float u_row, int *accepted_draft, double *closeness);
+// A lane's sampling policy (Sampling.hpp:56-83 in the reference): the tokens that weigh at least min_p of
+// the heaviest (0: all), then the top_k most likely of those (0: all), then their top_p nucleus (1: all).
+struct OrcSamplingPolicy { float temperature, min_p; uint32_t top_k; float top_p; };
+// distribution_end (sampling.metal:603-670): the last token the row keeps in the order of the logits
+// (larger first, among equals the smaller id first) as (key, last id), the kept mass, and the kept count
+// (returned). {0, 0} keeps everything; an end after the last token of its key's run has last id 0xFFFFFFFF. Pinned by brute force against a sort in the tests; masses sum in
+// fp64, so a nucleus within rounding of a token's boundary is reported through `closeness`.
+uint32_t orc_distribution_end(const float *logits, uint32_t vocab, const struct OrcSamplingPolicy *policy, uint32_t *key,
+                              uint32_t *last, float *mass, double *closeness);
+// orc_rejection_row and orc_rejection_law over the distribution the policy leaves.
+uint32_t orc_rejection_row_policy(const float *logits, uint32_t vocab, const struct OrcSamplingPolicy *policy, const float *q,
+                                  uint32_t draft_token, float u_child, float u_row, int *accepted_draft, double *closeness);
+void orc_rejection_law_policy(const float *logits, uint32_t vocab, const struct OrcSamplingPolicy *policy, const float *q,
+                              double *out);
 // The selection law of one sampled row in fp64, for the enumeration check
 // (target_sampling_metal_test.mm:2602-2631): out[t] = P(row selects t) when the draft proposes its
 // child from q and the row tests and redraws as above. It must equal softmax(logits / T).

@@ -2,6 +2,9 @@
 #include "oracle.h"
 #include "common.hpp"
 
+#include <algorithm>
+#include <cmath>
+#include <cstring>
 #include <limits>
 #include <vector>
 
@@ -51,9 +54,76 @@ Mass rowMass(const float *x, uint32_t V, float inv) {
   return row;
 }
 float tokenWeight(float logit, Mass m, float inv) { return unselectable(logit) ? 0.f : std::exp((logit - m.maximum) * inv); }
-float residualOf(float logit, float q, Mass m, float inv, bool rejected) {
-  const float w = tokenWeight(logit, m, inv);
-  return rejected ? std::max(w / m.sum - q, 0.f) : w;
+// sampling.metal:197-207: the order of the logits as an unsigned key
+uint32_t logitKey(float value) {
+  uint32_t bits;
+  std::memcpy(&bits, &value, 4);
+  bits = (bits << 1) ? bits : 0u;
+  return (bits & 0x80000000u) ? ~bits : bits | 0x80000000u;
+}
+struct OrderEnd { uint32_t key, last; };
+bool atOrBefore(uint32_t key, uint32_t token, OrderEnd end) { return key > end.key || (key == end.key && token <= end.last); }
+// A row's distribution: its maximum, the mass it keeps (m.sum) and the last token it keeps.
+struct Kept { Mass m; OrderEnd end; };
+float keptWeight(float logit, uint32_t token, const Kept &k, float inv) {
+  if (unselectable(logit) || !atOrBefore(logitKey(logit), token, k.end)) return 0.f;
+  return std::exp((logit - k.m.maximum) * inv);
+}
+float residualOf(float logit, uint32_t token, float q, const Kept &k, float inv, bool rejected) {
+  const float w = keptWeight(logit, token, k, inv);
+  return rejected ? std::max(w / k.m.sum - q, 0.f) : w;
+}
+void note(double *closeness, double value, double threshold);
+// distribution_end (sampling.metal:603-670) by a sort: the tokens in the order of the logits (larger
+// first, among equals the smaller id first); min_p keeps those at or above the logit that weighs min_p
+// of the heaviest, top_k the first top_k of those, top_p of those the tokens up to the one at which
+// their mass first exceeds top_p of the kept mass. Masses are summed in fp64 in that order; closeness
+// takes the relative distance of the nucleus from the masses either side of its last token.
+Kept distributionEnd(const float *x, uint32_t V, const OrcSamplingPolicy &policy, uint32_t *count, double *closeness) {
+  const float inv = 1.0f / policy.temperature;
+  Kept kept{rowMass(x, V, inv), {0u, 0u}};
+  std::vector<std::pair<uint32_t, uint32_t>> order;  // (key, id)
+  for (uint32_t t = 0; t < V; ++t)
+    if (!unselectable(x[t])) order.push_back({logitKey(x[t]), t});
+  std::sort(order.begin(), order.end(), [](const auto &a, const auto &b) { return a.first != b.first ? a.first > b.first : a.second < b.second; });
+  size_t keep = order.size();
+  const bool cuts = policy.min_p > 0.f || (policy.top_k && policy.top_k < V) || policy.top_p < 1.f;
+  if (count) *count = uint32_t(keep);
+  if (!cuts) return kept;
+  if (policy.min_p > 0.f) {
+    const uint32_t lowest = logitKey(std::min(kept.m.maximum + policy.temperature * std::log(policy.min_p), kept.m.maximum));
+    size_t n = 0;
+    while (n < order.size() && order[n].first >= lowest) ++n;
+    if (n < order.size()) { keep = n; kept.end = {lowest, 0xFFFFFFFFu}; }
+  }
+  if (policy.top_k && policy.top_k < keep) {
+    keep = policy.top_k;
+    kept.end = {order[keep - 1].first, order[keep - 1].second};
+  }
+  auto weight = [&](size_t i) { return double(tokenWeight(x[order[i].second], kept.m, inv)); };
+  double mass = 0;
+  for (size_t i = 0; i < keep; ++i) mass += weight(i);
+  if (policy.top_p < 1.f) {
+    const double nucleus = double(policy.top_p * float(mass));
+    double walked = 0;
+    for (size_t i = 0; i < keep; ++i) {
+      const double before = walked;
+      walked += weight(i);
+      if (walked > nucleus) {
+        note(closeness, walked, nucleus);
+        if (i) note(closeness, before, nucleus);
+        keep = i + 1;
+        kept.end = {order[i].first, order[i].second};
+        mass = walked;
+        break;
+      }
+    }
+  }
+  kept.m.sum = float(mass);
+  if (count) *count = uint32_t(keep);
+  // An end after the last token of its key's run is written with every id (the same kept set).
+  if (kept.end.key && (keep == order.size() || order[keep].first != kept.end.key)) kept.end.last = 0xFFFFFFFFu;
+  return kept;
 }
 void note(double *closeness, double value, double threshold) {
   if (!closeness) return;
@@ -103,15 +173,32 @@ uint32_t orc_accept_tree(const struct OrcTreeRow *tree, const uint32_t *tokens, 
   return kept;
 }
 
+uint32_t orc_distribution_end(const float *x, uint32_t V, const OrcSamplingPolicy *policy, uint32_t *key, uint32_t *last, float *mass,
+                              double *closeness) {
+  if (closeness) *closeness = 1.0;
+  uint32_t count = 0;
+  const Kept kept = distributionEnd(x, V, *policy, &count, closeness);
+  *key = kept.end.key;
+  *last = kept.end.last;
+  *mass = kept.m.sum;
+  return count;
+}
+
 uint32_t orc_rejection_row(const float *x, uint32_t V, float temperature, const float *q, uint32_t draft_token, float u_child,
                            float u_row, int *accepted_draft, double *closeness) {
-  const float inv = 1.0f / temperature;
-  const Mass mass = rowMass(x, V, inv);
+  const OrcSamplingPolicy policy{temperature, 0.f, 0u, 1.f};
+  return orc_rejection_row_policy(x, V, &policy, q, draft_token, u_child, u_row, accepted_draft, closeness);
+}
+
+uint32_t orc_rejection_row_policy(const float *x, uint32_t V, const OrcSamplingPolicy *policy, const float *q, uint32_t draft_token,
+                                  float u_child, float u_row, int *accepted_draft, double *closeness) {
+  const float inv = 1.0f / policy->temperature;
   if (closeness) *closeness = 1.0;
+  const Kept mass = distributionEnd(x, V, *policy, nullptr, closeness);
   if (accepted_draft) *accepted_draft = 0;
   bool rejected = false;
   if (q && draft_token != ORC_NO_TOKEN && draft_token < V) {
-    const float pc = tokenWeight(x[draft_token], mass, inv) / mass.sum;
+    const float pc = keptWeight(x[draft_token], draft_token, mass, inv) / mass.m.sum;
     note(closeness, double(u_child) * q[draft_token], pc);
     rejected = !(u_child * q[draft_token] < pc);   // accept iff u q < p (sampling.metal:790-800)
     if (!rejected) { if (accepted_draft) *accepted_draft = 1; return draft_token; }
@@ -125,7 +212,7 @@ uint32_t orc_rejection_row(const float *x, uint32_t V, float temperature, const 
       float s = 0.f;
       for (uint32_t i = 0; i < per; ++i) {
         const uint32_t t = begin + l * per + i;
-        if (t < end) s += residualOf(x[t], rejected ? q[t] : 0.f, mass, inv, rejected);
+        if (t < end) s += residualOf(x[t], t, rejected ? q[t] : 0.f, mass, inv, rejected);
       }
       lanes[l] = s;
     }
@@ -166,7 +253,7 @@ uint32_t orc_rejection_row(const float *x, uint32_t V, float temperature, const 
   for (uint32_t i = 0; i < per; ++i) {
     const uint32_t t = begin + chunk * per + i;
     if (t >= end) break;
-    const float w = residualOf(x[t], rejected ? q[t] : 0.f, mass, inv, rejected);
+    const float w = residualOf(x[t], t, rejected ? q[t] : 0.f, mass, inv, rejected);
     if (w > 0.f) lastToken = t;
     walked += w;
     if (selected == ORC_NO_TOKEN && w > 0.f && target < walked) {
@@ -181,10 +268,21 @@ uint32_t orc_rejection_row(const float *x, uint32_t V, float temperature, const 
 // P(select t) = q_t min(1, p_t / q_t) + (1 - sum_s q_s min(1, p_s / q_s)) * max(p_t - q_t, 0) / Z:
 // the first term is "child t drawn and accepted", the second "child rejected, residual draws t".
 void orc_rejection_law(const float *x, uint32_t V, float temperature, const float *q, double *out) {
+  const OrcSamplingPolicy policy{temperature, 0.f, 0u, 1.f};
+  orc_rejection_law_policy(x, V, &policy, q, out);
+}
+
+void orc_rejection_law_policy(const float *x, uint32_t V, const OrcSamplingPolicy *policy, const float *q, double *out) {
+  const float temperature = policy->temperature;
   std::vector<double> p(V);
   double mx = -std::numeric_limits<double>::infinity(), total = 0;
   for (uint32_t t = 0; t < V; ++t) if (!unselectable(x[t])) mx = std::max(mx, double(x[t]));
-  for (uint32_t t = 0; t < V; ++t) { p[t] = unselectable(x[t]) ? 0.0 : std::exp((double(x[t]) - mx) / temperature); total += p[t]; }
+  const Kept kept = distributionEnd(x, V, *policy, nullptr, nullptr);
+  for (uint32_t t = 0; t < V; ++t) {
+    const bool stays = !unselectable(x[t]) && atOrBefore(logitKey(x[t]), t, kept.end);
+    p[t] = stays ? std::exp((double(x[t]) - mx) / temperature) : 0.0;
+    total += p[t];
+  }
   for (uint32_t t = 0; t < V; ++t) p[t] /= total;
   double acceptMass = 0, Z = 0;
   for (uint32_t t = 0; t < V; ++t) { acceptMass += std::min(double(q[t]), p[t]); Z += std::max(p[t] - double(q[t]), 0.0); }

@@ -133,7 +133,11 @@ class DenseDimensions(ctypes.Structure):
 
 class VerifyLane(ctypes.Structure):
     _fields_ = [("rows", c_u32), ("committed", c_u32), ("table_first", c_u32), ("temperature", ctypes.c_float),
-                ("remaining", c_u32)]
+                ("remaining", c_u32), ("min_p", ctypes.c_float), ("top_k", c_u32), ("top_p", ctypes.c_float)]
+
+
+class SamplingPolicy(ctypes.Structure):
+    _fields_ = [("temperature", ctypes.c_float), ("min_p", ctypes.c_float), ("top_k", c_u32), ("top_p", ctypes.c_float)]
 
 
 class HybridDimensions(ctypes.Structure):
@@ -241,7 +245,7 @@ _sig("spo_moe_workspace_sizes", c_int, P(MoeShape), c_u32, P(c_u64))
 _sig("spo_moe_add_routing", c_int, c_p, c_p, c_u32, P(MoeWorkspace), P(MoeShape), c_u32)
 _sig("spo_moe_add_routed", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_u32, c_u32, P(MoeWorkspace), P(MoeShape), c_u32)
 _sig("spo_sampling_workspace", c_int, c_u32, P(c_u64))
-_sig("spo_sampling_add_verify", c_int, c_p, P(SamplingBuffers), c_u32, c_u32, P(LaneRows), P(ctypes.c_float), c_u32)
+_sig("spo_sampling_add_verify", c_int, c_p, P(SamplingBuffers), c_u32, c_u32, P(LaneRows), P(SamplingPolicy), c_u32)
 _sig("spo_sampling_add_acceptance", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, P(LaneRows), P(c_u32), c_u32, P(c_u32))
 _sig("spo_dense_verify_create", c_int, c_p, P(DenseDimensions), c_u32, c_u32, c_u32, P(c_p))
 _sig("spo_dense_verify_destroy", None, c_p)

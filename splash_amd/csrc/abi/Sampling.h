@@ -10,6 +10,15 @@
 #define SAMPLING_MAXIMUM_ROWS 16u    // rows of a lane's verify block
 #define SAMPLING_STOP_TOKENS 4u
 #define SAMPLING_NO_TOKEN 0xFFFFFFFFu  // a row with no selectable logit selects it (SPLASH_NO_TOKEN)
+// A sampled row's words of the decisions buffer: the accepted child or SAMPLING_NO_TOKEN, whether
+// the row draws from the residual, then the end of its distribution in the order of the logits
+// (larger logit first, smaller id first among equals): the last kept token's key and id, and the
+// mass and count of the kept tokens.
+#define SAMPLING_DECISION_WORDS 8u
+#define SAMPLING_END_KEY 2u
+#define SAMPLING_END_LAST 3u
+#define SAMPLING_END_MASS 4u
+#define SAMPLING_END_COUNT 5u
 
 // A lane's rows of the packed rows (SplashLaneRows).
 struct SamplingLaneRows {
@@ -26,8 +35,14 @@ struct TargetSamplingParams {
   uint32_t logits_stride; // floats between logits rows
   float temperature[SAMPLING_MAXIMUM_LANES];
   uint32_t sampling_mask; // lanes that sample; the others take the argmax
-  uint32_t reserved[3];
+  uint32_t truncating_mask; // lanes whose distribution ends before the last token (min_p, top_k or top_p cut it)
+  uint32_t reserved[2];
   struct SamplingLaneRows lane[SAMPLING_MAXIMUM_LANES];
+  // A sampling lane keeps the tokens that weigh at least min_p of the heaviest, then the top_k most
+  // likely of those (0: all), then their top_p nucleus (Sampling.hpp:58-83 in the reference).
+  float min_p[SAMPLING_MAXIMUM_LANES];
+  uint32_t top_k[SAMPLING_MAXIMUM_LANES];
+  float top_p[SAMPLING_MAXIMUM_LANES];
 };
 
 // decode_accept_tree: one thread per lane (AcceptBatchParams).
@@ -40,6 +55,6 @@ struct AcceptBatchParams {
 };
 
 #ifdef __cplusplus
-static_assert(sizeof(TargetSamplingParams) == 16 + 32 + 16 + 64, "target sampling parameters are 128 bytes on both sides");
+static_assert(sizeof(TargetSamplingParams) == 16 + 32 + 16 + 64 + 96, "target sampling parameters are 224 bytes on both sides");
 static_assert(sizeof(AcceptBatchParams) == 16 + 32 + 16 + 64, "acceptance parameters are 128 bytes on both sides");
 #endif

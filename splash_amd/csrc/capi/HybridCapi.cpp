@@ -20,7 +20,9 @@ std::vector<model::HybridLane> lanesOf(const spo_hybrid_lane *lanes, uint32_t co
   std::vector<model::HybridLane> out;
   for (uint32_t i = 0; i < count; ++i) {
     const spo_verify_lane &b = lanes[i].block;
-    out.push_back({{b.rows, b.committed, b.table_first, ops::SamplingPolicy{b.temperature}, b.remaining}, lanes[i].pending_path,
+    out.push_back({{b.rows, b.committed, b.table_first,
+                    ops::SamplingPolicy{b.temperature, b.min_p, b.top_k, b.top_p > 0.0f ? b.top_p : 1.0f}, b.remaining},
+                   lanes[i].pending_path,
                    lanes[i].parity});
   }
   return out;

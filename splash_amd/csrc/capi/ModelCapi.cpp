@@ -21,7 +21,9 @@ std::vector<model::VerifyLane> lanesOf(const spo_verify_lane *lanes, uint32_t co
   capi::require(lanes && count, "lanes");
   std::vector<model::VerifyLane> out;
   for (uint32_t i = 0; i < count; ++i)
-    out.push_back({lanes[i].rows, lanes[i].committed, lanes[i].table_first, ops::SamplingPolicy{lanes[i].temperature}, lanes[i].remaining});
+    out.push_back({lanes[i].rows, lanes[i].committed, lanes[i].table_first,
+                   ops::SamplingPolicy{lanes[i].temperature, lanes[i].min_p, lanes[i].top_k, lanes[i].top_p > 0.0f ? lanes[i].top_p : 1.0f},
+                   lanes[i].remaining});
   return out;
 }
 ops::AttentionPlan planOf(const model::DenseVerify &v, const std::vector<model::VerifyLane> &lanes) {
@@ -71,14 +73,14 @@ sp_status spo_sampling_workspace(uint32_t rows, uint64_t sizes[5]) {
   });
 }
 sp_status spo_sampling_add_verify(spo_graph *graph, const spo_sampling_buffers *b, uint32_t vocabulary, uint32_t logits_stride,
-                                  const spo_lane_rows *lanes, const float *temperatures, uint32_t count) {
+                                  const spo_lane_rows *lanes, const spo_sampling_policy *policy, uint32_t count) {
   return capi::guard([&] {
-    capi::require(graph && b && lanes && temperatures, "graph, buffers, lanes or temperatures");
+    capi::require(graph && b && lanes && policy, "graph, buffers, lanes or policies");
     ops::SamplingBuffers buffers{B(b->logits), B(b->tokens), B(b->partial_values), B(b->partial_indices), B(b->draft_probabilities),
                                  B(b->uniforms), B(b->masses), B(b->ranges), B(b->decisions), B(b->input_tokens), B(b->tree_rows)};
     std::vector<ops::LaneRows> rows;
     std::vector<ops::SamplingPolicy> policies;
-    for (uint32_t i = 0; i < count; ++i) { rows.push_back({lanes[i].first, lanes[i].rows}); policies.push_back({temperatures[i]}); }
+    for (uint32_t i = 0; i < count; ++i) { rows.push_back({lanes[i].first, lanes[i].rows}); policies.push_back({policy[i].temperature, policy[i].min_p, policy[i].top_k, policy[i].top_p}); }
     ops::Sampling::addVerify(capi::graphOf(graph), buffers, vocabulary, logits_stride, rows, policies);
   });
 }

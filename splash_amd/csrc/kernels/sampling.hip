@@ -15,6 +15,15 @@
 // point = u_row * sum, then its chunks and the hit chunk's tokens, each in id order; rounding
 // fall-backs take the last weighted range, chunk and token. A row without a child draws the same
 // way from p itself.
+//
+// A lane's min_p, top_k and top_p cut its rows' distributions (distribution_end, sampling.metal:
+// 603-670): in the order of the logits (larger first, among equals the smaller id first) a row keeps
+// the tokens at or above the logit that weighs min_p of the heaviest, then the first top_k of those,
+// then of those the tokens up to the one at which their mass first exceeds top_p of the kept mass.
+// The end is found by radix descent over the order-preserving key of a logit, four bits a pass, each
+// pass one scan of the row with a 16-bin histogram of counts and masses (a thread's tokens in id
+// order, the threads' sums in a fixed tree), then over the ids of the tokens tied at the last key.
+// Everything after it weighs nothing; p is renormalized by the kept mass.
 #include "abi/Sampling.h"
 #include "abi/PagedAttention.h"
 #include "backend/KernelRegistry.hpp"
@@ -188,14 +197,216 @@ __device__ __forceinline__ uint32_t child_token(const TargetSamplingParams &p, c
     if (tree[first + child].parent == local) return input_tokens[first + child];
   return SAMPLING_NO_TOKEN;
 }
+// The order of the logits as an unsigned key (sampling.metal:197-207): a larger logit has a larger
+// key; -0 and +0 share one; every finite logit's key is above that of -infinity.
+__device__ __forceinline__ uint32_t logit_key(float value) {
+  uint32_t bits = __builtin_bit_cast(uint32_t, value);
+  bits = (bits << 1) ? bits : 0u;
+  return (bits & 0x80000000u) ? ~bits : bits | 0x80000000u;
+}
+__device__ __forceinline__ float key_logit(uint32_t key) {
+  return __builtin_bit_cast(float, (key & 0x80000000u) ? key & 0x7FFFFFFFu : ~key);
+}
+constexpr uint32_t kLowestKey = 0x007FFFFFu;  // of -infinity
+// A position in the order: the tokens at or before it have a larger key, or its key and an id at
+// most `last`. {0, 0} lies after every token.
+struct OrderEnd {
+  uint32_t key, last;
+};
+__device__ __forceinline__ bool at_or_before(uint32_t key, uint32_t token, OrderEnd end) {
+  return key > end.key || (key == end.key && token <= end.last);
+}
+// A row's distribution: its maximum, the mass of the tokens it keeps and the last of them.
+struct Kept {
+  Mass mass;  // maximum, kept mass
+  OrderEnd end;
+};
+__device__ __forceinline__ Kept row_kept(const float *masses, const uint32_t *decisions, uint32_t row, float inverse, bool truncating) {
+  Kept kept{row_mass(masses, row, inverse), {0u, 0u}};
+  if (truncating) {
+    const uint32_t *words = decisions + size_t(row) * SAMPLING_DECISION_WORDS;
+    kept.end = {words[SAMPLING_END_KEY], words[SAMPLING_END_LAST]};
+    kept.mass.sum = __builtin_bit_cast(float, words[SAMPLING_END_MASS]);
+  }
+  return kept;
+}
 __device__ __forceinline__ float token_weight(float logit, Mass mass, float inverse) {
   return unselectable(logit) ? 0.f : expf((logit - mass.maximum) * inverse);
 }
-// The residual weight of token t: max(p_t - q_t, 0) after a rejection, p_t's weight otherwise.
-__device__ __forceinline__ float residual_of(float logit, float q, Mass mass, float inverse, bool rejected) {
-  const float w = token_weight(logit, mass, inverse);
-  return rejected ? fmaxf(w / mass.sum - q, 0.f) : w;
+// A token's weight in the row's distribution: its softmax weight at or before the end, else 0 (kept_weight, sampling.metal:672-679).
+__device__ __forceinline__ float kept_weight(float logit, uint32_t token, const Kept &kept, float inverse) {
+  if (unselectable(logit) || !at_or_before(logit_key(logit), token, kept.end)) return 0.f;
+  return expf((logit - kept.mass.maximum) * inverse);
 }
+// The residual weight of token t: max(p_t - q_t, 0) after a rejection, p_t's weight otherwise.
+__device__ __forceinline__ float residual_of(float logit, uint32_t token, float q, const Kept &kept, float inverse, bool rejected) {
+  const float w = kept_weight(logit, token, kept, inverse);
+  return rejected ? fmaxf(w / kept.mass.sum - q, 0.f) : w;
+}
+// ---------------------------------------------------------------------------------------------
+// decode_sample_distribution_end: grid (rows), 256 threads. Writes the row's end words of the
+// decisions buffer; rows of lanes that keep every token are left alone.
+// ---------------------------------------------------------------------------------------------
+struct Measure {
+  uint32_t count;
+  float mass;
+};
+struct EndScratch {
+  float mass[16][SAMPLING_THREADS];
+  uint32_t count[16][SAMPLING_THREADS];
+  float binMass[16];
+  uint32_t binCount[16];
+};
+// One scan of the row: the 16-bin histogram of `digit(token, key)` (0..15, or 16 to leave a token
+// out) over the selectable tokens at or before `end`, into scratch.binCount / binMass.
+template <class Digit>
+__device__ __forceinline__ void end_histogram(const float *x, uint32_t vocabulary, Mass mass, float inverse, OrderEnd end, Digit digit,
+                                              EndScratch &scratch, uint32_t tid) {
+#pragma unroll
+  for (uint32_t b = 0; b < 16; ++b) {
+    scratch.mass[b][tid] = 0.f;
+    scratch.count[b][tid] = 0u;
+  }
+  for (uint32_t token = tid; token < vocabulary; token += SAMPLING_THREADS) {
+    const float value = x[token];
+    if (unselectable(value)) continue;
+    const uint32_t key = logit_key(value);
+    if (!at_or_before(key, token, end)) continue;
+    const uint32_t b = digit(token, key);
+    if (b >= 16u) continue;
+    scratch.mass[b][tid] += expf((value - mass.maximum) * inverse);
+    scratch.count[b][tid] += 1u;
+  }
+  __syncthreads();
+  // Wavefront w sums bins 4 w .. 4 w + 3: a lane its four threads in order, the lanes in a fixed butterfly.
+  const uint32_t lane = tid & 63u, wave = tid >> 6;
+#pragma unroll
+  for (uint32_t i = 0; i < 4; ++i) {
+    const uint32_t b = 4u * wave + i;
+    float m = ((scratch.mass[b][lane] + scratch.mass[b][lane + 64u]) + scratch.mass[b][lane + 128u]) + scratch.mass[b][lane + 192u];
+    uint32_t c = scratch.count[b][lane] + scratch.count[b][lane + 64u] + scratch.count[b][lane + 128u] + scratch.count[b][lane + 192u];
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      m += __shfl_xor(m, o, 64);
+      c += uint32_t(__shfl_xor(int(c), o, 64));
+    }
+    if (lane == 0) {
+      scratch.binMass[b] = m;
+      scratch.binCount[b] = c;
+    }
+  }
+  __syncthreads();
+}
+// The last token kept of the tokens at or before `end` (of which `all` measures everything), in
+// order until their count exceeds `countTarget` (ByMass false) or their mass `massTarget` (ByMass
+// true); `kept` becomes the measure of the kept tokens. Every thread returns the same.
+template <bool ByMass>
+__device__ OrderEnd select_last(const float *x, uint32_t vocabulary, Mass mass, float inverse, OrderEnd end, uint32_t countTarget,
+                                float massTarget, Measure &kept, EndScratch &scratch, uint32_t tid) {
+  auto exceeded = [&](Measure m) { return ByMass ? m.mass > massTarget : m.count > countTarget; };
+  Measure above{0u, 0.f};
+  uint32_t prefix = 0, tied = 0;
+  for (int shift = 28; shift >= 0; shift -= 4) {
+    const uint32_t high = shift == 28 ? 0u : prefix >> (shift + 4);
+    end_histogram(x, vocabulary, mass, inverse, end,
+                  [&](uint32_t, uint32_t key) { return shift != 28 && (key >> (shift + 4)) != high ? 16u : (key >> shift) & 15u; }, scratch, tid);
+    int chosen = -1, lowest = -1;
+    Measure cumulative = above;
+    for (int b = 15; b >= 0 && chosen < 0; --b) {
+      if (!scratch.binCount[b]) continue;
+      const Measure next{cumulative.count + scratch.binCount[b], cumulative.mass + scratch.binMass[b]};
+      lowest = b;
+      if (exceeded(next)) chosen = b;
+      else cumulative = next;
+    }
+    if (chosen < 0) {
+      // The target is never exceeded: at the first pass every token stays; below it (a bin's mass and
+      // its parts' may round apart) the search ends in the last bin that holds a token.
+      if (shift == 28 || lowest < 0) {
+        kept = cumulative;
+        __syncthreads();
+        return end;
+      }
+      chosen = lowest;
+      cumulative = {cumulative.count - scratch.binCount[lowest], cumulative.mass - scratch.binMass[lowest]};
+    }
+    above = cumulative;
+    prefix |= uint32_t(chosen) << shift;
+    tied = scratch.binCount[chosen];
+    __syncthreads();  // every thread has read the bins before the next pass clears them
+  }
+  // `tied` tokens share the key `prefix` and one weight: as many of them stay as the target takes.
+  const float weight = expf((key_logit(prefix) - mass.maximum) * inverse);
+  uint32_t keep;
+  if (ByMass) {
+    keep = weight > 0.f ? uint32_t(fminf(fmaxf((massTarget - above.mass) / weight, 0.f), float(tied))) : tied;
+    keep = min(max(keep, 1u), tied);
+    while (keep > 1u && above.mass + float(keep - 1u) * weight > massTarget) --keep;
+    while (keep < tied && !(above.mass + float(keep) * weight > massTarget)) ++keep;
+  } else {
+    keep = min(max(countTarget + 1u - above.count, 1u), tied);
+  }
+  kept = {above.count + keep, above.mass + float(keep) * weight};
+  OrderEnd last{prefix, 0xFFFFFFFFu};
+  if (keep < tied) {
+    // The keep-th smallest id of the tied tokens at or before `end`, by the same descent over ids.
+    uint32_t bits = 4;
+    while (bits < 32 && (vocabulary - 1u) >> bits) bits += 4;
+    uint32_t id = 0, before = 0;
+    for (int shift = int(bits) - 4; shift >= 0; shift -= 4) {
+      const uint32_t high = shift + 4 >= 32 ? 0u : id >> (shift + 4);
+      end_histogram(x, vocabulary, mass, inverse, end,
+                    [&](uint32_t token, uint32_t key) {
+                      return key != prefix || (shift + 4 < 32 && (token >> (shift + 4)) != high) ? 16u : (token >> shift) & 15u;
+                    },
+                    scratch, tid);
+      uint32_t chosen = 15;
+      for (uint32_t b = 0; b < 16; ++b) {
+        if (before + scratch.binCount[b] >= keep) {
+          chosen = b;
+          break;
+        }
+        before += scratch.binCount[b];
+      }
+      id |= chosen << shift;
+      __syncthreads();
+    }
+    last.last = id;
+  }
+  return last;
+}
+
+__global__ __launch_bounds__(SAMPLING_THREADS) void decode_sample_distribution_end(const float *__restrict__ logits,
+                                                                                  const float *__restrict__ masses,
+                                                                                  uint32_t *__restrict__ decisions, TargetSamplingParams p) {
+  __shared__ EndScratch scratch;
+  const uint32_t row = blockIdx.x, tid = threadIdx.x, laneIndex = lane_of_row(p, row);
+  if (!((p.truncating_mask >> laneIndex) & 1u)) return;
+  const float temperature = p.temperature[laneIndex], inverse = 1.0f / temperature;
+  const Mass mass = row_mass(masses, row, inverse);
+  const float *x = logits + size_t(row) * p.logits_stride;
+  const float minP = p.min_p[laneIndex], topP = p.top_p[laneIndex];
+  const uint32_t topK = p.top_k[laneIndex];
+  OrderEnd end{0u, 0u};
+  // Everything, and what min_p keeps: the tokens at or above the logit that weighs min_p of the heaviest.
+  const uint32_t lowest = minP > 0.f ? logit_key(fminf(mass.maximum + temperature * logf(minP), mass.maximum)) : kLowestKey;
+  end_histogram(x, p.vocabulary, mass, inverse, end, [&](uint32_t, uint32_t key) { return key >= lowest ? 1u : 0u; }, scratch, tid);
+  Measure kept{scratch.binCount[1], scratch.binMass[1]};
+  const uint32_t admitted = scratch.binCount[0] + scratch.binCount[1];
+  __syncthreads();
+  if (minP > 0.f && kept.count < admitted) end = {lowest, 0xFFFFFFFFu};
+  if (topK && topK < kept.count) end = select_last<false>(x, p.vocabulary, mass, inverse, end, topK - 1u, 0.f, kept, scratch, tid);
+  if (topP < 1.0f) end = select_last<true>(x, p.vocabulary, mass, inverse, end, 0u, topP * kept.mass, kept, scratch, tid);
+  if (tid == 0) {
+    uint32_t *words = decisions + size_t(row) * SAMPLING_DECISION_WORDS;
+    words[SAMPLING_END_KEY] = end.key;
+    words[SAMPLING_END_LAST] = end.last;
+    words[SAMPLING_END_MASS] = __builtin_bit_cast(uint32_t, kept.mass);
+    words[SAMPLING_END_COUNT] = kept.count;
+  }
+}
+SP_REGISTER_KERNEL("decode_sample_distribution_end", &decode_sample_distribution_end);
+
 constexpr uint32_t kChunks = SAMPLING_THREADS;  // chunks of a range, one per thread
 __device__ __forceinline__ uint32_t range_tokens(uint32_t vocabulary) {
   return (vocabulary + SAMPLING_RANGES - 1) / SAMPLING_RANGES;
@@ -214,22 +425,23 @@ __global__ __launch_bounds__(256) void decode_sample_residual_ranges(const float
                                                                      TargetSamplingParams p) {
   constexpr uint32_t kPerRow = SAMPLING_RANGES / 4;
   const uint32_t row = blockIdx.x / kPerRow, range = (blockIdx.x % kPerRow) * 4u + (threadIdx.x >> 6), lane = threadIdx.x & 63u;
-  const float inverse = 1.0f / p.temperature[lane_of_row(p, row)];
-  const Mass mass = row_mass(masses, row, inverse);
+  const uint32_t laneIndex = lane_of_row(p, row);
+  const float inverse = 1.0f / p.temperature[laneIndex];
+  const Kept kept = row_kept(masses, decisions, row, inverse, (p.truncating_mask >> laneIndex) & 1u);
   const float *x = logits + size_t(row) * p.logits_stride, *q = draft + size_t(row) * p.logits_stride;
   const uint32_t child = child_token(p, tree, input_tokens, row);
   bool rejected = false;
   if (child != SAMPLING_NO_TOKEN && child < p.vocabulary) {
     // accept iff u_child * q < p (sampling.metal:790-800)
-    const float pc = token_weight(x[child], mass, inverse) / mass.sum;
+    const float pc = kept_weight(x[child], child, kept, inverse) / kept.mass.sum;
     rejected = !(uniforms[2 * row + 1] * q[child] < pc);
     if (blockIdx.x % kPerRow == 0 && threadIdx.x == 0) {
-      decisions[2 * row] = rejected ? SAMPLING_NO_TOKEN : child;
-      decisions[2 * row + 1] = rejected ? 1u : 0u;
+      decisions[SAMPLING_DECISION_WORDS * row] = rejected ? SAMPLING_NO_TOKEN : child;
+      decisions[SAMPLING_DECISION_WORDS * row + 1] = rejected ? 1u : 0u;
     }
   } else if (blockIdx.x % kPerRow == 0 && threadIdx.x == 0) {
-    decisions[2 * row] = SAMPLING_NO_TOKEN;
-    decisions[2 * row + 1] = 0u;
+    decisions[SAMPLING_DECISION_WORDS * row] = SAMPLING_NO_TOKEN;
+    decisions[SAMPLING_DECISION_WORDS * row + 1] = 0u;
   }
   if (child != SAMPLING_NO_TOKEN && child < p.vocabulary && !rejected) return;  // accepted: nothing to draw
   // the range's residual: a lane sums its tokens in id order, the lanes are added in order
@@ -238,7 +450,7 @@ __global__ __launch_bounds__(256) void decode_sample_residual_ranges(const float
   float sum = 0.f;
   for (uint32_t i = 0; i < per; ++i) {
     const uint32_t token = begin + lane * per + i;
-    if (token < end) sum += residual_of(x[token], rejected ? q[token] : 0.f, mass, inverse, rejected);
+    if (token < end) sum += residual_of(x[token], token, rejected ? q[token] : 0.f, kept, inverse, rejected);
   }
   float total = 0.f;
   for (int l = 0; l < 64; ++l) total += __shfl(sum, l, 64);
@@ -256,14 +468,14 @@ __global__ __launch_bounds__(64) void decode_sample_draw(const float *__restrict
   const uint32_t row = blockIdx.x, lane = threadIdx.x;
   const uint32_t laneIndex = lane_of_row(p, row);
   if (!((p.sampling_mask >> laneIndex) & 1u)) return;  // a greedy lane keeps its argmax
-  const uint32_t decision = decisions[2 * row];
+  const uint32_t decision = decisions[SAMPLING_DECISION_WORDS * row];
   if (decision != SAMPLING_NO_TOKEN) {
     if (lane == 0) tokens[row] = decision;
     return;
   }
-  const bool rejected = decisions[2 * row + 1] == 1u;
+  const bool rejected = decisions[SAMPLING_DECISION_WORDS * row + 1] == 1u;
   const float inverse = 1.0f / p.temperature[laneIndex];
-  const Mass mass = row_mass(masses, row, inverse);
+  const Kept kept = row_kept(masses, decisions, row, inverse, (p.truncating_mask >> laneIndex) & 1u);
   const float *x = logits + size_t(row) * p.logits_stride, *q = draft + size_t(row) * p.logits_stride;
   const float *r = ranges + row * SAMPLING_RANGES;
   float total = 0.f;
@@ -292,7 +504,7 @@ __global__ __launch_bounds__(64) void decode_sample_draw(const float *__restrict
   float sum = 0.f;
   for (uint32_t i = 0; i < per; ++i) {
     const uint32_t token = begin + lane * per + i;
-    if (token < end) sum += residual_of(x[token], rejected ? q[token] : 0.f, mass, inverse, rejected);
+    if (token < end) sum += residual_of(x[token], token, rejected ? q[token] : 0.f, kept, inverse, rejected);
   }
   uint32_t chunk = 64, lastChunk = 0;
   float chunkBefore = 0.f, lastChunkBefore = 0.f, cumulative = 0.f;
@@ -310,7 +522,7 @@ __global__ __launch_bounds__(64) void decode_sample_draw(const float *__restrict
     for (uint32_t i = 0; i < per; ++i) {
       const uint32_t token = begin + chunk * per + i;
       if (token >= end) break;
-      const float w = residual_of(x[token], rejected ? q[token] : 0.f, mass, inverse, rejected);
+      const float w = residual_of(x[token], token, rejected ? q[token] : 0.f, kept, inverse, rejected);
       if (w > 0.f) lastToken = token;
       walked += w;
       if (selected == SAMPLING_NO_TOKEN && w > 0.f && target < walked) selected = token;

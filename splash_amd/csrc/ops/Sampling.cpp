@@ -25,7 +25,7 @@ SamplingWorkspaceSize Sampling::workspace(uint32_t rows) noexcept {
   size.partialIndices = uint64_t{rows} * SAMPLING_SHARDS * 4;
   size.masses = uint64_t{rows} * SAMPLING_SHARDS * 8;
   size.ranges = uint64_t{rows} * SAMPLING_RANGES * 4;
-  size.decisions = uint64_t{rows} * 8;
+  size.decisions = uint64_t{rows} * SAMPLING_DECISION_WORDS * 4;
   return size;
 }
 
@@ -43,6 +43,13 @@ void Sampling::addVerify(hip::CommandGraph &graph, const SamplingBuffers &b, uin
     params.lane[l] = {lanes[l].first, lanes[l].rows};
     params.temperature[l] = policies[l].samples() ? policies[l].temperature : 1.0f;
     if (policies[l].samples()) params.sampling_mask |= 1u << l;
+    const SamplingPolicy &policy = policies[l];
+    if (!(policy.minP >= 0.0f) || !(policy.topP > 0.0f) || !(policy.temperature >= 0.0f))
+      throw std::invalid_argument("a sampling policy takes a temperature and a min_p of at least 0 and a top_p above 0");
+    if (policy.truncates(vocabulary)) params.truncating_mask |= 1u << l;
+    params.min_p[l] = policy.minP;
+    params.top_k[l] = policy.topK;
+    params.top_p[l] = policy.topP;
   }
   const SamplingWorkspaceSize need = workspace(rows);
   requireBytes(b.logits, (uint64_t{rows - 1} * logitsStride + vocabulary) * 4, "logits");
@@ -64,6 +71,8 @@ void Sampling::addVerify(hip::CommandGraph &graph, const SamplingBuffers &b, uin
   graph.add("decode_sample_argmax_reduce", {b.partialValues, b.partialIndices, b.tokens}, params, {rows, 1, 1}, {64, 1, 1});
   if (!params.sampling_mask) return;
   graph.add("decode_sample_mass_sharded", {b.logits, b.masses}, params, {rows * SAMPLING_SHARDS, 1, 1}, {SAMPLING_THREADS, 1, 1});
+  if (params.truncating_mask)
+    graph.add("decode_sample_distribution_end", {b.logits, b.masses, b.decisions}, params, {rows, 1, 1}, {SAMPLING_THREADS, 1, 1});
   graph.add("decode_sample_residual_ranges",
             {b.logits, b.draftProbabilities, b.masses, b.uniforms, b.treeRows, b.inputTokens, b.ranges, b.decisions}, params,
             {rows * (SAMPLING_RANGES / 4), 1, 1}, {256, 1, 1});

@@ -1,6 +1,7 @@
 // Acceptance of a verify block: ops::Sampling (runtime/ops/Sampling.hpp:64-254, Sampling.cpp:283-357
 // in the reference) over kernels/sampling.hip. addVerify selects each row's token (argmax, or
-// rejection sampling over the row's drafted child at temperature > 0); addAcceptance walks each
+// rejection sampling over the row's drafted child at temperature > 0, from the distribution the
+// lane's min_p, top_k and top_p leave); addAcceptance walks each
 // lane's block from its first row and writes the retained tokens, counts and retained-row mask.
 #pragma once
 #include "abi/Sampling.h"
@@ -11,11 +12,20 @@
 
 namespace splash::ops {
 
-// Sampling.hpp:64-110 in the reference, reduced to what the verify configurations use.
+// Sampling.hpp:56-83 in the reference, without penalties, constraints and the thinking cutoff.
 struct SamplingPolicy final {
   float temperature = 0.0f;
-  // Sampling.cpp:78-89: a policy samples iff temperature > 0.
-  [[nodiscard]] bool samples() const noexcept { return temperature > 0.0f; }
+  // A sampling lane keeps the tokens minP leaves it (those that weigh at least minP of the
+  // heaviest; 0 drops none), then its topK most likely of those (0, or a topK past the vocabulary:
+  // all), then its topP nucleus of those.
+  float minP = 0.0f;
+  uint32_t topK = 0;
+  float topP = 1.0f;
+  // A lane samples unless it keeps only its most likely token (Sampling.hpp:79-82).
+  [[nodiscard]] bool samples() const noexcept { return temperature > 0.0f && minP < 1.0f && topK != 1; }
+  [[nodiscard]] bool truncates(uint32_t vocabulary) const noexcept {
+    return samples() && (minP > 0.0f || (topK && topK < vocabulary) || topP < 1.0f);
+  }
 };
 
 struct LaneRows final {
@@ -32,7 +42,8 @@ struct SamplingBuffers final {
   // sampled rows only:
   hip::Buffer draftProbabilities;  // fp32 [rows][stride]: the distribution each row's child was drawn from
   hip::Buffer uniforms;            // fp32 [rows][2]: the row's draw, its child's test
-  hip::Buffer masses, ranges, decisions;
+  hip::Buffer masses, ranges;
+  hip::Buffer decisions;  // SAMPLING_DECISION_WORDS words a row: its child's test and the end of its distribution
   hip::Buffer inputTokens, treeRows;  // the block's input tokens and SplashTreeRow rows
 };
 struct AcceptanceBuffers final {

@@ -373,12 +373,14 @@ class Sampling:
         return list(sizes)
 
     @staticmethod
-    def add_verify(graph, buffers, vocabulary, stride, lanes, temperatures):
-        """buffers: dict of Buffer by the names of spo_sampling_buffers; lanes: [(first, rows)]."""
+    def add_verify(graph, buffers, vocabulary, stride, lanes, policies):
+        """buffers: dict of Buffer by the names of spo_sampling_buffers; lanes: [(first, rows)]; policies: a lane's
+        temperature, or (temperature, min_p, top_k, top_p)."""
         b = nat.SamplingBuffers(**{k: (v.handle if v is not None else None) for k, v in buffers.items()})
         arr = (nat.LaneRows * len(lanes))(*[nat.LaneRows(*l) for l in lanes])
-        temps = (ctypes.c_float * len(lanes))(*temperatures)
-        check(lib.spo_sampling_add_verify(graph.handle, ctypes.byref(b), vocabulary, stride, arr, temps, len(lanes)))
+        full = [p if isinstance(p, (tuple, list)) else (p, 0.0, 0, 1.0) for p in policies]
+        structs = (nat.SamplingPolicy * len(lanes))(*[nat.SamplingPolicy(*p) for p in full])
+        check(lib.spo_sampling_add_verify(graph.handle, ctypes.byref(b), vocabulary, stride, arr, structs, len(lanes)))
         graph._keep.extend(list(buffers.values()))
 
     @staticmethod

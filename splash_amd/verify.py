@@ -15,11 +15,13 @@ from . import ops
 
 
 class Lane:
-    def __init__(self, rows, committed, table_first=0, temperature=0.0, remaining=0xFFFFFFFF):
+    def __init__(self, rows, committed, table_first=0, temperature=0.0, remaining=0xFFFFFFFF, min_p=0.0, top_k=0, top_p=1.0):
         self.rows, self.committed, self.table_first, self.temperature, self.remaining = rows, committed, table_first, temperature, remaining
+        self.min_p, self.top_k, self.top_p = min_p, top_k, top_p
 
     def struct(self):
-        return nat.VerifyLane(self.rows, self.committed, self.table_first, self.temperature, self.remaining)
+        return nat.VerifyLane(self.rows, self.committed, self.table_first, self.temperature, self.remaining, self.min_p, self.top_k,
+                              self.top_p)
 
 
 class DenseVerify:

@@ -227,6 +227,48 @@ def rejection_row(logits, temperature, q, draft_token, u_child, u_row):
     return tok, bool(acc.value), close.value
 
 
+class SamplingPolicy(ctypes.Structure):
+    _fields_ = [("temperature", c_f), ("min_p", c_f), ("top_k", c_u32), ("top_p", c_f)]
+
+
+def distribution_end(logits, temperature, min_p=0.0, top_k=0, top_p=1.0):
+    """Returns (key, last id, kept mass, kept count, closeness)."""
+    x = np.ascontiguousarray(logits, dtype=np.float32)
+    policy = SamplingPolicy(temperature, min_p, top_k, top_p)
+    key, last, mass, close = c_u32(), c_u32(), c_f(), ctypes.c_double()
+    lib.orc_distribution_end.restype = c_u32
+    count = lib.orc_distribution_end(_p(x, f32p), c_u32(x.size), ctypes.byref(policy), ctypes.byref(key), ctypes.byref(last),
+                                     ctypes.byref(mass), ctypes.byref(close))
+    return key.value, last.value, mass.value, count, close.value
+
+
+def rejection_row_policy(logits, policy, q, draft_token, u_child, u_row):
+    """policy: (temperature, min_p, top_k, top_p). Returns (token, accepted_draft, closeness)."""
+    x = np.ascontiguousarray(logits, dtype=np.float32)
+    qq = np.ascontiguousarray(q, dtype=np.float32) if q is not None else None
+    acc, close = c_int(), ctypes.c_double()
+    lib.orc_rejection_row_policy.restype = c_u32
+    tok = lib.orc_rejection_row_policy(_p(x, f32p), c_u32(x.size), ctypes.byref(SamplingPolicy(*policy)), _p(qq, f32p), c_u32(draft_token),
+                                       c_f(u_child), c_f(u_row), ctypes.byref(acc), ctypes.byref(close))
+    return tok, bool(acc.value), close.value
+
+
+def rejection_law_policy(logits, policy, q):
+    x = np.ascontiguousarray(logits, dtype=np.float32)
+    qq = np.ascontiguousarray(q, dtype=np.float32)
+    out = np.empty(x.size, dtype=np.float64)
+    lib.orc_rejection_law_policy.restype = None
+    lib.orc_rejection_law_policy(_p(x, f32p), c_u32(x.size), ctypes.byref(SamplingPolicy(*policy)), _p(qq, f32p), _p(out, f64p))
+    return out
+
+
+def logit_key(values):
+    """The order-preserving unsigned key of fp32 logits (sampling.metal:197-207), vectorised."""
+    bits = np.ascontiguousarray(values, dtype=np.float32).view(np.uint32).copy()
+    bits[(bits << np.uint32(1)) == 0] = 0
+    return np.where(bits & 0x80000000, ~bits, bits | np.uint32(0x80000000)).astype(np.uint32)
+
+
 def rejection_law(logits, temperature, q):
     x = np.ascontiguousarray(logits, dtype=np.float32)
     qq = np.ascontiguousarray(q, dtype=np.float32)

@@ -171,3 +171,56 @@ def test_rejection_sampling_rows_match_oracle(backend):
     backend.run(g)
     mixed = b["tokens"].download(np.uint32)
     assert all(mixed[r] == orc.argmax(logits[r]) for r in range(8))
+
+
+@pytest.mark.parametrize("ties", [False, True])
+def test_truncated_distributions_match_oracle(backend, ties):
+    """min_p, top_k and top_p (distribution_end, sampling.metal:603-670): the end of every row's distribution -- the
+    last kept token's key and id, the kept count -- equals the oracle's sort, the kept mass to fp32 summation order,
+    and the rows' selections the oracle's over the cut distribution, except where a comparison lies within 1e-5 of its
+    threshold. With ties: logits on a grid of halves, so that top_k and the nucleus end inside runs of equal logits."""
+    print(f"case truncated sampling ties={ties}", flush=True)
+    rng = np.random.default_rng(11 + ties)
+    V = 151936 if not ties else 40000
+    lanes = [(0, 3), (3, 3), (6, 3), (9, 3), (12, 2), (14, 1), (15, 1)]
+    policies = [(0.7, 0.0, 50, 1.0), (0.7, 0.0, 0, 0.9), (1.2, 0.02, 0, 1.0), (0.5, 0.001, 1000, 0.95), (0.7, 0.0, V + 1, 1.0), (0.9, 0.0, 2, 0.5),
+                (0.0, 0.0, 0, 1.0)]
+    rows = 16
+    logits = (rng.standard_normal((rows, V)) * 2.5).astype(np.float32)
+    if ties:
+        logits = (np.round(logits * 2) / 2).astype(np.float32)
+    logits[4, rng.random(V) < 0.01] = -np.inf
+    dl = rng.standard_normal((rows, V)) * 2
+    draft = np.exp(dl - dl.max(axis=1, keepdims=True)); draft = (draft / draft.sum(axis=1, keepdims=True)).astype(np.float32)
+    tokens = np.zeros(rows, dtype=np.uint32)
+    tree = ops.chain_tree_rows([n for _, n in lanes])
+    for first, n in lanes:        # a lane's row r + 1 carries the child drawn at its row r: a likely token, or a draft draw
+        for r in range(first + 1, first + n):
+            d64 = draft[r - 1].astype(np.float64)
+            tokens[r] = int(np.argmax(logits[r - 1])) if r % 2 else int(rng.choice(V, p=d64 / d64.sum()))
+    uniforms = rng.random((rows, 2)).astype(np.float32)
+    b = sampling_buffers(backend, rows, V, logits, draft, uniforms, tokens, tree)
+    g = splash_amd.CommandGraph()
+    ops.Sampling.add_verify(g, b, V, V, lanes, policies)
+    backend.run(g)
+    got = b["tokens"].download(np.uint32)
+    words = b["decisions"].download(np.uint32).reshape(rows, 8)
+    checked = 0
+    for (first, n), policy in zip(lanes, policies):
+        T, min_p, top_k, top_p = policy
+        for r in range(first, first + n):
+            if T == 0.0:
+                assert got[r] == orc.argmax(logits[r])
+                continue
+            cuts = min_p > 0 or (top_k and top_k < V) or top_p < 1
+            key, last, mass, count, close_end = orc.distribution_end(logits[r], T, min_p, top_k, top_p)
+            if cuts and close_end > 1e-5:
+                assert (words[r, 2], words[r, 3], words[r, 5]) == (key, last, count), (r, policy)
+                assert abs(words[r, 4:5].view(np.float32)[0] - mass) <= 1e-5 * mass
+            child = int(tokens[r + 1]) if r + 1 < first + n else orc.NO_TOKEN
+            want, accepted, close = orc.rejection_row_policy(logits[r], policy, draft[r] if child != orc.NO_TOKEN else None, child,
+                                                             float(uniforms[r, 1]), float(uniforms[r, 0]))
+            if close > 1e-5:
+                assert got[r] == want, (r, policy, got[r], want, accepted)
+                checked += 1
+    assert checked >= 12

@@ -125,3 +125,75 @@ def test_rejection_row_accepts_iff_uq_below_p():
             if close > 1e-5:
                 assert accepted == (u * q[child] < p[child])
                 assert (tok == child) if accepted else (p[tok] > q[tok])   # a redraw comes from max(p - q, 0)
+
+
+def brute_force_end(x, T, min_p, top_k, top_p):
+    """distribution_end (sampling.metal:603-670) from its description alone, in fp64: the kept token ids, in order."""
+    finite = np.isfinite(x) | (x == np.inf)
+    ids = np.nonzero(finite)[0]
+    keys = orc.logit_key(x[ids]).astype(np.int64)
+    order = ids[np.lexsort((ids, -keys))]
+    mx = x[order[0]]
+    w = np.exp((x[order].astype(np.float64) - float(mx)) / T)
+    keep = len(order)
+    if min_p > 0:
+        threshold = np.float32(min(np.float32(mx) + np.float32(T) * np.float32(np.log(np.float32(min_p))), np.float32(mx)))
+        keep = int((orc.logit_key(x[order]) >= orc.logit_key(np.array([threshold], np.float32))[0]).sum())
+    if top_k and top_k < keep:
+        keep = top_k
+    mass = w[:keep].sum()
+    margin = 1.0
+    if top_p < 1:
+        cumulative = np.cumsum(w[:keep])
+        target = float(np.float32(top_p) * np.float32(mass))
+        crossing = np.nonzero(cumulative > target)[0]
+        if len(crossing):
+            keep = int(crossing[0]) + 1
+            margin = min(abs(cumulative[keep - 1] - target), abs(cumulative[keep - 2] - target) if keep > 1 else 1.0) / target
+    return order[:keep], margin
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_distribution_end_against_a_sort(seed):
+    """min_p, then top_k, then top_p, in the order of the logits with ties to the smaller id: the oracle's end keeps
+    exactly the tokens a sort keeps, also where whole runs of tokens share a logit."""
+    rng = np.random.default_rng(100 + seed)
+    V = int(rng.integers(5, 3000))
+    x = (rng.standard_normal(V) * 2.5).astype(np.float32)
+    if seed % 2:
+        x = (np.round(x * 2) / 2).astype(np.float32)      # many ties
+    x[rng.random(V) < 0.05] = -np.inf
+    x[0] = max(x[0], np.float32(0))
+    T = float(np.float32(rng.uniform(0.3, 1.5)))
+    for min_p, top_k, top_p in [(0.0, 0, 1.0), (0.05, 0, 1.0), (0.0, 7, 1.0), (0.0, 0, 0.9), (0.02, 40, 0.8), (0.0, V + 5, 0.5), (0.3, 2, 0.99)]:
+        min_p, top_p = float(np.float32(min_p)), float(np.float32(top_p))
+        kept, margin = brute_force_end(x, T, min_p, top_k, top_p)
+        key, last, mass, count, closeness = orc.distribution_end(x, T, min_p, top_k, top_p)
+        if margin < 1e-6:
+            continue
+        assert count == len(kept), (min_p, top_k, top_p)
+        keys, ids = orc.logit_key(x), np.arange(V)
+        stays = np.isfinite(x) & ((keys > key) | ((keys == key) & (ids <= last)))
+        assert np.array_equal(np.sort(kept), np.nonzero(stays)[0])
+        w = np.exp((x[kept].astype(np.float64) - float(x[kept[0]])) / T)
+        assert abs(mass - w.sum()) <= 1e-5 * w.sum()
+
+
+def test_truncated_rejection_law_is_the_renormalized_kept_distribution():
+    """The selection law of test-then-residual over a cut distribution is that distribution renormalized, whatever the
+    draft proposes (also tokens outside it), and a row's draw never leaves it."""
+    rng = np.random.default_rng(7)
+    for V, policy in ((14, (0.7, 0.0, 5, 1.0)), (40, (1.1, 0.05, 0, 0.9)), (300, (0.7, 0.01, 50, 0.7))):
+        x = (rng.standard_normal(V) * 3).astype(np.float32)
+        q = np.exp(rng.standard_normal(V) * 2); q = (q / q.sum()).astype(np.float32)
+        T = float(np.float32(policy[0]))
+        kept, _ = brute_force_end(x, T, float(np.float32(policy[1])), policy[2], float(np.float32(policy[3])))
+        p = np.zeros(V)
+        p[kept] = np.exp((x[kept].astype(np.float64) - float(x.max())) / T)
+        p /= p.sum()
+        law = orc.rejection_law_policy(x, policy, q)
+        assert np.abs(law - p).max() < 1e-12
+        for _ in range(200):
+            child = int(rng.integers(0, V))
+            tok, accepted, _ = orc.rejection_row_policy(x, policy, q, child, float(rng.random()), float(rng.random()))
+            assert p[tok] > 0 and (not accepted or tok == child)
