@@ -135,6 +135,11 @@ sp_status spo_norm_add_rms_table(spo_graph *graph, sp_buffer *input, sp_buffer *
                                  sp_buffer *table, uint32_t width, uint32_t rows);
 sp_status spo_embedding_add(spo_graph *graph, uint32_t format, sp_buffer *native_rows, uint32_t vocabulary,
                             uint32_t hidden, sp_buffer *tokens, sp_buffer *output, uint32_t rows);
+/* RowCopy::add (runtime/ops/RowCopy.hpp:9-28): `rows` rows of `width` bf16 values from row from_row of `source`
+ * (rows from_stride values apart, from value from_column on) to the like region of `destination`. */
+sp_status spo_row_copy_add(spo_graph *graph, sp_buffer *source, uint32_t from_row, uint32_t from_stride, uint32_t from_column,
+                           sp_buffer *destination, uint32_t to_row, uint32_t to_stride, uint32_t to_column, uint32_t rows,
+                           uint32_t width);
 typedef struct spo_rope_sequence { uint32_t first_row, rows, anchor; } spo_rope_sequence;
 sp_status spo_rope_add_tree_tables(spo_graph *graph, sp_buffer *inverse_frequency, sp_buffer *depth, sp_buffer *cosines,
                                    sp_buffer *sines, uint32_t pairs, const spo_rope_sequence *sequences, uint32_t count);

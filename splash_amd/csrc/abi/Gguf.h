@@ -53,8 +53,11 @@
 #define GGUF_Q6K_SCALES 3072u
 #define GGUF_Q6K_D 3328u
 #define GGUF_ROW_TILE 16u
-// The most rows one projection dispatch takes: four lanes of sixteen verify rows.
+// The most rows one workgroup takes: four lanes of sixteen verify rows. A dispatch of more rows
+// (eight lanes) runs pieces of this many rows side by side (grid.y); a piece's activation table,
+// output and residual rows, partials and counters follow those of the piece before it.
 #define GGUF_MAXIMUM_ROWS 64u
+#define GGUF_MAXIMUM_DISPATCH_ROWS 256u
 #define GGUF_MAXIMUM_SEGMENTS 3u
 #define GGUF_MAXIMUM_SPLITS 16u
 
@@ -87,6 +90,13 @@ GGUF_INLINE uint64_t gguf_table_sums16_offset(uint32_t k, uint32_t tiles) {
 }
 GGUF_INLINE uint64_t gguf_table_bytes(uint32_t k, uint32_t tiles) {
   return gguf_table_sums16_offset(k, tiles) + uint64_t(tiles) * (k / 16u) * 16u * 4u;
+}
+// Row tiles of a piece, and the tables of `tiles` row tiles in all: whole pieces' tables of four row
+// tiles each, then the last piece's (the single table of up to four row tiles is its own case).
+#define GGUF_PIECE_TILES (GGUF_MAXIMUM_ROWS / GGUF_ROW_TILE)
+GGUF_INLINE uint64_t gguf_tables_bytes(uint32_t k, uint32_t tiles) {
+  const uint32_t whole = tiles / GGUF_PIECE_TILES, rest = tiles % GGUF_PIECE_TILES;
+  return whole * gguf_table_bytes(k, GGUF_PIECE_TILES) + (rest ? gguf_table_bytes(k, rest) : 0u);
 }
 #endif
 

@@ -27,7 +27,16 @@ struct RopeTreeParams {
   uint32_t anchor[8];     // position of the sequence's row 0
 };
 
+// copy_rows_bf16: `rows` rows of `width` bf16 values between two row regions (the reference's
+// RowCopyParams, abi/RowCopy.h). One thread per value.
+struct RowCopyParams {
+  uint32_t rows, width;
+  uint32_t from_row, from_stride, from_column;
+  uint32_t to_row, to_stride, to_column;
+};
+
 #ifdef __cplusplus
+static_assert(sizeof(RowCopyParams) == 32, "row copy parameters are 32 bytes on both sides");
 static_assert(sizeof(NormParams) == 16, "norm parameters are 16 bytes on both sides");
 static_assert(sizeof(RopeTreeParams) == 112, "RoPE tree parameters are 112 bytes on both sides");
 #endif

@@ -55,6 +55,14 @@ sp_status spo_embedding_add(spo_graph *graph, uint32_t format, sp_buffer *native
     ops::Embedding::add(capi::graphOf(graph), {B(native_rows), format, vocabulary, hidden}, B(tokens), B(output), rows);
   });
 }
+sp_status spo_row_copy_add(spo_graph *graph, sp_buffer *source, uint32_t from_row, uint32_t from_stride, uint32_t from_column,
+                           sp_buffer *destination, uint32_t to_row, uint32_t to_stride, uint32_t to_column, uint32_t rows, uint32_t width) {
+  return capi::guard([&] {
+    capi::require(graph, "graph");
+    ops::RowCopy::add(capi::graphOf(graph), B(source), {from_row, from_stride, from_column}, B(destination), {to_row, to_stride, to_column},
+                      rows, width);
+  });
+}
 sp_status spo_rope_add_tree_tables(spo_graph *graph, sp_buffer *inverse_frequency, sp_buffer *depth, sp_buffer *cosines,
                                    sp_buffer *sines, uint32_t pairs, const spo_rope_sequence *sequences, uint32_t count) {
   return capi::guard([&] {

@@ -85,7 +85,7 @@ sp_status spo_graph_record(sp_backend *backend, const spo_graph *graph, sp_comma
 uint64_t spo_gguf_image_bytes(uint32_t format, uint32_t rows, uint32_t input_size) {
   return gguf_image_bytes(format, rows, input_size);
 }
-uint64_t spo_gguf_table_bytes(uint32_t input_size, uint32_t rows) { return gguf_table_bytes(input_size, gguf_row_tiles(rows)); }
+uint64_t spo_gguf_table_bytes(uint32_t input_size, uint32_t rows) { return gguf_tables_bytes(input_size, gguf_row_tiles(rows)); }
 sp_status spo_gguf_pack_image(uint32_t format, const uint8_t *native, uint32_t rows, uint32_t input_size, uint8_t *image) {
   return capi::guard([&] { capi::require(native && image, "rows or image"); ops::packGgufImage(format, native, rows, input_size, image); });
 }

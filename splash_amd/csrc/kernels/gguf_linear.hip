@@ -29,8 +29,12 @@ constexpr int kUnitTiles = 2;  // column tiles per wave
 // ---------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(64) void gguf_prepare_table(const uint16_t *__restrict__ input, uint8_t *__restrict__ table,
                                                          GgufPrepareParams p) {
-  const uint32_t g = blockIdx.x, t = blockIdx.y, lane = threadIdx.x, r = lane & 15u, kq = lane >> 4;
-  const uint32_t G = p.input_size / 32u, row = 16u * t + r;
+  const uint32_t g = blockIdx.x, lane = threadIdx.x, r = lane & 15u, kq = lane >> 4;
+  const uint32_t G = p.input_size / 32u, row = 16u * blockIdx.y + r;
+  // Row tile blockIdx.y is tile t of its piece's table, which holds `tiles` row tiles.
+  const uint32_t piece = blockIdx.y / GGUF_PIECE_TILES, t = blockIdx.y % GGUF_PIECE_TILES;
+  const uint32_t tiles = min(uint32_t(GGUF_PIECE_TILES), p.tiles - piece * GGUF_PIECE_TILES);
+  table += piece * gguf_table_bytes(p.input_size, GGUF_PIECE_TILES);
   float v[8];
 #pragma unroll
   for (uint32_t e = 0; e < 8; ++e) v[e] = 0.f;
@@ -61,8 +65,8 @@ __global__ __launch_bounds__(64) void gguf_prepare_table(const uint16_t *__restr
   }
   const float s0 = ((h0[0] + h0[1]) + h0[2]) + h0[3], s1 = ((h1[0] + h1[1]) + h1[2]) + h1[3];
   if (kq == 0) {
-    float *sums32 = reinterpret_cast<float *>(table + gguf_table_sums32_offset(p.input_size, p.tiles));
-    float *sums16 = reinterpret_cast<float *>(table + gguf_table_sums16_offset(p.input_size, p.tiles));
+    float *sums32 = reinterpret_cast<float *>(table + gguf_table_sums32_offset(p.input_size, tiles));
+    float *sums16 = reinterpret_cast<float *>(table + gguf_table_sums16_offset(p.input_size, tiles));
     sums32[(size_t(t) * G + g) * 16u + r] = s0 + s1;
     sums16[(size_t(t) * 2u * G + 2u * g) * 16u + r] = s0;
     sums16[(size_t(t) * 2u * G + 2u * g + 1u) * 16u + r] = s1;
@@ -581,6 +585,20 @@ __global__ __launch_bounds__(256) void gguf_decode(const uint8_t *__restrict__ s
                                                    void *__restrict__ out, const uint16_t *__restrict__ residual,
                                                    float *__restrict__ partials, uint32_t *__restrict__ counters,
                                                    GgufDecodeParams p) {
+  // Piece blockIdx.y: rows 64 y .. of the dispatch's, with its own table, rows, partials and counters.
+  if (const uint32_t piece = blockIdx.y) {
+    const uint32_t first = piece * GGUF_MAXIMUM_ROWS, partitioned = (p.units + 3u) / 4u - p.whole_groups;
+    const size_t rowBytes = size_t(p.out_stride) * (EP == GGUF_EPILOGUE_PLAIN_F32 ? 4u : 2u);
+    table += piece * gguf_table_bytes(p.input_size, GGUF_PIECE_TILES);
+    out = static_cast<uint8_t *>(out) + first * rowBytes;
+    if constexpr (EP == GGUF_EPILOGUE_GATE_UP_TABLE)
+      residual = reinterpret_cast<const uint16_t *>(reinterpret_cast<const uint8_t *>(residual) + piece * gguf_table_bytes(p.out_stride, GGUF_PIECE_TILES));
+    else residual += size_t(first) * p.out_stride;
+    partials += size_t(piece) * p.splits * partitioned * 4u * RT * 256u;
+    counters += piece * partitioned;
+    p.rows -= first;
+  }
+  p.rows = min(p.rows, uint32_t(GGUF_MAXIMUM_ROWS));
   decode_workgroup<FMT, RT, EP>(seg0, seg1, seg2, table, out, residual, partials, counters, p, blockIdx.x);
 }
 

@@ -70,7 +70,11 @@ __global__ __launch_bounds__(256) void norm_rms_table16(const uint16_t *__restri
                                                         uint16_t *__restrict__ output, uint8_t *__restrict__ table, NormParams p) {
   __shared__ float scratch[4];
   __shared__ __align__(16) uint16_t rowX[kStagedWidth], rowW[kStagedWidth];
-  const uint32_t row = blockIdx.x, tile = row / 16u, r = row % 16u, G = p.width / 32u;
+  const uint32_t row = blockIdx.x, r = row % 16u, G = p.width / 32u;
+  // Row tile row / 16 is tile `tile` of its piece's table, which holds `tiles` row tiles.
+  const uint32_t piece = row / 16u / GGUF_PIECE_TILES, tile = row / 16u % GGUF_PIECE_TILES;
+  const uint32_t tiles = min(uint32_t(GGUF_PIECE_TILES), p.tiles - piece * GGUF_PIECE_TILES);
+  table += piece * gguf_table_bytes(p.width, GGUF_PIECE_TILES);
   const bool live = row < p.rows;
   const uint16_t *x = input + size_t(live ? row : 0) * p.width, *w = weight;
   if (live && p.width <= kStagedWidth) {  // the width is a multiple of 256
@@ -82,8 +86,8 @@ __global__ __launch_bounds__(256) void norm_rms_table16(const uint16_t *__restri
   }
   const float inverse = live ? rms_inverse(x, p.width, scratch) : 0.f;
   uint2 *values = reinterpret_cast<uint2 *>(table);
-  float *sums32 = reinterpret_cast<float *>(table + gguf_table_sums32_offset(p.width, p.tiles));
-  float *sums16 = reinterpret_cast<float *>(table + gguf_table_sums16_offset(p.width, p.tiles));
+  float *sums32 = reinterpret_cast<float *>(table + gguf_table_sums32_offset(p.width, tiles));
+  float *sums16 = reinterpret_cast<float *>(table + gguf_table_sums16_offset(p.width, tiles));
   // run q covers inputs 4 q .. 4 q + 3: group g = q / 8, half = (q / 4) % 2, kq = q % 4
   for (uint32_t q = threadIdx.x; q < p.width / 4u; q += 256) {
     uint32_t bits[4] = {0, 0, 0, 0};
@@ -115,6 +119,16 @@ __global__ __launch_bounds__(256) void norm_rms_table16(const uint16_t *__restri
   }
 }
 SP_REGISTER_KERNEL("norm_rms_table16", &norm_rms_table16);
+
+// copy_rows_bf16: grid (ceil(rows * width / 256)), 256 threads.
+__global__ __launch_bounds__(256) void copy_rows_bf16(const uint16_t *__restrict__ source, uint16_t *__restrict__ destination, RowCopyParams p) {
+  const uint64_t index = uint64_t(blockIdx.x) * 256u + threadIdx.x;
+  if (index >= uint64_t(p.rows) * p.width) return;
+  const uint32_t row = uint32_t(index / p.width), column = uint32_t(index % p.width);
+  destination[(size_t(p.to_row) + row) * p.to_stride + p.to_column + column] =
+      source[(size_t(p.from_row) + row) * p.from_stride + p.from_column + column];
+}
+SP_REGISTER_KERNEL("copy_rows_bf16", &copy_rows_bf16);
 
 __global__ void rope_build_tree_tables(const float *__restrict__ inverse_frequency, const uint32_t *__restrict__ depth,
                                        float *__restrict__ cosines, float *__restrict__ sines, RopeTreeParams p) {

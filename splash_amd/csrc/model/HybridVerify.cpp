@@ -10,7 +10,7 @@ using hip::BufferStorage;
 
 namespace {
 // Rows one projection dispatch takes: a longer step runs its dense projections in pieces.
-constexpr uint32_t kProjectionRows = ops::kMaximumDecodeTileRows;
+constexpr uint32_t kProjectionRows = ops::kMaximumDispatchRows;
 template <class F> void forRowPieces(uint32_t rows, F &&piece) {
   for (uint32_t first = 0; first < rows; first += kProjectionRows) piece(first, std::min(kProjectionRows, rows - first));
 }

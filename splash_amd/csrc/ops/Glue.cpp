@@ -22,10 +22,10 @@ void Normalization::addRms(hip::CommandGraph &graph, const hip::Buffer &input, c
 PreparedInput Normalization::addRmsTable(hip::CommandGraph &graph, const hip::Buffer &input, const hip::Buffer &weight,
                                          const hip::Buffer &output, const LinearScratch &scratch, uint32_t width, uint32_t rows) {
   requireNorm(input, weight, output, width, rows);
-  if (width % GGUF_BLOCK || rows > kMaximumDecodeTileRows)
-    throw std::invalid_argument("the activation table takes up to 64 rows of whole 256-input super-blocks");
+  if (width % GGUF_BLOCK || rows > kMaximumDispatchRows)
+    throw std::invalid_argument("the activation table takes up to 256 rows of whole 256-input super-blocks");
   const uint32_t tiles = gguf_row_tiles(rows);
-  requireBytes(scratch.input, gguf_table_bytes(width, tiles), "projection table");
+  requireBytes(scratch.input, gguf_tables_bytes(width, tiles), "projection table");
   graph.add("norm_rms_table16", {input, weight, output, scratch.input}, NormParams{width, rows, tiles, 0},
             {tiles * GGUF_ROW_TILE, 1, 1}, {256, 1, 1});
   return {output, LinearInput::Table16};
@@ -62,6 +62,18 @@ void RoPE::addTreeTables(hip::CommandGraph &graph, const hip::Buffer &inverseFre
   requireBytes(cosines, uint64_t{params.rows} * pairs * 4, "RoPE cosine table");
   requireBytes(sines, uint64_t{params.rows} * pairs * 4, "RoPE sine table");
   graph.add("rope_build_tree_tables", {inverseFrequency, depth, cosines, sines}, params, {params.rows, 1, 1}, {pairs, 1, 1});
+}
+
+void RowCopy::add(hip::CommandGraph &graph, const hip::Buffer &source, RowRegion from, const hip::Buffer &destination, RowRegion to,
+                  uint32_t rows, uint32_t width) {
+  if (!rows || !width || from.column + uint64_t{width} > from.stride || to.column + uint64_t{width} > to.stride)
+    throw std::invalid_argument("invalid row copy");
+  auto regionBytes = [&](RowRegion r) { return ((uint64_t{r.row} + rows - 1) * r.stride + r.column + width) * 2; };
+  requireBytes(source, regionBytes(from), "row copy source");
+  requireBytes(destination, regionBytes(to), "row copy destination");
+  graph.add("copy_rows_bf16", {source, destination},
+            RowCopyParams{rows, width, from.row, from.stride, from.column, to.row, to.stride, to.column},
+            {uint32_t((uint64_t{rows} * width + 255) / 256), 1, 1}, {256, 1, 1});
 }
 
 } // namespace splash::ops

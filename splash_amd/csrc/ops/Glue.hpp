@@ -46,4 +46,17 @@ public:
                             const std::vector<RopeSequence> &sequences);
 };
 
+// Rows of `stride` bf16 values from row `row` of a buffer, of which a copy reads or writes the values
+// from `column` on (RowCopy.hpp:9-15 in the reference).
+struct RowRegion final {
+  uint32_t row = 0, stride = 0, column = 0;
+};
+// Copies rows of bf16 values between two row regions: a capture layer's output rows into their slot
+// of the draft's captured target hidden rows (RowCopy.hpp:17-28, QwenTarget.cpp addCapture).
+class RowCopy final {
+public:
+  static void add(hip::CommandGraph &graph, const hip::Buffer &source, RowRegion from, const hip::Buffer &destination, RowRegion to,
+                  uint32_t rows, uint32_t width);
+};
+
 } // namespace splash::ops

@@ -55,7 +55,7 @@ LinearPlan::LinearPlan(LinearWorkload workload, LinearConfig config, FloatOutput
 
 void LinearPlan::requireConfiguration() const {
   const auto [n, k] = workload_.matrix;
-  if (!workload_.rows || workload_.rows > kMaximumDecodeTileRows)
+  if (!workload_.rows || workload_.rows > kMaximumDispatchRows)
     throw std::invalid_argument("the block tile runs plans of 1 to 64 rows");
   if (!n || n % GGUF_TILE_COLUMNS || !k || k % GGUF_BLOCK)
     throw std::invalid_argument("block projections take whole 16-column tiles and 256-input super-blocks");
@@ -71,13 +71,16 @@ LinearScratchSize LinearPlan::scratchSize() const noexcept {
   const auto [n, k] = workload_.matrix;
   const uint32_t tiles = gguf_row_tiles(workload_.rows);
   LinearScratchSize size;
-  size.input = gguf_table_bytes(k, tiles);
+  size.input = gguf_tables_bytes(k, tiles);
   if (config_.splits > 1) {
     // [split][unit][row tile][4][64 lanes] fp32 partials over whole workgroups, and one counter per workgroup.
     // of the partitioned workgroups only
     const uint64_t groups = std::max<uint64_t>(1, groupsOf(n, workload_.epilogue) - config_.wholeGroups);
-    size.partials = uint64_t{config_.splits} * groups * kWavesAcross * tiles * 256u * sizeof(float);
-    size.counters = groups * sizeof(uint32_t);
+    // a piece of the dispatch's rows keeps its own, as many as a whole piece takes
+    // (the kernel's row tiles: 1, 2 or 4, which may be more than the rows fill)
+    const uint32_t pieces = rowPieces(workload_.rows), pieceTiles = storageRows() / GGUF_ROW_TILE;
+    size.partials = uint64_t{pieces} * config_.splits * groups * kWavesAcross * pieceTiles * 256u * sizeof(float);
+    size.counters = uint64_t{pieces} * groups * sizeof(uint32_t);
   }
   return size;
 }
@@ -135,11 +138,11 @@ LinearScratchSize Linear::scratchSize(LinearMatrix matrix, uint32_t rows) const 
 
 void Linear::addPrepare(hip::CommandGraph &graph, const hip::Buffer &input, const LinearScratch &scratch, uint32_t width,
                         uint32_t rows) {
-  if (!rows || rows > kMaximumDecodeTileRows) throw std::invalid_argument("the block tile runs plans of 1 to 64 rows");
+  if (!rows || rows > kMaximumDispatchRows) throw std::invalid_argument("a block projection takes 1 to 256 rows");
   if (!width || width % GGUF_BLOCK) throw std::invalid_argument("block projections take whole 256-input super-blocks");
   const uint32_t tiles = gguf_row_tiles(rows);
   requireBytes(input, uint64_t{rows} * width * 2, "projection input");
-  requireBytes(scratch.input, gguf_table_bytes(width, tiles), "projection table");
+  requireBytes(scratch.input, gguf_tables_bytes(width, tiles), "projection table");
   graph.add("gguf_prepare_table", {input, scratch.input}, GgufPrepareParams{width, rows, tiles, width},
             {width / 32, tiles, 1}, {64, 1, 1});
 }
@@ -173,7 +176,7 @@ PreparedInput Linear::add(hip::CommandGraph &graph, LinearBuffers b, const Proje
   if (b.nextTable && !gateUp) throw std::invalid_argument("only a block gate/up plan writes the next projection's table");
   if (writesTable) {
     if (n % GGUF_BLOCK) throw std::invalid_argument("a table epilogue takes whole super-blocks of output columns");
-    requireBytes(b.nextTable, gguf_table_bytes(n, tiles), "next projection table");
+    requireBytes(b.nextTable, gguf_tables_bytes(n, tiles), "next projection table");
     if (b.nextTable.sameView(b.scratch.input)) throw std::invalid_argument("the next projection's table is not the plan's own");
   }
   const bool prepared = b.prepared.layout == LinearInput::Table16 && b.prepared.source && b.input &&
@@ -214,7 +217,7 @@ PreparedInput Linear::add(hip::CommandGraph &graph, LinearBuffers b, const Proje
              w.epilogue == LinearEpilogue::Residual ? b.residual : writesTable ? b.nextTable : spare,
              c.splits > 1 ? b.scratch.partials : spare,
              c.splits > 1 ? b.scratch.counters : spare},
-            params, {c.wholeGroups + (groupsOf(n, w.epilogue) - c.wholeGroups) * c.splits, 1, 1}, {256, 1, 1});
+            params, {c.wholeGroups + (groupsOf(n, w.epilogue) - c.wholeGroups) * c.splits, rowPieces(w.rows), 1}, {256, 1, 1});
   (void)tiles;
   return {b.input, LinearInput::Table16};
 }

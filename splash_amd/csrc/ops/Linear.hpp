@@ -28,9 +28,12 @@ enum class LinearEpilogue : uint8_t { None, Residual, GateUp };
 // One tile: 16-column MFMA tiles, two per wave, 16/32/64 rows.
 enum class LinearTile : uint8_t { GgufMfma };
 inline constexpr uint32_t kMaximumDecodeTileRows = GGUF_MAXIMUM_ROWS;
+// A dispatch of more rows runs pieces of kMaximumDecodeTileRows rows side by side.
+inline constexpr uint32_t kMaximumDispatchRows = GGUF_MAXIMUM_DISPATCH_ROWS;
 
 // The tile height that holds `rows` rows (the reference's stagedTileRows, Linear.hpp:118-120).
 [[nodiscard]] constexpr uint32_t mfmaTileRows(uint32_t rows) noexcept { return rows <= 16 ? 16 : rows <= 32 ? 32 : 64; }
+[[nodiscard]] constexpr uint32_t rowPieces(uint32_t rows) noexcept { return (rows + kMaximumDecodeTileRows - 1) / kMaximumDecodeTileRows; }
 
 struct LinearWorkload final {
   LinearMatrix matrix;

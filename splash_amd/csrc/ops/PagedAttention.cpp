@@ -130,6 +130,7 @@ void PagedAttention::addAttention(hip::CommandGraph &graph, const AttentionPlan 
   const uint32_t width = g.qHeads * g.headDimension;
   if (outputTable) {
     if (width % GGUF_BLOCK) throw std::invalid_argument("an attention output table holds whole super-blocks");
+    if (rows > GGUF_MAXIMUM_ROWS) throw std::invalid_argument("the attention merge writes the table of up to 64 rows");
     params.table_tiles = gguf_row_tiles(rows);
     requireBytes(outputTable, gguf_table_bytes(width, params.table_tiles), "attention output table");
   }

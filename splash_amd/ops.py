@@ -363,6 +363,15 @@ class MoE:
 NO_TOKEN = 0xFFFFFFFF
 
 
+class RowCopy:
+    """ops::RowCopy: rows of bf16 values between two row regions (row, stride, column)."""
+
+    @staticmethod
+    def add(graph, source, from_region, destination, to_region, rows, width):
+        check(lib.spo_row_copy_add(graph.handle, source.handle, *from_region, destination.handle, *to_region, rows, width))
+        graph._keep.extend([source, destination])
+
+
 class Sampling:
     """ops::Sampling: addVerify (argmax or rejection sampling per row), addAcceptance (tree walk)."""
 

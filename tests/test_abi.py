@@ -71,6 +71,6 @@ def test_linear_plans_without_a_device():
     # the LM head fills the device in whole rounds; only the workgroups of the last, partial round split
     assert partials <= 16 * 255 * 4 * 256 * 4
     with pytest.raises(ValueError):
-        linear.scratch_size(5120, 25600, 65)
+        linear.scratch_size(5120, 25600, 257)
     with pytest.raises(ValueError):
         linear.scratch_size(5121, 25600, 16)

@@ -108,6 +108,41 @@ def test_rows_do_not_depend_on_the_block_or_the_partition(backend, fmt):
         assert np.all(np.abs(a.astype(np.float64) - want["exact"]) <= want["bound"])
 
 
+@pytest.mark.parametrize("fmt", [ops.FMT_Q4K, ops.FMT_Q6K])
+@pytest.mark.parametrize("M", [65, 80, 128, 200])
+def test_more_rows_than_a_workgroup_takes_run_as_pieces(backend, fmt, M):
+    """A dispatch of more than 64 rows (eight lanes of a hybrid step) runs 64-row pieces side by side: every row
+    carries the bits it has in a dispatch of its own piece alone, plain, split, with a residual and as a gate/up pair."""
+    print(f"case projection pieces fmt={fmt} M={M}", flush=True)
+    rng = np.random.default_rng(300 + M)
+    N, K = 320, 2048
+    native, gate_native = orc.make_native(fmt, N, K, 70), orc.make_native(fmt, N, K, 71)
+    x = orc.f32_to_bf16(rng.standard_normal((M, K)).astype(np.float32))
+    residual = orc.f32_to_bf16(rng.standard_normal((M, N)).astype(np.float32))
+    linear = ops.Linear(backend)
+    cases = [dict(float32=True, splits=1, whole_groups=0), dict(float32=True, splits=4, whole_groups=0), dict(splits=2, whole_groups=3),
+             dict(epilogue=ops.EPILOGUE_RESIDUAL, splits=4, whole_groups=1), dict(epilogue=ops.EPILOGUE_GATE_UP, splits=2, whole_groups=0)]
+    for case in cases:
+        extra = dict(case)
+        if extra.get("epilogue") == ops.EPILOGUE_RESIDUAL:
+            extra["residual_bits"] = residual
+        if extra.get("epilogue") == ops.EPILOGUE_GATE_UP:
+            extra["gate_native"] = gate_native
+        whole, _, _ = run_projection(backend, linear, fmt, [(N, native)], K, x, **extra)
+        for first in range(0, M, 64):
+            rows = slice(first, min(M, first + 64))
+            if "residual_bits" in extra:
+                extra["residual_bits"] = residual[rows]
+            piece, _, _ = run_projection(backend, linear, fmt, [(N, native)], K, x[rows], **extra)
+            assert piece.tobytes() == whole[rows].tobytes(), (case, first)
+            extra.pop("residual_bits", None)
+            if case.get("epilogue") == ops.EPILOGUE_RESIDUAL:
+                extra["residual_bits"] = residual
+    want = orc.gemm(fmt, native, x, N)
+    got, _, _ = run_projection(backend, linear, fmt, [(N, native)], K, x, float32=True)
+    assert np.all(np.abs(got.astype(np.float64) - want["exact"]) <= want["bound"])
+
+
 def test_fused_segments_equal_each_alone(backend):
     """A fused q|k|v dispatch gives each segment the bits it gets alone (LinearGguf.cpp:78-96)."""
     print("case fused segments", flush=True)
@@ -203,7 +238,7 @@ def test_linear_rejects_bad_buffers_before_adding_anything(backend):
     with pytest.raises(ValueError, match="too small"):
         linear.add(graph, proj, plan, small, x, scratch)
     with pytest.raises(ValueError):
-        linear.plan(proj, 65)
+        linear.plan(proj, 257)
     with pytest.raises(ValueError):
         linear.plan(proj, 16, splits=3)
     assert len(graph) == 0

@@ -68,6 +68,23 @@ def test_rope_tree_tables(backend):
     assert np.abs(sin.download(np.float32).reshape(7, pairs) - np.sin(angle)).max() < 2e-6
 
 
+def test_row_copy(backend):
+    """RowCopy.hpp:17-28: a capture copies a layer's output rows into its slot of wider rows."""
+    rng = np.random.default_rng(5)
+    source = rng.integers(0, 65536, (20, 96), dtype=np.uint16)
+    before = rng.integers(0, 65536, (24, 300), dtype=np.uint16)
+    destination = backend.from_array(before)
+    g = splash_amd.CommandGraph()
+    ops.RowCopy.add(g, backend.from_array(source), (3, 96, 16), destination, (5, 300, 100), 16, 64)
+    backend.run(g)
+    want = before.copy()
+    want[5:21, 100:164] = source[3:19, 16:80]
+    assert np.array_equal(destination.download(np.uint16).reshape(24, 300), want)
+    for bad in (((3, 96, 40), (5, 300, 100), 16, 64), ((3, 96, 16), (5, 300, 250), 16, 64), ((5, 96, 16), (5, 300, 100), 16, 64)):
+        with pytest.raises(ValueError):
+            ops.RowCopy.add(splash_amd.CommandGraph(), backend.from_array(source), bad[0], destination, bad[1], bad[2], bad[3])
+
+
 def sampling_buffers(backend, rows, V, logits, draft=None, uniforms=None, tokens=None, tree=None):
     sizes = ops.Sampling.workspace(rows)
     b = dict(logits=backend.from_array(logits.astype(np.float32)), tokens=backend.allocate_buffer(rows * 4),
