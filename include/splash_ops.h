@@ -211,6 +211,8 @@ sp_status spo_sampling_workspace(uint32_t rows, uint64_t sizes[5]);
 typedef struct spo_sampling_buffers {
   sp_buffer *logits, *tokens, *partial_values, *partial_indices;
   sp_buffer *draft_probabilities, *uniforms, *masses, *ranges, *decisions, *input_tokens, *tree_rows; /* sampled lanes */
+  sp_buffer *token_mask; /* constrained lanes: uint32 [rows][mask_words], bit t % 32 of word t / 32 of a row admits token t */
+  uint32_t mask_words;
 } spo_sampling_buffers;
 /* ops::SamplingPolicy (Sampling.hpp:56-83): temperature 0 is greedy; a sampling lane keeps the tokens that
  * weigh at least min_p of its heaviest (0: all), then the top_k most likely of those (0: all), then their
@@ -219,11 +221,15 @@ typedef struct spo_sampling_policy {
   float temperature, min_p;
   uint32_t top_k;
   float top_p;
+  uint32_t constrained;          /* the lane's rows admit only the tokens of their token_mask rows */
+  uint32_t excludes_stop_tokens; /* the lane never selects a stop token */
 } spo_sampling_policy;
-/* Sampling::addVerify (Sampling.cpp:283-328). */
+/* Sampling::addVerify (Sampling.cpp:283-328). The logits rows of a constrained or stop-excluding lane are rewritten
+ * first, -infinity at the tokens the lane does not admit (TargetRow::admits, sampling.metal:42-46).
+ * stop_tokens: four ids, 0xFFFFFFFF for none; NULL for none at all. */
 sp_status spo_sampling_add_verify(spo_graph *graph, const spo_sampling_buffers *buffers, uint32_t vocabulary,
                                   uint32_t logits_stride, const spo_lane_rows *lanes, const spo_sampling_policy *policies,
-                                  uint32_t count);
+                                  uint32_t count, const uint32_t *stop_tokens);
 /* Sampling::addAcceptance (Sampling.cpp:330-357). */
 sp_status spo_sampling_add_acceptance(spo_graph *graph, sp_buffer *input_tokens, sp_buffer *tree_rows, sp_buffer *tokens,
                                       sp_buffer *retained, sp_buffer *accepted_count, sp_buffer *retained_rows,

@@ -123,7 +123,7 @@ class MoeWorkspace(ctypes.Structure):
 
 class SamplingBuffers(ctypes.Structure):
     _fields_ = [(n, c_p) for n in ("logits", "tokens", "partial_values", "partial_indices", "draft_probabilities", "uniforms",
-                                   "masses", "ranges", "decisions", "input_tokens", "tree_rows")]
+                                   "masses", "ranges", "decisions", "input_tokens", "tree_rows", "token_mask")] + [("mask_words", c_u32)]
 
 
 class DenseDimensions(ctypes.Structure):
@@ -137,7 +137,8 @@ class VerifyLane(ctypes.Structure):
 
 
 class SamplingPolicy(ctypes.Structure):
-    _fields_ = [("temperature", ctypes.c_float), ("min_p", ctypes.c_float), ("top_k", c_u32), ("top_p", ctypes.c_float)]
+    _fields_ = [("temperature", ctypes.c_float), ("min_p", ctypes.c_float), ("top_k", c_u32), ("top_p", ctypes.c_float),
+                ("constrained", c_u32), ("excludes_stop_tokens", c_u32)]
 
 
 class HybridDimensions(ctypes.Structure):
@@ -246,7 +247,7 @@ _sig("spo_moe_add_routing", c_int, c_p, c_p, c_u32, P(MoeWorkspace), P(MoeShape)
 _sig("spo_moe_add_routed", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_u32, c_u32, P(MoeWorkspace), P(MoeShape), c_u32)
 _sig("spo_row_copy_add", c_int, c_p, c_p, c_u32, c_u32, c_u32, c_p, c_u32, c_u32, c_u32, c_u32, c_u32)
 _sig("spo_sampling_workspace", c_int, c_u32, P(c_u64))
-_sig("spo_sampling_add_verify", c_int, c_p, P(SamplingBuffers), c_u32, c_u32, P(LaneRows), P(SamplingPolicy), c_u32)
+_sig("spo_sampling_add_verify", c_int, c_p, P(SamplingBuffers), c_u32, c_u32, P(LaneRows), P(SamplingPolicy), c_u32, P(c_u32))
 _sig("spo_sampling_add_acceptance", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, P(LaneRows), P(c_u32), c_u32, P(c_u32))
 _sig("spo_dense_verify_create", c_int, c_p, P(DenseDimensions), c_u32, c_u32, c_u32, P(c_p))
 _sig("spo_dense_verify_destroy", None, c_p)

@@ -36,13 +36,17 @@ struct TargetSamplingParams {
   float temperature[SAMPLING_MAXIMUM_LANES];
   uint32_t sampling_mask; // lanes that sample; the others take the argmax
   uint32_t truncating_mask; // lanes whose distribution ends before the last token (min_p, top_k or top_p cut it)
-  uint32_t reserved[2];
+  uint32_t constrained_mask;   // lanes whose rows admit only the tokens of their constraint-mask rows
+  uint32_t exclude_stop_mask;  // lanes that ignore end-of-sequence: they never select a stop token
   struct SamplingLaneRows lane[SAMPLING_MAXIMUM_LANES];
   // A sampling lane keeps the tokens that weigh at least min_p of the heaviest, then the top_k most
   // likely of those (0: all), then their top_p nucleus (Sampling.hpp:58-83 in the reference).
   float min_p[SAMPLING_MAXIMUM_LANES];
   uint32_t top_k[SAMPLING_MAXIMUM_LANES];
   float top_p[SAMPLING_MAXIMUM_LANES];
+  uint32_t mask_words;      // words of a constraint-mask row (one a packed row): bit t % 32 of word t / 32 admits token t
+  uint32_t stop_tokens[SAMPLING_STOP_TOKENS];
+  uint32_t reserved[3];
 };
 
 // decode_accept_tree: one thread per lane (AcceptBatchParams).
@@ -55,6 +59,6 @@ struct AcceptBatchParams {
 };
 
 #ifdef __cplusplus
-static_assert(sizeof(TargetSamplingParams) == 16 + 32 + 16 + 64 + 96, "target sampling parameters are 224 bytes on both sides");
+static_assert(sizeof(TargetSamplingParams) == 16 + 32 + 16 + 64 + 96 + 32, "target sampling parameters are 256 bytes on both sides");
 static_assert(sizeof(AcceptBatchParams) == 16 + 32 + 16 + 64, "acceptance parameters are 128 bytes on both sides");
 #endif

@@ -81,15 +81,19 @@ sp_status spo_sampling_workspace(uint32_t rows, uint64_t sizes[5]) {
   });
 }
 sp_status spo_sampling_add_verify(spo_graph *graph, const spo_sampling_buffers *b, uint32_t vocabulary, uint32_t logits_stride,
-                                  const spo_lane_rows *lanes, const spo_sampling_policy *policy, uint32_t count) {
+                                  const spo_lane_rows *lanes, const spo_sampling_policy *policy, uint32_t count,
+                                  const uint32_t *stop_tokens) {
   return capi::guard([&] {
     capi::require(graph && b && lanes && policy, "graph, buffers, lanes or policies");
     ops::SamplingBuffers buffers{B(b->logits), B(b->tokens), B(b->partial_values), B(b->partial_indices), B(b->draft_probabilities),
-                                 B(b->uniforms), B(b->masses), B(b->ranges), B(b->decisions), B(b->input_tokens), B(b->tree_rows)};
+                                 B(b->uniforms), B(b->masses), B(b->ranges), B(b->decisions), B(b->input_tokens), B(b->tree_rows),
+                                 B(b->token_mask), b->mask_words};
     std::vector<ops::LaneRows> rows;
     std::vector<ops::SamplingPolicy> policies;
-    for (uint32_t i = 0; i < count; ++i) { rows.push_back({lanes[i].first, lanes[i].rows}); policies.push_back({policy[i].temperature, policy[i].min_p, policy[i].top_k, policy[i].top_p}); }
-    ops::Sampling::addVerify(capi::graphOf(graph), buffers, vocabulary, logits_stride, rows, policies);
+    for (uint32_t i = 0; i < count; ++i) { rows.push_back({lanes[i].first, lanes[i].rows}); policies.push_back({policy[i].temperature, policy[i].min_p, policy[i].top_k, policy[i].top_p, policy[i].constrained != 0, policy[i].excludes_stop_tokens != 0}); }
+    std::array<uint32_t, SAMPLING_STOP_TOKENS> stops{SAMPLING_NO_TOKEN, SAMPLING_NO_TOKEN, SAMPLING_NO_TOKEN, SAMPLING_NO_TOKEN};
+    if (stop_tokens) for (size_t s = 0; s < stops.size(); ++s) stops[s] = stop_tokens[s];
+    ops::Sampling::addVerify(capi::graphOf(graph), buffers, vocabulary, logits_stride, rows, policies, stops);
   });
 }
 sp_status spo_sampling_add_acceptance(spo_graph *graph, sp_buffer *input_tokens, sp_buffer *tree_rows, sp_buffer *tokens,

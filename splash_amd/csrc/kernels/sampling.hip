@@ -49,6 +49,35 @@ __device__ __forceinline__ Best wave_best(Best v) {
   return v;
 }
 
+__device__ __forceinline__ uint32_t lane_of(const TargetSamplingParams &p, uint32_t row) {
+  uint32_t lane = 0;
+  for (uint32_t l = 0; l < p.lanes; ++l)
+    if (row >= p.lane[l].first && row < p.lane[l].first + p.lane[l].rows) lane = l;
+  return lane;
+}
+// decode_sample_admit: grid (rows, ceil(vocabulary / 1024)), 256 threads. A row of a constrained lane
+// admits only the tokens of its constraint-mask row, a row of a lane that ignores end-of-sequence no
+// stop token (TargetRow::admits, sampling.metal:42-46): the logits of the others become -infinity,
+// which every selection kernel leaves out, before any of them reads the row.
+__global__ __launch_bounds__(256) void decode_sample_admit(float *__restrict__ logits, const uint32_t *__restrict__ token_mask,
+                                                           TargetSamplingParams p) {
+  const uint32_t row = blockIdx.x, lane = lane_of(p, row);
+  const bool constrained = (p.constrained_mask >> lane) & 1u, excludes = (p.exclude_stop_mask >> lane) & 1u;
+  if (!constrained && !excludes) return;
+  float *x = logits + size_t(row) * p.logits_stride;
+  const uint32_t *mask = token_mask + size_t(row) * p.mask_words;
+#pragma unroll
+  for (uint32_t i = 0; i < 4; ++i) {
+    const uint32_t token = (blockIdx.y * 4u + i) * 256u + threadIdx.x;
+    if (token >= p.vocabulary) continue;
+    bool admitted = !constrained || ((mask[token / 32u] >> (token % 32u)) & 1u);
+    if (excludes)
+      for (uint32_t s = 0; s < SAMPLING_STOP_TOKENS; ++s) admitted = admitted && token != p.stop_tokens[s];
+    if (!admitted) x[token] = -INFINITY;
+  }
+}
+SP_REGISTER_KERNEL("decode_sample_admit", &decode_sample_admit);
+
 // Grid (rows * SAMPLING_SHARDS), 256 threads. partial_values/indices [row][shard].
 __global__ __launch_bounds__(256) void decode_sample_argmax_sharded(const float *__restrict__ logits, float *__restrict__ partial_values,
                                                                     uint32_t *__restrict__ partial_indices, TargetSamplingParams p) {

@@ -30,7 +30,8 @@ SamplingWorkspaceSize Sampling::workspace(uint32_t rows) noexcept {
 }
 
 void Sampling::addVerify(hip::CommandGraph &graph, const SamplingBuffers &b, uint32_t vocabulary, uint32_t logitsStride,
-                         const std::vector<LaneRows> &lanes, const std::vector<SamplingPolicy> &policies) {
+                         const std::vector<LaneRows> &lanes, const std::vector<SamplingPolicy> &policies,
+                         const std::array<uint32_t, SAMPLING_STOP_TOKENS> &stopTokens) {
   const uint32_t rows = packedRows(lanes);
   if (policies.size() != lanes.size()) throw std::invalid_argument("acceptance takes one policy per lane");
   if (!vocabulary || logitsStride < vocabulary) throw std::invalid_argument("logits rows hold the vocabulary");
@@ -50,6 +51,14 @@ void Sampling::addVerify(hip::CommandGraph &graph, const SamplingBuffers &b, uin
     params.min_p[l] = policy.minP;
     params.top_k[l] = policy.topK;
     params.top_p[l] = policy.topP;
+    if (policy.constrained) params.constrained_mask |= 1u << l;
+    if (policy.excludesStopTokens) params.exclude_stop_mask |= 1u << l;
+  }
+  for (size_t s = 0; s < stopTokens.size(); ++s) params.stop_tokens[s] = stopTokens[s];
+  if (params.constrained_mask) {
+    if (uint64_t{b.maskWords} * 32 < vocabulary) throw std::invalid_argument("a constraint-mask row holds a bit for every token");
+    requireBytes(b.tokenMask, uint64_t{rows} * b.maskWords * 4, "constraint masks");
+    params.mask_words = b.maskWords;
   }
   const SamplingWorkspaceSize need = workspace(rows);
   requireBytes(b.logits, (uint64_t{rows - 1} * logitsStride + vocabulary) * 4, "logits");
@@ -65,6 +74,9 @@ void Sampling::addVerify(hip::CommandGraph &graph, const SamplingBuffers &b, uin
     requireBytes(b.inputTokens, uint64_t{rows} * 4, "input tokens");
     requireBytes(b.treeRows, uint64_t{rows} * sizeof(AttentionTreeRow), "verify tree rows");
   }
+  if (params.constrained_mask || params.exclude_stop_mask)
+    graph.add("decode_sample_admit", {b.logits, params.constrained_mask ? b.tokenMask : b.logits}, params,
+              {rows, (vocabulary + 1023) / 1024, 1}, {256, 1, 1});
   // Every row gets its argmax; the sampled lanes' rows are then overwritten by their draw.
   graph.add("decode_sample_argmax_sharded", {b.logits, b.partialValues, b.partialIndices}, params, {rows * SAMPLING_SHARDS, 1, 1},
             {SAMPLING_THREADS, 1, 1});

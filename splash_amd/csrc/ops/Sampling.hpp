@@ -21,6 +21,10 @@ struct SamplingPolicy final {
   float minP = 0.0f;
   uint32_t topK = 0;
   float topP = 1.0f;
+  // The lane's rows admit only the tokens of their rows of SamplingBuffers::tokenMask.
+  bool constrained = false;
+  // The lane ignores end-of-sequence: it never selects a stop token (addVerify's stopTokens).
+  bool excludesStopTokens = false;
   // A lane samples unless it keeps only its most likely token (Sampling.hpp:79-82).
   [[nodiscard]] bool samples() const noexcept { return temperature > 0.0f && minP < 1.0f && topK != 1; }
   [[nodiscard]] bool truncates(uint32_t vocabulary) const noexcept {
@@ -45,6 +49,9 @@ struct SamplingBuffers final {
   hip::Buffer masses, ranges;
   hip::Buffer decisions;  // SAMPLING_DECISION_WORDS words a row: its child's test and the end of its distribution
   hip::Buffer inputTokens, treeRows;  // the block's input tokens and SplashTreeRow rows
+  // Constrained lanes only: uint32 [rows][maskWords], bit t % 32 of word t / 32 of a row admits token t.
+  hip::Buffer tokenMask;
+  uint32_t maskWords = 0;
 };
 struct AcceptanceBuffers final {
   hip::Buffer inputTokens;    // uint32 [rows]
@@ -59,8 +66,12 @@ class Sampling final {
 public:
   [[nodiscard]] static SamplingWorkspaceSize workspace(uint32_t rows) noexcept;
   // One policy per lane. Throws for no or too many lanes, rows outside 1..16, or missing buffers.
+  // The logits rows of a constrained or stop-excluding lane are rewritten first: -infinity at the
+  // tokens the lane does not admit (TargetRow::admits in the reference, which reads a mask instead).
   static void addVerify(hip::CommandGraph &graph, const SamplingBuffers &buffers, uint32_t vocabulary, uint32_t logitsStride,
-                        const std::vector<LaneRows> &lanes, const std::vector<SamplingPolicy> &policies);
+                        const std::vector<LaneRows> &lanes, const std::vector<SamplingPolicy> &policies,
+                        const std::array<uint32_t, SAMPLING_STOP_TOKENS> &stopTokens = {SAMPLING_NO_TOKEN, SAMPLING_NO_TOKEN,
+                                                                                       SAMPLING_NO_TOKEN, SAMPLING_NO_TOKEN});
   static void addAcceptance(hip::CommandGraph &graph, const AcceptanceBuffers &buffers, const std::vector<LaneRows> &lanes,
                             const std::vector<uint32_t> &remaining, const std::array<uint32_t, SAMPLING_STOP_TOKENS> &stopTokens);
 };

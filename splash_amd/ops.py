@@ -382,15 +382,21 @@ class Sampling:
         return list(sizes)
 
     @staticmethod
-    def add_verify(graph, buffers, vocabulary, stride, lanes, policies):
-        """buffers: dict of Buffer by the names of spo_sampling_buffers; lanes: [(first, rows)]; policies: a lane's
-        temperature, or (temperature, min_p, top_k, top_p)."""
-        b = nat.SamplingBuffers(**{k: (v.handle if v is not None else None) for k, v in buffers.items()})
+    def add_verify(graph, buffers, vocabulary, stride, lanes, policies, stop_tokens=None):
+        """buffers: dict of Buffer by the names of spo_sampling_buffers (token_mask with mask_words for constrained
+        lanes); lanes: [(first, rows)]; policies: a lane's temperature, or (temperature, min_p, top_k, top_p[,
+        constrained, excludes_stop_tokens]); stop_tokens: up to four ids."""
+        words = buffers.get("mask_words", 0)
+        b = nat.SamplingBuffers(**{k: (v.handle if v is not None else None) for k, v in buffers.items() if k != "mask_words"},
+                                mask_words=words)
         arr = (nat.LaneRows * len(lanes))(*[nat.LaneRows(*l) for l in lanes])
-        full = [p if isinstance(p, (tuple, list)) else (p, 0.0, 0, 1.0) for p in policies]
+        full = [tuple(p) if isinstance(p, (tuple, list)) else (p, 0.0, 0, 1.0) for p in policies]
         structs = (nat.SamplingPolicy * len(lanes))(*[nat.SamplingPolicy(*p) for p in full])
-        check(lib.spo_sampling_add_verify(graph.handle, ctypes.byref(b), vocabulary, stride, arr, structs, len(lanes)))
-        graph._keep.extend(list(buffers.values()))
+        stops = None
+        if stop_tokens is not None:
+            stops = (ctypes.c_uint32 * 4)(*(list(stop_tokens) + [NO_TOKEN] * 4)[:4])
+        check(lib.spo_sampling_add_verify(graph.handle, ctypes.byref(b), vocabulary, stride, arr, structs, len(lanes), stops))
+        graph._keep.extend([v for k, v in buffers.items() if k != "mask_words"])
 
     @staticmethod
     def add_acceptance(graph, input_tokens, tree_rows, tokens, retained, accepted, retained_rows, lanes, remaining,

@@ -241,3 +241,55 @@ def test_truncated_distributions_match_oracle(backend, ties):
                 assert got[r] == want, (r, policy, got[r], want, accepted)
                 checked += 1
     assert checked >= 12
+
+
+def test_constraint_masks_and_stop_exclusion(backend):
+    """TargetRow::admits (sampling.metal:42-46): a constrained lane's rows select only tokens of their mask rows, a lane
+    that ignores end-of-sequence never a stop token, greedy or sampled; the other lanes' rows are untouched. The
+    oracle sees the same rows with -infinity at the tokens a lane does not admit."""
+    print("case sampling admits", flush=True)
+    rng = np.random.default_rng(21)
+    rows, V, words = 12, 5000, (5000 + 31) // 32
+    lanes = [(0, 3), (3, 3), (6, 3), (9, 3)]
+    # greedy constrained; sampled constrained + stop-excluding with a nucleus; greedy stop-excluding; plain sampled
+    policies = [(0.0, 0.0, 0, 1.0, 1, 0), (0.8, 0.0, 0, 0.9, 1, 1), (0.0, 0.0, 0, 1.0, 0, 1), (0.7, 0.0, 0, 1.0, 0, 0)]
+    logits = (rng.standard_normal((rows, V)) * 2.5).astype(np.float32)
+    stops = [int(np.argmax(logits[6])), int(np.argmax(logits[4])), 17]
+    allowed = rng.random((rows, V)) < 0.3
+    allowed[:, 0] = True
+    allowed[1] = False                              # a row that admits nothing selects the sentinel
+    bits = np.zeros((rows, words * 32), dtype=np.uint8)
+    bits[:, :V] = allowed
+    mask = np.packbits(bits.reshape(rows, words, 32), axis=2, bitorder="little").view(np.uint32).reshape(rows, words)
+    dl = rng.standard_normal((rows, V)) * 2
+    draft = np.exp(dl - dl.max(axis=1, keepdims=True)); draft = (draft / draft.sum(axis=1, keepdims=True)).astype(np.float32)
+    tokens = rng.integers(0, V, rows).astype(np.uint32)
+    uniforms = rng.random((rows, 2)).astype(np.float32)
+    tree = ops.chain_tree_rows([n for _, n in lanes])
+    b = sampling_buffers(backend, rows, V, logits, draft, uniforms, tokens, tree)
+    b["token_mask"], b["mask_words"] = backend.from_array(mask), words
+    g = splash_amd.CommandGraph()
+    ops.Sampling.add_verify(g, b, V, V, lanes, policies, stop_tokens=stops)
+    backend.run(g)
+    got = b["tokens"].download(np.uint32)
+    seen = b["logits"].download(np.float32).reshape(rows, V)
+    for (first, n), policy in zip(lanes, policies):
+        for r in range(first, first + n):
+            x = logits[r].copy()
+            if policy[4]:
+                x[~allowed[r]] = -np.inf
+            if policy[5]:
+                x[stops] = -np.inf
+            assert np.array_equal(seen[r], x)
+            if policy[0] == 0.0:
+                assert got[r] == orc.argmax(x), r
+                continue
+            child = int(tokens[r + 1]) if r + 1 < first + n else orc.NO_TOKEN
+            want, _, close = orc.rejection_row_policy(x, policy[:4], draft[r] if child != orc.NO_TOKEN else None, child,
+                                                      float(uniforms[r, 1]), float(uniforms[r, 0]))
+            if close > 1e-5:
+                assert got[r] == want, (r, got[r], want)
+            assert got[r] == orc.NO_TOKEN or np.isfinite(x[got[r]])
+    assert got[1] == orc.NO_TOKEN and got[6] != stops[0] and got[4] != stops[1]
+    with pytest.raises(ValueError, match="constraint"):
+        ops.Sampling.add_verify(splash_amd.CommandGraph(), {**b, "token_mask": None}, V, V, lanes, policies)
