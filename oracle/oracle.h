@@ -19,9 +19,11 @@
 //   orc_kv_quantize                 pinned: closed form, compiled reference header (oracle/_ref).
 //   orc_attention_*                 pinned by dense-softmax special cases and invariants.
 //   orc_gdn_*                       pinned by the fp64 textbook recurrence (orc_gdn_reference, the check
-//                                   the reference's own test makes) and fold/rollback invariants.
+//                                   the reference's own test makes) and fold/rollback invariants; tree
+//                                   blocks by the same recurrence along each row's path.
 //   orc_argmax / orc_accept_tree    pinned by brute force on tiny vocabularies.
 //   orc_rejection_*                 pinned by enumeration: selection law equals target to 1e-12.
+//   orc_distribution_end            pinned by an independent fp64 sort (min_p, top_k with ties, nucleus).
 //   orc_moe_*                       pinned by a stable sort and softmax closed form; the layer by the dense FFN it
 //                                   reduces to when every expert is the same.
 #pragma once
