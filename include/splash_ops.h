@@ -74,6 +74,15 @@ sp_status spo_linear_plan_with(const spo_projection *projection, spo_linear_plan
 sp_status spo_linear_add(const spo_linear *linear, spo_graph *graph, const spo_projection *projection,
                          const spo_projection *gate, const spo_linear_plan *plan, sp_buffer *input, sp_buffer *output,
                          sp_buffer *residual, sp_buffer *table, sp_buffer *partials, sp_buffer *counters, int prepared);
+/* Linear::add of a plan whose epilogue is 3 (residual + norm): output = bf16(residual + W input), and the RMS norm
+ * of those rows under norm_weight (bf16 [output size]) as the activation table of the projection that follows, in
+ * next_table (spo_gguf_table_bytes(output size, rows) bytes, not `table`): no norm dispatch runs between the two
+ * projections. One tensor, whole super-blocks of output columns, up to 64 rows, no more column groups of 64 than
+ * the device has compute units. */
+sp_status spo_linear_add_residual_norm(const spo_linear *linear, spo_graph *graph, const spo_projection *projection,
+                                       const spo_linear_plan *plan, sp_buffer *input, sp_buffer *output, sp_buffer *residual,
+                                       sp_buffer *norm_weight, sp_buffer *next_table, sp_buffer *table, sp_buffer *partials,
+                                       sp_buffer *counters, int prepared);
 /* Linear::addSwiGlu (Linear.hpp:352-354): output = residual + down(silu(gate x) * up x).
  * next_table (optional, spo_gguf_table_bytes(ffn, rows) bytes, not `table`): the gate/up pass
  * then writes the down projection's activation table from its epilogue and no separate table

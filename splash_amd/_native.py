@@ -221,6 +221,7 @@ _sig("spo_linear_destroy", None, c_p)
 _sig("spo_linear_plan_for", c_int, c_p, c_p, c_u32, c_u32, P(LinearPlan))
 _sig("spo_linear_plan_with", c_int, c_p, P(LinearPlan))
 _sig("spo_linear_add", c_int, c_p, c_p, c_p, c_p, P(LinearPlan), c_p, c_p, c_p, c_p, c_p, c_p, c_int)
+_sig("spo_linear_add_residual_norm", c_int, c_p, c_p, c_p, P(LinearPlan), c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_int)
 _sig("spo_linear_add_swiglu", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_u32, c_p, c_p, c_p, c_p)
 _sig("spo_linear_scratch_size", c_int, c_p, c_u32, c_u32, c_u32, P(c_u64), P(c_u64), P(c_u64))
 

@@ -117,6 +117,15 @@ struct GgufPrepareParams {
 // The same, and `out` also leaves as the next projection's activation table, written to the buffer
 // bound in the residual's place (columns a multiple of 256): kernel suffix _gt.
 #define GGUF_EPILOGUE_GATE_UP_TABLE 4u
+// out = bf16(v + res), and the RMS norm of those rows (weights bound in the second segment's slot) as
+// the activation table of the projection after it (bound in the third's): kernel suffix _rn. Each
+// workgroup that ends a column group leaves its rows' sums of squares over its 64 columns, counts itself in
+// and waits (a bounded wait) until every group has; then all of them know every row's inverse RMS and write
+// their own 64 columns of the table. The sums and three words (done, passed, expired) follow the
+// dispatch's partials and counters. One workgroup per column group waits, so the dispatch must hold
+// fewer column groups than the device runs workgroups at once.
+#define GGUF_EPILOGUE_RESIDUAL_NORM 5u
+#define GGUF_NORM_SYNC_WORDS 4u
 
 // gguf_decode_<fmt>_m<16|32|64>_<a|a_f32|r|g>: up to three column segments of one format in one
 // dispatch (the reference's GgufDecodeFusedParams, runtime/metal/abi/Gguf.h:168-178), tiles in

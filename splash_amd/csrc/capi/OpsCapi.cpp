@@ -14,7 +14,7 @@ using namespace splash;
 
 namespace {
 ops::LinearPlan toPlan(const ops::Projection &projection, const spo_linear_plan &p) {
-  if (p.epilogue > 2) throw std::invalid_argument("unknown linear epilogue");
+  if (p.epilogue > 3) throw std::invalid_argument("unknown linear epilogue");
   ops::LinearConfig config;
   config.splits = p.splits;
   config.wholeGroups = p.whole_groups;
@@ -151,7 +151,7 @@ sp_status spo_linear_plan_for(const spo_linear *linear, const spo_projection *pr
                               spo_linear_plan *out) {
   return capi::guard([&] {
     capi::require(linear && projection && out, "linear, projection or result");
-    if (epilogue > 2) throw std::invalid_argument("unknown linear epilogue");
+    if (epilogue > 3) throw std::invalid_argument("unknown linear epilogue");
     fromPlan(linear->linear.plan(projection->projection, rows, static_cast<ops::LinearEpilogue>(epilogue)), out);
   });
 }
@@ -174,6 +174,25 @@ sp_status spo_linear_add(const spo_linear *linear, spo_graph *graph, const spo_p
     if (prepared) buffers.prepared = {buffers.input, ops::LinearInput::Table16};
     linear->linear.add(graph->graph, std::move(buffers), projection->projection, toPlan(projection->projection, *plan),
                        gate ? &gate->projection : nullptr);
+  });
+}
+sp_status spo_linear_add_residual_norm(const spo_linear *linear, spo_graph *graph, const spo_projection *projection,
+                                       const spo_linear_plan *plan, sp_buffer *input, sp_buffer *output, sp_buffer *residual,
+                                       sp_buffer *norm_weight, sp_buffer *next_table, sp_buffer *table, sp_buffer *partials,
+                                       sp_buffer *counters, int prepared) {
+  return capi::guard([&] {
+    capi::require(linear && graph && projection && plan, "linear, graph, projection or plan");
+    ops::LinearBuffers buffers;
+    buffers.input = hip::Buffer::share(input);
+    buffers.output = hip::Buffer::share(output);
+    buffers.residual = hip::Buffer::share(residual);
+    buffers.normWeight = hip::Buffer::share(norm_weight);
+    buffers.nextTable = hip::Buffer::share(next_table);
+    buffers.scratch = scratchOf(table, partials, counters);
+    if (prepared) buffers.prepared = {buffers.input, ops::LinearInput::Table16};
+    const ops::LinearPlan full = toPlan(projection->projection, *plan);
+    if (full.workload().epilogue != ops::LinearEpilogue::ResidualNorm) throw std::invalid_argument("the plan does not norm its rows");
+    linear->linear.add(graph->graph, std::move(buffers), projection->projection, full);
   });
 }
 sp_status spo_linear_add_swiglu(const spo_linear *linear, spo_graph *graph, const spo_projection *gate,

@@ -360,6 +360,9 @@ __device__ __forceinline__ void decode_workgroup(const uint8_t *__restrict__ seg
   if (live) {
     if constexpr (kGateUp) {
       tile = {(unit & 1u ? seg1 : seg0) + size_t(unit >> 1) * blocks * kRecord, p.offset[0] + (unit >> 1) * GGUF_TILE_COLUMNS};
+    } else if constexpr (EP == GGUF_EPILOGUE_RESIDUAL_NORM) {
+      // one segment: the other two slots bind the norm's weights and the next projection's table
+      tile = {seg0 + size_t(unit) * blocks * kRecord, p.offset[0] + unit * GGUF_TILE_COLUMNS};
     } else {
       const uint8_t *const seg[3] = {seg0, seg1, seg2};
       tile = find_tile(unit, seg, p, kRecord);
@@ -562,6 +565,127 @@ __device__ __forceinline__ void decode_workgroup(const uint8_t *__restrict__ seg
         sums32[(size_t(t2) * G2 + g) * 16u + r] = halfSums[(t2 * 2u) * 16u + r] + halfSums[(t2 * 2u + 1u) * 16u + r];
       }
     }
+  } else if constexpr (EP == GGUF_EPILOGUE_RESIDUAL_NORM) {
+    // The residual rows leave as they do without the norm; their bf16 values stay in registers.
+    constexpr uint32_t kRows = 16u * RT;
+    const uint16_t *normWeight = reinterpret_cast<const uint16_t *>(seg1);
+    uint8_t *next = const_cast<uint8_t *>(seg2);
+    const uint32_t groupsAll = (p.units + 3u) / 4u, partitioned = groupsAll - p.whole_groups;
+    float *rowSquares = partials + (p.splits > 1 ? size_t(p.splits) * partitioned * 4u * RT * 256u : 0u);  // [group][row]
+    uint32_t *sync = counters + (p.splits > 1 ? partitioned : 0u);                                         // done, passed, expired
+    const bool owns = live && tile.image;
+    float hidden[RT][4], squares[RT][4];
+#pragma unroll
+    for (int t = 0; t < RT; ++t)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const uint32_t row = 16u * t + 4u * kq + v;
+        hidden[t][v] = 0.f;
+        if (owns && row < p.rows) {
+          const size_t at = size_t(row) * p.out_stride + tile.column + c;
+          const uint32_t bits = float_to_bf16_bits(acc[t][v] + bf16_bits_to_float(residual[at]));
+          static_cast<uint16_t *>(out)[at] = uint16_t(bits);
+          hidden[t][v] = bf16_bits_to_float(bits);
+        }
+        // the row's squares over the wave's 16 columns: the 16 lanes of one k quarter, by butterfly
+        float sq = hidden[t][v] * hidden[t][v];
+#pragma unroll
+        for (int o = 1; o < 16; o <<= 1) sq += __shfl_xor(sq, o, 64);
+        squares[t][v] = sq;
+      }
+    // The staging buffers are free once every wave has left the loop.
+    __syncthreads();
+    float *waveSquares = reinterpret_cast<float *>(&ldsA[0][0][0][0]);  // [wave][row]
+    float *partSums = waveSquares + 4u * kRows;                          // [part][row]
+    float *inverse = partSums + 256u;                                    // [row]
+    uint16_t *tileOut = reinterpret_cast<uint16_t *>(inverse + kRows);   // [wave][row tile][row][column]
+    float *halfSums = reinterpret_cast<float *>(tileOut + 4u * RT * 256u);  // [row tile][wave][row]
+    if (c == 0) {
+#pragma unroll
+      for (int t = 0; t < RT; ++t)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) waveSquares[wave * kRows + 16u * t + 4u * kq + v] = squares[t][v];
+    }
+    __syncthreads();
+    if (threadIdx.x < kRows) {
+      const float *w = waveSquares + threadIdx.x;
+      __hip_atomic_store(rowSquares + size_t(group) * kRows + threadIdx.x, ((w[0] + w[kRows]) + w[2u * kRows]) + w[3u * kRows],
+                         __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      __hip_atomic_fetch_add(sync, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      // Every group's last workgroup counts itself in; this one waits for them all, at most a
+      // fraction of a second (a dispatch that never completes a group leaves the third word set).
+      uint32_t budget = 1u << 18;
+      while (__hip_atomic_load(sync, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < groupsAll && --budget) __builtin_amdgcn_s_sleep(4);
+      if (!budget) __hip_atomic_store(sync + 2, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    // Every row's sum of squares: part q adds groups q, q + parts, ... in order, the parts are added in order.
+    {
+      constexpr uint32_t kParts = 256u / kRows;
+      const uint32_t row = threadIdx.x % kRows, part = threadIdx.x / kRows;
+      float sum = 0.f;
+      for (uint32_t g = part; g < groupsAll; g += kParts)
+        sum += __hip_atomic_load(rowSquares + size_t(g) * kRows + row, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      partSums[part * kRows + row] = sum;
+      __syncthreads();
+      if (threadIdx.x < kRows) {
+        float total = 0.f;
+        for (uint32_t q = 0; q < kParts; ++q) total += partSums[q * kRows + threadIdx.x];
+        inverse[threadIdx.x] = 1.0f / sqrtf(total / float(p.out_stride) + 1e-6f);
+      }
+      __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+      // The last workgroup through clears the two counts for the next dispatch.
+      const uint32_t passed = __hip_atomic_fetch_add(sync + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (passed == groupsAll - 1u) {
+        __hip_atomic_store(sync, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(sync + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+    // The normalized rows of the workgroup's 64 columns: two groups of the next projection's inputs.
+    const float weight = owns ? bf16_bits_to_float(normWeight[tile.column + c]) : 0.f;
+#pragma unroll
+    for (int t = 0; t < RT; ++t)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const uint32_t row = 16u * t + 4u * kq + v;
+        const uint32_t bits = owns && row < p.rows ? float_to_bf16_bits((hidden[t][v] * inverse[row]) * weight) : 0u;
+        tileOut[((wave * RT + t) * 16u + 4u * kq + v) * 16u + c] = uint16_t(bits);
+      }
+    __syncthreads();
+    const uint32_t G2 = p.out_stride / 32u;
+    uint2 *values = reinterpret_cast<uint2 *>(next);
+    float *sums32 = reinterpret_cast<float *>(next + gguf_table_sums32_offset(p.out_stride, tiles));
+    float *sums16 = reinterpret_cast<float *>(next + gguf_table_sums16_offset(p.out_stride, tiles));
+    // Piece (t, w, kq, r): inputs 16 (w % 2) + 4 kq .. + 3 of group 2 group + w / 2, row 16 t + r.
+    for (uint32_t piece = threadIdx.x; piece < 4u * RT * 64u; piece += 256u) {
+      const uint32_t r = piece & 15u, q4 = (piece >> 4) & 3u, w2 = (piece >> 6) & 3u, t2 = piece >> 8;
+      if (t2 >= tiles) continue;  // a whole wave: the kernel's row tiles past the table's
+      const uint32_t g2 = 2u * group + (w2 >> 1), h2 = w2 & 1u;
+      const uint2 raw = *reinterpret_cast<const uint2 *>(&tileOut[((w2 * RT + t2) * 16u + r) * 16u + 4u * q4]);
+      const uint32_t x0 = raw.x & 0xFFFFu, x1 = raw.x >> 16, x2 = raw.y & 0xFFFFu, x3 = raw.y >> 16;
+      values[((size_t(t2) * G2 + g2) * 64u + q4 * 16u + r) * 2u + h2] = make_uint2(x0 | (x2 << 16), x1 | (x3 << 16));
+      const float run = (bf16_bits_to_float(x0) + bf16_bits_to_float(x1)) + (bf16_bits_to_float(x2) + bf16_bits_to_float(x3));
+      const float r0 = __shfl(run, int(r), 64), r1 = __shfl(run, int(r) + 16, 64), r2 = __shfl(run, int(r) + 32, 64),
+                  r3 = __shfl(run, int(r) + 48, 64);
+      const float sum = ((r0 + r1) + r2) + r3;
+      if (q4 == 0) {
+        sums16[(size_t(t2) * 2u * G2 + 2u * g2 + h2) * 16u + r] = sum;
+        halfSums[(t2 * 4u + w2) * 16u + r] = sum;
+      }
+    }
+    __syncthreads();
+    if (threadIdx.x < tiles * 32u) {
+      const uint32_t t2 = threadIdx.x >> 5, pair = (threadIdx.x >> 4) & 1u, r = threadIdx.x & 15u;
+      sums32[(size_t(t2) * G2 + 2u * group + pair) * 16u + r] =
+          halfSums[(t2 * 4u + 2u * pair) * 16u + r] + halfSums[(t2 * 4u + 2u * pair + 1u) * 16u + r];
+    }
   } else {
     if (!live || !tile.image) return;
 #pragma unroll
@@ -632,7 +756,8 @@ SP_REGISTER_KERNEL("gguf_moe_decode_q6k_a", (&gguf_moe_decode<GGUF_FMT_Q6K, GGUF
   SP_REGISTER_KERNEL("gguf_decode_" fmt "_m" #rows "_a_f32", &gguf_decode<FMT, RT, GGUF_EPILOGUE_PLAIN_F32>); \
   SP_REGISTER_KERNEL("gguf_decode_" fmt "_m" #rows "_r", &gguf_decode<FMT, RT, GGUF_EPILOGUE_RESIDUAL>); \
   SP_REGISTER_KERNEL("gguf_decode_" fmt "_m" #rows "_g", &gguf_decode<FMT, RT, GGUF_EPILOGUE_GATE_UP>);  \
-  SP_REGISTER_KERNEL("gguf_decode_" fmt "_m" #rows "_gt", &gguf_decode<FMT, RT, GGUF_EPILOGUE_GATE_UP_TABLE>)
+  SP_REGISTER_KERNEL("gguf_decode_" fmt "_m" #rows "_gt", &gguf_decode<FMT, RT, GGUF_EPILOGUE_GATE_UP_TABLE>); \
+  SP_REGISTER_KERNEL("gguf_decode_" fmt "_m" #rows "_rn", &gguf_decode<FMT, RT, GGUF_EPILOGUE_RESIDUAL_NORM>)
 SP_GGUF_DECODE("q4k", GGUF_FMT_Q4K, 16, 1);
 SP_GGUF_DECODE("q4k", GGUF_FMT_Q4K, 32, 2);
 SP_GGUF_DECODE("q4k", GGUF_FMT_Q4K, 64, 4);

@@ -19,6 +19,7 @@ const char *epilogueSuffix(LinearEpilogue epilogue, FloatOutput destination, boo
   case LinearEpilogue::None: return destination == FloatOutput::Float32 ? "_a_f32" : "_a";
   case LinearEpilogue::Residual: return "_r";
   case LinearEpilogue::GateUp: return "_g";
+  case LinearEpilogue::ResidualNorm: return "_rn";
   }
   return "_a";
 }
@@ -82,6 +83,11 @@ LinearScratchSize LinearPlan::scratchSize() const noexcept {
     size.partials = uint64_t{pieces} * config_.splits * groups * kWavesAcross * pieceTiles * 256u * sizeof(float);
     size.counters = uint64_t{pieces} * groups * sizeof(uint32_t);
   }
+  if (workload_.epilogue == LinearEpilogue::ResidualNorm) {
+    // every column group's sums of squares of the rows, and the words its workgroups meet on
+    size.partials += uint64_t{groupsOf(n, workload_.epilogue)} * storageRows() * sizeof(float);
+    size.counters += GGUF_NORM_SYNC_WORDS * sizeof(uint32_t);
+  }
   return size;
 }
 
@@ -133,6 +139,8 @@ LinearScratchSize Linear::scratchSize(LinearMatrix matrix, uint32_t rows) const 
   LinearScratchSize size;
   for (LinearEpilogue e : {LinearEpilogue::None, LinearEpilogue::Residual, LinearEpilogue::GateUp})
     size.include(plan(LinearWorkload{matrix, rows, e}).scratchSize());
+  if (rows <= kMaximumDecodeTileRows && matrix.outputSize % GGUF_BLOCK == 0)
+    size.include(plan(LinearWorkload{matrix, rows, LinearEpilogue::ResidualNorm}).scratchSize());
   return size;
 }
 
@@ -165,15 +173,28 @@ PreparedInput Linear::add(hip::CommandGraph &graph, LinearBuffers b, const Proje
   const uint32_t tiles = gguf_row_tiles(w.rows);
   const uint64_t outBytes = plan.destination() == FloatOutput::Float32 ? 4 : 2;
   requireBytes(b.output, uint64_t{w.rows} * n * outBytes, "projection output");
-  if (w.epilogue == LinearEpilogue::Residual) requireBytes(b.residual, uint64_t{w.rows} * n * 2, "projection residual");
+  const bool norms = w.epilogue == LinearEpilogue::ResidualNorm;
+  if (w.epilogue == LinearEpilogue::Residual || norms) requireBytes(b.residual, uint64_t{w.rows} * n * 2, "projection residual");
   const LinearScratchSize need = plan.scratchSize();
   requireBytes(b.scratch.input, need.input, "projection table");
-  if (c.splits > 1) {
+  if (c.splits > 1 || norms) {
     requireBytes(b.scratch.partials, need.partials, "projection partials");
     requireBytes(b.scratch.counters, need.counters, "projection counters");
   }
+  if (norms) {
+    if (p.blocks().segments.size() != 1) throw std::invalid_argument("a projection that norms its rows is one tensor");
+    if (n % GGUF_BLOCK) throw std::invalid_argument("a table epilogue takes whole super-blocks of output columns");
+    if (w.rows > kMaximumDecodeTileRows) throw std::invalid_argument("a projection norms up to 64 rows");
+    // One workgroup per column group waits for the others: they all run at once only if the
+    // device holds that many beside the rest of the dispatch.
+    if (groupsOf(n, w.epilogue) > calibration_.computeUnits)
+      throw std::invalid_argument("a projection that norms its rows holds no more column groups than the device has compute units");
+    requireBytes(b.normWeight, uint64_t{n} * 2, "norm weight");
+    requireBytes(b.nextTable, gguf_tables_bytes(n, gguf_row_tiles(w.rows)), "next projection table");
+    if (b.nextTable.sameView(b.scratch.input)) throw std::invalid_argument("the next projection's table is not the plan's own");
+  }
   const bool writesTable = gateUp && bool(b.nextTable);
-  if (b.nextTable && !gateUp) throw std::invalid_argument("only a block gate/up plan writes the next projection's table");
+  if (b.nextTable && !gateUp && !norms) throw std::invalid_argument("only a gate/up or a norming plan writes the next projection's table");
   if (writesTable) {
     if (n % GGUF_BLOCK) throw std::invalid_argument("a table epilogue takes whole super-blocks of output columns");
     requireBytes(b.nextTable, gguf_tables_bytes(n, tiles), "next projection table");
@@ -212,11 +233,15 @@ PreparedInput Linear::add(hip::CommandGraph &graph, LinearBuffers b, const Proje
   const hip::Buffer &spare = b.scratch.input;
   const std::string name = std::string("gguf_decode_") + segments.front().name() + "_m" + std::to_string(plan.storageRows()) +
                            epilogueSuffix(w.epilogue, plan.destination(), writesTable);
+  if (norms) {
+    images[1] = b.normWeight;
+    images[2] = b.nextTable;
+  }
   graph.add(name,
             {images[0], images[1], images[2], b.scratch.input, b.output,
-             w.epilogue == LinearEpilogue::Residual ? b.residual : writesTable ? b.nextTable : spare,
-             c.splits > 1 ? b.scratch.partials : spare,
-             c.splits > 1 ? b.scratch.counters : spare},
+             w.epilogue == LinearEpilogue::Residual || norms ? b.residual : writesTable ? b.nextTable : spare,
+             c.splits > 1 || norms ? b.scratch.partials : spare,
+             c.splits > 1 || norms ? b.scratch.counters : spare},
             params, {c.wholeGroups + (groupsOf(n, w.epilogue) - c.wholeGroups) * c.splits, rowPieces(w.rows), 1}, {256, 1, 1});
   (void)tiles;
   return {b.input, LinearInput::Table16};

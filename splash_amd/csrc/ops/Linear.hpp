@@ -24,7 +24,10 @@ struct LinearMatrix final {
 
 // Linear.hpp:77 in the reference; UpWithGate (its two-pass gate/up) has no use here: the MFMA tile
 // runs every gate/up pair in one pass.
-enum class LinearEpilogue : uint8_t { None, Residual, GateUp };
+// ResidualNorm: the residual epilogue, and the RMS norm of its rows as the activation table of the
+// projection after it (the reference's residual projections feed a norm_rms_table16 dispatch; here
+// the projection's own workgroups write the table once every column group's sums of squares are in).
+enum class LinearEpilogue : uint8_t { None, Residual, GateUp, ResidualNorm };
 // One tile: 16-column MFMA tiles, two per wave, 16/32/64 rows.
 enum class LinearTile : uint8_t { GgufMfma };
 inline constexpr uint32_t kMaximumDecodeTileRows = GGUF_MAXIMUM_ROWS;
@@ -124,8 +127,11 @@ struct LinearBuffers final {
   hip::Buffer residual;
   LinearScratch scratch{};
   PreparedInput prepared{};
-  // Gate/up plans only: where the epilogue also writes `output` as an activation table.
+  // Gate/up plans: where the epilogue also writes `output` as an activation table. ResidualNorm
+  // plans: where it writes the normalized rows' table.
   hip::Buffer nextTable{};
+  // ResidualNorm plans: the norm's weights, bf16 [output size].
+  hip::Buffer normWeight{};
 };
 
 // What the plans read of the device (the reference's KernelCalibration, ops/KernelCalibration.hpp):

@@ -9,7 +9,7 @@ from ._native import lib, check
 from .backend import Buffer, STORAGE_PRIVATE
 
 FMT_Q4K, FMT_Q6K = 0, 4
-EPILOGUE_NONE, EPILOGUE_RESIDUAL, EPILOGUE_GATE_UP = 0, 1, 2
+EPILOGUE_NONE, EPILOGUE_RESIDUAL, EPILOGUE_GATE_UP, EPILOGUE_RESIDUAL_NORM = 0, 1, 2, 3
 
 
 def gguf_image_bytes(fmt, rows, input_size):
@@ -119,7 +119,19 @@ class Linear:
         c = max(p.scratch_counters for p in plans)
         return LinearScratch(backend, t, s, c)
 
-    def add(self, graph, projection, plan, input, output, scratch, residual=None, gate=None, prepared=False):
+    def add(self, graph, projection, plan, input, output, scratch, residual=None, gate=None, prepared=False, norm_weight=None,
+            next_table=None):
+        """norm_weight, next_table: of a plan with EPILOGUE_RESIDUAL_NORM, which also writes the RMS norm of its output
+        rows as the next projection's activation table."""
+        if plan.epilogue == EPILOGUE_RESIDUAL_NORM:
+            check(lib.spo_linear_add_residual_norm(self.handle, graph.handle, projection.handle, ctypes.byref(plan),
+                                                   input.handle if input else None, output.handle if output else None,
+                                                   residual.handle if residual else None,
+                                                   norm_weight.handle if norm_weight else None,
+                                                   next_table.handle if next_table else None, scratch.table.handle,
+                                                   scratch.partials.handle, scratch.counters.handle, int(prepared)))
+            graph._keep.extend([projection, input, output, residual, scratch, norm_weight, next_table])
+            return
         check(lib.spo_linear_add(self.handle, graph.handle, projection.handle, gate.handle if gate else None,
                                  ctypes.byref(plan), input.handle if input else None, output.handle if output else None,
                                  residual.handle if residual else None, scratch.table.handle, scratch.partials.handle,

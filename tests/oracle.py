@@ -302,6 +302,19 @@ def activation_table(x_bits, tiles=None):
     return values, np.ascontiguousarray(s32.transpose(0, 2, 1)), np.ascontiguousarray(s16.transpose(0, 2, 1))
 
 
+def table_rows(values, K, tiles):
+    """The bf16 rows [tiles * 16][K] an activation table's values hold (the inverse of activation_table's layout)."""
+    G = K // 32
+    order = np.array([0, 2, 1, 3])
+    e = np.arange(8)
+    kq = np.arange(4)
+    inputs = 16 * (e[None, :] // 4) + 4 * kq[:, None] + order[e[None, :] % 4]      # [kq][e]
+    v = np.asarray(values).reshape(tiles, G, 4, 16, 8).transpose(0, 3, 1, 2, 4)   # [t][r][g][kq][e]
+    rows = np.zeros((tiles, 16, G, 32), dtype=np.uint16)
+    rows[:, :, :, inputs] = v
+    return rows.reshape(tiles * 16, K)
+
+
 def split_activation_table(raw_bytes, K, tiles):
     """(values, sums32, sums16) views of a table downloaded as bytes."""
     G = K // 32

@@ -44,6 +44,12 @@ def test_image_dequantization_of_quantized_weights(backend, fmt):
     assert values.tobytes() == orc.dequant_rows(fmt, native, 64, 2048).tobytes()
 
 
+def ulp_key(bits):
+    """bf16 bit patterns as integers that order like their values."""
+    x = np.asarray(bits).astype(np.int32)
+    return np.where(x & 0x8000, 0x8000 - x, x)
+
+
 def run_projection(backend, linear, fmt, native_segments, K, x_bits, epilogue=ops.EPILOGUE_NONE, float32=False,
                    residual_bits=None, gate_native=None, splits=None, whole_groups=None):
     M = x_bits.shape[0]
@@ -221,6 +227,56 @@ def test_gate_up_table_epilogue_equals_the_table_pass(backend, M):
         wv, w32, w16 = orc.activation_table(mid)
         assert np.array_equal(values, wv)
         assert s32.tobytes() == w32.tobytes() and s16.tobytes() == w16.tobytes()
+
+
+@pytest.mark.parametrize("fmt,N,K,M,config", [(ops.FMT_Q4K, 5120, 8192, 16, None), (ops.FMT_Q6K, 5120, 5120, 16, None),
+                                              (ops.FMT_Q4K, 1024, 2048, 5, (1, 0)), (ops.FMT_Q4K, 1024, 2048, 40, (4, 3)),
+                                              (ops.FMT_Q6K, 768, 1024, 64, (2, 0))])
+def test_residual_norm_epilogue(backend, fmt, N, K, M, config):
+    """A residual projection may also write the RMS norm of its rows as the next projection's activation table:
+    its output rows are bit-identical to the plain residual projection's, the table is the table of rows within
+    a bf16 step of norm(output) (the row's sum of squares is added in another order), its sums are those of its own
+    values, and a second dispatch over the same scratch (whose counts the first cleared) repeats it bit for bit."""
+    print(f"case residual norm epilogue fmt={fmt} N={N} K={K} M={M} config={config}", flush=True)
+    rng = np.random.default_rng(N + M)
+    linear = ops.Linear(backend)
+    proj = ops.Projection.from_native(backend, [(fmt, N, orc.make_native(fmt, N, K, 9))], K)
+    x = backend.from_array(orc.f32_to_bf16(rng.standard_normal((M, K)).astype(np.float32)))
+    residual_bits = orc.f32_to_bf16(rng.standard_normal((M, N)).astype(np.float32))
+    weight_bits = orc.f32_to_bf16((1 + 0.1 * rng.standard_normal(N)).astype(np.float32))
+    residual, weight = backend.from_array(residual_bits), backend.from_array(weight_bits)
+    kwargs = dict(splits=config[0], whole_groups=config[1]) if config else {}
+    plain_plan = linear.plan(proj, M, ops.EPILOGUE_RESIDUAL, **kwargs)
+    plan = linear.plan(proj, M, ops.EPILOGUE_RESIDUAL_NORM, **kwargs)
+    assert (plan.splits, plan.whole_groups) == (plain_plan.splits, plain_plan.whole_groups)
+    scratch = linear.scratch_for(backend, [plan, plain_plan])
+    out_plain, out = backend.allocate_buffer(M * N * 2), backend.allocate_buffer(M * N * 2)
+    table = backend.allocate_buffer(ops.gguf_table_bytes(N, M))
+    graph = splash_amd.CommandGraph()
+    linear.add(graph, proj, plain_plan, x, out_plain, scratch, residual=residual)
+    backend.run(graph)
+    graph = splash_amd.CommandGraph()
+    linear.add(graph, proj, plan, x, out, scratch, residual=residual, norm_weight=weight, next_table=table)
+    assert len(graph) == 2          # the table pass of its own input, then the projection
+    backend.run(graph)
+    hidden = out.download(np.uint16).reshape(M, N)
+    assert np.array_equal(hidden, out_plain.download(np.uint16).reshape(M, N))
+    first = table.download(np.uint8)[:ops.gguf_table_bytes(N, M)].copy()
+    tiles = (M + 15) // 16
+    values, s32, s16 = orc.split_activation_table(first, N, tiles)
+    want = orc.rms_norm(hidden, weight_bits)
+    wv, _, _ = orc.activation_table(want)
+    steps = np.abs(ulp_key(values) - ulp_key(wv))
+    assert steps.max() <= 1 and (steps > 0).mean() < 1e-3, (steps.max(), (steps > 0).mean())
+    # the sums are those of the table's own values
+    own_values, own32, own16 = orc.activation_table(orc.table_rows(values, N, tiles))
+    assert np.array_equal(own_values, values) and own32.tobytes() == s32.tobytes() and own16.tobytes() == s16.tobytes()
+    sync = scratch.counters.download(np.uint32)
+    assert not sync.any()            # the counts are cleared and no wait expired
+    backend.run(graph)
+    assert np.array_equal(table.download(np.uint8)[:len(first)], first)
+    with pytest.raises(ValueError, match="next projection table"):
+        linear.add(splash_amd.CommandGraph(), proj, plan, x, out, scratch, residual=residual, norm_weight=weight)
 
 
 def test_linear_rejects_bad_buffers_before_adding_anything(backend):
