@@ -70,15 +70,19 @@ sp_status spo_linear_plan_for(const spo_linear *linear, const spo_projection *pr
  * fills storage_rows and scratch sizes from rows, epilogue, splits, whole_groups, float32. */
 sp_status spo_linear_plan_with(const spo_projection *projection, spo_linear_plan *plan);
 /* Linear::add (Linear.hpp:330-332). table/partials/counters are the LinearScratch; `prepared`
- * nonzero says the table already holds `input` (PreparedInput). gate only for a GateUp plan. */
+ * nonzero says the table already holds `input` (PreparedInput): 1 the table of the rows themselves, 2 the
+ * table a residual + norm plan wrote, whose rows still lack their inverse RMS (this projection applies it
+ * to its sums). gate only for a GateUp plan. */
 sp_status spo_linear_add(const spo_linear *linear, spo_graph *graph, const spo_projection *projection,
                          const spo_projection *gate, const spo_linear_plan *plan, sp_buffer *input, sp_buffer *output,
                          sp_buffer *residual, sp_buffer *table, sp_buffer *partials, sp_buffer *counters, int prepared);
-/* Linear::add of a plan whose epilogue is 3 (residual + norm): output = bf16(residual + W input), and the RMS norm
- * of those rows under norm_weight (bf16 [output size]) as the activation table of the projection that follows, in
- * next_table (spo_gguf_table_bytes(output size, rows) bytes, not `table`): no norm dispatch runs between the two
- * projections. One tensor, whole super-blocks of output columns, up to 64 rows, no more column groups of 64 than
- * the device has compute units. */
+/* Linear::add of a plan whose epilogue is 3 (residual + norm): output = bf16(residual + W input), and those rows
+ * as the activation table of the projection that follows their RMS norm under norm_weight (bf16 [output size]),
+ * in next_table (spo_gguf_table_bytes(output size, rows) bytes, not `table`): no norm dispatch runs between the
+ * two projections. The table holds bf16(output * norm_weight) and the sums of squares of the output rows; the
+ * projection that reads it (`prepared` 2) multiplies its sums by each row's inverse RMS, so its results differ from
+ * those of a norm pass, which rounds bf16(output * inverse RMS * norm_weight), by the rounding of that one bf16
+ * operand. One tensor, whole super-blocks of output columns. */
 sp_status spo_linear_add_residual_norm(const spo_linear *linear, spo_graph *graph, const spo_projection *projection,
                                        const spo_linear_plan *plan, sp_buffer *input, sp_buffer *output, sp_buffer *residual,
                                        sp_buffer *norm_weight, sp_buffer *next_table, sp_buffer *table, sp_buffer *partials,

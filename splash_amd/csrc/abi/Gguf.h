@@ -35,7 +35,10 @@
 // ACTIVATION TABLE of `tiles` row tiles (16 rows each, rows past the live ones zero) and G = K / 32
 // groups: values bf16 [tiles][G][64 lanes][8]: lane (r = l % 16, kq = l / 16) holds inputs
 // gguf_operand_input(kq, 0..7) of row 16 t + r; then sums32 fp32 [tiles][G][16 rows] and sums16
-// fp32 [tiles][2 G][16 rows], the fp32 sums of each row's 32 and 16 inputs in input order.
+// fp32 [tiles][2 G][16 rows], the fp32 sums of each row's 32 and 16 inputs in input order; then
+// squares fp32 [K / 64][16 tiles rows], read only of a table whose rows still lack a per-row scale
+// (GgufDecodeParams::deferred_scale): entry (j, r) is the sum of squares of row r's values over
+// columns 64 j .. 64 j + 63 of the rows the table was normed from.
 #pragma once
 #include <stdint.h>
 
@@ -88,8 +91,11 @@ GGUF_INLINE uint64_t gguf_table_sums32_offset(uint32_t k, uint32_t tiles) { retu
 GGUF_INLINE uint64_t gguf_table_sums16_offset(uint32_t k, uint32_t tiles) {
   return gguf_table_sums32_offset(k, tiles) + uint64_t(tiles) * (k / 32u) * 16u * 4u;
 }
-GGUF_INLINE uint64_t gguf_table_bytes(uint32_t k, uint32_t tiles) {
+GGUF_INLINE uint64_t gguf_table_squares_offset(uint32_t k, uint32_t tiles) {
   return gguf_table_sums16_offset(k, tiles) + uint64_t(tiles) * (k / 16u) * 16u * 4u;
+}
+GGUF_INLINE uint64_t gguf_table_bytes(uint32_t k, uint32_t tiles) {
+  return gguf_table_squares_offset(k, tiles) + uint64_t(tiles) * (k / 64u) * 16u * 4u;
 }
 // Row tiles of a piece, and the tables of `tiles` row tiles in all: whole pieces' tables of four row
 // tiles each, then the last piece's (the single table of up to four row tiles is its own case).
@@ -117,15 +123,14 @@ struct GgufPrepareParams {
 // The same, and `out` also leaves as the next projection's activation table, written to the buffer
 // bound in the residual's place (columns a multiple of 256): kernel suffix _gt.
 #define GGUF_EPILOGUE_GATE_UP_TABLE 4u
-// out = bf16(v + res), and the RMS norm of those rows (weights bound in the second segment's slot) as
-// the activation table of the projection after it (bound in the third's): kernel suffix _rn. Each
-// workgroup that ends a column group leaves its rows' sums of squares over its 64 columns, counts itself in
-// and waits (a bounded wait) until every group has; then all of them know every row's inverse RMS and write
-// their own 64 columns of the table. The sums and three words (done, passed, expired) follow the
-// dispatch's partials and counters. One workgroup per column group waits, so the dispatch must hold
-// fewer column groups than the device runs workgroups at once.
+// out = bf16(v + res), and those rows leave as the activation table of the projection after their RMS
+// norm (the norm's weights bound in the second segment's slot, the table in the third's): kernel
+// suffix _rn. A row's inverse RMS needs every column of the row, which no workgroup of the dispatch
+// has; so the table holds bf16(out * weight) and, in its squares region, each 64-column group's sums
+// of squares of `out`. The projection that reads the table sums them to the row's inverse RMS and
+// multiplies its sums by it (deferred_scale): a per-row factor commutes with the projection. One
+// tensor, whole super-blocks of output columns.
 #define GGUF_EPILOGUE_RESIDUAL_NORM 5u
-#define GGUF_NORM_SYNC_WORDS 4u
 
 // gguf_decode_<fmt>_m<16|32|64>_<a|a_f32|r|g>: up to three column segments of one format in one
 // dispatch (the reference's GgufDecodeFusedParams, runtime/metal/abi/Gguf.h:168-178), tiles in
@@ -140,6 +145,10 @@ struct GgufDecodeParams {
   uint32_t cols[3];     // columns per segment (multiples of 16); 0 past the last
   uint32_t offset[3];   // first destination column per segment
   uint32_t units;       // wave work units: one column tile each (gate/up: gate tile j is unit 2 j, up tile j unit 2 j + 1)
+  // Nonzero: the table's rows lack their RMS scale; every sum is multiplied by
+  // 1 / sqrt(sum of the row's squares entries / K + 1e-6) before the epilogue.
+  uint32_t deferred_scale;
+  uint32_t reserved[3];
 };
 
 // gguf_dequant_<fmt>: the image's fp32 values [N][K], for the bit-exactness test
@@ -159,7 +168,7 @@ struct GgufEmbedParams {
 
 #ifdef __cplusplus
 static_assert(sizeof(GgufPrepareParams) == 16, "prepare parameters are 16 bytes on both sides");
-static_assert(sizeof(GgufDecodeParams) == 48, "decode parameters are 48 bytes on both sides");
+static_assert(sizeof(GgufDecodeParams) == 64, "decode parameters are 64 bytes on both sides");
 static_assert(sizeof(GgufDequantParams) == 8, "dequant parameters are 8 bytes on both sides");
 static_assert(sizeof(GgufEmbedParams) == 12, "embedding parameters are 12 bytes on both sides");
 #endif

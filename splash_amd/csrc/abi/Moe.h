@@ -60,6 +60,6 @@ struct GgufMoeParams {
 
 #ifdef __cplusplus
 static_assert(sizeof(MoeRouteParams) == 16 && sizeof(MoeGroupParams) == 16 && sizeof(MoeGatherParams) == 16 &&
-                  sizeof(MoeCombineParams) == 16 && sizeof(GgufMoeParams) == 80,
+                  sizeof(MoeCombineParams) == 16 && sizeof(GgufMoeParams) == 96,
               "MoE parameters have the same size on both sides");
 #endif

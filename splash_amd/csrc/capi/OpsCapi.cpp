@@ -171,7 +171,7 @@ sp_status spo_linear_add(const spo_linear *linear, spo_graph *graph, const spo_p
     buffers.output = hip::Buffer::share(output);
     buffers.residual = hip::Buffer::share(residual);
     buffers.scratch = scratchOf(table, partials, counters);
-    if (prepared) buffers.prepared = {buffers.input, ops::LinearInput::Table16};
+    if (prepared) buffers.prepared = {buffers.input, prepared == 2 ? ops::LinearInput::TableUnscaled : ops::LinearInput::Table16};
     linear->linear.add(graph->graph, std::move(buffers), projection->projection, toPlan(projection->projection, *plan),
                        gate ? &gate->projection : nullptr);
   });
@@ -189,7 +189,7 @@ sp_status spo_linear_add_residual_norm(const spo_linear *linear, spo_graph *grap
     buffers.normWeight = hip::Buffer::share(norm_weight);
     buffers.nextTable = hip::Buffer::share(next_table);
     buffers.scratch = scratchOf(table, partials, counters);
-    if (prepared) buffers.prepared = {buffers.input, ops::LinearInput::Table16};
+    if (prepared) buffers.prepared = {buffers.input, prepared == 2 ? ops::LinearInput::TableUnscaled : ops::LinearInput::Table16};
     const ops::LinearPlan full = toPlan(projection->projection, *plan);
     if (full.workload().epilogue != ops::LinearEpilogue::ResidualNorm) throw std::invalid_argument("the plan does not norm its rows");
     linear->linear.add(graph->graph, std::move(buffers), projection->projection, full);

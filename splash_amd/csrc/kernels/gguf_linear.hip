@@ -21,7 +21,6 @@
 
 namespace splash::kernels {
 
-constexpr int kUnitTiles = 2;  // column tiles per wave
 #define GGUF_DECODE_UNIT_TILES 2
 
 // ---------------------------------------------------------------------------------------------
@@ -341,6 +340,7 @@ __device__ __forceinline__ void decode_workgroup(const uint8_t *__restrict__ seg
   __shared__ uint4 ldsA[2][RT][8][64];
   __shared__ float ldsSums[2][RT][4][64];
   __shared__ uint32_t arrived;
+  __shared__ float scaleParts[256], rowScale[16 * RT];  // of a table with a deferred scale
 
   const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6, c = lane & 15u, kq = lane >> 4;
   // Workgroup items: the whole groups first, then the partitioned ones part by part.
@@ -431,11 +431,33 @@ __device__ __forceinline__ void decode_workgroup(const uint8_t *__restrict__ seg
 #pragma unroll
       for (int q = 0; q < kSumShare; ++q) sumShare[q] += kSumsPerBlock * 4u * 16u * 4u;
     };
+    // Every row's inverse RMS from the squares the table's writer left, one entry a 64-column group:
+    // part q adds entries q, q + parts, ... in order, then the parts are added in order. The loads go
+    // out before the first weights', so the wait for them leaves those in flight.
+    constexpr uint32_t kRows = 16u * RT, kParts = 256u / kRows;
+    float squareSum = 0.f;
+    if (p.deferred_scale) {
+      const float *squares = reinterpret_cast<const float *>(table + gguf_table_squares_offset(p.input_size, tiles));
+      const uint32_t row = threadIdx.x % kRows, part = threadIdx.x / kRows, entries = p.input_size / 64u;
+      if (row < 16u * tiles)
+        for (uint32_t j = part; j < entries; j += kParts) squareSum += squares[size_t(j) * 16u * tiles + row];
+      __builtin_amdgcn_sched_barrier(0);
+    }
 #pragma unroll
     for (int s = 0; s < kStages - 1; ++s) {
       issue(stage[s]);
       // Keep the stages' loads in issue order: the loop's counted waits assume it on entry too.
       __builtin_amdgcn_sched_barrier(0);
+    }
+    if (p.deferred_scale) {
+      scaleParts[threadIdx.x] = squareSum;
+      __syncthreads();
+      if (threadIdx.x < kRows) {
+        float total = 0.f;
+        for (uint32_t q = 0; q < kParts; ++q) total += scaleParts[q * kRows + threadIdx.x];
+        rowScale[threadIdx.x] = 1.0f / sqrtf(total / float(p.input_size) + 1e-6f);
+      }
+      __syncthreads();
     }
     const uint32_t rounds = (count + kStages - 1) / kStages;
     uint32_t now = 0;
@@ -502,6 +524,12 @@ __device__ __forceinline__ void decode_workgroup(const uint8_t *__restrict__ seg
     }
     if (threadIdx.x == 0) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
+  if (p.deferred_scale) {
+#pragma unroll
+    for (int t = 0; t < RT; ++t)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) acc[t][v] *= rowScale[16u * t + 4u * kq + v];
+  }
 
   if constexpr (kGateUp) {
     // The up wave hands its sums to the gate wave beside it through LDS (the staging buffers are free).
@@ -566,99 +594,46 @@ __device__ __forceinline__ void decode_workgroup(const uint8_t *__restrict__ seg
       }
     }
   } else if constexpr (EP == GGUF_EPILOGUE_RESIDUAL_NORM) {
-    // The residual rows leave as they do without the norm; their bf16 values stay in registers.
+    // The residual rows leave as they do without the norm. Their table holds bf16(row * weight):
+    // the inverse RMS is left to the projection that reads it, from the sums of squares written here.
     constexpr uint32_t kRows = 16u * RT;
     const uint16_t *normWeight = reinterpret_cast<const uint16_t *>(seg1);
     uint8_t *next = const_cast<uint8_t *>(seg2);
-    const uint32_t groupsAll = (p.units + 3u) / 4u, partitioned = groupsAll - p.whole_groups;
-    float *rowSquares = partials + (p.splits > 1 ? size_t(p.splits) * partitioned * 4u * RT * 256u : 0u);  // [group][row]
-    uint32_t *sync = counters + (p.splits > 1 ? partitioned : 0u);                                         // done, passed, expired
     const bool owns = live && tile.image;
-    float hidden[RT][4], squares[RT][4];
+    const float weight = owns ? bf16_bits_to_float(normWeight[tile.column + c]) : 0.f;
+    // The staging buffers are free once every wave has left the loop.
+    __syncthreads();
+    float *waveSquares = reinterpret_cast<float *>(&ldsA[0][0][0][0]);          // [wave][row]
+    uint16_t *tileOut = reinterpret_cast<uint16_t *>(waveSquares + 4u * kRows);  // [wave][row tile][row][column]
+    float *halfSums = reinterpret_cast<float *>(tileOut + 4u * RT * 256u);       // [row tile][wave][row]
 #pragma unroll
     for (int t = 0; t < RT; ++t)
 #pragma unroll
       for (int v = 0; v < 4; ++v) {
         const uint32_t row = 16u * t + 4u * kq + v;
-        hidden[t][v] = 0.f;
+        float hidden = 0.f;
+        uint32_t scaled = 0;
         if (owns && row < p.rows) {
           const size_t at = size_t(row) * p.out_stride + tile.column + c;
           const uint32_t bits = float_to_bf16_bits(acc[t][v] + bf16_bits_to_float(residual[at]));
           static_cast<uint16_t *>(out)[at] = uint16_t(bits);
-          hidden[t][v] = bf16_bits_to_float(bits);
+          hidden = bf16_bits_to_float(bits);
+          scaled = float_to_bf16_bits(hidden * weight);
         }
+        tileOut[((wave * RT + t) * 16u + 4u * kq + v) * 16u + c] = uint16_t(scaled);
         // the row's squares over the wave's 16 columns: the 16 lanes of one k quarter, by butterfly
-        float sq = hidden[t][v] * hidden[t][v];
+        float sq = hidden * hidden;
 #pragma unroll
         for (int o = 1; o < 16; o <<= 1) sq += __shfl_xor(sq, o, 64);
-        squares[t][v] = sq;
+        if (c == 0) waveSquares[wave * kRows + row] = sq;
       }
-    // The staging buffers are free once every wave has left the loop.
     __syncthreads();
-    float *waveSquares = reinterpret_cast<float *>(&ldsA[0][0][0][0]);  // [wave][row]
-    float *partSums = waveSquares + 4u * kRows;                          // [part][row]
-    float *inverse = partSums + 256u;                                    // [row]
-    uint16_t *tileOut = reinterpret_cast<uint16_t *>(inverse + kRows);   // [wave][row tile][row][column]
-    float *halfSums = reinterpret_cast<float *>(tileOut + 4u * RT * 256u);  // [row tile][wave][row]
-    if (c == 0) {
-#pragma unroll
-      for (int t = 0; t < RT; ++t)
-#pragma unroll
-        for (int v = 0; v < 4; ++v) waveSquares[wave * kRows + 16u * t + 4u * kq + v] = squares[t][v];
-    }
-    __syncthreads();
-    if (threadIdx.x < kRows) {
+    if (threadIdx.x < 16u * tiles) {
       const float *w = waveSquares + threadIdx.x;
-      __hip_atomic_store(rowSquares + size_t(group) * kRows + threadIdx.x, ((w[0] + w[kRows]) + w[2u * kRows]) + w[3u * kRows],
-                         __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      float *squares = reinterpret_cast<float *>(next + gguf_table_squares_offset(p.out_stride, tiles));
+      squares[size_t(group) * 16u * tiles + threadIdx.x] = ((w[0] + w[kRows]) + w[2u * kRows]) + w[3u * kRows];
     }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-    __builtin_amdgcn_s_waitcnt(0);
-    __syncthreads();
-    if (threadIdx.x == 0) {
-      __hip_atomic_fetch_add(sync, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      // Every group's last workgroup counts itself in; this one waits for them all, at most a
-      // fraction of a second (a dispatch that never completes a group leaves the third word set).
-      uint32_t budget = 1u << 18;
-      while (__hip_atomic_load(sync, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < groupsAll && --budget) __builtin_amdgcn_s_sleep(4);
-      if (!budget) __hip_atomic_store(sync + 2, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    __syncthreads();
-    // Every row's sum of squares: part q adds groups q, q + parts, ... in order, the parts are added in order.
-    {
-      constexpr uint32_t kParts = 256u / kRows;
-      const uint32_t row = threadIdx.x % kRows, part = threadIdx.x / kRows;
-      float sum = 0.f;
-      for (uint32_t g = part; g < groupsAll; g += kParts)
-        sum += __hip_atomic_load(rowSquares + size_t(g) * kRows + row, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      partSums[part * kRows + row] = sum;
-      __syncthreads();
-      if (threadIdx.x < kRows) {
-        float total = 0.f;
-        for (uint32_t q = 0; q < kParts; ++q) total += partSums[q * kRows + threadIdx.x];
-        inverse[threadIdx.x] = 1.0f / sqrtf(total / float(p.out_stride) + 1e-6f);
-      }
-      __syncthreads();
-    }
-    if (threadIdx.x == 0) {
-      // The last workgroup through clears the two counts for the next dispatch.
-      const uint32_t passed = __hip_atomic_fetch_add(sync + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      if (passed == groupsAll - 1u) {
-        __hip_atomic_store(sync, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(sync + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      }
-    }
-    // The normalized rows of the workgroup's 64 columns: two groups of the next projection's inputs.
-    const float weight = owns ? bf16_bits_to_float(normWeight[tile.column + c]) : 0.f;
-#pragma unroll
-    for (int t = 0; t < RT; ++t)
-#pragma unroll
-      for (int v = 0; v < 4; ++v) {
-        const uint32_t row = 16u * t + 4u * kq + v;
-        const uint32_t bits = owns && row < p.rows ? float_to_bf16_bits((hidden[t][v] * inverse[row]) * weight) : 0u;
-        tileOut[((wave * RT + t) * 16u + 4u * kq + v) * 16u + c] = uint16_t(bits);
-      }
-    __syncthreads();
+    // The workgroup's 64 columns: two groups of the next projection's inputs.
     const uint32_t G2 = p.out_stride / 32u;
     uint2 *values = reinterpret_cast<uint2 *>(next);
     float *sums32 = reinterpret_cast<float *>(next + gguf_table_sums32_offset(p.out_stride, tiles));
@@ -718,6 +693,7 @@ __global__ __launch_bounds__(256) void gguf_decode(const uint8_t *__restrict__ s
     if constexpr (EP == GGUF_EPILOGUE_GATE_UP_TABLE)
       residual = reinterpret_cast<const uint16_t *>(reinterpret_cast<const uint8_t *>(residual) + piece * gguf_table_bytes(p.out_stride, GGUF_PIECE_TILES));
     else residual += size_t(first) * p.out_stride;
+    if constexpr (EP == GGUF_EPILOGUE_RESIDUAL_NORM) seg2 += piece * gguf_table_bytes(p.out_stride, GGUF_PIECE_TILES);
     partials += size_t(piece) * p.splits * partitioned * 4u * RT * 256u;
     counters += piece * partitioned;
     p.rows -= first;

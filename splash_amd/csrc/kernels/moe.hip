@@ -141,7 +141,7 @@ __global__ __launch_bounds__(64) void moe_gather_table(const uint16_t *__restric
                                                        MoeGatherParams p) {
   const uint32_t g = blockIdx.x, tile = blockIdx.y, lane = threadIdx.x, r = lane & 15u, kq = lane >> 4;
   if (tile >= tile_total[0]) return;
-  const uint32_t G = p.hidden / 32u, row = slot_row[tile * MOE_TILE_ROWS + r];
+  const uint32_t row = slot_row[tile * MOE_TILE_ROWS + r];
   uint8_t *table = tables + tile * p.table_bytes;
   float v[8];
   uint32_t bits[8] = {};

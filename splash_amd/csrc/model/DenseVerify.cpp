@@ -106,11 +106,16 @@ void DenseVerify::encodeEmbedding(hip::CommandGraph &graph, uint32_t rows) {
   ops::Embedding::add(graph, weights_.embedding, inputTokens_, hidden_[0], rows);
 }
 
-void DenseVerify::encodeLayer(hip::CommandGraph &graph, uint32_t layer, const ops::AttentionPlan &plan, uint32_t rows) {
+void DenseVerify::encodeLayer(hip::CommandGraph &graph, uint32_t layer, const ops::AttentionPlan &plan, uint32_t rows,
+                              bool inputReady, bool feedsNext) {
   const DenseLayer &w = weights_.layers.at(layer);
   const hip::Buffer &residual = hidden_[0], &next = hidden_[1];
   // Attention block: hidden[1] = hidden[0] + o(attention(qkv(norm(hidden[0])))).
-  ops::PreparedInput prepared = ops::Normalization::addRmsTable(graph, residual, w.inputNorm, normalized_, scratch_, dims_.hidden, rows);
+  // A table a residual projection's epilogue wrote stands for the normalized rows, which are then
+  // never stored; their inverse RMS is applied by the projection that reads the table.
+  const ops::PreparedInput ready{normalized_, ops::LinearInput::TableUnscaled};
+  ops::PreparedInput prepared =
+      inputReady ? ready : ops::Normalization::addRmsTable(graph, residual, w.inputNorm, normalized_, scratch_, dims_.hidden, rows);
   ops::LinearBuffers qkv;
   qkv.input = normalized_;
   qkv.output = qkv_;
@@ -121,6 +126,9 @@ void DenseVerify::encodeLayer(hip::CommandGraph &graph, uint32_t layer, const op
   ops::AttentionProjectionBuffers projection{qkv_, w.queryNorm, w.keyNorm, ropeCos_, ropeSin_};
   ops::PagedAttention::addProjection(graph, plan, projection, attentionWorkspace_, pages);
   ops::PagedAttention::addAttention(graph, plan, attentionWorkspace_, treeRows_, pages, attention_, nextTable_);
+  // The output projection adds the residual and, where its shape allows, norms the sum into the
+  // gate/up pass's table; the down projection does the same for the layer (or head) after it.
+  const bool outputNorms = linear_.normsRows(w.output, rows);
   ops::LinearBuffers output;
   output.input = attention_;
   output.output = next;
@@ -128,16 +136,32 @@ void DenseVerify::encodeLayer(hip::CommandGraph &graph, uint32_t layer, const op
   output.scratch = scratch_;
   output.scratch.input = nextTable_;
   output.prepared = {attention_, ops::LinearInput::Table16};
-  linear_.add(graph, output, w.output, linear_.plan(w.output, rows, ops::LinearEpilogue::Residual));
+  if (outputNorms) {
+    output.normWeight = w.postNorm;
+    output.nextTable = scratch_.input;
+  }
+  linear_.add(graph, output, w.output,
+              linear_.plan(w.output, rows, outputNorms ? ops::LinearEpilogue::ResidualNorm : ops::LinearEpilogue::Residual));
   // FFN block: hidden[0] = hidden[1] + down(silu(gate n) * up n), n = norm(hidden[1]).
-  prepared = ops::Normalization::addRmsTable(graph, next, w.postNorm, normalized_, scratch_, dims_.hidden, rows);
-  const ops::FfnBuffers ffn{normalized_, intermediate_, scratch_, nextTable_};
+  prepared = outputNorms ? ready : ops::Normalization::addRmsTable(graph, next, w.postNorm, normalized_, scratch_, dims_.hidden, rows);
+  ops::FfnBuffers ffn{normalized_, intermediate_, scratch_, nextTable_};
+  if (feedsNext) {
+    ffn.followingNorm = layer + 1 < dims_.layers ? weights_.layers[layer + 1].inputNorm : weights_.finalNorm;
+    ffn.followingTable = scratch_.input;
+  }
   linear_.addSwiGlu(graph, {&w.gate, &w.up, &w.down}, ffn, next, residual, rows, prepared);
 }
 
-void DenseVerify::encodeHead(hip::CommandGraph &graph, uint32_t rows) {
+bool DenseVerify::layersFeedNext(uint32_t rows) const noexcept {
+  for (const DenseLayer &l : weights_.layers)
+    if (!linear_.normsRows(l.down, rows)) return false;
+  return true;
+}
+
+void DenseVerify::encodeHead(hip::CommandGraph &graph, uint32_t rows, bool inputReady) {
   const ops::PreparedInput prepared =
-      ops::Normalization::addRmsTable(graph, hidden_[0], weights_.finalNorm, normalized_, scratch_, dims_.hidden, rows);
+      inputReady ? ops::PreparedInput{normalized_, ops::LinearInput::TableUnscaled}
+                 : ops::Normalization::addRmsTable(graph, hidden_[0], weights_.finalNorm, normalized_, scratch_, dims_.hidden, rows);
   ops::LinearBuffers head;
   head.input = normalized_;
   head.output = logits_;
@@ -170,8 +194,9 @@ void DenseVerify::encode(hip::CommandGraph &graph, const std::vector<VerifyLane>
   if (dims_.rotaryPairs)
     ops::RoPE::addTreeTables(graph, inverseFrequency_, depths_, ropeCos_, ropeSin_, dims_.rotaryPairs, rope);
   encodeEmbedding(graph, rows);
-  for (uint32_t layer = 0; layer < dims_.layers; ++layer) encodeLayer(graph, layer, plan, rows);
-  encodeHead(graph, rows);
+  const bool feeds = layersFeedNext(rows);
+  for (uint32_t layer = 0; layer < dims_.layers; ++layer) encodeLayer(graph, layer, plan, rows, feeds && layer > 0, feeds);
+  encodeHead(graph, rows, feeds);
   ops::Sampling::addVerify(graph, sampling_, dims_.vocabulary, dims_.vocabulary, laneRows, policies);
   const ops::AcceptanceBuffers acceptance{inputTokens_, treeRows_, tokens_, retained_, acceptedCount_, retainedRows_};
   ops::Sampling::addAcceptance(graph, acceptance, laneRows, remaining,

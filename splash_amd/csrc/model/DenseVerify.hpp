@@ -79,8 +79,14 @@ public:
   void encode(hip::CommandGraph &graph, const std::vector<VerifyLane> &lanes, bool commit = true);
   // Its parts, for per-kernel timing and tests.
   void encodeEmbedding(hip::CommandGraph &graph, uint32_t rows);
-  void encodeLayer(hip::CommandGraph &graph, uint32_t layer, const ops::AttentionPlan &plan, uint32_t rows);
-  void encodeHead(hip::CommandGraph &graph, uint32_t rows);
+  // A layer (or the head) whose predecessor in the same graph left the table of its normalized input
+  // in the projection scratch passes `inputReady`; a layer that passes `feedsNext` leaves that table
+  // for its successor. A part encoded on its own passes neither.
+  void encodeLayer(hip::CommandGraph &graph, uint32_t layer, const ops::AttentionPlan &plan, uint32_t rows,
+                   bool inputReady = false, bool feedsNext = false);
+  void encodeHead(hip::CommandGraph &graph, uint32_t rows, bool inputReady = false);
+  // Whether every layer's down projection can norm its rows for the layer after it.
+  [[nodiscard]] bool layersFeedNext(uint32_t rows) const noexcept;
 
 private:
   hip::Backend &backend_;

@@ -83,11 +83,6 @@ LinearScratchSize LinearPlan::scratchSize() const noexcept {
     size.partials = uint64_t{pieces} * config_.splits * groups * kWavesAcross * pieceTiles * 256u * sizeof(float);
     size.counters = uint64_t{pieces} * groups * sizeof(uint32_t);
   }
-  if (workload_.epilogue == LinearEpilogue::ResidualNorm) {
-    // every column group's sums of squares of the rows, and the words its workgroups meet on
-    size.partials += uint64_t{groupsOf(n, workload_.epilogue)} * storageRows() * sizeof(float);
-    size.counters += GGUF_NORM_SYNC_WORDS * sizeof(uint32_t);
-  }
   return size;
 }
 
@@ -139,7 +134,7 @@ LinearScratchSize Linear::scratchSize(LinearMatrix matrix, uint32_t rows) const 
   LinearScratchSize size;
   for (LinearEpilogue e : {LinearEpilogue::None, LinearEpilogue::Residual, LinearEpilogue::GateUp})
     size.include(plan(LinearWorkload{matrix, rows, e}).scratchSize());
-  if (rows <= kMaximumDecodeTileRows && matrix.outputSize % GGUF_BLOCK == 0)
+  if (matrix.outputSize % GGUF_BLOCK == 0)
     size.include(plan(LinearWorkload{matrix, rows, LinearEpilogue::ResidualNorm}).scratchSize());
   return size;
 }
@@ -177,18 +172,13 @@ PreparedInput Linear::add(hip::CommandGraph &graph, LinearBuffers b, const Proje
   if (w.epilogue == LinearEpilogue::Residual || norms) requireBytes(b.residual, uint64_t{w.rows} * n * 2, "projection residual");
   const LinearScratchSize need = plan.scratchSize();
   requireBytes(b.scratch.input, need.input, "projection table");
-  if (c.splits > 1 || norms) {
+  if (c.splits > 1) {
     requireBytes(b.scratch.partials, need.partials, "projection partials");
     requireBytes(b.scratch.counters, need.counters, "projection counters");
   }
   if (norms) {
     if (p.blocks().segments.size() != 1) throw std::invalid_argument("a projection that norms its rows is one tensor");
     if (n % GGUF_BLOCK) throw std::invalid_argument("a table epilogue takes whole super-blocks of output columns");
-    if (w.rows > kMaximumDecodeTileRows) throw std::invalid_argument("a projection norms up to 64 rows");
-    // One workgroup per column group waits for the others: they all run at once only if the
-    // device holds that many beside the rest of the dispatch.
-    if (groupsOf(n, w.epilogue) > calibration_.computeUnits)
-      throw std::invalid_argument("a projection that norms its rows holds no more column groups than the device has compute units");
     requireBytes(b.normWeight, uint64_t{n} * 2, "norm weight");
     requireBytes(b.nextTable, gguf_tables_bytes(n, gguf_row_tiles(w.rows)), "next projection table");
     if (b.nextTable.sameView(b.scratch.input)) throw std::invalid_argument("the next projection's table is not the plan's own");
@@ -200,7 +190,7 @@ PreparedInput Linear::add(hip::CommandGraph &graph, LinearBuffers b, const Proje
     requireBytes(b.nextTable, gguf_tables_bytes(n, tiles), "next projection table");
     if (b.nextTable.sameView(b.scratch.input)) throw std::invalid_argument("the next projection's table is not the plan's own");
   }
-  const bool prepared = b.prepared.layout == LinearInput::Table16 && b.prepared.source && b.input &&
+  const bool prepared = b.prepared.layout != LinearInput::Plain && b.prepared.source && b.input &&
                         b.prepared.source.sameView(b.input);
   if (!prepared) requireBytes(b.input, uint64_t{w.rows} * k * 2, "projection input");
 
@@ -229,6 +219,7 @@ PreparedInput Linear::add(hip::CommandGraph &graph, LinearBuffers b, const Proje
     }
   }
   params.units = unitsOf(n, w.epilogue);
+  params.deferred_scale = prepared && b.prepared.layout == LinearInput::TableUnscaled;
   // Unused bindings still name a buffer: the table stands in for them.
   const hip::Buffer &spare = b.scratch.input;
   const std::string name = std::string("gguf_decode_") + segments.front().name() + "_m" + std::to_string(plan.storageRows()) +
@@ -240,11 +231,10 @@ PreparedInput Linear::add(hip::CommandGraph &graph, LinearBuffers b, const Proje
   graph.add(name,
             {images[0], images[1], images[2], b.scratch.input, b.output,
              w.epilogue == LinearEpilogue::Residual || norms ? b.residual : writesTable ? b.nextTable : spare,
-             c.splits > 1 || norms ? b.scratch.partials : spare,
-             c.splits > 1 || norms ? b.scratch.counters : spare},
+             c.splits > 1 ? b.scratch.partials : spare, c.splits > 1 ? b.scratch.counters : spare},
             params, {c.wholeGroups + (groupsOf(n, w.epilogue) - c.wholeGroups) * c.splits, rowPieces(w.rows), 1}, {256, 1, 1});
   (void)tiles;
-  return {b.input, LinearInput::Table16};
+  return {b.input, prepared ? b.prepared.layout : LinearInput::Table16};
 }
 
 void Linear::addProjection(hip::CommandGraph &graph, hip::Buffer input, const Projection &projection, hip::Buffer output,
@@ -266,6 +256,11 @@ void Linear::addResidualProjection(hip::CommandGraph &graph, hip::Buffer input, 
   add(graph, std::move(buffers), projection, plan(projection, rows, LinearEpilogue::Residual));
 }
 
+bool Linear::normsRows(const Projection &projection, uint32_t rows) const noexcept {
+  return rows && rows <= kMaximumDispatchRows && projection.blocks().segments.size() == 1 &&
+         projection.outputSize % GGUF_BLOCK == 0;
+}
+
 void Linear::addSwiGlu(hip::CommandGraph &graph, const SwiGluProjections &ffn, const FfnBuffers &b, hip::Buffer residual,
                        hip::Buffer output, uint32_t rows, PreparedInput normalized) const {
   if (!ffn.gate || !ffn.up || !ffn.down) throw std::invalid_argument("a SwiGLU takes gate, up and down projections");
@@ -285,7 +280,12 @@ void Linear::addSwiGlu(hip::CommandGraph &graph, const SwiGluProjections &ffn, c
     down.scratch.input = b.nextTable;
     down.prepared = {b.intermediate, LinearInput::Table16};
   }
-  const LinearPlan downPlan = plan(*ffn.down, rows, LinearEpilogue::Residual);
+  const bool norms = bool(b.followingNorm);
+  if (norms) {
+    down.normWeight = b.followingNorm;
+    down.nextTable = b.followingTable;
+  }
+  const LinearPlan downPlan = plan(*ffn.down, rows, norms ? LinearEpilogue::ResidualNorm : LinearEpilogue::Residual);
   add(graph, std::move(pair), *ffn.up, pairPlan, ffn.gate);
   add(graph, std::move(down), *ffn.down, downPlan);
 }

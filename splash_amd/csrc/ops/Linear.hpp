@@ -91,11 +91,17 @@ struct FfnBuffers final {
   // Optional second activation table: the gate/up pass then writes the down projection's table
   // from its epilogue and the separate table pass is dropped.
   hip::Buffer nextTable{};
+  // Optional norm of the block's output rows: the down projection then also writes their RMS norm
+  // under these weights as the activation table of the projection that follows the block.
+  hip::Buffer followingNorm{}, followingTable{};
 };
 
 enum class LinearInput : uint8_t {
   Plain,    // bf16 [rows][K]
   Table16,  // the activation table of abi/Gguf.h
+  // The table a ResidualNorm plan wrote: rows times the norm's weights, and the sums of squares
+  // their inverse RMS comes from. The projection that reads it scales its own sums by that.
+  TableUnscaled,
 };
 // The scratch table currently holds `source` in `layout` (Linear.hpp:250-256 in the reference).
 struct PreparedInput final {
@@ -171,6 +177,8 @@ public:
                      uint32_t rows, LinearScratch scratch) const;
   void addResidualProjection(hip::CommandGraph &graph, hip::Buffer input, const Projection &projection,
                              hip::Buffer residual, hip::Buffer output, uint32_t rows, LinearScratch scratch) const;
+  // Whether a residual projection of this shape may also norm its rows (LinearEpilogue::ResidualNorm).
+  [[nodiscard]] bool normsRows(const Projection &projection, uint32_t rows) const noexcept;
   // output = residual + down(silu(gate x) * up x) of `rows` normalized rows.
   void addSwiGlu(hip::CommandGraph &graph, const SwiGluProjections &ffn, const FfnBuffers &buffers, hip::Buffer residual,
                  hip::Buffer output, uint32_t rows, PreparedInput normalized = {}) const;

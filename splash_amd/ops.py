@@ -10,6 +10,9 @@ from .backend import Buffer, STORAGE_PRIVATE
 
 FMT_Q4K, FMT_Q6K = 0, 4
 EPILOGUE_NONE, EPILOGUE_RESIDUAL, EPILOGUE_GATE_UP, EPILOGUE_RESIDUAL_NORM = 0, 1, 2, 3
+# `prepared` of Linear.add: the table holds the input rows; or the table a residual + norm plan wrote, whose rows lack
+# their inverse RMS
+PREPARED_TABLE, PREPARED_UNSCALED = 1, 2
 
 
 def gguf_image_bytes(fmt, rows, input_size):
@@ -121,8 +124,8 @@ class Linear:
 
     def add(self, graph, projection, plan, input, output, scratch, residual=None, gate=None, prepared=False, norm_weight=None,
             next_table=None):
-        """norm_weight, next_table: of a plan with EPILOGUE_RESIDUAL_NORM, which also writes the RMS norm of its output
-        rows as the next projection's activation table."""
+        """norm_weight, next_table: of a plan with EPILOGUE_RESIDUAL_NORM, which also writes its output rows times the
+        norm's weights as the next projection's activation table; that projection passes prepared=PREPARED_UNSCALED."""
         if plan.epilogue == EPILOGUE_RESIDUAL_NORM:
             check(lib.spo_linear_add_residual_norm(self.handle, graph.handle, projection.handle, ctypes.byref(plan),
                                                    input.handle if input else None, output.handle if output else None,

@@ -231,16 +231,19 @@ def test_gate_up_table_epilogue_equals_the_table_pass(backend, M):
 
 @pytest.mark.parametrize("fmt,N,K,M,config", [(ops.FMT_Q4K, 5120, 8192, 16, None), (ops.FMT_Q6K, 5120, 5120, 16, None),
                                               (ops.FMT_Q4K, 1024, 2048, 5, (1, 0)), (ops.FMT_Q4K, 1024, 2048, 40, (4, 3)),
-                                              (ops.FMT_Q6K, 768, 1024, 64, (2, 0))])
+                                              (ops.FMT_Q6K, 768, 1024, 64, (2, 0)), (ops.FMT_Q4K, 512, 1024, 100, None)])
 def test_residual_norm_epilogue(backend, fmt, N, K, M, config):
-    """A residual projection may also write the RMS norm of its rows as the next projection's activation table:
-    its output rows are bit-identical to the plain residual projection's, the table is the table of rows within
-    a bf16 step of norm(output) (the row's sum of squares is added in another order), its sums are those of its own
-    values, and a second dispatch over the same scratch (whose counts the first cleared) repeats it bit for bit."""
+    """A residual projection may also leave its rows as the activation table of the projection after their RMS
+    norm. Its output rows are bit-identical to the plain residual projection's; the table is bit for bit the
+    table of bf16(output * weight) (an exact fp32 product, rounded once) and ends with every 64-column group's
+    sums of squares of the output rows. The projection that reads the table as one that lacks its scale gives the
+    oracle's projection of those table rows times each row's inverse RMS, to the oracle's own error bound; against
+    the norm pass's rounding (bf16(output * inverse RMS * weight)) it differs by that one operand rounding."""
     print(f"case residual norm epilogue fmt={fmt} N={N} K={K} M={M} config={config}", flush=True)
     rng = np.random.default_rng(N + M)
     linear = ops.Linear(backend)
-    proj = ops.Projection.from_native(backend, [(fmt, N, orc.make_native(fmt, N, K, 9))], K)
+    native = orc.make_native(fmt, N, K, 9)
+    proj = ops.Projection.from_native(backend, [(fmt, N, native)], K)
     x = backend.from_array(orc.f32_to_bf16(rng.standard_normal((M, K)).astype(np.float32)))
     residual_bits = orc.f32_to_bf16(rng.standard_normal((M, N)).astype(np.float32))
     weight_bits = orc.f32_to_bf16((1 + 0.1 * rng.standard_normal(N)).astype(np.float32))
@@ -249,32 +252,65 @@ def test_residual_norm_epilogue(backend, fmt, N, K, M, config):
     plain_plan = linear.plan(proj, M, ops.EPILOGUE_RESIDUAL, **kwargs)
     plan = linear.plan(proj, M, ops.EPILOGUE_RESIDUAL_NORM, **kwargs)
     assert (plan.splits, plan.whole_groups) == (plain_plan.splits, plain_plan.whole_groups)
-    scratch = linear.scratch_for(backend, [plan, plain_plan])
+    # the projection after the norm: N inputs, 256 fp32 outputs
+    N2 = 256
+    native2 = orc.make_native(ops.FMT_Q4K, N2, N, 5)
+    proj2 = ops.Projection.from_native(backend, [(ops.FMT_Q4K, N2, native2)], N, float32=True)
+    plan2 = linear.plan(proj2, M)
+    scratch = linear.scratch_for(backend, [plan, plain_plan, plan2])
     out_plain, out = backend.allocate_buffer(M * N * 2), backend.allocate_buffer(M * N * 2)
-    table = backend.allocate_buffer(ops.gguf_table_bytes(N, M))
+    table_bytes = ops.gguf_table_bytes(N, M)
+    next_scratch = ops.LinearScratch(backend, table_bytes)
+    next_scratch.partials, next_scratch.counters = scratch.partials, scratch.counters
+    after = backend.allocate_buffer(M * N2 * 4)
+    normalized = backend.allocate_buffer(M * N * 2)   # stands for the rows the table holds; never read
     graph = splash_amd.CommandGraph()
     linear.add(graph, proj, plain_plan, x, out_plain, scratch, residual=residual)
     backend.run(graph)
     graph = splash_amd.CommandGraph()
-    linear.add(graph, proj, plan, x, out, scratch, residual=residual, norm_weight=weight, next_table=table)
+    linear.add(graph, proj, plan, x, out, scratch, residual=residual, norm_weight=weight, next_table=next_scratch.table)
     assert len(graph) == 2          # the table pass of its own input, then the projection
+    linear.add(graph, proj2, plan2, normalized, after, next_scratch, prepared=ops.PREPARED_UNSCALED)
+    assert len(graph) == 3          # no table pass: the table is there
     backend.run(graph)
     hidden = out.download(np.uint16).reshape(M, N)
     assert np.array_equal(hidden, out_plain.download(np.uint16).reshape(M, N))
-    first = table.download(np.uint8)[:ops.gguf_table_bytes(N, M)].copy()
-    tiles = (M + 15) // 16
-    values, s32, s16 = orc.split_activation_table(first, N, tiles)
-    want = orc.rms_norm(hidden, weight_bits)
-    wv, _, _ = orc.activation_table(want)
-    steps = np.abs(ulp_key(values) - ulp_key(wv))
-    assert steps.max() <= 1 and (steps > 0).mean() < 1e-3, (steps.max(), (steps > 0).mean())
-    # the sums are those of the table's own values
-    own_values, own32, own16 = orc.activation_table(orc.table_rows(values, N, tiles))
-    assert np.array_equal(own_values, values) and own32.tobytes() == s32.tobytes() and own16.tobytes() == s16.tobytes()
-    sync = scratch.counters.download(np.uint32)
-    assert not sync.any()            # the counts are cleared and no wait expired
+    raw = next_scratch.table.download(np.uint8)[:table_bytes].copy()
+    # pieces of 64 rows, each with a table of its own
+    scaled = orc.f32_to_bf16(orc.bf16_to_f32(hidden) * orc.bf16_to_f32(weight_bits)[None, :])
+    inverse = np.empty(M)
+    at = 0
+    for first in range(0, M, 64):
+        rows = min(64, M - first)
+        tiles = (rows + 15) // 16
+        size = ops.gguf_table_bytes(N, rows)
+        piece = raw[at:at + size]
+        at += size
+        values, s32, s16 = orc.split_activation_table(piece, N, tiles)
+        wv, w32, w16 = orc.activation_table(scaled[first:first + rows])
+        assert np.array_equal(values, wv)
+        assert s32.tobytes() == w32.tobytes() and s16.tobytes() == w16.tobytes()
+        squares = piece[size - (N // 64) * 16 * tiles * 4:].view(np.float32).reshape(N // 64, 16 * tiles)
+        h = orc.bf16_to_f32(hidden[first:first + rows]).astype(np.float64)
+        want = (h.reshape(rows, N // 64, 64) ** 2).sum(axis=2).T
+        assert np.allclose(squares[:, :rows], want, rtol=1e-5, atol=0)
+        assert not squares[:, rows:].any()
+        inverse[first:first + rows] = 1.0 / np.sqrt(want.sum(axis=0) / N + 1e-6)
+    assert at == table_bytes
+    got = after.download(np.float32).reshape(M, N2)
+    res = orc.gemm(ops.FMT_Q4K, native2, scaled, N2, want=("exact", "bound"))
+    error = np.abs(got - res["exact"] * inverse[:, None])
+    assert (error <= res["bound"] * inverse[:, None] * 1.01 + 1e-5 * np.abs(got)).all(), error.max()
+    # against the rounding points of a norm pass before the projection
+    normed = orc.rms_norm(hidden, weight_bits)
+    reference = orc.gemm(ops.FMT_Q4K, native2, normed, N2, want=("exact",))["exact"]
+    assert np.abs(got - reference).max() <= 2e-2 * np.sqrt((reference ** 2).mean())
+    cosine = (got * reference).sum() / np.sqrt((got ** 2).sum() * (reference ** 2).sum())
+    assert cosine >= 0.99999
+    # a second run repeats the table bit for bit
     backend.run(graph)
-    assert np.array_equal(table.download(np.uint8)[:len(first)], first)
+    assert np.array_equal(next_scratch.table.download(np.uint8)[:table_bytes], raw)
+    assert np.array_equal(after.download(np.float32).reshape(M, N2), got)
     with pytest.raises(ValueError, match="next projection table"):
         linear.add(splash_amd.CommandGraph(), proj, plan, x, out, scratch, residual=residual, norm_weight=weight)
 

@@ -56,7 +56,11 @@ def test_config1_verify_step(backend, rows, context):
     final = hidden_of()
     backend.run(gpu.encode_part(2, 0, [lane]))
     got_logits = gpu.buffer(verify.LOGITS).download(np.float32, rows * 32000).reshape(rows, 32000)
-    assert np.array_equal(got_logits, chain_logits)     # parts and whole are the same dispatches: bit-identical
+    # A part starts with a norm pass over its input rows; inside the whole step the projection before it wrote
+    # that table without the rows' inverse RMS, which the reading projection applies to its sums: one bf16
+    # operand rounding apart.
+    part_cos = (got_logits.astype(np.float64) * chain_logits).sum() / np.sqrt((got_logits.astype(np.float64) ** 2).sum() * (chain_logits.astype(np.float64) ** 2).sum())
+    assert part_cos >= 0.9999 and np.abs(got_logits - chain_logits).max() <= 2e-2, part_cos
     want_logits = model.oracle_head(final)
     cos = (got_logits.astype(np.float64) * want_logits).sum() / np.sqrt((got_logits.astype(np.float64) ** 2).sum() * (want_logits ** 2).sum())
     err = np.abs(got_logits - want_logits).max()
