@@ -161,7 +161,7 @@ template <int D, int G>
 __global__ __launch_bounds__(256, 2) void attention_q8_split(const _Float16 *__restrict__ queries, const float *__restrict__ qsums,
                                                           const AttentionTreeRow *__restrict__ tree,
                                                           const uint64_t *__restrict__ page_table, uint8_t *__restrict__ pool,
-                                                          float *__restrict__ partialO, float *__restrict__ partialML,
+                                                          _Float16 *__restrict__ partialO, float *__restrict__ partialML,
                                                           AttentionParams p) {
   constexpr int kStep = 64, JD = D / 32, DT = D / 16;
   constexpr int kTiles = (G + 3) / 4;  // fused-row tiles (one query head's 16 rows each) per wave
@@ -379,7 +379,10 @@ __global__ __launch_bounds__(256, 2) void attention_q8_split(const _Float16 *__r
     __syncthreads();
   }
 
-  // The split's partials: the code offset leaves with the row's sum of P, the 2^10 with a scale.
+  // The split's partials: the code offset leaves with the row's sum of P, the 2^10 with a scale. The
+  // outputs leave divided by the row's sum, a weighted mean of value rows whatever the split's
+  // length, as fp16: a lane's 4 DT values are contiguous (position 4 DT kq + 4 dt + i of the row
+  // holds dimension 16 dt + 4 kq + i), so a row's 2 D bytes go out as whole 16-byte stores.
 #pragma unroll
   for (int k = 0; k < kTiles; ++k) {
     if (!owns[k]) continue;
@@ -389,14 +392,17 @@ __global__ __launch_bounds__(256, 2) void attention_q8_split(const _Float16 *__r
     sum += __shfl_xor(sum, 32, 64);
     const size_t fused = ((size_t(z) * p.kv_heads + h) * p.splits + split) * (16u * G) + 16u * g + row;
     const float rowSum = o[k][DT][0] * kCodeOffset;
+    const float norm = sum > 0.f ? 1.0f / (sum * kPScale) : 0.f;
+    uint4 *mine = reinterpret_cast<uint4 *>(partialO + fused * D + 4u * DT * kq);
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-      float4 out;
-      out.x = (o[k][dt][0] - rowSum) * (1.0f / kPScale);
-      out.y = (o[k][dt][1] - rowSum) * (1.0f / kPScale);
-      out.z = (o[k][dt][2] - rowSum) * (1.0f / kPScale);
-      out.w = (o[k][dt][3] - rowSum) * (1.0f / kPScale);
-      *reinterpret_cast<float4 *>(partialO + fused * D + 16 * dt + 4 * kq) = out;
+    for (int dt = 0; dt < DT; dt += 2) {
+      f16x8 out;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        out[i] = _Float16((o[k][dt][i] - rowSum) * norm);
+        out[4 + i] = _Float16((o[k][dt + 1][i] - rowSum) * norm);
+      }
+      mine[dt / 2] = __builtin_bit_cast(uint4, out);
     }
     if (kq == 0) {
       partialML[2 * fused] = m[k];
@@ -411,14 +417,16 @@ SP_REGISTER_KERNEL("attention_q8_split_d64_g2", &attention_q8_split<64, 2>);
 // ---------------------------------------------------------------------------------------------
 // attention_reduce: grid (q_heads, 16, sequences), 256 threads. Merges the splits of one (head,
 // row) in a fixed order (paged_attention_tile.h:499-535) and writes bf16 [packed row][q_heads * D].
-// Thread (part, quad) sums splits part, part + P, ... of dimensions 4 quad .. 4 quad + 3, all its
-// loads in flight together; the P parts are then added in part order.
+// Thread (part, quad) sums splits part, part + P, ... of the row's positions 4 quad .. 4 quad + 3
+// (four dimensions in a row, in the order the split kernel leaves them), all its loads in flight
+// together; the P parts are then added in part order. A split weighs exp2(its maximum - the
+// largest) times its sum: its outputs arrive divided by that sum.
 // ---------------------------------------------------------------------------------------------
 // The _t variant also writes the rows as the activation table (abi/Gguf.h) of the projection that
 // follows, as gguf_prepare_table would from `out`; p.table_tiles is the table's row tiles. Rows of
 // a tile past the packed rows keep what the table held.
 template <int D, bool Table>
-__global__ __launch_bounds__(256) void attention_reduce(const float *__restrict__ partialO, const float *__restrict__ partialML,
+__global__ __launch_bounds__(256) void attention_reduce(const _Float16 *__restrict__ partialO, const float *__restrict__ partialML,
                                                         uint16_t *__restrict__ out, uint8_t *__restrict__ table,
                                                         const uint16_t *__restrict__ qkv, AttentionParams p) {
   constexpr uint32_t kQuads = D / 4, kParts = 256 / kQuads;
@@ -442,31 +450,34 @@ __global__ __launch_bounds__(256) void attention_reduce(const float *__restrict_
   }
   const float maximum = block_max<256>(ms, scratch, tid);
   const float weight = ms == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ms - maximum);
-  if (tid < ATTENTION_MAXIMUM_SPLITS) weights[tid] = weight;
+  if (tid < ATTENTION_MAXIMUM_SPLITS) weights[tid] = weight * ls;
   const float denominator = block_sum<256>(weight * ls, scratch, tid);  // block_sum's barriers publish the weights too
 
   const uint32_t part = tid / kQuads, quad = tid % kQuads;
   float4 total = make_float4(0.f, 0.f, 0.f, 0.f);
+  typedef __attribute__((ext_vector_type(4))) _Float16 f16x4;
   for (uint32_t s0 = part; s0 < p.splits; s0 += 4u * kParts) {
-    float4 held[4];
+    uint2 held[4];
 #pragma unroll
     for (uint32_t i = 0; i < 4u; ++i) {
       const uint32_t s = s0 + i * kParts;
-      held[i] = s < p.splits ? reinterpret_cast<const float4 *>(partialO + fusedOf(s) * D)[quad] : make_float4(0.f, 0.f, 0.f, 0.f);
+      held[i] = s < p.splits ? reinterpret_cast<const uint2 *>(partialO + fusedOf(s) * D)[quad] : make_uint2(0u, 0u);
     }
 #pragma unroll
     for (uint32_t i = 0; i < 4u; ++i) {
       const uint32_t s = s0 + i * kParts;
       const float w = s < p.splits ? weights[s] : 0.f;
       if (w != 0.f) {  // a split without a visible token may hold anything
-        total.x += w * held[i].x;
-        total.y += w * held[i].y;
-        total.z += w * held[i].z;
-        total.w += w * held[i].w;
+        const f16x4 x = __builtin_bit_cast(f16x4, held[i]);
+        total.x += w * float(x[0]);
+        total.y += w * float(x[1]);
+        total.z += w * float(x[2]);
+        total.w += w * float(x[3]);
       }
     }
   }
-  sums[part][quad] = total;
+  // position quad of the row is dimensions 16 (quad % DT) + 4 (quad / DT) ..
+  sums[part][4u * (quad % (D / 16u)) + quad / (D / 16u)] = total;
   __syncthreads();
   if (tid < D) {
     const float *flat = reinterpret_cast<const float *>(&sums[0][0]);

@@ -67,7 +67,7 @@ DenseVerify::DenseVerify(hip::Backend &backend, DenseDimensions d, uint32_t maxL
   maxSplits_ = ATTENTION_MAXIMUM_SPLITS;
   attentionWorkspace_.queries = device(fused * d.headDimension * 2, "staged queries");
   attentionWorkspace_.querySums = device(fused * 4, "query sums");
-  attentionWorkspace_.partials = device(fused * maxSplits_ * d.headDimension * 4, "attention partials");
+  attentionWorkspace_.partials = device(fused * maxSplits_ * d.headDimension * 2, "attention partials");
   attentionWorkspace_.partialSums = device(fused * maxSplits_ * 8, "attention partial sums");
   const ops::SamplingWorkspaceSize s = ops::Sampling::workspace(maxRows_);
   sampling_.logits = logits_;

@@ -82,7 +82,7 @@ HybridVerify::HybridVerify(hip::Backend &backend, HybridDimensions d, uint32_t m
   const uint64_t fused = uint64_t{maxLanes} * d.kvHeads * (d.qHeads / std::max(1u, d.kvHeads)) * 16;
   attentionWorkspace_.queries = device(fused * d.headDimension * 2, "staged queries");
   attentionWorkspace_.querySums = device(fused * 4, "query sums");
-  attentionWorkspace_.partials = device(fused * ATTENTION_MAXIMUM_SPLITS * d.headDimension * 4, "attention partials");
+  attentionWorkspace_.partials = device(fused * ATTENTION_MAXIMUM_SPLITS * d.headDimension * 2, "attention partials");
   attentionWorkspace_.partialSums = device(fused * ATTENTION_MAXIMUM_SPLITS * 8, "attention partial sums");
   const ops::MoeWorkspaceSize moe = ops::MoE::workspace(d.moeShape(), maxRows_);
   moeWorkspace_ = {device(moe.selected, "moe selected"),    device(moe.weights, "moe weights"),     device(moe.routeSlot, "moe route slots"),

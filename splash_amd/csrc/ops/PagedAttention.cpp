@@ -43,7 +43,7 @@ AttentionWorkspaceSize AttentionPlan::workspace() const noexcept {
   AttentionWorkspaceSize size;
   size.queries = fused * geometry_.headDimension * 2;
   size.querySums = fused * 4;
-  size.partials = fused * splits_ * geometry_.headDimension * 4;
+  size.partials = fused * splits_ * geometry_.headDimension * 2;
   size.partialSums = fused * splits_ * 8;
   return size;
 }

@@ -59,7 +59,7 @@ struct AttentionWorkspaceSize final {
 struct AttentionWorkspace final {
   hip::Buffer queries;      // staged fp16 query rows
   hip::Buffer querySums;    // their fp32 sums
-  hip::Buffer partials;     // fp32 split outputs
+  hip::Buffer partials;     // fp16 split outputs, each divided by its sum
   hip::Buffer partialSums;  // fp32 (max, sum) per split and fused row
 };
 
