@@ -24,7 +24,7 @@ HBM_PEAK_GBS = 8000.0   # MI355X published HBM3E bandwidth
 # HBM bytes per launch of the one-pass gate/up projection, by (hidden, ffn, rows): FETCH_SIZE + WRITE_SIZE of
 # rocprofv3 --pmc runs of this file, each scaled by what the counter reads for the copy kernel's known bytes
 # (profiles/verify_step_c4_hbm_traffic.md). Counters cannot be read from inside the run.
-GATE_UP_TRAFFIC_BYTES = {(5120, 25600, 16): 124.1e6}
+GATE_UP_TRAFFIC_BYTES = {(5120, 25600, 16): 124.2e6}
 
 WORKLOADS = {
     # hidden, q heads, kv heads, head dim, ffn, vocabulary, layers, context, rows
