@@ -145,6 +145,103 @@ def cpu_baseline(w):
                       f"({gemm_seconds + attention_seconds:.1f}s of CPU work on {cores} threads)"}
 
 
+def time_c2_ops(backend):
+    """BASELINE config 2: each projection of the 27B shape alone at M = 1, 4, 8, 16, 32 rows, over a ring of weight
+    copies larger than twice the 256 MB memory-side cache so that every pass reads HBM; per-dispatch GPU time (HIP
+    events around each dispatch), median over the ring passes after the first. Prints one JSON line."""
+    import splash_amd
+    from splash_amd import ops
+    rng = np.random.default_rng(0)
+    bf = lambda a: (np.ascontiguousarray(a, np.float32).view(np.uint32) >> 16).astype(np.uint16)
+    linear = ops.Linear(backend)
+    H, F, Q, KV = 5120, 25600, 8192, 1024
+    cases = [("gate_up", ops.FMT_Q4K, [F], H, ops.EPILOGUE_GATE_UP, 2), ("qkv", ops.FMT_Q4K, [Q, KV, KV], H, ops.EPILOGUE_NONE, 1),
+             ("o_proj", ops.FMT_Q4K, [H], Q, ops.EPILOGUE_RESIDUAL, 1), ("down", ops.FMT_Q6K, [H], F, ops.EPILOGUE_RESIDUAL, 1)]
+    results = []
+    for name, fmt, widths, K, epilogue, tensors in cases:
+        N = sum(widths)
+        weight_bytes = tensors * ops.gguf_image_bytes(fmt, N, K)
+        copies = int(np.ceil(2 * 268.4e6 / weight_bytes)) + 1
+        images = [rng.integers(0, 256, ops.gguf_image_bytes(fmt, n, K), dtype=np.uint8) for n in widths]
+        ring = [ops.Projection([(fmt, n, backend.from_array(im)) for n, im in zip(widths, images)], K) for _ in range(copies)]
+        gates = [ops.Projection([(fmt, N, backend.from_array(images[0]))], K) for _ in range(copies)] if tensors == 2 else None
+        for M in (1, 4, 8, 16, 32):
+            x = backend.from_array(bf(rng.standard_normal((M, K))))
+            out, residual = backend.allocate_buffer(M * N * 4), backend.allocate_buffer(M * N * 2)
+            plan = linear.plan(ring[0], M, epilogue)
+            scratch = linear.scratch_for(backend, [plan])
+            graph = splash_amd.CommandGraph()
+            linear.add(graph, ring[0], plan, x, out, scratch, residual=residual, gate=gates[0] if gates else None)   # table pass + first
+            passes = 4
+            for _ in range(passes):
+                for c in range(copies):
+                    linear.add(graph, ring[c], plan, x, out, scratch, residual=residual, gate=gates[c] if gates else None, prepared=True)
+            backend.set_dispatch_profiling(True)
+            _, _, per = backend.run(graph, profiled=True)
+            backend.set_dispatch_profiling(False)
+            us = float(np.median(np.array(per[2 + copies:]) * 1e6))
+            out_bytes = M * N * 2
+            algorithmic = weight_bytes + M * K * 2 + out_bytes
+            results.append({"op": name, "format": "q4_k" if fmt == ops.FMT_Q4K else "q6_k", "N": N * tensors if tensors == 2 else N, "K": K,
+                            "M": M, "splits": plan.splits, "us": round(us, 2), "GB/s": round(algorithmic / us / 1e3, 1),
+                            "frac": round(algorithmic / us / 1e3 / HBM_PEAK_GBS, 4)})
+            log(f"  {name:8s} M={M:2d} splits={plan.splits:2d} {us:7.2f} us {algorithmic / us / 1e3:7.1f} GB/s")
+            del graph, x, out, residual, scratch
+        del ring, gates
+    print(json.dumps({"metric": "projection us and GB/s by rows (config 2)", "unit": "us", "n_gpus": 1, "data": "synthetic: random images in a ring past the caches",
+                      "roofline_peak_gbs": HBM_PEAK_GBS, "results": results}), flush=True)
+
+
+def time_c3_ops(backend):
+    """BASELINE config 3: block-causal attention of a 16-row chain block (64 query / 8 KV heads of 128) over a paged
+    INT8 context of 8K, 32K and 128K tokens (256-token pages, random page table), the split pass and the merge, over a
+    ring of KV pools past the caches. Prints one JSON line."""
+    import splash_amd
+    from splash_amd import ops, synthetic
+    rng = np.random.default_rng(0)
+    bf = lambda a: (np.ascontiguousarray(a, np.float32).view(np.uint32) >> 16).astype(np.uint16)
+    QH, KVH, D, rows = 64, 8, 128, 16
+    results = []
+    for context in (8192, 32768, 131072):
+        pages = (context + ops.PAGE_TOKENS - 1) // ops.PAGE_TOKENS
+        kv_bytes = context * KVH * (2 * D + 4)
+        copies = int(np.ceil(2 * 268.4e6 / kv_bytes)) + 1
+        raw = synthetic.kv_pages(rng, KVH, D, 8)
+        raw = np.tile(raw, ((pages + 7) // 8, 1))[:pages]
+        table = rng.permutation(pages).astype(np.uint64)
+        pools = []
+        for _ in range(copies):
+            pool = ops.KvPages(backend, KVH, D, pages, table)
+            pool.upload(raw)
+            pools.append(pool)
+        plan = ops.AttentionPlan(QH, KVH, D, [(0, rows, context - rows, 0)])
+        workspace = ops.AttentionWorkspace(backend, plan)
+        qkv = backend.from_array(bf(rng.standard_normal((rows, (QH + 2 * KVH) * D))))
+        tree = backend.from_array(ops.chain_tree_rows([rows]))
+        out = backend.allocate_buffer(rows * QH * D * 2)
+        graph = splash_amd.CommandGraph()
+        ops.PagedAttention.add_projection(graph, plan, qkv, workspace, pools[0])
+        passes = 4
+        for _ in range(passes):
+            for pool in pools:
+                ops.PagedAttention.add_attention(graph, plan, workspace, tree, pool, out)
+        backend.set_dispatch_profiling(True)
+        _, _, per = backend.run(graph, profiled=True)
+        backend.set_dispatch_profiling(False)
+        pairs = np.array(per[1:]).reshape(-1, 2)[copies:] * 1e6
+        split_us, merge_us = float(np.median(pairs[:, 0])), float(np.median(pairs[:, 1]))
+        algorithmic = kv_bytes + rows * QH * D * 2 * 2 + pages * 8
+        results.append({"context": context, "splits": plan.splits, "split_us": round(split_us, 2), "merge_us": round(merge_us, 2),
+                        "GB/s": round(algorithmic / (split_us + merge_us) / 1e3, 1),
+                        "frac": round(algorithmic / (split_us + merge_us) / 1e3 / HBM_PEAK_GBS, 4),
+                        "TFLOP/s": round(4 * rows * QH * D * context / (split_us + merge_us) / 1e6, 1)})
+        log(f"  context {context:6d} splits {plan.splits:2d}: split {split_us:7.2f} us merge {merge_us:6.2f} us {algorithmic / (split_us + merge_us) / 1e3:7.1f} GB/s")
+        del graph, pools, workspace
+    print(json.dumps({"metric": "attention us and GB/s by context (config 3)", "unit": "us", "n_gpus": 1,
+                      "data": "synthetic: uniform INT8 codes, random page table, ring of pools past the caches",
+                      "roofline_peak_gbs": HBM_PEAK_GBS, "results": results}), flush=True)
+
+
 def time_c5_ops(backend):
     """Per-dispatch GPU time (HIP events around each dispatch) of the Gated DeltaNet step and the MoE layer at the
     35B-A3B shape of BASELINE config 5, batch 8 of 16-row blocks; weights and states in rings past the caches.
@@ -315,7 +412,12 @@ def main():
     ap.add_argument("--workload", default="c4", choices=sorted(WORKLOADS) + ["c5"])
     ap.add_argument("--lanes", type=int, default=1)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--ops", choices=["c5"], help="time the GDN step and the MoE layer of config 5 instead of the dense step")
+    ap.add_argument("--temperature", type=float, default=0.0,
+                    help="above 0: rejection-sampling acceptance at this temperature against a full-vocabulary draft "
+                         "distribution softmax(N(0, 2)) instead of greedy acceptance")
+    ap.add_argument("--ops", choices=["c2", "c3", "c5"],
+                    help="instead of the dense step: c2 the projections alone by rows, c3 attention alone by context, "
+                         "c5 the GDN step and the MoE layer of config 5")
     args = ap.parse_args()
     if args.gpus != 1:
         log("bench.py measures one GPU: this build runs the verify step on a single MI355X (no collectives); use --gpus 1")
@@ -323,8 +425,8 @@ def main():
     import splash_amd
     from splash_amd import ops, verify
     backend = splash_amd.Backend(0)
-    if args.ops == "c5":
-        time_c5_ops(backend)
+    if args.ops:
+        {"c2": time_c2_ops, "c3": time_c3_ops, "c5": time_c5_ops}[args.ops](backend)
         return
     if args.workload == "c5":
         bench_c5(backend, args)
@@ -336,11 +438,17 @@ def main():
     gpu = build_model(backend, w, args.lanes)
     log(f"model resident in {time.time() - t0:.1f}s; allocated {backend.memory_stats().allocated_bytes / 1e9:.2f} GB")
     context_pages = (w["context"] + ops.PAGE_TOKENS - 1) // ops.PAGE_TOKENS
-    lanes = [verify.Lane(w["rows"], w["context"] - w["rows"], table_first=i * context_pages) for i in range(args.lanes)]
+    lanes = [verify.Lane(w["rows"], w["context"] - w["rows"], table_first=i * context_pages, temperature=args.temperature)
+             for i in range(args.lanes)]
     rows = w["rows"] * args.lanes
     rng = np.random.default_rng(1)
-    gpu.set_block(lanes, rng.integers(0, w["vocabulary"], rows).astype(np.uint32))
+    gpu.set_block(lanes, rng.integers(0, w["vocabulary"], rows).astype(np.uint32), uniforms=rng.random((rows, 2), dtype=np.float32))
     graph = gpu.encode(lanes, commit=True)
+    if args.temperature > 0:
+        # the draft model's distributions of the block's rows: softmax of N(0, 2) logits over the whole vocabulary
+        draft = np.exp(rng.normal(0.0, 2.0, (rows, w["vocabulary"])).astype(np.float32))
+        draft /= draft.sum(axis=1, keepdims=True)
+        gpu.buffer(verify.DRAFT_PROBABILITIES).upload(draft.astype(np.float32))
     kernels = graph.kernels()
     step_bytes = gpu.step_bytes(lanes)
     log(f"step: {len(kernels)} dispatches, {step_bytes / 1e9:.3f} GB algorithmic")
@@ -382,7 +490,8 @@ def main():
         "data": "synthetic: native Q4_K/Q6_K blocks with uniform codes and model-like scales (every layer a copy in its own HBM), "
                 "uniform INT8 KV codes, uniform-random draft tokens, random page table",
         "config": {"workload": w["name"], "lanes": args.lanes, "rows_per_lane": w["rows"], "context_tokens": w["context"],
-                   "layers": w["layers"], "dispatches": len(kernels), "acceptance": "greedy"},
+                   "layers": w["layers"], "dispatches": len(kernels),
+                   "acceptance": f"rejection sampling, T = {args.temperature}" if args.temperature > 0 else "greedy"},
         "step_hbm": {"algorithmic_gb": round(step_bytes / 1e9, 3), "achieved_gbs": round(step_bytes / (ms * 1e-3) / 1e9, 1),
                      "frac_of_peak": round(step_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "wall_ms_per_step": round(wall_ms, 4)},
         "roofline": {"bound": "hbm", "kernel": gate_up, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
