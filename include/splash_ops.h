@@ -216,6 +216,13 @@ sp_status spo_moe_add_routing(spo_graph *graph, sp_buffer *scores, uint32_t scor
 sp_status spo_moe_add_routed(spo_graph *graph, sp_buffer *normalized, sp_buffer *residual, sp_buffer *output, sp_buffer *gate_images,
                              sp_buffer *up_images, sp_buffer *down_images, uint32_t format, uint32_t down_format,
                              const spo_moe_workspace *workspace, const spo_moe_shape *shape, uint32_t rows);
+/* The same, and the output rows also leave as the activation table (spo_gguf_table_bytes(hidden, rows) bytes) of the
+ * projection after their RMS norm under norm_weight (bf16 [hidden]), as spo_linear_add_residual_norm writes it: that
+ * projection is added with `prepared` = 2 and no norm dispatch runs before it. hidden a multiple of 256. */
+sp_status spo_moe_add_routed_norm(spo_graph *graph, sp_buffer *normalized, sp_buffer *residual, sp_buffer *output,
+                                  sp_buffer *gate_images, sp_buffer *up_images, sp_buffer *down_images, uint32_t format,
+                                  uint32_t down_format, const spo_moe_workspace *workspace, const spo_moe_shape *shape,
+                                  uint32_t rows, sp_buffer *norm_weight, sp_buffer *next_table);
 
 /* ---- Sampling (runtime/ops/Sampling.hpp:64-254, Sampling.cpp:283-357) ---- */
 typedef struct spo_lane_rows { uint32_t first, rows; } spo_lane_rows; /* SplashLaneRows */

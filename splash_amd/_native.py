@@ -246,6 +246,7 @@ _sig("spo_gdn_add_fold", c_int, c_p, c_p, c_p, c_p, c_u64, c_u64, c_u64, P(GdnSh
 _sig("spo_moe_workspace_sizes", c_int, P(MoeShape), c_u32, P(c_u64))
 _sig("spo_moe_add_routing", c_int, c_p, c_p, c_u32, P(MoeWorkspace), P(MoeShape), c_u32)
 _sig("spo_moe_add_routed", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_u32, c_u32, P(MoeWorkspace), P(MoeShape), c_u32)
+_sig("spo_moe_add_routed_norm", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_u32, c_u32, P(MoeWorkspace), P(MoeShape), c_u32, c_p, c_p)
 _sig("spo_row_copy_add", c_int, c_p, c_p, c_u32, c_u32, c_u32, c_p, c_u32, c_u32, c_u32, c_u32, c_u32)
 _sig("spo_sampling_workspace", c_int, c_u32, P(c_u64))
 _sig("spo_sampling_add_verify", c_int, c_p, P(SamplingBuffers), c_u32, c_u32, P(LaneRows), P(SamplingPolicy), c_u32, P(c_u32))

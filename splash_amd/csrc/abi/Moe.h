@@ -43,9 +43,12 @@ struct MoeGatherParams {
   uint64_t table_bytes;  // between tiles' tables
 };
 // moe_combine: grid (rows, hidden / 256), 256 threads: out = bf16(residual + sum_rank w y[slot]) in rank order.
+// table_tiles nonzero (hidden a multiple of 256): the rows also leave as the activation table (abi/Gguf.h, pieces of
+// 64 rows, table_tiles row tiles in all) of the projection after their RMS norm, as a residual projection's _rn
+// epilogue writes it: bf16(out * norm weight) and each 64-column group's sums of squares of `out`.
 struct MoeCombineParams {
   uint32_t rows, hidden, top_k;
-  uint32_t reserved;
+  uint32_t table_tiles;
 };
 
 // gguf_moe_decode_<fmt>_<a|gt>: grid (workgroups of one expert projection, maximum tiles), 256 threads.

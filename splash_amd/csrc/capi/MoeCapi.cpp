@@ -46,4 +46,16 @@ sp_status spo_moe_add_routed(spo_graph *graph, sp_buffer *normalized, sp_buffer 
   });
 }
 
+sp_status spo_moe_add_routed_norm(spo_graph *graph, sp_buffer *normalized, sp_buffer *residual, sp_buffer *output,
+                                  sp_buffer *gate_images, sp_buffer *up_images, sp_buffer *down_images, uint32_t format,
+                                  uint32_t down_format, const spo_moe_workspace *workspace, const spo_moe_shape *shape,
+                                  uint32_t rows, sp_buffer *norm_weight, sp_buffer *next_table) {
+  return capi::guard([&] {
+    capi::require(graph && workspace && shape && norm_weight && next_table, "graph, workspace, shape, norm weight or table");
+    ops::MoE::addRouted(capi::graphOf(graph), B(normalized), B(residual), B(output),
+                        ops::MoeExperts{B(gate_images), B(up_images), B(down_images), format, down_format}, workspaceOf(*workspace),
+                        shapeOf(*shape), rows, ops::MoeFollowingNorm{B(norm_weight), B(next_table)});
+  });
+}
+
 } // extern "C"

@@ -178,15 +178,57 @@ SP_REGISTER_KERNEL("moe_gather_table", &moe_gather_table);
 // moe_combine (moe.metal:367-392): out = bf16(residual + sum over the row's routes of w y) in rank order, fp32.
 __global__ __launch_bounds__(256) void moe_combine(const uint16_t *__restrict__ expert_output, const uint32_t *__restrict__ route_slot,
                                                    const float *__restrict__ weights, const uint16_t *__restrict__ residual,
-                                                   uint16_t *__restrict__ output, MoeCombineParams p) {
+                                                   uint16_t *__restrict__ output, const uint16_t *__restrict__ norm_weight,
+                                                   uint8_t *__restrict__ table, MoeCombineParams p) {
   const uint32_t row = blockIdx.x, d = blockIdx.y * 256u + threadIdx.x;
-  if (d >= p.hidden) return;
-  float value = bf16_bits_to_float(residual[size_t(row) * p.hidden + d]);
-  for (uint32_t rank = 0; rank < p.top_k; ++rank) {
-    const size_t route = size_t(row) * p.top_k + rank;
-    value += weights[route] * bf16_bits_to_float(expert_output[size_t(route_slot[route]) * p.hidden + d]);
+  const bool live = d < p.hidden;  // always, where a table is written
+  uint32_t bits = 0;
+  if (live) {
+    float value = bf16_bits_to_float(residual[size_t(row) * p.hidden + d]);
+    for (uint32_t rank = 0; rank < p.top_k; ++rank) {
+      const size_t route = size_t(row) * p.top_k + rank;
+      value += weights[route] * bf16_bits_to_float(expert_output[size_t(route_slot[route]) * p.hidden + d]);
+    }
+    bits = float_to_bf16_bits(value);
+    output[size_t(row) * p.hidden + d] = uint16_t(bits);
   }
-  output[size_t(row) * p.hidden + d] = uint16_t(float_to_bf16_bits(value));
+  if (!p.table_tiles) return;
+  // The row's piece of the table: lane l of a wave holds input 64 j + l of column group j. Runs of four
+  // inputs are one 8-byte piece of a table entry; lanes 4 i lead them.
+  const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6, r = row % 16u, G = p.hidden / 32u;
+  const uint32_t piece = row / 16u / GGUF_PIECE_TILES, tile = row / 16u % GGUF_PIECE_TILES;
+  const uint32_t tiles = min(uint32_t(GGUF_PIECE_TILES), p.table_tiles - piece * GGUF_PIECE_TILES);
+  table += piece * gguf_table_bytes(p.hidden, GGUF_PIECE_TILES);
+  const float hidden = bf16_bits_to_float(bits);
+  const uint32_t scaled = float_to_bf16_bits(hidden * bf16_bits_to_float(norm_weight[d]));
+  const float v = bf16_bits_to_float(scaled);
+  const uint32_t b1 = uint32_t(__shfl_down(int(scaled), 1, 64)), b2 = uint32_t(__shfl_down(int(scaled), 2, 64)),
+                 b3 = uint32_t(__shfl_down(int(scaled), 3, 64));
+  const float v1 = __shfl_down(v, 1, 64), v2 = __shfl_down(v, 2, 64), v3 = __shfl_down(v, 3, 64);
+  // sums of 16 inputs in input order: the four runs of a half are led by lanes 4 apart
+  float s = (v + v1) + (v2 + v3);
+  const float s1 = __shfl_down(s, 4, 64), s2 = __shfl_down(s, 8, 64), s3 = __shfl_down(s, 12, 64);
+  s = ((s + s1) + s2) + s3;
+  const float other = __shfl_down(s, 16, 64);
+  float square = hidden * hidden;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) square += __shfl_xor(square, o, 64);
+  const uint32_t q = d / 4u, g = q / 8u, half = (q / 4u) % 2u, kq = q % 4u;  // the run of input d
+  if ((lane & 3u) == 0) {
+    // operand elements 4 half + {0,1,2,3} are inputs 4 kq + {0,2,1,3} of the half
+    reinterpret_cast<uint2 *>(table)[((size_t(tile) * G + g) * 64u + kq * 16u + r) * 2u + half] =
+        make_uint2(scaled | (b2 << 16), b1 | (b3 << 16));
+    if (kq == 0) {
+      float *sums32 = reinterpret_cast<float *>(table + gguf_table_sums32_offset(p.hidden, tiles));
+      float *sums16 = reinterpret_cast<float *>(table + gguf_table_sums16_offset(p.hidden, tiles));
+      sums16[(size_t(tile) * 2u * G + 2u * g + half) * 16u + r] = s;
+      if (half == 0) sums32[(size_t(tile) * G + g) * 16u + r] = s + other;
+    }
+  }
+  if (lane == 0) {
+    float *squares = reinterpret_cast<float *>(table + gguf_table_squares_offset(p.hidden, tiles));
+    squares[size_t(blockIdx.y * 4u + wave) * 16u * tiles + 16u * tile + r] = square;
+  }
 }
 SP_REGISTER_KERNEL("moe_combine", &moe_combine);
 

@@ -143,7 +143,8 @@ void HybridVerify::encodeEmbedding(hip::CommandGraph &graph, uint32_t rows) {
   ops::Embedding::add(graph, weights_.embedding, inputTokens_, hidden_[0], rows);
 }
 
-void HybridVerify::encodeLayer(hip::CommandGraph &graph, uint32_t layer, const std::vector<HybridLane> &lanes) {
+void HybridVerify::encodeLayer(hip::CommandGraph &graph, uint32_t layer, const std::vector<HybridLane> &lanes, bool inputReady,
+                               bool feedsNext) {
   if (lanes.empty() || lanes.size() > maxLanes_) throw std::invalid_argument("the step takes 1 to its most lanes");
   const HybridLayer &w = weights_.layers.at(layer);
   const bool attends = dims_.attends(layer);
@@ -166,8 +167,10 @@ void HybridVerify::encodeLayer(hip::CommandGraph &graph, uint32_t layer, const s
     in.input = normalized;
     in.output = rowsOf(packed_, first, count, uint64_t{inputWidth} * 2);
     in.scratch = scratch_;
-    in.prepared = ops::Normalization::addRmsTable(graph, rowsOf(residual, first, count, hiddenBytes), w.inputNorm, normalized, scratch_,
-                                                  dims_.hidden, count);
+    // The layer before may have left the table of these rows, less their inverse RMS, from its combine.
+    in.prepared = inputReady ? ops::PreparedInput{normalized, ops::LinearInput::TableUnscaled}
+                             : ops::Normalization::addRmsTable(graph, rowsOf(residual, first, count, hiddenBytes), w.inputNorm, normalized,
+                                                               scratch_, dims_.hidden, count);
     linear_.add(graph, in, w.mixerInput, linear_.plan(w.mixerInput, count));
   });
   if (attends) {
@@ -205,10 +208,15 @@ void HybridVerify::encodeLayer(hip::CommandGraph &graph, uint32_t layer, const s
   });
   const ops::MoeShape moe = dims_.moeShape();
   ops::MoE::addRouting(graph, scores_, dims_.experts, moeWorkspace_, moe, rows);
-  ops::MoE::addRouted(graph, normalized_, next, residual, w.experts, moeWorkspace_, moe, rows);
+  ops::MoeFollowingNorm following;
+  if (feedsNext) {
+    following.weight = layer + 1 < dims_.layers ? weights_.layers[layer + 1].inputNorm : weights_.finalNorm;
+    following.table = scratch_.input;
+  }
+  ops::MoE::addRouted(graph, normalized_, next, residual, w.experts, moeWorkspace_, moe, rows, following);
 }
 
-void HybridVerify::encodeHead(hip::CommandGraph &graph, uint32_t rows) {
+void HybridVerify::encodeHead(hip::CommandGraph &graph, uint32_t rows, bool inputReady) {
   const uint64_t hiddenBytes = uint64_t{dims_.hidden} * 2;
   forRowPieces(rows, [&](uint32_t first, uint32_t count) {
     const hip::Buffer normalized = rowsOf(normalized_, first, count, hiddenBytes);
@@ -216,8 +224,9 @@ void HybridVerify::encodeHead(hip::CommandGraph &graph, uint32_t rows) {
     head.input = normalized;
     head.output = rowsOf(logits_, first, count, uint64_t{dims_.vocabulary} * 4);
     head.scratch = scratch_;
-    head.prepared = ops::Normalization::addRmsTable(graph, rowsOf(hidden_[0], first, count, hiddenBytes), weights_.finalNorm, normalized,
-                                                    scratch_, dims_.hidden, count);
+    head.prepared = inputReady ? ops::PreparedInput{normalized, ops::LinearInput::TableUnscaled}
+                               : ops::Normalization::addRmsTable(graph, rowsOf(hidden_[0], first, count, hiddenBytes), weights_.finalNorm,
+                                                                 normalized, scratch_, dims_.hidden, count);
     linear_.add(graph, head, weights_.head, linear_.plan(weights_.head, count));
   });
 }
@@ -242,8 +251,10 @@ void HybridVerify::encode(hip::CommandGraph &graph, const std::vector<HybridLane
   if (dims_.rotaryPairs)
     ops::RoPE::addTreeTables(graph, inverseFrequency_, depths_, ropeCos_, ropeSin_, dims_.rotaryPairs, rope);
   encodeEmbedding(graph, rows);
-  for (uint32_t layer = 0; layer < dims_.layers; ++layer) encodeLayer(graph, layer, lanes);
-  encodeHead(graph, rows);
+  // One piece of rows: a layer's combine can write the table the next layer's (or the head's) first projection reads.
+  const bool feeds = rows <= kProjectionRows && dims_.hidden % GGUF_BLOCK == 0;
+  for (uint32_t layer = 0; layer < dims_.layers; ++layer) encodeLayer(graph, layer, lanes, feeds && layer > 0, feeds);
+  encodeHead(graph, rows, feeds);
   ops::Sampling::addVerify(graph, sampling_, dims_.vocabulary, dims_.vocabulary, laneRows, policies);
   const ops::AcceptanceBuffers acceptance{inputTokens_, treeRows_, tokens_, retained_, acceptedCount_, retainedRows_};
   ops::Sampling::addAcceptance(graph, acceptance, laneRows, remaining,

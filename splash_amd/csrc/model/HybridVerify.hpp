@@ -124,8 +124,12 @@ public:
 
   void encode(hip::CommandGraph &graph, const std::vector<HybridLane> &lanes, bool commit = true);
   void encodeEmbedding(hip::CommandGraph &graph, uint32_t rows);
-  void encodeLayer(hip::CommandGraph &graph, uint32_t layer, const std::vector<HybridLane> &lanes);
-  void encodeHead(hip::CommandGraph &graph, uint32_t rows);
+  // A layer (or the head) whose predecessor in the same graph left the table of its input rows, less their inverse
+  // RMS, in the projection scratch passes `inputReady`; a layer that passes `feedsNext` leaves that table from its
+  // combine. A part encoded on its own passes neither.
+  void encodeLayer(hip::CommandGraph &graph, uint32_t layer, const std::vector<HybridLane> &lanes, bool inputReady = false,
+                   bool feedsNext = false);
+  void encodeHead(hip::CommandGraph &graph, uint32_t rows, bool inputReady = false);
 
 private:
   [[nodiscard]] ops::AttentionPlan planOf(const std::vector<HybridLane> &lanes) const;

@@ -57,8 +57,15 @@ void MoE::addRouting(hip::CommandGraph &graph, const hip::Buffer &scores, uint32
 }
 
 void MoE::addRouted(hip::CommandGraph &graph, const hip::Buffer &normalized, const hip::Buffer &residual, const hip::Buffer &output,
-                    const MoeExperts &experts, const MoeWorkspace &w, const MoeShape &shape, uint32_t rows) {
+                    const MoeExperts &experts, const MoeWorkspace &w, const MoeShape &shape, uint32_t rows,
+                    const MoeFollowingNorm &following) {
   requireShape(shape, rows);
+  const bool writesTable = bool(following.table);
+  if (writesTable) {
+    if (shape.hidden % GGUF_BLOCK) throw std::invalid_argument("a table epilogue takes whole super-blocks of columns");
+    requireBytes(following.weight, uint64_t{shape.hidden} * 2, "norm weight");
+    requireBytes(following.table, gguf_tables_bytes(shape.hidden, gguf_row_tiles(rows)), "next projection table");
+  }
   const MoeWorkspaceSize need = workspace(shape, rows);
   const uint32_t routes = rows * shape.topK, tiles = moe_maximum_tiles(routes, shape.experts);
   const std::string pairKernel = std::string("gguf_moe_decode_") + formatName(experts.format) + "_gt";
@@ -110,7 +117,10 @@ void MoE::addRouted(hip::CommandGraph &graph, const hip::Buffer &normalized, con
   down.out_row_bytes = shape.hidden * 2;
   graph.add(downKernel, {experts.down, experts.down, w.nextTables, w.expertOutput, w.nextTables, w.tileExpert, w.tileRows, w.tileTotal}, down,
             {(down.decode.units + 3) / 4, tiles, 1}, {256, 1, 1});
-  graph.add("moe_combine", {w.expertOutput, w.routeSlot, w.weights, residual, output}, MoeCombineParams{rows, shape.hidden, shape.topK, 0},
+  graph.add("moe_combine",
+            {w.expertOutput, w.routeSlot, w.weights, residual, output, writesTable ? following.weight : output,
+             writesTable ? following.table : output},
+            MoeCombineParams{rows, shape.hidden, shape.topK, writesTable ? gguf_row_tiles(rows) : 0u},
             {rows, (shape.hidden + 255) / 256, 1}, {256, 1, 1});
 }
 

@@ -37,6 +37,11 @@ struct MoeWorkspace final {
   hip::Buffer expertOutput;  // bf16 [slot][hidden]
 };
 
+struct MoeFollowingNorm final {
+  hip::Buffer weight;  // bf16 [hidden]
+  hip::Buffer table;   // gguf_tables_bytes(hidden, row tiles)
+};
+
 class MoE final {
 public:
   [[nodiscard]] static MoeWorkspaceSize workspace(const MoeShape &shape, uint32_t rows);
@@ -44,8 +49,12 @@ public:
   static void addRouting(hip::CommandGraph &graph, const hip::Buffer &scores, uint32_t scoreStride, const MoeWorkspace &workspace,
                          const MoeShape &shape, uint32_t rows);
   // output = bf16(residual + sum over a row's routes of weight * down(silu(gate x) * up x)) of its experts, x = normalized.
+  // `following` (optional): the output rows also leave as the activation table of the projection after their RMS
+  // norm under following.weight, as a LinearEpilogue::ResidualNorm plan writes it (that projection reads it as
+  // LinearInput::TableUnscaled).
   static void addRouted(hip::CommandGraph &graph, const hip::Buffer &normalized, const hip::Buffer &residual, const hip::Buffer &output,
-                        const MoeExperts &experts, const MoeWorkspace &workspace, const MoeShape &shape, uint32_t rows);
+                        const MoeExperts &experts, const MoeWorkspace &workspace, const MoeShape &shape, uint32_t rows,
+                        const MoeFollowingNorm &following = {});
 };
 
 } // namespace splash::ops

@@ -368,11 +368,18 @@ class MoE:
         graph._keep.extend([scores, self])
 
     def add_routed(self, graph, normalized, residual, output, gate_images, up_images, down_images, rows=None, fmt=FMT_Q4K,
-                   down_fmt=FMT_Q4K):
-        check(lib.spo_moe_add_routed(graph.handle, normalized.handle, residual.handle, output.handle, gate_images.handle, up_images.handle,
-                                     down_images.handle, fmt, down_fmt, ctypes.byref(self.workspace), ctypes.byref(self.shape),
-                                     rows or self.rows))
-        graph._keep.extend([normalized, residual, output, gate_images, up_images, down_images, self])
+                   down_fmt=FMT_Q4K, norm_weight=None, next_table=None):
+        """norm_weight, next_table: the output rows also leave as the table of the projection after their RMS norm (that
+        projection passes prepared=PREPARED_UNSCALED)."""
+        if next_table is not None:
+            check(lib.spo_moe_add_routed_norm(graph.handle, normalized.handle, residual.handle, output.handle, gate_images.handle,
+                                              up_images.handle, down_images.handle, fmt, down_fmt, ctypes.byref(self.workspace),
+                                              ctypes.byref(self.shape), rows or self.rows, norm_weight.handle, next_table.handle))
+        else:
+            check(lib.spo_moe_add_routed(graph.handle, normalized.handle, residual.handle, output.handle, gate_images.handle, up_images.handle,
+                                         down_images.handle, fmt, down_fmt, ctypes.byref(self.workspace), ctypes.byref(self.shape),
+                                         rows or self.rows))
+        graph._keep.extend([normalized, residual, output, gate_images, up_images, down_images, self, norm_weight, next_table])
 
 
 NO_TOKEN = 0xFFFFFFFF

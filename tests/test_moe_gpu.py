@@ -9,7 +9,7 @@ from tests import oracle as orc
 pytestmark = pytest.mark.gpu
 
 
-def run_layer(backend, rng, hidden, ffn, experts, top_k, rows, down_fmt=ops.FMT_Q4K):
+def run_layer(backend, rng, hidden, ffn, experts, top_k, rows, down_fmt=ops.FMT_Q4K, following=None):
     gate = [orc.make_native(ops.FMT_Q4K, ffn, hidden, 100 + e) for e in range(experts)]
     up = [orc.make_native(ops.FMT_Q4K, ffn, hidden, 300 + e) for e in range(experts)]
     down = [orc.make_native(down_fmt, hidden, ffn, 500 + e) for e in range(experts)]
@@ -23,7 +23,8 @@ def run_layer(backend, rng, hidden, ffn, experts, top_k, rows, down_fmt=ops.FMT_
     out = backend.allocate_buffer(rows * hidden * 2)
     graph = splash_amd.CommandGraph()
     moe.add_routing(graph, backend.from_array(scores))
-    moe.add_routed(graph, backend.from_array(x), backend.from_array(res), out, *images, down_fmt=down_fmt)
+    extra = dict(norm_weight=following[0], next_table=following[1]) if following else {}
+    moe.add_routed(graph, backend.from_array(x), backend.from_array(res), out, *images, down_fmt=down_fmt, **extra)
     assert len(graph) == 6
     backend.run(graph)
     got = out.download(np.uint16).reshape(rows, hidden)
@@ -81,6 +82,42 @@ def test_moe_layer_at_the_35b_shape(backend):
     rng = np.random.default_rng(9)
     moe, got, want = run_layer(backend, rng, 2048, 768, 128, 8, 128)
     check_layer(moe, got, want, 128, 128, 8)
+
+
+@pytest.mark.parametrize("rows", [20, 100])
+def test_combine_writes_the_next_norms_table(backend, rows):
+    """The combine may also leave its rows as the activation table of the projection after their RMS norm, as a
+    residual projection's norm epilogue does: the rows are unchanged, the table is bit for bit that of
+    bf16(row * weight) in pieces of 64 rows, with each 64-column group's sums of squares of the rows."""
+    print(f"case moe combine table rows={rows}", flush=True)
+    hidden, ffn, experts, top_k = 512, 256, 8, 2
+    rng = np.random.default_rng(rows)
+    _, plain, _ = run_layer(backend, np.random.default_rng(rows), hidden, ffn, experts, top_k, rows)
+    weight_bits = orc.f32_to_bf16((1 + 0.1 * rng.standard_normal(hidden)).astype(np.float32))
+    table_bytes = ops.gguf_table_bytes(hidden, rows)
+    table = backend.allocate_buffer(table_bytes)
+    _, got, _ = run_layer(backend, np.random.default_rng(rows), hidden, ffn, experts, top_k, rows,
+                          following=(backend.from_array(weight_bits), table))
+    assert np.array_equal(got, plain)
+    raw = table.download(np.uint8)[:table_bytes]
+    scaled = orc.f32_to_bf16(orc.bf16_to_f32(got) * orc.bf16_to_f32(weight_bits)[None, :])
+    at = 0
+    for first in range(0, rows, 64):
+        count = min(64, rows - first)
+        tiles = (count + 15) // 16
+        size = ops.gguf_table_bytes(hidden, count)
+        piece = raw[at:at + size]
+        at += size
+        values, s32, s16 = orc.split_activation_table(piece, hidden, tiles)
+        wv, w32, w16 = orc.activation_table(scaled[first:first + count])
+        live = orc.table_rows(values, hidden, tiles)[:count]
+        assert np.array_equal(live, orc.table_rows(wv, hidden, tiles)[:count])
+        rows_of = lambda sums: sums.transpose(0, 2, 1).reshape(tiles * 16, -1)[:count]     # [tile][entry][16 rows] -> [row][entry]
+        assert np.array_equal(rows_of(s32), rows_of(w32)) and np.array_equal(rows_of(s16), rows_of(w16))
+        squares = piece[size - (hidden // 64) * 16 * tiles * 4:].view(np.float32).reshape(hidden // 64, 16 * tiles)
+        h = orc.bf16_to_f32(got[first:first + count]).astype(np.float64)
+        assert np.allclose(squares[:, :count], (h.reshape(count, hidden // 64, 64) ** 2).sum(axis=2).T, rtol=1e-5, atol=0)
+    assert at == table_bytes
 
 
 def test_moe_rejects_bad_arguments(backend):
