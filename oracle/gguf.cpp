@@ -8,10 +8,14 @@ using namespace orc;
 
 namespace {
 
-constexpr uint32_t kQ4KBytes = 144, kQ6KBytes = 210, kBlock = 256;
+constexpr uint32_t kQ4KBytes = 144, kQ5KBytes = 176, kQ6KBytes = 210, kQ80Bytes = 34, kBlock = 256;
 constexpr uint32_t kQ6KScales = 128 + 64, kQ6KD = kQ6KScales + 16;  // GgufFormatReference.hpp:61
 
-uint32_t blockBytes(uint32_t fmt) { return fmt == ORC_FMT_Q4K ? kQ4KBytes : fmt == ORC_FMT_Q6K ? kQ6KBytes : 0; }
+// Bytes and elements of a native block: the K-quants' super-block of 256, Q8_0's group of 32.
+uint32_t blockBytes(uint32_t fmt) {
+  return fmt == ORC_FMT_Q4K ? kQ4KBytes : fmt == ORC_FMT_Q5K ? kQ5KBytes : fmt == ORC_FMT_Q6K ? kQ6KBytes : fmt == ORC_FMT_Q80 ? kQ80Bytes : 0;
+}
+uint32_t blockElements(uint32_t fmt) { return fmt == ORC_FMT_Q80 ? 32 : kBlock; }
 
 // GgufFormatReference.hpp:326-329
 void scaleMinK4(const uint8_t *sc, int j, uint8_t &s, uint8_t &m) {
@@ -23,14 +27,32 @@ void scaleMinK4(const uint8_t *sc, int j, uint8_t &s, uint8_t &m) {
 // (quant_formats.h:105-137); Q6_K has a scale per 16 and code - 32 (quant_formats.h:153-168).
 struct Group {
   uint8_t code[32];
-  float s[2];  // Q4_K: s[0] = s[1] = d * sc; Q6_K: one per 16 elements
-  float m;     // Q4_K: -dmin * mn; Q6_K: 0
-  int bias;    // Q4_K: 0; Q6_K: 32
+  float s[2];  // Q4_K, Q5_K: s[0] = s[1] = d * sc; Q6_K: one per 16 elements; Q8_0: d
+  float m;     // Q4_K, Q5_K: -dmin * mn; Q6_K, Q8_0: 0
+  int bias;    // Q4_K, Q5_K: 0; Q6_K: 32; Q8_0: 128 (code = value + 128)
 };
 void readGroup(uint32_t fmt, const uint8_t *row, uint32_t g, Group &out) {
+  if (fmt == ORC_FMT_Q80) {   // GgufFormatReference.hpp:453-458: value = d * int8
+    const uint8_t *blk = row + size_t(g) * kQ80Bytes;
+    uint16_t d16; std::memcpy(&d16, blk, 2);
+    for (int k = 0; k < 32; ++k) out.code[k] = uint8_t(int(int8_t(blk[2 + k])) + 128);
+    out.s[0] = out.s[1] = h2f(d16);
+    out.m = 0.f;
+    out.bias = 128;
+    return;
+  }
   const uint8_t *blk = row + size_t(g / 8) * blockBytes(fmt);
   const uint32_t j = g % 8;
-  if (fmt == ORC_FMT_Q4K) {
+  if (fmt == ORC_FMT_Q5K) {   // GgufFormatReference.hpp:405-416: the fifth bits in qh, bit j of byte k
+    uint16_t d16, m16; std::memcpy(&d16, blk, 2); std::memcpy(&m16, blk + 2, 2);
+    uint8_t sc, mn; scaleMinK4(blk + 4, int(j), sc, mn);
+    const uint8_t *qh = blk + 16, *q = blk + 48 + (j / 2) * 32;
+    const int sh = int(j % 2) * 4;
+    for (int k = 0; k < 32; ++k) out.code[k] = uint8_t(((q[k] >> sh) & 15) | (((qh[k] >> j) & 1) << 4));
+    out.s[0] = out.s[1] = h2f(d16) * float(sc);  // exact: 11 + 6 bits
+    out.m = -(h2f(m16) * float(mn));             // exact
+    out.bias = 0;
+  } else if (fmt == ORC_FMT_Q4K) {
     uint16_t d16, m16; std::memcpy(&d16, blk, 2); std::memcpy(&m16, blk + 2, 2);
     uint8_t sc, mn; scaleMinK4(blk + 4, int(j), sc, mn);
     const uint8_t *q = blk + 16 + (j / 2) * 32;
@@ -55,13 +77,13 @@ void readGroup(uint32_t fmt, const uint8_t *row, uint32_t g, Group &out) {
   }
 }
 
-// llama.cpp semantics (GgufFormatReference.hpp:370-381, :418-432): Q4_K d*sc*code - dmin*mn with one
-// rounding (both products exact); Q6_K d*sc*(q-32), exact.
+// llama.cpp semantics (GgufFormatReference.hpp:370-381, :405-432, :453-458): Q4_K and Q5_K d*sc*code - dmin*mn
+// with one rounding (both products exact); Q6_K d*sc*(q-32) and Q8_0 d*q, exact.
 void groupValues(uint32_t fmt, const uint8_t *row, uint32_t g, float *vals) {
   Group grp; readGroup(fmt, row, g, grp);
   for (int k = 0; k < 32; ++k) {
     const float s = grp.s[k / 16];
-    if (fmt == ORC_FMT_Q4K) vals[k] = s * float(grp.code[k]) + grp.m;   // s*code exact (<= 21 bits)
+    if (fmt == ORC_FMT_Q4K || fmt == ORC_FMT_Q5K) vals[k] = s * float(grp.code[k]) + grp.m;   // s*code exact (<= 22 bits)
     else vals[k] = s * float(int(grp.code[k]) - grp.bias);
   }
 }
@@ -204,7 +226,7 @@ void makeNativeWith(uint32_t fmt, uint32_t rows, uint32_t K, std::mt19937 &rng, 
     uint8_t *blk = native + b * bb;
     const uint16_t d = scale();
     std::memcpy(blk + off, &d, 2);
-    if (fmt == ORC_FMT_Q4K) { const uint16_t m = scale(); std::memcpy(blk + off + 2, &m, 2); }
+    if (fmt == ORC_FMT_Q4K || fmt == ORC_FMT_Q5K) { const uint16_t m = scale(); std::memcpy(blk + off + 2, &m, 2); }
   }
 }
 
@@ -219,7 +241,7 @@ float orc_bf2f(uint16_t b) { return bf2f(b); }
 
 uint64_t orc_row_bytes(uint32_t fmt, uint32_t K) {
   const uint32_t bb = blockBytes(fmt);
-  return bb && K % kBlock == 0 ? uint64_t(K / kBlock) * bb : 0;
+  return bb && K % kBlock == 0 ? uint64_t(K / blockElements(fmt)) * bb : 0;
 }
 
 int orc_fixture(uint32_t fmt, uint32_t rows, uint32_t K, uint32_t seed, uint8_t *native) {
@@ -237,8 +259,8 @@ int orc_make_native(uint32_t fmt, uint32_t rows, uint32_t K, uint32_t seed, uint
   if (!orc_row_bytes(fmt, K)) return -1;
   std::mt19937 rng(seed);
   // GgufFormatReference.hpp:295-323 scaleRange
-  std::uniform_real_distribution<float> range = fmt == ORC_FMT_Q4K
-      ? std::uniform_real_distribution<float>(0.0005f, 0.004f) : std::uniform_real_distribution<float>(0.00002f, 0.0001f);
+  std::uniform_real_distribution<float> range = fmt == ORC_FMT_Q6K
+      ? std::uniform_real_distribution<float>(0.00002f, 0.0001f) : std::uniform_real_distribution<float>(0.0005f, 0.004f);
   makeNativeWith(fmt, rows, K, rng, native, [&] { return f2h(range(rng)); });
   return 0;
 }
@@ -255,7 +277,7 @@ int orc_dequant_rows(uint32_t fmt, const uint8_t *native, uint32_t rows, uint32_
 
 int orc_quantize_rows(uint32_t fmt, const float *values, uint32_t rows, uint32_t K, uint8_t *native) {
   const uint64_t rb = orc_row_bytes(fmt, K);
-  if (!rb) return -1;
+  if (!rb || (fmt != ORC_FMT_Q4K && fmt != ORC_FMT_Q6K)) return -1;
   parallelFor(rows, 0, [&](uint32_t lo, uint32_t hi) {
     for (uint32_t r = lo; r < hi; ++r)
       for (uint32_t b = 0; b < K / kBlock; ++b) {
@@ -309,11 +331,16 @@ int orc_gemm(uint32_t fmt, const uint8_t *native, const uint16_t *x, uint32_t M,
           for (uint32_t g = 0; g < K / 32; ++g) {
             readGroup(fmt, row, g, grp);
             const float *s16 = sums16.data() + size_t(m) * (K / 16) + 2 * g;
-            if (fmt == ORC_FMT_Q4K) {
+            if (fmt == ORC_FMT_Q4K || fmt == ORC_FMT_Q5K) {
               float dot = 0;
               for (int k = 0; k < 32; ++k) dot = std::fma(xr[32 * g + k], float(128 + grp.code[k]), dot);
               acc = std::fma(dot, grp.s[0], acc);
               acc = std::fma(s16[0] + s16[1], grp.m - 128.f * grp.s[0], acc);
+            } else if (fmt == ORC_FMT_Q80) {
+              // the operand is the int8 value itself (linear_gguf_sgmatrix.metal:96-98), one scale a group, no min
+              float dot = 0;
+              for (int k = 0; k < 32; ++k) dot = std::fma(xr[32 * g + k], float(int(grp.code[k]) - 128), dot);
+              acc = std::fma(dot, grp.s[0], acc);
             } else {
               for (int h = 0; h < 2; ++h) {
                 float dot = -160.f * s16[h];

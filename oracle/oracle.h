@@ -35,7 +35,7 @@ extern "C" {
 #endif
 
 // Format ids follow the reference's GGUF_FMT_* numbering (runtime/metal/abi/QuantFormat.h:138-154).
-enum { ORC_FMT_Q4K = 0, ORC_FMT_Q6K = 4 };
+enum { ORC_FMT_Q4K = 0, ORC_FMT_Q5K = 3, ORC_FMT_Q6K = 4, ORC_FMT_Q80 = 6 };
 
 // ---- half / bfloat16 scalar conversions (round to nearest even) ----
 uint16_t orc_f2h(float f);

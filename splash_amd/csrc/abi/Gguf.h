@@ -26,6 +26,19 @@
 //     [3072, 3328)  scales: column c's 16 int8 scales at 3072 + 16 c.
 //     [3328, 3360)  d: column c's fp16 d at 3328 + 2 c.
 //
+//   Q5_K record, 2816 B (16 native blocks of 176 B):
+//     [   0, 2048)  low nibbles, arranged exactly as Q4_K's nibbles.
+//     [2048, 2560)  fifth bits: lane l owns 8 B at 2048 + 8 l: word h covers groups 4 h .. 4 h + 3; bit
+//                   4 (g % 4) + j is the fifth bit of the low half's code of operand register j of group g,
+//                   bit 16 + 4 (g % 4) + j that of its high half's.
+//     [2560, 2816)  meta: column c's native d, dmin and 12 scale bytes at 2560 + 16 c (as Q4_K's).
+//
+//   Q8_0 record, 4352 B (16 columns of eight native 34-B blocks):
+//     [   0, 4096)  values: four 1024-B parts; in part i lane l owns 16 B at 1024 i + 16 l: the int8 values of
+//                   inputs 4 kq .. 4 kq + 3 and 16 + 4 kq .. + 3 of group 2 i, then those of group 2 i + 1.
+//     [4096, 4352)  scales: column c's eight fp16 d (groups 0..7) at 4096 + 16 c.
+//   Its operands are the bf16 128 + value (0..255, exact); the 128 leaves as Q4_K's does, through the row sums.
+//
 // Within a group, lane (c, kq) holds eight codes as four registers of two bf16 operands
 // 128 + code: register j (0..3) holds inputs 16 (j / 2) + 4 kq + (j % 2) [low half] and that + 2
 // [high half]. Element e = 2 j + half of the lane's MFMA operand is therefore input
@@ -43,15 +56,24 @@
 #include <stdint.h>
 
 #define GGUF_FMT_Q4K 0u
+#define GGUF_FMT_Q5K 3u
 #define GGUF_FMT_Q6K 4u
+#define GGUF_FMT_Q80 6u
 #define GGUF_FMT_COUNT 26u
 
 #define GGUF_BLOCK 256u
 #define GGUF_TILE_COLUMNS 16u
 #define GGUF_Q4K_NATIVE 144u
+#define GGUF_Q5K_NATIVE 176u
 #define GGUF_Q6K_NATIVE 210u
+#define GGUF_Q80_NATIVE 272u  // eight 34-byte blocks: the bytes of 256 inputs
 #define GGUF_Q4K_RECORD (GGUF_TILE_COLUMNS * GGUF_Q4K_NATIVE)  // 2304
 #define GGUF_Q6K_RECORD (GGUF_TILE_COLUMNS * GGUF_Q6K_NATIVE)  // 3360
+#define GGUF_Q5K_RECORD (GGUF_TILE_COLUMNS * GGUF_Q5K_NATIVE)  // 2816
+#define GGUF_Q80_RECORD (GGUF_TILE_COLUMNS * GGUF_Q80_NATIVE)  // 4352
+#define GGUF_Q5K_HIGH 2048u
+#define GGUF_Q5K_META 2560u
+#define GGUF_Q80_SCALES 4096u
 #define GGUF_Q6K_HIGH 2048u
 #define GGUF_Q6K_SCALES 3072u
 #define GGUF_Q6K_D 3328u
@@ -65,17 +87,29 @@
 #define GGUF_MAXIMUM_SPLITS 16u
 
 #if defined(__HIPCC__) || defined(__cplusplus)
-#define GGUF_INLINE inline
+#define GGUF_INLINE constexpr inline
 #if defined(__HIPCC__)
 #undef GGUF_INLINE
-#define GGUF_INLINE __host__ __device__ inline
+#define GGUF_INLINE __host__ __device__ constexpr inline
 #endif
 
 GGUF_INLINE uint32_t gguf_record_bytes(uint32_t format) {
-  return format == GGUF_FMT_Q4K ? GGUF_Q4K_RECORD : format == GGUF_FMT_Q6K ? GGUF_Q6K_RECORD : 0u;
+  return format == GGUF_FMT_Q4K   ? GGUF_Q4K_RECORD
+         : format == GGUF_FMT_Q6K ? GGUF_Q6K_RECORD
+         : format == GGUF_FMT_Q5K ? GGUF_Q5K_RECORD
+         : format == GGUF_FMT_Q80 ? GGUF_Q80_RECORD
+                                  : 0u;
 }
 GGUF_INLINE uint32_t gguf_native_bytes(uint32_t format) {
-  return format == GGUF_FMT_Q4K ? GGUF_Q4K_NATIVE : format == GGUF_FMT_Q6K ? GGUF_Q6K_NATIVE : 0u;
+  return format == GGUF_FMT_Q4K   ? GGUF_Q4K_NATIVE
+         : format == GGUF_FMT_Q6K ? GGUF_Q6K_NATIVE
+         : format == GGUF_FMT_Q5K ? GGUF_Q5K_NATIVE
+         : format == GGUF_FMT_Q80 ? GGUF_Q80_NATIVE
+                                  : 0u;
+}
+// Kernel-name tag of a format.
+GGUF_INLINE const char *gguf_format_name(uint32_t format) {
+  return format == GGUF_FMT_Q4K ? "q4k" : format == GGUF_FMT_Q6K ? "q6k" : format == GGUF_FMT_Q5K ? "q5k" : format == GGUF_FMT_Q80 ? "q80" : "";
 }
 // Bytes of the image of an [N, K] tensor (N a multiple of 16, K of 256): those of its native rows.
 GGUF_INLINE uint64_t gguf_image_bytes(uint32_t format, uint32_t n, uint32_t k) {

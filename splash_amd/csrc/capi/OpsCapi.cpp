@@ -100,7 +100,7 @@ sp_status spo_gguf_add_dequant(spo_graph *graph, uint32_t format, sp_buffer *ima
       throw std::invalid_argument("a weight image holds whole tiles of a K-quant format");
     ops::requireBytes(hip::Buffer::share(image), gguf_image_bytes(format, rows, input_size), "weight image");
     ops::requireBytes(hip::Buffer::share(out), uint64_t{rows} * input_size * 4, "dequantized values");
-    graph->graph.add(format == GGUF_FMT_Q4K ? "gguf_dequant_q4k" : "gguf_dequant_q6k",
+    graph->graph.add(std::string("gguf_dequant_") + gguf_format_name(format),
                      {hip::Buffer::share(image), hip::Buffer::share(out)}, GgufDequantParams{input_size, rows},
                      {input_size / 256, rows / 16, 1}, {64, 1, 1});
   });

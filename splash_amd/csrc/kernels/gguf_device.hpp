@@ -1,4 +1,4 @@
-// Device-side decode of the Q4_K / Q6_K weight image (abi/Gguf.h): every kernel that reads the
+// Device-side decode of the K-quant and Q8_0 weight images (abi/Gguf.h): every kernel that reads the
 // image -- the projection tiles, the value dump of the bit-exactness test -- unpacks it through
 // these functions, so the test of one covers the others.
 #pragma once
@@ -56,6 +56,36 @@ template <bool High, uint32_t V0> __device__ __forceinline__ uint4 q6_operands(u
   r.y = with(V0 + 1, r.y);
   r.z = with(V0 + 2, r.z);
   r.w = with(V0 + 3, r.w);
+  return r;
+}
+
+// The same for Q5_K: the low nibbles as Q4_K's, then the fifth bits of registers R0 .. R0 + 3 of the record
+// half's fifth-bits word (abi/Gguf.h: bit r the low half's, bit 16 + r the high half's) at bit 4 of each half.
+template <bool High, uint32_t R0> __device__ __forceinline__ uint4 q5_operands(uint32_t wa, uint32_t wb, uint32_t hw) {
+  constexpr uint32_t kFifth = 0x00100010u;
+  uint4 r = q4_operands<High>(wa, wb);
+  auto with = [&](uint32_t reg, uint32_t low) -> uint32_t {
+    return and_or(reg > 4u ? hw >> (reg - 4u) : reg < 4u ? hw << (4u - reg) : hw, kFifth, low);
+  };
+  r.x = with(R0, r.x);
+  r.y = with(R0 + 1, r.y);
+  r.z = with(R0 + 2, r.z);
+  r.w = with(R0 + 3, r.w);
+  return r;
+}
+// Q8_0: the bf16 operands 128 + value of a group from the words of its inputs 4 kq .. 4 kq + 3 (wa) and
+// 16 + 4 kq .. + 3 (wb). value + 128 is the byte with its sign bit flipped; an integer up to 255 is exact in
+// fp32 and in bf16, whose bits are the fp32's upper half.
+__device__ __forceinline__ uint4 q8_operands(uint32_t wa, uint32_t wb) {
+  auto pair = [](uint32_t first, uint32_t second) -> uint32_t {  // bf16(first) in the low half, bf16(second) in the high
+    return __builtin_amdgcn_perm(__builtin_bit_cast(uint32_t, float(second)), __builtin_bit_cast(uint32_t, float(first)), 0x07060302u);
+  };
+  const uint32_t a = wa ^ 0x80808080u, b = wb ^ 0x80808080u;
+  uint4 r;
+  r.x = pair(a & 0xFFu, (a >> 16) & 0xFFu);
+  r.y = pair((a >> 8) & 0xFFu, a >> 24);
+  r.z = pair(b & 0xFFu, (b >> 16) & 0xFFu);
+  r.w = pair((b >> 8) & 0xFFu, b >> 24);
   return r;
 }
 

@@ -81,22 +81,25 @@ SP_REGISTER_KERNEL("gguf_prepare_table", &gguf_prepare_table);
 template <uint32_t FMT> struct Cursor {
   const uint4 *mine = nullptr;
   const uint4 *column = nullptr;
-  const uint16_t *d = nullptr;  // Q6_K only
+  const uint16_t *d = nullptr;   // Q6_K only
+  const uint2 *fifth = nullptr;  // Q5_K only
+  static constexpr uint32_t kColumnPart = FMT == GGUF_FMT_Q4K   ? 2048u
+                                          : FMT == GGUF_FMT_Q6K ? GGUF_Q6K_SCALES
+                                          : FMT == GGUF_FMT_Q5K ? GGUF_Q5K_META
+                                                                : GGUF_Q80_SCALES;
   __device__ __forceinline__ void open(const uint8_t *record, uint32_t lane) {
     const uint4 *p = reinterpret_cast<const uint4 *>(record);
     mine = p + lane;
-    if constexpr (FMT == GGUF_FMT_Q4K) {
-      column = p + 128 + (lane & 15u);
-    } else {
-      column = p + 192 + (lane & 15u);
-      d = reinterpret_cast<const uint16_t *>(record + GGUF_Q6K_D) + (lane & 15u);
-    }
+    column = p + kColumnPart / 16u + (lane & 15u);
+    if constexpr (FMT == GGUF_FMT_Q6K) d = reinterpret_cast<const uint16_t *>(record + GGUF_Q6K_D) + (lane & 15u);
+    if constexpr (FMT == GGUF_FMT_Q5K) fifth = reinterpret_cast<const uint2 *>(record + GGUF_Q5K_HIGH) + lane;
   }
   __device__ __forceinline__ void advance() {
-    constexpr uint32_t kVectors = (FMT == GGUF_FMT_Q4K ? GGUF_Q4K_RECORD : GGUF_Q6K_RECORD) / 16u;
+    constexpr uint32_t kVectors = gguf_record_bytes(FMT) / 16u;
     mine += kVectors;
     column += kVectors;
     if constexpr (FMT == GGUF_FMT_Q6K) d += kVectors * 8u;
+    if constexpr (FMT == GGUF_FMT_Q5K) fifth += kVectors * 2u;
   }
 };
 
@@ -121,7 +124,48 @@ template <> struct Record<GGUF_FMT_Q6K> {
   }
 };
 
+template <> struct Record<GGUF_FMT_Q5K> {
+  uint4 n0, n1, meta;
+  uint2 fifth;
+  __device__ __forceinline__ void load(const Cursor<GGUF_FMT_Q5K> &at) {
+    n0 = load_stream(at.mine);
+    n1 = load_stream(at.mine + 64);
+    meta = load_stream(at.column);
+    fifth = *at.fifth;
+  }
+};
+template <> struct Record<GGUF_FMT_Q80> {
+  uint4 v[4], scales;
+  __device__ __forceinline__ void load(const Cursor<GGUF_FMT_Q80> &at) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = load_stream(at.mine + 64 * i);
+    scales = load_stream(at.column);
+  }
+};
+
 // The eight groups' operand registers of a record, group g's in ops[g].
+__device__ __forceinline__ void record_operands(const Record<GGUF_FMT_Q5K> &r, uint4 ops[8]) {
+  ops[0] = q5_operands<false, 0>(r.n0.x, r.n0.y, r.fifth.x);
+  ops[1] = q5_operands<true, 4>(r.n0.x, r.n0.y, r.fifth.x);
+  ops[2] = q5_operands<false, 8>(r.n0.z, r.n0.w, r.fifth.x);
+  ops[3] = q5_operands<true, 12>(r.n0.z, r.n0.w, r.fifth.x);
+  ops[4] = q5_operands<false, 0>(r.n1.x, r.n1.y, r.fifth.y);
+  ops[5] = q5_operands<true, 4>(r.n1.x, r.n1.y, r.fifth.y);
+  ops[6] = q5_operands<false, 8>(r.n1.z, r.n1.w, r.fifth.y);
+  ops[7] = q5_operands<true, 12>(r.n1.z, r.n1.w, r.fifth.y);
+}
+__device__ __forceinline__ void record_operands(const Record<GGUF_FMT_Q80> &r, uint4 ops[8]) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    ops[2 * i] = q8_operands(r.v[i].x, r.v[i].y);
+    ops[2 * i + 1] = q8_operands(r.v[i].z, r.v[i].w);
+  }
+}
+// Group g's fp16 scale of a Q8_0 record's column.
+__device__ __forceinline__ float q8_scale(const uint4 &scales, uint32_t g) {
+  const uint32_t word = g < 2 ? scales.x : g < 4 ? scales.y : g < 6 ? scales.z : scales.w;
+  return half_bits_to_float((word >> (16u * (g & 1u))) & 0xFFFFu);
+}
 __device__ __forceinline__ void record_operands(const Record<GGUF_FMT_Q4K> &r, uint4 ops[8]) {
   ops[0] = q4_operands<false>(r.n0.x, r.n0.y);
   ops[1] = q4_operands<true>(r.n0.x, r.n0.y);
@@ -162,7 +206,16 @@ template <uint32_t FMT> __global__ __launch_bounds__(64) void gguf_dequant(const
   uint4 ops[8];
   record_operands(rec, ops);
   float *row = out + size_t(16u * tile + c) * p.input_size + size_t(b) * GGUF_BLOCK;
-  if constexpr (FMT == GGUF_FMT_Q4K) {
+  if constexpr (FMT == GGUF_FMT_Q80) {
+#pragma unroll
+    for (uint32_t g = 0; g < 8; ++g) {
+      const float d = q8_scale(rec.scales, g);
+      const uint32_t regs[4] = {ops[g].x, ops[g].y, ops[g].z, ops[g].w};
+#pragma unroll
+      for (uint32_t e = 0; e < 8; ++e)
+        row[32u * g + gguf_operand_input(kq, e)] = d * (bf16_bits_to_float((regs[e >> 1] >> (16u * (e & 1u))) & 0xFFFFu) - 128.f);  // exact
+    }
+  } else if constexpr (FMT == GGUF_FMT_Q4K || FMT == GGUF_FMT_Q5K) {
     const Q4KScales sc = q4k_scales(rec.meta);
 #pragma unroll
     for (uint32_t g = 0; g < 8; ++g) {
@@ -171,7 +224,7 @@ template <uint32_t FMT> __global__ __launch_bounds__(64) void gguf_dequant(const
       const uint32_t regs[4] = {ops[g].x, ops[g].y, ops[g].z, ops[g].w};
 #pragma unroll
       for (uint32_t e = 0; e < 8; ++e) {
-        const float code = float(operand_code(regs[e >> 1], e & 1u) & 0xFu);
+        const float code = float(operand_code(regs[e >> 1], e & 1u) & (FMT == GGUF_FMT_Q5K ? 0x1Fu : 0xFu));
         // d*sc*code is exact in fp32, so this is the one rounding of d*sc*code - dmin*mn.
         row[32u * g + gguf_operand_input(kq, e)] = __fmaf_rn(s, code, m);
       }
@@ -192,6 +245,8 @@ template <uint32_t FMT> __global__ __launch_bounds__(64) void gguf_dequant(const
 }
 SP_REGISTER_KERNEL("gguf_dequant_q4k", &gguf_dequant<GGUF_FMT_Q4K>);
 SP_REGISTER_KERNEL("gguf_dequant_q6k", &gguf_dequant<GGUF_FMT_Q6K>);
+SP_REGISTER_KERNEL("gguf_dequant_q5k", &gguf_dequant<GGUF_FMT_Q5K>);
+SP_REGISTER_KERNEL("gguf_dequant_q80", &gguf_dequant<GGUF_FMT_Q80>);
 
 // ---------------------------------------------------------------------------------------------
 // The decode projection.
@@ -200,6 +255,7 @@ SP_REGISTER_KERNEL("gguf_dequant_q6k", &gguf_dequant<GGUF_FMT_Q6K>);
 // moves no memory, so the software pipeline below needs no branch around a load and no
 // special case at the end of a range, and its address arithmetic is one 32-bit add per stream.
 using Resource = __amdgpu_buffer_rsrc_t;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
 __device__ __forceinline__ Resource make_resource(const void *base, uint32_t bytes) {
   // The base must be wave-uniform (it lives in scalar registers).
   const uint64_t v = reinterpret_cast<uint64_t>(base);
@@ -229,6 +285,21 @@ __device__ __forceinline__ void load_record(Record<GGUF_FMT_Q6K> &rec, Resource 
   // The lane's 16 l and the column's 16 c locate the record and c: d sits at record + 3328 + 2 c.
   const uint32_t lane = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
   rec.d = __builtin_amdgcn_raw_buffer_load_b16(r, int(mine - 16u * lane + GGUF_Q6K_D + 2u * (lane & 15u)), 0, kStreamOnce);
+}
+
+__device__ __forceinline__ void load_record(Record<GGUF_FMT_Q5K> &rec, Resource r, uint32_t mine, uint32_t column) {
+  rec.n0 = load128<kStreamOnce>(r, mine);
+  rec.n1 = load128<kStreamOnce>(r, mine + 1024u);
+  rec.meta = load128<kStreamOnce>(r, column);
+  // The lane's 8 bytes of fifth bits sit at record + 2048 + 8 l; `mine` is record + 16 l.
+  const uint32_t lane = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+  const u32x2 fifth = __builtin_amdgcn_raw_buffer_load_b64(r, int(mine - 8u * lane + GGUF_Q5K_HIGH), 0, kStreamOnce);
+  rec.fifth = make_uint2(fifth.x, fifth.y);
+}
+__device__ __forceinline__ void load_record(Record<GGUF_FMT_Q80> &rec, Resource r, uint32_t mine, uint32_t column) {
+#pragma unroll
+  for (uint32_t i = 0; i < 4; ++i) rec.v[i] = load128<kStreamOnce>(r, mine + 1024u * i);
+  rec.scales = load128<kStreamOnce>(r, column);
 }
 
 struct TileRef {
@@ -265,7 +336,30 @@ __device__ __forceinline__ void accumulate_record(const Record<FMT> &rec, const 
   uint4 ops[8];
   record_operands(rec, ops);
   const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
-  if constexpr (FMT == GGUF_FMT_Q4K) {
+  if constexpr (FMT == GGUF_FMT_Q80) {
+    // One fp16 scale a group; the operands' 128 leaves through the row sums: -128 d of groups kq and 4 + kq.
+    float s[8];
+#pragma unroll
+    for (uint32_t g = 0; g < 8; ++g) s[g] = q8_scale(rec.scales, g);
+    const uint32_t lowWord = kq == 0 ? rec.scales.x : kq == 1 ? rec.scales.x >> 16 : kq == 2 ? rec.scales.y : rec.scales.y >> 16;
+    const uint32_t highWord = kq == 0 ? rec.scales.z : kq == 1 ? rec.scales.z >> 16 : kq == 2 ? rec.scales.w : rec.scales.w >> 16;
+    const float c_lo = -128.f * half_bits_to_float(lowWord & 0xFFFFu), c_hi = -128.f * half_bits_to_float(highWord & 0xFFFFu);
+#pragma unroll
+    for (int t = 0; t < RT; ++t) {
+      acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(sums[t][0][lane], c_lo, acc[t], 0, 0, 0);
+      acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(sums[t][1][lane], c_hi, acc[t], 0, 0, 0);
+    }
+#pragma unroll
+    for (uint32_t g = 0; g < 8; ++g) {
+      const bf16x8 b = as_bf16x8(ops[g]);
+#pragma unroll
+      for (int t = 0; t < RT; ++t) {
+        const f32x4 dot = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a[t][g][lane]), b, zero, 0, 0, 0);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[t][i] = __fmaf_rn(dot[i], s[g], acc[t][i]);
+      }
+    }
+  } else if constexpr (FMT == GGUF_FMT_Q4K || FMT == GGUF_FMT_Q5K) {
     const Q4KScales sc = q4k_scales(rec.meta);
     float s[8];
 #pragma unroll
@@ -330,10 +424,11 @@ __device__ __forceinline__ void decode_workgroup(const uint8_t *__restrict__ seg
                                                  void *__restrict__ out, const uint16_t *__restrict__ residual,
                                                  float *__restrict__ partials, uint32_t *__restrict__ counters,
                                                  const GgufDecodeParams &p, const uint32_t item) {
-  constexpr uint32_t kRecord = FMT == GGUF_FMT_Q4K ? GGUF_Q4K_RECORD : GGUF_Q6K_RECORD;
+  constexpr uint32_t kRecord = gguf_record_bytes(FMT);
   constexpr bool kTable = EP == GGUF_EPILOGUE_GATE_UP_TABLE, kGateUp = EP == GGUF_EPILOGUE_GATE_UP || kTable;
-  constexpr uint32_t kColumnPart = FMT == GGUF_FMT_Q4K ? 2048u : GGUF_Q6K_SCALES;
-  constexpr uint32_t kSumsPerBlock = FMT == GGUF_FMT_Q4K ? 2 : 4;  // K = 4 MFMAs of row sums per super-block
+  constexpr uint32_t kColumnPart = Cursor<FMT>::kColumnPart;
+  constexpr bool kSums32 = FMT != GGUF_FMT_Q6K;                // the constant term rides on 32-input sums (Q6_K: 16)
+  constexpr uint32_t kSumsPerBlock = kSums32 ? 2 : 4;          // K = 4 MFMAs of row sums per super-block
   // The range's activations pass through LDS one super-block at a time (two buffers, one barrier
   // per super-block), each wave fetching a quarter of them, so a wave's vector-memory queue holds
   // almost only weights and the MFMA operands arrive on the LDS counter instead.
@@ -404,8 +499,8 @@ __device__ __forceinline__ void decode_workgroup(const uint8_t *__restrict__ seg
     uint32_t share[2];  // vector j of a row tile's super-block: byte offset of this thread's
 #pragma unroll
     for (int j = 0; j < 2; ++j) share[j] = (threadIdx.x + 256u * j) * 16u;
-    const uint32_t sumsAt = FMT == GGUF_FMT_Q4K ? gguf_table_sums32_offset(p.input_size, tiles) : gguf_table_sums16_offset(p.input_size, tiles);
-    const uint32_t sumGroups = FMT == GGUF_FMT_Q4K ? G : 2u * G;  // row-sum entries per row tile
+    const uint32_t sumsAt = kSums32 ? gguf_table_sums32_offset(p.input_size, tiles) : gguf_table_sums16_offset(p.input_size, tiles);
+    const uint32_t sumGroups = kSums32 ? G : 2u * G;  // row-sum entries per row tile
     const Resource sums = make_resource(table + sumsAt, tiles * sumGroups * 64u);
     // Threads past the staged sums repeat an earlier thread's (same value to the same slot).
     uint32_t sumShare[kSumShare], sumSlot[kSumShare];
@@ -740,5 +835,11 @@ SP_GGUF_DECODE("q4k", GGUF_FMT_Q4K, 64, 4);
 SP_GGUF_DECODE("q6k", GGUF_FMT_Q6K, 16, 1);
 SP_GGUF_DECODE("q6k", GGUF_FMT_Q6K, 32, 2);
 SP_GGUF_DECODE("q6k", GGUF_FMT_Q6K, 64, 4);
+SP_GGUF_DECODE("q5k", GGUF_FMT_Q5K, 16, 1);
+SP_GGUF_DECODE("q5k", GGUF_FMT_Q5K, 32, 2);
+SP_GGUF_DECODE("q5k", GGUF_FMT_Q5K, 64, 4);
+SP_GGUF_DECODE("q80", GGUF_FMT_Q80, 16, 1);
+SP_GGUF_DECODE("q80", GGUF_FMT_Q80, 32, 2);
+SP_GGUF_DECODE("q80", GGUF_FMT_Q80, 64, 4);
 
 } // namespace splash::kernels

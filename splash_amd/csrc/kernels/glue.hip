@@ -158,18 +158,29 @@ __global__ __launch_bounds__(64) void gguf_embed(const uint8_t *__restrict__ tab
     return;
   }
   const uint32_t blocks = p.hidden / 256u;
-  if constexpr (FMT == GGUF_FMT_Q4K) {
-    const uint8_t *blk = table + (size_t(token) * blocks + block) * GGUF_Q4K_NATIVE;
+  if constexpr (FMT == GGUF_FMT_Q4K || FMT == GGUF_FMT_Q5K) {
+    constexpr bool kFifth = FMT == GGUF_FMT_Q5K;   // Q5_K: 32 bytes of fifth bits between the scales and the nibbles
+    const uint8_t *blk = table + (size_t(token) * blocks + block) * (kFifth ? GGUF_Q5K_NATIVE : GGUF_Q4K_NATIVE);
     const float d = half_bits_to_float(blk[0] | (blk[1] << 8)), dmin = half_bits_to_float(blk[2] | (blk[3] << 8));
-    const uint8_t *sc = blk + 4, *qs = blk + 16;
+    const uint8_t *sc = blk + 4, *qh = blk + 16, *qs = blk + (kFifth ? 48 : 16);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const uint32_t k = tid + 64u * i, j = k / 32u, e = k % 32u;
       uint32_t s, m;
       if (j < 4) { s = sc[j] & 63u; m = sc[j + 4] & 63u; }
       else { s = (sc[j + 4] & 0xFu) | ((sc[j - 4] >> 6) << 4); m = (sc[j + 4] >> 4) | ((sc[j] >> 6) << 4); }
-      const uint32_t code = (qs[32u * (j / 2u) + e] >> (4u * (j % 2u))) & 15u;
+      uint32_t code = (qs[32u * (j / 2u) + e] >> (4u * (j % 2u))) & 15u;
+      if constexpr (kFifth) code |= ((qh[e] >> j) & 1u) << 4;
       o[k] = uint16_t(float_to_bf16_bits(__fmaf_rn(d * float(s), float(code), -(dmin * float(m)))));
+    }
+  } else if constexpr (FMT == GGUF_FMT_Q80) {
+    const uint8_t *blk = table + (size_t(token) * blocks + block) * GGUF_Q80_NATIVE;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t k = tid + 64u * i, j = k / 32u, e = k % 32u;
+      const uint8_t *group = blk + 34u * j;
+      const float d = half_bits_to_float(group[0] | (group[1] << 8));
+      o[k] = uint16_t(float_to_bf16_bits(d * float(int(int8_t(group[2u + e])))));
     }
   } else {
     const uint8_t *blk = table + (size_t(token) * blocks + block) * GGUF_Q6K_NATIVE;
@@ -186,5 +197,7 @@ __global__ __launch_bounds__(64) void gguf_embed(const uint8_t *__restrict__ tab
 }
 SP_REGISTER_KERNEL("gguf_embed_q4k", &gguf_embed<GGUF_FMT_Q4K>);
 SP_REGISTER_KERNEL("gguf_embed_q6k", &gguf_embed<GGUF_FMT_Q6K>);
+SP_REGISTER_KERNEL("gguf_embed_q5k", &gguf_embed<GGUF_FMT_Q5K>);
+SP_REGISTER_KERNEL("gguf_embed_q80", &gguf_embed<GGUF_FMT_Q80>);
 
 } // namespace splash::kernels

@@ -65,6 +65,35 @@ void packGgufImage(uint32_t formatId, const uint8_t *native, uint32_t rows, uint
               for (uint32_t w = 0; w < 4; ++w)
                 std::memcpy(rec + nibbleOffset(c, kq, h, w), qs + 64 * h + 32 * (w / 2) + 16 * (w % 2) + 4 * kq, 4);
           std::memcpy(rec + 2048 + 16 * c, blk, 16);
+        } else if (formatId == GGUF_FMT_Q5K) {
+          // Native: d, dmin, 12 scale bytes, qh[32] (bit j of byte i: the fifth bit of input i of group j), qs[128] as Q4_K's.
+          const uint8_t *qh = blk + 16, *qs = blk + 48;
+          for (uint32_t kq = 0; kq < 4; ++kq) {
+            for (uint32_t h = 0; h < 2; ++h) {
+              for (uint32_t w = 0; w < 4; ++w)
+                std::memcpy(rec + nibbleOffset(c, kq, h, w), qs + 64 * h + 32 * (w / 2) + 16 * (w % 2) + 4 * kq, 4);
+              uint32_t word = 0;
+              for (uint32_t gi = 0; gi < 4; ++gi)
+                for (uint32_t j = 0; j < 4; ++j)
+                  for (uint32_t half = 0; half < 2; ++half) {
+                    const uint32_t group = 4 * h + gi, input = gguf_operand_input(kq, 2 * j + half);
+                    word |= ((qh[input] >> group) & 1u) << (4 * gi + j + 16 * half);
+                  }
+              std::memcpy(rec + GGUF_Q5K_HIGH + 8 * (kq * 16 + c) + 4 * h, &word, 4);
+            }
+          }
+          std::memcpy(rec + GGUF_Q5K_META + 16 * c, blk, 16);
+        } else if (formatId == GGUF_FMT_Q80) {
+          // Native: eight blocks of (fp16 d, 32 int8).
+          for (uint32_t group = 0; group < 8; ++group) {
+            const uint8_t *q = blk + 34 * group + 2;
+            for (uint32_t kq = 0; kq < 4; ++kq) {
+              uint8_t *mine = rec + 1024 * (group / 2) + 16 * (kq * 16 + c) + 8 * (group % 2);
+              std::memcpy(mine, q + 4 * kq, 4);
+              std::memcpy(mine + 4, q + 16 + 4 * kq, 4);
+            }
+            std::memcpy(rec + GGUF_Q80_SCALES + 16 * c + 2 * group, blk + 34 * group, 2);
+          }
         } else {
           for (uint32_t kq = 0; kq < 4; ++kq) {
             for (uint32_t h = 0; h < 2; ++h)
@@ -120,6 +149,32 @@ void unpackGgufImage(uint32_t formatId, const uint8_t *image, uint32_t rows, uin
               for (uint32_t w = 0; w < 4; ++w)
                 std::memcpy(blk + 16 + 64 * h + 32 * (w / 2) + 16 * (w % 2) + 4 * kq, rec + nibbleOffset(c, kq, h, w), 4);
           std::memcpy(blk, rec + 2048 + 16 * c, 16);
+        } else if (formatId == GGUF_FMT_Q5K) {
+          uint8_t *qh = blk + 16, *qs = blk + 48;
+          for (uint32_t kq = 0; kq < 4; ++kq)
+            for (uint32_t h = 0; h < 2; ++h) {
+              for (uint32_t w = 0; w < 4; ++w)
+                std::memcpy(qs + 64 * h + 32 * (w / 2) + 16 * (w % 2) + 4 * kq, rec + nibbleOffset(c, kq, h, w), 4);
+              uint32_t word;
+              std::memcpy(&word, rec + GGUF_Q5K_HIGH + 8 * (kq * 16 + c) + 4 * h, 4);
+              for (uint32_t gi = 0; gi < 4; ++gi)
+                for (uint32_t j = 0; j < 4; ++j)
+                  for (uint32_t half = 0; half < 2; ++half) {
+                    const uint32_t group = 4 * h + gi, input = gguf_operand_input(kq, 2 * j + half);
+                    qh[input] = uint8_t(qh[input] | (((word >> (4 * gi + j + 16 * half)) & 1u) << group));
+                  }
+            }
+          std::memcpy(blk, rec + GGUF_Q5K_META + 16 * c, 16);
+        } else if (formatId == GGUF_FMT_Q80) {
+          for (uint32_t group = 0; group < 8; ++group) {
+            uint8_t *q = blk + 34 * group + 2;
+            for (uint32_t kq = 0; kq < 4; ++kq) {
+              const uint8_t *mine = rec + 1024 * (group / 2) + 16 * (kq * 16 + c) + 8 * (group % 2);
+              std::memcpy(q + 4 * kq, mine, 4);
+              std::memcpy(q + 16 + 4 * kq, mine + 4, 4);
+            }
+            std::memcpy(blk + 34 * group, rec + GGUF_Q80_SCALES + 16 * c + 2 * group, 2);
+          }
         } else {
           for (uint32_t kq = 0; kq < 4; ++kq) {
             uint32_t highWords[4];

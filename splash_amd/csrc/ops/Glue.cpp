@@ -1,5 +1,7 @@
 #include "ops/Glue.hpp"
 
+#include <string>
+
 #include <stdexcept>
 
 namespace splash::ops {
@@ -39,7 +41,7 @@ void Embedding::add(hip::CommandGraph &graph, const EmbeddingTable &table, const
   requireBytes(table.rows, uint64_t{table.vocabulary} * (table.hidden / GGUF_BLOCK) * gguf_native_bytes(table.formatId), "token table");
   requireBytes(tokens, uint64_t{rows} * 4, "input tokens");
   requireBytes(output, uint64_t{rows} * table.hidden * 2, "embedding output");
-  graph.add(table.formatId == GGUF_FMT_Q4K ? "gguf_embed_q4k" : "gguf_embed_q6k", {table.rows, tokens, output},
+  graph.add(std::string("gguf_embed_") + gguf_format_name(table.formatId), {table.rows, tokens, output},
             GgufEmbedParams{rows, table.vocabulary, table.hidden}, {rows, table.hidden / GGUF_BLOCK, 1}, {64, 1, 1});
 }
 

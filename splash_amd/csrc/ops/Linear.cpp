@@ -123,9 +123,8 @@ LinearPlan Linear::plan(LinearWorkload w, FloatOutput destination) const {
 }
 
 LinearPlan Linear::plan(const Projection &projection, uint32_t rows, LinearEpilogue epilogue) const {
-  uint32_t format = GGUF_FMT_Q4K;
-  for (const QuantizedSegment &segment : projection.blocks().segments)
-    if (segment.formatId == GGUF_FMT_Q6K) format = GGUF_FMT_Q6K;
+  // A dispatch's segments share one format (requireSegments).
+  const uint32_t format = projection.blocks().segments.empty() ? GGUF_FMT_Q4K : projection.blocks().segments.front().formatId;
   return plan(LinearWorkload{{projection.outputSize, projection.inputSize}, rows, epilogue, format},
               epilogue == LinearEpilogue::None ? projection.destination : FloatOutput::BFloat16);
 }

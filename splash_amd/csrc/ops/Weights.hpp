@@ -33,7 +33,7 @@ struct QuantizedSegment final {
   uint32_t columnOffset = 0;
   uint32_t formatId = GGUF_FMT_Q4K;
   // The kernel name token of its format (the reference's kQuantFormats[].name).
-  [[nodiscard]] const char *name() const noexcept { return formatId == GGUF_FMT_Q6K ? "q6k" : "q4k"; }
+  [[nodiscard]] const char *name() const noexcept { return gguf_format_name(formatId); }
 };
 
 struct BlockWeights final {

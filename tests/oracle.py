@@ -6,7 +6,7 @@ import os
 import numpy as np
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-FMT_Q4K, FMT_Q6K = 0, 4
+FMT_Q4K, FMT_Q5K, FMT_Q6K, FMT_Q80 = 0, 3, 4, 6
 NO_TOKEN = 0xFFFFFFFF
 
 _path = os.path.join(ROOT, "oracle", "liboracle.so")

@@ -31,13 +31,14 @@ def test_library_exports_every_declared_symbol():
 
 
 def test_kernels_are_registered_by_name():
-    for name in ("gguf_prepare_table", "gguf_dequant_q4k", "gguf_dequant_q6k", "gguf_decode_q4k_m16_a",
-                 "gguf_decode_q6k_m16_a_f32", "gguf_decode_q4k_m32_g", "gguf_decode_q6k_m64_r"):
+    for name in ("gguf_prepare_table", "gguf_dequant_q4k", "gguf_dequant_q6k", "gguf_dequant_q5k", "gguf_dequant_q80",
+                 "gguf_decode_q4k_m16_a", "gguf_decode_q6k_m16_a_f32", "gguf_decode_q4k_m32_g", "gguf_decode_q6k_m64_r",
+                 "gguf_decode_q5k_m16_gt", "gguf_decode_q80_m64_rn"):
         assert splash_amd.lib.sp_kernel_exists(name.encode()), name
     assert not splash_amd.lib.sp_kernel_exists(b"no_such_kernel")
 
 
-@pytest.mark.parametrize("fmt", [ops.FMT_Q4K, ops.FMT_Q6K])
+@pytest.mark.parametrize("fmt", [ops.FMT_Q4K, ops.FMT_Q6K, ops.FMT_Q5K, ops.FMT_Q80])
 def test_image_is_a_permutation_of_the_native_rows(fmt):
     """decode(retile(native)) == decode(native) follows from unpack(pack(native)) == native."""
     native = orc.fixture(fmt, 48, 768, 5)

@@ -24,7 +24,10 @@ def dequant_on_gpu(backend, fmt, native, rows, K):
     return out.download(np.float32).reshape(rows, K)
 
 
-@pytest.mark.parametrize("name,fmt", [("q4k", ops.FMT_Q4K), ("q6k", ops.FMT_Q6K)])
+ALL_FORMATS = [ops.FMT_Q4K, ops.FMT_Q6K, ops.FMT_Q5K, ops.FMT_Q80]
+
+
+@pytest.mark.parametrize("name,fmt", [("q4k", ops.FMT_Q4K), ("q6k", ops.FMT_Q6K), ("q5k", ops.FMT_Q5K), ("q80", ops.FMT_Q80)])
 def test_image_dequantization_matches_ggml_golden_hash(backend, name, fmt):
     """gguf_reference_test.mm:23-30 + gguf_dequant_test.mm:44-58: the kernels' unpacking of the
     re-tiled image gives GGML's fp32 values bit for bit."""
@@ -74,7 +77,7 @@ def check_interval(got_f32, oracle_result):
     assert not bad.any(), (int(bad.sum()), got_f32[bad][:4], lo[bad][:4], hi[bad][:4])
 
 
-@pytest.mark.parametrize("fmt", [ops.FMT_Q4K, ops.FMT_Q6K])
+@pytest.mark.parametrize("fmt", ALL_FORMATS)
 @pytest.mark.parametrize("M", [1, 4, 8, 16, 32, 64])
 def test_projection_lies_in_the_reference_interval(backend, fmt, M):
     """gguf_projection_test.mm:217-237: the bf16 result lies in [bf16(lo), bf16(hi)] of the fp64 dot
@@ -92,7 +95,7 @@ def test_projection_lies_in_the_reference_interval(backend, fmt, M):
     assert np.all(np.abs(got32.astype(np.float64) - want["exact"]) <= want["bound"])
 
 
-@pytest.mark.parametrize("fmt", [ops.FMT_Q4K, ops.FMT_Q6K])
+@pytest.mark.parametrize("fmt", ALL_FORMATS)
 def test_rows_do_not_depend_on_the_block_or_the_partition(backend, fmt):
     """Tested invariants of the reference (gguf_projection_test.mm): a row's result is bitwise the same
     alone or in a taller block, and splits sum in split order so a re-run is bit-identical."""
@@ -165,7 +168,7 @@ def test_fused_segments_equal_each_alone(backend):
         at += n
 
 
-@pytest.mark.parametrize("fmt", [ops.FMT_Q4K, ops.FMT_Q6K])
+@pytest.mark.parametrize("fmt", ALL_FORMATS)
 def test_residual_and_gate_up_epilogues(backend, fmt):
     """gguf_tile.h:10-16, gguf_linear.metal:34-71: bf16(v + res) and bf16(bf16(up) silu(bf16(gate)));
     the one-pass pair equals the two projections' fp32 sums put through the oracle's epilogue."""
