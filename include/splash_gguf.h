@@ -1,0 +1,55 @@
+/* GGUF files: the header parser and the step from a file's tensor to what the operators take.
+ * Replaces, for the verify step's weights, the reference's model::GgufFile / GgufTensor / GgufMetadata
+ * (runtime/model/GgufFile.hpp:24-150) and the image preparation of runtime/model/GgufImage.cpp: a tensor
+ * of a projection format (Q4_K, Q5_K, Q6_K, Q8_0) becomes the weight image spo_projection_create takes,
+ * a 16- or 32-bit float vector the bf16 weights of a norm. Status codes and the thread-local message of
+ * sp_last_error are those of splash_hip.h; a malformed file is SP_BACKEND_ERROR with the parser's message. */
+#pragma once
+#include "splash_hip.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct spg_file spg_file; /* model::GgufFile: the mapped file and its parsed header */
+
+/* GgufFile::GgufFile (GgufFile.hpp:117): GGUF version 3, one file. */
+sp_status spg_open(const char *path, spg_file **out);
+void spg_close(spg_file *file);
+
+/* GgufMetadata (GgufFile.hpp:95-107): integers and booleans as unsigned, floats as double, strings.
+ * A getter returns 0 when the key is absent or of another kind; spg_metadata_string returns the
+ * string's size with its terminator and copies up to `capacity` bytes. */
+int spg_metadata_unsigned(const spg_file *file, const char *key, uint64_t *value);
+int spg_metadata_float(const spg_file *file, const char *key, double *value);
+size_t spg_metadata_string(const spg_file *file, const char *key, char *out, size_t capacity);
+
+/* GgufFile::tensors / find (GgufFile.hpp:131-133). */
+typedef struct spg_tensor {
+  uint32_t ggml_type;   /* as the file stores it (ggml-common.h) */
+  uint32_t dimensions;  /* 1..4 */
+  uint64_t dims[4];     /* dims[0] is the row length */
+  uint64_t bytes;
+  uint32_t format;      /* the weight-image format (GGUF_FMT_* numbering) or 0xFFFFFFFF when the projections do not read the type */
+  uint32_t reserved;
+} spg_tensor;
+uint64_t spg_tensor_count(const spg_file *file);
+/* The tensor's name (size with terminator, copied up to `capacity`) and description; index below the count. */
+size_t spg_tensor_name(const spg_file *file, uint64_t index, char *out, size_t capacity);
+sp_status spg_tensor_info(const spg_file *file, uint64_t index, spg_tensor *out);
+/* Index of the tensor of that name, or -1. */
+int64_t spg_find(const spg_file *file, const char *name);
+/* The tensor's bytes in the mapped file, valid until spg_close. */
+const void *spg_tensor_data(const spg_file *file, uint64_t index);
+
+/* Rows [first_row, first_row + rows) (rows 0: all) of a two-dimensional tensor of a projection format, packed
+ * as the weight image and uploaded: whole 16-row tiles of whole 256-input super-blocks. The caller releases
+ * the buffer; format, rows and input size are what spo_projection_create takes beside it. */
+sp_status spg_load_image(sp_backend *backend, const spg_file *file, uint64_t index, uint32_t first_row, uint32_t rows,
+                         sp_buffer **image, uint32_t *format, uint32_t *out_rows, uint32_t *input_size);
+/* An F32, F16 or BF16 tensor as bf16 in device memory (a norm's weights). The caller releases the buffer. */
+sp_status spg_load_bf16(sp_backend *backend, const spg_file *file, uint64_t index, sp_buffer **out, uint64_t *elements);
+
+#ifdef __cplusplus
+}
+#endif

@@ -269,3 +269,23 @@ _sig("spo_hybrid_verify_layout", c_int, c_p, P(c_u64), P(c_u64), P(c_u64), P(Gdn
 _sig("spo_hybrid_verify_step_bytes", c_u64, c_p, P(HybridLane), c_u32)
 _sig("spo_hybrid_verify_encode", c_int, c_p, c_p, P(HybridLane), c_u32, c_int)
 _sig("spo_hybrid_verify_encode_part", c_int, c_p, c_p, c_u32, c_u32, P(HybridLane), c_u32)
+
+
+# ---- GGUF files (include/splash_gguf.h) ----
+class GgufTensor(ctypes.Structure):
+    _fields_ = [("ggml_type", c_u32), ("dimensions", c_u32), ("dims", ctypes.c_uint64 * 4), ("bytes", ctypes.c_uint64),
+                ("format", c_u32), ("reserved", c_u32)]
+
+
+_sig("spg_open", c_int, ctypes.c_char_p, P(c_p))
+_sig("spg_close", None, c_p)
+_sig("spg_metadata_unsigned", c_int, c_p, ctypes.c_char_p, P(ctypes.c_uint64))
+_sig("spg_metadata_float", c_int, c_p, ctypes.c_char_p, P(c_double))
+_sig("spg_metadata_string", ctypes.c_size_t, c_p, ctypes.c_char_p, ctypes.c_char_p, ctypes.c_size_t)
+_sig("spg_tensor_count", ctypes.c_uint64, c_p)
+_sig("spg_tensor_name", ctypes.c_size_t, c_p, ctypes.c_uint64, ctypes.c_char_p, ctypes.c_size_t)
+_sig("spg_tensor_info", c_int, c_p, ctypes.c_uint64, P(GgufTensor))
+_sig("spg_find", ctypes.c_int64, c_p, ctypes.c_char_p)
+_sig("spg_tensor_data", c_p, c_p, ctypes.c_uint64)
+_sig("spg_load_image", c_int, c_p, c_p, ctypes.c_uint64, c_u32, c_u32, P(c_p), P(c_u32), P(c_u32), P(c_u32))
+_sig("spg_load_bf16", c_int, c_p, c_p, ctypes.c_uint64, P(c_p), P(ctypes.c_uint64))

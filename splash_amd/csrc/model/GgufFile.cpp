@@ -1,0 +1,256 @@
+#include "model/GgufFile.hpp"
+
+#include "abi/Gguf.h"
+#include "ops/GgufImage.hpp"
+
+#include <array>
+#include <cmath>
+#include <cstring>
+#include <fcntl.h>
+#include <sys/mman.h>
+#include <sys/stat.h>
+#include <unistd.h>
+
+namespace splash::model {
+
+namespace {
+
+constexpr std::array<std::pair<uint32_t, GgmlTypeTraits>, 12> kTypes{{
+    {0, {"F32", 1, 4}},        {1, {"F16", 1, 2}},        {2, {"Q4_0", 32, 18}},    {3, {"Q4_1", 32, 20}},
+    {8, {"Q8_0", 32, 34}},     {10, {"Q2_K", 256, 84}},   {11, {"Q3_K", 256, 110}}, {12, {"Q4_K", 256, 144}},
+    {13, {"Q5_K", 256, 176}},  {14, {"Q6_K", 256, 210}},  {23, {"IQ4_XS", 256, 136}}, {30, {"BF16", 1, 2}},
+}};
+
+// GGUF metadata value types.
+enum : uint32_t { kU8, kI8, kU16, kI16, kU32, kI32, kF32, kBool, kString, kArray, kU64, kI64, kF64 };
+
+struct Reader {
+  const uint8_t *base;
+  uint64_t size, at = 0;
+  void need(uint64_t bytes) const {
+    if (bytes > size - at) throw GgufError("GGUF header is truncated");
+  }
+  template <class T> T take() {
+    need(sizeof(T));
+    T v;
+    std::memcpy(&v, base + at, sizeof(T));
+    at += sizeof(T);
+    return v;
+  }
+  std::string string() {
+    const uint64_t n = take<uint64_t>();
+    if (n > (1u << 24)) throw GgufError("GGUF string is too long");
+    need(n);
+    std::string s(reinterpret_cast<const char *>(base + at), n);
+    at += n;
+    return s;
+  }
+  void skipValue(uint32_t type) {
+    static constexpr uint32_t kBytes[] = {1, 1, 2, 2, 4, 4, 4, 1, 0, 0, 8, 8, 8};
+    if (type == kString) { (void)string(); return; }
+    if (type == kArray) {
+      const uint32_t inner = take<uint32_t>();
+      const uint64_t n = take<uint64_t>();
+      if (inner == kArray || inner > kF64) throw GgufError("unsupported GGUF array");
+      if (inner == kString) { for (uint64_t i = 0; i < n; ++i) (void)string(); return; }
+      if (n > (size - at) / kBytes[inner]) throw GgufError("GGUF header is truncated");
+      at += n * kBytes[inner];
+      return;
+    }
+    if (type > kF64) throw GgufError("unknown GGUF metadata type");
+    need(kBytes[type]);
+    at += kBytes[type];
+  }
+};
+
+float halfToFloat(uint16_t h) {
+  const uint32_t sign = uint32_t(h & 0x8000u) << 16, exponent = (h >> 10) & 31u, mantissa = h & 0x3FFu;
+  uint32_t bits;
+  if (exponent == 31) bits = sign | 0x7F800000u | (mantissa << 13);
+  else if (exponent) bits = sign | ((exponent + 112u) << 23) | (mantissa << 13);
+  else if (!mantissa) bits = sign;
+  else {
+    int shift = 0;
+    uint32_t m = mantissa;
+    while (!(m & 0x400u)) { m <<= 1; ++shift; }
+    bits = sign | ((113u - shift) << 23) | ((m & 0x3FFu) << 13);
+  }
+  float f;
+  std::memcpy(&f, &bits, 4);
+  return f;
+}
+uint16_t floatToBf16(float f) {  // nearest, ties to even
+  uint32_t v;
+  std::memcpy(&v, &f, 4);
+  if ((v & 0x7FFFFFFFu) > 0x7F800000u) return uint16_t((v >> 16) | 0x40u);
+  return uint16_t((v + 0x7FFFu + ((v >> 16) & 1u)) >> 16);
+}
+
+} // namespace
+
+const GgmlTypeTraits *ggmlTypeTraits(uint32_t type) noexcept {
+  for (const auto &[id, traits] : kTypes)
+    if (id == type) return &traits;
+  return nullptr;
+}
+
+std::optional<uint32_t> imageFormat(uint32_t ggmlType) noexcept {
+  switch (ggmlType) {
+    case ggml::kQ4_K: return GGUF_FMT_Q4K;
+    case ggml::kQ5_K: return GGUF_FMT_Q5K;
+    case ggml::kQ6_K: return GGUF_FMT_Q6K;
+    case ggml::kQ8_0: return GGUF_FMT_Q80;
+    default: return std::nullopt;
+  }
+}
+
+uint64_t GgufTensor::rows() const noexcept {
+  uint64_t n = dims.empty() ? 0 : 1;
+  for (size_t i = 1; i < dims.size(); ++i) n *= dims[i];
+  return n;
+}
+
+std::optional<uint64_t> GgufMetadata::unsignedValue(std::string_view key) const {
+  const auto it = unsigneds.find(key);
+  return it == unsigneds.end() ? std::nullopt : std::optional<uint64_t>(it->second);
+}
+std::optional<double> GgufMetadata::floatValue(std::string_view key) const {
+  const auto it = floats.find(key);
+  return it == floats.end() ? std::nullopt : std::optional<double>(it->second);
+}
+std::optional<std::string> GgufMetadata::stringValue(std::string_view key) const {
+  const auto it = strings.find(key);
+  return it == strings.end() ? std::nullopt : std::optional<std::string>(it->second);
+}
+
+GgufFile::GgufFile(const std::string &path) {
+  const int fd = ::open(path.c_str(), O_RDONLY);
+  if (fd < 0) throw GgufError("cannot open " + path);
+  struct stat st {};
+  if (::fstat(fd, &st) != 0 || st.st_size < 24) {
+    ::close(fd);
+    throw GgufError("not a GGUF file: " + path);
+  }
+  size_ = uint64_t(st.st_size);
+  void *mapped = ::mmap(nullptr, size_, PROT_READ, MAP_PRIVATE, fd, 0);
+  ::close(fd);
+  if (mapped == MAP_FAILED) throw GgufError("cannot map " + path);
+  base_ = static_cast<const uint8_t *>(mapped);
+  try {
+    Reader r{base_, size_};
+    if (r.take<uint32_t>() != 0x46554747u) throw GgufError("not a GGUF file: " + path);  // "GGUF"
+    const uint32_t version = r.take<uint32_t>();
+    if (version != 3) throw GgufError("unsupported GGUF version " + std::to_string(version));
+    const uint64_t tensorCount = r.take<uint64_t>(), valueCount = r.take<uint64_t>();
+    if (tensorCount > (1u << 20) || valueCount > (1u << 20)) throw GgufError("implausible GGUF counts");
+    for (uint64_t i = 0; i < valueCount; ++i) {
+      const std::string key = r.string();
+      const uint32_t type = r.take<uint32_t>();
+      switch (type) {
+        case kU8: metadata_.unsigneds[key] = r.take<uint8_t>(); break;
+        case kI8: metadata_.unsigneds[key] = uint64_t(int64_t(r.take<int8_t>())); break;
+        case kU16: metadata_.unsigneds[key] = r.take<uint16_t>(); break;
+        case kI16: metadata_.unsigneds[key] = uint64_t(int64_t(r.take<int16_t>())); break;
+        case kU32: metadata_.unsigneds[key] = r.take<uint32_t>(); break;
+        case kI32: metadata_.unsigneds[key] = uint64_t(int64_t(r.take<int32_t>())); break;
+        case kBool: metadata_.unsigneds[key] = r.take<uint8_t>() != 0; break;
+        case kU64: metadata_.unsigneds[key] = r.take<uint64_t>(); break;
+        case kI64: metadata_.unsigneds[key] = uint64_t(r.take<int64_t>()); break;
+        case kF32: metadata_.floats[key] = r.take<float>(); break;
+        case kF64: metadata_.floats[key] = r.take<double>(); break;
+        case kString: metadata_.strings[key] = r.string(); break;
+        default: r.skipValue(type); break;  // arrays (tokenizer tables) are not kept
+      }
+    }
+    const uint64_t alignment = metadata_.unsignedValue("general.alignment").value_or(32);
+    if (alignment < 8 || alignment > 65536 || (alignment & (alignment - 1))) throw GgufError("invalid GGUF alignment");
+    tensors_.reserve(tensorCount);
+    for (uint64_t i = 0; i < tensorCount; ++i) {
+      GgufTensor t;
+      t.name = r.string();
+      const uint32_t dimensions = r.take<uint32_t>();
+      if (!dimensions || dimensions > 4) throw GgufError("tensor has an unsupported rank: " + t.name);
+      for (uint32_t d = 0; d < dimensions; ++d) t.dims.push_back(r.take<uint64_t>());
+      t.type = r.take<uint32_t>();
+      t.offset = r.take<uint64_t>();
+      const GgmlTypeTraits *traits = ggmlTypeTraits(t.type);
+      if (!traits) throw GgufError("tensor " + t.name + " has unknown ggml type " + std::to_string(t.type));
+      if (!t.columns() || t.columns() % traits->blockElements) throw GgufError("tensor rows do not hold whole blocks: " + t.name);
+      if (t.rows() && t.columns() / traits->blockElements > UINT64_MAX / traits->blockBytes / t.rows())
+        throw GgufError("tensor is too large: " + t.name);
+      t.bytes = t.columns() / traits->blockElements * traits->blockBytes * t.rows();
+      if (t.offset % alignment) throw GgufError("tensor data is misaligned: " + t.name);
+      if (!index_.emplace(t.name, tensors_.size()).second) throw GgufError("duplicate tensor " + t.name);
+      tensors_.push_back(std::move(t));
+    }
+    dataStart_ = (r.at + alignment - 1) / alignment * alignment;
+    for (const GgufTensor &t : tensors_)
+      if (dataStart_ > size_ || t.offset > size_ - dataStart_ || t.bytes > size_ - dataStart_ - t.offset)
+        throw GgufError("tensor data lies past the end of the file: " + t.name);
+  } catch (...) {
+    ::munmap(const_cast<uint8_t *>(base_), size_);
+    base_ = nullptr;
+    throw;
+  }
+}
+
+GgufFile::~GgufFile() {
+  if (base_) ::munmap(const_cast<uint8_t *>(base_), size_);
+}
+
+const GgufTensor *GgufFile::find(std::string_view name) const noexcept {
+  const auto it = index_.find(name);
+  return it == index_.end() ? nullptr : &tensors_[it->second];
+}
+const GgufTensor &GgufFile::require(std::string_view name) const {
+  if (const GgufTensor *t = find(name)) return *t;
+  throw GgufError("missing tensor " + std::string(name));
+}
+const uint8_t *GgufFile::data(const GgufTensor &tensor) const { return base_ + dataStart_ + tensor.offset; }
+
+LoadedImage loadImage(hip::Backend &backend, const GgufFile &file, const GgufTensor &tensor, uint32_t firstRow, uint32_t rows) {
+  const std::optional<uint32_t> format = imageFormat(tensor.type);
+  if (!format) throw std::invalid_argument("tensor " + tensor.name + " is not of a projection format");
+  if (tensor.dims.size() != 2) throw std::invalid_argument("a projection tensor has two dimensions: " + tensor.name);
+  const uint64_t all = tensor.rows(), columns = tensor.columns();
+  if (!rows) rows = uint32_t(all - std::min<uint64_t>(all, firstRow));
+  if (!rows || uint64_t{firstRow} + rows > all || rows % GGUF_TILE_COLUMNS || firstRow % GGUF_TILE_COLUMNS || columns % GGUF_BLOCK ||
+      columns > UINT32_MAX)
+    throw std::invalid_argument("a weight image holds whole 16-row tiles of whole 256-input super-blocks: " + tensor.name);
+  const uint64_t rowBytes = columns / GGUF_BLOCK * gguf_native_bytes(*format);
+  const uint8_t *native = file.data(tensor) + uint64_t{firstRow} * rowBytes;
+  std::vector<uint8_t> image(gguf_image_bytes(*format, rows, uint32_t(columns)));
+  ops::packGgufImage(*format, native, rows, uint32_t(columns), image.data());
+  LoadedImage out;
+  out.formatId = *format;
+  out.rows = rows;
+  out.inputSize = uint32_t(columns);
+  out.image = backend.allocateBuffer(image.size(), hip::BufferStorage::Private, tensor.name.c_str());
+  out.image.upload(image.data(), image.size());
+  return out;
+}
+
+hip::Buffer loadBf16Vector(hip::Backend &backend, const GgufFile &file, const GgufTensor &tensor) {
+  if (tensor.type != ggml::kF32 && tensor.type != ggml::kF16 && tensor.type != ggml::kBF16)
+    throw std::invalid_argument("tensor " + tensor.name + " is not a 16- or 32-bit float vector");
+  const uint64_t n = tensor.elements();
+  std::vector<uint16_t> bits(n);
+  const uint8_t *data = file.data(tensor);
+  for (uint64_t i = 0; i < n; ++i) {
+    if (tensor.type == ggml::kBF16) std::memcpy(&bits[i], data + 2 * i, 2);
+    else if (tensor.type == ggml::kF16) {
+      uint16_t h;
+      std::memcpy(&h, data + 2 * i, 2);
+      bits[i] = floatToBf16(halfToFloat(h));
+    } else {
+      float f;
+      std::memcpy(&f, data + 4 * i, 4);
+      bits[i] = floatToBf16(f);
+    }
+  }
+  hip::Buffer out = backend.allocateBuffer(std::max<uint64_t>(n * 2, 16), hip::BufferStorage::Private, tensor.name.c_str());
+  out.upload(bits.data(), n * 2);
+  return out;
+}
+
+} // namespace splash::model

@@ -1,0 +1,98 @@
+// Header parser for llama.cpp GGUF files (version 3) and the step from a file's tensor to what the
+// operators take: the counterpart of the reference's runtime/model/GgufFile.hpp:24-150 (GgufFile,
+// GgufTensor, GgufMetadata) and of the image preparation in GgufImage.cpp, scoped to the formats
+// the projections read (Q4_K, Q5_K, Q6_K, Q8_0) and the 16/32-bit vectors of the norms. The file is
+// mapped read-only; tensor data is read in place.
+#pragma once
+#include "hip/Backend.hpp"
+
+#include <cstdint>
+#include <map>
+#include <optional>
+#include <stdexcept>
+#include <string>
+#include <string_view>
+#include <vector>
+
+namespace splash::model {
+
+class GgufError : public std::runtime_error {
+public:
+  using std::runtime_error::runtime_error;
+};
+
+// ggml type ids as GGUF tensor infos store them (ggml-common.h; GgufFile.hpp:35-66 in the reference).
+namespace ggml {
+inline constexpr uint32_t kF32 = 0, kF16 = 1, kQ8_0 = 8, kQ4_K = 12, kQ5_K = 13, kQ6_K = 14, kBF16 = 30;
+}
+struct GgmlTypeTraits {
+  const char *name;
+  uint32_t blockElements;
+  uint32_t blockBytes;
+};
+// nullptr for a type this parser cannot size.
+[[nodiscard]] const GgmlTypeTraits *ggmlTypeTraits(uint32_t type) noexcept;
+// The weight-image format (abi/Gguf.h) of a ggml type, if the projections read it.
+[[nodiscard]] std::optional<uint32_t> imageFormat(uint32_t ggmlType) noexcept;
+
+struct GgufTensor {
+  std::string name;
+  uint32_t type = 0;
+  std::vector<uint64_t> dims;  // dims[0] is the fastest (row length)
+  uint64_t offset = 0;         // in the file's tensor data
+  uint64_t bytes = 0;
+  [[nodiscard]] uint64_t columns() const noexcept { return dims.empty() ? 0 : dims[0]; }
+  [[nodiscard]] uint64_t rows() const noexcept;
+  [[nodiscard]] uint64_t elements() const noexcept { return columns() * rows(); }
+};
+
+// Scalar metadata by key: every integer and boolean as unsigned (a negative one as its two's
+// complement), every float as a double, and the strings (GgufFile.hpp:95-107).
+struct GgufMetadata {
+  std::map<std::string, uint64_t, std::less<>> unsigneds;
+  std::map<std::string, double, std::less<>> floats;
+  std::map<std::string, std::string, std::less<>> strings;
+  [[nodiscard]] std::optional<uint64_t> unsignedValue(std::string_view key) const;
+  [[nodiscard]] std::optional<double> floatValue(std::string_view key) const;
+  [[nodiscard]] std::optional<std::string> stringValue(std::string_view key) const;
+};
+
+class GgufFile final {
+public:
+  // Maps the file and parses its header; throws GgufError on a malformed or truncated file.
+  explicit GgufFile(const std::string &path);
+  ~GgufFile();
+  GgufFile(const GgufFile &) = delete;
+  GgufFile &operator=(const GgufFile &) = delete;
+
+  [[nodiscard]] const GgufMetadata &metadata() const noexcept { return metadata_; }
+  [[nodiscard]] const std::vector<GgufTensor> &tensors() const noexcept { return tensors_; }
+  [[nodiscard]] const GgufTensor *find(std::string_view name) const noexcept;
+  [[nodiscard]] const GgufTensor &require(std::string_view name) const;
+  // The tensor's bytes in the mapped file.
+  [[nodiscard]] const uint8_t *data(const GgufTensor &tensor) const;
+
+private:
+  const uint8_t *base_ = nullptr;
+  uint64_t size_ = 0;
+  uint64_t dataStart_ = 0;
+  GgufMetadata metadata_;
+  std::vector<GgufTensor> tensors_;
+  std::map<std::string, size_t, std::less<>> index_;
+};
+
+// A projection tensor's weight image in device memory.
+struct LoadedImage {
+  uint32_t formatId = 0;
+  uint32_t rows = 0;       // output size
+  uint32_t inputSize = 0;  // K
+  hip::Buffer image;
+};
+// Packs rows [firstRow, firstRow + rows) of a 2-D tensor of an image format (whole 16-row tiles of
+// whole 256-input super-blocks) and uploads them; rows = 0 takes all.
+[[nodiscard]] LoadedImage loadImage(hip::Backend &backend, const GgufFile &file, const GgufTensor &tensor, uint32_t firstRow = 0,
+                                    uint32_t rows = 0);
+// A 1-D F32, F16 or BF16 tensor as bf16 in device memory (the norms' weights).
+[[nodiscard]] hip::Buffer loadBf16Vector(hip::Backend &backend, const GgufFile &file, const GgufTensor &tensor);
+
+} // namespace splash::model

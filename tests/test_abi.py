@@ -15,10 +15,10 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 def declared_symbols():
     names = set()
-    for header in ("splash_hip.h", "splash_ops.h"):
+    for header in ("splash_hip.h", "splash_ops.h", "splash_gguf.h"):
         text = open(os.path.join(ROOT, "include", header)).read()
         text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-        names.update(re.findall(r"\b(spo?_[a-z0-9_]+)\s*\(", text))
+        names.update(re.findall(r"\b(sp[og]?_[a-z0-9_]+)\s*\(", text))
     names.discard("sp_completion")
     return sorted(names)
 

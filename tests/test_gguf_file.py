@@ -1,0 +1,113 @@
+"""The GGUF header parser (CPU) and the loading of a file's tensors as the operators' inputs (GPU)."""
+import numpy as np
+import pytest
+
+import splash_amd
+from splash_amd import gguf, ops
+from tests import gguf_writer as gw
+from tests import oracle as orc
+
+
+def model_file(path, alignment=32):
+    rng = np.random.default_rng(4)
+    tensors = [
+        ("blk.0.attn_q.weight", gw.GGML_Q4_K, [512, 96], orc.make_native(orc.FMT_Q4K, 96, 512, 1)),
+        ("blk.0.attn_v.weight", gw.GGML_Q6_K, [512, 32], orc.make_native(orc.FMT_Q6K, 32, 512, 2)),
+        ("blk.0.ffn_down.weight", gw.GGML_Q5_K, [768, 64], orc.make_native(orc.FMT_Q5K, 64, 768, 3)),
+        ("output.weight", gw.GGML_Q8_0, [512, 48], orc.make_native(orc.FMT_Q80, 48, 512, 4)),
+        ("blk.0.attn_norm.weight", gw.GGML_F32, [512], (1 + 0.1 * rng.standard_normal(512)).astype(np.float32)),
+        ("output_norm.weight", gw.GGML_BF16, [512], orc.f32_to_bf16((1 + 0.1 * rng.standard_normal(512)).astype(np.float32))),
+        ("blk.0.post_norm.weight", gw.GGML_F16, [512], (1 + 0.1 * rng.standard_normal(512)).astype(np.float16)),
+    ]
+    metadata = [("general.architecture", gw.STRING, "qwen3"), ("general.alignment", gw.U32, alignment),
+                ("qwen3.block_count", gw.U32, 1), ("qwen3.rope.freq_base", gw.F32, 1e6), ("qwen3.attention.layer_norm_rms_epsilon", gw.F64, 1e-6),
+                ("general.quantized", gw.BOOL, 1), ("general.negative", gw.I32, -2),
+                ("tokenizer.ggml.tokens", gw.ARRAY, (gw.STRING, ["a", "bc", "def"])), ("tokenizer.ggml.scores", gw.ARRAY, (gw.F32, [0.5, 1.5]))]
+    gw.write_gguf(path, metadata, tensors, alignment=alignment)
+    return tensors
+
+
+@pytest.mark.parametrize("alignment", [32, 64])
+def test_header_metadata_and_tensor_table(tmp_path, alignment):
+    path = tmp_path / "model.gguf"
+    tensors = model_file(path, alignment)
+    f = gguf.GgufFile(path)
+    assert f.string("general.architecture") == "qwen3" and f.unsigned("qwen3.block_count") == 1
+    assert f.float("qwen3.rope.freq_base") == 1e6 and f.float("qwen3.attention.layer_norm_rms_epsilon") == 1e-6
+    assert f.unsigned("general.quantized") == 1 and f.unsigned("general.negative") == 2 ** 64 - 2
+    assert f.string("missing") is None and f.unsigned("general.architecture") is None and f.string("tokenizer.ggml.tokens") is None
+    assert [t.name for t in f.tensors] == [t[0] for t in tensors]
+    for got, (name, kind, dims, data) in zip(f.tensors, tensors):
+        assert (got.ggml_type, got.dims, got.bytes) == (kind, dims, np.asarray(data).nbytes)
+        assert np.array_equal(f.data(got), np.frombuffer(np.ascontiguousarray(data).tobytes(), np.uint8))
+    assert [f.find(n).format for n in ("blk.0.attn_q.weight", "blk.0.attn_v.weight", "blk.0.ffn_down.weight", "output.weight")] == \
+        [ops.FMT_Q4K, ops.FMT_Q6K, ops.FMT_Q5K, ops.FMT_Q80]
+    assert f.find("output_norm.weight").format is None and f.find("nothing") is None
+
+
+def test_malformed_files_are_refused(tmp_path):
+    good = tmp_path / "good.gguf"
+    model_file(good)
+    raw = open(good, "rb").read()
+    cases = {"magic": b"GGML" + raw[4:], "version": raw[:4] + (2).to_bytes(4, "little") + raw[8:], "truncated header": raw[:200],
+             "truncated data": raw[:-4096], "empty": b""}
+    for name, content in cases.items():
+        path = tmp_path / f"{name}.gguf"
+        open(path, "wb").write(content)
+        with pytest.raises(splash_amd.SplashError):
+            gguf.GgufFile(path)
+    with pytest.raises(splash_amd.SplashError):
+        gguf.GgufFile(tmp_path / "absent.gguf")
+    # an unknown tensor type, rows that do not hold whole blocks, a misaligned offset, an alignment that is no power of two
+    x = np.zeros(144, np.uint8)
+    for name, tensors, alignment in (("type", [("t", 99, [256], x)], 32), ("blocks", [("t", gw.GGML_Q4_K, [100], x)], 32),
+                                      ("alignment", [("t", gw.GGML_Q4_K, [256], x)], 48)):
+        path = tmp_path / f"bad_{name}.gguf"
+        gw.write_gguf(path, [("general.alignment", gw.U32, alignment)], tensors, alignment=alignment)
+        with pytest.raises(splash_amd.SplashError):
+            gguf.GgufFile(path)
+
+
+@pytest.mark.gpu
+def test_projections_and_norms_load_from_a_file(backend, tmp_path):
+    """A file's tensors become the operators' inputs: each projection format's rows give the result of the same
+    native rows packed by hand, a slice of rows is that slice, and 16- and 32-bit vectors arrive as bf16."""
+    path = tmp_path / "model.gguf"
+    tensors = {t[0]: t for t in model_file(path)}
+    f = gguf.GgufFile(path)
+    linear = ops.Linear(backend)
+    rng = np.random.default_rng(8)
+    for name in ("blk.0.attn_q.weight", "blk.0.attn_v.weight", "blk.0.ffn_down.weight", "output.weight"):
+        print(f"case gguf file tensor {name}", flush=True)
+        _, _, (K, N), native = tensors[name]
+        fmt, rows, input_size, image = f.load_image(backend, f.find(name))
+        assert (rows, input_size) == (N, K) and fmt == f.find(name).format
+        assert np.array_equal(image.download(np.uint8)[:ops.gguf_image_bytes(fmt, N, K)], ops.pack_gguf_image(fmt, native, N, K))
+        x_bits = orc.f32_to_bf16(rng.standard_normal((5, K)).astype(np.float32))
+        results = []
+        for projection in (ops.Projection([(fmt, N, image)], K, float32=True), ops.Projection.from_native(backend, [(fmt, N, native)], K, float32=True)):
+            plan = linear.plan(projection, 5)
+            out = backend.allocate_buffer(5 * N * 4)
+            graph = splash_amd.CommandGraph()
+            linear.add(graph, projection, plan, backend.from_array(x_bits), out, linear.scratch_for(backend, [plan]))
+            backend.run(graph)
+            results.append(out.download(np.float32).reshape(5, N))
+        assert np.array_equal(results[0], results[1])
+        want = orc.gemm(fmt, native, x_bits, N, want=("exact", "bound"))
+        assert np.all(np.abs(results[0] - want["exact"]) <= want["bound"])
+    # rows 32..63 of a tensor alone
+    _, _, (K, N), native = tensors["blk.0.attn_q.weight"]
+    fmt, rows, _, image = f.load_image(backend, f.find("blk.0.attn_q.weight"), first_row=32, rows=32)
+    row_bytes = len(native) // N
+    assert rows == 32 and np.array_equal(image.download(np.uint8)[:ops.gguf_image_bytes(fmt, 32, K)],
+                                         ops.pack_gguf_image(fmt, native[32 * row_bytes:64 * row_bytes], 32, K))
+    with pytest.raises(ValueError):
+        f.load_image(backend, f.find("blk.0.attn_q.weight"), first_row=8, rows=16)
+    with pytest.raises(ValueError):
+        f.load_image(backend, f.find("output_norm.weight"))
+    for name in ("blk.0.attn_norm.weight", "output_norm.weight", "blk.0.post_norm.weight"):
+        data = tensors[name][3]
+        want = data if data.dtype == np.uint16 else orc.f32_to_bf16(np.asarray(data, np.float32))
+        assert np.array_equal(f.load_bf16(backend, f.find(name)).download(np.uint16)[:512], want)
+    with pytest.raises(ValueError):
+        f.load_bf16(backend, f.find("output.weight"))
