@@ -7,8 +7,8 @@
 // Nothing under splash_amd/ links, loads or calls it.
 //
 // Pin status of each group of functions (what fixes it besides its own formula):
-//   orc_dequant_rows (Q4_K, Q6_K)   pinned: SHA-256 goldens of upstream GGML over the 256x1024
-//                                   fixture (dev/tests/fixtures/weight-goldens/goldens.json:3,7)
+//   orc_dequant_rows (Q4_K, Q5_K,   pinned: SHA-256 goldens of upstream GGML over the 256x1024
+//     Q6_K, Q8_0)                   fixture (dev/tests/fixtures/weight-goldens/goldens.json:3,6,7,9)
 //                                   and the compiled reference header (oracle/_ref).
 //   orc_fixture                     pinned by the same goldens (a wrong byte order changes the hash).
 //   orc_quantize_q4k / q6k          PARITY UNPINNED: the K-quantizer lives in llama.cpp/ggml
@@ -50,7 +50,7 @@ uint64_t orc_row_bytes(uint32_t fmt, uint32_t K);
 int orc_fixture(uint32_t fmt, uint32_t rows, uint32_t K, uint32_t seed, uint8_t *native);
 // dev/tests/engine/GgufFormatReference.hpp:195-219,295-323 makeNative with realistic scales.
 int orc_make_native(uint32_t fmt, uint32_t rows, uint32_t K, uint32_t seed, uint8_t *native);
-// llama.cpp dequantize_row_q4_K / q6_K semantics (GgufFormatReference.hpp:370-381, :418-432).
+// llama.cpp dequantize_row_q4_K / q5_K / q6_K / q8_0 semantics (GgufFormatReference.hpp:370-381, :405-432, :453-458).
 int orc_dequant_rows(uint32_t fmt, const uint8_t *native, uint32_t rows, uint32_t K, float *out);
 // llama.cpp-style quantize_row_q4_K_ref / q6_K_ref (parity unpinned, see header).
 int orc_quantize_rows(uint32_t fmt, const float *values, uint32_t rows, uint32_t K, uint8_t *native);
