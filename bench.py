@@ -202,7 +202,8 @@ def time_c3_ops(backend):
     bf = lambda a: (np.ascontiguousarray(a, np.float32).view(np.uint32) >> 16).astype(np.uint16)
     QH, KVH, D, rows = 64, 8, 128, 16
     results = []
-    for context in (8192, 32768, 131072):
+    # the contexts BASELINE names, and one that ends 16 tokens past a page (the block after a full 32K history)
+    for context in (8192, 32768, 32768 + rows, 131072):
         pages = (context + ops.PAGE_TOKENS - 1) // ops.PAGE_TOKENS
         kv_bytes = context * KVH * (2 * D + 4)
         copies = int(np.ceil(2 * 268.4e6 / kv_bytes)) + 1

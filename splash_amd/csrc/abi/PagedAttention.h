@@ -17,6 +17,7 @@
 #include <stdint.h>
 
 #define ATTENTION_PAGE_TOKENS 256u
+#define ATTENTION_STEP_TOKENS 64u    // tokens the split kernel takes at a time; history splits hold whole steps
 #define ATTENTION_VALUE_BLOCK 64u
 #define ATTENTION_MAXIMUM_ROWS 16u      // rows of one sequence's verify block (SPLASH_TARGET_VERIFY_ROWS)
 #define ATTENTION_MAXIMUM_SEQUENCES 8u  // sequences of one dispatch
@@ -69,8 +70,8 @@ struct AttentionSequence {
   uint32_t committed;        // tokens in its cache before the block; row r is stored at slot committed + r
   uint32_t table_first;      // its first entry in the page table
   uint16_t rows;             // rows of its block, 1..16
-  uint16_t pages_per_split;  // logical pages of one history split, from its own length alone, so
-                             // that batching never changes a sequence's result; the last split takes the rest
+  uint16_t steps_per_split;  // steps (ATTENTION_STEP_TOKENS tokens) of one history split, from its own length alone,
+                             // so that batching never changes a sequence's result; the last split takes the rest
 };
 
 struct AttentionParams {

@@ -175,8 +175,9 @@ __global__ __launch_bounds__(256, 2) void attention_q8_split(const _Float16 *__r
   const uint32_t h = blockIdx.x, split = blockIdx.y, z = blockIdx.z;
   const AttentionSequence seq = p.sequence[z];
   const uint32_t total = seq.committed + seq.rows;
-  // The sequence's own splits: ceil(pages / pages_per_split) of them; later grid rows are empty.
-  const uint32_t span = uint32_t(seq.pages_per_split) * ATTENTION_PAGE_TOKENS;
+  // The sequence's own splits: ceil(steps / steps_per_split) of them; later grid rows are empty.
+  static_assert(kStep == int(ATTENTION_STEP_TOKENS) && ATTENTION_PAGE_TOKENS % ATTENTION_STEP_TOKENS == 0, "a page holds whole steps");
+  const uint32_t span = uint32_t(seq.steps_per_split) * ATTENTION_STEP_TOKENS;
   const uint32_t first = min(total, split * span), last = min(total, (split + 1) * span);
   const uint32_t steps = first < last ? (last - first + kStep - 1) / kStep : 0;
   const float scale2 = kLog2e / sqrtf(float(D));

@@ -8,12 +8,14 @@
 namespace splash::ops {
 
 AttentionSplits attentionSplits(uint64_t tokens) noexcept {
-  // About 64 splits of a long history, whole pages each: with 8 KV heads that is two workgroups
-  // per compute unit; a split never holds less than one page.
-  const uint32_t pages = std::max(1u, kv::Layout::pagesFor(tokens));
+  // About 64 splits of a long history, whole 64-token steps each (a page holds whole steps, so no
+  // step straddles two pages): with 8 KV heads that is two workgroups per compute unit whatever the
+  // length; a split holds at least four steps (a page's worth), below which its fixed cost outweighs it.
+  const uint64_t steps = std::max<uint64_t>(1, (tokens + ATTENTION_STEP_TOKENS - 1) / ATTENTION_STEP_TOKENS);
   AttentionSplits s;
-  s.pagesPerSplit = std::max(1u, (pages + 63) / 64);
-  s.splits = (pages + s.pagesPerSplit - 1) / s.pagesPerSplit;
+  constexpr uint64_t kSplits = 64;
+  s.stepsPerSplit = uint32_t(std::max<uint64_t>(4, (steps + kSplits - 1) / kSplits));
+  s.splits = uint32_t((steps + s.stepsPerSplit - 1) / s.stepsPerSplit);
   return s;
 }
 
@@ -62,7 +64,7 @@ AttentionParams AttentionPlan::params(uint64_t pageBytes) const noexcept {
   p.page_bytes = pageBytes;
   for (size_t i = 0; i < sequences_.size(); ++i)
     p.sequence[i] = {sequences_[i].firstRow, sequences_[i].committed, sequences_[i].tableFirst, uint16_t(sequences_[i].rows),
-                     uint16_t(partition_[i].pagesPerSplit)};
+                     uint16_t(partition_[i].stepsPerSplit)};
   return p;
 }
 
@@ -77,7 +79,7 @@ AttentionPlan PagedAttention::plan(const AttentionGeometry &geometry, std::vecto
   for (const AttentionRows &s : sequences) {
     if (!s.rows || s.rows > ATTENTION_MAXIMUM_ROWS) throw std::invalid_argument("a sequence's verify block holds 1 to 16 rows");
     const AttentionSplits part = attentionSplits(uint64_t{s.committed} + s.rows);
-    if (part.splits > ATTENTION_MAXIMUM_SPLITS || part.pagesPerSplit > 0xFFFF)
+    if (part.splits > ATTENTION_MAXIMUM_SPLITS || part.stepsPerSplit > 0xFFFF)
       throw std::invalid_argument("the sequence is longer than the attention kernels split");
     plan.partition_.push_back(part);
     plan.splits_ = std::max(plan.splits_, part.splits);

@@ -45,11 +45,11 @@ struct AttentionRows final {
 };
 
 // History splits of a sequence of `tokens` tokens (committed + rows): a split holds
-// pagesPerSplit logical pages; the partition follows the sequence alone
+// stepsPerSplit steps of ATTENTION_STEP_TOKENS tokens; the partition follows the sequence alone
 // (PagedAttention.cpp:125-146 in the reference states the same rule for its geometry).
 struct AttentionSplits final {
   uint32_t splits = 1;
-  uint32_t pagesPerSplit = 1;
+  uint32_t stepsPerSplit = 1;
 };
 [[nodiscard]] AttentionSplits attentionSplits(uint64_t tokens) noexcept;
 
