@@ -146,7 +146,7 @@ def cpu_baseline(w):
 
 
 def time_c2_ops(backend):
-    """BASELINE config 2: each projection of the 27B shape alone at M = 1, 4, 8, 16, 32 rows, over a ring of weight
+    """BASELINE.json config 2: each projection of the 27B shape alone at M = 1, 4, 8, 16, 32 rows, over a ring of weight
     copies larger than twice the 256 MB memory-side cache so that every pass reads HBM; per-dispatch GPU time (HIP
     events around each dispatch), median over the ring passes after the first. Prints one JSON line."""
     import splash_amd
@@ -193,7 +193,7 @@ def time_c2_ops(backend):
 
 
 def time_c3_ops(backend):
-    """BASELINE config 3: block-causal attention of a 16-row chain block (64 query / 8 KV heads of 128) over a paged
+    """BASELINE.json config 3: block-causal attention of a 16-row chain block (64 query / 8 KV heads of 128) over a paged
     INT8 context of 8K, 32K and 128K tokens (256-token pages, random page table), the split pass and the merge, over a
     ring of KV pools past the caches. Prints one JSON line."""
     import splash_amd
@@ -202,7 +202,7 @@ def time_c3_ops(backend):
     bf = lambda a: (np.ascontiguousarray(a, np.float32).view(np.uint32) >> 16).astype(np.uint16)
     QH, KVH, D, rows = 64, 8, 128, 16
     results = []
-    # the contexts BASELINE names, and one that ends 16 tokens past a page (the block after a full 32K history)
+    # the contexts BASELINE.json names, and one that ends 16 tokens past a page (the block after a full 32K history)
     for context in (8192, 32768, 32768 + rows, 131072):
         pages = (context + ops.PAGE_TOKENS - 1) // ops.PAGE_TOKENS
         kv_bytes = context * KVH * (2 * D + 4)
@@ -245,7 +245,7 @@ def time_c3_ops(backend):
 
 def time_c5_ops(backend):
     """Per-dispatch GPU time (HIP events around each dispatch) of the Gated DeltaNet step and the MoE layer at the
-    35B-A3B shape of BASELINE config 5, batch 8 of 16-row blocks; weights and states in rings past the caches.
+    35B-A3B shape of BASELINE.json config 5, batch 8 of 16-row blocks; weights and states in rings past the caches.
     Prints one JSON line; not the headline metric (that is the dense step)."""
     import splash_amd
     from splash_amd import ops
@@ -310,7 +310,7 @@ C5 = dict(hidden=2048, vocabulary=151936, layers=48, q_heads=32, kv_heads=4, hea
 
 
 def bench_c5(backend, args):
-    """BASELINE config 5 at full size: a step of 8 lanes x 16 rows that folds the 16 rows each lane accepted of the
+    """BASELINE.json config 5 at full size: a step of 8 lanes x 16 rows that folds the 16 rows each lane accepted of the
     step before (the worst case of the rollback protocol) and runs 16 new ones. Not the headline metric."""
     import splash_amd
     from splash_amd import ops, synthetic, verify

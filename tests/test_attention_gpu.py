@@ -114,7 +114,7 @@ def test_tree_rows_and_resubmission(backend):
 
 
 def test_long_context_32k(backend):
-    """BASELINE's 32K context at the 27B geometry: 64 q / 8 kv heads x 128, 16 rows, permuted page table."""
+    """BASELINE.json's 32K context at the 27B geometry: 64 q / 8 kv heads x 128, 16 rows, permuted page table."""
     print("case attention 32k", flush=True)
     rng = np.random.default_rng(32)
     got, want, want64, _, _, _, plan = run_block(backend, rng, 64, 8, 128, 16, 32768 - 16)

@@ -1,4 +1,4 @@
-"""End-to-end parity of the hybrid mixture-of-experts verify step (BASELINE config 5 at a small shape: three Gated
+"""End-to-end parity of the hybrid mixture-of-experts verify step (BASELINE.json config 5 at a small shape: three Gated
 DeltaNet layers and one attention layer, 16 experts top-2) against the oracle, through the C ABI: every layer
 teacher-forced from the GPU's own layer input, the step's parts bitwise the whole step, greedy acceptance exact,
 and the state rollback across two steps of two lanes (the accepted path of the first step is what the second folds)."""

@@ -77,7 +77,7 @@ def test_moe_layer_matches_the_oracle(backend, config):
 
 
 def test_moe_layer_at_the_35b_shape(backend):
-    """Hidden 2048, 128 experts of FFN 768, top-8, eight lanes of sixteen rows (BASELINE config 5's MoE layer)."""
+    """Hidden 2048, 128 experts of FFN 768, top-8, eight lanes of sixteen rows (BASELINE.json config 5's MoE layer)."""
     print("case moe 35B shape", flush=True)
     rng = np.random.default_rng(9)
     moe, got, want = run_layer(backend, rng, 2048, 768, 128, 8, 128)

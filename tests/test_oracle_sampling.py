@@ -19,7 +19,7 @@ def test_argmax_brute_force_ties_and_unselectable():
 
 
 def walk(tree, tokens, selected, remaining, stops):
-    """An independent restatement of the acceptance walk, recursive on children."""
+    """An independent restatement of the acceptance walk (sampling.metal:2044-2083), recursive on children."""
     rows = len(tree)
     path = [0]
     while True:

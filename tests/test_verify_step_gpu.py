@@ -1,4 +1,4 @@
-"""End-to-end parity of the dense verify step (BASELINE config 1) against the oracle, through the C ABI."""
+"""End-to-end parity of the dense verify step (BASELINE.json config 1) against the oracle, through the C ABI."""
 import numpy as np
 import pytest
 
