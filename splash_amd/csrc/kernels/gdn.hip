@@ -11,11 +11,13 @@
 // the row's products with k and q are tree sums over the half's 32 lanes, and each token keeps
 // the decay, memory, delta, update, output order of gdn.metal:270-298.
 //
-// A block whose rows are not a chain (some row's parent is not the row before it) takes its rows'
-// outputs from the committed state instead (gdn.metal:417-478): with S_j the state after the j-th
-// token of a row's path, S_j z = S_j-1 (d_j (z - c k_j)) + c v_j for c = beta_j (k_j . z), so the
-// row's output is S_-1 z_-1 + sum_j c_j v_j; a wave per row walks its path upward for z_-1 and the
-// coefficients, and the recurrence's waves add the path terms to the state's product with z_-1.
+// The block's rows never advance the state: every row, of a chain block as of a tree block, takes its
+// output from the committed state (the reference does so for tree blocks, gdn.metal:417-478; a chain is
+// the tree whose every row follows the row before it): with S_j the state after the j-th token of a
+// row's path, S_j z = S_j-1 (d_j (z - c k_j)) + c v_j for c = beta_j (k_j . z), so the row's output is
+// S_-1 z_-1 + sum_j c_j v_j; a wave per row walks its path upward for z_-1 and the coefficients, and
+// the recurrence's waves add the path terms to the state's product with z_-1: one product with the
+// state a row instead of the four passes over it that advancing it takes.
 #include "abi/Gdn.h"
 #include "abi/PagedAttention.h"  // AttentionTreeRow
 #include "backend/KernelRegistry.hpp"
@@ -113,10 +115,10 @@ __device__ __forceinline__ History history_of(const uint16_t *carried, const uin
 }
 
 // One token's delta-rule step on the wave's state rows (R pairs, a row per half-wave): decay,
-// memory, delta, update and, with `query`, the row's output.
-template <int R, bool Output>
+// memory, delta, update (gdn.metal:270-298).
+template <int R>
 __device__ __forceinline__ void advance(float (&state)[R][4], const uint16_t *key, const uint16_t *value_row, const uint32_t (&value_dim)[R],
-                                        float decay, float beta, const uint16_t *query, float (&result)[R], uint32_t column) {
+                                        float decay, float beta, uint32_t column) {
   const uint2 kb = *reinterpret_cast<const uint2 *>(key + column);
   const float k[4] = {bf16_bits_to_float(kb.x & 0xFFFFu), bf16_bits_to_float(kb.x >> 16), bf16_bits_to_float(kb.y & 0xFFFFu),
                       bf16_bits_to_float(kb.y >> 16)};
@@ -131,24 +133,11 @@ __device__ __forceinline__ void advance(float (&state)[R][4], const uint16_t *ke
     }
     memory[r] = half_sum(memory[r]);
   }
-  float q[4] = {0.f, 0.f, 0.f, 0.f};
-  if constexpr (Output) {
-    const uint2 qb = *reinterpret_cast<const uint2 *>(query + column);
-    q[0] = bf16_bits_to_float(qb.x & 0xFFFFu);
-    q[1] = bf16_bits_to_float(qb.x >> 16);
-    q[2] = bf16_bits_to_float(qb.y & 0xFFFFu);
-    q[3] = bf16_bits_to_float(qb.y >> 16);
-  }
 #pragma unroll
   for (int r = 0; r < R; ++r) {
     const float delta = (bf16_bits_to_float(value_row[value_dim[r]]) - memory[r]) * beta;
-    result[r] = 0.f;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      state[r][i] += k[i] * delta;
-      if constexpr (Output) result[r] += state[r][i] * q[i];
-    }
-    if constexpr (Output) result[r] = half_sum(result[r]);
+    for (int i = 0; i < 4; ++i) state[r][i] += k[i] * delta;
   }
 }
 
@@ -286,10 +275,7 @@ __global__ __launch_bounds__(64 * kWaves) void gdn_decode(const uint16_t *__rest
   }
   __syncthreads();
 
-  // Every thread reads the same paths, so the branch on them is uniform.
-  bool chain = true;
-  for (uint32_t token = 0; token < rows; ++token) chain = chain && paths[token] == (2u << token) - 1u;
-  if (!chain) {
+  {
     // ---- tree rows: transformed queries and path coefficients, a wave per row ----
     const uint32_t j = lane & 31u, column = 4u * j;
     for (uint32_t token = wave; token < rows; token += kWaves) {
@@ -336,32 +322,27 @@ __global__ __launch_bounds__(64 * kWaves) void gdn_decode(const uint16_t *__rest
         state[r][3] = loaded.w;
       }
       for (uint32_t token = 0; token < pendingRows; ++token)
-        advance<kInFlight, false>(state, pending.keys[token], pending.values[token], valueDim, pending.decay[token],
-                                  bf16_bits_to_float(pending.beta[token]), nullptr, result, column);
+        advance<kInFlight>(state, pending.keys[token], pending.values[token], valueDim, pending.decay[token],
+                           bf16_bits_to_float(pending.beta[token]), column);
 #pragma unroll
       for (int r = 0; r < kInFlight; ++r)
         *reinterpret_cast<float4 *>(stateOut + (size_t(head) * kDim + valueDim[r]) * kDim + column) =
             make_float4(state[r][0], state[r][1], state[r][2], state[r][3]);
       for (uint32_t token = 0; token < rows; ++token) {
-        if (chain) {
-          advance<kInFlight, true>(state, keys[token], values[token], valueDim, decays[token], bf16_bits_to_float(betas[token]),
-                                   queries[token], result, column);
-        } else {
-          // The path's terms, a lane per block row, beside the committed state's product with the
-          // transformed query (gdn.metal:363-377).
-          const uint32_t j = lane & 31u, pathRowIndex = j & (kRows - 1u);
-          const bool onPath = j < kRows && ((paths[token] >> j) & 1u);
-          const float coefficient = coefficients[token][pathRowIndex];
-          const float4 zq = *reinterpret_cast<const float4 *>(&transformed[token][column]);
+        // The path's terms, a lane per block row, beside the committed state's product with the
+        // transformed query (gdn.metal:363-377).
+        const uint32_t j = lane & 31u, pathRowIndex = j & (kRows - 1u);
+        const bool onPath = j < kRows && ((paths[token] >> j) & 1u);
+        const float coefficient = coefficients[token][pathRowIndex];
+        const float4 zq = *reinterpret_cast<const float4 *>(&transformed[token][column]);
 #pragma unroll
-          for (int r = 0; r < kInFlight; ++r) {
-            result[r] = onPath ? coefficient * bf16_bits_to_float(values[pathRowIndex][valueDim[r]]) : 0.0f;
-            result[r] += state[r][0] * zq.x;
-            result[r] += state[r][1] * zq.y;
-            result[r] += state[r][2] * zq.z;
-            result[r] += state[r][3] * zq.w;
-            result[r] = half_sum(result[r]);
-          }
+        for (int r = 0; r < kInFlight; ++r) {
+          result[r] = onPath ? coefficient * bf16_bits_to_float(values[pathRowIndex][valueDim[r]]) : 0.0f;
+          result[r] += state[r][0] * zq.x;
+          result[r] += state[r][1] * zq.y;
+          result[r] += state[r][2] * zq.z;
+          result[r] += state[r][3] * zq.w;
+          result[r] = half_sum(result[r]);
         }
         if ((lane & 31u) == 0) {
 #pragma unroll
@@ -426,7 +407,7 @@ __global__ __launch_bounds__(64 * kWaves) void gdn_fold(uint8_t *__restrict__ st
   const uint32_t half = lane >> 5, column = 4u * (lane & 31u);
   for (uint32_t batch = 0; batch < kDim / (2u * kWaves); batch += kInFlight) {
     uint32_t valueDim[kInFlight];
-    float state[kInFlight][4], result[kInFlight];
+    float state[kInFlight][4];
 #pragma unroll
     for (int r = 0; r < kInFlight; ++r) {
       valueDim[r] = (batch + r) * 2u * kWaves + wave * 2u + half;
@@ -437,8 +418,8 @@ __global__ __launch_bounds__(64 * kWaves) void gdn_fold(uint8_t *__restrict__ st
       state[r][3] = loaded.w;
     }
     for (uint32_t token = 0; token < rows; ++token)
-      advance<kInFlight, false>(state, pending.keys[token], pending.values[token], valueDim, pending.decay[token],
-                                bf16_bits_to_float(pending.beta[token]), nullptr, result, column);
+      advance<kInFlight>(state, pending.keys[token], pending.values[token], valueDim, pending.decay[token],
+                         bf16_bits_to_float(pending.beta[token]), column);
 #pragma unroll
     for (int r = 0; r < kInFlight; ++r)
       *reinterpret_cast<float4 *>(stateOut + (size_t(head) * kDim + valueDim[r]) * kDim + column) =
