@@ -15,6 +15,9 @@
 #define MOE_MAXIMUM_TOP 16u
 #define MOE_TILE_ROWS 16u
 #define MOE_NO_ROW 0xFFFFFFFFu
+// Words of moe_group_routes' bit matrix, a row an expert and a bit a route: experts * ceil(routes / 32) at most
+// (128 experts of 4096 routes, 256 experts of 2048).
+#define MOE_GROUP_WORDS 16384u
 
 // The most tiles `routes` routes over `experts` experts can take.
 #if defined(__HIPCC__)
@@ -30,7 +33,7 @@ struct MoeRouteParams {
   uint32_t rows, experts, top_k;
   uint32_t score_stride;  // floats between rows of scores
 };
-// moe_group_routes: one workgroup of 256 threads.
+// moe_group_routes: one workgroup of 1024 threads.
 struct MoeGroupParams {
   uint32_t routes;  // rows * top_k
   uint32_t experts, top_k;

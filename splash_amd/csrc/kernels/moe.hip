@@ -53,83 +53,73 @@ __global__ __launch_bounds__(64) void moe_route_select(const float *__restrict__
 }
 SP_REGISTER_KERNEL("moe_route_select", &moe_route_select);
 
-// moe_group_routes: one workgroup of 1024 threads. Thread (expert e, part) walks its part of the
-// routes, four expert ids a word, for expert e's; an expert's routes take their slots in route order
-// (the parts in order, each part's routes in order), so the grouping never depends on timing.
+// moe_group_routes: one workgroup of 1024 threads, work in proportion to the routes. Every route sets its bit
+// in its expert's row of a bit matrix (an OR: whatever order the threads run in, the matrix is the same);
+// a thread per expert counts its row word by word, which gives the expert's routes before each word and its
+// tiles; a route's place among its expert's is then those before its word plus the set bits below its own, so
+// an expert's routes keep their route order and the grouping never depends on timing.
 __global__ __launch_bounds__(1024) void moe_group_routes(const uint32_t *__restrict__ selected, uint32_t *__restrict__ route_slot,
                                                          uint32_t *__restrict__ slot_row, uint32_t *__restrict__ tile_expert,
                                                          uint32_t *__restrict__ tile_rows, uint32_t *__restrict__ tile_total,
                                                          MoeGroupParams p) {
-  constexpr uint32_t kStaged = 256u * MOE_MAXIMUM_TOP;  // routes of a step: 256 rows of up to 16
-  __shared__ uint32_t partCount[1024];                  // [part][expert]: then the part's first place among the expert's routes
-  __shared__ uint32_t counts[MOE_MAXIMUM_EXPERTS], firstTile[MOE_MAXIMUM_EXPERTS], waveTiles[16];
-  __shared__ __align__(16) uint8_t staged[kStaged];     // expert ids fit a byte
+  __shared__ uint32_t masks[MOE_GROUP_WORDS];   // [expert][word]: bit b of word w: route 32 w + b is the expert's
+  __shared__ uint16_t before[MOE_GROUP_WORDS];  // [expert][word]: the expert's routes before word w
+  __shared__ uint32_t firstTile[MOE_MAXIMUM_EXPERTS], waveTiles[MOE_MAXIMUM_EXPERTS / 64u];
+  constexpr uint32_t kMine = 256u * MOE_MAXIMUM_TOP / 1024u;  // routes a thread may own
   const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
-  // Expert columns: the experts rounded up to a power of two; the threads left over split the routes.
-  uint32_t columns = 4;
-  while (columns < p.experts) columns <<= 1;
-  const uint32_t parts = 1024u / columns, e = tid & (columns - 1u), part = tid / columns;
+  const uint32_t words = (p.routes + 31u) / 32u;
+  for (uint32_t i = tid; i < p.experts * words; i += 1024u) masks[i] = 0u;
   for (uint32_t slot = tid; slot < p.maximum_tiles * MOE_TILE_ROWS; slot += 1024u) slot_row[slot] = MOE_NO_ROW;
-  for (uint32_t route = tid; route < p.routes; route += 1024u) staged[route] = uint8_t(selected[route]);
-  __syncthreads();
-  const uint32_t words = (p.routes + 3u) / 4u, perPart = (words + parts - 1u) / parts;
-  const uint32_t firstWord = min(words, part * perPart), lastWord = min(words, firstWord + perPart);
-  const uint32_t pattern = e * 0x01010101u;
-  auto matches = [&](uint32_t word) -> uint32_t {  // bit 8 i + 7: route 4 word + i is expert e's
-    const uint32_t x = reinterpret_cast<const uint32_t *>(staged)[word] ^ pattern;
-    uint32_t zero = ~(((x & 0x7F7F7F7Fu) + 0x7F7F7F7Fu) | x | 0x7F7F7F7Fu);  // 0x80 in each zero byte, exactly
-    const uint32_t live = p.routes - 4u * word;
-    return live >= 4u ? zero : zero & ((1u << (8u * live)) - 1u);
-  };
-  uint32_t count = 0;
-  if (e < p.experts)
-    for (uint32_t word = firstWord; word < lastWord; ++word) count += uint32_t(__builtin_popcount(matches(word)));
-  partCount[part * columns + e] = count;
-  __syncthreads();
-  // The expert's routes in all: its parts' counts become their first places.
-  uint32_t total = 0;
-  if (tid < columns) {
-    for (uint32_t q = 0; q < parts; ++q) {
-      const uint32_t c = partCount[q * columns + tid];
-      partCount[q * columns + tid] = total;
-      total += c;
-    }
-    counts[tid] = total;
+  uint32_t mine[kMine];
+#pragma unroll
+  for (uint32_t i = 0; i < kMine; ++i) {
+    const uint32_t route = tid + 1024u * i;
+    mine[i] = route < p.routes ? selected[route] : 0u;
   }
+  __syncthreads();
+#pragma unroll
+  for (uint32_t i = 0; i < kMine; ++i) {
+    const uint32_t route = tid + 1024u * i;
+    if (route < p.routes) atomicOr(&masks[mine[i] * words + route / 32u], 1u << (route % 32u));
+  }
+  __syncthreads();
+  // The expert's routes in all, and before each word of its row.
+  uint32_t total = 0;
+  if (tid < p.experts)
+    for (uint32_t w = 0; w < words; ++w) {
+      before[tid * words + w] = uint16_t(total);
+      total += uint32_t(__builtin_popcount(masks[tid * words + w]));
+    }
   // First tiles: an exclusive sum of the experts' tile counts, by waves and then over the waves' sums.
-  const uint32_t tiles = tid < columns ? (total + MOE_TILE_ROWS - 1u) / MOE_TILE_ROWS : 0u;
+  const uint32_t tiles = (total + MOE_TILE_ROWS - 1u) / MOE_TILE_ROWS;
   uint32_t running = tiles;
 #pragma unroll
   for (int o = 1; o < 64; o <<= 1) {
     const uint32_t up = uint32_t(__shfl_up(int(running), o, 64));
     if (lane >= uint32_t(o)) running += up;
   }
-  if (lane == 63u) waveTiles[wave] = running;
+  if (lane == 63u && tid < MOE_MAXIMUM_EXPERTS) waveTiles[wave] = running;
   __syncthreads();
-  if (tid < columns) {
-    uint32_t before = 0;
-    for (uint32_t w = 0; w < wave; ++w) before += waveTiles[w];
-    firstTile[tid] = before + running - tiles;
-    if (tid == columns - 1u) tile_total[0] = before + running;
+  if (tid < MOE_MAXIMUM_EXPERTS) {
+    uint32_t start = 0;
+    for (uint32_t w = 0; w < wave; ++w) start += waveTiles[w];
+    firstTile[tid] = start + running - tiles;
+    if (tid == MOE_MAXIMUM_EXPERTS - 1u) tile_total[0] = start + running;
     for (uint32_t t = 0; t < tiles; ++t) {
       tile_expert[firstTile[tid] + t] = tid;
       tile_rows[firstTile[tid] + t] = min(MOE_TILE_ROWS, total - t * MOE_TILE_ROWS);
     }
   }
   __syncthreads();
-  if (e >= p.experts || !count) return;
-  const uint32_t first = firstTile[e];
-  uint32_t placed = partCount[part * columns + e];
-  for (uint32_t word = firstWord; word < lastWord; ++word) {
-    uint32_t mask = matches(word);
-    while (mask) {
-      const uint32_t route = 4u * word + (uint32_t(__builtin_ctz(mask)) >> 3);
-      mask &= mask - 1u;
-      const uint32_t slot = (first + placed / MOE_TILE_ROWS) * MOE_TILE_ROWS + placed % MOE_TILE_ROWS;
-      route_slot[route] = slot;
-      slot_row[slot] = route / p.top_k;
-      ++placed;
-    }
+#pragma unroll
+  for (uint32_t i = 0; i < kMine; ++i) {
+    const uint32_t route = tid + 1024u * i;
+    if (route >= p.routes) continue;
+    const uint32_t at = mine[i] * words + route / 32u;
+    const uint32_t placed = before[at] + uint32_t(__builtin_popcount(masks[at] & ((1u << (route % 32u)) - 1u)));
+    const uint32_t slot = (firstTile[mine[i]] + placed / MOE_TILE_ROWS) * MOE_TILE_ROWS + placed % MOE_TILE_ROWS;
+    route_slot[route] = slot;
+    slot_row[slot] = route / p.top_k;
   }
 }
 SP_REGISTER_KERNEL("moe_group_routes", &moe_group_routes);

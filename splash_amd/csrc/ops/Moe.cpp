@@ -11,6 +11,9 @@ constexpr uint32_t kMaximumRows = 256;  // rows of a step: eight lanes of sixtee
 void requireShape(const MoeShape &shape, uint32_t rows) {
   if (!shape.valid()) throw std::invalid_argument("invalid MoE shape");
   if (!rows || rows > kMaximumRows) throw std::invalid_argument("a MoE step takes 1 to 256 rows");
+  // The grouping kernel's bit matrix, a row an expert and a bit a route, lives in one workgroup's LDS.
+  if (uint64_t{shape.experts} * ((uint64_t{rows} * shape.topK + 31) / 32) > MOE_GROUP_WORDS)
+    throw std::invalid_argument("too many experts for that many routes: experts * ceil(rows * top_k / 32) is at most 16384");
 }
 const char *formatName(uint32_t format) {
   if (format == GGUF_FMT_Q4K) return "q4k";
