@@ -182,12 +182,14 @@ typedef struct spo_gdn_decode_buffers { /* ops::GdnDecodeBuffers (GDN.hpp:122-15
   sp_buffer *packed, *convolution_weights, *states, *tape, *decay_weights, *time_bias, *mixer_norm, *hidden;
   uint32_t float_norm; /* the output norm's weights are fp32 */
   sp_buffer *tree_rows; /* the step's rows' places in their blocks (SplashTreeRow, 8 bytes a row) */
+  sp_buffer *hidden_table; /* optional (NULL: none): the hidden rows also as the activation table of the projection that
+                              reads them, spo_gguf_table_bytes(value_heads * 128, rows) bytes; that projection is added
+                              with `prepared` 1 and no table pass runs before it */
 } spo_gdn_decode_buffers;
 /* GDN::addDecode (GDN.hpp:184): the step of 1 to 8 lanes of one layer. The state a step writes is
  * the one BEFORE its rows (the lane's pending path folded in); its rows go to the lane's tape.
- * A lane whose rows are a chain runs the sequential recurrence; any other tree's rows each read the
- * state before the block along their own path (GDN.hpp:143-147), and every row's convolution reads
- * its path's tokens. */
+ * Every row, of a chain as of any other tree, reads the state before the block along its own path
+ * (GDN.hpp:143-147), and every row's convolution reads its path's tokens. */
 sp_status spo_gdn_add_decode(spo_graph *graph, const spo_gdn_decode_buffers *buffers, const spo_gdn_shape *shape, uint32_t layer,
                              const spo_gdn_state_strides *state, uint32_t tiled_heads, const spo_gdn_lane *lanes, uint32_t count);
 /* GDN::addFold (GDN.hpp:198): the state after the first `rows` rows of the path a lane retained of a

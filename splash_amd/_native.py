@@ -106,7 +106,7 @@ class GdnLane(ctypes.Structure):
 
 class GdnDecodeBuffers(ctypes.Structure):
     _fields_ = [(n, c_p) for n in ("packed", "convolution_weights", "states", "tape", "decay_weights", "time_bias", "mixer_norm",
-                                   "hidden")] + [("float_norm", c_u32), ("tree_rows", c_p)]
+                                   "hidden")] + [("float_norm", c_u32), ("tree_rows", c_p), ("hidden_table", c_p)]
 
 
 class MoeShape(ctypes.Structure):

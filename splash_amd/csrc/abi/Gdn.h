@@ -74,7 +74,8 @@ struct GdnDecodeParams {
   uint32_t flags;
   uint32_t layer;
   uint32_t lanes;
-  uint32_t reserved;
+  uint32_t table_tiles;  // nonzero: the hidden rows also leave as the activation table (abi/Gguf.h, pieces of 64 rows,
+                         // table_tiles row tiles in all) of the projection that reads them
   uint64_t conv_layer_bytes;
   uint64_t recurrent_layer_bytes;
   uint64_t convolution_state_bytes;

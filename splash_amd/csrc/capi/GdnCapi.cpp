@@ -42,7 +42,8 @@ sp_status spo_gdn_add_decode(spo_graph *graph, const spo_gdn_decode_buffers *b, 
   return capi::guard([&] {
     capi::require(graph && b && shape && state && lanes, "graph, buffers, shape, strides or lanes");
     ops::GdnDecodeBuffers buffers{B(b->packed), B(b->convolution_weights), B(b->states), B(b->tape), B(b->decay_weights),
-                                  B(b->time_bias), B(b->mixer_norm), b->float_norm != 0, B(b->hidden), B(b->tree_rows)};
+                                  B(b->time_bias), B(b->mixer_norm), b->float_norm != 0, B(b->hidden), B(b->tree_rows),
+                                  b->hidden_table ? B(b->hidden_table) : hip::Buffer{}};
     std::vector<ops::GdnLaneStep> list;
     for (uint32_t i = 0; i < count; ++i)
       list.push_back({lanes[i].first_row, lanes[i].rows, lanes[i].pending_path, lanes[i].pending_tape, lanes[i].step_tape,

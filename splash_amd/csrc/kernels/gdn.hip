@@ -19,6 +19,7 @@
 // the recurrence's waves add the path terms to the state's product with z_-1: one product with the
 // state a row instead of the four passes over it that advancing it takes.
 #include "abi/Gdn.h"
+#include "abi/Gguf.h"
 #include "abi/PagedAttention.h"  // AttentionTreeRow
 #include "backend/KernelRegistry.hpp"
 #include "kernels/device_common.hpp"
@@ -152,7 +153,8 @@ __global__ __launch_bounds__(64 * kWaves) void gdn_decode(const uint16_t *__rest
                                                   uint8_t *__restrict__ states, uint8_t *__restrict__ tape,
                                                   const float *__restrict__ a_scale, const uint16_t *__restrict__ dt_bias,
                                                   const void *__restrict__ norm_weight, uint16_t *__restrict__ hidden,
-                                                  const AttentionTreeRow *__restrict__ tree, GdnDecodeParams p) {
+                                                  const AttentionTreeRow *__restrict__ tree, uint8_t *__restrict__ table,
+                                                  GdnDecodeParams p) {
   __shared__ __align__(16) uint16_t queries[kRows][kDim], keys[kRows][kDim], values[kRows][kDim], outputs[kRows][kDim];
   __shared__ __align__(16) float transformed[kRows][kDim];
   __shared__ float coefficients[kRows][kRows];
@@ -368,7 +370,34 @@ __global__ __launch_bounds__(64 * kWaves) void gdn_decode(const uint16_t *__rest
       const float normalized = round_bf16((value[part] * inverse) * weight);
       const float z = bf16_bits_to_float(rowsIn[size_t(token) * P + zOffset + head * kDim + d]);
       const float gated = (normalized * ((p.flags & GDN_SIGMOID_GATE) ? 1.0f : z)) / (1.0f + exp2_fast(-kLog2e * z));
-      hidden[(size_t(L.first_row + token) * s.value_heads + outHead) * kDim + d] = uint16_t(float_to_bf16_bits(gated));
+      const uint32_t bits = float_to_bf16_bits(gated);
+      hidden[(size_t(L.first_row + token) * s.value_heads + outHead) * kDim + d] = uint16_t(bits);
+      outputs[token][d] = uint16_t(bits);  // this wave's row: read above, and below for the table
+    }
+    if (p.table_tiles) {
+      // The row's 128 values of this head as 32 runs of four inputs, a lane a run: the pieces, and the sums of 16
+      // and 32 inputs in input order, that gguf_prepare_table would write of the hidden rows.
+      const uint32_t packedRow = L.first_row + token, r = packedRow % 16u, width = s.value_heads * kDim, G = width / 32u;
+      const uint32_t piece = packedRow / 16u / GGUF_PIECE_TILES, tile = packedRow / 16u % GGUF_PIECE_TILES;
+      const uint32_t tiles = min(uint32_t(GGUF_PIECE_TILES), p.table_tiles - piece * GGUF_PIECE_TILES);
+      uint8_t *mine = table + piece * gguf_table_bytes(width, GGUF_PIECE_TILES);
+      const uint32_t run = lane & 31u, q = outHead * (kDim / 4u) + run, g = q / 8u, half = (q / 4u) % 2u, kq = q % 4u;
+      const uint2 raw = *reinterpret_cast<const uint2 *>(&outputs[token][4u * run]);
+      const uint32_t x0 = raw.x & 0xFFFFu, x1 = raw.x >> 16, x2 = raw.y & 0xFFFFu, x3 = raw.y >> 16;
+      float sum = (bf16_bits_to_float(x0) + bf16_bits_to_float(x1)) + (bf16_bits_to_float(x2) + bf16_bits_to_float(x3));
+      const float s1 = __shfl_down(sum, 1, 64), s2 = __shfl_down(sum, 2, 64), s3 = __shfl_down(sum, 3, 64);
+      sum = ((sum + s1) + s2) + s3;
+      const float other = __shfl_down(sum, 4, 64);
+      if (lane < 32u) {
+        // operand elements 4 half + {0,1,2,3} are inputs 4 kq + {0,2,1,3} of the half
+        reinterpret_cast<uint2 *>(mine)[((size_t(tile) * G + g) * 64u + kq * 16u + r) * 2u + half] = make_uint2(x0 | (x2 << 16), x1 | (x3 << 16));
+        if (kq == 0) {
+          float *sums32 = reinterpret_cast<float *>(mine + gguf_table_sums32_offset(width, tiles));
+          float *sums16 = reinterpret_cast<float *>(mine + gguf_table_sums16_offset(width, tiles));
+          sums16[(size_t(tile) * 2u * G + 2u * g + half) * 16u + r] = sum;
+          if (half == 0) sums32[(size_t(tile) * G + g) * 16u + r] = sum + other;
+        }
+      }
     }
   }
 }

@@ -500,17 +500,21 @@ __global__ __launch_bounds__(256) void attention_reduce(const _Float16 *__restri
     if (tid < D / 4u) {
       // Run q: inputs 4 q .. 4 q + 3 of the packed row (norm_rms_table16 writes the same pieces).
       const uint32_t width = p.q_heads * D, G = width / 32u, q = head * (D / 4u) + tid;
-      const uint32_t packed = seq.first_row + row, tile = packed / 16u, r = packed % 16u;
+      // Row tile packed / 16 is a tile of its 64-row piece's table, which holds `tiles` row tiles.
+      const uint32_t packed = seq.first_row + row, r = packed % 16u;
+      const uint32_t piece = packed / 16u / GGUF_PIECE_TILES, tile = packed / 16u % GGUF_PIECE_TILES;
+      const uint32_t tiles = min(uint32_t(GGUF_PIECE_TILES), p.table_tiles - piece * GGUF_PIECE_TILES);
+      uint8_t *mine = table + piece * gguf_table_bytes(width, GGUF_PIECE_TILES);
       const uint32_t x0 = staged[4 * tid], x1 = staged[4 * tid + 1], x2 = staged[4 * tid + 2], x3 = staged[4 * tid + 3];
       const uint32_t g = q / 8u, half = (q / 4u) % 2u, kq = q % 4u;
-      reinterpret_cast<uint2 *>(table)[((size_t(tile) * G + g) * 64u + kq * 16u + r) * 2u + half] = make_uint2(x0 | (x2 << 16), x1 | (x3 << 16));
+      reinterpret_cast<uint2 *>(mine)[((size_t(tile) * G + g) * 64u + kq * 16u + r) * 2u + half] = make_uint2(x0 | (x2 << 16), x1 | (x3 << 16));
       float s = (bf16_bits_to_float(x0) + bf16_bits_to_float(x1)) + (bf16_bits_to_float(x2) + bf16_bits_to_float(x3));
       const float s1 = __shfl_down(s, 1, 64), s2 = __shfl_down(s, 2, 64), s3 = __shfl_down(s, 3, 64);
       s = ((s + s1) + s2) + s3;
       const float other = __shfl_down(s, 4, 64);
       if (kq == 0) {
-        float *sums32 = reinterpret_cast<float *>(table + gguf_table_sums32_offset(width, p.table_tiles));
-        float *sums16 = reinterpret_cast<float *>(table + gguf_table_sums16_offset(width, p.table_tiles));
+        float *sums32 = reinterpret_cast<float *>(mine + gguf_table_sums32_offset(width, tiles));
+        float *sums16 = reinterpret_cast<float *>(mine + gguf_table_sums16_offset(width, tiles));
         sums16[(size_t(tile) * 2u * G + 2u * g + half) * 16u + r] = s;
         if (half == 0) sums32[(size_t(tile) * G + g) * 16u + r] = s + other;
       }

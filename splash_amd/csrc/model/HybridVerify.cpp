@@ -79,6 +79,7 @@ HybridVerify::HybridVerify(hip::Backend &backend, HybridDimensions d, uint32_t m
   scratch_.input = device(size.input, "linear table");
   scratch_.partials = device(size.partials, "linear partials");
   scratch_.counters = device(std::max<uint64_t>(size.counters, 4), "linear counters");
+  mixedTable_ = device(gguf_tables_bytes(std::max(d.attentionWidth(), d.gdnWidth()), gguf_row_tiles(pieceRows)), "mixer output table");
   const uint64_t fused = uint64_t{maxLanes} * d.kvHeads * (d.qHeads / std::max(1u, d.kvHeads)) * 16;
   attentionWorkspace_.queries = device(fused * d.headDimension * 2, "staged queries");
   attentionWorkspace_.querySums = device(fused * 4, "query sums");
@@ -160,7 +161,9 @@ void HybridVerify::encodeLayer(hip::CommandGraph &graph, uint32_t layer, const s
       w.router.inputSize != dims_.hidden)
     throw std::invalid_argument("the layer's projections do not fit the model");
 
-  // Mixer: hidden[1] = hidden[0] + out(mixer(in(norm(hidden[0])))).
+  // Mixer: hidden[1] = hidden[0] + out(mixer(in(norm(hidden[0])))). With one piece of rows the mixer's last kernel
+  // writes its output rows' activation table beside them.
+  const bool mixerTable = rows <= kProjectionRows;
   forRowPieces(rows, [&](uint32_t first, uint32_t count) {
     const hip::Buffer normalized = rowsOf(normalized_, first, count, hiddenBytes);
     ops::LinearBuffers in;
@@ -177,7 +180,7 @@ void HybridVerify::encodeLayer(hip::CommandGraph &graph, uint32_t layer, const s
     const ops::AttentionPlan plan = planOf(lanes);
     const ops::KvPages pages{pageTable_, kvPools_.at(index), pageBytes_};
     ops::PagedAttention::addProjection(graph, plan, {packed_, w.queryNorm, w.keyNorm, ropeCos_, ropeSin_}, attentionWorkspace_, pages);
-    ops::PagedAttention::addAttention(graph, plan, attentionWorkspace_, treeRows_, pages, mixed_, {}, packed_);
+    ops::PagedAttention::addAttention(graph, plan, attentionWorkspace_, treeRows_, pages, mixed_, mixerTable ? mixedTable_ : hip::Buffer{}, packed_);
   } else {
     std::vector<ops::GdnLaneStep> steps;
     uint32_t firstRow = 0;
@@ -187,12 +190,21 @@ void HybridVerify::encodeLayer(hip::CommandGraph &graph, uint32_t layer, const s
                        tapeOffset(uint32_t(i), lane.parity, index), cellOffset(uint32_t(i), lane.parity), cellOffset(uint32_t(i), lane.parity ^ 1u)});
       firstRow += lane.block.rows;
     }
-    ops::GdnDecodeBuffers buffers{packed_, w.convolutionWeights, states_, tape_, w.decay, w.timeBias, w.mixerNorm, false, mixed_, treeRows_};
+    ops::GdnDecodeBuffers buffers{packed_, w.convolutionWeights, states_, tape_, w.decay, w.timeBias, w.mixerNorm, false, mixed_, treeRows_,
+                                  mixerTable ? mixedTable_ : hip::Buffer{}};
     ops::GDN::addDecode(graph, buffers, dims_.gdnShape(), index, strides_, ops::GdnHeadOrder::Grouped, steps);
   }
   forRowPieces(rows, [&](uint32_t first, uint32_t count) {
-    linear_.addResidualProjection(graph, rowsOf(mixed_, first, count, uint64_t{mixedWidth} * 2), w.mixerOutput,
-                                  rowsOf(residual, first, count, hiddenBytes), rowsOf(next, first, count, hiddenBytes), count, scratch_);
+    ops::LinearBuffers out;
+    out.input = rowsOf(mixed_, first, count, uint64_t{mixedWidth} * 2);
+    out.output = rowsOf(next, first, count, hiddenBytes);
+    out.residual = rowsOf(residual, first, count, hiddenBytes);
+    out.scratch = scratch_;
+    if (mixerTable) {  // the mixer wrote the table of its output rows
+      out.scratch.input = mixedTable_;
+      out.prepared = {out.input, ops::LinearInput::Table16};
+    }
+    linear_.add(graph, out, w.mixerOutput, linear_.plan(w.mixerOutput, count, ops::LinearEpilogue::Residual));
   });
 
   // FFN: hidden[0] = hidden[1] + sum over a row's experts of weight * expert(norm(hidden[1])).

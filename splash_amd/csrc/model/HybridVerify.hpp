@@ -146,6 +146,7 @@ private:
   ops::GdnStateStrides strides_;
   hip::Buffer kvAll_, states_, tape_;
   hip::Buffer hidden_[2], normalized_, packed_, mixed_, scores_, logits_, draft_;
+  hip::Buffer mixedTable_;  // the activation table of the mixer's output rows, written by the mixer's last kernel
   hip::Buffer inverseFrequency_, ropeCos_, ropeSin_;
   hip::Buffer inputTokens_, treeRows_, depths_, uniforms_, tokens_, retained_, acceptedCount_, retainedRows_;
   hip::Buffer pageTable_;

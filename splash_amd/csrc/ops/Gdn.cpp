@@ -1,4 +1,5 @@
 #include "ops/Gdn.hpp"
+#include "abi/Gguf.h"
 #include "abi/PagedAttention.h"  // AttentionTreeRow
 #include "ops/Linear.hpp"  // requireBytes
 
@@ -62,7 +63,13 @@ void GDN::addDecode(hip::CommandGraph &graph, const GdnDecodeBuffers &b, const G
   requireBytes(b.mixerNorm, uint64_t{GDN_HEAD_DIMENSION} * (b.floatNorm ? 4 : 2), "GDN output norm");
   requireBytes(b.hidden, uint64_t{rows} * shape.valueHeads * GDN_HEAD_DIMENSION * 2, "GDN hidden rows");
   requireBytes(b.tree, uint64_t{rows} * sizeof(AttentionTreeRow), "GDN tree rows");
-  graph.add("gdn_decode", {b.packed, b.convolutionWeights, b.states, b.tape, b.decayWeights, b.timeBias, b.mixerNorm, b.hidden, b.tree},
+  if (b.hiddenTable) {
+    requireBytes(b.hiddenTable, gguf_tables_bytes(shape.valueHeads * GDN_HEAD_DIMENSION, gguf_row_tiles(rows)), "GDN hidden table");
+    params.table_tiles = gguf_row_tiles(rows);
+  }
+  graph.add("gdn_decode",
+            {b.packed, b.convolutionWeights, b.states, b.tape, b.decayWeights, b.timeBias, b.mixerNorm, b.hidden, b.tree,
+             b.hiddenTable ? b.hiddenTable : b.hidden},
             params,
             {shape.valueHeads, uint32_t(lanes.size()), 1}, {1024, 1, 1});
 }

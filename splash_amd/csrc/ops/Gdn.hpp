@@ -55,10 +55,12 @@ struct GdnDecodeBuffers final {
   hip::Buffer mixerNorm;           // bf16 or fp32 [128]
   bool floatNorm = false;
   hip::Buffer hidden;              // bf16 [rows][valueHeads * 128]
-  // The step's rows' places in their blocks' trees (AttentionTreeRow, a row each): a chain's rows
-  // run the sequential recurrence, another tree's rows each read the state before the block along
-  // their own path, and every row's convolution reads its path's tokens (GDN.hpp:143-147).
+  // The step's rows' places in their blocks' trees (AttentionTreeRow, a row each): every row reads the
+  // state before the block along its own path, and its convolution reads its path's tokens (GDN.hpp:143-147).
   hip::Buffer tree;
+  // Optional: the hidden rows also leave as the activation table (gguf_tables_bytes(valueHeads * 128, row tiles)) of
+  // the projection that reads them, so no table pass runs before it.
+  hip::Buffer hiddenTable{};
 };
 struct GdnFoldBuffers final {
   hip::Buffer states;

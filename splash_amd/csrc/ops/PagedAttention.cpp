@@ -132,9 +132,8 @@ void PagedAttention::addAttention(hip::CommandGraph &graph, const AttentionPlan 
   const uint32_t width = g.qHeads * g.headDimension;
   if (outputTable) {
     if (width % GGUF_BLOCK) throw std::invalid_argument("an attention output table holds whole super-blocks");
-    if (rows > GGUF_MAXIMUM_ROWS) throw std::invalid_argument("the attention merge writes the table of up to 64 rows");
     params.table_tiles = gguf_row_tiles(rows);
-    requireBytes(outputTable, gguf_table_bytes(width, params.table_tiles), "attention output table");
+    requireBytes(outputTable, gguf_tables_bytes(width, params.table_tiles), "attention output table");
   }
   graph.add("attention_q8_split" + kernelSuffix(g) + "_g" + std::to_string(g.group()),
             {w.queries, w.querySums, treeRows, pages.pageTable, pages.pool, w.partials, w.partialSums}, params,

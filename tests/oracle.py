@@ -326,6 +326,23 @@ def split_activation_table(raw_bytes, K, tiles):
     return values, s32, s16
 
 
+def assert_table_holds(raw_bytes, x_bits, piece_bytes):
+    """A downloaded activation table equals the one the bf16 rows x_bits [M][K] define, piece by piece of 64 rows;
+    piece_bytes(rows) is a piece's size. Rows of a tile past M are not compared: a writer of live rows leaves them."""
+    M, K = x_bits.shape
+    at = 0
+    for first in range(0, M, 64):
+        count = min(64, M - first)
+        tiles = (count + 15) // 16
+        size = piece_bytes(count)
+        values, s32, s16 = split_activation_table(raw_bytes[at:at + size], K, tiles)
+        wv, w32, w16 = activation_table(x_bits[first:first + count])
+        assert np.array_equal(table_rows(values, K, tiles)[:count], table_rows(wv, K, tiles)[:count])
+        live = lambda sums: sums.transpose(0, 2, 1).reshape(tiles * 16, -1)[:count]
+        assert live(s32).tobytes() == live(w32).tobytes() and live(s16).tobytes() == live(w16).tobytes()
+        at += size
+
+
 # ---- Gated DeltaNet ----
 class GdnShape(ctypes.Structure):
     _fields_ = [("key_heads", c_u32), ("value_heads", c_u32), ("conv_dim", c_u32), ("packed_width", c_u32), ("flags", c_u32)]

@@ -188,11 +188,43 @@ def test_attention_output_table(backend, rows, committed):
         backend.run(graph)
         outs.append(out.download(np.uint16).reshape(rows, width))
     assert np.array_equal(outs[0], outs[1])
-    values, s32, s16 = orc.split_activation_table(table.download(np.uint8), width, 1)
-    wv, w32, w16 = orc.activation_table(outs[1])
-    live = np.arange(64) % 16 < rows   # rows of the tile past the block keep what the table held (zeros here)
-    assert np.array_equal(values[:, :, live], wv[:, :, live])
-    assert s32[..., :rows].tobytes() == w32[..., :rows].tobytes() and s16[..., :rows].tobytes() == w16[..., :rows].tobytes()
+    orc.assert_table_holds(table.download(np.uint8), outs[1], lambda count: ops.gguf_table_bytes(width, count))
+
+
+def test_attention_output_table_in_pieces(backend):
+    """More than 64 rows over several sequences: the table is written piece by piece of 64 rows, and a sequence
+    whose rows straddle two pieces lands in both."""
+    print("case attention output table pieces", flush=True)
+    rng = np.random.default_rng(78)
+    q_heads, kv_heads, D = 16, 8, 64
+    seqs = [(16, 200), (16, 64), (16, 900), (9, 130), (16, 10), (14, 300)]   # 87 rows: 64 + 23, the fifth straddles
+    PT = ops.PAGE_TOKENS
+    pages = [(c + r + PT - 1) // PT for r, c in seqs]
+    phys = sum(pages) + 1
+    perm = rng.permutation(phys)[:sum(pages)]
+    codes = lambda: rng.integers(-127, 128, (phys, kv_heads, PT, D)).astype(np.int8)
+    scales = lambda: rng.uniform(0.002, 0.02, (phys, kv_heads, PT)).astype(np.float32)
+    kv = ops.KvPages(backend, kv_heads, D, phys, perm)
+    kv.upload(kv.pack_pages(codes(), scales(), codes(), scales()))
+    total = sum(r for r, _ in seqs)
+    width = q_heads * D
+    qkv = backend.from_array(orc.f32_to_bf16(rng.standard_normal((total, (q_heads + 2 * kv_heads) * D)).astype(np.float32)))
+    batch, first, table_first = [], 0, 0
+    for (r, c), n in zip(seqs, pages):
+        batch.append((first, r, c, table_first))
+        first += r
+        table_first += n
+    plan = ops.AttentionPlan(q_heads, kv_heads, D, batch)
+    ws = ops.AttentionWorkspace(backend, plan)
+    tree = backend.from_array(ops.chain_tree_rows([r for r, _ in seqs]))
+    out = backend.allocate_buffer(total * width * 2)
+    table = backend.allocate_buffer(ops.gguf_table_bytes(width, total))
+    graph = splash_amd.CommandGraph()
+    ops.PagedAttention.add_projection(graph, plan, qkv, ws, kv)
+    ops.PagedAttention.add_attention(graph, plan, ws, tree, kv, out, output_table=table)
+    backend.run(graph)
+    orc.assert_table_holds(table.download(np.uint8), out.download(np.uint16).reshape(total, width),
+                           lambda count: ops.gguf_table_bytes(width, count))
 
 
 @pytest.mark.parametrize("geometry", [(32, 4, 128), (16, 8, 64)])

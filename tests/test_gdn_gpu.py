@@ -62,11 +62,16 @@ class Layer:
                               step_tape=self.slot(lane, parity, layer), current_cell=self.cell(lane, cur), next_cell=self.cell(lane, nxt)))
             first += block.shape[0]
         graph = splash_amd.CommandGraph()
+        width = self.shape.value_heads * 128
+        table = self.backend.allocate_buffer(ops.gguf_table_bytes(width, rows))
         buffers = dict(packed=self.backend.from_array(packed), states=self.states, tape=self.tape, hidden=hidden,
-                       tree_rows=self.backend.from_array(tree), **self.weights)
+                       tree_rows=self.backend.from_array(tree), hidden_table=table, **self.weights)
         self.gdn.add_decode(graph, buffers, layer, lanes, float_norm=self.float_norm)
         self.backend.run(graph)
-        out = hidden.download(np.uint16).reshape(rows, self.shape.value_heads * 128)
+        out = hidden.download(np.uint16).reshape(rows, width)
+        # the hidden rows also left as the activation table of the projection that reads them: bit for bit the table
+        # pass's, piece by piece of 64 rows (rows of a tile past the step's keep what the buffer held)
+        orc.assert_table_holds(table.download(np.uint8), out, lambda count: ops.gguf_table_bytes(width, count))
         return [out[l["first_row"]:l["first_row"] + l["rows"]] for l in lanes]
 
 
