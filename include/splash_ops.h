@@ -41,7 +41,10 @@ sp_status spo_gguf_unpack_image(uint32_t format, const uint8_t *image, uint32_t 
 sp_status spo_gguf_add_dequant(spo_graph *graph, uint32_t format, sp_buffer *image, sp_buffer *out, uint32_t rows,
                                uint32_t input_size);
 
-/* ---- Projection (Weights.hpp:170-186): segments tile the leading output columns in order ---- */
+/* ---- Projection (Weights.hpp:170-186): segments tile the leading output columns in order. Segments may differ
+ *      in format, as the reference's fused q|k|v takes a format per segment (gguf_linear.metal:237-261,
+ *      LinearGguf.cpp:78-96): such a projection runs as one dispatch of a kernel that holds every format, under a
+ *      plain bf16 plan (no epilogue, whole_groups 0), each segment a multiple of 64 columns. ---- */
 sp_status spo_projection_create(uint32_t segments, const uint32_t *formats, const uint32_t *output_sizes,
                                 uint32_t input_size, sp_buffer *const *images, int float32_destination,
                                 spo_projection **out);

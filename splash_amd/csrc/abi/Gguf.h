@@ -170,6 +170,8 @@ struct GgufPrepareParams {
 // dispatch (the reference's GgufDecodeFusedParams, runtime/metal/abi/Gguf.h:168-178), tiles in
 // segment order; a single tensor is one segment. A gate/up pair binds gate as segment 0 and up as
 // segment 1, both of cols[0] columns. Grid (whole_groups + (groups - whole_groups) * splits), 256 threads: a wave per unit.
+// gguf_decode_mixed_m<16|32|64>_a: segments of different formats (formats[]), each whole workgroups
+// (multiples of 64 columns), whole_groups 0: grid groups * splits.
 struct GgufDecodeParams {
   uint32_t input_size;  // K
   uint32_t rows;        // live rows
@@ -182,7 +184,7 @@ struct GgufDecodeParams {
   // Nonzero: the table's rows lack their RMS scale; every sum is multiplied by
   // 1 / sqrt(sum of the row's squares entries / K + 1e-6) before the epilogue.
   uint32_t deferred_scale;
-  uint32_t reserved[3];
+  uint32_t formats[3];  // gguf_decode_mixed_*: each segment's format; the kernels of one format leave it zero
 };
 
 // gguf_dequant_<fmt>: the image's fp32 values [N][K], for the bit-exactness test

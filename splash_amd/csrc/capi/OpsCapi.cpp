@@ -18,9 +18,8 @@ ops::LinearPlan toPlan(const ops::Projection &projection, const spo_linear_plan 
   ops::LinearConfig config;
   config.splits = p.splits;
   config.wholeGroups = p.whole_groups;
-  return ops::Linear::plan(ops::LinearWorkload{{projection.outputSize, projection.inputSize}, p.rows,
-                                               static_cast<ops::LinearEpilogue>(p.epilogue)},
-                           config, p.float32 ? ops::FloatOutput::Float32 : ops::FloatOutput::BFloat16);
+  return ops::Linear::plan(ops::workloadOf(projection, p.rows, static_cast<ops::LinearEpilogue>(p.epilogue)), config,
+                           p.float32 ? ops::FloatOutput::Float32 : ops::FloatOutput::BFloat16);
 }
 void fromPlan(const ops::LinearPlan &plan, spo_linear_plan *out) {
   const ops::LinearScratchSize size = plan.scratchSize();

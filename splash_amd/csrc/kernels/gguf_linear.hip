@@ -418,12 +418,20 @@ __device__ __forceinline__ void accumulate_record(const Record<FMT> &rec, const 
 // is tile u of its concatenated segments; of a gate/up pair, unit 2 j is gate tile j and unit
 // 2 j + 1 up tile j, so the two halves of a pair sit in neighbouring waves of one workgroup.
 // `item` is the workgroup's place in the dispatch (blockIdx.x of gguf_decode).
+// A workgroup's LDS, which the kernel declares once whatever formats its workgroups decode.
+template <int RT> struct DecodeShared {
+  uint4 a[2][RT][8][64];
+  float sums[2][RT][4][64];
+  uint32_t arrived;
+  float scaleParts[256], rowScale[16 * RT];  // of a table with a deferred scale
+};
+
 template <uint32_t FMT, int RT, uint32_t EP>
-__device__ __forceinline__ void decode_workgroup(const uint8_t *__restrict__ seg0, const uint8_t *__restrict__ seg1,
-                                                 const uint8_t *__restrict__ seg2, const uint8_t *__restrict__ table,
-                                                 void *__restrict__ out, const uint16_t *__restrict__ residual,
-                                                 float *__restrict__ partials, uint32_t *__restrict__ counters,
-                                                 const GgufDecodeParams &p, const uint32_t item) {
+__device__ __forceinline__ void decode_workgroup(DecodeShared<RT> &shared, const uint8_t *__restrict__ seg0,
+                                                 const uint8_t *__restrict__ seg1, const uint8_t *__restrict__ seg2,
+                                                 const uint8_t *__restrict__ table, void *__restrict__ out,
+                                                 const uint16_t *__restrict__ residual, float *__restrict__ partials,
+                                                 uint32_t *__restrict__ counters, const GgufDecodeParams &p, const uint32_t item) {
   constexpr uint32_t kRecord = gguf_record_bytes(FMT);
   constexpr bool kTable = EP == GGUF_EPILOGUE_GATE_UP_TABLE, kGateUp = EP == GGUF_EPILOGUE_GATE_UP || kTable;
   constexpr uint32_t kColumnPart = Cursor<FMT>::kColumnPart;
@@ -432,10 +440,11 @@ __device__ __forceinline__ void decode_workgroup(const uint8_t *__restrict__ seg
   // The range's activations pass through LDS one super-block at a time (two buffers, one barrier
   // per super-block), each wave fetching a quarter of them, so a wave's vector-memory queue holds
   // almost only weights and the MFMA operands arrive on the LDS counter instead.
-  __shared__ uint4 ldsA[2][RT][8][64];
-  __shared__ float ldsSums[2][RT][4][64];
-  __shared__ uint32_t arrived;
-  __shared__ float scaleParts[256], rowScale[16 * RT];  // of a table with a deferred scale
+  auto &ldsA = shared.a;
+  auto &ldsSums = shared.sums;
+  uint32_t &arrived = shared.arrived;
+  auto &scaleParts = shared.scaleParts;
+  auto &rowScale = shared.rowScale;
 
   const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6, c = lane & 15u, kq = lane >> 4;
   // Workgroup items: the whole groups first, then the partitioned ones part by part.
@@ -794,8 +803,69 @@ __global__ __launch_bounds__(256) void gguf_decode(const uint8_t *__restrict__ s
     p.rows -= first;
   }
   p.rows = min(p.rows, uint32_t(GGUF_MAXIMUM_ROWS));
-  decode_workgroup<FMT, RT, EP>(seg0, seg1, seg2, table, out, residual, partials, counters, p, blockIdx.x);
+  __shared__ DecodeShared<RT> shared;
+  decode_workgroup<FMT, RT, EP>(shared, seg0, seg1, seg2, table, out, residual, partials, counters, p, blockIdx.x);
 }
+
+// Segments of different formats in one dispatch (the reference's fused projection takes a format per segment,
+// gguf_linear.metal:237-261): p.formats names each segment's. Segments hold whole workgroups (multiples of 64
+// columns), every workgroup takes one of p.splits parts of K (whole_groups 0), and a workgroup runs its segment's
+// format as a projection of that segment alone, its partials and counters after those of the segments before it.
+template <int RT>
+__global__ __launch_bounds__(256) void gguf_decode_mixed(const uint8_t *__restrict__ seg0, const uint8_t *__restrict__ seg1,
+                                                         const uint8_t *__restrict__ seg2, const uint8_t *__restrict__ table,
+                                                         void *__restrict__ out, const uint16_t *__restrict__ residual,
+                                                         float *__restrict__ partials, uint32_t *__restrict__ counters,
+                                                         GgufDecodeParams p) {
+  constexpr uint32_t kGroupFloats = 4u * RT * 256u;  // a workgroup's partials of one part
+  const uint32_t groups = p.units / 4u;
+  if (const uint32_t piece = blockIdx.y) {
+    const uint32_t first = piece * GGUF_MAXIMUM_ROWS;
+    table += piece * gguf_table_bytes(p.input_size, GGUF_PIECE_TILES);
+    out = static_cast<uint8_t *>(out) + size_t(first) * p.out_stride * 2u;
+    partials += size_t(piece) * p.splits * groups * kGroupFloats;
+    counters += piece * groups;
+    p.rows -= first;
+  }
+  p.rows = min(p.rows, uint32_t(GGUF_MAXIMUM_ROWS));
+  const uint32_t group = blockIdx.x / p.splits, split = blockIdx.x % p.splits;
+  uint32_t segment = 0, before = 0;
+#pragma unroll
+  for (uint32_t s = 0; s < 2u; ++s)
+    if (segment == s && group >= before + p.cols[s] / 64u) {
+      before += p.cols[s] / 64u;
+      segment = s + 1u;
+    }
+  const uint8_t *image = segment == 0 ? seg0 : segment == 1 ? seg1 : seg2;
+  GgufDecodeParams mine = p;
+  mine.cols[0] = p.cols[segment];
+  mine.cols[1] = mine.cols[2] = 0;
+  mine.offset[0] = p.offset[segment];
+  mine.units = p.cols[segment] / GGUF_TILE_COLUMNS;
+  mine.whole_groups = 0;
+  partials += size_t(before) * p.splits * kGroupFloats;
+  counters += before;
+  const uint32_t item = (group - before) * p.splits + split;
+  __shared__ DecodeShared<RT> shared;
+  switch (p.formats[segment]) {
+  case GGUF_FMT_Q4K:
+    decode_workgroup<GGUF_FMT_Q4K, RT, GGUF_EPILOGUE_PLAIN>(shared, image, image, image, table, out, residual, partials, counters, mine, item);
+    break;
+  case GGUF_FMT_Q5K:
+    decode_workgroup<GGUF_FMT_Q5K, RT, GGUF_EPILOGUE_PLAIN>(shared, image, image, image, table, out, residual, partials, counters, mine, item);
+    break;
+  case GGUF_FMT_Q6K:
+    decode_workgroup<GGUF_FMT_Q6K, RT, GGUF_EPILOGUE_PLAIN>(shared, image, image, image, table, out, residual, partials, counters, mine, item);
+    break;
+  case GGUF_FMT_Q80:
+    decode_workgroup<GGUF_FMT_Q80, RT, GGUF_EPILOGUE_PLAIN>(shared, image, image, image, table, out, residual, partials, counters, mine, item);
+    break;
+  default: break;
+  }
+}
+SP_REGISTER_KERNEL("gguf_decode_mixed_m16_a", &gguf_decode_mixed<1>);
+SP_REGISTER_KERNEL("gguf_decode_mixed_m32_a", &gguf_decode_mixed<2>);
+SP_REGISTER_KERNEL("gguf_decode_mixed_m64_a", &gguf_decode_mixed<4>);
 
 // The routed experts of a mixture-of-experts layer (the reference's moe_expert_gguf_*, abi/MoE.h):
 // grid (workgroups of one expert projection, tile slots). Tile t holds up to 16 rows routed to
@@ -813,7 +883,8 @@ __global__ __launch_bounds__(256) void gguf_moe_decode(const uint8_t *__restrict
   const uint32_t expert = tile_expert[tile];
   GgufDecodeParams p = m.decode;
   p.rows = tile_rows[tile];
-  decode_workgroup<FMT, 1, EP>(seg0 + expert * m.expert_bytes, seg1 + expert * m.expert_bytes, seg0 + expert * m.expert_bytes,
+  __shared__ DecodeShared<1> shared;
+  decode_workgroup<FMT, 1, EP>(shared, seg0 + expert * m.expert_bytes, seg1 + expert * m.expert_bytes, seg0 + expert * m.expert_bytes,
                                tables + tile * m.table_bytes, out + size_t(tile) * 16u * m.out_row_bytes,
                                reinterpret_cast<const uint16_t *>(next_tables + tile * m.next_table_bytes), nullptr, nullptr, p,
                                blockIdx.x);

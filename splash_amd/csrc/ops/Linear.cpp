@@ -39,8 +39,6 @@ void requireSegments(const Projection &p, LinearMatrix matrix) {
   if (segments.empty() || segments.size() > GGUF_MAXIMUM_SEGMENTS)
     throw std::invalid_argument("a block projection dispatch takes one to three segments");
   for (const QuantizedSegment &s : segments) {
-    if (s.formatId != segments.front().formatId)
-      throw std::invalid_argument("the segments of one block dispatch share a format");
     if (s.outputSize % GGUF_TILE_COLUMNS || s.inputSize % GGUF_BLOCK)
       throw std::invalid_argument("block segments hold whole 16-column tiles of whole 256-input super-blocks");
     requireBytes(s.image, gguf_image_bytes(s.formatId, s.outputSize, s.inputSize), "block weight image");
@@ -48,6 +46,17 @@ void requireSegments(const Projection &p, LinearMatrix matrix) {
 }
 
 } // namespace
+
+LinearWorkload workloadOf(const Projection &projection, uint32_t rows, LinearEpilogue epilogue) {
+  LinearWorkload w{{projection.outputSize, projection.inputSize}, rows, epilogue};
+  const std::vector<QuantizedSegment> &segments = projection.blocks().segments;
+  if (!segments.empty()) w.formatId = segments.front().formatId;
+  for (const QuantizedSegment &s : segments) {
+    w.severalFormats |= s.formatId != segments.front().formatId;
+    if (gguf_record_bytes(s.formatId) > gguf_record_bytes(w.formatId)) w.formatId = s.formatId;
+  }
+  return w;
+}
 
 LinearPlan::LinearPlan(LinearWorkload workload, LinearConfig config, FloatOutput destination)
     : workload_(workload), config_(config), destination_(destination) {
@@ -66,6 +75,9 @@ void LinearPlan::requireConfiguration() const {
   if (c.wholeGroups > groupsOf(n, workload_.epilogue)) throw std::invalid_argument("more whole workgroups than the projection has");
   if (destination_ == FloatOutput::Float32 && workload_.epilogue != LinearEpilogue::None)
     throw std::invalid_argument("only a plain block plan writes fp32");
+  if (workload_.severalFormats &&
+      (workload_.epilogue != LinearEpilogue::None || destination_ != FloatOutput::BFloat16 || c.wholeGroups || n % 64))
+    throw std::invalid_argument("segments of several formats take a plain bf16 plan whose workgroups all partition K");
 }
 
 LinearScratchSize LinearPlan::scratchSize() const noexcept {
@@ -108,7 +120,7 @@ LinearPlan Linear::plan(LinearWorkload w, FloatOutput destination) const {
   if (groups * most * 4 < calibration_.computeUnits) most = std::min(LinearConfig::kMaximumSplits, blocks);
   LinearConfig config;
   const uint32_t units = calibration_.computeUnits;
-  if (groups >= 2 * units && groups % units) {
+  if (!w.severalFormats && groups >= 2 * units && groups % units) {
     // Enough workgroups to fill the device without partitioning, but a remainder that would leave
     // most units idle at the end: the whole rounds run unsplit and the remainder is partitioned
     // into about one piece per unit, dispatched last.
@@ -123,10 +135,7 @@ LinearPlan Linear::plan(LinearWorkload w, FloatOutput destination) const {
 }
 
 LinearPlan Linear::plan(const Projection &projection, uint32_t rows, LinearEpilogue epilogue) const {
-  // A dispatch's segments share one format (requireSegments).
-  const uint32_t format = projection.blocks().segments.empty() ? GGUF_FMT_Q4K : projection.blocks().segments.front().formatId;
-  return plan(LinearWorkload{{projection.outputSize, projection.inputSize}, rows, epilogue, format},
-              epilogue == LinearEpilogue::None ? projection.destination : FloatOutput::BFloat16);
+  return plan(workloadOf(projection, rows, epilogue), epilogue == LinearEpilogue::None ? projection.destination : FloatOutput::BFloat16);
 }
 
 LinearScratchSize Linear::scratchSize(LinearMatrix matrix, uint32_t rows) const {
@@ -135,6 +144,10 @@ LinearScratchSize Linear::scratchSize(LinearMatrix matrix, uint32_t rows) const 
     size.include(plan(LinearWorkload{matrix, rows, e}).scratchSize());
   if (matrix.outputSize % GGUF_BLOCK == 0)
     size.include(plan(LinearWorkload{matrix, rows, LinearEpilogue::ResidualNorm}).scratchSize());
+  // segments of several formats partition every workgroup, however many the matrix has
+  if (matrix.outputSize % 64 == 0)
+    for (uint32_t format : {GGUF_FMT_Q4K, GGUF_FMT_Q6K})
+      size.include(plan(LinearWorkload{matrix, rows, LinearEpilogue::None, format, true}).scratchSize());
   return size;
 }
 
@@ -156,6 +169,11 @@ PreparedInput Linear::add(hip::CommandGraph &graph, LinearBuffers b, const Proje
   const auto [n, k] = w.matrix;
   // Everything is checked before anything is added.
   requireSegments(p, w.matrix);
+  const bool mixed = workloadOf(p, w.rows, w.epilogue).severalFormats;
+  if (mixed != w.severalFormats) throw std::invalid_argument("the plan is not of this projection's formats");
+  if (mixed)
+    for (const QuantizedSegment &s : p.blocks().segments)
+      if (s.outputSize % 64) throw std::invalid_argument("segments of several formats hold whole 64-column workgroups");
   const bool gateUp = w.epilogue == LinearEpilogue::GateUp;
   if (gateUp != (gate != nullptr)) throw std::invalid_argument("a block gate/up plan takes a gate projection, no other does");
   if (gate) {
@@ -214,6 +232,7 @@ PreparedInput Linear::add(hip::CommandGraph &graph, LinearBuffers b, const Proje
       if (s < segments.size()) {
         params.cols[s] = segment.outputSize;
         params.offset[s] = segment.columnOffset;
+        if (mixed) params.formats[s] = segment.formatId;
       }
     }
   }
@@ -221,7 +240,7 @@ PreparedInput Linear::add(hip::CommandGraph &graph, LinearBuffers b, const Proje
   params.deferred_scale = prepared && b.prepared.layout == LinearInput::TableUnscaled;
   // Unused bindings still name a buffer: the table stands in for them.
   const hip::Buffer &spare = b.scratch.input;
-  const std::string name = std::string("gguf_decode_") + segments.front().name() + "_m" + std::to_string(plan.storageRows()) +
+  const std::string name = std::string("gguf_decode_") + (mixed ? "mixed" : segments.front().name()) + "_m" + std::to_string(plan.storageRows()) +
                            epilogueSuffix(w.epilogue, plan.destination(), writesTable);
   if (norms) {
     images[1] = b.normWeight;

@@ -45,8 +45,15 @@ struct LinearWorkload final {
   // The widest record format among the projection's segments: it sets how many workgroups a
   // compute unit holds at once.
   uint32_t formatId = GGUF_FMT_Q4K;
+  // Segments of different formats (one dispatch of the mixed kernel): whole 64-column workgroups a
+  // segment, every workgroup one part of K, bf16 rows without an epilogue.
+  bool severalFormats = false;
   auto operator<=>(const LinearWorkload &) const = default;
 };
+
+// A plan's workload for `rows` rows of a projection: its matrix, its segments' widest record format and
+// whether they differ.
+[[nodiscard]] LinearWorkload workloadOf(const Projection &projection, uint32_t rows, LinearEpilogue epilogue);
 
 struct LinearConfig final {
   LinearTile tile = LinearTile::GgufMfma;

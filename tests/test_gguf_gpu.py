@@ -168,6 +168,46 @@ def test_fused_segments_equal_each_alone(backend):
         at += n
 
 
+@pytest.mark.parametrize("formats", [(ops.FMT_Q4K, ops.FMT_Q4K, ops.FMT_Q6K), (ops.FMT_Q80, ops.FMT_Q5K, ops.FMT_Q6K),
+                                     (ops.FMT_Q6K, ops.FMT_Q4K)])
+@pytest.mark.parametrize("M", [16, 40, 80])
+def test_segments_of_several_formats_equal_each_alone(backend, formats, M):
+    """The reference's fused projection takes a format per segment (gguf_linear.metal:237-261): one dispatch gives
+    each segment the bits it gets alone under the same partition of K, and the device's own plan stays in the
+    reference interval."""
+    print(f"case mixed segments formats={formats} M={M}", flush=True)
+    rng = np.random.default_rng(19)
+    K, sizes = 2048, (256, 64, 128)[:len(formats)]
+    natives = [orc.make_native(f, n, K, 70 + i) for i, (f, n) in enumerate(zip(formats, sizes))]
+    x = orc.f32_to_bf16(rng.standard_normal((M, K)).astype(np.float32))
+    linear = ops.Linear(backend)
+
+    def run(segments, **config):
+        proj = ops.Projection.from_native(backend, segments, K)
+        plan = linear.plan(proj, M, ops.EPILOGUE_NONE, **config)
+        out = backend.allocate_buffer(M * proj.output_size * 2)
+        graph = splash_amd.CommandGraph()
+        linear.add(graph, proj, plan, backend.from_array(x), out, linear.scratch_for(backend, [plan]))
+        assert ("mixed" in graph.kernels()[-1]) == (len({f for f, _, _ in segments}) > 1)
+        backend.run(graph)
+        return out.download(np.uint16).reshape(M, proj.output_size)
+
+    everything = list(zip(formats, sizes, natives))
+    for splits in (1, 2, 8):
+        fused, at = run(everything, splits=splits, whole_groups=0), 0
+        for segment in everything:
+            alone = run([segment], splits=splits, whole_groups=0)
+            assert np.array_equal(fused[:, at:at + segment[1]], alone), (splits, segment[0])
+            at += segment[1]
+    fused, at = run(everything), 0
+    for f, n, native in everything:
+        check_interval(orc.bf16_to_f32(fused[:, at:at + n]), orc.gemm(f, native, x, n))
+        at += n
+    # whole workgroups a segment, and no epilogue
+    with pytest.raises(splash_amd.SplashError):
+        run([(formats[0], 32, natives[0][:natives[0].size // sizes[0] * 32]), everything[-1]])
+
+
 @pytest.mark.parametrize("fmt", ALL_FORMATS)
 def test_residual_and_gate_up_epilogues(backend, fmt):
     """gguf_tile.h:10-16, gguf_linear.metal:34-71: bf16(v + res) and bf16(bf16(up) silu(bf16(gate)));
