@@ -1,7 +1,7 @@
 /* GGUF files: the header parser and the step from a file's tensor to what the operators take.
  * Replaces, for the verify step's weights, the reference's model::GgufFile / GgufTensor / GgufMetadata
  * (runtime/model/GgufFile.hpp:24-150) and the image preparation of runtime/model/GgufImage.cpp: a tensor
- * of a projection format (Q4_K, Q5_K, Q6_K, Q8_0) becomes the weight image spo_projection_create takes,
+ * of a projection format (Q4_K, Q5_K, Q6_K, Q8_0, IQ4_XS, IQ4_NL) becomes the weight image spo_projection_create takes,
  * a 16- or 32-bit float vector the bf16 weights of a norm. Status codes and the thread-local message of
  * sp_last_error are those of splash_hip.h; a malformed file is SP_BACKEND_ERROR with the parser's message. */
 #pragma once

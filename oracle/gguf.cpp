@@ -8,14 +8,17 @@ using namespace orc;
 
 namespace {
 
-constexpr uint32_t kQ4KBytes = 144, kQ5KBytes = 176, kQ6KBytes = 210, kQ80Bytes = 34, kBlock = 256;
+constexpr uint32_t kQ4KBytes = 144, kQ5KBytes = 176, kQ6KBytes = 210, kQ80Bytes = 34, kIQ4XSBytes = 136, kIQ4NLBytes = 18, kBlock = 256;
+// The 4-bit non-linear codebook of IQ4_NL and IQ4_XS (ggml's kvalues_iq4nl; GgufFormatReference.hpp:382-403 reads it).
+constexpr int8_t kIQ4Values[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
 constexpr uint32_t kQ6KScales = 128 + 64, kQ6KD = kQ6KScales + 16;  // GgufFormatReference.hpp:61
 
 // Bytes and elements of a native block: the K-quants' super-block of 256, Q8_0's group of 32.
 uint32_t blockBytes(uint32_t fmt) {
-  return fmt == ORC_FMT_Q4K ? kQ4KBytes : fmt == ORC_FMT_Q5K ? kQ5KBytes : fmt == ORC_FMT_Q6K ? kQ6KBytes : fmt == ORC_FMT_Q80 ? kQ80Bytes : 0;
+  return fmt == ORC_FMT_Q4K ? kQ4KBytes : fmt == ORC_FMT_Q5K ? kQ5KBytes : fmt == ORC_FMT_Q6K ? kQ6KBytes : fmt == ORC_FMT_Q80 ? kQ80Bytes
+         : fmt == ORC_FMT_IQ4XS ? kIQ4XSBytes : fmt == ORC_FMT_IQ4NL ? kIQ4NLBytes : 0;
 }
-uint32_t blockElements(uint32_t fmt) { return fmt == ORC_FMT_Q80 ? 32 : kBlock; }
+uint32_t blockElements(uint32_t fmt) { return fmt == ORC_FMT_Q80 || fmt == ORC_FMT_IQ4NL ? 32 : kBlock; }
 
 // GgufFormatReference.hpp:326-329
 void scaleMinK4(const uint8_t *sc, int j, uint8_t &s, uint8_t &m) {
@@ -27,9 +30,9 @@ void scaleMinK4(const uint8_t *sc, int j, uint8_t &s, uint8_t &m) {
 // (quant_formats.h:105-137); Q6_K has a scale per 16 and code - 32 (quant_formats.h:153-168).
 struct Group {
   uint8_t code[32];
-  float s[2];  // Q4_K, Q5_K: s[0] = s[1] = d * sc; Q6_K: one per 16 elements; Q8_0: d
-  float m;     // Q4_K, Q5_K: -dmin * mn; Q6_K, Q8_0: 0
-  int bias;    // Q4_K, Q5_K: 0; Q6_K: 32; Q8_0: 128 (code = value + 128)
+  float s[2];  // Q4_K, Q5_K: s[0] = s[1] = d * sc; Q6_K: one per 16 elements; Q8_0, IQ4_NL: d; IQ4_XS: d * (ls - 32)
+  float m;     // Q4_K, Q5_K: -dmin * mn; the others: 0
+  int bias;    // Q4_K, Q5_K: 0; Q6_K: 32; Q8_0, IQ4_NL, IQ4_XS: 128 (code = value or codebook value + 128)
 };
 void readGroup(uint32_t fmt, const uint8_t *row, uint32_t g, Group &out) {
   if (fmt == ORC_FMT_Q80) {   // GgufFormatReference.hpp:453-458: value = d * int8
@@ -41,8 +44,27 @@ void readGroup(uint32_t fmt, const uint8_t *row, uint32_t g, Group &out) {
     out.bias = 128;
     return;
   }
+  if (fmt == ORC_FMT_IQ4NL) {   // GgufFormatReference.hpp:394-403: value = d * codebook[nibble]; byte k's low nibble is
+    const uint8_t *blk = row + size_t(g) * kIQ4NLBytes;   // input k, its high nibble input 16 + k
+    uint16_t d16; std::memcpy(&d16, blk, 2);
+    for (int k = 0; k < 32; ++k) out.code[k] = uint8_t(kIQ4Values[k < 16 ? blk[2 + k] & 15 : blk[2 + k - 16] >> 4] + 128);
+    out.s[0] = out.s[1] = h2f(d16);
+    out.m = 0.f;
+    out.bias = 128;
+    return;
+  }
   const uint8_t *blk = row + size_t(g / 8) * blockBytes(fmt);
   const uint32_t j = g % 8;
+  if (fmt == ORC_FMT_IQ4XS) {   // GgufFormatReference.hpp:382-393: a 6-bit scale a group, value = d * (ls - 32) * codebook[nibble]
+    uint16_t d16, high; std::memcpy(&d16, blk, 2); std::memcpy(&high, blk + 2, 2);
+    const int ls = ((blk[4 + j / 2] >> (4 * (j % 2))) & 15) | (((high >> (2 * j)) & 3) << 4);
+    const uint8_t *qs = blk + 8 + 16 * j;
+    for (int k = 0; k < 32; ++k) out.code[k] = uint8_t(kIQ4Values[k < 16 ? qs[k] & 15 : qs[k - 16] >> 4] + 128);
+    out.s[0] = out.s[1] = h2f(d16) * float(ls - 32);  // exact: 11 + 6 bits
+    out.m = 0.f;
+    out.bias = 128;
+    return;
+  }
   if (fmt == ORC_FMT_Q5K) {   // GgufFormatReference.hpp:405-416: the fifth bits in qh, bit j of byte k
     uint16_t d16, m16; std::memcpy(&d16, blk, 2); std::memcpy(&m16, blk + 2, 2);
     uint8_t sc, mn; scaleMinK4(blk + 4, int(j), sc, mn);
@@ -78,7 +100,7 @@ void readGroup(uint32_t fmt, const uint8_t *row, uint32_t g, Group &out) {
 }
 
 // llama.cpp semantics (GgufFormatReference.hpp:370-381, :405-432, :453-458): Q4_K and Q5_K d*sc*code - dmin*mn
-// with one rounding (both products exact); Q6_K d*sc*(q-32) and Q8_0 d*q, exact.
+// with one rounding (both products exact); Q6_K d*sc*(q-32), Q8_0 d*q and the IQ4 codebook formats' s*value, exact.
 void groupValues(uint32_t fmt, const uint8_t *row, uint32_t g, float *vals) {
   Group grp; readGroup(fmt, row, g, grp);
   for (int k = 0; k < 32; ++k) {
@@ -259,8 +281,9 @@ int orc_make_native(uint32_t fmt, uint32_t rows, uint32_t K, uint32_t seed, uint
   if (!orc_row_bytes(fmt, K)) return -1;
   std::mt19937 rng(seed);
   // GgufFormatReference.hpp:295-323 scaleRange
-  std::uniform_real_distribution<float> range = fmt == ORC_FMT_Q6K
-      ? std::uniform_real_distribution<float>(0.00002f, 0.0001f) : std::uniform_real_distribution<float>(0.0005f, 0.004f);
+  std::uniform_real_distribution<float> range = fmt == ORC_FMT_Q6K     ? std::uniform_real_distribution<float>(0.00002f, 0.0001f)
+                                                : fmt == ORC_FMT_IQ4XS ? std::uniform_real_distribution<float>(0.00002f, 0.00015f)
+                                                                       : std::uniform_real_distribution<float>(0.0005f, 0.004f);
   makeNativeWith(fmt, rows, K, rng, native, [&] { return f2h(range(rng)); });
   return 0;
 }
@@ -336,8 +359,9 @@ int orc_gemm(uint32_t fmt, const uint8_t *native, const uint16_t *x, uint32_t M,
               for (int k = 0; k < 32; ++k) dot = std::fma(xr[32 * g + k], float(128 + grp.code[k]), dot);
               acc = std::fma(dot, grp.s[0], acc);
               acc = std::fma(s16[0] + s16[1], grp.m - 128.f * grp.s[0], acc);
-            } else if (fmt == ORC_FMT_Q80) {
-              // the operand is the int8 value itself (linear_gguf_sgmatrix.metal:96-98), one scale a group, no min
+            } else if (fmt == ORC_FMT_Q80 || fmt == ORC_FMT_IQ4XS || fmt == ORC_FMT_IQ4NL) {
+              // the operand is the int8 value itself (linear_gguf_sgmatrix.metal:96-98), or the codebook's
+              // (:94-95), one scale a group, no min
               float dot = 0;
               for (int k = 0; k < 32; ++k) dot = std::fma(xr[32 * g + k], float(int(grp.code[k]) - 128), dot);
               acc = std::fma(dot, grp.s[0], acc);

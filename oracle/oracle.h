@@ -8,7 +8,7 @@
 //
 // Pin status of each group of functions (what fixes it besides its own formula):
 //   orc_dequant_rows (Q4_K, Q5_K,   pinned: SHA-256 goldens of upstream GGML over the 256x1024
-//     Q6_K, Q8_0)                   fixture (dev/tests/fixtures/weight-goldens/goldens.json:3,6,7,9)
+//     Q6_K, Q8_0, IQ4_XS, IQ4_NL)   fixture (dev/tests/fixtures/weight-goldens/goldens.json:3-7,9)
 //                                   and the compiled reference header (oracle/_ref).
 //   orc_fixture                     pinned by the same goldens (a wrong byte order changes the hash).
 //   orc_quantize_q4k / q6k          PARITY UNPINNED: the K-quantizer lives in llama.cpp/ggml
@@ -35,7 +35,7 @@ extern "C" {
 #endif
 
 // Format ids follow the reference's GGUF_FMT_* numbering (runtime/metal/abi/QuantFormat.h:138-154).
-enum { ORC_FMT_Q4K = 0, ORC_FMT_Q5K = 3, ORC_FMT_Q6K = 4, ORC_FMT_Q80 = 6 };
+enum { ORC_FMT_Q4K = 0, ORC_FMT_IQ4XS = 1, ORC_FMT_IQ4NL = 2, ORC_FMT_Q5K = 3, ORC_FMT_Q6K = 4, ORC_FMT_Q80 = 6 };
 
 // ---- half / bfloat16 scalar conversions (round to nearest even) ----
 uint16_t orc_f2h(float f);

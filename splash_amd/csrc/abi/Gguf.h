@@ -39,6 +39,14 @@
 //     [4096, 4352)  scales: column c's eight fp16 d (groups 0..7) at 4096 + 16 c.
 //   Its operands are the bf16 128 + value (0..255, exact); the 128 leaves as Q4_K's does, through the row sums.
 //
+//   IQ4_XS record, 2176 B (16 native blocks of 136 B), and IQ4_NL record, 2304 B (16 columns of eight native 18-B blocks):
+//     [   0, 2048)  nibbles: two 1024-B halves h; in half h lane l owns 16 B at 1024 h + 16 l, whose word i holds the
+//                   lane's eight codes of group 4 h + i as the native bytes do: byte j's low nibble the code of input
+//                   4 kq + j, its high nibble that of input 16 + 4 kq + j.
+//     [2048, ...)   IQ4_XS: column c's native d, scales_h and four scales_l bytes at 2048 + 8 c;
+//                   IQ4_NL: column c's eight fp16 d (groups 0..7) at 2048 + 16 c.
+//   A code names a value of the 16-entry codebook (-127 .. 113); the operands are the bf16 128 + value, as Q8_0's.
+//
 // Within a group, lane (c, kq) holds eight codes as four registers of two bf16 operands
 // 128 + code: register j (0..3) holds inputs 16 (j / 2) + 4 kq + (j % 2) [low half] and that + 2
 // [high half]. Element e = 2 j + half of the lane's MFMA operand is therefore input
@@ -56,6 +64,8 @@
 #include <stdint.h>
 
 #define GGUF_FMT_Q4K 0u
+#define GGUF_FMT_IQ4XS 1u
+#define GGUF_FMT_IQ4NL 2u
 #define GGUF_FMT_Q5K 3u
 #define GGUF_FMT_Q6K 4u
 #define GGUF_FMT_Q80 6u
@@ -67,6 +77,11 @@
 #define GGUF_Q5K_NATIVE 176u
 #define GGUF_Q6K_NATIVE 210u
 #define GGUF_Q80_NATIVE 272u  // eight 34-byte blocks: the bytes of 256 inputs
+#define GGUF_IQ4XS_NATIVE 136u
+#define GGUF_IQ4NL_NATIVE 144u  // eight 18-byte blocks
+#define GGUF_IQ4XS_RECORD (GGUF_TILE_COLUMNS * GGUF_IQ4XS_NATIVE)  // 2176
+#define GGUF_IQ4NL_RECORD (GGUF_TILE_COLUMNS * GGUF_IQ4NL_NATIVE)  // 2304
+#define GGUF_IQ4_SCALES 2048u
 #define GGUF_Q4K_RECORD (GGUF_TILE_COLUMNS * GGUF_Q4K_NATIVE)  // 2304
 #define GGUF_Q6K_RECORD (GGUF_TILE_COLUMNS * GGUF_Q6K_NATIVE)  // 3360
 #define GGUF_Q5K_RECORD (GGUF_TILE_COLUMNS * GGUF_Q5K_NATIVE)  // 2816
@@ -98,6 +113,8 @@ GGUF_INLINE uint32_t gguf_record_bytes(uint32_t format) {
          : format == GGUF_FMT_Q6K ? GGUF_Q6K_RECORD
          : format == GGUF_FMT_Q5K ? GGUF_Q5K_RECORD
          : format == GGUF_FMT_Q80 ? GGUF_Q80_RECORD
+         : format == GGUF_FMT_IQ4XS ? GGUF_IQ4XS_RECORD
+         : format == GGUF_FMT_IQ4NL ? GGUF_IQ4NL_RECORD
                                   : 0u;
 }
 GGUF_INLINE uint32_t gguf_native_bytes(uint32_t format) {
@@ -105,11 +122,19 @@ GGUF_INLINE uint32_t gguf_native_bytes(uint32_t format) {
          : format == GGUF_FMT_Q6K ? GGUF_Q6K_NATIVE
          : format == GGUF_FMT_Q5K ? GGUF_Q5K_NATIVE
          : format == GGUF_FMT_Q80 ? GGUF_Q80_NATIVE
+         : format == GGUF_FMT_IQ4XS ? GGUF_IQ4XS_NATIVE
+         : format == GGUF_FMT_IQ4NL ? GGUF_IQ4NL_NATIVE
                                   : 0u;
 }
 // Kernel-name tag of a format.
 GGUF_INLINE const char *gguf_format_name(uint32_t format) {
-  return format == GGUF_FMT_Q4K ? "q4k" : format == GGUF_FMT_Q6K ? "q6k" : format == GGUF_FMT_Q5K ? "q5k" : format == GGUF_FMT_Q80 ? "q80" : "";
+  return format == GGUF_FMT_Q4K     ? "q4k"
+         : format == GGUF_FMT_Q6K   ? "q6k"
+         : format == GGUF_FMT_Q5K   ? "q5k"
+         : format == GGUF_FMT_Q80   ? "q80"
+         : format == GGUF_FMT_IQ4XS ? "iq4xs"
+         : format == GGUF_FMT_IQ4NL ? "iq4nl"
+                                    : "";
 }
 // Bytes of the image of an [N, K] tensor (N a multiple of 16, K of 256): those of its native rows.
 GGUF_INLINE uint64_t gguf_image_bytes(uint32_t format, uint32_t n, uint32_t k) {

@@ -76,17 +76,34 @@ template <bool High, uint32_t R0> __device__ __forceinline__ uint4 q5_operands(u
 // Q8_0: the bf16 operands 128 + value of a group from the words of its inputs 4 kq .. 4 kq + 3 (wa) and
 // 16 + 4 kq .. + 3 (wb). value + 128 is the byte with its sign bit flipped; an integer up to 255 is exact in
 // fp32 and in bf16, whose bits are the fp32's upper half.
-__device__ __forceinline__ uint4 q8_operands(uint32_t wa, uint32_t wb) {
+// The operands of a group from its bytes 0..255 themselves: a the inputs 4 kq .. 4 kq + 3, b the inputs 16 + 4 kq .. + 3.
+__device__ __forceinline__ uint4 byte_operands(uint32_t a, uint32_t b) {
   auto pair = [](uint32_t first, uint32_t second) -> uint32_t {  // bf16(first) in the low half, bf16(second) in the high
     return __builtin_amdgcn_perm(__builtin_bit_cast(uint32_t, float(second)), __builtin_bit_cast(uint32_t, float(first)), 0x07060302u);
   };
-  const uint32_t a = wa ^ 0x80808080u, b = wb ^ 0x80808080u;
   uint4 r;
   r.x = pair(a & 0xFFu, (a >> 16) & 0xFFu);
   r.y = pair((a >> 8) & 0xFFu, a >> 24);
   r.z = pair(b & 0xFFu, (b >> 16) & 0xFFu);
   r.w = pair((b >> 8) & 0xFFu, b >> 24);
   return r;
+}
+__device__ __forceinline__ uint4 q8_operands(uint32_t wa, uint32_t wb) { return byte_operands(wa ^ 0x80808080u, wb ^ 0x80808080u); }
+
+// IQ4_XS and IQ4_NL: 128 + the codebook value of each of four codes (one a byte, 0..15), by two byte permutes over the
+// codebook's halves and a select on the codes' bit 3. The codebook (ggml's kvalues_iq4nl):
+// -127 -104 -83 -65 -49 -35 -22 -10 1 13 25 38 53 69 89 113.
+__device__ __forceinline__ uint32_t iq4_bytes(uint32_t codes) {
+  constexpr uint32_t kT0 = 0x3F2D1801u, kT1 = 0x766A5D4Fu, kT2 = 0xA6998D81u, kT3 = 0xF1D9C5B5u;  // 128 + value, code 0 lowest
+  const uint32_t index = codes & 0x07070707u;
+  const uint32_t low = __builtin_amdgcn_perm(kT1, kT0, index), high = __builtin_amdgcn_perm(kT3, kT2, index);
+  const uint32_t upper = ((codes >> 3) & 0x01010101u) * 0xFFu;  // 0xFF in the bytes of codes 8..15
+  return (high & upper) | (low & ~upper);
+}
+// The operands of a group from the word of the lane's eight codes (abi/Gguf.h): low nibbles inputs 4 kq .. + 3, high
+// nibbles inputs 16 + 4 kq .. + 3.
+__device__ __forceinline__ uint4 iq4_operands(uint32_t word) {
+  return byte_operands(iq4_bytes(word & 0x0F0F0F0Fu), iq4_bytes((word >> 4) & 0x0F0F0F0Fu));
 }
 
 // The code (0..15, or 0..63 for Q6_K) in half `half` of operand register `reg`.

@@ -83,16 +83,19 @@ template <uint32_t FMT> struct Cursor {
   const uint4 *column = nullptr;
   const uint16_t *d = nullptr;   // Q6_K only
   const uint2 *fifth = nullptr;  // Q5_K only
+  const uint2 *meta8 = nullptr;  // IQ4_XS only: its column's eight bytes
   static constexpr uint32_t kColumnPart = FMT == GGUF_FMT_Q4K   ? 2048u
                                           : FMT == GGUF_FMT_Q6K ? GGUF_Q6K_SCALES
                                           : FMT == GGUF_FMT_Q5K ? GGUF_Q5K_META
-                                                                : GGUF_Q80_SCALES;
+                                          : FMT == GGUF_FMT_Q80 ? GGUF_Q80_SCALES
+                                                                : GGUF_IQ4_SCALES;
   __device__ __forceinline__ void open(const uint8_t *record, uint32_t lane) {
     const uint4 *p = reinterpret_cast<const uint4 *>(record);
     mine = p + lane;
     column = p + kColumnPart / 16u + (lane & 15u);
     if constexpr (FMT == GGUF_FMT_Q6K) d = reinterpret_cast<const uint16_t *>(record + GGUF_Q6K_D) + (lane & 15u);
     if constexpr (FMT == GGUF_FMT_Q5K) fifth = reinterpret_cast<const uint2 *>(record + GGUF_Q5K_HIGH) + lane;
+    if constexpr (FMT == GGUF_FMT_IQ4XS) meta8 = reinterpret_cast<const uint2 *>(record + GGUF_IQ4_SCALES) + (lane & 15u);
   }
   __device__ __forceinline__ void advance() {
     constexpr uint32_t kVectors = gguf_record_bytes(FMT) / 16u;
@@ -100,6 +103,7 @@ template <uint32_t FMT> struct Cursor {
     column += kVectors;
     if constexpr (FMT == GGUF_FMT_Q6K) d += kVectors * 8u;
     if constexpr (FMT == GGUF_FMT_Q5K) fifth += kVectors * 2u;
+    if constexpr (FMT == GGUF_FMT_IQ4XS) meta8 += kVectors * 2u;
   }
 };
 
@@ -143,7 +147,43 @@ template <> struct Record<GGUF_FMT_Q80> {
   }
 };
 
+template <> struct Record<GGUF_FMT_IQ4XS> {
+  uint4 n0, n1;
+  uint2 meta;  // x: d | scales_h << 16; y: the low four bits of the eight groups' scales
+  __device__ __forceinline__ void load(const Cursor<GGUF_FMT_IQ4XS> &at) {
+    n0 = load_stream(at.mine);
+    n1 = load_stream(at.mine + 64);
+    meta = *at.meta8;
+  }
+};
+template <> struct Record<GGUF_FMT_IQ4NL> {
+  uint4 n0, n1, scales;
+  __device__ __forceinline__ void load(const Cursor<GGUF_FMT_IQ4NL> &at) {
+    n0 = load_stream(at.mine);
+    n1 = load_stream(at.mine + 64);
+    scales = load_stream(at.column);
+  }
+};
+
 // The eight groups' operand registers of a record, group g's in ops[g].
+template <uint32_t FMT>
+__device__ __forceinline__ void iq4_record_operands(const Record<FMT> &r, uint4 ops[8]) {
+  ops[0] = iq4_operands(r.n0.x);
+  ops[1] = iq4_operands(r.n0.y);
+  ops[2] = iq4_operands(r.n0.z);
+  ops[3] = iq4_operands(r.n0.w);
+  ops[4] = iq4_operands(r.n1.x);
+  ops[5] = iq4_operands(r.n1.y);
+  ops[6] = iq4_operands(r.n1.z);
+  ops[7] = iq4_operands(r.n1.w);
+}
+__device__ __forceinline__ void record_operands(const Record<GGUF_FMT_IQ4XS> &r, uint4 ops[8]) { iq4_record_operands(r, ops); }
+__device__ __forceinline__ void record_operands(const Record<GGUF_FMT_IQ4NL> &r, uint4 ops[8]) { iq4_record_operands(r, ops); }
+// Group g's scale of an IQ4_XS record's column: d * (ls - 32), ls its six bits of scales_l and scales_h (exact).
+__device__ __forceinline__ float iq4xs_scale(const uint2 &meta, uint32_t g) {
+  const uint32_t ls = ((meta.y >> (4u * g)) & 15u) | (((meta.x >> (16u + 2u * g)) & 3u) << 4);
+  return half_bits_to_float(meta.x & 0xFFFFu) * float(int(ls) - 32);
+}
 __device__ __forceinline__ void record_operands(const Record<GGUF_FMT_Q5K> &r, uint4 ops[8]) {
   ops[0] = q5_operands<false, 0>(r.n0.x, r.n0.y, r.fifth.x);
   ops[1] = q5_operands<true, 4>(r.n0.x, r.n0.y, r.fifth.x);
@@ -166,6 +206,10 @@ __device__ __forceinline__ float q8_scale(const uint4 &scales, uint32_t g) {
   const uint32_t word = g < 2 ? scales.x : g < 4 ? scales.y : g < 6 ? scales.z : scales.w;
   return half_bits_to_float((word >> (16u * (g & 1u))) & 0xFFFFu);
 }
+// Group g's scale of a record of one of the formats whose groups carry one scale and no minimum.
+__device__ __forceinline__ float group_scale(const Record<GGUF_FMT_Q80> &r, uint32_t g) { return q8_scale(r.scales, g); }
+__device__ __forceinline__ float group_scale(const Record<GGUF_FMT_IQ4NL> &r, uint32_t g) { return q8_scale(r.scales, g); }
+__device__ __forceinline__ float group_scale(const Record<GGUF_FMT_IQ4XS> &r, uint32_t g) { return iq4xs_scale(r.meta, g); }
 __device__ __forceinline__ void record_operands(const Record<GGUF_FMT_Q4K> &r, uint4 ops[8]) {
   ops[0] = q4_operands<false>(r.n0.x, r.n0.y);
   ops[1] = q4_operands<true>(r.n0.x, r.n0.y);
@@ -206,10 +250,10 @@ template <uint32_t FMT> __global__ __launch_bounds__(64) void gguf_dequant(const
   uint4 ops[8];
   record_operands(rec, ops);
   float *row = out + size_t(16u * tile + c) * p.input_size + size_t(b) * GGUF_BLOCK;
-  if constexpr (FMT == GGUF_FMT_Q80) {
+  if constexpr (FMT == GGUF_FMT_Q80 || FMT == GGUF_FMT_IQ4XS || FMT == GGUF_FMT_IQ4NL) {
 #pragma unroll
     for (uint32_t g = 0; g < 8; ++g) {
-      const float d = q8_scale(rec.scales, g);
+      const float d = group_scale(rec, g);
       const uint32_t regs[4] = {ops[g].x, ops[g].y, ops[g].z, ops[g].w};
 #pragma unroll
       for (uint32_t e = 0; e < 8; ++e)
@@ -247,6 +291,8 @@ SP_REGISTER_KERNEL("gguf_dequant_q4k", &gguf_dequant<GGUF_FMT_Q4K>);
 SP_REGISTER_KERNEL("gguf_dequant_q6k", &gguf_dequant<GGUF_FMT_Q6K>);
 SP_REGISTER_KERNEL("gguf_dequant_q5k", &gguf_dequant<GGUF_FMT_Q5K>);
 SP_REGISTER_KERNEL("gguf_dequant_q80", &gguf_dequant<GGUF_FMT_Q80>);
+SP_REGISTER_KERNEL("gguf_dequant_iq4xs", &gguf_dequant<GGUF_FMT_IQ4XS>);
+SP_REGISTER_KERNEL("gguf_dequant_iq4nl", &gguf_dequant<GGUF_FMT_IQ4NL>);
 
 // ---------------------------------------------------------------------------------------------
 // The decode projection.
@@ -302,6 +348,20 @@ __device__ __forceinline__ void load_record(Record<GGUF_FMT_Q80> &rec, Resource 
   rec.scales = load128<kStreamOnce>(r, column);
 }
 
+__device__ __forceinline__ void load_record(Record<GGUF_FMT_IQ4XS> &rec, Resource r, uint32_t mine, uint32_t) {
+  rec.n0 = load128<kStreamOnce>(r, mine);
+  rec.n1 = load128<kStreamOnce>(r, mine + 1024u);
+  // The column's 8 bytes sit at record + 2048 + 8 c; `mine` is record + 16 l.
+  const uint32_t lane = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+  const u32x2 meta = __builtin_amdgcn_raw_buffer_load_b64(r, int(mine - 16u * lane + GGUF_IQ4_SCALES + 8u * (lane & 15u)), 0, kStreamOnce);
+  rec.meta = make_uint2(meta.x, meta.y);
+}
+__device__ __forceinline__ void load_record(Record<GGUF_FMT_IQ4NL> &rec, Resource r, uint32_t mine, uint32_t column) {
+  rec.n0 = load128<kStreamOnce>(r, mine);
+  rec.n1 = load128<kStreamOnce>(r, mine + 1024u);
+  rec.scales = load128<kStreamOnce>(r, column);
+}
+
 struct TileRef {
   const uint8_t *image;  // the tile's first record; null for a tile past the dispatch's last
   uint32_t column;       // its first destination column
@@ -336,14 +396,21 @@ __device__ __forceinline__ void accumulate_record(const Record<FMT> &rec, const 
   uint4 ops[8];
   record_operands(rec, ops);
   const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
-  if constexpr (FMT == GGUF_FMT_Q80) {
-    // One fp16 scale a group; the operands' 128 leaves through the row sums: -128 d of groups kq and 4 + kq.
+  if constexpr (FMT == GGUF_FMT_Q80 || FMT == GGUF_FMT_IQ4XS || FMT == GGUF_FMT_IQ4NL) {
+    // One scale a group; the operands' 128 leaves through the row sums: -128 s of groups kq and 4 + kq.
     float s[8];
 #pragma unroll
-    for (uint32_t g = 0; g < 8; ++g) s[g] = q8_scale(rec.scales, g);
-    const uint32_t lowWord = kq == 0 ? rec.scales.x : kq == 1 ? rec.scales.x >> 16 : kq == 2 ? rec.scales.y : rec.scales.y >> 16;
-    const uint32_t highWord = kq == 0 ? rec.scales.z : kq == 1 ? rec.scales.z >> 16 : kq == 2 ? rec.scales.w : rec.scales.w >> 16;
-    const float c_lo = -128.f * half_bits_to_float(lowWord & 0xFFFFu), c_hi = -128.f * half_bits_to_float(highWord & 0xFFFFu);
+    for (uint32_t g = 0; g < 8; ++g) s[g] = group_scale(rec, g);
+    float c_lo, c_hi;
+    if constexpr (FMT == GGUF_FMT_IQ4XS) {
+      c_lo = -128.f * iq4xs_scale(rec.meta, kq);
+      c_hi = -128.f * iq4xs_scale(rec.meta, 4u + kq);
+    } else {
+      const uint32_t lowWord = kq == 0 ? rec.scales.x : kq == 1 ? rec.scales.x >> 16 : kq == 2 ? rec.scales.y : rec.scales.y >> 16;
+      const uint32_t highWord = kq == 0 ? rec.scales.z : kq == 1 ? rec.scales.z >> 16 : kq == 2 ? rec.scales.w : rec.scales.w >> 16;
+      c_lo = -128.f * half_bits_to_float(lowWord & 0xFFFFu);
+      c_hi = -128.f * half_bits_to_float(highWord & 0xFFFFu);
+    }
 #pragma unroll
     for (int t = 0; t < RT; ++t) {
       acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(sums[t][0][lane], c_lo, acc[t], 0, 0, 0);
@@ -837,17 +904,19 @@ __global__ __launch_bounds__(256) void gguf_decode_mixed(const uint8_t *__restri
       segment = s + 1u;
     }
   const uint8_t *image = segment == 0 ? seg0 : segment == 1 ? seg1 : seg2;
+  auto of = [&](const uint32_t (&field)[3]) { return segment == 0 ? field[0] : segment == 1 ? field[1] : field[2]; };
+  const uint32_t format = of(p.formats);
   GgufDecodeParams mine = p;
-  mine.cols[0] = p.cols[segment];
+  mine.cols[0] = of(p.cols);
   mine.cols[1] = mine.cols[2] = 0;
-  mine.offset[0] = p.offset[segment];
-  mine.units = p.cols[segment] / GGUF_TILE_COLUMNS;
+  mine.offset[0] = of(p.offset);
+  mine.units = mine.cols[0] / GGUF_TILE_COLUMNS;
   mine.whole_groups = 0;
   partials += size_t(before) * p.splits * kGroupFloats;
   counters += before;
   const uint32_t item = (group - before) * p.splits + split;
   __shared__ DecodeShared<RT> shared;
-  switch (p.formats[segment]) {
+  switch (format) {
   case GGUF_FMT_Q4K:
     decode_workgroup<GGUF_FMT_Q4K, RT, GGUF_EPILOGUE_PLAIN>(shared, image, image, image, table, out, residual, partials, counters, mine, item);
     break;
@@ -859,6 +928,12 @@ __global__ __launch_bounds__(256) void gguf_decode_mixed(const uint8_t *__restri
     break;
   case GGUF_FMT_Q80:
     decode_workgroup<GGUF_FMT_Q80, RT, GGUF_EPILOGUE_PLAIN>(shared, image, image, image, table, out, residual, partials, counters, mine, item);
+    break;
+  case GGUF_FMT_IQ4XS:
+    decode_workgroup<GGUF_FMT_IQ4XS, RT, GGUF_EPILOGUE_PLAIN>(shared, image, image, image, table, out, residual, partials, counters, mine, item);
+    break;
+  case GGUF_FMT_IQ4NL:
+    decode_workgroup<GGUF_FMT_IQ4NL, RT, GGUF_EPILOGUE_PLAIN>(shared, image, image, image, table, out, residual, partials, counters, mine, item);
     break;
   default: break;
   }
@@ -912,5 +987,11 @@ SP_GGUF_DECODE("q5k", GGUF_FMT_Q5K, 64, 4);
 SP_GGUF_DECODE("q80", GGUF_FMT_Q80, 16, 1);
 SP_GGUF_DECODE("q80", GGUF_FMT_Q80, 32, 2);
 SP_GGUF_DECODE("q80", GGUF_FMT_Q80, 64, 4);
+SP_GGUF_DECODE("iq4xs", GGUF_FMT_IQ4XS, 16, 1);
+SP_GGUF_DECODE("iq4xs", GGUF_FMT_IQ4XS, 32, 2);
+SP_GGUF_DECODE("iq4xs", GGUF_FMT_IQ4XS, 64, 4);
+SP_GGUF_DECODE("iq4nl", GGUF_FMT_IQ4NL, 16, 1);
+SP_GGUF_DECODE("iq4nl", GGUF_FMT_IQ4NL, 32, 2);
+SP_GGUF_DECODE("iq4nl", GGUF_FMT_IQ4NL, 64, 4);
 
 } // namespace splash::kernels

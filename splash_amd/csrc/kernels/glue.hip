@@ -173,6 +173,27 @@ __global__ __launch_bounds__(64) void gguf_embed(const uint8_t *__restrict__ tab
       if constexpr (kFifth) code |= ((qh[e] >> j) & 1u) << 4;
       o[k] = uint16_t(float_to_bf16_bits(__fmaf_rn(d * float(s), float(code), -(dmin * float(m)))));
     }
+  } else if constexpr (FMT == GGUF_FMT_IQ4XS || FMT == GGUF_FMT_IQ4NL) {
+    // value = scale * codebook[nibble]: byte e % 16 of the group's 16 holds inputs e (low nibble) and 16 + e (high)
+    constexpr int kCodebook[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
+    constexpr bool kXs = FMT == GGUF_FMT_IQ4XS;
+    const uint8_t *blk = table + (size_t(token) * blocks + block) * (kXs ? GGUF_IQ4XS_NATIVE : GGUF_IQ4NL_NATIVE);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t k = tid + 64u * i, j = k / 32u, e = k % 32u;
+      float scale;
+      const uint8_t *qs;
+      if constexpr (kXs) {
+        const uint32_t high = blk[2] | (blk[3] << 8), ls = ((blk[4u + j / 2u] >> (4u * (j % 2u))) & 15u) | (((high >> (2u * j)) & 3u) << 4);
+        scale = half_bits_to_float(blk[0] | (blk[1] << 8)) * float(int(ls) - 32);
+        qs = blk + 8u + 16u * j;
+      } else {
+        scale = half_bits_to_float(blk[18u * j] | (blk[18u * j + 1u] << 8));
+        qs = blk + 18u * j + 2u;
+      }
+      const uint32_t code = e < 16u ? qs[e] & 15u : qs[e - 16u] >> 4;
+      o[k] = uint16_t(float_to_bf16_bits(scale * float(kCodebook[code])));
+    }
   } else if constexpr (FMT == GGUF_FMT_Q80) {
     const uint8_t *blk = table + (size_t(token) * blocks + block) * GGUF_Q80_NATIVE;
 #pragma unroll
@@ -199,5 +220,7 @@ SP_REGISTER_KERNEL("gguf_embed_q4k", &gguf_embed<GGUF_FMT_Q4K>);
 SP_REGISTER_KERNEL("gguf_embed_q6k", &gguf_embed<GGUF_FMT_Q6K>);
 SP_REGISTER_KERNEL("gguf_embed_q5k", &gguf_embed<GGUF_FMT_Q5K>);
 SP_REGISTER_KERNEL("gguf_embed_q80", &gguf_embed<GGUF_FMT_Q80>);
+SP_REGISTER_KERNEL("gguf_embed_iq4xs", &gguf_embed<GGUF_FMT_IQ4XS>);
+SP_REGISTER_KERNEL("gguf_embed_iq4nl", &gguf_embed<GGUF_FMT_IQ4NL>);
 
 } // namespace splash::kernels

@@ -15,10 +15,11 @@ namespace splash::model {
 
 namespace {
 
-constexpr std::array<std::pair<uint32_t, GgmlTypeTraits>, 12> kTypes{{
+constexpr std::array<std::pair<uint32_t, GgmlTypeTraits>, 13> kTypes{{
     {0, {"F32", 1, 4}},        {1, {"F16", 1, 2}},        {2, {"Q4_0", 32, 18}},    {3, {"Q4_1", 32, 20}},
     {8, {"Q8_0", 32, 34}},     {10, {"Q2_K", 256, 84}},   {11, {"Q3_K", 256, 110}}, {12, {"Q4_K", 256, 144}},
-    {13, {"Q5_K", 256, 176}},  {14, {"Q6_K", 256, 210}},  {23, {"IQ4_XS", 256, 136}}, {30, {"BF16", 1, 2}},
+    {13, {"Q5_K", 256, 176}},  {14, {"Q6_K", 256, 210}},  {20, {"IQ4_NL", 32, 18}},   {23, {"IQ4_XS", 256, 136}},
+    {30, {"BF16", 1, 2}},
 }};
 
 // GGUF metadata value types.
@@ -100,6 +101,8 @@ std::optional<uint32_t> imageFormat(uint32_t ggmlType) noexcept {
     case ggml::kQ5_K: return GGUF_FMT_Q5K;
     case ggml::kQ6_K: return GGUF_FMT_Q6K;
     case ggml::kQ8_0: return GGUF_FMT_Q80;
+    case ggml::kIQ4_XS: return GGUF_FMT_IQ4XS;
+    case ggml::kIQ4_NL: return GGUF_FMT_IQ4NL;
     default: return std::nullopt;
   }
 }

@@ -23,7 +23,7 @@ public:
 
 // ggml type ids as GGUF tensor infos store them (ggml-common.h; GgufFile.hpp:35-66 in the reference).
 namespace ggml {
-inline constexpr uint32_t kF32 = 0, kF16 = 1, kQ8_0 = 8, kQ4_K = 12, kQ5_K = 13, kQ6_K = 14, kBF16 = 30;
+inline constexpr uint32_t kF32 = 0, kF16 = 1, kQ8_0 = 8, kQ4_K = 12, kQ5_K = 13, kQ6_K = 14, kIQ4_NL = 20, kIQ4_XS = 23, kBF16 = 30;
 }
 struct GgmlTypeTraits {
   const char *name;

@@ -83,6 +83,16 @@ void packGgufImage(uint32_t formatId, const uint8_t *native, uint32_t rows, uint
             }
           }
           std::memcpy(rec + GGUF_Q5K_META + 16 * c, blk, 16);
+        } else if (formatId == GGUF_FMT_IQ4XS || formatId == GGUF_FMT_IQ4NL) {
+          // Native IQ4_XS: d, scales_h, scales_l[4], qs[128]; IQ4_NL: eight blocks of (fp16 d, qs[16]). Byte j of a
+          // group's 16 holds inputs j (low nibble) and 16 + j (high): the record's words are native words, moved.
+          const bool xs = formatId == GGUF_FMT_IQ4XS;
+          for (uint32_t group = 0; group < 8; ++group) {
+            const uint8_t *qs = xs ? blk + 8 + 16 * group : blk + 18 * group + 2;
+            for (uint32_t kq = 0; kq < 4; ++kq) std::memcpy(rec + nibbleOffset(c, kq, group / 4, group % 4), qs + 4 * kq, 4);
+            if (!xs) std::memcpy(rec + GGUF_IQ4_SCALES + 16 * c + 2 * group, blk + 18 * group, 2);
+          }
+          if (xs) std::memcpy(rec + GGUF_IQ4_SCALES + 8 * c, blk, 8);
         } else if (formatId == GGUF_FMT_Q80) {
           // Native: eight blocks of (fp16 d, 32 int8).
           for (uint32_t group = 0; group < 8; ++group) {
@@ -165,6 +175,14 @@ void unpackGgufImage(uint32_t formatId, const uint8_t *image, uint32_t rows, uin
                   }
             }
           std::memcpy(blk, rec + GGUF_Q5K_META + 16 * c, 16);
+        } else if (formatId == GGUF_FMT_IQ4XS || formatId == GGUF_FMT_IQ4NL) {
+          const bool xs = formatId == GGUF_FMT_IQ4XS;
+          for (uint32_t group = 0; group < 8; ++group) {
+            uint8_t *qs = xs ? blk + 8 + 16 * group : blk + 18 * group + 2;
+            for (uint32_t kq = 0; kq < 4; ++kq) std::memcpy(qs + 4 * kq, rec + nibbleOffset(c, kq, group / 4, group % 4), 4);
+            if (!xs) std::memcpy(blk + 18 * group, rec + GGUF_IQ4_SCALES + 16 * c + 2 * group, 2);
+          }
+          if (xs) std::memcpy(blk, rec + GGUF_IQ4_SCALES + 8 * c, 8);
         } else if (formatId == GGUF_FMT_Q80) {
           for (uint32_t group = 0; group < 8; ++group) {
             uint8_t *q = blk + 34 * group + 2;

@@ -8,7 +8,8 @@ from . import _native as nat
 from ._native import lib, check
 from .backend import Buffer, STORAGE_PRIVATE
 
-FMT_Q4K, FMT_Q5K, FMT_Q6K, FMT_Q80 = 0, 3, 4, 6
+FMT_Q4K, FMT_IQ4XS, FMT_IQ4NL, FMT_Q5K, FMT_Q6K, FMT_Q80 = 0, 1, 2, 3, 4, 6
+FORMATS = (FMT_Q4K, FMT_Q6K, FMT_Q5K, FMT_Q80, FMT_IQ4XS, FMT_IQ4NL)   # the formats with a weight image
 EPILOGUE_NONE, EPILOGUE_RESIDUAL, EPILOGUE_GATE_UP, EPILOGUE_RESIDUAL_NORM = 0, 1, 2, 3
 # `prepared` of Linear.add: the table holds the input rows; or the table a residual + norm plan wrote, whose rows lack
 # their inverse RMS

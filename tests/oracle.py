@@ -6,7 +6,8 @@ import os
 import numpy as np
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-FMT_Q4K, FMT_Q5K, FMT_Q6K, FMT_Q80 = 0, 3, 4, 6
+FMT_Q4K, FMT_IQ4XS, FMT_IQ4NL, FMT_Q5K, FMT_Q6K, FMT_Q80 = 0, 1, 2, 3, 4, 6
+ALL_FORMATS = [("q4k", FMT_Q4K), ("q6k", FMT_Q6K), ("q5k", FMT_Q5K), ("q80", FMT_Q80), ("iq4xs", FMT_IQ4XS), ("iq4nl", FMT_IQ4NL)]
 NO_TOKEN = 0xFFFFFFFF
 
 _path = os.path.join(ROOT, "oracle", "liboracle.so")

@@ -33,19 +33,20 @@ def test_library_exports_every_declared_symbol():
 def test_kernels_are_registered_by_name():
     for name in ("gguf_prepare_table", "gguf_dequant_q4k", "gguf_dequant_q6k", "gguf_dequant_q5k", "gguf_dequant_q80",
                  "gguf_decode_q4k_m16_a", "gguf_decode_q6k_m16_a_f32", "gguf_decode_q4k_m32_g", "gguf_decode_q6k_m64_r",
-                 "gguf_decode_q5k_m16_gt", "gguf_decode_q80_m64_rn", "gguf_decode_mixed_m16_a", "gguf_decode_mixed_m64_a"):
+                 "gguf_decode_q5k_m16_gt", "gguf_decode_q80_m64_rn", "gguf_decode_mixed_m16_a", "gguf_decode_mixed_m64_a",
+                 "gguf_dequant_iq4xs", "gguf_decode_iq4xs_m16_rn", "gguf_decode_iq4nl_m32_gt", "gguf_embed_iq4xs", "gguf_embed_iq4nl"):
         assert splash_amd.lib.sp_kernel_exists(name.encode()), name
     assert not splash_amd.lib.sp_kernel_exists(b"no_such_kernel")
 
 
-@pytest.mark.parametrize("fmt", [ops.FMT_Q4K, ops.FMT_Q6K, ops.FMT_Q5K, ops.FMT_Q80])
+@pytest.mark.parametrize("fmt", ops.FORMATS)
 def test_image_is_a_permutation_of_the_native_rows(fmt):
     """decode(retile(native)) == decode(native) follows from unpack(pack(native)) == native."""
     native = orc.fixture(fmt, 48, 768, 5)
     image = ops.pack_gguf_image(fmt, native, 48, 768)
     assert image.size == native.size == ops.gguf_image_bytes(fmt, 48, 768)
     assert np.array_equal(ops.unpack_gguf_image(fmt, image, 48, 768), native)
-    if fmt == ops.FMT_Q4K:  # byte-for-byte re-ordering
+    if fmt in (ops.FMT_Q4K, ops.FMT_IQ4XS, ops.FMT_IQ4NL, ops.FMT_Q80):  # byte-for-byte re-ordering
         assert np.array_equal(np.sort(image), np.sort(native))
 
 

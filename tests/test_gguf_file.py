@@ -15,6 +15,8 @@ def model_file(path, alignment=32):
         ("blk.0.attn_v.weight", gw.GGML_Q6_K, [512, 32], orc.make_native(orc.FMT_Q6K, 32, 512, 2)),
         ("blk.0.ffn_down.weight", gw.GGML_Q5_K, [768, 64], orc.make_native(orc.FMT_Q5K, 64, 768, 3)),
         ("output.weight", gw.GGML_Q8_0, [512, 48], orc.make_native(orc.FMT_Q80, 48, 512, 4)),
+        ("blk.0.ffn_gate.weight", gw.GGML_IQ4_XS, [512, 64], orc.make_native(orc.FMT_IQ4XS, 64, 512, 5)),
+        ("blk.0.ffn_up.weight", gw.GGML_IQ4_NL, [512, 64], orc.make_native(orc.FMT_IQ4NL, 64, 512, 6)),
         ("blk.0.attn_norm.weight", gw.GGML_F32, [512], (1 + 0.1 * rng.standard_normal(512)).astype(np.float32)),
         ("output_norm.weight", gw.GGML_BF16, [512], orc.f32_to_bf16((1 + 0.1 * rng.standard_normal(512)).astype(np.float32))),
         ("blk.0.post_norm.weight", gw.GGML_F16, [512], (1 + 0.1 * rng.standard_normal(512)).astype(np.float16)),
@@ -40,8 +42,9 @@ def test_header_metadata_and_tensor_table(tmp_path, alignment):
     for got, (name, kind, dims, data) in zip(f.tensors, tensors):
         assert (got.ggml_type, got.dims, got.bytes) == (kind, dims, np.asarray(data).nbytes)
         assert np.array_equal(f.data(got), np.frombuffer(np.ascontiguousarray(data).tobytes(), np.uint8))
-    assert [f.find(n).format for n in ("blk.0.attn_q.weight", "blk.0.attn_v.weight", "blk.0.ffn_down.weight", "output.weight")] == \
-        [ops.FMT_Q4K, ops.FMT_Q6K, ops.FMT_Q5K, ops.FMT_Q80]
+    assert [f.find(n).format for n in ("blk.0.attn_q.weight", "blk.0.attn_v.weight", "blk.0.ffn_down.weight", "output.weight",
+                                       "blk.0.ffn_gate.weight", "blk.0.ffn_up.weight")] == \
+        [ops.FMT_Q4K, ops.FMT_Q6K, ops.FMT_Q5K, ops.FMT_Q80, ops.FMT_IQ4XS, ops.FMT_IQ4NL]
     assert f.find("output_norm.weight").format is None and f.find("nothing") is None
 
 
@@ -77,7 +80,8 @@ def test_projections_and_norms_load_from_a_file(backend, tmp_path):
     f = gguf.GgufFile(path)
     linear = ops.Linear(backend)
     rng = np.random.default_rng(8)
-    for name in ("blk.0.attn_q.weight", "blk.0.attn_v.weight", "blk.0.ffn_down.weight", "output.weight"):
+    for name in ("blk.0.attn_q.weight", "blk.0.attn_v.weight", "blk.0.ffn_down.weight", "output.weight", "blk.0.ffn_gate.weight",
+                 "blk.0.ffn_up.weight"):
         print(f"case gguf file tensor {name}", flush=True)
         _, _, (K, N), native = tensors[name]
         fmt, rows, input_size, image = f.load_image(backend, f.find(name))

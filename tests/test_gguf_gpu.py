@@ -24,10 +24,10 @@ def dequant_on_gpu(backend, fmt, native, rows, K):
     return out.download(np.float32).reshape(rows, K)
 
 
-ALL_FORMATS = [ops.FMT_Q4K, ops.FMT_Q6K, ops.FMT_Q5K, ops.FMT_Q80]
+ALL_FORMATS = list(ops.FORMATS)
 
 
-@pytest.mark.parametrize("name,fmt", [("q4k", ops.FMT_Q4K), ("q6k", ops.FMT_Q6K), ("q5k", ops.FMT_Q5K), ("q80", ops.FMT_Q80)])
+@pytest.mark.parametrize("name,fmt", orc.ALL_FORMATS)
 def test_image_dequantization_matches_ggml_golden_hash(backend, name, fmt):
     """gguf_reference_test.mm:23-30 + gguf_dequant_test.mm:44-58: the kernels' unpacking of the
     re-tiled image gives GGML's fp32 values bit for bit."""
@@ -168,7 +168,7 @@ def test_fused_segments_equal_each_alone(backend):
         at += n
 
 
-@pytest.mark.parametrize("formats", [(ops.FMT_Q4K, ops.FMT_Q4K, ops.FMT_Q6K), (ops.FMT_Q80, ops.FMT_Q5K, ops.FMT_Q6K),
+@pytest.mark.parametrize("formats", [(ops.FMT_Q4K, ops.FMT_Q4K, ops.FMT_Q6K), (ops.FMT_Q80, ops.FMT_Q5K, ops.FMT_Q6K), (ops.FMT_IQ4XS, ops.FMT_Q4K, ops.FMT_IQ4NL),
                                      (ops.FMT_Q6K, ops.FMT_Q4K)])
 @pytest.mark.parametrize("M", [16, 40, 80])
 def test_segments_of_several_formats_equal_each_alone(backend, formats, M):

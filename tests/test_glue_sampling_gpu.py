@@ -39,7 +39,7 @@ def test_rms_norm_and_its_activation_table(backend, rows, width):
     assert np.array_equal(table.download(), table2.download())
 
 
-@pytest.mark.parametrize("fmt", [ops.FMT_Q4K, ops.FMT_Q6K, ops.FMT_Q5K, ops.FMT_Q80])
+@pytest.mark.parametrize("fmt", ops.FORMATS)
 def test_embedding_gathers_native_rows(backend, fmt):
     """embedding.metal:10-18: bf16(decode(row)); a token past the vocabulary gives zeros."""
     vocab, hidden = 500, 1024

@@ -14,7 +14,7 @@ GOLDENS = json.load(open(os.path.join(HERE, "golden", "gguf_dequantization.json"
 ROWS, COLUMNS, SEED = 256, 1024, 7
 
 
-@pytest.mark.parametrize("name,fmt", [("q4k", orc.FMT_Q4K), ("q6k", orc.FMT_Q6K), ("q5k", orc.FMT_Q5K), ("q80", orc.FMT_Q80)])
+@pytest.mark.parametrize("name,fmt", orc.ALL_FORMATS)
 def test_dequant_matches_ggml_golden_hash(name, fmt):
     native = orc.fixture(fmt, ROWS, COLUMNS, SEED + fmt)
     values = orc.dequant_rows(fmt, native, ROWS, COLUMNS)
@@ -22,7 +22,7 @@ def test_dequant_matches_ggml_golden_hash(name, fmt):
 
 
 @pytest.mark.skipif(orc.ref is None, reason="oracle/_ref was not built (no reference tree)")
-@pytest.mark.parametrize("fmt", [orc.FMT_Q4K, orc.FMT_Q6K, orc.FMT_Q5K, orc.FMT_Q80])
+@pytest.mark.parametrize("fmt", [f for _, f in orc.ALL_FORMATS])
 def test_restatement_equals_compiled_reference(fmt):
     native = orc.fixture(fmt, 64, 1024, 99)
     assert np.array_equal(native, orc.fixture(fmt, 64, 1024, 99, library=orc.ref))
