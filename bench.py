@@ -303,6 +303,39 @@ def time_c5_ops(backend):
                       "expert_gbs": round(weights / float(med[3] + med[4]) / 1e3, 1)}}), flush=True)
 
 
+def time_state_codec(backend):
+    """The cached form of a lane's recurrent layers at the 35B-A3B shape (36 GDN layers of 32 value heads x 128 x 128 fp32,
+    75.5 MB a lane): quantize and dequantize over a ring of lanes' states past the caches, per-dispatch GPU time (HIP
+    events around each dispatch). Algorithmic bytes a value: 4 read + 1 + 2/32 written, and the reverse. Prints one JSON
+    line; not the headline metric."""
+    import splash_amd
+    from splash_amd import ops
+    rng = np.random.default_rng(0)
+    layers, rows, columns, copies = 36, 32 * 128, 128, 8
+    shape = ops.StateCodec.shape(layers, rows, columns)
+    state_bytes, codes_bytes = layers * rows * columns * 4, layers * ops.StateCodec.layer_bytes(rows, columns)
+    base = rng.standard_normal(state_bytes // 4).astype(np.float32)
+    states = [backend.from_array(base) for _ in range(copies)]
+    codes = [backend.allocate_buffer(codes_bytes) for _ in range(copies)]
+    graph = splash_amd.CommandGraph()
+    for _ in range(4):
+        for c in range(copies):
+            ops.StateCodec.add_quantize(graph, states[c], codes[c], shape)
+        for c in range(copies):
+            ops.StateCodec.add_dequantize(graph, codes[c], states[c], shape)
+    backend.set_dispatch_profiling(True)
+    _, _, per = backend.run(graph, profiled=True)
+    backend.set_dispatch_profiling(False)
+    per = np.array(per).reshape(4, 2, copies)[1:] * 1e6
+    moved = state_bytes + codes_bytes
+    result = {"ops": "state", "n_gpus": 1, "data": "synthetic", "workload": "36 layers x 4096 rows x 128 fp32 values a lane",
+              "bytes": moved}
+    for name, us in (("state_quantize", float(np.median(per[:, 0]))), ("state_dequantize", float(np.median(per[:, 1])))):
+        result[name] = {"us": round(us, 1), "achieved_gbs": round(moved / us / 1e3, 1), "frac": round(moved / us / 1e3 / HBM_PEAK_GBS, 4)}
+        log(f"  {name:16s} {us:7.1f} us {moved / us / 1e3:7.1f} GB/s")
+    print(json.dumps(result), flush=True)
+
+
 C5 = dict(hidden=2048, vocabulary=151936, layers=48, q_heads=32, kv_heads=4, head_dim=128, gdn_key_heads=16, gdn_value_heads=32,
           experts=128, top_k=8, expert_ffn=768, context=16384, rows=16, lanes=8,
           name="35B-A3B-shaped hybrid MoE verify step: 36 GDN + 12 attention layers, 128 experts top-8 (Q4_K), 16-token draft, "
@@ -416,9 +449,9 @@ def main():
     ap.add_argument("--temperature", type=float, default=0.0,
                     help="above 0: rejection-sampling acceptance at this temperature against a full-vocabulary draft "
                          "distribution softmax(N(0, 2)) instead of greedy acceptance")
-    ap.add_argument("--ops", choices=["c2", "c3", "c5"],
+    ap.add_argument("--ops", choices=["c2", "c3", "c5", "state"],
                     help="instead of the dense step: c2 the projections alone by rows, c3 attention alone by context, "
-                         "c5 the GDN step and the MoE layer of config 5")
+                         "c5 the GDN step and the MoE layer of config 5, state the recurrent layers' cached form")
     args = ap.parse_args()
     if args.gpus != 1:
         log("bench.py measures one GPU: this build runs the verify step on a single MI355X (no collectives); use --gpus 1")
@@ -427,7 +460,7 @@ def main():
     from splash_amd import ops, verify
     backend = splash_amd.Backend(0)
     if args.ops:
-        {"c2": time_c2_ops, "c3": time_c3_ops, "c5": time_c5_ops}[args.ops](backend)
+        {"c2": time_c2_ops, "c3": time_c3_ops, "c5": time_c5_ops, "state": time_state_codec}[args.ops](backend)
         return
     if args.workload == "c5":
         bench_c5(backend, args)

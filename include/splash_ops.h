@@ -202,6 +202,20 @@ sp_status spo_gdn_add_fold(spo_graph *graph, sp_buffer *states, sp_buffer *tape,
                            uint64_t state_cell, uint64_t fold_cell, const spo_gdn_shape *shape, uint32_t layers, uint32_t rows,
                            const spo_gdn_state_strides *state);
 
+/* ---- StateCodec (runtime/ops/StateCodec.hpp:11-49; runtime/metal/abi/StateCodec.h): the cached form of the
+ *      recurrent layers, int8 codes row by row and then a bf16 scale per block of 32 values ---- */
+typedef struct spo_state_codec_shape { /* ops::StateCodecShape (StateCodec.hpp:17-34) */
+  uint32_t layers, rows, columns; /* a layer's value rows (every value head's) of `columns` values, a multiple of 32 */
+  uint32_t bf16_state;            /* the running state holds bf16 values (GdnStateFormat::BFloat16), else fp32 */
+  uint64_t state_layer_bytes, codes_layer_bytes; /* between consecutive layers of the running and of the cached state */
+} spo_state_codec_shape;
+/* state_codec_layer_bytes (abi/StateCodec.h:31-33): a cached layer's bytes. */
+uint64_t spo_state_codec_layer_bytes(uint32_t rows, uint32_t columns);
+/* StateCodec::addQuantize / addDequantize / addCopy (StateCodec.hpp:41-48); the buffers start at the first layer. */
+sp_status spo_state_codec_add_quantize(spo_graph *graph, sp_buffer *state, sp_buffer *codes, const spo_state_codec_shape *shape);
+sp_status spo_state_codec_add_dequantize(spo_graph *graph, sp_buffer *codes, sp_buffer *state, const spo_state_codec_shape *shape);
+sp_status spo_state_codec_add_copy(spo_graph *graph, sp_buffer *from, sp_buffer *to, const spo_state_codec_shape *shape);
+
 /* ---- MoE (runtime/ops/MoE.hpp:403-410, MoE.cpp:143-287; runtime/metal/abi/MoE.h:23-245) ---- */
 typedef struct spo_moe_shape { uint32_t hidden, ffn, experts, top_k; } spo_moe_shape;
 typedef struct spo_moe_workspace { /* in the order of spo_moe_workspace_sizes */

@@ -26,6 +26,8 @@
 //   orc_distribution_end            pinned by an independent fp64 sort (min_p, top_k with ties, nucleus).
 //   orc_moe_*                       pinned by a stable sort and softmax closed form; the layer by the dense FFN it
 //                                   reduces to when every expert is the same.
+//   orc_state_codes / _values       pinned: the compiled reference header (oracle/_ref, StateCodecReference.hpp) bit for
+//                                   bit, and the closed form (a value restores within half its block's step).
 #pragma once
 #include <stddef.h>
 #include <stdint.h>
@@ -192,6 +194,12 @@ void orc_moe_route(const float *scores, uint32_t rows, uint32_t experts, uint32_
 // y bf16 [rows][top_k][hidden] the expert outputs of the routes.
 void orc_moe_combine(const uint16_t *y, const float *weights, const uint16_t *residual, uint32_t rows, uint32_t top_k,
                      uint32_t hidden, uint16_t *out);
+
+// ---- the cached form of Gated DeltaNet recurrent layers (runtime/ops/StateCodec.hpp, metal/abi/StateCodec.h) ----
+// A layer of `rows` value rows of `columns` values: int8 codes row by row, then a bf16 scale per block of 32.
+uint64_t orc_state_codec_bytes(uint32_t rows, uint32_t columns);
+int orc_state_codes(const float *values, uint32_t rows, uint32_t columns, uint8_t *image);
+int orc_state_values(const uint8_t *image, uint32_t rows, uint32_t columns, float *values);
 
 #ifdef __cplusplus
 }

@@ -4,6 +4,7 @@
 // when it is there and skips the cross-check when it is not.
 #include "GgufFormatReference.hpp"
 #include "Q8PageFormatReference.hpp"
+#include "StateCodecReference.hpp"
 
 #include <cstdint>
 #include <random>
@@ -52,4 +53,11 @@ void ref_dot_bound(const float *x, const float *w, uint32_t K, double *value, do
 float ref_kv_scale(float maximum) { return splash::kv::reference_detail::storedScale(maximum); }
 int ref_kv_code(float value, float maximum) { return splash::kv::reference_detail::quantize(value, maximum); }
 
+
+// StateCodecReference.hpp:38-61
+int ref_state_codes(const float *values, uint32_t rows, uint32_t columns, uint8_t *image) {
+  const std::vector<uint8_t> v = splash::test::stateCodesReference(values, rows, columns);
+  std::copy(v.begin(), v.end(), image);
+  return 0;
+}
 }

@@ -109,6 +109,11 @@ class GdnDecodeBuffers(ctypes.Structure):
                                    "hidden")] + [("float_norm", c_u32), ("tree_rows", c_p), ("hidden_table", c_p)]
 
 
+class StateCodecShape(ctypes.Structure):
+    _fields_ = [("layers", c_u32), ("rows", c_u32), ("columns", c_u32), ("bf16_state", c_u32), ("state_layer_bytes", c_u64),
+                ("codes_layer_bytes", c_u64)]
+
+
 class MoeShape(ctypes.Structure):
     _fields_ = [("hidden", c_u32), ("ffn", c_u32), ("experts", c_u32), ("top_k", c_u32)]
 
@@ -243,6 +248,9 @@ _sig("spo_rope_add_tree_tables", c_int, c_p, c_p, c_p, c_p, c_p, c_u32, P(RopeSe
 _sig("spo_gdn_layout", c_int, P(GdnShape), c_u32, P(GdnStateStrides), P(c_u64), P(c_u64))
 _sig("spo_gdn_add_decode", c_int, c_p, P(GdnDecodeBuffers), P(GdnShape), c_u32, P(GdnStateStrides), c_u32, P(GdnLane), c_u32)
 _sig("spo_gdn_add_fold", c_int, c_p, c_p, c_p, c_p, c_u64, c_u64, c_u64, P(GdnShape), c_u32, c_u32, P(GdnStateStrides))
+_sig("spo_state_codec_layer_bytes", c_u64, c_u32, c_u32)
+for _name in ("spo_state_codec_add_quantize", "spo_state_codec_add_dequantize", "spo_state_codec_add_copy"):
+    _sig(_name, c_int, c_p, c_p, c_p, P(StateCodecShape))
 _sig("spo_moe_workspace_sizes", c_int, P(MoeShape), c_u32, P(c_u64))
 _sig("spo_moe_add_routing", c_int, c_p, c_p, c_u32, P(MoeWorkspace), P(MoeShape), c_u32)
 _sig("spo_moe_add_routed", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_u32, c_u32, P(MoeWorkspace), P(MoeShape), c_u32)

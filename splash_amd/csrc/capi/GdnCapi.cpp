@@ -2,6 +2,7 @@
 #include "capi/Guard.hpp"
 #include "capi/Handles.hpp"
 #include "ops/Gdn.hpp"
+#include "ops/StateCodec.hpp"
 #include "splash_ops.h"
 
 using namespace splash;
@@ -63,4 +64,32 @@ sp_status spo_gdn_add_fold(spo_graph *graph, sp_buffer *states, sp_buffer *tape,
   });
 }
 
+
+uint64_t spo_state_codec_layer_bytes(uint32_t rows, uint32_t columns) { return state_codec_layer_bytes(rows, columns); }
+
+namespace {
+ops::StateCodecShape codecShapeOf(const spo_state_codec_shape &s) {
+  return {s.layers, s.rows, s.columns, s.state_layer_bytes, s.codes_layer_bytes,
+          s.bf16_state ? ops::GdnStateFormat::BFloat16 : ops::GdnStateFormat::Float32};
+}
+} // namespace
+
+sp_status spo_state_codec_add_quantize(spo_graph *graph, sp_buffer *state, sp_buffer *codes, const spo_state_codec_shape *shape) {
+  return capi::guard([&] {
+    capi::require(graph && shape, "graph or shape");
+    ops::StateCodec::addQuantize(capi::graphOf(graph), B(state), B(codes), codecShapeOf(*shape));
+  });
+}
+sp_status spo_state_codec_add_dequantize(spo_graph *graph, sp_buffer *codes, sp_buffer *state, const spo_state_codec_shape *shape) {
+  return capi::guard([&] {
+    capi::require(graph && shape, "graph or shape");
+    ops::StateCodec::addDequantize(capi::graphOf(graph), B(codes), B(state), codecShapeOf(*shape));
+  });
+}
+sp_status spo_state_codec_add_copy(spo_graph *graph, sp_buffer *from, sp_buffer *to, const spo_state_codec_shape *shape) {
+  return capi::guard([&] {
+    capi::require(graph && shape, "graph or shape");
+    ops::StateCodec::addCopy(capi::graphOf(graph), B(from), B(to), codecShapeOf(*shape));
+  });
+}
 } // extern "C"

@@ -278,6 +278,35 @@ class PagedAttention:
         graph._keep.extend([plan, retained, pages])
 
 
+class StateCodec:
+    """ops::StateCodec: a running state's recurrent layers as int8 codes with a bf16 scale per block of 32 values."""
+
+    @staticmethod
+    def layer_bytes(rows, columns):
+        return lib.spo_state_codec_layer_bytes(rows, columns)
+
+    @staticmethod
+    def shape(layers, rows, columns, state_layer_bytes=None, codes_layer_bytes=None, bf16_state=False):
+        state = rows * columns * (2 if bf16_state else 4)
+        return nat.StateCodecShape(layers, rows, columns, int(bf16_state), state if state_layer_bytes is None else state_layer_bytes,
+                                   StateCodec.layer_bytes(rows, columns) if codes_layer_bytes is None else codes_layer_bytes)
+
+    @staticmethod
+    def add_quantize(graph, state, codes, shape):
+        check(lib.spo_state_codec_add_quantize(graph.handle, state.handle, codes.handle, ctypes.byref(shape)))
+        graph._keep.extend([state, codes])
+
+    @staticmethod
+    def add_dequantize(graph, codes, state, shape):
+        check(lib.spo_state_codec_add_dequantize(graph.handle, codes.handle, state.handle, ctypes.byref(shape)))
+        graph._keep.extend([state, codes])
+
+    @staticmethod
+    def add_copy(graph, source, destination, shape):
+        check(lib.spo_state_codec_add_copy(graph.handle, source.handle, destination.handle, ctypes.byref(shape)))
+        graph._keep.extend([source, destination])
+
+
 def chain_tree_rows(rows_per_sequence):
     """SplashTreeRow of chains: ancestors (2 << r) - 1, parent r - 1, depth r, packed per sequence."""
     out = []

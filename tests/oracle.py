@@ -476,3 +476,26 @@ def moe_layer(x_bits, residual_bits, scores, top_k, gate_native, up_native, down
         down = gemm(down_fmt, down_native[e], mid, hidden, want=("chain",))["chain"]
         y[r, k] = f32_to_bf16(down)
     return selected, weights, y, moe_combine(y, weights, residual_bits)
+
+
+# ---- the cached form of recurrent layers ----
+def state_codec_bytes(rows, columns):
+    lib.orc_state_codec_bytes.restype = ctypes.c_uint64
+    return lib.orc_state_codec_bytes(c_u32(rows), c_u32(columns))
+
+
+def state_codes(values, library=None):
+    """fp32 [rows][columns] -> the layer's codes and scales (uint8)."""
+    values = np.ascontiguousarray(values, dtype=np.float32)
+    rows, columns = values.shape
+    image = np.zeros(state_codec_bytes(rows, columns), dtype=np.uint8)
+    fn = (library or lib).ref_state_codes if library is not None else lib.orc_state_codes
+    assert fn(_p(values, f32p), c_u32(rows), c_u32(columns), _p(image, u8p)) == 0
+    return image
+
+
+def state_values(image, rows, columns):
+    image = np.ascontiguousarray(image, dtype=np.uint8)
+    values = np.empty((rows, columns), dtype=np.float32)
+    assert lib.orc_state_values(_p(image, u8p), c_u32(rows), c_u32(columns), _p(values, f32p)) == 0
+    return values
