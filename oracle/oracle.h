@@ -22,6 +22,8 @@
 //                                   the reference's own test makes) and fold/rollback invariants; tree
 //                                   blocks by the same recurrence along each row's path.
 //   orc_argmax / orc_accept_tree    pinned by brute force on tiny vocabularies.
+//   orc_penalize                    pinned by a brute-force restatement over explicit path contexts (tests) and the
+//                                   closed cases of the reference's test (prompt-only, saturation, unselectable).
 //   orc_rejection_*                 pinned by enumeration: selection law equals target to 1e-12.
 //   orc_distribution_end            pinned by an independent fp64 sort (min_p, top_k with ties, nucleus).
 //   orc_moe_*                       pinned by a stable sort and softmax closed form; the layer by the dense FFN it
@@ -124,6 +126,11 @@ struct OrcTreeRow { uint32_t ancestors; uint16_t parent; uint16_t depth; };
 uint32_t orc_accept_tree(const struct OrcTreeRow *tree, const uint32_t *tokens, const uint32_t *selected,
                          uint32_t rows, uint32_t remaining, const uint32_t *stop_tokens, uint32_t stops,
                          uint32_t *out_tokens, uint32_t *accepted, uint32_t *retained_rows);
+// sampling.metal:991-1051 decode_sample_penalize for one lane's block: logits fp32 [rows][stride] rewritten in place
+// from the lane's penalty words [vocab] (bit 31: a prompt token; the rest: the output's count), its input tokens and
+// tree rows. frequency * count, + presence and the subtraction each round once (no fused multiply-add).
+void orc_penalize(float *logits, uint32_t rows, uint32_t vocab, uint32_t stride, const uint32_t *words, const uint32_t *inputs,
+                  const struct OrcTreeRow *tree, float repetition, float presence, float frequency);
 // One sampled verify row under the textbook full-vocabulary rule in the reference's order of
 // operations (sampling.metal:713-885): weight_t = exp((logit_t - max) / T); p = weight / total;
 // accept the drafted token iff u_child * q[draft] < p[draft]; else draw from max(p - q, 0)

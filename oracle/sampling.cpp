@@ -136,6 +136,32 @@ void note(double *closeness, double value, double threshold) {
 extern "C" {
 
 // sampling.metal:1896-1997: larger value, ties to the lowest id, NaN and -inf skipped.
+void orc_penalize(float *logits, uint32_t rows, uint32_t vocab, uint32_t stride, const uint32_t *words, const uint32_t *inputs,
+                  const struct OrcTreeRow *tree, float repetition, float presence, float frequency) {
+  const float largest = std::numeric_limits<float>::max();
+  const float inverse = std::min(1.0f / repetition, largest);   // Sampling.cpp:147-149
+  for (uint32_t token = 0; token < vocab; ++token) {
+    uint32_t drafted = 0;
+    for (uint32_t row = 1; row < rows; ++row) drafted |= uint32_t(inputs[row] == token) << row;
+    const uint32_t word = words[token];
+    if (!word && !drafted) continue;
+    for (uint32_t row = 0; row < rows; ++row) {
+      const uint32_t count = (word & 0x7FFFFFFFu) + uint32_t(__builtin_popcount(drafted & tree[row].ancestors & ~1u));
+      if (!count && !(word & 0x80000000u)) continue;
+      float &logit = logits[size_t(row) * stride + token];
+      uint32_t bits; std::memcpy(&bits, &logit, 4);
+      if ((bits & 0x7FFFFFFFu) > 0x7F800000u || bits == 0xFF800000u) continue;   // unselectable: NaN or -infinity
+      float value = logit * (logit > 0.0f ? inverse : repetition);
+      if (count) {
+        const float product = frequency * float(count);
+        const float lowered = product + presence;
+        value = value - lowered;
+      }
+      logit = std::min(std::max(value, -largest), largest);
+    }
+  }
+}
+
 uint32_t orc_argmax(const float *logits, uint32_t vocab) {
   float best = -std::numeric_limits<float>::infinity();
   uint32_t index = ORC_NO_TOKEN;

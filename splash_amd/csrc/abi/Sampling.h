@@ -49,6 +49,27 @@ struct TargetSamplingParams {
   uint32_t reserved[3];
 };
 
+// A token's word of a penalty table row (Sampling.h:121-125 in the reference): the prompt bit marks a prompt token, the
+// count is how often the target selected the token.
+#define SAMPLING_PENALTY_PROMPT_BIT 0x80000000u
+#define SAMPLING_PENALTY_COUNT_MASK 0x7FFFFFFFu
+
+// decode_sample_penalize: grid (ceil(vocabulary / 256), entries), 256 threads. Entry e rewrites the logits rows of
+// lane[e] from row table_row[e] of the penalty table (the reference's SamplingPenaltyParams, abi/Sampling.h:127-142).
+// repetition_inverse is 1 / repetition, saturated to the largest float.
+struct SamplingPenaltyParams {
+  uint32_t vocabulary;
+  uint32_t entries;
+  uint32_t logits_stride;  // floats between logits rows
+  uint32_t reserved;
+  struct SamplingLaneRows lane[SAMPLING_MAXIMUM_LANES];
+  uint32_t table_row[SAMPLING_MAXIMUM_LANES];
+  float repetition[SAMPLING_MAXIMUM_LANES];
+  float repetition_inverse[SAMPLING_MAXIMUM_LANES];
+  float presence[SAMPLING_MAXIMUM_LANES];
+  float frequency[SAMPLING_MAXIMUM_LANES];
+};
+
 // decode_accept_tree: one thread per lane (AcceptBatchParams).
 struct AcceptBatchParams {
   uint32_t lanes;
@@ -60,5 +81,6 @@ struct AcceptBatchParams {
 
 #ifdef __cplusplus
 static_assert(sizeof(TargetSamplingParams) == 16 + 32 + 16 + 64 + 96 + 32, "target sampling parameters are 256 bytes on both sides");
+static_assert(sizeof(SamplingPenaltyParams) == 16 + 64 + 5 * 32, "penalty parameters are 240 bytes on both sides");
 static_assert(sizeof(AcceptBatchParams) == 16 + 32 + 16 + 64, "acceptance parameters are 128 bytes on both sides");
 #endif

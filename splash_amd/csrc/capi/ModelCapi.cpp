@@ -110,6 +110,34 @@ sp_status spo_sampling_add_acceptance(spo_graph *graph, sp_buffer *input_tokens,
   });
 }
 
+sp_status spo_sampling_rebuild_penalty_words(uint32_t *words, uint32_t vocabulary, const uint32_t *history, uint64_t history_tokens,
+                                             uint64_t generated_tokens, uint32_t pending_token, int mark_prompt) {
+  return capi::guard([&] {
+    capi::require(words && history, "words or history");
+    ops::Sampling::rebuildPenaltyWords({words, vocabulary}, {history, size_t(history_tokens)}, generated_tokens,
+                                       pending_token == SAMPLING_NO_TOKEN ? std::nullopt : std::optional<uint32_t>(pending_token),
+                                       mark_prompt != 0);
+  });
+}
+sp_status spo_sampling_count_penalty_tokens(uint32_t *words, uint32_t vocabulary, const uint32_t *selected, uint64_t count) {
+  return capi::guard([&] {
+    capi::require(words && (selected || !count), "words or selected tokens");
+    ops::Sampling::countPenaltyTokens({words, vocabulary}, {selected, size_t(count)});
+  });
+}
+sp_status spo_sampling_add_penalties(spo_graph *graph, sp_buffer *logits, sp_buffer *words, sp_buffer *input_tokens,
+                                     sp_buffer *tree_rows, uint32_t vocabulary, uint32_t logits_stride, const spo_lane_rows *lanes,
+                                     const spo_sampling_penalties *penalties, uint32_t count) {
+  return capi::guard([&] {
+    capi::require(graph && lanes && penalties, "graph, lanes or penalties");
+    std::vector<ops::PenalizedLane> list;
+    for (uint32_t i = 0; i < count; ++i)
+      list.push_back({{lanes[i].first, lanes[i].rows}, penalties[i].table_row,
+                      {penalties[i].repetition, penalties[i].presence, penalties[i].frequency}});
+    ops::Sampling::addPenalties(capi::graphOf(graph), B(logits), B(words), B(input_tokens), B(tree_rows), vocabulary, logits_stride, list);
+  });
+}
+
 sp_status spo_dense_verify_create(sp_backend *backend, const spo_dense_dimensions *d, uint32_t max_lanes, uint32_t physical_pages,
                                   uint32_t page_table_entries, spo_dense_verify **out) {
   return capi::guard([&] {

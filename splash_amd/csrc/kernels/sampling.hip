@@ -29,6 +29,8 @@
 #include "backend/KernelRegistry.hpp"
 #include "kernels/device_common.hpp"
 
+#include <cfloat>
+
 namespace splash::kernels {
 
 __device__ __forceinline__ bool unselectable(float v) { return !(v > -INFINITY); }  // NaN or -inf (sampling.metal:986-989)
@@ -77,6 +79,42 @@ __global__ __launch_bounds__(256) void decode_sample_admit(float *__restrict__ l
   }
 }
 SP_REGISTER_KERNEL("decode_sample_admit", &decode_sample_admit);
+
+// The sampling penalties of one logit (sampling.metal:991-1008): repetition divides a positive logit and multiplies a
+// negative one when the prompt or the output holds the token; presence and frequency lower it by the output's count of
+// the token. The result saturates, so no rewritten logit is infinite; an unselectable logit stays as it is.
+__device__ __forceinline__ float penalize_logit(float value, uint32_t count, float repetition, float repetition_inverse,
+                                                float presence, float frequency) {
+  if (unselectable(value)) return value;
+  value *= value > 0.0f ? repetition_inverse : repetition;
+  if (count) value -= frequency * float(count) + presence;
+  return fminf(fmaxf(value, -FLT_MAX), FLT_MAX);
+}
+// decode_sample_penalize (sampling.metal:1016-1051): one thread per vocabulary token and entry, the entry's lane's
+// logits rewritten in place. A row's context adds the draft tokens of its path: bit r of `drafted` is set when the
+// lane's input row r holds the token, which the rows below row r in the block's tree add to the output; a row counts
+// the bits of its ancestors but its anchor on top of the table's count.
+__global__ __launch_bounds__(256) void decode_sample_penalize(float *__restrict__ logits, const uint32_t *__restrict__ words,
+                                                              const uint32_t *__restrict__ input_tokens,
+                                                              const AttentionTreeRow *__restrict__ tree, SamplingPenaltyParams p) {
+  const uint32_t token = blockIdx.x * 256u + threadIdx.x, entry = blockIdx.y;
+  if (token >= p.vocabulary) return;
+  const SamplingLaneRows lane = p.lane[entry];
+  const uint32_t *inputs = input_tokens + lane.first;
+  uint32_t drafted = 0;
+  for (uint32_t row = 1; row < lane.rows; ++row) drafted |= uint32_t(inputs[row] == token) << row;
+  const uint32_t word = words[size_t(p.table_row[entry]) * p.vocabulary + token];
+  if (!word && !drafted) return;
+  float *column = logits + size_t(lane.first) * p.logits_stride + token;
+  for (uint32_t row = 0; row < lane.rows; ++row) {
+    const uint32_t path = tree[lane.first + row].ancestors;
+    const uint32_t count = (word & SAMPLING_PENALTY_COUNT_MASK) + uint32_t(__popc(drafted & path & ~1u));
+    if (!count && !(word & SAMPLING_PENALTY_PROMPT_BIT)) continue;
+    float &logit = column[size_t(row) * p.logits_stride];
+    logit = penalize_logit(logit, count, p.repetition[entry], p.repetition_inverse[entry], p.presence[entry], p.frequency[entry]);
+  }
+}
+SP_REGISTER_KERNEL("decode_sample_penalize", &decode_sample_penalize);
 
 // Grid (rows * SAMPLING_SHARDS), 256 threads. partial_values/indices [row][shard].
 __global__ __launch_bounds__(256) void decode_sample_argmax_sharded(const float *__restrict__ logits, float *__restrict__ partial_values,

@@ -3,6 +3,8 @@
 #include "ops/Linear.hpp"  // requireBytes
 
 #include <algorithm>
+#include <cmath>
+#include <limits>
 #include <stdexcept>
 
 namespace splash::ops {
@@ -18,6 +20,62 @@ uint32_t packedRows(const std::vector<LaneRows> &lanes) {
   return rows;
 }
 } // namespace
+
+void Sampling::rebuildPenaltyWords(std::span<uint32_t> words, std::span<const uint32_t> history, uint64_t generatedTokens,
+                                   std::optional<uint32_t> pendingToken, bool markPrompt) {
+  if (history.size() <= generatedTokens) throw std::logic_error("request history holds no prompt");
+  const auto inside = [&](uint32_t token) {
+    if (token >= words.size()) throw std::invalid_argument("penalty token is outside the vocabulary");
+  };
+  for (uint32_t token : history) inside(token);
+  if (pendingToken) inside(*pendingToken);
+  const size_t prompt = history.size() - generatedTokens;
+  std::fill(words.begin(), words.end(), 0u);
+  if (markPrompt)
+    for (size_t i = 0; i < prompt; ++i) words[history[i]] |= SAMPLING_PENALTY_PROMPT_BIT;
+  for (size_t i = prompt; i < history.size(); ++i) ++words[history[i]];
+  if (pendingToken) ++words[*pendingToken];
+}
+
+void Sampling::countPenaltyTokens(std::span<uint32_t> words, std::span<const uint32_t> selected) {
+  for (uint32_t token : selected)
+    if (token >= words.size()) throw std::invalid_argument("penalty token is outside the vocabulary");
+  for (uint32_t token : selected) ++words[token];
+}
+
+void Sampling::addPenalties(hip::CommandGraph &graph, const hip::Buffer &logits, const hip::Buffer &words,
+                            const hip::Buffer &inputTokens, const hip::Buffer &treeRows, uint32_t vocabulary, uint32_t logitsStride,
+                            const std::vector<PenalizedLane> &lanes) {
+  if (!vocabulary || logitsStride < vocabulary) throw std::invalid_argument("logits rows hold the vocabulary");
+  std::vector<LaneRows> rowsOf;
+  for (const PenalizedLane &l : lanes) rowsOf.push_back(l.rows);
+  const uint32_t rows = packedRows(rowsOf);
+  SamplingPenaltyParams params{};
+  params.vocabulary = vocabulary;
+  params.logits_stride = logitsStride;
+  for (const PenalizedLane &l : lanes) {
+    if (!l.penalties.active()) continue;
+    if (!(l.penalties.repetition > 0.0f) || !std::isfinite(l.penalties.repetition) || !std::isfinite(l.penalties.presence) ||
+        !std::isfinite(l.penalties.frequency))
+      throw std::invalid_argument("a repetition penalty is positive and every penalty finite");
+    // the kernel indexes the whole table by this row
+    requireBytes(words, (uint64_t{l.tableRow} + 1) * vocabulary * 4, "penalty table");
+    const uint32_t entry = params.entries++;
+    params.lane[entry] = {l.rows.first, l.rows.rows};
+    params.table_row[entry] = l.tableRow;
+    params.repetition[entry] = l.penalties.repetition;
+    // 1 / 2^-149 overflows; the saturated inverse keeps the product finite
+    params.repetition_inverse[entry] = std::min(1.0f / l.penalties.repetition, std::numeric_limits<float>::max());
+    params.presence[entry] = l.penalties.presence;
+    params.frequency[entry] = l.penalties.frequency;
+  }
+  if (!params.entries) return;
+  requireBytes(logits, (uint64_t{rows - 1} * logitsStride + vocabulary) * 4, "logits");
+  requireBytes(treeRows, uint64_t{rows} * sizeof(AttentionTreeRow), "verify tree rows");
+  requireBytes(inputTokens, uint64_t{rows} * 4, "input tokens");
+  graph.add("decode_sample_penalize", {logits, words, inputTokens, treeRows}, params, {(vocabulary + 255) / 256, params.entries, 1},
+            {256, 1, 1});
+}
 
 SamplingWorkspaceSize Sampling::workspace(uint32_t rows) noexcept {
   SamplingWorkspaceSize size;

@@ -8,6 +8,8 @@
 #include "hip/Backend.hpp"
 
 #include <array>
+#include <optional>
+#include <span>
 #include <vector>
 
 namespace splash::ops {
@@ -30,6 +32,16 @@ struct SamplingPolicy final {
   [[nodiscard]] bool truncates(uint32_t vocabulary) const noexcept {
     return samples() && (minP > 0.0f || (topK && topK < vocabulary) || topP < 1.0f);
   }
+};
+
+// The sampling penalties, which rewrite a lane's target logits before its policy selects from them (the reference's
+// SamplingPenalties, runtime/ops/Sampling.hpp:17-29): repetition scales the logit of every token the prompt or the
+// output holds, presence and frequency lower that of every token the output holds. The defaults change nothing.
+struct SamplingPenalties final {
+  float repetition = 1.0f;
+  float presence = 0.0f;
+  float frequency = 0.0f;
+  [[nodiscard]] bool active() const noexcept { return repetition != 1.0f || presence != 0.0f || frequency != 0.0f; }
 };
 
 struct LaneRows final {
@@ -62,8 +74,28 @@ struct AcceptanceBuffers final {
   hip::Buffer retainedRows;   // uint32 [lanes]: mask of the block rows retained
 };
 
+// A lane whose logits rows the penalties rewrite, from row `tableRow` of the penalty table.
+struct PenalizedLane final {
+  LaneRows rows;
+  uint32_t tableRow = 0;
+  SamplingPenalties penalties;
+};
+
 class Sampling final {
 public:
+  // A request's penalty words (abi/Sampling.h), rebuilt from its history of prompt and generated tokens: the prompt
+  // bit on every prompt token (markPrompt), the count of every generated token and of a pending one
+  // (Sampling.cpp:91-114 in the reference). Throws for a token outside the vocabulary (words.size()).
+  static void rebuildPenaltyWords(std::span<uint32_t> words, std::span<const uint32_t> history, uint64_t generatedTokens,
+                                  std::optional<uint32_t> pendingToken, bool markPrompt);
+  // Counts the tokens one step selected into a request's penalty words (Sampling.cpp:116-121).
+  static void countPenaltyTokens(std::span<uint32_t> words, std::span<const uint32_t> selected);
+  // Rewrites the logits rows of the lanes whose penalties are active, in place, before addVerify reads them
+  // (Sampling::addPenalties, Sampling.cpp:129-172): `words` holds uint32 [table rows][vocabulary]; a row of a lane also
+  // counts the draft tokens of its path, from the block's input tokens and tree rows. Nothing when no lane is active.
+  static void addPenalties(hip::CommandGraph &graph, const hip::Buffer &logits, const hip::Buffer &words,
+                           const hip::Buffer &inputTokens, const hip::Buffer &treeRows, uint32_t vocabulary,
+                           uint32_t logitsStride, const std::vector<PenalizedLane> &lanes);
   [[nodiscard]] static SamplingWorkspaceSize workspace(uint32_t rows) noexcept;
   // One policy per lane. Throws for no or too many lanes, rows outside 1..16, or missing buffers.
   // The logits rows of a constrained or stop-excluding lane are rewritten first: -infinity at the

@@ -434,6 +434,32 @@ class Sampling:
         return list(sizes)
 
     @staticmethod
+    def rebuild_penalty_words(vocabulary, history, generated_tokens, pending_token=None, mark_prompt=True):
+        """Sampling::rebuildPenaltyWords: a request's penalty words (uint32 [vocabulary]) from its history."""
+        words = np.zeros(vocabulary, dtype=np.uint32)
+        history = np.ascontiguousarray(history, dtype=np.uint32)
+        check(lib.spo_sampling_rebuild_penalty_words(words.ctypes.data_as(ctypes.POINTER(ctypes.c_uint32)), vocabulary,
+                                                     history.ctypes.data_as(ctypes.POINTER(ctypes.c_uint32)), len(history),
+                                                     generated_tokens, 0xFFFFFFFF if pending_token is None else pending_token,
+                                                     int(mark_prompt)))
+        return words
+
+    @staticmethod
+    def count_penalty_tokens(words, selected):
+        selected = np.ascontiguousarray(selected, dtype=np.uint32)
+        check(lib.spo_sampling_count_penalty_tokens(words.ctypes.data_as(ctypes.POINTER(ctypes.c_uint32)), len(words),
+                                                    selected.ctypes.data_as(ctypes.POINTER(ctypes.c_uint32)), len(selected)))
+
+    @staticmethod
+    def add_penalties(graph, logits, words, input_tokens, tree_rows, vocabulary, stride, lanes, penalties):
+        """lanes: [(first, rows)]; penalties: a lane's (repetition, presence, frequency, table_row)."""
+        rows = (nat.LaneRows * len(lanes))(*[nat.LaneRows(f, r) for f, r in lanes])
+        entries = (nat.SamplingPenalties * len(lanes))(*[nat.SamplingPenalties(*p) for p in penalties])
+        check(lib.spo_sampling_add_penalties(graph.handle, logits.handle, words.handle, input_tokens.handle, tree_rows.handle,
+                                             vocabulary, stride, rows, entries, len(lanes)))
+        graph._keep.extend([logits, words, input_tokens, tree_rows])
+
+    @staticmethod
     def add_verify(graph, buffers, vocabulary, stride, lanes, policies, stop_tokens=None):
         """buffers: dict of Buffer by the names of spo_sampling_buffers (token_mask with mask_words for constrained
         lanes); lanes: [(first, rows)]; policies: a lane's temperature, or (temperature, min_p, top_k, top_p[,

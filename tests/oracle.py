@@ -499,3 +499,16 @@ def state_values(image, rows, columns):
     values = np.empty((rows, columns), dtype=np.float32)
     assert lib.orc_state_values(_p(image, u8p), c_u32(rows), c_u32(columns), _p(values, f32p)) == 0
     return values
+
+
+def penalize(logits, words, inputs, tree, repetition, presence, frequency):
+    """decode_sample_penalize for one lane's block: fp32 [rows][vocab] -> the rewritten rows."""
+    out = np.ascontiguousarray(logits, dtype=np.float32).copy()
+    rows, vocab = out.shape
+    words = np.ascontiguousarray(words, dtype=np.uint32)
+    inputs = np.ascontiguousarray(inputs, dtype=np.uint32)
+    tree = np.ascontiguousarray(tree)
+    lib.orc_penalize.restype = None
+    lib.orc_penalize(_p(out, f32p), c_u32(rows), c_u32(vocab), c_u32(vocab), _p(words, u32p), _p(inputs, u32p),
+                     tree.ctypes.data_as(ctypes.c_void_p), c_f(repetition), c_f(presence), c_f(frequency))
+    return out

@@ -76,3 +76,24 @@ def test_linear_plans_without_a_device():
         linear.scratch_size(5120, 25600, 257)
     with pytest.raises(ValueError):
         linear.scratch_size(5121, 25600, 16)
+
+
+def test_penalty_words_follow_the_request_history():
+    """Sampling::rebuildPenaltyWords / countPenaltyTokens (Sampling.cpp:91-121): the prompt bit on prompt tokens, the
+    count of generated and pending tokens."""
+    history = [5, 9, 5, 2, 7, 7, 9]   # four prompt tokens, three generated
+    words = ops.Sampling.rebuild_penalty_words(12, history, 3, pending_token=7)
+    want = np.zeros(12, dtype=np.uint32)
+    want[[5, 9, 2]] = 0x80000000
+    want[7] += 3
+    want[9] += 1
+    assert np.array_equal(words, want)
+    assert np.array_equal(ops.Sampling.rebuild_penalty_words(12, history, 3, mark_prompt=False) & 0x80000000, np.zeros(12, np.uint32))
+    ops.Sampling.count_penalty_tokens(words, [7, 0, 0])
+    want[7] += 1
+    want[0] += 2
+    assert np.array_equal(words, want)
+    for bad in (lambda: ops.Sampling.rebuild_penalty_words(12, history, 7), lambda: ops.Sampling.rebuild_penalty_words(8, history, 3),
+                lambda: ops.Sampling.count_penalty_tokens(words, [12])):
+        with pytest.raises(splash_amd.SplashError):
+            bad()

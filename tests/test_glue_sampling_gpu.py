@@ -293,3 +293,51 @@ def test_constraint_masks_and_stop_exclusion(backend):
     assert got[1] == orc.NO_TOKEN and got[6] != stops[0] and got[4] != stops[1]
     with pytest.raises(ValueError, match="constraint"):
         ops.Sampling.add_verify(splash_amd.CommandGraph(), {**b, "token_mask": None}, V, V, lanes, policies)
+
+
+@pytest.mark.parametrize("stride_pad", [0, 40])
+def test_penalties_rewrite_the_penalized_lanes_only(backend, stride_pad):
+    """decode_sample_penalize (sampling.metal:1016-1051) against the oracle, bit for bit: three lanes of chain and tree
+    blocks, two penalized from their own rows of the penalty table, one not; extreme repetition penalties saturate;
+    unselectable logits stay; the unpenalized lane's rows and the padding between rows keep their bits."""
+    print(f"case penalties stride_pad={stride_pad}", flush=True)
+    from tests.test_oracle_sampling import penalty_case, random_tree
+    rng = np.random.default_rng(21)
+    V = 1000
+    stride = V + stride_pad
+    blocks = [(16, None), (9, random_tree(rng, 9)), (5, None)]
+    lanes, trees, logits, inputs, tables = [], [], [], [], []
+    first = 0
+    for rows, tree in blocks:
+        tree = tree if tree is not None else ops.chain_tree_rows([rows])
+        x, words, tokens = penalty_case(rng, rows, V, tree)
+        lanes.append((first, rows)); trees.append(tree); logits.append(x); inputs.append(tokens); tables.append(words)
+        first += rows
+    total = first
+    padded = np.full((total, stride), np.float32(123.0), dtype=np.float32)
+    padded[:, :V] = np.concatenate(logits)
+    # lane 0 reads table row 2, lane 1 is not penalized, lane 2 reads table row 0
+    table = np.zeros((3, V), dtype=np.uint32)
+    table[2], table[0], table[1] = tables[0], tables[2], rng.integers(0, 2 ** 32, V, dtype=np.uint32)
+    for penalties in ([(1.3, 0.5, 0.25, 2), (1.0, 0.0, 0.0, 1), (0.8, 0.3, 0.0, 0)], [(1e-45, 0.0, 0.0, 2), (1.0, 0.0, 0.0, 1), (3e38, 1e38, 3e38, 0)]):
+        buffer = backend.from_array(padded)
+        graph = splash_amd.CommandGraph()
+        ops.Sampling.add_penalties(graph, buffer, backend.from_array(table), backend.from_array(np.concatenate(inputs)),
+                                   backend.from_array(np.concatenate(trees)), V, stride, lanes, penalties)
+        assert graph.kernels() == ["decode_sample_penalize"]
+        backend.run(graph)
+        got = buffer.download(np.float32).reshape(total, stride)
+        assert np.all(got[:, V:] == np.float32(123.0))
+        for (f, rows), x, words, tokens, tree, p in zip(lanes, logits, tables, inputs, trees, penalties):
+            want = orc.penalize(x, words, tokens, tree, *p[:3]) if p[:3] != (1.0, 0.0, 0.0) else x
+            assert got[f:f + rows, :V].tobytes() == want.tobytes(), p
+    # nothing is added when no lane's penalties are active; a table too short for a lane's row is refused
+    graph = splash_amd.CommandGraph()
+    args = (backend.from_array(padded), backend.from_array(table), backend.from_array(np.concatenate(inputs)),
+            backend.from_array(np.concatenate(trees)), V, stride, lanes)
+    ops.Sampling.add_penalties(graph, *args, [(1.0, 0.0, 0.0, 9)] * 3)
+    assert len(graph) == 0
+    with pytest.raises(splash_amd.SplashError):
+        ops.Sampling.add_penalties(graph, *args, [(1.1, 0.0, 0.0, 3)] + [(1.0, 0.0, 0.0, 0)] * 2)
+    with pytest.raises(splash_amd.SplashError):
+        ops.Sampling.add_penalties(graph, *args, [(0.0, 0.0, 0.0, 0)] * 3)

@@ -197,3 +197,61 @@ def test_truncated_rejection_law_is_the_renormalized_kept_distribution():
             child = int(rng.integers(0, V))
             tok, accepted, _ = orc.rejection_row_policy(x, policy, q, child, float(rng.random()), float(rng.random()))
             assert p[tok] > 0 and (not accepted or tok == child)
+
+
+def penalty_case(rng, rows, vocab, tree):
+    """A block's logits with the special values the reference's test covers (target_sampling_metal_test.mm:27-30,
+    :791-860), its penalty words and its draft tokens."""
+    logits = (rng.standard_normal((rows, vocab)) * 4).astype(np.float32)
+    logits[:, 3] = -np.inf
+    logits[rows // 2, 5] = np.nan
+    logits[:, 7] = np.float32(3e38)
+    logits[:, 8] = np.float32(-3e38)
+    logits[:, 9] = 0.0
+    words = np.zeros(vocab, dtype=np.uint32)
+    words[rng.choice(vocab, vocab // 3, replace=False)] = rng.integers(1, 5, vocab // 3)
+    words[rng.choice(vocab, vocab // 4, replace=False)] |= 0x80000000
+    words[[3, 5, 7, 8, 9]] |= 0x80000001
+    inputs = rng.integers(0, vocab, rows).astype(np.uint32)
+    inputs[1:4] = inputs[1] if rows > 3 else inputs[1:4]     # a token drafted at several rows of a path
+    return logits, words, inputs
+
+
+def brute_force_penalty(logits, words, inputs, tree, repetition, presence, frequency):
+    """Row r's context: the table's count of the token plus the rows of r's path, its anchor aside, that drafted it."""
+    out = logits.copy()
+    f32 = np.float32
+    largest = np.finfo(np.float32).max
+    with np.errstate(over="ignore", divide="ignore"):
+        inverse = min(f32(1) / f32(repetition), largest)
+    for r in range(logits.shape[0]):
+        path = [j for j in range(1, logits.shape[0]) if (int(tree[r]["ancestors"]) >> j) & 1]
+        for t in range(logits.shape[1]):
+            count = int(words[t] & 0x7FFFFFFF) + sum(1 for j in path if inputs[j] == t)
+            if (count == 0 and not (words[t] >> 31)) or np.isnan(logits[r, t]) or logits[r, t] == -np.inf:
+                continue
+            with np.errstate(over="ignore"):
+                value = f32(logits[r, t]) * (inverse if logits[r, t] > 0 else f32(repetition))
+                if count:
+                    value = f32(value - f32(f32(f32(frequency) * f32(count)) + f32(presence)))
+            out[r, t] = min(max(value, -largest), largest)
+    return out
+
+
+@pytest.mark.parametrize("penalties", [(1.3, 0.5, 0.25), (1.0, 0.7, 0.0), (0.8, 0.0, 0.0), (1e-45, 0.0, 0.0), (3e38, 1e38, 3e38)])
+def test_penalties_against_explicit_path_contexts(penalties):
+    rng = np.random.default_rng(11)
+    for rows, tree in ((9, random_tree(rng, 9)), (16, None), (1, None)):
+        if tree is None:
+            tree = np.zeros(rows, dtype=np.dtype([("ancestors", "<u4"), ("parent", "<u2"), ("depth", "<u2")]))
+            for r in range(rows):
+                tree[r] = ((2 << r) - 1, max(r - 1, 0) if r else 0xFFFF, r)
+        logits, words, inputs = penalty_case(rng, rows, 64, tree)
+        got = orc.penalize(logits, words, inputs, tree, *penalties)
+        want = brute_force_penalty(logits, words, inputs, tree, *penalties)
+        assert got.tobytes() == want.tobytes()
+        assert np.isfinite(got[np.isfinite(logits)]).all()                       # saturates, never overflows
+        assert np.all(got[:, 3] == -np.inf) and np.isnan(got[rows // 2, 5])      # unselectable logits stay
+        untouched = ((words == 0)[None, :] & (got.view(np.uint32) != logits.view(np.uint32)))
+        for r, t in zip(*np.nonzero(untouched)):                                 # only a drafted token of the path changes
+            assert any(inputs[j] == t for j in range(1, rows) if (int(tree[r]["ancestors"]) >> j) & 1)
