@@ -24,6 +24,8 @@
 //   orc_argmax / orc_accept_tree    pinned by brute force on tiny vocabularies.
 //   orc_penalize                    pinned by a brute-force restatement over explicit path contexts (tests) and the
 //                                   closed cases of the reference's test (prompt-only, saturation, unselectable).
+//   orc_thinking_cutoff             pinned by an independent walk over explicit depth-ordered paths (tests) and the
+//                                   closed form on chains.
 //   orc_rejection_*                 pinned by enumeration: selection law equals target to 1e-12.
 //   orc_distribution_end            pinned by an independent fp64 sort (min_p, top_k with ties, nucleus).
 //   orc_moe_*                       pinned by a stable sort and softmax closed form; the layer by the dense FFN it
@@ -131,6 +133,12 @@ uint32_t orc_accept_tree(const struct OrcTreeRow *tree, const uint32_t *tokens, 
 // tree rows. frequency * count, + presence and the subtraction each round once (no fused multiply-add).
 void orc_penalize(float *logits, uint32_t rows, uint32_t vocab, uint32_t stride, const uint32_t *words, const uint32_t *inputs,
                   const struct OrcTreeRow *tree, float repetition, float presence, float frequency);
+// sampling.metal:1999-2042 decode_sample_thinking_cutoff for one lane's block: selections rewritten in place. masks
+// (uint32 [rows][mask_words], NULL unless waits) are the rows' constraint masks; end[0 .. count) the end tokens the
+// block's rows can hold, close the last token of the whole end.
+void orc_thinking_cutoff(uint32_t *selected, uint32_t rows, uint32_t vocab, const uint32_t *inputs, const struct OrcTreeRow *tree,
+                         const uint32_t *masks, uint32_t mask_words, uint32_t cutoff_row, const uint32_t *end, uint32_t count,
+                         uint32_t close, uint32_t also_ends, int waits);
 // One sampled verify row under the textbook full-vocabulary rule in the reference's order of
 // operations (sampling.metal:713-885): weight_t = exp((logit_t - max) / T); p = weight / total;
 // accept the drafted token iff u_child * q[draft] < p[draft]; else draw from max(p - q, 0)

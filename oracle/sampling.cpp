@@ -162,6 +162,26 @@ void orc_penalize(float *logits, uint32_t rows, uint32_t vocab, uint32_t stride,
   }
 }
 
+void orc_thinking_cutoff(uint32_t *selected, uint32_t rows, uint32_t vocab, const uint32_t *inputs, const struct OrcTreeRow *tree,
+                         const uint32_t *masks, uint32_t mask_words, uint32_t cutoff_row, const uint32_t *end, uint32_t count,
+                         uint32_t close, uint32_t also_ends, int waits) {
+  for (uint32_t at = 0; at < rows; ++at) {
+    const uint32_t path = tree[at].ancestors, depth = tree[at].depth;
+    uint32_t cut = 0;
+    for (uint32_t walk = path; walk; walk &= walk - 1, ++cut) {
+      const uint32_t row = uint32_t(__builtin_ctz(walk));
+      if (cut >= cutoff_row && (!waits || ((masks[size_t(row) * mask_words + end[0] / 32] >> (end[0] % 32)) & 1u))) break;
+    }
+    if (cut > depth || depth - cut >= count) continue;
+    bool ended = false;
+    for (uint32_t walk = path & ~1u; walk; walk &= walk - 1) {
+      const uint32_t before = uint32_t(__builtin_ctz(walk));
+      ended = ended || (tree[before].depth <= cut && (inputs[before] == close || inputs[before] == also_ends));
+    }
+    if (!ended && selected[at] < vocab) selected[at] = end[depth - cut];
+  }
+}
+
 uint32_t orc_argmax(const float *logits, uint32_t vocab) {
   float best = -std::numeric_limits<float>::infinity();
   uint32_t index = ORC_NO_TOKEN;

@@ -145,6 +145,10 @@ class SamplingPenalties(ctypes.Structure):
     _fields_ = [("repetition", ctypes.c_float), ("presence", ctypes.c_float), ("frequency", ctypes.c_float), ("table_row", c_u32)]
 
 
+class ThinkingCutoff(ctypes.Structure):
+    _fields_ = [("row", c_u32), ("end_count", c_u32), ("also_ends", c_u32), ("waits_for_mask", c_u32), ("end", P(c_u32))]
+
+
 class SamplingPolicy(ctypes.Structure):
     _fields_ = [("temperature", ctypes.c_float), ("min_p", ctypes.c_float), ("top_k", c_u32), ("top_p", ctypes.c_float),
                 ("constrained", c_u32), ("excludes_stop_tokens", c_u32)]
@@ -265,6 +269,7 @@ _sig("spo_sampling_add_verify", c_int, c_p, P(SamplingBuffers), c_u32, c_u32, P(
 _sig("spo_sampling_rebuild_penalty_words", c_int, P(c_u32), c_u32, P(c_u32), c_u64, c_u64, c_u32, c_int)
 _sig("spo_sampling_count_penalty_tokens", c_int, P(c_u32), c_u32, P(c_u32), c_u64)
 _sig("spo_sampling_add_penalties", c_int, c_p, c_p, c_p, c_p, c_p, c_u32, c_u32, P(LaneRows), P(SamplingPenalties), c_u32)
+_sig("spo_sampling_add_thinking_cutoff", c_int, c_p, c_p, c_p, c_u32, c_p, c_p, c_u32, P(LaneRows), P(ThinkingCutoff), c_u32)
 _sig("spo_sampling_add_acceptance", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, P(LaneRows), P(c_u32), c_u32, P(c_u32))
 _sig("spo_dense_verify_create", c_int, c_p, P(DenseDimensions), c_u32, c_u32, c_u32, P(c_p))
 _sig("spo_dense_verify_destroy", None, c_p)

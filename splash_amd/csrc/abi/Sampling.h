@@ -70,6 +70,25 @@ struct SamplingPenaltyParams {
   float frequency[SAMPLING_MAXIMUM_LANES];
 };
 
+// decode_sample_thinking_cutoff: grid (lanes), one thread a lane (the reference's ThinkingCutoffParams,
+// abi/Sampling.h:147-172). A lane whose `row` is below its rows cuts each row's path at the path's row of depth `row`:
+// the path's row of depth cut + i selects its end token tokens[i], for each i below `count`, unless a draft token on
+// the path up to the cut is `close` or `also_ends`, which ended thinking first. The end of a lane in waiting_mask, a
+// constrained one, waits for its mask: a path's cut is instead the first of its rows from depth `row` on whose
+// constraint-mask row admits tokens[0]. A row whose selection is SAMPLING_NO_TOKEN keeps it.
+struct ThinkingCutoffParams {
+  uint32_t vocabulary;
+  uint32_t lanes;
+  uint32_t waiting_mask;
+  uint32_t mask_words;  // words of a constraint-mask row (one a packed row)
+  struct SamplingLaneRows lane[SAMPLING_MAXIMUM_LANES];
+  uint32_t row[SAMPLING_MAXIMUM_LANES];
+  uint32_t count[SAMPLING_MAXIMUM_LANES];
+  uint32_t close[SAMPLING_MAXIMUM_LANES];
+  uint32_t also_ends[SAMPLING_MAXIMUM_LANES];
+  uint32_t tokens[SAMPLING_MAXIMUM_LANES][SAMPLING_MAXIMUM_ROWS];
+};
+
 // decode_accept_tree: one thread per lane (AcceptBatchParams).
 struct AcceptBatchParams {
   uint32_t lanes;
@@ -82,5 +101,6 @@ struct AcceptBatchParams {
 #ifdef __cplusplus
 static_assert(sizeof(TargetSamplingParams) == 16 + 32 + 16 + 64 + 96 + 32, "target sampling parameters are 256 bytes on both sides");
 static_assert(sizeof(SamplingPenaltyParams) == 16 + 64 + 5 * 32, "penalty parameters are 240 bytes on both sides");
+static_assert(sizeof(ThinkingCutoffParams) == 16 + 64 + 4 * 32 + 512, "thinking cutoff parameters are 720 bytes on both sides");
 static_assert(sizeof(AcceptBatchParams) == 16 + 32 + 16 + 64, "acceptance parameters are 128 bytes on both sides");
 #endif

@@ -138,6 +138,25 @@ sp_status spo_sampling_add_penalties(spo_graph *graph, sp_buffer *logits, sp_buf
   });
 }
 
+sp_status spo_sampling_add_thinking_cutoff(spo_graph *graph, sp_buffer *input_tokens, sp_buffer *token_mask, uint32_t mask_words,
+                                           sp_buffer *tree_rows, sp_buffer *tokens, uint32_t vocabulary, const spo_lane_rows *lanes,
+                                           const spo_thinking_cutoff *cutoffs, uint32_t count) {
+  return capi::guard([&] {
+    capi::require(graph && lanes && cutoffs, "graph, lanes or cutoffs");
+    std::vector<ops::LaneRows> rows;
+    std::vector<std::optional<ops::ThinkingCutoff>> list;
+    for (uint32_t i = 0; i < count; ++i) {
+      rows.push_back({lanes[i].first, lanes[i].rows});
+      if (!cutoffs[i].end_count) { list.push_back(std::nullopt); continue; }
+      capi::require(cutoffs[i].end, "a cutoff's end tokens");
+      list.push_back(ops::ThinkingCutoff{cutoffs[i].row, {cutoffs[i].end, cutoffs[i].end + cutoffs[i].end_count}, cutoffs[i].also_ends,
+                                         cutoffs[i].waits_for_mask != 0});
+    }
+    ops::Sampling::addThinkingCutoff(capi::graphOf(graph), B(input_tokens), token_mask ? B(token_mask) : hip::Buffer{}, mask_words,
+                                     B(tree_rows), B(tokens), vocabulary, rows, list);
+  });
+}
+
 sp_status spo_dense_verify_create(sp_backend *backend, const spo_dense_dimensions *d, uint32_t max_lanes, uint32_t physical_pages,
                                   uint32_t page_table_entries, spo_dense_verify **out) {
   return capi::guard([&] {

@@ -116,6 +116,38 @@ __global__ __launch_bounds__(256) void decode_sample_penalize(float *__restrict_
 }
 SP_REGISTER_KERNEL("decode_sample_penalize", &decode_sample_penalize);
 
+// decode_sample_thinking_cutoff (sampling.metal:1999-2042): one thread a lane rewrites, among the lane's selections,
+// those of the rows its thinking end reaches.
+__global__ __launch_bounds__(64) void decode_sample_thinking_cutoff(const uint32_t *__restrict__ input_tokens,
+                                                                    const uint32_t *__restrict__ token_mask,
+                                                                    const AttentionTreeRow *__restrict__ tree,
+                                                                    uint32_t *__restrict__ tokens, ThinkingCutoffParams p) {
+  const uint32_t lane = blockIdx.x;
+  if (threadIdx.x || lane >= p.lanes) return;
+  const uint32_t rows = p.lane[lane].rows, first = p.lane[lane].first;
+  const bool waits = (p.waiting_mask >> lane) & 1u;
+  const uint32_t start = p.tokens[lane][0];
+  for (uint32_t at = 0; at < rows; ++at) {
+    const uint32_t path = tree[first + at].ancestors, depth = tree[first + at].depth;
+    // The path's rows ascend from its anchor, one a depth; one past the row's depth where the path holds no cut.
+    uint32_t cut = 0;
+    for (uint32_t walk = path; walk; walk &= walk - 1u, ++cut)
+      if (cut >= p.row[lane] &&
+          (!waits || ((token_mask[size_t(first + uint32_t(__ffs(int(walk)) - 1)) * p.mask_words + start / 32u] >> (start % 32u)) & 1u)))
+        break;
+    if (cut > depth || depth - cut >= p.count[lane]) continue;
+    bool ended = false;
+    for (uint32_t walk = path & ~1u; walk; walk &= walk - 1u) {
+      const uint32_t before = uint32_t(__ffs(int(walk)) - 1);
+      const uint32_t draft = input_tokens[first + before];
+      ended = ended || (tree[first + before].depth <= cut && (draft == p.close[lane] || draft == p.also_ends[lane]));
+    }
+    // A row with no selectable logit keeps its sentinel, so the lane fails.
+    if (!ended && tokens[first + at] < p.vocabulary) tokens[first + at] = p.tokens[lane][depth - cut];
+  }
+}
+SP_REGISTER_KERNEL("decode_sample_thinking_cutoff", &decode_sample_thinking_cutoff);
+
 // Grid (rows * SAMPLING_SHARDS), 256 threads. partial_values/indices [row][shard].
 __global__ __launch_bounds__(256) void decode_sample_argmax_sharded(const float *__restrict__ logits, float *__restrict__ partial_values,
                                                                     uint32_t *__restrict__ partial_indices, TargetSamplingParams p) {

@@ -77,6 +77,48 @@ void Sampling::addPenalties(hip::CommandGraph &graph, const hip::Buffer &logits,
             {256, 1, 1});
 }
 
+void Sampling::addThinkingCutoff(hip::CommandGraph &graph, const hip::Buffer &inputTokens, const hip::Buffer &tokenMask,
+                                 uint32_t maskWords, const hip::Buffer &treeRows, const hip::Buffer &tokens, uint32_t vocabulary,
+                                 const std::vector<LaneRows> &lanes, const std::vector<std::optional<ThinkingCutoff>> &cutoffs) {
+  const uint32_t rows = packedRows(lanes);
+  if (cutoffs.size() != lanes.size()) throw std::invalid_argument("a thinking cutoff, or none, per lane");
+  if (!vocabulary) throw std::invalid_argument("invalid sampling geometry");
+  ThinkingCutoffParams params{};
+  params.vocabulary = vocabulary;
+  params.lanes = uint32_t(lanes.size());
+  params.mask_words = maskWords;
+  bool cuts = false;
+  for (size_t l = 0; l < lanes.size(); ++l) {
+    params.lane[l] = {lanes[l].first, lanes[l].rows};
+    const std::optional<ThinkingCutoff> &cutoff = cutoffs[l];
+    params.row[l] = cutoff ? cutoff->row : lanes[l].rows;
+    if (params.row[l] >= lanes[l].rows) {
+      params.row[l] = SAMPLING_MAXIMUM_ROWS;  // past every depth: the lane's rows keep their selections
+      continue;
+    }
+    if (cutoff->end.empty()) throw std::invalid_argument("a thinking cutoff has no end");
+    if (cutoff->waitsForMask) {
+      if (cutoff->end.front() >= vocabulary)
+        throw std::invalid_argument("a thinking end that waits for a mask starts outside the vocabulary");
+      if (uint64_t{maskWords} * 32 < vocabulary) throw std::invalid_argument("a constraint-mask row holds a bit for every token");
+      requireBytes(tokenMask, uint64_t{rows} * maskWords * 4, "constraint masks");
+      params.waiting_mask |= 1u << l;
+    }
+    // The rows from the cutoff's on take as many of its end as the lane's rows hold.
+    params.count[l] = uint32_t(std::min<size_t>(cutoff->end.size(), lanes[l].rows - cutoff->row));
+    std::copy_n(cutoff->end.begin(), params.count[l], params.tokens[l]);
+    params.close[l] = cutoff->end.back();
+    params.also_ends[l] = cutoff->alsoEnds;
+    cuts = true;
+  }
+  if (!cuts) return;
+  requireBytes(inputTokens, uint64_t{rows} * 4, "input tokens");
+  requireBytes(treeRows, uint64_t{rows} * sizeof(AttentionTreeRow), "verify tree rows");
+  requireBytes(tokens, uint64_t{rows} * 4, "selected tokens");
+  graph.add("decode_sample_thinking_cutoff", {inputTokens, params.waiting_mask ? tokenMask : inputTokens, treeRows, tokens}, params,
+            {uint32_t(lanes.size()), 1, 1}, {64, 1, 1});
+}
+
 SamplingWorkspaceSize Sampling::workspace(uint32_t rows) noexcept {
   SamplingWorkspaceSize size;
   size.partialValues = uint64_t{rows} * SAMPLING_SHARDS * 4;

@@ -74,6 +74,18 @@ struct AcceptanceBuffers final {
   hip::Buffer retainedRows;   // uint32 [lanes]: mask of the block rows retained
 };
 
+// Where a lane's thinking budget runs out in a selection (the reference's ThinkingCutoff, Sampling.hpp:30-55): its
+// selected rows of depth `row` on take the `end` tokens in order, as many as the block holds, unless a draft token on
+// the row's path up to depth `row` is the last of `end`, which closes thinking, or `alsoEnds`. An end that waits for
+// the mask of a constrained lane starts instead, along each row's path, at the first of the path's rows from depth
+// `row` on whose constraint-mask row admits its first token.
+struct ThinkingCutoff final {
+  uint32_t row = 0;
+  std::vector<uint32_t> end;
+  uint32_t alsoEnds = SAMPLING_NO_TOKEN;
+  bool waitsForMask = false;
+};
+
 // A lane whose logits rows the penalties rewrite, from row `tableRow` of the penalty table.
 struct PenalizedLane final {
   LaneRows rows;
@@ -104,6 +116,13 @@ public:
                         const std::vector<LaneRows> &lanes, const std::vector<SamplingPolicy> &policies,
                         const std::array<uint32_t, SAMPLING_STOP_TOKENS> &stopTokens = {SAMPLING_NO_TOKEN, SAMPLING_NO_TOKEN,
                                                                                        SAMPLING_NO_TOKEN, SAMPLING_NO_TOKEN});
+  // After addVerify: the selections of the rows each lane's thinking end reaches become its end tokens
+  // (decode_sample_thinking_cutoff, Sampling.cpp:41-78 and :314-327 in the reference). One optional cutoff a lane; a
+  // lane without one, or whose cutoff row is past its rows, keeps its selections. Nothing when no lane is cut.
+  // tokenMask (uint32 [rows][maskWords]) only for a lane whose end waits for its mask.
+  static void addThinkingCutoff(hip::CommandGraph &graph, const hip::Buffer &inputTokens, const hip::Buffer &tokenMask,
+                                uint32_t maskWords, const hip::Buffer &treeRows, const hip::Buffer &tokens, uint32_t vocabulary,
+                                const std::vector<LaneRows> &lanes, const std::vector<std::optional<ThinkingCutoff>> &cutoffs);
   static void addAcceptance(hip::CommandGraph &graph, const AcceptanceBuffers &buffers, const std::vector<LaneRows> &lanes,
                             const std::vector<uint32_t> &remaining, const std::array<uint32_t, SAMPLING_STOP_TOKENS> &stopTokens);
 };

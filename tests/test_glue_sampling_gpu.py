@@ -341,3 +341,50 @@ def test_penalties_rewrite_the_penalized_lanes_only(backend, stride_pad):
         ops.Sampling.add_penalties(graph, *args, [(1.1, 0.0, 0.0, 3)] + [(1.0, 0.0, 0.0, 0)] * 2)
     with pytest.raises(splash_amd.SplashError):
         ops.Sampling.add_penalties(graph, *args, [(0.0, 0.0, 0.0, 0)] * 3)
+
+
+def test_thinking_cutoff_rewrites_the_reached_rows(backend):
+    """decode_sample_thinking_cutoff (sampling.metal:1999-2042) against the oracle over lanes of chains and trees: a lane
+    cut at its first row, one in the middle of its block, one whose end waits for its constraint masks, one with no
+    cutoff and one whose cutoff lies past its rows."""
+    print("case thinking cutoff", flush=True)
+    from tests.test_oracle_sampling import random_tree
+    rng = np.random.default_rng(23)
+    vocab, words = 70, 3
+    for trial in range(20):
+        sizes = [int(rng.integers(1, 17)) for _ in range(5)]
+        trees = [random_tree(rng, n) if (trial + i) % 2 else ops.chain_tree_rows([n]) for i, n in enumerate(sizes)]
+        lanes, first = [], 0
+        for n in sizes:
+            lanes.append((first, n)); first += n
+        total = first
+        selected = rng.integers(0, vocab, total).astype(np.uint32)
+        selected[rng.random(total) < 0.1] = 0xFFFFFFFF
+        inputs = rng.integers(0, 10, total).astype(np.uint32)
+        masks = rng.integers(0, 2 ** 32, (total, words), dtype=np.uint32)
+        end = lambda: [int(t) for t in rng.integers(0, 10, int(rng.integers(1, 6)))]
+        cutoffs = [(0, end()), (int(rng.integers(0, sizes[1])), end(), int(rng.integers(0, 10))),
+                   (int(rng.integers(0, sizes[2])), end(), 0xFFFFFFFF, True), None, (sizes[4] + 1, end())]
+        tokens = backend.from_array(selected)
+        graph = splash_amd.CommandGraph()
+        ops.Sampling.add_thinking_cutoff(graph, backend.from_array(inputs), backend.from_array(np.concatenate(trees)), tokens, vocab, lanes,
+                                         cutoffs, token_mask=backend.from_array(masks), mask_words=words)
+        assert graph.kernels() == ["decode_sample_thinking_cutoff"]
+        backend.run(graph)
+        got = tokens.download(np.uint32)
+        for (f, n), tree, c in zip(lanes, trees, cutoffs):
+            want = selected[f:f + n]
+            if c is not None:
+                want = orc.thinking_cutoff(want, inputs[f:f + n], tree, vocab, c[0], c[1], c[2] if len(c) > 2 else 0xFFFFFFFF,
+                                           masks[f:f + n] if len(c) > 3 and c[3] else None)
+            assert np.array_equal(got[f:f + n], want), (trial, c)
+    # no lane is cut: nothing is added; an empty end and a waiting end outside the vocabulary are refused
+    graph = splash_amd.CommandGraph()
+    args = (backend.from_array(inputs), backend.from_array(np.concatenate(trees)), tokens, vocab, lanes)
+    ops.Sampling.add_thinking_cutoff(graph, *args, [None, (sizes[1], [1]), None, None, None])
+    assert len(graph) == 0
+    with pytest.raises(splash_amd.SplashError):
+        ops.Sampling.add_thinking_cutoff(graph, *args, [(0, [vocab + 1], 0xFFFFFFFF, True), None, None, None, None],
+                                         token_mask=backend.from_array(masks), mask_words=words)
+    with pytest.raises(splash_amd.SplashError):
+        ops.Sampling.add_thinking_cutoff(graph, *args, [(0, [1], 0xFFFFFFFF, True), None, None, None, None])   # no masks

@@ -255,3 +255,73 @@ def test_penalties_against_explicit_path_contexts(penalties):
         untouched = ((words == 0)[None, :] & (got.view(np.uint32) != logits.view(np.uint32)))
         for r, t in zip(*np.nonzero(untouched)):                                 # only a drafted token of the path changes
             assert any(inputs[j] == t for j in range(1, rows) if (int(tree[r]["ancestors"]) >> j) & 1)
+
+
+def cutoff_by_depth(selected, inputs, tree, vocab, row, end, also_ends, masks):
+    """The thinking cutoff told by depth: a row's path as the list of its rows in depth order; the cut is the first depth
+    from `row` on (whose mask admits end[0], for an end that waits); the rows of depth cut + i take end[i] unless a
+    drafted token of the path at depths 1..cut closes thinking."""
+    out = list(selected)
+    rows = len(selected)
+    count = min(len(end), rows - row) if row < rows else 0
+    for at in range(rows):
+        path = sorted((j for j in range(rows) if (int(tree[at]["ancestors"]) >> j) & 1), key=lambda j: int(tree[j]["depth"]))
+        assert [int(tree[j]["depth"]) for j in path] == list(range(len(path)))
+        depth = len(path) - 1
+        cut = next((d for d in range(row, len(path))
+                    if masks is None or (int(masks[path[d]][end[0] // 32]) >> (end[0] % 32)) & 1), None)
+        if cut is None or depth - cut >= count:
+            continue
+        if any(int(inputs[j]) in (end[-1], also_ends) for j in path[1:cut + 1]):
+            continue
+        if out[at] < vocab:
+            out[at] = end[depth - cut]
+    return np.array(out, dtype=np.uint32)
+
+
+def test_thinking_cutoff_against_a_walk_by_depth():
+    rng = np.random.default_rng(17)
+    vocab = 50
+    for trial in range(300):
+        rows = int(rng.integers(1, 17))
+        tree = random_tree(rng, rows) if trial % 3 else None
+        if tree is None:
+            tree = np.zeros(rows, dtype=np.dtype([("ancestors", "<u4"), ("parent", "<u2"), ("depth", "<u2")]))
+            for r in range(rows):
+                tree[r] = ((2 << r) - 1, max(r - 1, 0) if r else 0xFFFF, r)
+        selected = rng.integers(0, vocab, rows).astype(np.uint32)
+        selected[rng.random(rows) < 0.1] = orc.NO_TOKEN
+        inputs = rng.integers(0, 12, rows).astype(np.uint32)     # a small alphabet, so closes and also-ends occur
+        end = [int(t) for t in rng.integers(0, 12, int(rng.integers(1, 5)))]
+        row = int(rng.integers(0, rows + 2))
+        also = int(rng.integers(0, 12)) if trial % 2 else orc.NO_TOKEN
+        masks = None
+        if trial % 4 == 0:
+            masks = rng.integers(0, 2 ** 32, (rows, 2), dtype=np.uint32)
+        got = orc.thinking_cutoff(selected, inputs, tree, vocab, row, end, also, masks)
+        want = cutoff_by_depth(selected, inputs, tree, vocab, row, end, also, masks)
+        assert np.array_equal(got, want), (trial, rows, row, end)
+
+
+def test_thinking_cutoff_on_a_chain_closed_form():
+    """A chain whose drafts never close: rows row .. row + len(end) - 1 take the end in order; a close token drafted at a
+    depth up to the cut keeps every selection; a row without a selectable logit keeps its sentinel."""
+    rows, vocab = 12, 100
+    tree = np.zeros(rows, dtype=np.dtype([("ancestors", "<u4"), ("parent", "<u2"), ("depth", "<u2")]))
+    for r in range(rows):
+        tree[r] = ((2 << r) - 1, max(r - 1, 0) if r else 0xFFFF, r)
+    selected = np.arange(rows, dtype=np.uint32) + 50
+    inputs = np.full(rows, 7, dtype=np.uint32)
+    got = orc.thinking_cutoff(selected, inputs, tree, vocab, 4, [90, 91, 92])
+    want = selected.copy(); want[4:7] = [90, 91, 92]
+    assert np.array_equal(got, want)
+    got = orc.thinking_cutoff(selected, inputs, tree, vocab, 10, [90, 91, 92])     # the block holds two of the three
+    want = selected.copy(); want[10:12] = [90, 91]
+    assert np.array_equal(got, want)
+    closed = inputs.copy(); closed[3] = 92                                          # thinking closed before the cut
+    assert np.array_equal(orc.thinking_cutoff(selected, closed, tree, vocab, 4, [90, 91, 92]), selected)
+    closed = inputs.copy(); closed[5] = 92                                          # after the cut: not looked at
+    assert np.array_equal(orc.thinking_cutoff(selected, closed, tree, vocab, 4, [90, 91, 92])[4:7], [90, 91, 92])
+    failed = selected.copy(); failed[5] = orc.NO_TOKEN
+    assert orc.thinking_cutoff(failed, inputs, tree, vocab, 4, [90, 91, 92])[5] == orc.NO_TOKEN
+    assert np.array_equal(orc.thinking_cutoff(selected, inputs, tree, vocab, 12, [90]), selected)   # past the block
