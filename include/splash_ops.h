@@ -217,7 +217,13 @@ sp_status spo_state_codec_add_dequantize(spo_graph *graph, sp_buffer *codes, sp_
 sp_status spo_state_codec_add_copy(spo_graph *graph, sp_buffer *from, sp_buffer *to, const spo_state_codec_shape *shape);
 
 /* ---- MoE (runtime/ops/MoE.hpp:403-410, MoE.cpp:143-287; runtime/metal/abi/MoE.h:23-245) ---- */
-typedef struct spo_moe_shape { uint32_t hidden, ffn, experts, top_k; } spo_moe_shape;
+typedef struct spo_moe_shape {
+  uint32_t hidden, ffn, experts, top_k;
+  /* The shared expert (MoE.hpp:50-63): shared_slices experts of the routed experts' width that every row visits after
+   * its routed ones, ids experts .. experts + shared_slices - 1, their images after the routed experts' in the same
+   * buffers; shared_gate: each weighs sigmoid(row . scalar gate), else 1. */
+  uint32_t shared_slices, shared_gate;
+} spo_moe_shape;
 typedef struct spo_moe_workspace { /* in the order of spo_moe_workspace_sizes */
   sp_buffer *selected, *weights, *route_slot, *slot_row, *tile_expert, *tile_rows, *tile_total, *tables, *next_tables,
       *intermediate, *expert_output;
@@ -228,7 +234,7 @@ sp_status spo_moe_workspace_sizes(const spo_moe_shape *shape, uint32_t rows, uin
  * experts by (score descending, id ascending) in selected, their weights exp2((s_r - s_0) log2 e) / sum
  * in rank order, and the routes grouped by expert into tiles of up to 16 rows. */
 sp_status spo_moe_add_routing(spo_graph *graph, sp_buffer *scores, uint32_t score_stride, const spo_moe_workspace *workspace,
-                              const spo_moe_shape *shape, uint32_t rows);
+                              const spo_moe_shape *shape, uint32_t rows, sp_buffer *input, sp_buffer *shared_scalar_gate);
 /* MoE::addRouted (MoE.cpp:242-287): output = bf16(residual + sum over a row's routes, in rank order, of
  * weight * down_e(silu(gate_e x) * up_e x)). *_images hold every expert's re-tiled image of the tensor,
  * expert e at e * spo_gguf_image_bytes(format, rows of the tensor, its inputs). */
@@ -358,6 +364,7 @@ typedef struct spo_hybrid_dimensions {
   float rope_theta;
   uint32_t gdn_key_heads, gdn_value_heads, gdn_packed_width; /* packed row [q|k|v|z|b|a], whole column tiles */
   uint32_t experts, top_k, expert_ffn;
+  uint32_t shared_slices, shared_gate; /* the shared expert, as in spo_moe_shape */
 } spo_hybrid_dimensions;
 typedef struct spo_hybrid_lane {
   spo_verify_lane block;
@@ -372,6 +379,7 @@ typedef struct spo_hybrid_layer {
   const spo_projection *router;                                       /* hidden -> experts, fp32 scores */
   sp_buffer *gate_images, *up_images, *down_images;                   /* every expert's image of each tensor */
   uint32_t expert_format, expert_down_format;
+  sp_buffer *shared_scalar_gate; /* fp32 [hidden], of a gated shared expert (NULL otherwise) */
 } spo_hybrid_layer;
 sp_status spo_hybrid_verify_create(sp_backend *backend, const spo_hybrid_dimensions *dimensions, uint32_t max_lanes,
                                    uint32_t physical_pages, uint32_t page_table_entries, spo_hybrid_verify **out);

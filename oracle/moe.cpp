@@ -31,6 +31,26 @@ void orc_moe_route(const float *scores, uint32_t rows, uint32_t experts, uint32_
   }
 }
 
+void orc_moe_shared_weights(const uint16_t *x, const float *gate, uint32_t rows, uint32_t hidden, float *weights) {
+  for (uint32_t r = 0; r < rows; ++r) {
+    float partial[64];
+    for (uint32_t l = 0; l < 64; ++l) {
+      float sum = 0.f;
+      for (uint32_t d = l; d < hidden; d += 64) {
+        const float product = bf2f(x[size_t(r) * hidden + d]) * gate[d];
+        sum += product;
+      }
+      partial[l] = sum;
+    }
+    for (uint32_t distance = 32; distance; distance >>= 1) {
+      float next[64];
+      for (uint32_t l = 0; l < 64; ++l) next[l] = partial[l] + partial[l ^ distance];
+      std::memcpy(partial, next, sizeof next);
+    }
+    weights[r] = 1.0f / (1.0f + std::exp2(-1.44269504089f * partial[0]));
+  }
+}
+
 // kernels/shared/moe.metal:367-392: out = bf16(residual + sum over ranks of w y), fp32 in rank order.
 // y bf16 [rows][top_k][hidden]: the expert output of each route.
 void orc_moe_combine(const uint16_t *y, const float *weights, const uint16_t *residual, uint32_t rows, uint32_t top_k, uint32_t hidden,

@@ -115,7 +115,7 @@ class StateCodecShape(ctypes.Structure):
 
 
 class MoeShape(ctypes.Structure):
-    _fields_ = [("hidden", c_u32), ("ffn", c_u32), ("experts", c_u32), ("top_k", c_u32)]
+    _fields_ = [("hidden", c_u32), ("ffn", c_u32), ("experts", c_u32), ("top_k", c_u32), ("shared_slices", c_u32), ("shared_gate", c_u32)]
 
 
 MOE_WORKSPACE_FIELDS = ("selected", "weights", "route_slot", "slot_row", "tile_expert", "tile_rows", "tile_total", "tables", "next_tables",
@@ -157,7 +157,8 @@ class SamplingPolicy(ctypes.Structure):
 class HybridDimensions(ctypes.Structure):
     _fields_ = [(n, c_u32) for n in ("hidden", "vocabulary", "layers", "attention_interval", "q_heads", "kv_heads", "head_dim",
                                      "rotary_pairs", "normalize_heads", "gated_attention")] + [("rope_theta", ctypes.c_float)] + [
-        (n, c_u32) for n in ("gdn_key_heads", "gdn_value_heads", "gdn_packed_width", "experts", "top_k", "expert_ffn")]
+        (n, c_u32) for n in ("gdn_key_heads", "gdn_value_heads", "gdn_packed_width", "experts", "top_k", "expert_ffn", "shared_slices",
+                             "shared_gate")]
 
 
 class HybridLane(ctypes.Structure):
@@ -167,7 +168,8 @@ class HybridLane(ctypes.Structure):
 class HybridLayer(ctypes.Structure):
     _fields_ = [(n, c_p) for n in ("mixer_input", "mixer_output", "input_norm", "post_norm", "query_norm", "key_norm",
                                    "convolution_weights", "decay_weights", "time_bias", "mixer_norm", "router", "gate_images",
-                                   "up_images", "down_images")] + [("expert_format", c_u32), ("expert_down_format", c_u32)]
+                                   "up_images", "down_images")] + [("expert_format", c_u32), ("expert_down_format", c_u32),
+                                                                    ("shared_scalar_gate", c_p)]
 
 
 def _sig(name, restype, *argtypes):
@@ -260,7 +262,7 @@ _sig("spo_state_codec_layer_bytes", c_u64, c_u32, c_u32)
 for _name in ("spo_state_codec_add_quantize", "spo_state_codec_add_dequantize", "spo_state_codec_add_copy"):
     _sig(_name, c_int, c_p, c_p, c_p, P(StateCodecShape))
 _sig("spo_moe_workspace_sizes", c_int, P(MoeShape), c_u32, P(c_u64))
-_sig("spo_moe_add_routing", c_int, c_p, c_p, c_u32, P(MoeWorkspace), P(MoeShape), c_u32)
+_sig("spo_moe_add_routing", c_int, c_p, c_p, c_u32, P(MoeWorkspace), P(MoeShape), c_u32, c_p, c_p)
 _sig("spo_moe_add_routed", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_u32, c_u32, P(MoeWorkspace), P(MoeShape), c_u32)
 _sig("spo_moe_add_routed_norm", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_u32, c_u32, P(MoeWorkspace), P(MoeShape), c_u32, c_p, c_p)
 _sig("spo_row_copy_add", c_int, c_p, c_p, c_u32, c_u32, c_u32, c_p, c_u32, c_u32, c_u32, c_u32, c_u32)

@@ -28,10 +28,16 @@ inline uint32_t moe_maximum_tiles(uint32_t routes, uint32_t experts) {
   return full + partial;
 }
 
-// moe_route_select: grid (rows), 64 threads.
+// moe_route_select: grid (rows), 64 threads. A row's routes are its top_k routed experts and then the `shared` slices
+// of the shared expert, ids `experts` on, which every row visits (the reference's moe_shared_slice, moe.metal:5-8):
+// weighted by the sigmoid of the row's product with the block's fp32 scalar gate (shared_gated), or by 1.
 struct MoeRouteParams {
   uint32_t rows, experts, top_k;
   uint32_t score_stride;  // floats between rows of scores
+  uint32_t shared;        // slices of the shared expert
+  uint32_t shared_gated;
+  uint32_t input_size;    // of the rows the scalar gate multiplies (bf16)
+  uint32_t reserved;
 };
 // moe_group_routes: one workgroup of 1024 threads.
 struct MoeGroupParams {
@@ -65,7 +71,7 @@ struct GgufMoeParams {
 };
 
 #ifdef __cplusplus
-static_assert(sizeof(MoeRouteParams) == 16 && sizeof(MoeGroupParams) == 16 && sizeof(MoeGatherParams) == 16 &&
+static_assert(sizeof(MoeRouteParams) == 32 && sizeof(MoeGroupParams) == 16 && sizeof(MoeGatherParams) == 16 &&
                   sizeof(MoeCombineParams) == 16 && sizeof(GgufMoeParams) == 96,
               "MoE parameters have the same size on both sides");
 #endif

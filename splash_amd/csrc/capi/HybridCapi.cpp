@@ -55,6 +55,8 @@ sp_status spo_hybrid_verify_create(sp_backend *backend, const spo_hybrid_dimensi
     dims.experts = d->experts;
     dims.topK = d->top_k;
     dims.expertFfn = d->expert_ffn;
+    dims.sharedSlices = d->shared_slices;
+    dims.sharedGate = d->shared_gate != 0;
     holder->verify = std::make_unique<model::HybridVerify>(*holder->backend, dims, max_lanes, physical_pages, page_table_entries);
     *out = holder.release();
   });
@@ -80,6 +82,7 @@ sp_status spo_hybrid_verify_set_layer(spo_hybrid_verify *verify, uint32_t layer,
     out.router = capi::projectionOf(l->router);
     out.router.destination = ops::FloatOutput::Float32;
     out.experts = {B(l->gate_images), B(l->up_images), B(l->down_images), l->expert_format, l->expert_down_format};
+    if (l->shared_scalar_gate) out.sharedScalarGate = B(l->shared_scalar_gate);
     w.layers[layer] = std::move(out);
   });
 }

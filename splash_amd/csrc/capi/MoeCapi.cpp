@@ -8,7 +8,7 @@ using namespace splash;
 
 namespace {
 hip::Buffer B(sp_buffer *b) { return hip::Buffer::share(b); }
-ops::MoeShape shapeOf(const spo_moe_shape &s) { return {s.hidden, s.ffn, s.experts, s.top_k}; }
+ops::MoeShape shapeOf(const spo_moe_shape &s) { return {s.hidden, s.ffn, s.experts, s.top_k, s.shared_slices, s.shared_gate != 0}; }
 ops::MoeWorkspace workspaceOf(const spo_moe_workspace &w) {
   return {B(w.selected), B(w.weights), B(w.route_slot), B(w.slot_row), B(w.tile_expert), B(w.tile_rows), B(w.tile_total), B(w.tables),
           B(w.next_tables), B(w.intermediate), B(w.expert_output)};
@@ -28,10 +28,11 @@ sp_status spo_moe_workspace_sizes(const spo_moe_shape *shape, uint32_t rows, uin
 }
 
 sp_status spo_moe_add_routing(spo_graph *graph, sp_buffer *scores, uint32_t score_stride, const spo_moe_workspace *workspace,
-                              const spo_moe_shape *shape, uint32_t rows) {
+                              const spo_moe_shape *shape, uint32_t rows, sp_buffer *input, sp_buffer *shared_scalar_gate) {
   return capi::guard([&] {
     capi::require(graph && workspace && shape, "graph, workspace or shape");
-    ops::MoE::addRouting(capi::graphOf(graph), B(scores), score_stride, workspaceOf(*workspace), shapeOf(*shape), rows);
+    ops::MoE::addRouting(capi::graphOf(graph), B(scores), score_stride, workspaceOf(*workspace), shapeOf(*shape), rows,
+                         input ? B(input) : hip::Buffer{}, shared_scalar_gate ? B(shared_scalar_gate) : hip::Buffer{});
   });
 }
 

@@ -9,11 +9,28 @@ namespace splash::kernels {
 
 // moe_route_select (moe.metal:23-113): one wave per row; lane l holds experts l, l + 64, ... Each
 // rank takes the highest remaining score and, among equals, the lowest expert id.
-__global__ __launch_bounds__(64) void moe_route_select(const float *__restrict__ scores, uint32_t *__restrict__ selected,
+// A gated shared expert's weight is the sigmoid of the row's product with the scalar gate: lane l sums dimensions l,
+// l + 64, ... in order, the lanes' sums add by the wave's exchanges at distances 32, 16, ... 1.
+__global__ __launch_bounds__(64) void moe_route_select(const float *__restrict__ scores, const uint16_t *__restrict__ input,
+                                                       const float *__restrict__ shared_gate, uint32_t *__restrict__ selected,
                                                        float *__restrict__ weights, MoeRouteParams p) {
   constexpr uint32_t kPerLane = MOE_MAXIMUM_EXPERTS / 64u;
   __shared__ float ordered[MOE_MAXIMUM_TOP];
-  const uint32_t row = blockIdx.x, lane = threadIdx.x;
+  const uint32_t row = blockIdx.x, lane = threadIdx.x, perRow = p.top_k + p.shared;
+  if (p.shared) {
+    float weight = 1.0f;
+    if (p.shared_gated) {
+      const uint16_t *x = input + size_t(row) * p.input_size;
+      float scalar = 0.f;
+      for (uint32_t d = lane; d < p.input_size; d += 64u) scalar += bf16_bits_to_float(x[d]) * shared_gate[d];
+      scalar = wave_sum(scalar);
+      weight = 1.0f / (1.0f + __builtin_amdgcn_exp2f(-1.44269504089f * scalar));
+    }
+    if (lane < p.shared) {
+      selected[size_t(row) * perRow + p.top_k + lane] = p.experts + lane;
+      weights[size_t(row) * perRow + p.top_k + lane] = weight;
+    }
+  }
   float mine[kPerLane];
 #pragma unroll
   for (uint32_t slot = 0; slot < kPerLane; ++slot) {
@@ -41,14 +58,14 @@ __global__ __launch_bounds__(64) void moe_route_select(const float *__restrict__
     }
     if (lane == 0) {
       ordered[rank] = rowBest;
-      selected[size_t(row) * p.top_k + rank] = winner;
+      selected[size_t(row) * perRow + rank] = winner;
     }
   }
   __syncthreads();
   if (lane < p.top_k) {
     float denominator = 0.f;
     for (uint32_t other = 0; other < p.top_k; ++other) denominator += __builtin_amdgcn_exp2f((ordered[other] - ordered[0]) * 1.44269504089f);
-    weights[size_t(row) * p.top_k + lane] = __builtin_amdgcn_exp2f((ordered[lane] - ordered[0]) * 1.44269504089f) / denominator;
+    weights[size_t(row) * perRow + lane] = __builtin_amdgcn_exp2f((ordered[lane] - ordered[0]) * 1.44269504089f) / denominator;
   }
 }
 SP_REGISTER_KERNEL("moe_route_select", &moe_route_select);

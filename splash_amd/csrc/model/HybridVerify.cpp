@@ -116,7 +116,7 @@ uint64_t HybridVerify::stepBytes(const std::vector<HybridLane> &lanes) const {
   uint64_t bytes = weights_.head.weightBytes();
   for (const HybridLayer &l : weights_.layers) {
     bytes += l.mixerInput.weightBytes() + l.mixerOutput.weightBytes() + l.router.weightBytes();
-    bytes += uint64_t{moe.experts} * (2 * gguf_image_bytes(l.experts.format, moe.ffn, moe.hidden) +
+    bytes += uint64_t{moe.allExperts()} * (2 * gguf_image_bytes(l.experts.format, moe.ffn, moe.hidden) +
                                       gguf_image_bytes(l.experts.downFormat, moe.hidden, moe.ffn));
   }
   uint32_t rows = 0;
@@ -219,7 +219,7 @@ void HybridVerify::encodeLayer(hip::CommandGraph &graph, uint32_t layer, const s
     linear_.add(graph, router, w.router, linear_.plan(w.router, count));
   });
   const ops::MoeShape moe = dims_.moeShape();
-  ops::MoE::addRouting(graph, scores_, dims_.experts, moeWorkspace_, moe, rows);
+  ops::MoE::addRouting(graph, scores_, dims_.experts, moeWorkspace_, moe, rows, normalized_, w.sharedScalarGate);
   ops::MoeFollowingNorm following;
   if (feedsNext) {
     following.weight = layer + 1 < dims_.layers ? weights_.layers[layer + 1].inputNorm : weights_.finalNorm;

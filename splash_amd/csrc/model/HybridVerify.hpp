@@ -36,6 +36,9 @@ struct HybridDimensions final {
   uint32_t gdnKeyHeads = 0, gdnValueHeads = 0;
   uint32_t gdnPackedWidth = 0;  // the GDN input projection's width (whole column tiles)
   uint32_t experts = 0, topK = 0, expertFfn = 0;
+  // The shared expert: slices of the routed experts' width every row visits, gated by the layer's scalar gate or not.
+  uint32_t sharedSlices = 0;
+  bool sharedGate = false;
 
   [[nodiscard]] bool attends(uint32_t layer) const noexcept { return (layer + 1) % attentionInterval == 0; }
   [[nodiscard]] uint32_t attentionLayers() const noexcept { return layers / attentionInterval; }
@@ -56,7 +59,7 @@ struct HybridDimensions final {
     s.packedWidth = gdnPackedWidth;
     return s;
   }
-  [[nodiscard]] ops::MoeShape moeShape() const noexcept { return {hidden, expertFfn, experts, topK}; }
+  [[nodiscard]] ops::MoeShape moeShape() const noexcept { return {hidden, expertFfn, experts, topK, sharedSlices, sharedGate}; }
 };
 
 struct HybridLayer final {
@@ -66,7 +69,8 @@ struct HybridLayer final {
   hip::Buffer queryNorm, keyNorm;                                   // attention layers: bf16 [head dimension]
   hip::Buffer convolutionWeights, decay, timeBias, mixerNorm;       // GDN layers (mixerNorm bf16 [128])
   ops::Projection router;                                           // hidden -> experts, fp32 scores
-  ops::MoeExperts experts;
+  ops::MoeExperts experts;                                          // the shared slices' images after the routed experts'
+  hip::Buffer sharedScalarGate;                                     // fp32 [hidden], of a gated shared expert
 };
 
 struct HybridWeights final {

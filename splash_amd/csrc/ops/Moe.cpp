@@ -12,8 +12,8 @@ void requireShape(const MoeShape &shape, uint32_t rows) {
   if (!shape.valid()) throw std::invalid_argument("invalid MoE shape");
   if (!rows || rows > kMaximumRows) throw std::invalid_argument("a MoE step takes 1 to 256 rows");
   // The grouping kernel's bit matrix, a row an expert and a bit a route, lives in one workgroup's LDS.
-  if (uint64_t{shape.experts} * ((uint64_t{rows} * shape.topK + 31) / 32) > MOE_GROUP_WORDS)
-    throw std::invalid_argument("too many experts for that many routes: experts * ceil(rows * top_k / 32) is at most 16384");
+  if (uint64_t{shape.allExperts()} * ((uint64_t{rows} * shape.routesPerRow() + 31) / 32) > MOE_GROUP_WORDS)
+    throw std::invalid_argument("too many experts for that many routes: experts * ceil(rows * routes a row / 32) is at most 16384");
 }
 const char *formatName(uint32_t format) {
   if (format == GGUF_FMT_Q4K) return "q4k";
@@ -24,7 +24,8 @@ const char *formatName(uint32_t format) {
 
 MoeWorkspaceSize MoE::workspace(const MoeShape &shape, uint32_t rows) {
   requireShape(shape, rows);
-  const uint64_t routes = uint64_t{rows} * shape.topK, tiles = moe_maximum_tiles(uint32_t(routes), shape.experts), slots = tiles * MOE_TILE_ROWS;
+  const uint64_t routes = uint64_t{rows} * shape.routesPerRow(), tiles = moe_maximum_tiles(uint32_t(routes), shape.allExperts()),
+                 slots = tiles * MOE_TILE_ROWS;
   MoeWorkspaceSize s;
   s.selected = routes * 4;
   s.weights = routes * 4;
@@ -40,8 +41,12 @@ MoeWorkspaceSize MoE::workspace(const MoeShape &shape, uint32_t rows) {
 }
 
 void MoE::addRouting(hip::CommandGraph &graph, const hip::Buffer &scores, uint32_t scoreStride, const MoeWorkspace &w,
-                     const MoeShape &shape, uint32_t rows) {
+                     const MoeShape &shape, uint32_t rows, const hip::Buffer &input, const hip::Buffer &sharedScalarGate) {
   requireShape(shape, rows);
+  if (shape.sharedGate) {
+    requireBytes(input, uint64_t{rows} * shape.hidden * 2, "router input rows");
+    requireBytes(sharedScalarGate, uint64_t{shape.hidden} * 4, "shared expert gate");
+  }
   if (scoreStride < shape.experts) throw std::invalid_argument("a row of scores holds every expert's");
   const MoeWorkspaceSize need = workspace(shape, rows);
   requireBytes(scores, (uint64_t{rows - 1} * scoreStride + shape.experts) * 4, "router scores");
@@ -52,11 +57,14 @@ void MoE::addRouting(hip::CommandGraph &graph, const hip::Buffer &scores, uint32
   requireBytes(w.tileExpert, need.tileExpert, "tile experts");
   requireBytes(w.tileRows, need.tileRows, "tile rows");
   requireBytes(w.tileTotal, 4, "tile count");
-  const uint32_t routes = rows * shape.topK;
-  graph.add("moe_route_select", {scores, w.selected, w.weights}, MoeRouteParams{rows, shape.experts, shape.topK, scoreStride}, {rows, 1, 1},
+  const uint32_t routes = rows * shape.routesPerRow();
+  graph.add("moe_route_select", {scores, shape.sharedGate ? input : scores, shape.sharedGate ? sharedScalarGate : scores, w.selected, w.weights},
+            MoeRouteParams{rows, shape.experts, shape.topK, scoreStride, shape.sharedSlices, shape.sharedGate, shape.hidden, 0}, {rows, 1, 1},
             {64, 1, 1});
+  // The grouping and the combine take the shared slices as further experts and routes of a row.
   graph.add("moe_group_routes", {w.selected, w.routeSlot, w.slotRow, w.tileExpert, w.tileRows, w.tileTotal},
-            MoeGroupParams{routes, shape.experts, shape.topK, moe_maximum_tiles(routes, shape.experts)}, {1, 1, 1}, {1024, 1, 1});
+            MoeGroupParams{routes, shape.allExperts(), shape.routesPerRow(), moe_maximum_tiles(routes, shape.allExperts())}, {1, 1, 1},
+            {1024, 1, 1});
 }
 
 void MoE::addRouted(hip::CommandGraph &graph, const hip::Buffer &normalized, const hip::Buffer &residual, const hip::Buffer &output,
@@ -70,7 +78,7 @@ void MoE::addRouted(hip::CommandGraph &graph, const hip::Buffer &normalized, con
     requireBytes(following.table, gguf_tables_bytes(shape.hidden, gguf_row_tiles(rows)), "next projection table");
   }
   const MoeWorkspaceSize need = workspace(shape, rows);
-  const uint32_t routes = rows * shape.topK, tiles = moe_maximum_tiles(routes, shape.experts);
+  const uint32_t routes = rows * shape.routesPerRow(), tiles = moe_maximum_tiles(routes, shape.allExperts());
   const std::string pairKernel = std::string("gguf_moe_decode_") + formatName(experts.format) + "_gt";
   if (experts.format != GGUF_FMT_Q4K) throw std::invalid_argument("routed gate and up projections are Q4_K");
   const std::string downKernel = std::string("gguf_moe_decode_") + formatName(experts.downFormat) + "_a";
@@ -79,9 +87,9 @@ void MoE::addRouted(hip::CommandGraph &graph, const hip::Buffer &normalized, con
   requireBytes(normalized, uint64_t{rows} * shape.hidden * 2, "normalized rows");
   requireBytes(residual, uint64_t{rows} * shape.hidden * 2, "residual rows");
   requireBytes(output, uint64_t{rows} * shape.hidden * 2, "MoE output");
-  requireBytes(experts.gate, pairBytes * shape.experts, "expert gate images");
-  requireBytes(experts.up, pairBytes * shape.experts, "expert up images");
-  requireBytes(experts.down, downBytes * shape.experts, "expert down images");
+  requireBytes(experts.gate, pairBytes * shape.allExperts(), "expert gate images");
+  requireBytes(experts.up, pairBytes * shape.allExperts(), "expert up images");
+  requireBytes(experts.down, downBytes * shape.allExperts(), "expert down images");
   requireBytes(w.routeSlot, need.routeSlot, "route slots");
   requireBytes(w.slotRow, need.slotRow, "slot rows");
   requireBytes(w.tileExpert, need.tileExpert, "tile experts");
@@ -123,7 +131,7 @@ void MoE::addRouted(hip::CommandGraph &graph, const hip::Buffer &normalized, con
   graph.add("moe_combine",
             {w.expertOutput, w.routeSlot, w.weights, residual, output, writesTable ? following.weight : output,
              writesTable ? following.table : output},
-            MoeCombineParams{rows, shape.hidden, shape.topK, writesTable ? gguf_row_tiles(rows) : 0u},
+            MoeCombineParams{rows, shape.hidden, shape.routesPerRow(), writesTable ? gguf_row_tiles(rows) : 0u},
             {rows, (shape.hidden + 255) / 256, 1}, {256, 1, 1});
 }
 

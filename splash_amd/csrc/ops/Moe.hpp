@@ -9,9 +9,18 @@ namespace splash::ops {
 
 struct MoeShape final {
   uint32_t hidden = 0, ffn = 0, experts = 0, topK = 0;
+  // The shared expert is sharedSlices experts every row visits after its routed ones, ids experts to
+  // experts + sharedSlices - 1, each of the routed experts' width (a shared expert sharedSlices times that wide is
+  // their sum); with sharedGate each slice's weight is the sigmoid of the row's product with the block's scalar gate,
+  // else 1 (the reference's MoeShape, runtime/ops/MoE.hpp:50-63). Their images follow the routed experts' in the
+  // same buffers, in the same formats.
+  uint32_t sharedSlices = 0;
+  bool sharedGate = false;
+  [[nodiscard]] uint32_t routesPerRow() const noexcept { return topK + sharedSlices; }
+  [[nodiscard]] uint32_t allExperts() const noexcept { return experts + sharedSlices; }
   [[nodiscard]] bool valid() const noexcept {
-    return hidden && hidden % GGUF_BLOCK == 0 && ffn && ffn % GGUF_BLOCK == 0 && experts && experts <= MOE_MAXIMUM_EXPERTS && topK &&
-           topK <= MOE_MAXIMUM_TOP && topK <= experts;
+    return hidden && hidden % GGUF_BLOCK == 0 && ffn && ffn % GGUF_BLOCK == 0 && experts && allExperts() <= MOE_MAXIMUM_EXPERTS && topK &&
+           routesPerRow() <= MOE_MAXIMUM_TOP && topK <= experts && sharedSlices <= 64 && (sharedSlices || !sharedGate);
   }
 };
 // Every expert's re-tiled image of a tensor, expert e at e * gguf_image_bytes(format, rows, inputs).
@@ -45,9 +54,11 @@ struct MoeFollowingNorm final {
 class MoE final {
 public:
   [[nodiscard]] static MoeWorkspaceSize workspace(const MoeShape &shape, uint32_t rows);
-  // Selects and weighs each row's experts from its fp32 router scores ([rows][scoreStride]) and groups the routes.
+  // Selects and weighs each row's experts from its fp32 router scores ([rows][scoreStride]), appends the shape's shared
+  // slices to every row's routes and groups the routes. `input` (the normalized rows, bf16 [rows][hidden]) and
+  // `sharedScalarGate` (fp32 [hidden]) only for a gated shared expert (MoE.hpp:410-416 in the reference).
   static void addRouting(hip::CommandGraph &graph, const hip::Buffer &scores, uint32_t scoreStride, const MoeWorkspace &workspace,
-                         const MoeShape &shape, uint32_t rows);
+                         const MoeShape &shape, uint32_t rows, const hip::Buffer &input = {}, const hip::Buffer &sharedScalarGate = {});
   // output = bf16(residual + sum over a row's routes of weight * down(silu(gate x) * up x)) of its experts, x = normalized.
   // `following` (optional): the output rows also leave as the activation table of the projection after their RMS
   // norm under following.weight, as a LinearEpilogue::ResidualNorm plan writes it (that projection reads it as

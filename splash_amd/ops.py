@@ -384,18 +384,20 @@ class GDN:
 class MoE:
     """ops::MoE: routing (addRouting) and the routed experts with their weighted sum (addRouted)."""
 
-    def __init__(self, backend, hidden, ffn, experts, top_k, rows):
-        self.shape = nat.MoeShape(hidden, ffn, experts, top_k)
+    def __init__(self, backend, hidden, ffn, experts, top_k, rows, shared_slices=0, shared_gate=False):
+        self.shape = nat.MoeShape(hidden, ffn, experts, top_k, shared_slices, int(shared_gate))
         self.rows = rows
         sizes = (ctypes.c_uint64 * 11)()
         check(lib.spo_moe_workspace_sizes(ctypes.byref(self.shape), rows, sizes))
         self.buffers = {n: backend.allocate_buffer(max(int(b), 16), STORAGE_PRIVATE, "moe " + n) for n, b in zip(nat.MOE_WORKSPACE_FIELDS, sizes)}
         self.workspace = nat.MoeWorkspace(**{n: b.handle for n, b in self.buffers.items()})
 
-    def add_routing(self, graph, scores, rows=None, score_stride=None):
+    def add_routing(self, graph, scores, rows=None, score_stride=None, input=None, shared_scalar_gate=None):
+        """input (the normalized rows) and shared_scalar_gate (fp32 [hidden]): of a shape with a gated shared expert."""
         check(lib.spo_moe_add_routing(graph.handle, scores.handle, score_stride or self.shape.experts, ctypes.byref(self.workspace),
-                                      ctypes.byref(self.shape), rows or self.rows))
-        graph._keep.extend([scores, self])
+                                      ctypes.byref(self.shape), rows or self.rows, input.handle if input is not None else None,
+                                      shared_scalar_gate.handle if shared_scalar_gate is not None else None))
+        graph._keep.extend([scores, self, input, shared_scalar_gate])
 
     def add_routed(self, graph, normalized, residual, output, gate_images, up_images, down_images, rows=None, fmt=FMT_Q4K,
                    down_fmt=FMT_Q4K, norm_weight=None, next_table=None):

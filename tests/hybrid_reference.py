@@ -9,12 +9,13 @@ from tests import oracle as orc
 
 class HybridModel:
     def __init__(self, seed, hidden, vocabulary, layers, q_heads, kv_heads, head_dim, gdn_key_heads, gdn_value_heads, experts, top_k,
-                 expert_ffn, attention_interval=4, rope_theta=1e6, gated_attention=False):
+                 expert_ffn, attention_interval=4, rope_theta=1e6, gated_attention=False, shared_slices=0, shared_gate=False):
         self.dims = dict(hidden=hidden, vocabulary=vocabulary, layers=layers, q_heads=q_heads, kv_heads=kv_heads, head_dim=head_dim,
                          gdn_key_heads=gdn_key_heads, gdn_value_heads=gdn_value_heads, experts=experts, top_k=top_k, expert_ffn=expert_ffn,
                          attention_interval=attention_interval)
         self.rope_theta = rope_theta
         self.gated = gated_attention       # a query head's rows of the projection: its queries, then its gate
+        self.shared_slices, self.shared_gate = shared_slices, shared_gate   # the shared expert, after the routed experts
         rng = np.random.default_rng(seed)
         self.rng = rng
         D = head_dim
@@ -30,8 +31,11 @@ class HybridModel:
         self.layers = []
         for l in range(layers):
             w = dict(input_norm=norm(hidden), post_norm=norm(hidden), router=quant(experts, hidden, orc.FMT_Q6K, 0.05),
-                     gate=[quant(expert_ffn, hidden) for _ in range(experts)], up=[quant(expert_ffn, hidden) for _ in range(experts)],
-                     down=[quant(hidden, expert_ffn) for _ in range(experts)])
+                     gate=[quant(expert_ffn, hidden) for _ in range(experts + shared_slices)],
+                     up=[quant(expert_ffn, hidden) for _ in range(experts + shared_slices)],
+                     down=[quant(hidden, expert_ffn) for _ in range(experts + shared_slices)])
+            if shared_gate:
+                w["shared_scalar_gate"] = (rng.standard_normal(hidden) * 0.05).astype(np.float32)
             if self.attends(l):
                 w.update(q=quant(q_heads * D * (2 if self.gated else 1), hidden), k=quant(kv_heads * D, hidden), v=quant(kv_heads * D, hidden),
                          o=quant(hidden, q_heads * D), q_norm=norm(D), k_norm=norm(D))
@@ -57,7 +61,7 @@ class HybridModel:
         gpu = verify.HybridVerify(backend, d["hidden"], d["vocabulary"], d["layers"], d["q_heads"], d["kv_heads"], d["head_dim"],
                                   d["gdn_key_heads"], d["gdn_value_heads"], d["experts"], d["top_k"], d["expert_ffn"],
                                   attention_interval=d["attention_interval"], rope_theta=self.rope_theta, max_lanes=max_lanes,
-                                  gated_attention=self.gated,
+                                  gated_attention=self.gated, shared_slices=self.shared_slices, shared_gate=self.shared_gate,
                                   physical_pages=self.physical_pages, page_table_entries=max_lanes * pages_per_lane)
         assert gpu.dims.gdn_packed_width == self.packed_width
         self.table = np.random.default_rng(99).permutation(self.physical_pages)[:max_lanes * pages_per_lane].astype(np.uint64)
@@ -69,6 +73,8 @@ class HybridModel:
             common = dict(input_norm=backend.from_array(w["input_norm"]), post_norm=backend.from_array(w["post_norm"]),
                           router=P([(orc.FMT_Q6K, d["experts"], w["router"])], H, True), gate_images=images(orc.FMT_Q4K, w["gate"], F, H),
                           up_images=images(orc.FMT_Q4K, w["up"], F, H), down_images=images(orc.FMT_Q4K, w["down"], H, F))
+            if self.shared_gate:
+                common["shared_scalar_gate"] = backend.from_array(w["shared_scalar_gate"])
             if self.attends(i):
                 gpu.set_layer(i, P([(orc.FMT_Q4K, d["q_heads"] * D * (2 if self.gated else 1), w["q"]), (orc.FMT_Q4K, d["kv_heads"] * D, w["k"]),
                                     (orc.FMT_Q4K, d["kv_heads"] * D, w["v"])], H), P([(orc.FMT_Q4K, H, w["o"])], d["q_heads"] * D),
@@ -201,7 +207,8 @@ class HybridModel:
         w, d = self.layers[li], self.dims
         n = orc.rms_norm(hidden1, w["post_norm"])
         scores = self._project(orc.FMT_Q6K, w["router"], n, d["experts"]).astype(np.float32)
-        _, _, _, out = orc.moe_layer(n, hidden1, scores, d["top_k"], w["gate"], w["up"], w["down"], d["expert_ffn"])
+        _, _, _, out = orc.moe_layer(n, hidden1, scores, d["top_k"], w["gate"], w["up"], w["down"], d["expert_ffn"],
+                                     shared=self.shared_slices, shared_gate=w.get("shared_scalar_gate"))
         return scores, out
 
     def oracle_head(self, hidden):

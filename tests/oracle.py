@@ -444,12 +444,22 @@ lib.orc_moe_combine.restype = None
 lib.orc_moe_combine.argtypes = [u16p, f32p, u16p, c_u32, c_u32, c_u32, u16p]
 
 
-def moe_route(scores, top_k):
+def moe_route(scores, top_k, shared=0, x_bits=None, shared_gate=None):
+    """Each row's routes: its top_k routed experts, then `shared` slices of the shared expert (ids experts on), each
+    weighing sigmoid(x . shared_gate) or, without a gate, 1."""
     scores = np.ascontiguousarray(scores, np.float32)
     rows, experts = scores.shape
     selected = np.zeros((rows, top_k), np.uint32)
     weights = np.zeros((rows, top_k), np.float32)
     lib.orc_moe_route(_p(scores, f32p), rows, experts, experts, top_k, _p(selected, u32p), _p(weights, f32p))
+    if shared:
+        gate = np.ones(rows, np.float32)
+        if shared_gate is not None:
+            x = np.ascontiguousarray(x_bits, np.uint16)
+            g = np.ascontiguousarray(shared_gate, np.float32)
+            lib.orc_moe_shared_weights(_p(x, u16p), _p(g, f32p), rows, x.shape[1], _p(gate, f32p))
+        selected = np.concatenate([selected, np.tile(experts + np.arange(shared, dtype=np.uint32), (rows, 1))], axis=1)
+        weights = np.concatenate([weights, np.tile(gate[:, None], (1, shared))], axis=1)
     return selected, weights
 
 
@@ -461,12 +471,14 @@ def moe_combine(y_bits, weights, residual_bits):
     return out
 
 
-def moe_layer(x_bits, residual_bits, scores, top_k, gate_native, up_native, down_native, ffn, fmt=FMT_Q4K, down_fmt=FMT_Q4K):
-    """The routed experts of a layer: x bf16 [rows][hidden] (normalized), natives per expert. Each expert's
-    rows go through the oracle's projections together; a row's result does not depend on the rows beside it."""
+def moe_layer(x_bits, residual_bits, scores, top_k, gate_native, up_native, down_native, ffn, fmt=FMT_Q4K, down_fmt=FMT_Q4K,
+              shared=0, shared_gate=None):
+    """The routed experts of a layer: x bf16 [rows][hidden] (normalized), natives per expert (the shared slices' after
+    the routed experts'). Each expert's rows go through the oracle's projections together; a row's result does not
+    depend on the rows beside it."""
     rows, hidden = x_bits.shape
-    selected, weights = moe_route(scores, top_k)
-    y = np.zeros((rows, top_k, hidden), np.uint16)
+    selected, weights = moe_route(scores, top_k, shared, x_bits, shared_gate)
+    y = np.zeros((rows, top_k + shared, hidden), np.uint16)
     for e in np.unique(selected):
         r, k = np.nonzero(selected == e)
         xe = np.ascontiguousarray(x_bits[r])

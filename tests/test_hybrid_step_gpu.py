@@ -136,6 +136,20 @@ def test_config5_more_rows_than_one_projection_takes(backend, gated):
     check_step(backend, model, gpu, lanes, rng.integers(0, SHAPE["vocabulary"], 80).astype(np.uint32))
 
 
+@pytest.mark.parametrize("gate", [True, False])
+def test_config5_with_a_shared_expert(backend, gate):
+    """The reference's Qwen3.5 MoE blocks add a shared expert every row visits (MoE.hpp:50-63), gated by the sigmoid of
+    the row's product with the block's scalar gate: two lanes, layer by layer against the oracle."""
+    print(f"case config 5 hybrid shared expert gate={gate}", flush=True)
+    model = HybridModel(seed=43, shared_slices=1, shared_gate=gate, **SHAPE)
+    gpu = model.build_gpu(backend, max_lanes=2, pages_per_lane=1)
+    rng = np.random.default_rng(8)
+    model.seed_context(rng)
+    model.seed_states(rng, lanes=2)
+    lanes = [verify.HybridLane(16, 40, table_first=0), verify.HybridLane(9, 100, table_first=1)]
+    check_step(backend, model, gpu, lanes, rng.integers(0, SHAPE["vocabulary"], 25).astype(np.uint32))
+
+
 def test_hybrid_rejects_bad_arguments(backend):
     with pytest.raises(ValueError):
         verify.HybridVerify(backend, **{**SHAPE, "layers": 5})            # not whole groups of four layers

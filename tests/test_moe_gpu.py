@@ -9,32 +9,38 @@ from tests import oracle as orc
 pytestmark = pytest.mark.gpu
 
 
-def run_layer(backend, rng, hidden, ffn, experts, top_k, rows, down_fmt=ops.FMT_Q4K, following=None):
-    gate = [orc.make_native(ops.FMT_Q4K, ffn, hidden, 100 + e) for e in range(experts)]
-    up = [orc.make_native(ops.FMT_Q4K, ffn, hidden, 300 + e) for e in range(experts)]
-    down = [orc.make_native(down_fmt, hidden, ffn, 500 + e) for e in range(experts)]
+def run_layer(backend, rng, hidden, ffn, experts, top_k, rows, down_fmt=ops.FMT_Q4K, following=None, shared=0, gated=False):
+    """shared: slices of a shared expert, whose images follow the routed experts'; gated: they weigh sigmoid(x . gate)."""
+    gate = [orc.make_native(ops.FMT_Q4K, ffn, hidden, 100 + e) for e in range(experts + shared)]
+    up = [orc.make_native(ops.FMT_Q4K, ffn, hidden, 300 + e) for e in range(experts + shared)]
+    down = [orc.make_native(down_fmt, hidden, ffn, 500 + e) for e in range(experts + shared)]
     images = [backend.from_array(np.concatenate([ops.pack_gguf_image(f, n, r, k) for n in natives]))
               for natives, f, r, k in ((gate, ops.FMT_Q4K, ffn, hidden), (up, ops.FMT_Q4K, ffn, hidden), (down, down_fmt, hidden, ffn))]
     x = orc.f32_to_bf16(rng.standard_normal((rows, hidden)).astype(np.float32))
     res = orc.f32_to_bf16(rng.standard_normal((rows, hidden)).astype(np.float32))
     scores = rng.standard_normal((rows, experts)).astype(np.float32)
     scores[0, :] = 0.5                                 # a row of ties: experts 0..top_k-1 in id order
-    moe = ops.MoE(backend, hidden, ffn, experts, top_k, rows)
+    moe = ops.MoE(backend, hidden, ffn, experts, top_k, rows, shared_slices=shared, shared_gate=gated)
     out = backend.allocate_buffer(rows * hidden * 2)
     graph = splash_amd.CommandGraph()
-    moe.add_routing(graph, backend.from_array(scores))
+    scalar_gate = (rng.standard_normal(hidden) * 0.05).astype(np.float32) if gated else None
+    moe.add_routing(graph, backend.from_array(scores), input=backend.from_array(x) if gated else None,
+                    shared_scalar_gate=backend.from_array(scalar_gate) if gated else None)
     extra = dict(norm_weight=following[0], next_table=following[1]) if following else {}
     moe.add_routed(graph, backend.from_array(x), backend.from_array(res), out, *images, down_fmt=down_fmt, **extra)
     assert len(graph) == 6
     backend.run(graph)
     got = out.download(np.uint16).reshape(rows, hidden)
-    want = orc.moe_layer(x, res, scores, top_k, gate, up, down, ffn, down_fmt=down_fmt)
+    want = orc.moe_layer(x, res, scores, top_k, gate, up, down, ffn, down_fmt=down_fmt, shared=shared, shared_gate=scalar_gate)
     return moe, got, want
 
 
-def check_layer(moe, got, want, rows, experts, top_k):
+def check_layer(moe, got, want, rows, experts, top_k, shared=0):
     selected, weights, y, out = want
     b = moe.buffers
+    routed = top_k
+    top_k, experts = top_k + shared, experts + shared      # the shared slices are further routes of a row, and experts
+    assert np.array_equal(selected[:, routed:], np.tile(experts - shared + np.arange(shared), (rows, 1)))
     got_selected = b["selected"].download(np.uint32)[:rows * top_k].reshape(rows, top_k)
     assert np.array_equal(got_selected, selected)                        # routing is exact, ties by id
     got_weights = b["weights"].download(np.float32)[:rows * top_k].reshape(rows, top_k)
@@ -74,6 +80,21 @@ def test_moe_layer_matches_the_oracle(backend, config):
     rng = np.random.default_rng(experts)
     moe, got, want = run_layer(backend, rng, hidden, ffn, experts, top_k, rows)
     check_layer(moe, got, want, rows, experts, top_k)
+
+
+@pytest.mark.parametrize("config", [(512, 256, 8, 2, 20, 1, True), (256, 256, 6, 3, 40, 2, False), (1024, 512, 64, 4, 48, 1, False),
+                                    (2048, 768, 128, 8, 128, 1, True)])
+def test_shared_expert_slices_ride_every_row(backend, config):
+    """The shared expert as further routes of every row (moe.metal:5-8, :42-65; MoE.hpp:50-63): ids `experts` on, gated
+    by the sigmoid of the row's product with the block's scalar gate or weighing 1, through the same grouping, expert
+    projections and combine; the last case is a 35B-A3B layer with its shared expert."""
+    print(f"case moe shared {config}", flush=True)
+    hidden, ffn, experts, top_k, rows, shared, gated = config
+    rng = np.random.default_rng(experts + shared)
+    moe, got, want = run_layer(backend, rng, hidden, ffn, experts, top_k, rows, shared=shared, gated=gated)
+    check_layer(moe, got, want, rows, experts, top_k, shared)
+    if not gated:
+        assert np.all(want[1][:, top_k:] == 1.0)
 
 
 def test_moe_layer_at_the_35b_shape(backend):
