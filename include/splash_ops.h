@@ -365,6 +365,7 @@ typedef struct spo_hybrid_dimensions {
   uint32_t gdn_key_heads, gdn_value_heads, gdn_packed_width; /* packed row [q|k|v|z|b|a], whole column tiles */
   uint32_t experts, top_k, expert_ffn;
   uint32_t shared_slices, shared_gate; /* the shared expert, as in spo_moe_shape */
+  uint32_t dense_ffn; /* with experts 0: every layer's FFN is a dense SwiGLU of this width (QwenTarget.cpp:351-370) */
 } spo_hybrid_dimensions;
 typedef struct spo_hybrid_lane {
   spo_verify_lane block;
@@ -380,6 +381,7 @@ typedef struct spo_hybrid_layer {
   sp_buffer *gate_images, *up_images, *down_images;                   /* every expert's image of each tensor */
   uint32_t expert_format, expert_down_format;
   sp_buffer *shared_scalar_gate; /* fp32 [hidden], of a gated shared expert (NULL otherwise) */
+  const spo_projection *ffn_gate, *ffn_up, *ffn_down; /* a dense model's SwiGLU (router and images NULL) */
 } spo_hybrid_layer;
 sp_status spo_hybrid_verify_create(sp_backend *backend, const spo_hybrid_dimensions *dimensions, uint32_t max_lanes,
                                    uint32_t physical_pages, uint32_t page_table_entries, spo_hybrid_verify **out);

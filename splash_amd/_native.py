@@ -158,7 +158,7 @@ class HybridDimensions(ctypes.Structure):
     _fields_ = [(n, c_u32) for n in ("hidden", "vocabulary", "layers", "attention_interval", "q_heads", "kv_heads", "head_dim",
                                      "rotary_pairs", "normalize_heads", "gated_attention")] + [("rope_theta", ctypes.c_float)] + [
         (n, c_u32) for n in ("gdn_key_heads", "gdn_value_heads", "gdn_packed_width", "experts", "top_k", "expert_ffn", "shared_slices",
-                             "shared_gate")]
+                             "shared_gate", "dense_ffn")]
 
 
 class HybridLane(ctypes.Structure):
@@ -169,7 +169,8 @@ class HybridLayer(ctypes.Structure):
     _fields_ = [(n, c_p) for n in ("mixer_input", "mixer_output", "input_norm", "post_norm", "query_norm", "key_norm",
                                    "convolution_weights", "decay_weights", "time_bias", "mixer_norm", "router", "gate_images",
                                    "up_images", "down_images")] + [("expert_format", c_u32), ("expert_down_format", c_u32),
-                                                                    ("shared_scalar_gate", c_p)]
+                                                                    ("shared_scalar_gate", c_p), ("ffn_gate", c_p), ("ffn_up", c_p),
+                                                                    ("ffn_down", c_p)]
 
 
 def _sig(name, restype, *argtypes):

@@ -57,6 +57,7 @@ sp_status spo_hybrid_verify_create(sp_backend *backend, const spo_hybrid_dimensi
     dims.expertFfn = d->expert_ffn;
     dims.sharedSlices = d->shared_slices;
     dims.sharedGate = d->shared_gate != 0;
+    dims.denseFfn = d->dense_ffn;
     holder->verify = std::make_unique<model::HybridVerify>(*holder->backend, dims, max_lanes, physical_pages, page_table_entries);
     *out = holder.release();
   });
@@ -65,7 +66,9 @@ void spo_hybrid_verify_destroy(spo_hybrid_verify *verify) { delete verify; }
 
 sp_status spo_hybrid_verify_set_layer(spo_hybrid_verify *verify, uint32_t layer, const spo_hybrid_layer *l) {
   return capi::guard([&] {
-    capi::require(verify && l && l->mixer_input && l->mixer_output && l->router, "verify, layer or projections");
+    capi::require(verify && l && l->mixer_input && l->mixer_output, "verify, layer or projections");
+    const bool dense = verify->verify->dimensions().dense();
+    capi::require(dense ? (l->ffn_gate && l->ffn_up && l->ffn_down) : l->router != nullptr, "the layer's FFN");
     model::HybridWeights &w = verify->verify->weights();
     if (layer >= w.layers.size()) throw std::invalid_argument("no such layer");
     model::HybridLayer out;
@@ -79,9 +82,15 @@ sp_status spo_hybrid_verify_set_layer(spo_hybrid_verify *verify, uint32_t layer,
     out.decay = B(l->decay_weights);
     out.timeBias = B(l->time_bias);
     out.mixerNorm = B(l->mixer_norm);
-    out.router = capi::projectionOf(l->router);
-    out.router.destination = ops::FloatOutput::Float32;
-    out.experts = {B(l->gate_images), B(l->up_images), B(l->down_images), l->expert_format, l->expert_down_format};
+    if (dense) {
+      out.ffnGate = capi::projectionOf(l->ffn_gate);
+      out.ffnUp = capi::projectionOf(l->ffn_up);
+      out.ffnDown = capi::projectionOf(l->ffn_down);
+    } else {
+      out.router = capi::projectionOf(l->router);
+      out.router.destination = ops::FloatOutput::Float32;
+      out.experts = {B(l->gate_images), B(l->up_images), B(l->down_images), l->expert_format, l->expert_down_format};
+    }
     if (l->shared_scalar_gate) out.sharedScalarGate = B(l->shared_scalar_gate);
     w.layers[layer] = std::move(out);
   });

@@ -27,7 +27,8 @@ HybridVerify::HybridVerify(hip::Backend &backend, HybridDimensions d, uint32_t m
       d.gdnPackedWidth % GGUF_TILE_COLUMNS || d.experts % GGUF_TILE_COLUMNS)
     throw std::invalid_argument("the model's widths hold whole super-blocks and its projections whole column tiles");
   if (!d.gdnShape().valid()) throw std::invalid_argument("invalid GDN shape");
-  if (!d.moeShape().valid()) throw std::invalid_argument("invalid MoE shape");
+  if (d.dense() ? (!d.denseFfn || d.denseFfn % GGUF_BLOCK) : !d.moeShape().valid())
+    throw std::invalid_argument(d.dense() ? "a dense FFN holds whole super-blocks" : "invalid MoE shape");
   maxRows_ = maxLanes * ATTENTION_MAXIMUM_ROWS;
   weights_.layers.resize(d.layers);
   const ops::kv::Layout layout{d.kvHeads, d.headDimension};
@@ -74,8 +75,14 @@ HybridVerify::HybridVerify(hip::Backend &backend, HybridDimensions d, uint32_t m
   ops::LinearScratchSize size;
   for (ops::LinearMatrix m : {ops::LinearMatrix{d.qkvWidth(), d.hidden}, ops::LinearMatrix{d.hidden, d.attentionWidth()},
                               ops::LinearMatrix{d.gdnPackedWidth, d.hidden}, ops::LinearMatrix{d.hidden, d.gdnWidth()},
-                              ops::LinearMatrix{d.experts, d.hidden}, ops::LinearMatrix{d.vocabulary, d.hidden}})
+                              d.dense() ? ops::LinearMatrix{d.denseFfn, d.hidden} : ops::LinearMatrix{d.experts, d.hidden},
+                              d.dense() ? ops::LinearMatrix{d.hidden, d.denseFfn} : ops::LinearMatrix{d.experts, d.hidden},
+                              ops::LinearMatrix{d.vocabulary, d.hidden}})
     size.include(linear_.scratchSize(m, pieceRows));
+  if (d.dense()) {
+    intermediate_ = device(R * d.denseFfn * 2, "SwiGLU rows");
+    ffnTable_ = device(gguf_tables_bytes(d.denseFfn, gguf_row_tiles(pieceRows)), "SwiGLU table");
+  }
   scratch_.input = device(size.input, "linear table");
   scratch_.partials = device(size.partials, "linear partials");
   scratch_.counters = device(std::max<uint64_t>(size.counters, 4), "linear counters");
@@ -85,7 +92,7 @@ HybridVerify::HybridVerify(hip::Backend &backend, HybridDimensions d, uint32_t m
   attentionWorkspace_.querySums = device(fused * 4, "query sums");
   attentionWorkspace_.partials = device(fused * ATTENTION_MAXIMUM_SPLITS * d.headDimension * 2, "attention partials");
   attentionWorkspace_.partialSums = device(fused * ATTENTION_MAXIMUM_SPLITS * 8, "attention partial sums");
-  const ops::MoeWorkspaceSize moe = ops::MoE::workspace(d.moeShape(), maxRows_);
+  const ops::MoeWorkspaceSize moe = d.dense() ? ops::MoeWorkspaceSize{} : ops::MoE::workspace(d.moeShape(), maxRows_);
   moeWorkspace_ = {device(moe.selected, "moe selected"),    device(moe.weights, "moe weights"),     device(moe.routeSlot, "moe route slots"),
                    device(moe.slotRow, "moe slot rows"),    device(moe.tileExpert, "moe tile experts"), device(moe.tileRows, "moe tile rows"),
                    device(moe.tileTotal, "moe tile count"), device(moe.tables, "moe tables"),       device(moe.nextTables, "moe SwiGLU tables"),
@@ -115,9 +122,14 @@ uint64_t HybridVerify::stepBytes(const std::vector<HybridLane> &lanes) const {
   const ops::MoeShape moe = dims_.moeShape();
   uint64_t bytes = weights_.head.weightBytes();
   for (const HybridLayer &l : weights_.layers) {
-    bytes += l.mixerInput.weightBytes() + l.mixerOutput.weightBytes() + l.router.weightBytes();
+    bytes += l.mixerInput.weightBytes() + l.mixerOutput.weightBytes();
+    if (dims_.dense()) {
+      bytes += l.ffnGate.weightBytes() + l.ffnUp.weightBytes() + l.ffnDown.weightBytes();
+      continue;
+    }
+    bytes += l.router.weightBytes();
     bytes += uint64_t{moe.allExperts()} * (2 * gguf_image_bytes(l.experts.format, moe.ffn, moe.hidden) +
-                                      gguf_image_bytes(l.experts.downFormat, moe.hidden, moe.ffn));
+                                           gguf_image_bytes(l.experts.downFormat, moe.hidden, moe.ffn));
   }
   uint32_t rows = 0;
   for (const HybridLane &lane : lanes) {
@@ -157,9 +169,12 @@ void HybridVerify::encodeLayer(hip::CommandGraph &graph, uint32_t layer, const s
   const uint64_t hiddenBytes = uint64_t{dims_.hidden} * 2;
   const uint32_t inputWidth = w.mixerInput.outputSize, mixedWidth = w.mixerOutput.inputSize;
   if (inputWidth != (attends ? dims_.qkvWidth() : dims_.gdnPackedWidth) || mixedWidth != (attends ? dims_.attentionWidth() : dims_.gdnWidth()) ||
-      w.mixerInput.inputSize != dims_.hidden || w.mixerOutput.outputSize != dims_.hidden || w.router.outputSize != dims_.experts ||
-      w.router.inputSize != dims_.hidden)
+      w.mixerInput.inputSize != dims_.hidden || w.mixerOutput.outputSize != dims_.hidden)
     throw std::invalid_argument("the layer's projections do not fit the model");
+  if (dims_.dense() ? (w.ffnGate.outputSize != dims_.denseFfn || w.ffnUp.outputSize != dims_.denseFfn || w.ffnDown.inputSize != dims_.denseFfn ||
+                       w.ffnGate.inputSize != dims_.hidden || w.ffnUp.inputSize != dims_.hidden || w.ffnDown.outputSize != dims_.hidden)
+                    : (w.router.outputSize != dims_.experts || w.router.inputSize != dims_.hidden))
+    throw std::invalid_argument("the layer's FFN does not fit the model");
 
   // Mixer: hidden[1] = hidden[0] + out(mixer(in(norm(hidden[0])))). With one piece of rows the mixer's last kernel
   // writes its output rows' activation table beside them.
@@ -207,6 +222,22 @@ void HybridVerify::encodeLayer(hip::CommandGraph &graph, uint32_t layer, const s
     linear_.add(graph, out, w.mixerOutput, linear_.plan(w.mixerOutput, count, ops::LinearEpilogue::Residual));
   });
 
+  if (dims_.dense()) {
+    // FFN: hidden[0] = hidden[1] + down(silu(gate n) * up n), n = norm(hidden[1]).
+    forRowPieces(rows, [&](uint32_t first, uint32_t count) {
+      const hip::Buffer normalized = rowsOf(normalized_, first, count, hiddenBytes);
+      const ops::PreparedInput prepared = ops::Normalization::addRmsTable(graph, rowsOf(next, first, count, hiddenBytes), w.postNorm, normalized,
+                                                                          scratch_, dims_.hidden, count);
+      ops::FfnBuffers ffn{normalized, rowsOf(intermediate_, first, count, uint64_t{dims_.denseFfn} * 2), scratch_, ffnTable_};
+      if (feedsNext) {
+        ffn.followingNorm = layer + 1 < dims_.layers ? weights_.layers[layer + 1].inputNorm : weights_.finalNorm;
+        ffn.followingTable = scratch_.input;
+      }
+      linear_.addSwiGlu(graph, {&w.ffnGate, &w.ffnUp, &w.ffnDown}, ffn, rowsOf(next, first, count, hiddenBytes),
+                        rowsOf(residual, first, count, hiddenBytes), count, prepared);
+    });
+    return;
+  }
   // FFN: hidden[0] = hidden[1] + sum over a row's experts of weight * expert(norm(hidden[1])).
   forRowPieces(rows, [&](uint32_t first, uint32_t count) {
     const hip::Buffer normalized = rowsOf(normalized_, first, count, hiddenBytes);
@@ -264,7 +295,9 @@ void HybridVerify::encode(hip::CommandGraph &graph, const std::vector<HybridLane
     ops::RoPE::addTreeTables(graph, inverseFrequency_, depths_, ropeCos_, ropeSin_, dims_.rotaryPairs, rope);
   encodeEmbedding(graph, rows);
   // One piece of rows: a layer's combine can write the table the next layer's (or the head's) first projection reads.
-  const bool feeds = rows <= kProjectionRows && dims_.hidden % GGUF_BLOCK == 0;
+  bool feeds = rows <= kProjectionRows && dims_.hidden % GGUF_BLOCK == 0;
+  if (dims_.dense())
+    for (const HybridLayer &l : weights_.layers) feeds = feeds && linear_.normsRows(l.ffnDown, rows);
   for (uint32_t layer = 0; layer < dims_.layers; ++layer) encodeLayer(graph, layer, lanes, feeds && layer > 0, feeds);
   encodeHead(graph, rows, feeds);
   ops::Sampling::addVerify(graph, sampling_, dims_.vocabulary, dims_.vocabulary, laneRows, policies);

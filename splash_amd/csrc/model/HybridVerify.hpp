@@ -36,6 +36,10 @@ struct HybridDimensions final {
   uint32_t gdnKeyHeads = 0, gdnValueHeads = 0;
   uint32_t gdnPackedWidth = 0;  // the GDN input projection's width (whole column tiles)
   uint32_t experts = 0, topK = 0, expertFfn = 0;
+  // experts == 0: every layer's FFN is a dense SwiGLU of this width instead of a mixture of experts (the reference's
+  // dense Qwen3.5 targets: the same mixers over QwenTarget::addDenseFfn, QwenTarget.cpp:351-370).
+  uint32_t denseFfn = 0;
+  [[nodiscard]] bool dense() const noexcept { return experts == 0; }
   // The shared expert: slices of the routed experts' width every row visits, gated by the layer's scalar gate or not.
   uint32_t sharedSlices = 0;
   bool sharedGate = false;
@@ -68,6 +72,7 @@ struct HybridLayer final {
   hip::Buffer inputNorm, postNorm;                                  // bf16 [hidden]
   hip::Buffer queryNorm, keyNorm;                                   // attention layers: bf16 [head dimension]
   hip::Buffer convolutionWeights, decay, timeBias, mixerNorm;       // GDN layers (mixerNorm bf16 [128])
+  ops::Projection ffnGate, ffnUp, ffnDown;                          // a dense model's SwiGLU
   ops::Projection router;                                           // hidden -> experts, fp32 scores
   ops::MoeExperts experts;                                          // the shared slices' images after the routed experts'
   hip::Buffer sharedScalarGate;                                     // fp32 [hidden], of a gated shared expert
@@ -151,6 +156,7 @@ private:
   hip::Buffer kvAll_, states_, tape_;
   hip::Buffer hidden_[2], normalized_, packed_, mixed_, scores_, logits_, draft_;
   hip::Buffer mixedTable_;  // the activation table of the mixer's output rows, written by the mixer's last kernel
+  hip::Buffer intermediate_, ffnTable_;  // a dense model's SwiGLU rows and their activation table
   hip::Buffer inverseFrequency_, ropeCos_, ropeSin_;
   hip::Buffer inputTokens_, treeRows_, depths_, uniforms_, tokens_, retained_, acceptedCount_, retainedRows_;
   hip::Buffer pageTable_;

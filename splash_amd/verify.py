@@ -118,14 +118,15 @@ class HybridVerify:
 
     def __init__(self, backend, hidden, vocabulary, layers, q_heads, kv_heads, head_dim, gdn_key_heads, gdn_value_heads, experts, top_k,
                  expert_ffn, attention_interval=4, rotary_pairs=None, normalize_heads=True, rope_theta=1e6, gdn_packed_width=None,
-                 max_lanes=1, physical_pages=2, page_table_entries=None, gated_attention=False, shared_slices=0, shared_gate=False):
+                 max_lanes=1, physical_pages=2, page_table_entries=None, gated_attention=False, shared_slices=0, shared_gate=False, dense_ffn=0):
+        """experts 0 and dense_ffn: every layer's FFN is a dense SwiGLU of that width instead of a mixture of experts."""
         self.backend = backend
         pairs = head_dim // 2 if rotary_pairs is None else rotary_pairs
         conv = (2 * gdn_key_heads + gdn_value_heads) * 128
         packed = gdn_packed_width or (conv + gdn_value_heads * 128 + 2 * gdn_value_heads + 15) // 16 * 16
         self.dims = nat.HybridDimensions(hidden, vocabulary, layers, attention_interval, q_heads, kv_heads, head_dim, pairs,
                                          int(normalize_heads), int(gated_attention), rope_theta, gdn_key_heads, gdn_value_heads, packed, experts, top_k, expert_ffn,
-                                         shared_slices, int(shared_gate))
+                                         shared_slices, int(shared_gate), dense_ffn)
         h = ctypes.c_void_p()
         entries = page_table_entries if page_table_entries is not None else physical_pages
         check(lib.spo_hybrid_verify_create(backend.handle, ctypes.byref(self.dims), max_lanes, physical_pages, entries, ctypes.byref(h)))
@@ -162,17 +163,18 @@ class HybridVerify:
         check(lib.spo_hybrid_verify_buffer(self.handle, which, index, ctypes.byref(out)))
         return Buffer(out.value)
 
-    def set_layer(self, layer, mixer_input, mixer_output, input_norm, post_norm, router, gate_images, up_images, down_images,
+    def set_layer(self, layer, mixer_input, mixer_output, input_norm, post_norm, router=None, gate_images=None, up_images=None, down_images=None,
                   query_norm=None, key_norm=None, convolution_weights=None, decay_weights=None, time_bias=None, mixer_norm=None,
-                  expert_format=ops.FMT_Q4K, expert_down_format=ops.FMT_Q4K, shared_scalar_gate=None):
+                  expert_format=ops.FMT_Q4K, expert_down_format=ops.FMT_Q4K, shared_scalar_gate=None, ffn=None):
+        """ffn: (gate, up, down) projections of a dense model's layer, which has no router and no expert images."""
         handle = lambda b: b.handle if b is not None else None
         w = nat.HybridLayer(mixer_input.handle, mixer_output.handle, handle(input_norm), handle(post_norm), handle(query_norm),
                             handle(key_norm), handle(convolution_weights), handle(decay_weights), handle(time_bias), handle(mixer_norm),
-                            router.handle, handle(gate_images), handle(up_images), handle(down_images), expert_format, expert_down_format,
-                            handle(shared_scalar_gate))
+                            handle(router), handle(gate_images), handle(up_images), handle(down_images), expert_format, expert_down_format,
+                            handle(shared_scalar_gate), *([p.handle for p in ffn] if ffn else [None, None, None]))
         check(lib.spo_hybrid_verify_set_layer(self.handle, layer, ctypes.byref(w)))
         self._keep.extend([mixer_input, mixer_output, input_norm, post_norm, router, gate_images, up_images, down_images, query_norm,
-                           key_norm, convolution_weights, decay_weights, time_bias, mixer_norm, shared_scalar_gate])
+                           key_norm, convolution_weights, decay_weights, time_bias, mixer_norm, shared_scalar_gate, ffn])
 
     def set_head(self, embedding_format, embedding_rows, final_norm, head):
         check(lib.spo_hybrid_verify_set_head(self.handle, embedding_format, embedding_rows.handle, final_norm.handle, head.handle))

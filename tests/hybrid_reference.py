@@ -9,13 +9,14 @@ from tests import oracle as orc
 
 class HybridModel:
     def __init__(self, seed, hidden, vocabulary, layers, q_heads, kv_heads, head_dim, gdn_key_heads, gdn_value_heads, experts, top_k,
-                 expert_ffn, attention_interval=4, rope_theta=1e6, gated_attention=False, shared_slices=0, shared_gate=False):
+                 expert_ffn, attention_interval=4, rope_theta=1e6, gated_attention=False, shared_slices=0, shared_gate=False, dense_ffn=0):
         self.dims = dict(hidden=hidden, vocabulary=vocabulary, layers=layers, q_heads=q_heads, kv_heads=kv_heads, head_dim=head_dim,
                          gdn_key_heads=gdn_key_heads, gdn_value_heads=gdn_value_heads, experts=experts, top_k=top_k, expert_ffn=expert_ffn,
                          attention_interval=attention_interval)
         self.rope_theta = rope_theta
         self.gated = gated_attention       # a query head's rows of the projection: its queries, then its gate
         self.shared_slices, self.shared_gate = shared_slices, shared_gate   # the shared expert, after the routed experts
+        self.dense_ffn = dense_ffn         # with experts 0: a dense SwiGLU of this width in every layer
         rng = np.random.default_rng(seed)
         self.rng = rng
         D = head_dim
@@ -30,10 +31,14 @@ class HybridModel:
             return orc.f32_to_bf16((1 + 0.1 * rng.standard_normal(n)).astype(np.float32))
         self.layers = []
         for l in range(layers):
-            w = dict(input_norm=norm(hidden), post_norm=norm(hidden), router=quant(experts, hidden, orc.FMT_Q6K, 0.05),
-                     gate=[quant(expert_ffn, hidden) for _ in range(experts + shared_slices)],
-                     up=[quant(expert_ffn, hidden) for _ in range(experts + shared_slices)],
-                     down=[quant(hidden, expert_ffn) for _ in range(experts + shared_slices)])
+            if experts:
+                w = dict(input_norm=norm(hidden), post_norm=norm(hidden), router=quant(experts, hidden, orc.FMT_Q6K, 0.05),
+                         gate=[quant(expert_ffn, hidden) for _ in range(experts + shared_slices)],
+                         up=[quant(expert_ffn, hidden) for _ in range(experts + shared_slices)],
+                         down=[quant(hidden, expert_ffn) for _ in range(experts + shared_slices)])
+            else:
+                w = dict(input_norm=norm(hidden), post_norm=norm(hidden), ffn_gate=quant(dense_ffn, hidden), ffn_up=quant(dense_ffn, hidden),
+                         ffn_down=quant(hidden, dense_ffn, orc.FMT_Q6K))
             if shared_gate:
                 w["shared_scalar_gate"] = (rng.standard_normal(hidden) * 0.05).astype(np.float32)
             if self.attends(l):
@@ -62,6 +67,7 @@ class HybridModel:
                                   d["gdn_key_heads"], d["gdn_value_heads"], d["experts"], d["top_k"], d["expert_ffn"],
                                   attention_interval=d["attention_interval"], rope_theta=self.rope_theta, max_lanes=max_lanes,
                                   gated_attention=self.gated, shared_slices=self.shared_slices, shared_gate=self.shared_gate,
+                                  dense_ffn=self.dense_ffn,
                                   physical_pages=self.physical_pages, page_table_entries=max_lanes * pages_per_lane)
         assert gpu.dims.gdn_packed_width == self.packed_width
         self.table = np.random.default_rng(99).permutation(self.physical_pages)[:max_lanes * pages_per_lane].astype(np.uint64)
@@ -70,9 +76,13 @@ class HybridModel:
         P = lambda segs, k, f32=False: ops.Projection.from_native(backend, segs, k, float32=f32)
         images = lambda fmt, natives, n, k: backend.from_array(np.concatenate([ops.pack_gguf_image(fmt, x, n, k) for x in natives]))
         for i, w in enumerate(self.layers):
-            common = dict(input_norm=backend.from_array(w["input_norm"]), post_norm=backend.from_array(w["post_norm"]),
-                          router=P([(orc.FMT_Q6K, d["experts"], w["router"])], H, True), gate_images=images(orc.FMT_Q4K, w["gate"], F, H),
-                          up_images=images(orc.FMT_Q4K, w["up"], F, H), down_images=images(orc.FMT_Q4K, w["down"], H, F))
+            common = dict(input_norm=backend.from_array(w["input_norm"]), post_norm=backend.from_array(w["post_norm"]))
+            if d["experts"]:
+                common.update(router=P([(orc.FMT_Q6K, d["experts"], w["router"])], H, True), gate_images=images(orc.FMT_Q4K, w["gate"], F, H),
+                              up_images=images(orc.FMT_Q4K, w["up"], F, H), down_images=images(orc.FMT_Q4K, w["down"], H, F))
+            else:
+                common.update(ffn=(P([(orc.FMT_Q4K, self.dense_ffn, w["ffn_gate"])], H), P([(orc.FMT_Q4K, self.dense_ffn, w["ffn_up"])], H),
+                                   P([(orc.FMT_Q6K, H, w["ffn_down"])], self.dense_ffn)))
             if self.shared_gate:
                 common["shared_scalar_gate"] = backend.from_array(w["shared_scalar_gate"])
             if self.attends(i):
@@ -206,6 +216,10 @@ class HybridModel:
         """(router scores, output rows) of the layer's mixture of experts."""
         w, d = self.layers[li], self.dims
         n = orc.rms_norm(hidden1, w["post_norm"])
+        if not d["experts"]:   # a dense SwiGLU: no router
+            mid = orc.swiglu(self._project(orc.FMT_Q4K, w["ffn_gate"], n, self.dense_ffn), self._project(orc.FMT_Q4K, w["ffn_up"], n, self.dense_ffn))
+            down = self._project(orc.FMT_Q6K, w["ffn_down"], mid, d["hidden"])
+            return None, orc.f32_to_bf16((down + orc.bf16_to_f32(hidden1)).astype(np.float32))
         scores = self._project(orc.FMT_Q6K, w["router"], n, d["experts"]).astype(np.float32)
         _, _, _, out = orc.moe_layer(n, hidden1, scores, d["top_k"], w["gate"], w["up"], w["down"], d["expert_ffn"],
                                      shared=self.shared_slices, shared_gate=w.get("shared_scalar_gate"))

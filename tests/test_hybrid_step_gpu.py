@@ -56,7 +56,7 @@ def check_step(backend, model, gpu, lanes, tokens):
         assert ok, ("mixer", layer, detail)
         # the FFN from the GPU's own mixer output
         scores, want = model.oracle_ffn(hidden_of(1), layer)
-        sure = sure_routes(scores, d["top_k"])
+        sure = sure_routes(scores, d["top_k"]) if scores is not None else np.ones(rows, dtype=bool)   # a dense FFN routes nothing
         assert sure.mean() >= 0.9
         ok, detail = close_bf16(hidden_of()[sure], want[sure])
         assert ok, ("ffn", layer, detail)
@@ -148,6 +148,24 @@ def test_config5_with_a_shared_expert(backend, gate):
     model.seed_states(rng, lanes=2)
     lanes = [verify.HybridLane(16, 40, table_first=0), verify.HybridLane(9, 100, table_first=1)]
     check_step(backend, model, gpu, lanes, rng.integers(0, SHAPE["vocabulary"], 25).astype(np.uint32))
+
+
+def test_dense_ffn_under_the_hybrid_mixers(backend):
+    """The reference's dense Qwen3.5 targets run the same Gated DeltaNet and attention mixers over a dense SwiGLU
+    (QwenTarget.cpp:351-370) instead of a mixture of experts: experts 0 and a dense FFN width, layer by layer against
+    the oracle, two lanes, and a second step that folds what the first accepted."""
+    print("case hybrid dense FFN", flush=True)
+    shape = {**SHAPE, "experts": 0, "top_k": 0, "expert_ffn": 0}
+    model = HybridModel(seed=44, dense_ffn=768, **shape)
+    gpu = model.build_gpu(backend, max_lanes=2, pages_per_lane=1)
+    rng = np.random.default_rng(12)
+    model.seed_context(rng)
+    model.seed_states(rng, lanes=2)
+    lanes = [verify.HybridLane(16, 33, table_first=0), verify.HybridLane(7, 90, table_first=1)]
+    _, (selected, retained, accepted, masks) = check_step(backend, model, gpu, lanes, rng.integers(0, SHAPE["vocabulary"], 23).astype(np.uint32))
+    following = [verify.HybridLane(16, 33 + int(retained[0]), table_first=0, pending_path=int(masks[0]), parity=1),
+                 verify.HybridLane(7, 90 + int(retained[1]), table_first=1, pending_path=int(masks[1]), parity=1)]
+    check_step(backend, model, gpu, following, rng.integers(0, SHAPE["vocabulary"], 23).astype(np.uint32))
 
 
 def test_hybrid_rejects_bad_arguments(backend):
