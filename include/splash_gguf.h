@@ -6,6 +6,7 @@
  * sp_last_error are those of splash_hip.h; a malformed file is SP_BACKEND_ERROR with the parser's message. */
 #pragma once
 #include "splash_hip.h"
+#include "splash_ops.h"
 
 #ifdef __cplusplus
 extern "C" {
@@ -49,6 +50,18 @@ sp_status spg_load_image(sp_backend *backend, const spg_file *file, uint64_t ind
                          sp_buffer **image, uint32_t *format, uint32_t *out_rows, uint32_t *input_size);
 /* An F32, F16 or BF16 tensor as bf16 in device memory (a norm's weights). The caller releases the buffer. */
 sp_status spg_load_bf16(sp_backend *backend, const spg_file *file, uint64_t index, sp_buffer **out, uint64_t *elements);
+
+/* A dense decoder from a file (the reference's GgufTargetLoader and planImages for its targets, GgufTarget.hpp:24-75,
+ * GgufImage.cpp:474-520, :696-713). spg_dense_dimensions reads the geometry from the metadata of the file's
+ * architecture (block_count, embedding_length, feed_forward_length, attention.head_count / head_count_kv / key_length,
+ * rope.freq_base; the vocabulary is token_embd.weight's rows; per-head q/k norms when blk.0.attn_q_norm.weight exists);
+ * spo_dense_verify_load_gguf then loads every weight of a driver created with those dimensions: blk.N.attn_norm,
+ * attn_q | attn_k | attn_v as one projection of three segments, each of its tensor's format, attn_q_norm, attn_k_norm,
+ * attn_output, ffn_norm, ffn_gate, ffn_up, ffn_down, output_norm, token_embd (native rows, for the token gather) and
+ * output.weight, or the token table again when the file ties them. A malformed file, a missing tensor, a type the
+ * path does not read or a tensor the loader would ignore (a bias) is SP_BACKEND_ERROR naming all of them. */
+sp_status spg_dense_dimensions(const spg_file *file, spo_dense_dimensions *out);
+sp_status spo_dense_verify_load_gguf(spo_dense_verify *verify, const spg_file *file);
 
 #ifdef __cplusplus
 }

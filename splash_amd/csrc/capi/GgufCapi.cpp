@@ -1,6 +1,7 @@
 // The C entry points of include/splash_gguf.h over model::GgufFile.
 #include "splash_gguf.h"
 #include "capi/Guard.hpp"
+#include "capi/Handles.hpp"
 #include "model/GgufFile.hpp"
 
 #include <algorithm>
@@ -12,6 +13,13 @@ using namespace splash;
 struct spg_file {
   std::unique_ptr<model::GgufFile> file;
 };
+
+namespace splash::capi {
+const model::GgufFile &ggufOf(const spg_file *file) {
+  require(file, "file");
+  return *file->file;
+}
+} // namespace splash::capi
 
 namespace {
 size_t copyOut(const std::string &text, char *out, size_t capacity) {

@@ -9,7 +9,14 @@ struct spo_graph { splash::hip::CommandGraph graph; };
 struct spo_projection { splash::ops::Projection projection; };
 struct spo_linear { splash::ops::Linear linear; };
 
+struct spg_file;
+namespace splash::model {
+class GgufFile;
+}
+
 namespace splash::capi {
+// The parsed file behind a handle of include/splash_gguf.h.
+const model::GgufFile &ggufOf(const spg_file *file);
 inline hip::CommandGraph &graphOf(spo_graph *graph) { return graph->graph; }
 inline const ops::Projection &projectionOf(const spo_projection *projection) { return projection->projection; }
 } // namespace splash::capi

@@ -3,6 +3,8 @@
 #include "capi/Guard.hpp"
 #include "capi/Handles.hpp"
 #include "model/DenseVerify.hpp"
+#include "model/GgufTarget.hpp"
+#include "splash_gguf.h"
 #include "ops/Glue.hpp"
 #include "ops/Sampling.hpp"
 
@@ -170,6 +172,20 @@ sp_status spo_dense_verify_create(sp_backend *backend, const spo_dense_dimension
   });
 }
 void spo_dense_verify_destroy(spo_dense_verify *verify) { delete verify; }
+
+sp_status spg_dense_dimensions(const spg_file *file, spo_dense_dimensions *out) {
+  return capi::guard([&] {
+    capi::require(out, "result");
+    const model::DenseDimensions d = model::ggufDenseDimensions(capi::ggufOf(file));
+    *out = {d.hidden, d.qHeads, d.kvHeads, d.headDimension, d.ffn, d.vocabulary, d.layers, d.rotaryPairs, d.normalizeHeads ? 1u : 0u, d.ropeTheta};
+  });
+}
+sp_status spo_dense_verify_load_gguf(spo_dense_verify *verify, const spg_file *file) {
+  return capi::guard([&] {
+    capi::require(verify, "verify");
+    model::loadGgufDenseWeights(*verify->backend, capi::ggufOf(file), *verify->verify);
+  });
+}
 
 sp_status spo_dense_verify_set_layer(spo_dense_verify *verify, uint32_t layer, const spo_projection *qkv, const spo_projection *output,
                                      const spo_projection *gate, const spo_projection *up, const spo_projection *down,

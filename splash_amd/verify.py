@@ -38,6 +38,18 @@ class DenseVerify:
         self.physical_pages = physical_pages
         self._keep = []
 
+    @classmethod
+    def from_gguf(cls, backend, gguf_file, max_lanes=1, physical_pages=2, page_table_entries=None):
+        """A driver of the geometry the file's metadata names, with every weight loaded from the file
+        (spg_dense_dimensions, spo_dense_verify_load_gguf)."""
+        d = nat.DenseDimensions()
+        check(lib.spg_dense_dimensions(gguf_file.handle, ctypes.byref(d)))
+        self = cls(backend, d.hidden, d.q_heads, d.kv_heads, d.head_dim, d.ffn, d.vocabulary, d.layers, d.rotary_pairs,
+                   bool(d.normalize_heads), d.rope_theta, max_lanes, physical_pages, page_table_entries)
+        check(lib.spo_dense_verify_load_gguf(self.handle, gguf_file.handle))
+        self._keep.append(gguf_file)
+        return self
+
     def __del__(self):
         try:
             lib.spo_dense_verify_destroy(self.handle)

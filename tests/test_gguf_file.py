@@ -115,3 +115,99 @@ def test_projections_and_norms_load_from_a_file(backend, tmp_path):
         assert np.array_equal(f.load_bf16(backend, f.find(name)).download(np.uint16)[:512], want)
     with pytest.raises(ValueError):
         f.load_bf16(backend, f.find("output.weight"))
+
+
+def dense_model_file(path, model, value_format, tied, extra=(), skip=()):
+    """A dense decoder's GGUF as llama.cpp names its tensors: blk.N.attn_q / attn_k / attn_v (the values requantized to
+    `value_format`, as a Q4_K_M file keeps them) ..., norms as F32, the token table, and the head unless tied."""
+    d = model.dims
+    H, D, F, V = d["hidden"], d["head_dim"], d["ffn"], d["vocabulary"]
+    kinds = {orc.FMT_Q4K: gw.GGML_Q4_K, orc.FMT_Q6K: gw.GGML_Q6_K, orc.FMT_Q5K: gw.GGML_Q5_K, orc.FMT_Q80: gw.GGML_Q8_0}
+    f32 = lambda bits: orc.bf16_to_f32(bits).astype(np.float32)
+    tensors = [("token_embd.weight", gw.GGML_Q4_K, [H, V], model.embedding)]
+    for i, w in enumerate(model.layers):
+        p = f"blk.{i}."
+        tensors += [(p + "attn_norm.weight", gw.GGML_F32, [H], f32(w["input_norm"])),
+                    (p + "attn_q.weight", gw.GGML_Q4_K, [H, d["q_heads"] * D], w["q"]),
+                    (p + "attn_k.weight", gw.GGML_Q4_K, [H, d["kv_heads"] * D], w["k"]),
+                    (p + "attn_v.weight", kinds[value_format], [H, d["kv_heads"] * D], w["v"]),
+                    (p + "attn_q_norm.weight", gw.GGML_F32, [D], f32(w["q_norm"])),
+                    (p + "attn_k_norm.weight", gw.GGML_BF16, [D], w["k_norm"]),
+                    (p + "attn_output.weight", gw.GGML_Q4_K, [d["q_heads"] * D, H], w["o"]),
+                    (p + "ffn_norm.weight", gw.GGML_F32, [H], f32(w["post_norm"])),
+                    (p + "ffn_gate.weight", gw.GGML_Q4_K, [H, F], w["gate"]), (p + "ffn_up.weight", gw.GGML_Q4_K, [H, F], w["up"]),
+                    (p + "ffn_down.weight", kinds[model.down_format], [F, H], w["down"])]
+    tensors.append(("output_norm.weight", gw.GGML_F32, [H], f32(model.final_norm)))
+    if not tied:
+        tensors.append(("output.weight", gw.GGML_Q6_K, [H, V], model.head))
+    tensors = [t for t in tensors if t[0] not in skip] + list(extra)
+    metadata = [("general.architecture", gw.STRING, "qwen3"), ("qwen3.block_count", gw.U32, d["layers"]),
+                ("qwen3.embedding_length", gw.U32, H), ("qwen3.feed_forward_length", gw.U32, F),
+                ("qwen3.attention.head_count", gw.U32, d["q_heads"]), ("qwen3.attention.head_count_kv", gw.U32, d["kv_heads"]),
+                ("qwen3.attention.key_length", gw.U32, D), ("qwen3.attention.value_length", gw.U32, D),
+                ("qwen3.attention.layer_norm_rms_epsilon", gw.F32, 1e-6), ("qwen3.rope.freq_base", gw.F32, model.rope_theta)]
+    gw.write_gguf(path, metadata, tensors)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("value_format,tied", [(orc.FMT_Q6K, False), (orc.FMT_Q4K, True)])
+def test_a_dense_decoder_loads_from_a_file(tmp_path, value_format, tied):
+    """spg_dense_dimensions and spo_dense_verify_load_gguf: the driver built from a file gives, bit for bit, the logits
+    and the acceptance of the driver built by hand from the same tensors: q | k | v fused with the values in another
+    format than the queries and keys, a tied head, and the refusal of tensors the loader would ignore."""
+    from splash_amd import verify
+    from tests.dense_reference import DenseModel
+    backend = splash_amd.Backend(0)
+    model = DenseModel(seed=5, hidden=512, q_heads=16, kv_heads=8, head_dim=64, ffn=768, vocabulary=2048, layers=2, down_format=orc.FMT_Q6K)
+    if value_format != orc.FMT_Q4K:   # the values in the format a Q4_K_M file keeps them in
+        for w in model.layers:
+            w["v"] = orc.quantize_rows(value_format, orc.dequant_rows(orc.FMT_Q4K, w["v"], 512, 512))
+    if tied:
+        model.head = model.embedding
+    path = tmp_path / "dense.gguf"
+    dense_model_file(path, model, value_format, tied)
+    rows, context = 16, 200
+    rng = np.random.default_rng(1)
+    tokens = rng.integers(0, 2048, rows).astype(np.uint32)
+    pages = (context + 16 + ops.PAGE_TOKENS - 1) // ops.PAGE_TOKENS
+    loaded = verify.DenseVerify.from_gguf(backend, gguf.GgufFile(path), max_lanes=1, physical_pages=pages + 1, page_table_entries=pages)
+    d = loaded.dims
+    assert (d.hidden, d.q_heads, d.kv_heads, d.head_dim, d.ffn, d.vocabulary, d.layers, d.rotary_pairs, d.normalize_heads) == \
+        (512, 16, 8, 64, 768, 2048, 2, 32, 1) and d.rope_theta == model.rope_theta
+
+    def hand_built():
+        from splash_amd import ops as o
+        P = lambda segs, k, f32=False: o.Projection.from_native(backend, segs, k, float32=f32)
+        gpu = verify.DenseVerify(backend, 512, 16, 8, 64, 768, 2048, 2, rope_theta=model.rope_theta, max_lanes=1, physical_pages=pages + 1,
+                                 page_table_entries=pages)
+        for i, w in enumerate(model.layers):
+            gpu.set_layer(i, P([(orc.FMT_Q4K, 1024, w["q"]), (orc.FMT_Q4K, 512, w["k"]), (value_format, 512, w["v"])], 512),
+                          P([(orc.FMT_Q4K, 512, w["o"])], 1024), P([(orc.FMT_Q4K, 768, w["gate"])], 512), P([(orc.FMT_Q4K, 768, w["up"])], 512),
+                          P([(orc.FMT_Q6K, 512, w["down"])], 768), backend.from_array(w["input_norm"]), backend.from_array(w["post_norm"]),
+                          backend.from_array(w["q_norm"]), backend.from_array(w["k_norm"]))
+        gpu.set_head(orc.FMT_Q4K, backend.from_array(model.embedding), backend.from_array(model.final_norm),
+                     P([(orc.FMT_Q4K if tied else orc.FMT_Q6K, 2048, model.head)], 512, True))
+        return gpu
+    outputs = []
+    for gpu in (loaded, hand_built()):
+        model.physical_pages = pages + 1
+        model.table = np.random.default_rng(99).permutation(pages + 1)[:pages].astype(np.uint64)
+        gpu.buffer(verify.PAGE_TABLE).upload(model.table)
+        model.seed_context(gpu, context, np.random.default_rng(3))
+        lane = verify.Lane(rows, context)
+        gpu.set_block([lane], tokens)
+        backend.run(gpu.encode([lane], commit=True))
+        outputs.append((gpu.buffer(verify.LOGITS).download(np.float32, rows * 2048), gpu.results([lane])))
+    assert outputs[0][0].tobytes() == outputs[1][0].tobytes()
+    for a, b in zip(outputs[0][1], outputs[1][1]):
+        assert np.array_equal(a, b)
+    assert np.isfinite(outputs[0][0]).all() and np.abs(outputs[0][0]).max() > 0
+    # a tensor the loader would ignore, a missing one and a wrong shape are refused, all named in one message
+    bad = tmp_path / "bad.gguf"
+    dense_model_file(bad, model, value_format, tied, extra=[("blk.0.attn_q.bias", gw.GGML_F32, [512], np.zeros(512, np.float32))])
+    with pytest.raises(splash_amd.SplashError, match="attn_q.bias"):
+        verify.DenseVerify.from_gguf(backend, gguf.GgufFile(bad), physical_pages=pages + 1)
+    dense_model_file(bad, model, value_format, tied, skip=("blk.1.ffn_up.weight", "output_norm.weight"))
+    with pytest.raises(splash_amd.SplashError, match="blk.1.ffn_up.weight is missing; output_norm.weight is missing"):
+        verify.DenseVerify.from_gguf(backend, gguf.GgufFile(bad), physical_pages=pages + 1)
+    backend.close()
