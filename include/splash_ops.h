@@ -223,6 +223,8 @@ typedef struct spo_moe_shape {
    * its routed ones, ids experts .. experts + shared_slices - 1, their images after the routed experts' in the same
    * buffers; shared_gate: each weighs sigmoid(row . scalar gate), else 1. */
   uint32_t shared_slices, shared_gate;
+  uint32_t sigmoid_router; /* MoeRouter::SigmoidNormalized (moe.metal:21, :104-110) instead of the softmax of the selected scores */
+  uint32_t reserved;
 } spo_moe_shape;
 typedef struct spo_moe_workspace { /* in the order of spo_moe_workspace_sizes */
   sp_buffer *selected, *weights, *route_slot, *slot_row, *tile_expert, *tile_rows, *tile_total, *tables, *next_tables,

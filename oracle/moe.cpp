@@ -31,6 +31,18 @@ void orc_moe_route(const float *scores, uint32_t rows, uint32_t experts, uint32_
   }
 }
 
+void orc_moe_route_sigmoid(const float *scores, uint32_t rows, uint32_t experts, uint32_t stride, uint32_t top_k, uint32_t *selected,
+                           float *weights) {
+  orc_moe_route(scores, rows, experts, stride, top_k, selected, weights);   // the selection is the router's; only the weights differ
+  const auto sigmoid = [](float x) { return 1.0f / (1.0f + std::exp2(-1.44269504089f * x)); };
+  for (uint32_t r = 0; r < rows; ++r) {
+    float denominator = 0.f;
+    for (uint32_t k = 0; k < top_k; ++k) denominator += sigmoid(scores[size_t(r) * stride + selected[size_t(r) * top_k + k]]);
+    for (uint32_t k = 0; k < top_k; ++k)
+      weights[size_t(r) * top_k + k] = sigmoid(scores[size_t(r) * stride + selected[size_t(r) * top_k + k]]) / (denominator + 1e-20f);
+  }
+}
+
 void orc_moe_shared_weights(const uint16_t *x, const float *gate, uint32_t rows, uint32_t hidden, float *weights) {
   for (uint32_t r = 0; r < rows; ++r) {
     float partial[64];

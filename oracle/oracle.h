@@ -205,6 +205,10 @@ int orc_gdn_reference(const struct OrcGdnShape *s, const uint16_t *packed, uint3
 // and their weights exp2((s_r - s_0) log2 e) / sum, the sum in rank order.
 void orc_moe_route(const float *scores, uint32_t rows, uint32_t experts, uint32_t stride, uint32_t top_k, uint32_t *selected,
                    float *weights);
+// The same selection under the sigmoid router (moe.metal:104-110): weight of rank r = sigmoid(s_r) / (sum over the k
+// selected of sigmoid(s) + 1e-20), the sum in rank order.
+void orc_moe_route_sigmoid(const float *scores, uint32_t rows, uint32_t experts, uint32_t stride, uint32_t top_k, uint32_t *selected,
+                           float *weights);
 // kernels/shared/moe.metal:42-65: a gated shared expert's weight of each row, sigmoid(x . gate) with e^-t as
 // exp2(-log2(e) t): 64 partial sums, partial l over dimensions l, l + 64, ... in order (a product and a sum, each
 // rounded), added pairwise at distances 32, 16, ... 1.

@@ -115,7 +115,8 @@ class StateCodecShape(ctypes.Structure):
 
 
 class MoeShape(ctypes.Structure):
-    _fields_ = [("hidden", c_u32), ("ffn", c_u32), ("experts", c_u32), ("top_k", c_u32), ("shared_slices", c_u32), ("shared_gate", c_u32)]
+    _fields_ = [("hidden", c_u32), ("ffn", c_u32), ("experts", c_u32), ("top_k", c_u32), ("shared_slices", c_u32), ("shared_gate", c_u32),
+                ("sigmoid_router", c_u32), ("reserved", c_u32)]
 
 
 MOE_WORKSPACE_FIELDS = ("selected", "weights", "route_slot", "slot_row", "tile_expert", "tile_rows", "tile_total", "tables", "next_tables",

@@ -37,7 +37,9 @@ struct MoeRouteParams {
   uint32_t shared;        // slices of the shared expert
   uint32_t shared_gated;
   uint32_t input_size;    // of the rows the scalar gate multiplies (bf16)
-  uint32_t reserved;
+  // 0: the softmax of the selected scores; 1: each one's sigmoid over the sum of theirs plus 1e-20, summed in rank
+  // order (the reference's MoeRouter::SigmoidNormalized, moe.metal:104-110).
+  uint32_t sigmoid_router;
 };
 // moe_group_routes: one workgroup of 1024 threads.
 struct MoeGroupParams {

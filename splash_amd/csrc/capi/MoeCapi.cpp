@@ -8,7 +8,7 @@ using namespace splash;
 
 namespace {
 hip::Buffer B(sp_buffer *b) { return hip::Buffer::share(b); }
-ops::MoeShape shapeOf(const spo_moe_shape &s) { return {s.hidden, s.ffn, s.experts, s.top_k, s.shared_slices, s.shared_gate != 0}; }
+ops::MoeShape shapeOf(const spo_moe_shape &s) { return {s.hidden, s.ffn, s.experts, s.top_k, s.shared_slices, s.shared_gate != 0, s.sigmoid_router != 0}; }
 ops::MoeWorkspace workspaceOf(const spo_moe_workspace &w) {
   return {B(w.selected), B(w.weights), B(w.route_slot), B(w.slot_row), B(w.tile_expert), B(w.tile_rows), B(w.tile_total), B(w.tables),
           B(w.next_tables), B(w.intermediate), B(w.expert_output)};

@@ -64,8 +64,14 @@ __global__ __launch_bounds__(64) void moe_route_select(const float *__restrict__
   __syncthreads();
   if (lane < p.top_k) {
     float denominator = 0.f;
-    for (uint32_t other = 0; other < p.top_k; ++other) denominator += __builtin_amdgcn_exp2f((ordered[other] - ordered[0]) * 1.44269504089f);
-    weights[size_t(row) * perRow + lane] = __builtin_amdgcn_exp2f((ordered[lane] - ordered[0]) * 1.44269504089f) / denominator;
+    if (p.sigmoid_router) {
+      const auto sigmoid = [](float x) { return 1.0f / (1.0f + __builtin_amdgcn_exp2f(-1.44269504089f * x)); };
+      for (uint32_t other = 0; other < p.top_k; ++other) denominator += sigmoid(ordered[other]);
+      weights[size_t(row) * perRow + lane] = sigmoid(ordered[lane]) / (denominator + 1e-20f);
+    } else {
+      for (uint32_t other = 0; other < p.top_k; ++other) denominator += __builtin_amdgcn_exp2f((ordered[other] - ordered[0]) * 1.44269504089f);
+      weights[size_t(row) * perRow + lane] = __builtin_amdgcn_exp2f((ordered[lane] - ordered[0]) * 1.44269504089f) / denominator;
+    }
   }
 }
 SP_REGISTER_KERNEL("moe_route_select", &moe_route_select);

@@ -59,7 +59,7 @@ void MoE::addRouting(hip::CommandGraph &graph, const hip::Buffer &scores, uint32
   requireBytes(w.tileTotal, 4, "tile count");
   const uint32_t routes = rows * shape.routesPerRow();
   graph.add("moe_route_select", {scores, shape.sharedGate ? input : scores, shape.sharedGate ? sharedScalarGate : scores, w.selected, w.weights},
-            MoeRouteParams{rows, shape.experts, shape.topK, scoreStride, shape.sharedSlices, shape.sharedGate, shape.hidden, 0}, {rows, 1, 1},
+            MoeRouteParams{rows, shape.experts, shape.topK, scoreStride, shape.sharedSlices, shape.sharedGate, shape.hidden, shape.sigmoidRouter}, {rows, 1, 1},
             {64, 1, 1});
   // The grouping and the combine take the shared slices as further experts and routes of a row.
   graph.add("moe_group_routes", {w.selected, w.routeSlot, w.slotRow, w.tileExpert, w.tileRows, w.tileTotal},

@@ -16,6 +16,9 @@ struct MoeShape final {
   // same buffers, in the same formats.
   uint32_t sharedSlices = 0;
   bool sharedGate = false;
+  // The routed experts' weights: the softmax of the selected scores, or each one's sigmoid over the sum of theirs
+  // (the reference's MoeRouter, moe.metal:21, :96-110).
+  bool sigmoidRouter = false;
   [[nodiscard]] uint32_t routesPerRow() const noexcept { return topK + sharedSlices; }
   [[nodiscard]] uint32_t allExperts() const noexcept { return experts + sharedSlices; }
   [[nodiscard]] bool valid() const noexcept {

@@ -384,8 +384,8 @@ class GDN:
 class MoE:
     """ops::MoE: routing (addRouting) and the routed experts with their weighted sum (addRouted)."""
 
-    def __init__(self, backend, hidden, ffn, experts, top_k, rows, shared_slices=0, shared_gate=False):
-        self.shape = nat.MoeShape(hidden, ffn, experts, top_k, shared_slices, int(shared_gate))
+    def __init__(self, backend, hidden, ffn, experts, top_k, rows, shared_slices=0, shared_gate=False, sigmoid_router=False):
+        self.shape = nat.MoeShape(hidden, ffn, experts, top_k, shared_slices, int(shared_gate), int(sigmoid_router), 0)
         self.rows = rows
         sizes = (ctypes.c_uint64 * 11)()
         check(lib.spo_moe_workspace_sizes(ctypes.byref(self.shape), rows, sizes))

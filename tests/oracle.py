@@ -444,14 +444,15 @@ lib.orc_moe_combine.restype = None
 lib.orc_moe_combine.argtypes = [u16p, f32p, u16p, c_u32, c_u32, c_u32, u16p]
 
 
-def moe_route(scores, top_k, shared=0, x_bits=None, shared_gate=None):
+def moe_route(scores, top_k, shared=0, x_bits=None, shared_gate=None, sigmoid_router=False):
     """Each row's routes: its top_k routed experts, then `shared` slices of the shared expert (ids experts on), each
     weighing sigmoid(x . shared_gate) or, without a gate, 1."""
     scores = np.ascontiguousarray(scores, np.float32)
     rows, experts = scores.shape
     selected = np.zeros((rows, top_k), np.uint32)
     weights = np.zeros((rows, top_k), np.float32)
-    lib.orc_moe_route(_p(scores, f32p), rows, experts, experts, top_k, _p(selected, u32p), _p(weights, f32p))
+    route = lib.orc_moe_route_sigmoid if sigmoid_router else lib.orc_moe_route
+    route(_p(scores, f32p), rows, experts, experts, top_k, _p(selected, u32p), _p(weights, f32p))
     if shared:
         gate = np.ones(rows, np.float32)
         if shared_gate is not None:
@@ -472,12 +473,12 @@ def moe_combine(y_bits, weights, residual_bits):
 
 
 def moe_layer(x_bits, residual_bits, scores, top_k, gate_native, up_native, down_native, ffn, fmt=FMT_Q4K, down_fmt=FMT_Q4K,
-              shared=0, shared_gate=None):
+              shared=0, shared_gate=None, sigmoid_router=False):
     """The routed experts of a layer: x bf16 [rows][hidden] (normalized), natives per expert (the shared slices' after
     the routed experts'). Each expert's rows go through the oracle's projections together; a row's result does not
     depend on the rows beside it."""
     rows, hidden = x_bits.shape
-    selected, weights = moe_route(scores, top_k, shared, x_bits, shared_gate)
+    selected, weights = moe_route(scores, top_k, shared, x_bits, shared_gate, sigmoid_router)
     y = np.zeros((rows, top_k + shared, hidden), np.uint16)
     for e in np.unique(selected):
         r, k = np.nonzero(selected == e)

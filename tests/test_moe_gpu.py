@@ -9,7 +9,7 @@ from tests import oracle as orc
 pytestmark = pytest.mark.gpu
 
 
-def run_layer(backend, rng, hidden, ffn, experts, top_k, rows, down_fmt=ops.FMT_Q4K, following=None, shared=0, gated=False):
+def run_layer(backend, rng, hidden, ffn, experts, top_k, rows, down_fmt=ops.FMT_Q4K, following=None, shared=0, gated=False, sigmoid=False):
     """shared: slices of a shared expert, whose images follow the routed experts'; gated: they weigh sigmoid(x . gate)."""
     gate = [orc.make_native(ops.FMT_Q4K, ffn, hidden, 100 + e) for e in range(experts + shared)]
     up = [orc.make_native(ops.FMT_Q4K, ffn, hidden, 300 + e) for e in range(experts + shared)]
@@ -20,7 +20,7 @@ def run_layer(backend, rng, hidden, ffn, experts, top_k, rows, down_fmt=ops.FMT_
     res = orc.f32_to_bf16(rng.standard_normal((rows, hidden)).astype(np.float32))
     scores = rng.standard_normal((rows, experts)).astype(np.float32)
     scores[0, :] = 0.5                                 # a row of ties: experts 0..top_k-1 in id order
-    moe = ops.MoE(backend, hidden, ffn, experts, top_k, rows, shared_slices=shared, shared_gate=gated)
+    moe = ops.MoE(backend, hidden, ffn, experts, top_k, rows, shared_slices=shared, shared_gate=gated, sigmoid_router=sigmoid)
     out = backend.allocate_buffer(rows * hidden * 2)
     graph = splash_amd.CommandGraph()
     scalar_gate = (rng.standard_normal(hidden) * 0.05).astype(np.float32) if gated else None
@@ -31,7 +31,8 @@ def run_layer(backend, rng, hidden, ffn, experts, top_k, rows, down_fmt=ops.FMT_
     assert len(graph) == 6
     backend.run(graph)
     got = out.download(np.uint16).reshape(rows, hidden)
-    want = orc.moe_layer(x, res, scores, top_k, gate, up, down, ffn, down_fmt=down_fmt, shared=shared, shared_gate=scalar_gate)
+    want = orc.moe_layer(x, res, scores, top_k, gate, up, down, ffn, down_fmt=down_fmt, shared=shared, shared_gate=scalar_gate,
+                         sigmoid_router=sigmoid)
     return moe, got, want
 
 
@@ -95,6 +96,18 @@ def test_shared_expert_slices_ride_every_row(backend, config):
     check_layer(moe, got, want, rows, experts, top_k, shared)
     if not gated:
         assert np.all(want[1][:, top_k:] == 1.0)
+
+
+def test_sigmoid_router_weighs_by_normalized_sigmoids(backend):
+    """MoeRouter::SigmoidNormalized (moe.metal:21, :104-110): the same selection, each weight its score's sigmoid over the
+    sum of the selected ones'; with an ungated shared expert twice the routed width (two slices), as the reference's
+    Flint blocks have it."""
+    print("case moe sigmoid router", flush=True)
+    rng = np.random.default_rng(31)
+    moe, got, want = run_layer(backend, rng, 512, 256, 16, 4, 40, shared=2, sigmoid=True)
+    check_layer(moe, got, want, 40, 16, 4, 2)
+    weights = want[1][:, :4]
+    assert np.all(np.abs(weights.sum(axis=1) - 1) < 1e-5) and np.all(np.diff(weights, axis=1) <= 1e-7)
 
 
 def test_moe_layer_at_the_35b_shape(backend):
