@@ -109,3 +109,43 @@ def test_config1_accepts_a_self_consistent_draft(backend):
     selected, retained, accepted, mask = gpu.results([lane])
     assert accepted[0] == 4 and retained[0] == 5 and mask[0] == 0b11111
     assert np.array_equal(selected[:4], planted[1:5]) and selected[4] == tokens[5]
+
+
+def test_a_context_built_from_tokens_alone(backend):
+    """No seeded KV: from an empty context, three blocks of sixteen prompt tokens run through the step one after the
+    other (their rows' keys and values stay in the pages whatever the acceptance says; the caller advances the lane's
+    committed tokens itself), then a verify block over the 48-token context the GPU wrote. Against the oracle run the
+    same way, storing its own keys and values: logits within the bf16 tolerance of a chain of four steps (cosine >=
+    0.999, max-abs 5e-2), and the empty history (committed 0) is a case of its own for the attention's partition."""
+    print("case config 1 context from tokens", flush=True)
+    model = DenseModel(seed=13, hidden=1024, q_heads=16, kv_heads=8, head_dim=64, ffn=3072, vocabulary=32000, layers=2)
+    rng = np.random.default_rng(2)
+    gpu = model.build_gpu(backend, max_lanes=1, context_tokens=64)
+    pages = model.physical_pages
+    zero = lambda shape, dtype: np.zeros(shape, dtype=dtype)
+    model.context = [[zero((pages, 8, ops.PAGE_TOKENS, 64), np.int8), zero((pages, 8, ops.PAGE_TOKENS), np.float32),
+                      zero((pages, 8, ops.PAGE_TOKENS, 64), np.int8), zero((pages, 8, ops.PAGE_TOKENS), np.float32)] for _ in range(2)]
+    for layer in range(2):   # the pools start as whatever the allocation held: clear them as the oracle's context is
+        gpu.buffer(verify.KV_POOL, layer).fill(0)
+    prompt = rng.integers(0, 32000, 48).astype(np.uint32)
+    for block in range(3):
+        tokens = prompt[16 * block:16 * block + 16]
+        lane = verify.Lane(16, 16 * block)
+        gpu.set_block([lane], tokens)
+        backend.run(gpu.encode([lane], commit=False))
+        got = gpu.buffer(verify.LOGITS).download(np.float32, 16 * 32000).reshape(16, 32000)
+        want = model.oracle_step(tokens, 16 * block)["logits"]
+        cos = (got.astype(np.float64) * want).sum() / np.sqrt((got.astype(np.float64) ** 2).sum() * (want ** 2).sum())
+        assert cos >= 0.999 and np.abs(got - want).max() <= 5e-2, (block, cos, np.abs(got - want).max())
+    draft = rng.integers(0, 32000, 16).astype(np.uint32)
+    lane = verify.Lane(16, 48)
+    gpu.set_block([lane], draft)
+    backend.run(gpu.encode([lane], commit=True))
+    got = gpu.buffer(verify.LOGITS).download(np.float32, 16 * 32000).reshape(16, 32000)
+    want = model.oracle_step(draft, 48)
+    cos = (got.astype(np.float64) * want["logits"]).sum() / np.sqrt((got.astype(np.float64) ** 2).sum() * (want["logits"] ** 2).sum())
+    assert cos >= 0.999 and np.abs(got - want["logits"]).max() <= 5e-2, (cos, np.abs(got - want["logits"]).max())
+    selected, retained, accepted, mask = gpu.results([lane])
+    picks = np.array([orc.argmax(got[r]) for r in range(16)], dtype=np.uint32)
+    kept, acc, m = orc.accept_tree(ops.chain_tree_rows([16]), draft, picks)
+    assert retained[0] == len(kept) and accepted[0] == acc and mask[0] == m and np.array_equal(selected[:len(kept)], kept)
