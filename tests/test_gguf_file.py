@@ -211,3 +211,27 @@ def test_a_dense_decoder_loads_from_a_file(tmp_path, value_format, tied):
     with pytest.raises(splash_amd.SplashError, match="blk.1.ffn_up.weight is missing; output_norm.weight is missing"):
         verify.DenseVerify.from_gguf(backend, gguf.GgufFile(bad), physical_pages=pages + 1)
     backend.close()
+
+
+def test_dense_geometry_from_metadata(tmp_path):
+    """spg_dense_dimensions (no device): the geometry a file's metadata and token table name; a missing key, another
+    epsilon and a partial rotary embedding are refused."""
+    from splash_amd import _native as nat
+    import ctypes
+    from tests.dense_reference import DenseModel
+    model = DenseModel(seed=6, hidden=256, q_heads=4, kv_heads=2, head_dim=64, ffn=256, vocabulary=256, layers=1, rope_theta=5e5)
+    path = tmp_path / "tiny.gguf"
+    dense_model_file(path, model, orc.FMT_Q4K, tied=True)
+    d = nat.DenseDimensions()
+    f = gguf.GgufFile(path)
+    splash_amd.check(splash_amd.lib.spg_dense_dimensions(f.handle, ctypes.byref(d)))
+    assert (d.hidden, d.q_heads, d.kv_heads, d.head_dim, d.ffn, d.vocabulary, d.layers, d.rotary_pairs, d.normalize_heads, d.rope_theta) == \
+        (256, 4, 2, 64, 256, 256, 1, 32, 1, 5e5)
+    raw = open(path, "rb").read()
+    for name, edit in (("key", lambda b: b.replace(b"qwen3.block_count", b"qwen3.block_coumt")),
+                       ("architecture", lambda b: b.replace(b"general.architecture", b"general.architectura"))):
+        bad = tmp_path / f"{name}.gguf"
+        open(bad, "wb").write(edit(raw))
+        broken = gguf.GgufFile(bad)
+        with pytest.raises(splash_amd.SplashError):
+            splash_amd.check(splash_amd.lib.spg_dense_dimensions(broken.handle, ctypes.byref(d)))
