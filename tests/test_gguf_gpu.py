@@ -407,3 +407,43 @@ def test_backend_one_command_in_flight_and_unknown_kernel(backend):
     rec = backend.record(g2)
     rec.submit().wait()
     assert np.array_equal(out.download(np.float32), first)
+
+
+@pytest.mark.parametrize("name,fmt,widths,K", [("gate_up", ops.FMT_Q4K, (25600,), 5120), ("fused_qkv", ops.FMT_Q4K, (5120, 1024, 1024), 5120),
+                                               ("down", ops.FMT_Q6K, (5120,), 25600)])
+def test_config2_projections_at_full_size(backend, name, fmt, widths, K):
+    """BASELINE.json config 2's shapes (K 5120 with N 25600 and the fused 5120 + 2 x 1024; the down projection K 25600,
+    N 5120 in Q6_K) at M = 1, 4, 8, 16, 32 rows, through properties that do not need the oracle over the whole matrix:
+    a sample of columns lies in the reference interval of the fp64 dot (gguf_projection_test.mm:217-237); doubling the
+    input doubles every fp32 output bit for bit; and a row's result is the same in a block of any height."""
+    print(f"case config 2 full size {name}", flush=True)
+    rng = np.random.default_rng(len(name))
+    natives = [orc.make_native(fmt, n, K, 900 + i) for i, n in enumerate(widths)]
+    N = sum(widths)
+    proj = ops.Projection.from_native(backend, [(fmt, n, native) for n, native in zip(widths, natives)], K, float32=True)
+    linear = ops.Linear(backend)
+    x = orc.f32_to_bf16(rng.standard_normal((32, K)).astype(np.float32))
+    row_bytes = natives[0].size // widths[0]
+    sample = np.sort(rng.choice(widths[0], 48, replace=False))
+    sampled_native = np.concatenate([natives[0][c * row_bytes:(c + 1) * row_bytes] for c in sample])
+    want = orc.gemm(fmt, sampled_native, x, len(sample), want=("exact", "bound"))
+
+    def run(rows_bits, plan):
+        out = backend.allocate_buffer(rows_bits.shape[0] * N * 4)
+        graph = splash_amd.CommandGraph()
+        linear.add(graph, proj, plan, backend.from_array(rows_bits), out, linear.scratch_for(backend, [plan]))
+        backend.run(graph)
+        return out.download(np.float32).reshape(rows_bits.shape[0], N)
+    tallest = linear.plan(proj, 32, ops.EPILOGUE_NONE)
+    full = run(x, tallest)
+    for M in (1, 4, 8, 16, 32):
+        got = run(x[:M], linear.plan(proj, M, ops.EPILOGUE_NONE))
+        assert np.all(np.abs(got[:, sample].astype(np.float64) - want["exact"][:M]) <= want["bound"][:M]), M
+        assert np.isfinite(got).all()
+        # the same partition of K as the tallest block's: the rows are its rows, bit for bit
+        same = linear.plan(proj, M, ops.EPILOGUE_NONE, splits=tallest.splits, whole_groups=tallest.whole_groups)
+        if same.storage_rows == tallest.storage_rows:
+            assert run(x[:M], same).tobytes() == full[:M].tobytes(), M
+    doubled = orc.f32_to_bf16(2 * orc.bf16_to_f32(x[:16]))
+    plan = linear.plan(proj, 16, ops.EPILOGUE_NONE)
+    assert (2 * run(x[:16], plan)).tobytes() == run(doubled, plan).tobytes()
