@@ -964,9 +964,16 @@ __global__ __launch_bounds__(256) void gguf_moe_decode(const uint8_t *__restrict
                                reinterpret_cast<const uint16_t *>(next_tables + tile * m.next_table_bytes), nullptr, nullptr, p,
                                blockIdx.x);
 }
-SP_REGISTER_KERNEL("gguf_moe_decode_q4k_gt", (&gguf_moe_decode<GGUF_FMT_Q4K, GGUF_EPILOGUE_GATE_UP_TABLE>));
-SP_REGISTER_KERNEL("gguf_moe_decode_q4k_a", (&gguf_moe_decode<GGUF_FMT_Q4K, GGUF_EPILOGUE_PLAIN>));
-SP_REGISTER_KERNEL("gguf_moe_decode_q6k_a", (&gguf_moe_decode<GGUF_FMT_Q6K, GGUF_EPILOGUE_PLAIN>));
+// Every image format serves the experts' one-pass gate/up (_gt) and their down projection (_a).
+#define SP_GGUF_MOE_DECODE(fmt, FMT)                                                                                  \
+  SP_REGISTER_KERNEL("gguf_moe_decode_" fmt "_gt", (&gguf_moe_decode<FMT, GGUF_EPILOGUE_GATE_UP_TABLE>));             \
+  SP_REGISTER_KERNEL("gguf_moe_decode_" fmt "_a", (&gguf_moe_decode<FMT, GGUF_EPILOGUE_PLAIN>))
+SP_GGUF_MOE_DECODE("q4k", GGUF_FMT_Q4K);
+SP_GGUF_MOE_DECODE("q6k", GGUF_FMT_Q6K);
+SP_GGUF_MOE_DECODE("q5k", GGUF_FMT_Q5K);
+SP_GGUF_MOE_DECODE("q80", GGUF_FMT_Q80);
+SP_GGUF_MOE_DECODE("iq4xs", GGUF_FMT_IQ4XS);
+SP_GGUF_MOE_DECODE("iq4nl", GGUF_FMT_IQ4NL);
 
 #define SP_GGUF_DECODE(fmt, FMT, rows, RT)                                                              \
   SP_REGISTER_KERNEL("gguf_decode_" fmt "_m" #rows "_a", &gguf_decode<FMT, RT, GGUF_EPILOGUE_PLAIN>);   \

@@ -16,9 +16,8 @@ void requireShape(const MoeShape &shape, uint32_t rows) {
     throw std::invalid_argument("too many experts for that many routes: experts * ceil(rows * routes a row / 32) is at most 16384");
 }
 const char *formatName(uint32_t format) {
-  if (format == GGUF_FMT_Q4K) return "q4k";
-  if (format == GGUF_FMT_Q6K) return "q6k";
-  throw std::invalid_argument("no routed expert kernel for this format");
+  if (!gguf_record_bytes(format)) throw std::invalid_argument("no routed expert kernel for this format");
+  return gguf_format_name(format);
 }
 } // namespace
 
@@ -80,7 +79,6 @@ void MoE::addRouted(hip::CommandGraph &graph, const hip::Buffer &normalized, con
   const MoeWorkspaceSize need = workspace(shape, rows);
   const uint32_t routes = rows * shape.routesPerRow(), tiles = moe_maximum_tiles(routes, shape.allExperts());
   const std::string pairKernel = std::string("gguf_moe_decode_") + formatName(experts.format) + "_gt";
-  if (experts.format != GGUF_FMT_Q4K) throw std::invalid_argument("routed gate and up projections are Q4_K");
   const std::string downKernel = std::string("gguf_moe_decode_") + formatName(experts.downFormat) + "_a";
   const uint64_t pairBytes = gguf_image_bytes(experts.format, shape.ffn, shape.hidden);
   const uint64_t downBytes = gguf_image_bytes(experts.downFormat, shape.hidden, shape.ffn);

@@ -9,13 +9,14 @@ from tests import oracle as orc
 pytestmark = pytest.mark.gpu
 
 
-def run_layer(backend, rng, hidden, ffn, experts, top_k, rows, down_fmt=ops.FMT_Q4K, following=None, shared=0, gated=False, sigmoid=False):
+def run_layer(backend, rng, hidden, ffn, experts, top_k, rows, down_fmt=ops.FMT_Q4K, following=None, shared=0, gated=False, sigmoid=False,
+              fmt=ops.FMT_Q4K):
     """shared: slices of a shared expert, whose images follow the routed experts'; gated: they weigh sigmoid(x . gate)."""
-    gate = [orc.make_native(ops.FMT_Q4K, ffn, hidden, 100 + e) for e in range(experts + shared)]
-    up = [orc.make_native(ops.FMT_Q4K, ffn, hidden, 300 + e) for e in range(experts + shared)]
+    gate = [orc.make_native(fmt, ffn, hidden, 100 + e) for e in range(experts + shared)]
+    up = [orc.make_native(fmt, ffn, hidden, 300 + e) for e in range(experts + shared)]
     down = [orc.make_native(down_fmt, hidden, ffn, 500 + e) for e in range(experts + shared)]
     images = [backend.from_array(np.concatenate([ops.pack_gguf_image(f, n, r, k) for n in natives]))
-              for natives, f, r, k in ((gate, ops.FMT_Q4K, ffn, hidden), (up, ops.FMT_Q4K, ffn, hidden), (down, down_fmt, hidden, ffn))]
+              for natives, f, r, k in ((gate, fmt, ffn, hidden), (up, fmt, ffn, hidden), (down, down_fmt, hidden, ffn))]
     x = orc.f32_to_bf16(rng.standard_normal((rows, hidden)).astype(np.float32))
     res = orc.f32_to_bf16(rng.standard_normal((rows, hidden)).astype(np.float32))
     scores = rng.standard_normal((rows, experts)).astype(np.float32)
@@ -27,11 +28,11 @@ def run_layer(backend, rng, hidden, ffn, experts, top_k, rows, down_fmt=ops.FMT_
     moe.add_routing(graph, backend.from_array(scores), input=backend.from_array(x) if gated else None,
                     shared_scalar_gate=backend.from_array(scalar_gate) if gated else None)
     extra = dict(norm_weight=following[0], next_table=following[1]) if following else {}
-    moe.add_routed(graph, backend.from_array(x), backend.from_array(res), out, *images, down_fmt=down_fmt, **extra)
+    moe.add_routed(graph, backend.from_array(x), backend.from_array(res), out, *images, fmt=fmt, down_fmt=down_fmt, **extra)
     assert len(graph) == 6
     backend.run(graph)
     got = out.download(np.uint16).reshape(rows, hidden)
-    want = orc.moe_layer(x, res, scores, top_k, gate, up, down, ffn, down_fmt=down_fmt, shared=shared, shared_gate=scalar_gate,
+    want = orc.moe_layer(x, res, scores, top_k, gate, up, down, ffn, fmt=fmt, down_fmt=down_fmt, shared=shared, shared_gate=scalar_gate,
                          sigmoid_router=sigmoid)
     return moe, got, want
 
@@ -96,6 +97,16 @@ def test_shared_expert_slices_ride_every_row(backend, config):
     check_layer(moe, got, want, rows, experts, top_k, shared)
     if not gated:
         assert np.all(want[1][:, top_k:] == 1.0)
+
+
+@pytest.mark.parametrize("fmt,down_fmt", [(ops.FMT_IQ4XS, ops.FMT_Q5K), (ops.FMT_Q5K, ops.FMT_Q6K), (ops.FMT_Q80, ops.FMT_IQ4NL), (ops.FMT_Q6K, ops.FMT_Q80)])
+def test_expert_tensors_of_every_image_format(backend, fmt, down_fmt):
+    """The experts of a real file are not all Q4_K: every weight-image format serves the one-pass gate/up and the down
+    projection of the routed experts."""
+    print(f"case moe formats {fmt} {down_fmt}", flush=True)
+    rng = np.random.default_rng(fmt * 7 + down_fmt)
+    moe, got, want = run_layer(backend, rng, 512, 256, 8, 2, 24, fmt=fmt, down_fmt=down_fmt)
+    check_layer(moe, got, want, 24, 8, 2)
 
 
 def test_sigmoid_router_weighs_by_normalized_sigmoids(backend):
