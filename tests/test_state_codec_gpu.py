@@ -137,3 +137,43 @@ def test_extents_are_checked_before_anything_is_added(backend):
     assert len(graph) == 0
     ops.StateCodec.add_quantize(graph, state, codes, shape)
     assert graph.kernels() == ["state_quantize"]
+
+
+def test_a_lane_restored_from_its_coded_state_goes_on_within_a_percent(backend):
+    """State capture end to end: a Gated DeltaNet lane's cell (what GDN::addFold or a step leaves) is coded, restored
+    into another cell by the codec, and the lane's next block runs from both. The restored state is within the 1 %
+    the reference measured on its models (state_codec_metal_test.mm:8-10), the coded form is the oracle's byte for
+    byte, and the block's outputs from the restored cell stay within a percent of those from the exact one."""
+    print("case state codec restores a GDN lane", flush=True)
+    from tests.gdn_case import make_rows, make_state
+    from tests.test_gdn_gpu import Layer
+    rng = np.random.default_rng(41)
+    key_heads, value_heads = 4, 8
+    layer = Layer(backend, rng, key_heads, value_heads, lanes=1, cells=4)
+    conv, state = make_state(rng, layer.shape)
+    layer.write_cell(0, 0, conv, state)
+    first = make_rows(rng, layer.shape, 16)
+    layer.step([(0, first, 0, 0, 0, 1)])                       # cell 1: the state before the block; tape 0: its rows
+    second = make_rows(rng, layer.shape, 16)
+    exact = layer.step([(0, second, 0xFFFF, 1, 1, 2)])[0]      # folds the sixteen rows, runs the next block; cell 2 holds the fold
+    conv2, state2 = layer.read_cell(0, 2)
+    # code cell 2's recurrent layer, restore it into cell 3 beside a copy of the convolution carry
+    st, gdn = layer.gdn.strides, layer.gdn
+    rows, columns = value_heads * 128, 128
+    shape = ops.StateCodec.shape(1, rows, columns, st.recurrent_layer_bytes, ops.StateCodec.layer_bytes(rows, columns))
+    view = lambda cell: layer.states.view(layer.cell(0, cell) + st.convolution_state_bytes, st.recurrent_layer_bytes)
+    codes = backend.allocate_buffer(ops.StateCodec.layer_bytes(rows, columns))
+    graph = splash_amd.CommandGraph()
+    ops.StateCodec.add_quantize(graph, view(2), codes, shape)
+    ops.StateCodec.add_dequantize(graph, codes, view(3), shape)
+    backend.run(graph)
+    assert np.array_equal(codes.download(np.uint8), orc.state_codes(state2.reshape(rows, columns)))
+    layer.states.upload(np.ascontiguousarray(conv2), layer.cell(0, 3))
+    _, restored = layer.read_cell(0, 3)
+    assert np.linalg.norm(restored - state2) <= 0.01 * np.linalg.norm(state2)
+    third = make_rows(rng, layer.shape, 16)
+    from_exact = layer.step([(0, third, 0, 0, 2, 1)])[0]
+    from_restored = layer.step([(0, third, 0, 0, 3, 1)])[0]
+    a, b = orc.bf16_to_f32(from_exact).astype(np.float64), orc.bf16_to_f32(from_restored).astype(np.float64)
+    assert np.linalg.norm(a - b) <= 0.01 * np.linalg.norm(a), np.linalg.norm(a - b) / np.linalg.norm(a)
+    assert np.isfinite(b).all() and exact.shape == from_exact.shape
