@@ -109,7 +109,7 @@ def cpu_baseline(w):
     rng = np.random.default_rng(5)
     rows, H, F = w["rows"], w["hidden"], w["ffn"]
     x = orc.f32_to_bf16(rng.standard_normal((rows, H)).astype(np.float32))
-    PASSES = 60
+    PASSES = 120
     sample_n = F      # the whole gate projection, and a quarter of the down projection's columns
     t0 = time.time()
     bytes_done = 0
