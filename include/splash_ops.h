@@ -313,6 +313,17 @@ sp_status spo_sampling_add_acceptance(spo_graph *graph, sp_buffer *input_tokens,
                                       const spo_lane_rows *lanes, const uint32_t *remaining, uint32_t count,
                                       const uint32_t stop_tokens[4]);
 
+/* ---- DraftSelector::addVerifyRows (runtime/ops/DraftSelector.hpp:139-147; StepRows, LaneRows.hpp:49-67): a decode
+ *      step's rows from the trees a draft selector grew. Each lane's tree holds tree_sizes[lane] rows of 16 (tokens,
+ *      SplashTreeRow rows, fp32 pairs of draft probability and estimate), best first; the step takes every lane's
+ *      anchor and the best other rows by estimate that `rows` and `lane_cap` hold, none estimated below `floor`,
+ *      numbers each lane's in preorder and writes their tokens, tree rows, lane rows {first, rows} and sources (the
+ *      tree row each is; 0xFFFFFFFF for the rows past the lanes', which belong to no lane). The selector's scoring
+ *      kernels are not part of this library. ---- */
+sp_status spo_draft_add_verify_rows(spo_graph *graph, sp_buffer *tree_tokens, sp_buffer *trees, sp_buffer *tree_scores,
+                                    sp_buffer *tree_sizes, sp_buffer *input_tokens, sp_buffer *tree_rows, sp_buffer *lane_rows,
+                                    sp_buffer *verify_sources, uint32_t lanes, uint32_t rows, uint32_t lane_cap, float floor);
+
 /* ---- The dense verify step (the reference's model layer: QwenTarget.cpp:206-395, :457-496;
  *      Runtime.cpp:2677-2717, :2883-2892) ---- */
 typedef struct spo_dense_verify spo_dense_verify;

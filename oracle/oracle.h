@@ -26,6 +26,8 @@
 //                                   closed cases of the reference's test (prompt-only, saturation, unselectable).
 //   orc_thinking_cutoff             pinned by an independent walk over explicit depth-ordered paths (tests) and the
 //                                   closed form on chains.
+//   orc_draft_verify_rows           pinned by an independent statement (a stable sort of the estimates, a recursive
+//                                   preorder) in the tests.
 //   orc_rejection_*                 pinned by enumeration: selection law equals target to 1e-12.
 //   orc_distribution_end            pinned by an independent fp64 sort (min_p, top_k with ties, nucleus).
 //   orc_moe_*                       pinned by a stable sort and softmax closed form; the layer by the dense FFN it
@@ -139,6 +141,12 @@ void orc_penalize(float *logits, uint32_t rows, uint32_t vocab, uint32_t stride,
 void orc_thinking_cutoff(uint32_t *selected, uint32_t rows, uint32_t vocab, const uint32_t *inputs, const struct OrcTreeRow *tree,
                          const uint32_t *masks, uint32_t mask_words, uint32_t cutoff_row, const uint32_t *end, uint32_t count,
                          uint32_t close, uint32_t also_ends, int waits);
+// sampling.metal:1799-1895 draft_verify_rows: a decode step's rows from each lane's tree (16 rows a lane: tokens, tree
+// rows, {draft probability, estimate} pairs; sizes[lane] rows held). Outputs as the kernel writes them: tokens, tree rows
+// and sources [rows], lane_rows {first, rows} [lanes].
+void orc_draft_verify_rows(const uint32_t *tree_tokens, const struct OrcTreeRow *trees, const float *scores, const uint32_t *sizes,
+                           uint32_t lanes, uint32_t rows, uint32_t lane_cap, float floor, uint32_t *tokens, struct OrcTreeRow *tree,
+                           uint32_t *lane_rows, uint32_t *sources);
 // One sampled verify row under the textbook full-vocabulary rule in the reference's order of
 // operations (sampling.metal:713-885): weight_t = exp((logit_t - max) / T); p = weight / total;
 // accept the drafted token iff u_child * q[draft] < p[draft]; else draw from max(p - q, 0)

@@ -182,6 +182,66 @@ void orc_thinking_cutoff(uint32_t *selected, uint32_t rows, uint32_t vocab, cons
   }
 }
 
+void orc_draft_verify_rows(const uint32_t *tree_tokens, const struct OrcTreeRow *trees, const float *scores, const uint32_t *sizes,
+                           uint32_t lanes, uint32_t rows, uint32_t lane_cap, float floor, uint32_t *tokens, struct OrcTreeRow *tree,
+                           uint32_t *lane_rows, uint32_t *sources) {
+  constexpr uint32_t kRows = 16;
+  std::vector<float> estimates;
+  std::vector<uint32_t> owners;
+  for (uint32_t lane = 0; lane < lanes; ++lane)
+    for (uint32_t row = 1; row < sizes[lane]; ++row) {
+      const float estimate = scores[(lane * kRows + row) * 2 + 1];
+      size_t at = estimates.size();
+      estimates.push_back(estimate);
+      owners.push_back(lane);
+      for (; at > 0 && estimates[at - 1] < estimate; --at) {   // an earlier row first among equal ones
+        estimates[at] = estimates[at - 1];
+        owners[at] = owners[at - 1];
+      }
+      estimates[at] = estimate;
+      owners[at] = lane;
+    }
+  std::vector<uint32_t> taken_of(lanes, 1);
+  uint32_t taken = lanes;
+  for (size_t i = 0; i < estimates.size() && taken < rows; ++i) {
+    if (estimates[i] < floor) break;
+    if (taken_of[owners[i]] == lane_cap) continue;
+    ++taken_of[owners[i]];
+    ++taken;
+  }
+  uint32_t first = 0;
+  for (uint32_t lane = 0; lane < lanes; ++lane) {
+    const uint32_t mine = taken_of[lane];
+    uint32_t order[kRows], placed[kRows], stack[kRows], size = 0, next = 0;
+    stack[size++] = 0;
+    while (size) {
+      const uint32_t row = stack[--size];
+      placed[row] = next;
+      order[next++] = row;
+      for (uint32_t child = mine; child-- > row + 1;)
+        if (trees[lane * kRows + child].parent == row) stack[size++] = child;
+    }
+    uint32_t ancestors[kRows], depths[kRows];
+    for (uint32_t at = 0; at < next; ++at) {
+      const uint32_t row = order[at];
+      const uint32_t up = at ? placed[trees[lane * kRows + row].parent] : 0xFFFFu;
+      ancestors[at] = (at ? ancestors[up] : 0u) | (1u << at);
+      depths[at] = at ? depths[up] + 1 : 0;
+      tokens[first + at] = tree_tokens[lane * kRows + row];
+      tree[first + at] = {ancestors[at], uint16_t(up), uint16_t(depths[at])};
+      sources[first + at] = row;
+    }
+    lane_rows[2 * lane] = first;
+    lane_rows[2 * lane + 1] = next;
+    first += next;
+  }
+  for (uint32_t row = first; row < rows; ++row) {
+    tokens[row] = tree_tokens[0];
+    tree[row] = {0u, 0xFFFFu, 0};
+    sources[row] = 0xFFFFFFFFu;
+  }
+}
+
 uint32_t orc_argmax(const float *logits, uint32_t vocab) {
   float best = -std::numeric_limits<float>::infinity();
   uint32_t index = ORC_NO_TOKEN;

@@ -89,6 +89,18 @@ struct ThinkingCutoffParams {
   uint32_t tokens[SAMPLING_MAXIMUM_LANES][SAMPLING_MAXIMUM_ROWS];
 };
 
+// draft_verify_rows: one thread lays out a decode step's rows from the trees a draft selector grew (the reference's
+// VerifyRowsParams, abi/Sampling.h:270-298): `rows` rows over `lanes` lanes, each lane its anchor and the best of its
+// tree's other rows by estimate that the step's rows and the lanes' cap hold, none estimated below `floor`; the rows
+// past the lanes' belong to no lane.
+#define SAMPLING_TREE_ROOT 0xFFFFu  // the parent of a row without one (SPLASH_TREE_ROOT)
+struct VerifyRowsParams {
+  uint32_t lanes;
+  uint32_t rows;
+  uint32_t lane_cap;
+  float floor;
+};
+
 // decode_accept_tree: one thread per lane (AcceptBatchParams).
 struct AcceptBatchParams {
   uint32_t lanes;
@@ -102,5 +114,6 @@ struct AcceptBatchParams {
 static_assert(sizeof(TargetSamplingParams) == 16 + 32 + 16 + 64 + 96 + 32, "target sampling parameters are 256 bytes on both sides");
 static_assert(sizeof(SamplingPenaltyParams) == 16 + 64 + 5 * 32, "penalty parameters are 240 bytes on both sides");
 static_assert(sizeof(ThinkingCutoffParams) == 16 + 64 + 4 * 32 + 512, "thinking cutoff parameters are 720 bytes on both sides");
+static_assert(sizeof(VerifyRowsParams) == 16, "verify rows parameters are 16 bytes on both sides");
 static_assert(sizeof(AcceptBatchParams) == 16 + 32 + 16 + 64, "acceptance parameters are 128 bytes on both sides");
 #endif

@@ -5,6 +5,7 @@
 #include "model/DenseVerify.hpp"
 #include "model/GgufTarget.hpp"
 #include "splash_gguf.h"
+#include "ops/DraftSelector.hpp"
 #include "ops/Glue.hpp"
 #include "ops/Sampling.hpp"
 
@@ -156,6 +157,18 @@ sp_status spo_sampling_add_thinking_cutoff(spo_graph *graph, sp_buffer *input_to
     }
     ops::Sampling::addThinkingCutoff(capi::graphOf(graph), B(input_tokens), token_mask ? B(token_mask) : hip::Buffer{}, mask_words,
                                      B(tree_rows), B(tokens), vocabulary, rows, list);
+  });
+}
+
+sp_status spo_draft_add_verify_rows(spo_graph *graph, sp_buffer *tree_tokens, sp_buffer *trees, sp_buffer *tree_scores,
+                                    sp_buffer *tree_sizes, sp_buffer *input_tokens, sp_buffer *tree_rows, sp_buffer *lane_rows,
+                                    sp_buffer *verify_sources, uint32_t lanes, uint32_t rows, uint32_t lane_cap, float floor) {
+  return capi::guard([&] {
+    capi::require(graph, "graph");
+    ops::DraftSelector::addVerifyRows(capi::graphOf(graph),
+                                      {B(tree_tokens), B(trees), B(tree_scores), B(tree_sizes), B(input_tokens), B(tree_rows), B(lane_rows),
+                                       B(verify_sources)},
+                                      {lanes, rows, lane_cap}, floor);
   });
 }
 

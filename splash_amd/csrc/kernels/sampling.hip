@@ -148,6 +148,79 @@ __global__ __launch_bounds__(64) void decode_sample_thinking_cutoff(const uint32
 }
 SP_REGISTER_KERNEL("decode_sample_thinking_cutoff", &decode_sample_thinking_cutoff);
 
+// draft_verify_rows (sampling.metal:1799-1895): lane l's tree holds sizes[l] rows from row l * 16 of tree_tokens, trees
+// and scores (a row's draft probability and its estimate, the chance that the target accepts it), in the order the
+// selector took them, best first. A lane's rows are numbered in preorder, the earlier-taken child first, so that the
+// likeliest path of its tree lies on its first rows; the rows of no lane carry lane 0's anchor, no path and no source.
+__global__ __launch_bounds__(64) void draft_verify_rows(const uint32_t *__restrict__ tree_tokens, const AttentionTreeRow *__restrict__ trees,
+                                                        const float2 *__restrict__ scores, const uint32_t *__restrict__ sizes,
+                                                        uint32_t *__restrict__ tokens, AttentionTreeRow *__restrict__ tree,
+                                                        SamplingLaneRows *__restrict__ lane_rows, uint32_t *__restrict__ sources,
+                                                        VerifyRowsParams p) {
+  constexpr uint32_t kLanes = SAMPLING_MAXIMUM_LANES, kRows = SAMPLING_MAXIMUM_ROWS;
+  if (blockIdx.x || threadIdx.x) return;
+  // Every lane's rows past its anchor by estimate, a lane's earlier row first among equal ones.
+  float estimates[kLanes * kRows];
+  uint32_t owners[kLanes * kRows];
+  uint32_t count = 0;
+  for (uint32_t lane = 0; lane < p.lanes; ++lane)
+    for (uint32_t row = 1; row < min(sizes[lane], kRows); ++row) {
+      const float estimate = scores[lane * kRows + row].y;
+      uint32_t at = count++;
+      for (; at > 0 && estimates[at - 1] < estimate; --at) {
+        estimates[at] = estimates[at - 1];
+        owners[at] = owners[at - 1];
+      }
+      estimates[at] = estimate;
+      owners[at] = lane;
+    }
+  // The best of them that the step's rows and the lanes' cap hold, none below the floor: they fall, so the first
+  // below it ends them.
+  uint32_t taken_of[kLanes];
+  for (uint32_t lane = 0; lane < p.lanes; ++lane) taken_of[lane] = 1;
+  uint32_t taken = p.lanes;
+  for (uint32_t i = 0; i < count && taken < p.rows; ++i) {
+    if (estimates[i] < p.floor) break;
+    if (taken_of[owners[i]] == p.lane_cap) continue;
+    ++taken_of[owners[i]];
+    ++taken;
+  }
+  uint32_t first = 0;
+  for (uint32_t lane = 0; lane < p.lanes; ++lane) {
+    const uint32_t mine = taken_of[lane];
+    uint32_t parent[kRows], order[kRows], placed[kRows], stack[kRows];
+    for (uint32_t row = 0; row < mine; ++row) parent[row] = trees[lane * kRows + row].parent;
+    // Preorder: a row's children follow it, each with its subtree, in the order the tree took them.
+    uint32_t size = 0, next = 0;
+    stack[size++] = 0;
+    while (size) {
+      const uint32_t row = stack[--size];
+      placed[row] = next;
+      order[next++] = row;
+      for (uint32_t child = mine; child-- > row + 1;)
+        if (parent[child] == row && size < kRows) stack[size++] = child;
+    }
+    uint32_t ancestors[kRows], depths[kRows];
+    for (uint32_t at = 0; at < next; ++at) {
+      const uint32_t row = order[at];
+      const uint32_t up = at ? placed[parent[row]] : SAMPLING_TREE_ROOT;
+      ancestors[at] = (at ? ancestors[up] : 0u) | (1u << at);
+      depths[at] = at ? depths[up] + 1u : 0u;
+      tokens[first + at] = tree_tokens[lane * kRows + row];
+      tree[first + at] = AttentionTreeRow{ancestors[at], uint16_t(up), uint16_t(depths[at])};
+      sources[first + at] = row;
+    }
+    lane_rows[lane] = SamplingLaneRows{first, next};
+    first += next;
+  }
+  for (uint32_t row = first; row < p.rows; ++row) {
+    tokens[row] = tree_tokens[0];
+    tree[row] = AttentionTreeRow{0u, uint16_t(SAMPLING_TREE_ROOT), uint16_t(0)};
+    sources[row] = SAMPLING_NO_TOKEN;
+  }
+}
+SP_REGISTER_KERNEL("draft_verify_rows", &draft_verify_rows);
+
 // Grid (rows * SAMPLING_SHARDS), 256 threads. partial_values/indices [row][shard].
 __global__ __launch_bounds__(256) void decode_sample_argmax_sharded(const float *__restrict__ logits, float *__restrict__ partial_values,
                                                                     uint32_t *__restrict__ partial_indices, TargetSamplingParams p) {

@@ -307,6 +307,17 @@ class StateCodec:
         graph._keep.extend([source, destination])
 
 
+class DraftSelector:
+    """ops::DraftSelector::addVerifyRows: a decode step's rows from the trees a draft selector grew."""
+
+    @staticmethod
+    def add_verify_rows(graph, tree_tokens, trees, tree_scores, tree_sizes, input_tokens, tree_rows, lane_rows, verify_sources, lanes,
+                        rows, lane_cap, floor=0.0):
+        buffers = [tree_tokens, trees, tree_scores, tree_sizes, input_tokens, tree_rows, lane_rows, verify_sources]
+        check(lib.spo_draft_add_verify_rows(graph.handle, *[b.handle for b in buffers], lanes, rows, lane_cap, floor))
+        graph._keep.extend(buffers)
+
+
 def chain_tree_rows(rows_per_sequence):
     """SplashTreeRow of chains: ancestors (2 << r) - 1, parent r - 1, depth r, packed per sequence."""
     out = []

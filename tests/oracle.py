@@ -544,3 +544,23 @@ def thinking_cutoff(selected, inputs, tree, vocab, row, end, also_ends=NO_TOKEN,
                             _p(m, u32p), c_u32(m.shape[1] if m is not None else 0), c_u32(row), _p(tokens, u32p), c_u32(count),
                             c_u32(end[-1]), c_u32(also_ends), c_int(m is not None))
     return out
+
+
+TREE_DTYPE = np.dtype([("ancestors", "<u4"), ("parent", "<u2"), ("depth", "<u2")])
+
+
+def draft_verify_rows(tree_tokens, trees, scores, sizes, rows, lane_cap, floor=0.0):
+    """draft_verify_rows: (tokens [rows], tree rows [rows], lane rows [lanes][2], sources [rows]) of a step laid out from
+    each lane's tree: tree_tokens uint32 [lanes][16], trees TREE_DTYPE [lanes][16], scores fp32 [lanes][16][2]."""
+    lanes = len(sizes)
+    tree_tokens = np.ascontiguousarray(tree_tokens, dtype=np.uint32)
+    trees = np.ascontiguousarray(trees, dtype=TREE_DTYPE)
+    scores = np.ascontiguousarray(scores, dtype=np.float32)
+    sizes = np.ascontiguousarray(sizes, dtype=np.uint32)
+    tokens, tree = np.zeros(rows, np.uint32), np.zeros(rows, TREE_DTYPE)
+    lane_rows, sources = np.zeros((lanes, 2), np.uint32), np.zeros(rows, np.uint32)
+    lib.orc_draft_verify_rows.restype = None
+    lib.orc_draft_verify_rows(_p(tree_tokens, u32p), trees.ctypes.data_as(ctypes.c_void_p), _p(scores, f32p), _p(sizes, u32p), c_u32(lanes),
+                              c_u32(rows), c_u32(lane_cap), c_f(floor), _p(tokens, u32p), tree.ctypes.data_as(ctypes.c_void_p),
+                              _p(lane_rows, u32p), _p(sources, u32p))
+    return tokens, tree, lane_rows, sources

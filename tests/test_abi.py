@@ -35,7 +35,7 @@ def test_kernels_are_registered_by_name():
                  "gguf_decode_q4k_m16_a", "gguf_decode_q6k_m16_a_f32", "gguf_decode_q4k_m32_g", "gguf_decode_q6k_m64_r",
                  "gguf_decode_q5k_m16_gt", "gguf_decode_q80_m64_rn", "gguf_decode_mixed_m16_a", "gguf_decode_mixed_m64_a",
                  "gguf_dequant_iq4xs", "gguf_decode_iq4xs_m16_rn", "gguf_decode_iq4nl_m32_gt", "gguf_embed_iq4xs", "gguf_embed_iq4nl", "state_quantize", "state_dequantize_bf16_state", "state_copy",
-                 "decode_sample_penalize", "decode_sample_thinking_cutoff"):
+                 "decode_sample_penalize", "decode_sample_thinking_cutoff", "draft_verify_rows"):
         assert splash_amd.lib.sp_kernel_exists(name.encode()), name
     assert not splash_amd.lib.sp_kernel_exists(b"no_such_kernel")
 

@@ -388,3 +388,42 @@ def test_thinking_cutoff_rewrites_the_reached_rows(backend):
                                          token_mask=backend.from_array(masks), mask_words=words)
     with pytest.raises(splash_amd.SplashError):
         ops.Sampling.add_thinking_cutoff(graph, *args, [(0, [1], 0xFFFFFFFF, True), None, None, None, None])   # no masks
+
+
+def test_verify_rows_are_laid_out_from_the_trees(backend):
+    """draft_verify_rows (sampling.metal:1799-1895) against the oracle, bit for bit: tokens, tree rows, lane rows and
+    sources over random trees, caps, floors and tied estimates; and its outputs are what the acceptance walk reads."""
+    print("case draft verify rows", flush=True)
+    from tests.draft_case import grown_trees
+    rng = np.random.default_rng(37)
+    for trial in range(40):
+        lanes = int(rng.integers(1, 9))
+        tokens, trees, scores, sizes = grown_trees(rng, lanes, ties=trial % 3 == 0)
+        lane_cap = int(rng.integers(1, 17))
+        rows = int(rng.integers(lanes, lanes * lane_cap + 1))
+        floor = float(rng.choice([0.0, 0.3, 0.7]))
+        out = [backend.from_array(np.full(rows, 0xA5A5A5A5, np.uint32)), backend.from_array(np.zeros(rows, dtype=orc.TREE_DTYPE)),
+               backend.from_array(np.zeros((lanes, 2), np.uint32)), backend.from_array(np.full(rows, 0xA5A5A5A5, np.uint32))]
+        graph = splash_amd.CommandGraph()
+        ops.DraftSelector.add_verify_rows(graph, backend.from_array(tokens), backend.from_array(trees), backend.from_array(scores),
+                                          backend.from_array(sizes), *out, lanes, rows, lane_cap, floor)
+        backend.run(graph)
+        want = orc.draft_verify_rows(tokens, trees, scores, sizes, rows, lane_cap, floor)
+        got = (out[0].download(np.uint32), out[1].download(np.uint8).view(orc.TREE_DTYPE), out[2].download(np.uint32).reshape(lanes, 2),
+               out[3].download(np.uint32))
+        for g, w in zip(got, want):
+            assert np.array_equal(g, w), (trial, lanes, rows, lane_cap, floor)
+    # the step's rows feed the acceptance walk as they are: every lane accepts the path its selections name
+    lane_list = [(int(f), int(n)) for f, n in got[2]]
+    selected = rng.integers(0, 50000, rows).astype(np.uint32)
+    tb, ret, acc, mask = (backend.from_array(selected), backend.allocate_buffer(lanes * 4), backend.allocate_buffer(lanes * 4),
+                          backend.allocate_buffer(lanes * 4))
+    graph = splash_amd.CommandGraph()
+    ops.Sampling.add_acceptance(graph, out[0], out[1], tb, ret, acc, mask, lane_list, [0xFFFFFFFF] * lanes, [0xFFFFFFFF] * 4)
+    backend.run(graph)
+    for i, (f, n) in enumerate(lane_list):
+        kept, a, m = orc.accept_tree(got[1][f:f + n], got[0][f:f + n], selected[f:f + n])
+        assert ret.download(np.uint32)[i] == len(kept) and acc.download(np.uint32)[i] == a and mask.download(np.uint32)[i] == m
+    with pytest.raises(splash_amd.SplashError):
+        ops.DraftSelector.add_verify_rows(graph, backend.from_array(tokens), backend.from_array(trees), backend.from_array(scores),
+                                          backend.from_array(sizes), *out, lanes, lanes * lane_cap + 1, lane_cap, 0.0)

@@ -325,3 +325,29 @@ def test_thinking_cutoff_on_a_chain_closed_form():
     failed = selected.copy(); failed[5] = orc.NO_TOKEN
     assert orc.thinking_cutoff(failed, inputs, tree, vocab, 4, [90, 91, 92])[5] == orc.NO_TOKEN
     assert np.array_equal(orc.thinking_cutoff(selected, inputs, tree, vocab, 12, [90]), selected)   # past the block
+
+
+def test_verify_rows_layout_against_a_sort_and_a_recursive_preorder():
+    from tests.draft_case import grown_trees, layout_by_sorting
+    rng = np.random.default_rng(29)
+    for trial in range(200):
+        lanes = int(rng.integers(1, 9))
+        tokens, trees, scores, sizes = grown_trees(rng, lanes, ties=trial % 3 == 0)
+        lane_cap = int(rng.integers(1, 17))
+        rows = int(rng.integers(lanes, lanes * lane_cap + 1))
+        floor = float(rng.choice([0.0, 0.3, 0.7]))
+        got = orc.draft_verify_rows(tokens, trees, scores, sizes, rows, lane_cap, floor)
+        want = layout_by_sorting(tokens, trees, scores, sizes, rows, lane_cap, floor)
+        for g, w in zip(got, want):
+            assert np.array_equal(g, w), (trial, lanes, rows, lane_cap, floor)
+        # what the verify path relies on: a lane's first row is its anchor, parents precede children, a row's ancestors
+        # are its parent's and itself, and the rows of no lane are on no path
+        _, tree, lane_rows, sources = got
+        for first, count in lane_rows:
+            assert count >= 1 and int(tree[first]["ancestors"]) == 1 and int(tree[first]["parent"]) == 0xFFFF
+            for at in range(1, count):
+                up = int(tree[first + at]["parent"])
+                assert up < at and int(tree[first + at]["ancestors"]) == int(tree[first + up]["ancestors"]) | (1 << at)
+                assert int(tree[first + at]["depth"]) == int(tree[first + up]["depth"]) + 1
+        used = int(lane_rows[-1][0] + lane_rows[-1][1])
+        assert np.all(sources[used:] == orc.NO_TOKEN) and np.all(tree[used:]["ancestors"] == 0)
