@@ -336,6 +336,39 @@ def time_state_codec(backend):
     print(json.dumps(result), flush=True)
 
 
+def time_draft_candidates(backend):
+    """The draft selector's candidates and edge scores at the headline vocabulary (151936 columns) for 1 and 8 lanes:
+    per-dispatch GPU time (HIP events around each dispatch) over a ring of logits past the caches. Algorithmic bytes of the
+    top-16 kernel: the 7 proposal rows a lane of fp32 logits, read once. Prints one JSON line; not the headline metric."""
+    import splash_amd
+    from splash_amd import ops
+    rng = np.random.default_rng(0)
+    vocabulary, copies = 151936, 8
+    result = {"ops": "draft", "n_gpus": 1, "data": "synthetic", "workload": "7 proposal rows a lane of 151936 fp32 logits, rank-256 codebooks"}
+    before, after = (backend.from_array((rng.standard_normal((vocabulary, 256)).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16))
+                     for _ in range(2))
+    for lanes in (1, 8):
+        logits = [backend.from_array(rng.standard_normal((lanes * 8, vocabulary)).astype(np.float32)) for _ in range(copies)]
+        hidden = backend.from_array((rng.standard_normal((lanes * 8, 256)).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16))
+        scratch = backend.allocate_buffer(ops.DraftSelector.candidate_scratch_bytes(lanes, vocabulary))
+        out = [backend.allocate_buffer(lanes * 7 * 16 * 4), backend.allocate_buffer(lanes * 7 * 16 * 4), backend.allocate_buffer(lanes * 7 * 256 * 4)]
+        graph = splash_amd.CommandGraph()
+        for _ in range(4):
+            for c in range(copies):
+                ops.DraftSelector.add_candidates(graph, logits[c], hidden, scratch, *out, before, after, vocabulary, vocabulary, vocabulary,
+                                                 [1] * lanes)
+        backend.set_dispatch_profiling(True)
+        _, _, per = backend.run(graph, profiled=True)
+        backend.set_dispatch_profiling(False)
+        per = np.array(per).reshape(4, copies, 2)[1:] * 1e6
+        moved = lanes * 7 * vocabulary * 4
+        top, edges = float(np.median(per[:, :, 0])), float(np.median(per[:, :, 1]))
+        result[f"lanes_{lanes}"] = {"top16_us": round(top, 1), "top16_gbs": round(moved / top / 1e3, 1),
+                                    "top16_frac": round(moved / top / 1e3 / HBM_PEAK_GBS, 4), "edges_us": round(edges, 1)}
+        log(f"  {lanes} lane(s): top16 {top:6.1f} us {moved / top / 1e3:7.1f} GB/s, edges {edges:6.1f} us")
+    print(json.dumps(result), flush=True)
+
+
 C5 = dict(hidden=2048, vocabulary=151936, layers=48, q_heads=32, kv_heads=4, head_dim=128, gdn_key_heads=16, gdn_value_heads=32,
           experts=128, top_k=8, expert_ffn=768, context=16384, rows=16, lanes=8,
           name="35B-A3B-shaped hybrid MoE verify step: 36 GDN + 12 attention layers, 128 experts top-8 (Q4_K), 16-token draft, "
@@ -449,7 +482,7 @@ def main():
     ap.add_argument("--temperature", type=float, default=0.0,
                     help="above 0: rejection-sampling acceptance at this temperature against a full-vocabulary draft "
                          "distribution softmax(N(0, 2)) instead of greedy acceptance")
-    ap.add_argument("--ops", choices=["c2", "c3", "c5", "state"],
+    ap.add_argument("--ops", choices=["c2", "c3", "c5", "state", "draft"],
                     help="instead of the dense step: c2 the projections alone by rows, c3 attention alone by context, "
                          "c5 the GDN step and the MoE layer of config 5, state the recurrent layers' cached form")
     args = ap.parse_args()
@@ -460,7 +493,7 @@ def main():
     from splash_amd import ops, verify
     backend = splash_amd.Backend(0)
     if args.ops:
-        {"c2": time_c2_ops, "c3": time_c3_ops, "c5": time_c5_ops, "state": time_state_codec}[args.ops](backend)
+        {"c2": time_c2_ops, "c3": time_c3_ops, "c5": time_c5_ops, "state": time_state_codec, "draft": time_draft_candidates}[args.ops](backend)
         return
     if args.workload == "c5":
         bench_c5(backend, args)

@@ -318,8 +318,21 @@ sp_status spo_sampling_add_acceptance(spo_graph *graph, sp_buffer *input_tokens,
  *      SplashTreeRow rows, fp32 pairs of draft probability and estimate), best first; the step takes every lane's
  *      anchor and the best other rows by estimate that `rows` and `lane_cap` hold, none estimated below `floor`,
  *      numbers each lane's in preorder and writes their tokens, tree rows, lane rows {first, rows} and sources (the
- *      tree row each is; 0xFFFFFFFF for the rows past the lanes', which belong to no lane). The selector's scoring
- *      kernels are not part of this library. ---- */
+ *      tree row each is; 0xFFFFFFFF for the rows past the lanes', which belong to no lane). ---- */
+/* The first two kernels of DraftSelector::add (runtime/ops/DraftSelector.cpp:37-140; draft_select_top16_sharded and
+ * draft_select_edges, runtime/metal/kernels/decode/sampling.metal:1099-1356): of each of a lane's 7 proposal positions
+ * (rows 1-7 of its 8 query rows of `logits`, fp32 [lanes * 8][columns], columns = leading + vocabulary - trailing) the 16
+ * tokens of the largest logits, the larger first and among equal ones the smaller column (`candidates` uint32
+ * [lanes * 7][16], `unary` their logits; 0xFFFFFFFF and -inf where the columns run out), and `edges` fp32
+ * [lanes * 7][16][16]: [predecessor][candidate] the sum over the selector's rank of 256 of predecessor_codebook[token
+ * of the position before, anchors[lane] at position 0 (row 0 alone)] x selector_hidden[row] x successor_codebook[token],
+ * bf16 factors, fp32 sums. Codebooks bf16 [vocabulary][256]; selector_hidden bf16 [lanes * 8][256]; `scratch` of
+ * spo_draft_candidate_scratch_bytes. Up to 524288 columns. Growing the tree over them is not part of this library. */
+sp_status spo_draft_candidate_scratch_bytes(uint32_t lanes, uint32_t columns, uint64_t *bytes);
+sp_status spo_draft_add_candidates(spo_graph *graph, sp_buffer *logits, sp_buffer *selector_hidden, sp_buffer *scratch,
+                                   sp_buffer *candidates, sp_buffer *unary, sp_buffer *edges, sp_buffer *predecessor_codebook,
+                                   sp_buffer *successor_codebook, uint32_t leading, uint32_t trailing, uint32_t vocabulary,
+                                   const uint32_t *anchors, uint32_t lanes);
 sp_status spo_draft_add_verify_rows(spo_graph *graph, sp_buffer *tree_tokens, sp_buffer *trees, sp_buffer *tree_scores,
                                     sp_buffer *tree_sizes, sp_buffer *input_tokens, sp_buffer *tree_rows, sp_buffer *lane_rows,
                                     sp_buffer *verify_sources, uint32_t lanes, uint32_t rows, uint32_t lane_cap, float floor);

@@ -28,6 +28,10 @@
 //                                   closed form on chains.
 //   orc_draft_verify_rows           pinned by an independent statement (a stable sort of the estimates, a recursive
 //                                   preorder) in the tests.
+//   orc_draft_candidates            pinned by a lexicographic sort of (logit descending, column ascending) in the tests,
+//                                   ties, signed zeros and short rows among the cases.
+//   orc_draft_edges                 pinned by the fp64 trilinear sum over the decoded bf16 factors (numpy einsum), to the
+//                                   rounding of its fp32 products.
 //   orc_rejection_*                 pinned by enumeration: selection law equals target to 1e-12.
 //   orc_distribution_end            pinned by an independent fp64 sort (min_p, top_k with ties, nucleus).
 //   orc_moe_*                       pinned by a stable sort and softmax closed form; the layer by the dense FFN it
@@ -147,6 +151,16 @@ void orc_thinking_cutoff(uint32_t *selected, uint32_t rows, uint32_t vocab, cons
 void orc_draft_verify_rows(const uint32_t *tree_tokens, const struct OrcTreeRow *trees, const float *scores, const uint32_t *sizes,
                            uint32_t lanes, uint32_t rows, uint32_t lane_cap, float floor, uint32_t *tokens, struct OrcTreeRow *tree,
                            uint32_t *lane_rows, uint32_t *sources);
+// sampling.metal:1099-1264: of each proposal position's logits row (rows 1-7 of a lane's eight, fp32 [lanes * 8][columns])
+// the sixteen columns of the largest logits, the larger first, the smaller column first among equal ones; candidates their
+// tokens (a column at or past `leading` is token column - leading + trailing), unary their logits, [lanes * 7][16];
+// 0xffffffff and -infinity where the columns run out.
+void orc_draft_candidates(const float *logits, uint32_t lanes, uint32_t columns, uint32_t leading, uint32_t trailing,
+                          uint32_t *candidates, float *unary);
+// sampling.metal:1271-1356: edges fp32 [lanes * 7][16][16], [predecessor][candidate]; hidden bf16 [lanes * 8][256], codebooks
+// bf16 [vocabulary][256]. Position 0 writes its row 0 alone (predecessor anchors[lane]).
+void orc_draft_edges(const uint32_t *candidates, const uint32_t *anchors, uint32_t lanes, uint32_t vocabulary, const uint16_t *hidden,
+                     const uint16_t *predecessor_codebook, const uint16_t *successor_codebook, float *edges);
 // One sampled verify row under the textbook full-vocabulary rule in the reference's order of
 // operations (sampling.metal:713-885): weight_t = exp((logit_t - max) / T); p = weight / total;
 // accept the drafted token iff u_child * q[draft] < p[draft]; else draw from max(p - q, 0)

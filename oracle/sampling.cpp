@@ -182,6 +182,65 @@ void orc_thinking_cutoff(uint32_t *selected, uint32_t rows, uint32_t vocab, cons
   }
 }
 
+// sampling.metal:1050-1052 top_beats, :1099-1232 draft_select_top16_sharded, :1236-1264 top16_merge_shards: a sorted list
+// of sixteen, begun as empty entries (-infinity, token 0xffffffff), takes every column that beats its last entry; shards
+// and their merge select what one list over the whole row does. A column's token is itself below `leading`, else
+// column - leading + trailing. Rows 1-7 of a lane's eight query rows are its proposal positions.
+void orc_draft_candidates(const float *logits, uint32_t lanes, uint32_t columns, uint32_t leading, uint32_t trailing,
+                          uint32_t *candidates, float *unary) {
+  constexpr uint32_t K = 16, kPositions = 7, kQueryRows = 8;
+  for (uint32_t row = 0; row < lanes * kPositions; ++row) {
+    const float *x = logits + (size_t(row / kPositions) * kQueryRows + row % kPositions + 1) * columns;
+    float values[K];
+    uint32_t ids[K];
+    for (uint32_t i = 0; i < K; ++i) values[i] = -INFINITY, ids[i] = 0xffffffffu;
+    const auto beats = [](float value, uint32_t token, float other, uint32_t other_token) {
+      return value > other || (value == other && token < other_token);
+    };
+    for (uint32_t column = 0; column < columns; ++column) {
+      if (!beats(x[column], column, values[K - 1], ids[K - 1])) continue;
+      uint32_t at = K - 1;
+      for (; at > 0 && beats(x[column], column, values[at - 1], ids[at - 1]); --at) values[at] = values[at - 1], ids[at] = ids[at - 1];
+      values[at] = x[column], ids[at] = column;
+    }
+    for (uint32_t i = 0; i < K; ++i) {
+      candidates[row * K + i] = ids[i] < leading || ids[i] == 0xffffffffu ? ids[i] : ids[i] - leading + trailing;
+      unary[row * K + i] = values[i];
+    }
+  }
+}
+
+// sampling.metal:1271-1356 draft_select_edges: edges[row][predecessor][candidate] = sum over the rank of 256 of
+// (predecessor_codebook[predecessor token] * hidden[row]) * successor_codebook[candidate token], the factors bf16, each
+// product rounded to fp32; tokens clamp to the vocabulary. The reference leaves the order of the sum to its simdgroup
+// reduction; this one adds in fp64. Position 0 scores its anchor's row alone.
+void orc_draft_edges(const uint32_t *candidates, const uint32_t *anchors, uint32_t lanes, uint32_t vocabulary, const uint16_t *hidden,
+                     const uint16_t *predecessor_codebook, const uint16_t *successor_codebook, float *edges) {
+  constexpr uint32_t K = 16, kPositions = 7, kQueryRows = 8, kRank = 256;
+  const auto f = [](uint16_t bits) {
+    const uint32_t u = uint32_t{bits} << 16;
+    float v;
+    std::memcpy(&v, &u, 4);
+    return v;
+  };
+  for (uint32_t row = 0; row < lanes * kPositions; ++row) {
+    const uint32_t lane = row / kPositions, position = row % kPositions;
+    const uint16_t *h = hidden + (size_t(lane) * kQueryRows + position + 1) * kRank;
+    for (uint32_t predecessor = 0; predecessor < (position ? K : 1u); ++predecessor) {
+      const uint32_t before = std::min(position ? candidates[(row - 1) * K + predecessor] : anchors[lane], vocabulary - 1);
+      for (uint32_t candidate = 0; candidate < K; ++candidate) {
+        const uint32_t token = std::min(candidates[row * K + candidate], vocabulary - 1);
+        double sum = 0.0;
+        for (uint32_t d = 0; d < kRank; ++d) {
+          const float context = f(predecessor_codebook[size_t(before) * kRank + d]) * f(h[d]);
+          sum += double(context * f(successor_codebook[size_t(token) * kRank + d]));
+        }
+        edges[(size_t(row) * K + predecessor) * K + candidate] = float(sum);
+      }
+    }
+  }
+}
+
 void orc_draft_verify_rows(const uint32_t *tree_tokens, const struct OrcTreeRow *trees, const float *scores, const uint32_t *sizes,
                            uint32_t lanes, uint32_t rows, uint32_t lane_cap, float floor, uint32_t *tokens, struct OrcTreeRow *tree,
                            uint32_t *lane_rows, uint32_t *sources) {

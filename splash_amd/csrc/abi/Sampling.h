@@ -101,6 +101,27 @@ struct VerifyRowsParams {
   float floor;
 };
 
+// draft_select_top16_sharded, draft_select_edges (the reference's SelectorBatchParams, abi/Sampling.h:184-194, and
+// abi/ExecutionGeometry.h:6-7, :60-65): a lane's draft proposes DRAFT_PROPOSAL_TOKENS positions, rows 1-7 of its
+// DRAFT_QUERY_ROWS query rows, over the `columns` tokens of the draft's vocabulary: the target's first `leading`
+// tokens and those from `trailing` on. A workgroup of the first kernel selects among DRAFT_SHARD_COLUMNS columns.
+#define DRAFT_QUERY_ROWS 8u
+#define DRAFT_PROPOSAL_TOKENS 7u
+#define DRAFT_CANDIDATES 16u
+#define DRAFT_SELECTOR_RANK 256u
+#define DRAFT_SHARD_COLUMNS 4096u
+#define DRAFT_MAXIMUM_SHARDS 128u
+struct DraftSelectParams {
+  uint32_t anchor[SAMPLING_MAXIMUM_LANES];
+  uint32_t lanes;
+  uint32_t vocabulary;
+  uint32_t columns;
+  uint32_t leading;
+  uint32_t trailing;
+  uint32_t shards;
+  uint32_t reserved[2];
+};
+
 // decode_accept_tree: one thread per lane (AcceptBatchParams).
 struct AcceptBatchParams {
   uint32_t lanes;
@@ -114,6 +135,7 @@ struct AcceptBatchParams {
 static_assert(sizeof(TargetSamplingParams) == 16 + 32 + 16 + 64 + 96 + 32, "target sampling parameters are 256 bytes on both sides");
 static_assert(sizeof(SamplingPenaltyParams) == 16 + 64 + 5 * 32, "penalty parameters are 240 bytes on both sides");
 static_assert(sizeof(ThinkingCutoffParams) == 16 + 64 + 4 * 32 + 512, "thinking cutoff parameters are 720 bytes on both sides");
+static_assert(sizeof(DraftSelectParams) == 32 + 32, "draft selector parameters are 64 bytes on both sides");
 static_assert(sizeof(VerifyRowsParams) == 16, "verify rows parameters are 16 bytes on both sides");
 static_assert(sizeof(AcceptBatchParams) == 16 + 32 + 16 + 64, "acceptance parameters are 128 bytes on both sides");
 #endif

@@ -160,6 +160,25 @@ sp_status spo_sampling_add_thinking_cutoff(spo_graph *graph, sp_buffer *input_to
   });
 }
 
+sp_status spo_draft_candidate_scratch_bytes(uint32_t lanes, uint32_t columns, uint64_t *bytes) {
+  return capi::guard([&] {
+    capi::require(bytes, "result");
+    *bytes = ops::DraftSelector::candidateScratchBytes(lanes, columns);
+  });
+}
+
+sp_status spo_draft_add_candidates(spo_graph *graph, sp_buffer *logits, sp_buffer *selector_hidden, sp_buffer *scratch,
+                                   sp_buffer *candidates, sp_buffer *unary, sp_buffer *edges, sp_buffer *predecessor_codebook,
+                                   sp_buffer *successor_codebook, uint32_t leading, uint32_t trailing, uint32_t vocabulary,
+                                   const uint32_t *anchors, uint32_t lanes) {
+  return capi::guard([&] {
+    capi::require(graph && (anchors || !lanes), "graph or anchors");
+    ops::DraftSelector::addCandidates(capi::graphOf(graph), {B(logits), B(selector_hidden), B(scratch), B(candidates), B(unary), B(edges)},
+                                      {B(predecessor_codebook), B(successor_codebook)}, {leading, trailing}, vocabulary,
+                                      std::span<const uint32_t>(anchors, lanes));
+  });
+}
+
 sp_status spo_draft_add_verify_rows(spo_graph *graph, sp_buffer *tree_tokens, sp_buffer *trees, sp_buffer *tree_scores,
                                     sp_buffer *tree_sizes, sp_buffer *input_tokens, sp_buffer *tree_rows, sp_buffer *lane_rows,
                                     sp_buffer *verify_sources, uint32_t lanes, uint32_t rows, uint32_t lane_cap, float floor) {

@@ -308,7 +308,22 @@ class StateCodec:
 
 
 class DraftSelector:
-    """ops::DraftSelector::addVerifyRows: a decode step's rows from the trees a draft selector grew."""
+    """ops::DraftSelector: every proposal position's candidates and edge scores, and a decode step's rows from the trees
+    a draft selector grew."""
+
+    @staticmethod
+    def candidate_scratch_bytes(lanes, columns):
+        out = ctypes.c_uint64()
+        check(lib.spo_draft_candidate_scratch_bytes(lanes, columns, ctypes.byref(out)))
+        return out.value
+
+    @staticmethod
+    def add_candidates(graph, logits, selector_hidden, scratch, candidates, unary, edges, predecessor_codebook, successor_codebook,
+                       leading, trailing, vocabulary, anchors):
+        buffers = [logits, selector_hidden, scratch, candidates, unary, edges, predecessor_codebook, successor_codebook]
+        array = (ctypes.c_uint32 * max(len(anchors), 1))(*anchors)
+        check(lib.spo_draft_add_candidates(graph.handle, *[b.handle for b in buffers], leading, trailing, vocabulary, array, len(anchors)))
+        graph._keep.extend(buffers)
 
     @staticmethod
     def add_verify_rows(graph, tree_tokens, trees, tree_scores, tree_sizes, input_tokens, tree_rows, lane_rows, verify_sources, lanes,

@@ -60,3 +60,51 @@ def layout_by_sorting(tokens, trees, scores, sizes, rows, lane_cap, floor):
         out_tokens.append(int(tokens[0, 0])); out_tree.append((0, 0xFFFF, 0)); out_sources.append(0xFFFFFFFF)
     return (np.array(out_tokens, np.uint32), np.array(out_tree, dtype=orc.TREE_DTYPE), np.array(lane_rows, np.uint32),
             np.array(out_sources, np.uint32))
+
+
+def bf16_bits(values):
+    """fp32 values truncated to bf16 bit patterns (uint16): test data need no rounding."""
+    return (np.ascontiguousarray(values, dtype=np.float32).view(np.uint32) >> 16).astype(np.uint16)
+
+
+def bf16_values(bits):
+    return (np.asarray(bits, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+def proposal_logits(rng, lanes, columns, kind):
+    """fp32 [lanes * 8][columns] draft logits: plain, heavily tied (few distinct values, signed zeros among them), or
+    mostly -infinity so that a row has fewer than sixteen finite columns."""
+    shape = (lanes * 8, columns)
+    if kind == "tied":
+        return rng.choice(np.array([-2.0, -0.0, 0.0, 1.5, 3.0], np.float32), shape)
+    logits = (rng.standard_normal(shape) * 4).astype(np.float32)
+    if kind == "sparse":
+        logits[rng.random(shape) < 0.999] = -np.inf
+    return logits
+
+
+def candidates_by_sorting(logits, lanes, leading, trailing):
+    """The same candidates from a lexicographic sort: logit descending, column ascending; -0 equals +0."""
+    columns = logits.shape[1]
+    candidates, unary = np.full((lanes * 7, 16), 0xFFFFFFFF, np.uint32), np.full((lanes * 7, 16), -np.inf, np.float32)
+    for row in range(lanes * 7):
+        x = logits[row // 7 * 8 + row % 7 + 1]
+        order = np.lexsort((np.arange(columns), -(x.astype(np.float64) + 0.0)))[:16]
+        tokens = np.where(order < leading, order, order - leading + trailing)
+        candidates[row, :len(order)] = tokens
+        unary[row, :len(order)] = x[order]
+    return candidates, unary
+
+
+def edges_by_einsum(candidates, anchors, vocabulary, hidden, before, after):
+    """fp64 sum over the rank of predecessor x hidden x successor of the decoded bf16 factors; NaN where the kernel writes
+    nothing (position 0's rows past the anchor's)."""
+    h, b, a = (bf16_values(x).astype(np.float64) for x in (hidden, before, after))
+    out = np.full((candidates.shape[0], 16, 16), np.nan)
+    for row in range(candidates.shape[0]):
+        lane, position = divmod(row, 7)
+        previous = candidates[row - 1] if position else np.array([anchors[lane]], np.uint32)
+        previous, tokens = np.minimum(previous, vocabulary - 1), np.minimum(candidates[row], vocabulary - 1)
+        scores = np.einsum("pd,d,cd->pc", b[previous], h[lane * 8 + position + 1], a[tokens])
+        out[row, :len(previous)] = scores
+    return out

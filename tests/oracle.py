@@ -549,6 +549,32 @@ def thinking_cutoff(selected, inputs, tree, vocab, row, end, also_ends=NO_TOKEN,
 TREE_DTYPE = np.dtype([("ancestors", "<u4"), ("parent", "<u2"), ("depth", "<u2")])
 
 
+def draft_candidates(logits, lanes, leading=None, trailing=None):
+    """(candidates uint32 [lanes * 7][16], unary fp32 [lanes * 7][16]) of logits fp32 [lanes * 8][columns]."""
+    logits = np.ascontiguousarray(logits, dtype=np.float32)
+    columns = logits.shape[1]
+    leading = columns if leading is None else leading
+    trailing = leading if trailing is None else trailing
+    candidates, unary = np.zeros((lanes * 7, 16), np.uint32), np.zeros((lanes * 7, 16), np.float32)
+    lib.orc_draft_candidates.restype = None
+    lib.orc_draft_candidates(_p(logits, f32p), c_u32(lanes), c_u32(columns), c_u32(leading), c_u32(trailing), _p(candidates, u32p),
+                             _p(unary, f32p))
+    return candidates, unary
+
+
+def draft_edges(candidates, anchors, vocabulary, hidden, predecessor_codebook, successor_codebook):
+    """edges fp32 [lanes * 7][16][16]; hidden and the codebooks as bf16 bit patterns (uint16)."""
+    candidates = np.ascontiguousarray(candidates, dtype=np.uint32)
+    anchors = np.ascontiguousarray(anchors, dtype=np.uint32)
+    hidden, before, after = (np.ascontiguousarray(a, dtype=np.uint16) for a in (hidden, predecessor_codebook, successor_codebook))
+    edges = np.zeros((candidates.shape[0], 16, 16), np.float32)
+    u16p = ctypes.POINTER(ctypes.c_uint16)
+    lib.orc_draft_edges.restype = None
+    lib.orc_draft_edges(_p(candidates, u32p), _p(anchors, u32p), c_u32(len(anchors)), c_u32(vocabulary), _p(hidden, u16p), _p(before, u16p),
+                        _p(after, u16p), _p(edges, f32p))
+    return edges
+
+
 def draft_verify_rows(tree_tokens, trees, scores, sizes, rows, lane_cap, floor=0.0):
     """draft_verify_rows: (tokens [rows], tree rows [rows], lane rows [lanes][2], sources [rows]) of a step laid out from
     each lane's tree: tree_tokens uint32 [lanes][16], trees TREE_DTYPE [lanes][16], scores fp32 [lanes][16][2]."""

@@ -427,3 +427,52 @@ def test_verify_rows_are_laid_out_from_the_trees(backend):
     with pytest.raises(splash_amd.SplashError):
         ops.DraftSelector.add_verify_rows(graph, backend.from_array(tokens), backend.from_array(trees), backend.from_array(scores),
                                           backend.from_array(sizes), *out, lanes, lanes * lane_cap + 1, lane_cap, 0.0)
+
+
+def test_draft_candidates_and_edges(backend):
+    """draft_select_top16_sharded and draft_select_edges (sampling.metal:1099-1356) against the oracle: candidates and
+    their logits bit for bit (ties, signed zeros, short rows, rows of few finite columns, a draft vocabulary that skips a
+    range, a vocabulary of several shards with a ragged last one); edge scores to the fp32 rounding of a 256-term sum,
+    2^-20 of the terms' largest magnitude times 256, the order of the sum being the kernel's own."""
+    print("case draft candidates and edges", flush=True)
+    from tests.draft_case import bf16_bits, bf16_values, proposal_logits
+    rng = np.random.default_rng(73)
+    cases = [("plain", 151936, 151936, 151936, 1), ("plain", 32000, 20000, 139936, 8), ("tied", 20000, 8000, 9000, 3),
+             ("sparse", 40000, 40000, 40000, 2), ("plain", 9, 4, 10, 2), ("tied", 8193, 8193, 8193, 1), ("sparse", 300000, 300000, 300000, 1)]
+    for kind, columns, leading, trailing, lanes in cases:
+        print("  ", kind, columns, lanes, flush=True)
+        vocabulary = columns - leading + trailing
+        logits = proposal_logits(rng, lanes, columns, kind)
+        codebook_rows = min(vocabulary, 4096)      # random rows, repeated up to the vocabulary
+        hidden, before, after = (bf16_bits(rng.standard_normal(shape)) for shape in
+                                 ((lanes * 8, 256), (codebook_rows, 256), (codebook_rows, 256)))
+        anchors = rng.integers(0, vocabulary, lanes).astype(np.uint32)
+        out = [backend.from_array(np.full((lanes * 7, 16), 0xA5A5A5A5, np.uint32)), backend.from_array(np.zeros((lanes * 7, 16), np.float32)),
+               backend.from_array(np.zeros((lanes * 7, 16, 16), np.float32))]
+        scratch = backend.allocate_buffer(ops.DraftSelector.candidate_scratch_bytes(lanes, columns))
+        graph = splash_amd.CommandGraph()
+        ops.DraftSelector.add_candidates(graph, backend.from_array(logits), backend.from_array(hidden), scratch, *out,
+                                         backend.from_array(_padded(before, vocabulary)), backend.from_array(_padded(after, vocabulary)),
+                                         leading, trailing, vocabulary, list(anchors))
+        backend.run(graph)
+        candidates, unary = out[0].download(np.uint32).reshape(-1, 16), out[1].download(np.float32).reshape(-1, 16)
+        want = orc.draft_candidates(logits, lanes, leading, trailing)
+        assert np.array_equal(candidates, want[0]), (kind, columns)
+        assert np.array_equal(unary.view(np.uint32), want[1].view(np.uint32)), (kind, columns)
+        edges = out[2].download(np.float32).reshape(-1, 16, 16)
+        want_edges = orc.draft_edges(want[0], anchors, vocabulary, hidden, _padded(before, vocabulary), _padded(after, vocabulary))
+        scale = np.abs(bf16_values(hidden)).max() * np.abs(bf16_values(before)).max() * np.abs(bf16_values(after)).max() * 256
+        assert np.abs(edges - want_edges).max() <= 2.0 ** -20 * scale, (kind, columns)
+        assert np.abs(want_edges).max() > 10
+    with pytest.raises(splash_amd.SplashError):      # a draft's tokens lie in its vocabulary
+        ops.DraftSelector.add_candidates(graph, backend.from_array(logits), backend.from_array(hidden), scratch, *out,
+                                         backend.from_array(before), backend.from_array(after), 10, 5, 8193, [0])
+    with pytest.raises(splash_amd.SplashError):      # more columns than the selector's shards hold
+        ops.DraftSelector.add_candidates(graph, backend.from_array(logits), backend.from_array(hidden), scratch, *out,
+                                         backend.from_array(before), backend.from_array(after), 600000, 600000, 600000, [0])
+
+
+def _padded(codebook, vocabulary):
+    """A codebook of `vocabulary` rows whose rows past the given ones repeat them."""
+    rows = codebook.shape[0]
+    return codebook if rows == vocabulary else codebook[np.arange(vocabulary) % rows]

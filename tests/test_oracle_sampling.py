@@ -351,3 +351,39 @@ def test_verify_rows_layout_against_a_sort_and_a_recursive_preorder():
                 assert int(tree[first + at]["depth"]) == int(tree[first + up]["depth"]) + 1
         used = int(lane_rows[-1][0] + lane_rows[-1][1])
         assert np.all(sources[used:] == orc.NO_TOKEN) and np.all(tree[used:]["ancestors"] == 0)
+
+
+def test_draft_candidates_are_the_sorted_heads_of_the_rows():
+    """orc_draft_candidates against a lexicographic sort (logit descending, column ascending): plain rows, rows of few
+    distinct values with signed zeros, rows with fewer finite columns than candidates, fewer columns than candidates, and a
+    draft vocabulary that skips a range of the target's tokens."""
+    from tests.draft_case import candidates_by_sorting, proposal_logits
+    rng = np.random.default_rng(71)
+    for kind, columns, leading, trailing in [("plain", 5000, 5000, 5000), ("tied", 3000, 1000, 4000), ("sparse", 20000, 12000, 13000),
+                                             ("plain", 9, 4, 10), ("tied", 40, 0, 7)]:
+        lanes = int(rng.integers(1, 4))
+        logits = proposal_logits(rng, lanes, columns, kind)
+        got = orc.draft_candidates(logits, lanes, leading, trailing)
+        want = candidates_by_sorting(logits, lanes, leading, trailing)
+        assert np.array_equal(got[0], want[0]), kind
+        assert np.array_equal(got[1].view(np.uint32), want[1].view(np.uint32)), kind   # signed zeros as the row holds them
+
+
+def test_draft_edges_are_the_trilinear_sums():
+    """orc_draft_edges against the fp64 einsum of the decoded factors: each of the 256 products is rounded to fp32 once or
+    twice (2^-23 relative each), so the sums agree to 2^-22 of the sum of the products' magnitudes; position 0 scores its
+    anchor alone and a token past the vocabulary reads its last row."""
+    from tests.draft_case import bf16_bits, bf16_values, edges_by_einsum
+    rng = np.random.default_rng(72)
+    lanes, vocabulary = 2, 300
+    hidden, before, after = (bf16_bits(rng.standard_normal(shape)) for shape in ((lanes * 8, 256), (vocabulary, 256), (vocabulary, 256)))
+    candidates = rng.integers(0, vocabulary, (lanes * 7, 16)).astype(np.uint32)
+    candidates[3, 5] = 0xFFFFFFFF
+    anchors = np.array([7, 299], np.uint32)
+    got = orc.draft_edges(candidates, anchors, vocabulary, hidden, before, after)
+    want = edges_by_einsum(candidates, anchors, vocabulary, hidden, before, after)
+    written = ~np.isnan(want)
+    assert written.sum() == lanes * (16 + 6 * 256) and not got[~written].any()
+    scale = np.abs(bf16_values(hidden)).max() * np.abs(bf16_values(before)).max() * np.abs(bf16_values(after)).max() * 256
+    assert np.abs(got[written] - want[written]).max() <= 2.0 ** -22 * scale
+    assert np.abs(want[written]).max() > 10      # the scores are far from zero: a dropped factor would show
