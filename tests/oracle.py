@@ -590,3 +590,32 @@ def draft_verify_rows(tree_tokens, trees, scores, sizes, rows, lane_cap, floor=0
                               c_u32(rows), c_u32(lane_cap), c_f(floor), _p(tokens, u32p), tree.ctypes.data_as(ctypes.c_void_p),
                               _p(lane_rows, u32p), _p(sources, u32p))
     return tokens, tree, lane_rows, sources
+
+
+# ---- glue: rope tables, the sigmoid router, the shared expert's gate ----
+lib.orc_rope_tables.restype = None
+lib.orc_rope_tables.argtypes = [c_u32, u32p, c_u32, f32p, c_u32, f32p, f32p]
+lib.orc_moe_shared_weights.restype = None
+lib.orc_moe_shared_weights.argtypes = [u16p, f32p, c_u32, c_u32, f32p]
+
+
+def rope_tables(anchor, depth, invfreq):
+    depth = np.ascontiguousarray(depth, np.uint32)
+    invfreq = np.ascontiguousarray(invfreq, np.float32)
+    cosv = np.empty((len(depth), len(invfreq)), np.float32)
+    sinv = np.empty_like(cosv)
+    lib.orc_rope_tables(c_u32(anchor), _p(depth, u32p), c_u32(len(depth)), _p(invfreq, f32p), c_u32(len(invfreq)), _p(cosv, f32p),
+                        _p(sinv, f32p))
+    return cosv, sinv
+
+
+def silu(x):
+    return np.array([lib.orc_silu(float(v)) for v in np.ravel(x)], np.float32).reshape(np.shape(x))
+
+
+def moe_shared_weights(x_bits, gate):
+    x = np.ascontiguousarray(x_bits, np.uint16)
+    g = np.ascontiguousarray(gate, np.float32)
+    out = np.empty(x.shape[0], np.float32)
+    lib.orc_moe_shared_weights(_p(x, u16p), _p(g, f32p), x.shape[0], x.shape[1], _p(out, f32p))
+    return out
