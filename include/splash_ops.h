@@ -361,11 +361,15 @@ sp_status spo_dense_verify_set_layer(spo_dense_verify *verify, uint32_t layer, c
                                      sp_buffer *query_norm, sp_buffer *key_norm);
 sp_status spo_dense_verify_set_head(spo_dense_verify *verify, uint32_t embedding_format, sp_buffer *embedding_rows,
                                     sp_buffer *final_norm, const spo_projection *head);
-/* The step's buffers; each call returns a new reference (release it). `index` is the layer for KV pools. */
+/* The step's buffers; each call returns a new reference (release it). `index` is the layer for KV pools and the
+   stream (0 or 1) for the hidden rows. The last three hold what the layer that ran last left in them: its fused
+   q|k|v rows before the head norms, its attention rows before the output projection, its SwiGLU rows before the
+   down projection (what a layer-by-layer check of the step reads). */
 typedef enum spo_verify_buffer {
   SPO_VERIFY_INPUT_TOKENS = 0, SPO_VERIFY_TREE_ROWS, SPO_VERIFY_DEPTHS, SPO_VERIFY_UNIFORMS, SPO_VERIFY_TOKENS,
   SPO_VERIFY_RETAINED, SPO_VERIFY_ACCEPTED, SPO_VERIFY_RETAINED_ROWS, SPO_VERIFY_PAGE_TABLE, SPO_VERIFY_KV_POOL,
-  SPO_VERIFY_LOGITS, SPO_VERIFY_DRAFT_PROBABILITIES, SPO_VERIFY_HIDDEN
+  SPO_VERIFY_LOGITS, SPO_VERIFY_DRAFT_PROBABILITIES, SPO_VERIFY_HIDDEN,
+  SPO_VERIFY_QKV_ROWS = 15, SPO_VERIFY_ATTENTION_ROWS = 16, SPO_VERIFY_FFN_ROWS = 17
 } spo_verify_buffer;
 sp_status spo_dense_verify_buffer(spo_dense_verify *verify, spo_verify_buffer which, uint32_t index, sp_buffer **out);
 uint64_t spo_dense_verify_page_bytes(const spo_dense_verify *verify);

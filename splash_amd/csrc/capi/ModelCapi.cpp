@@ -261,6 +261,9 @@ sp_status spo_dense_verify_buffer(spo_dense_verify *verify, spo_verify_buffer wh
     case SPO_VERIFY_LOGITS: b = v.logits(); break;
     case SPO_VERIFY_DRAFT_PROBABILITIES: b = v.draftProbabilities(); break;
     case SPO_VERIFY_HIDDEN: b = v.hidden(index); break;
+    case SPO_VERIFY_QKV_ROWS: b = v.qkvRows(); break;
+    case SPO_VERIFY_ATTENTION_ROWS: b = v.attentionRows(); break;
+    case SPO_VERIFY_FFN_ROWS: b = v.ffnRows(); break;
     default: throw std::invalid_argument("no such verify buffer");
     }
     sp_buffer_retain(b.handle());

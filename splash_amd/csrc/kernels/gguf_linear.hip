@@ -490,7 +490,7 @@ template <int RT> struct DecodeShared {
   uint4 a[2][RT][8][64];
   float sums[2][RT][4][64];
   uint32_t arrived;
-  float scaleParts[256], rowScale[16 * RT];  // of a table with a deferred scale
+  float scaleParts[256 * RT], rowScale[16 * RT];  // of a table with a deferred scale
 };
 
 template <uint32_t FMT, int RT, uint32_t EP>
@@ -603,15 +603,23 @@ __device__ __forceinline__ void decode_workgroup(DecodeShared<RT> &shared, const
       for (int q = 0; q < kSumShare; ++q) sumShare[q] += kSumsPerBlock * 4u * 16u * 4u;
     };
     // Every row's inverse RMS from the squares the table's writer left, one entry a 64-column group:
-    // part q adds entries q, q + parts, ... in order, then the parts are added in order. The loads go
-    // out before the first weights', so the wait for them leaves those in flight.
-    constexpr uint32_t kRows = 16u * RT, kParts = 256u / kRows;
-    float squareSum = 0.f;
+    // part q of 16 adds entries q, q + 16, ... in order, then the 16 parts are added in order -- the same
+    // sums whatever the kernel's row tiles, so a row's result does not depend on the block's height. A
+    // thread takes RT parts of its row. The loads go out before the first weights', so the wait for
+    // them leaves those in flight.
+    constexpr uint32_t kRows = 16u * RT, kParts = 16u, kThreadParts = 256u / kRows;
+    float squareSum[RT];
+#pragma unroll
+    for (int i = 0; i < RT; ++i) squareSum[i] = 0.f;
     if (p.deferred_scale) {
       const float *squares = reinterpret_cast<const float *>(table + gguf_table_squares_offset(p.input_size, tiles));
-      const uint32_t row = threadIdx.x % kRows, part = threadIdx.x / kRows, entries = p.input_size / 64u;
-      if (row < 16u * tiles)
-        for (uint32_t j = part; j < entries; j += kParts) squareSum += squares[size_t(j) * 16u * tiles + row];
+      const uint32_t row = threadIdx.x % kRows, entries = p.input_size / 64u;
+      if (row < 16u * tiles) {
+#pragma unroll
+        for (int i = 0; i < RT; ++i)
+          for (uint32_t j = threadIdx.x / kRows + kThreadParts * i; j < entries; j += kParts)
+            squareSum[i] += squares[size_t(j) * 16u * tiles + row];
+      }
       __builtin_amdgcn_sched_barrier(0);
     }
 #pragma unroll
@@ -621,7 +629,8 @@ __device__ __forceinline__ void decode_workgroup(DecodeShared<RT> &shared, const
       __builtin_amdgcn_sched_barrier(0);
     }
     if (p.deferred_scale) {
-      scaleParts[threadIdx.x] = squareSum;
+#pragma unroll
+      for (int i = 0; i < RT; ++i) scaleParts[256u * i + threadIdx.x] = squareSum[i];   // part (threadIdx.x / kRows + kThreadParts i) of row threadIdx.x % kRows
       __syncthreads();
       if (threadIdx.x < kRows) {
         float total = 0.f;

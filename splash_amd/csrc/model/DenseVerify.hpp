@@ -71,6 +71,9 @@ public:
   [[nodiscard]] const hip::Buffer &logits() const noexcept { return logits_; }
   [[nodiscard]] const hip::Buffer &draftProbabilities();  // allocated on first use
   [[nodiscard]] const hip::Buffer &hidden(uint32_t index) const noexcept { return hidden_[index & 1]; }
+  [[nodiscard]] const hip::Buffer &qkvRows() const noexcept { return qkv_; }
+  [[nodiscard]] const hip::Buffer &attentionRows() const noexcept { return attention_; }
+  [[nodiscard]] const hip::Buffer &ffnRows() const noexcept { return intermediate_; }
   [[nodiscard]] uint64_t pageBytes() const noexcept { return pageBytes_; }
   // Algorithmic bytes one step of `lanes` streams from HBM: weights once, each lane's KV, logits.
   [[nodiscard]] uint64_t stepBytes(const std::vector<VerifyLane> &lanes) const;

@@ -11,7 +11,7 @@ from .backend import Buffer, CommandGraph, STORAGE_PRIVATE
 from . import ops
 
 (INPUT_TOKENS, TREE_ROWS, DEPTHS, UNIFORMS, TOKENS, RETAINED, ACCEPTED, RETAINED_ROWS, PAGE_TABLE, KV_POOL, LOGITS,
- DRAFT_PROBABILITIES, HIDDEN, GDN_STATES, GDN_TAPE) = range(15)
+ DRAFT_PROBABILITIES, HIDDEN, GDN_STATES, GDN_TAPE, QKV_ROWS, ATTENTION_ROWS, FFN_ROWS) = range(18)
 
 
 class Lane:

@@ -36,7 +36,8 @@ def build_context(rng, backend, q_heads, kv_heads, D, rows, committed, extra_pag
     return kv, (kc, ks, vc, vs), table
 
 
-def run_block(backend, rng, q_heads, kv_heads, D, rows, committed, pairs=0, normalize=False, ancestors=None):
+def run_block(backend, rng, q_heads, kv_heads, D, rows, committed, pairs=0, normalize=False, ancestors=None, oracle_kv_heads=None):
+    """oracle_kv_heads: the KV heads the oracle evaluates (all by default); `got` then holds their query heads only."""
     kv, logical, table = build_context(rng, backend, q_heads, kv_heads, D, rows, committed)
     kc, ks, vc, vs = (a.copy() for a in logical)
     width = (q_heads + 2 * kv_heads) * D
@@ -70,7 +71,14 @@ def run_block(backend, rng, q_heads, kv_heads, D, rows, committed, pairs=0, norm
         p, s = table[t // ops.PAGE_TOKENS], t % ops.PAGE_TOKENS
         kc[p, :, s], ks[p, :, s], vc[p, :, s], vs[p, :, s] = kcod[r], kscl[r], vcod[r], vscl[r]
     anc = tree["ancestors"].astype(np.uint32)
-    want, want64 = orc.attention(q, kc, ks, vc, vs, table, anc, committed)
+    if oracle_kv_heads is not None:
+        group = q_heads // kv_heads
+        mine = np.concatenate([np.arange(h * group, (h + 1) * group) for h in oracle_kv_heads])
+        sub = lambda a: np.ascontiguousarray(a[:, list(oracle_kv_heads)])
+        want, want64 = orc.attention(np.ascontiguousarray(q[:, mine]), sub(kc), sub(ks), sub(vc), sub(vs), table, anc, committed)
+        got = got[:, mine]
+    else:
+        want, want64 = orc.attention(q, kc, ks, vc, vs, table, anc, committed)
     stored = kv.unpack_pages(kv.download())
     return got, want, want64, stored, (kc, ks, vc, vs), table, plan
 
@@ -111,6 +119,23 @@ def test_tree_rows_and_resubmission(backend):
     rng = np.random.default_rng(4)
     again, *_ = run_block(backend, rng, 64, 8, 128, rows, committed, ancestors=anc)
     assert np.array_equal(got, again)
+
+
+@pytest.mark.parametrize("context,heads", [(8192, None), (131072, (1, 6))])
+def test_config3_contexts_of_8k_and_128k(backend, context, heads):
+    """BASELINE.json config 3's other contexts at its geometry (64 q / 8 kv heads x 128, a 16-row chain block ending the
+    context, permuted page table), with the head norms and RoPE of the step; at 128K the oracle evaluates two of the
+    eight KV heads (16 of the 64 query heads), the GPU all of them. The attention's gate: cosine >= 0.9999 and max-abs
+    < 0.02 against the fp64 softmax over the stored INT8 pages."""
+    print(f"case attention config 3 context={context}", flush=True)
+    rng = np.random.default_rng(context)
+    got, want, want64, _, _, _, plan = run_block(backend, rng, 64, 8, 128, 16, context - 16, pairs=64, normalize=True,
+                                                 oracle_kv_heads=heads)
+    assert got.shape[1] == (64 if heads is None else 8 * len(heads))
+    cos, err = tolerance(got, want64)
+    assert cos >= 0.9999 and err < 0.02, (cos, err)
+    cos2, err2 = tolerance(got, orc.bf16_to_f32(want).astype(np.float64))
+    assert cos2 >= 0.9999 and err2 < 0.02, (cos2, err2)
 
 
 def test_long_context_32k(backend):
