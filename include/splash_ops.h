@@ -312,6 +312,18 @@ sp_status spo_sampling_add_acceptance(spo_graph *graph, sp_buffer *input_tokens,
                                       sp_buffer *retained, sp_buffer *accepted_count, sp_buffer *retained_rows,
                                       const spo_lane_rows *lanes, const uint32_t *remaining, uint32_t count,
                                       const uint32_t stop_tokens[4]);
+/* No counterpart in the reference. For callers that cannot allocate device memory or a workspace (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc): the greedy selection of spo_sampling_add_verify --
+ * every row's largest logit, the lower id among equals, NaN and -infinity never, 0xFFFFFFFF for a row with no
+ * selectable logit -- launched directly on `stream` (a hipStream_t; NULL is the null stream) over device pointers:
+ * logits fp32 [rows][logits_stride], tokens uint32 [rows]. The shards' partial results live in a device array of the
+ * library (64 KiB a GPU, held until the process ends) instead of a workspace argument: the call allocates nothing,
+ * frees nothing and returns once its two kernels are launched. At most SPO_SAMPLING_STATIC_MAXIMUM_ROWS rows a call
+ * (more is SP_INVALID_ARGUMENT). Every call on one GPU shares that GPU's array: calls that overlap on one GPU
+ * (different streams, or threads) race; calls in stream order on one stream do not. */
+#define SPO_SAMPLING_STATIC_MAXIMUM_ROWS 256u
+sp_status spo_sampling_greedy_rows_static(const float *logits, uint32_t rows, uint32_t vocabulary, uint32_t logits_stride,
+                                          uint32_t *tokens, void *stream);
 
 /* ---- DraftSelector::addVerifyRows (runtime/ops/DraftSelector.hpp:139-147; StepRows, LaneRows.hpp:49-67): a decode
  *      step's rows from the trees a draft selector grew. Each lane's tree holds tree_sizes[lane] rows of 16 (tokens,

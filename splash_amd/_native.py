@@ -276,6 +276,7 @@ _sig("spo_sampling_add_penalties", c_int, c_p, c_p, c_p, c_p, c_p, c_u32, c_u32,
 _sig("spo_sampling_add_thinking_cutoff", c_int, c_p, c_p, c_p, c_u32, c_p, c_p, c_u32, P(LaneRows), P(ThinkingCutoff), c_u32)
 _sig("spo_draft_add_verify_rows", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_u32, c_u32, c_u32, ctypes.c_float)
 _sig("spo_sampling_add_acceptance", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, P(LaneRows), P(c_u32), c_u32, P(c_u32))
+_sig("spo_sampling_greedy_rows_static", c_int, ctypes.c_void_p, c_u32, c_u32, c_u32, ctypes.c_void_p, ctypes.c_void_p)
 _sig("spg_dense_dimensions", c_int, c_p, P(DenseDimensions))
 _sig("spo_dense_verify_load_gguf", c_int, c_p, c_p)
 _sig("spo_dense_verify_create", c_int, c_p, P(DenseDimensions), c_u32, c_u32, c_u32, P(c_p))

@@ -705,3 +705,80 @@ __global__ __launch_bounds__(64) void decode_sample_draw(const float *__restrict
 SP_REGISTER_KERNEL("decode_sample_draw", &decode_sample_draw);
 
 } // namespace splash::kernels
+
+// ---- Greedy selection of packed logits rows without any allocation ------------------------------
+// spo_sampling_greedy_rows_static (include/splash_ops.h) is the argmax pair above for callers that
+// cannot allocate: the shards' partials live in a file-scope device array instead of a workspace.
+// Host code never uses the array's name as an address: each device's copy is looked up once with
+// hipGetSymbolAddress and that pointer is what the kernels get.
+#include "backend/Internal.hpp"
+#include "splash_ops.h"
+
+#include <hip/hip_runtime.h>
+#include <mutex>
+
+namespace splash::kernels {
+namespace {
+
+struct GreedyPartial {
+  float value;
+  uint32_t index;
+};
+constexpr uint32_t kStaticRows = SPO_SAMPLING_STATIC_MAXIMUM_ROWS;
+constexpr int kMaximumDevices = 64;
+static __device__ __align__(256) unsigned char scratch[kStaticRows * SAMPLING_SHARDS * sizeof(GreedyPartial)];
+
+std::mutex scratchMutex;
+void *scratchOfDevice[kMaximumDevices];  // each device holds its own copy of the array, at its own address
+
+// The current device's copy of the scratch array (looked up on the device's first call).
+hipError_t deviceScratch(void **out) {
+  int device = -1;
+  hipError_t status = hipGetDevice(&device);
+  if (status != hipSuccess) return status;
+  if (device < 0 || device >= kMaximumDevices) return hipErrorInvalidDevice;
+  std::lock_guard<std::mutex> lock(scratchMutex);
+  if (!scratchOfDevice[device]) {
+    void *address = nullptr;
+    status = hipGetSymbolAddress(&address, HIP_SYMBOL(scratch));
+    if (status != hipSuccess) return status;
+    scratchOfDevice[device] = address;
+  }
+  *out = scratchOfDevice[device];
+  return hipSuccess;
+}
+
+} // namespace
+} // namespace splash::kernels
+
+extern "C" sp_status spo_sampling_greedy_rows_static(const float *logits, uint32_t rows, uint32_t vocabulary, uint32_t logits_stride,
+                                                     uint32_t *tokens, void *stream) {
+  using namespace splash::kernels;
+  auto fail = [](sp_status code, const std::string &message) {
+    splash::hipbackend::setLastError(message);
+    return code;
+  };
+  if (!logits || !tokens) return fail(SP_INVALID_ARGUMENT, "null logits or tokens");
+  if (!rows || rows > kStaticRows)
+    return fail(SP_INVALID_ARGUMENT, "the static greedy selection takes 1 to " + std::to_string(kStaticRows) + " rows");
+  if (!vocabulary || logits_stride < vocabulary) return fail(SP_INVALID_ARGUMENT, "a logits row holds its vocabulary");
+  void *memory = nullptr;
+  hipError_t status = deviceScratch(&memory);
+  if (status != hipSuccess) return fail(SP_BACKEND_ERROR, std::string("hipGetSymbolAddress: ") + hipGetErrorString(status));
+  // Every (row, shard) partial of this call is written by the first kernel before the second reads
+  // it, so nothing of an earlier call's contents is read and nothing needs clearing.
+  float *values = static_cast<float *>(memory);
+  uint32_t *indices = reinterpret_cast<uint32_t *>(values + size_t(kStaticRows) * SAMPLING_SHARDS);
+  TargetSamplingParams p{};
+  p.vocabulary = vocabulary;
+  p.rows = rows;
+  p.lanes = 1;
+  p.logits_stride = logits_stride;
+  p.lane[0] = SamplingLaneRows{0, rows};
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  hipLaunchKernelGGL(decode_sample_argmax_sharded, dim3(rows * SAMPLING_SHARDS), dim3(256), 0, s, logits, values, indices, p);
+  hipLaunchKernelGGL(decode_sample_argmax_reduce, dim3(rows), dim3(64), 0, s, values, indices, tokens, p);
+  status = hipGetLastError();
+  if (status != hipSuccess) return fail(SP_BACKEND_ERROR, std::string("launch: ") + hipGetErrorString(status));
+  return SP_OK;
+}

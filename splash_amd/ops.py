@@ -521,6 +521,15 @@ class Sampling:
         check(lib.spo_sampling_add_verify(graph.handle, ctypes.byref(b), vocabulary, stride, arr, structs, len(lanes), stops))
         graph._keep.extend([v for k, v in buffers.items() if k != "mask_words"])
 
+    STATIC_MAXIMUM_ROWS = 256
+
+    @staticmethod
+    def greedy_rows_static(logits, rows, vocabulary, stride, tokens, stream=None):
+        """spo_sampling_greedy_rows_static: every row's greedy selection, launched on `stream` (a hipStream_t as an
+        integer; None is the null stream) with no allocation; logits and tokens are device Buffers. Returns once
+        the kernels are launched: the caller synchronizes the stream."""
+        check(lib.spo_sampling_greedy_rows_static(logits.gpu_address, rows, vocabulary, stride, tokens.gpu_address, stream))
+
     @staticmethod
     def add_acceptance(graph, input_tokens, tree_rows, tokens, retained, accepted, retained_rows, lanes, remaining,
                        stop_tokens=(NO_TOKEN,) * 4):
