@@ -394,6 +394,20 @@ sp_status spo_dense_verify_encode(spo_dense_verify *verify, spo_graph *graph, co
 sp_status spo_dense_verify_encode_part(spo_dense_verify *verify, spo_graph *graph, uint32_t part, uint32_t index,
                                        const spo_verify_lane *lanes, uint32_t count);
 
+/* A completed step's results, checked as Runtime::finalizeDecode checks them before a lane commits (Runtime.cpp:2943-2972,
+ * invalidSelection :1559-1582): per lane 1 <= retained <= min(rows, remaining), popcount(retained_rows) == retained with
+ * bit 0 set and no bit at or past the lane's rows, accepted < rows and <= retained, every retained token below
+ * `vocabulary`. SP_BACKEND_ERROR with the lane and the rule in sp_last_error() otherwise. Host arrays only: lanes[i]
+ * gives lane i's first packed row and its rows, tokens holds the step's packed rows. */
+sp_status spo_verify_check_results(const spo_lane_rows *lanes, const uint32_t *remaining, uint32_t count, uint32_t step_rows,
+                                   uint32_t vocabulary, const uint32_t *tokens, const uint32_t *retained, const uint32_t *accepted,
+                                   const uint32_t *retained_rows);
+/* Reads a completed step's results out of the driver's buffers (call after the command's ticket has been waited for),
+ * checks them as spo_verify_check_results does, and copies them: tokens uint32 [the lanes' rows, packed], the others
+ * uint32 [count]. */
+sp_status spo_dense_verify_results(spo_dense_verify *verify, const spo_verify_lane *lanes, uint32_t count, uint32_t *tokens,
+                                   uint32_t *retained, uint32_t *accepted, uint32_t *retained_rows);
+
 /* ---- The hybrid mixture-of-experts verify step (the reference's Qwen3.5 target with Gated
  *      DeltaNet mixers: QwenTarget.cpp:206-255 the GDN mixer, :263-347 the attention mixer, :372-395
  *      the MoE routing, :457-496 the layer recipe; Runtime.cpp:2701-2707 tape parity and pending
@@ -435,6 +449,9 @@ sp_status spo_hybrid_verify_set_head(spo_hybrid_verify *verify, uint32_t embeddi
 #define SPO_VERIFY_GDN_STATES 13
 #define SPO_VERIFY_GDN_TAPE 14
 sp_status spo_hybrid_verify_buffer(spo_hybrid_verify *verify, uint32_t which, uint32_t index, sp_buffer **out);
+/* As spo_dense_verify_results. */
+sp_status spo_hybrid_verify_results(spo_hybrid_verify *verify, const spo_hybrid_lane *lanes, uint32_t count, uint32_t *tokens,
+                                    uint32_t *retained, uint32_t *accepted, uint32_t *retained_rows);
 /* Where the recurrent state lives: a lane's cell of a parity at (lane * 2 + parity) * cell_bytes in the
  * states buffer (strides as spo_gdn_layout gives them for the model's GDN layers), GDN layer g's tape of
  * a lane's step of a parity at ((lane * 2 + parity) * gdn_layers + g) * tape_layer_bytes in the tape buffer. */

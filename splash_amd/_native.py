@@ -277,6 +277,8 @@ _sig("spo_sampling_add_thinking_cutoff", c_int, c_p, c_p, c_p, c_u32, c_p, c_p, 
 _sig("spo_draft_add_verify_rows", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_u32, c_u32, c_u32, ctypes.c_float)
 _sig("spo_sampling_add_acceptance", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, P(LaneRows), P(c_u32), c_u32, P(c_u32))
 _sig("spo_sampling_greedy_rows_static", c_int, ctypes.c_void_p, c_u32, c_u32, c_u32, ctypes.c_void_p, ctypes.c_void_p)
+_sig("spo_verify_check_results", c_int, P(LaneRows), P(c_u32), c_u32, c_u32, c_u32, P(c_u32), P(c_u32), P(c_u32), P(c_u32))
+_sig("spo_dense_verify_results", c_int, c_p, P(VerifyLane), c_u32, P(c_u32), P(c_u32), P(c_u32), P(c_u32))
 _sig("spg_dense_dimensions", c_int, c_p, P(DenseDimensions))
 _sig("spo_dense_verify_load_gguf", c_int, c_p, c_p)
 _sig("spo_dense_verify_create", c_int, c_p, P(DenseDimensions), c_u32, c_u32, c_u32, P(c_p))
@@ -297,6 +299,7 @@ _sig("spo_hybrid_verify_layout", c_int, c_p, P(c_u64), P(c_u64), P(c_u64), P(Gdn
 _sig("spo_hybrid_verify_step_bytes", c_u64, c_p, P(HybridLane), c_u32)
 _sig("spo_hybrid_verify_encode", c_int, c_p, c_p, P(HybridLane), c_u32, c_int)
 _sig("spo_hybrid_verify_encode_part", c_int, c_p, c_p, c_u32, c_u32, P(HybridLane), c_u32)
+_sig("spo_hybrid_verify_results", c_int, c_p, P(HybridLane), c_u32, P(c_u32), P(c_u32), P(c_u32), P(c_u32))
 
 
 # ---- GGUF files (include/splash_gguf.h) ----

@@ -3,6 +3,7 @@
 #include "capi/Guard.hpp"
 #include "capi/Handles.hpp"
 #include "model/HybridVerify.hpp"
+#include "model/StepResults.hpp"
 
 #include <memory>
 
@@ -105,6 +106,18 @@ sp_status spo_hybrid_verify_set_head(spo_hybrid_verify *verify, uint32_t embeddi
     w.finalNorm = B(final_norm);
     w.head = capi::projectionOf(head);
     w.head.destination = ops::FloatOutput::Float32;
+  });
+}
+sp_status spo_hybrid_verify_results(spo_hybrid_verify *verify, const spo_hybrid_lane *lanes, uint32_t count, uint32_t *tokens,
+                                    uint32_t *retained, uint32_t *accepted, uint32_t *retained_rows) {
+  return capi::guard([&] {
+    capi::require(verify && lanes && count && tokens && retained && accepted && retained_rows, "verify, lanes or results");
+    model::HybridVerify &v = *verify->verify;
+    std::vector<model::StepLane> list;
+    uint32_t first = 0;
+    for (uint32_t i = 0; i < count; ++i) { list.push_back({first, lanes[i].block.rows, lanes[i].block.remaining}); first += lanes[i].block.rows; }
+    model::readStepResults(list, v.tokens(), v.retained(), v.acceptedCount(), v.retainedRows(), v.dimensions().vocabulary, tokens, retained,
+                           accepted, retained_rows);
   });
 }
 sp_status spo_hybrid_verify_buffer(spo_hybrid_verify *verify, uint32_t which, uint32_t index, sp_buffer **out) {

@@ -3,6 +3,7 @@
 #include "capi/Guard.hpp"
 #include "capi/Handles.hpp"
 #include "model/DenseVerify.hpp"
+#include "model/StepResults.hpp"
 #include "model/GgufTarget.hpp"
 #include "splash_gguf.h"
 #include "ops/DraftSelector.hpp"
@@ -268,6 +269,33 @@ sp_status spo_dense_verify_buffer(spo_dense_verify *verify, spo_verify_buffer wh
     }
     sp_buffer_retain(b.handle());
     *out = b.handle();
+  });
+}
+sp_status spo_verify_check_results(const spo_lane_rows *lanes, const uint32_t *remaining, uint32_t count, uint32_t step_rows,
+                                   uint32_t vocabulary, const uint32_t *tokens, const uint32_t *retained, const uint32_t *accepted,
+                                   const uint32_t *retained_rows) {
+  return capi::guard([&] {
+    capi::require(lanes && count && tokens && retained && accepted && retained_rows, "lanes or results");
+    std::vector<model::StepLane> list;
+    std::vector<model::StepLaneResult> results;
+    for (uint32_t i = 0; i < count; ++i) {
+      list.push_back({lanes[i].first, lanes[i].rows, remaining ? remaining[i] : 0xFFFFFFFFu});
+      if (uint64_t{lanes[i].first} + lanes[i].rows > step_rows) throw hip::BackendError("lane " + std::to_string(i) + ": its rows are not rows of the step");
+      results.push_back({retained[i], accepted[i], retained_rows[i], tokens + lanes[i].first});
+    }
+    model::validateStepResults(list, results, step_rows, vocabulary);
+  });
+}
+sp_status spo_dense_verify_results(spo_dense_verify *verify, const spo_verify_lane *lanes, uint32_t count, uint32_t *tokens,
+                                   uint32_t *retained, uint32_t *accepted, uint32_t *retained_rows) {
+  return capi::guard([&] {
+    capi::require(verify && tokens && retained && accepted && retained_rows, "verify or results");
+    model::DenseVerify &v = *verify->verify;
+    std::vector<model::StepLane> list;
+    uint32_t first = 0;
+    for (const model::VerifyLane &l : lanesOf(lanes, count)) { list.push_back({first, l.rows, l.remaining}); first += l.rows; }
+    model::readStepResults(list, v.tokens(), v.retained(), v.acceptedCount(), v.retainedRows(), v.dimensions().vocabulary, tokens, retained,
+                           accepted, retained_rows);
   });
 }
 uint64_t spo_dense_verify_page_bytes(const spo_dense_verify *verify) { return verify ? verify->verify->pageBytes() : 0; }

@@ -71,8 +71,22 @@ struct Loader {
 
 } // namespace
 
+// The architectures whose dense decoder tensors, head geometry and RoPE pairing (dimension i with i + pairs, GGML's
+// "neox" rotation) these kernels compute: the Qwen families the reference targets (requireMetadata,
+// runtime/model/GgufImage.cpp:874-916, takes its model's own architecture and nothing else). A llama-architecture
+// file permutes its query and key rows for the interleaved rotation: it would load and give wrong logits.
+bool denseArchitecture(const std::string &name) {
+  static const std::set<std::string> known = {"qwen2", "qwen3", "qwen35"};
+  return known.count(name) != 0;
+}
+
 DenseDimensions ggufDenseDimensions(const GgufFile &file) {
-  const std::string a = architectureOf(file) + ".";
+  const std::string name = architectureOf(file);
+  if (!denseArchitecture(name))
+    throw GgufError("GGUF architecture " + name + " is not one the dense driver computes (qwen2, qwen3, qwen35)");
+  const std::string a = name + ".";
+  // What the metadata names and the kernels do not do, collected so that one error names all of it.
+  Problems problems;
   DenseDimensions d;
   d.layers = requireUnsigned(file, a + "block_count");
   d.hidden = requireUnsigned(file, a + "embedding_length");
@@ -82,13 +96,18 @@ DenseDimensions ggufDenseDimensions(const GgufFile &file) {
   const std::optional<uint64_t> keyLength = file.metadata().unsignedValue(a + "attention.key_length");
   d.headDimension = keyLength ? uint32_t(*keyLength) : d.hidden / d.qHeads;
   const std::optional<uint64_t> valueLength = file.metadata().unsignedValue(a + "attention.value_length");
-  if (valueLength && *valueLength != d.headDimension) throw GgufError("keys and values of different lengths are not supported");
+  if (valueLength && *valueLength != d.headDimension) problems.add("keys and values of different lengths are not supported");
   const std::optional<uint64_t> rotary = file.metadata().unsignedValue(a + "rope.dimension_count");
-  if (rotary && *rotary != d.headDimension) throw GgufError("a partial rotary embedding is not supported by the dense driver");
+  if (rotary && *rotary != d.headDimension) problems.add("a partial rotary embedding is not supported by the dense driver");
   d.rotaryPairs = d.headDimension / 2;
-  d.ropeTheta = float(file.metadata().floatValue(a + "rope.freq_base").value_or(10000.0));
+  const std::optional<double> base = file.metadata().floatValue(a + "rope.freq_base");
+  if (!base || !(*base > 0)) problems.add("GGUF metadata lacks " + a + "rope.freq_base");
+  d.ropeTheta = float(base.value_or(0.0));
+  if (const std::optional<std::string> scaling = file.metadata().stringValue(a + "rope.scaling.type"); scaling && *scaling != "none")
+    problems.add("rope.scaling.type " + *scaling + " is not computed (expected none)");
   const double epsilon = file.metadata().floatValue(a + "attention.layer_norm_rms_epsilon").value_or(1e-6);
-  if (std::fabs(epsilon - 1e-6) > 1e-12) throw GgufError("the norms' epsilon is 1e-6 in these kernels; the file names another");
+  if (std::fabs(epsilon - 1e-6) > 1e-12) problems.add("the norms' epsilon is 1e-6 in these kernels; the file names another");
+  if (!problems.text.empty()) throw GgufError("GGUF metadata this build cannot follow: " + problems.text);
   const GgufTensor &table = file.require("token_embd.weight");
   if (table.dims.size() != 2 || table.dims[0] != d.hidden) throw GgufError("token_embd.weight is not vocabulary x hidden");
   d.vocabulary = uint32_t(table.dims[1]);

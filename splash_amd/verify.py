@@ -104,12 +104,18 @@ class DenseVerify:
         if uniforms is not None:
             self.buffer(UNIFORMS).contents()[:rows * 8] = np.asarray(uniforms, dtype=np.float32).reshape(rows, 2).view(np.uint8).ravel()
 
+    _results_call = "spo_dense_verify_results"
+
     def results(self, lanes):
-        """(selected/retained tokens per packed row, retained count, accepted count, retained-row mask) per lane."""
-        rows = sum(l.rows for l in lanes)
-        n = len(lanes)
-        rd = lambda which, count: self.buffer(which).contents()[:count * 4].view(np.uint32).copy()
-        return rd(TOKENS, rows), rd(RETAINED, n), rd(ACCEPTED, n), rd(RETAINED_ROWS, n)
+        """(selected/retained tokens per packed row, retained count, accepted count, retained-row mask) per lane, read
+        from the driver's buffers after the step's command completed and checked as Runtime::finalizeDecode checks them
+        (a SplashError names the lane and the rule a result breaks)."""
+        rows, n = sum(l.rows for l in lanes), len(lanes)
+        tokens = np.zeros(rows, np.uint32)
+        retained, accepted, mask = (np.zeros(n, np.uint32) for _ in range(3))
+        p = lambda a: a.ctypes.data_as(ctypes.POINTER(ctypes.c_uint32))
+        check(getattr(lib, self._results_call)(self.handle, self._lanes(lanes), n, p(tokens), p(retained), p(accepted), p(mask)))
+        return tokens, retained, accepted, mask
 
 
 class HybridLane(Lane):
@@ -212,3 +218,15 @@ class HybridVerify:
 
     set_block = DenseVerify.set_block
     results = DenseVerify.results
+    _results_call = "spo_hybrid_verify_results"
+
+
+def check_results(lanes, tokens, retained, accepted, retained_rows, vocabulary, remaining=None, step_rows=None):
+    """spo_verify_check_results over host arrays: lanes [(first, rows)]."""
+    arr = (nat.LaneRows * len(lanes))(*[nat.LaneRows(*l) for l in lanes])
+    u32 = lambda a: np.ascontiguousarray(a, np.uint32)
+    tokens, retained, accepted, retained_rows = u32(tokens), u32(retained), u32(accepted), u32(retained_rows)
+    rem = u32(remaining) if remaining is not None else None
+    p = lambda a: a.ctypes.data_as(ctypes.POINTER(ctypes.c_uint32)) if a is not None else None
+    rows = step_rows if step_rows is not None else len(tokens)
+    check(lib.spo_verify_check_results(arr, p(rem), len(lanes), rows, vocabulary, p(tokens), p(retained), p(accepted), p(retained_rows)))

@@ -117,7 +117,7 @@ def test_projections_and_norms_load_from_a_file(backend, tmp_path):
         f.load_bf16(backend, f.find("output.weight"))
 
 
-def dense_model_file(path, model, value_format, tied, extra=(), skip=()):
+def dense_model_file(path, model, value_format, tied, extra=(), skip=(), more_metadata=()):
     """A dense decoder's GGUF as llama.cpp names its tensors: blk.N.attn_q / attn_k / attn_v (the values requantized to
     `value_format`, as a Q4_K_M file keeps them) ..., norms as F32, the token table, and the head unless tied."""
     d = model.dims
@@ -146,7 +146,7 @@ def dense_model_file(path, model, value_format, tied, extra=(), skip=()):
                 ("qwen3.attention.head_count", gw.U32, d["q_heads"]), ("qwen3.attention.head_count_kv", gw.U32, d["kv_heads"]),
                 ("qwen3.attention.key_length", gw.U32, D), ("qwen3.attention.value_length", gw.U32, D),
                 ("qwen3.attention.layer_norm_rms_epsilon", gw.F32, 1e-6), ("qwen3.rope.freq_base", gw.F32, model.rope_theta)]
-    gw.write_gguf(path, metadata, tensors)
+    gw.write_gguf(path, metadata + list(more_metadata), tensors)
 
 
 @pytest.mark.gpu
@@ -228,10 +228,31 @@ def test_dense_geometry_from_metadata(tmp_path):
     assert (d.hidden, d.q_heads, d.kv_heads, d.head_dim, d.ffn, d.vocabulary, d.layers, d.rotary_pairs, d.normalize_heads, d.rope_theta) == \
         (256, 4, 2, 64, 256, 256, 1, 32, 1, 5e5)
     raw = open(path, "rb").read()
-    for name, edit in (("key", lambda b: b.replace(b"qwen3.block_count", b"qwen3.block_coumt")),
-                       ("architecture", lambda b: b.replace(b"general.architecture", b"general.architectura"))):
+    # Same-length byte edits of the file: a key that is no longer there, an architecture whose rows are laid out for
+    # another rotation (llama: interleaved pairs), a missing RoPE base; each is refused with a message that names it.
+    for name, edit, message in (("key", lambda b: b.replace(b"qwen3.block_count", b"qwen3.block_coumt"), "block_count"),
+                                ("architecture", lambda b: b.replace(b"general.architecture", b"general.architectura"), "architecture"),
+                                ("llama", lambda b: b.replace(b"qwen3", b"llama"), "llama is not one the dense driver computes"),
+                                ("base", lambda b: b.replace(b"qwen3.rope.freq_base", b"qwen3.rope.freq_bass"), "rope.freq_base")):
         bad = tmp_path / f"{name}.gguf"
         open(bad, "wb").write(edit(raw))
         broken = gguf.GgufFile(bad)
-        with pytest.raises(splash_amd.SplashError):
+        with pytest.raises(splash_amd.SplashError, match=message):
             splash_amd.check(splash_amd.lib.spg_dense_dimensions(broken.handle, ctypes.byref(d)))
+    # a long-context file (YaRN or linear RoPE scaling) has no tensor the loader would miss: its metadata refuses it,
+    # and one error names everything the metadata asks for that the kernels do not do
+    for scaling, refused in (("none", False), ("yarn", True), ("linear", True)):
+        scaled = tmp_path / f"{scaling}.gguf"
+        dense_model_file(scaled, model, orc.FMT_Q4K, tied=True, more_metadata=[("qwen3.rope.scaling.type", gw.STRING, scaling)])
+        g = gguf.GgufFile(scaled)
+        if refused:
+            with pytest.raises(splash_amd.SplashError, match=f"rope.scaling.type {scaling}"):
+                splash_amd.check(splash_amd.lib.spg_dense_dimensions(g.handle, ctypes.byref(d)))
+        else:
+            splash_amd.check(splash_amd.lib.spg_dense_dimensions(g.handle, ctypes.byref(d)))
+    both = tmp_path / "both.gguf"
+    dense_model_file(both, model, orc.FMT_Q4K, tied=True, more_metadata=[("qwen3.rope.scaling.type", gw.STRING, "yarn"),
+                                                                         ("qwen3.rope.dimension_count", gw.U32, 32)])
+    g = gguf.GgufFile(both)
+    with pytest.raises(splash_amd.SplashError, match="partial rotary.*rope.scaling.type yarn"):
+        splash_amd.check(splash_amd.lib.spg_dense_dimensions(g.handle, ctypes.byref(d)))
