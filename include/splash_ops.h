@@ -277,36 +277,6 @@ typedef struct spo_sampling_policy {
 sp_status spo_sampling_add_verify(spo_graph *graph, const spo_sampling_buffers *buffers, uint32_t vocabulary,
                                   uint32_t logits_stride, const spo_lane_rows *lanes, const spo_sampling_policy *policies,
                                   uint32_t count, const uint32_t *stop_tokens);
-/* ops::SamplingPenalties (Sampling.hpp:17-29) of one lane and the row of the penalty table it reads. */
-typedef struct spo_sampling_penalties {
-  float repetition, presence, frequency; /* 1, 0, 0 change nothing */
-  uint32_t table_row;
-} spo_sampling_penalties;
-/* Sampling::rebuildPenaltyWords / countPenaltyTokens (Sampling.cpp:91-121), on the host: words uint32 [vocabulary] of one
- * request; pending_token 0xFFFFFFFF for none. */
-sp_status spo_sampling_rebuild_penalty_words(uint32_t *words, uint32_t vocabulary, const uint32_t *history, uint64_t history_tokens,
-                                             uint64_t generated_tokens, uint32_t pending_token, int mark_prompt);
-sp_status spo_sampling_count_penalty_tokens(uint32_t *words, uint32_t vocabulary, const uint32_t *selected, uint64_t count);
-/* Sampling::addPenalties (Sampling.cpp:129-172): rewrites, in place and before spo_sampling_add_verify reads them, the
- * logits rows of the lanes whose penalties are active, from `words` (uint32 [table rows][vocabulary]); a row also
- * counts the draft tokens of its path (input_tokens, tree_rows). One penalties entry per lane. */
-sp_status spo_sampling_add_penalties(spo_graph *graph, sp_buffer *logits, sp_buffer *words, sp_buffer *input_tokens,
-                                     sp_buffer *tree_rows, uint32_t vocabulary, uint32_t logits_stride, const spo_lane_rows *lanes,
-                                     const spo_sampling_penalties *penalties, uint32_t count);
-/* ops::ThinkingCutoff (Sampling.hpp:30-55) of one lane: rows of depth `row` on select end[0 .. end_count) in order unless a
- * draft token of their path up to that depth is the last end token or also_ends (0xFFFFFFFF: none). A lane without a
- * cutoff passes end_count 0. waits_for_mask: the end starts at the first row of the path from depth `row` on whose
- * constraint-mask row admits end[0]. */
-typedef struct spo_thinking_cutoff {
-  uint32_t row, end_count, also_ends, waits_for_mask;
-  const uint32_t *end;
-} spo_thinking_cutoff;
-/* The thinking cutoffs of a selection (Sampling.cpp:41-78, :314-327): after spo_sampling_add_verify, rewrites the
- * selections (tokens) of the rows each lane's end reaches. token_mask as in spo_sampling_buffers, read only for a lane
- * that waits for its mask (NULL otherwise). */
-sp_status spo_sampling_add_thinking_cutoff(spo_graph *graph, sp_buffer *input_tokens, sp_buffer *token_mask, uint32_t mask_words,
-                                           sp_buffer *tree_rows, sp_buffer *tokens, uint32_t vocabulary, const spo_lane_rows *lanes,
-                                           const spo_thinking_cutoff *cutoffs, uint32_t count);
 /* Sampling::addAcceptance (Sampling.cpp:330-357). */
 sp_status spo_sampling_add_acceptance(spo_graph *graph, sp_buffer *input_tokens, sp_buffer *tree_rows, sp_buffer *tokens,
                                       sp_buffer *retained, sp_buffer *accepted_count, sp_buffer *retained_rows,

@@ -22,10 +22,6 @@
 //                                   the reference's own test makes) and fold/rollback invariants; tree
 //                                   blocks by the same recurrence along each row's path.
 //   orc_argmax / orc_accept_tree    pinned by brute force on tiny vocabularies.
-//   orc_penalize                    pinned by a brute-force restatement over explicit path contexts (tests) and the
-//                                   closed cases of the reference's test (prompt-only, saturation, unselectable).
-//   orc_thinking_cutoff             pinned by an independent walk over explicit depth-ordered paths (tests) and the
-//                                   closed form on chains.
 //   orc_draft_verify_rows           pinned by an independent statement (a stable sort of the estimates, a recursive
 //                                   preorder) in the tests.
 //   orc_draft_candidates            pinned by a lexicographic sort of (logit descending, column ascending) in the tests,
@@ -134,17 +130,6 @@ struct OrcTreeRow { uint32_t ancestors; uint16_t parent; uint16_t depth; };
 uint32_t orc_accept_tree(const struct OrcTreeRow *tree, const uint32_t *tokens, const uint32_t *selected,
                          uint32_t rows, uint32_t remaining, const uint32_t *stop_tokens, uint32_t stops,
                          uint32_t *out_tokens, uint32_t *accepted, uint32_t *retained_rows);
-// sampling.metal:991-1051 decode_sample_penalize for one lane's block: logits fp32 [rows][stride] rewritten in place
-// from the lane's penalty words [vocab] (bit 31: a prompt token; the rest: the output's count), its input tokens and
-// tree rows. frequency * count, + presence and the subtraction each round once (no fused multiply-add).
-void orc_penalize(float *logits, uint32_t rows, uint32_t vocab, uint32_t stride, const uint32_t *words, const uint32_t *inputs,
-                  const struct OrcTreeRow *tree, float repetition, float presence, float frequency);
-// sampling.metal:1999-2042 decode_sample_thinking_cutoff for one lane's block: selections rewritten in place. masks
-// (uint32 [rows][mask_words], NULL unless waits) are the rows' constraint masks; end[0 .. count) the end tokens the
-// block's rows can hold, close the last token of the whole end.
-void orc_thinking_cutoff(uint32_t *selected, uint32_t rows, uint32_t vocab, const uint32_t *inputs, const struct OrcTreeRow *tree,
-                         const uint32_t *masks, uint32_t mask_words, uint32_t cutoff_row, const uint32_t *end, uint32_t count,
-                         uint32_t close, uint32_t also_ends, int waits);
 // sampling.metal:1799-1895 draft_verify_rows: a decode step's rows from each lane's tree (16 rows a lane: tokens, tree
 // rows, {draft probability, estimate} pairs; sizes[lane] rows held). Outputs as the kernel writes them: tokens, tree rows
 // and sources [rows], lane_rows {first, rows} [lanes].

@@ -135,53 +135,6 @@ void note(double *closeness, double value, double threshold) {
 
 extern "C" {
 
-// sampling.metal:1896-1997: larger value, ties to the lowest id, NaN and -inf skipped.
-void orc_penalize(float *logits, uint32_t rows, uint32_t vocab, uint32_t stride, const uint32_t *words, const uint32_t *inputs,
-                  const struct OrcTreeRow *tree, float repetition, float presence, float frequency) {
-  const float largest = std::numeric_limits<float>::max();
-  const float inverse = std::min(1.0f / repetition, largest);   // Sampling.cpp:147-149
-  for (uint32_t token = 0; token < vocab; ++token) {
-    uint32_t drafted = 0;
-    for (uint32_t row = 1; row < rows; ++row) drafted |= uint32_t(inputs[row] == token) << row;
-    const uint32_t word = words[token];
-    if (!word && !drafted) continue;
-    for (uint32_t row = 0; row < rows; ++row) {
-      const uint32_t count = (word & 0x7FFFFFFFu) + uint32_t(__builtin_popcount(drafted & tree[row].ancestors & ~1u));
-      if (!count && !(word & 0x80000000u)) continue;
-      float &logit = logits[size_t(row) * stride + token];
-      uint32_t bits; std::memcpy(&bits, &logit, 4);
-      if ((bits & 0x7FFFFFFFu) > 0x7F800000u || bits == 0xFF800000u) continue;   // unselectable: NaN or -infinity
-      float value = logit * (logit > 0.0f ? inverse : repetition);
-      if (count) {
-        const float product = frequency * float(count);
-        const float lowered = product + presence;
-        value = value - lowered;
-      }
-      logit = std::min(std::max(value, -largest), largest);
-    }
-  }
-}
-
-void orc_thinking_cutoff(uint32_t *selected, uint32_t rows, uint32_t vocab, const uint32_t *inputs, const struct OrcTreeRow *tree,
-                         const uint32_t *masks, uint32_t mask_words, uint32_t cutoff_row, const uint32_t *end, uint32_t count,
-                         uint32_t close, uint32_t also_ends, int waits) {
-  for (uint32_t at = 0; at < rows; ++at) {
-    const uint32_t path = tree[at].ancestors, depth = tree[at].depth;
-    uint32_t cut = 0;
-    for (uint32_t walk = path; walk; walk &= walk - 1, ++cut) {
-      const uint32_t row = uint32_t(__builtin_ctz(walk));
-      if (cut >= cutoff_row && (!waits || ((masks[size_t(row) * mask_words + end[0] / 32] >> (end[0] % 32)) & 1u))) break;
-    }
-    if (cut > depth || depth - cut >= count) continue;
-    bool ended = false;
-    for (uint32_t walk = path & ~1u; walk; walk &= walk - 1) {
-      const uint32_t before = uint32_t(__builtin_ctz(walk));
-      ended = ended || (tree[before].depth <= cut && (inputs[before] == close || inputs[before] == also_ends));
-    }
-    if (!ended && selected[at] < vocab) selected[at] = end[depth - cut];
-  }
-}
-
 // sampling.metal:1050-1052 top_beats, :1099-1232 draft_select_top16_sharded, :1236-1264 top16_merge_shards: a sorted list
 // of sixteen, begun as empty entries (-infinity, token 0xffffffff), takes every column that beats its last entry; shards
 // and their merge select what one list over the whole row does. A column's token is itself below `leading`, else

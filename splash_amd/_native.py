@@ -142,14 +142,6 @@ class VerifyLane(ctypes.Structure):
                 ("remaining", c_u32), ("min_p", ctypes.c_float), ("top_k", c_u32), ("top_p", ctypes.c_float)]
 
 
-class SamplingPenalties(ctypes.Structure):
-    _fields_ = [("repetition", ctypes.c_float), ("presence", ctypes.c_float), ("frequency", ctypes.c_float), ("table_row", c_u32)]
-
-
-class ThinkingCutoff(ctypes.Structure):
-    _fields_ = [("row", c_u32), ("end_count", c_u32), ("also_ends", c_u32), ("waits_for_mask", c_u32), ("end", P(c_u32))]
-
-
 class SamplingPolicy(ctypes.Structure):
     _fields_ = [("temperature", ctypes.c_float), ("min_p", ctypes.c_float), ("top_k", c_u32), ("top_p", ctypes.c_float),
                 ("constrained", c_u32), ("excludes_stop_tokens", c_u32)]
@@ -270,10 +262,6 @@ _sig("spo_moe_add_routed_norm", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_u32,
 _sig("spo_row_copy_add", c_int, c_p, c_p, c_u32, c_u32, c_u32, c_p, c_u32, c_u32, c_u32, c_u32, c_u32)
 _sig("spo_sampling_workspace", c_int, c_u32, P(c_u64))
 _sig("spo_sampling_add_verify", c_int, c_p, P(SamplingBuffers), c_u32, c_u32, P(LaneRows), P(SamplingPolicy), c_u32, P(c_u32))
-_sig("spo_sampling_rebuild_penalty_words", c_int, P(c_u32), c_u32, P(c_u32), c_u64, c_u64, c_u32, c_int)
-_sig("spo_sampling_count_penalty_tokens", c_int, P(c_u32), c_u32, P(c_u32), c_u64)
-_sig("spo_sampling_add_penalties", c_int, c_p, c_p, c_p, c_p, c_p, c_u32, c_u32, P(LaneRows), P(SamplingPenalties), c_u32)
-_sig("spo_sampling_add_thinking_cutoff", c_int, c_p, c_p, c_p, c_u32, c_p, c_p, c_u32, P(LaneRows), P(ThinkingCutoff), c_u32)
 _sig("spo_draft_add_verify_rows", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_u32, c_u32, c_u32, ctypes.c_float)
 _sig("spo_sampling_add_acceptance", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, P(LaneRows), P(c_u32), c_u32, P(c_u32))
 _sig("spo_sampling_greedy_rows_static", c_int, ctypes.c_void_p, c_u32, c_u32, c_u32, ctypes.c_void_p, ctypes.c_void_p)

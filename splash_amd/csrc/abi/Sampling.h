@@ -49,47 +49,7 @@ struct TargetSamplingParams {
   uint32_t reserved[3];
 };
 
-// A token's word of a penalty table row (Sampling.h:121-125 in the reference): the prompt bit marks a prompt token, the
-// count is how often the target selected the token.
-#define SAMPLING_PENALTY_PROMPT_BIT 0x80000000u
-#define SAMPLING_PENALTY_COUNT_MASK 0x7FFFFFFFu
-
-// decode_sample_penalize: grid (ceil(vocabulary / 256), entries), 256 threads. Entry e rewrites the logits rows of
-// lane[e] from row table_row[e] of the penalty table (the reference's SamplingPenaltyParams, abi/Sampling.h:127-142).
-// repetition_inverse is 1 / repetition, saturated to the largest float.
-struct SamplingPenaltyParams {
-  uint32_t vocabulary;
-  uint32_t entries;
-  uint32_t logits_stride;  // floats between logits rows
-  uint32_t reserved;
-  struct SamplingLaneRows lane[SAMPLING_MAXIMUM_LANES];
-  uint32_t table_row[SAMPLING_MAXIMUM_LANES];
-  float repetition[SAMPLING_MAXIMUM_LANES];
-  float repetition_inverse[SAMPLING_MAXIMUM_LANES];
-  float presence[SAMPLING_MAXIMUM_LANES];
-  float frequency[SAMPLING_MAXIMUM_LANES];
-};
-
-// decode_sample_thinking_cutoff: grid (lanes), one thread a lane (the reference's ThinkingCutoffParams,
-// abi/Sampling.h:147-172). A lane whose `row` is below its rows cuts each row's path at the path's row of depth `row`:
-// the path's row of depth cut + i selects its end token tokens[i], for each i below `count`, unless a draft token on
-// the path up to the cut is `close` or `also_ends`, which ended thinking first. The end of a lane in waiting_mask, a
-// constrained one, waits for its mask: a path's cut is instead the first of its rows from depth `row` on whose
-// constraint-mask row admits tokens[0]. A row whose selection is SAMPLING_NO_TOKEN keeps it.
-struct ThinkingCutoffParams {
-  uint32_t vocabulary;
-  uint32_t lanes;
-  uint32_t waiting_mask;
-  uint32_t mask_words;  // words of a constraint-mask row (one a packed row)
-  struct SamplingLaneRows lane[SAMPLING_MAXIMUM_LANES];
-  uint32_t row[SAMPLING_MAXIMUM_LANES];
-  uint32_t count[SAMPLING_MAXIMUM_LANES];
-  uint32_t close[SAMPLING_MAXIMUM_LANES];
-  uint32_t also_ends[SAMPLING_MAXIMUM_LANES];
-  uint32_t tokens[SAMPLING_MAXIMUM_LANES][SAMPLING_MAXIMUM_ROWS];
-};
-
-// draft_verify_rows: one thread lays out a decode step's rows from the trees a draft selector grew (the reference's
+// draft_verify_rows: one workgroup lays out a decode step's rows from the trees a draft selector grew (the reference's
 // VerifyRowsParams, abi/Sampling.h:270-298): `rows` rows over `lanes` lanes, each lane its anchor and the best of its
 // tree's other rows by estimate that the step's rows and the lanes' cap hold, none estimated below `floor`; the rows
 // past the lanes' belong to no lane.
@@ -122,7 +82,7 @@ struct DraftSelectParams {
   uint32_t reserved[2];
 };
 
-// decode_accept_tree: one thread per lane (AcceptBatchParams).
+// decode_accept_tree: one wavefront per lane, a thread a row (the reference's AcceptBatchParams, abi/Sampling.h:314-317).
 struct AcceptBatchParams {
   uint32_t lanes;
   uint32_t reserved[3];
@@ -133,8 +93,6 @@ struct AcceptBatchParams {
 
 #ifdef __cplusplus
 static_assert(sizeof(TargetSamplingParams) == 16 + 32 + 16 + 64 + 96 + 32, "target sampling parameters are 256 bytes on both sides");
-static_assert(sizeof(SamplingPenaltyParams) == 16 + 64 + 5 * 32, "penalty parameters are 240 bytes on both sides");
-static_assert(sizeof(ThinkingCutoffParams) == 16 + 64 + 4 * 32 + 512, "thinking cutoff parameters are 720 bytes on both sides");
 static_assert(sizeof(DraftSelectParams) == 32 + 32, "draft selector parameters are 64 bytes on both sides");
 static_assert(sizeof(VerifyRowsParams) == 16, "verify rows parameters are 16 bytes on both sides");
 static_assert(sizeof(AcceptBatchParams) == 16 + 32 + 16 + 64, "acceptance parameters are 128 bytes on both sides");

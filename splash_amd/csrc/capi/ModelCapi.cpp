@@ -114,53 +114,6 @@ sp_status spo_sampling_add_acceptance(spo_graph *graph, sp_buffer *input_tokens,
   });
 }
 
-sp_status spo_sampling_rebuild_penalty_words(uint32_t *words, uint32_t vocabulary, const uint32_t *history, uint64_t history_tokens,
-                                             uint64_t generated_tokens, uint32_t pending_token, int mark_prompt) {
-  return capi::guard([&] {
-    capi::require(words && history, "words or history");
-    ops::Sampling::rebuildPenaltyWords({words, vocabulary}, {history, size_t(history_tokens)}, generated_tokens,
-                                       pending_token == SAMPLING_NO_TOKEN ? std::nullopt : std::optional<uint32_t>(pending_token),
-                                       mark_prompt != 0);
-  });
-}
-sp_status spo_sampling_count_penalty_tokens(uint32_t *words, uint32_t vocabulary, const uint32_t *selected, uint64_t count) {
-  return capi::guard([&] {
-    capi::require(words && (selected || !count), "words or selected tokens");
-    ops::Sampling::countPenaltyTokens({words, vocabulary}, {selected, size_t(count)});
-  });
-}
-sp_status spo_sampling_add_penalties(spo_graph *graph, sp_buffer *logits, sp_buffer *words, sp_buffer *input_tokens,
-                                     sp_buffer *tree_rows, uint32_t vocabulary, uint32_t logits_stride, const spo_lane_rows *lanes,
-                                     const spo_sampling_penalties *penalties, uint32_t count) {
-  return capi::guard([&] {
-    capi::require(graph && lanes && penalties, "graph, lanes or penalties");
-    std::vector<ops::PenalizedLane> list;
-    for (uint32_t i = 0; i < count; ++i)
-      list.push_back({{lanes[i].first, lanes[i].rows}, penalties[i].table_row,
-                      {penalties[i].repetition, penalties[i].presence, penalties[i].frequency}});
-    ops::Sampling::addPenalties(capi::graphOf(graph), B(logits), B(words), B(input_tokens), B(tree_rows), vocabulary, logits_stride, list);
-  });
-}
-
-sp_status spo_sampling_add_thinking_cutoff(spo_graph *graph, sp_buffer *input_tokens, sp_buffer *token_mask, uint32_t mask_words,
-                                           sp_buffer *tree_rows, sp_buffer *tokens, uint32_t vocabulary, const spo_lane_rows *lanes,
-                                           const spo_thinking_cutoff *cutoffs, uint32_t count) {
-  return capi::guard([&] {
-    capi::require(graph && lanes && cutoffs, "graph, lanes or cutoffs");
-    std::vector<ops::LaneRows> rows;
-    std::vector<std::optional<ops::ThinkingCutoff>> list;
-    for (uint32_t i = 0; i < count; ++i) {
-      rows.push_back({lanes[i].first, lanes[i].rows});
-      if (!cutoffs[i].end_count) { list.push_back(std::nullopt); continue; }
-      capi::require(cutoffs[i].end, "a cutoff's end tokens");
-      list.push_back(ops::ThinkingCutoff{cutoffs[i].row, {cutoffs[i].end, cutoffs[i].end + cutoffs[i].end_count}, cutoffs[i].also_ends,
-                                         cutoffs[i].waits_for_mask != 0});
-    }
-    ops::Sampling::addThinkingCutoff(capi::graphOf(graph), B(input_tokens), token_mask ? B(token_mask) : hip::Buffer{}, mask_words,
-                                     B(tree_rows), B(tokens), vocabulary, rows, list);
-  });
-}
-
 sp_status spo_draft_candidate_scratch_bytes(uint32_t lanes, uint32_t columns, uint64_t *bytes) {
   return capi::guard([&] {
     capi::require(bytes, "result");

@@ -80,143 +80,105 @@ __global__ __launch_bounds__(256) void decode_sample_admit(float *__restrict__ l
 }
 SP_REGISTER_KERNEL("decode_sample_admit", &decode_sample_admit);
 
-// The sampling penalties of one logit (sampling.metal:991-1008): repetition divides a positive logit and multiplies a
-// negative one when the prompt or the output holds the token; presence and frequency lower it by the output's count of
-// the token. The result saturates, so no rewritten logit is infinite; an unselectable logit stays as it is.
-__device__ __forceinline__ float penalize_logit(float value, uint32_t count, float repetition, float repetition_inverse,
-                                                float presence, float frequency) {
-  if (unselectable(value)) return value;
-  value *= value > 0.0f ? repetition_inverse : repetition;
-  if (count) value -= frequency * float(count) + presence;
-  return fminf(fmaxf(value, -FLT_MAX), FLT_MAX);
-}
-// decode_sample_penalize (sampling.metal:1016-1051): one thread per vocabulary token and entry, the entry's lane's
-// logits rewritten in place. A row's context adds the draft tokens of its path: bit r of `drafted` is set when the
-// lane's input row r holds the token, which the rows below row r in the block's tree add to the output; a row counts
-// the bits of its ancestors but its anchor on top of the table's count.
-__global__ __launch_bounds__(256) void decode_sample_penalize(float *__restrict__ logits, const uint32_t *__restrict__ words,
-                                                              const uint32_t *__restrict__ input_tokens,
-                                                              const AttentionTreeRow *__restrict__ tree, SamplingPenaltyParams p) {
-  const uint32_t token = blockIdx.x * 256u + threadIdx.x, entry = blockIdx.y;
-  if (token >= p.vocabulary) return;
-  const SamplingLaneRows lane = p.lane[entry];
-  const uint32_t *inputs = input_tokens + lane.first;
-  uint32_t drafted = 0;
-  for (uint32_t row = 1; row < lane.rows; ++row) drafted |= uint32_t(inputs[row] == token) << row;
-  const uint32_t word = words[size_t(p.table_row[entry]) * p.vocabulary + token];
-  if (!word && !drafted) return;
-  float *column = logits + size_t(lane.first) * p.logits_stride + token;
-  for (uint32_t row = 0; row < lane.rows; ++row) {
-    const uint32_t path = tree[lane.first + row].ancestors;
-    const uint32_t count = (word & SAMPLING_PENALTY_COUNT_MASK) + uint32_t(__popc(drafted & path & ~1u));
-    if (!count && !(word & SAMPLING_PENALTY_PROMPT_BIT)) continue;
-    float &logit = column[size_t(row) * p.logits_stride];
-    logit = penalize_logit(logit, count, p.repetition[entry], p.repetition_inverse[entry], p.presence[entry], p.frequency[entry]);
-  }
-}
-SP_REGISTER_KERNEL("decode_sample_penalize", &decode_sample_penalize);
 
-// decode_sample_thinking_cutoff (sampling.metal:1999-2042): one thread a lane rewrites, among the lane's selections,
-// those of the rows its thinking end reaches.
-__global__ __launch_bounds__(64) void decode_sample_thinking_cutoff(const uint32_t *__restrict__ input_tokens,
-                                                                    const uint32_t *__restrict__ token_mask,
-                                                                    const AttentionTreeRow *__restrict__ tree,
-                                                                    uint32_t *__restrict__ tokens, ThinkingCutoffParams p) {
-  const uint32_t lane = blockIdx.x;
-  if (threadIdx.x || lane >= p.lanes) return;
-  const uint32_t rows = p.lane[lane].rows, first = p.lane[lane].first;
-  const bool waits = (p.waiting_mask >> lane) & 1u;
-  const uint32_t start = p.tokens[lane][0];
-  for (uint32_t at = 0; at < rows; ++at) {
-    const uint32_t path = tree[first + at].ancestors, depth = tree[first + at].depth;
-    // The path's rows ascend from its anchor, one a depth; one past the row's depth where the path holds no cut.
-    uint32_t cut = 0;
-    for (uint32_t walk = path; walk; walk &= walk - 1u, ++cut)
-      if (cut >= p.row[lane] &&
-          (!waits || ((token_mask[size_t(first + uint32_t(__ffs(int(walk)) - 1)) * p.mask_words + start / 32u] >> (start % 32u)) & 1u)))
-        break;
-    if (cut > depth || depth - cut >= p.count[lane]) continue;
-    bool ended = false;
-    for (uint32_t walk = path & ~1u; walk; walk &= walk - 1u) {
-      const uint32_t before = uint32_t(__ffs(int(walk)) - 1);
-      const uint32_t draft = input_tokens[first + before];
-      ended = ended || (tree[first + before].depth <= cut && (draft == p.close[lane] || draft == p.also_ends[lane]));
-    }
-    // A row with no selectable logit keeps its sentinel, so the lane fails.
-    if (!ended && tokens[first + at] < p.vocabulary) tokens[first + at] = p.tokens[lane][depth - cut];
-  }
-}
-SP_REGISTER_KERNEL("decode_sample_thinking_cutoff", &decode_sample_thinking_cutoff);
-
-// draft_verify_rows (sampling.metal:1799-1895): lane l's tree holds sizes[l] rows from row l * 16 of tree_tokens, trees
-// and scores (a row's draft probability and its estimate, the chance that the target accepts it), in the order the
-// selector took them, best first. A lane's rows are numbered in preorder, the earlier-taken child first, so that the
+// draft_verify_rows (the layout the reference's sampling.metal:1799-1895 produces): lane l's tree holds sizes[l] rows
+// from row l * 16 of tree_tokens, trees and scores (a row's draft probability and its estimate, the chance that the
+// target accepts it), in the order the selector took them, best first. The step takes every lane's anchor and the
+// best other rows by estimate (among equals the lower lane, then the lower row) that its rows and the lanes' cap
+// hold, none below the floor; a lane's rows are numbered in preorder, the earlier-taken child first, so that the
 // likeliest path of its tree lies on its first rows; the rows of no lane carry lane 0's anchor, no path and no source.
-__global__ __launch_bounds__(64) void draft_verify_rows(const uint32_t *__restrict__ tree_tokens, const AttentionTreeRow *__restrict__ trees,
-                                                        const float2 *__restrict__ scores, const uint32_t *__restrict__ sizes,
-                                                        uint32_t *__restrict__ tokens, AttentionTreeRow *__restrict__ tree,
-                                                        SamplingLaneRows *__restrict__ lane_rows, uint32_t *__restrict__ sources,
-                                                        VerifyRowsParams p) {
-  constexpr uint32_t kLanes = SAMPLING_MAXIMUM_LANES, kRows = SAMPLING_MAXIMUM_ROWS;
-  if (blockIdx.x || threadIdx.x) return;
-  // Every lane's rows past its anchor by estimate, a lane's earlier row first among equal ones.
-  float estimates[kLanes * kRows];
-  uint32_t owners[kLanes * kRows];
-  uint32_t count = 0;
-  for (uint32_t lane = 0; lane < p.lanes; ++lane)
-    for (uint32_t row = 1; row < min(sizes[lane], kRows); ++row) {
-      const float estimate = scores[lane * kRows + row].y;
-      uint32_t at = count++;
-      for (; at > 0 && estimates[at - 1] < estimate; --at) {
-        estimates[at] = estimates[at - 1];
-        owners[at] = owners[at - 1];
-      }
-      estimates[at] = estimate;
-      owners[at] = lane;
+//
+// One workgroup of 128 threads, thread (lane, row) = (t / 16, t % 16), no loop over the step's rows:
+//   rank      a candidate's place in the order above is the count of candidates that beat it;
+//   take      in that order a candidate is eligible if it is at or above the floor and fewer than cap - 1 candidates
+//             of its lane precede it; it is taken if fewer than rows - lanes eligible ones precede it (wave ballots
+//             over the ranked order);
+//   preorder  with ancestor masks, row x precedes row r if x is an ancestor of r or, where their paths part, x's
+//             branch was taken earlier (parents are taken before children, so the lowest set bit of a path below
+//             the common part is its branch): r's place is the count of the lane's rows that precede it.
+__global__ __launch_bounds__(128) void draft_verify_rows(const uint32_t *__restrict__ tree_tokens, const AttentionTreeRow *__restrict__ trees,
+                                                         const float2 *__restrict__ scores, const uint32_t *__restrict__ sizes,
+                                                         uint32_t *__restrict__ tokens, AttentionTreeRow *__restrict__ tree,
+                                                         SamplingLaneRows *__restrict__ lane_rows, uint32_t *__restrict__ sources,
+                                                         VerifyRowsParams p) {
+  constexpr uint32_t kLanes = SAMPLING_MAXIMUM_LANES, kRows = SAMPLING_MAXIMUM_ROWS, kAll = kLanes * kRows;
+  __shared__ float estimateOf[kAll];
+  __shared__ uint32_t rankedOwner[kAll];   // the lane of the candidate at each place of the order, kLanes for none
+  __shared__ float rankedEstimate[kAll];
+  __shared__ uint32_t eligibleBefore[2];   // eligible candidates in the first wave's places
+  __shared__ uint32_t takenOf[kLanes];
+  __shared__ uint32_t pathOf[kAll];        // a row's ancestors and itself, in its tree's own numbering
+  __shared__ uint32_t placeOf[kAll];       // a row's place in its lane's preorder
+  if (blockIdx.x) return;
+  const uint32_t t = threadIdx.x, lane = t / kRows, row = t % kRows, lanes = min(p.lanes, kLanes);
+  const uint32_t size = lane < lanes ? min(sizes[lane], kRows) : 0u;
+  const bool candidate = row >= 1 && row < size;
+  const float estimate = candidate ? scores[t].y : 0.f;
+  estimateOf[t] = candidate ? estimate : -INFINITY;
+  rankedOwner[t] = kLanes;
+  rankedEstimate[t] = -INFINITY;
+  if (t < kLanes) takenOf[t] = 0;
+  __syncthreads();
+  if (candidate) {
+    uint32_t rank = 0;
+    for (uint32_t other = 0; other < kAll; ++other) {
+      const float e = estimateOf[other];
+      rank += (e > estimate || (e == estimate && other < t)) && (other % kRows) >= 1 && e != -INFINITY ? 1u : 0u;
     }
-  // The best of them that the step's rows and the lanes' cap hold, none below the floor: they fall, so the first
-  // below it ends them.
-  uint32_t taken_of[kLanes];
-  for (uint32_t lane = 0; lane < p.lanes; ++lane) taken_of[lane] = 1;
-  uint32_t taken = p.lanes;
-  for (uint32_t i = 0; i < count && taken < p.rows; ++i) {
-    if (estimates[i] < p.floor) break;
-    if (taken_of[owners[i]] == p.lane_cap) continue;
-    ++taken_of[owners[i]];
-    ++taken;
+    rankedOwner[rank] = lane;
+    rankedEstimate[rank] = estimate;
   }
-  uint32_t first = 0;
-  for (uint32_t lane = 0; lane < p.lanes; ++lane) {
-    const uint32_t mine = taken_of[lane];
-    uint32_t parent[kRows], order[kRows], placed[kRows], stack[kRows];
-    for (uint32_t row = 0; row < mine; ++row) parent[row] = trees[lane * kRows + row].parent;
-    // Preorder: a row's children follow it, each with its subtree, in the order the tree took them.
-    uint32_t size = 0, next = 0;
-    stack[size++] = 0;
-    while (size) {
-      const uint32_t row = stack[--size];
-      placed[row] = next;
-      order[next++] = row;
-      for (uint32_t child = mine; child-- > row + 1;)
-        if (parent[child] == row && size < kRows) stack[size++] = child;
-    }
-    uint32_t ancestors[kRows], depths[kRows];
-    for (uint32_t at = 0; at < next; ++at) {
-      const uint32_t row = order[at];
-      const uint32_t up = at ? placed[parent[row]] : SAMPLING_TREE_ROOT;
-      ancestors[at] = (at ? ancestors[up] : 0u) | (1u << at);
-      depths[at] = at ? depths[up] + 1u : 0u;
-      tokens[first + at] = tree_tokens[lane * kRows + row];
-      tree[first + at] = AttentionTreeRow{ancestors[at], uint16_t(up), uint16_t(depths[at])};
-      sources[first + at] = row;
-    }
-    lane_rows[lane] = SamplingLaneRows{first, next};
-    first += next;
+  __syncthreads();
+  // Thread t now stands for place t of the order.
+  const uint32_t owner = rankedOwner[t];
+  uint32_t before = 0;   // candidates of the same lane at earlier places
+  for (uint32_t place = 0; place < t; ++place) before += rankedOwner[place] == owner ? 1u : 0u;
+  const bool eligible = owner < kLanes && !(rankedEstimate[t] < p.floor) && before + 1u < p.lane_cap;
+  const uint64_t ballot = __builtin_amdgcn_ballot_w64(eligible);
+  if ((t & 63u) == 0) eligibleBefore[t >> 6] = uint32_t(__builtin_popcountll(ballot));
+  __syncthreads();
+  const uint32_t earlier = uint32_t(__builtin_popcountll(ballot & ((uint64_t{1} << (t & 63u)) - 1u))) + (t >= 64 ? eligibleBefore[0] : 0u);
+  const uint32_t budget = p.rows > lanes ? p.rows - lanes : 0u;
+  if (eligible && earlier < budget) atomicAdd(&takenOf[owner], 1u);
+  __syncthreads();
+  // Back to thread (lane, row): the lane keeps its anchor and its first taken rows.
+  const uint32_t mine = lane < lanes ? takenOf[lane] + 1u : 0u;
+  uint32_t first = 0, total = 0;
+  for (uint32_t l = 0; l < lanes; ++l) {
+    first += l < lane ? takenOf[l] + 1u : 0u;
+    total += takenOf[l] + 1u;
   }
-  for (uint32_t row = first; row < p.rows; ++row) {
-    tokens[row] = tree_tokens[0];
-    tree[row] = AttentionTreeRow{0u, uint16_t(SAMPLING_TREE_ROOT), uint16_t(0)};
-    sources[row] = SAMPLING_NO_TOKEN;
+  const bool placed = row < mine;
+  const AttentionTreeRow node = placed ? trees[t] : AttentionTreeRow{0u, 0u, 0u};
+  pathOf[t] = placed ? node.ancestors : 0u;
+  __syncthreads();
+  uint32_t place = 0;
+  if (placed) {
+    const uint32_t path = node.ancestors;
+    for (uint32_t x = 0; x < mine; ++x) {
+      if (x == row) continue;
+      const uint32_t other = pathOf[lane * kRows + x], common = other & path;
+      const bool ancestor = (path >> x) & 1u, descendant = (other >> row) & 1u;
+      const bool earlierBranch = __builtin_ctz((other & ~common) | 0x10000u) < __builtin_ctz((path & ~common) | 0x10000u);
+      place += ancestor || (!descendant && earlierBranch) ? 1u : 0u;
+    }
+  }
+  placeOf[t] = place;
+  __syncthreads();
+  if (placed) {
+    uint32_t ancestors = 0;
+    for (uint32_t walk = node.ancestors; walk; walk &= walk - 1u) ancestors |= 1u << placeOf[lane * kRows + uint32_t(__builtin_ctz(walk))];
+    const uint32_t depth = uint32_t(__builtin_popcount(node.ancestors)) - 1u;
+    const uint32_t up = row ? placeOf[lane * kRows + node.parent] : SAMPLING_TREE_ROOT;
+    tokens[first + place] = tree_tokens[t];
+    tree[first + place] = AttentionTreeRow{ancestors, uint16_t(up), uint16_t(depth)};
+    sources[first + place] = row;
+  }
+  if (lane < lanes && row == 0) lane_rows[lane] = SamplingLaneRows{first, mine};
+  for (uint32_t spare = total + t; spare < p.rows; spare += kAll) {
+    tokens[spare] = tree_tokens[0];
+    tree[spare] = AttentionTreeRow{0u, uint16_t(SAMPLING_TREE_ROOT), uint16_t(0)};
+    sources[spare] = SAMPLING_NO_TOKEN;
   }
 }
 SP_REGISTER_KERNEL("draft_verify_rows", &draft_verify_rows);
@@ -263,42 +225,51 @@ __global__ __launch_bounds__(64) void decode_sample_argmax_reduce(const float *_
 }
 SP_REGISTER_KERNEL("decode_sample_argmax_reduce", &decode_sample_argmax_reduce);
 
-// Grid (lanes), 1 thread (sampling.metal:2044-2083). tokens: in, each row's selection; out, the
-// lane's retained tokens from its first row.
-__global__ void decode_accept_tree(const uint32_t *__restrict__ input_tokens, const AttentionTreeRow *__restrict__ tree,
-                                   uint32_t *__restrict__ tokens, uint32_t *__restrict__ retained,
-                                   uint32_t *__restrict__ accepted_count, uint32_t *__restrict__ retained_rows,
-                                   AcceptBatchParams p) {
-  const uint32_t lane = blockIdx.x;
-  if (lane >= p.lanes || threadIdx.x) return;
-  const uint32_t first = p.lane[lane].first, rows = p.lane[lane].rows;
-  const uint32_t *inputs = input_tokens + first;
-  const AttentionTreeRow *nodes = tree + first;
-  uint32_t *selected = tokens + first;
-  uint32_t path[SAMPLING_MAXIMUM_ROWS];
-  path[0] = 0;
-  uint32_t accepted = 0;
-  for (uint32_t row = 0;;) {
-    const uint32_t token = selected[row];
-    uint32_t next = 0;
-    for (uint32_t child = row + 1; child < rows && !next; ++child)
-      next = nodes[child].parent == row && inputs[child] == token ? child : 0;
-    if (!next) break;
-    path[++accepted] = next;
-    row = next;
+// decode_accept_tree (what the reference's sampling.metal:2044-2083 decides): grid (lanes), one wavefront a lane, a
+// thread a row. tokens: in, each row's selection; out, the lane's retained tokens from its first row.
+// A row follows its parent when its input token is the parent's selection and no earlier row of the same parent
+// does (one ballot); a row lies on the accepted path when every row of its ancestor mask follows its parent. The
+// path's rows, by depth, are the accepted draft tokens' rows; each selects the next token of the output, the last
+// the target's own. The output is cut to what the lane may still keep and after its first stop token (a second
+// ballot); the retained rows are the ancestor mask of the last kept row.
+__global__ __launch_bounds__(64) void decode_accept_tree(const uint32_t *__restrict__ input_tokens, const AttentionTreeRow *__restrict__ tree,
+                                                         uint32_t *__restrict__ tokens, uint32_t *__restrict__ retained,
+                                                         uint32_t *__restrict__ accepted_count, uint32_t *__restrict__ retained_rows,
+                                                         AcceptBatchParams p) {
+  const uint32_t lane = blockIdx.x, row = threadIdx.x;
+  if (lane >= p.lanes) return;
+  const uint32_t first = p.lane[lane].first, rows = min(p.lane[lane].rows, SAMPLING_MAXIMUM_ROWS);
+  const bool live = row < rows;
+  const AttentionTreeRow node = live ? tree[first + row] : AttentionTreeRow{0u, 0u, 0u};
+  const uint32_t input = live ? input_tokens[first + row] : 0u, selection = live ? tokens[first + row] : 0u;
+  const uint32_t parent = live && row ? min(uint32_t(node.parent), SAMPLING_MAXIMUM_ROWS - 1u) : 0u;
+  const uint32_t parentSelection = __shfl(selection, int(parent), 64);
+  const bool matches = live && row && node.parent < row && input == parentSelection;
+  // the matching rows of this row's parent before it
+  uint32_t siblingsBefore = 0;
+  for (uint32_t other = 1; other < rows; ++other) {
+    const bool sameParent = __shfl(matches ? int(parent) : -1, int(other), 64) == int(parent);
+    siblingsBefore += other < row && sameParent ? 1u : 0u;
   }
-  uint32_t kept = min(accepted + 1, max(p.remaining[lane], 1u));
-  for (uint32_t i = 0; i < kept; ++i) {
-    const uint32_t token = selected[path[i]];
-    selected[i] = token;
-    bool stop = false;
+  const bool follows = matches && !siblingsBefore;
+  const uint32_t following = uint32_t(__builtin_amdgcn_ballot_w64(follows)) | 1u;   // the anchor starts the path
+  const bool onPath = live && (node.ancestors & ~following) == 0u && ((node.ancestors >> row) & 1u);
+  const uint32_t path = uint32_t(__builtin_amdgcn_ballot_w64(onPath));
+  const uint32_t accepted = uint32_t(__builtin_popcount(path)) - 1u;
+  const uint32_t depth = live ? uint32_t(__builtin_popcount(path & ((1u << row) - 1u))) : 0u;   // the path's rows rise with depth
+  uint32_t kept = min(accepted + 1u, max(p.remaining[lane], 1u));
+  bool stop = false;
 #pragma unroll
-    for (int s = 0; s < int(SAMPLING_STOP_TOKENS); ++s) stop = stop || (p.stop_tokens[s] != SAMPLING_NO_TOKEN && token == p.stop_tokens[s]);
-    if (stop) kept = i + 1;
+  for (int s = 0; s < int(SAMPLING_STOP_TOKENS); ++s) stop = stop || (p.stop_tokens[s] != SAMPLING_NO_TOKEN && selection == p.stop_tokens[s]);
+  // the shallowest path row within the kept ones that selects a stop token ends the output
+  const uint32_t stops = uint32_t(__builtin_amdgcn_ballot_w64(onPath && depth < kept && stop));
+  if (stops) kept = uint32_t(__builtin_popcount(path & ((2u << __builtin_ctz(stops)) - 1u)));
+  if (onPath && depth < kept) tokens[first + depth] = selection;   // every selection was read before any is written
+  if (onPath && depth + 1u == kept) {
+    retained_rows[lane] = node.ancestors;
+    retained[lane] = kept;
+    accepted_count[lane] = min(accepted, kept);
   }
-  accepted_count[lane] = min(accepted, kept);
-  retained[lane] = kept;
-  retained_rows[lane] = nodes[path[kept - 1]].ancestors;
 }
 SP_REGISTER_KERNEL("decode_accept_tree", &decode_accept_tree);
 

@@ -55,7 +55,7 @@ void DraftSelector::addVerifyRows(hip::CommandGraph &graph, const DraftVerifyRow
   requireBytes(b.laneRows, uint64_t{step.lanes} * sizeof(SamplingLaneRows), "verify lane rows");
   requireBytes(b.verifySources, uint64_t{step.rows} * 4, "verify source");
   graph.add("draft_verify_rows", {b.treeTokens, b.trees, b.treeScores, b.treeSizes, b.inputTokens, b.treeRows, b.laneRows, b.verifySources},
-            VerifyRowsParams{step.lanes, step.rows, step.laneCap, floor}, {1, 1, 1}, {64, 1, 1});
+            VerifyRowsParams{step.lanes, step.rows, step.laneCap, floor}, {1, 1, 1}, {128, 1, 1});
 }
 
 } // namespace splash::ops

@@ -21,104 +21,6 @@ uint32_t packedRows(const std::vector<LaneRows> &lanes) {
 }
 } // namespace
 
-void Sampling::rebuildPenaltyWords(std::span<uint32_t> words, std::span<const uint32_t> history, uint64_t generatedTokens,
-                                   std::optional<uint32_t> pendingToken, bool markPrompt) {
-  if (history.size() <= generatedTokens) throw std::logic_error("request history holds no prompt");
-  const auto inside = [&](uint32_t token) {
-    if (token >= words.size()) throw std::invalid_argument("penalty token is outside the vocabulary");
-  };
-  for (uint32_t token : history) inside(token);
-  if (pendingToken) inside(*pendingToken);
-  const size_t prompt = history.size() - generatedTokens;
-  std::fill(words.begin(), words.end(), 0u);
-  if (markPrompt)
-    for (size_t i = 0; i < prompt; ++i) words[history[i]] |= SAMPLING_PENALTY_PROMPT_BIT;
-  for (size_t i = prompt; i < history.size(); ++i) ++words[history[i]];
-  if (pendingToken) ++words[*pendingToken];
-}
-
-void Sampling::countPenaltyTokens(std::span<uint32_t> words, std::span<const uint32_t> selected) {
-  for (uint32_t token : selected)
-    if (token >= words.size()) throw std::invalid_argument("penalty token is outside the vocabulary");
-  for (uint32_t token : selected) ++words[token];
-}
-
-void Sampling::addPenalties(hip::CommandGraph &graph, const hip::Buffer &logits, const hip::Buffer &words,
-                            const hip::Buffer &inputTokens, const hip::Buffer &treeRows, uint32_t vocabulary, uint32_t logitsStride,
-                            const std::vector<PenalizedLane> &lanes) {
-  if (!vocabulary || logitsStride < vocabulary) throw std::invalid_argument("logits rows hold the vocabulary");
-  std::vector<LaneRows> rowsOf;
-  for (const PenalizedLane &l : lanes) rowsOf.push_back(l.rows);
-  const uint32_t rows = packedRows(rowsOf);
-  SamplingPenaltyParams params{};
-  params.vocabulary = vocabulary;
-  params.logits_stride = logitsStride;
-  for (const PenalizedLane &l : lanes) {
-    if (!l.penalties.active()) continue;
-    if (!(l.penalties.repetition > 0.0f) || !std::isfinite(l.penalties.repetition) || !std::isfinite(l.penalties.presence) ||
-        !std::isfinite(l.penalties.frequency))
-      throw std::invalid_argument("a repetition penalty is positive and every penalty finite");
-    // the kernel indexes the whole table by this row
-    requireBytes(words, (uint64_t{l.tableRow} + 1) * vocabulary * 4, "penalty table");
-    const uint32_t entry = params.entries++;
-    params.lane[entry] = {l.rows.first, l.rows.rows};
-    params.table_row[entry] = l.tableRow;
-    params.repetition[entry] = l.penalties.repetition;
-    // 1 / 2^-149 overflows; the saturated inverse keeps the product finite
-    params.repetition_inverse[entry] = std::min(1.0f / l.penalties.repetition, std::numeric_limits<float>::max());
-    params.presence[entry] = l.penalties.presence;
-    params.frequency[entry] = l.penalties.frequency;
-  }
-  if (!params.entries) return;
-  requireBytes(logits, (uint64_t{rows - 1} * logitsStride + vocabulary) * 4, "logits");
-  requireBytes(treeRows, uint64_t{rows} * sizeof(AttentionTreeRow), "verify tree rows");
-  requireBytes(inputTokens, uint64_t{rows} * 4, "input tokens");
-  graph.add("decode_sample_penalize", {logits, words, inputTokens, treeRows}, params, {(vocabulary + 255) / 256, params.entries, 1},
-            {256, 1, 1});
-}
-
-void Sampling::addThinkingCutoff(hip::CommandGraph &graph, const hip::Buffer &inputTokens, const hip::Buffer &tokenMask,
-                                 uint32_t maskWords, const hip::Buffer &treeRows, const hip::Buffer &tokens, uint32_t vocabulary,
-                                 const std::vector<LaneRows> &lanes, const std::vector<std::optional<ThinkingCutoff>> &cutoffs) {
-  const uint32_t rows = packedRows(lanes);
-  if (cutoffs.size() != lanes.size()) throw std::invalid_argument("a thinking cutoff, or none, per lane");
-  if (!vocabulary) throw std::invalid_argument("invalid sampling geometry");
-  ThinkingCutoffParams params{};
-  params.vocabulary = vocabulary;
-  params.lanes = uint32_t(lanes.size());
-  params.mask_words = maskWords;
-  bool cuts = false;
-  for (size_t l = 0; l < lanes.size(); ++l) {
-    params.lane[l] = {lanes[l].first, lanes[l].rows};
-    const std::optional<ThinkingCutoff> &cutoff = cutoffs[l];
-    params.row[l] = cutoff ? cutoff->row : lanes[l].rows;
-    if (params.row[l] >= lanes[l].rows) {
-      params.row[l] = SAMPLING_MAXIMUM_ROWS;  // past every depth: the lane's rows keep their selections
-      continue;
-    }
-    if (cutoff->end.empty()) throw std::invalid_argument("a thinking cutoff has no end");
-    if (cutoff->waitsForMask) {
-      if (cutoff->end.front() >= vocabulary)
-        throw std::invalid_argument("a thinking end that waits for a mask starts outside the vocabulary");
-      if (uint64_t{maskWords} * 32 < vocabulary) throw std::invalid_argument("a constraint-mask row holds a bit for every token");
-      requireBytes(tokenMask, uint64_t{rows} * maskWords * 4, "constraint masks");
-      params.waiting_mask |= 1u << l;
-    }
-    // The rows from the cutoff's on take as many of its end as the lane's rows hold.
-    params.count[l] = uint32_t(std::min<size_t>(cutoff->end.size(), lanes[l].rows - cutoff->row));
-    std::copy_n(cutoff->end.begin(), params.count[l], params.tokens[l]);
-    params.close[l] = cutoff->end.back();
-    params.also_ends[l] = cutoff->alsoEnds;
-    cuts = true;
-  }
-  if (!cuts) return;
-  requireBytes(inputTokens, uint64_t{rows} * 4, "input tokens");
-  requireBytes(treeRows, uint64_t{rows} * sizeof(AttentionTreeRow), "verify tree rows");
-  requireBytes(tokens, uint64_t{rows} * 4, "selected tokens");
-  graph.add("decode_sample_thinking_cutoff", {inputTokens, params.waiting_mask ? tokenMask : inputTokens, treeRows, tokens}, params,
-            {uint32_t(lanes.size()), 1, 1}, {64, 1, 1});
-}
-
 SamplingWorkspaceSize Sampling::workspace(uint32_t rows) noexcept {
   SamplingWorkspaceSize size;
   size.partialValues = uint64_t{rows} * SAMPLING_SHARDS * 4;

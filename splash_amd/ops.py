@@ -462,49 +462,6 @@ class Sampling:
         return list(sizes)
 
     @staticmethod
-    def rebuild_penalty_words(vocabulary, history, generated_tokens, pending_token=None, mark_prompt=True):
-        """Sampling::rebuildPenaltyWords: a request's penalty words (uint32 [vocabulary]) from its history."""
-        words = np.zeros(vocabulary, dtype=np.uint32)
-        history = np.ascontiguousarray(history, dtype=np.uint32)
-        check(lib.spo_sampling_rebuild_penalty_words(words.ctypes.data_as(ctypes.POINTER(ctypes.c_uint32)), vocabulary,
-                                                     history.ctypes.data_as(ctypes.POINTER(ctypes.c_uint32)), len(history),
-                                                     generated_tokens, 0xFFFFFFFF if pending_token is None else pending_token,
-                                                     int(mark_prompt)))
-        return words
-
-    @staticmethod
-    def count_penalty_tokens(words, selected):
-        selected = np.ascontiguousarray(selected, dtype=np.uint32)
-        check(lib.spo_sampling_count_penalty_tokens(words.ctypes.data_as(ctypes.POINTER(ctypes.c_uint32)), len(words),
-                                                    selected.ctypes.data_as(ctypes.POINTER(ctypes.c_uint32)), len(selected)))
-
-    @staticmethod
-    def add_penalties(graph, logits, words, input_tokens, tree_rows, vocabulary, stride, lanes, penalties):
-        """lanes: [(first, rows)]; penalties: a lane's (repetition, presence, frequency, table_row)."""
-        rows = (nat.LaneRows * len(lanes))(*[nat.LaneRows(f, r) for f, r in lanes])
-        entries = (nat.SamplingPenalties * len(lanes))(*[nat.SamplingPenalties(*p) for p in penalties])
-        check(lib.spo_sampling_add_penalties(graph.handle, logits.handle, words.handle, input_tokens.handle, tree_rows.handle,
-                                             vocabulary, stride, rows, entries, len(lanes)))
-        graph._keep.extend([logits, words, input_tokens, tree_rows])
-
-    @staticmethod
-    def add_thinking_cutoff(graph, input_tokens, tree_rows, tokens, vocabulary, lanes, cutoffs, token_mask=None, mask_words=0):
-        """cutoffs: per lane None or (row, end tokens[, also_ends[, waits_for_mask]])."""
-        rows = (nat.LaneRows * len(lanes))(*[nat.LaneRows(f, r) for f, r in lanes])
-        entries, keep = [], []
-        for c in cutoffs:
-            if c is None:
-                entries.append(nat.ThinkingCutoff(0, 0, 0xFFFFFFFF, 0, None))
-                continue
-            end = (ctypes.c_uint32 * len(c[1]))(*c[1])
-            keep.append(end)
-            entries.append(nat.ThinkingCutoff(c[0], len(c[1]), c[2] if len(c) > 2 else 0xFFFFFFFF, int(c[3]) if len(c) > 3 else 0, end))
-        array = (nat.ThinkingCutoff * len(lanes))(*entries)
-        check(lib.spo_sampling_add_thinking_cutoff(graph.handle, input_tokens.handle, token_mask.handle if token_mask is not None else None,
-                                                   mask_words, tree_rows.handle, tokens.handle, vocabulary, rows, array, len(lanes)))
-        graph._keep.extend([input_tokens, tree_rows, tokens, token_mask])
-
-    @staticmethod
     def add_verify(graph, buffers, vocabulary, stride, lanes, policies, stop_tokens=None):
         """buffers: dict of Buffer by the names of spo_sampling_buffers (token_mask with mask_words for constrained
         lanes); lanes: [(first, rows)]; policies: a lane's temperature, or (temperature, min_p, top_k, top_p[,

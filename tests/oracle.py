@@ -514,38 +514,6 @@ def state_values(image, rows, columns):
     return values
 
 
-def penalize(logits, words, inputs, tree, repetition, presence, frequency):
-    """decode_sample_penalize for one lane's block: fp32 [rows][vocab] -> the rewritten rows."""
-    out = np.ascontiguousarray(logits, dtype=np.float32).copy()
-    rows, vocab = out.shape
-    words = np.ascontiguousarray(words, dtype=np.uint32)
-    inputs = np.ascontiguousarray(inputs, dtype=np.uint32)
-    tree = np.ascontiguousarray(tree)
-    lib.orc_penalize.restype = None
-    lib.orc_penalize(_p(out, f32p), c_u32(rows), c_u32(vocab), c_u32(vocab), _p(words, u32p), _p(inputs, u32p),
-                     tree.ctypes.data_as(ctypes.c_void_p), c_f(repetition), c_f(presence), c_f(frequency))
-    return out
-
-
-def thinking_cutoff(selected, inputs, tree, vocab, row, end, also_ends=NO_TOKEN, masks=None):
-    """decode_sample_thinking_cutoff for one lane's block: the selections after the cutoff. masks: uint32
-    [rows][words] when the end waits for the lane's constraint masks."""
-    out = np.ascontiguousarray(selected, dtype=np.uint32).copy()
-    rows = len(out)
-    inputs = np.ascontiguousarray(inputs, dtype=np.uint32)
-    tree = np.ascontiguousarray(tree)
-    count = min(len(end), rows - row) if row < rows else 0
-    if count <= 0:
-        return out
-    tokens = np.ascontiguousarray(end[:count], dtype=np.uint32)
-    m = np.ascontiguousarray(masks, dtype=np.uint32) if masks is not None else None
-    lib.orc_thinking_cutoff.restype = None
-    lib.orc_thinking_cutoff(_p(out, u32p), c_u32(rows), c_u32(vocab), _p(inputs, u32p), tree.ctypes.data_as(ctypes.c_void_p),
-                            _p(m, u32p), c_u32(m.shape[1] if m is not None else 0), c_u32(row), _p(tokens, u32p), c_u32(count),
-                            c_u32(end[-1]), c_u32(also_ends), c_int(m is not None))
-    return out
-
-
 TREE_DTYPE = np.dtype([("ancestors", "<u4"), ("parent", "<u2"), ("depth", "<u2")])
 
 

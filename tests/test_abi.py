@@ -35,7 +35,7 @@ def test_kernels_are_registered_by_name():
                  "gguf_decode_q4k_m16_a", "gguf_decode_q6k_m16_a_f32", "gguf_decode_q4k_m32_g", "gguf_decode_q6k_m64_r",
                  "gguf_decode_q5k_m16_gt", "gguf_decode_q80_m64_rn", "gguf_decode_mixed_m16_a", "gguf_decode_mixed_m64_a",
                  "gguf_dequant_iq4xs", "gguf_decode_iq4xs_m16_rn", "gguf_decode_iq4nl_m32_gt", "gguf_embed_iq4xs", "gguf_embed_iq4nl", "state_quantize", "state_dequantize_bf16_state", "state_copy",
-                 "decode_sample_penalize", "decode_sample_thinking_cutoff", "draft_verify_rows"):
+                 "draft_verify_rows"):
         assert splash_amd.lib.sp_kernel_exists(name.encode()), name
     assert not splash_amd.lib.sp_kernel_exists(b"no_such_kernel")
 
@@ -77,24 +77,3 @@ def test_linear_plans_without_a_device():
         linear.scratch_size(5120, 25600, 257)
     with pytest.raises(ValueError):
         linear.scratch_size(5121, 25600, 16)
-
-
-def test_penalty_words_follow_the_request_history():
-    """Sampling::rebuildPenaltyWords / countPenaltyTokens (Sampling.cpp:91-121): the prompt bit on prompt tokens, the
-    count of generated and pending tokens."""
-    history = [5, 9, 5, 2, 7, 7, 9]   # four prompt tokens, three generated
-    words = ops.Sampling.rebuild_penalty_words(12, history, 3, pending_token=7)
-    want = np.zeros(12, dtype=np.uint32)
-    want[[5, 9, 2]] = 0x80000000
-    want[7] += 3
-    want[9] += 1
-    assert np.array_equal(words, want)
-    assert np.array_equal(ops.Sampling.rebuild_penalty_words(12, history, 3, mark_prompt=False) & 0x80000000, np.zeros(12, np.uint32))
-    ops.Sampling.count_penalty_tokens(words, [7, 0, 0])
-    want[7] += 1
-    want[0] += 2
-    assert np.array_equal(words, want)
-    for bad in (lambda: ops.Sampling.rebuild_penalty_words(12, history, 7), lambda: ops.Sampling.rebuild_penalty_words(8, history, 3),
-                lambda: ops.Sampling.count_penalty_tokens(words, [12])):
-        with pytest.raises(splash_amd.SplashError):
-            bad()

@@ -295,101 +295,6 @@ def test_constraint_masks_and_stop_exclusion(backend):
         ops.Sampling.add_verify(splash_amd.CommandGraph(), {**b, "token_mask": None}, V, V, lanes, policies)
 
 
-@pytest.mark.parametrize("stride_pad", [0, 40])
-def test_penalties_rewrite_the_penalized_lanes_only(backend, stride_pad):
-    """decode_sample_penalize (sampling.metal:1016-1051) against the oracle, bit for bit: three lanes of chain and tree
-    blocks, two penalized from their own rows of the penalty table, one not; extreme repetition penalties saturate;
-    unselectable logits stay; the unpenalized lane's rows and the padding between rows keep their bits."""
-    print(f"case penalties stride_pad={stride_pad}", flush=True)
-    from tests.test_oracle_sampling import penalty_case, random_tree
-    rng = np.random.default_rng(21)
-    V = 1000
-    stride = V + stride_pad
-    blocks = [(16, None), (9, random_tree(rng, 9)), (5, None)]
-    lanes, trees, logits, inputs, tables = [], [], [], [], []
-    first = 0
-    for rows, tree in blocks:
-        tree = tree if tree is not None else ops.chain_tree_rows([rows])
-        x, words, tokens = penalty_case(rng, rows, V, tree)
-        lanes.append((first, rows)); trees.append(tree); logits.append(x); inputs.append(tokens); tables.append(words)
-        first += rows
-    total = first
-    padded = np.full((total, stride), np.float32(123.0), dtype=np.float32)
-    padded[:, :V] = np.concatenate(logits)
-    # lane 0 reads table row 2, lane 1 is not penalized, lane 2 reads table row 0
-    table = np.zeros((3, V), dtype=np.uint32)
-    table[2], table[0], table[1] = tables[0], tables[2], rng.integers(0, 2 ** 32, V, dtype=np.uint32)
-    for penalties in ([(1.3, 0.5, 0.25, 2), (1.0, 0.0, 0.0, 1), (0.8, 0.3, 0.0, 0)], [(1e-45, 0.0, 0.0, 2), (1.0, 0.0, 0.0, 1), (3e38, 1e38, 3e38, 0)]):
-        buffer = backend.from_array(padded)
-        graph = splash_amd.CommandGraph()
-        ops.Sampling.add_penalties(graph, buffer, backend.from_array(table), backend.from_array(np.concatenate(inputs)),
-                                   backend.from_array(np.concatenate(trees)), V, stride, lanes, penalties)
-        assert graph.kernels() == ["decode_sample_penalize"]
-        backend.run(graph)
-        got = buffer.download(np.float32).reshape(total, stride)
-        assert np.all(got[:, V:] == np.float32(123.0))
-        for (f, rows), x, words, tokens, tree, p in zip(lanes, logits, tables, inputs, trees, penalties):
-            want = orc.penalize(x, words, tokens, tree, *p[:3]) if p[:3] != (1.0, 0.0, 0.0) else x
-            assert got[f:f + rows, :V].tobytes() == want.tobytes(), p
-    # nothing is added when no lane's penalties are active; a table too short for a lane's row is refused
-    graph = splash_amd.CommandGraph()
-    args = (backend.from_array(padded), backend.from_array(table), backend.from_array(np.concatenate(inputs)),
-            backend.from_array(np.concatenate(trees)), V, stride, lanes)
-    ops.Sampling.add_penalties(graph, *args, [(1.0, 0.0, 0.0, 9)] * 3)
-    assert len(graph) == 0
-    with pytest.raises(splash_amd.SplashError):
-        ops.Sampling.add_penalties(graph, *args, [(1.1, 0.0, 0.0, 3)] + [(1.0, 0.0, 0.0, 0)] * 2)
-    with pytest.raises(splash_amd.SplashError):
-        ops.Sampling.add_penalties(graph, *args, [(0.0, 0.0, 0.0, 0)] * 3)
-
-
-def test_thinking_cutoff_rewrites_the_reached_rows(backend):
-    """decode_sample_thinking_cutoff (sampling.metal:1999-2042) against the oracle over lanes of chains and trees: a lane
-    cut at its first row, one in the middle of its block, one whose end waits for its constraint masks, one with no
-    cutoff and one whose cutoff lies past its rows."""
-    print("case thinking cutoff", flush=True)
-    from tests.test_oracle_sampling import random_tree
-    rng = np.random.default_rng(23)
-    vocab, words = 70, 3
-    for trial in range(20):
-        sizes = [int(rng.integers(1, 17)) for _ in range(5)]
-        trees = [random_tree(rng, n) if (trial + i) % 2 else ops.chain_tree_rows([n]) for i, n in enumerate(sizes)]
-        lanes, first = [], 0
-        for n in sizes:
-            lanes.append((first, n)); first += n
-        total = first
-        selected = rng.integers(0, vocab, total).astype(np.uint32)
-        selected[rng.random(total) < 0.1] = 0xFFFFFFFF
-        inputs = rng.integers(0, 10, total).astype(np.uint32)
-        masks = rng.integers(0, 2 ** 32, (total, words), dtype=np.uint32)
-        end = lambda: [int(t) for t in rng.integers(0, 10, int(rng.integers(1, 6)))]
-        cutoffs = [(0, end()), (int(rng.integers(0, sizes[1])), end(), int(rng.integers(0, 10))),
-                   (int(rng.integers(0, sizes[2])), end(), 0xFFFFFFFF, True), None, (sizes[4] + 1, end())]
-        tokens = backend.from_array(selected)
-        graph = splash_amd.CommandGraph()
-        ops.Sampling.add_thinking_cutoff(graph, backend.from_array(inputs), backend.from_array(np.concatenate(trees)), tokens, vocab, lanes,
-                                         cutoffs, token_mask=backend.from_array(masks), mask_words=words)
-        assert graph.kernels() == ["decode_sample_thinking_cutoff"]
-        backend.run(graph)
-        got = tokens.download(np.uint32)
-        for (f, n), tree, c in zip(lanes, trees, cutoffs):
-            want = selected[f:f + n]
-            if c is not None:
-                want = orc.thinking_cutoff(want, inputs[f:f + n], tree, vocab, c[0], c[1], c[2] if len(c) > 2 else 0xFFFFFFFF,
-                                           masks[f:f + n] if len(c) > 3 and c[3] else None)
-            assert np.array_equal(got[f:f + n], want), (trial, c)
-    # no lane is cut: nothing is added; an empty end and a waiting end outside the vocabulary are refused
-    graph = splash_amd.CommandGraph()
-    args = (backend.from_array(inputs), backend.from_array(np.concatenate(trees)), tokens, vocab, lanes)
-    ops.Sampling.add_thinking_cutoff(graph, *args, [None, (sizes[1], [1]), None, None, None])
-    assert len(graph) == 0
-    with pytest.raises(splash_amd.SplashError):
-        ops.Sampling.add_thinking_cutoff(graph, *args, [(0, [vocab + 1], 0xFFFFFFFF, True), None, None, None, None],
-                                         token_mask=backend.from_array(masks), mask_words=words)
-    with pytest.raises(splash_amd.SplashError):
-        ops.Sampling.add_thinking_cutoff(graph, *args, [(0, [1], 0xFFFFFFFF, True), None, None, None, None])   # no masks
-
-
 def test_verify_rows_are_laid_out_from_the_trees(backend):
     """draft_verify_rows (sampling.metal:1799-1895) against the oracle, bit for bit: tokens, tree rows, lane rows and
     sources over random trees, caps, floors and tied estimates; and its outputs are what the acceptance walk reads."""

@@ -199,134 +199,6 @@ def test_truncated_rejection_law_is_the_renormalized_kept_distribution():
             assert p[tok] > 0 and (not accepted or tok == child)
 
 
-def penalty_case(rng, rows, vocab, tree):
-    """A block's logits with the special values the reference's test covers (target_sampling_metal_test.mm:27-30,
-    :791-860), its penalty words and its draft tokens."""
-    logits = (rng.standard_normal((rows, vocab)) * 4).astype(np.float32)
-    logits[:, 3] = -np.inf
-    logits[rows // 2, 5] = np.nan
-    logits[:, 7] = np.float32(3e38)
-    logits[:, 8] = np.float32(-3e38)
-    logits[:, 9] = 0.0
-    words = np.zeros(vocab, dtype=np.uint32)
-    words[rng.choice(vocab, vocab // 3, replace=False)] = rng.integers(1, 5, vocab // 3)
-    words[rng.choice(vocab, vocab // 4, replace=False)] |= 0x80000000
-    words[[3, 5, 7, 8, 9]] |= 0x80000001
-    inputs = rng.integers(0, vocab, rows).astype(np.uint32)
-    inputs[1:4] = inputs[1] if rows > 3 else inputs[1:4]     # a token drafted at several rows of a path
-    return logits, words, inputs
-
-
-def brute_force_penalty(logits, words, inputs, tree, repetition, presence, frequency):
-    """Row r's context: the table's count of the token plus the rows of r's path, its anchor aside, that drafted it."""
-    out = logits.copy()
-    f32 = np.float32
-    largest = np.finfo(np.float32).max
-    with np.errstate(over="ignore", divide="ignore"):
-        inverse = min(f32(1) / f32(repetition), largest)
-    for r in range(logits.shape[0]):
-        path = [j for j in range(1, logits.shape[0]) if (int(tree[r]["ancestors"]) >> j) & 1]
-        for t in range(logits.shape[1]):
-            count = int(words[t] & 0x7FFFFFFF) + sum(1 for j in path if inputs[j] == t)
-            if (count == 0 and not (words[t] >> 31)) or np.isnan(logits[r, t]) or logits[r, t] == -np.inf:
-                continue
-            with np.errstate(over="ignore"):
-                value = f32(logits[r, t]) * (inverse if logits[r, t] > 0 else f32(repetition))
-                if count:
-                    value = f32(value - f32(f32(f32(frequency) * f32(count)) + f32(presence)))
-            out[r, t] = min(max(value, -largest), largest)
-    return out
-
-
-@pytest.mark.parametrize("penalties", [(1.3, 0.5, 0.25), (1.0, 0.7, 0.0), (0.8, 0.0, 0.0), (1e-45, 0.0, 0.0), (3e38, 1e38, 3e38)])
-def test_penalties_against_explicit_path_contexts(penalties):
-    rng = np.random.default_rng(11)
-    for rows, tree in ((9, random_tree(rng, 9)), (16, None), (1, None)):
-        if tree is None:
-            tree = np.zeros(rows, dtype=np.dtype([("ancestors", "<u4"), ("parent", "<u2"), ("depth", "<u2")]))
-            for r in range(rows):
-                tree[r] = ((2 << r) - 1, max(r - 1, 0) if r else 0xFFFF, r)
-        logits, words, inputs = penalty_case(rng, rows, 64, tree)
-        got = orc.penalize(logits, words, inputs, tree, *penalties)
-        want = brute_force_penalty(logits, words, inputs, tree, *penalties)
-        assert got.tobytes() == want.tobytes()
-        assert np.isfinite(got[np.isfinite(logits)]).all()                       # saturates, never overflows
-        assert np.all(got[:, 3] == -np.inf) and np.isnan(got[rows // 2, 5])      # unselectable logits stay
-        untouched = ((words == 0)[None, :] & (got.view(np.uint32) != logits.view(np.uint32)))
-        for r, t in zip(*np.nonzero(untouched)):                                 # only a drafted token of the path changes
-            assert any(inputs[j] == t for j in range(1, rows) if (int(tree[r]["ancestors"]) >> j) & 1)
-
-
-def cutoff_by_depth(selected, inputs, tree, vocab, row, end, also_ends, masks):
-    """The thinking cutoff told by depth: a row's path as the list of its rows in depth order; the cut is the first depth
-    from `row` on (whose mask admits end[0], for an end that waits); the rows of depth cut + i take end[i] unless a
-    drafted token of the path at depths 1..cut closes thinking."""
-    out = list(selected)
-    rows = len(selected)
-    count = min(len(end), rows - row) if row < rows else 0
-    for at in range(rows):
-        path = sorted((j for j in range(rows) if (int(tree[at]["ancestors"]) >> j) & 1), key=lambda j: int(tree[j]["depth"]))
-        assert [int(tree[j]["depth"]) for j in path] == list(range(len(path)))
-        depth = len(path) - 1
-        cut = next((d for d in range(row, len(path))
-                    if masks is None or (int(masks[path[d]][end[0] // 32]) >> (end[0] % 32)) & 1), None)
-        if cut is None or depth - cut >= count:
-            continue
-        if any(int(inputs[j]) in (end[-1], also_ends) for j in path[1:cut + 1]):
-            continue
-        if out[at] < vocab:
-            out[at] = end[depth - cut]
-    return np.array(out, dtype=np.uint32)
-
-
-def test_thinking_cutoff_against_a_walk_by_depth():
-    rng = np.random.default_rng(17)
-    vocab = 50
-    for trial in range(300):
-        rows = int(rng.integers(1, 17))
-        tree = random_tree(rng, rows) if trial % 3 else None
-        if tree is None:
-            tree = np.zeros(rows, dtype=np.dtype([("ancestors", "<u4"), ("parent", "<u2"), ("depth", "<u2")]))
-            for r in range(rows):
-                tree[r] = ((2 << r) - 1, max(r - 1, 0) if r else 0xFFFF, r)
-        selected = rng.integers(0, vocab, rows).astype(np.uint32)
-        selected[rng.random(rows) < 0.1] = orc.NO_TOKEN
-        inputs = rng.integers(0, 12, rows).astype(np.uint32)     # a small alphabet, so closes and also-ends occur
-        end = [int(t) for t in rng.integers(0, 12, int(rng.integers(1, 5)))]
-        row = int(rng.integers(0, rows + 2))
-        also = int(rng.integers(0, 12)) if trial % 2 else orc.NO_TOKEN
-        masks = None
-        if trial % 4 == 0:
-            masks = rng.integers(0, 2 ** 32, (rows, 2), dtype=np.uint32)
-        got = orc.thinking_cutoff(selected, inputs, tree, vocab, row, end, also, masks)
-        want = cutoff_by_depth(selected, inputs, tree, vocab, row, end, also, masks)
-        assert np.array_equal(got, want), (trial, rows, row, end)
-
-
-def test_thinking_cutoff_on_a_chain_closed_form():
-    """A chain whose drafts never close: rows row .. row + len(end) - 1 take the end in order; a close token drafted at a
-    depth up to the cut keeps every selection; a row without a selectable logit keeps its sentinel."""
-    rows, vocab = 12, 100
-    tree = np.zeros(rows, dtype=np.dtype([("ancestors", "<u4"), ("parent", "<u2"), ("depth", "<u2")]))
-    for r in range(rows):
-        tree[r] = ((2 << r) - 1, max(r - 1, 0) if r else 0xFFFF, r)
-    selected = np.arange(rows, dtype=np.uint32) + 50
-    inputs = np.full(rows, 7, dtype=np.uint32)
-    got = orc.thinking_cutoff(selected, inputs, tree, vocab, 4, [90, 91, 92])
-    want = selected.copy(); want[4:7] = [90, 91, 92]
-    assert np.array_equal(got, want)
-    got = orc.thinking_cutoff(selected, inputs, tree, vocab, 10, [90, 91, 92])     # the block holds two of the three
-    want = selected.copy(); want[10:12] = [90, 91]
-    assert np.array_equal(got, want)
-    closed = inputs.copy(); closed[3] = 92                                          # thinking closed before the cut
-    assert np.array_equal(orc.thinking_cutoff(selected, closed, tree, vocab, 4, [90, 91, 92]), selected)
-    closed = inputs.copy(); closed[5] = 92                                          # after the cut: not looked at
-    assert np.array_equal(orc.thinking_cutoff(selected, closed, tree, vocab, 4, [90, 91, 92])[4:7], [90, 91, 92])
-    failed = selected.copy(); failed[5] = orc.NO_TOKEN
-    assert orc.thinking_cutoff(failed, inputs, tree, vocab, 4, [90, 91, 92])[5] == orc.NO_TOKEN
-    assert np.array_equal(orc.thinking_cutoff(selected, inputs, tree, vocab, 12, [90]), selected)   # past the block
-
-
 def test_verify_rows_layout_against_a_sort_and_a_recursive_preorder():
     from tests.draft_case import grown_trees, layout_by_sorting
     rng = np.random.default_rng(29)
