@@ -21,10 +21,50 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0   # MI355X published HBM3E bandwidth
-# HBM bytes per launch of the one-pass gate/up projection, by (hidden, ffn, rows): FETCH_SIZE + WRITE_SIZE of
-# rocprofv3 --pmc runs of this file, each scaled by what the counter reads for the copy kernel's known bytes
-# (profiles/verify_step_c4_hbm_traffic.md). Counters cannot be read from inside the run.
-GATE_UP_TRAFFIC_BYTES = {(5120, 25600, 16): 124.2e6}
+# Counters cannot be read from inside the run: the HBM bytes a launch of the dominant kernel moves come from the
+# committed summary of two rocprofv3 --pmc runs of this file (FETCH_SIZE, then WRITE_SIZE), each scaled by what the same
+# counter reads, in the same run, for plain read and copy kernels of known size (--calibrate-traffic).
+TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "verify_step_c4_hbm_traffic.md")
+
+
+def measured_traffic(kernel):
+    """(bytes per launch, where it was measured) of `kernel` from the committed traffic summary: its line
+    `traffic <kernel>: <bytes> bytes per launch` and the summary's `measured at: <commit, date>` line; (None, None) when
+    the summary does not hold the kernel."""
+    import re
+    try:
+        text = open(TRAFFIC_SUMMARY).read()
+    except OSError:
+        return None, None
+    found = re.search(r"^traffic " + re.escape(kernel) + r": (\d+) bytes per launch", text, re.M)
+    where = re.search(r"^measured at: (.+)$", text, re.M)
+    return (int(found.group(1)) if found else None), (where.group(1).strip() if where else None)
+
+
+def calibrate_traffic(backend):
+    """Plain kernels of known size for the counters' scale, over buffers nothing has read: read_bytes streams 256 MiB
+    (its fetch counter against 268,435,456 bytes), copy_bytes moves 256 MiB (fetch and write counters against the
+    same), four times each over buffers of their own. Their grids (2051 and 4099 workgroups) tell them from every
+    other dispatch of the run."""
+    import ctypes
+    import splash_amd
+
+    class P(ctypes.Structure):
+        _fields_ = [("vectors", ctypes.c_uint64)]
+    size = 256 << 20
+    sources = [backend.allocate_buffer(size, label="calibration source") for _ in range(8)]
+    targets = [backend.allocate_buffer(size, label="calibration target") for _ in range(4)]
+    folded = backend.allocate_buffer(1 << 20)
+    for b in sources:
+        b.fill(0x5A)
+    g = splash_amd.CommandGraph()
+    for i in range(4):
+        g.add("read_bytes", [sources[i], folded], P(size // 16), (2051, 1, 1), (256, 1, 1))
+    for i in range(4):
+        g.add("copy_bytes", [sources[4 + i], targets[i]], P(size // 16), (4099, 1, 1), (256, 1, 1))
+    backend.run(g)
+    log(f"traffic calibration: 4 reads and 4 copies of {size} bytes")
+
 
 WORKLOADS = {
     # hidden, q heads, kv heads, head dim, ffn, vocabulary, layers, context, rows
@@ -479,6 +519,9 @@ def main():
     ap.add_argument("--workload", default="c4", choices=sorted(WORKLOADS) + ["c5"])
     ap.add_argument("--lanes", type=int, default=1)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-traffic", action="store_true",
+                    help="after the steps, run plain read and copy kernels of known size: the scale of the FETCH_SIZE / "
+                         "WRITE_SIZE counters of a rocprofv3 --pmc run of this command")
     ap.add_argument("--temperature", type=float, default=0.0,
                     help="above 0: rejection-sampling acceptance at this temperature against a full-vocabulary draft "
                          "distribution softmax(N(0, 2)) instead of greedy acceptance")
@@ -550,6 +593,9 @@ def main():
     H, F = w["hidden"], w["ffn"]
     gate_up_bytes = 2 * F * H * 0.5625 + rows * H * 2 + rows * F * 2     # both tensors once + bf16 rows in and out
     achieved = gate_up_bytes / avg / 1e9
+    traffic, traffic_at = measured_traffic(gate_up) if args.workload == "c4" and args.lanes == 1 else (None, None)
+    if args.calibrate_traffic:
+        calibrate_traffic(backend)
     result = {
         "metric": "verify-step ms + % HBM roofline, 27B-shape Q4_K, 16-tok draft, 32K ctx" if args.workload == "c4" else "verify-step ms (config 1)",
         "value": round(ms, 4), "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
@@ -562,7 +608,8 @@ def main():
         "step_hbm": {"algorithmic_gb": round(step_bytes / 1e9, 3), "achieved_gbs": round(step_bytes / (ms * 1e-3) / 1e9, 1),
                      "frac_of_peak": round(step_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "wall_ms_per_step": round(wall_ms, 4)},
         "roofline": {"bound": "hbm", "kernel": gate_up, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": GATE_UP_TRAFFIC_BYTES.get((w["hidden"], w["ffn"], rows)), "launches": len(by_kernel[gate_up]),
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic, "traffic_measured_at": traffic_at,
+                     "launches": len(by_kernel[gate_up]),
                      "avg_us": round(avg * 1e6, 2), "algorithmic_bytes": int(gate_up_bytes), "largest_total": dominant},
     }
     if not args.no_cpu_baseline:

@@ -608,25 +608,45 @@ __device__ __forceinline__ void decode_workgroup(DecodeShared<RT> &shared, const
     // thread takes RT parts of its row. The loads go out before the first weights', so the wait for
     // them leaves those in flight.
     constexpr uint32_t kRows = 16u * RT, kParts = 16u, kThreadParts = 256u / kRows;
-    float squareSum[RT];
+    // Eight entries of a part are loaded together and added in their order afterwards, so a part costs one round trip
+    // to the cache, not one an entry; the first eight go out before the first weights and are added once those are
+    // on their way. The squares are read through a resource of their own: an entry past the table's, a row past its
+    // rows and every entry of a table without a deferred scale read as zero without touching memory (a squares entry
+    // is a sum of squares: adding 0 changes nothing).
+    constexpr uint32_t kChunk = 8u;
+    float squareSum[RT], loaded[RT][kChunk];
 #pragma unroll
     for (int i = 0; i < RT; ++i) squareSum[i] = 0.f;
-    if (p.deferred_scale) {
-      const float *squares = reinterpret_cast<const float *>(table + gguf_table_squares_offset(p.input_size, tiles));
-      const uint32_t row = threadIdx.x % kRows, entries = p.input_size / 64u;
-      if (row < 16u * tiles) {
+    const uint32_t squareRow = threadIdx.x % kRows, squareEntries = p.input_size / 64u, squareStride = 16u * tiles * 4u;
+    const Resource squares = make_resource(table + gguf_table_squares_offset(p.input_size, tiles),
+                                           p.deferred_scale && squareRow < 16u * tiles ? squareEntries * squareStride : 0u);
+    auto loadSquares = [&](int i, uint32_t base) {
 #pragma unroll
-        for (int i = 0; i < RT; ++i)
-          for (uint32_t j = threadIdx.x / kRows + kThreadParts * i; j < entries; j += kParts)
-            squareSum[i] += squares[size_t(j) * 16u * tiles + row];
-      }
-      __builtin_amdgcn_sched_barrier(0);
-    }
+      for (uint32_t e = 0; e < kChunk; ++e)
+        loaded[i][e] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(squares, int((base + kParts * e) * squareStride + squareRow * 4u), 0, 0));
+    };
+    auto addSquares = [&](int i) {
+#pragma unroll
+      for (uint32_t e = 0; e < kChunk; ++e) squareSum[i] += loaded[i][e];
+    };
+#pragma unroll
+    for (int i = 0; i < RT; ++i) loadSquares(i, threadIdx.x / kRows + kThreadParts * i);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int s = 0; s < kStages - 1; ++s) {
       issue(stage[s]);
       // Keep the stages' loads in issue order: the loop's counted waits assume it on entry too.
       __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll
+    for (int i = 0; i < RT; ++i) {
+      addSquares(i);
+      // a wider table: the part's further entries, eight at a time (these waits do reach the weights')
+      if (p.deferred_scale)
+        for (uint32_t base = threadIdx.x / kRows + kThreadParts * i + kParts * kChunk; base < squareEntries; base += kParts * kChunk) {
+          loadSquares(i, base);
+          addSquares(i);
+        }
     }
     if (p.deferred_scale) {
 #pragma unroll
