@@ -260,6 +260,12 @@ typedef struct spo_sampling_buffers {
   sp_buffer *draft_probabilities, *uniforms, *masses, *ranges, *decisions, *input_tokens, *tree_rows; /* sampled lanes */
   sp_buffer *token_mask; /* constrained lanes: uint32 [rows][mask_words], bit t % 32 of word t / 32 of a row admits token t */
   uint32_t mask_words;
+  /* A tree block's sampled rows (the reference's DrawChildren, sampling.metal:680-690; NULL for blocks whose rows have
+   * one child tested against a full-vocabulary draft distribution): each row's sixteen candidates -- uint32 ids and fp32
+   * draft probabilities [rows][16] --, the candidate indices of the children its draft drew in the order drawn (bytes
+   * [rows][4], 0xFF past them) and a uniform for each child's test (fp32 [rows][4]). With these the sampled lanes' rows
+   * run recursive rejection sampling over their children (sampling.metal:697-880); draft_probabilities is not read. */
+  sp_buffer *candidate_ids, *candidate_probabilities, *candidate_draws, *child_uniforms;
 } spo_sampling_buffers;
 /* ops::SamplingPolicy (Sampling.hpp:56-83): temperature 0 is greedy; a sampling lane keeps the tokens that
  * weigh at least min_p of its heaviest (0: all), then the top_k most likely of those (0: all), then their

@@ -171,6 +171,13 @@ void orc_rejection_law_policy(const float *logits, uint32_t vocab, const struct 
 // The selection law of one sampled row in fp64, for the enumeration check
 // (target_sampling_metal_test.mm:2602-2631): out[t] = P(row selects t) when the draft proposes its
 // child from q and the row tests and redraws as above. It must equal softmax(logits / T).
+// sampling.metal:697-880: a verify row of a tree block: up to four drawn children among sixteen candidates (ids, their
+// draft probabilities q, the candidate indices drawn in order, 0xFF for none, one uniform a child), then the last
+// residual's draw at u_row. Returns the selected token.
+uint32_t orc_children_row(const float *x, uint32_t V, const struct OrcSamplingPolicy *policy, const uint32_t *ids, const float *q,
+                          const uint8_t *draws, uint32_t n_draws, const float *u_children, float u_row, double *closeness);
+// The law of that selection over the draft's draws without replacement, by enumeration in fp64: out[t] = P(select t).
+void orc_children_law(const double *p_target, uint32_t V, const uint32_t *ids, const double *q, uint32_t n_draws, double *out);
 void orc_rejection_law(const float *logits, uint32_t vocab, float temperature, const float *q, double *out);
 
 // ---- Gated DeltaNet ----

@@ -383,6 +383,183 @@ uint32_t orc_rejection_row_policy(const float *x, uint32_t V, const OrcSamplingP
   return selected != ORC_NO_TOKEN ? selected : lastToken;
 }
 
+// sampling.metal:697-880 (vocabulary_draw with children): a verify row of a tree block tests the children its draft drew
+// among the sixteen candidates ids[] (draft probabilities q[], candidate indices draws[0 .. n_draws) in the order drawn,
+// one uniform a child): child c is selected iff u_c q_c < p_c; on a rejection the target's distribution becomes its
+// residual max(p - q, 0) over the candidates with the mass outside them kept, renormalized, and the draft's loses the
+// child, renormalized. A row that selects none draws at point = u_row (inside + outside): a candidate with residual
+// weight in index order, or past them a token outside the candidates by the target's own weights in id order. Sums
+// in fp32 in the orders of the kernel: ranges of (V + 255) / 256 tokens, 64 lane chunks a range, tokens of a chunk.
+uint32_t orc_children_row(const float *x, uint32_t V, const OrcSamplingPolicy *policy, const uint32_t *ids, const float *q_in,
+                          const uint8_t *draws, uint32_t n_draws, const float *u_children, float u_row, double *closeness) {
+  constexpr uint32_t K = 16;
+  const float inv = 1.0f / policy->temperature;
+  if (closeness) *closeness = 1.0;
+  const Kept mass = distributionEnd(x, V, *policy, nullptr, closeness);
+  const uint32_t size = (V + kRanges - 1) / kRanges, per = (size + 63) / 64;
+  std::vector<float> ranges(kRanges, 0.f), lanes(64);
+  bool excluding = false;
+  uint32_t excluded[K];
+  auto weightOf = [&](uint32_t t) {
+    if (excluding)
+      for (uint32_t i = 0; i < K; ++i)
+        if (excluded[i] == t) return 0.f;
+    return keptWeight(x[t], t, mass, inv);
+  };
+  auto laneSums = [&](uint32_t range) {
+    const uint32_t begin = range * size, end = std::min(V, begin + size);
+    for (uint32_t l = 0; l < 64; ++l) {
+      float s = 0.f;
+      for (uint32_t i = 0; i < per; ++i) {
+        const uint32_t t = begin + l * per + i;
+        if (t < end) s += weightOf(t);
+      }
+      lanes[l] = s;
+    }
+  };
+  for (uint32_t j = 0; j < kRanges; ++j) {
+    laneSums(j);
+    float s = 0.f;
+    for (int l = 0; l < 64; ++l) s += lanes[l];
+    ranges[j] = s;
+  }
+  float total = 0.f;
+  for (uint32_t j = 0; j < kRanges; ++j) total += ranges[j];
+  if (!(total > 0.f)) return ORC_NO_TOKEN;
+  float target = u_row * total;
+  if (n_draws && draws[0] != 0xFF) {
+    float p[K], q[K];
+    for (uint32_t i = 0; i < K; ++i) {
+      const float w = ids[i] < V ? keptWeight(x[ids[i]], ids[i], mass, inv) : 0.f;
+      if (ids[i] < V) ranges[ids[i] / size] = std::max(ranges[ids[i] / size] - w, 0.f);
+      excluded[i] = ids[i];
+      p[i] = w / total;
+      q[i] = q_in[i];
+    }
+    float outsideWeight = 0.f;
+    for (uint32_t j = 0; j < kRanges; ++j) outsideWeight += ranges[j];
+    float outside = outsideWeight / total;
+    for (uint32_t child = 0; child < n_draws && child < 4; ++child) {
+      const uint32_t c = draws[child];
+      if (c == 0xFF) break;
+      note(closeness, double(u_children[child]) * q[c], p[c]);
+      if (u_children[child] * q[c] < p[c]) return ids[c];
+      float residual = outside;
+      for (uint32_t i = 0; i < K; ++i) residual += std::max(p[i] - q[i], 0.f);
+      if (!(residual > 0.f)) break;
+      for (uint32_t i = 0; i < K; ++i) p[i] = std::max(p[i] - q[i], 0.f) / residual;
+      outside /= residual;
+      q[c] = 0.f;
+      float rest = 0.f;
+      for (uint32_t i = 0; i < K; ++i) rest += q[i];
+      for (uint32_t i = 0; rest > 0.f && i < K; ++i) q[i] /= rest;
+    }
+    float inside = 0.f;
+    for (uint32_t i = 0; i < K; ++i) inside += p[i];
+    const float point = u_row * (inside + outside);
+    float cumulative = 0.f;
+    uint32_t last = K;
+    for (uint32_t i = 0; i < K && !(point < cumulative); ++i)
+      if (p[i] > 0.f) {
+        last = i;
+        note(closeness, point, cumulative + p[i]);
+        if (cumulative > 0) note(closeness, point, cumulative);
+        cumulative += p[i];
+      }
+    if (last < K && (point < cumulative || !(outside > 0.f))) return ids[last];
+    excluding = true;
+    target = (point - inside) / outside * outsideWeight;
+  }
+  // the range that holds the target; the last weighted one on a rounding shortfall
+  uint32_t hit = kRanges, lastWeighted = 0;
+  float before = 0.f, lastBefore = 0.f, cumulative = 0.f;
+  for (uint32_t j = 0; j < kRanges && hit == kRanges; ++j) {
+    if (ranges[j] > 0.f) { lastWeighted = j; lastBefore = cumulative; }
+    if (ranges[j] > 0.f && target < cumulative + ranges[j]) {
+      hit = j; before = cumulative;
+      note(closeness, double(target), double(cumulative) + ranges[j]);
+      if (cumulative > 0) note(closeness, double(target), cumulative);
+    }
+    cumulative += ranges[j];
+  }
+  if (hit == kRanges) { hit = lastWeighted; before = lastBefore; }
+  float within = target - before;
+  laneSums(hit);   // with the candidates left out when the draw is past them
+  uint32_t chunk = 64, lastChunk = 0;
+  float chunkBefore = 0.f, lastChunkBefore = 0.f;
+  cumulative = 0.f;
+  for (uint32_t l = 0; l < 64; ++l) {
+    if (lanes[l] > 0.f) { lastChunk = l; lastChunkBefore = cumulative; }
+    if (chunk == 64 && lanes[l] > 0.f && within < cumulative + lanes[l]) {
+      chunk = l; chunkBefore = cumulative;
+      note(closeness, double(within) + before, double(cumulative) + lanes[l] + before);
+    }
+    cumulative += lanes[l];
+  }
+  if (chunk == 64) { chunk = lastChunk; chunkBefore = lastChunkBefore; }
+  within -= chunkBefore;
+  const uint32_t begin = hit * size, end = std::min(V, begin + size);
+  uint32_t selected = ORC_NO_TOKEN, lastToken = ORC_NO_TOKEN;
+  float walked = 0.f;
+  for (uint32_t i = 0; i < per; ++i) {
+    const uint32_t t = begin + chunk * per + i;
+    if (t >= end) break;
+    const float w = weightOf(t);
+    if (w > 0.f) lastToken = t;
+    walked += w;
+    if (selected == ORC_NO_TOKEN && w > 0.f && within < walked) {
+      selected = t;
+      note(closeness, double(within) + before + chunkBefore, double(walked) + before + chunkBefore);
+      note(closeness, double(within) + before + chunkBefore, double(walked - w) + before + chunkBefore);
+    }
+  }
+  return selected != ORC_NO_TOKEN ? selected : lastToken;
+}
+
+// The law of that selection when the draft draws its n_draws children from q without replacement (each next child from
+// the rest of q, renormalized), in fp64 by enumerating every sequence of rejected children
+// (target_sampling_metal_test.mm:2560-2600): out[t] = P(the row selects t). It equals the target's own distribution
+// whatever q and the candidates are: that is what the rule is for.
+void orc_children_law(const double *p_target, uint32_t V, const uint32_t *ids, const double *q_in, uint32_t n_draws, double *out) {
+  constexpr uint32_t K = 16;
+  struct State { double p[K], q[K], outside; };
+  std::vector<bool> candidate(V, false);
+  double outsideMass = 0;
+  for (uint32_t i = 0; i < K; ++i) if (ids[i] < V) candidate[ids[i]] = true;
+  for (uint32_t t = 0; t < V; ++t) { out[t] = 0; if (!candidate[t]) outsideMass += p_target[t]; }
+  State start{};
+  for (uint32_t i = 0; i < K; ++i) { start.p[i] = ids[i] < V ? p_target[ids[i]] : 0.0; start.q[i] = q_in[i]; }
+  start.outside = outsideMass;
+  struct Walker {
+    const double *p_target; uint32_t V; const uint32_t *ids; const std::vector<bool> &candidate; double outsideMass; double *out;
+    void step(const State &r, uint32_t left, double weight) {
+      double draft = 0;
+      for (double v : r.q) draft += v;
+      if (!left || !(draft > 0)) {
+        for (uint32_t i = 0; i < K; ++i) if (ids[i] < V) out[ids[i]] += weight * r.p[i];
+        for (uint32_t t = 0; t < V && outsideMass > 0; ++t) if (!candidate[t]) out[t] += weight * r.outside * p_target[t] / outsideMass;
+        return;
+      }
+      for (uint32_t i = 0; i < K; ++i) {
+        if (!(r.q[i] > 0)) continue;
+        const double drawn = r.q[i] / draft, accept = std::min(1.0, r.p[i] / r.q[i] * draft);   // q renormalized to its rest
+        if (ids[i] < V) out[ids[i]] += weight * drawn * accept;
+        if (accept < 1.0) {
+          State next = r;
+          double residual = next.outside;
+          for (uint32_t j = 0; j < K; ++j) residual += std::max(next.p[j] - next.q[j] / draft, 0.0);
+          if (!(residual > 0)) continue;
+          for (uint32_t j = 0; j < K; ++j) next.p[j] = std::max(next.p[j] - next.q[j] / draft, 0.0) / residual;
+          next.outside /= residual;
+          next.q[i] = 0;
+          step(next, left - 1, weight * drawn * (1.0 - accept));
+        }
+      }
+    }
+  } walker{p_target, V, ids, candidate, outsideMass, out};
+  walker.step(start, n_draws, 1.0);
+}
+
 // P(select t) = q_t min(1, p_t / q_t) + (1 - sum_s q_s min(1, p_s / q_s)) * max(p_t - q_t, 0) / Z:
 // the first term is "child t drawn and accepted", the second "child rejected, residual draws t".
 void orc_rejection_law(const float *x, uint32_t V, float temperature, const float *q, double *out) {

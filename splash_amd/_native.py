@@ -129,7 +129,8 @@ class MoeWorkspace(ctypes.Structure):
 
 class SamplingBuffers(ctypes.Structure):
     _fields_ = [(n, c_p) for n in ("logits", "tokens", "partial_values", "partial_indices", "draft_probabilities", "uniforms",
-                                   "masses", "ranges", "decisions", "input_tokens", "tree_rows", "token_mask")] + [("mask_words", c_u32)]
+                                   "masses", "ranges", "decisions", "input_tokens", "tree_rows", "token_mask")] + [("mask_words", c_u32)] + [
+        (n, c_p) for n in ("candidate_ids", "candidate_probabilities", "candidate_draws", "child_uniforms")]
 
 
 class DenseDimensions(ctypes.Structure):

@@ -9,6 +9,9 @@
 #define SAMPLING_MAXIMUM_LANES 8u
 #define SAMPLING_MAXIMUM_ROWS 16u    // rows of a lane's verify block
 #define SAMPLING_STOP_TOKENS 4u
+#define SAMPLING_CANDIDATES 16u     // candidates of a row's next position (SPLASH_DRAFT_CANDIDATES)
+#define SAMPLING_TREE_CHILDREN 4u   // children a row's draft draws at most (SPLASH_TREE_CHILDREN)
+#define SAMPLING_NO_DRAW 0xFFu      // past a row's drawn children
 #define SAMPLING_NO_TOKEN 0xFFFFFFFFu  // a row with no selectable logit selects it (SPLASH_NO_TOKEN)
 // A sampled row's words of the decisions buffer: the accepted child or SAMPLING_NO_TOKEN, whether
 // the row draws from the residual, then the end of its distribution in the order of the logits
@@ -46,7 +49,10 @@ struct TargetSamplingParams {
   float top_p[SAMPLING_MAXIMUM_LANES];
   uint32_t mask_words;      // words of a constraint-mask row (one a packed row): bit t % 32 of word t / 32 admits token t
   uint32_t stop_tokens[SAMPLING_STOP_TOKENS];
-  uint32_t reserved[3];
+  // A tree block's sampled rows test the children their draft drew among SAMPLING_CANDIDATES candidates
+  // (decode_sample_draw_children) instead of one child against a full-vocabulary draft distribution.
+  uint32_t candidate_children;
+  uint32_t reserved[2];
 };
 
 // draft_verify_rows: one workgroup lays out a decode step's rows from the trees a draft selector grew (the reference's

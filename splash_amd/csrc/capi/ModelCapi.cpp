@@ -91,7 +91,8 @@ sp_status spo_sampling_add_verify(spo_graph *graph, const spo_sampling_buffers *
     capi::require(graph && b && lanes && policy, "graph, buffers, lanes or policies");
     ops::SamplingBuffers buffers{B(b->logits), B(b->tokens), B(b->partial_values), B(b->partial_indices), B(b->draft_probabilities),
                                  B(b->uniforms), B(b->masses), B(b->ranges), B(b->decisions), B(b->input_tokens), B(b->tree_rows),
-                                 B(b->token_mask), b->mask_words};
+                                 B(b->token_mask), b->mask_words, B(b->candidate_ids), B(b->candidate_probabilities), B(b->candidate_draws),
+                                 B(b->child_uniforms)};
     std::vector<ops::LaneRows> rows;
     std::vector<ops::SamplingPolicy> policies;
     for (uint32_t i = 0; i < count; ++i) { rows.push_back({lanes[i].first, lanes[i].rows}); policies.push_back({policy[i].temperature, policy[i].min_p, policy[i].top_k, policy[i].top_p, policy[i].constrained != 0, policy[i].excludes_stop_tokens != 0}); }

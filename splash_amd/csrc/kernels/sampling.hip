@@ -572,7 +572,8 @@ __global__ __launch_bounds__(256) void decode_sample_residual_ranges(const float
   const float inverse = 1.0f / p.temperature[laneIndex];
   const Kept kept = row_kept(masses, decisions, row, inverse, (p.truncating_mask >> laneIndex) & 1u);
   const float *x = logits + size_t(row) * p.logits_stride, *q = draft + size_t(row) * p.logits_stride;
-  const uint32_t child = child_token(p, tree, input_tokens, row);
+  // a row that tests candidate children sums the ranges of its whole distribution: the draw kernel does the tests
+  const uint32_t child = p.candidate_children ? SAMPLING_NO_TOKEN : child_token(p, tree, input_tokens, row);
   bool rejected = false;
   if (child != SAMPLING_NO_TOKEN && child < p.vocabulary) {
     // accept iff u_child * q < p (sampling.metal:790-800)
@@ -674,6 +675,170 @@ __global__ __launch_bounds__(64) void decode_sample_draw(const float *__restrict
   }
 }
 SP_REGISTER_KERNEL("decode_sample_draw", &decode_sample_draw);
+
+// decode_sample_draw_children (the rule of the reference's vocabulary_draw with children, sampling.metal:697-880): grid
+// (rows), 64 threads. A sampled row of a tree block tests the children its draft drew among its SAMPLING_CANDIDATES
+// candidates -- ids [row][16], their draft probabilities q [row][16], the candidate indices drawn in order draws
+// [row][4] (bytes, SAMPLING_NO_DRAW past them), a uniform a child child_uniforms [row][4] -- by recursive rejection
+// sampling without replacement: child c is selected iff u_c q_c < p_c; a rejection leaves the target its residual
+// max(p - q, 0) over the candidates and its mass outside them, renormalized, and the draft its rest, renormalized. A
+// row that selects none draws at u_row of the last residual: a candidate in index order, or past them a token
+// outside them in id order by the target's own weights. The ranges hold the row's kept weights (the ranges kernel
+// ran without a child); the candidates' weights leave them here. Lanes 0..15 weigh a candidate each, lane 0 decides,
+// the wavefront walks the drawn range.
+__global__ __launch_bounds__(64) void decode_sample_draw_children(const float *__restrict__ logits, const float *__restrict__ masses,
+                                                                  const float *__restrict__ uniforms, const float *__restrict__ ranges,
+                                                                  const uint32_t *__restrict__ decisions,
+                                                                  const uint32_t *__restrict__ candidate_ids,
+                                                                  const float *__restrict__ candidate_q,
+                                                                  const uint8_t *__restrict__ draws,
+                                                                  const float *__restrict__ child_uniforms,
+                                                                  uint32_t *__restrict__ tokens, TargetSamplingParams p) {
+  constexpr uint32_t K = SAMPLING_CANDIDATES;
+  __shared__ float rangeWeight[SAMPLING_RANGES];
+  __shared__ float candidateWeight[K];
+  __shared__ uint32_t excludedIds[K];
+  __shared__ uint32_t decided[4];  // selected (1) or walking (0), token or range, target bits, excluding
+  const uint32_t row = blockIdx.x, lane = threadIdx.x;
+  const uint32_t laneIndex = lane_of_row(p, row);
+  if (!((p.sampling_mask >> laneIndex) & 1u)) return;  // a greedy lane keeps its argmax
+  const float inverse = 1.0f / p.temperature[laneIndex];
+  const Kept kept = row_kept(masses, decisions, row, inverse, (p.truncating_mask >> laneIndex) & 1u);
+  const float *x = logits + size_t(row) * p.logits_stride;
+  const uint32_t size = range_tokens(p.vocabulary);
+  for (uint32_t j = lane; j < SAMPLING_RANGES; j += 64u) rangeWeight[j] = ranges[row * SAMPLING_RANGES + j];
+  if (lane < K) {
+    const uint32_t id = candidate_ids[row * K + lane];
+    excludedIds[lane] = id;
+    candidateWeight[lane] = id < p.vocabulary ? kept_weight(x[id], id, kept, inverse) : 0.f;
+  }
+  __syncthreads();
+  if (lane == 0) {
+    float total = 0.f;
+    for (uint32_t j = 0; j < SAMPLING_RANGES; ++j) total += rangeWeight[j];
+    bool selected = false, excluding = false;
+    uint32_t token = SAMPLING_NO_TOKEN;
+    float target = uniforms[2 * row] * total;
+    const uint8_t *drawn = draws + row * SAMPLING_TREE_CHILDREN;
+    if (!(total > 0.f)) {
+      selected = true;  // nothing selectable: the sentinel
+    } else if (drawn[0] != SAMPLING_NO_DRAW) {
+      float pc[K], qc[K];
+      for (uint32_t i = 0; i < K; ++i) {
+        const uint32_t id = excludedIds[i];
+        const float weight = candidateWeight[i];
+        if (id < p.vocabulary) rangeWeight[id / size] = fmaxf(rangeWeight[id / size] - weight, 0.f);
+        pc[i] = weight / total;
+        qc[i] = candidate_q[row * K + i];
+      }
+      float outsideWeight = 0.f;
+      for (uint32_t j = 0; j < SAMPLING_RANGES; ++j) outsideWeight += rangeWeight[j];
+      float outside = outsideWeight / total;
+      for (uint32_t child = 0; child < SAMPLING_TREE_CHILDREN && !selected; ++child) {
+        const uint32_t c = drawn[child];
+        if (c >= K) break;
+        // a dynamic index into a register array would spill: pick the child's p and q by comparison
+        float pChild = 0.f, qChild = 0.f;
+        for (uint32_t i = 0; i < K; ++i) { pChild = i == c ? pc[i] : pChild; qChild = i == c ? qc[i] : qChild; }
+        if (child_uniforms[row * SAMPLING_TREE_CHILDREN + child] * qChild < pChild) {
+          selected = true;
+          token = excludedIds[c];
+          break;
+        }
+        float residual = outside;
+        for (uint32_t i = 0; i < K; ++i) residual += fmaxf(pc[i] - qc[i], 0.f);
+        if (!(residual > 0.f)) break;
+        for (uint32_t i = 0; i < K; ++i) pc[i] = fmaxf(pc[i] - qc[i], 0.f) / residual;
+        outside /= residual;
+        float rest = 0.f;
+        for (uint32_t i = 0; i < K; ++i) { qc[i] = i == c ? 0.f : qc[i]; rest += qc[i]; }
+        for (uint32_t i = 0; rest > 0.f && i < K; ++i) qc[i] /= rest;
+      }
+      if (!selected) {
+        float inside = 0.f;
+        for (uint32_t i = 0; i < K; ++i) inside += pc[i];
+        const float point = uniforms[2 * row] * (inside + outside);
+        float cumulative = 0.f;
+        uint32_t last = K;
+        for (uint32_t i = 0; i < K && !(point < cumulative); ++i)
+          if (pc[i] > 0.f) {
+            last = i;
+            cumulative += pc[i];
+          }
+        if (last < K && (point < cumulative || !(outside > 0.f))) {
+          selected = true;
+          token = excludedIds[last];
+        } else {
+          excluding = true;
+          target = (point - inside) / outside * outsideWeight;
+        }
+      }
+    }
+    uint32_t hit = 0;
+    float within = 0.f;
+    if (!selected) {
+      // the first weighted range whose end lies past the target; the last weighted one on a rounding shortfall
+      float cumulative = 0.f;
+      for (uint32_t j = 0; j < SAMPLING_RANGES; ++j) {
+        const float weight = rangeWeight[j];
+        if (!(weight > 0.f)) continue;
+        hit = j;
+        within = target - cumulative;
+        cumulative += weight;
+        if (cumulative > target) break;
+      }
+    }
+    decided[0] = selected ? 1u : 0u;
+    decided[1] = selected ? token : hit;
+    decided[2] = __builtin_bit_cast(uint32_t, within);
+    decided[3] = excluding ? 1u : 0u;
+  }
+  __syncthreads();
+  if (decided[0]) {
+    if (lane == 0) tokens[row] = decided[1];
+    return;
+  }
+  const uint32_t hit = decided[1];
+  const bool excluding = decided[3] != 0u;
+  float target = __builtin_bit_cast(float, decided[2]);
+  auto weigh = [&](uint32_t token) {
+    bool out = false;
+    if (excluding)
+      for (uint32_t i = 0; i < K; ++i) out = out || excludedIds[i] == token;
+    return out ? 0.f : kept_weight(x[token], token, kept, inverse);
+  };
+  // the range's lanes' chunks, as the ranges kernel summed them (less the candidates), walked in lane order
+  const uint32_t begin = hit * size, end = min(p.vocabulary, begin + size), per = (size + 63u) / 64u;
+  float sum = 0.f;
+  for (uint32_t i = 0; i < per; ++i) {
+    const uint32_t token = begin + lane * per + i;
+    if (token < end) sum += weigh(token);
+  }
+  uint32_t chunk = 64, lastChunk = 0;
+  float chunkBefore = 0.f, lastChunkBefore = 0.f, cumulative = 0.f;
+  for (int l = 0; l < 64; ++l) {
+    const float c = __shfl(sum, l, 64);
+    if (c > 0.f) { lastChunk = uint32_t(l); lastChunkBefore = cumulative; }
+    if (chunk == 64 && c > 0.f && target < cumulative + c) { chunk = uint32_t(l); chunkBefore = cumulative; }
+    cumulative += c;
+  }
+  if (chunk == 64) { chunk = lastChunk; chunkBefore = lastChunkBefore; }
+  target -= chunkBefore;
+  if (lane == 0) {
+    uint32_t selected = SAMPLING_NO_TOKEN, lastToken = SAMPLING_NO_TOKEN;
+    float walked = 0.f;
+    for (uint32_t i = 0; i < per; ++i) {
+      const uint32_t token = begin + chunk * per + i;
+      if (token >= end) break;
+      const float w = weigh(token);
+      if (w > 0.f) lastToken = token;
+      walked += w;
+      if (selected == SAMPLING_NO_TOKEN && w > 0.f && target < walked) selected = token;
+    }
+    tokens[row] = selected != SAMPLING_NO_TOKEN ? selected : lastToken;
+  }
+}
+SP_REGISTER_KERNEL("decode_sample_draw_children", &decode_sample_draw_children);
 
 } // namespace splash::kernels
 

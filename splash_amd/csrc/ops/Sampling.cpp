@@ -67,8 +67,17 @@ void Sampling::addVerify(hip::CommandGraph &graph, const SamplingBuffers &b, uin
   requireBytes(b.tokens, uint64_t{rows} * 4, "selected tokens");
   requireBytes(b.partialValues, need.partialValues, "argmax partial values");
   requireBytes(b.partialIndices, need.partialIndices, "argmax partial indices");
+  const bool children = bool(b.candidateIds);
+  params.candidate_children = children ? 1u : 0u;
   if (params.sampling_mask) {
-    requireBytes(b.draftProbabilities, (uint64_t{rows - 1} * logitsStride + vocabulary) * 4, "draft probabilities");
+    if (children) {
+      requireBytes(b.candidateIds, uint64_t{rows} * SAMPLING_CANDIDATES * 4, "candidate ids");
+      requireBytes(b.candidateProbabilities, uint64_t{rows} * SAMPLING_CANDIDATES * 4, "candidate probabilities");
+      requireBytes(b.candidateDraws, uint64_t{rows} * SAMPLING_TREE_CHILDREN, "drawn children");
+      requireBytes(b.childUniforms, uint64_t{rows} * SAMPLING_TREE_CHILDREN * 4, "child uniforms");
+    } else {
+      requireBytes(b.draftProbabilities, (uint64_t{rows - 1} * logitsStride + vocabulary) * 4, "draft probabilities");
+    }
     requireBytes(b.uniforms, uint64_t{rows} * 8, "sampling uniforms");
     requireBytes(b.masses, need.masses, "sampling masses");
     requireBytes(b.ranges, need.ranges, "sampling ranges");
@@ -87,11 +96,18 @@ void Sampling::addVerify(hip::CommandGraph &graph, const SamplingBuffers &b, uin
   graph.add("decode_sample_mass_sharded", {b.logits, b.masses}, params, {rows * SAMPLING_SHARDS, 1, 1}, {SAMPLING_THREADS, 1, 1});
   if (params.truncating_mask)
     graph.add("decode_sample_distribution_end", {b.logits, b.masses, b.decisions}, params, {rows, 1, 1}, {SAMPLING_THREADS, 1, 1});
+  // with candidate children no full-vocabulary draft distribution is read: the logits stand in for its binding
   graph.add("decode_sample_residual_ranges",
-            {b.logits, b.draftProbabilities, b.masses, b.uniforms, b.treeRows, b.inputTokens, b.ranges, b.decisions}, params,
-            {rows * (SAMPLING_RANGES / 4), 1, 1}, {256, 1, 1});
-  graph.add("decode_sample_draw", {b.logits, b.draftProbabilities, b.masses, b.uniforms, b.ranges, b.decisions, b.tokens}, params,
-            {rows, 1, 1}, {64, 1, 1});
+            {b.logits, children ? b.logits : b.draftProbabilities, b.masses, b.uniforms, b.treeRows, b.inputTokens, b.ranges, b.decisions},
+            params, {rows * (SAMPLING_RANGES / 4), 1, 1}, {256, 1, 1});
+  if (children)
+    graph.add("decode_sample_draw_children",
+              {b.logits, b.masses, b.uniforms, b.ranges, b.decisions, b.candidateIds, b.candidateProbabilities, b.candidateDraws,
+               b.childUniforms, b.tokens},
+              params, {rows, 1, 1}, {64, 1, 1});
+  else
+    graph.add("decode_sample_draw", {b.logits, b.draftProbabilities, b.masses, b.uniforms, b.ranges, b.decisions, b.tokens}, params,
+              {rows, 1, 1}, {64, 1, 1});
 }
 
 void Sampling::addAcceptance(hip::CommandGraph &graph, const AcceptanceBuffers &b, const std::vector<LaneRows> &lanes,

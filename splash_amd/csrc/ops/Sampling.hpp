@@ -55,6 +55,11 @@ struct SamplingBuffers final {
   // Constrained lanes only: uint32 [rows][maskWords], bit t % 32 of word t / 32 of a row admits token t.
   hip::Buffer tokenMask;
   uint32_t maskWords = 0;
+  // A tree block's sampled rows (Sampling.hpp:119-136 in the reference, DrawChildren): each row's sixteen candidates
+  // (uint32 ids and fp32 draft probabilities [rows][16]), the candidate indices of the children its draft drew, in the
+  // order drawn (bytes [rows][4], 0xFF past them), and a uniform for each child's test (fp32 [rows][4]). With these the
+  // sampled lanes' rows run recursive rejection sampling over their children; draftProbabilities is then not read.
+  hip::Buffer candidateIds, candidateProbabilities, candidateDraws, childUniforms;
 };
 struct AcceptanceBuffers final {
   hip::Buffer inputTokens;    // uint32 [rows]

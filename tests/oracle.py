@@ -587,3 +587,32 @@ def moe_shared_weights(x_bits, gate):
     out = np.empty(x.shape[0], np.float32)
     lib.orc_moe_shared_weights(_p(x, u16p), _p(g, f32p), x.shape[0], x.shape[1], _p(out, f32p))
     return out
+
+
+# ---- a tree block's sampled rows: up to four drawn children among sixteen candidates ----
+def children_row(logits, policy, ids, q, draws, u_children, u_row):
+    """orc_children_row: (token, closeness). policy: (temperature, min_p, top_k, top_p); draws: candidate indices in the
+    order drawn (at most four)."""
+    x = np.ascontiguousarray(logits, np.float32)
+    ids = np.ascontiguousarray(ids, np.uint32)
+    q = np.ascontiguousarray(q, np.float32)
+    d = np.full(4, 0xFF, np.uint8)
+    d[:len(draws)] = draws
+    u = np.zeros(4, np.float32)
+    u[:len(u_children)] = u_children
+    pol = SamplingPolicy(*policy)
+    close = ctypes.c_double()
+    lib.orc_children_row.restype = c_u32
+    token = lib.orc_children_row(_p(x, f32p), c_u32(x.size), ctypes.byref(pol), _p(ids, u32p), _p(q, f32p), _p(d, u8p), c_u32(len(draws)),
+                                 _p(u, f32p), c_f(u_row), ctypes.byref(close))
+    return token, close.value
+
+
+def children_law(p_target, ids, q, n_draws):
+    p = np.ascontiguousarray(p_target, np.float64)
+    ids = np.ascontiguousarray(ids, np.uint32)
+    q = np.ascontiguousarray(q, np.float64)
+    out = np.zeros(p.size, np.float64)
+    lib.orc_children_law.restype = None
+    lib.orc_children_law(_p(p, f64p), c_u32(p.size), _p(ids, u32p), _p(q, f64p), c_u32(n_draws), _p(out, f64p))
+    return out

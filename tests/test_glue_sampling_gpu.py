@@ -190,6 +190,70 @@ def test_rejection_sampling_rows_match_oracle(backend):
     assert all(mixed[r] == orc.argmax(logits[r]) for r in range(8))
 
 
+@pytest.mark.parametrize("V,policy", [(151936, (0.7, 0.0, 0, 1.0)), (32000, (0.9, 0.0, 40, 0.95))])
+def test_tree_rows_test_their_drawn_children(backend, V, policy):
+    """sampling.metal:697-880 (vocabulary_draw with children): every sampled row of a tree block tests the children its
+    draft drew among sixteen candidates, one to four of them or none, then draws from the last residual: among the
+    candidates or, past them, outside them. Token for token the oracle's, except where one of its comparisons lies within
+    1e-5 of its threshold (target_sampling_metal_test.mm:2645-2709); a greedy lane beside keeps its argmax."""
+    print(f"case children rows V={V}", flush=True)
+    rng = np.random.default_rng(V)
+    rows, K = 16, 16
+    logits = (rng.standard_normal((rows, V)) * 2.5).astype(np.float32)
+    logits[2, rng.random(V) < 0.02] = -np.inf
+    for r in (1, 4, 6, 9):                                 # peaked rows: a child that is the likeliest token is accepted
+        logits[r, rng.integers(0, V, 2)] += np.float32(14.0)
+    T = policy[0]
+    ids = np.zeros((rows, K), np.uint32)
+    q = np.zeros((rows, K), np.float32)
+    draws = np.full((rows, 4), 0xFF, np.uint8)
+    for r in range(rows):
+        # the candidates: the row's likeliest tokens mixed with random ones, so that children are accepted and rejected
+        top = np.argsort(-logits[r])[:8]
+        ids[r] = rng.permutation(np.concatenate([top, rng.choice(V, 8, replace=False)]))[:K]
+        if r == 5:
+            ids[r, 12:] = 0xFFFFFFFF                    # a draft row of fewer comparable logits
+        weights = -np.log(0.5 * (rng.random(K) + 1.0))
+        weights[ids[r] >= V] = 0
+        if r % 3 == 0:
+            weights[rng.integers(0, K, 3)] = 0
+        q[r] = (weights / weights.sum()).astype(np.float32)
+        count = r % 5                                   # 0 .. 4 children
+        keys = sorted(((np.log(q[r, i]) - np.log(-np.log(rng.random() + 1e-300)), i) for i in range(K) if q[r, i] > 0), reverse=True)
+        for c, (_, i) in enumerate(keys[:count]):
+            draws[r, c] = i
+    if True:   # a row whose candidates hold none of its mass and whose children are all rejected: the draw lands outside them
+        ids[7] = rng.choice(np.where(logits[7] < -3)[0], K, replace=False)
+        draws[7] = [0, 1, 2, 3]
+    child_uniforms = rng.random((rows, 4)).astype(np.float32)
+    uniforms = rng.random((rows, 2)).astype(np.float32)
+    tokens = rng.integers(0, V, rows).astype(np.uint32)
+    tree = ops.chain_tree_rows([rows])
+    b = sampling_buffers(backend, rows, V, logits, None, uniforms, tokens, tree)
+    b.update(candidate_ids=backend.from_array(ids), candidate_probabilities=backend.from_array(q), candidate_draws=backend.from_array(draws),
+             child_uniforms=backend.from_array(child_uniforms))
+    g = splash_amd.CommandGraph()
+    ops.Sampling.add_verify(g, b, V, V, [(0, 12), (12, 4)], [policy, 0.0])
+    assert "decode_sample_draw_children" in g.kernels() and "decode_sample_draw" not in g.kernels()
+    backend.run(g)
+    got = b["tokens"].download(np.uint32)
+    checked = children_selected = outside = 0
+    for r in range(12):
+        n = int((draws[r] != 0xFF).sum())
+        want, close = orc.children_row(logits[r], policy, ids[r], q[r], list(draws[r, :n]), child_uniforms[r], float(uniforms[r, 0]))
+        if close > 1e-5:
+            assert got[r] == want, (r, n, got[r], want)
+            checked += 1
+            children_selected += int(n and got[r] in ids[r, draws[r, :n]])
+            outside += int(got[r] not in ids[r])
+    assert checked >= 9 and children_selected >= 1 and outside >= 1
+    assert all(got[r] == orc.argmax(logits[r]) for r in range(12, 16))
+    # the buffers are checked before anything is added
+    short = dict(b, candidate_draws=backend.allocate_buffer(16))
+    with pytest.raises(ValueError, match="drawn children"):
+        ops.Sampling.add_verify(splash_amd.CommandGraph(), short, V, V, [(0, 12), (12, 4)], [policy, 0.0])
+
+
 @pytest.mark.parametrize("ties", [False, True])
 def test_truncated_distributions_match_oracle(backend, ties):
     """min_p, top_k and top_p (distribution_end, sampling.metal:603-670): the end of every row's distribution -- the

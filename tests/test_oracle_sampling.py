@@ -259,3 +259,93 @@ def test_draft_edges_are_the_trilinear_sums():
     scale = np.abs(bf16_values(hidden)).max() * np.abs(bf16_values(before)).max() * np.abs(bf16_values(after)).max() * 256
     assert np.abs(got[written] - want[written]).max() <= 2.0 ** -22 * scale
     assert np.abs(want[written]).max() > 10      # the scores are far from zero: a dropped factor would show
+
+
+# ------------------------------------------------------------------ a tree block's sampled rows (sampling.metal:697-880)
+def _dirichlet(rng, n, zeros):
+    v = -np.log(0.5 * (rng.random(n) + 1.0) + 1e-9)
+    v[rng.integers(0, n, zeros)] = 0.0
+    return v / v.sum()
+
+
+def test_children_law_is_the_target_distribution_whatever_the_draft():
+    """The proof harness of the reference (target_sampling_metal_test.mm:2602-2631): over 300 random targets and drafts of
+    one to four children, some candidates outside the target's support and some of its mass outside the candidates, the
+    enumerated law of the selection is the target's to 1e-12. A wrong residual, a missing renormalization of p or of
+    the draft's rest, or a draw past the candidates that forgets their mass all break it."""
+    rng = np.random.default_rng(0x7272)
+    worst = 0.0
+    for trial in range(300):
+        p = _dirichlet(rng, 24, trial % 5)
+        ids = rng.permutation(24)[:16].astype(np.uint32)
+        q = _dirichlet(rng, 16, trial % 7)
+        law = orc.children_law(p, ids, q, 1 + trial % 4)
+        worst = max(worst, float(np.abs(law - p).max()))
+    assert worst < 1e-12, worst
+    # candidates past the vocabulary (a draft row of fewer comparable logits lists 0xffffffff) weigh nothing
+    p = _dirichlet(rng, 10, 0)
+    ids = np.concatenate([rng.permutation(10)[:6], np.full(10, 0xFFFFFFFF)]).astype(np.uint32)
+    q = np.concatenate([_dirichlet(rng, 6, 0), np.zeros(10)])
+    assert np.abs(orc.children_law(p, ids, q, 3) - p).max() < 1e-12
+
+
+def _gumbel_draws(rng, q, count):
+    keys = [(np.log(q[i]) - np.log(-np.log(rng.random() + 1e-300)), i) for i in range(len(q)) if q[i] > 0]
+    return [i for _, i in sorted(keys, reverse=True)[:count]]
+
+
+def test_children_row_follows_the_target_distribution():
+    """The row itself over many seeds (the reference's followsDistribution, target_sampling_metal_test.mm:3019): children
+    drawn without replacement from q, uniform tests and draws; the selected tokens' frequencies are the target's."""
+    rng = np.random.default_rng(9)
+    V, T, N = 40, 0.8, 30000
+    logits = (rng.standard_normal(V) * 1.5).astype(np.float32)
+    logits[[3, 17]] = -np.inf
+    p = np.where(np.isfinite(logits), np.exp((logits.astype(np.float64) - logits[np.isfinite(logits)].max()) / T), 0)
+    p /= p.sum()
+    ids = rng.permutation(V)[:16].astype(np.uint32)
+    q = _dirichlet(rng, 16, 2).astype(np.float32)
+    for draws_n in (1, 4):
+        counts = np.zeros(V)
+        for _ in range(N):
+            draws = _gumbel_draws(rng, q.astype(np.float64), draws_n)
+            token, _ = orc.children_row(logits, (T, 0.0, 0, 1.0), ids, q, draws, rng.random(4).astype(np.float32), float(rng.random()))
+            counts[token] += 1
+        freq = counts / N
+        assert np.all(np.abs(freq - p) <= 4 * np.sqrt(p * (1 - p) / N) + 5e-4), (draws_n, np.abs(freq - p).max())
+        assert counts[3] == 0 and counts[17] == 0
+
+
+def test_children_row_decisions_at_their_thresholds():
+    rng = np.random.default_rng(10)
+    V, T = 64, 0.7
+    logits = (rng.standard_normal(V) * 2).astype(np.float32)
+    w = np.exp((logits.astype(np.float64) - logits.max()) / T)
+    p = w / w.sum()
+    ids = np.arange(8, 24).astype(np.uint32)
+    q = np.full(16, 1 / 16, np.float32)
+    policy = (T, 0.0, 0, 1.0)
+    # a child is selected iff u q < p: just below and just above the threshold p / q
+    c = 5
+    threshold = p[ids[c]] / q[c]
+    if threshold < 1:
+        assert orc.children_row(logits, policy, ids, q, [c], [np.float32(threshold * 0.999)], 0.5)[0] == ids[c]
+        assert orc.children_row(logits, policy, ids, q, [c], [np.float32(min(threshold * 1.001, 0.99999))], 0.5)[0] != ids[c] or threshold * 1.001 >= 1
+    assert orc.children_row(logits, policy, ids, q, [c], [0.0], 0.5)[0] == ids[c]                 # u = 0 always accepts a possible child
+    # a second child is tested after the first is rejected, against the residual: with q concentrated on the first child
+    # (q0 = 1 - eps), its rejection leaves p almost untouched elsewhere and the draft's rest uniform over the others
+    q2 = np.full(16, 1e-3 / 15, np.float32); q2[0] = 1 - 1e-3
+    token, _ = orc.children_row(logits, policy, ids, q2, [0, 7], [0.999999, 0.0], 0.5)
+    assert token == ids[7]
+    # no children: the row draws from its whole distribution, exactly as the one-child rule's row without a child does
+    for u in (0.0, 0.3, 0.77, 0.999):
+        assert orc.children_row(logits, policy, ids, q, [], [], u)[0] == orc.rejection_row(logits, T, None, orc.NO_TOKEN, 0.0, u)[0]
+    # every child rejected and all of the target's mass on the candidates' complement: the draw lands outside them
+    far = np.full(V, -np.inf, np.float32); far[[40, 50]] = [0.0, 1.0]
+    token, _ = orc.children_row(far, policy, ids, q, [1, 2, 3, 4], [0.5] * 4, 0.99)
+    assert token in (40, 50)
+    # the draw over the candidates walks them in index order: with the mass on candidates only, u_row picks by cumulative p
+    only = np.full(V, -np.inf, np.float32); only[ids[2]] = 0.0; only[ids[9]] = 0.0
+    qz = np.zeros(16, np.float32); qz[0] = 1.0                                      # the drawn child has no target mass: rejected
+    assert orc.children_row(only, policy, ids, qz, [0], [0.5], 0.25)[0] == ids[2]
+    assert orc.children_row(only, policy, ids, qz, [0], [0.5], 0.75)[0] == ids[9]
