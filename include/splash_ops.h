@@ -357,7 +357,11 @@ typedef enum spo_verify_buffer {
   SPO_VERIFY_INPUT_TOKENS = 0, SPO_VERIFY_TREE_ROWS, SPO_VERIFY_DEPTHS, SPO_VERIFY_UNIFORMS, SPO_VERIFY_TOKENS,
   SPO_VERIFY_RETAINED, SPO_VERIFY_ACCEPTED, SPO_VERIFY_RETAINED_ROWS, SPO_VERIFY_PAGE_TABLE, SPO_VERIFY_KV_POOL,
   SPO_VERIFY_LOGITS, SPO_VERIFY_DRAFT_PROBABILITIES, SPO_VERIFY_HIDDEN,
-  SPO_VERIFY_QKV_ROWS = 15, SPO_VERIFY_ATTENTION_ROWS = 16, SPO_VERIFY_FFN_ROWS = 17
+  SPO_VERIFY_QKV_ROWS = 15, SPO_VERIFY_ATTENTION_ROWS = 16, SPO_VERIFY_FFN_ROWS = 17,
+  /* the sampled rows' candidate children (spo_sampling_buffers): index 0 ids, 1 probabilities, 2 drawn children, 3 child
+     uniforms; host-visible, allocated by the first call, after which every step's sampled lanes test candidate
+     children instead of one child against the full-vocabulary draft probabilities */
+  SPO_VERIFY_CANDIDATE_CHILDREN = 18
 } spo_verify_buffer;
 sp_status spo_dense_verify_buffer(spo_dense_verify *verify, spo_verify_buffer which, uint32_t index, sp_buffer **out);
 uint64_t spo_dense_verify_page_bytes(const spo_dense_verify *verify);

@@ -219,6 +219,7 @@ sp_status spo_dense_verify_buffer(spo_dense_verify *verify, spo_verify_buffer wh
     case SPO_VERIFY_QKV_ROWS: b = v.qkvRows(); break;
     case SPO_VERIFY_ATTENTION_ROWS: b = v.attentionRows(); break;
     case SPO_VERIFY_FFN_ROWS: b = v.ffnRows(); break;
+    case SPO_VERIFY_CANDIDATE_CHILDREN: b = v.candidateChildren(index); break;
     default: throw std::invalid_argument("no such verify buffer");
     }
     sp_buffer_retain(b.handle());

@@ -90,6 +90,27 @@ const hip::Buffer &DenseVerify::draftProbabilities() {
   return draft_;
 }
 
+const hip::Buffer &DenseVerify::candidateChildren(uint32_t which) {
+  if (!sampling_.candidateIds) {
+    const uint64_t R = maxRows_;
+    auto shared = [&](uint64_t bytes, const char *label) { return backend_.allocateBuffer(bytes, BufferStorage::Shared, label); };
+    sampling_.candidateIds = shared(R * SAMPLING_CANDIDATES * 4, "candidate ids");
+    sampling_.candidateProbabilities = shared(R * SAMPLING_CANDIDATES * 4, "candidate probabilities");
+    sampling_.candidateDraws = shared(R * SAMPLING_TREE_CHILDREN, "drawn children");
+    sampling_.childUniforms = shared(R * SAMPLING_TREE_CHILDREN * 4, "child uniforms");
+    // no children drawn until a draft says so: such rows draw from their whole distribution
+    std::vector<uint8_t> none(R * SAMPLING_TREE_CHILDREN, uint8_t(SAMPLING_NO_DRAW));
+    sampling_.candidateDraws.upload(none.data(), none.size());
+  }
+  switch (which) {
+  case 0: return sampling_.candidateIds;
+  case 1: return sampling_.candidateProbabilities;
+  case 2: return sampling_.candidateDraws;
+  case 3: return sampling_.childUniforms;
+  default: throw std::invalid_argument("no such candidate buffer");
+  }
+}
+
 uint64_t DenseVerify::stepBytes(const std::vector<VerifyLane> &lanes) const {
   uint64_t bytes = weights_.head.weightBytes();
   for (const DenseLayer &l : weights_.layers)
@@ -190,7 +211,7 @@ void DenseVerify::encode(hip::CommandGraph &graph, const std::vector<VerifyLane>
   }
   const ops::AttentionGeometry geometry{dims_.qHeads, dims_.kvHeads, dims_.headDimension, dims_.rotaryPairs, dims_.normalizeHeads};
   const ops::AttentionPlan plan = ops::PagedAttention::plan(geometry, sequences);
-  if (samples) (void)draftProbabilities();
+  if (samples && !sampling_.candidateIds) (void)draftProbabilities();
   if (dims_.rotaryPairs)
     ops::RoPE::addTreeTables(graph, inverseFrequency_, depths_, ropeCos_, ropeSin_, dims_.rotaryPairs, rope);
   encodeEmbedding(graph, rows);

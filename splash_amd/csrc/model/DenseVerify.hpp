@@ -70,6 +70,11 @@ public:
   [[nodiscard]] const hip::Buffer &kvPool(uint32_t layer) const { return kvPools_.at(layer); }
   [[nodiscard]] const hip::Buffer &logits() const noexcept { return logits_; }
   [[nodiscard]] const hip::Buffer &draftProbabilities();  // allocated on first use
+  // The sampled rows of tree blocks test the children their draft drew among sixteen candidates (Sampling.hpp,
+  // candidateIds ..): the four host-visible buffers a draft writes, allocated on first use -- which: 0 ids uint32
+  // [rows][16], 1 probabilities fp32 [rows][16], 2 drawn children bytes [rows][4], 3 child uniforms fp32 [rows][4].
+  // Once they exist, every step's sampled lanes read them instead of the full-vocabulary draft probabilities.
+  [[nodiscard]] const hip::Buffer &candidateChildren(uint32_t which);
   [[nodiscard]] const hip::Buffer &hidden(uint32_t index) const noexcept { return hidden_[index & 1]; }
   [[nodiscard]] const hip::Buffer &qkvRows() const noexcept { return qkv_; }
   [[nodiscard]] const hip::Buffer &attentionRows() const noexcept { return attention_; }

@@ -11,7 +11,7 @@ from .backend import Buffer, CommandGraph, STORAGE_PRIVATE
 from . import ops
 
 (INPUT_TOKENS, TREE_ROWS, DEPTHS, UNIFORMS, TOKENS, RETAINED, ACCEPTED, RETAINED_ROWS, PAGE_TABLE, KV_POOL, LOGITS,
- DRAFT_PROBABILITIES, HIDDEN, GDN_STATES, GDN_TAPE, QKV_ROWS, ATTENTION_ROWS, FFN_ROWS) = range(18)
+ DRAFT_PROBABILITIES, HIDDEN, GDN_STATES, GDN_TAPE, QKV_ROWS, ATTENTION_ROWS, FFN_ROWS, CANDIDATE_CHILDREN) = range(19)
 
 
 class Lane:
@@ -105,6 +105,13 @@ class DenseVerify:
             self.buffer(UNIFORMS).contents()[:rows * 8] = np.asarray(uniforms, dtype=np.float32).reshape(rows, 2).view(np.uint8).ravel()
 
     _results_call = "spo_dense_verify_results"
+
+    def set_candidate_children(self, ids, probabilities, draws, child_uniforms):
+        """The sampled rows' candidate children, by packed row: ids uint32 [rows][16], probabilities fp32 [rows][16], draws
+        bytes [rows][4] (0xFF past a row's drawn children), child_uniforms fp32 [rows][4]."""
+        for which, array, dtype in ((0, ids, np.uint32), (1, probabilities, np.float32), (2, draws, np.uint8), (3, child_uniforms, np.float32)):
+            raw = np.ascontiguousarray(array, dtype).view(np.uint8).ravel()
+            self.buffer(CANDIDATE_CHILDREN, which).contents()[:raw.size] = raw
 
     def results(self, lanes):
         """(selected/retained tokens per packed row, retained count, accepted count, retained-row mask) per lane, read

@@ -149,3 +149,63 @@ def test_a_context_built_from_tokens_alone(backend):
     picks = np.array([orc.argmax(got[r]) for r in range(16)], dtype=np.uint32)
     kept, acc, m = orc.accept_tree(ops.chain_tree_rows([16]), draft, picks)
     assert retained[0] == len(kept) and accepted[0] == acc and mask[0] == m and np.array_equal(selected[:len(kept)], kept)
+
+
+def test_a_sampled_tree_block_tests_its_drawn_children(backend):
+    """A tree block through the driver with sampled acceptance: every row tests the children its draft drew among its
+    sixteen candidates (sampling.metal:697-880), the acceptance walk follows the selected children. The candidates of a
+    row are the likeliest tokens of the target itself at that row (found by running the step as the tree grows), so
+    children are accepted and rejected; against the oracle's rows over the step's own logits and its walk."""
+    print("case config 1 sampled tree block", flush=True)
+    V, T, rows = 32000, 0.03, 8          # a peaked target: its likeliest token is accepted, the others seldom
+    model = DenseModel(seed=14, hidden=1024, q_heads=16, kv_heads=8, head_dim=64, ffn=3072, vocabulary=V, layers=2)
+    rng = np.random.default_rng(8)
+    context = 200
+    gpu = model.build_gpu(backend, max_lanes=1, context_tokens=context + 16)
+    model.seed_context(gpu, context, rng)
+    parents = [0xFFFF, 0, 0, 1, 1, 2, 3, 3]
+    tree = np.zeros(rows, dtype=orc.TREE_DTYPE)
+    for r, parent in enumerate(parents):
+        tree[r] = ((1 << r) | (0 if r == 0 else int(tree[parent]["ancestors"])), parent, 0 if r == 0 else int(tree[parent]["depth"]) + 1)
+    children_of = {r: [c for c in range(rows) if parents[c] == r] for r in range(rows)}
+    tokens = np.zeros(rows, dtype=np.uint32)
+    tokens[0] = 4321
+    ids = np.zeros((rows, 16), np.uint32)
+    q = np.zeros((rows, 16), np.float32)
+    draws = np.full((rows, 4), 0xFF, np.uint8)
+    child_uniforms = rng.random((rows, 4)).astype(np.float32)
+    uniforms = rng.random((rows, 2)).astype(np.float32)
+    lane = verify.Lane(rows, context, temperature=T)
+    logits_of = lambda: gpu.buffer(verify.LOGITS).download(np.float32, rows * V).reshape(rows, V)
+    for r in range(rows):       # parents come before children: a row's candidates from the target's own logits at that row
+        gpu.set_block([lane], tokens, tree_rows=tree, uniforms=uniforms)
+        gpu.set_candidate_children(ids, q, draws, child_uniforms)
+        backend.run(gpu.encode([lane], commit=False))
+        row_logits = logits_of()[r].astype(np.float64)
+        top = np.argsort(-row_logits)[:16]
+        ids[r] = rng.permutation(top)
+        w = np.exp((row_logits[ids[r]] - row_logits.max()) / (2 * T))        # a flatter draft than the target
+        q[r] = (w / w.sum()).astype(np.float32)
+        best = int(np.argmax(row_logits[ids[r]]))
+        order = ([best] if r % 2 == 0 else []) + [i for i in rng.permutation(16) if i != best]   # even rows draw the likeliest first
+        for c, (child, index) in enumerate(zip(children_of[r], order)):
+            draws[r, c] = index
+            tokens[child] = ids[r, index]
+    gpu.set_block([lane], tokens, tree_rows=tree, uniforms=uniforms)
+    gpu.set_candidate_children(ids, q, draws, child_uniforms)
+    graph = gpu.encode([lane], commit=False)
+    assert "decode_sample_draw_children" in graph.kernels()
+    backend.run(graph)
+    logits = logits_of()
+    selected, retained, accepted, mask = gpu.results([lane])
+    want_rows, sure = [], True
+    for r in range(rows):
+        n = int((draws[r] != 0xFF).sum())
+        want, close = orc.children_row(logits[r], (T, 0.0, 0, 1.0), ids[r], q[r], list(draws[r, :n]), child_uniforms[r], float(uniforms[r, 0]))
+        want_rows.append(want)
+        sure &= close > 1e-5
+    kept, acc, m = orc.accept_tree(tree, tokens, np.array(want_rows, np.uint32))
+    print(f"  oracle rows {want_rows}; kept {list(kept)} accepted {acc} mask {m:#x}; sure {sure}", flush=True)
+    if sure:
+        assert retained[0] == len(kept) and accepted[0] == acc and mask[0] == m and np.array_equal(selected[:len(kept)], kept)
+    assert 1 <= retained[0] <= rows and (not sure or accepted[0] >= 1)
