@@ -1,15 +1,21 @@
 """A random-init hybrid decoder (Gated DeltaNet and attention mixers over a mixture-of-experts FFN) for the
 parity tests: its weights, the GPU model built from them, and the oracle's evaluation of each layer.
 Test infrastructure only."""
+from concurrent.futures import ThreadPoolExecutor
+
 import numpy as np
 
 from splash_amd import ops, verify
 from tests import oracle as orc
+from tests.dense_reference import device_copy
 
 
 class HybridModel:
     def __init__(self, seed, hidden, vocabulary, layers, q_heads, kv_heads, head_dim, gdn_key_heads, gdn_value_heads, experts, top_k,
-                 expert_ffn, attention_interval=4, rope_theta=1e6, gated_attention=False, shared_slices=0, shared_gate=False, dense_ffn=0):
+                 expert_ffn, attention_interval=4, rope_theta=1e6, gated_attention=False, shared_slices=0, shared_gate=False, dense_ffn=0,
+                 distinct_layers=None, threads=8):
+        """`distinct_layers` weight sets are drawn (a multiple of the attention interval, so that a set's mixer is its
+        layers'), layer l holding set l % distinct_layers; all of them by default."""
         self.dims = dict(hidden=hidden, vocabulary=vocabulary, layers=layers, q_heads=q_heads, kv_heads=kv_heads, head_dim=head_dim,
                          gdn_key_heads=gdn_key_heads, gdn_value_heads=gdn_value_heads, experts=experts, top_k=top_k, expert_ffn=expert_ffn,
                          attention_interval=attention_interval)
@@ -24,18 +30,28 @@ class HybridModel:
         self.packed_width = (conv + gdn_value_heads * 128 + 2 * gdn_value_heads + 15) // 16 * 16
         self.gdn_shape = orc.gdn_shape(gdn_key_heads, gdn_value_heads, packed_width=self.packed_width)
 
+        pool = ThreadPoolExecutor(max(1, threads))
+
         def quant(n, k, fmt=orc.FMT_Q4K, scale=0.02):
             return orc.quantize_rows(fmt, (rng.standard_normal((n, k)) * scale).astype(np.float32))
 
+        def quant_many(count, n, k):
+            # a layer's experts: each from a generator spawned from the model's, quantized on the pool's threads
+            work = lambda g: orc.quantize_rows(orc.FMT_Q4K, (g.standard_normal((n, k), dtype=np.float32) * np.float32(0.02)))
+            return list(pool.map(work, rng.spawn(count)))
+
         def norm(n):
             return orc.f32_to_bf16((1 + 0.1 * rng.standard_normal(n)).astype(np.float32))
+        self.distinct = layers if distinct_layers is None else distinct_layers
+        assert self.distinct == layers or self.distinct % attention_interval == 0
         self.layers = []
-        for l in range(layers):
+        for l in range(self.distinct):
             if experts:
+                many = experts * expert_ffn * hidden >= (1 << 24)
                 w = dict(input_norm=norm(hidden), post_norm=norm(hidden), router=quant(experts, hidden, orc.FMT_Q6K, 0.05),
-                         gate=[quant(expert_ffn, hidden) for _ in range(experts + shared_slices)],
-                         up=[quant(expert_ffn, hidden) for _ in range(experts + shared_slices)],
-                         down=[quant(hidden, expert_ffn) for _ in range(experts + shared_slices)])
+                         gate=quant_many(experts + shared_slices, expert_ffn, hidden) if many else [quant(expert_ffn, hidden) for _ in range(experts + shared_slices)],
+                         up=quant_many(experts + shared_slices, expert_ffn, hidden) if many else [quant(expert_ffn, hidden) for _ in range(experts + shared_slices)],
+                         down=quant_many(experts + shared_slices, hidden, expert_ffn) if many else [quant(hidden, expert_ffn) for _ in range(experts + shared_slices)])
             else:
                 w = dict(input_norm=norm(hidden), post_norm=norm(hidden), ffn_gate=quant(dense_ffn, hidden), ffn_up=quant(dense_ffn, hidden),
                          ffn_down=quant(hidden, dense_ffn, orc.FMT_Q6K))
@@ -51,6 +67,8 @@ class HybridModel:
                          a_scale=(-np.exp(rng.uniform(-1.0, 1.0, gdn_value_heads))).astype(np.float32),
                          dt_bias=orc.f32_to_bf16(rng.uniform(-1.0, 1.0, gdn_value_heads).astype(np.float32)), mixer_norm=norm(128))
             self.layers.append(w)
+        self.layers = [self.layers[l % self.distinct] for l in range(layers)]
+        pool.shutdown()
         self.embedding = quant(vocabulary, hidden)
         self.final_norm = norm(hidden)
         self.head = quant(vocabulary, hidden, orc.FMT_Q6K)
@@ -75,7 +93,12 @@ class HybridModel:
         D, H, F = d["head_dim"], d["hidden"], d["expert_ffn"]
         P = lambda segs, k, f32=False: ops.Projection.from_native(backend, segs, k, float32=f32)
         images = lambda fmt, natives, n, k: backend.from_array(np.concatenate([ops.pack_gguf_image(fmt, x, n, k) for x in natives]))
+        built = {}
         for i, w in enumerate(self.layers):
+            if i >= self.distinct:      # a layer of a set already resident: its buffers again
+                args, kwargs = built[i % self.distinct]
+                gpu.set_layer(i, *args, **kwargs)
+                continue
             common = dict(input_norm=backend.from_array(w["input_norm"]), post_norm=backend.from_array(w["post_norm"]))
             if d["experts"]:
                 common.update(router=P([(orc.FMT_Q6K, d["experts"], w["router"])], H, True), gate_images=images(orc.FMT_Q4K, w["gate"], F, H),
@@ -86,34 +109,42 @@ class HybridModel:
             if self.shared_gate:
                 common["shared_scalar_gate"] = backend.from_array(w["shared_scalar_gate"])
             if self.attends(i):
-                gpu.set_layer(i, P([(orc.FMT_Q4K, d["q_heads"] * D * (2 if self.gated else 1), w["q"]), (orc.FMT_Q4K, d["kv_heads"] * D, w["k"]),
-                                    (orc.FMT_Q4K, d["kv_heads"] * D, w["v"])], H), P([(orc.FMT_Q4K, H, w["o"])], d["q_heads"] * D),
-                              query_norm=backend.from_array(w["q_norm"]), key_norm=backend.from_array(w["k_norm"]), **common)
+                args = (P([(orc.FMT_Q4K, d["q_heads"] * D * (2 if self.gated else 1), w["q"]), (orc.FMT_Q4K, d["kv_heads"] * D, w["k"]),
+                           (orc.FMT_Q4K, d["kv_heads"] * D, w["v"])], H), P([(orc.FMT_Q4K, H, w["o"])], d["q_heads"] * D))
+                kwargs = dict(query_norm=backend.from_array(w["q_norm"]), key_norm=backend.from_array(w["k_norm"]), **common)
             else:
-                gpu.set_layer(i, P([(orc.FMT_Q4K, self.packed_width, w["mixer_in"])], H),
-                              P([(orc.FMT_Q4K, H, w["mixer_out"])], d["gdn_value_heads"] * 128),
-                              convolution_weights=backend.from_array(w["conv_w"]), decay_weights=backend.from_array(w["a_scale"]),
+                args = (P([(orc.FMT_Q4K, self.packed_width, w["mixer_in"])], H), P([(orc.FMT_Q4K, H, w["mixer_out"])], d["gdn_value_heads"] * 128))
+                kwargs = dict(convolution_weights=backend.from_array(w["conv_w"]), decay_weights=backend.from_array(w["a_scale"]),
                               time_bias=backend.from_array(w["dt_bias"]), mixer_norm=backend.from_array(w["mixer_norm"]), **common)
+            built[i] = (args, kwargs)
+            gpu.set_layer(i, *args, **kwargs)
         gpu.set_head(orc.FMT_Q4K, backend.from_array(self.embedding), backend.from_array(self.final_norm),
                      P([(orc.FMT_Q6K, d["vocabulary"], self.head)], H, True))
         self.gpu = gpu
         return gpu
 
-    def seed_context(self, rng):
-        """A seeded INT8 context in every physical page of every attention layer."""
+    def seed_context(self, rng, distinct=None):
+        """A seeded INT8 context in every physical page of every attention layer; `distinct` contexts are drawn, attention
+        layer a holding context a % distinct (copied on the device)."""
         d, gpu = self.dims, self.gpu
         H, D, PT = d["kv_heads"], d["head_dim"], ops.PAGE_TOKENS
         helper = ops.KvPages.__new__(ops.KvPages)
         helper.kv_heads, helper.head_dim, helper.page_bytes = H, D, gpu.page_bytes
-        self.context = []
-        for layer in range(d["layers"] // d["attention_interval"]):
+        attention_layers = d["layers"] // d["attention_interval"]
+        distinct = attention_layers if distinct is None else distinct
+        drawn = []
+        for layer in range(distinct):
             def quant(x):
                 mx = np.abs(x).max(axis=-1, keepdims=True)
                 codes = np.clip(np.rint(x * np.float32(127.0) / mx), -127, 127).astype(np.int8)
                 return codes, (mx[..., 0] / np.float32(127.0)).astype(np.float16).astype(np.float32)
             (kc, ks), (vc, vs) = (quant(rng.standard_normal((self.physical_pages, H, PT, D)).astype(np.float32)) for _ in range(2))
-            self.context.append([kc, ks, vc, vs])
+            drawn.append([kc, ks, vc, vs])
             gpu.buffer(verify.KV_POOL, layer).upload(helper.pack_pages(kc, ks, vc, vs))
+        for layer in range(distinct, attention_layers):
+            device_copy(gpu.backend, gpu.buffer(verify.KV_POOL, layer % distinct), gpu.buffer(verify.KV_POOL, layer),
+                        self.physical_pages * gpu.page_bytes)
+        self.context = [drawn[a % distinct] for a in range(attention_layers)]
 
     def seed_states(self, rng, lanes, parity=0):
         """Random recurrent states and convolution carries in every lane's cell of `parity`."""
@@ -130,16 +161,15 @@ class HybridModel:
     def read_cell(self, lane, parity, gdn_layer):
         gpu, shape = self.gpu, self.gdn_shape
         st = gpu.strides
-        raw = gpu.buffer(verify.GDN_STATES).download(np.uint8)
+        states = gpu.buffer(verify.GDN_STATES)
         base = gpu.cell_offset(lane, parity)
-        conv = raw[base + gdn_layer * st.convolution_layer_bytes:][:3 * shape.conv_dim * 2].view(np.uint16).reshape(3, shape.conv_dim)
+        conv = states.download(np.uint16, 3 * shape.conv_dim, base + gdn_layer * st.convolution_layer_bytes).reshape(3, shape.conv_dim)
         at = base + st.convolution_state_bytes + gdn_layer * st.recurrent_layer_bytes
-        return conv.copy(), raw[at:at + st.recurrent_layer_bytes].view(np.float32).reshape(shape.value_heads, 128, 128).copy()
+        return conv.copy(), states.download(np.float32, st.recurrent_layer_bytes // 4, at).reshape(shape.value_heads, 128, 128).copy()
 
     def read_tape(self, lane, parity, gdn_layer):
         gpu = self.gpu
-        raw = gpu.buffer(verify.GDN_TAPE).download(np.uint8)
-        return raw[gpu.tape_offset(lane, parity, gdn_layer):][:gpu.tape_layer_bytes].copy()
+        return gpu.buffer(verify.GDN_TAPE).download(np.uint8, gpu.tape_layer_bytes, gpu.tape_offset(lane, parity, gdn_layer)).copy()
 
     # ------------------------------------------------------------------ oracle side
     def _project(self, fmt, native, x_bits, n):

