@@ -255,29 +255,33 @@ def time_c3_ops(backend):
             pool = ops.KvPages(backend, KVH, D, pages, table)
             pool.upload(raw)
             pools.append(pool)
-        plan = ops.AttentionPlan(QH, KVH, D, [(0, rows, context - rows, 0)])
-        workspace = ops.AttentionWorkspace(backend, plan)
         qkv = backend.from_array(bf(rng.standard_normal((rows, (QH + 2 * KVH) * D))))
         tree = backend.from_array(ops.chain_tree_rows([rows]))
         out = backend.allocate_buffer(rows * QH * D * 2)
-        graph = splash_amd.CommandGraph()
-        ops.PagedAttention.add_projection(graph, plan, qkv, workspace, pools[0])
-        passes = 4
-        for _ in range(passes):
-            for pool in pools:
-                ops.PagedAttention.add_attention(graph, plan, workspace, tree, pool, out)
-        backend.set_dispatch_profiling(True)
-        _, _, per = backend.run(graph, profiled=True)
-        backend.set_dispatch_profiling(False)
-        pairs = np.array(per[1:]).reshape(-1, 2)[copies:] * 1e6
-        split_us, merge_us = float(np.median(pairs[:, 0])), float(np.median(pairs[:, 1]))
         algorithmic = kv_bytes + rows * QH * D * 2 * 2 + pages * 8
-        results.append({"context": context, "splits": plan.splits, "split_us": round(split_us, 2), "merge_us": round(merge_us, 2),
-                        "GB/s": round(algorithmic / (split_us + merge_us) / 1e3, 1),
-                        "frac": round(algorithmic / (split_us + merge_us) / 1e3 / HBM_PEAK_GBS, 4),
-                        "TFLOP/s": round(4 * rows * QH * D * context / (split_us + merge_us) / 1e6, 1)})
-        log(f"  context {context:6d} splits {plan.splits:2d}: split {split_us:7.2f} us merge {merge_us:6.2f} us {algorithmic / (split_us + merge_us) / 1e3:7.1f} GB/s")
-        del graph, pools, workspace
+        for int8_queries in (False, True):
+            plan = ops.AttentionPlan(QH, KVH, D, [(0, rows, context - rows, 0)], int8_queries=int8_queries)
+            workspace = ops.AttentionWorkspace(backend, plan)
+            graph = splash_amd.CommandGraph()
+            ops.PagedAttention.add_projection(graph, plan, qkv, workspace, pools[0])
+            passes = 4
+            for _ in range(passes):
+                for pool in pools:
+                    ops.PagedAttention.add_attention(graph, plan, workspace, tree, pool, out)
+            backend.set_dispatch_profiling(True)
+            _, _, per = backend.run(graph, profiled=True)
+            backend.set_dispatch_profiling(False)
+            pairs = np.array(per[1:]).reshape(-1, 2)[copies:] * 1e6
+            split_us, merge_us = float(np.median(pairs[:, 0])), float(np.median(pairs[:, 1]))
+            results.append({"context": context, "queries": "int8" if int8_queries else "bf16", "splits": plan.splits,
+                            "split_us": round(split_us, 2), "merge_us": round(merge_us, 2),
+                            "GB/s": round(algorithmic / (split_us + merge_us) / 1e3, 1),
+                            "frac": round(algorithmic / (split_us + merge_us) / 1e3 / HBM_PEAK_GBS, 4),
+                            "TFLOP/s": round(4 * rows * QH * D * context / (split_us + merge_us) / 1e6, 1)})
+            log(f"  context {context:6d} {'int8' if int8_queries else 'bf16'} queries, splits {plan.splits:2d}: split {split_us:7.2f} us "
+                f"merge {merge_us:6.2f} us {algorithmic / (split_us + merge_us) / 1e3:7.1f} GB/s")
+            del graph, workspace
+        del pools
     print(json.dumps({"metric": "attention us and GB/s by context (config 3)", "unit": "us", "n_gpus": 1,
                       "data": "synthetic: uniform INT8 codes, random page table, ring of pools past the caches",
                       "roofline_peak_gbs": HBM_PEAK_GBS, "results": results}), flush=True)

@@ -110,6 +110,8 @@ typedef struct spo_attention_geometry {
   uint32_t normalize;    /* RMS-norm q and k heads */
   uint32_t gated;        /* the projection row holds each query head's queries, then its gate; the output rows
                             are multiplied by the gates' sigmoids (kernels/common/attention_gate.h:19-44) */
+  uint32_t int8_queries; /* the block's queries score as INT8 codes with a scale per head and row, exactly in int32
+                            (the "q8q" kernels, PagedAttention.cpp:380-383); 0: as the bf16 rows */
 } spo_attention_geometry;
 typedef struct spo_attention_rows { /* one sequence: ops::AttentionRows / AttentionHistory */
   uint32_t first_row, rows, committed, table_first;

@@ -76,6 +76,21 @@ void orc_attention_prepare(const struct OrcAttention *a, const uint16_t *qkv, co
   }
 }
 
+// common/int8_activations.h:22-28 (int8_activation_block, int8_activation_code).
+void orc_int8_activation_block(const float *x, uint32_t n, int8_t *codes, float *scale) {
+  float largest = 0.f;
+  bool finite = true;
+  for (uint32_t i = 0; i < n; ++i) {
+    finite = finite && std::isfinite(x[i]);
+    largest = std::max(largest, std::fabs(x[i]));
+  }
+  const bool coded = largest > 0x1p-100f;
+  const float inverse = coded ? 127.0f / largest : 0.0f;
+  for (uint32_t i = 0; i < n; ++i)
+    codes[i] = finite ? int8_t(std::clamp(std::nearbyint(x[i] * inverse), -127.0f, 127.0f)) : int8_t(0);
+  *scale = !finite ? std::numeric_limits<float>::quiet_NaN() : coded ? largest / 127.0f : 0.0f;
+}
+
 // paged_attention_tile.h:179-285 (page softmax), :427-463 (page loop), :499-535 (split merge).
 void orc_attention(const struct OrcAttention *a, const uint16_t *q, const int8_t *kcodes, const float *kscales,
                    const int8_t *vcodes, const float *vscales, const uint32_t *page_table,
@@ -96,6 +111,14 @@ void orc_attention(const struct OrcAttention *a, const uint16_t *q, const int8_t
     for (uint32_t item = lo; item < hi; ++item) {
       const uint32_t r = item / a->q_heads, qh = item % a->q_heads, kh = qh / group;
       const uint16_t *qr = q + (size_t(r) * a->q_heads + qh) * D;
+      // INT8 queries: the row's codes and scale; the score product is then exact in int32
+      std::vector<int8_t> qcodes(D);
+      float qscale = 1.f;
+      if (a->int8_queries) {
+        std::vector<float> values(D);
+        for (uint32_t d = 0; d < D; ++d) values[d] = bf2f(qr[d]);
+        orc_int8_activation_block(values.data(), D, qcodes.data(), &qscale);
+      }
       // ---- fp32 page loop with ordered split merge ----
       std::vector<float> sm(splits, -std::numeric_limits<float>::infinity()), sl(splits, 0.f);
       std::vector<std::vector<float>> so(splits, std::vector<float>(D, 0.f));
@@ -112,7 +135,13 @@ void orc_attention(const struct OrcAttention *a, const uint16_t *q, const int8_t
           for (uint32_t t = 0; t < PT; ++t) {
             if (!visible(r, p * PT + t)) { score[t] = -std::numeric_limits<float>::infinity(); continue; }
             float dot = 0.f;
-            for (uint32_t d = 0; d < D; ++d) dot += bf2f(qr[d]) * float(kp[size_t(t) * D + d]);
+            if (a->int8_queries) {
+              int32_t exact = 0;
+              for (uint32_t d = 0; d < D; ++d) exact += int32_t(qcodes[d]) * int32_t(kp[size_t(t) * D + d]);
+              dot = float(exact) * qscale;
+            } else {
+              for (uint32_t d = 0; d < D; ++d) dot += bf2f(qr[d]) * float(kp[size_t(t) * D + d]);
+            }
             score[t] = dot * ks[t] * inv_sqrt;
             pageMax = std::max(pageMax, score[t]);
           }

@@ -99,6 +99,7 @@ struct OrcAttention {
   uint32_t splits;      // history splits merged in split order (1 = none)
   uint32_t pages_per_split;
   uint32_t half_scale;  // scales are fp16 values (already rounded) -- informational
+  uint32_t int8_queries; // the page loop scores INT8 codes of each (row, head)'s queries (paged_attention_tile.h:294-322)
 };
 // q/k per-head RMS norm + partial RoPE + staging (attention_qkv_prepare.h:28-91).
 // qkv bf16 [rows][(q_heads + 2 kv_heads) * D]; qw/kw bf16 [D] norm weights (NULL = no norm);
@@ -107,6 +108,10 @@ struct OrcAttention {
 void orc_attention_prepare(const struct OrcAttention *a, const uint16_t *qkv, const uint16_t *qw, const uint16_t *kw,
                            const float *cosv, const float *sinv, uint32_t pairs, uint16_t *q_out, float *k_out,
                            float *v_out);
+// common/int8_activations.h:22-28: a block of activations as INT8 codes and one scale: with m the block's largest
+// magnitude, code = clamp(rint(x * (127 / m)), -127, 127) (ties to even, the quotient rounded first) and scale = m / 127;
+// a block whose m is 2^-100 or less codes as zeros with scale 0; one that holds an infinity or a NaN takes a NaN scale.
+void orc_int8_activation_block(const float *x, uint32_t n, int8_t *codes, float *scale);
 // Block-causal attention over paged INT8 KV, page by page with the online softmax of
 // paged_attention_tile.h:179-285 and the ordered split merge of :499-535.
 // pages: page_table[p] names the physical page of logical page p. A physical page holds

@@ -75,7 +75,8 @@ class LinearPlan(ctypes.Structure):
 
 
 class AttentionGeometry(ctypes.Structure):
-    _fields_ = [("q_heads", c_u32), ("kv_heads", c_u32), ("head_dim", c_u32), ("rotary_pairs", c_u32), ("normalize", c_u32), ("gated", c_u32)]
+    _fields_ = [("q_heads", c_u32), ("kv_heads", c_u32), ("head_dim", c_u32), ("rotary_pairs", c_u32), ("normalize", c_u32), ("gated", c_u32),
+                ("int8_queries", c_u32)]
 
 
 class AttentionRows(ctypes.Structure):

@@ -84,6 +84,9 @@ struct AttentionParams {
   uint32_t sequences;
   uint32_t table_tiles;      // attention_reduce_*_t: row tiles of the activation table it writes
   uint32_t gated;            // 1: the output rows are multiplied by the sigmoid of their heads' gates (attention_gate.h:19-44)
+  uint32_t int8_queries;     // 1: queries are staged as INT8 codes with one scale a (row, head) and scored by an
+                             // INT8 x INT8 product (the reference's q8q kernels, paged_attention_tile.h:294-322)
+  uint32_t reserved;
   uint64_t page_bytes;       // bytes between physical pages of the layer's pool
   struct AttentionSequence sequence[ATTENTION_MAXIMUM_SEQUENCES];
 };
@@ -102,6 +105,6 @@ struct AttentionCommitParams {
 #ifdef __cplusplus
 static_assert(sizeof(AttentionTreeRow) == 8, "a tree row is 8 bytes on both sides");
 static_assert(sizeof(AttentionSequence) == 16, "an attention sequence is 16 bytes on both sides");
-static_assert(sizeof(AttentionParams) == 48 + 16 * ATTENTION_MAXIMUM_SEQUENCES, "attention parameters are 176 bytes on both sides");
+static_assert(sizeof(AttentionParams) == 56 + 16 * ATTENTION_MAXIMUM_SEQUENCES, "attention parameters are 184 bytes on both sides");
 static_assert(sizeof(AttentionCommitParams) == 32 + 16 * ATTENTION_MAXIMUM_SEQUENCES, "commit parameters are 160 bytes on both sides");
 #endif

@@ -32,7 +32,7 @@ sp_status spo_attention_plan_create(const spo_attention_geometry *geometry, cons
     for (uint32_t i = 0; i < count; ++i)
       rows.push_back({sequences[i].first_row, sequences[i].rows, sequences[i].committed, sequences[i].table_first});
     const ops::AttentionGeometry g{geometry->q_heads, geometry->kv_heads, geometry->head_dim, geometry->rotary_pairs,
-                                   geometry->normalize != 0, geometry->gated != 0};
+                                   geometry->normalize != 0, geometry->gated != 0, geometry->int8_queries != 0};
     *out = new spo_attention_plan{ops::PagedAttention::plan(g, std::move(rows))};
   });
 }

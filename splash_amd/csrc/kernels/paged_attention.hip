@@ -92,7 +92,8 @@ __global__ __launch_bounds__(D) void attention_q8_qkv(const uint16_t *__restrict
     if (query) {
       const uint32_t kv = head / group, g = head % group;
       const size_t at = ((size_t(z) * p.kv_heads + kv) * group + g) * 16u + row;
-      queries[at * D + tid] = _Float16(0.f);
+      if (p.int8_queries) reinterpret_cast<int8_t *>(queries)[at * D + tid] = 0;
+      else queries[at * D + tid] = _Float16(0.f);
       if (tid == 0) qsums[at] = 0.f;
     }
     return;
@@ -123,6 +124,20 @@ __global__ __launch_bounds__(D) void attention_q8_qkv(const uint16_t *__restrict
   if (query) {
     const uint32_t kv = index / group, g = index % group;
     const size_t at = ((size_t(z) * p.kv_heads + kv) * group + g) * 16u + row;
+    if (p.int8_queries) {
+      // common/int8_activations.h:22-28: code = clamp(rint(x (127 / m))), the quotient rounded first; scale = m / 127; a
+      // head at or below 2^-100 codes as zeros with scale 0; one that is not finite takes a NaN scale. The codes lie
+      // where the fp16 queries would, one byte a dimension, and the scale in the sums' slot.
+      const uint32_t bits = __builtin_bit_cast(uint32_t, result);
+      const float notFinite = block_max<D>((bits & 0x7F800000u) == 0x7F800000u ? 1.f : 0.f, scratch, tid);
+      const float largest = block_max<D>(fabsf(result), scratch, tid);
+      const bool coded = largest > 0x1p-100f;
+      const float inverse = coded ? 127.0f / largest : 0.0f;
+      const float code = fminf(fmaxf(rintf(result * inverse), -127.0f), 127.0f);
+      reinterpret_cast<int8_t *>(queries)[at * D + tid] = notFinite != 0.f ? int8_t(0) : int8_t(code);
+      if (tid == 0) qsums[at] = notFinite != 0.f ? __builtin_bit_cast(float, 0x7FC00000u) : coded ? largest / 127.0f : 0.0f;
+      return;
+    }
     const _Float16 staged = _Float16(result);
     queries[at * D + tid] = staged;
     const float sum = block_sum<D>(float(staged), scratch, tid);
@@ -157,7 +172,11 @@ SP_REGISTER_KERNEL("attention_q8_qkv_d64", &attention_q8_qkv<64>);
 // Partials: O fp32 [sequence][kv head][split][16 G fused rows][D], (max, sum) fp32 pairs
 // [sequence][kv head][split][16 G]; the max is in the log2 domain of the scaled scores.
 // ---------------------------------------------------------------------------------------------
-template <int D, int G>
+// I8: the queries are INT8 codes with a scale a fused row (attention_q8_qkv staged them so): the score product is one
+// v_mfma_i32_16x16x64_i8 per 64 dimensions on the keys' stored bytes, which pass through LDS as they are (no widening,
+// no offset to remove), and a row's scale multiplies its scores after the product.
+typedef __attribute__((ext_vector_type(4))) int i32x4;
+template <int D, int G, bool I8>
 __global__ __launch_bounds__(256, 2) void attention_q8_split(const _Float16 *__restrict__ queries, const float *__restrict__ qsums,
                                                           const AttentionTreeRow *__restrict__ tree,
                                                           const uint64_t *__restrict__ page_table, uint8_t *__restrict__ pool,
@@ -167,7 +186,9 @@ __global__ __launch_bounds__(256, 2) void attention_q8_split(const _Float16 *__r
   constexpr int kTiles = (G + 3) / 4;  // fused-row tiles (one query head's 16 rows each) per wave
   constexpr int kKeyVectors = kStep * D / 16 / 256, kValueVectors = kKeyVectors;
   static_assert(kKeyVectors >= 1, "a step's keys fill the workgroup's loads");
-  __shared__ __align__(16) _Float16 ldsK[2][kStep][D + 8];
+  // keys: fp16 numbers 1152 + code, or (I8) the stored bytes, a token's row padded by 16 bytes either way
+  constexpr int kKeyRow = I8 ? (D + 16) / 2 : D + 8;  // in fp16 units
+  __shared__ __align__(16) _Float16 ldsK[2][kStep][kKeyRow];
   __shared__ __align__(16) _Float16 ldsV[2][D][kStep + 8];
   __shared__ __align__(16) float ldsKS[2][kStep], ldsVS[2][kStep];
 
@@ -183,17 +204,26 @@ __global__ __launch_bounds__(256, 2) void attention_q8_split(const _Float16 *__r
   const float scale2 = kLog2e / sqrtf(float(D));
 
   // This wave's query rows as MFMA operands, their sums and their rows' visibility masks.
-  f16x8 q[kTiles][JD];
-  float qsum[kTiles];
+  constexpr int JQ = D / 64;  // INT8 products of 64 dimensions
+  f16x8 q[I8 ? 1 : kTiles][I8 ? 1 : JD];
+  i32x4 q8[I8 ? kTiles : 1][I8 ? JQ : 1];
+  float qsum[kTiles];  // fp16 queries: the code offset's share of a score; INT8 queries: the row's scale
   bool owns[kTiles];
 #pragma unroll
   for (int k = 0; k < kTiles; ++k) {
     const uint32_t g = wave + 4u * k;
     owns[k] = g < uint32_t(G);
     const size_t at = ((size_t(z) * p.kv_heads + h) * G + (owns[k] ? g : 0u)) * 16u + row;
+    if constexpr (I8) {
+      const int8_t *codes = reinterpret_cast<const int8_t *>(queries) + at * D;
 #pragma unroll
-    for (int j = 0; j < JD; ++j) q[k][j] = *reinterpret_cast<const f16x8 *>(queries + at * D + 32 * j + 8 * kq);
-    qsum[k] = -(qsums[at] * kCodeOffset);
+      for (int j = 0; j < JQ; ++j) q8[k][j] = *reinterpret_cast<const i32x4 *>(codes + 64 * j + 16 * kq);
+      qsum[k] = qsums[at];
+    } else {
+#pragma unroll
+      for (int j = 0; j < JD; ++j) q[k][j] = *reinterpret_cast<const f16x8 *>(queries + at * D + 32 * j + 8 * kq);
+      qsum[k] = -(qsums[at] * kCodeOffset);
+    }
   }
   const uint32_t ancestors = row < seq.rows ? tree[seq.first_row + row].ancestors : 0u;
 
@@ -242,12 +272,16 @@ __global__ __launch_bounds__(256, 2) void attention_q8_split(const _Float16 *__r
 #pragma unroll
     for (int n = 0; n < kKeyVectors; ++n) {
       const uint32_t v = tid + 256u * n, token = v / (D / 16), dq = v % (D / 16);
-      const uint4 x = make_uint4(keyLoad[n].x ^ 0x80808080u, keyLoad[n].y ^ 0x80808080u, keyLoad[n].z ^ 0x80808080u,
-                                 keyLoad[n].w ^ 0x80808080u);
-      const uint2 a = bytes_to_f16(x.x), b = bytes_to_f16(x.y), c = bytes_to_f16(x.z), d = bytes_to_f16(x.w);
-      uint4 *out = reinterpret_cast<uint4 *>(&ldsK[buffer][token][16 * dq]);
-      out[0] = make_uint4(a.x, a.y, b.x, b.y);
-      out[1] = make_uint4(c.x, c.y, d.x, d.y);
+      if constexpr (I8) {
+        *reinterpret_cast<uint4 *>(reinterpret_cast<int8_t *>(&ldsK[buffer][token][0]) + 16 * dq) = keyLoad[n];
+      } else {
+        const uint4 x = make_uint4(keyLoad[n].x ^ 0x80808080u, keyLoad[n].y ^ 0x80808080u, keyLoad[n].z ^ 0x80808080u,
+                                   keyLoad[n].w ^ 0x80808080u);
+        const uint2 a = bytes_to_f16(x.x), b = bytes_to_f16(x.y), c = bytes_to_f16(x.z), d = bytes_to_f16(x.w);
+        uint4 *out = reinterpret_cast<uint4 *>(&ldsK[buffer][token][16 * dq]);
+        out[0] = make_uint4(a.x, a.y, b.x, b.y);
+        out[1] = make_uint4(c.x, c.y, d.x, d.y);
+      }
     }
 #pragma unroll
     for (int n = 0; n < kValueVectors; ++n) {
@@ -279,15 +313,31 @@ __global__ __launch_bounds__(256, 2) void attention_q8_split(const _Float16 *__r
     f32x4 s[kTiles][4];
 #pragma unroll
     for (int tt = 0; tt < 4; ++tt) {
-      f16x8 key[JD];
+      if constexpr (I8) {
+        // the keys' bytes against the queries' codes, exact in int32; the row's scale follows with the key's
+        i32x4 key[JQ];
+        const int8_t *bytes = reinterpret_cast<const int8_t *>(&ldsK[buffer][16 * tt + row][0]);
 #pragma unroll
-      for (int j = 0; j < JD; ++j) key[j] = *reinterpret_cast<const f16x8 *>(&ldsK[buffer][16 * tt + row][32 * j + 8 * kq]);
+        for (int j = 0; j < JQ; ++j) key[j] = *reinterpret_cast<const i32x4 *>(bytes + 64 * j + 16 * kq);
 #pragma unroll
-      for (int k = 0; k < kTiles; ++k) {
-        f32x4 acc = {qsum[k], qsum[k], qsum[k], qsum[k]};
+        for (int k = 0; k < kTiles; ++k) {
+          i32x4 acc = {0, 0, 0, 0};
 #pragma unroll
-        for (int j = 0; j < JD; ++j) acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(key[j], q[k][j], acc, 0, 0, 0);
-        s[k][tt] = acc;
+          for (int j = 0; j < JQ; ++j) acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(key[j], q8[k][j], acc, 0, 0, 0);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) s[k][tt][i] = float(acc[i]) * qsum[k];
+        }
+      } else {
+        f16x8 key[JD];
+#pragma unroll
+        for (int j = 0; j < JD; ++j) key[j] = *reinterpret_cast<const f16x8 *>(&ldsK[buffer][16 * tt + row][32 * j + 8 * kq]);
+#pragma unroll
+        for (int k = 0; k < kTiles; ++k) {
+          f32x4 acc = {qsum[k], qsum[k], qsum[k], qsum[k]};
+#pragma unroll
+          for (int j = 0; j < JD; ++j) acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(key[j], q[k][j], acc, 0, 0, 0);
+          s[k][tt] = acc;
+        }
       }
     }
     f32x4 keyScale[4], valueScale[4];
@@ -411,9 +461,12 @@ __global__ __launch_bounds__(256, 2) void attention_q8_split(const _Float16 *__r
     }
   }
 }
-SP_REGISTER_KERNEL("attention_q8_split_d128_g8", &attention_q8_split<128, 8>);
-SP_REGISTER_KERNEL("attention_q8_split_d128_g4", &attention_q8_split<128, 4>);
-SP_REGISTER_KERNEL("attention_q8_split_d64_g2", &attention_q8_split<64, 2>);
+SP_REGISTER_KERNEL("attention_q8_split_d128_g8", &attention_q8_split<128, 8, false>);
+SP_REGISTER_KERNEL("attention_q8_split_d128_g4", &attention_q8_split<128, 4, false>);
+SP_REGISTER_KERNEL("attention_q8_split_d64_g2", &attention_q8_split<64, 2, false>);
+SP_REGISTER_KERNEL("attention_q8q_split_d128_g8", &attention_q8_split<128, 8, true>);
+SP_REGISTER_KERNEL("attention_q8q_split_d128_g4", &attention_q8_split<128, 4, true>);
+SP_REGISTER_KERNEL("attention_q8q_split_d64_g2", &attention_q8_split<64, 2, true>);
 
 // ---------------------------------------------------------------------------------------------
 // attention_reduce: grid (q_heads, 16, sequences), 256 threads. Merges the splits of one (head,

@@ -59,6 +59,7 @@ AttentionParams AttentionPlan::params(uint64_t pageBytes) const noexcept {
   p.normalize = geometry_.normalize;
   p.qkv_stride = geometry_.packedWidth();
   p.gated = geometry_.gated;
+  p.int8_queries = geometry_.int8Queries;
   p.splits = splits_;
   p.sequences = uint32_t(sequences_.size());
   p.page_bytes = pageBytes;
@@ -135,7 +136,7 @@ void PagedAttention::addAttention(hip::CommandGraph &graph, const AttentionPlan 
     params.table_tiles = gguf_row_tiles(rows);
     requireBytes(outputTable, gguf_tables_bytes(width, params.table_tiles), "attention output table");
   }
-  graph.add("attention_q8_split" + kernelSuffix(g) + "_g" + std::to_string(g.group()),
+  graph.add(std::string(g.int8Queries ? "attention_q8q_split" : "attention_q8_split") + kernelSuffix(g) + "_g" + std::to_string(g.group()),
             {w.queries, w.querySums, treeRows, pages.pageTable, pages.pool, w.partials, w.partialSums}, params,
             {g.kvHeads, plan.splits(), plan.sequences().size()}, {256, 1, 1});
   graph.add("attention_reduce" + kernelSuffix(g) + (outputTable ? "_t" : ""),

@@ -31,6 +31,9 @@ struct AttentionGeometry final {
   // The projection row holds each query head's queries, then its gate, and the output rows are
   // multiplied by the gates' sigmoids (the reference's Gated geometries, attention_gate.h:19-44).
   bool gated = false;
+  // The block's queries score as INT8 codes with one scale per head and row against the INT8 keys, exact in int32 (the
+  // reference's "q8q" kernels, PagedAttention.cpp:380-383, paged_attention_tile.h:287-332); otherwise as the bf16 rows.
+  bool int8Queries = false;
   [[nodiscard]] uint32_t group() const noexcept { return kvHeads ? qHeads / kvHeads : 0; }
   [[nodiscard]] uint32_t packedWidth() const noexcept { return ((gated ? 2 : 1) * qHeads + 2 * kvHeads) * headDimension; }
   [[nodiscard]] kv::Layout layout() const noexcept { return {kvHeads, headDimension}; }

@@ -215,10 +215,10 @@ class KvPages:
 class AttentionPlan:
     """ops::AttentionPlan: geometry + sequences + history splits."""
 
-    def __init__(self, q_heads, kv_heads, head_dim, sequences, rotary_pairs=0, normalize=False, gated=False):
+    def __init__(self, q_heads, kv_heads, head_dim, sequences, rotary_pairs=0, normalize=False, gated=False, int8_queries=False):
         """sequences: [(first_row, rows, committed, table_first)]; gated: a projection row holds each query head's
         queries, then its gate, and the output rows are multiplied by the gates' sigmoids."""
-        g = nat.AttentionGeometry(q_heads, kv_heads, head_dim, rotary_pairs, int(normalize), int(gated))
+        g = nat.AttentionGeometry(q_heads, kv_heads, head_dim, rotary_pairs, int(normalize), int(gated), int(int8_queries))
         rows = (nat.AttentionRows * len(sequences))(*[nat.AttentionRows(*s) for s in sequences])
         h = ctypes.c_void_p()
         check(lib.spo_attention_plan_create(ctypes.byref(g), rows, len(sequences), ctypes.byref(h)))

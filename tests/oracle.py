@@ -144,7 +144,7 @@ def projection_interval(exact, bound):
 
 class OrcAttention(ctypes.Structure):
     _fields_ = [("q_heads", c_u32), ("kv_heads", c_u32), ("head_dim", c_u32), ("rows", c_u32), ("committed", c_u32),
-                ("page_tokens", c_u32), ("splits", c_u32), ("pages_per_split", c_u32), ("half_scale", c_u32)]
+                ("page_tokens", c_u32), ("splits", c_u32), ("pages_per_split", c_u32), ("half_scale", c_u32), ("int8_queries", c_u32)]
 
 
 def kv_quantize(values, half_scale=True):
@@ -172,12 +172,21 @@ def attention_prepare(q_heads, kv_heads, head_dim, qkv_bits, qw, kw, cosv, sinv,
     return q, k, v
 
 
+def int8_activation_block(values):
+    """common/int8_activations.h: (codes int8, scale) of one block of float32 values."""
+    x = np.ascontiguousarray(values, np.float32).ravel()
+    codes = np.empty(x.size, np.int8)
+    scale = c_f()
+    lib.orc_int8_activation_block(_p(x, f32p), c_u32(x.size), _p(codes, i8p), ctypes.byref(scale))
+    return codes, scale.value
+
+
 def attention(q_bits, kcodes, kscales, vcodes, vscales, page_table, ancestors, committed, splits=1, pages_per_split=1 << 20,
-              want64=True, threads=0):
+              want64=True, threads=0, int8_queries=False):
     """q_bits uint16 [rows][q_heads][D]; K/V logical pages [phys][kv_heads][256][D] int8, scales [phys][kv_heads][256]."""
     rows, q_heads, D = q_bits.shape
     kv_heads, PT = kcodes.shape[1], kcodes.shape[2]
-    a = OrcAttention(q_heads, kv_heads, D, rows, committed, PT, splits, pages_per_split, 1)
+    a = OrcAttention(q_heads, kv_heads, D, rows, committed, PT, splits, pages_per_split, 1, int(int8_queries))
     out = np.empty((rows, q_heads, D), dtype=np.uint16)
     out64 = np.empty((rows, q_heads, D), dtype=np.float64) if want64 else None
     q_bits = np.ascontiguousarray(q_bits, dtype=np.uint16)

@@ -36,8 +36,10 @@ def build_context(rng, backend, q_heads, kv_heads, D, rows, committed, extra_pag
     return kv, (kc, ks, vc, vs), table
 
 
-def run_block(backend, rng, q_heads, kv_heads, D, rows, committed, pairs=0, normalize=False, ancestors=None, oracle_kv_heads=None):
-    """oracle_kv_heads: the KV heads the oracle evaluates (all by default); `got` then holds their query heads only."""
+def run_block(backend, rng, q_heads, kv_heads, D, rows, committed, pairs=0, normalize=False, ancestors=None, oracle_kv_heads=None,
+              int8_queries=False):
+    """oracle_kv_heads: the KV heads the oracle evaluates (all by default); `got` then holds their query heads only.
+    int8_queries: the plan and the oracle's page loop score INT8 query codes (its fp64 reference keeps the bf16 rows)."""
     kv, logical, table = build_context(rng, backend, q_heads, kv_heads, D, rows, committed)
     kc, ks, vc, vs = (a.copy() for a in logical)
     width = (q_heads + 2 * kv_heads) * D
@@ -49,7 +51,8 @@ def run_block(backend, rng, q_heads, kv_heads, D, rows, committed, pairs=0, norm
     tree = ops.chain_tree_rows([rows])
     if ancestors is not None:
         tree["ancestors"] = ancestors
-    plan = ops.AttentionPlan(q_heads, kv_heads, D, [(0, rows, committed, 0)], rotary_pairs=pairs, normalize=normalize)
+    plan = ops.AttentionPlan(q_heads, kv_heads, D, [(0, rows, committed, 0)], rotary_pairs=pairs, normalize=normalize,
+                             int8_queries=int8_queries)
     ws = ops.AttentionWorkspace(backend, plan)
     out = backend.allocate_buffer(rows * q_heads * D * 2)
     graph = splash_amd.CommandGraph()
@@ -75,10 +78,11 @@ def run_block(backend, rng, q_heads, kv_heads, D, rows, committed, pairs=0, norm
         group = q_heads // kv_heads
         mine = np.concatenate([np.arange(h * group, (h + 1) * group) for h in oracle_kv_heads])
         sub = lambda a: np.ascontiguousarray(a[:, list(oracle_kv_heads)])
-        want, want64 = orc.attention(np.ascontiguousarray(q[:, mine]), sub(kc), sub(ks), sub(vc), sub(vs), table, anc, committed)
+        want, want64 = orc.attention(np.ascontiguousarray(q[:, mine]), sub(kc), sub(ks), sub(vc), sub(vs), table, anc, committed,
+                                     int8_queries=int8_queries)
         got = got[:, mine]
     else:
-        want, want64 = orc.attention(q, kc, ks, vc, vs, table, anc, committed)
+        want, want64 = orc.attention(q, kc, ks, vc, vs, table, anc, committed, int8_queries=int8_queries)
     stored = kv.unpack_pages(kv.download())
     return got, want, want64, stored, (kc, ks, vc, vs), table, plan
 
@@ -136,6 +140,38 @@ def test_config3_contexts_of_8k_and_128k(backend, context, heads):
     assert cos >= 0.9999 and err < 0.02, (cos, err)
     cos2, err2 = tolerance(got, orc.bf16_to_f32(want).astype(np.float64))
     assert cos2 >= 0.9999 and err2 < 0.02, (cos2, err2)
+
+
+@pytest.mark.parametrize("geometry", [(64, 8, 128), (16, 8, 64), (32, 4, 128)])
+@pytest.mark.parametrize("rows,committed", [(16, 0), (1, 255), (7, 1000), (16, 4096 + 37), (16, 32768 - 16)])
+def test_int8_queries_score_their_codes(backend, geometry, rows, committed):
+    """The "q8q" kernels (PagedAttention.cpp:380-383, paged_attention_tile.h:287-332): a head's queries of a row become
+    INT8 codes with one scale (int8_activations.h:22-28) and the score products are exact in int32. Against the oracle's
+    page loop over the same codes the output holds the bf16-query path's closeness; against the fp64 softmax of the
+    bf16 rows it passes the reference's gate (q8_flash_attention_metal_test.mm:788-799: cosine > 0.9995, max-abs <
+    0.02 of a value's range); and over the longer contexts it lies nearer the oracle that codes the queries than the
+    reference that does not, which a kernel that scored the bf16 rows would not."""
+    q_heads, kv_heads, D = geometry
+    if committed > 30000 and geometry != (64, 8, 128):
+        pytest.skip("the long context runs at the headline geometry")
+    print(f"case attention int8 queries geometry={geometry} rows={rows} committed={committed}", flush=True)
+    rng = np.random.default_rng(rows * 11 + committed)
+    got, want, want64, _, logical, _, _ = run_block(backend, rng, q_heads, kv_heads, D, rows, committed, pairs=D // 4,
+                                                    normalize=True, int8_queries=True)
+    coded = orc.bf16_to_f32(want).astype(np.float64)
+    # the reference's gate is stated on values within 1 (its valuePattern, q8_flash_attention_metal_test.mm:189-196); these
+    # are unit normals, so the bound on an output, a weighted mean of values, scales with the largest value stored
+    largest = float(np.abs(logical[2].astype(np.float32) * logical[3][..., None]).max())
+    cos, err = tolerance(got, want64)
+    assert cos > 0.9995 and err < 0.02 * max(1.0, largest), (cos, err, largest)
+    cos2, err2 = tolerance(got, coded)
+    assert cos2 >= 0.9999 and err2 < 0.02, (cos2, err2)
+    g = orc.bf16_to_f32(got).astype(np.float64)
+    near, far = np.sqrt(((g - coded) ** 2).mean()), np.sqrt(((g - want64) ** 2).mean())
+    print(f"  rms to the coded oracle {near:.3e}, to the fp64 reference of the bf16 rows {far:.3e}", flush=True)
+    # (short contexts leave outputs near 1, where the bf16 rounding of the output outweighs the queries' rounding)
+    if committed >= 1000:
+        assert near < 0.7 * far, (near, far)
 
 
 def test_long_context_32k(backend):

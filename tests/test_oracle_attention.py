@@ -105,3 +105,70 @@ def test_page_table_permutation_and_tree_rows():
     q2[2] = q[3]
     chain, _ = orc.attention(q2, kc2, ks2, vc2, vs2, table, anc, 300)
     assert np.array_equal(tree[3], chain[2])
+
+
+def test_int8_activation_block_follows_its_closed_form():
+    """common/int8_activations.h:22-28: code = clamp(rint(x * (127 / m))) with the quotient rounded first, scale = m / 127;
+    a block at or below 2^-100 codes as zeros with scale 0; a block holding an infinity or a NaN takes a NaN scale. Against
+    numpy float32 arithmetic written from that rule (not from the oracle's code), and its invariants."""
+    import numpy as np
+    from tests import oracle as orc
+    rng = np.random.default_rng(3)
+    for _ in range(50):
+        x = (rng.standard_normal(128) * rng.uniform(1e-3, 30)).astype(np.float32)
+        codes, scale = orc.int8_activation_block(x)
+        m = np.abs(x).max()
+        inverse = np.float32(127.0) / m                                        # correctly rounded float32 quotient
+        want = np.clip(np.rint(x * inverse), -127, 127).astype(np.int8)        # float32 product, ties to even
+        assert np.array_equal(codes, want) and scale == np.float32(m) / np.float32(127.0)
+        assert np.abs(codes).max() == 127                                      # the largest magnitude codes as +-127
+        assert np.abs(codes.astype(np.float64) * scale - x).max() <= 0.5001 * scale   # a value restores within half a step
+    # the quotient 127 / m is rounded before the product: for this pair x * (127 / m) rounds to 112, where x * 127 / m
+    # (the KV store's order of operations) would give 113
+    m, x = np.float32(0.5596824884414673), np.float32(0.4957817494869232)
+    assert np.rint(x * (np.float32(127) / m)) == 112 and np.rint(x * np.float32(127) / m) == 113
+    codes, scale = orc.int8_activation_block(np.array([m, x, -x], np.float32))
+    assert list(codes) == [127, 112, -112] and scale == m / np.float32(127.0)
+    # ties go to even: with m = 127 the codes are rint(x)
+    codes, _ = orc.int8_activation_block(np.array([127.0, 0.5, 1.5, 2.5, -0.5, -1.5], np.float32))
+    assert list(codes) == [127, 0, 2, 2, 0, -2]
+    codes, scale = orc.int8_activation_block(np.full(8, 2.0 ** -101, np.float32))
+    assert not codes.any() and scale == 0.0
+    codes, scale = orc.int8_activation_block(np.zeros(8, np.float32))
+    assert not codes.any() and scale == 0.0
+    for bad in (np.inf, -np.inf, np.nan):
+        _, scale = orc.int8_activation_block(np.array([1.0, bad, 2.0], np.float32))
+        assert np.isnan(scale)
+
+
+def test_int8_query_attention_scores_the_codes_exactly():
+    """paged_attention_tile.h:294-322: with INT8 queries the score product runs on the queries' codes and the row's scale
+    multiplies it. On one page with unit key scales and a one-hot value per token the page loop's output is the softmax
+    itself: it equals the fp64 softmax of (codes . keys) * qscale / sqrt(D); and against bf16 queries it stays inside the
+    reference's attention gate."""
+    import numpy as np
+    from tests import oracle as orc
+    rng = np.random.default_rng(4)
+    q_heads, kv_heads, D, rows, committed = 4, 2, 64, 3, 40
+    q = orc.f32_to_bf16(rng.standard_normal((rows, q_heads, D)).astype(np.float32))
+    kc = rng.integers(-127, 128, (1, kv_heads, 256, D)).astype(np.int8)
+    ks = np.full((1, kv_heads, 256), 0.02, np.float32)
+    vc = np.zeros((1, kv_heads, 256, D), np.int8)
+    for t in range(D):
+        vc[0, :, t, t] = 100                                                   # token t's value is 100 e_t
+    vs = np.full((1, kv_heads, 256), 0.01, np.float32)
+    anc = np.array([(2 << r) - 1 for r in range(rows)], np.uint32)
+    table = np.zeros(1, np.uint32)
+    got, _ = orc.attention(q, kc, ks, vc, vs, table, anc, committed, int8_queries=True)
+    exact, exact64 = orc.attention(q, kc, ks, vc, vs, table, anc, committed)
+    got = orc.bf16_to_f32(got).astype(np.float64)
+    for r in range(rows):
+        for h in range(q_heads):
+            codes, scale = orc.int8_activation_block(orc.bf16_to_f32(q[r, h]))
+            visible = committed + r + 1
+            s = (kc[0, h // 2, :visible].astype(np.int64) @ codes.astype(np.int64)).astype(np.float64) * scale * 0.02 / np.sqrt(D)
+            p = np.exp(s - s.max()); p /= p.sum()
+            want = np.zeros(D); want[:min(D, visible)] = p[:D]                 # P . V with V = e_t: the probabilities themselves
+            assert np.abs(got[r, h] - want).max() <= 2.0 ** -8 * max(want.max(), 1e-3) + 1e-6
+    cos = (got * exact64).sum() / np.sqrt((got ** 2).sum() * (exact64 ** 2).sum())
+    assert cos >= 0.9995 and np.abs(got - exact64).max() < 0.02
