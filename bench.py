@@ -523,6 +523,8 @@ def main():
     ap.add_argument("--workload", default="c4", choices=sorted(WORKLOADS) + ["c5"])
     ap.add_argument("--lanes", type=int, default=1)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--chain", action="store_true",
+                    help="one dispatch for a layer's four projections after its attention instead of a dispatch each")
     ap.add_argument("--calibrate-traffic", action="store_true",
                     help="after the steps, run plain read and copy kernels of known size: the scale of the FETCH_SIZE / "
                          "WRITE_SIZE counters of a rocprofv3 --pmc run of this command")
@@ -557,6 +559,8 @@ def main():
     rows = w["rows"] * args.lanes
     rng = np.random.default_rng(1)
     gpu.set_block(lanes, rng.integers(0, w["vocabulary"], rows).astype(np.uint32), uniforms=rng.random((rows, 2), dtype=np.float32))
+    if args.chain:
+        gpu.set_chained(True)
     graph = gpu.encode(lanes, commit=True)
     if args.temperature > 0:
         # the draft model's distributions of the block's rows: softmax of N(0, 2) logits over the whole vocabulary
@@ -592,10 +596,20 @@ def main():
     for total, name in totals[:8]:
         log(f"  {name:36s} x{len(by_kernel[name]):3d}  avg {total / len(by_kernel[name]) * 1e6:8.2f} us  total {total * 1e3:7.3f} ms")
     dominant = totals[0][1]
-    gate_up = [k for k in by_kernel if k.endswith("_g") or k.endswith("_gt")][0]
-    avg = sum(by_kernel[gate_up]) / len(by_kernel[gate_up])
     H, F = w["hidden"], w["ffn"]
-    gate_up_bytes = 2 * F * H * 0.5625 + rows * H * 2 + rows * F * 2     # both tensors once + bf16 rows in and out
+    QW, QKV = w["q_heads"] * w["head_dim"], (w["q_heads"] + 2 * w["kv_heads"]) * w["head_dim"]
+    chains = [k for k in by_kernel if k.startswith("gguf_decode_chain")]
+    if chains:
+        # A layer's chained dispatch: output (Q4_K), gate and up (Q4_K), down (Q6_K) and the next layer's q|k|v (Q4_K),
+        # every tensor once, and the bf16 rows in and out of each; the last layer's, which ends with the LM head, is left out.
+        gate_up = chains[0]
+        launches = by_kernel[gate_up][:-1]
+        gate_up_bytes = (H * QW + 2 * F * H + QKV * H) * 0.5625 + H * F * 0.8203125 + rows * 2 * (QW + 3 * H + 2 * F + QKV)
+    else:
+        gate_up = [k for k in by_kernel if k.endswith("_g") or k.endswith("_gt")][0]
+        launches = by_kernel[gate_up]
+        gate_up_bytes = 2 * F * H * 0.5625 + rows * H * 2 + rows * F * 2     # both tensors once + bf16 rows in and out
+    avg = sum(launches) / len(launches)
     achieved = gate_up_bytes / avg / 1e9
     traffic, traffic_at = measured_traffic(gate_up) if args.workload == "c4" and args.lanes == 1 else (None, None)
     if args.calibrate_traffic:
@@ -613,7 +627,7 @@ def main():
                      "frac_of_peak": round(step_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "wall_ms_per_step": round(wall_ms, 4)},
         "roofline": {"bound": "hbm", "kernel": gate_up, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic, "traffic_measured_at": traffic_at,
-                     "launches": len(by_kernel[gate_up]),
+                     "launches": len(launches),
                      "avg_us": round(avg * 1e6, 2), "algorithmic_bytes": int(gate_up_bytes), "largest_total": dominant},
     }
     if not args.no_cpu_baseline:

@@ -98,6 +98,36 @@ sp_status spo_linear_add_swiglu(const spo_linear *linear, spo_graph *graph, cons
                                 const spo_projection *up, const spo_projection *down, sp_buffer *normalized,
                                 sp_buffer *intermediate, sp_buffer *residual, sp_buffer *output, uint32_t rows,
                                 sp_buffer *table, sp_buffer *partials, sp_buffer *counters, sp_buffer *next_table);
+/* Linear::addChain: up to four projections of up to 64 rows as ONE dispatch, each reading what the one before it wrote
+ * (the table its epilogue leaves in next_table, the residual rows), in place of the reference's one dispatch a
+ * projection with a kernel boundary between them (QwenTarget.cpp:457-496 encodes a layer's projections one after the
+ * other): the next link's workgroups fetch their first weights while the link before drains and wait for its count of
+ * finished workgroups. A link is what spo_linear_add / spo_linear_add_residual_norm take: a plain plan (epilogue 0), a
+ * gate/up plan with next_table (2), or a residual + norm plan (3); `prepared` is 1 or 2 for every link (its table
+ * exists or the link before writes it); every link's table, partials and counters are its own, and no table is written
+ * that an earlier link of the chain read. `progress`: SPO_CHAIN_PROGRESS_BYTES bytes the chain owns, zero before its
+ * first dispatch; the word at SPO_CHAIN_STATUS_OFFSET reads nonzero after a dispatch in which a workgroup's bounded
+ * wait gave up (then the results are not to be used, and the caller zeroes the buffer). Results equal those of the
+ * links dispatched one by one, bit for bit. */
+#define SPO_CHAIN_LINKS 4u
+#define SPO_CHAIN_PROGRESS_BYTES 65792u
+#define SPO_CHAIN_STATUS_OFFSET 16u
+typedef struct spo_chain_link {
+  const spo_projection *projection, *gate;
+  spo_linear_plan plan;
+  sp_buffer *input, *output, *residual, *norm_weight, *next_table, *table, *partials, *counters;
+  int32_t prepared;
+  uint32_t reserved;
+} spo_chain_link;
+sp_status spo_linear_add_chain(const spo_linear *linear, spo_graph *graph, const spo_chain_link *links, uint32_t count,
+                               sp_buffer *progress);
+/* Linear::add (Linear.hpp:330-332) of one link's buffers, as a dispatch of its own: every field of LinearBuffers, so
+ * also a gate/up plan that writes the next projection's table (next_table) outside Linear::addSwiGlu. */
+sp_status spo_linear_add_link(const spo_linear *linear, spo_graph *graph, const spo_chain_link *link);
+/* KernelCalibration::chainSpinLimit: the polls (about a microsecond each) a chained projection's workgroup waits for the
+ * link before it, of chains added from now on. 0 makes every wait that finds the count short give up at once, which is
+ * how a host tests the failure path without a kernel that does not end. */
+sp_status spo_linear_set_chain_spin_limit(spo_linear *linear, uint32_t polls);
 /* Linear::scratchSize (Linear.hpp:319): of every plan of up to `rows` rows of the matrix. */
 sp_status spo_linear_scratch_size(const spo_linear *linear, uint32_t output_size, uint32_t input_size, uint32_t rows,
                                   uint64_t *table, uint64_t *partials, uint64_t *counters);
@@ -389,6 +419,11 @@ sp_status spo_verify_check_results(const spo_lane_rows *lanes, const uint32_t *r
  * uint32 [count]. */
 sp_status spo_dense_verify_results(spo_dense_verify *verify, const spo_verify_lane *lanes, uint32_t count, uint32_t *tokens,
                                    uint32_t *retained, uint32_t *accepted, uint32_t *retained_rows);
+/* Whether steps encoded from now on chain a layer's projections after its attention into one dispatch
+ * (spo_linear_add_chain: output, gate/up, down and the next layer's q|k|v, the LM head after the last layer) where
+ * their shapes allow: off by default; the results are the same bit for bit. spo_dense_verify_results fails with
+ * SP_BACKEND_ERROR after a step in which a chained projection's bounded wait gave up. */
+sp_status spo_dense_verify_set_chained(spo_dense_verify *verify, int chained);
 
 /* ---- The hybrid mixture-of-experts verify step (the reference's Qwen3.5 target with Gated
  *      DeltaNet mixers: QwenTarget.cpp:206-255 the GDN mixer, :263-347 the attention mixer, :372-395

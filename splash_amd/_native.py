@@ -74,6 +74,12 @@ class LinearPlan(ctypes.Structure):
                 ("float32", c_u32), ("scratch_input", c_u64), ("scratch_partials", c_u64), ("scratch_counters", c_u64)]
 
 
+class ChainLink(ctypes.Structure):
+    _fields_ = [("projection", c_p), ("gate", c_p), ("plan", LinearPlan), ("input", c_p), ("output", c_p), ("residual", c_p),
+                ("norm_weight", c_p), ("next_table", c_p), ("table", c_p), ("partials", c_p), ("counters", c_p),
+                ("prepared", ctypes.c_int32), ("reserved", c_u32)]
+
+
 class AttentionGeometry(ctypes.Structure):
     _fields_ = [("q_heads", c_u32), ("kv_heads", c_u32), ("head_dim", c_u32), ("rotary_pairs", c_u32), ("normalize", c_u32), ("gated", c_u32),
                 ("int8_queries", c_u32)]
@@ -234,6 +240,9 @@ _sig("spo_linear_plan_with", c_int, c_p, P(LinearPlan))
 _sig("spo_linear_add", c_int, c_p, c_p, c_p, c_p, P(LinearPlan), c_p, c_p, c_p, c_p, c_p, c_p, c_int)
 _sig("spo_linear_add_residual_norm", c_int, c_p, c_p, c_p, P(LinearPlan), c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_int)
 _sig("spo_linear_add_swiglu", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_u32, c_p, c_p, c_p, c_p)
+_sig("spo_linear_set_chain_spin_limit", c_int, c_p, c_u32)
+_sig("spo_linear_add_link", c_int, c_p, c_p, P(ChainLink))
+_sig("spo_linear_add_chain", c_int, c_p, c_p, P(ChainLink), c_u32, c_p)
 _sig("spo_linear_scratch_size", c_int, c_p, c_u32, c_u32, c_u32, P(c_u64), P(c_u64), P(c_u64))
 
 _sig("spo_kv_page_bytes", c_u64, c_u32, c_u32)
@@ -268,6 +277,7 @@ _sig("spo_draft_add_verify_rows", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p,
 _sig("spo_sampling_add_acceptance", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, P(LaneRows), P(c_u32), c_u32, P(c_u32))
 _sig("spo_sampling_greedy_rows_static", c_int, ctypes.c_void_p, c_u32, c_u32, c_u32, ctypes.c_void_p, ctypes.c_void_p)
 _sig("spo_verify_check_results", c_int, P(LaneRows), P(c_u32), c_u32, c_u32, c_u32, P(c_u32), P(c_u32), P(c_u32), P(c_u32))
+_sig("spo_dense_verify_set_chained", c_int, c_p, c_int)
 _sig("spo_dense_verify_results", c_int, c_p, P(VerifyLane), c_u32, P(c_u32), P(c_u32), P(c_u32), P(c_u32))
 _sig("spg_dense_dimensions", c_int, c_p, P(DenseDimensions))
 _sig("spo_dense_verify_load_gguf", c_int, c_p, c_p)

@@ -57,9 +57,11 @@
 // groups: values bf16 [tiles][G][64 lanes][8]: lane (r = l % 16, kq = l / 16) holds inputs
 // gguf_operand_input(kq, 0..7) of row 16 t + r; then sums32 fp32 [tiles][G][16 rows] and sums16
 // fp32 [tiles][2 G][16 rows], the fp32 sums of each row's 32 and 16 inputs in input order; then
-// squares fp32 [K / 64][16 tiles rows], read only of a table whose rows still lack a per-row scale
-// (GgufDecodeParams::deferred_scale): entry (j, r) is the sum of squares of row r's values over
-// columns 64 j .. 64 j + 63 of the rows the table was normed from.
+// squares fp32 [K / 64][gguf_squares_stride(tiles)], read only of a table whose rows still lack a per-row scale
+// (GgufDecodeParams::deferred_scale): entry (j, r), r < 16 tiles, is the sum of squares of row r's values over
+// columns 64 j .. 64 j + 63 of the rows the table was normed from. An entry fills whole 128-byte lines, as a group's
+// values and a workgroup's 16-input sums do: each has one writer (the workgroup that owns those columns), which is what
+// lets a projection chained behind the writer read them through its cache (gguf_decode_chain).
 #pragma once
 #include <stdint.h>
 
@@ -153,8 +155,9 @@ GGUF_INLINE uint64_t gguf_table_sums16_offset(uint32_t k, uint32_t tiles) {
 GGUF_INLINE uint64_t gguf_table_squares_offset(uint32_t k, uint32_t tiles) {
   return gguf_table_sums16_offset(k, tiles) + uint64_t(tiles) * (k / 16u) * 16u * 4u;
 }
+GGUF_INLINE uint32_t gguf_squares_stride(uint32_t tiles) { return tiles < 2u ? 32u : tiles * 16u; }  // floats an entry
 GGUF_INLINE uint64_t gguf_table_bytes(uint32_t k, uint32_t tiles) {
-  return gguf_table_squares_offset(k, tiles) + uint64_t(tiles) * (k / 64u) * 16u * 4u;
+  return gguf_table_squares_offset(k, tiles) + uint64_t(k / 64u) * gguf_squares_stride(tiles) * 4u;
 }
 // Row tiles of a piece, and the tables of `tiles` row tiles in all: whole pieces' tables of four row
 // tiles each, then the last piece's (the single table of up to four row tiles is its own case).
@@ -212,6 +215,38 @@ struct GgufDecodeParams {
   uint32_t formats[3];  // gguf_decode_mixed_*: each segment's format; the kernels of one format leave it zero
 };
 
+// gguf_decode_chain_m<16|32|64>: up to four projections of up to 64 rows in one dispatch, each a gguf_decode (or, with
+// `mixed`, a gguf_decode_mixed) dispatch of its own eight buffers, link i + 1 reading what link i's epilogue wrote (the
+// next projection's table, the residual rows). Grid: the links' grids one after the other; 256 threads. After the
+// links' buffers the kernel binds `progress`, GGUF_CHAIN_PROGRESS_WORDS words that are zero between dispatches:
+// GGUF_CHAIN_LINKS counts of finished workgroups; a status word, nonzero once a workgroup's wait for the link before it
+// ran out of polls (the results are then not to be used); and from word GGUF_CHAIN_FLAGS_AT each link's GGUF_CHAIN_FLAGS
+// go flags, GGUF_CHAIN_FLAG_STRIDE words apart (a flag a 256-byte block, so that the workgroups that wait, each
+// polling flag `its index % GGUF_CHAIN_FLAGS`, spread over the memory channels: a word that every waiting workgroup of
+// the device polls slows the whole dispatch down). The workgroup that completes a link's count sets that link's flags
+// and clears the flags of the link before. Every link has its own table, partials and counters, and no buffer a link
+// writes is read earlier in the dispatch.
+#define GGUF_CHAIN_LINKS 4u
+#define GGUF_CHAIN_FLAGS 64u
+#define GGUF_CHAIN_FLAG_STRIDE 64u
+#define GGUF_CHAIN_FLAGS_AT 64u
+#define GGUF_CHAIN_PROGRESS_WORDS (GGUF_CHAIN_FLAGS_AT + GGUF_CHAIN_LINKS * GGUF_CHAIN_FLAGS * GGUF_CHAIN_FLAG_STRIDE)
+struct GgufChainLink {
+  struct GgufDecodeParams p;
+  uint32_t first_item;  // the link's first workgroup of the dispatch
+  uint32_t format;      // GGUF_FMT_* of its segments (the formats of a mixed link are p.formats)
+  uint32_t epilogue;    // GGUF_EPILOGUE_PLAIN, _PLAIN_F32, _GATE_UP_TABLE or _RESIDUAL_NORM
+  uint32_t mixed;       // nonzero: segments of several formats, plain bf16 rows
+  uint32_t groups;      // workgroups that write the link's results: each counts itself in when they are out
+  uint32_t reserved[3];
+};
+struct GgufChainParams {
+  uint32_t links;       // 1..GGUF_CHAIN_LINKS
+  uint32_t spin_limit;  // polls of a workgroup's wait before it gives up
+  uint32_t reserved[2];
+  struct GgufChainLink link[GGUF_CHAIN_LINKS];
+};
+
 // gguf_dequant_<fmt>: the image's fp32 values [N][K], for the bit-exactness test
 // (the reference's gguf_dequant_test.metal). Grid (K / 256, N / 16), 64 threads.
 struct GgufDequantParams {
@@ -230,6 +265,7 @@ struct GgufEmbedParams {
 #ifdef __cplusplus
 static_assert(sizeof(GgufPrepareParams) == 16, "prepare parameters are 16 bytes on both sides");
 static_assert(sizeof(GgufDecodeParams) == 64, "decode parameters are 64 bytes on both sides");
+static_assert(sizeof(GgufChainLink) == 96 && sizeof(GgufChainParams) == 400, "chain parameters are 400 bytes on both sides");
 static_assert(sizeof(GgufDequantParams) == 8, "dequant parameters are 8 bytes on both sides");
 static_assert(sizeof(GgufEmbedParams) == 12, "embedding parameters are 12 bytes on both sides");
 #endif

@@ -249,8 +249,15 @@ sp_status spo_dense_verify_results(spo_dense_verify *verify, const spo_verify_la
     std::vector<model::StepLane> list;
     uint32_t first = 0;
     for (const model::VerifyLane &l : lanesOf(lanes, count)) { list.push_back({first, l.rows, l.remaining}); first += l.rows; }
+    if (v.takeChainStatus()) throw hip::BackendError("a chained projection's wait for the one before it gave up: the step's results are void");
     model::readStepResults(list, v.tokens(), v.retained(), v.acceptedCount(), v.retainedRows(), v.dimensions().vocabulary, tokens, retained,
                            accepted, retained_rows);
+  });
+}
+sp_status spo_dense_verify_set_chained(spo_dense_verify *verify, int chained) {
+  return capi::guard([&] {
+    capi::require(verify, "verify");
+    verify->verify->setChained(chained != 0);
   });
 }
 uint64_t spo_dense_verify_page_bytes(const spo_dense_verify *verify) { return verify ? verify->verify->pageBytes() : 0; }

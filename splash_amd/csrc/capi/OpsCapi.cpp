@@ -145,6 +145,14 @@ sp_status spo_linear_create_calibrated(uint32_t compute_units, uint32_t groups_p
   });
 }
 void spo_linear_destroy(spo_linear *linear) { delete linear; }
+sp_status spo_linear_set_chain_spin_limit(spo_linear *linear, uint32_t polls) {
+  return capi::guard([&] {
+    capi::require(linear, "linear");
+    ops::KernelCalibration calibration = linear->linear.calibration();
+    calibration.chainSpinLimit = polls;
+    linear->linear = ops::Linear(calibration);
+  });
+}
 
 sp_status spo_linear_plan_for(const spo_linear *linear, const spo_projection *projection, uint32_t rows, uint32_t epilogue,
                               spo_linear_plan *out) {
@@ -192,6 +200,36 @@ sp_status spo_linear_add_residual_norm(const spo_linear *linear, spo_graph *grap
     const ops::LinearPlan full = toPlan(projection->projection, *plan);
     if (full.workload().epilogue != ops::LinearEpilogue::ResidualNorm) throw std::invalid_argument("the plan does not norm its rows");
     linear->linear.add(graph->graph, std::move(buffers), projection->projection, full);
+  });
+}
+namespace {
+ops::ChainedProjection linkOf(const spo_chain_link &l) {
+  capi::require(l.projection, "a link's projection");
+  ops::LinearBuffers buffers;
+  buffers.input = hip::Buffer::share(l.input);
+  buffers.output = hip::Buffer::share(l.output);
+  buffers.residual = hip::Buffer::share(l.residual);
+  buffers.normWeight = hip::Buffer::share(l.norm_weight);
+  buffers.nextTable = hip::Buffer::share(l.next_table);
+  buffers.scratch = scratchOf(l.table, l.partials, l.counters);
+  if (l.prepared) buffers.prepared = {buffers.input, l.prepared == 2 ? ops::LinearInput::TableUnscaled : ops::LinearInput::Table16};
+  return {std::move(buffers), &l.projection->projection, toPlan(l.projection->projection, l.plan), l.gate ? &l.gate->projection : nullptr};
+}
+} // namespace
+sp_status spo_linear_add_chain(const spo_linear *linear, spo_graph *graph, const spo_chain_link *links, uint32_t count,
+                               sp_buffer *progress) {
+  return capi::guard([&] {
+    capi::require(linear && graph && links && progress, "linear, graph, links or progress");
+    std::vector<ops::ChainedProjection> chain;
+    for (uint32_t i = 0; i < count; ++i) chain.push_back(linkOf(links[i]));
+    linear->linear.addChain(graph->graph, std::move(chain), hip::Buffer::share(progress));
+  });
+}
+sp_status spo_linear_add_link(const spo_linear *linear, spo_graph *graph, const spo_chain_link *link) {
+  return capi::guard([&] {
+    capi::require(linear && graph && link, "linear, graph or link");
+    ops::ChainedProjection one = linkOf(*link);
+    linear->linear.add(graph->graph, std::move(one.buffers), *one.projection, one.plan, one.gate);
   });
 }
 sp_status spo_linear_add_swiglu(const spo_linear *linear, spo_graph *graph, const spo_projection *gate,

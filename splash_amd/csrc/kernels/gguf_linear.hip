@@ -493,12 +493,66 @@ template <int RT> struct DecodeShared {
   float scaleParts[256 * RT], rowScale[16 * RT];  // of a table with a deferred scale
 };
 
-template <uint32_t FMT, int RT, uint32_t EP>
+// A projection's place in a chain of projections that share one dispatch (gguf_decode_chain): link i + 1 reads what link
+// i's epilogues wrote, so its workgroups, which the device starts after every workgroup of link i, fetch their first
+// weights, which depend on nothing, and then wait for link i's count of finished workgroups. Results that a later link
+// reads leave through agent-scope stores, which go to the memory side of the compute dies' caches, and are counted in
+// only once those stores have completed; the reader finds no older copy of them in its own die's cache because nothing
+// of the dispatch read those addresses before (every link has tables, partials and counters of its own) and every
+// cache line it reads through the cache had a single writer.
+struct ChainPosition {
+  // The link before's go flag this workgroup polls (one of GGUF_CHAIN_FLAGS words in cache lines of their own, so that the
+  // device's waiting workgroups do not all ask one memory channel for one word); null for the first link.
+  uint32_t *wait;
+  uint32_t *done;       // this link's count, of doneTarget workgroups
+  uint32_t doneTarget;
+  uint32_t *flags;      // this link's go flags, which the workgroup that completes the count sets; null for the last link
+  uint32_t *flagsBefore;  // the link before's, which that workgroup clears: every workgroup of this link has passed them
+  uint32_t spinLimit;   // polls a workgroup waits before it gives up and reports through *status
+  uint32_t *status;
+};
+template <bool Coherent, class T> __device__ __forceinline__ void store_result(T *at, T value) {
+  if constexpr (Coherent) __hip_atomic_store(at, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  else *at = value;
+}
+template <bool Coherent, class T> __device__ __forceinline__ T load_result(const T *at) {
+  if constexpr (Coherent) return __hip_atomic_load(at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  else return *at;
+}
+// The wait of a link's workgroup: one thread polls, with a bound, so that every wave ends whatever the count does.
+__device__ __forceinline__ void chain_wait(const ChainPosition &chain) {
+  if (chain.wait) {
+    if (threadIdx.x == 0) {
+      uint32_t polls = 0;
+      while (__hip_atomic_load(chain.wait, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0u) {
+        if (++polls > chain.spinLimit) {
+          __hip_atomic_store(chain.status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          break;
+        }
+        __builtin_amdgcn_s_sleep(8);
+      }
+    }
+    __syncthreads();
+  }
+#ifdef SP_CHAIN_TRACE
+  if (threadIdx.x == 0) reinterpret_cast<uint64_t *>(chain.status - GGUF_CHAIN_LINKS + GGUF_CHAIN_PROGRESS_WORDS)[blockIdx.x * 4u + 1u] = wall_clock64();
+#endif
+  // nothing that reads the link before's results moves above the wait
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+  __builtin_amdgcn_sched_barrier(0);
+}
+
+template <uint32_t FMT, int RT, uint32_t EP, bool Chain = false>
 __device__ __forceinline__ void decode_workgroup(DecodeShared<RT> &shared, const uint8_t *__restrict__ seg0,
                                                  const uint8_t *__restrict__ seg1, const uint8_t *__restrict__ seg2,
                                                  const uint8_t *__restrict__ table, void *__restrict__ out,
                                                  const uint16_t *__restrict__ residual, float *__restrict__ partials,
-                                                 uint32_t *__restrict__ counters, const GgufDecodeParams &p, const uint32_t item) {
+                                                 uint32_t *__restrict__ counters, const GgufDecodeParams &p, const uint32_t item,
+                                                 const ChainPosition &chain = ChainPosition{}) {
+  // A chained link reads only what has one writer a cache line: a group's values, a workgroup's 16-input sums, a squares
+  // entry. The 32-input sums have two (a gate/up workgroup writes 64 bytes of them), so a chained link adds the two
+  // 16-input sums they are the sum of, the same fp32 addition their writer made.
+  constexpr bool kPairSums = Chain && FMT != GGUF_FMT_Q6K;
   constexpr uint32_t kRecord = gguf_record_bytes(FMT);
   constexpr bool kTable = EP == GGUF_EPILOGUE_GATE_UP_TABLE, kGateUp = EP == GGUF_EPILOGUE_GATE_UP || kTable;
   constexpr uint32_t kColumnPart = Cursor<FMT>::kColumnPart;
@@ -562,6 +616,7 @@ __device__ __forceinline__ void decode_workgroup(DecodeShared<RT> &shared, const
       Record<FMT> rec;
       uint4 a[2 * RT];       // this thread's share of the super-block's RT * 8 * 64 operand vectors
       float sum[kSumShare];  // and of its row sums
+      float second[kPairSums ? kSumShare : 1];  // a chained link: the other 16-input half of a 32-input sum
     };
     Stage stage[kStages];
     // A wave without a tile reads an empty range.
@@ -575,32 +630,43 @@ __device__ __forceinline__ void decode_workgroup(DecodeShared<RT> &shared, const
     uint32_t share[2];  // vector j of a row tile's super-block: byte offset of this thread's
 #pragma unroll
     for (int j = 0; j < 2; ++j) share[j] = (threadIdx.x + 256u * j) * 16u;
-    const uint32_t sumsAt = kSums32 ? gguf_table_sums32_offset(p.input_size, tiles) : gguf_table_sums16_offset(p.input_size, tiles);
+    const uint32_t sumsAt = kSums32 && !kPairSums ? gguf_table_sums32_offset(p.input_size, tiles) : gguf_table_sums16_offset(p.input_size, tiles);
     const uint32_t sumGroups = kSums32 ? G : 2u * G;  // row-sum entries per row tile
-    const Resource sums = make_resource(table + sumsAt, tiles * sumGroups * 64u);
+    const Resource sums = make_resource(table + sumsAt, tiles * (kPairSums ? 2u * G : sumGroups) * 64u);
     // Threads past the staged sums repeat an earlier thread's (same value to the same slot).
     uint32_t sumShare[kSumShare], sumSlot[kSumShare];
 #pragma unroll
     for (int q = 0; q < kSumShare; ++q) {
       const uint32_t at = (threadIdx.x + 256u * q) % kSumFloats;
       const uint32_t t = at / (kSumsPerBlock * 64u), j = (at / 64u) % kSumsPerBlock, l = at % 64u;
-      sumShare[q] = ((t * sumGroups + kSumsPerBlock * 4u * b0 + 4u * j + (l >> 4)) * 16u + (l & 15u)) * 4u;
+      sumShare[q] = ((t * sumGroups + kSumsPerBlock * 4u * b0 + 4u * j + (l >> 4)) * 16u * (kPairSums ? 2u : 1u) + (l & 15u)) * 4u;
       sumSlot[q] = (t * 4u + j) * 64u + l;
     }
-    auto issue = [&](Stage &st) {
+    auto issueTable = [&](Stage &st) {
 #pragma unroll
       for (int j = 0; j < 2 * RT; ++j) st.a[j] = load128<0>(values[j / 2], share[j % 2]);
 #pragma unroll
       for (int q = 0; q < kSumShare; ++q)
         st.sum[q] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(sums, int(sumShare[q]), 0, 0));
-      load_record(st.rec, weights, mine, column);
-      mine += kRecord;
-      column += kRecord;
+      if constexpr (kPairSums) {
+#pragma unroll
+        for (int q = 0; q < kSumShare; ++q)
+          st.second[q] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(sums, int(sumShare[q] + 64u), 0, 0));
+      }
 #pragma unroll
       for (int j = 0; j < 2; ++j) share[j] += 8192u;
       // Sums past the range are the next range's or, past the table, zeros: staged and never used.
 #pragma unroll
-      for (int q = 0; q < kSumShare; ++q) sumShare[q] += kSumsPerBlock * 4u * 16u * 4u;
+      for (int q = 0; q < kSumShare; ++q) sumShare[q] += kSumsPerBlock * 4u * 16u * 4u * (kPairSums ? 2u : 1u);
+    };
+    auto issueWeights = [&](Stage &st) {
+      load_record(st.rec, weights, mine, column);
+      mine += kRecord;
+      column += kRecord;
+    };
+    auto issue = [&](Stage &st) {
+      issueTable(st);
+      issueWeights(st);
     };
     // Every row's inverse RMS from the squares the table's writer left, one entry a 64-column group:
     // part q of 16 adds entries q, q + 16, ... in order, then the 16 parts are added in order -- the same
@@ -617,7 +683,7 @@ __device__ __forceinline__ void decode_workgroup(DecodeShared<RT> &shared, const
     float squareSum[RT], loaded[RT][kChunk];
 #pragma unroll
     for (int i = 0; i < RT; ++i) squareSum[i] = 0.f;
-    const uint32_t squareRow = threadIdx.x % kRows, squareEntries = p.input_size / 64u, squareStride = 16u * tiles * 4u;
+    const uint32_t squareRow = threadIdx.x % kRows, squareEntries = p.input_size / 64u, squareStride = gguf_squares_stride(tiles) * 4u;
     const Resource squares = make_resource(table + gguf_table_squares_offset(p.input_size, tiles),
                                            p.deferred_scale && squareRow < 16u * tiles ? squareEntries * squareStride : 0u);
     auto loadSquares = [&](int i, uint32_t base) {
@@ -629,14 +695,32 @@ __device__ __forceinline__ void decode_workgroup(DecodeShared<RT> &shared, const
 #pragma unroll
       for (uint32_t e = 0; e < kChunk; ++e) squareSum[i] += loaded[i][e];
     };
+    if constexpr (Chain) {
+      // The first stages' weights go out, then the wait for the link before, then what that link wrote.
 #pragma unroll
-    for (int i = 0; i < RT; ++i) loadSquares(i, threadIdx.x / kRows + kThreadParts * i);
-    __builtin_amdgcn_sched_barrier(0);
+      for (int s = 0; s < kStages - 1; ++s) {
+        issueWeights(stage[s]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      chain_wait(chain);
 #pragma unroll
-    for (int s = 0; s < kStages - 1; ++s) {
-      issue(stage[s]);
-      // Keep the stages' loads in issue order: the loop's counted waits assume it on entry too.
+      for (int i = 0; i < RT; ++i) loadSquares(i, threadIdx.x / kRows + kThreadParts * i);
       __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int s = 0; s < kStages - 1; ++s) {
+        issueTable(stage[s]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < RT; ++i) loadSquares(i, threadIdx.x / kRows + kThreadParts * i);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int s = 0; s < kStages - 1; ++s) {
+        issue(stage[s]);
+        // Keep the stages' loads in issue order: the loop's counted waits assume it on entry too.
+        __builtin_amdgcn_sched_barrier(0);
+      }
     }
 #pragma unroll
     for (int i = 0; i < RT; ++i) {
@@ -668,7 +752,8 @@ __device__ __forceinline__ void decode_workgroup(DecodeShared<RT> &shared, const
 #pragma unroll
         for (int j = 0; j < 2 * RT; ++j) (&ldsA[buffer][0][0][0])[threadIdx.x + 256u * j] = stage[u].a[j];
 #pragma unroll
-        for (int q = 0; q < kSumShare; ++q) (&ldsSums[buffer][0][0][0])[sumSlot[q]] = stage[u].sum[q];
+        for (int q = 0; q < kSumShare; ++q)
+          (&ldsSums[buffer][0][0][0])[sumSlot[q]] = kPairSums ? stage[u].sum[q] + stage[u].second[q] : stage[u].sum[q];
         __syncthreads();
         issue(stage[(u + kStages - 1) % kStages]);
         if (now < count) accumulate_record<FMT, RT>(stage[u].rec, ldsA[buffer], ldsSums[buffer], acc, lane, kq);
@@ -676,6 +761,9 @@ __device__ __forceinline__ void decode_workgroup(DecodeShared<RT> &shared, const
     }
   }
 
+#ifdef SP_CHAIN_TRACE
+  if constexpr (Chain) if (threadIdx.x == 0) reinterpret_cast<uint64_t *>(chain.status - GGUF_CHAIN_LINKS + GGUF_CHAIN_PROGRESS_WORDS)[blockIdx.x * 4u + 2u] = wall_clock64();
+#endif
   // Element (t, v) of this lane is row 16 t + 4 kq + v, column tile.column + c.
   if (splits > 1) {
     // Partials [split][partitioned unit][t][v][lane]: whole-wave contiguous stores and loads.
@@ -768,7 +856,7 @@ __device__ __forceinline__ void decode_workgroup(DecodeShared<RT> &shared, const
       __syncthreads();
       uint8_t *next = reinterpret_cast<uint8_t *>(const_cast<uint16_t *>(residual));
       const uint32_t G2 = p.out_stride / 32u, g = group;
-      uint2 *values = reinterpret_cast<uint2 *>(next);
+      uint64_t *values = reinterpret_cast<uint64_t *>(next);
       float *sums32 = reinterpret_cast<float *>(next + gguf_table_sums32_offset(p.out_stride, tiles));
       float *sums16 = reinterpret_cast<float *>(next + gguf_table_sums16_offset(p.out_stride, tiles));
       // Piece (t, half, kq, r): inputs 16 half + 4 kq .. + 3 of row 16 t + r; a wave holds one (t, half).
@@ -777,20 +865,21 @@ __device__ __forceinline__ void decode_workgroup(DecodeShared<RT> &shared, const
         if (t2 >= tiles) continue;  // a whole wave: the kernel's row tiles past the table's
         const uint2 raw = *reinterpret_cast<const uint2 *>(&tileOut[((h2 * RT + t2) * 16u + r) * 16u + 4u * q4]);
         const uint32_t x0 = raw.x & 0xFFFFu, x1 = raw.x >> 16, x2 = raw.y & 0xFFFFu, x3 = raw.y >> 16;
-        values[((size_t(t2) * G2 + g) * 64u + q4 * 16u + r) * 2u + h2] = make_uint2(x0 | (x2 << 16), x1 | (x3 << 16));
+        store_result<Chain>(&values[((size_t(t2) * G2 + g) * 64u + q4 * 16u + r) * 2u + h2],
+                            uint64_t(x0 | (x2 << 16)) | uint64_t(x1 | (x3 << 16)) << 32);
         const float run = (bf16_bits_to_float(x0) + bf16_bits_to_float(x1)) + (bf16_bits_to_float(x2) + bf16_bits_to_float(x3));
         const float r0 = __shfl(run, int(r), 64), r1 = __shfl(run, int(r) + 16, 64), r2 = __shfl(run, int(r) + 32, 64),
                     r3 = __shfl(run, int(r) + 48, 64);
         const float sum = ((r0 + r1) + r2) + r3;
         if (q4 == 0) {
-          sums16[(size_t(t2) * 2u * G2 + 2u * g + h2) * 16u + r] = sum;
+          store_result<Chain>(&sums16[(size_t(t2) * 2u * G2 + 2u * g + h2) * 16u + r], sum);
           halfSums[(t2 * 2u + h2) * 16u + r] = sum;
         }
       }
       __syncthreads();
       if (threadIdx.x < tiles * 16u) {
         const uint32_t t2 = threadIdx.x >> 4, r = threadIdx.x & 15u;
-        sums32[(size_t(t2) * G2 + g) * 16u + r] = halfSums[(t2 * 2u) * 16u + r] + halfSums[(t2 * 2u + 1u) * 16u + r];
+        store_result<Chain>(&sums32[(size_t(t2) * G2 + g) * 16u + r], halfSums[(t2 * 2u) * 16u + r] + halfSums[(t2 * 2u + 1u) * 16u + r]);
       }
     }
   } else if constexpr (EP == GGUF_EPILOGUE_RESIDUAL_NORM) {
@@ -815,8 +904,8 @@ __device__ __forceinline__ void decode_workgroup(DecodeShared<RT> &shared, const
         uint32_t scaled = 0;
         if (owns && row < p.rows) {
           const size_t at = size_t(row) * p.out_stride + tile.column + c;
-          const uint32_t bits = float_to_bf16_bits(acc[t][v] + bf16_bits_to_float(residual[at]));
-          static_cast<uint16_t *>(out)[at] = uint16_t(bits);
+          const uint32_t bits = float_to_bf16_bits(acc[t][v] + bf16_bits_to_float(load_result<Chain>(&residual[at])));
+          store_result<Chain>(&static_cast<uint16_t *>(out)[at], uint16_t(bits));
           hidden = bf16_bits_to_float(bits);
           scaled = float_to_bf16_bits(hidden * weight);
         }
@@ -831,11 +920,11 @@ __device__ __forceinline__ void decode_workgroup(DecodeShared<RT> &shared, const
     if (threadIdx.x < 16u * tiles) {
       const float *w = waveSquares + threadIdx.x;
       float *squares = reinterpret_cast<float *>(next + gguf_table_squares_offset(p.out_stride, tiles));
-      squares[size_t(group) * 16u * tiles + threadIdx.x] = ((w[0] + w[kRows]) + w[2u * kRows]) + w[3u * kRows];
+      store_result<Chain>(&squares[size_t(group) * gguf_squares_stride(tiles) + threadIdx.x], ((w[0] + w[kRows]) + w[2u * kRows]) + w[3u * kRows]);
     }
     // The workgroup's 64 columns: two groups of the next projection's inputs.
     const uint32_t G2 = p.out_stride / 32u;
-    uint2 *values = reinterpret_cast<uint2 *>(next);
+    uint64_t *values = reinterpret_cast<uint64_t *>(next);
     float *sums32 = reinterpret_cast<float *>(next + gguf_table_sums32_offset(p.out_stride, tiles));
     float *sums16 = reinterpret_cast<float *>(next + gguf_table_sums16_offset(p.out_stride, tiles));
     // Piece (t, w, kq, r): inputs 16 (w % 2) + 4 kq .. + 3 of group 2 group + w / 2, row 16 t + r.
@@ -845,36 +934,63 @@ __device__ __forceinline__ void decode_workgroup(DecodeShared<RT> &shared, const
       const uint32_t g2 = 2u * group + (w2 >> 1), h2 = w2 & 1u;
       const uint2 raw = *reinterpret_cast<const uint2 *>(&tileOut[((w2 * RT + t2) * 16u + r) * 16u + 4u * q4]);
       const uint32_t x0 = raw.x & 0xFFFFu, x1 = raw.x >> 16, x2 = raw.y & 0xFFFFu, x3 = raw.y >> 16;
-      values[((size_t(t2) * G2 + g2) * 64u + q4 * 16u + r) * 2u + h2] = make_uint2(x0 | (x2 << 16), x1 | (x3 << 16));
+      store_result<Chain>(&values[((size_t(t2) * G2 + g2) * 64u + q4 * 16u + r) * 2u + h2],
+                          uint64_t(x0 | (x2 << 16)) | uint64_t(x1 | (x3 << 16)) << 32);
       const float run = (bf16_bits_to_float(x0) + bf16_bits_to_float(x1)) + (bf16_bits_to_float(x2) + bf16_bits_to_float(x3));
       const float r0 = __shfl(run, int(r), 64), r1 = __shfl(run, int(r) + 16, 64), r2 = __shfl(run, int(r) + 32, 64),
                   r3 = __shfl(run, int(r) + 48, 64);
       const float sum = ((r0 + r1) + r2) + r3;
       if (q4 == 0) {
-        sums16[(size_t(t2) * 2u * G2 + 2u * g2 + h2) * 16u + r] = sum;
+        store_result<Chain>(&sums16[(size_t(t2) * 2u * G2 + 2u * g2 + h2) * 16u + r], sum);
         halfSums[(t2 * 4u + w2) * 16u + r] = sum;
       }
     }
     __syncthreads();
     if (threadIdx.x < tiles * 32u) {
       const uint32_t t2 = threadIdx.x >> 5, pair = (threadIdx.x >> 4) & 1u, r = threadIdx.x & 15u;
-      sums32[(size_t(t2) * G2 + 2u * group + pair) * 16u + r] =
-          halfSums[(t2 * 4u + 2u * pair) * 16u + r] + halfSums[(t2 * 4u + 2u * pair + 1u) * 16u + r];
+      store_result<Chain>(&sums32[(size_t(t2) * G2 + 2u * group + pair) * 16u + r],
+                          halfSums[(t2 * 4u + 2u * pair) * 16u + r] + halfSums[(t2 * 4u + 2u * pair + 1u) * 16u + r]);
     }
   } else {
-    if (!live || !tile.image) return;
+    if (live && tile.image) {
 #pragma unroll
-    for (int t = 0; t < RT; ++t)
+      for (int t = 0; t < RT; ++t)
 #pragma unroll
-      for (int v = 0; v < 4; ++v) {
-        const uint32_t row = 16u * t + 4u * kq + v;
-        if (row >= p.rows) continue;
-        const size_t at = size_t(row) * p.out_stride + tile.column + c;
-        if constexpr (EP == GGUF_EPILOGUE_PLAIN_F32) static_cast<float *>(out)[at] = acc[t][v];
-        else if constexpr (EP == GGUF_EPILOGUE_RESIDUAL)
-          static_cast<uint16_t *>(out)[at] = uint16_t(float_to_bf16_bits(acc[t][v] + bf16_bits_to_float(residual[at])));
-        else static_cast<uint16_t *>(out)[at] = uint16_t(float_to_bf16_bits(acc[t][v]));
+        for (int v = 0; v < 4; ++v) {
+          const uint32_t row = 16u * t + 4u * kq + v;
+          if (row >= p.rows) continue;
+          const size_t at = size_t(row) * p.out_stride + tile.column + c;
+          if constexpr (EP == GGUF_EPILOGUE_PLAIN_F32) static_cast<float *>(out)[at] = acc[t][v];
+          else if constexpr (EP == GGUF_EPILOGUE_RESIDUAL)
+            store_result<Chain>(&static_cast<uint16_t *>(out)[at],
+                                uint16_t(float_to_bf16_bits(acc[t][v] + bf16_bits_to_float(load_result<Chain>(&residual[at])))));
+          else static_cast<uint16_t *>(out)[at] = uint16_t(float_to_bf16_bits(acc[t][v]));
+        }
+    }
+  }
+  if constexpr (Chain) {
+    // The workgroup's results are out (its stores have completed) before it counts itself in; the one that completes
+    // the count clears the count it waited for, which every workgroup of this link has passed by then.
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+#ifdef SP_CHAIN_TRACE
+    if (threadIdx.x == 0) reinterpret_cast<uint64_t *>(chain.status - GGUF_CHAIN_LINKS + GGUF_CHAIN_PROGRESS_WORDS)[blockIdx.x * 4u + 3u] = wall_clock64();
+#endif
+    if (threadIdx.x < 64u) {
+      uint32_t before = 0;
+      if (threadIdx.x == 0) before = __hip_atomic_fetch_add(chain.done, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      before = uint32_t(__builtin_amdgcn_readfirstlane(int(before)));
+      if (before + 1u == chain.doneTarget) {
+        // the link is complete: its count returns to zero (nobody reads it), the next link's workgroups may go, and the
+        // flags this link's workgroups waited for are cleared for the next dispatch; a lane a flag
+        static_assert(GGUF_CHAIN_FLAGS == 64u, "one wave sets a link's flags");
+        if (threadIdx.x == 0) __hip_atomic_store(chain.done, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (chain.flags) __hip_atomic_store(chain.flags + threadIdx.x * GGUF_CHAIN_FLAG_STRIDE, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (chain.flagsBefore)
+          __hip_atomic_store(chain.flagsBefore + threadIdx.x * GGUF_CHAIN_FLAG_STRIDE, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
+    }
   }
 }
 
@@ -970,6 +1086,111 @@ __global__ __launch_bounds__(256) void gguf_decode_mixed(const uint8_t *__restri
 SP_REGISTER_KERNEL("gguf_decode_mixed_m16_a", &gguf_decode_mixed<1>);
 SP_REGISTER_KERNEL("gguf_decode_mixed_m32_a", &gguf_decode_mixed<2>);
 SP_REGISTER_KERNEL("gguf_decode_mixed_m64_a", &gguf_decode_mixed<4>);
+
+// A chain of up to four projections in one dispatch (GgufChainParams): link i's workgroups are items
+// link[i].first_item .. of the grid, in link order, so the device has started every workgroup of a link before any of
+// the next one's, and a workgroup that waits for the link before (ChainPosition) waits only for workgroups that are
+// running or done. Each link binds the eight buffers of a gguf_decode dispatch; `progress` (abi/Gguf.h) holds a count
+// of finished workgroups per link, a status word that a wait that ran out of polls sets, and each link's go flags.
+// A link of several formats is a plain one, as gguf_decode_mixed's. Rows of one piece (up to 64).
+template <uint32_t FMT, int RT>
+__device__ __forceinline__ void chain_link(DecodeShared<RT> &shared, uint32_t epilogue, const uint8_t *seg0, const uint8_t *seg1,
+                                           const uint8_t *seg2, const uint8_t *table, void *out, const uint16_t *residual,
+                                           float *partials, uint32_t *counters, const GgufDecodeParams &p, uint32_t item,
+                                           const ChainPosition &chain) {
+  switch (epilogue) {
+  case GGUF_EPILOGUE_PLAIN:
+    decode_workgroup<FMT, RT, GGUF_EPILOGUE_PLAIN, true>(shared, seg0, seg1, seg2, table, out, residual, partials, counters, p, item, chain);
+    break;
+  case GGUF_EPILOGUE_PLAIN_F32:
+    decode_workgroup<FMT, RT, GGUF_EPILOGUE_PLAIN_F32, true>(shared, seg0, seg1, seg2, table, out, residual, partials, counters, p, item, chain);
+    break;
+  case GGUF_EPILOGUE_GATE_UP_TABLE:
+    decode_workgroup<FMT, RT, GGUF_EPILOGUE_GATE_UP_TABLE, true>(shared, seg0, seg1, seg2, table, out, residual, partials, counters, p, item, chain);
+    break;
+  case GGUF_EPILOGUE_RESIDUAL_NORM:
+    decode_workgroup<FMT, RT, GGUF_EPILOGUE_RESIDUAL_NORM, true>(shared, seg0, seg1, seg2, table, out, residual, partials, counters, p, item, chain);
+    break;
+  default: break;
+  }
+}
+
+#define SP_CHAIN_LINK_PARAMETERS(n)                                                                                              \
+  const uint8_t *__restrict__ seg0_##n, const uint8_t *__restrict__ seg1_##n, const uint8_t *__restrict__ seg2_##n,             \
+      const uint8_t *__restrict__ table_##n, void *__restrict__ out_##n, const uint16_t *__restrict__ residual_##n,             \
+      float *__restrict__ partials_##n, uint32_t *__restrict__ counters_##n
+template <int RT>
+__global__ __launch_bounds__(256) void gguf_decode_chain(SP_CHAIN_LINK_PARAMETERS(0), SP_CHAIN_LINK_PARAMETERS(1),
+                                                         SP_CHAIN_LINK_PARAMETERS(2), SP_CHAIN_LINK_PARAMETERS(3),
+                                                         uint32_t *__restrict__ progress, GgufChainParams cp) {
+  uint32_t link = 0;
+#pragma unroll
+  for (uint32_t l = 1; l < GGUF_CHAIN_LINKS; ++l)
+    if (l < cp.links && blockIdx.x >= cp.link[l].first_item) link = l;
+  auto pick = [&](auto a, auto b, auto c, auto d) { return link == 0 ? a : link == 1 ? b : link == 2 ? c : d; };
+  const uint8_t *seg0 = pick(seg0_0, seg0_1, seg0_2, seg0_3), *seg1 = pick(seg1_0, seg1_1, seg1_2, seg1_3);
+  const uint8_t *seg2 = pick(seg2_0, seg2_1, seg2_2, seg2_3), *table = pick(table_0, table_1, table_2, table_3);
+  void *out = pick(out_0, out_1, out_2, out_3);
+  const uint16_t *residual = pick(residual_0, residual_1, residual_2, residual_3);
+  float *partials = pick(partials_0, partials_1, partials_2, partials_3);
+  uint32_t *counters = pick(counters_0, counters_1, counters_2, counters_3);
+  const GgufChainLink &mine = cp.link[link];  // (the parameters lie in constant memory: an indexed scalar load)
+  ChainPosition chain;
+  auto flagsOf = [&](uint32_t l) { return progress + GGUF_CHAIN_FLAGS_AT + l * GGUF_CHAIN_FLAGS * GGUF_CHAIN_FLAG_STRIDE; };
+  chain.flagsBefore = link ? flagsOf(link - 1u) : nullptr;
+  chain.wait = link ? chain.flagsBefore + (blockIdx.x % GGUF_CHAIN_FLAGS) * GGUF_CHAIN_FLAG_STRIDE : nullptr;
+  chain.done = progress + link;
+  chain.doneTarget = mine.groups;
+  chain.flags = link + 1u == cp.links ? nullptr : flagsOf(link);
+  chain.spinLimit = cp.spin_limit;
+  chain.status = progress + GGUF_CHAIN_LINKS;
+#ifdef SP_CHAIN_TRACE
+  if (threadIdx.x == 0) reinterpret_cast<uint64_t *>(chain.status - GGUF_CHAIN_LINKS + GGUF_CHAIN_PROGRESS_WORDS)[blockIdx.x * 4u] = wall_clock64();
+#endif
+  GgufDecodeParams p = mine.p;
+  p.rows = min(p.rows, uint32_t(GGUF_MAXIMUM_ROWS));
+  uint32_t item = blockIdx.x - mine.first_item;
+  uint32_t format = mine.format, epilogue = mine.epilogue;
+  if (mine.mixed) {
+    // as gguf_decode_mixed: the workgroup's segment alone, in that segment's format
+    constexpr uint32_t kGroupFloats = 4u * RT * 256u;
+    const uint32_t group = item / p.splits, split = item % p.splits;
+    uint32_t segment = 0, past = 0;
+#pragma unroll
+    for (uint32_t s = 0; s < 2u; ++s)
+      if (segment == s && group >= past + p.cols[s] / 64u) {
+        past += p.cols[s] / 64u;
+        segment = s + 1u;
+      }
+    auto of = [&](const uint32_t (&field)[3]) { return segment == 0 ? field[0] : segment == 1 ? field[1] : field[2]; };
+    seg0 = segment == 0 ? seg0 : segment == 1 ? seg1 : seg2;
+    format = of(p.formats);
+    const uint32_t columns = of(p.cols), offset = of(p.offset);
+    p.cols[0] = columns;
+    p.cols[1] = p.cols[2] = 0;
+    p.offset[0] = offset;
+    p.units = columns / GGUF_TILE_COLUMNS;
+    p.whole_groups = 0;
+    partials += size_t(past) * p.splits * kGroupFloats;
+    counters += past;
+    item = (group - past) * p.splits + split;
+    epilogue = GGUF_EPILOGUE_PLAIN;
+  }
+  __shared__ DecodeShared<RT> shared;
+  switch (format) {
+  case GGUF_FMT_Q4K: chain_link<GGUF_FMT_Q4K, RT>(shared, epilogue, seg0, seg1, seg2, table, out, residual, partials, counters, p, item, chain); break;
+  case GGUF_FMT_Q5K: chain_link<GGUF_FMT_Q5K, RT>(shared, epilogue, seg0, seg1, seg2, table, out, residual, partials, counters, p, item, chain); break;
+  case GGUF_FMT_Q6K: chain_link<GGUF_FMT_Q6K, RT>(shared, epilogue, seg0, seg1, seg2, table, out, residual, partials, counters, p, item, chain); break;
+  case GGUF_FMT_Q80: chain_link<GGUF_FMT_Q80, RT>(shared, epilogue, seg0, seg1, seg2, table, out, residual, partials, counters, p, item, chain); break;
+  case GGUF_FMT_IQ4XS: chain_link<GGUF_FMT_IQ4XS, RT>(shared, epilogue, seg0, seg1, seg2, table, out, residual, partials, counters, p, item, chain); break;
+  case GGUF_FMT_IQ4NL: chain_link<GGUF_FMT_IQ4NL, RT>(shared, epilogue, seg0, seg1, seg2, table, out, residual, partials, counters, p, item, chain); break;
+  default: break;
+  }
+}
+#undef SP_CHAIN_LINK_PARAMETERS
+SP_REGISTER_KERNEL("gguf_decode_chain_m16", &gguf_decode_chain<1>);
+SP_REGISTER_KERNEL("gguf_decode_chain_m32", &gguf_decode_chain<2>);
+SP_REGISTER_KERNEL("gguf_decode_chain_m64", &gguf_decode_chain<4>);
 
 // The routed experts of a mixture-of-experts layer (the reference's moe_expert_gguf_*, abi/MoE.h):
 // grid (workgroups of one expert projection, tile slots). Tile t holds up to 16 rows routed to

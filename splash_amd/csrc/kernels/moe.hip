@@ -240,7 +240,7 @@ __global__ __launch_bounds__(256) void moe_combine(const uint16_t *__restrict__ 
   }
   if (lane == 0) {
     float *squares = reinterpret_cast<float *>(table + gguf_table_squares_offset(p.hidden, tiles));
-    squares[size_t(blockIdx.y * 4u + wave) * 16u * tiles + 16u * tile + r] = square;
+    squares[size_t(blockIdx.y * 4u + wave) * gguf_squares_stride(tiles) + 16u * tile + r] = square;
   }
 }
 SP_REGISTER_KERNEL("moe_combine", &moe_combine);

@@ -62,6 +62,15 @@ DenseVerify::DenseVerify(hip::Backend &backend, DenseDimensions d, uint32_t maxL
   scratch_.counters = device(std::max<uint64_t>(size.counters, 4), "linear counters");
   // The attention merge and the gate/up pass write the table of the projection after them here.
   nextTable_ = device(gguf_table_bytes(std::max(d.attentionWidth(), d.ffn), gguf_row_tiles(maxRows_)), "linear table 2");
+  // Chained projections each keep a table, partials and counters of their own.
+  chainTables_[0] = device(gguf_table_bytes(d.hidden, gguf_row_tiles(maxRows_)), "gate/up table");
+  chainTables_[1] = device(gguf_table_bytes(d.ffn, gguf_row_tiles(maxRows_)), "down table");
+  for (ops::LinearScratch &link : chainScratch_) {
+    link.partials = device(size.partials, "chained partials");
+    link.counters = device(std::max<uint64_t>(size.counters, 4), "chained counters");
+  }
+  chainProgress_ = device(GGUF_CHAIN_PROGRESS_WORDS * 4, "chain progress");
+  chainProgress_.fill(0, GGUF_CHAIN_PROGRESS_WORDS * 4);
   // Attention workspace for the most splits any sequence may take.
   const uint64_t fused = uint64_t{maxLanes} * d.kvHeads * (d.qHeads / d.kvHeads) * 16;
   maxSplits_ = ATTENTION_MAXIMUM_SPLITS;
@@ -173,6 +182,86 @@ void DenseVerify::encodeLayer(hip::CommandGraph &graph, uint32_t layer, const op
   linear_.addSwiGlu(graph, {&w.gate, &w.up, &w.down}, ffn, next, residual, rows, prepared);
 }
 
+bool DenseVerify::chains(uint32_t rows) const noexcept {
+  if (!chained_ || rows > ops::kMaximumDecodeTileRows || !layersFeedNext(rows)) return false;
+  for (const DenseLayer &l : weights_.layers)
+    if (!linear_.normsRows(l.output, rows)) return false;
+  return true;
+}
+
+uint32_t DenseVerify::takeChainStatus() {
+  if (!encodedChains_) return 0;
+  uint32_t status = 0;
+  chainProgress_.download(&status, 4, GGUF_CHAIN_LINKS * 4);
+  if (status) chainProgress_.fill(0, GGUF_CHAIN_PROGRESS_WORDS * 4);
+  return status;
+}
+
+// The layers with their projections chained: the first layer's q|k|v on its own, then a layer's head norms, RoPE and
+// cache store, its attention, and one dispatch of its output projection, gate/up pair, down projection and the q|k|v
+// projection of the layer after it (after the last layer, the LM head).
+void DenseVerify::encodeChainedLayers(hip::CommandGraph &graph, const ops::AttentionPlan &plan, uint32_t rows) {
+  const hip::Buffer &tableQkv = scratch_.input, &tableOutput = nextTable_, &tableGateUp = chainTables_[0], &tableDown = chainTables_[1];
+  const ops::PreparedInput ready{normalized_, ops::LinearInput::TableUnscaled};
+  auto scratchOf = [&](uint32_t link, const hip::Buffer &table) {
+    ops::LinearScratch scratch = chainScratch_[link];
+    scratch.input = table;
+    return scratch;
+  };
+  {
+    const DenseLayer &first = weights_.layers.front();
+    ops::LinearBuffers qkv;
+    qkv.input = normalized_;
+    qkv.output = qkv_;
+    qkv.scratch = scratch_;
+    qkv.prepared = ops::Normalization::addRmsTable(graph, hidden_[0], first.inputNorm, normalized_, scratch_, dims_.hidden, rows);
+    linear_.add(graph, qkv, first.qkv, linear_.plan(first.qkv, rows));
+  }
+  for (uint32_t layer = 0; layer < dims_.layers; ++layer) {
+    const DenseLayer &w = weights_.layers[layer];
+    const bool lastLayer = layer + 1 == dims_.layers;
+    const ops::KvPages pages{pageTable_, kvPools_.at(layer), pageBytes_};
+    ops::AttentionProjectionBuffers projection{qkv_, w.queryNorm, w.keyNorm, ropeCos_, ropeSin_};
+    ops::PagedAttention::addProjection(graph, plan, projection, attentionWorkspace_, pages);
+    ops::PagedAttention::addAttention(graph, plan, attentionWorkspace_, treeRows_, pages, attention_, tableOutput);
+    std::vector<ops::ChainedProjection> links;
+    ops::LinearBuffers output;
+    output.input = attention_;
+    output.output = hidden_[1];
+    output.residual = hidden_[0];
+    output.scratch = scratchOf(0, tableOutput);
+    output.prepared = {attention_, ops::LinearInput::Table16};
+    output.normWeight = w.postNorm;
+    output.nextTable = tableGateUp;
+    links.push_back({output, &w.output, linear_.plan(w.output, rows, ops::LinearEpilogue::ResidualNorm)});
+    ops::LinearBuffers pair;
+    pair.input = normalized_;
+    pair.output = intermediate_;
+    pair.scratch = scratchOf(1, tableGateUp);
+    pair.prepared = ready;
+    pair.nextTable = tableDown;
+    links.push_back({pair, &w.up, linear_.plan(w.up, rows, ops::LinearEpilogue::GateUp), &w.gate});
+    ops::LinearBuffers down;
+    down.input = intermediate_;
+    down.output = hidden_[0];
+    down.residual = hidden_[1];
+    down.scratch = scratchOf(2, tableDown);
+    down.prepared = {intermediate_, ops::LinearInput::Table16};
+    down.normWeight = lastLayer ? weights_.finalNorm : weights_.layers[layer + 1].inputNorm;
+    down.nextTable = tableQkv;
+    links.push_back({down, &w.down, linear_.plan(w.down, rows, ops::LinearEpilogue::ResidualNorm)});
+    const ops::Projection &following = lastLayer ? weights_.head : weights_.layers[layer + 1].qkv;
+    ops::LinearBuffers next;
+    next.input = normalized_;
+    next.output = lastLayer ? logits_ : qkv_;
+    next.scratch = scratchOf(3, tableQkv);
+    next.prepared = ready;
+    links.push_back({next, &following, linear_.plan(following, rows)});
+    linear_.addChain(graph, std::move(links), chainProgress_);
+  }
+  encodedChains_ = true;
+}
+
 bool DenseVerify::layersFeedNext(uint32_t rows) const noexcept {
   for (const DenseLayer &l : weights_.layers)
     if (!linear_.normsRows(l.down, rows)) return false;
@@ -215,9 +304,13 @@ void DenseVerify::encode(hip::CommandGraph &graph, const std::vector<VerifyLane>
   if (dims_.rotaryPairs)
     ops::RoPE::addTreeTables(graph, inverseFrequency_, depths_, ropeCos_, ropeSin_, dims_.rotaryPairs, rope);
   encodeEmbedding(graph, rows);
-  const bool feeds = layersFeedNext(rows);
-  for (uint32_t layer = 0; layer < dims_.layers; ++layer) encodeLayer(graph, layer, plan, rows, feeds && layer > 0, feeds);
-  encodeHead(graph, rows, feeds);
+  if (chains(rows)) {
+    encodeChainedLayers(graph, plan, rows);
+  } else {
+    const bool feeds = layersFeedNext(rows);
+    for (uint32_t layer = 0; layer < dims_.layers; ++layer) encodeLayer(graph, layer, plan, rows, feeds && layer > 0, feeds);
+    encodeHead(graph, rows, feeds);
+  }
   ops::Sampling::addVerify(graph, sampling_, dims_.vocabulary, dims_.vocabulary, laneRows, policies);
   const ops::AcceptanceBuffers acceptance{inputTokens_, treeRows_, tokens_, retained_, acceptedCount_, retainedRows_};
   ops::Sampling::addAcceptance(graph, acceptance, laneRows, remaining,

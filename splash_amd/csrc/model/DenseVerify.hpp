@@ -95,6 +95,14 @@ public:
   void encodeHead(hip::CommandGraph &graph, uint32_t rows, bool inputReady = false);
   // Whether every layer's down projection can norm its rows for the layer after it.
   [[nodiscard]] bool layersFeedNext(uint32_t rows) const noexcept;
+  // A layer's four projections after its attention -- output, gate/up, down and the next layer's q|k|v (the LM head
+  // after the last layer) -- leave as one dispatch (ops::Linear::addChain) where the shapes allow it: off by default.
+  // The results are those of the separate dispatches, bit for bit.
+  void setChained(bool chained) noexcept { chained_ = chained; }
+  [[nodiscard]] bool chained() const noexcept { return chained_; }
+  // Nonzero after a step in which a chained projection's wait for the one before it gave up: the step's results are
+  // then not to be used. Reads the device's word (a copy of four bytes) and clears it.
+  [[nodiscard]] uint32_t takeChainStatus();
 
 private:
   hip::Backend &backend_;
@@ -111,6 +119,12 @@ private:
   std::vector<hip::Buffer> kvPools_;
   ops::LinearScratch scratch_;
   hip::Buffer nextTable_;
+  // chained projections: the gate/up and down tables, each link's partials and counters, the chain's progress words
+  hip::Buffer chainTables_[2], chainProgress_;
+  ops::LinearScratch chainScratch_[GGUF_CHAIN_LINKS];
+  bool chained_ = false, encodedChains_ = false;
+  void encodeChainedLayers(hip::CommandGraph &graph, const ops::AttentionPlan &plan, uint32_t rows);
+  [[nodiscard]] bool chains(uint32_t rows) const noexcept;
   ops::AttentionWorkspace attentionWorkspace_;
   ops::SamplingBuffers sampling_;
   uint32_t maxSplits_ = 0;

@@ -162,8 +162,28 @@ void Linear::addPrepare(hip::CommandGraph &graph, const hip::Buffer &input, cons
             {width / 32, tiles, 1}, {64, 1, 1});
 }
 
+// One validated projection dispatch: what Linear::add hands the graph, and what a chain holds of each link.
+struct Linear::Resolved {
+  std::string kernel;
+  std::array<hip::Buffer, 8> buffers;
+  GgufDecodeParams params{};
+  uint32_t items = 0, pieces = 1, groups = 0;
+  uint32_t format = 0, epilogue = 0;
+  bool mixed = false, prepared = false;
+  PreparedInput after;
+};
+
 PreparedInput Linear::add(hip::CommandGraph &graph, LinearBuffers b, const Projection &p, const LinearPlan &plan,
                           const Projection *gate) const {
+  const LinearWorkload w = plan.workload();
+  const hip::Buffer input = b.input, table = b.scratch.input;
+  const Resolved r = resolve(std::move(b), p, plan, gate);
+  if (!r.prepared) addPrepare(graph, input, LinearScratch{table, {}, {}}, w.matrix.inputSize, w.rows);
+  graph.add(r.kernel, {r.buffers.begin(), r.buffers.end()}, r.params, {r.items, r.pieces, 1}, {256, 1, 1});
+  return r.after;
+}
+
+Linear::Resolved Linear::resolve(LinearBuffers b, const Projection &p, const LinearPlan &plan, const Projection *gate) const {
   const LinearWorkload w = plan.workload();
   const LinearConfig c = plan.configuration();
   const auto [n, k] = w.matrix;
@@ -211,8 +231,6 @@ PreparedInput Linear::add(hip::CommandGraph &graph, LinearBuffers b, const Proje
                         b.prepared.source.sameView(b.input);
   if (!prepared) requireBytes(b.input, uint64_t{w.rows} * k * 2, "projection input");
 
-  if (!prepared) addPrepare(graph, b.input, b.scratch, k, w.rows);
-
   GgufDecodeParams params{};
   params.input_size = k;
   params.rows = w.rows;
@@ -246,13 +264,74 @@ PreparedInput Linear::add(hip::CommandGraph &graph, LinearBuffers b, const Proje
     images[1] = b.normWeight;
     images[2] = b.nextTable;
   }
-  graph.add(name,
-            {images[0], images[1], images[2], b.scratch.input, b.output,
-             w.epilogue == LinearEpilogue::Residual || norms ? b.residual : writesTable ? b.nextTable : spare,
-             c.splits > 1 ? b.scratch.partials : spare, c.splits > 1 ? b.scratch.counters : spare},
-            params, {c.wholeGroups + (groupsOf(n, w.epilogue) - c.wholeGroups) * c.splits, rowPieces(w.rows), 1}, {256, 1, 1});
+  Resolved r;
+  r.kernel = name;
+  r.buffers = {images[0], images[1], images[2], b.scratch.input, b.output,
+               w.epilogue == LinearEpilogue::Residual || norms ? b.residual : writesTable ? b.nextTable : spare,
+               c.splits > 1 ? b.scratch.partials : spare, c.splits > 1 ? b.scratch.counters : spare};
+  r.params = params;
+  r.groups = groupsOf(n, w.epilogue);
+  r.items = c.wholeGroups + (r.groups - c.wholeGroups) * c.splits;
+  r.pieces = rowPieces(w.rows);
+  r.format = segments.front().formatId;
+  r.epilogue = norms ? GGUF_EPILOGUE_RESIDUAL_NORM
+               : gateUp ? (writesTable ? GGUF_EPILOGUE_GATE_UP_TABLE : GGUF_EPILOGUE_GATE_UP)
+               : w.epilogue == LinearEpilogue::Residual ? GGUF_EPILOGUE_RESIDUAL
+               : plan.destination() == FloatOutput::Float32 ? GGUF_EPILOGUE_PLAIN_F32 : GGUF_EPILOGUE_PLAIN;
+  r.mixed = mixed;
+  r.prepared = prepared;
+  r.after = {b.input, prepared ? b.prepared.layout : LinearInput::Table16};
   (void)tiles;
-  return {b.input, prepared ? b.prepared.layout : LinearInput::Table16};
+  return r;
+}
+
+void Linear::addChain(hip::CommandGraph &graph, std::vector<ChainedProjection> links, const hip::Buffer &progress) const {
+  if (links.empty() || links.size() > GGUF_CHAIN_LINKS) throw std::invalid_argument("a chain holds one to four projections");
+  requireBytes(progress, GGUF_CHAIN_PROGRESS_WORDS * 4, "chain progress");
+  GgufChainParams chain{};
+  chain.links = uint32_t(links.size());
+  chain.spin_limit = calibration_.chainSpinLimit;
+  std::vector<hip::Buffer> buffers;
+  std::vector<Resolved> resolved;
+  const uint32_t storage = links.front().plan.storageRows();
+  uint32_t items = 0;
+  for (size_t i = 0; i < links.size(); ++i) {
+    ChainedProjection &link = links[i];
+    if (!link.projection) throw std::invalid_argument("a chain link names its projection");
+    if (link.plan.storageRows() != storage || rowPieces(link.plan.workload().rows) != 1)
+      throw std::invalid_argument("a chain's projections share one tile height of up to 64 rows");
+    resolved.push_back(resolve(link.buffers, *link.projection, link.plan, link.gate));
+    const Resolved &r = resolved.back();
+    if (!r.prepared) throw std::invalid_argument("a chained projection reads a table that is already there or that the link before it writes");
+    if (r.epilogue == GGUF_EPILOGUE_RESIDUAL || r.epilogue == GGUF_EPILOGUE_GATE_UP)
+      throw std::invalid_argument("a chained projection is plain, a gate/up pair that writes the next table, or a residual one that norms its rows");
+    // a link's table, partials and counters are its own, and nothing the dispatch has read is written later
+    for (size_t j = 0; j < i; ++j) {
+      const LinearBuffers &other = links[j].buffers;
+      if (other.scratch.input.sameView(link.buffers.scratch.input)) throw std::invalid_argument("chained projections read tables of their own");
+      if (link.plan.configuration().splits > 1 && links[j].plan.configuration().splits > 1 &&
+          (other.scratch.partials.sameView(link.buffers.scratch.partials) || other.scratch.counters.sameView(link.buffers.scratch.counters)))
+        throw std::invalid_argument("chained projections keep partials and counters of their own");
+      if (link.buffers.nextTable && link.buffers.nextTable.sameView(other.scratch.input))
+        throw std::invalid_argument("a chained projection writes no table an earlier link read");
+    }
+    GgufChainLink &out = chain.link[i];
+    out.p = r.params;
+    out.first_item = items;
+    out.format = r.format;
+    out.epilogue = r.epilogue;
+    out.mixed = r.mixed;
+    out.groups = r.groups;
+    items += r.items;
+    buffers.insert(buffers.end(), r.buffers.begin(), r.buffers.end());
+  }
+  // links past the last bind the first one's buffers and take no workgroup
+  for (size_t i = links.size(); i < GGUF_CHAIN_LINKS; ++i) {
+    chain.link[i].first_item = items;
+    buffers.insert(buffers.end(), resolved.front().buffers.begin(), resolved.front().buffers.end());
+  }
+  buffers.push_back(progress);
+  graph.add("gguf_decode_chain_m" + std::to_string(storage), std::move(buffers), chain, {items, 1, 1}, {256, 1, 1});
 }
 
 void Linear::addProjection(hip::CommandGraph &graph, hip::Buffer input, const Projection &projection, hip::Buffer output,

@@ -13,6 +13,7 @@
 #include <compare>
 #include <cstdint>
 #include <string>
+#include <vector>
 
 namespace splash::ops {
 
@@ -158,6 +159,17 @@ struct KernelCalibration final {
   // Fewest super-blocks a workgroup's K range keeps.
   uint32_t minimumBlocksPerWave = 5;
   uint32_t groupsPerUnitQ6K = 3;
+  // Polls of a chained projection's workgroup for the link before it (about a microsecond each) before it gives up.
+  uint32_t chainSpinLimit = 1u << 16;
+};
+
+class Linear;
+// One projection of a chain (Linear::addChain): what Linear::add takes.
+struct ChainedProjection final {
+  LinearBuffers buffers;
+  const Projection *projection = nullptr;
+  LinearPlan plan;
+  const Projection *gate = nullptr;
 };
 
 class Linear final {
@@ -180,6 +192,13 @@ public:
   // Returns what the scratch table describes after the dispatch.
   PreparedInput add(hip::CommandGraph &graph, LinearBuffers buffers, const Projection &projection,
                     const LinearPlan &plan, const Projection *gate = nullptr) const;
+  // Up to four projections of up to 64 rows as one dispatch, each reading what the one before it wrote (the table its
+  // epilogue leaves, the residual rows): the next link's workgroups fetch their first weights while the link before
+  // them drains, and wait for its count of finished workgroups instead of a kernel boundary. Every link's input is
+  // prepared (a table that exists or that the link before writes), its table, partials and counters are its own, and
+  // `progress` (GGUF_CHAIN_PROGRESS_WORDS words, zero before the first dispatch) is the chain's; its last word reads
+  // nonzero after a dispatch in which a wait gave up.
+  void addChain(hip::CommandGraph &graph, std::vector<ChainedProjection> links, const hip::Buffer &progress) const;
   void addProjection(hip::CommandGraph &graph, hip::Buffer input, const Projection &projection, hip::Buffer output,
                      uint32_t rows, LinearScratch scratch) const;
   void addResidualProjection(hip::CommandGraph &graph, hip::Buffer input, const Projection &projection,
@@ -191,6 +210,9 @@ public:
                  hip::Buffer output, uint32_t rows, PreparedInput normalized = {}) const;
 
 private:
+  struct Resolved;
+  [[nodiscard]] Resolved resolve(LinearBuffers buffers, const Projection &projection, const LinearPlan &plan,
+                                 const Projection *gate) const;
   KernelCalibration calibration_;
 };
 

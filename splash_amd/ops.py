@@ -142,6 +142,41 @@ class Linear:
                                  scratch.counters.handle, int(prepared)))
         graph._keep.extend([projection, gate, input, output, residual, scratch])
 
+    CHAIN_PROGRESS_BYTES = 65792
+
+    def set_chain_spin_limit(self, polls):
+        check(lib.spo_linear_set_chain_spin_limit(self.handle, polls))
+    CHAIN_STATUS_OFFSET = 16
+
+    @staticmethod
+    def _fill_link(slot, link):
+        handle = lambda b: b.handle if b is not None else None
+        scratch = link["scratch"]
+        slot.projection, slot.gate = link["projection"].handle, handle(link.get("gate"))
+        slot.plan = link["plan"]
+        slot.input, slot.output, slot.residual = handle(link.get("input")), handle(link.get("output")), handle(link.get("residual"))
+        slot.norm_weight, slot.next_table = handle(link.get("norm_weight")), handle(link.get("next_table"))
+        slot.table, slot.partials, slot.counters = scratch.table.handle, scratch.partials.handle, scratch.counters.handle
+        slot.prepared = int(link.get("prepared", 0))
+
+    def add_chain(self, graph, links, progress):
+        """Up to four projections as one dispatch, each reading what the one before it wrote. links: dicts of add()'s
+        arguments (projection, plan, input, output, scratch, and residual, gate, prepared, norm_weight, next_table as
+        that link takes them); progress: CHAIN_PROGRESS_BYTES bytes the chain owns, zero before its first dispatch."""
+        array = (nat.ChainLink * len(links))()
+        for slot, link in zip(array, links):
+            self._fill_link(slot, link)
+            graph._keep.extend(link.values())
+        check(lib.spo_linear_add_chain(self.handle, graph.handle, array, len(links), progress.handle))
+        graph._keep.append(progress)
+
+    def add_link(self, graph, **link):
+        """One link as a dispatch of its own (Linear::add of all its buffers)."""
+        slot = nat.ChainLink()
+        self._fill_link(slot, link)
+        check(lib.spo_linear_add_link(self.handle, graph.handle, ctypes.byref(slot)))
+        graph._keep.extend(link.values())
+
     def add_swiglu(self, graph, gate, up, down, normalized, intermediate, residual, output, rows, scratch, next_table=None):
         """next_table: a second activation table (gguf_table_bytes(ffn, rows)); the gate/up pass then writes
         the down projection's table itself."""

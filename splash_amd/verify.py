@@ -106,6 +106,11 @@ class DenseVerify:
 
     _results_call = "spo_dense_verify_results"
 
+    def set_chained(self, chained):
+        """Whether steps encoded from now on chain a layer's projections after its attention into one dispatch (off by
+        default): the results are the same bit for bit."""
+        check(lib.spo_dense_verify_set_chained(self.handle, int(bool(chained))))
+
     def set_candidate_children(self, ids, probabilities, draws, child_uniforms):
         """The sampled rows' candidate children, by packed row: ids uint32 [rows][16], probabilities fp32 [rows][16], draws
         bytes [rows][4] (0xFF past a row's drawn children), child_uniforms fp32 [rows][4]."""

@@ -333,7 +333,8 @@ def test_residual_norm_epilogue(backend, fmt, N, K, M, config):
         wv, w32, w16 = orc.activation_table(scaled[first:first + rows])
         assert np.array_equal(values, wv)
         assert s32.tobytes() == w32.tobytes() and s16.tobytes() == w16.tobytes()
-        squares = piece[size - (N // 64) * 16 * tiles * 4:].view(np.float32).reshape(N // 64, 16 * tiles)
+        stride = max(16 * tiles, 32)     # floats an entry: whole 128-byte lines
+        squares = piece[size - (N // 64) * stride * 4:].view(np.float32).reshape(N // 64, stride)[:, :16 * tiles]
         h = orc.bf16_to_f32(hidden[first:first + rows]).astype(np.float64)
         want = (h.reshape(rows, N // 64, 64) ** 2).sum(axis=2).T
         assert np.allclose(squares[:, :rows], want, rtol=1e-5, atol=0)

@@ -159,7 +159,8 @@ def test_combine_writes_the_next_norms_table(backend, rows):
         assert np.array_equal(live, orc.table_rows(wv, hidden, tiles)[:count])
         rows_of = lambda sums: sums.transpose(0, 2, 1).reshape(tiles * 16, -1)[:count]     # [tile][entry][16 rows] -> [row][entry]
         assert np.array_equal(rows_of(s32), rows_of(w32)) and np.array_equal(rows_of(s16), rows_of(w16))
-        squares = piece[size - (hidden // 64) * 16 * tiles * 4:].view(np.float32).reshape(hidden // 64, 16 * tiles)
+        stride = max(16 * tiles, 32)     # floats an entry: whole 128-byte lines
+        squares = piece[size - (hidden // 64) * stride * 4:].view(np.float32).reshape(hidden // 64, stride)[:, :16 * tiles]
         h = orc.bf16_to_f32(got[first:first + count]).astype(np.float64)
         assert np.allclose(squares[:, :count], (h.reshape(count, hidden // 64, 64) ** 2).sum(axis=2).T, rtol=1e-5, atol=0)
     assert at == table_bytes

@@ -214,3 +214,36 @@ def test_a_sampled_tree_block_tests_its_drawn_children(backend):
     if sure:
         assert retained[0] == len(kept) and accepted[0] == acc and mask[0] == m and np.array_equal(selected[:len(kept)], kept)
     assert 1 <= retained[0] <= rows and (not sure or accepted[0] >= 1)
+
+
+@pytest.mark.parametrize("lanes_rows", [[16], [7, 16, 3]])
+def test_chained_projections_change_nothing(backend, lanes_rows):
+    """A step whose layers dispatch their four projections after the attention as one chain (a layer's output, gate/up
+    and down projections and the next layer's q|k|v, the LM head after the last) gives the logits, the hidden rows and
+    the results of the step that dispatches them one by one, bit for bit, on repeated runs, in far fewer dispatches."""
+    print(f"case chained step lanes={lanes_rows}", flush=True)
+    model = DenseModel(seed=15, hidden=1024, q_heads=16, kv_heads=8, head_dim=64, ffn=3072, vocabulary=32000, layers=4)
+    rng = np.random.default_rng(8)
+    contexts = [300 + 111 * i for i in range(len(lanes_rows))]
+    gpu = model.build_gpu(backend, max_lanes=len(lanes_rows), context_tokens=[c + 16 for c in contexts])
+    model.seed_context(gpu, None, rng)
+    lanes = [verify.Lane(rows, committed, table_first=first) for rows, committed, first in zip(lanes_rows, contexts, model.table_first)]
+    total = sum(lanes_rows)
+    gpu.set_block(lanes, rng.integers(0, 32000, total).astype(np.uint32))
+
+    def run(chained):
+        gpu.set_chained(chained)
+        graph = gpu.encode(lanes, commit=False)
+        outcomes = []
+        for _ in range(3):
+            backend.run(graph)
+            outcomes.append((gpu.buffer(verify.LOGITS).download(np.float32, total * 32000).copy(),
+                             gpu.buffer(verify.HIDDEN, 0).download(np.uint16, total * 1024).copy(), gpu.results(lanes)))
+        return len(graph), outcomes
+    plain_dispatches, plain = run(False)
+    chained_dispatches, chained = run(True)
+    assert chained_dispatches == plain_dispatches - 3 * 4   # four projections become one in each of the four layers
+    for logits, hidden, results in plain[1:] + chained:
+        assert np.array_equal(logits, plain[0][0]) and np.array_equal(hidden, plain[0][1])
+        for got, want in zip(results, plain[0][2]):
+            assert np.array_equal(got, want)
