@@ -787,24 +787,32 @@ __device__ __forceinline__ void decode_workgroup(DecodeShared<RT> &shared, const
     if (threadIdx.x == 0) arrived = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
     if (arrived != splits - 1) return;
-    // The last arriver sums the splits in split order; the loads of a round of eight are in flight together.
+    // The last arriver sums the splits in split order; the loads of a round are in flight together (the loop's staging
+    // registers are free by now), so the sum costs one or two round trips to the coherence point whatever the splits.
+    constexpr uint32_t kRound = RT == 1 ? 16u : RT == 2 ? 8u : 4u;
 #pragma unroll
     for (int t = 0; t < RT; ++t)
 #pragma unroll
       for (int v = 0; v < 4; ++v) acc[t][v] = 0.f;
-    for (uint32_t s0 = 0; s0 < splits; s0 += 4u) {
-      float part[4][RT][4];
+    for (uint32_t s0 = 0; s0 < splits; s0 += kRound) {
+      float part[kRound][RT][4];
 #pragma unroll
-      for (uint32_t s = 0; s < 4u; ++s)
+      for (uint32_t s = 0; s < kRound; ++s) {
+        if (s0 + s < splits) {
 #pragma unroll
-        for (int t = 0; t < RT; ++t)
+          for (int t = 0; t < RT; ++t)
 #pragma unroll
-          for (int v = 0; v < 4; ++v) {
-            const uint32_t from = s0 + s < splits ? s0 + s : s0;
-            part[s][t][v] = __hip_atomic_load(mineAt + size_t(from) * stride + (t * 4 + v) * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          }
+            for (int v = 0; v < 4; ++v)
+              part[s][t][v] = __hip_atomic_load(mineAt + size_t(s0 + s) * stride + (t * 4 + v) * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        } else {
 #pragma unroll
-      for (uint32_t s = 0; s < 4u; ++s)
+          for (int t = 0; t < RT; ++t)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) part[s][t][v] = 0.f;
+        }
+      }
+#pragma unroll
+      for (uint32_t s = 0; s < kRound; ++s)
 #pragma unroll
         for (int t = 0; t < RT; ++t)
 #pragma unroll
