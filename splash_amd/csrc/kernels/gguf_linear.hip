@@ -534,9 +534,6 @@ __device__ __forceinline__ void chain_wait(const ChainPosition &chain) {
     }
     __syncthreads();
   }
-#ifdef SP_CHAIN_TRACE
-  if (threadIdx.x == 0) reinterpret_cast<uint64_t *>(chain.status - GGUF_CHAIN_LINKS + GGUF_CHAIN_PROGRESS_WORDS)[blockIdx.x * 4u + 1u] = wall_clock64();
-#endif
   // nothing that reads the link before's results moves above the wait
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
   __builtin_amdgcn_sched_barrier(0);
@@ -761,9 +758,6 @@ __device__ __forceinline__ void decode_workgroup(DecodeShared<RT> &shared, const
     }
   }
 
-#ifdef SP_CHAIN_TRACE
-  if constexpr (Chain) if (threadIdx.x == 0) reinterpret_cast<uint64_t *>(chain.status - GGUF_CHAIN_LINKS + GGUF_CHAIN_PROGRESS_WORDS)[blockIdx.x * 4u + 2u] = wall_clock64();
-#endif
   // Element (t, v) of this lane is row 16 t + 4 kq + v, column tile.column + c.
   if (splits > 1) {
     // Partials [split][partitioned unit][t][v][lane]: whole-wave contiguous stores and loads.
@@ -982,9 +976,6 @@ __device__ __forceinline__ void decode_workgroup(DecodeShared<RT> &shared, const
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
-#ifdef SP_CHAIN_TRACE
-    if (threadIdx.x == 0) reinterpret_cast<uint64_t *>(chain.status - GGUF_CHAIN_LINKS + GGUF_CHAIN_PROGRESS_WORDS)[blockIdx.x * 4u + 3u] = wall_clock64();
-#endif
     if (threadIdx.x < 64u) {
       uint32_t before = 0;
       if (threadIdx.x == 0) before = __hip_atomic_fetch_add(chain.done, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -1152,9 +1143,6 @@ __global__ __launch_bounds__(256) void gguf_decode_chain(SP_CHAIN_LINK_PARAMETER
   chain.flags = link + 1u == cp.links ? nullptr : flagsOf(link);
   chain.spinLimit = cp.spin_limit;
   chain.status = progress + GGUF_CHAIN_LINKS;
-#ifdef SP_CHAIN_TRACE
-  if (threadIdx.x == 0) reinterpret_cast<uint64_t *>(chain.status - GGUF_CHAIN_LINKS + GGUF_CHAIN_PROGRESS_WORDS)[blockIdx.x * 4u] = wall_clock64();
-#endif
   GgufDecodeParams p = mine.p;
   p.rows = min(p.rows, uint32_t(GGUF_MAXIMUM_ROWS));
   uint32_t item = blockIdx.x - mine.first_item;
