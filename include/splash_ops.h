@@ -347,12 +347,28 @@ sp_status spo_sampling_greedy_rows_static(const float *logits, uint32_t rows, ui
  * [lanes * 7][16][16]: [predecessor][candidate] the sum over the selector's rank of 256 of predecessor_codebook[token
  * of the position before, anchors[lane] at position 0 (row 0 alone)] x selector_hidden[row] x successor_codebook[token],
  * bf16 factors, fp32 sums. Codebooks bf16 [vocabulary][256]; selector_hidden bf16 [lanes * 8][256]; `scratch` of
- * spo_draft_candidate_scratch_bytes. Up to 524288 columns. Growing the tree over them is not part of this library. */
+ * spo_draft_candidate_scratch_bytes. Up to 524288 columns. */
 sp_status spo_draft_candidate_scratch_bytes(uint32_t lanes, uint32_t columns, uint64_t *bytes);
 sp_status spo_draft_add_candidates(spo_graph *graph, sp_buffer *logits, sp_buffer *selector_hidden, sp_buffer *scratch,
                                    sp_buffer *candidates, sp_buffer *unary, sp_buffer *edges, sp_buffer *predecessor_codebook,
                                    sp_buffer *successor_codebook, uint32_t leading, uint32_t trailing, uint32_t vocabulary,
                                    const uint32_t *anchors, uint32_t lanes);
+/* The third kernel of DraftSelector::add (DraftSelector.cpp:96-118; draft_select_tree, sampling.metal:1357-1766, its
+ * rule in abi/Sampling.h:209-255): each lane's tree over those candidates and edges, best first by the estimate that the
+ * target accepts the path to a row, up to 16 rows a lane, as spo_draft_add_verify_rows and the sampled rows of a verify
+ * step (spo_sampling_buffers' candidate fields: a row's next-position probabilities and drawn children) read them.
+ * chain_tokens uint32 [lanes][15] and chain_rates fp32 [lanes][15][4] hold each lane's host chain (its rate by its
+ * agreement with the draft at its depth: the draft's likeliest, another candidate, none, past the draft's positions);
+ * tree_draws bytes [lanes][16][4], tree_next fp32 [lanes][16][16], tree_caps fp32 [lanes][16]. */
+typedef struct spo_draft_tree_lane {
+  uint32_t anchor, depth, children, chain; /* depth < 16, children 1..4, chain <= 15 */
+  float slope, intercept[7], temperature;  /* estimate = sigmoid(slope * logit(q) + intercept[position]); temperature 0: greedy */
+  uint32_t noise[2];                        /* the 64-bit seed of a sampled lane's draws, low word first */
+} spo_draft_tree_lane;
+sp_status spo_draft_add_tree(spo_graph *graph, sp_buffer *candidates, sp_buffer *unary, sp_buffer *edges, sp_buffer *chain_tokens,
+                             sp_buffer *chain_rates, sp_buffer *tree_tokens, sp_buffer *trees, sp_buffer *tree_scores,
+                             sp_buffer *tree_sizes, sp_buffer *tree_draws, sp_buffer *tree_next, sp_buffer *tree_caps,
+                             const spo_draft_tree_lane *lanes, uint32_t count);
 sp_status spo_draft_add_verify_rows(spo_graph *graph, sp_buffer *tree_tokens, sp_buffer *trees, sp_buffer *tree_scores,
                                     sp_buffer *tree_sizes, sp_buffer *input_tokens, sp_buffer *tree_rows, sp_buffer *lane_rows,
                                     sp_buffer *verify_sources, uint32_t lanes, uint32_t rows, uint32_t lane_cap, float floor);

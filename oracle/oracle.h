@@ -24,6 +24,9 @@
 //   orc_argmax / orc_accept_tree    pinned by brute force on tiny vocabularies.
 //   orc_draft_verify_rows           pinned by an independent statement (a stable sort of the estimates, a recursive
 //                                   preorder) in the tests.
+//   orc_draft_tree                  pinned by an independent statement in the tests (every path's entry enumerated in fp64,
+//                                   a stable sort by estimate, cases whose order hangs on less than 1e-4 set aside), by the
+//                                   caps' and estimates' invariants, and by the frequencies of a sampled row's draws.
 //   orc_draft_candidates            pinned by a lexicographic sort of (logit descending, column ascending) in the tests,
 //                                   ties, signed zeros and short rows among the cases.
 //   orc_draft_edges                 pinned by the fp64 trilinear sum over the decoded bf16 factors (numpy einsum), to the
@@ -141,6 +144,19 @@ uint32_t orc_accept_tree(const struct OrcTreeRow *tree, const uint32_t *tokens, 
 void orc_draft_verify_rows(const uint32_t *tree_tokens, const struct OrcTreeRow *trees, const float *scores, const uint32_t *sizes,
                            uint32_t lanes, uint32_t rows, uint32_t lane_cap, float floor, uint32_t *tokens, struct OrcTreeRow *tree,
                            uint32_t *lane_rows, uint32_t *sources);
+// sampling.metal:1357-1766 draft_select_tree for one lane: candidates uint32 [7][16], unary fp32 [7][16], edges fp32
+// [7][16][16] ([position][predecessor][candidate]; position 0 reads predecessor 0 alone), the lane's host chain (15 tokens, a
+// rate for each of 4 agreements a token) and parameters (Sampling.h:242-252, one lane's). Outputs, 16 rows: tokens, tree
+// rows, {draft probability, estimate} pairs, the rows held, each row's drawn children (candidate indices, 0xFF past them),
+// its next position's probabilities, and its cap.
+struct OrcDraftTreeLane {
+  uint32_t anchor, depth, chain, children;
+  float slope, intercept[7], temperature;
+  uint32_t noise[2];
+};
+void orc_draft_tree(const uint32_t *candidates, const float *unary, const float *edges, const uint32_t *chain_tokens,
+                    const float *chain_rates, const struct OrcDraftTreeLane *lane, uint32_t *tokens, struct OrcTreeRow *tree,
+                    float *scores, uint32_t *size, uint8_t *draws, float *next, float *caps);
 // sampling.metal:1099-1264: of each proposal position's logits row (rows 1-7 of a lane's eight, fp32 [lanes * 8][columns])
 // the sixteen columns of the largest logits, the larger first, the smaller column first among equal ones; candidates their
 // tokens (a column at or past `leading` is token column - leading + trailing), unary their logits, [lanes * 7][16];

@@ -273,6 +273,12 @@ _sig("spo_moe_add_routed_norm", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_u32,
 _sig("spo_row_copy_add", c_int, c_p, c_p, c_u32, c_u32, c_u32, c_p, c_u32, c_u32, c_u32, c_u32, c_u32)
 _sig("spo_sampling_workspace", c_int, c_u32, P(c_u64))
 _sig("spo_sampling_add_verify", c_int, c_p, P(SamplingBuffers), c_u32, c_u32, P(LaneRows), P(SamplingPolicy), c_u32, P(c_u32))
+class DraftTreeLane(ctypes.Structure):
+    _fields_ = [("anchor", c_u32), ("depth", c_u32), ("children", c_u32), ("chain", c_u32), ("slope", ctypes.c_float),
+                ("intercept", ctypes.c_float * 7), ("temperature", ctypes.c_float), ("noise", c_u32 * 2)]
+
+
+_sig("spo_draft_add_tree", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, P(DraftTreeLane), c_u32)
 _sig("spo_draft_add_verify_rows", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_u32, c_u32, c_u32, ctypes.c_float)
 _sig("spo_sampling_add_acceptance", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, P(LaneRows), P(c_u32), c_u32, P(c_u32))
 _sig("spo_sampling_greedy_rows_static", c_int, ctypes.c_void_p, c_u32, c_u32, c_u32, ctypes.c_void_p, ctypes.c_void_p)

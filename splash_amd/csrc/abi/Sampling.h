@@ -88,6 +88,32 @@ struct DraftSelectParams {
   uint32_t reserved[2];
 };
 
+// draft_select_tree: one wavefront a lane grows the lane's tree over the candidates and edges of draft_select_edges (the
+// reference's DraftTreeParams, abi/Sampling.h:209-255). A row's estimate is the probability that the target accepts the
+// path to it, the product of its steps' estimates: a step to a draft candidate at proposal position p, of probability q
+// among the position's candidates after its parent's, sigmoid(slope * logit(q) + intercept[p]), at most its cap (what the
+// parent's host-chain child and the steps the parent drew before it left of 1); a step to host chain token d, its rate
+// for its agreement with the draft at depth d (DRAFT_CHAIN_AGREEMENTS: the draft's likeliest there, another of its
+// candidates, none, past its positions). The tree grows best first by estimate, a draft row taking children[l]
+// candidates (a greedy lane's likeliest; a sampled lane's Gumbel-top-k draws from the probabilities at its temperature,
+// with noise[l] as the anchor's key) and a chain row the chain's next token, one row a token path, until it holds
+// DRAFT_TREE_ROWS rows, depth[l] + 1 rows, or nothing no deeper than depth[l] is left. Grid (lanes), 64 threads.
+#define DRAFT_TREE_ROWS 16u
+#define DRAFT_CHAIN_TOKENS (DRAFT_TREE_ROWS - 1u)
+#define DRAFT_CHAIN_AGREEMENTS 4u
+struct DraftTreeParams {
+  uint32_t anchor[SAMPLING_MAXIMUM_LANES];
+  uint32_t depth[SAMPLING_MAXIMUM_LANES];     // the deepest row a walk of the tree may retain
+  uint32_t chain[SAMPLING_MAXIMUM_LANES];     // tokens of the lane's host chain (0: none)
+  uint32_t children[SAMPLING_MAXIMUM_LANES];  // 1..SAMPLING_TREE_CHILDREN
+  uint32_t lanes;
+  uint32_t reserved[3];
+  float slope[SAMPLING_MAXIMUM_LANES];
+  float intercept[SAMPLING_MAXIMUM_LANES][DRAFT_PROPOSAL_TOKENS];
+  float temperature[SAMPLING_MAXIMUM_LANES];
+  uint32_t noise[SAMPLING_MAXIMUM_LANES][2];  // a 64-bit seed, low word first
+};
+
 // decode_accept_tree: one wavefront per lane, a thread a row (the reference's AcceptBatchParams, abi/Sampling.h:314-317).
 struct AcceptBatchParams {
   uint32_t lanes;
@@ -100,6 +126,7 @@ struct AcceptBatchParams {
 #ifdef __cplusplus
 static_assert(sizeof(TargetSamplingParams) == 16 + 32 + 16 + 64 + 96 + 32, "target sampling parameters are 256 bytes on both sides");
 static_assert(sizeof(DraftSelectParams) == 32 + 32, "draft selector parameters are 64 bytes on both sides");
+static_assert(sizeof(DraftTreeParams) == 4 * 32 + 16 + 32 + 224 + 32 + 64, "draft tree parameters are 496 bytes on both sides");
 static_assert(sizeof(VerifyRowsParams) == 16, "verify rows parameters are 16 bytes on both sides");
 static_assert(sizeof(AcceptBatchParams) == 16 + 32 + 16 + 64, "acceptance parameters are 128 bytes on both sides");
 #endif

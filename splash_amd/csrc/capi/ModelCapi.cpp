@@ -134,6 +134,32 @@ sp_status spo_draft_add_candidates(spo_graph *graph, sp_buffer *logits, sp_buffe
   });
 }
 
+sp_status spo_draft_add_tree(spo_graph *graph, sp_buffer *candidates, sp_buffer *unary, sp_buffer *edges, sp_buffer *chain_tokens,
+                             sp_buffer *chain_rates, sp_buffer *tree_tokens, sp_buffer *trees, sp_buffer *tree_scores,
+                             sp_buffer *tree_sizes, sp_buffer *tree_draws, sp_buffer *tree_next, sp_buffer *tree_caps,
+                             const spo_draft_tree_lane *lanes, uint32_t count) {
+  return capi::guard([&] {
+    capi::require(graph && lanes, "graph or lanes");
+    std::vector<ops::DraftTreeLane> list;
+    for (uint32_t l = 0; l < count; ++l) {
+      ops::DraftTreeLane lane;
+      lane.anchor = lanes[l].anchor;
+      lane.depth = lanes[l].depth;
+      lane.children = lanes[l].children;
+      lane.chain = lanes[l].chain;
+      lane.slope = lanes[l].slope;
+      for (size_t p = 0; p < lane.intercept.size(); ++p) lane.intercept[p] = lanes[l].intercept[p];
+      lane.temperature = lanes[l].temperature;
+      lane.noise = uint64_t{lanes[l].noise[1]} << 32 | lanes[l].noise[0];
+      list.push_back(lane);
+    }
+    ops::DraftSelector::addTree(capi::graphOf(graph),
+                                {B(candidates), B(unary), B(edges), B(chain_tokens), B(chain_rates), B(tree_tokens), B(trees), B(tree_scores),
+                                 B(tree_sizes), B(tree_draws), B(tree_next), B(tree_caps)},
+                                list);
+  });
+}
+
 sp_status spo_draft_add_verify_rows(spo_graph *graph, sp_buffer *tree_tokens, sp_buffer *trees, sp_buffer *tree_scores,
                                     sp_buffer *tree_sizes, sp_buffer *input_tokens, sp_buffer *tree_rows, sp_buffer *lane_rows,
                                     sp_buffer *verify_sources, uint32_t lanes, uint32_t rows, uint32_t lane_cap, float floor) {

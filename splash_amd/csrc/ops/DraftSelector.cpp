@@ -40,6 +40,47 @@ void DraftSelector::addCandidates(hip::CommandGraph &graph, const DraftCandidate
             {static_cast<uint32_t>(rows), 1, 1}, {256, 1, 1});
 }
 
+void DraftSelector::addTree(hip::CommandGraph &graph, const DraftTreeBuffers &b, std::span<const DraftTreeLane> lanes) {
+  if (lanes.empty() || lanes.size() > SAMPLING_MAXIMUM_LANES) throw std::invalid_argument("invalid draft selector batch");
+  DraftTreeParams params{};
+  params.lanes = static_cast<uint32_t>(lanes.size());
+  for (uint32_t l = 0; l < params.lanes; ++l) {
+    const DraftTreeLane &lane = lanes[l];
+    if (!lane.children || lane.children > SAMPLING_TREE_CHILDREN) throw std::invalid_argument("a draft row takes one to four children");
+    if (lane.depth >= DRAFT_TREE_ROWS || lane.chain > DRAFT_CHAIN_TOKENS) throw std::invalid_argument("a tree is no deeper than a verify block's rows after its anchor");
+    if (!(lane.temperature >= 0.0f) || !std::isfinite(lane.temperature) || !std::isfinite(lane.slope))
+      throw std::invalid_argument("invalid draft tree lane");
+    for (float value : lane.intercept)
+      if (!std::isfinite(value)) throw std::invalid_argument("invalid draft tree lane");
+    params.anchor[l] = lane.anchor;
+    params.depth[l] = lane.depth;
+    params.chain[l] = lane.chain;
+    params.children[l] = lane.children;
+    params.slope[l] = lane.slope;
+    for (uint32_t p = 0; p < DRAFT_PROPOSAL_TOKENS; ++p) params.intercept[l][p] = lane.intercept[p];
+    params.temperature[l] = lane.temperature;
+    params.noise[l][0] = static_cast<uint32_t>(lane.noise);
+    params.noise[l][1] = static_cast<uint32_t>(lane.noise >> 32);
+  }
+  const uint64_t positions = uint64_t{params.lanes} * DRAFT_PROPOSAL_TOKENS, rows = uint64_t{params.lanes} * DRAFT_TREE_ROWS;
+  requireBytes(b.candidates, positions * DRAFT_CANDIDATES * 4, "draft candidate");
+  requireBytes(b.unary, positions * DRAFT_CANDIDATES * 4, "draft candidate score");
+  requireBytes(b.edges, positions * DRAFT_CANDIDATES * DRAFT_CANDIDATES * 4, "draft edge score");
+  requireBytes(b.chainTokens, uint64_t{params.lanes} * DRAFT_CHAIN_TOKENS * 4, "draft chain token");
+  requireBytes(b.chainRates, uint64_t{params.lanes} * DRAFT_CHAIN_TOKENS * DRAFT_CHAIN_AGREEMENTS * 4, "draft chain rate");
+  requireBytes(b.treeTokens, rows * 4, "draft tree token");
+  requireBytes(b.trees, rows * sizeof(AttentionTreeRow), "draft tree row");
+  requireBytes(b.treeScores, rows * 8, "draft tree score");
+  requireBytes(b.treeSizes, uint64_t{params.lanes} * 4, "draft tree size");
+  requireBytes(b.treeDraws, rows * SAMPLING_TREE_CHILDREN, "draft tree draws");
+  requireBytes(b.treeNext, rows * DRAFT_CANDIDATES * 4, "draft tree next probabilities");
+  requireBytes(b.treeCaps, rows * 4, "draft tree cap");
+  graph.add("draft_select_tree",
+            {b.candidates, b.unary, b.edges, b.chainTokens, b.chainRates, b.treeTokens, b.trees, b.treeScores, b.treeSizes, b.treeDraws,
+             b.treeNext, b.treeCaps},
+            params, {params.lanes, 1, 1}, {64, 1, 1});
+}
+
 void DraftSelector::addVerifyRows(hip::CommandGraph &graph, const DraftVerifyRowsBuffers &b, const StepRows &step, float floor) {
   if (!step.lanes || step.lanes > SAMPLING_MAXIMUM_LANES || !step.laneCap || step.laneCap > SAMPLING_MAXIMUM_ROWS ||
       step.rows < step.lanes || step.rows > uint64_t{step.lanes} * step.laneCap)

@@ -1,12 +1,13 @@
 // The draft side's steps either side of its tree: every proposal position's candidates and their edge scores (the first
 // two kernels of the reference's ops::DraftSelector::add, runtime/ops/DraftSelector.cpp:37-140), and laying a decode
 // step's rows out from the trees a draft selector grew (ops::DraftSelector::addVerifyRows, runtime/ops/
-// DraftSelector.hpp:139-147; StepRows, runtime/ops/LaneRows.hpp:49-67). Growing the tree over the candidates
-// (draft_select_tree) is not part of this library.
+// DraftSelector.hpp:139-147; StepRows, runtime/ops/LaneRows.hpp:49-67), and between them the tree each lane grows over
+// its candidates (draft_select_tree, DraftSelector.cpp:96-118).
 #pragma once
 #include "abi/Sampling.h"
 #include "hip/Backend.hpp"
 
+#include <array>
 #include <cstdint>
 #include <span>
 
@@ -56,8 +57,33 @@ struct DraftCandidateBuffers final {
   hip::Buffer edges;           // fp32 [lanes * 7][16][16]: [predecessor][candidate]; position 0 writes row 0 alone
 };
 
+// A lane of DraftSelector::addTree (the reference's DraftTreeLane, runtime/ops/DraftSelector.hpp:59-92).
+struct DraftTreeLane final {
+  uint32_t anchor = 0;       // the token the lane's tree grows from
+  uint32_t depth = 0;        // the deepest row a walk of the tree may retain
+  uint32_t children = 1;     // candidates a draft row takes: 1..SAMPLING_TREE_CHILDREN
+  uint32_t chain = 0;        // tokens of the lane's host chain (chainTokens), 0 for none
+  float slope = 1.0f;        // the lane's acceptance model: sigmoid(slope * logit(q) + intercept[position])
+  std::array<float, DRAFT_PROPOSAL_TOKENS> intercept{};
+  float temperature = 0.0f;  // 0: the likeliest candidates; above: draws from the probabilities at that temperature
+  uint64_t noise = 0;        // the seed of a sampled lane's draws
+};
+
+struct DraftTreeBuffers final {
+  hip::Buffer candidates, unary, edges;  // as addCandidates left them
+  hip::Buffer chainTokens;   // uint32 [lanes][15]: each lane's host chain
+  hip::Buffer chainRates;    // fp32 [lanes][15][4]: a chain token's rate by its agreement with the draft at its depth
+  hip::Buffer treeTokens, trees, treeScores, treeSizes;  // as addVerifyRows reads them
+  hip::Buffer treeDraws;     // bytes [lanes][16][4]: a row's drawn children (candidate indices), SAMPLING_NO_DRAW past them
+  hip::Buffer treeNext;      // fp32 [lanes][16][16]: a row's next position's probabilities (at the lane's temperature)
+  hip::Buffer treeCaps;      // fp32 [lanes][16]: the cap of the draft step that made or joined a row
+};
+
 class DraftSelector final {
 public:
+  // Each lane's tree over the candidates and edges addCandidates left, best first by estimate (abi/Sampling.h,
+  // DraftTreeParams): rows 16 l .. of the tree buffers, lane l's sizes[l] of them.
+  static void addTree(hip::CommandGraph &graph, const DraftTreeBuffers &buffers, std::span<const DraftTreeLane> lanes);
   [[nodiscard]] static uint32_t candidateShards(uint32_t columns) noexcept { return (columns + DRAFT_SHARD_COLUMNS - 1) / DRAFT_SHARD_COLUMNS; }
   [[nodiscard]] static uint64_t candidateScratchBytes(uint32_t lanes, uint32_t columns) noexcept {
     return uint64_t{lanes} * DRAFT_PROPOSAL_TOKENS * candidateShards(columns) * DRAFT_CANDIDATES * 8;

@@ -361,6 +361,22 @@ class DraftSelector:
         graph._keep.extend(buffers)
 
     @staticmethod
+    def add_tree(graph, candidates, unary, edges, chain_tokens, chain_rates, tree_tokens, trees, tree_scores, tree_sizes, tree_draws,
+                 tree_next, tree_caps, lanes):
+        """lanes: dicts of anchor, depth, children and, as the lane has them, chain, slope, intercept (7), temperature, noise."""
+        array = (nat.DraftTreeLane * len(lanes))()
+        for slot, lane in zip(array, lanes):
+            slot.anchor, slot.depth, slot.children, slot.chain = lane["anchor"], lane["depth"], lane["children"], lane.get("chain", 0)
+            slot.slope, slot.temperature = lane.get("slope", 1.0), lane.get("temperature", 0.0)
+            slot.intercept = (ctypes.c_float * 7)(*lane.get("intercept", [0.0] * 7))
+            noise = lane.get("noise", 0)
+            slot.noise = (ctypes.c_uint32 * 2)(noise & 0xFFFFFFFF, noise >> 32)
+        buffers = [candidates, unary, edges, chain_tokens, chain_rates, tree_tokens, trees, tree_scores, tree_sizes, tree_draws, tree_next,
+                   tree_caps]
+        check(lib.spo_draft_add_tree(graph.handle, *[b.handle for b in buffers], array, len(lanes)))
+        graph._keep.extend(buffers)
+
+    @staticmethod
     def add_verify_rows(graph, tree_tokens, trees, tree_scores, tree_sizes, input_tokens, tree_rows, lane_rows, verify_sources, lanes,
                         rows, lane_cap, floor=0.0):
         buffers = [tree_tokens, trees, tree_scores, tree_sizes, input_tokens, tree_rows, lane_rows, verify_sources]

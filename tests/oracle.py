@@ -569,6 +569,36 @@ def draft_verify_rows(tree_tokens, trees, scores, sizes, rows, lane_cap, floor=0
     return tokens, tree, lane_rows, sources
 
 
+class DraftTreeLane(ctypes.Structure):
+    """One lane's DraftTreeParams (Sampling.h:242-252)."""
+    _fields_ = [("anchor", c_u32), ("depth", c_u32), ("chain", c_u32), ("children", c_u32), ("slope", c_f), ("intercept", c_f * 7),
+                ("temperature", c_f), ("noise", c_u32 * 2)]
+
+
+def draft_tree_lane(anchor, depth, children, slope=1.0, intercept=None, temperature=0.0, noise=0, chain=0):
+    lane = DraftTreeLane(anchor, depth, chain, children, slope, (c_f * 7)(*(intercept if intercept is not None else [0.0] * 7)), temperature,
+                         (c_u32 * 2)(noise & 0xFFFFFFFF, noise >> 32))
+    return lane
+
+
+def draft_tree(candidates, unary, edges, lane, chain_tokens=None, chain_rates=None):
+    """draft_select_tree of one lane: candidates uint32 [7][16], unary fp32 [7][16], edges fp32 [7][16][16]. Returns a dict:
+    tokens [n], tree TREE_DTYPE [n], q [n], estimate [n], draws uint8 [n][4], next fp32 [n][16], caps [n]."""
+    candidates = np.ascontiguousarray(candidates, np.uint32)
+    unary, edges = np.ascontiguousarray(unary, np.float32), np.ascontiguousarray(edges, np.float32)
+    chain_tokens = np.ascontiguousarray(chain_tokens if chain_tokens is not None else np.zeros(15), np.uint32)
+    chain_rates = np.ascontiguousarray(chain_rates if chain_rates is not None else np.zeros((15, 4)), np.float32)
+    tokens, tree, scores = np.zeros(16, np.uint32), np.zeros(16, TREE_DTYPE), np.zeros((16, 2), np.float32)
+    size = c_u32(0)
+    draws, nxt, caps = np.zeros((16, 4), np.uint8), np.zeros((16, 16), np.float32), np.zeros(16, np.float32)
+    lib.orc_draft_tree.restype = None
+    lib.orc_draft_tree(_p(candidates, u32p), _p(unary, f32p), _p(edges, f32p), _p(chain_tokens, u32p), _p(chain_rates, f32p), ctypes.byref(lane),
+                       _p(tokens, u32p), tree.ctypes.data_as(ctypes.c_void_p), _p(scores, f32p), ctypes.byref(size), _p(draws, u8p),
+                       _p(nxt, f32p), _p(caps, f32p))
+    n = size.value
+    return dict(tokens=tokens[:n], tree=tree[:n], q=scores[:n, 0], estimate=scores[:n, 1], draws=draws[:n], next=nxt[:n], caps=caps[:n])
+
+
 # ---- glue: rope tables, the sigmoid router, the shared expert's gate ----
 lib.orc_rope_tables.restype = None
 lib.orc_rope_tables.argtypes = [c_u32, u32p, c_u32, f32p, c_u32, f32p, f32p]
