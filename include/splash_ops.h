@@ -369,6 +369,16 @@ sp_status spo_draft_add_tree(spo_graph *graph, sp_buffer *candidates, sp_buffer 
                              sp_buffer *chain_rates, sp_buffer *tree_tokens, sp_buffer *trees, sp_buffer *tree_scores,
                              sp_buffer *tree_sizes, sp_buffer *tree_draws, sp_buffer *tree_next, sp_buffer *tree_caps,
                              const spo_draft_tree_lane *lanes, uint32_t count);
+/* The step's side of the trees, row by row of the step (no counterpart kernel in the reference, whose sampled selection
+ * reads the trees through verify_sources itself, sampling.metal:697-780): for every row the candidates of its next
+ * position (candidate_ids uint32 [rows][16], candidate_probabilities fp32 [rows][16]) and the children its draft drew
+ * (candidate_draws bytes [rows][4], 0xFF past them) -- spo_sampling_buffers' candidate fields -- and its depth (depths
+ * uint32 [rows], what the RoPE tables take), from verify_sources, lane_rows and tree_rows as spo_draft_add_verify_rows
+ * wrote them and candidates, tree_next and tree_draws of the trees. */
+sp_status spo_draft_add_verify_children(spo_graph *graph, sp_buffer *verify_sources, sp_buffer *lane_rows, sp_buffer *tree_rows,
+                                        sp_buffer *candidates, sp_buffer *tree_next, sp_buffer *tree_draws, sp_buffer *candidate_ids,
+                                        sp_buffer *candidate_probabilities, sp_buffer *candidate_draws, sp_buffer *depths,
+                                        uint32_t lanes, uint32_t rows);
 sp_status spo_draft_add_verify_rows(spo_graph *graph, sp_buffer *tree_tokens, sp_buffer *trees, sp_buffer *tree_scores,
                                     sp_buffer *tree_sizes, sp_buffer *input_tokens, sp_buffer *tree_rows, sp_buffer *lane_rows,
                                     sp_buffer *verify_sources, uint32_t lanes, uint32_t rows, uint32_t lane_cap, float floor);

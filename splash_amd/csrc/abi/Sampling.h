@@ -114,6 +114,17 @@ struct DraftTreeParams {
   uint32_t noise[SAMPLING_MAXIMUM_LANES][2];  // a 64-bit seed, low word first
 };
 
+// draft_verify_children: what a verify step's sampled rows read of the trees, row by row of the step (grid (rows), 64
+// threads): a row's depth, and of the tree row it is (sources, draft_verify_rows) the candidates of its next position
+// (ids, their probabilities at the lane's temperature) and the children its draft drew among them; a row of no lane, or
+// one whose children would lie past the draft's positions, gets no candidates and no drawn child (SAMPLING_NO_DRAW),
+// so that its selection draws from its whole distribution.
+struct VerifyChildrenParams {
+  uint32_t lanes;
+  uint32_t rows;
+  uint32_t reserved[2];
+};
+
 // decode_accept_tree: one wavefront per lane, a thread a row (the reference's AcceptBatchParams, abi/Sampling.h:314-317).
 struct AcceptBatchParams {
   uint32_t lanes;
@@ -127,6 +138,7 @@ struct AcceptBatchParams {
 static_assert(sizeof(TargetSamplingParams) == 16 + 32 + 16 + 64 + 96 + 32, "target sampling parameters are 256 bytes on both sides");
 static_assert(sizeof(DraftSelectParams) == 32 + 32, "draft selector parameters are 64 bytes on both sides");
 static_assert(sizeof(DraftTreeParams) == 4 * 32 + 16 + 32 + 224 + 32 + 64, "draft tree parameters are 496 bytes on both sides");
+static_assert(sizeof(VerifyChildrenParams) == 16, "verify children parameters are 16 bytes on both sides");
 static_assert(sizeof(VerifyRowsParams) == 16, "verify rows parameters are 16 bytes on both sides");
 static_assert(sizeof(AcceptBatchParams) == 16 + 32 + 16 + 64, "acceptance parameters are 128 bytes on both sides");
 #endif

@@ -160,6 +160,19 @@ sp_status spo_draft_add_tree(spo_graph *graph, sp_buffer *candidates, sp_buffer 
   });
 }
 
+sp_status spo_draft_add_verify_children(spo_graph *graph, sp_buffer *verify_sources, sp_buffer *lane_rows, sp_buffer *tree_rows,
+                                        sp_buffer *candidates, sp_buffer *tree_next, sp_buffer *tree_draws, sp_buffer *candidate_ids,
+                                        sp_buffer *candidate_probabilities, sp_buffer *candidate_draws, sp_buffer *depths,
+                                        uint32_t lanes, uint32_t rows) {
+  return capi::guard([&] {
+    capi::require(graph, "graph");
+    ops::DraftSelector::addVerifyChildren(capi::graphOf(graph),
+                                          {B(verify_sources), B(lane_rows), B(tree_rows), B(candidates), B(tree_next), B(tree_draws),
+                                           B(candidate_ids), B(candidate_probabilities), B(candidate_draws), B(depths)},
+                                          {lanes, rows, SAMPLING_MAXIMUM_ROWS});
+  });
+}
+
 sp_status spo_draft_add_verify_rows(spo_graph *graph, sp_buffer *tree_tokens, sp_buffer *trees, sp_buffer *tree_scores,
                                     sp_buffer *tree_sizes, sp_buffer *input_tokens, sp_buffer *tree_rows, sp_buffer *lane_rows,
                                     sp_buffer *verify_sources, uint32_t lanes, uint32_t rows, uint32_t lane_cap, float floor) {

@@ -289,4 +289,26 @@ __global__ __launch_bounds__(64) void draft_select_tree(const uint32_t *__restri
 }
 SP_REGISTER_KERNEL("draft_select_tree", &draft_select_tree);
 
+// The trees' side of a sampled verify step, gathered by the step's rows (abi/Sampling.h, VerifyChildrenParams).
+__global__ __launch_bounds__(64) void draft_verify_children(const uint32_t *__restrict__ sources, const SamplingLaneRows *__restrict__ lane_rows,
+                                                            const AttentionTreeRow *__restrict__ step_tree, const uint32_t *__restrict__ candidates,
+                                                            const float *__restrict__ tree_next, const uint8_t *__restrict__ tree_draws,
+                                                            uint32_t *__restrict__ ids, float *__restrict__ probabilities,
+                                                            uint8_t *__restrict__ draws, uint32_t *__restrict__ depths, VerifyChildrenParams p) {
+  const uint32_t row = blockIdx.x, tid = threadIdx.x;
+  if (row >= p.rows) return;
+  uint32_t lane = SAMPLING_MAXIMUM_LANES;
+  for (uint32_t l = 0; l < min(p.lanes, uint32_t(SAMPLING_MAXIMUM_LANES)); ++l)
+    if (row >= lane_rows[l].first && row < lane_rows[l].first + lane_rows[l].rows) lane = l;
+  const uint32_t source = sources[row], depth = step_tree[row].depth;
+  const bool drafted = lane < SAMPLING_MAXIMUM_LANES && source < kRows && depth < kPositions;
+  if (tid == 0) depths[row] = lane < SAMPLING_MAXIMUM_LANES ? depth : 0u;
+  if (tid < kCandidates) {
+    ids[size_t(row) * kCandidates + tid] = drafted ? candidates[(size_t(lane) * kPositions + depth) * kCandidates + tid] : SAMPLING_NO_TOKEN;
+    probabilities[size_t(row) * kCandidates + tid] = drafted ? tree_next[(size_t(lane) * kRows + source) * kCandidates + tid] : 0.f;
+  }
+  if (tid < kChildren) draws[size_t(row) * kChildren + tid] = drafted ? tree_draws[(size_t(lane) * kRows + source) * kChildren + tid] : uint8_t(SAMPLING_NO_DRAW);
+}
+SP_REGISTER_KERNEL("draft_verify_children", &draft_verify_children);
+
 } // namespace splash::kernels

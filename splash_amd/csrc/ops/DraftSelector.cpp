@@ -81,6 +81,25 @@ void DraftSelector::addTree(hip::CommandGraph &graph, const DraftTreeBuffers &b,
             params, {params.lanes, 1, 1}, {64, 1, 1});
 }
 
+void DraftSelector::addVerifyChildren(hip::CommandGraph &graph, const DraftVerifyChildrenBuffers &b, const StepRows &step) {
+  if (!step.lanes || step.lanes > SAMPLING_MAXIMUM_LANES || step.rows < step.lanes) throw std::invalid_argument("invalid decode step rows");
+  const uint64_t treeRows = uint64_t{step.lanes} * DRAFT_TREE_ROWS;
+  requireBytes(b.verifySources, uint64_t{step.rows} * 4, "verify source");
+  requireBytes(b.laneRows, uint64_t{step.lanes} * sizeof(SamplingLaneRows), "verify lane rows");
+  requireBytes(b.treeRows, uint64_t{step.rows} * sizeof(AttentionTreeRow), "verify tree row");
+  requireBytes(b.candidates, uint64_t{step.lanes} * DRAFT_PROPOSAL_TOKENS * DRAFT_CANDIDATES * 4, "draft candidate");
+  requireBytes(b.treeNext, treeRows * DRAFT_CANDIDATES * 4, "draft tree next probabilities");
+  requireBytes(b.treeDraws, treeRows * SAMPLING_TREE_CHILDREN, "draft tree draws");
+  requireBytes(b.candidateIds, uint64_t{step.rows} * SAMPLING_CANDIDATES * 4, "candidate ids");
+  requireBytes(b.candidateProbabilities, uint64_t{step.rows} * SAMPLING_CANDIDATES * 4, "candidate probabilities");
+  requireBytes(b.candidateDraws, uint64_t{step.rows} * SAMPLING_TREE_CHILDREN, "drawn children");
+  requireBytes(b.depths, uint64_t{step.rows} * 4, "row depths");
+  graph.add("draft_verify_children",
+            {b.verifySources, b.laneRows, b.treeRows, b.candidates, b.treeNext, b.treeDraws, b.candidateIds, b.candidateProbabilities,
+             b.candidateDraws, b.depths},
+            VerifyChildrenParams{step.lanes, step.rows, {0, 0}}, {step.rows, 1, 1}, {64, 1, 1});
+}
+
 void DraftSelector::addVerifyRows(hip::CommandGraph &graph, const DraftVerifyRowsBuffers &b, const StepRows &step, float floor) {
   if (!step.lanes || step.lanes > SAMPLING_MAXIMUM_LANES || !step.laneCap || step.laneCap > SAMPLING_MAXIMUM_ROWS ||
       step.rows < step.lanes || step.rows > uint64_t{step.lanes} * step.laneCap)

@@ -79,8 +79,21 @@ struct DraftTreeBuffers final {
   hip::Buffer treeCaps;      // fp32 [lanes][16]: the cap of the draft step that made or joined a row
 };
 
+// The step's rows (addVerifyRows' outputs) and the trees they came from, and what a sampled verify step reads of them.
+struct DraftVerifyChildrenBuffers final {
+  hip::Buffer verifySources, laneRows, treeRows;  // of the step, as addVerifyRows wrote them
+  hip::Buffer candidates, treeNext, treeDraws;    // of the trees (addCandidates, addTree)
+  hip::Buffer candidateIds;            // uint32 [rows][16]: the candidates of a row's next position
+  hip::Buffer candidateProbabilities;  // fp32 [rows][16]
+  hip::Buffer candidateDraws;          // bytes [rows][4]: the children the draft drew, SAMPLING_NO_DRAW past them
+  hip::Buffer depths;                  // uint32 [rows]: a row's depth below its lane's anchor (the RoPE tables' input)
+};
+
 class DraftSelector final {
 public:
+  // The candidate children of every row of the step (ops::SamplingBuffers' candidate fields) and the rows' depths, from
+  // the trees: a step then takes its tree blocks from the draft side without a copy through the host.
+  static void addVerifyChildren(hip::CommandGraph &graph, const DraftVerifyChildrenBuffers &buffers, const StepRows &step);
   // Each lane's tree over the candidates and edges addCandidates left, best first by estimate (abi/Sampling.h,
   // DraftTreeParams): rows 16 l .. of the tree buffers, lane l's sizes[l] of them.
   static void addTree(hip::CommandGraph &graph, const DraftTreeBuffers &buffers, std::span<const DraftTreeLane> lanes);

@@ -377,6 +377,14 @@ class DraftSelector:
         graph._keep.extend(buffers)
 
     @staticmethod
+    def add_verify_children(graph, verify_sources, lane_rows, tree_rows, candidates, tree_next, tree_draws, candidate_ids,
+                            candidate_probabilities, candidate_draws, depths, lanes, rows):
+        buffers = [verify_sources, lane_rows, tree_rows, candidates, tree_next, tree_draws, candidate_ids, candidate_probabilities,
+                   candidate_draws, depths]
+        check(lib.spo_draft_add_verify_children(graph.handle, *[b.handle for b in buffers], lanes, rows))
+        graph._keep.extend(buffers)
+
+    @staticmethod
     def add_verify_rows(graph, tree_tokens, trees, tree_scores, tree_sizes, input_tokens, tree_rows, lane_rows, verify_sources, lanes,
                         rows, lane_cap, floor=0.0):
         buffers = [tree_tokens, trees, tree_scores, tree_sizes, input_tokens, tree_rows, lane_rows, verify_sources]

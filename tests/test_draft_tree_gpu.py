@@ -171,3 +171,84 @@ def test_tree_rejects_bad_lanes(backend):
                          (dict(anchor=1, depth=3, children=1, temperature=-1.0), "invalid draft tree lane")]:
         with pytest.raises(splash_amd.SplashError, match=message):
             grow(backend, [lattice], [bad])
+
+
+def test_a_tree_feeds_the_step_without_the_host(backend):
+    """A sampled lane's tree goes from the draft side's kernels straight into the dense driver's input buffers (tokens,
+    tree rows, depths, candidate children), and the step's results are those of the same step with its inputs written by
+    the host from the oracle's tree: the draft side and the verify step meet on the device."""
+    from splash_amd import verify
+    from tests.dense_reference import DenseModel
+    print("case tree into the step on the device", flush=True)
+    V, rows, context, T = 32000, 16, 300, 0.9
+    model = DenseModel(seed=21, hidden=1024, q_heads=16, kv_heads=8, head_dim=64, ffn=3072, vocabulary=V, layers=2)
+    rng = np.random.default_rng(31)
+    gpu = model.build_gpu(backend, max_lanes=1, context_tokens=context + 16)
+    model.seed_context(gpu, None, rng)
+    # a synthetic draft: logits and selector rows of one lane
+    rank = 256
+    logits = rng.normal(0, 2.0, (8, V)).astype(np.float32)
+    hidden = orc.f32_to_bf16(rng.normal(0, 1, (8, rank)).astype(np.float32))
+    before = orc.f32_to_bf16(rng.normal(0, 0.08, (V, rank)).astype(np.float32))
+    after = orc.f32_to_bf16(rng.normal(0, 0.08, (V, rank)).astype(np.float32))
+    anchor = 777
+    draft_lane = dict(anchor=anchor, depth=15, children=3, intercept=[0.3] * 7, temperature=T, noise=12345678901234567)
+    up = backend.from_array
+    b = dict(candidates=backend.allocate_buffer(7 * 16 * 4), unary=backend.allocate_buffer(7 * 16 * 4), edges=backend.allocate_buffer(7 * 256 * 4),
+             scratch=backend.allocate_buffer(ops.DraftSelector.candidate_scratch_bytes(1, V)), tokens=backend.allocate_buffer(64),
+             trees=backend.allocate_buffer(128), scores=backend.allocate_buffer(128), sizes=backend.allocate_buffer(16), draws=backend.allocate_buffer(64),
+             next=backend.allocate_buffer(1024), caps=backend.allocate_buffer(64), lane_rows=backend.allocate_buffer(16), sources=backend.allocate_buffer(64))
+    lane = verify.Lane(rows, context, temperature=T)
+    uniforms = rng.random((rows, 2)).astype(np.float32)
+    child_uniforms = rng.random((rows, 4)).astype(np.float32)
+    # the step's graph exists before its inputs do: its shape is the lane's 16 rows
+    gpu.set_block([lane], np.zeros(rows, np.uint32), uniforms=uniforms)
+    gpu.set_candidate_children(np.zeros((rows, 16), np.uint32), np.zeros((rows, 16), np.float32), np.full((rows, 4), 0xFF, np.uint8), child_uniforms)
+    step = gpu.encode([lane], commit=False)
+    assert "decode_sample_draw_children" in step.kernels()
+    children = [gpu.buffer(verify.CANDIDATE_CHILDREN, which) for which in range(3)]
+    draft = splash_amd.CommandGraph()
+    ops.DraftSelector.add_candidates(draft, up(logits), up(hidden), b["scratch"], b["candidates"], b["unary"], b["edges"], up(before), up(after),
+                                     V, V, V, [anchor])
+    ops.DraftSelector.add_tree(draft, b["candidates"], b["unary"], b["edges"], up(np.zeros((1, 15), np.uint32)), up(np.zeros((1, 15, 4), np.float32)),
+                               b["tokens"], b["trees"], b["scores"], b["sizes"], b["draws"], b["next"], b["caps"], [draft_lane])
+    ops.DraftSelector.add_verify_rows(draft, b["tokens"], b["trees"], b["scores"], b["sizes"], gpu.buffer(verify.INPUT_TOKENS),
+                                      gpu.buffer(verify.TREE_ROWS), b["lane_rows"], b["sources"], 1, rows, rows)
+    ops.DraftSelector.add_verify_children(draft, b["sources"], b["lane_rows"], gpu.buffer(verify.TREE_ROWS), b["candidates"], b["next"], b["draws"],
+                                          children[0], children[1], children[2], gpu.buffer(verify.DEPTHS), 1, rows)
+    backend.run(draft)
+    backend.run(step)
+    device_results = gpu.results([lane])
+    device_logits = gpu.buffer(verify.LOGITS).download(np.float32, rows * V).copy()
+    assert b["sizes"].download(np.uint32)[0] == rows and list(b["lane_rows"].download(np.uint32)[:2]) == [0, rows]
+    # the same step from the host: the oracle's tree over the GPU's own candidates and edges, laid out and gathered in numpy
+    candidates = b["candidates"].download(np.uint32).reshape(7, 16)
+    unary, edges = b["unary"].download(np.float32).reshape(7, 16), b["edges"].download(np.float32).reshape(7, 16, 16)
+    oracle_lane = orc.draft_tree_lane(anchor=anchor, depth=15, children=3, intercept=[0.3] * 7, temperature=T, noise=draft_lane["noise"])
+    if stated_tree(candidates, unary, edges, oracle_lane) is None:
+        pytest.skip("a drawn lattice whose order hangs on the rounding of exp")
+    grown = orc.draft_tree(candidates, unary, edges, oracle_lane)
+    assert len(grown["tokens"]) == rows
+    scores = np.stack([grown["q"], grown["estimate"]], axis=1)[None]
+    w_tokens, w_tree, w_lane_rows, w_sources = orc.draft_verify_rows(grown["tokens"][None], grown["tree"][None], scores, [rows], rows, rows)
+    ids = np.full((rows, 16), 0xFFFFFFFF, np.uint32)
+    q = np.zeros((rows, 16), np.float32)
+    draws = np.full((rows, 4), 0xFF, np.uint8)
+    for r in range(rows):
+        depth, source = int(w_tree["depth"][r]), int(w_sources[r])
+        if depth < 7:
+            ids[r], q[r], draws[r] = candidates[depth], grown["next"][source], grown["draws"][source]
+    got_ids = children[0].download(np.uint32)[:rows * 16].reshape(rows, 16)
+    got_draws = children[2].download(np.uint8)[:rows * 4].reshape(rows, 4)
+    assert np.array_equal(got_ids, ids) and np.array_equal(got_draws, draws)
+    assert np.allclose(children[1].download(np.float32)[:rows * 16].reshape(rows, 16), q, rtol=1e-4, atol=1e-7)
+    assert np.array_equal(gpu.buffer(verify.INPUT_TOKENS).download(np.uint32)[:rows], w_tokens)
+    assert np.array_equal(gpu.buffer(verify.DEPTHS).download(np.uint32)[:rows], w_tree["depth"].astype(np.uint32))
+    # ... and run from the host's copies of exactly what the device wrote (its probabilities, to the last bit)
+    q_device = children[1].download(np.float32)[:rows * 16].reshape(rows, 16).copy()
+    gpu.set_block([lane], w_tokens, tree_rows=w_tree, uniforms=uniforms)
+    gpu.set_candidate_children(ids, q_device, draws, child_uniforms)
+    backend.run(step)
+    assert np.array_equal(gpu.buffer(verify.LOGITS).download(np.float32, rows * V), device_logits)
+    for got, want in zip(gpu.results([lane]), device_results):
+        assert np.array_equal(got, want)
