@@ -525,6 +525,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--chain", action="store_true",
                     help="one dispatch for a layer's four projections after its attention instead of a dispatch each")
+    ap.add_argument("--fused-prepare", action="store_true",
+                    help="a layer's q|k|v projection prepares its attention block itself: one dispatch instead of the "
+                         "projection and the prepare kernel")
     ap.add_argument("--calibrate-traffic", action="store_true",
                     help="after the steps, run plain read and copy kernels of known size: the scale of the FETCH_SIZE / "
                          "WRITE_SIZE counters of a rocprofv3 --pmc run of this command")
@@ -561,6 +564,8 @@ def main():
     gpu.set_block(lanes, rng.integers(0, w["vocabulary"], rows).astype(np.uint32), uniforms=rng.random((rows, 2), dtype=np.float32))
     if args.chain:
         gpu.set_chained(True)
+    if args.fused_prepare:
+        gpu.set_fused_prepare(True)
     graph = gpu.encode(lanes, commit=True)
     if args.temperature > 0:
         # the draft model's distributions of the block's rows: softmax of N(0, 2) logits over the whole vocabulary

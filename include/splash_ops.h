@@ -163,6 +163,19 @@ sp_status spo_attention_add_projection(spo_graph *graph, const spo_attention_pla
                                        sp_buffer *query_norm, sp_buffer *key_norm, sp_buffer *rope_cos,
                                        sp_buffer *rope_sin, sp_buffer *queries, sp_buffer *query_sums,
                                        sp_buffer *page_table, sp_buffer *pool, uint64_t page_bytes);
+/* The block's q|k|v projection and spo_attention_add_projection's work as ONE dispatch, where the reference runs the
+ * projection and its prepare kernel one after the other (QwenTarget.cpp:457-470, PagedAttention.cpp:441-464): the
+ * workgroup that completes a head's columns norms, rotates, stages or stores it. `qkv` is what spo_linear_add_link
+ * takes (a plain bf16 plan; its output is the block's packed rows); its partials hold plan.splits x
+ * (output size / 64) x storage_rows x 256 bytes and its counters 4 bytes a 64 columns, whatever the plan's parts. The
+ * packed rows, staged queries, their sums and the cache bytes equal those of the two dispatches bit for bit.
+ * spo_attention_fuses_projection: 1 when the kernels take the pair (up to 64 rows, every workgroup one part of K,
+ * heads of 64 or 128 dimensions whole in the projection's tensors, fp16 queries, no gates), else 0. */
+int spo_attention_fuses_projection(const spo_attention_plan *plan, const spo_projection *projection, const spo_linear_plan *linear_plan);
+sp_status spo_attention_add_fused_projection(const spo_linear *linear, spo_graph *graph, const spo_chain_link *qkv,
+                                             const spo_attention_plan *plan, sp_buffer *query_norm, sp_buffer *key_norm,
+                                             sp_buffer *rope_cos, sp_buffer *rope_sin, sp_buffer *queries,
+                                             sp_buffer *query_sums, sp_buffer *page_table, sp_buffer *pool, uint64_t page_bytes);
 /* PagedAttention::addAttention (PagedAttention.cpp:466-607): split, then ordered reduce.
  * output_table (optional, spo_gguf_table_bytes(q_heads * head_dim, rows) bytes): the reduce also
  * writes the rows as the activation table of the projection that follows. packed_qkv: the rows'
@@ -450,6 +463,10 @@ sp_status spo_dense_verify_results(spo_dense_verify *verify, const spo_verify_la
  * their shapes allow: off by default; the results are the same bit for bit. spo_dense_verify_results fails with
  * SP_BACKEND_ERROR after a step in which a chained projection's bounded wait gave up. */
 sp_status spo_dense_verify_set_chained(spo_dense_verify *verify, int chained);
+/* DenseVerify::setFusedPrepare: a layer's q|k|v projection also prepares its attention block
+ * (spo_attention_add_fused_projection) where the kernels take the pair: off by default (on MI355X the two dispatches
+ * are the faster at the 27B shape); the results are the same bit for bit. */
+sp_status spo_dense_verify_set_fused_prepare(spo_dense_verify *verify, int fused);
 
 /* ---- The hybrid mixture-of-experts verify step (the reference's Qwen3.5 target with Gated
  *      DeltaNet mixers: QwenTarget.cpp:206-255 the GDN mixer, :263-347 the attention mixer, :372-395

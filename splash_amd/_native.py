@@ -253,6 +253,8 @@ _sig("spo_attention_plan_destroy", None, c_p)
 _sig("spo_attention_plan_splits", c_u32, c_p)
 _sig("spo_attention_workspace", c_int, c_p, P(c_u64))
 _sig("spo_attention_add_projection", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_u64)
+_sig("spo_attention_fuses_projection", c_int, c_p, c_p, P(LinearPlan))
+_sig("spo_attention_add_fused_projection", c_int, c_p, c_p, P(ChainLink), c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_u64)
 _sig("spo_attention_add_attention", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_u64, c_p, c_p, c_p)
 _sig("spo_attention_add_path_commit", c_int, c_p, c_p, c_p, c_p, c_p, c_u64)
 
@@ -285,6 +287,7 @@ _sig("spo_sampling_add_acceptance", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, P(
 _sig("spo_sampling_greedy_rows_static", c_int, ctypes.c_void_p, c_u32, c_u32, c_u32, ctypes.c_void_p, ctypes.c_void_p)
 _sig("spo_verify_check_results", c_int, P(LaneRows), P(c_u32), c_u32, c_u32, c_u32, P(c_u32), P(c_u32), P(c_u32), P(c_u32))
 _sig("spo_dense_verify_set_chained", c_int, c_p, c_int)
+_sig("spo_dense_verify_set_fused_prepare", c_int, c_p, c_int)
 _sig("spo_dense_verify_results", c_int, c_p, P(VerifyLane), c_u32, P(c_u32), P(c_u32), P(c_u32), P(c_u32))
 _sig("spg_dense_dimensions", c_int, c_p, P(DenseDimensions))
 _sig("spo_dense_verify_load_gguf", c_int, c_p, c_p)

@@ -193,6 +193,13 @@ struct GgufPrepareParams {
 // multiplies its sums by it (deferred_scale): a per-row factor commutes with the projection. One
 // tensor, whole super-blocks of output columns.
 #define GGUF_EPILOGUE_RESIDUAL_NORM 5u
+// out = bf16(v), the fused q|k|v rows, and on them the work of attention_q8_qkv (abi/PagedAttention.h): the q and k heads'
+// RMS norms, RoPE, the staged queries and their sums, the block's keys and values quantized into their page slots: kernels
+// gguf_decode_qkv_<fmt>_m<rows> and gguf_decode_qkv_mixed_m<rows> (GgufQkvParams). A head's 64 or 128 columns lie in one
+// or two workgroups times `splits` parts of K; all of them leave partials and the last to arrive finishes the head, so
+// the dispatch keeps partials and counters even unsplit, every workgroup takes a part (whole_groups 0), and the
+// segments hold whole heads.
+#define GGUF_EPILOGUE_QKV_PREPARE 6u
 
 // gguf_decode_<fmt>_m<16|32|64>_<a|a_f32|r|g>: up to three column segments of one format in one
 // dispatch (the reference's GgufDecodeFusedParams, runtime/metal/abi/Gguf.h:168-178), tiles in
@@ -246,6 +253,16 @@ struct GgufChainParams {
   uint32_t reserved[2];
   struct GgufChainLink link[GGUF_CHAIN_LINKS];
 };
+
+#ifdef ATTENTION_MAXIMUM_SEQUENCES
+// gguf_decode_qkv_*: a decode projection's parameters and the attention block's (abi/PagedAttention.h, included first).
+// Binds seg0..2, table, out, partials, counters, then the query and key norm weights, the RoPE cosine and sine tables,
+// the staged queries and their sums, the page table and the layer's pool, as attention_q8_qkv does.
+struct GgufQkvParams {
+  struct GgufDecodeParams decode;
+  struct AttentionParams attention;
+};
+#endif
 
 // gguf_dequant_<fmt>: the image's fp32 values [N][K], for the bit-exactness test
 // (the reference's gguf_dequant_test.metal). Grid (K / 256, N / 16), 64 threads.

@@ -6,7 +6,6 @@
 
 using namespace splash;
 
-struct spo_attention_plan { ops::AttentionPlan plan; };
 
 namespace {
 ops::KvPages pagesOf(sp_buffer *table, sp_buffer *pool, uint64_t pageBytes) {

@@ -4,10 +4,12 @@
 #include "hip/Backend.hpp"
 
 #include "ops/Linear.hpp"
+#include "ops/PagedAttention.hpp"
 
 struct spo_graph { splash::hip::CommandGraph graph; };
 struct spo_projection { splash::ops::Projection projection; };
 struct spo_linear { splash::ops::Linear linear; };
+struct spo_attention_plan { splash::ops::AttentionPlan plan; };
 
 struct spg_file;
 namespace splash::model {

@@ -299,6 +299,12 @@ sp_status spo_dense_verify_set_chained(spo_dense_verify *verify, int chained) {
     verify->verify->setChained(chained != 0);
   });
 }
+sp_status spo_dense_verify_set_fused_prepare(spo_dense_verify *verify, int fused) {
+  return capi::guard([&] {
+    capi::require(verify, "verify");
+    verify->verify->setFusedPrepare(fused != 0);
+  });
+}
 uint64_t spo_dense_verify_page_bytes(const spo_dense_verify *verify) { return verify ? verify->verify->pageBytes() : 0; }
 uint64_t spo_dense_verify_step_bytes(const spo_dense_verify *verify, const spo_verify_lane *lanes, uint32_t count) {
   uint64_t bytes = 0;

@@ -232,6 +232,28 @@ sp_status spo_linear_add_link(const spo_linear *linear, spo_graph *graph, const 
     linear->linear.add(graph->graph, std::move(one.buffers), *one.projection, one.plan, one.gate);
   });
 }
+int spo_attention_fuses_projection(const spo_attention_plan *plan, const spo_projection *projection, const spo_linear_plan *linear_plan) {
+  if (!plan || !projection || !linear_plan) return 0;
+  try {
+    return ops::PagedAttention::fusesProjection(plan->plan, projection->projection, toPlan(projection->projection, *linear_plan)) ? 1 : 0;
+  } catch (...) {
+    return 0;
+  }
+}
+sp_status spo_attention_add_fused_projection(const spo_linear *linear, spo_graph *graph, const spo_chain_link *qkv,
+                                             const spo_attention_plan *plan, sp_buffer *query_norm, sp_buffer *key_norm,
+                                             sp_buffer *rope_cos, sp_buffer *rope_sin, sp_buffer *queries, sp_buffer *query_sums,
+                                             sp_buffer *page_table, sp_buffer *pool, uint64_t page_bytes) {
+  return capi::guard([&] {
+    capi::require(linear && graph && qkv && plan, "linear, graph, projection or plan");
+    ops::ChainedProjection one = linkOf(*qkv);
+    ops::AttentionProjectionBuffers b{one.buffers.output, hip::Buffer::share(query_norm), hip::Buffer::share(key_norm),
+                                      hip::Buffer::share(rope_cos), hip::Buffer::share(rope_sin)};
+    ops::AttentionWorkspace w{hip::Buffer::share(queries), hip::Buffer::share(query_sums), {}, {}};
+    ops::PagedAttention::addFusedProjection(graph->graph, linear->linear, std::move(one.buffers), *one.projection, one.plan, plan->plan, b, w,
+                                            ops::KvPages{hip::Buffer::share(page_table), hip::Buffer::share(pool), page_bytes});
+  });
+}
 sp_status spo_linear_add_swiglu(const spo_linear *linear, spo_graph *graph, const spo_projection *gate,
                                 const spo_projection *up, const spo_projection *down, sp_buffer *normalized,
                                 sp_buffer *intermediate, sp_buffer *residual, sp_buffer *output, uint32_t rows,

@@ -14,6 +14,8 @@
 // a workgroup that share tiles sum their ranges through LDS in wave order, and `splits` workgroups
 // (grid.y) sum theirs through fp32 partials in split order, the last arriver applying the
 // epilogue (the reference's split_reduce.h:28-54), so a result never depends on arrival order.
+#include "abi/PagedAttention.h"
+
 #include "abi/Gguf.h"
 #include "abi/Moe.h"
 #include "backend/KernelRegistry.hpp"
@@ -539,13 +541,221 @@ __device__ __forceinline__ void chain_wait(const ChainPosition &chain) {
   __builtin_amdgcn_sched_barrier(0);
 }
 
+// The head norms, RoPE and cache store of attention_q8_qkv (kernels/paged_attention.hip; the reference's
+// attention_qkv_prepare.h:59-66, attention_store.h:52-85) as the epilogue of the fused q|k|v projection
+// (GGUF_EPILOGUE_QKV_PREPARE): what that kernel binds and its parameters.
+struct QkvPrepare {
+  const uint16_t *queryNorm, *keyNorm;
+  const float *ropeCos, *ropeSin;
+  _Float16 *queries;
+  float *querySums;
+  const uint64_t *pageTable;
+  uint8_t *pool;
+  const AttentionParams *attention;
+};
+// One head's rows, a wave a row at a time, four rows a wave of each 16: `tile` holds the head's columns of every packed
+// row as the projection's bf16 results (the values attention_q8_qkv reads back from the packed rows), lane l of a wave
+// elements l and l + 64 of its row. Every sum and maximum is taken as attention_q8_qkv's 64-lane waves take them (a
+// butterfly over elements 0..63, one over 64..127, then the two added in that order), so the staged queries, their sums,
+// the cached codes and scales are that kernel's bit for bit.
+// What a row needs from memory does not depend on the projection's sums -- its sequence, its RoPE angles, its page --
+// so a wave fetches that of its four rows ahead (QkvRowsAhead), before the sums' own loads, and the epilogue waits
+// for one round trip instead of one a row.
+struct QkvRowAhead {
+  uint32_t z, row, token;   // the sequence (sequences: the packed row is in no block), the row of its block, its slot in the page
+  float cosine[2], sine[2];
+  uint64_t page;            // the physical page of the row's slot
+};
+struct QkvHead {
+  bool query, key;
+  uint32_t index, group;    // the head among its kind; query heads a KV head
+  uint32_t weight[2];       // the head norm's weights of this lane's elements, as loaded (converted where they are used, so
+                            // that nothing waits for them before the other loads have left)
+};
+__device__ __forceinline__ QkvHead qkv_head(uint32_t head, const QkvPrepare &q) {
+  const AttentionParams &a = *q.attention;
+  const uint32_t lane = threadIdx.x & 63u, halves = a.head_dim / 64u;
+  QkvHead h;
+  h.query = head < a.q_heads;
+  h.key = !h.query && head < a.q_heads + a.kv_heads;
+  h.index = h.query ? head : h.key ? head - a.q_heads : head - a.q_heads - a.kv_heads;
+  h.group = a.q_heads / a.kv_heads;
+  h.weight[0] = h.weight[1] = 0;
+  if (a.normalize && (h.query || h.key))
+    _Pragma("unroll") for (uint32_t e = 0; e < 2u; ++e) if (e < halves) h.weight[e] = (h.query ? q.queryNorm : q.keyNorm)[lane + 64u * e];
+  return h;
+}
+__device__ __forceinline__ void qkv_rows_ahead(QkvRowAhead (&ahead)[4], const QkvHead &h, uint32_t first, uint32_t rows, const QkvPrepare &q) {
+  const AttentionParams &a = *q.attention;
+  const uint32_t lane = threadIdx.x & 63u, halves = a.head_dim / 64u;
+  // a wave's rows are the same in every lane: the search of their sequences runs on the scalar unit
+  const uint32_t wave = uint32_t(__builtin_amdgcn_readfirstlane(int(threadIdx.x >> 6)));
+  uint32_t entry[4] = {0, 0, 0, 0};
+#pragma unroll
+  for (uint32_t i = 0; i < 4; ++i) ahead[i].z = a.sequences;
+  for (uint32_t s = 0; s < a.sequences; ++s) {
+    const AttentionSequence seq = a.sequence[s];
+#pragma unroll
+    for (uint32_t i = 0; i < 4; ++i) {
+      const uint32_t packed = first + wave + 4u * i;
+      if (packed < rows && packed - seq.first_row < seq.rows) {
+        const uint32_t slot = seq.committed + (packed - seq.first_row);
+        ahead[i].z = s;
+        ahead[i].row = packed - seq.first_row;
+        ahead[i].token = slot % ATTENTION_PAGE_TOKENS;
+        entry[i] = seq.table_first + slot / ATTENTION_PAGE_TOKENS;
+      }
+    }
+  }
+#pragma unroll
+  for (uint32_t i = 0; i < 4; ++i) {
+    QkvRowAhead &r = ahead[i];
+    if (r.z == a.sequences) continue;
+    const uint32_t packed = first + wave + 4u * i;
+    if (a.rotary_pairs && (h.query || h.key))
+      _Pragma("unroll") for (uint32_t e = 0; e < 2u; ++e) if (e < halves) {
+        const uint32_t at = lane + 64u * e;
+        if (at < 2u * a.rotary_pairs) {
+          const uint32_t pair = at < a.rotary_pairs ? at : at - a.rotary_pairs;
+          r.cosine[e] = q.ropeCos[size_t(packed) * a.rotary_pairs + pair];
+          r.sine[e] = q.ropeSin[size_t(packed) * a.rotary_pairs + pair];
+        }
+      }
+    if (!h.query) r.page = q.pageTable[entry[i]];
+  }
+}
+// A wave's four rows move through the stages together: the reductions of different rows are independent chains the
+// hardware overlaps, and no row waits for the stores of the one before it.
+__device__ __forceinline__ void qkv_prepare_rows(const float (*tile)[128], float (*staged)[4][128], const QkvRowAhead (&ahead)[4],
+                                                 const QkvHead &head, uint32_t first, const QkvPrepare &q) {
+  const AttentionParams &a = *q.attention;
+  const uint32_t lane = threadIdx.x & 63u, wave = uint32_t(__builtin_amdgcn_readfirstlane(int(threadIdx.x >> 6)));
+  const uint32_t D = a.head_dim, halves = D / 64u;
+  const bool query = head.query, key = head.key, two = halves == 2u;
+  const uint32_t index = head.index, group = head.group;
+  // the weights' bits become floats here and no earlier: the conversion placed at their load would wait for it there
+  uint32_t weightBits[2] = {head.weight[0], head.weight[1]};
+  asm volatile("" : "+v"(weightBits[0]), "+v"(weightBits[1]));
+  const float weight[2] = {bf16_bits_to_float(weightBits[0]), bf16_bits_to_float(weightBits[1])};
+  bool valid[4];
+  float result[4][2];
+#pragma unroll
+  for (uint32_t i = 0; i < 4; ++i) {
+    valid[i] = ahead[i].z != a.sequences;
+    const uint32_t packed = first + wave + 4u * i;
+    result[i][0] = valid[i] ? tile[packed][lane] : 0.f;
+    result[i][1] = valid[i] && two ? tile[packed][lane + 64u] : 0.f;
+  }
+  if (a.normalize && (query || key)) {
+    // attention_qkv_prepare.h:59-66: inv = rsqrt(sum x^2 / D + 1e-6); n = bf16(x inv w)
+    float total[4], high[4];
+#pragma unroll
+    for (uint32_t i = 0; i < 4; ++i) total[i] = wave_sum(result[i][0] * result[i][0]);
+    if (two) {
+#pragma unroll
+      for (uint32_t i = 0; i < 4; ++i) high[i] = wave_sum(result[i][1] * result[i][1]);
+#pragma unroll
+      for (uint32_t i = 0; i < 4; ++i) total[i] += high[i];
+    }
+#pragma unroll
+    for (uint32_t i = 0; i < 4; ++i) {
+      const float inverse = 1.0f / sqrtf(total[i] / float(D) + 1e-6f);
+      result[i][0] = round_bf16(result[i][0] * inverse * weight[0]);
+      if (two) result[i][1] = round_bf16(result[i][1] * inverse * weight[1]);
+    }
+  }
+  if (a.rotary_pairs && (query || key)) {
+#pragma unroll
+    for (uint32_t i = 0; i < 4; ++i) {
+      staged[wave][i][lane] = result[i][0];
+      if (two) staged[wave][i][lane + 64u] = result[i][1];
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+    for (uint32_t i = 0; i < 4; ++i)
+      _Pragma("unroll") for (uint32_t h = 0; h < 2u; ++h) if (h < halves) {
+        const uint32_t at = lane + 64u * h;
+        if (valid[i] && at < 2u * a.rotary_pairs) {
+          const uint32_t pair = at < a.rotary_pairs ? at : at - a.rotary_pairs;
+          const float low = staged[wave][i][pair], other = staged[wave][i][pair + a.rotary_pairs];
+          const float cosine = ahead[i].cosine[h], sine = ahead[i].sine[h];
+          result[i][h] = at < a.rotary_pairs ? round_bf16(low * cosine - other * sine) : round_bf16(other * cosine + low * sine);
+        }
+      }
+    __builtin_amdgcn_wave_barrier();
+  }
+  if (query) {
+    _Float16 half[4][2];
+    float sum[4], high[4];
+#pragma unroll
+    for (uint32_t i = 0; i < 4; ++i) {
+      half[i][0] = _Float16(result[i][0]);
+      half[i][1] = _Float16(result[i][1]);
+      sum[i] = wave_sum(float(half[i][0]));
+    }
+    if (two) {
+#pragma unroll
+      for (uint32_t i = 0; i < 4; ++i) high[i] = wave_sum(float(half[i][1]));
+#pragma unroll
+      for (uint32_t i = 0; i < 4; ++i) sum[i] += high[i];
+    }
+#pragma unroll
+    for (uint32_t i = 0; i < 4; ++i) {
+      if (!valid[i]) continue;
+      const size_t at = (size_t(ahead[i].z) * a.kv_heads * group + index) * 16u + ahead[i].row;
+      q.queries[at * D + lane] = half[i][0];
+      if (two) q.queries[at * D + lane + 64u] = half[i][1];
+      if (lane == 0) q.querySums[at] = sum[i];
+    }
+    return;
+  }
+  // attention_store.h:52-85: scale = max / 127, code = clamp(rint(v 127 / max)); the scale is stored fp16.
+  float largest[4];
+#pragma unroll
+  for (uint32_t i = 0; i < 4; ++i) largest[i] = wave_max(fmaxf(fabsf(result[i][0]), fabsf(result[i][1])));
+#pragma unroll
+  for (uint32_t i = 0; i < 4; ++i) {
+    if (!valid[i]) continue;
+    const QkvRowAhead &r = ahead[i];
+    uint8_t *page = q.pool + r.page * a.page_bytes;
+    _Pragma("unroll") for (uint32_t h = 0; h < 2u; ++h) if (h < halves) {
+      int code = 0;
+      if (largest[i] != 0.0f) {
+        code = int(rintf(result[i][h] * 127.0f / largest[i]));
+        code = code < -127 ? -127 : code > 127 ? 127 : code;
+      }
+      const uint32_t dim = lane + 64u * h;
+      if (key) reinterpret_cast<int8_t *>(page)[attention_key_index(index, r.token, dim, D)] = int8_t(code);
+      else reinterpret_cast<int8_t *>(page + attention_page_values_offset(a.kv_heads, D))[attention_value_index(index, r.token, dim, D)] = int8_t(code);
+    }
+    if (lane == 0) {
+      uint16_t *scales = reinterpret_cast<uint16_t *>(page + (key ? attention_page_key_scales_offset(a.kv_heads, D) : attention_page_value_scales_offset(a.kv_heads, D)));
+      scales[attention_scale_index(index, r.token)] = uint16_t(float_to_half_bits(largest[i] == 0.0f ? 0.0f : largest[i] / 127.0f));
+    }
+  }
+}
+// the staged rows past a sequence's block are zero (the attention kernel reads 16 rows a head)
+__device__ __forceinline__ void qkv_clear_rows(const QkvHead &head, const QkvPrepare &q) {
+  const AttentionParams &a = *q.attention;
+  const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6, D = a.head_dim, halves = D / 64u;
+  if (!head.query) return;
+  for (uint32_t z = 0; z < a.sequences; ++z)
+    for (uint32_t row = a.sequence[z].rows + wave; row < 16u; row += 4u) {
+      const size_t at = (size_t(z) * a.kv_heads * head.group + head.index) * 16u + row;
+      _Pragma("unroll") for (uint32_t h = 0; h < 2u; ++h) if (h < halves) q.queries[at * D + lane + 64u * h] = _Float16(0.f);
+      if (lane == 0) q.querySums[at] = 0.f;
+    }
+}
+
 template <uint32_t FMT, int RT, uint32_t EP, bool Chain = false>
 __device__ __forceinline__ void decode_workgroup(DecodeShared<RT> &shared, const uint8_t *__restrict__ seg0,
                                                  const uint8_t *__restrict__ seg1, const uint8_t *__restrict__ seg2,
                                                  const uint8_t *__restrict__ table, void *__restrict__ out,
                                                  const uint16_t *__restrict__ residual, float *__restrict__ partials,
                                                  uint32_t *__restrict__ counters, const GgufDecodeParams &p, const uint32_t item,
-                                                 const ChainPosition &chain = ChainPosition{}) {
+                                                 const ChainPosition &chain = ChainPosition{}, const QkvPrepare *prepare = nullptr) {
   // A chained link reads only what has one writer a cache line: a group's values, a workgroup's 16-input sums, a squares
   // entry. The 32-input sums have two (a gate/up workgroup writes 64 bytes of them), so a chained link adds the two
   // 16-input sums they are the sum of, the same fp32 addition their writer made.
@@ -758,7 +968,134 @@ __device__ __forceinline__ void decode_workgroup(DecodeShared<RT> &shared, const
     }
   }
 
+  // The sum of a unit's parts in part order; the loads of a round are in flight together (the loop's staging registers
+  // are free by now), so the sum costs one or two round trips to the coherence point whatever the parts.
+  auto orderedSum = [&](const float *from, size_t stride, uint32_t parts) {
+    constexpr uint32_t kRound = RT == 1 ? 16u : RT == 2 ? 8u : 4u;
+#pragma unroll
+    for (int t = 0; t < RT; ++t)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) acc[t][v] = 0.f;
+    for (uint32_t s0 = 0; s0 < parts; s0 += kRound) {
+      float part[kRound][RT][4];
+#pragma unroll
+      for (uint32_t s = 0; s < kRound; ++s) {
+        if (s0 + s < parts) {
+#pragma unroll
+          for (int t = 0; t < RT; ++t)
+#pragma unroll
+            for (int v = 0; v < 4; ++v)
+              part[s][t][v] = __hip_atomic_load(from + size_t(s0 + s) * stride + (t * 4 + v) * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        } else {
+#pragma unroll
+          for (int t = 0; t < RT; ++t)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) part[s][t][v] = 0.f;
+        }
+      }
+#pragma unroll
+      for (uint32_t s = 0; s < kRound; ++s)
+#pragma unroll
+        for (int t = 0; t < RT; ++t)
+#pragma unroll
+          for (int v = 0; v < 4; ++v) acc[t][v] += s0 + s < parts ? part[s][t][v] : 0.f;
+    }
+  };
   // Element (t, v) of this lane is row 16 t + 4 kq + v, column tile.column + c.
+  if constexpr (EP == GGUF_EPILOGUE_QKV_PREPARE) {
+    // A head's columns lie in one or two workgroups (64 columns each) times `splits` parts of K: every one of them leaves
+    // its sums as partials and counts itself in on the head's counter, and the last to arrive sums each column tile's
+    // parts in part order (the sums of the plain projection), writes the packed rows and runs the head's norms, RoPE
+    // and cache store on them.
+    const AttentionParams &a = *prepare->attention;
+    const uint32_t halves = a.head_dim / 64u, headOf = group / halves;
+    const size_t stride = size_t((p.units + 3u) / 4u) * 4u * RT * 256u;
+    float *mineAt = partials + (size_t(unit) * RT * 4u) * 64u + lane;
+    if (live) {
+#pragma unroll
+      for (int t = 0; t < RT; ++t)
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+          __hip_atomic_store(mineAt + size_t(split) * stride + (t * 4 + v) * 64, acc[t][v], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    if (threadIdx.x == 0) arrived = __hip_atomic_fetch_add(counters + headOf, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (arrived != halves * splits - 1u) return;
+    if (threadIdx.x == 0) __hip_atomic_store(counters + headOf, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    // the staging buffers are free: the head's rows as floats, then a row a wave for the RoPE exchange
+    float (*headRows)[128] = reinterpret_cast<float (*)[128]>(&ldsA[0][0][0][0]);
+    float (*waveRows)[4][128] = reinterpret_cast<float (*)[4][128]>(reinterpret_cast<char *>(&ldsA[0][0][0][0]) + 16u * RT * 128u * 4u);
+    static_assert(sizeof(shared.a) >= 16u * RT * 128u * 4u + 4u * 4u * 128u * 4u, "the staging buffers hold a head's rows and a wave's four");
+    const uint8_t *const seg[3] = {seg0, seg1, seg2};
+    const uint32_t firstColumn = uint32_t(__builtin_amdgcn_readfirstlane(int(find_tile(headOf * halves * 4u, seg, p, kRecord).column)));
+    const uint32_t rows = min(p.rows, 16u * RT);
+    // what the first rows need from memory, in flight with the sums' own loads
+    const QkvHead head = qkv_head(firstColumn / a.head_dim, *prepare);
+    QkvRowAhead ahead[4];
+    qkv_rows_ahead(ahead, head, 0u, rows, *prepare);
+    // A head of two halves at one row tile and up to eight parts: both halves' parts in flight together.
+    constexpr uint32_t kBoth = RT == 1 ? 8u : 0u;
+    float sums[2][RT][4];
+    if (kBoth && halves == 2u && splits <= kBoth) {
+      float part[2][kBoth ? kBoth : 1u][4];
+#pragma unroll
+      for (uint32_t half = 0; half < 2u; ++half) {
+        const float *from = partials + (size_t((headOf * 2u + half) * 4u + wave) * RT * 4u) * 64u + lane;
+#pragma unroll
+        for (uint32_t s = 0; s < kBoth; ++s)
+#pragma unroll
+          for (int v = 0; v < 4; ++v)
+            part[half][s][v] = s < splits ? __hip_atomic_load(from + size_t(s) * stride + v * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0.f;
+      }
+#pragma unroll
+      for (uint32_t half = 0; half < 2u; ++half)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          float total = 0.f;
+#pragma unroll
+          for (uint32_t s = 0; s < kBoth; ++s) total += s < splits ? part[half][s][v] : 0.f;
+          sums[half][0][v] = total;
+        }
+    } else {
+#pragma unroll
+      for (uint32_t half = 0; half < 2u; ++half) {
+        if (half >= halves) break;
+        orderedSum(partials + (size_t((headOf * halves + half) * 4u + wave) * RT * 4u) * 64u + lane, stride, splits);
+#pragma unroll
+        for (int t = 0; t < RT; ++t)
+#pragma unroll
+          for (int v = 0; v < 4; ++v) sums[half][t][v] = acc[t][v];
+      }
+    }
+#pragma unroll
+    for (uint32_t half = 0; half < 2u; ++half) {
+      if (half >= halves) break;
+      const uint32_t column = find_tile((headOf * halves + half) * 4u + wave, seg, p, kRecord).column;
+#pragma unroll
+      for (int t = 0; t < RT; ++t)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          const uint32_t row = 16u * t + 4u * kq + v;
+          if (row >= p.rows) continue;
+          const float sum = p.deferred_scale ? sums[half][t][v] * rowScale[row] : sums[half][t][v];
+          const uint32_t bits = float_to_bf16_bits(sum);
+          static_cast<uint16_t *>(out)[size_t(row) * p.out_stride + column + c] = uint16_t(bits);
+          headRows[row][half * 64u + 16u * wave + c] = bf16_bits_to_float(bits);
+        }
+    }
+    __syncthreads();
+    for (uint32_t first = 0; first < rows; first += 16u) {
+      if (first) qkv_rows_ahead(ahead, head, first, rows, *prepare);
+      // everything fetched ahead has arrived before the first store leaves: no later wait counts stores
+      __builtin_amdgcn_s_waitcnt(0);
+      qkv_prepare_rows(headRows, waveRows, ahead, head, first, *prepare);
+    }
+    qkv_clear_rows(head, *prepare);
+    return;
+  }
   if (splits > 1) {
     // Partials [split][partitioned unit][t][v][lane]: whole-wave contiguous stores and loads.
     const uint32_t partitioned = (p.units + 3u) / 4u - p.whole_groups;  // workgroups
@@ -781,37 +1118,7 @@ __device__ __forceinline__ void decode_workgroup(DecodeShared<RT> &shared, const
     if (threadIdx.x == 0) arrived = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
     if (arrived != splits - 1) return;
-    // The last arriver sums the splits in split order; the loads of a round are in flight together (the loop's staging
-    // registers are free by now), so the sum costs one or two round trips to the coherence point whatever the splits.
-    constexpr uint32_t kRound = RT == 1 ? 16u : RT == 2 ? 8u : 4u;
-#pragma unroll
-    for (int t = 0; t < RT; ++t)
-#pragma unroll
-      for (int v = 0; v < 4; ++v) acc[t][v] = 0.f;
-    for (uint32_t s0 = 0; s0 < splits; s0 += kRound) {
-      float part[kRound][RT][4];
-#pragma unroll
-      for (uint32_t s = 0; s < kRound; ++s) {
-        if (s0 + s < splits) {
-#pragma unroll
-          for (int t = 0; t < RT; ++t)
-#pragma unroll
-            for (int v = 0; v < 4; ++v)
-              part[s][t][v] = __hip_atomic_load(mineAt + size_t(s0 + s) * stride + (t * 4 + v) * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        } else {
-#pragma unroll
-          for (int t = 0; t < RT; ++t)
-#pragma unroll
-            for (int v = 0; v < 4; ++v) part[s][t][v] = 0.f;
-        }
-      }
-#pragma unroll
-      for (uint32_t s = 0; s < kRound; ++s)
-#pragma unroll
-        for (int t = 0; t < RT; ++t)
-#pragma unroll
-          for (int v = 0; v < 4; ++v) acc[t][v] += s0 + s < splits ? part[s][t][v] : 0.f;
-    }
+    orderedSum(mineAt, stride, splits);
     if (threadIdx.x == 0) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
   if (p.deferred_scale) {
@@ -1086,6 +1393,69 @@ SP_REGISTER_KERNEL("gguf_decode_mixed_m16_a", &gguf_decode_mixed<1>);
 SP_REGISTER_KERNEL("gguf_decode_mixed_m32_a", &gguf_decode_mixed<2>);
 SP_REGISTER_KERNEL("gguf_decode_mixed_m64_a", &gguf_decode_mixed<4>);
 
+// The fused q|k|v projection that also prepares the attention block (GGUF_EPILOGUE_QKV_PREPARE): one format, or a format
+// a segment as gguf_decode_mixed. Rows of one piece (up to 64).
+#define SP_QKV_PARAMETERS                                                                                                        \
+  const uint8_t *__restrict__ seg0, const uint8_t *__restrict__ seg1, const uint8_t *__restrict__ seg2,                          \
+      const uint8_t *__restrict__ table, void *__restrict__ out, float *__restrict__ partials, uint32_t *__restrict__ counters,  \
+      const uint16_t *__restrict__ query_norm, const uint16_t *__restrict__ key_norm, const float *__restrict__ rope_cos,       \
+      const float *__restrict__ rope_sin, _Float16 *__restrict__ queries, float *__restrict__ query_sums,                       \
+      const uint64_t *__restrict__ page_table, uint8_t *__restrict__ pool, GgufQkvParams qp
+template <uint32_t FMT, int RT> __global__ __launch_bounds__(256) void gguf_decode_qkv(SP_QKV_PARAMETERS) {
+  GgufDecodeParams p = qp.decode;
+  p.rows = min(p.rows, uint32_t(GGUF_MAXIMUM_ROWS));
+  const QkvPrepare prepare{query_norm, key_norm, rope_cos, rope_sin, queries, query_sums, page_table, pool, &qp.attention};
+  __shared__ DecodeShared<RT> shared;
+  decode_workgroup<FMT, RT, GGUF_EPILOGUE_QKV_PREPARE>(shared, seg0, seg1, seg2, table, out, nullptr, partials, counters, p, blockIdx.x,
+                                                       ChainPosition{}, &prepare);
+}
+template <int RT> __global__ __launch_bounds__(256) void gguf_decode_qkv_mixed(SP_QKV_PARAMETERS) {
+  constexpr uint32_t kGroupFloats = 4u * RT * 256u;
+  GgufDecodeParams p = qp.decode;
+  p.rows = min(p.rows, uint32_t(GGUF_MAXIMUM_ROWS));
+  const QkvPrepare prepare{query_norm, key_norm, rope_cos, rope_sin, queries, query_sums, page_table, pool, &qp.attention};
+  const uint32_t group = blockIdx.x / p.splits, split = blockIdx.x % p.splits;
+  uint32_t segment = 0, before = 0;
+#pragma unroll
+  for (uint32_t s = 0; s < 2u; ++s)
+    if (segment == s && group >= before + p.cols[s] / 64u) {
+      before += p.cols[s] / 64u;
+      segment = s + 1u;
+    }
+  const uint8_t *image = segment == 0 ? seg0 : segment == 1 ? seg1 : seg2;
+  auto of = [&](const uint32_t (&field)[3]) { return segment == 0 ? field[0] : segment == 1 ? field[1] : field[2]; };
+  const uint32_t format = of(p.formats);
+  GgufDecodeParams mine = p;
+  mine.cols[0] = of(p.cols);
+  mine.cols[1] = mine.cols[2] = 0;
+  mine.offset[0] = of(p.offset);
+  mine.units = mine.cols[0] / GGUF_TILE_COLUMNS;
+  mine.whole_groups = 0;
+  partials += size_t(before) * p.splits * kGroupFloats;
+  counters += before;
+  const uint32_t item = (group - before) * p.splits + split;
+  __shared__ DecodeShared<RT> shared;
+#define SP_QKV_FORMAT(F)                                                                                                          \
+  case F:                                                                                                                         \
+    decode_workgroup<F, RT, GGUF_EPILOGUE_QKV_PREPARE>(shared, image, image, image, table, out, nullptr, partials, counters, mine, item, \
+                                                       ChainPosition{}, &prepare);                                                \
+    break
+  switch (format) {
+    SP_QKV_FORMAT(GGUF_FMT_Q4K);
+    SP_QKV_FORMAT(GGUF_FMT_Q5K);
+    SP_QKV_FORMAT(GGUF_FMT_Q6K);
+    SP_QKV_FORMAT(GGUF_FMT_Q80);
+    SP_QKV_FORMAT(GGUF_FMT_IQ4XS);
+    SP_QKV_FORMAT(GGUF_FMT_IQ4NL);
+  default: break;
+  }
+#undef SP_QKV_FORMAT
+}
+#undef SP_QKV_PARAMETERS
+SP_REGISTER_KERNEL("gguf_decode_qkv_mixed_m16", &gguf_decode_qkv_mixed<1>);
+SP_REGISTER_KERNEL("gguf_decode_qkv_mixed_m32", &gguf_decode_qkv_mixed<2>);
+SP_REGISTER_KERNEL("gguf_decode_qkv_mixed_m64", &gguf_decode_qkv_mixed<4>);
+
 // A chain of up to four projections in one dispatch (GgufChainParams): link i's workgroups are items
 // link[i].first_item .. of the grid, in link order, so the device has started every workgroup of a link before any of
 // the next one's, and a workgroup that waits for the link before (ChainPosition) waits only for workgroups that are
@@ -1227,7 +1597,8 @@ SP_GGUF_MOE_DECODE("iq4nl", GGUF_FMT_IQ4NL);
   SP_REGISTER_KERNEL("gguf_decode_" fmt "_m" #rows "_r", &gguf_decode<FMT, RT, GGUF_EPILOGUE_RESIDUAL>); \
   SP_REGISTER_KERNEL("gguf_decode_" fmt "_m" #rows "_g", &gguf_decode<FMT, RT, GGUF_EPILOGUE_GATE_UP>);  \
   SP_REGISTER_KERNEL("gguf_decode_" fmt "_m" #rows "_gt", &gguf_decode<FMT, RT, GGUF_EPILOGUE_GATE_UP_TABLE>); \
-  SP_REGISTER_KERNEL("gguf_decode_" fmt "_m" #rows "_rn", &gguf_decode<FMT, RT, GGUF_EPILOGUE_RESIDUAL_NORM>)
+  SP_REGISTER_KERNEL("gguf_decode_" fmt "_m" #rows "_rn", &gguf_decode<FMT, RT, GGUF_EPILOGUE_RESIDUAL_NORM>);                             \
+  SP_REGISTER_KERNEL("gguf_decode_qkv_" fmt "_m" #rows, &gguf_decode_qkv<FMT, RT>)
 SP_GGUF_DECODE("q4k", GGUF_FMT_Q4K, 16, 1);
 SP_GGUF_DECODE("q4k", GGUF_FMT_Q4K, 32, 2);
 SP_GGUF_DECODE("q4k", GGUF_FMT_Q4K, 64, 4);

@@ -57,6 +57,13 @@ DenseVerify::DenseVerify(hip::Backend &backend, DenseDimensions d, uint32_t maxL
                               ops::LinearMatrix{d.ffn, d.hidden}, ops::LinearMatrix{d.hidden, d.ffn},
                               ops::LinearMatrix{d.vocabulary, d.hidden}})
     size.include(linear_.scratchSize(m, maxRows_));
+  // a q|k|v projection that prepares its attention block keeps partials whatever its plan's parts
+  for (uint32_t rows : {16u, 32u, 64u})
+    for (uint32_t format : {GGUF_FMT_Q4K, GGUF_FMT_Q6K})
+      for (bool several : {false, true})
+        if (!several || d.qkvWidth() % 64 == 0)
+          size.include(ops::Linear::attentionScratchSize(linear_.plan(
+              ops::LinearWorkload{{d.qkvWidth(), d.hidden}, std::min(rows, maxRows_), ops::LinearEpilogue::None, format, several})));
   scratch_.input = device(size.input, "linear table");
   scratch_.partials = device(size.partials, "linear partials");
   scratch_.counters = device(std::max<uint64_t>(size.counters, 4), "linear counters");
@@ -151,10 +158,17 @@ void DenseVerify::encodeLayer(hip::CommandGraph &graph, uint32_t layer, const op
   qkv.output = qkv_;
   qkv.scratch = scratch_;
   qkv.prepared = prepared;
-  linear_.add(graph, qkv, w.qkv, linear_.plan(w.qkv, rows));
+  const ops::LinearPlan qkvPlan = linear_.plan(w.qkv, rows);
   const ops::KvPages pages{pageTable_, kvPools_.at(layer), pageBytes_};
   ops::AttentionProjectionBuffers projection{qkv_, w.queryNorm, w.keyNorm, ropeCos_, ropeSin_};
-  ops::PagedAttention::addProjection(graph, plan, projection, attentionWorkspace_, pages);
+  const ops::LinearScratchSize fusedNeed = ops::Linear::attentionScratchSize(qkvPlan);
+  if (fusedPrepare_ && ops::PagedAttention::fusesProjection(plan, w.qkv, qkvPlan) &&
+      scratch_.partials.sizeBytes() >= fusedNeed.partials && scratch_.counters.sizeBytes() >= fusedNeed.counters) {
+    ops::PagedAttention::addFusedProjection(graph, linear_, qkv, w.qkv, qkvPlan, plan, projection, attentionWorkspace_, pages);
+  } else {
+    linear_.add(graph, qkv, w.qkv, qkvPlan);
+    ops::PagedAttention::addProjection(graph, plan, projection, attentionWorkspace_, pages);
+  }
   ops::PagedAttention::addAttention(graph, plan, attentionWorkspace_, treeRows_, pages, attention_, nextTable_);
   // The output projection adds the residual and, where its shape allows, norms the sum into the
   // gate/up pass's table; the down projection does the same for the layer (or head) after it.

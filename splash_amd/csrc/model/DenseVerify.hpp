@@ -100,6 +100,13 @@ public:
   // The results are those of the separate dispatches, bit for bit.
   void setChained(bool chained) noexcept { chained_ = chained; }
   [[nodiscard]] bool chained() const noexcept { return chained_; }
+  // A layer's q|k|v projection also prepares its attention block (ops::PagedAttention::addFusedProjection) where the
+  // kernels take the pair: off by default (the projection and the prepare kernel run one after the other). The results
+  // are the same bit for bit; on MI355X the one dispatch is the slower of the two at the 27B shape, since the workgroup
+  // that completes a head prepares its sixteen rows alone (four a wave, about 4 us of vector arithmetic), where the
+  // prepare kernel spreads them over 1280 workgroups.
+  void setFusedPrepare(bool fused) noexcept { fusedPrepare_ = fused; }
+  [[nodiscard]] bool fusedPrepare() const noexcept { return fusedPrepare_; }
   // Nonzero after a step in which a chained projection's wait for the one before it gave up: the step's results are
   // then not to be used. Reads the device's word (a copy of four bytes) and clears it.
   [[nodiscard]] uint32_t takeChainStatus();
@@ -122,7 +129,7 @@ private:
   // chained projections: the gate/up and down tables, each link's partials and counters, the chain's progress words
   hip::Buffer chainTables_[2], chainProgress_;
   ops::LinearScratch chainScratch_[GGUF_CHAIN_LINKS];
-  bool chained_ = false, encodedChains_ = false;
+  bool chained_ = false, encodedChains_ = false, fusedPrepare_ = false;
   void encodeChainedLayers(hip::CommandGraph &graph, const ops::AttentionPlan &plan, uint32_t rows);
   [[nodiscard]] bool chains(uint32_t rows) const noexcept;
   ops::AttentionWorkspace attentionWorkspace_;

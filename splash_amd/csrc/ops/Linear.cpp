@@ -334,6 +334,67 @@ void Linear::addChain(hip::CommandGraph &graph, std::vector<ChainedProjection> l
   graph.add("gguf_decode_chain_m" + std::to_string(storage), std::move(buffers), chain, {items, 1, 1}, {256, 1, 1});
 }
 
+bool Linear::preparesAttention(const Projection &p, const LinearPlan &plan, const AttentionParams &a) noexcept {
+  const LinearWorkload w = plan.workload();
+  const uint32_t D = a.head_dim;
+  if (w.epilogue != LinearEpilogue::None || plan.destination() != FloatOutput::BFloat16) return false;
+  if (rowPieces(w.rows) != 1 || plan.configuration().wholeGroups) return false;
+  if ((D != 64 && D != 128) || a.gated || a.int8_queries || !a.kv_heads) return false;
+  if (w.matrix.outputSize != (a.q_heads + 2 * a.kv_heads) * D || a.qkv_stride != w.matrix.outputSize) return false;
+  if (!a.sequences || a.sequences > ATTENTION_MAXIMUM_SEQUENCES) return false;
+  for (uint32_t s = 0; s < a.sequences; ++s)
+    if (uint64_t{a.sequence[s].first_row} + a.sequence[s].rows > w.rows) return false;
+  for (const QuantizedSegment &s : p.blocks().segments)
+    if (s.outputSize % D || s.columnOffset % D) return false;
+  return true;
+}
+
+LinearScratchSize Linear::attentionScratchSize(const LinearPlan &plan) noexcept {
+  // [part][workgroup][4 waves][row tile][4][64 lanes] fp32 sums, and a counter a head (at most one a workgroup)
+  const LinearWorkload w = plan.workload();
+  const uint64_t groups = groupsOf(w.matrix.outputSize, w.epilogue), pieceTiles = plan.storageRows() / GGUF_ROW_TILE;
+  LinearScratchSize size = plan.scratchSize();
+  size.partials = plan.configuration().splits * groups * kWavesAcross * pieceTiles * 256u * sizeof(float);
+  size.counters = groups * sizeof(uint32_t);
+  return size;
+}
+
+PreparedInput Linear::addWithAttention(hip::CommandGraph &graph, LinearBuffers b, const Projection &p, const LinearPlan &plan,
+                                       const AttentionPrepareBindings &attention) const {
+  const LinearWorkload w = plan.workload();
+  const AttentionParams &a = attention.params;
+  const hip::Buffer input = b.input, table = b.scratch.input, partials = b.scratch.partials, counters = b.scratch.counters;
+  const Resolved r = resolve(std::move(b), p, plan, nullptr);
+  if (!preparesAttention(p, plan, a)) throw std::invalid_argument("no fused kernel prepares this attention block from this projection");
+  const LinearScratchSize need = attentionScratchSize(plan);
+  requireBytes(partials, need.partials, "projection partials");
+  requireBytes(counters, need.counters, "projection counters");
+  const uint32_t rows = w.rows, D = a.head_dim;
+  if (a.normalize) {
+    requireBytes(attention.queryNorm, D * 2, "query norm weight");
+    requireBytes(attention.keyNorm, D * 2, "key norm weight");
+  }
+  if (a.rotary_pairs) {
+    requireBytes(attention.ropeCos, uint64_t{rows} * a.rotary_pairs * 4, "RoPE cosine table");
+    requireBytes(attention.ropeSin, uint64_t{rows} * a.rotary_pairs * 4, "RoPE sine table");
+  }
+  const uint64_t fused = uint64_t{a.sequences} * a.q_heads * 16;
+  requireBytes(attention.queries, fused * D * 2, "staged queries");
+  requireBytes(attention.querySums, fused * 4, "staged query sums");
+  if (!attention.pageTable || !attention.pool) throw std::invalid_argument("the fused projection stores into the layer's pages");
+  if (!r.prepared) addPrepare(graph, input, LinearScratch{table, {}, {}}, w.matrix.inputSize, rows);
+  const hip::Buffer &spare = table;
+  const std::string name = std::string("gguf_decode_qkv_") + (r.mixed ? "mixed" : p.blocks().segments.front().name()) + "_m" +
+                           std::to_string(plan.storageRows());
+  graph.add(name,
+            {r.buffers[0], r.buffers[1], r.buffers[2], r.buffers[3], r.buffers[4], partials, counters,
+             a.normalize ? attention.queryNorm : spare, a.normalize ? attention.keyNorm : spare,
+             a.rotary_pairs ? attention.ropeCos : spare, a.rotary_pairs ? attention.ropeSin : spare, attention.queries,
+             attention.querySums, attention.pageTable, attention.pool},
+            GgufQkvParams{r.params, a}, {r.items, 1, 1}, {256, 1, 1});
+  return r.after;
+}
+
 void Linear::addProjection(hip::CommandGraph &graph, hip::Buffer input, const Projection &projection, hip::Buffer output,
                            uint32_t rows, LinearScratch scratch) const {
   LinearBuffers buffers;

@@ -5,6 +5,8 @@
 // before any dispatch is added; producers and consumers hand the prepared activation table along
 // as PreparedInput.
 #pragma once
+#include "abi/PagedAttention.h"
+
 #include "abi/Gguf.h"
 #include "hip/Backend.hpp"
 #include "ops/Weights.hpp"
@@ -172,6 +174,13 @@ struct ChainedProjection final {
   const Projection *gate = nullptr;
 };
 
+// What the fused q|k|v projection binds of its attention block (kernels gguf_decode_qkv_*): attention_q8_qkv's buffers
+// after the packed rows, in that kernel's order, and its parameters.
+struct AttentionPrepareBindings final {
+  hip::Buffer queryNorm, keyNorm, ropeCos, ropeSin, queries, querySums, pageTable, pool;
+  AttentionParams params{};
+};
+
 class Linear final {
 public:
   explicit Linear(const sp_device_info &device) noexcept;
@@ -199,6 +208,16 @@ public:
   // `progress` (GGUF_CHAIN_PROGRESS_WORDS words, zero before the first dispatch) is the chain's; its last word reads
   // nonzero after a dispatch in which a wait gave up.
   void addChain(hip::CommandGraph &graph, std::vector<ChainedProjection> links, const hip::Buffer &progress) const;
+  // The q|k|v projection of an attention block with the block's head norms, RoPE, query staging and cache store as its
+  // epilogue (GGUF_EPILOGUE_QKV_PREPARE), in place of the projection and attention_q8_qkv after it: the same packed
+  // rows, staged queries and cache bytes. preparesAttention: whether the kernels take the pair (a plain bf16 plan of one
+  // piece of rows whose workgroups all take a part of K, heads of 64 or 128 dimensions that lie whole in the
+  // projection's segments, fp16 queries, no gates). The dispatch keeps partials and counters whatever the plan's parts
+  // (attentionScratchSize).
+  [[nodiscard]] static bool preparesAttention(const Projection &projection, const LinearPlan &plan, const AttentionParams &attention) noexcept;
+  [[nodiscard]] static LinearScratchSize attentionScratchSize(const LinearPlan &plan) noexcept;
+  PreparedInput addWithAttention(hip::CommandGraph &graph, LinearBuffers buffers, const Projection &projection,
+                                 const LinearPlan &plan, const AttentionPrepareBindings &attention) const;
   void addProjection(hip::CommandGraph &graph, hip::Buffer input, const Projection &projection, hip::Buffer output,
                      uint32_t rows, LinearScratch scratch) const;
   void addResidualProjection(hip::CommandGraph &graph, hip::Buffer input, const Projection &projection,

@@ -115,6 +115,24 @@ void PagedAttention::addProjection(hip::CommandGraph &graph, const AttentionPlan
             {g.headDimension, 1, 1});
 }
 
+bool PagedAttention::fusesProjection(const AttentionPlan &plan, const Projection &projection, const LinearPlan &linearPlan) noexcept {
+  return linearPlan.workload().rows == totalRows(plan.sequences()) && Linear::preparesAttention(projection, linearPlan, plan.params(0));
+}
+
+PreparedInput PagedAttention::addFusedProjection(hip::CommandGraph &graph, const Linear &linear, LinearBuffers linearBuffers,
+                                                 const Projection &projection, const LinearPlan &linearPlan, const AttentionPlan &plan,
+                                                 const AttentionProjectionBuffers &b, const AttentionWorkspace &w, const KvPages &pages) {
+  if (!fusesProjection(plan, projection, linearPlan)) throw std::invalid_argument("no fused kernel prepares this attention block from this projection");
+  if (!b.qkv.sameView(linearBuffers.output)) throw std::invalid_argument("the fused projection writes the block's packed rows");
+  const AttentionWorkspaceSize need = plan.workspace();
+  requireBytes(w.queries, need.queries, "staged queries");
+  requireBytes(w.querySums, need.querySums, "staged query sums");
+  requirePages(plan, pages);
+  return linear.addWithAttention(graph, std::move(linearBuffers), projection, linearPlan,
+                                 AttentionPrepareBindings{b.queryNorm, b.keyNorm, b.ropeCos, b.ropeSin, w.queries, w.querySums,
+                                                          pages.pageTable, pages.pool, plan.params(pages.pageBytes)});
+}
+
 void PagedAttention::addAttention(hip::CommandGraph &graph, const AttentionPlan &plan, const AttentionWorkspace &w,
                                   const hip::Buffer &treeRows, const KvPages &pages, const hip::Buffer &output,
                                   const hip::Buffer &outputTable, const hip::Buffer &packed) {

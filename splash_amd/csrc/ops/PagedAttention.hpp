@@ -6,6 +6,7 @@
 #pragma once
 #include "abi/PagedAttention.h"
 #include "hip/Backend.hpp"
+#include "ops/Linear.hpp"
 
 #include <cstdint>
 #include <vector>
@@ -100,6 +101,15 @@ public:
   // q/k norm + RoPE + query staging + INT8 store of the block's K and V (PagedAttention.cpp:441-464).
   static void addProjection(hip::CommandGraph &graph, const AttentionPlan &plan, const AttentionProjectionBuffers &buffers,
                             const AttentionWorkspace &workspace, const KvPages &pages);
+  // The q|k|v projection and addProjection's work in ONE dispatch (Linear::addWithAttention), where the reference runs the
+  // projection and its prepare kernel one after the other (QwenTarget.cpp:457-470): `projection` writes the packed
+  // rows into buffers.qkv (which is `linear.output`) and the last workgroup of each head prepares it. The same packed
+  // rows, staged queries and cache bytes as the two dispatches. fusesProjection: whether the kernels take the pair.
+  [[nodiscard]] static bool fusesProjection(const AttentionPlan &plan, const Projection &projection, const LinearPlan &linearPlan) noexcept;
+  static PreparedInput addFusedProjection(hip::CommandGraph &graph, const Linear &linear, LinearBuffers linearBuffers,
+                                          const Projection &projection, const LinearPlan &linearPlan, const AttentionPlan &plan,
+                                          const AttentionProjectionBuffers &buffers, const AttentionWorkspace &workspace,
+                                          const KvPages &pages);
   // Split + reduce (PagedAttention.cpp:466-607): output bf16 [packed rows][q heads * D].
   // outputTable (optional): the reduce also writes the rows as the activation table of the
   // projection that follows (gguf_table_bytes(q heads * D, rows)), which then needs no table pass.

@@ -298,6 +298,25 @@ class PagedAttention:
         graph._keep.extend([plan, qkv, workspace, pages, query_norm, key_norm, rope_cos, rope_sin])
 
     @staticmethod
+    def fuses_projection(plan, projection, linear_plan):
+        """Whether the q|k|v projection of this plan can prepare the attention block from its epilogue."""
+        return bool(lib.spo_attention_fuses_projection(plan.handle, projection.handle, ctypes.byref(linear_plan)))
+
+    @staticmethod
+    def add_fused_projection(graph, linear, attention, workspace, pages, query_norm=None, key_norm=None, rope_cos=None, rope_sin=None,
+                             **qkv):
+        """The q|k|v projection (`qkv`: a link as Linear.add_link takes it, whose output is the block's packed rows) and
+        add_projection's work for the block of the plan `attention` in one dispatch."""
+        h = lambda b: b.handle if b is not None else None
+        slot = nat.ChainLink()
+        linear._fill_link(slot, qkv)
+        check(lib.spo_attention_add_fused_projection(linear.handle, graph.handle, ctypes.byref(slot), attention.handle, h(query_norm),
+                                                     h(key_norm), h(rope_cos), h(rope_sin), workspace.queries.handle,
+                                                     workspace.query_sums.handle, pages.table.handle, pages.pool.handle,
+                                                     pages.page_bytes))
+        graph._keep.extend([attention, workspace, pages, query_norm, key_norm, rope_cos, rope_sin, *qkv.values()])
+
+    @staticmethod
     def add_attention(graph, plan, workspace, tree_rows, pages, output, output_table=None, packed_qkv=None):
         check(lib.spo_attention_add_attention(graph.handle, plan.handle, workspace.queries.handle, workspace.query_sums.handle,
                                               workspace.partials.handle, workspace.partial_sums.handle, tree_rows.handle,

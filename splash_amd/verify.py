@@ -111,6 +111,11 @@ class DenseVerify:
         default): the results are the same bit for bit."""
         check(lib.spo_dense_verify_set_chained(self.handle, int(bool(chained))))
 
+    def set_fused_prepare(self, fused):
+        """Whether a layer's q|k|v projection also prepares its attention block where the kernels take the pair (off by
+        default): the results are the same bit for bit."""
+        check(lib.spo_dense_verify_set_fused_prepare(self.handle, int(bool(fused))))
+
     def set_candidate_children(self, ids, probabilities, draws, child_uniforms):
         """The sampled rows' candidate children, by packed row: ids uint32 [rows][16], probabilities fp32 [rows][16], draws
         bytes [rows][4] (0xFF past a row's drawn children), child_uniforms fp32 [rows][4]."""

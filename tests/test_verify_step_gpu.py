@@ -247,3 +247,37 @@ def test_chained_projections_change_nothing(backend, lanes_rows):
         assert np.array_equal(logits, plain[0][0]) and np.array_equal(hidden, plain[0][1])
         for got, want in zip(results, plain[0][2]):
             assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("lanes_rows", [[16], [7, 16, 3]])
+def test_the_fused_prepare_changes_nothing(backend, lanes_rows):
+    """A step whose q|k|v projections prepare their attention blocks themselves (off by default) gives the logits, the
+    hidden rows, the cache and the results of the step that runs the prepare kernel after each projection, bit for bit,
+    with a dispatch a layer fewer."""
+    print(f"case fused prepare step lanes={lanes_rows}", flush=True)
+    model = DenseModel(seed=16, hidden=1024, q_heads=16, kv_heads=8, head_dim=64, ffn=3072, vocabulary=32000, layers=4)
+    rng = np.random.default_rng(9)
+    contexts = [250 + 111 * i for i in range(len(lanes_rows))]
+    gpu = model.build_gpu(backend, max_lanes=len(lanes_rows), context_tokens=[c + 16 for c in contexts])
+    model.seed_context(gpu, None, rng)
+    lanes = [verify.Lane(rows, committed, table_first=first) for rows, committed, first in zip(lanes_rows, contexts, model.table_first)]
+    total = sum(lanes_rows)
+    gpu.set_block(lanes, rng.integers(0, 32000, total).astype(np.uint32))
+
+    def run(fused):
+        gpu.set_fused_prepare(fused)
+        graph = gpu.encode(lanes, commit=False)
+        outcomes = []
+        for _ in range(2):
+            backend.run(graph)
+            outcomes.append((gpu.buffer(verify.LOGITS).download(np.float32, total * 32000).copy(),
+                             gpu.buffer(verify.HIDDEN, 0).download(np.uint16, total * 1024).copy(),
+                             np.concatenate([gpu.buffer(verify.KV_POOL, layer).download(np.uint8) for layer in range(4)]), gpu.results(lanes)))
+        return len(graph), outcomes
+    fused_dispatches, fused = run(True)
+    plain_dispatches, plain = run(False)
+    assert fused_dispatches == plain_dispatches - 4
+    for logits, hidden, pool, results in plain[1:] + fused:
+        assert np.array_equal(logits, plain[0][0]) and np.array_equal(hidden, plain[0][1]) and np.array_equal(pool, plain[0][2])
+        for got, want in zip(results, plain[0][3]):
+            assert np.array_equal(got, want)
