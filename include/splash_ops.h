@@ -64,6 +64,11 @@ typedef struct spo_linear_plan {
   uint32_t splits, whole_groups; /* LinearConfig: K partitions, and the leading workgroups that take K whole */
   uint32_t storage_rows;    /* LinearPlan::storageRows */
   uint32_t float32;         /* LinearPlan::destination */
+  /* LinearTile: 0 the register rule (exact 128 + code operands, one fp32 multiply-add a group;
+   * linear_gguf_sgmatrix.metal:140-288), 1 the staged rule (weights decoded with fp32 group coefficients and rounded
+   * once to half, products accumulated in fp32; kernels/common/gguf_staged.h:12-66, gguf_linear.metal:120-140): plain
+   * and residual plans of one format, set with spo_linear_plan_with. */
+  uint32_t tile, reserved;
   uint64_t scratch_input, scratch_partials, scratch_counters; /* LinearPlan::scratchSize */
 } spo_linear_plan;
 /* Linear::plan(projection, rows, epilogue) (Linear.hpp:307-309): the device's plan. */

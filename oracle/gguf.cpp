@@ -312,6 +312,41 @@ int orc_quantize_rows(uint32_t fmt, const float *values, uint32_t rows, uint32_t
   return 0;
 }
 
+int orc_gemm_staged(uint32_t fmt, const uint8_t *native, const uint16_t *x, uint32_t M, uint32_t K, uint32_t N,
+                    double *exact, double *bound, float *staged, double *accumulation, int threads) {
+  const uint64_t rb = orc_row_bytes(fmt, K);
+  if (!rb) return -1;
+  std::vector<float> xf(size_t(M) * K);
+  for (size_t i = 0; i < xf.size(); ++i) xf[i] = bf2f(x[i]);
+  parallelFor(N, threads, [&](uint32_t lo, uint32_t hi) {
+    std::vector<float> w(K), w16(K);
+    for (uint32_t n = lo; n < hi; ++n) {
+      const uint8_t *row = native + n * rb;
+      for (uint32_t g = 0; g < K / 32; ++g) groupValues(fmt, row, g, w.data() + 32 * g);
+      for (uint32_t k = 0; k < K; ++k) w16[k] = h2f(f2h(w[k]));   // gguf_staged.h:12-19: rounded once to half
+      for (uint32_t m = 0; m < M; ++m) {
+        const float *xr = xf.data() + size_t(m) * K;
+        // GgufFormatReference.hpp:717-742: dot and projectionBound(staged)
+        double value = 0, magnitude = 0, inputs = 0, largest = 0, rounded = 0;
+        for (uint32_t k = 0; k < K; ++k) {
+          value += double(xr[k]) * w[k];
+          magnitude += std::fabs(double(xr[k]) * w[k]);
+          inputs += std::fabs(xr[k]);
+          largest = std::max(largest, double(std::fabs(w[k])));
+          rounded += double(xr[k]) * w16[k];
+        }
+        const size_t at = size_t(m) * N + n;
+        const double chain = std::ldexp(inputs * largest, -16);
+        if (exact) exact[at] = value;
+        if (bound) bound[at] = chain + std::ldexp(magnitude, -11) + std::ldexp(inputs, -25);
+        if (staged) staged[at] = float(rounded);
+        if (accumulation) accumulation[at] = chain;
+      }
+    }
+  });
+  return 0;
+}
+
 int orc_gemm(uint32_t fmt, const uint8_t *native, const uint16_t *x, uint32_t M, uint32_t K, uint32_t N,
              double *exact, double *bound, float *chain, int threads) {
   const uint64_t rb = orc_row_bytes(fmt, K);

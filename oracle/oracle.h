@@ -72,6 +72,15 @@ int orc_quantize_rows(uint32_t fmt, const float *values, uint32_t rows, uint32_t
 // Any of the three outputs may be NULL. threads <= 0 uses every core.
 int orc_gemm(uint32_t fmt, const uint8_t *native, const uint16_t *x, uint32_t M, uint32_t K, uint32_t N,
              double *exact, double *bound, float *chain, int threads);
+// The staged tile's projection (kernels/common/gguf_staged.h:12-66: every weight decoded with fp32 group coefficients
+// and rounded once to half; gguf_linear.metal:1-12: fp32 accumulation of its products with the bf16 inputs).
+// exact:  fp64 dot product with the weights' fp32 values (what the reference's test measures from).
+// bound:  projectionBound(staged) (GgufFormatReference.hpp:739-742): 2^-16 sum|x| max|w| + 2^-11 sum|x w| + 2^-25 sum|x|.
+// staged: the fp64 dot product with the weights rounded to half, rounded to fp32: what the tile computes but for the
+//         order and roundings of its fp32 accumulation, which 2^-16 sum|x| max|w| (accumulation) bounds.
+// Pinned by the reference's own dot and projectionBound (oracle/_ref) and numpy's float16 rounding of orc_dequant_rows.
+int orc_gemm_staged(uint32_t fmt, const uint8_t *native, const uint16_t *x, uint32_t M, uint32_t K, uint32_t N,
+                    double *exact, double *bound, float *staged, double *accumulation, int threads);
 // Epilogues on fp32 sums (kernels/common/gguf_tile.h:10-16, gguf_linear.metal:34-71).
 uint16_t orc_epilogue_plain(float v);
 uint16_t orc_epilogue_residual(float v, uint16_t residual);

@@ -50,6 +50,13 @@ void ref_dot_bound(const float *x, const float *w, uint32_t K, double *value, do
   *bound = projectionBound(d, false);
 }
 
+// The staged tile's bound of the same pair.
+void ref_dot_bound_staged(const float *x, const float *w, uint32_t K, double *value, double *bound) {
+  const Dot d = dot(x, w, K);
+  *value = d.value;
+  *bound = projectionBound(d, true);
+}
+
 float ref_kv_scale(float maximum) { return splash::kv::reference_detail::storedScale(maximum); }
 int ref_kv_code(float value, float maximum) { return splash::kv::reference_detail::quantize(value, maximum); }
 

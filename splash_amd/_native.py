@@ -71,7 +71,7 @@ class MemoryStats(ctypes.Structure):
 
 class LinearPlan(ctypes.Structure):
     _fields_ = [("rows", c_u32), ("epilogue", c_u32), ("splits", c_u32), ("whole_groups", c_u32), ("storage_rows", c_u32),
-                ("float32", c_u32), ("scratch_input", c_u64), ("scratch_partials", c_u64), ("scratch_counters", c_u64)]
+                ("float32", c_u32), ("tile", c_u32), ("reserved", c_u32), ("scratch_input", c_u64), ("scratch_partials", c_u64), ("scratch_counters", c_u64)]
 
 
 class ChainLink(ctypes.Structure):

@@ -482,6 +482,70 @@ __device__ __forceinline__ void accumulate_record(const Record<FMT> &rec, const 
   }
 }
 
+// The staged rule (the reference's staged tile, kernels/common/gguf_staged.h:12-66: every weight decoded with fp32 group
+// coefficients and rounded once to half, products with the bf16 inputs accumulated in fp32): a group's eight values of
+// this lane as halves, each split into the bf16 that holds its leading eight significant bits and the bf16 that holds
+// the rest (a half has eleven), so that two bf16 MFMAs multiply the inputs by the half exactly; the constant terms ride
+// in the values, so the row sums stay unread.
+__device__ __forceinline__ void staged_operands(const float (&value)[8], bf16x8 &high, bf16x8 &low) {
+  uint32_t highWords[4], lowWords[4];
+#pragma unroll
+  for (uint32_t e = 0; e < 8; e += 2) {
+    uint32_t h[2], l[2];
+#pragma unroll
+    for (uint32_t i = 0; i < 2; ++i) {
+      const float rounded = float(_Float16(value[e + i]));                    // the staged tile's half
+      const uint32_t bits = __float_as_uint(rounded), lead = bits & 0xFFFF0000u;  // a bf16: sign, exponent, seven fraction bits
+      h[i] = lead >> 16;
+      l[i] = __float_as_uint(rounded - __uint_as_float(lead)) >> 16;           // at most three significant bits: a bf16 holds them
+    }
+    highWords[e / 2] = h[0] | (h[1] << 16);
+    lowWords[e / 2] = l[0] | (l[1] << 16);
+  }
+  high = as_bf16x8(make_uint4(highWords[0], highWords[1], highWords[2], highWords[3]));
+  low = as_bf16x8(make_uint4(lowWords[0], lowWords[1], lowWords[2], lowWords[3]));
+}
+template <uint32_t FMT, int RT>
+__device__ __forceinline__ void accumulate_record_staged(const Record<FMT> &rec, const uint4 (*a)[8][64], f32x4 (&acc)[RT], uint32_t lane,
+                                                         uint32_t kq) {
+  uint4 ops[8];
+  record_operands(rec, ops);
+  Q4KScales sc{};
+  float d6 = 0.f;
+  if constexpr (FMT == GGUF_FMT_Q4K || FMT == GGUF_FMT_Q5K) sc = q4k_scales(rec.meta);
+  if constexpr (FMT == GGUF_FMT_Q6K) d6 = half_bits_to_float(rec.d);
+#pragma unroll
+  for (uint32_t g = 0; g < 8; ++g) {
+    const uint32_t regs[4] = {ops[g].x, ops[g].y, ops[g].z, ops[g].w};
+    float value[8];
+    // the fp32 values of gguf_dequant, each exact or rounded once
+    if constexpr (FMT == GGUF_FMT_Q80 || FMT == GGUF_FMT_IQ4XS || FMT == GGUF_FMT_IQ4NL) {
+      const float d = group_scale(rec, g);
+#pragma unroll
+      for (uint32_t e = 0; e < 8; ++e) value[e] = d * (bf16_bits_to_float((regs[e >> 1] >> (16u * (e & 1u))) & 0xFFFFu) - 128.f);
+    } else if constexpr (FMT == GGUF_FMT_Q4K || FMT == GGUF_FMT_Q5K) {
+      const float s = sc.d * byte_of(g < 4 ? sc.sc_lo : sc.sc_hi, g & 3u);
+      const float m = -(sc.dmin * byte_of(g < 4 ? sc.mn_lo : sc.mn_hi, g & 3u));
+#pragma unroll
+      for (uint32_t e = 0; e < 8; ++e)
+        value[e] = __fmaf_rn(s, float(operand_code(regs[e >> 1], e & 1u) & (FMT == GGUF_FMT_Q5K ? 0x1Fu : 0xFu)), m);
+    } else {
+#pragma unroll
+      for (uint32_t e = 0; e < 8; ++e)
+        value[e] = (d6 * q6_scale(rec.scales, 2u * g + (e >> 2))) * float(int(operand_code(regs[e >> 1], e & 1u) & 0x3Fu) - 32);
+    }
+    bf16x8 high, low;
+    staged_operands(value, high, low);
+#pragma unroll
+    for (int t = 0; t < RT; ++t) {
+      const bf16x8 rows = as_bf16x8(a[t][g][lane]);
+      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(rows, high, acc[t], 0, 0, 0);
+      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(rows, low, acc[t], 0, 0, 0);
+    }
+  }
+  (void)kq;
+}
+
 // Work split: a wave owns one column tile over the workgroup's K range; the four waves of a
 // workgroup walk that range in step and share its activations through LDS. Unit u of a dispatch
 // is tile u of its concatenated segments; of a gate/up pair, unit 2 j is gate tile j and unit
@@ -749,7 +813,7 @@ __device__ __forceinline__ void qkv_clear_rows(const QkvHead &head, const QkvPre
     }
 }
 
-template <uint32_t FMT, int RT, uint32_t EP, bool Chain = false>
+template <uint32_t FMT, int RT, uint32_t EP, bool Chain = false, bool Staged = false>
 __device__ __forceinline__ void decode_workgroup(DecodeShared<RT> &shared, const uint8_t *__restrict__ seg0,
                                                  const uint8_t *__restrict__ seg1, const uint8_t *__restrict__ seg2,
                                                  const uint8_t *__restrict__ table, void *__restrict__ out,
@@ -963,7 +1027,10 @@ __device__ __forceinline__ void decode_workgroup(DecodeShared<RT> &shared, const
           (&ldsSums[buffer][0][0][0])[sumSlot[q]] = kPairSums ? stage[u].sum[q] + stage[u].second[q] : stage[u].sum[q];
         __syncthreads();
         issue(stage[(u + kStages - 1) % kStages]);
-        if (now < count) accumulate_record<FMT, RT>(stage[u].rec, ldsA[buffer], ldsSums[buffer], acc, lane, kq);
+        if (now < count) {
+          if constexpr (Staged) accumulate_record_staged<FMT, RT>(stage[u].rec, ldsA[buffer], acc, lane, kq);
+          else accumulate_record<FMT, RT>(stage[u].rec, ldsA[buffer], ldsSums[buffer], acc, lane, kq);
+        }
       }
     }
   }
@@ -1300,7 +1367,7 @@ __device__ __forceinline__ void decode_workgroup(DecodeShared<RT> &shared, const
   }
 }
 
-template <uint32_t FMT, int RT, uint32_t EP>
+template <uint32_t FMT, int RT, uint32_t EP, bool Staged = false>
 __global__ __launch_bounds__(256) void gguf_decode(const uint8_t *__restrict__ seg0, const uint8_t *__restrict__ seg1,
                                                    const uint8_t *__restrict__ seg2, const uint8_t *__restrict__ table,
                                                    void *__restrict__ out, const uint16_t *__restrict__ residual,
@@ -1322,7 +1389,7 @@ __global__ __launch_bounds__(256) void gguf_decode(const uint8_t *__restrict__ s
   }
   p.rows = min(p.rows, uint32_t(GGUF_MAXIMUM_ROWS));
   __shared__ DecodeShared<RT> shared;
-  decode_workgroup<FMT, RT, EP>(shared, seg0, seg1, seg2, table, out, residual, partials, counters, p, blockIdx.x);
+  decode_workgroup<FMT, RT, EP, false, Staged>(shared, seg0, seg1, seg2, table, out, residual, partials, counters, p, blockIdx.x);
 }
 
 // Segments of different formats in one dispatch (the reference's fused projection takes a format per segment,
@@ -1598,7 +1665,10 @@ SP_GGUF_MOE_DECODE("iq4nl", GGUF_FMT_IQ4NL);
   SP_REGISTER_KERNEL("gguf_decode_" fmt "_m" #rows "_g", &gguf_decode<FMT, RT, GGUF_EPILOGUE_GATE_UP>);  \
   SP_REGISTER_KERNEL("gguf_decode_" fmt "_m" #rows "_gt", &gguf_decode<FMT, RT, GGUF_EPILOGUE_GATE_UP_TABLE>); \
   SP_REGISTER_KERNEL("gguf_decode_" fmt "_m" #rows "_rn", &gguf_decode<FMT, RT, GGUF_EPILOGUE_RESIDUAL_NORM>);                             \
-  SP_REGISTER_KERNEL("gguf_decode_qkv_" fmt "_m" #rows, &gguf_decode_qkv<FMT, RT>)
+  SP_REGISTER_KERNEL("gguf_decode_qkv_" fmt "_m" #rows, &gguf_decode_qkv<FMT, RT>);                     \
+  SP_REGISTER_KERNEL("gguf_staged_" fmt "_m" #rows "_a", &gguf_decode<FMT, RT, GGUF_EPILOGUE_PLAIN, true>); \
+  SP_REGISTER_KERNEL("gguf_staged_" fmt "_m" #rows "_a_f32", &gguf_decode<FMT, RT, GGUF_EPILOGUE_PLAIN_F32, true>); \
+  SP_REGISTER_KERNEL("gguf_staged_" fmt "_m" #rows "_r", &gguf_decode<FMT, RT, GGUF_EPILOGUE_RESIDUAL, true>)
 SP_GGUF_DECODE("q4k", GGUF_FMT_Q4K, 16, 1);
 SP_GGUF_DECODE("q4k", GGUF_FMT_Q4K, 32, 2);
 SP_GGUF_DECODE("q4k", GGUF_FMT_Q4K, 64, 4);

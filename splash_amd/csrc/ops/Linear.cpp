@@ -78,6 +78,9 @@ void LinearPlan::requireConfiguration() const {
   if (workload_.severalFormats &&
       (workload_.epilogue != LinearEpilogue::None || destination_ != FloatOutput::BFloat16 || c.wholeGroups || n % 64))
     throw std::invalid_argument("segments of several formats take a plain bf16 plan whose workgroups all partition K");
+  if (c.tile == LinearTile::GgufStaged &&
+      (workload_.severalFormats || (workload_.epilogue != LinearEpilogue::None && workload_.epilogue != LinearEpilogue::Residual)))
+    throw std::invalid_argument("the staged rule takes plain and residual plans of one format");
 }
 
 LinearScratchSize LinearPlan::scratchSize() const noexcept {
@@ -258,8 +261,9 @@ Linear::Resolved Linear::resolve(LinearBuffers b, const Projection &p, const Lin
   params.deferred_scale = prepared && b.prepared.layout == LinearInput::TableUnscaled;
   // Unused bindings still name a buffer: the table stands in for them.
   const hip::Buffer &spare = b.scratch.input;
-  const std::string name = std::string("gguf_decode_") + (mixed ? "mixed" : segments.front().name()) + "_m" + std::to_string(plan.storageRows()) +
-                           epilogueSuffix(w.epilogue, plan.destination(), writesTable);
+  const bool staged = c.tile == LinearTile::GgufStaged;
+  const std::string name = std::string(staged ? "gguf_staged_" : "gguf_decode_") + (mixed ? "mixed" : segments.front().name()) + "_m" +
+                           std::to_string(plan.storageRows()) + epilogueSuffix(w.epilogue, plan.destination(), writesTable);
   if (norms) {
     images[1] = b.normWeight;
     images[2] = b.nextTable;
@@ -300,6 +304,7 @@ void Linear::addChain(hip::CommandGraph &graph, std::vector<ChainedProjection> l
     if (!link.projection) throw std::invalid_argument("a chain link names its projection");
     if (link.plan.storageRows() != storage || rowPieces(link.plan.workload().rows) != 1)
       throw std::invalid_argument("a chain's projections share one tile height of up to 64 rows");
+    if (link.plan.configuration().tile != LinearTile::GgufMfma) throw std::invalid_argument("chained projections run the register rule");
     resolved.push_back(resolve(link.buffers, *link.projection, link.plan, link.gate));
     const Resolved &r = resolved.back();
     if (!r.prepared) throw std::invalid_argument("a chained projection reads a table that is already there or that the link before it writes");
@@ -338,7 +343,7 @@ bool Linear::preparesAttention(const Projection &p, const LinearPlan &plan, cons
   const LinearWorkload w = plan.workload();
   const uint32_t D = a.head_dim;
   if (w.epilogue != LinearEpilogue::None || plan.destination() != FloatOutput::BFloat16) return false;
-  if (rowPieces(w.rows) != 1 || plan.configuration().wholeGroups) return false;
+  if (rowPieces(w.rows) != 1 || plan.configuration().wholeGroups || plan.configuration().tile != LinearTile::GgufMfma) return false;
   if ((D != 64 && D != 128) || a.gated || a.int8_queries || !a.kv_heads) return false;
   if (w.matrix.outputSize != (a.q_heads + 2 * a.kv_heads) * D || a.qkv_stride != w.matrix.outputSize) return false;
   if (!a.sequences || a.sequences > ATTENTION_MAXIMUM_SEQUENCES) return false;

@@ -31,8 +31,11 @@ struct LinearMatrix final {
 // projection after it (the reference's residual projections feed a norm_rms_table16 dispatch; here
 // the projection's own workgroups write the table once every column group's sums of squares are in).
 enum class LinearEpilogue : uint8_t { None, Residual, GateUp, ResidualNorm };
-// One tile: 16-column MFMA tiles, two per wave, 16/32/64 rows.
-enum class LinearTile : uint8_t { GgufMfma };
+// 16-column MFMA tiles of 16/32/64 rows under one of two arithmetic rules: GgufMfma, the register rule (exact operands
+// 128 + code, one fp32 multiply-add a group; the reference's Apple9 register tile), and GgufStaged, the staged rule
+// (every weight decoded with fp32 group coefficients and rounded once to half, the products accumulated in fp32; the
+// reference's staged tile, kernels/common/gguf_staged.h:12-66), which takes plain and residual plans of one format.
+enum class LinearTile : uint8_t { GgufMfma, GgufStaged };
 inline constexpr uint32_t kMaximumDecodeTileRows = GGUF_MAXIMUM_ROWS;
 // A dispatch of more rows runs pieces of kMaximumDecodeTileRows rows side by side.
 inline constexpr uint32_t kMaximumDispatchRows = GGUF_MAXIMUM_DISPATCH_ROWS;

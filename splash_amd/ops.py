@@ -106,14 +106,17 @@ class Linear:
         except Exception:
             pass
 
-    def plan(self, projection, rows, epilogue=EPILOGUE_NONE, splits=None, whole_groups=None):
+    def plan(self, projection, rows, epilogue=EPILOGUE_NONE, splits=None, whole_groups=None, staged=False):
+        """staged: the plan runs the staged rule (weights rounded once to half, products accumulated in fp32) instead of
+        the register rule."""
         p = nat.LinearPlan()
         check(lib.spo_linear_plan_for(self.handle, projection.handle, rows, epilogue, ctypes.byref(p)))
-        if splits is not None or whole_groups is not None:
+        if splits is not None or whole_groups is not None or staged:
             if splits is not None:
                 p.splits = splits
             if whole_groups is not None:
                 p.whole_groups = whole_groups
+            p.tile = 1 if staged else 0
             check(lib.spo_linear_plan_with(projection.handle, ctypes.byref(p)))
         return p
 

@@ -109,6 +109,19 @@ def gemm(fmt, native, x_bf16, N, want=("exact", "bound", "chain"), threads=0):
     return out
 
 
+def gemm_staged(fmt, native, x_bf16, N, threads=0):
+    """The staged tile's projection. Returns dict of exact (f64), bound (f64: the reference's staged projectionBound),
+    staged (f32: the fp64 dot with half-rounded weights) and accumulation (f64: the bound of the fp32 accumulation alone),
+    each [M][N]."""
+    x = np.ascontiguousarray(x_bf16, dtype=np.uint16)
+    M, K = x.shape
+    exact, bound = np.empty((M, N), dtype=np.float64), np.empty((M, N), dtype=np.float64)
+    staged, accumulation = np.empty((M, N), dtype=np.float32), np.empty((M, N), dtype=np.float64)
+    assert lib.orc_gemm_staged(c_u32(fmt), _p(native, u8p), _p(x, u16p), c_u32(M), c_u32(K), c_u32(N), _p(exact, f64p),
+                               _p(bound, f64p), _p(staged, f32p), _p(accumulation, f64p), c_int(threads)) == 0
+    return dict(exact=exact, bound=bound, staged=staged, accumulation=accumulation)
+
+
 def rms_norm(x_bf16, w_bf16):
     x = np.ascontiguousarray(x_bf16, dtype=np.uint16)
     w = np.ascontiguousarray(w_bf16, dtype=np.uint16)

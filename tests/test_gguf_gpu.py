@@ -54,12 +54,12 @@ def ulp_key(bits):
 
 
 def run_projection(backend, linear, fmt, native_segments, K, x_bits, epilogue=ops.EPILOGUE_NONE, float32=False,
-                   residual_bits=None, gate_native=None, splits=None, whole_groups=None):
+                   residual_bits=None, gate_native=None, splits=None, whole_groups=None, staged=False):
     M = x_bits.shape[0]
     proj = ops.Projection.from_native(backend, [(fmt, n, nat) for n, nat in native_segments], K, float32=float32)
     gate = ops.Projection.from_native(backend, [(fmt, native_segments[0][0], gate_native)], K) if gate_native is not None else None
     N = proj.output_size
-    plan = linear.plan(proj, M, epilogue, splits=splits, whole_groups=whole_groups)
+    plan = linear.plan(proj, M, epilogue, splits=splits, whole_groups=whole_groups, staged=staged)
     scratch = linear.scratch_for(backend, [plan])
     x = backend.from_array(x_bits, label="x")
     out = backend.allocate_buffer(M * N * (4 if float32 else 2), label="out")
@@ -448,3 +448,56 @@ def test_config2_projections_at_full_size(backend, name, fmt, widths, K):
     doubled = orc.f32_to_bf16(2 * orc.bf16_to_f32(x[:16]))
     plan = linear.plan(proj, 16, ops.EPILOGUE_NONE)
     assert (2 * run(x[:16], plan)).tobytes() == run(doubled, plan).tobytes()
+
+
+@pytest.mark.parametrize("fmt", ALL_FORMATS)
+@pytest.mark.parametrize("M", [1, 16, 40, 64, 100])
+def test_the_staged_rule_rounds_each_weight_once_to_half(backend, fmt, M):
+    """The staged tile (kernels/common/gguf_staged.h:12-66; gguf_projection_test.mm:217-237 with staged = true): the
+    bf16 result lies in [bf16(lo), bf16(hi)] of the fp64 dot +- projectionBound(staged). The fp32 result, beyond that,
+    lies within the accumulation term alone (2^-16 sum|x| max|w|) of the fp64 dot over the HALF-ROUNDED weights, which
+    the same products over unrounded weights miss (the two dots differ by up to 2^-11 sum|x w|): the weights are halves.
+    With a residual; bit-identical re-runs over K partitions."""
+    print(f"case staged projection fmt={fmt} M={M}", flush=True)
+    rng = np.random.default_rng(500 + M)
+    N, K = 192, 2048
+    native = orc.make_native(fmt, N, K, 60 + M)
+    x = orc.f32_to_bf16(rng.standard_normal((M, K)).astype(np.float32))
+    linear = ops.Linear(backend)
+    want = orc.gemm_staged(fmt, native, x, N)
+    got, plan, _ = run_projection(backend, linear, fmt, [(N, native)], K, x, staged=True)
+    assert plan.tile == 1
+    check_interval(orc.bf16_to_f32(got), want)
+    got32, _, _ = run_projection(backend, linear, fmt, [(N, native)], K, x, float32=True, staged=True)
+    distance = np.abs(got32.astype(np.float64) - want["staged"].astype(np.float64))
+    assert np.all(distance <= want["accumulation"] + np.abs(want["staged"]) * 2.0 ** -23), float((distance / want["accumulation"]).max())
+    # ... and the unrounded weights' dot is further away than that for most outputs: the test tells the two apart
+    assert np.mean(np.abs(want["exact"] - want["staged"]) > 2 * distance) > 0.5
+    residual = orc.f32_to_bf16(rng.standard_normal((M, N)).astype(np.float32))
+    with_residual, _, _ = run_projection(backend, linear, fmt, [(N, native)], K, x, epilogue=ops.EPILOGUE_RESIDUAL, residual_bits=residual,
+                                         staged=True)
+    # gguf_projection_test.mm:242-245: fl(p + r) is monotonic, so the sum's interval is the rounded sums of the ends
+    r = orc.bf16_to_f32(residual)
+    lo = np.nextafter((want["exact"] - want["bound"]).astype(np.float32), -np.inf) + r
+    hi = np.nextafter((want["exact"] + want["bound"]).astype(np.float32), np.inf) + r
+    value = orc.bf16_to_f32(with_residual)
+    assert np.all((value >= orc.bf16_to_f32(orc.f32_to_bf16(lo))) & (value <= orc.bf16_to_f32(orc.f32_to_bf16(hi))))
+    for splits in (1, 2, 8):
+        a, _, _ = run_projection(backend, linear, fmt, [(N, native)], K, x, float32=True, splits=splits, whole_groups=0, staged=True)
+        b, _, _ = run_projection(backend, linear, fmt, [(N, native)], K, x, float32=True, splits=splits, whole_groups=0, staged=True)
+        assert a.tobytes() == b.tobytes()
+        assert np.all(np.abs(a.astype(np.float64) - want["exact"]) <= want["bound"])
+
+
+def test_the_staged_rule_takes_plain_and_residual_plans_of_one_format(backend):
+    linear = ops.Linear(backend)
+    K = 1024
+    one = ops.Projection.from_native(backend, [(ops.FMT_Q4K, 128, orc.make_native(ops.FMT_Q4K, 128, K, 1))], K)
+    with pytest.raises(splash_amd.SplashError):
+        linear.plan(one, 16, ops.EPILOGUE_GATE_UP, staged=True)
+    with pytest.raises(splash_amd.SplashError):
+        linear.plan(one, 16, ops.EPILOGUE_RESIDUAL_NORM, staged=True)
+    mixed = ops.Projection.from_native(backend, [(ops.FMT_Q4K, 64, orc.make_native(ops.FMT_Q4K, 64, K, 2)),
+                                                 (ops.FMT_Q6K, 64, orc.make_native(ops.FMT_Q6K, 64, K, 3))], K)
+    with pytest.raises(splash_amd.SplashError):
+        linear.plan(mixed, 16, staged=True)

@@ -76,3 +76,42 @@ def test_register_chain_lies_inside_projection_bound(fmt):
     w = orc.dequant_rows(fmt, native, N, K).astype(np.float64)
     ref = orc.bf16_to_f32(x).astype(np.float64) @ w.T
     assert np.allclose(r["exact"], ref, rtol=1e-12, atol=1e-12)
+
+
+ALL_FORMATS = [orc.FMT_Q4K, orc.FMT_Q6K, orc.FMT_Q5K, orc.FMT_Q80, orc.FMT_IQ4XS, orc.FMT_IQ4NL]
+
+
+@pytest.mark.parametrize("fmt", ALL_FORMATS)
+def test_staged_projection_is_the_half_rounded_weights_and_the_reference_bound(fmt):
+    """orc_gemm_staged against statements of its own parts: its exact dot and its staged value are numpy fp64 products
+    over the dequantized weights and over numpy's float16 rounding of them (gguf_staged.h:12-19: each value rounded
+    once to half); its bounds are the reference's own dot + projectionBound(staged) and (register tile) on sample
+    pairs (a dropped 2^-11 or 2^-25 term, or the accumulation term over sum|x w| instead of sum|x| max|w|, fails)."""
+    rng = np.random.default_rng(17 + fmt)
+    N, K, M = 48, 1024, 6
+    native = orc.make_native(fmt, N, K, 31 + fmt)
+    x = orc.f32_to_bf16(rng.standard_normal((M, K)).astype(np.float32))
+    r = orc.gemm_staged(fmt, native, x, N)
+    w = orc.dequant_rows(fmt, native, N, K)
+    xf = orc.bf16_to_f32(x).astype(np.float64)
+    assert np.allclose(r["exact"], xf @ w.astype(np.float64).T, rtol=1e-12, atol=1e-12)
+    w16 = w.astype(np.float16).astype(np.float64)
+    assert np.any(w16 != w)     # the rounding is one: these weights are not halves already
+    assert np.array_equal(r["staged"], (xf @ w16.T).astype(np.float32))
+    # the staged value lies inside the reference's interval, and its distance is of the rounding's size
+    assert np.all(np.abs(r["staged"] - r["exact"]) <= r["bound"])
+    assert np.all(r["accumulation"] < r["bound"])
+    if orc.ref is None:
+        pytest.skip("oracle/_ref is not built here")
+    f64p = orc.ctypes.POINTER(orc.ctypes.c_double)
+    for fn in (orc.ref.ref_dot_bound, orc.ref.ref_dot_bound_staged):
+        fn.argtypes = [orc.f32p, orc.f32p, orc.c_u32, f64p, f64p]
+        fn.restype = None
+    xf32 = orc.bf16_to_f32(x)
+    for m, n in [(0, 0), (3, 17), (5, 47), (2, 31)]:
+        value, staged_bound, plain_bound = (orc.ctypes.c_double() for _ in range(3))
+        xr, wr = np.ascontiguousarray(xf32[m]), np.ascontiguousarray(w[n])
+        orc.ref.ref_dot_bound_staged(orc._p(xr, orc.f32p), orc._p(wr, orc.f32p), K, orc.ctypes.byref(value), orc.ctypes.byref(staged_bound))
+        orc.ref.ref_dot_bound(orc._p(xr, orc.f32p), orc._p(wr, orc.f32p), K, orc.ctypes.byref(value), orc.ctypes.byref(plain_bound))
+        assert value.value == r["exact"][m, n]
+        assert staged_bound.value == r["bound"][m, n] and plain_bound.value == r["accumulation"][m, n]
