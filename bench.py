@@ -232,6 +232,46 @@ def time_c2_ops(backend):
                       "roofline_peak_gbs": HBM_PEAK_GBS, "results": results}), flush=True)
 
 
+def time_prefill_ops(backend):
+    """The prefill projection (ops.Linear.add_prefill: the staged rule over a chunk of rows, 128 x 128 a workgroup) at the
+    27B shape's matrices and chunks of 512, 2048 and 8192 rows: GPU time of a chunk's dispatches (its table passes and its
+    projection; HIP events around each dispatch), median of five. The operations counted are the algorithm's, 2 M N K;
+    the kernel issues two bf16 MFMAs a product (a half weight is two bf16 parts). Prints one JSON line; the dense MFMA
+    peak is bf16's."""
+    import splash_amd
+    from splash_amd import ops
+    rng = np.random.default_rng(0)
+    bf = lambda a: (np.ascontiguousarray(a, np.float32).view(np.uint32) >> 16).astype(np.uint16)
+    H, F, Q, KV = 5120, 25600, 8192, 1024
+    peak = 2500.0
+    results = []
+    for name, fmt, N, K in (("qkv", ops.FMT_Q4K, Q + 2 * KV, H), ("gate", ops.FMT_Q4K, F, H), ("down", ops.FMT_Q6K, H, F)):
+        projection = ops.Projection([(fmt, N, backend.from_array(rng.integers(0, 256, ops.gguf_image_bytes(fmt, N, K), dtype=np.uint8)))], K)
+        for M in (512, 2048, 8192):
+            x = backend.from_array(bf(rng.standard_normal((M, K))))
+            out = backend.allocate_buffer(M * N * 2)
+            table = backend.allocate_buffer(ops.Linear.prefill_table_bytes(K, M))
+            graph = splash_amd.CommandGraph()
+            repeats = 6
+            for _ in range(repeats):
+                ops.Linear.add_prefill(graph, projection, x, out, table, M)
+            per_chunk = len(graph) // repeats
+            backend.set_dispatch_profiling(True)
+            _, _, per = backend.run(graph, profiled=True)
+            backend.set_dispatch_profiling(False)
+            chunks = np.array(per).reshape(repeats, per_chunk)[1:] * 1e6
+            us, gemm_us = float(np.median(chunks.sum(axis=1))), float(np.median(chunks[:, -1]))
+            tflops = 2.0 * M * N * K / us / 1e6
+            results.append({"op": name, "format": "q4_k" if fmt == ops.FMT_Q4K else "q6_k", "N": N, "K": K, "M": M, "us": round(us, 1),
+                            "projection_us": round(gemm_us, 1), "TFLOP/s": round(tflops, 1), "frac": round(tflops / peak, 4)})
+            log(f"  {name:5s} M={M:5d}: {us:9.1f} us a chunk ({gemm_us:9.1f} us the projection) {tflops:7.1f} TFLOP/s")
+            del graph, x, out, table
+        del projection
+    print(json.dumps({"metric": "prefill projection us and TFLOP/s by rows", "unit": "us", "n_gpus": 1,
+                      "data": "synthetic: random images, N(0, 1) rows", "roofline": {"bound": "mfma", "peak": peak, "unit": "TFLOP/s"},
+                      "results": results}), flush=True)
+
+
 def time_c3_ops(backend):
     """BASELINE.json config 3: block-causal attention of a 16-row chain block (64 query / 8 KV heads of 128) over a paged
     INT8 context of 8K, 32K and 128K tokens (256-token pages, random page table), the split pass and the merge, over a
@@ -534,7 +574,7 @@ def main():
     ap.add_argument("--temperature", type=float, default=0.0,
                     help="above 0: rejection-sampling acceptance at this temperature against a full-vocabulary draft "
                          "distribution softmax(N(0, 2)) instead of greedy acceptance")
-    ap.add_argument("--ops", choices=["c2", "c3", "c5", "state", "draft"],
+    ap.add_argument("--ops", choices=["c2", "c3", "c5", "state", "draft", "prefill"],
                     help="instead of the dense step: c2 the projections alone by rows, c3 attention alone by context, "
                          "c5 the GDN step and the MoE layer of config 5, state the recurrent layers' cached form")
     args = ap.parse_args()
@@ -545,7 +585,8 @@ def main():
     from splash_amd import ops, verify
     backend = splash_amd.Backend(0)
     if args.ops:
-        {"c2": time_c2_ops, "c3": time_c3_ops, "c5": time_c5_ops, "state": time_state_codec, "draft": time_draft_candidates}[args.ops](backend)
+        {"c2": time_c2_ops, "c3": time_c3_ops, "c5": time_c5_ops, "state": time_state_codec, "draft": time_draft_candidates,
+         "prefill": time_prefill_ops}[args.ops](backend)
         return
     if args.workload == "c5":
         bench_c5(backend, args)

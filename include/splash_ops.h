@@ -133,6 +133,15 @@ sp_status spo_linear_add_link(const spo_linear *linear, spo_graph *graph, const 
  * link before it, of chains added from now on. 0 makes every wait that finds the count short give up at once, which is
  * how a host tests the failure path without a kernel that does not end. */
 sp_status spo_linear_set_chain_spin_limit(spo_linear *linear, uint32_t polls);
+/* Linear::addPrefill: a chunk of 1 to 16384 rows (a prompt's) through the projection under the staged rule, a workgroup
+ * 128 rows x 128 columns with K whole: the counterpart of the reference's prefill tile (LinearTile::GgufPrefill,
+ * gguf_linear.metal:79-118, Linear.hpp:330-332 with a prefill plan). output = bf16 (fp32 for a projection created so)
+ * of input x W^T, plus the bf16 residual rows when `residual` is not NULL. Every tensor of the projection holds a
+ * multiple of 128 columns. `table`: spo_linear_prefill_table_bytes(input size, rows) bytes of the rows' activation
+ * tables, which the dispatches write first. */
+uint64_t spo_linear_prefill_table_bytes(uint32_t input_size, uint32_t rows);
+sp_status spo_linear_add_prefill(spo_graph *graph, const spo_projection *projection, sp_buffer *input, sp_buffer *output,
+                                 sp_buffer *residual, sp_buffer *table, uint32_t rows);
 /* Linear::scratchSize (Linear.hpp:319): of every plan of up to `rows` rows of the matrix. */
 sp_status spo_linear_scratch_size(const spo_linear *linear, uint32_t output_size, uint32_t input_size, uint32_t rows,
                                   uint64_t *table, uint64_t *partials, uint64_t *counters);

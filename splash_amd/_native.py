@@ -243,6 +243,8 @@ _sig("spo_linear_add_swiglu", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p
 _sig("spo_linear_set_chain_spin_limit", c_int, c_p, c_u32)
 _sig("spo_linear_add_link", c_int, c_p, c_p, P(ChainLink))
 _sig("spo_linear_add_chain", c_int, c_p, c_p, P(ChainLink), c_u32, c_p)
+_sig("spo_linear_prefill_table_bytes", c_u64, c_u32, c_u32)
+_sig("spo_linear_add_prefill", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_u32)
 _sig("spo_linear_scratch_size", c_int, c_p, c_u32, c_u32, c_u32, P(c_u64), P(c_u64), P(c_u64))
 
 _sig("spo_kv_page_bytes", c_u64, c_u32, c_u32)

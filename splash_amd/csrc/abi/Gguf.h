@@ -177,6 +177,19 @@ struct GgufPrepareParams {
   uint32_t row_stride;  // elements between input rows
 };
 
+// gguf_prefill_<fmt>_{a,a_f32,r}: a chunk of rows under the staged rule. Binds the segment's image, the rows' activation
+// tables (64-row pieces one after the other, each gguf_table_bytes(input_size, GGUF_PIECE_TILES) on from the one before),
+// out (bf16, or fp32 for _a_f32) and the residual rows (bf16; any buffer when unused). Grid (columns / 128,
+// ceil(rows / 128)), 256 threads.
+struct GgufPrefillParams {
+  uint32_t input_size;
+  uint32_t rows;
+  uint32_t columns;     // of this segment: a multiple of 128
+  uint32_t out_stride;  // elements between output (and residual) rows
+  uint32_t out_offset;  // the segment's first output column
+  uint32_t reserved[3];
+};
+
 // Epilogues of a decode projection (the reference's LinearEpilogue, runtime/ops/Linear.hpp:77).
 #define GGUF_EPILOGUE_PLAIN 0u     // out = bf16(v)         kernel suffix _a
 #define GGUF_EPILOGUE_PLAIN_F32 1u // out = v               kernel suffix _a_f32

@@ -270,6 +270,17 @@ sp_status spo_linear_add_swiglu(const spo_linear *linear, spo_graph *graph, cons
                              hip::Buffer::share(residual), hip::Buffer::share(output), rows);
   });
 }
+uint64_t spo_linear_prefill_table_bytes(uint32_t input_size, uint32_t rows) {
+  return input_size && input_size % GGUF_BLOCK == 0 && rows ? ops::Linear::prefillTableBytes(input_size, rows) : 0;
+}
+sp_status spo_linear_add_prefill(spo_graph *graph, const spo_projection *projection, sp_buffer *input, sp_buffer *output,
+                                 sp_buffer *residual, sp_buffer *table, uint32_t rows) {
+  return capi::guard([&] {
+    capi::require(graph && projection, "graph or projection");
+    ops::Linear::addPrefill(graph->graph, hip::Buffer::share(input), projection->projection, hip::Buffer::share(output),
+                            hip::Buffer::share(residual), hip::Buffer::share(table), rows);
+  });
+}
 sp_status spo_linear_scratch_size(const spo_linear *linear, uint32_t output_size, uint32_t input_size, uint32_t rows,
                                   uint64_t *table, uint64_t *partials, uint64_t *counters) {
   return capi::guard([&] {

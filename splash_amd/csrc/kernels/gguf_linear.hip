@@ -505,37 +505,48 @@ __device__ __forceinline__ void staged_operands(const float (&value)[8], bf16x8 
   high = as_bf16x8(make_uint4(highWords[0], highWords[1], highWords[2], highWords[3]));
   low = as_bf16x8(make_uint4(lowWords[0], lowWords[1], lowWords[2], lowWords[3]));
 }
+// A record's coefficients of the staged rule and a group's two operands.
+template <uint32_t FMT> struct StagedCoefficients {
+  Q4KScales sc{};
+  float d6 = 0.f;
+  __device__ __forceinline__ explicit StagedCoefficients(const Record<FMT> &rec) {
+    if constexpr (FMT == GGUF_FMT_Q4K || FMT == GGUF_FMT_Q5K) sc = q4k_scales(rec.meta);
+    if constexpr (FMT == GGUF_FMT_Q6K) d6 = half_bits_to_float(rec.d);
+  }
+};
+template <uint32_t FMT>
+__device__ __forceinline__ void staged_group(const Record<FMT> &rec, const StagedCoefficients<FMT> &k, const uint4 &operand, uint32_t g,
+                                             bf16x8 &high, bf16x8 &low) {
+  const uint32_t regs[4] = {operand.x, operand.y, operand.z, operand.w};
+  float value[8];
+  // the fp32 values of gguf_dequant, each exact or rounded once
+  if constexpr (FMT == GGUF_FMT_Q80 || FMT == GGUF_FMT_IQ4XS || FMT == GGUF_FMT_IQ4NL) {
+    const float d = group_scale(rec, g);
+#pragma unroll
+    for (uint32_t e = 0; e < 8; ++e) value[e] = d * (bf16_bits_to_float((regs[e >> 1] >> (16u * (e & 1u))) & 0xFFFFu) - 128.f);
+  } else if constexpr (FMT == GGUF_FMT_Q4K || FMT == GGUF_FMT_Q5K) {
+    const float s = k.sc.d * byte_of(g < 4 ? k.sc.sc_lo : k.sc.sc_hi, g & 3u);
+    const float m = -(k.sc.dmin * byte_of(g < 4 ? k.sc.mn_lo : k.sc.mn_hi, g & 3u));
+#pragma unroll
+    for (uint32_t e = 0; e < 8; ++e)
+      value[e] = __fmaf_rn(s, float(operand_code(regs[e >> 1], e & 1u) & (FMT == GGUF_FMT_Q5K ? 0x1Fu : 0xFu)), m);
+  } else {
+#pragma unroll
+    for (uint32_t e = 0; e < 8; ++e)
+      value[e] = (k.d6 * q6_scale(rec.scales, 2u * g + (e >> 2))) * float(int(operand_code(regs[e >> 1], e & 1u) & 0x3Fu) - 32);
+  }
+  staged_operands(value, high, low);
+}
 template <uint32_t FMT, int RT>
 __device__ __forceinline__ void accumulate_record_staged(const Record<FMT> &rec, const uint4 (*a)[8][64], f32x4 (&acc)[RT], uint32_t lane,
                                                          uint32_t kq) {
   uint4 ops[8];
   record_operands(rec, ops);
-  Q4KScales sc{};
-  float d6 = 0.f;
-  if constexpr (FMT == GGUF_FMT_Q4K || FMT == GGUF_FMT_Q5K) sc = q4k_scales(rec.meta);
-  if constexpr (FMT == GGUF_FMT_Q6K) d6 = half_bits_to_float(rec.d);
+  const StagedCoefficients<FMT> k(rec);
 #pragma unroll
   for (uint32_t g = 0; g < 8; ++g) {
-    const uint32_t regs[4] = {ops[g].x, ops[g].y, ops[g].z, ops[g].w};
-    float value[8];
-    // the fp32 values of gguf_dequant, each exact or rounded once
-    if constexpr (FMT == GGUF_FMT_Q80 || FMT == GGUF_FMT_IQ4XS || FMT == GGUF_FMT_IQ4NL) {
-      const float d = group_scale(rec, g);
-#pragma unroll
-      for (uint32_t e = 0; e < 8; ++e) value[e] = d * (bf16_bits_to_float((regs[e >> 1] >> (16u * (e & 1u))) & 0xFFFFu) - 128.f);
-    } else if constexpr (FMT == GGUF_FMT_Q4K || FMT == GGUF_FMT_Q5K) {
-      const float s = sc.d * byte_of(g < 4 ? sc.sc_lo : sc.sc_hi, g & 3u);
-      const float m = -(sc.dmin * byte_of(g < 4 ? sc.mn_lo : sc.mn_hi, g & 3u));
-#pragma unroll
-      for (uint32_t e = 0; e < 8; ++e)
-        value[e] = __fmaf_rn(s, float(operand_code(regs[e >> 1], e & 1u) & (FMT == GGUF_FMT_Q5K ? 0x1Fu : 0xFu)), m);
-    } else {
-#pragma unroll
-      for (uint32_t e = 0; e < 8; ++e)
-        value[e] = (d6 * q6_scale(rec.scales, 2u * g + (e >> 2))) * float(int(operand_code(regs[e >> 1], e & 1u) & 0x3Fu) - 32);
-    }
     bf16x8 high, low;
-    staged_operands(value, high, low);
+    staged_group(rec, k, ops[g], g, high, low);
 #pragma unroll
     for (int t = 0; t < RT; ++t) {
       const bf16x8 rows = as_bf16x8(a[t][g][lane]);
@@ -1687,5 +1698,120 @@ SP_GGUF_DECODE("iq4xs", GGUF_FMT_IQ4XS, 64, 4);
 SP_GGUF_DECODE("iq4nl", GGUF_FMT_IQ4NL, 16, 1);
 SP_GGUF_DECODE("iq4nl", GGUF_FMT_IQ4NL, 32, 2);
 SP_GGUF_DECODE("iq4nl", GGUF_FMT_IQ4NL, 64, 4);
+
+// ---------------------------------------------------------------------------------------------
+// gguf_prefill_<fmt>_{a,a_f32,r}: the staged rule over a chunk of many rows (the reference's prefill tile,
+// gguf_linear.metal:79-118: a shared stage of dequantized weights, each simdgroup its rows). Here the weights stay in
+// registers and the rows pass through LDS: a workgroup owns 128 rows x 128 columns, a wave 32 of the columns (two
+// records a super-block) over all of the rows, so an operand of rows read from LDS meets four MFMAs (two records, each
+// the half's two bf16 parts). Rows come from the activation tables of their 64-row pieces (gguf_prepare_table), half a
+// super-block at a time through two LDS buffers. Grid (columns / 128, ceil(rows / 128)), 256 threads; K whole.
+// ---------------------------------------------------------------------------------------------
+template <uint32_t FMT, uint32_t EP>
+__global__ __launch_bounds__(256, 2) void gguf_prefill(const uint8_t *__restrict__ image, const uint8_t *__restrict__ tables,
+                                                       void *__restrict__ out, const uint16_t *__restrict__ residual,
+                                                       GgufPrefillParams p) {
+  constexpr uint32_t kRecord = gguf_record_bytes(FMT);
+  __shared__ uint4 rowsStage[2][8][4][64];   // [buffer][row tile][group of the half][lane]: 64 KiB
+  const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6, c = lane & 15u, kq = lane >> 4;
+  const uint32_t blocks = p.input_size / GGUF_BLOCK, G = p.input_size / 32u;
+  const uint32_t firstTile = blockIdx.y * 8u, totalTiles = (p.rows + 15u) / 16u;
+  const uint32_t tilesHere = min(8u, totalTiles - firstTile);
+  const uint64_t pieceBytes = gguf_table_bytes(p.input_size, GGUF_PIECE_TILES);
+  // this wave's two column tiles
+  const uint32_t tile0 = (blockIdx.x * 4u + wave) * 2u;
+  Cursor<FMT> cursor[2];
+  Record<FMT> rec[2], next[2];
+#pragma unroll
+  for (uint32_t r = 0; r < 2; ++r) {
+    cursor[r].open(image + size_t(tile0 + r) * blocks * kRecord, lane);
+    next[r].load(cursor[r]);
+  }
+  f32x4 acc[2][8];
+#pragma unroll
+  for (uint32_t r = 0; r < 2; ++r)
+#pragma unroll
+    for (uint32_t t = 0; t < 8; ++t) acc[r][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+  // A half super-block of the rows: 8 tiles x 4 groups x 64 lanes of 16 bytes, 8 a thread.
+  uint4 held[8];
+  auto fetch = [&](uint32_t half) {   // half counts half super-blocks from the start of K
+#pragma unroll
+    for (uint32_t i = 0; i < 8; ++i) {
+      const uint32_t at = threadIdx.x + 256u * i, t = at >> 8, g = (at >> 6) & 3u, l = at & 63u;
+      const uint32_t tile = firstTile + t;
+      held[i] = make_uint4(0u, 0u, 0u, 0u);
+      if (t < tilesHere) {
+        const uint4 *values = reinterpret_cast<const uint4 *>(tables + uint64_t(tile / GGUF_PIECE_TILES) * pieceBytes);
+        held[i] = values[(size_t(tile % GGUF_PIECE_TILES) * G + half * 4u + g) * 64u + l];
+      }
+    }
+  };
+  auto store = [&](uint32_t buffer) {
+#pragma unroll
+    for (uint32_t i = 0; i < 8; ++i) (&rowsStage[buffer][0][0][0])[threadIdx.x + 256u * i] = held[i];
+  };
+  const uint32_t halves = 2u * blocks;
+  fetch(0);
+  store(0);
+  __syncthreads();
+  for (uint32_t block = 0; block < blocks; ++block) {
+    // a new super-block: its records, and the next one's on their way
+    uint4 ops[2][8];
+#pragma unroll
+    for (uint32_t r = 0; r < 2; ++r) {
+      rec[r] = next[r];
+      cursor[r].advance();
+      if (block + 1 < blocks) next[r].load(cursor[r]);
+      record_operands(rec[r], ops[r]);
+    }
+    const StagedCoefficients<FMT> k[2] = {StagedCoefficients<FMT>(rec[0]), StagedCoefficients<FMT>(rec[1])};
+#pragma unroll
+    for (uint32_t h = 0; h < 2; ++h) {   // the super-block's halves: LDS buffer h
+      const uint32_t half = 2u * block + h;
+      if (half + 1 < halves) fetch(half + 1);
+#pragma unroll
+      for (uint32_t r = 0; r < 2; ++r)
+#pragma unroll
+        for (uint32_t g = 0; g < 4; ++g) {
+          bf16x8 high, low;
+          staged_group(rec[r], k[r], ops[r][4u * h + g], 4u * h + g, high, low);
+#pragma unroll
+          for (uint32_t t = 0; t < 8; ++t) {
+            if (t >= tilesHere) break;
+            const bf16x8 rows = as_bf16x8(rowsStage[h][t][g][lane]);
+            acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(rows, high, acc[r][t], 0, 0, 0);
+            acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(rows, low, acc[r][t], 0, 0, 0);
+          }
+        }
+      if (half + 1 < halves) store(h ^ 1u);
+      __syncthreads();
+    }
+  }
+  // Element (t, v) of this lane is row 16 (firstTile + t) + 4 kq + v, column 16 (tile0 + r) + c.
+#pragma unroll
+  for (uint32_t r = 0; r < 2; ++r)
+#pragma unroll
+    for (uint32_t t = 0; t < 8; ++t)
+#pragma unroll
+      for (uint32_t v = 0; v < 4; ++v) {
+        const uint32_t row = 16u * (firstTile + t) + 4u * kq + v;
+        if (row >= p.rows) continue;
+        const size_t at = size_t(row) * p.out_stride + p.out_offset + 16u * (tile0 + r) + c;
+        if constexpr (EP == GGUF_EPILOGUE_PLAIN_F32) static_cast<float *>(out)[at] = acc[r][t][v];
+        else if constexpr (EP == GGUF_EPILOGUE_RESIDUAL)
+          static_cast<uint16_t *>(out)[at] = uint16_t(float_to_bf16_bits(acc[r][t][v] + bf16_bits_to_float(residual[at])));
+        else static_cast<uint16_t *>(out)[at] = uint16_t(float_to_bf16_bits(acc[r][t][v]));
+      }
+}
+#define SP_GGUF_PREFILL(fmt, FMT)                                                                          \
+  SP_REGISTER_KERNEL("gguf_prefill_" fmt "_a", &gguf_prefill<FMT, GGUF_EPILOGUE_PLAIN>);                 \
+  SP_REGISTER_KERNEL("gguf_prefill_" fmt "_a_f32", &gguf_prefill<FMT, GGUF_EPILOGUE_PLAIN_F32>);         \
+  SP_REGISTER_KERNEL("gguf_prefill_" fmt "_r", &gguf_prefill<FMT, GGUF_EPILOGUE_RESIDUAL>)
+SP_GGUF_PREFILL("q4k", GGUF_FMT_Q4K);
+SP_GGUF_PREFILL("q6k", GGUF_FMT_Q6K);
+SP_GGUF_PREFILL("q5k", GGUF_FMT_Q5K);
+SP_GGUF_PREFILL("q80", GGUF_FMT_Q80);
+SP_GGUF_PREFILL("iq4xs", GGUF_FMT_IQ4XS);
+SP_GGUF_PREFILL("iq4nl", GGUF_FMT_IQ4NL);
 
 } // namespace splash::kernels

@@ -400,6 +400,51 @@ PreparedInput Linear::addWithAttention(hip::CommandGraph &graph, LinearBuffers b
   return r.after;
 }
 
+uint64_t Linear::prefillTableBytes(uint32_t inputSize, uint32_t rows) noexcept {
+  return gguf_tables_bytes(inputSize, gguf_row_tiles(rows));
+}
+
+namespace {
+hip::Buffer viewOf(const hip::Buffer &base, uint64_t offset, uint64_t length) {
+  sp_buffer *raw = nullptr;
+  hip::throwStatus(sp_buffer_view(base.handle(), offset, length, &raw));
+  return hip::Buffer::adopt(raw);
+}
+} // namespace
+
+void Linear::addPrefill(hip::CommandGraph &graph, const hip::Buffer &input, const Projection &p, const hip::Buffer &output,
+                        const hip::Buffer &residual, const hip::Buffer &table, uint32_t rows) {
+  const uint32_t n = p.outputSize, k = p.inputSize;
+  if (!rows || rows > kMaximumPrefillRows) throw std::invalid_argument("a prefill chunk takes 1 to 16384 rows");
+  requireSegments(p, {n, k});
+  for (const QuantizedSegment &s : p.blocks().segments)
+    if (s.outputSize % 128 || s.columnOffset % 16) throw std::invalid_argument("a prefill projection's tensors hold whole 128-column workgroups");
+  const bool float32 = p.destination == FloatOutput::Float32;
+  if (float32 && residual) throw std::invalid_argument("only a plain prefill projection writes fp32");
+  requireBytes(input, uint64_t{rows} * k * 2, "projection input");
+  requireBytes(output, uint64_t{rows} * n * (float32 ? 4 : 2), "projection output");
+  if (residual) requireBytes(residual, uint64_t{rows} * n * 2, "projection residual");
+  requireBytes(table, prefillTableBytes(k, rows), "projection tables");
+  // the rows' tables, 256 rows (four 64-row pieces) a pass
+  const uint64_t pieceBytes = gguf_table_bytes(k, GGUF_PIECE_TILES);
+  for (uint32_t first = 0; first < rows; first += kMaximumDispatchRows) {
+    const uint32_t count = std::min(kMaximumDispatchRows, rows - first);
+    const uint64_t tableAt = uint64_t{first / GGUF_MAXIMUM_ROWS} * pieceBytes;
+    addPrepare(graph, viewOf(input, uint64_t{first} * k * 2, uint64_t{count} * k * 2),
+               LinearScratch{viewOf(table, tableAt, gguf_tables_bytes(k, gguf_row_tiles(count))), {}, {}}, k, count);
+  }
+  for (const QuantizedSegment &s : p.blocks().segments) {
+    GgufPrefillParams params{};
+    params.input_size = k;
+    params.rows = rows;
+    params.columns = s.outputSize;
+    params.out_stride = n;
+    params.out_offset = s.columnOffset;
+    graph.add(std::string("gguf_prefill_") + s.name() + (residual ? "_r" : float32 ? "_a_f32" : "_a"),
+              {s.image, table, output, residual ? residual : output}, params, {s.outputSize / 128, (rows + 127) / 128, 1}, {256, 1, 1});
+  }
+}
+
 void Linear::addProjection(hip::CommandGraph &graph, hip::Buffer input, const Projection &projection, hip::Buffer output,
                            uint32_t rows, LinearScratch scratch) const {
   LinearBuffers buffers;

@@ -221,6 +221,15 @@ public:
   [[nodiscard]] static LinearScratchSize attentionScratchSize(const LinearPlan &plan) noexcept;
   PreparedInput addWithAttention(hip::CommandGraph &graph, LinearBuffers buffers, const Projection &projection,
                                  const LinearPlan &plan, const AttentionPrepareBindings &attention) const;
+  // A chunk of many rows (a prompt's, up to kMaximumPrefillRows) under the staged rule, a workgroup 128 rows x 128
+  // columns with K whole (kernels gguf_prefill_*; the reference's prefill tile, gguf_linear.metal:79-118, and
+  // LinearTile::GgufPrefill): output = bf16 or fp32 (the projection's destination) of input x W^T, plus the residual
+  // rows when `residual` names them. Every segment's columns are a multiple of 128. `table` holds the rows'
+  // activation tables (prefillTableBytes), which the dispatch writes first.
+  static constexpr uint32_t kMaximumPrefillRows = 16384;
+  [[nodiscard]] static uint64_t prefillTableBytes(uint32_t inputSize, uint32_t rows) noexcept;
+  static void addPrefill(hip::CommandGraph &graph, const hip::Buffer &input, const Projection &projection, const hip::Buffer &output,
+                         const hip::Buffer &residual, const hip::Buffer &table, uint32_t rows);
   void addProjection(hip::CommandGraph &graph, hip::Buffer input, const Projection &projection, hip::Buffer output,
                      uint32_t rows, LinearScratch scratch) const;
   void addResidualProjection(hip::CommandGraph &graph, hip::Buffer input, const Projection &projection,

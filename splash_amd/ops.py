@@ -189,6 +189,18 @@ class Linear:
                                         next_table.handle if next_table is not None else None))
         graph._keep.extend([gate, up, down, normalized, intermediate, residual, output, scratch, next_table])
 
+    @staticmethod
+    def prefill_table_bytes(input_size, rows):
+        return lib.spo_linear_prefill_table_bytes(input_size, rows)
+
+    @staticmethod
+    def add_prefill(graph, projection, input, output, table, rows, residual=None):
+        """A chunk of up to 16384 rows through the projection under the staged rule (Linear::addPrefill). table:
+        prefill_table_bytes(input size, rows) bytes."""
+        check(lib.spo_linear_add_prefill(graph.handle, projection.handle, input.handle, output.handle,
+                                         residual.handle if residual is not None else None, table.handle, rows))
+        graph._keep.extend([projection, input, output, table, residual])
+
     def scratch_size(self, output_size, input_size, rows):
         t, s, c = ctypes.c_uint64(), ctypes.c_uint64(), ctypes.c_uint64()
         check(lib.spo_linear_scratch_size(self.handle, output_size, input_size, rows, ctypes.byref(t), ctypes.byref(s),
