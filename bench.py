@@ -568,6 +568,9 @@ def main():
     ap.add_argument("--fused-prepare", action="store_true",
                     help="a layer's q|k|v projection prepares its attention block itself: one dispatch instead of the "
                          "projection and the prepare kernel")
+    ap.add_argument("--prompt-chunk", type=int, default=0,
+                    help="instead of the verify step: a chunk of this many prompt tokens (up to 16 x --lanes) of one "
+                         "sequence through every layer in one pass over the weights (DenseVerify.encode_prefill)")
     ap.add_argument("--calibrate-traffic", action="store_true",
                     help="after the steps, run plain read and copy kernels of known size: the scale of the FETCH_SIZE / "
                          "WRITE_SIZE counters of a rocprofv3 --pmc run of this command")
@@ -607,6 +610,20 @@ def main():
         gpu.set_chained(True)
     if args.fused_prepare:
         gpu.set_fused_prepare(True)
+    if args.prompt_chunk:
+        # a prompt chunk that ends the context: every layer, no head
+        tokens = args.prompt_chunk
+        gpu.set_prefill_block(rng.integers(0, w["vocabulary"], tokens).astype(np.uint32))
+        command = backend.record(gpu.encode_prefill(0, w["context"] - tokens, tokens))
+        for _ in range(args.warmup):
+            command.submit().wait()
+        seconds = sum(command.submit().wait()[0] for _ in range(args.steps)) / args.steps
+        log(f"prompt chunk of {tokens} tokens: {seconds * 1e3:.3f} ms, {tokens / seconds:.0f} tokens/s")
+        print(json.dumps({"metric": "prompt chunk ms (every layer of the 27B shape, one pass over the weights)", "value": round(seconds * 1e3, 4),
+                          "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "tokens": tokens,
+                          "tokens_per_s": round(tokens / seconds, 1), "higher_is_better": False, "data": "synthetic",
+                          "config": {"workload": w["name"] if "name" in w else args.workload, "context_tokens": w["context"]}}), flush=True)
+        return
     graph = gpu.encode(lanes, commit=True)
     if args.temperature > 0:
         # the draft model's distributions of the block's rows: softmax of N(0, 2) logits over the whole vocabulary

@@ -476,6 +476,15 @@ sp_status spo_dense_verify_results(spo_dense_verify *verify, const spo_verify_la
  * (spo_linear_add_chain: output, gate/up, down and the next layer's q|k|v, the LM head after the last layer) where
  * their shapes allow: off by default; the results are the same bit for bit. spo_dense_verify_results fails with
  * SP_BACKEND_ERROR after a step in which a chained projection's bounded wait gave up. */
+/* DenseVerify::encodePrefill: a chunk of 1 to 16 x max_lanes prompt tokens of ONE sequence (its pages from table_first,
+ * `committed` tokens cached before the chunk) in one pass over the weights, where the reference prefills a prompt in
+ * chunks (Runtime.cpp's chunked prefill over QwenTarget.cpp:457-496): the tokens go in SPO_VERIFY_INPUT_TOKENS, a chain
+ * of tree rows a block of sixteen in SPO_VERIFY_TREE_ROWS, each row's depth in its block in SPO_VERIFY_DEPTHS, as a
+ * step's. Every layer runs, the head and the acceptance do not: the tokens' keys and values are in the pages and the
+ * hidden rows where a step leaves them, bit for bit those of the blocks run one step after the other; the caller
+ * advances the sequence's committed tokens. */
+sp_status spo_dense_verify_encode_prefill(spo_dense_verify *verify, spo_graph *graph, uint32_t table_first, uint32_t committed,
+                                          uint32_t tokens);
 sp_status spo_dense_verify_set_chained(spo_dense_verify *verify, int chained);
 /* DenseVerify::setFusedPrepare: a layer's q|k|v projection also prepares its attention block
  * (spo_attention_add_fused_projection) where the kernels take the pair: off by default (on MI355X the two dispatches

@@ -293,6 +293,13 @@ sp_status spo_dense_verify_results(spo_dense_verify *verify, const spo_verify_la
                            accepted, retained_rows);
   });
 }
+sp_status spo_dense_verify_encode_prefill(spo_dense_verify *verify, spo_graph *graph, uint32_t table_first, uint32_t committed,
+                                          uint32_t tokens) {
+  return capi::guard([&] {
+    capi::require(verify && graph, "verify or graph");
+    verify->verify->encodePrefill(capi::graphOf(graph), table_first, committed, tokens);
+  });
+}
 sp_status spo_dense_verify_set_chained(spo_dense_verify *verify, int chained) {
   return capi::guard([&] {
     capi::require(verify, "verify");

@@ -294,6 +294,25 @@ void DenseVerify::encodeHead(hip::CommandGraph &graph, uint32_t rows, bool input
   linear_.add(graph, head, weights_.head, linear_.plan(weights_.head, rows));
 }
 
+void DenseVerify::encodePrefill(hip::CommandGraph &graph, uint32_t tableFirst, uint32_t committed, uint32_t tokens) {
+  if (!tokens || tokens > maxRows_) throw std::invalid_argument("a prompt chunk takes 1 to 16 tokens a lane of the driver");
+  std::vector<ops::AttentionRows> sequences;
+  std::vector<ops::RopeSequence> rope;
+  for (uint32_t first = 0; first < tokens; first += ATTENTION_MAXIMUM_ROWS) {
+    const uint32_t rows = std::min<uint32_t>(ATTENTION_MAXIMUM_ROWS, tokens - first);
+    sequences.push_back({first, rows, committed + first, tableFirst});
+    rope.push_back({first, rows, committed + first});
+  }
+  const ops::AttentionGeometry geometry{dims_.qHeads, dims_.kvHeads, dims_.headDimension, dims_.rotaryPairs, dims_.normalizeHeads};
+  const ops::AttentionPlan plan = ops::PagedAttention::plan(geometry, sequences);
+  if (dims_.rotaryPairs)
+    ops::RoPE::addTreeTables(graph, inverseFrequency_, depths_, ropeCos_, ropeSin_, dims_.rotaryPairs, rope);
+  encodeEmbedding(graph, tokens);
+  const bool feeds = layersFeedNext(tokens);
+  for (uint32_t layer = 0; layer < dims_.layers; ++layer)
+    encodeLayer(graph, layer, plan, tokens, feeds && layer > 0, feeds && layer + 1 < dims_.layers);
+}
+
 void DenseVerify::encode(hip::CommandGraph &graph, const std::vector<VerifyLane> &lanes, bool commit) {
   if (lanes.empty() || lanes.size() > maxLanes_) throw std::invalid_argument("the step takes 1 to its most lanes");
   std::vector<ops::AttentionRows> sequences;

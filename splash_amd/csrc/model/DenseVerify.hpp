@@ -100,6 +100,13 @@ public:
   // The results are those of the separate dispatches, bit for bit.
   void setChained(bool chained) noexcept { chained_ = chained; }
   [[nodiscard]] bool chained() const noexcept { return chained_; }
+  // A chunk of a sequence's prompt (1 to 16 x maxLanes tokens, its input tokens, chain tree rows a block of sixteen and
+  // depths where a step's are) in one pass over the weights: the chunk runs as blocks of sixteen rows of one sequence,
+  // block i's history ending where block i - 1's rows end, through every layer and no head, so the tokens' keys and
+  // values are in the pages and the hidden rows where a step leaves them. The counterpart of the reference's chunked
+  // prefill (Runtime.cpp's prefill chunks over QwenTarget's layers) with the verify step's own kernels: the pools and
+  // the hidden rows are those of the blocks run one step after the other, bit for bit.
+  void encodePrefill(hip::CommandGraph &graph, uint32_t tableFirst, uint32_t committed, uint32_t tokens);
   // A layer's q|k|v projection also prepares its attention block (ops::PagedAttention::addFusedProjection) where the
   // kernels take the pair: off by default (the projection and the prepare kernel run one after the other). The results
   // are the same bit for bit; on MI355X the one dispatch is the slower of the two at the 27B shape, since the workgroup

@@ -92,6 +92,20 @@ class DenseVerify:
         graph._keep.append(self)
         return graph
 
+    def encode_prefill(self, table_first, committed, tokens, graph=None):
+        """A chunk of `tokens` prompt tokens of one sequence in one pass over the weights (every layer, no head): see
+        set_prefill_block for its inputs."""
+        graph = graph or CommandGraph()
+        check(lib.spo_dense_verify_encode_prefill(self.handle, graph.handle, table_first, committed, tokens))
+        graph._keep.append(self)
+        return graph
+
+    def set_prefill_block(self, tokens):
+        """A prompt chunk's inputs: its tokens, a chain of tree rows a block of sixteen, each row's depth in its block."""
+        tokens = np.asarray(tokens, dtype=np.uint32)
+        blocks = [min(16, tokens.size - at) for at in range(0, tokens.size, 16)]
+        self.set_block([Lane(rows, 0) for rows in blocks], tokens)
+
     def set_block(self, lanes, tokens, tree_rows=None, uniforms=None):
         """Writes the step's host-visible inputs: packed input tokens, tree rows (chains by default), depths."""
         rows = sum(l.rows for l in lanes)

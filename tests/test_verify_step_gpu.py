@@ -281,3 +281,40 @@ def test_the_fused_prepare_changes_nothing(backend, lanes_rows):
         assert np.array_equal(logits, plain[0][0]) and np.array_equal(hidden, plain[0][1]) and np.array_equal(pool, plain[0][2])
         for got, want in zip(results, plain[0][3]):
             assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("prompt_tokens", [64, 53])
+def test_a_prompt_chunk_in_one_pass_equals_its_blocks_one_by_one(backend, prompt_tokens):
+    """Prefill through the path's own kernels: a chunk of up to 64 prompt tokens as blocks of sixteen rows of ONE sequence
+    in one pass over the weights (block i's history ends where block i - 1's rows end; its keys and values are in the
+    pages before any block attends) leaves the pools and the hidden rows of the same blocks run one step after the
+    other, bit for bit."""
+    print(f"case prompt chunk tokens={prompt_tokens}", flush=True)
+    model = DenseModel(seed=17, hidden=1024, q_heads=16, kv_heads=8, head_dim=64, ffn=3072, vocabulary=32000, layers=3)
+    rng = np.random.default_rng(4)
+    gpu = model.build_gpu(backend, max_lanes=4, context_tokens=[prompt_tokens + 300])
+    model.seed_context(gpu, None, rng)
+    first, committed = model.table_first[0], 250      # the chunk crosses a page
+    prompt = rng.integers(0, 32000, prompt_tokens).astype(np.uint32)
+    blocks = [(16 * b, min(16, prompt_tokens - 16 * b)) for b in range((prompt_tokens + 15) // 16)]
+    pools = lambda: np.concatenate([gpu.buffer(verify.KV_POOL, layer).download(np.uint8) for layer in range(3)])
+    start = pools()
+    # one step a block
+    hidden = []
+    for at, rows in blocks:
+        lane = verify.Lane(rows, committed + at, table_first=first)
+        gpu.set_block([lane], prompt[at:at + rows])
+        backend.run(gpu.encode([lane], commit=False))
+        hidden.append(gpu.buffer(verify.HIDDEN, 0).download(np.uint16, rows * 1024).copy())
+    want_pools, want_hidden = pools(), np.concatenate(hidden)
+    assert (want_pools != start).any()
+    for layer in range(3):
+        gpu.buffer(verify.KV_POOL, layer).upload(start.reshape(3, -1)[layer])
+    # the chunk in one pass
+    graph = gpu.encode_prefill(first, committed, prompt_tokens)
+    gpu.set_prefill_block(prompt)
+    backend.run(graph)
+    assert np.array_equal(pools(), want_pools)
+    assert np.array_equal(gpu.buffer(verify.HIDDEN, 0).download(np.uint16, prompt_tokens * 1024), want_hidden)
+    # fewer passes over the weights: a layer's dispatches once, not once a block
+    assert len(graph) < len(gpu.encode([verify.Lane(16, committed, table_first=first)], commit=False)) 
