@@ -11,8 +11,8 @@ using hip::BufferStorage;
 DenseVerify::DenseVerify(hip::Backend &backend, DenseDimensions d, uint32_t maxLanes, uint32_t physicalPages,
                          uint32_t pageTableEntries)
     : backend_(backend), dims_(d), linear_(backend.deviceInfo()), maxLanes_(maxLanes) {
-  if (!d.hidden || !d.layers || !d.vocabulary || !d.ffn || !maxLanes || maxLanes > 4)
-    throw std::invalid_argument("a dense verify step takes a model and 1 to 4 lanes");
+  if (!d.hidden || !d.layers || !d.vocabulary || !d.ffn || !maxLanes || maxLanes > ATTENTION_MAXIMUM_SEQUENCES)
+    throw std::invalid_argument("a dense verify step takes a model and 1 to 8 lanes");
   if (d.hidden % GGUF_BLOCK || d.ffn % GGUF_BLOCK || d.attentionWidth() % GGUF_BLOCK || d.vocabulary % GGUF_TILE_COLUMNS)
     throw std::invalid_argument("the model's widths hold whole super-blocks and its vocabulary whole column tiles");
   maxRows_ = maxLanes * ATTENTION_MAXIMUM_ROWS;

@@ -283,16 +283,16 @@ def test_the_fused_prepare_changes_nothing(backend, lanes_rows):
             assert np.array_equal(got, want)
 
 
-@pytest.mark.parametrize("prompt_tokens", [64, 53])
+@pytest.mark.parametrize("prompt_tokens", [64, 53, 128])
 def test_a_prompt_chunk_in_one_pass_equals_its_blocks_one_by_one(backend, prompt_tokens):
-    """Prefill through the path's own kernels: a chunk of up to 64 prompt tokens as blocks of sixteen rows of ONE sequence
+    """Prefill through the path's own kernels: a chunk of up to 128 prompt tokens as blocks of sixteen rows of ONE sequence
     in one pass over the weights (block i's history ends where block i - 1's rows end; its keys and values are in the
     pages before any block attends) leaves the pools and the hidden rows of the same blocks run one step after the
     other, bit for bit."""
     print(f"case prompt chunk tokens={prompt_tokens}", flush=True)
     model = DenseModel(seed=17, hidden=1024, q_heads=16, kv_heads=8, head_dim=64, ffn=3072, vocabulary=32000, layers=3)
     rng = np.random.default_rng(4)
-    gpu = model.build_gpu(backend, max_lanes=4, context_tokens=[prompt_tokens + 300])
+    gpu = model.build_gpu(backend, max_lanes=(prompt_tokens + 15) // 16, context_tokens=[prompt_tokens + 300])
     model.seed_context(gpu, None, rng)
     first, committed = model.table_first[0], 250      # the chunk crosses a page
     prompt = rng.integers(0, 32000, prompt_tokens).astype(np.uint32)
@@ -318,3 +318,31 @@ def test_a_prompt_chunk_in_one_pass_equals_its_blocks_one_by_one(backend, prompt
     assert np.array_equal(gpu.buffer(verify.HIDDEN, 0).download(np.uint16, prompt_tokens * 1024), want_hidden)
     # fewer passes over the weights: a layer's dispatches once, not once a block
     assert len(graph) < len(gpu.encode([verify.Lane(16, committed, table_first=first)], commit=False)) 
+
+
+def test_eight_lanes_equal_each_lane_alone(backend):
+    """The driver's most lanes: eight lanes of unequal blocks and histories in one step give, lane by lane, the logits,
+    selections and acceptance each lane gives alone, bit for bit."""
+    print("case eight lanes", flush=True)
+    model = DenseModel(seed=19, hidden=1024, q_heads=16, kv_heads=8, head_dim=64, ffn=3072, vocabulary=32000, layers=2)
+    rng = np.random.default_rng(6)
+    rows = [16, 3, 9, 16, 1, 12, 16, 7]
+    contexts = [100 + 97 * i for i in range(8)]
+    gpu = model.build_gpu(backend, max_lanes=8, context_tokens=[c + 16 for c in contexts])
+    model.seed_context(gpu, None, rng)
+    lanes = [verify.Lane(r, c, table_first=f) for r, c, f in zip(rows, contexts, model.table_first)]
+    tokens = rng.integers(0, 32000, sum(rows)).astype(np.uint32)
+    gpu.set_block(lanes, tokens)
+    backend.run(gpu.encode(lanes, commit=False))
+    logits = gpu.buffer(verify.LOGITS).download(np.float32, sum(rows) * 32000).reshape(-1, 32000).copy()
+    selected, retained, accepted, mask = (np.array(a).copy() for a in gpu.results(lanes))
+    first = 0
+    for i, lane in enumerate(lanes):
+        gpu.set_block([lane], tokens[first:first + lane.rows])
+        backend.run(gpu.encode([lane], commit=False))
+        alone = gpu.buffer(verify.LOGITS).download(np.float32, lane.rows * 32000).reshape(-1, 32000)
+        assert np.array_equal(alone, logits[first:first + lane.rows]), i
+        s1, r1, a1, m1 = gpu.results([lane])
+        assert r1[0] == retained[i] and a1[0] == accepted[i] and m1[0] == mask[i], i
+        assert np.array_equal(np.asarray(s1)[:r1[0]], selected[first:first + r1[0]]), i
+        first += lane.rows
