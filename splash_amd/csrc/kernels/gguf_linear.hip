@@ -563,9 +563,14 @@ __device__ __forceinline__ void accumulate_record_staged(const Record<FMT> &rec,
 // 2 j + 1 up tile j, so the two halves of a pair sit in neighbouring waves of one workgroup.
 // `item` is the workgroup's place in the dispatch (blockIdx.x of gguf_decode).
 // A workgroup's LDS, which the kernel declares once whatever formats its workgroups decode.
+// The four-tile kernels keep ONE buffer of a super-block's activations (two barriers a super-block instead of one): at
+// 32 KiB instead of 64 a compute unit holds three of their workgroups, not two, which their waits on LDS and on the
+// weight stream need more than they need the barrier. `spare` extends the buffer for the epilogues that lay rows out in it.
 template <int RT> struct DecodeShared {
-  uint4 a[2][RT][8][64];
-  float sums[2][RT][4][64];
+  static constexpr int kBuffers = RT > 2 ? 1 : 2;
+  uint4 a[kBuffers][RT][8][64];
+  uint4 spare[RT > 2 ? 512 : 1];
+  float sums[kBuffers][RT][4][64];
   uint32_t arrived;
   float scaleParts[256 * RT], rowScale[16 * RT];  // of a table with a deferred scale
 };
@@ -1030,7 +1035,7 @@ __device__ __forceinline__ void decode_workgroup(DecodeShared<RT> &shared, const
     for (uint32_t round = 0; round < rounds; ++round) {
 #pragma unroll
       for (int u = 0; u < kStages; ++u, ++now) {
-        const uint32_t buffer = now & 1u;
+        const uint32_t buffer = DecodeShared<RT>::kBuffers == 2 ? (now & 1u) : 0u;
 #pragma unroll
         for (int j = 0; j < 2 * RT; ++j) (&ldsA[buffer][0][0][0])[threadIdx.x + 256u * j] = stage[u].a[j];
 #pragma unroll
@@ -1042,6 +1047,7 @@ __device__ __forceinline__ void decode_workgroup(DecodeShared<RT> &shared, const
           if constexpr (Staged) accumulate_record_staged<FMT, RT>(stage[u].rec, ldsA[buffer], acc, lane, kq);
           else accumulate_record<FMT, RT>(stage[u].rec, ldsA[buffer], ldsSums[buffer], acc, lane, kq);
         }
+        if constexpr (DecodeShared<RT>::kBuffers == 1) __syncthreads();   // every wave has read the buffer before the next super-block lands in it
       }
     }
   }
@@ -1106,7 +1112,8 @@ __device__ __forceinline__ void decode_workgroup(DecodeShared<RT> &shared, const
     // the staging buffers are free: the head's rows as floats, then a row a wave for the RoPE exchange
     float (*headRows)[128] = reinterpret_cast<float (*)[128]>(&ldsA[0][0][0][0]);
     float (*waveRows)[4][128] = reinterpret_cast<float (*)[4][128]>(reinterpret_cast<char *>(&ldsA[0][0][0][0]) + 16u * RT * 128u * 4u);
-    static_assert(sizeof(shared.a) >= 16u * RT * 128u * 4u + 4u * 4u * 128u * 4u, "the staging buffers hold a head's rows and a wave's four");
+    static_assert(sizeof(shared.a) + (RT > 2 ? sizeof(shared.spare) : 0u) >= 16u * RT * 128u * 4u + 4u * 4u * 128u * 4u,
+                  "the staging buffers hold a head's rows and a wave's four");
     const uint8_t *const seg[3] = {seg0, seg1, seg2};
     const uint32_t firstColumn = uint32_t(__builtin_amdgcn_readfirstlane(int(find_tile(headOf * halves * 4u, seg, p, kRecord).column)));
     const uint32_t rows = min(p.rows, 16u * RT);
@@ -1379,7 +1386,7 @@ __device__ __forceinline__ void decode_workgroup(DecodeShared<RT> &shared, const
 }
 
 template <uint32_t FMT, int RT, uint32_t EP, bool Staged = false>
-__global__ __launch_bounds__(256) void gguf_decode(const uint8_t *__restrict__ seg0, const uint8_t *__restrict__ seg1,
+__global__ __launch_bounds__(256, RT > 2 ? 3 : 1) void gguf_decode(const uint8_t *__restrict__ seg0, const uint8_t *__restrict__ seg1,
                                                    const uint8_t *__restrict__ seg2, const uint8_t *__restrict__ table,
                                                    void *__restrict__ out, const uint16_t *__restrict__ residual,
                                                    float *__restrict__ partials, uint32_t *__restrict__ counters,
