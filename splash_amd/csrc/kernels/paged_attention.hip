@@ -415,7 +415,16 @@ __global__ __launch_bounds__(256, 2) void attention_q8_split(const _Float16 *__r
   // Steps wholly inside the committed history come first, in a loop of their own.
   const uint32_t plain = first < seq.committed ? min(steps, (seq.committed - first) / kStep) : 0u;
   uint32_t step = 0;
+  // A SIMD holds one wave of each of a compute unit's two workgroups and issues the older one's instructions first, so
+  // the workgroup placed second runs every step behind the first and then finishes alone on an idle unit. The waves
+  // take turns instead: a wave's priority is up on the steps whose parity is its wave slot's.
+  const uint32_t slot = __builtin_amdgcn_s_getreg((3 << 11) | 4) & 1u;   // HW_ID's wave slot, bit 0
+  auto takeTurn = [&](uint32_t s) {
+    if ((s + slot) & 1u) __builtin_amdgcn_s_setprio(2);
+    else __builtin_amdgcn_s_setprio(0);
+  };
   for (; step < plain; ++step) {
+    takeTurn(step);
     const uint32_t buffer = step & 1u;
     if (step + 1 < steps) load(step + 1);
     compute(buffer, first + step * kStep, std::false_type{});
@@ -423,6 +432,7 @@ __global__ __launch_bounds__(256, 2) void attention_q8_split(const _Float16 *__r
     __syncthreads();
   }
   for (; step < steps; ++step) {
+    takeTurn(step);
     const uint32_t buffer = step & 1u;
     if (step + 1 < steps) load(step + 1);
     compute(buffer, first + step * kStep, std::true_type{});
