@@ -392,6 +392,41 @@ __device__ __forceinline__ TileRef find_tile(uint32_t index, const uint8_t *cons
 // One record's contribution to a wave's sums. `a` and `sums` are the workgroup's staged
 // activations of the record's super-block in LDS: a[t][g][lane] the MFMA operand of row tile t,
 // group g; sums[t][j][lane] the row sums of the j-th K = 4 MFMA.
+// acc[t] = fma(dot(step, t), scale(step), acc[t]) over a record's `Steps` steps in order, every row tile. With four row
+// tiles a step's products are issued before the multiply-adds of the step before it, so that those run while the matrix
+// cores work (each element's multiply-adds keep their order: the sums are the same).
+template <int RT, uint32_t Steps, class Dot, class Scale>
+__device__ __forceinline__ void scaled_groups(f32x4 (&acc)[RT], Dot dot, Scale scale) {
+  if constexpr (RT > 2) {
+    f32x4 held[2][RT];
+#pragma unroll
+    for (int t = 0; t < RT; ++t) held[0][t] = dot(0u, t);
+#pragma unroll
+    for (uint32_t j = 1; j <= Steps; ++j) {
+      if (j < Steps) {
+#pragma unroll
+        for (int t = 0; t < RT; ++t) held[j & 1u][t] = dot(j, t);
+      }
+      const float s = scale(j - 1u);
+#pragma unroll
+      for (int t = 0; t < RT; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[t][i] = __fmaf_rn(held[(j - 1u) & 1u][t][i], s, acc[t][i]);
+    }
+  } else {
+#pragma unroll
+    for (uint32_t j = 0; j < Steps; ++j) {
+      const float s = scale(j);
+#pragma unroll
+      for (int t = 0; t < RT; ++t) {
+        const f32x4 product = dot(j, t);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[t][i] = __fmaf_rn(product[i], s, acc[t][i]);
+      }
+    }
+  }
+}
+
 template <uint32_t FMT, int RT>
 __device__ __forceinline__ void accumulate_record(const Record<FMT> &rec, const uint4 (*a)[8][64], const float (*sums)[4][64],
                                                   f32x4 (&acc)[RT], uint32_t lane, uint32_t kq) {
@@ -418,16 +453,9 @@ __device__ __forceinline__ void accumulate_record(const Record<FMT> &rec, const 
       acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(sums[t][0][lane], c_lo, acc[t], 0, 0, 0);
       acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(sums[t][1][lane], c_hi, acc[t], 0, 0, 0);
     }
-#pragma unroll
-    for (uint32_t g = 0; g < 8; ++g) {
-      const bf16x8 b = as_bf16x8(ops[g]);
-#pragma unroll
-      for (int t = 0; t < RT; ++t) {
-        const f32x4 dot = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a[t][g][lane]), b, zero, 0, 0, 0);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) acc[t][i] = __fmaf_rn(dot[i], s[g], acc[t][i]);
-      }
-    }
+    scaled_groups<RT, 8>(acc, [&](uint32_t g, int t) {
+      return __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a[t][g][lane]), as_bf16x8(ops[g]), zero, 0, 0, 0);
+    }, [&](uint32_t g) { return s[g]; });
   } else if constexpr (FMT == GGUF_FMT_Q4K || FMT == GGUF_FMT_Q5K) {
     const Q4KScales sc = q4k_scales(rec.meta);
     float s[8];
@@ -442,16 +470,9 @@ __device__ __forceinline__ void accumulate_record(const Record<FMT> &rec, const 
       acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(sums[t][0][lane], c_lo, acc[t], 0, 0, 0);
       acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(sums[t][1][lane], c_hi, acc[t], 0, 0, 0);
     }
-#pragma unroll
-    for (uint32_t g = 0; g < 8; ++g) {
-      const bf16x8 b = as_bf16x8(ops[g]);
-#pragma unroll
-      for (int t = 0; t < RT; ++t) {
-        const f32x4 dot = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a[t][g][lane]), b, zero, 0, 0, 0);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) acc[t][i] = __fmaf_rn(dot[i], s[g], acc[t][i]);
-      }
-    }
+    scaled_groups<RT, 8>(acc, [&](uint32_t g, int t) {
+      return __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a[t][g][lane]), as_bf16x8(ops[g]), zero, 0, 0, 0);
+    }, [&](uint32_t g) { return s[g]; });
   } else {
     const float d = half_bits_to_float(rec.d);
     // Constant terms of 16-input blocks 4 j + kq: -160 d sc (operand 128 + q, value q - 32).
@@ -462,23 +483,14 @@ __device__ __forceinline__ void accumulate_record(const Record<FMT> &rec, const 
 #pragma unroll
       for (int t = 0; t < RT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(sums[t][j][lane], coef, acc[t], 0, 0, 0);
     }
-#pragma unroll
-    for (uint32_t g = 0; g < 8; ++g) {
-#pragma unroll
-      for (int t = 0; t < RT; ++t) {
-        const uint4 av = a[t][g][lane];
-#pragma unroll
-        for (uint32_t h = 0; h < 2; ++h) {
-          const float s = d * q6_scale(rec.scales, 2u * g + h);
-          const uint2 bw = h ? make_uint2(ops[g].z, ops[g].w) : make_uint2(ops[g].x, ops[g].y);
-          const uint2 aw = h ? make_uint2(av.z, av.w) : make_uint2(av.x, av.y);
-          const f32x4 dot = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4, aw),
-                                                                      __builtin_bit_cast(s16x4, bw), zero, 0, 0, 0);
-#pragma unroll
-          for (int i = 0; i < 4; ++i) acc[t][i] = __fmaf_rn(dot[i], s, acc[t][i]);
-        }
-      }
-    }
+    // a step is half a group: 16 inputs under one scale
+    scaled_groups<RT, 16>(acc, [&](uint32_t j, int t) {
+      const uint32_t g = j >> 1;
+      const uint4 av = a[t][g][lane];
+      const uint2 bw = j & 1u ? make_uint2(ops[g].z, ops[g].w) : make_uint2(ops[g].x, ops[g].y);
+      const uint2 aw = j & 1u ? make_uint2(av.z, av.w) : make_uint2(av.x, av.y);
+      return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4, aw), __builtin_bit_cast(s16x4, bw), zero, 0, 0, 0);
+    }, [&](uint32_t j) { return d * q6_scale(rec.scales, j); });
   }
 }
 
