@@ -227,6 +227,28 @@ def time_c2_ops(backend):
                             "frac": round(algorithmic / us / 1e3 / HBM_PEAK_GBS, 4)})
             log(f"  {name:8s} M={M:2d} splits={plan.splits:2d} {us:7.2f} us {algorithmic / us / 1e3:7.1f} GB/s")
             del graph, x, out, residual, scratch
+        # the column rule (every addition in the reference's order) at its one and two rows: a dispatch a tensor
+        for M in (1, 2):
+            x = backend.from_array(bf(rng.standard_normal((M, K))))
+            out, residual = backend.allocate_buffer(M * N * 4), backend.allocate_buffer(M * N * 2)
+            plan = linear.plan(ring[0], M, epilogue, column=True)
+            scratch = linear.scratch_for(backend, [plan])
+            graph = splash_amd.CommandGraph()
+            passes, each = 3, len(widths)
+            for _ in range(passes):
+                for c in range(copies):
+                    linear.add(graph, ring[c], plan, x, out, scratch, residual=residual, gate=gates[c] if gates else None)
+            backend.set_dispatch_profiling(True)
+            _, _, per = backend.run(graph, profiled=True)
+            backend.set_dispatch_profiling(False)
+            adds = np.array(per).reshape(passes * copies, each).sum(axis=1)
+            us = float(np.median(adds[copies:]) * 1e6)
+            algorithmic = weight_bytes + M * K * 2 + M * N * 2
+            results.append({"op": name, "rule": "column", "format": "q4_k" if fmt == ops.FMT_Q4K else "q6_k", "N": N * tensors if tensors == 2 else N,
+                            "K": K, "M": M, "dispatches": each, "us": round(us, 2), "GB/s": round(algorithmic / us / 1e3, 1),
+                            "frac": round(algorithmic / us / 1e3 / HBM_PEAK_GBS, 4)})
+            log(f"  {name:8s} M={M:2d} column rule {us:7.2f} us {algorithmic / us / 1e3:7.1f} GB/s ({each} dispatches)")
+            del graph, x, out, residual, scratch
         del ring, gates
     print(json.dumps({"metric": "projection us and GB/s by rows (config 2)", "unit": "us", "n_gpus": 1, "data": "synthetic: random images in a ring past the caches",
                       "roofline_peak_gbs": HBM_PEAK_GBS, "results": results}), flush=True)

@@ -67,7 +67,10 @@ typedef struct spo_linear_plan {
   /* LinearTile: 0 the register rule (exact 128 + code operands, one fp32 multiply-add a group;
    * linear_gguf_sgmatrix.metal:140-288), 1 the staged rule (weights decoded with fp32 group coefficients and rounded
    * once to half, products accumulated in fp32; kernels/common/gguf_staged.h:12-66, gguf_linear.metal:120-140): plain
-   * and residual plans of one format, set with spo_linear_plan_with. */
+   * and residual plans of one format, set with spo_linear_plan_with; 2 the column rule (LinearTile::GgufColumn,
+   * kernels/common/gguf_column_tile.h:25-68, kernels/decode/linear_gguf_column.metal:33-66; LinearGguf.cpp:141-147): one
+   * or two rows, unsplit, half weights and every addition in the reference's order, so the results are the reference's bit
+   * for bit; plain, residual and one-pass gate/up plans, a dispatch a tensor over the rows as they are. */
   uint32_t tile, reserved;
   uint64_t scratch_input, scratch_partials, scratch_counters; /* LinearPlan::scratchSize */
 } spo_linear_plan;

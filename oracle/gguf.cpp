@@ -347,6 +347,45 @@ int orc_gemm_staged(uint32_t fmt, const uint8_t *native, const uint16_t *x, uint
   return 0;
 }
 
+// The column tile's projection (kernels/common/gguf_column_tile.h:25-68, kernels/decode/linear_gguf_column.metal:33-66):
+// weights rounded once to half; per group of 32 one fp32 chain of its products in element order (each product of a
+// half and a bf16 is exact in fp32, so every step rounds once), added to the sum of its part of K; part s of eight holds
+// groups [s G / 8, (s + 1) G / 8); the parts are added in order. out[m][n] is that fp32 total, before any epilogue.
+int orc_gemv_column(uint32_t fmt, const uint8_t *native, const uint16_t *x, uint32_t M, uint32_t K, uint32_t N, float *out,
+                    int threads) {
+  const uint64_t rb = orc_row_bytes(fmt, K);
+  if (!rb) return -1;
+  const uint32_t G = K / 32, kParts = 8;
+  std::vector<float> xf(size_t(M) * K);
+  for (size_t i = 0; i < xf.size(); ++i) xf[i] = bf2f(x[i]);
+  parallelFor(N, threads, [&](uint32_t lo, uint32_t hi) {
+    std::vector<float> w(K);
+    for (uint32_t n = lo; n < hi; ++n) {
+      const uint8_t *row = native + n * rb;
+      for (uint32_t g = 0; g < G; ++g) groupValues(fmt, row, g, w.data() + 32 * g);
+      for (uint32_t k = 0; k < K; ++k) w[k] = h2f(f2h(w[k]));
+      for (uint32_t m = 0; m < M; ++m) {
+        const float *xr = xf.data() + size_t(m) * K;
+        float total = 0.0f;
+        for (uint32_t s = 0; s < kParts; ++s) {
+          float sums = 0.0f;
+          for (uint32_t g = s * G / kParts; g < (s + 1) * G / kParts; ++g) {
+            float sum = 0.0f;
+            for (uint32_t i = 0; i < 32; ++i) {
+              const float product = w[32 * g + i] * xr[32 * g + i];   // exact: 11 + 8 significant bits
+              sum = sum + product;
+            }
+            sums += sum;
+          }
+          total += sums;
+        }
+        out[size_t(m) * N + n] = total;
+      }
+    }
+  });
+  return 0;
+}
+
 int orc_gemm(uint32_t fmt, const uint8_t *native, const uint16_t *x, uint32_t M, uint32_t K, uint32_t N,
              double *exact, double *bound, float *chain, int threads) {
   const uint64_t rb = orc_row_bytes(fmt, K);

@@ -81,6 +81,12 @@ int orc_gemm(uint32_t fmt, const uint8_t *native, const uint16_t *x, uint32_t M,
 // Pinned by the reference's own dot and projectionBound (oracle/_ref) and numpy's float16 rounding of orc_dequant_rows.
 int orc_gemm_staged(uint32_t fmt, const uint8_t *native, const uint16_t *x, uint32_t M, uint32_t K, uint32_t N,
                     double *exact, double *bound, float *staged, double *accumulation, int threads);
+// The column tile's fp32 totals out[M][N] (kernels/common/gguf_column_tile.h:25-68, linear_gguf_column.metal:33-66):
+// half weights, a group's 32 products added in element order, groups added to their part of K (eight parts of
+// G / 8 groups, by integer division of s G), the parts added in order. Pinned by closed forms that only this order
+// satisfies (tests/test_oracle_gguf.py) and by the staged interval of orc_gemm_staged.
+int orc_gemv_column(uint32_t fmt, const uint8_t *native, const uint16_t *x, uint32_t M, uint32_t K, uint32_t N, float *out,
+                    int threads);
 // Epilogues on fp32 sums (kernels/common/gguf_tile.h:10-16, gguf_linear.metal:34-71).
 uint16_t orc_epilogue_plain(float v);
 uint16_t orc_epilogue_residual(float v, uint16_t residual);

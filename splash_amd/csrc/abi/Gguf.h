@@ -190,6 +190,19 @@ struct GgufPrefillParams {
   uint32_t reserved[3];
 };
 
+// gguf_column_<fmt>_{a,a_f32,r,g}: one or two rows under the reference's column rule (its GgufColumnParams,
+// metal/abi/Gguf.h:45-55; GGUF_COLUMN_SPLITS parts of K there and here). Binds the tensor's image, a one-pass gate/up's
+// up image (the first is the gate's; the tensor's again otherwise), the rows (bf16 [rows][input_size]), out and the
+// residual rows (any buffer when unused). Grid (the tensor's 16-column tiles), 512 threads.
+#define GGUF_COLUMN_ROWS 2u
+struct GgufColumnParams {
+  uint32_t rows;        // 1 to GGUF_COLUMN_ROWS
+  uint32_t input_size;
+  uint32_t out_stride;  // elements between output (and residual) rows
+  uint32_t out_offset;  // the tensor's first output column
+  uint32_t reserved[4];
+};
+
 // Epilogues of a decode projection (the reference's LinearEpilogue, runtime/ops/Linear.hpp:77).
 #define GGUF_EPILOGUE_PLAIN 0u     // out = bf16(v)         kernel suffix _a
 #define GGUF_EPILOGUE_PLAIN_F32 1u // out = v               kernel suffix _a_f32

@@ -18,8 +18,8 @@ ops::LinearPlan toPlan(const ops::Projection &projection, const spo_linear_plan 
   ops::LinearConfig config;
   config.splits = p.splits;
   config.wholeGroups = p.whole_groups;
-  if (p.tile > 1) throw std::invalid_argument("unknown linear tile");
-  config.tile = p.tile ? ops::LinearTile::GgufStaged : ops::LinearTile::GgufMfma;
+  if (p.tile > 2) throw std::invalid_argument("unknown linear tile");
+  config.tile = static_cast<ops::LinearTile>(p.tile);
   return ops::Linear::plan(ops::workloadOf(projection, p.rows, static_cast<ops::LinearEpilogue>(p.epilogue)), config,
                            p.float32 ? ops::FloatOutput::Float32 : ops::FloatOutput::BFloat16);
 }
@@ -31,7 +31,7 @@ void fromPlan(const ops::LinearPlan &plan, spo_linear_plan *out) {
   out->whole_groups = plan.configuration().wholeGroups;
   out->storage_rows = plan.storageRows();
   out->float32 = plan.destination() == ops::FloatOutput::Float32;
-  out->tile = plan.configuration().tile == ops::LinearTile::GgufStaged ? 1u : 0u;
+  out->tile = uint32_t(plan.configuration().tile);
   out->reserved = 0;
   out->scratch_input = size.input;
   out->scratch_partials = size.partials;

@@ -526,11 +526,11 @@ template <uint32_t FMT> struct StagedCoefficients {
     if constexpr (FMT == GGUF_FMT_Q6K) d6 = half_bits_to_float(rec.d);
   }
 };
+// A group's eight values of this lane in fp32, element e the lane's input gguf_operand_input(kq, e).
 template <uint32_t FMT>
-__device__ __forceinline__ void staged_group(const Record<FMT> &rec, const StagedCoefficients<FMT> &k, const uint4 &operand, uint32_t g,
-                                             bf16x8 &high, bf16x8 &low) {
+__device__ __forceinline__ void staged_values(const Record<FMT> &rec, const StagedCoefficients<FMT> &k, const uint4 &operand, uint32_t g,
+                                              float (&value)[8]) {
   const uint32_t regs[4] = {operand.x, operand.y, operand.z, operand.w};
-  float value[8];
   // the fp32 values of gguf_dequant, each exact or rounded once
   if constexpr (FMT == GGUF_FMT_Q80 || FMT == GGUF_FMT_IQ4XS || FMT == GGUF_FMT_IQ4NL) {
     const float d = group_scale(rec, g);
@@ -547,6 +547,12 @@ __device__ __forceinline__ void staged_group(const Record<FMT> &rec, const Stage
     for (uint32_t e = 0; e < 8; ++e)
       value[e] = (k.d6 * q6_scale(rec.scales, 2u * g + (e >> 2))) * float(int(operand_code(regs[e >> 1], e & 1u) & 0x3Fu) - 32);
   }
+}
+template <uint32_t FMT>
+__device__ __forceinline__ void staged_group(const Record<FMT> &rec, const StagedCoefficients<FMT> &k, const uint4 &operand, uint32_t g,
+                                             bf16x8 &high, bf16x8 &low) {
+  float value[8];
+  staged_values(rec, k, operand, g, value);
   staged_operands(value, high, low);
 }
 template <uint32_t FMT, int RT>
@@ -1717,6 +1723,152 @@ SP_GGUF_DECODE("iq4xs", GGUF_FMT_IQ4XS, 64, 4);
 SP_GGUF_DECODE("iq4nl", GGUF_FMT_IQ4NL, 16, 1);
 SP_GGUF_DECODE("iq4nl", GGUF_FMT_IQ4NL, 32, 2);
 SP_GGUF_DECODE("iq4nl", GGUF_FMT_IQ4NL, 64, 4);
+
+// ---------------------------------------------------------------------------------------------
+// gguf_column_<fmt>_{a,a_f32,r,g}: one or two rows under the reference's column rule (kernels/common/gguf_column_tile.h:25-68,
+// kernels/decode/linear_gguf_column.metal:33-66), whose every addition is ordered, so the results are the reference's
+// bit for bit: each weight rounded once to half (the staged rule's), a group's 32 products with the row added one after
+// the other in input order (each product exact in fp32), the group's sum added to the sum of its part of K, the eight
+// parts -- groups [s G / 8, (s + 1) G / 8) of G = K / 32 -- added in order, then the epilogue.
+// A workgroup (512 threads) owns one 16-column tile; wave s sums part s. A wave decodes a record in the image's lane
+// order (lane (c, kq) holds inputs gguf_operand_input(kq, 0..7) of each group of column c), lays the halves out in LDS
+// by input, and lane (c, q) then runs the chains of groups 2 q and 2 q + 1 of column c; the part's running sum passes
+// from q to q + 1 (and from 3 to the next record's 0), so groups are added in order. The rows are read as they are
+// (bf16 [rows][K]): no activation table. Grid (the tensor's column tiles); of a one-pass gate/up, a workgroup sums
+// tile t of both tensors.
+// ---------------------------------------------------------------------------------------------
+constexpr uint32_t kColumnParts = 8u;       // the reference's GGUF_COLUMN_SPLITS
+constexpr uint32_t kColumnStride = 8u * 32u + 8u;  // halves of a column's record in LDS: eight groups and a pad against bank conflicts
+struct ColumnShared {
+  _Float16 weights[kColumnParts][16][kColumnStride];
+  float parts[kColumnParts][2][GGUF_COLUMN_ROWS][16];
+};
+template <uint32_t FMT, uint32_t EP>
+__global__ __launch_bounds__(512, 4) void gguf_column(const uint8_t *__restrict__ image, const uint8_t *__restrict__ upImage,
+                                                        const uint16_t *__restrict__ input, void *__restrict__ out,
+                                                        const uint16_t *__restrict__ residual, GgufColumnParams p) {
+  constexpr bool kGateUp = EP == GGUF_EPILOGUE_GATE_UP;
+  constexpr uint32_t kTensors = kGateUp ? 2u : 1u, kRecord = gguf_record_bytes(FMT);
+  __shared__ ColumnShared shared;
+  const uint32_t lane = threadIdx.x & 63u, part = threadIdx.x >> 6, c = lane & 15u, kq = lane >> 4;
+  const uint32_t blocks = p.input_size / GGUF_BLOCK, G = p.input_size / 32u;
+  const uint32_t first = uint32_t(__builtin_amdgcn_readfirstlane(int(part * G / kColumnParts)));
+  const uint32_t last = uint32_t(__builtin_amdgcn_readfirstlane(int((part + 1u) * G / kColumnParts)));
+  float running[kTensors][GGUF_COLUMN_ROWS];
+#pragma unroll
+  for (uint32_t t = 0; t < kTensors; ++t)
+#pragma unroll
+    for (uint32_t r = 0; r < GGUF_COLUMN_ROWS; ++r) running[t][r] = 0.f;
+  _Float16 (*mine)[kColumnStride] = shared.weights[part];
+  for (uint32_t b = first / 8u; 8u * b < last; ++b) {
+#pragma unroll
+    for (uint32_t t = 0; t < kTensors; ++t) {
+      const uint8_t *tensor = (t ? upImage : image) + (size_t(blockIdx.x) * blocks + b) * kRecord;
+      const Resource weights = make_resource(tensor, kRecord);
+      Record<FMT> rec;
+      load_record(rec, weights, 16u * lane, Cursor<FMT>::kColumnPart + 16u * c);
+      uint4 ops[8];
+      record_operands(rec, ops);
+      const StagedCoefficients<FMT> k(rec);
+#pragma unroll
+      for (uint32_t g = 0; g < 8; ++g) {
+        if (8u * b + g < first || 8u * b + g >= last) continue;   // the whole wave: a group of another part
+        float value[8];
+        staged_values(rec, k, ops[g], g, value);
+        _Float16 h[8];
+#pragma unroll
+        for (uint32_t e = 0; e < 8; ++e) h[e] = _Float16(value[e]);
+        // elements 0..3 are inputs 4 kq + {0, 2, 1, 3}, elements 4..7 those + 16
+        typedef __attribute__((ext_vector_type(4))) _Float16 f16x4;
+        *reinterpret_cast<f16x4 *>(&mine[c][32u * g + 4u * kq]) = f16x4{h[0], h[2], h[1], h[3]};
+        *reinterpret_cast<f16x4 *>(&mine[c][32u * g + 16u + 4u * kq]) = f16x4{h[4], h[6], h[5], h[7]};
+      }
+      // the wave's own writes, read back by its own lanes: no other wave touches this part's rows
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0)
+      __builtin_amdgcn_wave_barrier();
+      float chain[2][GGUF_COLUMN_ROWS];
+      bool active[2];
+#pragma unroll
+      for (uint32_t j = 0; j < 2; ++j) {
+        const uint32_t g = 2u * kq + j, group = 8u * b + g;
+        active[j] = group >= first && group < last;
+#pragma unroll
+        for (uint32_t r = 0; r < GGUF_COLUMN_ROWS; ++r) chain[j][r] = 0.f;
+        if (!active[j]) continue;
+        typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
+        f16x8 w[4];
+#pragma unroll
+        for (uint32_t v = 0; v < 4; ++v) w[v] = *reinterpret_cast<const f16x8 *>(&mine[c][32u * g + 8u * v]);
+#pragma unroll
+        for (uint32_t r = 0; r < GGUF_COLUMN_ROWS; ++r) {
+          if (r >= p.rows) break;
+          const uint4 *x = reinterpret_cast<const uint4 *>(input + size_t(r) * p.input_size + 32u * group);
+          float sum = 0.f;
+#pragma unroll
+          for (uint32_t v = 0; v < 4; ++v) {
+            const uint4 q = x[v];
+            const uint32_t words[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+            for (uint32_t i = 0; i < 8; ++i)
+              sum = __fmaf_rn(float(w[v][i]), bf16_bits_to_float((words[i >> 1] >> (16u * (i & 1u))) & 0xFFFFu), sum);
+          }
+          chain[j][r] = sum;
+        }
+      }
+      // every lane has read the record's halves before the next record's land
+      __builtin_amdgcn_wave_barrier();
+      // the part's sum so far passes through the lanes of a column in group order
+#pragma unroll
+      for (uint32_t q = 0; q < 4; ++q) {
+#pragma unroll
+        for (uint32_t r = 0; r < GGUF_COLUMN_ROWS; ++r) {
+          const float incoming = __shfl(running[t][r], int((lane + 48u) & 63u), 64);
+          if (kq == q) {
+            float sum = incoming;
+            if (active[0]) sum += chain[0][r];
+            if (active[1]) sum += chain[1][r];
+            running[t][r] = sum;
+          }
+        }
+      }
+    }
+  }
+  if (kq == 3u) {
+#pragma unroll
+    for (uint32_t t = 0; t < kTensors; ++t)
+#pragma unroll
+      for (uint32_t r = 0; r < GGUF_COLUMN_ROWS; ++r) shared.parts[part][t][r][c] = running[t][r];
+  }
+  __syncthreads();
+  if (threadIdx.x >= 16u * GGUF_COLUMN_ROWS) return;
+  const uint32_t r = threadIdx.x >> 4, column = threadIdx.x & 15u;
+  if (r >= p.rows) return;
+  float total[kTensors];
+#pragma unroll
+  for (uint32_t t = 0; t < kTensors; ++t) {
+    total[t] = 0.f;
+    for (uint32_t s = 0; s < kColumnParts; ++s) total[t] += shared.parts[s][t][r][column];
+  }
+  const size_t at = size_t(r) * p.out_stride + p.out_offset + 16u * blockIdx.x + column;
+  if constexpr (kGateUp)   // the first tensor is the gate's
+    static_cast<uint16_t *>(out)[at] = uint16_t(float_to_bf16_bits(round_bf16(total[1]) * silu(round_bf16(total[0]))));
+  else if constexpr (EP == GGUF_EPILOGUE_PLAIN_F32) static_cast<float *>(out)[at] = total[0];
+  else if constexpr (EP == GGUF_EPILOGUE_RESIDUAL)
+    static_cast<uint16_t *>(out)[at] = uint16_t(float_to_bf16_bits(total[0] + bf16_bits_to_float(residual[at])));
+  else static_cast<uint16_t *>(out)[at] = uint16_t(float_to_bf16_bits(total[0]));
+}
+#define SP_GGUF_COLUMN(fmt, FMT)                                                                   \
+  SP_REGISTER_KERNEL("gguf_column_" fmt "_a", &gguf_column<FMT, GGUF_EPILOGUE_PLAIN>);             \
+  SP_REGISTER_KERNEL("gguf_column_" fmt "_a_f32", &gguf_column<FMT, GGUF_EPILOGUE_PLAIN_F32>);     \
+  SP_REGISTER_KERNEL("gguf_column_" fmt "_r", &gguf_column<FMT, GGUF_EPILOGUE_RESIDUAL>);          \
+  SP_REGISTER_KERNEL("gguf_column_" fmt "_g", &gguf_column<FMT, GGUF_EPILOGUE_GATE_UP>)
+SP_GGUF_COLUMN("q4k", GGUF_FMT_Q4K);
+SP_GGUF_COLUMN("q6k", GGUF_FMT_Q6K);
+SP_GGUF_COLUMN("q5k", GGUF_FMT_Q5K);
+SP_GGUF_COLUMN("q80", GGUF_FMT_Q80);
+SP_GGUF_COLUMN("iq4xs", GGUF_FMT_IQ4XS);
+SP_GGUF_COLUMN("iq4nl", GGUF_FMT_IQ4NL);
 
 // ---------------------------------------------------------------------------------------------
 // gguf_prefill_<fmt>_{a,a_f32,r}: the staged rule over a chunk of many rows (the reference's prefill tile,

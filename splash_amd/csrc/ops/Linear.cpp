@@ -75,9 +75,12 @@ void LinearPlan::requireConfiguration() const {
   if (c.wholeGroups > groupsOf(n, workload_.epilogue)) throw std::invalid_argument("more whole workgroups than the projection has");
   if (destination_ == FloatOutput::Float32 && workload_.epilogue != LinearEpilogue::None)
     throw std::invalid_argument("only a plain block plan writes fp32");
-  if (workload_.severalFormats &&
+  if (workload_.severalFormats && c.tile != LinearTile::GgufColumn &&
       (workload_.epilogue != LinearEpilogue::None || destination_ != FloatOutput::BFloat16 || c.wholeGroups || n % 64))
     throw std::invalid_argument("segments of several formats take a plain bf16 plan whose workgroups all partition K");
+  if (c.tile == LinearTile::GgufColumn &&
+      (workload_.rows > GGUF_COLUMN_ROWS || c.splits != 1 || c.wholeGroups || workload_.epilogue == LinearEpilogue::ResidualNorm))
+    throw std::invalid_argument("the column tile takes up to two rows, unsplit, and does not norm its rows");
   if (c.tile == LinearTile::GgufStaged &&
       (workload_.severalFormats || (workload_.epilogue != LinearEpilogue::None && workload_.epilogue != LinearEpilogue::Residual)))
     throw std::invalid_argument("the staged rule takes plain and residual plans of one format");
@@ -179,11 +182,45 @@ struct Linear::Resolved {
 PreparedInput Linear::add(hip::CommandGraph &graph, LinearBuffers b, const Projection &p, const LinearPlan &plan,
                           const Projection *gate) const {
   const LinearWorkload w = plan.workload();
+  if (plan.configuration().tile == LinearTile::GgufColumn) return addColumn(graph, std::move(b), p, plan, gate);
   const hip::Buffer input = b.input, table = b.scratch.input;
   const Resolved r = resolve(std::move(b), p, plan, gate);
   if (!r.prepared) addPrepare(graph, input, LinearScratch{table, {}, {}}, w.matrix.inputSize, w.rows);
   graph.add(r.kernel, {r.buffers.begin(), r.buffers.end()}, r.params, {r.items, r.pieces, 1}, {256, 1, 1});
   return r.after;
+}
+
+// The column tile: a dispatch a tensor, each of its own format, over the rows as they are (the reference's
+// Linear::addGgufColumn, LinearGguf.cpp:508-520).
+PreparedInput Linear::addColumn(hip::CommandGraph &graph, LinearBuffers b, const Projection &p, const LinearPlan &plan,
+                                const Projection *gate) const {
+  const LinearWorkload w = plan.workload();
+  const auto [n, k] = w.matrix;
+  requireSegments(p, w.matrix);
+  const bool gateUp = w.epilogue == LinearEpilogue::GateUp, residual = w.epilogue == LinearEpilogue::Residual;
+  if (gateUp != (gate != nullptr)) throw std::invalid_argument("a block gate/up plan takes a gate projection, no other does");
+  if (gate) {
+    requireSegments(*gate, w.matrix);
+    if (p.blocks().segments.size() != 1 || gate->blocks().segments.size() != 1 ||
+        gate->blocks().segments.front().formatId != p.blocks().segments.front().formatId)
+      throw std::invalid_argument("a one-pass block gate/up takes single tensors of one format");
+  }
+  const bool float32 = plan.destination() == FloatOutput::Float32;
+  requireBytes(b.input, uint64_t{w.rows} * k * 2, "projection input");
+  requireBytes(b.output, uint64_t{w.rows} * n * (float32 ? 4 : 2), "projection output");
+  if (residual) requireBytes(b.residual, uint64_t{w.rows} * n * 2, "projection residual");
+  for (const QuantizedSegment &s : p.blocks().segments) {
+    GgufColumnParams params{};
+    params.rows = w.rows;
+    params.input_size = k;
+    params.out_stride = n;
+    params.out_offset = s.columnOffset;
+    const hip::Buffer &image = gate ? gate->blocks().segments.front().image : s.image;
+    graph.add(std::string("gguf_column_") + s.name() + (gateUp ? "_g" : residual ? "_r" : float32 ? "_a_f32" : "_a"),
+              {image, s.image, b.input, b.output, residual ? b.residual : b.output}, params, {s.outputSize / GGUF_TILE_COLUMNS, 1, 1},
+              {512, 1, 1});
+  }
+  return {b.input, LinearInput::Plain};
 }
 
 Linear::Resolved Linear::resolve(LinearBuffers b, const Projection &p, const LinearPlan &plan, const Projection *gate) const {

@@ -35,7 +35,10 @@ enum class LinearEpilogue : uint8_t { None, Residual, GateUp, ResidualNorm };
 // 128 + code, one fp32 multiply-add a group; the reference's Apple9 register tile), and GgufStaged, the staged rule
 // (every weight decoded with fp32 group coefficients and rounded once to half, the products accumulated in fp32; the
 // reference's staged tile, kernels/common/gguf_staged.h:12-66), which takes plain and residual plans of one format.
-enum class LinearTile : uint8_t { GgufMfma, GgufStaged };
+// GgufColumn: a plan of one or two rows under the reference's column rule (kernels/common/gguf_column_tile.h:25-68:
+// half weights, every addition in a fixed order, eight parts of K), whose results are the reference's bit for bit;
+// unsplit, every epilogue but the norming one, a dispatch a tensor. It reads the rows as they are, no activation table.
+enum class LinearTile : uint8_t { GgufMfma, GgufStaged, GgufColumn };
 inline constexpr uint32_t kMaximumDecodeTileRows = GGUF_MAXIMUM_ROWS;
 // A dispatch of more rows runs pieces of kMaximumDecodeTileRows rows side by side.
 inline constexpr uint32_t kMaximumDispatchRows = GGUF_MAXIMUM_DISPATCH_ROWS;
@@ -242,6 +245,8 @@ public:
 
 private:
   struct Resolved;
+  PreparedInput addColumn(hip::CommandGraph &graph, LinearBuffers buffers, const Projection &projection, const LinearPlan &plan,
+                          const Projection *gate) const;
   [[nodiscard]] Resolved resolve(LinearBuffers buffers, const Projection &projection, const LinearPlan &plan,
                                  const Projection *gate) const;
   KernelCalibration calibration_;

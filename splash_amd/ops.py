@@ -106,10 +106,15 @@ class Linear:
         except Exception:
             pass
 
-    def plan(self, projection, rows, epilogue=EPILOGUE_NONE, splits=None, whole_groups=None, staged=False):
+    def plan(self, projection, rows, epilogue=EPILOGUE_NONE, splits=None, whole_groups=None, staged=False, column=False):
         """staged: the plan runs the staged rule (weights rounded once to half, products accumulated in fp32) instead of
-        the register rule."""
+        the register rule. column: the plan (one or two rows) runs the column rule, every addition in a fixed order."""
         p = nat.LinearPlan()
+        if column:
+            p.rows, p.epilogue, p.float32 = rows, epilogue, int(projection.float32 and epilogue == EPILOGUE_NONE)
+            p.splits, p.whole_groups, p.tile = 1, 0, 2
+            check(lib.spo_linear_plan_with(projection.handle, ctypes.byref(p)))
+            return p
         check(lib.spo_linear_plan_for(self.handle, projection.handle, rows, epilogue, ctypes.byref(p)))
         if splits is not None or whole_groups is not None or staged:
             if splits is not None:

@@ -122,6 +122,15 @@ def gemm_staged(fmt, native, x_bf16, N, threads=0):
     return dict(exact=exact, bound=bound, staged=staged, accumulation=accumulation)
 
 
+def gemv_column(fmt, native, x_bf16, N, threads=0):
+    """The column tile's fp32 totals [M][N]: every addition in the reference's order."""
+    x = np.ascontiguousarray(x_bf16, dtype=np.uint16)
+    M, K = x.shape
+    out = np.empty((M, N), dtype=np.float32)
+    assert lib.orc_gemv_column(c_u32(fmt), _p(native, u8p), _p(x, u16p), c_u32(M), c_u32(K), c_u32(N), _p(out, f32p), c_int(threads)) == 0
+    return out
+
+
 def rms_norm(x_bf16, w_bf16):
     x = np.ascontiguousarray(x_bf16, dtype=np.uint16)
     w = np.ascontiguousarray(w_bf16, dtype=np.uint16)

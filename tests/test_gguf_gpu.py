@@ -501,3 +501,88 @@ def test_the_staged_rule_takes_plain_and_residual_plans_of_one_format(backend):
                                                  (ops.FMT_Q6K, 64, orc.make_native(ops.FMT_Q6K, 64, K, 3))], K)
     with pytest.raises(splash_amd.SplashError):
         linear.plan(mixed, 16, staged=True)
+
+
+def run_column(backend, linear, segments, K, x_bits, epilogue=ops.EPILOGUE_NONE, float32=False, residual_bits=None, gate=None):
+    """segments: (format, columns, native rows) of the projection's tensors. The column tile reads the rows as they are."""
+    M = x_bits.shape[0]
+    proj = ops.Projection.from_native(backend, segments, K, float32=float32)
+    gate_proj = ops.Projection.from_native(backend, [gate], K) if gate is not None else None
+    N = proj.output_size
+    plan = linear.plan(proj, M, epilogue, column=True)
+    assert plan.tile == 2 and plan.splits == 1
+    scratch = linear.scratch_for(backend, [plan])
+    out = backend.allocate_buffer(M * N * (4 if float32 else 2), label="out")
+    out.fill(0xEE)
+    res = backend.from_array(residual_bits, label="residual") if residual_bits is not None else None
+    graph = splash_amd.CommandGraph()
+    linear.add(graph, proj, plan, backend.from_array(x_bits, label="x"), out, scratch, residual=res, gate=gate_proj)
+    assert len(graph) == len(segments)      # a dispatch a tensor and no table pass
+    backend.run(graph)
+    return out.download(np.float32 if float32 else np.uint16).reshape(M, N)
+
+
+@pytest.mark.parametrize("fmt", ALL_FORMATS)
+@pytest.mark.parametrize("M,K", [(1, 1280), (2, 2048), (2, 5120), (1, 256)])
+def test_the_column_tile_adds_in_the_reference_order(backend, fmt, M, K):
+    """linear_gguf_column.metal:33-66 and gguf_column_tile.h:25-68 fix every addition of a column's sum, so the fp32
+    totals are the oracle's bit for bit (K = 1280 and 256: parts that end inside a super-block, parts of less than a
+    group's worth), and the epilogues those of the tiles on them."""
+    print(f"case column tile fmt={fmt} M={M} K={K}", flush=True)
+    rng = np.random.default_rng(K + M)
+    N = 80
+    native = orc.make_native(fmt, N, K, 17 + M)
+    x = orc.f32_to_bf16(rng.standard_normal((M, K)).astype(np.float32))
+    linear = ops.Linear(backend)
+    want = orc.gemv_column(fmt, native, x, N)
+    got32 = run_column(backend, linear, [(fmt, N, native)], K, x, float32=True)
+    assert got32.tobytes() == want.tobytes(), int((got32 != want).sum())
+    got = run_column(backend, linear, [(fmt, N, native)], K, x)
+    assert np.array_equal(got, orc.f32_to_bf16(want))
+    res = orc.f32_to_bf16(rng.standard_normal((M, N)).astype(np.float32))
+    got = run_column(backend, linear, [(fmt, N, native)], K, x, epilogue=ops.EPILOGUE_RESIDUAL, residual_bits=res)
+    assert np.array_equal(got, orc.f32_to_bf16(want + orc.bf16_to_f32(res)))
+    gate_native = orc.make_native(fmt, N, K, 18 + M)
+    pair = run_column(backend, linear, [(fmt, N, native)], K, x, epilogue=ops.EPILOGUE_GATE_UP, gate=(fmt, N, gate_native))
+    swiglu = orc.swiglu(orc.gemv_column(fmt, gate_native, x, N), want)
+    diff = np.abs(pair.astype(np.int32) - swiglu.astype(np.int32))   # exp2's last bits differ between the CPU and the GPU
+    assert diff.max() <= 1 and (diff > 0).mean() < 0.02, (diff.max(), (diff > 0).mean())
+
+
+def test_the_column_tile_takes_a_format_a_tensor_and_closed_forms(backend):
+    """A fused projection's tensors, each of its own format, are a dispatch each at their columns; and the closed forms
+    that pin the oracle's order hold on the GPU: 2^24 then ones in a group, ones then 2^24."""
+    print("case column tile segments", flush=True)
+    rng = np.random.default_rng(3)
+    K, M = 2304, 2
+    parts = [(ops.FMT_Q4K, 64, orc.make_native(ops.FMT_Q4K, 64, K, 1)), (ops.FMT_Q6K, 16, orc.make_native(ops.FMT_Q6K, 16, K, 2)),
+             (ops.FMT_IQ4XS, 32, orc.make_native(ops.FMT_IQ4XS, 32, K, 3))]
+    x = orc.f32_to_bf16(rng.standard_normal((M, K)).astype(np.float32))
+    linear = ops.Linear(backend)
+    got = run_column(backend, linear, parts, K, x, float32=True)
+    want = np.concatenate([orc.gemv_column(f, nat, x, n) for f, n, nat in parts], axis=1)
+    assert got.tobytes() == want.tobytes()
+    # Q8_0 rows of ones under a scale of one: a block is the fp16 scale and 32 codes
+    K = 256
+    blocks = np.zeros((16, K // 32, 34), dtype=np.uint8)
+    blocks[:, :, :2] = np.frombuffer(np.float16(1.0).tobytes(), dtype=np.uint8)
+    blocks[:, :, 2:] = 1
+    native = np.ascontiguousarray(blocks.reshape(16, -1))
+    values = np.zeros((2, K), dtype=np.float32)
+    values[:, :32] = 1.0
+    values[0, 0] = 2.0 ** 24      # row 0: the ones after it are lost
+    values[1, 31] = 2.0 ** 24     # row 1: 31 first, then 2^24 + 31 rounds to 2^24 + 32
+    got = run_column(backend, linear, [(ops.FMT_Q80, 16, native)], K, orc.f32_to_bf16(values), float32=True)
+    assert np.all(got[0] == 2.0 ** 24) and np.all(got[1] == 2.0 ** 24 + 32)
+
+
+def test_the_column_tile_rejects_what_it_does_not_run(backend):
+    linear = ops.Linear(backend)
+    K, N = 512, 32
+    proj = ops.Projection.from_native(backend, [(ops.FMT_Q4K, N, orc.make_native(ops.FMT_Q4K, N, K, 1))], K)
+    with pytest.raises(splash_amd.SplashError):
+        linear.plan(proj, 3, column=True)                      # more than two rows
+    plan = linear.plan(proj, 2, column=True)
+    plan.splits = 2
+    with pytest.raises(splash_amd.SplashError):
+        ops.check(ops.lib.spo_linear_plan_with(proj.handle, ops.ctypes.byref(plan)))     # a partition of K

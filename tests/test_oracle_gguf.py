@@ -115,3 +115,88 @@ def test_staged_projection_is_the_half_rounded_weights_and_the_reference_bound(f
         orc.ref.ref_dot_bound(orc._p(xr, orc.f32p), orc._p(wr, orc.f32p), K, orc.ctypes.byref(value), orc.ctypes.byref(plain_bound))
         assert value.value == r["exact"][m, n]
         assert staged_bound.value == r["bound"][m, n] and plain_bound.value == r["accumulation"][m, n]
+
+
+# ---- the column tile's order (orc_gemv_column; kernels/common/gguf_column_tile.h:25-68) ----
+def q80_rows(codes, d=1.0):
+    """Q8_0 native rows of int8 codes [N][K] under one scale d: a block is the fp16 scale, then 32 codes."""
+    codes = np.asarray(codes, dtype=np.int8)
+    N, K = codes.shape
+    blocks = np.zeros((N, K // 32, 34), dtype=np.uint8)
+    blocks[:, :, :2] = np.frombuffer(np.float16(d).tobytes(), dtype=np.uint8)
+    blocks[:, :, 2:] = codes.reshape(N, K // 32, 32).view(np.uint8)
+    return np.ascontiguousarray(blocks.reshape(N, -1))
+
+
+def column_total(codes, x, d=1.0):
+    x_bits = orc.f32_to_bf16(np.asarray(x, dtype=np.float32)[None, :])
+    assert np.array_equal(orc.bf16_to_f32(x_bits)[0], np.asarray(x, dtype=np.float32))   # the inputs are bf16 numbers
+    return float(orc.gemv_column(orc.FMT_Q80, q80_rows(np.asarray(codes)[None, :], d), x_bits, 1)[0, 0])
+
+
+def test_the_column_rule_adds_a_group_in_element_order():
+    """Weights 1, one input 2^24 and 31 inputs 1 in a group: added in element order after 2^24 every 1 is lost (a tie
+    rounds to the even 2^24); with 2^24 last the ones make 31 first and 2^24 + 31 rounds to 2^24 + 32. A pairwise or
+    reversed order gives the other number in each case."""
+    K = 256
+    ones = np.zeros(K, dtype=np.int8)
+    ones[:32] = 1
+    x = np.zeros(K, dtype=np.float32)
+    x[:32] = 1.0
+    x[0] = 2.0 ** 24
+    assert column_total(ones, x) == 2.0 ** 24
+    x[0], x[31] = 1.0, 2.0 ** 24
+    assert column_total(ones, x) == 2.0 ** 24 + 32
+
+
+def test_the_column_rule_restarts_its_chain_every_group_and_sums_parts_apart():
+    """K = 1280: eight parts of five groups, so parts end inside super-blocks. Group 0 sums to 2^24 and each later group of
+    its part holds 32 ones: a chain that ran on through the groups would lose every one, a chain a group adds 32 a
+    group. Then a one in each group of part 1: added to a sum that ran over all groups each would be lost after 2^24;
+    added to their own part's sum they make 5, and (2^24 + 128) + 5 rounds once, to the even 2^24 + 132. Last, 2^24 in
+    part 7 after 35 ones in parts 0 to 6: the parts are added from the first, so 35 + 2^24 rounds to 2^24 + 36; with
+    2^24 first every part would be lost."""
+    K = 1280
+    codes = np.ones(K, dtype=np.int8)
+    x = np.zeros(K, dtype=np.float32)
+    x[0] = 2.0 ** 24          # group 0: the chain holds 2^24 (its other inputs are 0)
+    x[32:160] = 1.0           # groups 1..4, the rest of part 0: 32 each
+    assert column_total(codes, x) == 2.0 ** 24 + 128
+    for g in range(5, 10):    # part 1: a one a group, 5 in all
+        x[32 * g] = 1.0
+    want = np.float32(np.float32(2.0 ** 24 + 128) + np.float32(5.0))   # one rounding of the parts' sum: ties to even
+    assert column_total(codes, x) == float(want) and float(want) == 2.0 ** 24 + 132
+    # the eight parts are added in order from the first: a 2^24 in part 7 arrives after everything else
+    x = np.zeros(K, dtype=np.float32)
+    x[32 * 35] = 2.0 ** 24    # part 7 = groups 35..39
+    for g in range(0, 35):
+        x[32 * g] = 1.0       # parts 0..6: 5 each, 35 in all, exact
+    assert column_total(codes, x) == 2.0 ** 24 + 36   # 35 + 2^24 rounds to even: + 36; 2^24 first would lose every part
+
+
+def test_the_column_rule_rounds_each_weight_to_half_first():
+    """A scale of 1 + 2^-10 and code 3: the fp32 value 3 + 3 * 2^-10 is not a half (their spacing at 3 is 2^-9), and the
+    total is the half it rounds to times the input, not the fp32 value times the input."""
+    K = 256
+    codes = np.zeros(K, dtype=np.int8)
+    codes[0] = 3
+    x = np.zeros(K, dtype=np.float32)
+    x[0] = 1.0
+    d = np.float16(1.0 + 2.0 ** -10)                  # a half: the block's scale field is one
+    value = np.float32(d) * np.float32(3)              # 3 + 3 * 2^-10: fp32 holds it, a half (spacing 2^-9 at 3) does not
+    assert float(np.float16(value)) != float(value)
+    assert column_total(codes, x, d=float(d)) == float(np.float16(value))
+
+
+@pytest.mark.parametrize("name,fmt", orc.ALL_FORMATS)
+def test_the_column_rule_lies_in_the_staged_interval(name, fmt):
+    """On random weights and rows the totals lie within the reference's bound for a staged projection of the exact dot
+    (projectionBound(staged)) and within the accumulation term of the dot over the half-rounded weights."""
+    rng = np.random.default_rng(5)
+    N, K, M = 48, 1280, 2
+    native = orc.make_native(fmt, N, K, 9)
+    x = orc.f32_to_bf16(rng.standard_normal((M, K)).astype(np.float32))
+    got = orc.gemv_column(fmt, native, x, N).astype(np.float64)
+    want = orc.gemm_staged(fmt, native, x, N)
+    assert np.all(np.abs(got - want["exact"]) <= want["bound"])
+    assert np.all(np.abs(got - want["staged"].astype(np.float64)) <= want["accumulation"] + np.abs(want["staged"]) * 2.0 ** -23)
