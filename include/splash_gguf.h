@@ -16,6 +16,12 @@ typedef struct spg_file spg_file; /* model::GgufFile: the mapped file and its pa
 
 /* GgufFile::GgufFile (GgufFile.hpp:117): GGUF version 3, one file. */
 sp_status spg_open(const char *path, spg_file **out);
+/* The parts of a split GGUF (NAME-0000K-of-0000N.gguf, K = 1..N) in split order, which is their name order
+ * (GgufFile.hpp:118-124, GgufFile.cpp:167-201, GgufTarget.cpp:19-46): the first part's metadata is the file's, and its
+ * split.count and split.tensors.count, where stated, must be the parts and tensors read, so a part alone is refused; a
+ * later part's split.no must be its place; a part of no tensors may end at its header. Tensors keep one numbering
+ * across the parts. count 1 is spg_open. */
+sp_status spg_open_parts(const char *const *paths, uint32_t count, spg_file **out);
 void spg_close(spg_file *file);
 
 /* GgufMetadata (GgufFile.hpp:95-107): integers and booleans as unsigned, floats as double, strings.

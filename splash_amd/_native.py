@@ -322,6 +322,7 @@ class GgufTensor(ctypes.Structure):
 
 
 _sig("spg_open", c_int, ctypes.c_char_p, P(c_p))
+_sig("spg_open_parts", c_int, P(ctypes.c_char_p), c_u32, P(c_p))
 _sig("spg_close", None, c_p)
 _sig("spg_metadata_unsigned", c_int, c_p, ctypes.c_char_p, P(ctypes.c_uint64))
 _sig("spg_metadata_float", c_int, c_p, ctypes.c_char_p, P(c_double))

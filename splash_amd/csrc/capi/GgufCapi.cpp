@@ -51,6 +51,19 @@ sp_status spg_open(const char *path, spg_file **out) {
     *out = holder.release();
   });
 }
+sp_status spg_open_parts(const char *const *paths, uint32_t count, spg_file **out) {
+  return capi::guard([&] {
+    capi::require(paths && count && out, "paths or result");
+    std::vector<std::string> parts;
+    for (uint32_t i = 0; i < count; ++i) {
+      capi::require(paths[i], "a part's path");
+      parts.emplace_back(paths[i]);
+    }
+    auto holder = std::make_unique<spg_file>();
+    holder->file = std::make_unique<model::GgufFile>(parts);
+    *out = holder.release();
+  });
+}
 void spg_close(spg_file *file) { delete file; }
 
 int spg_metadata_unsigned(const spg_file *file, const char *key, uint64_t *value) {

@@ -126,7 +126,23 @@ std::optional<std::string> GgufMetadata::stringValue(std::string_view key) const
   return it == strings.end() ? std::nullopt : std::optional<std::string>(it->second);
 }
 
-GgufFile::GgufFile(const std::string &path) {
+GgufFile::GgufFile(const std::string &path) : GgufFile(std::vector<std::string>{path}) {}
+
+GgufFile::GgufFile(const std::vector<std::string> &paths) {
+  if (paths.empty()) throw GgufError("a GGUF has at least one file");
+  try {
+    for (size_t file = 0; file < paths.size(); ++file) parse(paths[file], uint32_t(file));
+    if (metadata_.unsignedValue("split.count").value_or(1) != parts_.size())
+      throw GgufError("the GGUF's split.count does not match its " + std::to_string(parts_.size()) + " file(s)");
+    if (metadata_.unsignedValue("split.tensors.count").value_or(tensors_.size()) != tensors_.size())
+      throw GgufError("the GGUF's files hold another number of tensors than split.tensors.count");
+  } catch (...) {
+    unmap();
+    throw;
+  }
+}
+
+void GgufFile::parse(const std::string &path, uint32_t file) {
   const int fd = ::open(path.c_str(), O_RDONLY);
   if (fd < 0) throw GgufError("cannot open " + path);
   struct stat st {};
@@ -134,72 +150,82 @@ GgufFile::GgufFile(const std::string &path) {
     ::close(fd);
     throw GgufError("not a GGUF file: " + path);
   }
-  size_ = uint64_t(st.st_size);
-  void *mapped = ::mmap(nullptr, size_, PROT_READ, MAP_PRIVATE, fd, 0);
+  Part part;
+  part.size = uint64_t(st.st_size);
+  void *mapped = ::mmap(nullptr, part.size, PROT_READ, MAP_PRIVATE, fd, 0);
   ::close(fd);
   if (mapped == MAP_FAILED) throw GgufError("cannot map " + path);
-  base_ = static_cast<const uint8_t *>(mapped);
-  try {
-    Reader r{base_, size_};
-    if (r.take<uint32_t>() != 0x46554747u) throw GgufError("not a GGUF file: " + path);  // "GGUF"
-    const uint32_t version = r.take<uint32_t>();
-    if (version != 3) throw GgufError("unsupported GGUF version " + std::to_string(version));
-    const uint64_t tensorCount = r.take<uint64_t>(), valueCount = r.take<uint64_t>();
-    if (tensorCount > (1u << 20) || valueCount > (1u << 20)) throw GgufError("implausible GGUF counts");
-    for (uint64_t i = 0; i < valueCount; ++i) {
-      const std::string key = r.string();
-      const uint32_t type = r.take<uint32_t>();
-      switch (type) {
-        case kU8: metadata_.unsigneds[key] = r.take<uint8_t>(); break;
-        case kI8: metadata_.unsigneds[key] = uint64_t(int64_t(r.take<int8_t>())); break;
-        case kU16: metadata_.unsigneds[key] = r.take<uint16_t>(); break;
-        case kI16: metadata_.unsigneds[key] = uint64_t(int64_t(r.take<int16_t>())); break;
-        case kU32: metadata_.unsigneds[key] = r.take<uint32_t>(); break;
-        case kI32: metadata_.unsigneds[key] = uint64_t(int64_t(r.take<int32_t>())); break;
-        case kBool: metadata_.unsigneds[key] = r.take<uint8_t>() != 0; break;
-        case kU64: metadata_.unsigneds[key] = r.take<uint64_t>(); break;
-        case kI64: metadata_.unsigneds[key] = uint64_t(r.take<int64_t>()); break;
-        case kF32: metadata_.floats[key] = r.take<float>(); break;
-        case kF64: metadata_.floats[key] = r.take<double>(); break;
-        case kString: metadata_.strings[key] = r.string(); break;
-        default: r.skipValue(type); break;  // arrays (tokenizer tables) are not kept
-      }
+  part.base = static_cast<const uint8_t *>(mapped);
+  parts_.push_back(part);   // unmapped with the others if the header is refused
+  Reader r{part.base, part.size};
+  if (r.take<uint32_t>() != 0x46554747u) throw GgufError("not a GGUF file: " + path);  // "GGUF"
+  const uint32_t version = r.take<uint32_t>();
+  if (version != 3) throw GgufError("unsupported GGUF version " + std::to_string(version));
+  const uint64_t tensorCount = r.take<uint64_t>(), valueCount = r.take<uint64_t>();
+  if (tensorCount > (1u << 20) || valueCount > (1u << 20)) throw GgufError("implausible GGUF counts");
+  // Only the first part's metadata is kept: a later part repeats split.* alone, whose split.no must be its place.
+  GgufMetadata later;
+  GgufMetadata &metadata = file ? later : metadata_;
+  for (uint64_t i = 0; i < valueCount; ++i) {
+    const std::string key = r.string();
+    const uint32_t type = r.take<uint32_t>();
+    if (file && key == "split.no" && type != kU16 && type != kU32) throw GgufError("invalid split.no in " + path);
+    switch (type) {
+      case kU8: metadata.unsigneds[key] = r.take<uint8_t>(); break;
+      case kI8: metadata.unsigneds[key] = uint64_t(int64_t(r.take<int8_t>())); break;
+      case kU16: metadata.unsigneds[key] = r.take<uint16_t>(); break;
+      case kI16: metadata.unsigneds[key] = uint64_t(int64_t(r.take<int16_t>())); break;
+      case kU32: metadata.unsigneds[key] = r.take<uint32_t>(); break;
+      case kI32: metadata.unsigneds[key] = uint64_t(int64_t(r.take<int32_t>())); break;
+      case kBool: metadata.unsigneds[key] = r.take<uint8_t>() != 0; break;
+      case kU64: metadata.unsigneds[key] = r.take<uint64_t>(); break;
+      case kI64: metadata.unsigneds[key] = uint64_t(r.take<int64_t>()); break;
+      case kF32: metadata.floats[key] = r.take<float>(); break;
+      case kF64: metadata.floats[key] = r.take<double>(); break;
+      case kString: metadata.strings[key] = r.string(); break;
+      default: r.skipValue(type); break;  // arrays (tokenizer tables) are not kept
     }
-    const uint64_t alignment = metadata_.unsignedValue("general.alignment").value_or(32);
-    if (alignment < 8 || alignment > 65536 || (alignment & (alignment - 1))) throw GgufError("invalid GGUF alignment");
-    tensors_.reserve(tensorCount);
-    for (uint64_t i = 0; i < tensorCount; ++i) {
-      GgufTensor t;
-      t.name = r.string();
-      const uint32_t dimensions = r.take<uint32_t>();
-      if (!dimensions || dimensions > 4) throw GgufError("tensor has an unsupported rank: " + t.name);
-      for (uint32_t d = 0; d < dimensions; ++d) t.dims.push_back(r.take<uint64_t>());
-      t.type = r.take<uint32_t>();
-      t.offset = r.take<uint64_t>();
-      const GgmlTypeTraits *traits = ggmlTypeTraits(t.type);
-      if (!traits) throw GgufError("tensor " + t.name + " has unknown ggml type " + std::to_string(t.type));
-      if (!t.columns() || t.columns() % traits->blockElements) throw GgufError("tensor rows do not hold whole blocks: " + t.name);
-      if (t.rows() && t.columns() / traits->blockElements > UINT64_MAX / traits->blockBytes / t.rows())
-        throw GgufError("tensor is too large: " + t.name);
-      t.bytes = t.columns() / traits->blockElements * traits->blockBytes * t.rows();
-      if (t.offset % alignment) throw GgufError("tensor data is misaligned: " + t.name);
-      if (!index_.emplace(t.name, tensors_.size()).second) throw GgufError("duplicate tensor " + t.name);
-      tensors_.push_back(std::move(t));
-    }
-    dataStart_ = (r.at + alignment - 1) / alignment * alignment;
-    for (const GgufTensor &t : tensors_)
-      if (dataStart_ > size_ || t.offset > size_ - dataStart_ || t.bytes > size_ - dataStart_ - t.offset)
-        throw GgufError("tensor data lies past the end of the file: " + t.name);
-  } catch (...) {
-    ::munmap(const_cast<uint8_t *>(base_), size_);
-    base_ = nullptr;
-    throw;
+  }
+  if (file && later.unsignedValue("split.no").value_or(file) != file) throw GgufError("GGUF split file " + path + " is out of order");
+  const uint64_t alignment = metadata.unsignedValue("general.alignment").value_or(metadata_.unsignedValue("general.alignment").value_or(32));
+  if (alignment < 8 || alignment > 65536 || (alignment & (alignment - 1))) throw GgufError("invalid GGUF alignment");
+  const size_t firstTensor = tensors_.size();
+  tensors_.reserve(firstTensor + tensorCount);
+  for (uint64_t i = 0; i < tensorCount; ++i) {
+    GgufTensor t;
+    t.name = r.string();
+    t.file = file;
+    const uint32_t dimensions = r.take<uint32_t>();
+    if (!dimensions || dimensions > 4) throw GgufError("tensor has an unsupported rank: " + t.name);
+    for (uint32_t d = 0; d < dimensions; ++d) t.dims.push_back(r.take<uint64_t>());
+    t.type = r.take<uint32_t>();
+    t.offset = r.take<uint64_t>();
+    const GgmlTypeTraits *traits = ggmlTypeTraits(t.type);
+    if (!traits) throw GgufError("tensor " + t.name + " has unknown ggml type " + std::to_string(t.type));
+    if (!t.columns() || t.columns() % traits->blockElements) throw GgufError("tensor rows do not hold whole blocks: " + t.name);
+    if (t.rows() && t.columns() / traits->blockElements > UINT64_MAX / traits->blockBytes / t.rows())
+      throw GgufError("tensor is too large: " + t.name);
+    t.bytes = t.columns() / traits->blockElements * traits->blockBytes * t.rows();
+    if (t.offset % alignment) throw GgufError("tensor data is misaligned: " + t.name);
+    if (!index_.emplace(t.name, tensors_.size()).second) throw GgufError("duplicate tensor " + t.name);
+    tensors_.push_back(std::move(t));
+  }
+  Part &mine = parts_.back();
+  mine.dataStart = (r.at + alignment - 1) / alignment * alignment;
+  for (size_t i = firstTensor; i < tensors_.size(); ++i) {
+    const GgufTensor &t = tensors_[i];
+    if (mine.dataStart > mine.size || t.offset > mine.size - mine.dataStart || t.bytes > mine.size - mine.dataStart - t.offset)
+      throw GgufError("tensor data lies past the end of the file: " + t.name);
   }
 }
 
-GgufFile::~GgufFile() {
-  if (base_) ::munmap(const_cast<uint8_t *>(base_), size_);
+void GgufFile::unmap() noexcept {
+  for (const Part &part : parts_)
+    if (part.base) ::munmap(const_cast<uint8_t *>(part.base), part.size);
+  parts_.clear();
 }
+
+GgufFile::~GgufFile() { unmap(); }
 
 const GgufTensor *GgufFile::find(std::string_view name) const noexcept {
   const auto it = index_.find(name);
@@ -209,7 +235,10 @@ const GgufTensor &GgufFile::require(std::string_view name) const {
   if (const GgufTensor *t = find(name)) return *t;
   throw GgufError("missing tensor " + std::string(name));
 }
-const uint8_t *GgufFile::data(const GgufTensor &tensor) const { return base_ + dataStart_ + tensor.offset; }
+const uint8_t *GgufFile::data(const GgufTensor &tensor) const {
+  const Part &part = parts_.at(tensor.file);
+  return part.base + part.dataStart + tensor.offset;
+}
 
 LoadedImage loadImage(hip::Backend &backend, const GgufFile &file, const GgufTensor &tensor, uint32_t firstRow, uint32_t rows) {
   const std::optional<uint32_t> format = imageFormat(tensor.type);

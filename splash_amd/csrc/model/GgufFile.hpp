@@ -39,8 +39,9 @@ struct GgufTensor {
   std::string name;
   uint32_t type = 0;
   std::vector<uint64_t> dims;  // dims[0] is the fastest (row length)
-  uint64_t offset = 0;         // in the file's tensor data
+  uint64_t offset = 0;         // in the tensor data of the file that holds it
   uint64_t bytes = 0;
+  uint32_t file = 0;           // which part of a split GGUF holds it (GgufFile.hpp:74 in the reference)
   [[nodiscard]] uint64_t columns() const noexcept { return dims.empty() ? 0 : dims[0]; }
   [[nodiscard]] uint64_t rows() const noexcept;
   [[nodiscard]] uint64_t elements() const noexcept { return columns() * rows(); }
@@ -61,6 +62,11 @@ class GgufFile final {
 public:
   // Maps the file and parses its header; throws GgufError on a malformed or truncated file.
   explicit GgufFile(const std::string &path);
+  // The parts of a split GGUF in split order (GgufFile.hpp:118-124, GgufFile.cpp:167-201 in the reference): the first
+  // part's metadata is kept, and its split.count and split.tensors.count, where it states them, must describe the parts
+  // read (a part read alone is refused); a later part's split.no must be its place; a part of no tensors may end at
+  // its header. One path is the single file.
+  explicit GgufFile(const std::vector<std::string> &paths);
   ~GgufFile();
   GgufFile(const GgufFile &) = delete;
   GgufFile &operator=(const GgufFile &) = delete;
@@ -71,11 +77,17 @@ public:
   [[nodiscard]] const GgufTensor &require(std::string_view name) const;
   // The tensor's bytes in the mapped file.
   [[nodiscard]] const uint8_t *data(const GgufTensor &tensor) const;
+  [[nodiscard]] size_t parts() const noexcept { return parts_.size(); }
 
 private:
-  const uint8_t *base_ = nullptr;
-  uint64_t size_ = 0;
-  uint64_t dataStart_ = 0;
+  struct Part {
+    const uint8_t *base = nullptr;
+    uint64_t size = 0;
+    uint64_t dataStart = 0;
+  };
+  void parse(const std::string &path, uint32_t file);
+  void unmap() noexcept;
+  std::vector<Part> parts_;
   GgufMetadata metadata_;
   std::vector<GgufTensor> tensors_;
   std::map<std::string, size_t, std::less<>> index_;

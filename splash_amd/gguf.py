@@ -23,11 +23,16 @@ class Tensor:
 
 
 class GgufFile:
-    """model::GgufFile: a mapped GGUF (version 3) file, its scalar metadata and its tensor table."""
+    """model::GgufFile: a mapped GGUF (version 3) file, its scalar metadata and its tensor table. `path` may be the
+    list of a split GGUF's parts in split order."""
 
     def __init__(self, path):
         handle = ctypes.c_void_p()
-        check(lib.spg_open(str(path).encode(), ctypes.byref(handle)))
+        if isinstance(path, (list, tuple)):
+            parts = (ctypes.c_char_p * len(path))(*[str(p).encode() for p in path])
+            check(lib.spg_open_parts(parts, len(path), ctypes.byref(handle)))
+        else:
+            check(lib.spg_open(str(path).encode(), ctypes.byref(handle)))
         self.handle = handle
         self.tensors = []
         for i in range(lib.spg_tensor_count(handle)):

@@ -117,7 +117,7 @@ def test_projections_and_norms_load_from_a_file(backend, tmp_path):
         f.load_bf16(backend, f.find("output.weight"))
 
 
-def dense_model_file(path, model, value_format, tied, extra=(), skip=(), more_metadata=()):
+def dense_model_file(path, model, value_format, tied, extra=(), skip=(), more_metadata=(), parts=1):
     """A dense decoder's GGUF as llama.cpp names its tensors: blk.N.attn_q / attn_k / attn_v (the values requantized to
     `value_format`, as a Q4_K_M file keeps them) ..., norms as F32, the token table, and the head unless tied."""
     d = model.dims
@@ -146,12 +146,59 @@ def dense_model_file(path, model, value_format, tied, extra=(), skip=(), more_me
                 ("qwen3.attention.head_count", gw.U32, d["q_heads"]), ("qwen3.attention.head_count_kv", gw.U32, d["kv_heads"]),
                 ("qwen3.attention.key_length", gw.U32, D), ("qwen3.attention.value_length", gw.U32, D),
                 ("qwen3.attention.layer_norm_rms_epsilon", gw.F32, 1e-6), ("qwen3.rope.freq_base", gw.F32, model.rope_theta)]
-    gw.write_gguf(path, metadata + list(more_metadata), tensors)
+    if parts == 1:
+        gw.write_gguf(path, metadata + list(more_metadata), tensors)
+        return path
+    return write_split(path, metadata + list(more_metadata), tensors, parts)
+
+
+def write_split(path, metadata, tensors, parts):
+    """The file as a split GGUF of `parts` parts, NAME-0000K-of-0000N.gguf: the first holds the metadata and no tensor
+    (as llama.cpp's splitter may leave it), the others the tensors in order and split.* alone."""
+    stem = str(path)[:-len(".gguf")]
+    names = [f"{stem}-{k + 1:05d}-of-{parts:05d}.gguf" for k in range(parts)]
+    split = lambda k: [("split.no", gw.U16, k), ("split.count", gw.U16, parts), ("split.tensors.count", gw.I32, len(tensors))]
+    gw.write_gguf(names[0], list(metadata) + split(0), [])
+    share = (len(tensors) + parts - 2) // (parts - 1)
+    for k in range(1, parts):
+        gw.write_gguf(names[k], split(k), tensors[(k - 1) * share:k * share])
+    return names
+
+
+def test_a_split_file_reads_as_one(tmp_path):
+    """GgufFile.cpp:167-201: the parts in split order are one file, with the first part's metadata and one tensor
+    numbering; a part alone, parts out of order, a part missing or twice, and a wrong tensor count are refused."""
+    whole = tmp_path / "whole.gguf"
+    tensors = model_file(whole)
+    raw = open(whole, "rb").read()
+    assert raw[:4] == b"GGUF"
+    metadata = [("general.architecture", gw.STRING, "qwen3"), ("qwen3.block_count", gw.U32, 1)]
+    names = write_split(tmp_path / "model.gguf", metadata, tensors, 3)
+    f, one = gguf.GgufFile(names), gguf.GgufFile(whole)
+    assert f.string("general.architecture") == "qwen3" and f.unsigned("split.count") == 3 and f.unsigned("split.no") == 0
+    assert [t.name for t in f.tensors] == [t.name for t in one.tensors]
+    for a, b in zip(f.tensors, one.tensors):
+        assert (a.ggml_type, a.dims, a.bytes, a.format) == (b.ggml_type, b.dims, b.bytes, b.format)
+        assert np.array_equal(f.data(a), one.data(b))
+    assert f.find("output.weight").name == "output.weight"
+    for bad in ([names[1]], names[:2], [names[0], names[2], names[1]], names + [names[2]], [names[1], names[0], names[2]]):
+        with pytest.raises(splash_amd.SplashError):
+            gguf.GgufFile(bad)
+    # another number of tensors than the first part states
+    short = write_split(tmp_path / "short.gguf", metadata, tensors, 3)
+    gw.write_gguf(short[2], [("split.no", gw.U16, 2), ("split.count", gw.U16, 3)], [])
+    with pytest.raises(splash_amd.SplashError, match="split.tensors.count"):
+        gguf.GgufFile(short)
+    # a single file that says it is a part of several
+    alone = tmp_path / "alone.gguf"
+    gw.write_gguf(alone, metadata + [("split.count", gw.U16, 2)], tensors)
+    with pytest.raises(splash_amd.SplashError, match="split.count"):
+        gguf.GgufFile(alone)
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("value_format,tied", [(orc.FMT_Q6K, False), (orc.FMT_Q4K, True)])
-def test_a_dense_decoder_loads_from_a_file(tmp_path, value_format, tied):
+@pytest.mark.parametrize("value_format,tied,parts", [(orc.FMT_Q6K, False, 1), (orc.FMT_Q4K, True, 1), (orc.FMT_Q6K, False, 3)])
+def test_a_dense_decoder_loads_from_a_file(tmp_path, value_format, tied, parts):
     """spg_dense_dimensions and spo_dense_verify_load_gguf: the driver built from a file gives, bit for bit, the logits
     and the acceptance of the driver built by hand from the same tensors: q | k | v fused with the values in another
     format than the queries and keys, a tied head, and the refusal of tensors the loader would ignore."""
@@ -164,8 +211,7 @@ def test_a_dense_decoder_loads_from_a_file(tmp_path, value_format, tied):
             w["v"] = orc.quantize_rows(value_format, orc.dequant_rows(orc.FMT_Q4K, w["v"], 512, 512))
     if tied:
         model.head = model.embedding
-    path = tmp_path / "dense.gguf"
-    dense_model_file(path, model, value_format, tied)
+    path = dense_model_file(tmp_path / "dense.gguf", model, value_format, tied, parts=parts)   # a path, or a split file's parts
     rows, context = 16, 200
     rng = np.random.default_rng(1)
     tokens = rng.integers(0, 2048, rows).astype(np.uint32)
