@@ -226,6 +226,55 @@ def test_batched_sequences_equal_each_alone(backend):
         assert np.array_equal(together[s[0]:s[0] + s[1]], alone[s[0]:s[0] + s[1]])
 
 
+def test_sequences_share_the_pages_of_a_common_prefix(backend):
+    """A page table names physical pages, so sequences with a common prefix may name the same ones (what the engine's
+    prefix cache hands out): three sequences of one 600-token history share its two full pages and keep the page they
+    write their own rows into apart. Each gives the result of a sequence that owns copies of every page, bit for bit,
+    and the shared pages keep their bytes."""
+    print("case attention shared prefix", flush=True)
+    rng = np.random.default_rng(8)
+    q_heads, kv_heads, D, PT = 32, 4, 128, ops.PAGE_TOKENS
+    committed, rows_each = 600, [16, 9, 16]
+    full = committed // PT                     # the prefix's full pages: shared; the page after them holds 88 tokens and the rows
+    k = rng.standard_normal((full + 1, kv_heads, PT, D)).astype(np.float32)
+    v = rng.standard_normal((full + 1, kv_heads, PT, D)).astype(np.float32)
+    mx = np.abs(k).max(-1, keepdims=True); kc = np.clip(np.rint(k * 127 / mx), -127, 127).astype(np.int8); ks = mx[..., 0] / 127
+    mx = np.abs(v).max(-1, keepdims=True); vc = np.clip(np.rint(v * 127 / mx), -127, 127).astype(np.int8); vs = mx[..., 0] / 127
+    width = (q_heads + 2 * kv_heads) * D
+    total_rows = sum(rows_each)
+    qkv = orc.f32_to_bf16(rng.standard_normal((total_rows, width)).astype(np.float32))
+    tree = ops.chain_tree_rows(rows_each)
+
+    def run(shared):
+        # physical pages: the prefix's (once when shared, once a sequence otherwise), then a tail page a sequence
+        n = len(rows_each)
+        prefix_of = (lambda s: list(range(full))) if shared else (lambda s: list(range(s * full, (s + 1) * full)))
+        tails = (full if shared else n * full)
+        table = np.array([page for s in range(n) for page in prefix_of(s) + [tails + s]], dtype=np.uint64)
+        phys = tails + n
+        source = np.array([p for s in range(1 if shared else n) for p in range(full)] + [full] * n)   # which logical page a physical one holds
+        kv = ops.KvPages(backend, kv_heads, D, phys, table)
+        packed = kv.pack_pages(kc[source], ks[source], vc[source], vs[source])
+        kv.upload(packed)
+        sequences, first = [], 0
+        for s, r in enumerate(rows_each):
+            sequences.append((first, r, committed, s * (full + 1)))
+            first += r
+        plan = ops.AttentionPlan(q_heads, kv_heads, D, sequences)
+        ws = ops.AttentionWorkspace(backend, plan)
+        out = backend.allocate_buffer(total_rows * q_heads * D * 2)
+        g = splash_amd.CommandGraph()
+        ops.PagedAttention.add_projection(g, plan, backend.from_array(qkv), ws, kv)
+        ops.PagedAttention.add_attention(g, plan, ws, backend.from_array(tree), kv, out)
+        backend.run(g)
+        return out.download(np.uint16).reshape(total_rows, q_heads * D), kv.download(), packed
+    shared, pool, before = run(True)
+    apart, _, _ = run(False)
+    assert np.array_equal(shared, apart)
+    assert np.array_equal(pool[:full], before[:full])            # nobody wrote the shared pages
+    assert (pool[full:] != before[full:]).any(axis=1).all()       # every sequence stored its rows in its own page
+
+
 @pytest.mark.parametrize("rows,committed", [(16, 300), (5, 1000)])
 def test_attention_output_table(backend, rows, committed):
     """The split merge may also write its rows as the next projection's activation table: the rows are
