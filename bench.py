@@ -619,6 +619,10 @@ def main():
     w = WORKLOADS[args.workload]
     info = backend.device_info()
     log(f"device {info.name.decode()} {info.arch.decode()} CUs {info.compute_units}")
+    if args.prompt_chunk:
+        if args.prompt_chunk > 128:
+            raise SystemExit("a prompt chunk holds up to 128 tokens (16 rows of each of the driver's eight lanes)")
+        args.lanes = max(args.lanes, (args.prompt_chunk + 15) // 16)    # the driver's rows: 16 a lane
     t0 = time.time()
     gpu = build_model(backend, w, args.lanes)
     log(f"model resident in {time.time() - t0:.1f}s; allocated {backend.memory_stats().allocated_bytes / 1e9:.2f} GB")
