@@ -392,12 +392,13 @@ __device__ __forceinline__ TileRef find_tile(uint32_t index, const uint8_t *cons
 // One record's contribution to a wave's sums. `a` and `sums` are the workgroup's staged
 // activations of the record's super-block in LDS: a[t][g][lane] the MFMA operand of row tile t,
 // group g; sums[t][j][lane] the row sums of the j-th K = 4 MFMA.
-// acc[t] = fma(dot(step, t), scale(step), acc[t]) over a record's `Steps` steps in order, every row tile. With four row
-// tiles a step's products are issued before the multiply-adds of the step before it, so that those run while the matrix
-// cores work (each element's multiply-adds keep their order: the sums are the same).
+// acc[t] = fma(dot(step, t), scale(step), acc[t]) over a record's `Steps` steps in order, every row tile. A step's
+// products are issued before the multiply-adds of the step before it, so that those run while the matrix cores work
+// (each element's multiply-adds keep their order: the sums are the same).
 template <int RT, uint32_t Steps, class Dot, class Scale>
 __device__ __forceinline__ void scaled_groups(f32x4 (&acc)[RT], Dot dot, Scale scale) {
-  if constexpr (RT > 2) {
+  // (not the two-tile Q6_K kernel, whose sixteen steps of two products would cost it a wave a SIMD in registers)
+  if constexpr (!(RT == 2 && Steps == 16)) {
     f32x4 held[2][RT];
 #pragma unroll
     for (int t = 0; t < RT; ++t) held[0][t] = dot(0u, t);
