@@ -190,7 +190,7 @@ def time_c2_ops(backend):
     copies larger than twice the 256 MB memory-side cache so that every pass reads HBM; per-dispatch GPU time (HIP
     events around each dispatch), median over the ring passes after the first. Prints one JSON line."""
     import splash_amd
-    from splash_amd import ops
+    from splash_amd import ops, synthetic
     rng = np.random.default_rng(0)
     bf = lambda a: (np.ascontiguousarray(a, np.float32).view(np.uint32) >> 16).astype(np.uint16)
     linear = ops.Linear(backend)
@@ -205,6 +205,21 @@ def time_c2_ops(backend):
         images = [rng.integers(0, 256, ops.gguf_image_bytes(fmt, n, K), dtype=np.uint8) for n in widths]
         ring = [ops.Projection([(fmt, n, backend.from_array(im)) for n, im in zip(widths, images)], K) for _ in range(copies)]
         gates = [ops.Projection([(fmt, N, backend.from_array(images[0]))], K) for _ in range(copies)] if tensors == 2 else None
+        # the CPU oracle's register-rule projection of the same matrices on this host's cores, whole, at 16 rows
+        from tests import oracle as orc
+        natives = [synthetic.native(rng, fmt, n, K) for n in widths] * tensors
+        x16 = orc.f32_to_bf16(rng.standard_normal((16, K)).astype(np.float32))
+        rounds = []
+        for _ in range(5):
+            t0 = time.time()
+            for nat, n in zip(natives, list(widths) * tensors):
+                orc.gemm(fmt, nat, x16, n, want=("chain",), threads=0)
+            rounds.append(time.time() - t0)
+        cpu_us = float(np.median(rounds[1:]) * 1e6)
+        log(f"  {name:8s} M=16 on the CPU ({os.cpu_count()} threads): {cpu_us / 1e3:8.2f} ms")
+        results.append({"op": name, "device": "cpu", "cores": os.cpu_count(), "kind": "port", "M": 16, "us": round(cpu_us, 1),
+                        "GB/s": round(weight_bytes / cpu_us / 1e3, 2)})
+        del natives
         for M in (1, 4, 8, 16, 32):
             x = backend.from_array(bf(rng.standard_normal((M, K))))
             out, residual = backend.allocate_buffer(M * N * 4), backend.allocate_buffer(M * N * 2)
@@ -321,6 +336,22 @@ def time_c3_ops(backend):
         tree = backend.from_array(ops.chain_tree_rows([rows]))
         out = backend.allocate_buffer(rows * QH * D * 2)
         algorithmic = kv_bytes + rows * QH * D * 2 * 2 + pages * 8
+        if context % ops.PAGE_TOKENS == 0:
+            # the CPU oracle's page loop over the same shape on this host's cores: every head up to 32K, two of the
+            # eight KV heads (a quarter of the work, scaled) at 128K
+            from tests import oracle as orc
+            heads = KVH if context <= 32768 else 2
+            kc = rng.integers(-127, 128, (pages, heads, ops.PAGE_TOKENS, D)).astype(np.int8)
+            ks = np.full((pages, heads, ops.PAGE_TOKENS), 0.03, dtype=np.float32)
+            q = orc.f32_to_bf16(rng.standard_normal((rows, heads * (QH // KVH), D)).astype(np.float32))
+            anc = np.array([(2 << r) - 1 for r in range(rows)], dtype=np.uint32)
+            t0 = time.time()
+            orc.attention(q, kc, ks, kc, ks, np.arange(pages, dtype=np.uint32), anc, context - rows, want64=False, threads=0)
+            cpu_us = (time.time() - t0) * 1e6 * KVH / heads
+            log(f"  context {context:6d} on the CPU ({os.cpu_count()} threads, {heads} of {KVH} KV heads timed): {cpu_us / 1e3:9.1f} ms")
+            results.append({"context": context, "device": "cpu", "cores": os.cpu_count(), "kind": "port", "kv_heads_timed": heads,
+                            "us": round(cpu_us, 1), "GB/s": round(algorithmic / cpu_us / 1e3, 3)})
+            del kc, ks, q
         for int8_queries in (False, True):
             plan = ops.AttentionPlan(QH, KVH, D, [(0, rows, context - rows, 0)], int8_queries=int8_queries)
             workspace = ops.AttentionWorkspace(backend, plan)
