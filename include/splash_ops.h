@@ -358,7 +358,10 @@ sp_status spo_sampling_add_acceptance(spo_graph *graph, sp_buffer *input_tokens,
  * library (64 KiB a GPU, held until the process ends) instead of a workspace argument: the call allocates nothing,
  * frees nothing and returns once its two kernels are launched. At most SPO_SAMPLING_STATIC_MAXIMUM_ROWS rows a call
  * (more is SP_INVALID_ARGUMENT). Every call on one GPU shares that GPU's array: calls that overlap on one GPU
- * (different streams, or threads) race; calls in stream order on one stream do not. */
+ * (different streams, or threads) race; calls in stream order on one stream do not. A GPU's FIRST call looks the
+ * array's address up (hipGetSymbolAddress, under a mutex; it may load the code object), which is not a call to make
+ * under stream capture: make one call per GPU outside any capture first (any row count, e.g. at start-up); every
+ * later call on that GPU is two kernel launches and nothing else. */
 #define SPO_SAMPLING_STATIC_MAXIMUM_ROWS 256u
 sp_status spo_sampling_greedy_rows_static(const float *logits, uint32_t rows, uint32_t vocabulary, uint32_t logits_stride,
                                           uint32_t *tokens, void *stream);
@@ -447,8 +450,8 @@ typedef enum spo_verify_buffer {
   SPO_VERIFY_LOGITS, SPO_VERIFY_DRAFT_PROBABILITIES, SPO_VERIFY_HIDDEN,
   SPO_VERIFY_QKV_ROWS = 15, SPO_VERIFY_ATTENTION_ROWS = 16, SPO_VERIFY_FFN_ROWS = 17,
   /* the sampled rows' candidate children (spo_sampling_buffers): index 0 ids, 1 probabilities, 2 drawn children, 3 child
-     uniforms; host-visible, allocated by the first call, after which every step's sampled lanes test candidate
-     children instead of one child against the full-vocabulary draft probabilities */
+     uniforms; host-visible, allocated by the first call. Fetching them changes no step: spo_dense_verify_set_test_children
+     chooses which test the sampled lanes of later steps run */
   SPO_VERIFY_CANDIDATE_CHILDREN = 18
 } spo_verify_buffer;
 sp_status spo_dense_verify_buffer(spo_dense_verify *verify, spo_verify_buffer which, uint32_t index, sp_buffer **out);
@@ -478,7 +481,20 @@ sp_status spo_dense_verify_results(spo_dense_verify *verify, const spo_verify_la
 /* Whether steps encoded from now on chain a layer's projections after its attention into one dispatch
  * (spo_linear_add_chain: output, gate/up, down and the next layer's q|k|v, the LM head after the last layer) where
  * their shapes allow: off by default; the results are the same bit for bit. spo_dense_verify_results fails with
- * SP_BACKEND_ERROR after a step in which a chained projection's bounded wait gave up. */
+ * SP_BACKEND_ERROR after a step in which a chained projection's bounded wait gave up. A chained dispatch rests on
+ * two things HIP does not promise: that the device starts a grid's workgroups in index order (a link's workgroups are
+ * started before any of the next link's), and that a link's results, stored with agent scope and counted in only after
+ * the stores completed, are seen by a later link that never read those addresses before. The bounded wait turns a
+ * break of either into a status, never a hang. */
+/* Whether the sampled lanes of steps encoded from now on test the children their draft drew among sixteen candidates
+ * (SPO_VERIFY_CANDIDATE_CHILDREN; sampling.metal:697-880) or, the default, one child against the full-vocabulary draft
+ * distribution (SPO_VERIFY_DRAFT_PROBABILITIES). A step reads only the buffers of the test it runs. */
+sp_status spo_dense_verify_set_test_children(spo_dense_verify *verify, int on);
+/* The chained projections' status of the last completed step, for a caller that reads logits or hidden rows through
+ * spo_dense_verify_buffer without spo_dense_verify_results: *status 0 when every wait was met (always, of a step that
+ * chains nothing), nonzero when one gave up and what the step left is void. Reading it clears it. No counterpart in the
+ * reference, whose projections are a dispatch each. */
+sp_status spo_dense_verify_chain_status(spo_dense_verify *verify, uint32_t *status);
 /* DenseVerify::encodePrefill: a chunk of 1 to 16 x max_lanes prompt tokens of ONE sequence (its pages from table_first,
  * `committed` tokens cached before the chunk) in one pass over the weights, where the reference prefills a prompt in
  * chunks (Runtime.cpp's chunked prefill over QwenTarget.cpp:457-496): the tokens go in SPO_VERIFY_INPUT_TOKENS, a chain

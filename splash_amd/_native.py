@@ -289,6 +289,8 @@ _sig("spo_sampling_add_acceptance", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, P(
 _sig("spo_sampling_greedy_rows_static", c_int, ctypes.c_void_p, c_u32, c_u32, c_u32, ctypes.c_void_p, ctypes.c_void_p)
 _sig("spo_verify_check_results", c_int, P(LaneRows), P(c_u32), c_u32, c_u32, c_u32, P(c_u32), P(c_u32), P(c_u32), P(c_u32))
 _sig("spo_dense_verify_set_chained", c_int, c_p, c_int)
+_sig("spo_dense_verify_chain_status", c_int, c_p, ctypes.POINTER(ctypes.c_uint32))
+_sig("spo_dense_verify_set_test_children", c_int, c_p, c_int)
 _sig("spo_dense_verify_encode_prefill", c_int, c_p, c_p, c_u32, c_u32, c_u32)
 _sig("spo_dense_verify_set_fused_prepare", c_int, c_p, c_int)
 _sig("spo_dense_verify_results", c_int, c_p, P(VerifyLane), c_u32, P(c_u32), P(c_u32), P(c_u32), P(c_u32))

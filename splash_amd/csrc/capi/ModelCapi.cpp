@@ -300,6 +300,18 @@ sp_status spo_dense_verify_encode_prefill(spo_dense_verify *verify, spo_graph *g
     verify->verify->encodePrefill(capi::graphOf(graph), table_first, committed, tokens);
   });
 }
+sp_status spo_dense_verify_set_test_children(spo_dense_verify *verify, int on) {
+  return capi::guard([&] {
+    capi::require(verify, "verify");
+    verify->verify->setTestChildren(on != 0);
+  });
+}
+sp_status spo_dense_verify_chain_status(spo_dense_verify *verify, uint32_t *status) {
+  return capi::guard([&] {
+    capi::require(verify && status, "verify or status");
+    *status = verify->verify->takeChainStatus();
+  });
+}
 sp_status spo_dense_verify_set_chained(spo_dense_verify *verify, int chained) {
   return capi::guard([&] {
     capi::require(verify, "verify");

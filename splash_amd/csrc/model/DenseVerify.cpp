@@ -107,22 +107,22 @@ const hip::Buffer &DenseVerify::draftProbabilities() {
 }
 
 const hip::Buffer &DenseVerify::candidateChildren(uint32_t which) {
-  if (!sampling_.candidateIds) {
+  if (!children_.candidateIds) {
     const uint64_t R = maxRows_;
     auto shared = [&](uint64_t bytes, const char *label) { return backend_.allocateBuffer(bytes, BufferStorage::Shared, label); };
-    sampling_.candidateIds = shared(R * SAMPLING_CANDIDATES * 4, "candidate ids");
-    sampling_.candidateProbabilities = shared(R * SAMPLING_CANDIDATES * 4, "candidate probabilities");
-    sampling_.candidateDraws = shared(R * SAMPLING_TREE_CHILDREN, "drawn children");
-    sampling_.childUniforms = shared(R * SAMPLING_TREE_CHILDREN * 4, "child uniforms");
+    children_.candidateIds = shared(R * SAMPLING_CANDIDATES * 4, "candidate ids");
+    children_.candidateProbabilities = shared(R * SAMPLING_CANDIDATES * 4, "candidate probabilities");
+    children_.candidateDraws = shared(R * SAMPLING_TREE_CHILDREN, "drawn children");
+    children_.childUniforms = shared(R * SAMPLING_TREE_CHILDREN * 4, "child uniforms");
     // no children drawn until a draft says so: such rows draw from their whole distribution
     std::vector<uint8_t> none(R * SAMPLING_TREE_CHILDREN, uint8_t(SAMPLING_NO_DRAW));
-    sampling_.candidateDraws.upload(none.data(), none.size());
+    children_.candidateDraws.upload(none.data(), none.size());
   }
   switch (which) {
-  case 0: return sampling_.candidateIds;
-  case 1: return sampling_.candidateProbabilities;
-  case 2: return sampling_.candidateDraws;
-  case 3: return sampling_.childUniforms;
+  case 0: return children_.candidateIds;
+  case 1: return children_.candidateProbabilities;
+  case 2: return children_.candidateDraws;
+  case 3: return children_.childUniforms;
   default: throw std::invalid_argument("no such candidate buffer");
   }
 }
@@ -333,7 +333,7 @@ void DenseVerify::encode(hip::CommandGraph &graph, const std::vector<VerifyLane>
   }
   const ops::AttentionGeometry geometry{dims_.qHeads, dims_.kvHeads, dims_.headDimension, dims_.rotaryPairs, dims_.normalizeHeads};
   const ops::AttentionPlan plan = ops::PagedAttention::plan(geometry, sequences);
-  if (samples && !sampling_.candidateIds) (void)draftProbabilities();
+  if (samples && !testChildren_) (void)draftProbabilities();
   if (dims_.rotaryPairs)
     ops::RoPE::addTreeTables(graph, inverseFrequency_, depths_, ropeCos_, ropeSin_, dims_.rotaryPairs, rope);
   encodeEmbedding(graph, rows);
@@ -344,7 +344,15 @@ void DenseVerify::encode(hip::CommandGraph &graph, const std::vector<VerifyLane>
     for (uint32_t layer = 0; layer < dims_.layers; ++layer) encodeLayer(graph, layer, plan, rows, feeds && layer > 0, feeds);
     encodeHead(graph, rows, feeds);
   }
-  ops::Sampling::addVerify(graph, sampling_, dims_.vocabulary, dims_.vocabulary, laneRows, policies);
+  // the sampled lanes' test is the step's choice (setTestChildren), not a property of which buffers were ever fetched
+  ops::SamplingBuffers sampling = sampling_;
+  if (testChildren_) {
+    sampling.candidateIds = children_.candidateIds;
+    sampling.candidateProbabilities = children_.candidateProbabilities;
+    sampling.candidateDraws = children_.candidateDraws;
+    sampling.childUniforms = children_.childUniforms;
+  }
+  ops::Sampling::addVerify(graph, sampling, dims_.vocabulary, dims_.vocabulary, laneRows, policies);
   const ops::AcceptanceBuffers acceptance{inputTokens_, treeRows_, tokens_, retained_, acceptedCount_, retainedRows_};
   ops::Sampling::addAcceptance(graph, acceptance, laneRows, remaining,
                                {SAMPLING_NO_TOKEN, SAMPLING_NO_TOKEN, SAMPLING_NO_TOKEN, SAMPLING_NO_TOKEN});

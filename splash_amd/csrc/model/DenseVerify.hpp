@@ -73,8 +73,11 @@ public:
   // The sampled rows of tree blocks test the children their draft drew among sixteen candidates (Sampling.hpp,
   // candidateIds ..): the four host-visible buffers a draft writes, allocated on first use -- which: 0 ids uint32
   // [rows][16], 1 probabilities fp32 [rows][16], 2 drawn children bytes [rows][4], 3 child uniforms fp32 [rows][4].
-  // Once they exist, every step's sampled lanes read them instead of the full-vocabulary draft probabilities.
+  // Fetching them changes no step: setTestChildren chooses, for the steps encoded after it, whether sampled lanes
+  // read them or the full-vocabulary draft probabilities (the default).
   [[nodiscard]] const hip::Buffer &candidateChildren(uint32_t which);
+  void setTestChildren(bool on) { testChildren_ = on; if (on) (void)candidateChildren(0); }
+  [[nodiscard]] bool testChildren() const noexcept { return testChildren_; }
   [[nodiscard]] const hip::Buffer &hidden(uint32_t index) const noexcept { return hidden_[index & 1]; }
   [[nodiscard]] const hip::Buffer &qkvRows() const noexcept { return qkv_; }
   [[nodiscard]] const hip::Buffer &attentionRows() const noexcept { return attention_; }
@@ -136,7 +139,8 @@ private:
   // chained projections: the gate/up and down tables, each link's partials and counters, the chain's progress words
   hip::Buffer chainTables_[2], chainProgress_;
   ops::LinearScratch chainScratch_[GGUF_CHAIN_LINKS];
-  bool chained_ = false, encodedChains_ = false, fusedPrepare_ = false;
+  bool chained_ = false, encodedChains_ = false, fusedPrepare_ = false, testChildren_ = false;
+  ops::SamplingBuffers children_;   // the four candidate-children buffers, bound into a step's sampling buffers when it tests them
   void encodeChainedLayers(hip::CommandGraph &graph, const ops::AttentionPlan &plan, uint32_t rows);
   [[nodiscard]] bool chains(uint32_t rows) const noexcept;
   ops::AttentionWorkspace attentionWorkspace_;

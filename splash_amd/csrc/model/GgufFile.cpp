@@ -6,6 +6,7 @@
 #include <array>
 #include <cmath>
 #include <cstring>
+#include <set>
 #include <fcntl.h>
 #include <sys/mman.h>
 #include <sys/stat.h>
@@ -162,12 +163,14 @@ void GgufFile::parse(const std::string &path, uint32_t file) {
   const uint32_t version = r.take<uint32_t>();
   if (version != 3) throw GgufError("unsupported GGUF version " + std::to_string(version));
   const uint64_t tensorCount = r.take<uint64_t>(), valueCount = r.take<uint64_t>();
-  if (tensorCount > (1u << 20) || valueCount > (1u << 20)) throw GgufError("implausible GGUF counts");
+  if (tensorCount > 16384 || valueCount > 16384) throw GgufError("implausible GGUF header counts");
   // Only the first part's metadata is kept: a later part repeats split.* alone, whose split.no must be its place.
   GgufMetadata later;
   GgufMetadata &metadata = file ? later : metadata_;
+  std::set<std::string, std::less<>> keys;   // a key holds one value (GgufFile.cpp:191-194 of the reference)
   for (uint64_t i = 0; i < valueCount; ++i) {
     const std::string key = r.string();
+    if (!keys.insert(key).second) throw GgufError("duplicate GGUF metadata key: " + key);
     const uint32_t type = r.take<uint32_t>();
     if (file && key == "split.no" && type != kU16 && type != kU32) throw GgufError("invalid split.no in " + path);
     switch (type) {
@@ -187,7 +190,8 @@ void GgufFile::parse(const std::string &path, uint32_t file) {
     }
   }
   if (file && later.unsignedValue("split.no").value_or(file) != file) throw GgufError("GGUF split file " + path + " is out of order");
-  const uint64_t alignment = metadata.unsignedValue("general.alignment").value_or(metadata_.unsignedValue("general.alignment").value_or(32));
+  // the first part's alignment holds for every part: a later part's metadata is read for its split.no alone
+  const uint64_t alignment = metadata_.unsignedValue("general.alignment").value_or(32);
   if (alignment < 8 || alignment > 65536 || (alignment & (alignment - 1))) throw GgufError("invalid GGUF alignment");
   const size_t firstTensor = tensors_.size();
   tensors_.reserve(firstTensor + tensorCount);

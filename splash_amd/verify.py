@@ -125,14 +125,27 @@ class DenseVerify:
         default): the results are the same bit for bit."""
         check(lib.spo_dense_verify_set_chained(self.handle, int(bool(chained))))
 
+    def chain_status(self):
+        """0 when every chained projection of the last completed step met its wait, nonzero when one gave up (the step's
+        logits, hidden rows and results are void then); reading it clears it."""
+        status = ctypes.c_uint32()
+        check(lib.spo_dense_verify_chain_status(self.handle, ctypes.byref(status)))
+        return status.value
+
     def set_fused_prepare(self, fused):
         """Whether a layer's q|k|v projection also prepares its attention block where the kernels take the pair (off by
         default): the results are the same bit for bit."""
         check(lib.spo_dense_verify_set_fused_prepare(self.handle, int(bool(fused))))
 
+    def test_children(self, on=True):
+        """Whether the sampled lanes of steps encoded from now on test their draft's drawn children among sixteen
+        candidates, or (the default) one child against the full-vocabulary draft probabilities."""
+        check(lib.spo_dense_verify_set_test_children(self.handle, int(bool(on))))
+
     def set_candidate_children(self, ids, probabilities, draws, child_uniforms):
         """The sampled rows' candidate children, by packed row: ids uint32 [rows][16], probabilities fp32 [rows][16], draws
-        bytes [rows][4] (0xFF past a row's drawn children), child_uniforms fp32 [rows][4]."""
+        bytes [rows][4] (0xFF past a row's drawn children), child_uniforms fp32 [rows][4]; later steps test them."""
+        self.test_children(True)
         for which, array, dtype in ((0, ids, np.uint32), (1, probabilities, np.float32), (2, draws, np.uint8), (3, child_uniforms, np.float32)):
             raw = np.ascontiguousarray(array, dtype).view(np.uint8).ravel()
             self.buffer(CANDIDATE_CHILDREN, which).contents()[:raw.size] = raw

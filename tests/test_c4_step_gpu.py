@@ -1,7 +1,7 @@
 """Parity of the dense verify step at BASELINE.json's headline shape (config 4: 64 layers, hidden 5120, 64 q / 8 kv
 heads x 128, SwiGLU 25600, vocabulary 151936, Q4_K with Q6_K down-projection and LM head, 32K INT8 context, 16-row
-draft block), through the C ABI. The 64 layers share one drawn weight set and one drawn context (each layer's context
-is its own copy in HBM): what a layer adds to the step is depth, which the free-running checks cover, not new arithmetic.
+draft block), through the C ABI. The 64 layers cycle through four drawn weight sets and four drawn contexts (each
+layer's weights and context are its own copy in HBM), so that a layer's roundings meet other weights in the next.
 
 Tolerances: hidden rows and logits, teacher-forced (each GPU layer against the oracle run on the GPU's own layer input):
 cosine >= 0.9999 and |delta| <= max(2e-2, two bf16 steps); greedy ids, accepted counts and retained masks bit-exact
@@ -51,9 +51,9 @@ def stage_close(name, got_bits, want_bits, steps_allowed=2, cos_floor=0.99999):
 @pytest.fixture(scope="module")
 def c4(backend):
     print("case config 4: building the 27B-shaped model", flush=True)
-    model = DenseModel(seed=41, down_format=orc.FMT_Q6K, distinct_layers=1, **C4)
+    model = DenseModel(seed=41, down_format=orc.FMT_Q6K, distinct_layers=4, **C4)
     gpu = model.build_gpu(backend, max_lanes=4, context_tokens=[c + 16 for c in LANE_COMMITTED])
-    model.seed_context(gpu, None, np.random.default_rng(42), distinct=1)
+    model.seed_context(gpu, None, np.random.default_rng(42), distinct=4)
     print("case config 4: model resident", flush=True)
     yield model, gpu
     del gpu
@@ -69,7 +69,9 @@ def logits_of(gpu, rows):
 
 def test_config4_layers_and_head_teacher_forced_and_greedy_acceptance(backend, c4):
     """Layers 0, 31 and 63 and the head at the headline shape against the oracle, each from the GPU's own input rows;
-    greedy acceptance of the step bit-exact against the oracle's walk over the step's logits."""
+    greedy acceptance of the step bit-exact against the oracle's walk over the step's logits; and the oracle's own
+    chain of all 64 layers run free beside them, against which the step (its norms left to the projections that read
+    them) drifts no further than its parts run one by one (each after a norm pass)."""
     model, gpu = c4
     print("case config 4 teacher-forced layers, batch 1, 32K context", flush=True)
     rows, committed = LANE_ROWS[0], LANE_COMMITTED[0]
@@ -91,9 +93,15 @@ def test_config4_layers_and_head_teacher_forced_and_greedy_acceptance(backend, c
     hidden_of = lambda: rows_of(verify.HIDDEN, H)
     backend.run(gpu.encode_part(0, 0, lane))
     assert np.array_equal(hidden_of(), model.oracle_embedding(tokens))
+    free = model.oracle_embedding(tokens)       # the oracle's own chain, fed nothing of the GPU's
     for layer in range(64):
         before = hidden_of() if layer in (0, 31, 63) else None
         backend.run(gpu.encode_part(1, layer, lane))
+        free = model.oracle_layer(free, layer, committed, model.table_first[0])
+        if layer % 16 == 15:
+            g, w = orc.bf16_to_f32(hidden_of()).astype(np.float64), orc.bf16_to_f32(free).astype(np.float64)
+            print(f" after layer {layer}, parts against the oracle's chain: cosine {cosine(g, w):.6f} relative rms "
+                  f"{np.sqrt(((g - w) ** 2).mean() / (w ** 2).mean()):.4f}", flush=True)
         if before is None:
             continue
         print(f" layer {layer}", flush=True)
@@ -146,6 +154,22 @@ def test_config4_layers_and_head_teacher_forced_and_greedy_acceptance(backend, c
     drift = float(np.abs(step_logits - got).max())
     print(f"  whole step vs parts, free-running over 64 layers: cosine {cosine(step_logits, got):.6f} max-abs {drift:.4f}", flush=True)
     assert cosine(step_logits, got) >= 0.999
+    # Both against the oracle's own chain: six bf16 roundings a layer, each now and then a step apart between a sum
+    # taken in fp32 and one taken exactly, over 64 layers of distinct weights (the differences add in quadrature:
+    # about 0.7 % of the rows' size after a layer, 5 % after 64). The step's deferred norms must not add to that:
+    # its logits lie as near the chain's as the parts' do, and where the chain's top two are well apart the ids agree.
+    chain = model.oracle_head(free)
+    rms = lambda a: float(np.sqrt(((a - chain) ** 2).mean()))
+    chain_ids = chain.argmax(axis=1)
+    part2 = np.partition(chain, -2, axis=1)
+    apart = part2[:, -1] - part2[:, -2] > 0.25
+    print(f"  against the oracle's chain: step cosine {cosine(step_logits, chain):.6f} rms {rms(step_logits):.4f} max-abs "
+          f"{np.abs(step_logits - chain).max():.4f}; parts cosine {cosine(got, chain):.6f} rms {rms(got):.4f} max-abs "
+          f"{np.abs(got - chain).max():.4f}; logits rms {float(np.sqrt((chain ** 2).mean())):.3f}; ids equal "
+          f"{int((step_logits.argmax(axis=1) == chain_ids).sum())}/16 (step) {int((got.argmax(axis=1) == chain_ids).sum())}/16 (parts)", flush=True)
+    assert cosine(step_logits, chain) >= 0.998 and cosine(got, chain) >= 0.998
+    assert rms(step_logits) <= 1.15 * rms(got)
+    assert np.array_equal(step_logits.argmax(axis=1)[apart], chain_ids[apart])
 
 
 def test_config4_batch_of_four_lanes_equals_each_lane_alone(backend, c4):

@@ -69,6 +69,13 @@ def test_malformed_files_are_refused(tmp_path):
         gw.write_gguf(path, [("general.alignment", gw.U32, alignment)], tensors, alignment=alignment)
         with pytest.raises(splash_amd.SplashError):
             gguf.GgufFile(path)
+    # a key holds one value (the reference's GgufFile.cpp:191-194, as llama.cpp's reader): a repeated key is refused,
+    # whatever its second value
+    twice = tmp_path / "twice.gguf"
+    gw.write_gguf(twice, [("general.architecture", gw.STRING, "qwen3"), ("qwen3.block_count", gw.U32, 1), ("qwen3.block_count", gw.U32, 2)],
+                  [("t", gw.GGML_Q4_K, [256], x)])
+    with pytest.raises(splash_amd.SplashError, match="duplicate GGUF metadata key"):
+        gguf.GgufFile(twice)
 
 
 @pytest.mark.gpu
@@ -189,6 +196,16 @@ def test_a_split_file_reads_as_one(tmp_path):
     gw.write_gguf(short[2], [("split.no", gw.U16, 2), ("split.count", gw.U16, 3)], [])
     with pytest.raises(splash_amd.SplashError, match="split.tensors.count"):
         gguf.GgufFile(short)
+    # a later part's general.alignment is not read: its tensors lie at the first part's alignment (here 32, which the
+    # part's own claim of 4096 would refuse for offsets that are multiples of 32 only)
+    claims = write_split(tmp_path / "claims.gguf", metadata, tensors, 3)
+    share = (len(tensors) + 1) // 2
+    gw.write_gguf(claims[2], [("split.no", gw.U16, 2), ("split.count", gw.U16, 3), ("general.alignment", gw.U32, 4096)], tensors[share:], alignment=32)
+    claimed = gguf.GgufFile(claims)
+    offsets = np.cumsum([0] + [(np.asarray(d).nbytes + 31) // 32 * 32 for _, _, _, d in tensors[share:]])[:-1]
+    assert any(int(o) % 4096 for o in offsets)                                 # the layout really is the first part's
+    for a, b in zip(claimed.tensors, one.tensors):
+        assert a.name == b.name and np.array_equal(claimed.data(a), one.data(b))
     # a single file that says it is a part of several
     alone = tmp_path / "alone.gguf"
     gw.write_gguf(alone, metadata + [("split.count", gw.U16, 2)], tensors)

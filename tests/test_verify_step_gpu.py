@@ -83,6 +83,14 @@ def test_config1_verify_step(backend, rows, context):
     cos = (chain_logits.astype(np.float64) * want["logits"]).sum() / np.sqrt((chain_logits.astype(np.float64) ** 2).sum() * (want["logits"] ** 2).sum())
     err = np.abs(chain_logits - want["logits"]).max()
     assert cos >= 0.9999 and err <= 5e-2, (cos, err)
+    # Where that difference comes from is not the step's deferred norms: the parts, each after a norm pass that rounds as
+    # the oracle's does, lie as far from the oracle's chain (the stages that move are the SwiGLU rows and the attention
+    # rows, where a sum taken in fp32 and one taken exactly fall on two sides of a bf16 rounding now and then, and a
+    # large activation is worth 3e-2 a step).
+    rms = lambda a: float(np.sqrt(((a - want["logits"]) ** 2).mean()))
+    print(f"  free-running against the oracle's chain: step max-abs {err:.4f} rms {rms(chain_logits):.5f}; parts max-abs "
+          f"{np.abs(got_logits - want['logits']).max():.4f} rms {rms(got_logits):.5f}", flush=True)
+    assert rms(chain_logits) <= 1.15 * rms(got_logits)
     sure = top2_gap(want["logits"]) > 1e-1
     assert np.array_equal(gpu_argmax[sure], want["selected"][sure])
     # where the oracle's top two are closer than that, the GPU's choice is still one of the oracle's near-ties
@@ -237,6 +245,7 @@ def test_chained_projections_change_nothing(backend, lanes_rows):
         outcomes = []
         for _ in range(3):
             backend.run(graph)
+            assert gpu.chain_status() == 0           # what a reader of the buffers asks before it trusts them
             outcomes.append((gpu.buffer(verify.LOGITS).download(np.float32, total * 32000).copy(),
                              gpu.buffer(verify.HIDDEN, 0).download(np.uint16, total * 1024).copy(), gpu.results(lanes)))
         return len(graph), outcomes
