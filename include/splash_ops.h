@@ -263,6 +263,28 @@ sp_status spo_gdn_add_decode(spo_graph *graph, const spo_gdn_decode_buffers *buf
 sp_status spo_gdn_add_fold(spo_graph *graph, sp_buffer *states, sp_buffer *tape, sp_buffer *retained_rows, uint64_t step_tape,
                            uint64_t state_cell, uint64_t fold_cell, const spo_gdn_shape *shape, uint32_t layers, uint32_t rows,
                            const spo_gdn_state_strides *state);
+typedef struct spo_gdn_prefill_buffers { /* ops::GdnPrefillBuffers (GDN.hpp:75-93) */
+  sp_buffer *packed, *convolution_weights, *states, *decay_weights, *time_bias, *mixer_norm;
+  uint32_t float_norm; /* the output norm's weights are fp32 */
+  uint32_t reserved;
+  sp_buffer *queries, *keys;    /* bf16 [tokens][key_heads * 128], written by the prepare pass */
+  sp_buffer *values;            /* bf16 [tokens][value_heads * 128] */
+  sp_buffer *decay, *beta;      /* fp32 and bf16 [tokens][value_heads] */
+  sp_buffer *recurrent_rows;    /* bf16 [tokens][value_heads * 128]: the scan's rows before the gated norm */
+  sp_buffer *hidden;            /* bf16 [tokens][value_heads * 128] */
+  uint64_t current_cell, next_cell; /* byte offsets in the states buffer: the cell the chunk starts from, the one it leaves */
+} spo_gdn_prefill_buffers;
+typedef struct spo_gdn_prefill_capture { /* ops::GdnPrefillCapture (GDN.hpp:95-104): the cell after the chunk's first `tokens` rows */
+  uint32_t tokens, reserved;
+  uint64_t cell;
+} spo_gdn_prefill_capture;
+/* GDN::addPrefill (GDN.hpp:166-181, GDN.cpp:132-222): a prompt chunk of `tokens` rows of one lane and layer, every row
+ * entering the state: a prepare and a scan dispatch for each run between captures (ascending, inside the rows; a run
+ * continues from the cell the run before wrote, and no run writes the cell it reads), then one gate dispatch over all
+ * rows. The cells hold, bit for bit, what the same rows leave when they enter as accepted verify blocks. */
+sp_status spo_gdn_add_prefill(spo_graph *graph, const spo_gdn_prefill_buffers *buffers, const spo_gdn_shape *shape, uint32_t layer,
+                              uint32_t tokens, const spo_gdn_state_strides *state, uint32_t tiled_heads,
+                              const spo_gdn_prefill_capture *captures, uint32_t count);
 
 /* ---- StateCodec (runtime/ops/StateCodec.hpp:11-49; runtime/metal/abi/StateCodec.h): the cached form of the
  *      recurrent layers, int8 codes row by row and then a bf16 scale per block of 32 values ---- */

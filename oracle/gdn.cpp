@@ -309,6 +309,90 @@ int orc_gdn_fold(const OrcGdnShape *s, const uint16_t *conv_in, const float *sta
   return 0;
 }
 
+// A prompt chunk of `tokens` rows of one lane and layer (kernels/prefill/gdn.metal:196-262 the prepare pass,
+// :24-160 the scan, :312-341 the gate; GDN.cpp:176-222): every row enters the state. Row t's taps are rows
+// t - 3 .. t of the carried inputs followed by the chunk's own; its k, v and gates are those a decode step
+// leaves on its tape for the same rows, a state row's recurrence is foldRow's, and its output reads the state
+// after its own token, o_t = S_t q_t (prefill/gdn.metal:124-141). The reference's prefill sums a row's dot
+// products eight lanes of sixteen columns at a time where its decode kernels sum 32 lanes of four; this
+// restatement keeps the decode order for both, so that a chunk and the same rows as accepted blocks leave one
+// state, and is held to the reference's fp64 bounds for the pass (gdn_metal_test.mm:283-409).
+int orc_gdn_prefill(const OrcGdnShape *s, const uint16_t *packed, uint32_t tokens, const uint16_t *conv_weights, const float *a_scale,
+                    const uint16_t *dt_bias, const void *norm_weight, const uint16_t *conv_in, const float *state_in, uint16_t *queries,
+                    uint16_t *keys, uint16_t *values, float *decay, uint16_t *beta, uint16_t *conv_out, float *state_out,
+                    uint16_t *recurrent, uint16_t *hidden) {
+  if (!tokens || s->conv_dim != (2 * s->key_heads + s->value_heads) * kDim) return -1;
+  const uint32_t KH = s->key_heads, VH = s->value_heads, C = s->conv_dim, P = s->packed_width, perKey = VH / KH;
+  const uint32_t keyWidth = KH * kDim, valueWidth = VH * kDim, zOffset = C, bOffset = C + valueWidth, aOffset = bOffset + VH;
+  auto input = [&](uint32_t position) { return position < 3 ? conv_in + size_t(position) * C : packed + size_t(position - 3) * P; };
+  std::vector<uint16_t> conv(C);
+  for (uint32_t t = 0; t < tokens; ++t) {
+    for (uint32_t c = 0; c < C; ++c) {
+      float value = 0.f;
+      for (uint32_t tap = 0; tap < kTaps; ++tap) value += bf2f(input(t + tap)[c]) * bf2f(conv_weights[size_t(c) * kTaps + tap]);
+      value = bf2f(f2bf(value));
+      conv[c] = f2bf(silu(value));
+    }
+    for (uint32_t kh = 0; kh < KH; ++kh) {
+      float q[kDim], k[kDim];
+      for (uint32_t d = 0; d < kDim; ++d) {
+        q[d] = bf2f(conv[kh * kDim + d]);
+        k[d] = bf2f(conv[keyWidth + kh * kDim + d]);
+      }
+      const float qs = 1.0f / std::sqrt(sumSquares128(q) / float(kDim) + kEps), ks = 1.0f / std::sqrt(sumSquares128(k) / float(kDim) + kEps);
+      for (uint32_t d = 0; d < kDim; ++d) {
+        queries[size_t(t) * keyWidth + kh * kDim + d] = f2bf(bf2f(f2bf(q[d] * qs)) * 0.0078125f);
+        keys[size_t(t) * keyWidth + kh * kDim + d] = f2bf(bf2f(f2bf(k[d] * ks)) * 0.08838834765f);
+      }
+    }
+    for (uint32_t c = 0; c < valueWidth; ++c) values[size_t(t) * valueWidth + c] = conv[2 * keyWidth + c];
+    for (uint32_t h = 0; h < VH; ++h) {
+      const float b = bf2f(packed[size_t(t) * P + bOffset + h]);
+      beta[size_t(t) * VH + h] = f2bf(sigmoid(b));
+      const float x = bf2f(f2bf(bf2f(packed[size_t(t) * P + aOffset + h]) + bf2f(dt_bias[h])));
+      const float softplus = bf2f(f2bf(std::max(x, 0.0f) + std::log2(1.0f + std::exp2(-1.44269504089f * std::fabs(x))) * 0.69314718056f));
+      decay[size_t(t) * VH + h] = std::exp(a_scale[h] * softplus);
+    }
+  }
+  for (uint32_t r = 0; r < 3; ++r) std::copy(input(tokens + r), input(tokens + r) + C, conv_out + size_t(r) * C);
+  // per value head: its rows' k, q, v and gates side by side, then each state row through the chunk
+  std::vector<uint16_t> hk(size_t(tokens) * kDim), hq(size_t(tokens) * kDim), hv(size_t(tokens) * kDim), hb(tokens), out(size_t(tokens) * kDim);
+  std::vector<float> hd(tokens);
+  for (uint32_t h = 0; h < VH; ++h) {
+    const uint32_t kh = h / perKey;
+    for (uint32_t t = 0; t < tokens; ++t) {
+      std::copy(keys + size_t(t) * keyWidth + kh * kDim, keys + size_t(t) * keyWidth + (kh + 1) * kDim, hk.begin() + size_t(t) * kDim);
+      std::copy(queries + size_t(t) * keyWidth + kh * kDim, queries + size_t(t) * keyWidth + (kh + 1) * kDim, hq.begin() + size_t(t) * kDim);
+      std::copy(values + size_t(t) * valueWidth + h * kDim, values + size_t(t) * valueWidth + (h + 1) * kDim, hv.begin() + size_t(t) * kDim);
+      hd[t] = decay[size_t(t) * VH + h];
+      hb[t] = beta[size_t(t) * VH + h];
+    }
+    for (uint32_t r = 0; r < kDim; ++r) {
+      float state[kDim];
+      const size_t base = (size_t(h) * kDim + r) * kDim;
+      std::copy(state_in + base, state_in + base + kDim, state);
+      foldRow(state, r, tokens, hk.data(), hv.data(), hd.data(), hb.data(), hq.data(), out.data());
+      std::copy(state, state + kDim, state_out + base);
+    }
+    const uint32_t outHead = (s->flags & 1u) ? (h % perKey) * KH + h / perKey : h;
+    for (uint32_t t = 0; t < tokens; ++t) {
+      float value[kDim];
+      for (uint32_t d = 0; d < kDim; ++d) {
+        recurrent[size_t(t) * valueWidth + h * kDim + d] = out[size_t(t) * kDim + d];
+        value[d] = bf2f(out[size_t(t) * kDim + d]);
+      }
+      const float inverse = 1.0f / std::sqrt(sumSquares128(value) / float(kDim) + kEps);
+      for (uint32_t d = 0; d < kDim; ++d) {
+        const float w = (s->flags & 4u) ? static_cast<const float *>(norm_weight)[d] : bf2f(static_cast<const uint16_t *>(norm_weight)[d]);
+        const float normalized = bf2f(f2bf((value[d] * inverse) * w));
+        const float z = bf2f(packed[size_t(t) * P + zOffset + h * kDim + d]);
+        hidden[(size_t(t) * VH + outHead) * kDim + d] = f2bf((normalized * ((s->flags & 2u) ? 1.0f : z)) / (1.0f + std::exp2(-1.44269504089f * z)));
+      }
+    }
+  }
+  return 0;
+}
+
 // The reference's own check of a decode step (gdn_decode_metal_test.mm:373-522): convolution + SiLU,
 // normalized heads, gates and the recurrence in fp64 from the same packed rows, no intermediate
 // rounding but the stored bf16 inputs. Outputs: k and v rows [rows][kv_width], beta and decay

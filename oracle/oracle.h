@@ -245,6 +245,17 @@ int orc_gdn_decode(const struct OrcGdnShape *s, const uint16_t *packed, uint32_t
 // hold it (gdn.metal:630-698, exact cells). Returns 1 and writes nothing when the path is shorter.
 int orc_gdn_fold(const struct OrcGdnShape *s, const uint16_t *conv_in, const float *state_in, uint8_t *step_tape,
                  uint32_t path, uint32_t rows, uint16_t *conv_out, float *state_out);
+// A prompt chunk of `tokens` rows of one lane and layer (kernels/prefill/gdn.metal, GDN.cpp:176-222): queries and keys
+// bf16 [tokens][kh * 128], values [tokens][vh * 128], decay fp32 and beta bf16 [tokens][vh], the carry and the state
+// after the chunk, the scan's rows (recurrent, bf16 [tokens][vh * 128]: o_t = S_t q_t) and their gated norm (hidden).
+// Pinned by the fp64 check below under the reference's bounds for the pass (gdn_metal_test.mm:283-409: prepared rows
+// within 2 bf16 steps, scan rows within one step + 1e-5, state within 1e-5, gated rows within 2 steps and at most 1 %
+// of them off the fp64 rounding), and bit for bit by orc_gdn_decode + orc_gdn_fold over the same rows as accepted
+// blocks (tests/test_oracle_gdn.py).
+int orc_gdn_prefill(const struct OrcGdnShape *s, const uint16_t *packed, uint32_t tokens, const uint16_t *conv_weights,
+                    const float *a_scale, const uint16_t *dt_bias, const void *norm_weight, const uint16_t *conv_in,
+                    const float *state_in, uint16_t *queries, uint16_t *keys, uint16_t *values, float *decay, uint16_t *beta,
+                    uint16_t *conv_out, float *state_out, uint16_t *recurrent, uint16_t *hidden);
 // The fp64 check of a step the reference's test makes (gdn_decode_metal_test.mm:373-522).
 int orc_gdn_reference(const struct OrcGdnShape *s, const uint16_t *packed, uint32_t rows, const uint16_t *conv_weights,
                       const float *a_scale, const uint16_t *dt_bias, const uint16_t *conv_in, const float *state_in,

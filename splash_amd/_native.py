@@ -116,6 +116,17 @@ class GdnDecodeBuffers(ctypes.Structure):
                                    "hidden")] + [("float_norm", c_u32), ("tree_rows", c_p), ("hidden_table", c_p)]
 
 
+class GdnPrefillBuffers(ctypes.Structure):
+    _fields_ = [(n, c_p) for n in ("packed", "convolution_weights", "states", "decay_weights", "time_bias", "mixer_norm")] + \
+               [("float_norm", c_u32), ("reserved", c_u32)] + \
+               [(n, c_p) for n in ("queries", "keys", "values", "decay", "beta", "recurrent_rows", "hidden")] + \
+               [("current_cell", c_u64), ("next_cell", c_u64)]
+
+
+class GdnPrefillCapture(ctypes.Structure):
+    _fields_ = [("tokens", c_u32), ("reserved", c_u32), ("cell", c_u64)]
+
+
 class StateCodecShape(ctypes.Structure):
     _fields_ = [("layers", c_u32), ("rows", c_u32), ("columns", c_u32), ("bf16_state", c_u32), ("state_layer_bytes", c_u64),
                 ("codes_layer_bytes", c_u64)]
@@ -266,6 +277,7 @@ _sig("spo_embedding_add", c_int, c_p, c_u32, c_p, c_u32, c_u32, c_p, c_p, c_u32)
 _sig("spo_rope_add_tree_tables", c_int, c_p, c_p, c_p, c_p, c_p, c_u32, P(RopeSequence), c_u32)
 _sig("spo_gdn_layout", c_int, P(GdnShape), c_u32, P(GdnStateStrides), P(c_u64), P(c_u64))
 _sig("spo_gdn_add_decode", c_int, c_p, P(GdnDecodeBuffers), P(GdnShape), c_u32, P(GdnStateStrides), c_u32, P(GdnLane), c_u32)
+_sig("spo_gdn_add_prefill", c_int, c_p, P(GdnPrefillBuffers), P(GdnShape), c_u32, c_u32, P(GdnStateStrides), c_u32, P(GdnPrefillCapture), c_u32)
 _sig("spo_gdn_add_fold", c_int, c_p, c_p, c_p, c_p, c_u64, c_u64, c_u64, P(GdnShape), c_u32, c_u32, P(GdnStateStrides))
 _sig("spo_state_codec_layer_bytes", c_u64, c_u32, c_u32)
 for _name in ("spo_state_codec_add_quantize", "spo_state_codec_add_dequantize", "spo_state_codec_add_copy"):

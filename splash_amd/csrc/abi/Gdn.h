@@ -100,7 +100,27 @@ struct GdnFoldParams {
   uint64_t fold_cell;   // the cell the fold writes
 };
 
+// gdn_prefill_prepare / gdn_prefill_scan / gdn_prefill_gate: one run of a prompt chunk of one lane, `tokens`
+// rows that all enter the state (the reference's GDNPrefillParams, runtime/ops/GDN.cpp:176-222): the run reads
+// the layer's convolution carry and recurrent state of `current_cell` and writes those after its rows to
+// `next_cell`, another cell. No tape: a prompt's rows are never rolled back.
+#define GDN_SCAN_STATE_ROWS 8u    // state rows of one scan workgroup (the reference's SPLASH_GDN_SCAN_STATE_ROWS is 16)
+#define GDN_SCAN_BLOCK 16u        // tokens a scan workgroup stages at a time
+struct GdnPrefillParams {
+  struct GdnShapeParams shape;
+  uint32_t flags;
+  uint32_t layer;
+  uint32_t tokens;        // rows of the run
+  uint32_t first;         // the run's first row in the chunk's buffers (packed rows and every buffer of rows)
+  uint64_t conv_layer_bytes;
+  uint64_t recurrent_layer_bytes;
+  uint64_t convolution_state_bytes;
+  uint64_t current_cell;
+  uint64_t next_cell;
+};
+
 #ifdef __cplusplus
+static_assert(sizeof(GdnPrefillParams) == 72, "GDN prefill parameters are 72 bytes on both sides");
 static_assert(sizeof(GdnLane) == 48, "a GDN lane is 48 bytes on both sides");
 static_assert(sizeof(GdnDecodeParams) == 56 + 48 * GDN_MAXIMUM_LANES, "GDN decode parameters are 440 bytes on both sides");
 static_assert(sizeof(GdnFoldParams) == 80, "GDN fold parameters are 80 bytes on both sides");

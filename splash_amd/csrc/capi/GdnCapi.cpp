@@ -64,6 +64,20 @@ sp_status spo_gdn_add_fold(spo_graph *graph, sp_buffer *states, sp_buffer *tape,
   });
 }
 
+sp_status spo_gdn_add_prefill(spo_graph *graph, const spo_gdn_prefill_buffers *b, const spo_gdn_shape *shape, uint32_t layer,
+                              uint32_t tokens, const spo_gdn_state_strides *state, uint32_t tiled_heads,
+                              const spo_gdn_prefill_capture *captures, uint32_t count) {
+  return capi::guard([&] {
+    capi::require(graph && b && shape && state && (captures || !count), "graph, buffers, shape, strides or captures");
+    ops::GdnPrefillBuffers buffers{B(b->packed), B(b->convolution_weights), B(b->states), B(b->decay_weights), B(b->time_bias),
+                                   B(b->mixer_norm), b->float_norm != 0, B(b->queries), B(b->keys), B(b->values), B(b->decay),
+                                   B(b->beta), B(b->recurrent_rows), B(b->hidden), b->current_cell, b->next_cell};
+    std::vector<ops::GdnPrefillCapture> list;
+    for (uint32_t i = 0; i < count; ++i) list.push_back({captures[i].tokens, captures[i].cell});
+    ops::GDN::addPrefill(capi::graphOf(graph), buffers, shapeOf(*shape), layer, tokens, stridesOf(*state),
+                         tiled_heads ? ops::GdnHeadOrder::Tiled : ops::GdnHeadOrder::Grouped, list);
+  });
+}
 
 uint64_t spo_state_codec_layer_bytes(uint32_t rows, uint32_t columns) { return state_codec_layer_bytes(rows, columns); }
 

@@ -115,14 +115,82 @@ __device__ __forceinline__ History history_of(const uint16_t *carried, const uin
   return h;
 }
 
+// A row's convolution + SiLU of one channel from its four taps, oldest first (gdn_primitives.h:37-50).
+__device__ __forceinline__ float conv_silu(const uint16_t *const (&taps)[kTaps], const uint16_t *conv_weights, uint32_t channel) {
+  float value = 0.f;
+#pragma unroll
+  for (uint32_t tap = 0; tap < kTaps; ++tap)
+    value += bf16_bits_to_float(taps[tap][channel]) * bf16_bits_to_float(conv_weights[size_t(channel) * kTaps + tap]);
+  value = round_bf16(value);
+  return round_bf16(silu_of(value));
+}
+
+// A row's normalized, scaled query and key and its value of one head as bf16 bits, lane l the
+// dimensions l and 64 + l (gdn.metal:198-232): q and k are RMS-normed over the head, rounded, then
+// scaled by 1/128 and 1/sqrt(128).
+struct HeadRow {
+  uint32_t query[2], key[2], value[2];
+};
+__device__ __forceinline__ HeadRow head_row(const uint16_t *const (&taps)[kTaps], const uint16_t *conv_weights, uint32_t qChannel,
+                                            uint32_t kChannel, uint32_t vChannel, uint32_t lane) {
+  float q[2], k[2], v[2];
+#pragma unroll
+  for (uint32_t part = 0; part < 2; ++part) {
+    const uint32_t d = lane + 64u * part;
+    q[part] = conv_silu(taps, conv_weights, qChannel + d);
+    k[part] = conv_silu(taps, conv_weights, kChannel + d);
+    v[part] = conv_silu(taps, conv_weights, vChannel + d);
+  }
+  const float qScale = 1.0f / sqrtf(head_sum(q[0] * q[0], q[1] * q[1]) / float(kDim) + 1e-6f);
+  const float kScale = 1.0f / sqrtf(head_sum(k[0] * k[0], k[1] * k[1]) / float(kDim) + 1e-6f);
+  HeadRow row;
+#pragma unroll
+  for (uint32_t part = 0; part < 2; ++part) {
+    row.query[part] = float_to_bf16_bits(round_bf16(q[part] * qScale) * 0.0078125f);
+    row.key[part] = float_to_bf16_bits(round_bf16(k[part] * kScale) * 0.08838834765f);
+    row.value[part] = float_to_bf16_bits(v[part]);
+  }
+  return row;
+}
+
+// A row's gates of one value head (gdn_primitives.h:65-73): beta = bf16(sigmoid(b)); decay =
+// exp(a_scale bf16(softplus(bf16(a + dt_bias)))).
+struct Gates {
+  uint32_t beta;
+  float decay;
+};
+__device__ __forceinline__ Gates gates_of(const uint16_t *inputs, uint32_t bOffset, uint32_t aOffset, uint32_t head,
+                                          const float *a_scale, const uint16_t *dt_bias) {
+  Gates g;
+  g.beta = float_to_bf16_bits(sigmoid_of(bf16_bits_to_float(inputs[bOffset + head])));
+  const float x = round_bf16(bf16_bits_to_float(inputs[aOffset + head]) + bf16_bits_to_float(dt_bias[head]));
+  const float softplus = round_bf16(fmaxf(x, 0.0f) + __builtin_amdgcn_logf(1.0f + exp2_fast(-kLog2e * fabsf(x))) * 0.69314718056f);
+  g.decay = exp2_fast(kLog2e * (a_scale[head] * softplus));
+  return g;
+}
+
+// The gated output norm of a row's 128 recurrent values of one head, lane l the dimensions l and
+// 64 + l, as bf16 bits (gdn.metal:489-526): RMS norm with the mixer's weight, rounded, times silu(z)
+// (or sigmoid(z)) of the row's gate columns `z`.
+__device__ __forceinline__ void gated_norm(const float (&value)[2], const void *norm_weight, uint32_t flags, const uint16_t *z_row,
+                                           uint32_t lane, uint32_t (&bits)[2]) {
+  const float inverse = 1.0f / sqrtf(head_sum(value[0] * value[0], value[1] * value[1]) / float(kDim) + 1e-6f);
+#pragma unroll
+  for (uint32_t part = 0; part < 2; ++part) {
+    const uint32_t d = lane + 64u * part;
+    const float weight = (flags & GDN_FLOAT_NORM) ? static_cast<const float *>(norm_weight)[d]
+                                                  : bf16_bits_to_float(static_cast<const uint16_t *>(norm_weight)[d]);
+    const float normalized = round_bf16((value[part] * inverse) * weight);
+    const float z = bf16_bits_to_float(z_row[d]);
+    const float gated = (normalized * ((flags & GDN_SIGMOID_GATE) ? 1.0f : z)) / (1.0f + exp2_fast(-kLog2e * z));
+    bits[part] = float_to_bf16_bits(gated);
+  }
+}
+
 // One token's delta-rule step on the wave's state rows (R pairs, a row per half-wave): decay,
-// memory, delta, update (gdn.metal:270-298).
+// memory, delta, update (gdn.metal:270-298). k: the lane's four key columns; value: each row's value.
 template <int R>
-__device__ __forceinline__ void advance(float (&state)[R][4], const uint16_t *key, const uint16_t *value_row, const uint32_t (&value_dim)[R],
-                                        float decay, float beta, uint32_t column) {
-  const uint2 kb = *reinterpret_cast<const uint2 *>(key + column);
-  const float k[4] = {bf16_bits_to_float(kb.x & 0xFFFFu), bf16_bits_to_float(kb.x >> 16), bf16_bits_to_float(kb.y & 0xFFFFu),
-                      bf16_bits_to_float(kb.y >> 16)};
+__device__ __forceinline__ void advance_rows(float (&state)[R][4], const float (&k)[4], const float (&value)[R], float decay, float beta) {
   float memory[R];
 #pragma unroll
   for (int r = 0; r < R; ++r) {
@@ -136,10 +204,22 @@ __device__ __forceinline__ void advance(float (&state)[R][4], const uint16_t *ke
   }
 #pragma unroll
   for (int r = 0; r < R; ++r) {
-    const float delta = (bf16_bits_to_float(value_row[value_dim[r]]) - memory[r]) * beta;
+    const float delta = (value[r] - memory[r]) * beta;
 #pragma unroll
     for (int i = 0; i < 4; ++i) state[r][i] += k[i] * delta;
   }
+}
+// The same from a token's staged key row and value row (bf16 in LDS).
+template <int R>
+__device__ __forceinline__ void advance(float (&state)[R][4], const uint16_t *key, const uint16_t *value_row, const uint32_t (&value_dim)[R],
+                                        float decay, float beta, uint32_t column) {
+  const uint2 kb = *reinterpret_cast<const uint2 *>(key + column);
+  const float k[4] = {bf16_bits_to_float(kb.x & 0xFFFFu), bf16_bits_to_float(kb.x >> 16), bf16_bits_to_float(kb.y & 0xFFFFu),
+                      bf16_bits_to_float(kb.y >> 16)};
+  float value[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) value[r] = bf16_bits_to_float(value_row[value_dim[r]]);
+  advance_rows<R>(state, k, value, decay, beta);
 }
 
 constexpr int kInFlight = 4;  // row pairs a wave advances together, to overlap their reductions
@@ -215,52 +295,28 @@ __global__ __launch_bounds__(64 * kWaves) void gdn_decode(const uint16_t *__rest
         taps[tap] = depth + tap < kTaps - 1 ? history.row[depth + tap] : rowsIn + size_t(row) * P;
       }
     }
-    auto conv = [&](uint32_t channel) -> float {
-      float value = 0.f;
-#pragma unroll
-      for (uint32_t tap = 0; tap < kTaps; ++tap)
-        value += bf16_bits_to_float(taps[tap][channel]) * bf16_bits_to_float(conv_weights[size_t(channel) * kTaps + tap]);
-      value = round_bf16(value);
-      return round_bf16(silu_of(value));
-    };
-    float q[2], k[2], v[2];
-#pragma unroll
-    for (uint32_t part = 0; part < 2; ++part) {
-      const uint32_t d = lane + 64u * part;
-      q[part] = conv(qChannel + d);
-      k[part] = conv(kChannel + d);
-      v[part] = conv(vChannel + d);
-    }
-    const float qScale = 1.0f / sqrtf(head_sum(q[0] * q[0], q[1] * q[1]) / float(kDim) + 1e-6f);
-    const float kScale = 1.0f / sqrtf(head_sum(k[0] * k[0], k[1] * k[1]) / float(kDim) + 1e-6f);
+    const HeadRow row = head_row(taps, conv_weights, qChannel, kChannel, vChannel, lane);
     const uint16_t *inputs = rowsIn + size_t(token) * P;
 #pragma unroll
     for (uint32_t part = 0; part < 2; ++part) {
       const uint32_t d = lane + 64u * part;
-      const uint32_t query = float_to_bf16_bits(round_bf16(q[part] * qScale) * 0.0078125f);
-      const uint32_t key = float_to_bf16_bits(round_bf16(k[part] * kScale) * 0.08838834765f);
-      const uint32_t value = float_to_bf16_bits(v[part]);
-      queries[token][d] = uint16_t(query);
-      keys[token][d] = uint16_t(key);
-      values[token][d] = uint16_t(value);
+      queries[token][d] = uint16_t(row.query[part]);
+      keys[token][d] = uint16_t(row.key[part]);
+      values[token][d] = uint16_t(row.value[part]);
       stepTape.inputs[size_t(token) * C + vChannel + d] = inputs[vChannel + d];
-      stepTape.kv[size_t(token) * kvWidth + keyWidth + head * kDim + d] = uint16_t(value);
+      stepTape.kv[size_t(token) * kvWidth + keyWidth + head * kDim + d] = uint16_t(row.value[part]);
       if (sharedWriter) {
         stepTape.inputs[size_t(token) * C + qChannel + d] = inputs[qChannel + d];
         stepTape.inputs[size_t(token) * C + kChannel + d] = inputs[kChannel + d];
-        stepTape.kv[size_t(token) * kvWidth + keyHead * kDim + d] = uint16_t(key);
+        stepTape.kv[size_t(token) * kvWidth + keyHead * kDim + d] = uint16_t(row.key[part]);
       }
     }
     if (lane == 0) {
-      // gdn_primitives.h:65-73: beta = bf16(sigmoid(b)); decay = exp(a_scale bf16(softplus(bf16(a + dt_bias))))
-      const uint32_t beta = float_to_bf16_bits(sigmoid_of(bf16_bits_to_float(inputs[bOffset + head])));
-      const float x = round_bf16(bf16_bits_to_float(inputs[aOffset + head]) + bf16_bits_to_float(dt_bias[head]));
-      const float softplus = round_bf16(fmaxf(x, 0.0f) + __builtin_amdgcn_logf(1.0f + exp2_fast(-kLog2e * fabsf(x))) * 0.69314718056f);
-      const float decay = exp2_fast(kLog2e * (a_scale[head] * softplus));
-      stepTape.beta[token * s.value_heads + head] = uint16_t(beta);
-      stepTape.decay[token * s.value_heads + head] = decay;
-      betas[token] = uint16_t(beta);
-      decays[token] = decay;
+      const Gates gates = gates_of(inputs, bOffset, aOffset, head, a_scale, dt_bias);
+      stepTape.beta[token * s.value_heads + head] = uint16_t(gates.beta);
+      stepTape.decay[token * s.value_heads + head] = gates.decay;
+      betas[token] = uint16_t(gates.beta);
+      decays[token] = gates.decay;
       paths[token] = path;
     }
   }
@@ -361,18 +417,13 @@ __global__ __launch_bounds__(64 * kWaves) void gdn_decode(const uint16_t *__rest
     float value[2];
 #pragma unroll
     for (uint32_t part = 0; part < 2; ++part) value[part] = bf16_bits_to_float(outputs[token][lane + 64u * part]);
-    const float inverse = 1.0f / sqrtf(head_sum(value[0] * value[0], value[1] * value[1]) / float(kDim) + 1e-6f);
+    uint32_t gated[2];
+    gated_norm(value, norm_weight, p.flags, rowsIn + size_t(token) * P + zOffset + head * kDim, lane, gated);
 #pragma unroll
     for (uint32_t part = 0; part < 2; ++part) {
       const uint32_t d = lane + 64u * part;
-      const float weight = (p.flags & GDN_FLOAT_NORM) ? static_cast<const float *>(norm_weight)[d]
-                                                       : bf16_bits_to_float(static_cast<const uint16_t *>(norm_weight)[d]);
-      const float normalized = round_bf16((value[part] * inverse) * weight);
-      const float z = bf16_bits_to_float(rowsIn[size_t(token) * P + zOffset + head * kDim + d]);
-      const float gated = (normalized * ((p.flags & GDN_SIGMOID_GATE) ? 1.0f : z)) / (1.0f + exp2_fast(-kLog2e * z));
-      const uint32_t bits = float_to_bf16_bits(gated);
-      hidden[(size_t(L.first_row + token) * s.value_heads + outHead) * kDim + d] = uint16_t(bits);
-      outputs[token][d] = uint16_t(bits);  // this wave's row: read above, and below for the table
+      hidden[(size_t(L.first_row + token) * s.value_heads + outHead) * kDim + d] = uint16_t(gated[part]);
+      outputs[token][d] = uint16_t(gated[part]);  // this wave's row: read above, and below for the table
     }
     if (p.table_tiles) {
       // The row's 128 values of this head as 32 runs of four inputs, a lane a run: the pieces, and the sums of 16
@@ -456,5 +507,230 @@ __global__ __launch_bounds__(64 * kWaves) void gdn_fold(uint8_t *__restrict__ st
   }
 }
 SP_REGISTER_KERNEL("gdn_fold", &gdn_fold);
+
+// ---- prefill: a prompt chunk, whose rows all enter the state (the reference's kernels/prefill/gdn.metal) ----
+//
+// Three passes over a run of `tokens` rows of one lane and layer. The rows' k, v and gates are those
+// a verify step would leave on its tape for the same rows (the same device functions compute both) and
+// a state row's recurrence is `advance`, the fold's: a prompt that enters the state through these
+// kernels leaves the cell, bit for bit, that the same rows leave when they enter as accepted verify
+// blocks. Only the outputs differ in form: here a row reads the state after its own token, o = S_t q_t
+// (gdn.metal:291-298), where a verify block's rows read the state before the block.
+
+// gdn_prefill_prepare: grid (value_heads, ceil(tokens / 4)), 256 threads, a wave per (row, value head),
+// lane l the dimensions l and 64 + l: convolution + SiLU, q/k norms, gates (prefill/gdn.metal:196-262).
+// The head's value rows, its gates and, from the first value head of a key head, the key head's query
+// and key rows leave to the run's buffers; the workgroups of the first rows also write the convolution
+// carry after the run's last row.
+__global__ __launch_bounds__(256) void gdn_prefill_prepare(const uint16_t *__restrict__ packed, const uint16_t *__restrict__ conv_weights,
+                                                           uint8_t *__restrict__ states, const float *__restrict__ a_scale,
+                                                           const uint16_t *__restrict__ dt_bias, uint16_t *__restrict__ queries,
+                                                           uint16_t *__restrict__ keys, uint16_t *__restrict__ values,
+                                                           float *__restrict__ decay, uint16_t *__restrict__ beta, GdnPrefillParams p) {
+  const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6, head = blockIdx.x, token = blockIdx.y * 4u + wave;
+  const GdnShapeParams s = p.shape;
+  const uint32_t perKey = s.value_heads / s.key_heads, keyHead = head / perKey, keyWidth = s.key_heads * kDim;
+  const uint32_t valueWidth = s.value_heads * kDim, C = s.conv_dim, P = s.packed_width;
+  const uint32_t bOffset = C + valueWidth, aOffset = bOffset + s.value_heads;
+  const bool sharedWriter = head % perKey == 0;
+  const uint16_t *convIn = reinterpret_cast<const uint16_t *>(states + p.current_cell + uint64_t(p.layer) * p.conv_layer_bytes);
+  uint16_t *convOut = reinterpret_cast<uint16_t *>(states + p.next_cell + uint64_t(p.layer) * p.conv_layer_bytes);
+  const uint32_t qChannel = keyHead * kDim, kChannel = keyWidth + keyHead * kDim, vChannel = 2 * keyWidth + head * kDim;
+  // input position i of the run's history: the carried rows, then the run's own (gdn_primitives.h:20-35)
+  auto input = [&](uint32_t position) __attribute__((always_inline)) -> const uint16_t * {
+    return position < kTaps - 1 ? convIn + size_t(position) * C : packed + size_t(p.first + position - (kTaps - 1)) * P;
+  };
+  if (blockIdx.y == 0 && wave < kTaps - 1) {
+    const uint16_t *source = input(p.tokens + wave);
+#pragma unroll
+    for (uint32_t part = 0; part < 2; ++part) {
+      const uint32_t d = lane + 64u * part;
+      convOut[size_t(wave) * C + vChannel + d] = source[vChannel + d];
+      if (sharedWriter) {
+        convOut[size_t(wave) * C + qChannel + d] = source[qChannel + d];
+        convOut[size_t(wave) * C + kChannel + d] = source[kChannel + d];
+      }
+    }
+  }
+  if (token >= p.tokens) return;
+  const uint16_t *taps[kTaps];
+#pragma unroll
+  for (uint32_t tap = 0; tap < kTaps; ++tap) taps[tap] = input(token + tap);
+  const HeadRow row = head_row(taps, conv_weights, qChannel, kChannel, vChannel, lane);
+  const size_t at = size_t(p.first) + token;  // the row's place in the chunk's buffers
+#pragma unroll
+  for (uint32_t part = 0; part < 2; ++part) {
+    const uint32_t d = lane + 64u * part;
+    values[at * valueWidth + head * kDim + d] = uint16_t(row.value[part]);
+    if (sharedWriter) {
+      queries[at * keyWidth + keyHead * kDim + d] = uint16_t(row.query[part]);
+      keys[at * keyWidth + keyHead * kDim + d] = uint16_t(row.key[part]);
+    }
+  }
+  if (lane == 0) {
+    const Gates gates = gates_of(packed + at * P, bOffset, aOffset, head, a_scale, dt_bias);
+    beta[at * s.value_heads + head] = uint16_t(gates.beta);
+    decay[at * s.value_heads + head] = gates.decay;
+  }
+}
+SP_REGISTER_KERNEL("gdn_prefill_prepare", &gdn_prefill_prepare);
+
+// gdn_prefill_scan: grid (value_heads * 128 / GDN_SCAN_STATE_ROWS), 256 threads. A workgroup carries GDN_SCAN_STATE_ROWS
+// rows of a head's state through the run in registers, token by token (prefill/gdn.metal:11-23): a wave holds a
+// pair of rows, a row per half-wave, lane j of a half the key columns 4 j .. 4 j + 3, as the fold does.
+// Blocks of GDN_SCAN_BLOCK tokens of k, q, v and gates are staged in LDS while the block after them is
+// in flight to registers, so the dependent chain of a token reads LDS only; a block's outputs collect
+// in LDS and leave as whole 16-byte runs. Eight rows a workgroup put two workgroups on a compute unit and
+// two waves on a SIMD, each other's cover for the chain's latencies.
+__global__ __launch_bounds__(256) void gdn_prefill_scan(const uint16_t *__restrict__ queries, const uint16_t *__restrict__ keys,
+                                                        const uint16_t *__restrict__ values, const float *__restrict__ decay,
+                                                        const uint16_t *__restrict__ beta, uint8_t *__restrict__ states,
+                                                        uint16_t *__restrict__ recurrent_rows, GdnPrefillParams p) {
+  constexpr uint32_t B = GDN_SCAN_BLOCK, R = GDN_SCAN_STATE_ROWS, kGroups = kDim / R, kPairs = R / 8, kPieces = R / 8;
+  static_assert(B * kDim * 2 == 256 * 16, "a thread stages sixteen bytes of a block's keys and of its queries");
+  static_assert(R == 4 * 2 * kPairs && R % 8 == 0, "four waves of kPairs pairs of rows hold a workgroup's state rows, whole 16-byte pieces of a token's values");
+  __shared__ __align__(16) uint16_t sk[2][B][kDim], sq[2][B][kDim];
+  __shared__ __align__(16) uint16_t sv[2][B][R], so[B][R];
+  __shared__ float sd[2][B];
+  __shared__ uint16_t sb[2][B];
+  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+  const GdnShapeParams s = p.shape;
+  const uint32_t head = blockIdx.x / kGroups, rowBase = (blockIdx.x % kGroups) * R;
+  const uint32_t keyHead = head / (s.value_heads / s.key_heads), keyWidth = s.key_heads * kDim, valueWidth = s.value_heads * kDim;
+  const uint32_t half = lane >> 5, column = 4u * (lane & 31u), tokens = p.tokens;
+  const float *stateIn = reinterpret_cast<const float *>(states + p.current_cell + p.convolution_state_bytes + uint64_t(p.layer) * p.recurrent_layer_bytes);
+  float *stateOut = reinterpret_cast<float *>(states + p.next_cell + p.convolution_state_bytes + uint64_t(p.layer) * p.recurrent_layer_bytes);
+  uint32_t local[kPairs];
+  float state[kPairs][4];
+#pragma unroll
+  for (uint32_t r = 0; r < kPairs; ++r) {
+    local[r] = (r * 4u + wave) * 2u + half;
+    const float4 loaded = *reinterpret_cast<const float4 *>(stateIn + (size_t(head) * kDim + rowBase + local[r]) * kDim + column);
+    state[r][0] = loaded.x;
+    state[r][1] = loaded.y;
+    state[r][2] = loaded.z;
+    state[r][3] = loaded.w;
+  }
+  // Rows at or past `tokens` keep what the registers held and are staged as they are: the loop below stops at the
+  // run's last token, so those slots are never read.
+  uint4 keyFetch = make_uint4(0, 0, 0, 0), queryFetch = keyFetch, valueFetch = keyFetch;
+  float decayFetch = 0.f;
+  uint16_t betaFetch = 0;
+  auto fetch = [&](uint32_t start) __attribute__((always_inline)) {
+    const uint32_t token = start + tid / 16u;
+    if (token < tokens) {
+      const size_t at = (size_t(p.first) + token) * keyWidth + keyHead * kDim + (tid % 16u) * 8u;
+      keyFetch = *reinterpret_cast<const uint4 *>(keys + at);
+      queryFetch = *reinterpret_cast<const uint4 *>(queries + at);
+    }
+    if (tid < kPieces * B && start + tid / kPieces < tokens)
+      valueFetch = *reinterpret_cast<const uint4 *>(values + (size_t(p.first) + start + tid / kPieces) * valueWidth + head * kDim + rowBase + (tid % kPieces) * 8u);
+    if (tid < B && start + tid < tokens) {
+      decayFetch = decay[(size_t(p.first) + start + tid) * s.value_heads + head];
+      betaFetch = beta[(size_t(p.first) + start + tid) * s.value_heads + head];
+    }
+  };
+  auto stage = [&](uint32_t buffer) __attribute__((always_inline)) {
+    *reinterpret_cast<uint4 *>(&sk[buffer][tid / 16u][(tid % 16u) * 8u]) = keyFetch;
+    *reinterpret_cast<uint4 *>(&sq[buffer][tid / 16u][(tid % 16u) * 8u]) = queryFetch;
+    if (tid < kPieces * B) *reinterpret_cast<uint4 *>(&sv[buffer][tid / kPieces][(tid % kPieces) * 8u]) = valueFetch;
+    if (tid < B) {
+      sd[buffer][tid] = decayFetch;
+      sb[buffer][tid] = betaFetch;
+    }
+  };
+  fetch(0);
+  stage(0);
+  __syncthreads();
+  for (uint32_t start = 0, buffer = 0; start < tokens; start += B, buffer ^= 1u) {
+    const bool more = start + B < tokens;
+    if (more) fetch(start + B);
+    const uint32_t count = min(B, tokens - start);
+    // A token's operands leave LDS one token ahead of their use, and a token's output is off the state's dependent
+    // chain: its lanes' products wait one token, and their sum over the half-wave runs beside the next token's update.
+    struct Operands {
+      uint2 key, query;
+      float decay;
+      uint32_t beta, value[kPairs];
+    };
+    auto operands = [&](uint32_t t) __attribute__((always_inline)) {
+      Operands o;
+      o.key = *reinterpret_cast<const uint2 *>(&sk[buffer][t][column]);
+      o.query = *reinterpret_cast<const uint2 *>(&sq[buffer][t][column]);
+      o.decay = sd[buffer][t];
+      o.beta = sb[buffer][t];
+#pragma unroll
+      for (uint32_t r = 0; r < kPairs; ++r) o.value[r] = sv[buffer][t][local[r]];
+      return o;
+    };
+    float partial[kPairs] = {};
+    Operands ahead = operands(0);
+    for (uint32_t t = 0; t <= count; ++t) {
+      float sum[kPairs];
+#pragma unroll
+      for (uint32_t r = 0; r < kPairs; ++r) sum[r] = partial[r];
+      if (t < count) {
+        const Operands now = ahead;
+        ahead = operands(min(t + 1u, B - 1u));  // past the block's last token: a staged slot nobody uses
+        const float k[4] = {bf16_bits_to_float(now.key.x & 0xFFFFu), bf16_bits_to_float(now.key.x >> 16),
+                            bf16_bits_to_float(now.key.y & 0xFFFFu), bf16_bits_to_float(now.key.y >> 16)};
+        const float q[4] = {bf16_bits_to_float(now.query.x & 0xFFFFu), bf16_bits_to_float(now.query.x >> 16),
+                            bf16_bits_to_float(now.query.y & 0xFFFFu), bf16_bits_to_float(now.query.y >> 16)};
+        float value[kPairs];
+#pragma unroll
+        for (uint32_t r = 0; r < kPairs; ++r) value[r] = bf16_bits_to_float(now.value[r]);
+        advance_rows<kPairs>(state, k, value, now.decay, bf16_bits_to_float(now.beta));
+#pragma unroll
+        for (uint32_t r = 0; r < kPairs; ++r) {
+          partial[r] = 0.f;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) partial[r] += state[r][i] * q[i];
+        }
+      }
+      if (t > 0) {
+#pragma unroll
+        for (uint32_t r = 0; r < kPairs; ++r) sum[r] = half_sum(sum[r]);
+        if ((lane & 31u) == 0) {
+#pragma unroll
+          for (uint32_t r = 0; r < kPairs; ++r) so[t - 1][local[r]] = uint16_t(float_to_bf16_bits(sum[r]));
+        }
+      }
+    }
+    __syncthreads();  // the block's outputs are whole, and no wave reads its staged rows any more
+    if (tid < kPieces * count)
+      *reinterpret_cast<uint4 *>(recurrent_rows + (size_t(p.first) + start + tid / kPieces) * valueWidth + head * kDim + rowBase + (tid % kPieces) * 8u) =
+          *reinterpret_cast<const uint4 *>(&so[tid / kPieces][(tid % kPieces) * 8u]);
+    if (more) stage(buffer ^ 1u);
+    __syncthreads();
+  }
+#pragma unroll
+  for (uint32_t r = 0; r < kPairs; ++r)
+    *reinterpret_cast<float4 *>(stateOut + (size_t(head) * kDim + rowBase + local[r]) * kDim + column) =
+        make_float4(state[r][0], state[r][1], state[r][2], state[r][3]);
+}
+SP_REGISTER_KERNEL("gdn_prefill_scan", &gdn_prefill_scan);
+
+// gdn_prefill_gate: grid (value_heads, ceil(tokens / 4)), 256 threads, a wave per (row, value head): the gated
+// output norm of the scan's rows (prefill/gdn.metal:312-341, gdn.metal:489-526).
+__global__ __launch_bounds__(256) void gdn_prefill_gate(const uint16_t *__restrict__ recurrent_rows, const uint16_t *__restrict__ packed,
+                                                        const void *__restrict__ norm_weight, uint16_t *__restrict__ hidden,
+                                                        GdnPrefillParams p) {
+  const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6, head = blockIdx.x;
+  if (blockIdx.y * 4u + wave >= p.tokens) return;
+  const size_t token = size_t(p.first) + blockIdx.y * 4u + wave;
+  const GdnShapeParams s = p.shape;
+  const uint32_t perKey = s.value_heads / s.key_heads, valueWidth = s.value_heads * kDim;
+  const uint32_t outHead = (p.flags & GDN_TILED_HEADS) ? (head % perKey) * s.key_heads + head / perKey : head;
+  float value[2];
+#pragma unroll
+  for (uint32_t part = 0; part < 2; ++part)
+    value[part] = bf16_bits_to_float(recurrent_rows[token * valueWidth + head * kDim + lane + 64u * part]);
+  uint32_t gated[2];
+  gated_norm(value, norm_weight, p.flags, packed + token * s.packed_width + s.conv_dim + head * kDim, lane, gated);
+#pragma unroll
+  for (uint32_t part = 0; part < 2; ++part)
+    hidden[(token * s.value_heads + outHead) * kDim + lane + 64u * part] = uint16_t(gated[part]);
+}
+SP_REGISTER_KERNEL("gdn_prefill_gate", &gdn_prefill_gate);
 
 } // namespace splash::kernels

@@ -1,6 +1,6 @@
 // ops::GDN of the reference (runtime/ops/GDN.hpp:16-203, GDN.cpp:225-330) for the verify step: the
-// decode step of up to eight lanes with its tape, and the fold of a step's accepted rows alone,
-// over kernels/gdn.hip. Prefill and the cached states' codes are not part of the verify step.
+// decode step of up to eight lanes with its tape, the fold of a step's accepted rows alone, and the prompt
+// chunk that builds the state a lane's first step starts from (GDN.hpp:75-104, :166-181), over kernels/gdn.hip.
 #pragma once
 #include "abi/Gdn.h"
 #include "hip/Backend.hpp"
@@ -71,8 +71,40 @@ struct GdnFoldBuffers final {
   uint64_t foldCell = 0;     // the cell the fold writes
 };
 
+// A prompt chunk of one lane and layer (GDN.hpp:75-93): the chunk's packed rows, the lane's cells, and the
+// buffers of rows the three passes hand to each other. A chunk's rows all enter the state; nothing is taped.
+struct GdnPrefillBuffers final {
+  hip::Buffer packed;              // bf16 [tokens][packedWidth]
+  hip::Buffer convolutionWeights;  // bf16 [convolutionDimension][4]
+  hip::Buffer states;              // the cells
+  hip::Buffer decayWeights;        // fp32 [valueHeads]
+  hip::Buffer timeBias;            // bf16 [valueHeads]
+  hip::Buffer mixerNorm;           // bf16 or fp32 [128]
+  bool floatNorm = false;
+  hip::Buffer queries, keys;       // bf16 [tokens][keyHeads * 128]: normalized, scaled
+  hip::Buffer values;              // bf16 [tokens][valueHeads * 128]
+  hip::Buffer decay;               // fp32 [tokens][valueHeads]
+  hip::Buffer beta;                // bf16 [tokens][valueHeads]
+  hip::Buffer recurrentRows;       // bf16 [tokens][valueHeads * 128]: the scan's outputs before the gated norm
+  hip::Buffer hidden;              // bf16 [tokens][valueHeads * 128]
+  uint64_t currentCell = 0;        // the cell the chunk starts from
+  uint64_t nextCell = 0;           // the cell after its last row
+};
+// A state a chunk leaves on the way (GDN.hpp:95-104): the cell after its first `tokens` rows, convolution carry and
+// recurrent state as a chunk ending there would leave them. What a cached state codes (ops::StateCodec) is such a cell.
+struct GdnPrefillCapture final {
+  uint32_t tokens = 0;
+  uint64_t cell = 0;
+};
+
 class GDN final {
 public:
+  // A chunk of `tokens` rows of one lane, in runs that end at the captures (ascending, inside the rows): each run is
+  // a prepare and a scan dispatch that continue from the cell the run before wrote, and one gate dispatch covers all
+  // rows (GDN.cpp:176-222). The scan is sequential, so the runs compute bit for bit what one run computes.
+  static void addPrefill(hip::CommandGraph &graph, const GdnPrefillBuffers &buffers, const GdnShape &shape, uint32_t layer,
+                         uint32_t tokens, const GdnStateStrides &state, GdnHeadOrder order,
+                         const std::vector<GdnPrefillCapture> &captures = {});
   // The step of 1 to 8 lanes of one layer.
   static void addDecode(hip::CommandGraph &graph, const GdnDecodeBuffers &buffers, const GdnShape &shape, uint32_t layer,
                         const GdnStateStrides &state, GdnHeadOrder order, const std::vector<GdnLaneStep> &lanes);

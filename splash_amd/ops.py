@@ -476,7 +476,8 @@ class RoPE:
 
 
 class GDN:
-    """ops::GDN: the verify step of Gated DeltaNet layers (addDecode) and the fold of a step's accepted rows (addFold)."""
+    """ops::GDN: the verify step of Gated DeltaNet layers (addDecode), the fold of a step's accepted rows (addFold) and the
+    prompt chunk that builds a lane's state (addPrefill)."""
 
     def __init__(self, key_heads, value_heads, packed_width=None, sigmoid_gate=False, layers=1):
         conv = (2 * key_heads + value_heads) * 128
@@ -497,6 +498,23 @@ class GDN:
                                                        l["step_tape"], l["current_cell"], l["next_cell"]) for l in lanes])
         check(lib.spo_gdn_add_decode(graph.handle, ctypes.byref(b), ctypes.byref(self.shape), layer, ctypes.byref(self.strides),
                                      int(tiled_heads), arr, len(lanes)))
+        graph._keep.extend(list(buffers.values()))
+
+    def prefill_workspace(self, backend, tokens):
+        """The buffers of rows a chunk of `tokens` rows hands from pass to pass (and its hidden rows)."""
+        kw, vw, vh = self.shape.key_heads * 128, self.shape.value_heads * 128, self.shape.value_heads
+        sizes = dict(queries=tokens * kw * 2, keys=tokens * kw * 2, values=tokens * vw * 2, decay=tokens * vh * 4, beta=tokens * vh * 2,
+                     recurrent_rows=tokens * vw * 2, hidden=tokens * vw * 2)
+        return {n: backend.allocate_buffer(max(b, 16), STORAGE_PRIVATE, "gdn prefill " + n) for n, b in sizes.items()}
+
+    def add_prefill(self, graph, buffers, layer, tokens, current_cell, next_cell, captures=(), tiled_heads=False, float_norm=False):
+        """GDN::addPrefill: a prompt chunk of one lane and layer. buffers: dict of Buffer by the names of
+        spo_gdn_prefill_buffers; captures: [(tokens, cell)], ascending inside the rows."""
+        b = nat.GdnPrefillBuffers(**{k: v.handle for k, v in buffers.items()}, float_norm=int(float_norm), current_cell=current_cell,
+                                  next_cell=next_cell)
+        arr = (nat.GdnPrefillCapture * max(1, len(captures)))(*[nat.GdnPrefillCapture(t, 0, c) for t, c in captures])
+        check(lib.spo_gdn_add_prefill(graph.handle, ctypes.byref(b), ctypes.byref(self.shape), layer, tokens, ctypes.byref(self.strides),
+                                      int(tiled_heads), arr, len(captures)))
         graph._keep.extend(list(buffers.values()))
 
     def add_fold(self, graph, states, tape, retained_rows, step_tape, state_cell, fold_cell, rows):

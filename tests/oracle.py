@@ -435,6 +435,31 @@ lib.orc_gdn_reference.restype = c_int
 lib.orc_gdn_reference.argtypes = [ctypes.POINTER(GdnShape), u16p, c_u32, u16p, f32p, u16p, u16p, f32p, f64p, f64p, f64p, f64p, f64p]
 
 
+lib.orc_gdn_prefill.restype = c_int
+lib.orc_gdn_prefill.argtypes = [ctypes.POINTER(GdnShape), u16p, c_u32, u16p, f32p, u16p, ctypes.c_void_p, u16p, f32p, u16p, u16p, u16p, f32p,
+                                u16p, u16p, f32p, u16p, u16p]
+
+
+def gdn_prefill(shape, packed, conv_weights, a_scale, dt_bias, norm_weight, conv_in, state_in):
+    """A prompt chunk of one lane and layer. Returns dict(queries, keys, values, decay, beta, conv_out, state_out,
+    recurrent, hidden)."""
+    tokens, vh, kh = packed.shape[0], shape.value_heads, shape.key_heads
+    out = dict(queries=np.zeros((tokens, kh * 128), np.uint16), keys=np.zeros((tokens, kh * 128), np.uint16),
+               values=np.zeros((tokens, vh * 128), np.uint16), decay=np.zeros((tokens, vh), np.float32),
+               beta=np.zeros((tokens, vh), np.uint16), conv_out=np.zeros((3, shape.conv_dim), np.uint16),
+               state_out=np.zeros((vh, 128, 128), np.float32), recurrent=np.zeros((tokens, vh * 128), np.uint16),
+               hidden=np.zeros((tokens, vh * 128), np.uint16))
+    packed, conv_weights, a_scale, dt_bias, norm_weight, conv_in, state_in = (np.ascontiguousarray(x) for x in (
+        packed, conv_weights, a_scale, dt_bias, norm_weight, conv_in, state_in))
+    rc = lib.orc_gdn_prefill(ctypes.byref(shape), _p(packed, u16p), tokens, _p(conv_weights, u16p), _p(a_scale, f32p), _p(dt_bias, u16p),
+                             norm_weight.ctypes.data_as(ctypes.c_void_p), _p(conv_in, u16p), _p(state_in, f32p),
+                             _p(out["queries"], u16p), _p(out["keys"], u16p), _p(out["values"], u16p), _p(out["decay"], f32p),
+                             _p(out["beta"], u16p), _p(out["conv_out"], u16p), _p(out["state_out"], f32p), _p(out["recurrent"], u16p),
+                             _p(out["hidden"], u16p))
+    assert rc == 0
+    return out
+
+
 def gdn_fold(shape, conv_in, state_in, step_tape, path, rows):
     conv_out = np.zeros((3, shape.conv_dim), np.uint16)
     state_out = np.zeros_like(state_in)

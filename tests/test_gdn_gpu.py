@@ -6,7 +6,7 @@ import pytest
 import splash_amd
 from splash_amd import ops
 from tests import oracle as orc
-from tests.gdn_case import make_layer, make_rows, make_state, make_tree, path_rows, tree_rows_array, ulps
+from tests.gdn_case import check_prefill_against_fp64, make_layer, make_rows, make_state, make_tree, path_rows, tree_rows_array, ulps
 
 pytestmark = pytest.mark.gpu
 
@@ -278,3 +278,114 @@ def test_gdn_rejects_bad_arguments(backend):
     with pytest.raises(ValueError):
         ops.GDN(3, 4)
     assert len(graph) == 0
+
+
+class Chunk:
+    """A prompt chunk through GDN::addPrefill on a Layer's cells; returns the passes' rows as arrays."""
+
+    def __init__(self, layer, tokens):
+        self.layer, self.tokens = layer, tokens
+        self.work = layer.gdn.prefill_workspace(layer.backend, tokens)
+
+    def run(self, packed, lane, current, nxt, captures=(), tiled_heads=False):
+        layer = self.layer
+        graph = splash_amd.CommandGraph()
+        buffers = dict(packed=layer.backend.from_array(packed), states=layer.states, **layer.weights, **self.work)
+        layer.gdn.add_prefill(graph, buffers, 0, packed.shape[0], layer.cell(lane, current), layer.cell(lane, nxt),
+                              captures=[(t, layer.cell(lane, c)) for t, c in captures], tiled_heads=tiled_heads,
+                              float_norm=layer.float_norm)
+        layer.backend.run(graph)
+        shape, tokens = layer.shape, packed.shape[0]
+        kw, vw, vh = shape.key_heads * 128, shape.value_heads * 128, shape.value_heads
+        take = lambda name, dtype, width: self.work[name].download(dtype)[:tokens * width].reshape(tokens, width).copy()
+        conv_out, state_out = layer.read_cell(lane, nxt)
+        return dict(queries=take("queries", np.uint16, kw), keys=take("keys", np.uint16, kw), values=take("values", np.uint16, vw),
+                    decay=take("decay", np.float32, vh), beta=take("beta", np.uint16, vh), recurrent=take("recurrent_rows", np.uint16, vw),
+                    hidden=take("hidden", np.uint16, vw), conv_out=conv_out, state_out=state_out)
+
+
+@pytest.mark.parametrize("heads,tokens,float_norm", [((2, 4), 1, False), ((2, 4), 53, False), ((16, 32), 100, True), ((2, 2), 2048, False)])
+def test_prefill_passes_the_reference_checks_and_matches_the_oracle(backend, heads, tokens, float_norm):
+    """gdn_metal_test.mm:215-418: each pass of the chunk against fp64 arithmetic over the pass's own inputs, under the
+    reference's bounds; and the chunk against the oracle's, whose exp2 and log2 differ from the GPU's in their last bits."""
+    print(f"case gdn prefill heads={heads} tokens={tokens}", flush=True)
+    rng = np.random.default_rng(41)
+    layer = Layer(backend, rng, *heads, lanes=1, float_norm=float_norm)
+    shape = layer.shape
+    conv_in, state_in = make_state(rng, shape)
+    packed = make_rows(rng, shape, tokens)
+    layer.write_cell(0, 0, conv_in, state_in)
+    got = Chunk(layer, tokens).run(packed, 0, 0, 1)
+    check_prefill_against_fp64(shape, layer.conv_w, layer.a_scale, layer.dt_bias, layer.norm, packed, conv_in, state_in, got)
+    if tokens > 512:
+        return
+    want = orc.gdn_prefill(shape, packed, layer.conv_w, layer.a_scale, layer.dt_bias, layer.norm, conv_in, state_in)
+    assert np.array_equal(got["conv_out"], want["conv_out"])
+    for name in ("queries", "keys", "values"):
+        assert ulps(got[name], want[name]).max() <= 1 and (ulps(got[name], want[name]) > 0).mean() < 0.01, name
+    assert ulps(got["beta"], want["beta"]).max() <= 1
+    assert np.all(np.abs(got["decay"] - want["decay"]) <= 1e-5 * want["decay"] + 1e-12)
+    assert np.abs(got["state_out"] - want["state_out"]).max() <= 1e-4 * np.abs(want["state_out"]).max()
+
+
+def test_prefill_leaves_the_cell_of_the_same_rows_as_accepted_blocks(backend):
+    """Bitwise on the GPU: a chunk's k, v and gates are the tape's, and the cell it leaves is the one the same rows leave
+    as verify blocks accepted whole (a step per block, then the fold of the last); a chunk in runs with captures equals
+    the chunk whole, and each capture the chunk that ends there (gdn_metal_test.mm:426-480, :560-700)."""
+    print("case gdn prefill invariants", flush=True)
+    rng = np.random.default_rng(42)
+    layer = Layer(backend, rng, 4, 8, lanes=1, cells=6)
+    shape = layer.shape
+    conv_in, state_in = make_state(rng, shape)
+    tokens = 45
+    packed = make_rows(rng, shape, tokens)
+    layer.write_cell(0, 0, conv_in, state_in)
+    chunk = Chunk(layer, tokens)
+    whole = chunk.run(packed, 0, 0, 1)
+    # the same rows as blocks of 16, 16 and 13, each accepted whole
+    kw = shape.key_heads * 128
+    cells, path, parity, retained = (0, 2), 0, 0, None
+    for first, rows in ((0, 16), (16, 16), (32, 13)):
+        layer.step([(0, packed[first:first + rows], path, parity, cells[0], cells[1])])
+        _, kv, decay, beta = orc.gdn_split_tape(shape, layer.read_tape(0, parity))
+        assert np.array_equal(kv[:rows, :kw], whole["keys"][first:first + rows])
+        assert np.array_equal(kv[:rows, kw:], whole["values"][first:first + rows])
+        assert decay[:rows].tobytes() == whole["decay"][first:first + rows].tobytes()
+        assert np.array_equal(beta[:rows], whole["beta"][first:first + rows])
+        path, parity, cells = (1 << rows) - 1, parity ^ 1, (cells[1], cells[0] if cells[0] != 0 else 3)
+    graph = splash_amd.CommandGraph()
+    layer.gdn.add_fold(graph, layer.states, layer.tape, backend.from_array(np.array([path], np.uint32)), layer.slot(0, parity ^ 1),
+                       layer.cell(0, cells[0]), layer.cell(0, 4), 13)
+    backend.run(graph)
+    conv, state = layer.read_cell(0, 4)
+    assert np.array_equal(conv, whole["conv_out"]) and state.tobytes() == whole["state_out"].tobytes()
+    # runs: captures after 7 and 32 rows
+    layer.write_cell(0, 0, conv_in, state_in)
+    runs = chunk.run(packed, 0, 0, 1, captures=[(7, 2), (32, 3)])
+    for name in whole:
+        assert runs[name].tobytes() == whole[name].tobytes(), name
+    for count, cell in ((7, 2), (32, 3)):
+        layer.write_cell(0, 0, conv_in, state_in)
+        part = Chunk(layer, count).run(packed[:count], 0, 0, 5)
+        conv, state = layer.read_cell(0, cell)
+        assert np.array_equal(conv, part["conv_out"]) and state.tobytes() == part["state_out"].tobytes()
+    with pytest.raises(ValueError):
+        chunk.run(packed, 0, 0, 0)                       # a run reads and writes different cells
+    with pytest.raises(ValueError):
+        chunk.run(packed, 0, 0, 1, captures=[(45, 2)])   # a capture lies inside the rows
+
+
+def test_prefill_head_order(backend):
+    """Tiled heads leave at (h % heads per key) * key heads + h / heads per key (gdn_metal_test.mm:703-745)."""
+    rng = np.random.default_rng(43)
+    layer = Layer(backend, rng, 2, 4, lanes=1)
+    conv_in, state_in = make_state(rng, layer.shape)
+    packed = make_rows(rng, layer.shape, 9)
+    layer.write_cell(0, 0, conv_in, state_in)
+    chunk = Chunk(layer, 9)
+    grouped = chunk.run(packed, 0, 0, 1)
+    tiled = chunk.run(packed, 0, 0, 1, tiled_heads=True)
+    assert tiled["state_out"].tobytes() == grouped["state_out"].tobytes()
+    g, t = grouped["hidden"].reshape(9, 4, 128), tiled["hidden"].reshape(9, 4, 128)
+    for head in range(4):
+        assert np.array_equal(t[:, (head % 2) * 2 + head // 2], g[:, head])

@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 
 from tests import oracle as orc
-from tests.gdn_case import make_layer, make_rows, make_state, make_tree, path_rows, ulps
+from tests.gdn_case import check_prefill_against_fp64, make_layer, make_rows, make_state, make_tree, path_rows, ulps
 
 
 def test_step_matches_the_fp64_recurrence():
@@ -174,3 +174,52 @@ def test_a_tree_path_folds_like_its_chain():
     assert np.array_equal(conv1, conv2) and state1.tobytes() == state2.tobytes() and np.array_equal(hidden1, hidden2)
     rc, convf, statef = orc.gdn_fold(shape, conv0, state0, tape0, path, len(along))
     assert rc == 0 and np.array_equal(convf, conv1) and statef.tobytes() == state1.tobytes()
+
+
+def _prefill_case(seed, heads, tokens, float_norm=False):
+    rng = np.random.default_rng(seed)
+    shape, conv_w, a_scale, dt_bias, norm = make_layer(rng, *heads, float_norm=float_norm)
+    packed = make_rows(rng, shape, tokens)
+    conv_in, state_in = make_state(rng, shape)
+    return shape, conv_w, a_scale, dt_bias, norm, packed, conv_in, state_in
+
+
+@pytest.mark.parametrize("heads,tokens,float_norm", [((2, 4), 40, False), ((1, 2), 1, True), ((2, 2), 19, False)])
+def test_prefill_matches_the_fp64_checks_of_the_reference(heads, tokens, float_norm):
+    case = _prefill_case(31, heads, tokens, float_norm)
+    shape, conv_w, a_scale, dt_bias, norm, packed, conv_in, state_in = case
+    got = orc.gdn_prefill(shape, packed, conv_w, a_scale, dt_bias, norm, conv_in, state_in)
+    check_prefill_against_fp64(*case, got)
+
+
+def test_prefill_leaves_the_state_of_the_same_rows_as_accepted_blocks():
+    """A chunk's k, v and gates are the tape's, and its cell is, bit for bit, the one the rows leave when they enter as
+    verify blocks that are accepted whole (a decode step per block, the next step's fold after it)."""
+    shape, conv_w, a_scale, dt_bias, norm, packed, conv_in, state_in = _prefill_case(32, (2, 4), 40)
+    got = orc.gdn_prefill(shape, packed, conv_w, a_scale, dt_bias, norm, conv_in, state_in)
+    conv, state, tape, path = conv_in, state_in, None, 0
+    kw = shape.key_heads * 128
+    for first, rows in ((0, 16), (16, 16), (32, 8)):
+        conv, state, tape, _ = orc.gdn_decode(shape, packed[first:first + rows], conv_w, a_scale, dt_bias, norm, conv, state,
+                                              pending_tape=tape, pending_path=path)
+        path = (1 << rows) - 1
+        _, kv, decay, beta = orc.gdn_split_tape(shape, tape)
+        assert np.array_equal(kv[:rows, :kw], got["keys"][first:first + rows])
+        assert np.array_equal(kv[:rows, kw:], got["values"][first:first + rows])
+        assert decay[:rows].tobytes() == got["decay"][first:first + rows].tobytes()
+        assert np.array_equal(beta[:rows], got["beta"][first:first + rows])
+    rc, conv, state = orc.gdn_fold(shape, conv, state, tape, path, 8)
+    assert rc == 0
+    assert np.array_equal(conv, got["conv_out"]) and state.tobytes() == got["state_out"].tobytes()
+
+
+def test_prefill_in_two_runs_is_the_chunk():
+    """gdn_metal_test.mm:426-480: a chunk continued from the cell its first rows left equals the chunk run whole."""
+    shape, conv_w, a_scale, dt_bias, norm, packed, conv_in, state_in = _prefill_case(33, (2, 4), 37)
+    whole = orc.gdn_prefill(shape, packed, conv_w, a_scale, dt_bias, norm, conv_in, state_in)
+    first = orc.gdn_prefill(shape, packed[:21], conv_w, a_scale, dt_bias, norm, conv_in, state_in)
+    second = orc.gdn_prefill(shape, packed[21:], conv_w, a_scale, dt_bias, norm, first["conv_out"], first["state_out"])
+    for name in ("queries", "keys", "values", "beta", "recurrent", "hidden"):
+        assert np.array_equal(np.concatenate([first[name], second[name]]), whole[name]), name
+    assert np.concatenate([first["decay"], second["decay"]]).tobytes() == whole["decay"].tobytes()
+    assert np.array_equal(second["conv_out"], whole["conv_out"]) and second["state_out"].tobytes() == whole["state_out"].tobytes()
