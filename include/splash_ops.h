@@ -201,6 +201,28 @@ sp_status spo_attention_add_attention(spo_graph *graph, const spo_attention_plan
                                       sp_buffer *query_sums, sp_buffer *partials, sp_buffer *partial_sums,
                                       sp_buffer *tree_rows, sp_buffer *page_table, sp_buffer *pool, uint64_t page_bytes,
                                       sp_buffer *output, sp_buffer *output_table, sp_buffer *packed_qkv);
+/* Prompt chunks: the plan over kv::ChunkedPrefillParams (PagedAttention.hpp:28-39, :270-275; PagedAttention.cpp:351-389).
+ * A chunk is `tokens` rows (1 to 2048, SPLASH_PREFILL_TOKEN_BUDGET) of one sequence at positions from `committed`,
+ * attending causally; it runs as tiles of 16 rows, eight tiles a dispatch, each tile's history split by its own length
+ * alone, so a row's result is bit for bit the one its tile gives as a verify block. The workspace holds the staged
+ * queries of every tile and the partials of the largest dispatch. add_chunk_projection stores every row's K and V
+ * before add_chunk_attention lets any row attend; buffers as the single-dispatch calls', over all the chunks' rows
+ * (tree_rows: a chain a tile; output_table: the one table of all the rows). */
+typedef struct spo_attention_chunk_plan spo_attention_chunk_plan;
+typedef struct spo_attention_chunk { uint32_t first_row, tokens, committed, table_first; } spo_attention_chunk;
+sp_status spo_attention_chunk_plan_create(const spo_attention_geometry *geometry, const spo_attention_chunk *chunks, uint32_t count,
+                                          spo_attention_chunk_plan **out);
+void spo_attention_chunk_plan_destroy(spo_attention_chunk_plan *plan);
+uint32_t spo_attention_chunk_plan_dispatches(const spo_attention_chunk_plan *plan);
+sp_status spo_attention_chunk_workspace(const spo_attention_chunk_plan *plan, uint64_t sizes[4]);
+sp_status spo_attention_add_chunk_projection(spo_graph *graph, const spo_attention_chunk_plan *plan, sp_buffer *qkv,
+                                             sp_buffer *query_norm, sp_buffer *key_norm, sp_buffer *rope_cos, sp_buffer *rope_sin,
+                                             sp_buffer *queries, sp_buffer *query_sums, sp_buffer *page_table, sp_buffer *pool,
+                                             uint64_t page_bytes);
+sp_status spo_attention_add_chunk_attention(spo_graph *graph, const spo_attention_chunk_plan *plan, sp_buffer *queries,
+                                            sp_buffer *query_sums, sp_buffer *partials, sp_buffer *partial_sums,
+                                            sp_buffer *tree_rows, sp_buffer *page_table, sp_buffer *pool, uint64_t page_bytes,
+                                            sp_buffer *output, sp_buffer *output_table, sp_buffer *packed_qkv);
 /* PagedAttention::addPathCommit (PagedAttention.cpp:647-667). */
 sp_status spo_attention_add_path_commit(spo_graph *graph, const spo_attention_plan *plan, sp_buffer *retained,
                                         sp_buffer *page_table, sp_buffer *pool, uint64_t page_bytes);
@@ -455,6 +477,12 @@ typedef struct spo_verify_lane {
 } spo_verify_lane;
 sp_status spo_dense_verify_create(sp_backend *backend, const spo_dense_dimensions *dimensions, uint32_t max_lanes,
                                   uint32_t physical_pages, uint32_t page_table_entries, spo_dense_verify **out);
+/* The same with room for prompt chunks of up to prefill_rows rows (spo_dense_verify_encode_prefill; 0: a step's most,
+ * 16 x max_lanes; at most 2048, SPLASH_PREFILL_TOKEN_BUDGET): the rows' buffers (input tokens, tree rows, depths, hidden
+ * rows, q|k|v and attention rows) are sized for it. */
+sp_status spo_dense_verify_create_chunked(sp_backend *backend, const spo_dense_dimensions *dimensions, uint32_t max_lanes,
+                                          uint32_t physical_pages, uint32_t page_table_entries, uint32_t prefill_rows,
+                                          spo_dense_verify **out);
 void spo_dense_verify_destroy(spo_dense_verify *verify);
 sp_status spo_dense_verify_set_layer(spo_dense_verify *verify, uint32_t layer, const spo_projection *qkv,
                                      const spo_projection *output, const spo_projection *gate, const spo_projection *up,
@@ -517,7 +545,7 @@ sp_status spo_dense_verify_set_test_children(spo_dense_verify *verify, int on);
  * chains nothing), nonzero when one gave up and what the step left is void. Reading it clears it. No counterpart in the
  * reference, whose projections are a dispatch each. */
 sp_status spo_dense_verify_chain_status(spo_dense_verify *verify, uint32_t *status);
-/* DenseVerify::encodePrefill: a chunk of 1 to 16 x max_lanes prompt tokens of ONE sequence (its pages from table_first,
+/* DenseVerify::encodePrefill: a chunk of 1 to 16 x max_lanes (or the prefill_rows it was created with) prompt tokens of ONE sequence (its pages from table_first,
  * `committed` tokens cached before the chunk) in one pass over the weights, where the reference prefills a prompt in
  * chunks (Runtime.cpp's chunked prefill over QwenTarget.cpp:457-496): the tokens go in SPO_VERIFY_INPUT_TOKENS, a chain
  * of tree rows a block of sixteen in SPO_VERIFY_TREE_ROWS, each row's depth in its block in SPO_VERIFY_DEPTHS, as a

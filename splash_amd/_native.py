@@ -269,6 +269,12 @@ _sig("spo_attention_add_projection", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c
 _sig("spo_attention_fuses_projection", c_int, c_p, c_p, P(LinearPlan))
 _sig("spo_attention_add_fused_projection", c_int, c_p, c_p, P(ChainLink), c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_u64)
 _sig("spo_attention_add_attention", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_u64, c_p, c_p, c_p)
+_sig("spo_attention_chunk_plan_create", c_int, P(AttentionGeometry), P(AttentionRows), c_u32, P(c_p))
+_sig("spo_attention_chunk_plan_destroy", None, c_p)
+_sig("spo_attention_chunk_plan_dispatches", c_u32, c_p)
+_sig("spo_attention_chunk_workspace", c_int, c_p, P(c_u64))
+_sig("spo_attention_add_chunk_projection", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_u64)
+_sig("spo_attention_add_chunk_attention", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_u64, c_p, c_p, c_p)
 _sig("spo_attention_add_path_commit", c_int, c_p, c_p, c_p, c_p, c_p, c_u64)
 
 _sig("spo_norm_add_rms", c_int, c_p, c_p, c_p, c_p, c_u32, c_u32)
@@ -309,6 +315,7 @@ _sig("spo_dense_verify_results", c_int, c_p, P(VerifyLane), c_u32, P(c_u32), P(c
 _sig("spg_dense_dimensions", c_int, c_p, P(DenseDimensions))
 _sig("spo_dense_verify_load_gguf", c_int, c_p, c_p)
 _sig("spo_dense_verify_create", c_int, c_p, P(DenseDimensions), c_u32, c_u32, c_u32, P(c_p))
+_sig("spo_dense_verify_create_chunked", c_int, c_p, P(DenseDimensions), c_u32, c_u32, c_u32, c_u32, P(c_p))
 _sig("spo_dense_verify_destroy", None, c_p)
 _sig("spo_dense_verify_set_layer", c_int, c_p, c_u32, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p)
 _sig("spo_dense_verify_set_head", c_int, c_p, c_u32, c_p, c_p, c_p)

@@ -10,6 +10,7 @@ struct spo_graph { splash::hip::CommandGraph graph; };
 struct spo_projection { splash::ops::Projection projection; };
 struct spo_linear { splash::ops::Linear linear; };
 struct spo_attention_plan { splash::ops::AttentionPlan plan; };
+struct spo_attention_chunk_plan { splash::ops::AttentionChunkPlan plan; };
 
 struct spg_file;
 namespace splash::model {

@@ -187,13 +187,17 @@ sp_status spo_draft_add_verify_rows(spo_graph *graph, sp_buffer *tree_tokens, sp
 
 sp_status spo_dense_verify_create(sp_backend *backend, const spo_dense_dimensions *d, uint32_t max_lanes, uint32_t physical_pages,
                                   uint32_t page_table_entries, spo_dense_verify **out) {
+  return spo_dense_verify_create_chunked(backend, d, max_lanes, physical_pages, page_table_entries, 0, out);
+}
+sp_status spo_dense_verify_create_chunked(sp_backend *backend, const spo_dense_dimensions *d, uint32_t max_lanes, uint32_t physical_pages,
+                                          uint32_t page_table_entries, uint32_t prefill_rows, spo_dense_verify **out) {
   return capi::guard([&] {
     capi::require(backend && d && out, "backend, dimensions or result");
     auto holder = std::make_unique<spo_dense_verify>();
     holder->backend = std::make_unique<hip::Backend>(backend);
     model::DenseDimensions dims{d->hidden, d->q_heads, d->kv_heads, d->head_dim, d->ffn, d->vocabulary, d->layers,
                                 d->rotary_pairs, d->normalize_heads != 0, d->rope_theta};
-    holder->verify = std::make_unique<model::DenseVerify>(*holder->backend, dims, max_lanes, physical_pages, page_table_entries);
+    holder->verify = std::make_unique<model::DenseVerify>(*holder->backend, dims, max_lanes, physical_pages, page_table_entries, prefill_rows);
     *out = holder.release();
   });
 }

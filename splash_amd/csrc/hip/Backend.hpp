@@ -64,6 +64,12 @@ public:
   void fill(int byte, uint64_t bytes, uint64_t offset = 0) const {
     throwStatus(sp_buffer_fill(handle_.get(), offset, byte, bytes));
   }
+  // Bytes [offset, offset + length) of this buffer as a buffer of their own; the view keeps the base alive.
+  [[nodiscard]] Buffer slice(uint64_t offsetBytes, uint64_t lengthBytes) const {
+    sp_buffer *raw = nullptr;
+    throwStatus(sp_buffer_view(handle_.get(), offsetBytes, lengthBytes, &raw));
+    return adopt(raw);
+  }
   // Adopts a handle the caller owns one reference of.
   static Buffer adopt(sp_buffer *raw) {
     Buffer b;

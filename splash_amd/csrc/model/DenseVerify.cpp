@@ -8,38 +8,55 @@ namespace splash::model {
 
 using hip::BufferStorage;
 
+namespace {
+// A long chunk's projections run in windows of this many rows (whole 64-row pieces of the activation tables).
+constexpr uint32_t kWindowRows = ops::kMaximumDispatchRows;
+// Rows [first, first + count) of a buffer of rows of `rowBytes` bytes.
+hip::Buffer rowsOf(const hip::Buffer &buffer, uint32_t first, uint32_t count, uint64_t rowBytes) {
+  return buffer.slice(first * rowBytes, count * rowBytes);
+}
+// The activation tables (k inputs a row) of rows [first, first + count) of the tables of a chunk's rows: 64-row
+// pieces lie one after the other, and `first` is a multiple of 64.
+hip::Buffer tablesOf(const hip::Buffer &tables, uint32_t k, uint32_t first, uint32_t count) {
+  return tables.slice(uint64_t{first / GGUF_MAXIMUM_ROWS} * gguf_table_bytes(k, GGUF_PIECE_TILES), gguf_tables_bytes(k, gguf_row_tiles(count)));
+}
+} // namespace
+
 DenseVerify::DenseVerify(hip::Backend &backend, DenseDimensions d, uint32_t maxLanes, uint32_t physicalPages,
-                         uint32_t pageTableEntries)
+                         uint32_t pageTableEntries, uint32_t prefillRows)
     : backend_(backend), dims_(d), linear_(backend.deviceInfo()), maxLanes_(maxLanes) {
+  if (prefillRows > ops::kMaximumChunkRows) throw std::invalid_argument("a prompt chunk holds at most 2048 rows");
   if (!d.hidden || !d.layers || !d.vocabulary || !d.ffn || !maxLanes || maxLanes > ATTENTION_MAXIMUM_SEQUENCES)
     throw std::invalid_argument("a dense verify step takes a model and 1 to 8 lanes");
   if (d.hidden % GGUF_BLOCK || d.ffn % GGUF_BLOCK || d.attentionWidth() % GGUF_BLOCK || d.vocabulary % GGUF_TILE_COLUMNS)
     throw std::invalid_argument("the model's widths hold whole super-blocks and its vocabulary whole column tiles");
   maxRows_ = maxLanes * ATTENTION_MAXIMUM_ROWS;
+  rowCapacity_ = std::max(maxRows_, prefillRows);
+  const uint32_t windowRows = std::min(rowCapacity_, std::max(maxRows_, kWindowRows));  // the most rows of one projection dispatch
   weights_.layers.resize(d.layers);
   const ops::kv::Layout layout{d.kvHeads, d.headDimension};
   pageBytes_ = layout.bytesPerLayerPage();
   auto device = [&](uint64_t bytes, const char *label) { return backend.allocateBuffer(std::max<uint64_t>(bytes, 16), BufferStorage::Private, label); };
   auto shared = [&](uint64_t bytes, const char *label) { return backend.allocateBuffer(std::max<uint64_t>(bytes, 16), BufferStorage::Shared, label); };
-  const uint64_t R = maxRows_;
-  hidden_[0] = device(R * d.hidden * 2, "hidden 0");
-  hidden_[1] = device(R * d.hidden * 2, "hidden 1");
-  normalized_ = device(R * d.hidden * 2, "normalized");
-  qkv_ = device(R * d.qkvWidth() * 2, "qkv");
-  attention_ = device(R * d.attentionWidth() * 2, "attention output");
-  intermediate_ = device(R * d.ffn * 2, "ffn intermediate");
+  const uint64_t R = maxRows_, C = rowCapacity_;
+  hidden_[0] = device(C * d.hidden * 2, "hidden 0");
+  hidden_[1] = device(C * d.hidden * 2, "hidden 1");
+  normalized_ = device(C * d.hidden * 2, "normalized");
+  qkv_ = device(C * d.qkvWidth() * 2, "qkv");
+  attention_ = device(C * d.attentionWidth() * 2, "attention output");
+  intermediate_ = device(uint64_t{windowRows} * d.ffn * 2, "ffn intermediate");
   logits_ = device(R * d.vocabulary * 4, "logits");
-  ropeCos_ = device(R * std::max(1u, d.rotaryPairs) * 4, "rope cos");
-  ropeSin_ = device(R * std::max(1u, d.rotaryPairs) * 4, "rope sin");
+  ropeCos_ = device(C * std::max(1u, d.rotaryPairs) * 4, "rope cos");
+  ropeSin_ = device(C * std::max(1u, d.rotaryPairs) * 4, "rope sin");
   inverseFrequency_ = device(std::max(1u, d.rotaryPairs) * 4, "rope inverse frequency");
   if (d.rotaryPairs) {
     std::vector<float> inv(d.rotaryPairs);
     for (uint32_t i = 0; i < d.rotaryPairs; ++i) inv[i] = float(std::pow(double(d.ropeTheta), -double(i) / d.rotaryPairs));
     inverseFrequency_.upload(inv.data(), inv.size() * 4);
   }
-  inputTokens_ = shared(R * 4, "input tokens");
-  treeRows_ = shared(R * sizeof(AttentionTreeRow), "tree rows");
-  depths_ = shared(R * 4, "row depths");
+  inputTokens_ = shared(C * 4, "input tokens");
+  treeRows_ = shared(C * sizeof(AttentionTreeRow), "tree rows");
+  depths_ = shared(C * 4, "row depths");
   uniforms_ = shared(R * 8, "uniforms");
   tokens_ = shared(R * 4, "selected tokens");
   retained_ = shared(maxLanes * 4, "retained");
@@ -56,7 +73,9 @@ DenseVerify::DenseVerify(hip::Backend &backend, DenseDimensions d, uint32_t maxL
   for (ops::LinearMatrix m : {ops::LinearMatrix{d.qkvWidth(), d.hidden}, ops::LinearMatrix{d.hidden, d.attentionWidth()},
                               ops::LinearMatrix{d.ffn, d.hidden}, ops::LinearMatrix{d.hidden, d.ffn},
                               ops::LinearMatrix{d.vocabulary, d.hidden}})
-    size.include(linear_.scratchSize(m, maxRows_));
+    size.include(linear_.scratchSize(m, windowRows));
+  // the table of a chunk's normalized rows holds every window's: a layer's last projection leaves it for the next layer
+  size.input = std::max<uint64_t>(size.input, gguf_tables_bytes(d.hidden, gguf_row_tiles(rowCapacity_)));
   // a q|k|v projection that prepares its attention block keeps partials whatever its plan's parts
   for (uint32_t rows : {16u, 32u, 64u})
     for (uint32_t format : {GGUF_FMT_Q4K, GGUF_FMT_Q6K})
@@ -68,7 +87,9 @@ DenseVerify::DenseVerify(hip::Backend &backend, DenseDimensions d, uint32_t maxL
   scratch_.partials = device(size.partials, "linear partials");
   scratch_.counters = device(std::max<uint64_t>(size.counters, 4), "linear counters");
   // The attention merge and the gate/up pass write the table of the projection after them here.
-  nextTable_ = device(gguf_table_bytes(std::max(d.attentionWidth(), d.ffn), gguf_row_tiles(maxRows_)), "linear table 2");
+  nextTable_ = device(gguf_tables_bytes(std::max(d.attentionWidth(), d.ffn), gguf_row_tiles(windowRows)), "linear table 2");
+  if (rowCapacity_ > maxRows_)
+    chunkAttentionTable_ = device(gguf_tables_bytes(d.attentionWidth(), gguf_row_tiles(rowCapacity_)), "chunk attention table");
   // Chained projections each keep a table, partials and counters of their own.
   chainTables_[0] = device(gguf_table_bytes(d.hidden, gguf_row_tiles(maxRows_)), "gate/up table");
   chainTables_[1] = device(gguf_table_bytes(d.ffn, gguf_row_tiles(maxRows_)), "down table");
@@ -79,10 +100,13 @@ DenseVerify::DenseVerify(hip::Backend &backend, DenseDimensions d, uint32_t maxL
   chainProgress_ = device(GGUF_CHAIN_PROGRESS_WORDS * 4, "chain progress");
   chainProgress_.fill(0, GGUF_CHAIN_PROGRESS_WORDS * 4);
   // Attention workspace for the most splits any sequence may take.
-  const uint64_t fused = uint64_t{maxLanes} * d.kvHeads * (d.qHeads / d.kvHeads) * 16;
+  // Staged queries for every tile of the longest chunk; partials for the tiles of one dispatch.
+  const uint64_t fusedTile = uint64_t{d.kvHeads} * (d.qHeads / d.kvHeads) * 16;
+  const uint64_t staged = fusedTile * std::max(maxLanes, gguf_row_tiles(rowCapacity_));
+  const uint64_t fused = fusedTile * (rowCapacity_ > maxRows_ ? ATTENTION_MAXIMUM_SEQUENCES : maxLanes);
   maxSplits_ = ATTENTION_MAXIMUM_SPLITS;
-  attentionWorkspace_.queries = device(fused * d.headDimension * 2, "staged queries");
-  attentionWorkspace_.querySums = device(fused * 4, "query sums");
+  attentionWorkspace_.queries = device(staged * d.headDimension * 2, "staged queries");
+  attentionWorkspace_.querySums = device(staged * 4, "query sums");
   attentionWorkspace_.partials = device(fused * maxSplits_ * d.headDimension * 2, "attention partials");
   attentionWorkspace_.partialSums = device(fused * maxSplits_ * 8, "attention partial sums");
   const ops::SamplingWorkspaceSize s = ops::Sampling::workspace(maxRows_);
@@ -294,8 +318,97 @@ void DenseVerify::encodeHead(hip::CommandGraph &graph, uint32_t rows, bool input
   linear_.add(graph, head, weights_.head, linear_.plan(weights_.head, rows));
 }
 
+// A layer of a long chunk: every window's q|k|v rows, the chunked attention over all of them, then every window's output
+// projection and SwiGLU. Each window's projections and tables are the ones encodeLayer gives a step of its rows.
+void DenseVerify::encodeChunkLayer(hip::CommandGraph &graph, uint32_t layer, const ops::AttentionChunkPlan &plan, uint32_t tokens,
+                                   bool inputReady, bool feedsNext) {
+  const DenseLayer &w = weights_.layers.at(layer);
+  const uint64_t hiddenBytes = uint64_t{dims_.hidden} * 2;
+  struct Window {
+    uint32_t first, rows;
+    hip::Buffer residual, next, normalized, qkv, attention;
+    ops::LinearScratch scratch;  // the driver's partials and counters, the window's own tables of normalized rows
+  };
+  std::vector<Window> windows;
+  for (uint32_t first = 0; first < tokens; first += kWindowRows) {
+    Window v;
+    v.first = first;
+    v.rows = std::min(kWindowRows, tokens - first);
+    v.residual = rowsOf(hidden_[0], first, v.rows, hiddenBytes);
+    v.next = rowsOf(hidden_[1], first, v.rows, hiddenBytes);
+    v.normalized = rowsOf(normalized_, first, v.rows, hiddenBytes);
+    v.qkv = rowsOf(qkv_, first, v.rows, uint64_t{dims_.qkvWidth()} * 2);
+    v.attention = rowsOf(attention_, first, v.rows, uint64_t{dims_.attentionWidth()} * 2);
+    v.scratch = scratch_;
+    v.scratch.input = tablesOf(scratch_.input, dims_.hidden, first, v.rows);
+    windows.push_back(std::move(v));
+  }
+  for (const Window &v : windows) {
+    const ops::PreparedInput prepared =
+        inputReady ? ops::PreparedInput{v.normalized, ops::LinearInput::TableUnscaled}
+                   : ops::Normalization::addRmsTable(graph, v.residual, w.inputNorm, v.normalized, v.scratch, dims_.hidden, v.rows);
+    ops::LinearBuffers qkv;
+    qkv.input = v.normalized;
+    qkv.output = v.qkv;
+    qkv.scratch = v.scratch;
+    qkv.prepared = prepared;
+    linear_.add(graph, qkv, w.qkv, linear_.plan(w.qkv, v.rows));
+  }
+  const ops::KvPages pages{pageTable_, kvPools_.at(layer), pageBytes_};
+  ops::PagedAttention::addChunkProjection(graph, plan, {qkv_, w.queryNorm, w.keyNorm, ropeCos_, ropeSin_}, attentionWorkspace_, pages);
+  ops::PagedAttention::addChunkAttention(graph, plan, attentionWorkspace_, treeRows_, pages, attention_, chunkAttentionTable_);
+  for (const Window &v : windows) {
+    const ops::PreparedInput ready{v.normalized, ops::LinearInput::TableUnscaled};
+    const bool outputNorms = linear_.normsRows(w.output, v.rows);
+    ops::LinearBuffers output;
+    output.input = v.attention;
+    output.output = v.next;
+    output.residual = v.residual;
+    output.scratch = v.scratch;
+    output.scratch.input = tablesOf(chunkAttentionTable_, dims_.attentionWidth(), v.first, v.rows);
+    output.prepared = {v.attention, ops::LinearInput::Table16};
+    if (outputNorms) {
+      output.normWeight = w.postNorm;
+      output.nextTable = v.scratch.input;
+    }
+    linear_.add(graph, output, w.output,
+                linear_.plan(w.output, v.rows, outputNorms ? ops::LinearEpilogue::ResidualNorm : ops::LinearEpilogue::Residual));
+    const ops::PreparedInput prepared =
+        outputNorms ? ready : ops::Normalization::addRmsTable(graph, v.next, w.postNorm, v.normalized, v.scratch, dims_.hidden, v.rows);
+    ops::FfnBuffers ffn{v.normalized, intermediate_, v.scratch, nextTable_};
+    if (feedsNext) {
+      ffn.followingNorm = layer + 1 < dims_.layers ? weights_.layers[layer + 1].inputNorm : weights_.finalNorm;
+      ffn.followingTable = v.scratch.input;
+    }
+    linear_.addSwiGlu(graph, {&w.gate, &w.up, &w.down}, ffn, v.next, v.residual, v.rows, prepared);
+  }
+}
+
 void DenseVerify::encodePrefill(hip::CommandGraph &graph, uint32_t tableFirst, uint32_t committed, uint32_t tokens) {
-  if (!tokens || tokens > maxRows_) throw std::invalid_argument("a prompt chunk takes 1 to 16 tokens a lane of the driver");
+  if (!tokens || tokens > rowCapacity_) throw std::invalid_argument("a prompt chunk takes 1 to the driver's most prefill rows");
+  if (tokens > maxRows_) {
+    const ops::AttentionGeometry geometry{dims_.qHeads, dims_.kvHeads, dims_.headDimension, dims_.rotaryPairs, dims_.normalizeHeads};
+    const ops::AttentionChunkPlan plan = ops::PagedAttention::planChunks(geometry, {{0, tokens, committed, tableFirst}});
+    if (dims_.rotaryPairs) {
+      // the RoPE tables eight blocks a dispatch, each dispatch over its own rows of the depths and tables
+      const uint32_t span = ATTENTION_MAXIMUM_SEQUENCES * ATTENTION_MAXIMUM_ROWS;
+      for (uint32_t first = 0; first < tokens; first += span) {
+        const uint32_t count = std::min(span, tokens - first);
+        std::vector<ops::RopeSequence> rope;
+        for (uint32_t at = 0; at < count; at += ATTENTION_MAXIMUM_ROWS)
+          rope.push_back({at, std::min<uint32_t>(ATTENTION_MAXIMUM_ROWS, count - at), committed + first + at});
+        const uint64_t tableBytes = uint64_t{dims_.rotaryPairs} * 4;
+        ops::RoPE::addTreeTables(graph, inverseFrequency_, rowsOf(depths_, first, count, 4), rowsOf(ropeCos_, first, count, tableBytes),
+                                 rowsOf(ropeSin_, first, count, tableBytes), dims_.rotaryPairs, rope);
+      }
+    }
+    encodeEmbedding(graph, tokens);
+    // every window is a step's worth of rows at most, so what holds for one holds for all
+    const bool feeds = layersFeedNext(std::min(tokens, kWindowRows));
+    for (uint32_t layer = 0; layer < dims_.layers; ++layer)
+      encodeChunkLayer(graph, layer, plan, tokens, feeds && layer > 0, feeds && layer + 1 < dims_.layers);
+    return;
+  }
   std::vector<ops::AttentionRows> sequences;
   std::vector<ops::RopeSequence> rope;
   for (uint32_t first = 0; first < tokens; first += ATTENTION_MAXIMUM_ROWS) {

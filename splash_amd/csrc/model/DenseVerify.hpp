@@ -50,9 +50,11 @@ struct VerifyLane final {
 
 class DenseVerify final {
 public:
-  // maxLanes x 16 rows at most; the KV pool holds `physicalPages` pages per layer.
+  // maxLanes x 16 rows a step at most; the KV pool holds `physicalPages` pages per layer. prefillRows: the most rows of
+  // a prompt chunk (encodePrefill), 0 for a step's most, up to ops::kMaximumChunkRows; the rows' buffers are sized for it.
   DenseVerify(hip::Backend &backend, DenseDimensions dimensions, uint32_t maxLanes, uint32_t physicalPages,
-              uint32_t pageTableEntries);
+              uint32_t pageTableEntries, uint32_t prefillRows = 0);
+  [[nodiscard]] uint32_t prefillRows() const noexcept { return rowCapacity_; }
 
   [[nodiscard]] const DenseDimensions &dimensions() const noexcept { return dims_; }
   DenseWeights &weights() noexcept { return weights_; }
@@ -103,12 +105,14 @@ public:
   // The results are those of the separate dispatches, bit for bit.
   void setChained(bool chained) noexcept { chained_ = chained; }
   [[nodiscard]] bool chained() const noexcept { return chained_; }
-  // A chunk of a sequence's prompt (1 to 16 x maxLanes tokens, its input tokens, chain tree rows a block of sixteen and
-  // depths where a step's are) in one pass over the weights: the chunk runs as blocks of sixteen rows of one sequence,
+  // A chunk of a sequence's prompt (1 to prefillRows() tokens, its input tokens, chain tree rows a block of sixteen and
+  // depths where a step's are) in one pass over the layers: the chunk runs as blocks of sixteen rows of one sequence,
   // block i's history ending where block i - 1's rows end, through every layer and no head, so the tokens' keys and
   // values are in the pages and the hidden rows where a step leaves them. The counterpart of the reference's chunked
   // prefill (Runtime.cpp's prefill chunks over QwenTarget's layers) with the verify step's own kernels: the pools and
-  // the hidden rows are those of the blocks run one step after the other, bit for bit.
+  // the hidden rows are those of the blocks run one step after the other, bit for bit. A chunk of more rows than a
+  // step's runs layer by layer: the projections in windows of ops::kMaximumDispatchRows rows around one chunked
+  // attention (ops::PagedAttention::planChunks) over all of them.
   void encodePrefill(hip::CommandGraph &graph, uint32_t tableFirst, uint32_t committed, uint32_t tokens);
   // A layer's q|k|v projection also prepares its attention block (ops::PagedAttention::addFusedProjection) where the
   // kernels take the pair: off by default (the projection and the prepare kernel run one after the other). The results
@@ -126,7 +130,7 @@ private:
   DenseDimensions dims_;
   DenseWeights weights_;
   ops::Linear linear_;
-  uint32_t maxRows_ = 0, maxLanes_ = 0;
+  uint32_t maxRows_ = 0, maxLanes_ = 0, rowCapacity_ = 0;
   uint64_t pageBytes_ = 0, layerBytes_ = 0;
   hip::Buffer kvAll_;
   hip::Buffer hidden_[2], normalized_, qkv_, attention_, intermediate_, logits_, draft_;
@@ -141,6 +145,9 @@ private:
   ops::LinearScratch chainScratch_[GGUF_CHAIN_LINKS];
   bool chained_ = false, encodedChains_ = false, fusedPrepare_ = false, testChildren_ = false;
   ops::SamplingBuffers children_;   // the four candidate-children buffers, bound into a step's sampling buffers when it tests them
+  hip::Buffer chunkAttentionTable_;  // a long chunk's attention rows as the output projection's tables, every window's
+  void encodeChunkLayer(hip::CommandGraph &graph, uint32_t layer, const ops::AttentionChunkPlan &plan, uint32_t tokens, bool first,
+                        bool feedsNext);
   void encodeChainedLayers(hip::CommandGraph &graph, const ops::AttentionPlan &plan, uint32_t rows);
   [[nodiscard]] bool chains(uint32_t rows) const noexcept;
   ops::AttentionWorkspace attentionWorkspace_;

@@ -135,9 +135,10 @@ PreparedInput PagedAttention::addFusedProjection(hip::CommandGraph &graph, const
 
 void PagedAttention::addAttention(hip::CommandGraph &graph, const AttentionPlan &plan, const AttentionWorkspace &w,
                                   const hip::Buffer &treeRows, const KvPages &pages, const hip::Buffer &output,
-                                  const hip::Buffer &outputTable, const hip::Buffer &packed) {
+                                  const hip::Buffer &outputTable, const hip::Buffer &packed, uint32_t tableRows) {
   const AttentionGeometry &g = plan.geometry();
   const uint32_t rows = totalRows(plan.sequences());
+  if (tableRows && tableRows < rows) throw std::invalid_argument("the output table holds the dispatch's rows");
   const AttentionWorkspaceSize need = plan.workspace();
   requireBytes(w.queries, need.queries, "staged queries");
   requireBytes(w.querySums, need.querySums, "staged query sums");
@@ -151,7 +152,7 @@ void PagedAttention::addAttention(hip::CommandGraph &graph, const AttentionPlan 
   const uint32_t width = g.qHeads * g.headDimension;
   if (outputTable) {
     if (width % GGUF_BLOCK) throw std::invalid_argument("an attention output table holds whole super-blocks");
-    params.table_tiles = gguf_row_tiles(rows);
+    params.table_tiles = gguf_row_tiles(tableRows ? tableRows : rows);
     requireBytes(outputTable, gguf_tables_bytes(width, params.table_tiles), "attention output table");
   }
   graph.add(std::string(g.int8Queries ? "attention_q8q_split" : "attention_q8_split") + kernelSuffix(g) + "_g" + std::to_string(g.group()),
@@ -160,6 +161,83 @@ void PagedAttention::addAttention(hip::CommandGraph &graph, const AttentionPlan 
   graph.add("attention_reduce" + kernelSuffix(g) + (outputTable ? "_t" : ""),
             {w.partials, w.partialSums, output, outputTable ? outputTable : output, g.gated ? packed : output}, params,
             {g.qHeads, ATTENTION_MAXIMUM_ROWS, plan.sequences().size()}, {256, 1, 1});
+}
+
+AttentionWorkspaceSize AttentionChunkPlan::workspace() const noexcept {
+  AttentionWorkspaceSize size;
+  for (const AttentionPlan &plan : dispatches_) {
+    const AttentionWorkspaceSize one = plan.workspace();
+    size.queries += one.queries;
+    size.querySums += one.querySums;
+    size.partials = std::max(size.partials, one.partials);
+    size.partialSums = std::max(size.partialSums, one.partialSums);
+  }
+  return size;
+}
+
+AttentionChunkPlan PagedAttention::planChunks(const AttentionGeometry &geometry, const std::vector<AttentionChunk> &chunks) {
+  if (chunks.empty()) throw std::invalid_argument("a chunked attention takes at least one chunk");
+  std::vector<AttentionRows> tiles;
+  AttentionChunkPlan plan;
+  plan.geometry_ = geometry;
+  for (const AttentionChunk &chunk : chunks) {
+    if (!chunk.tokens || chunk.tokens > kMaximumChunkRows) throw std::invalid_argument("a prompt chunk holds 1 to 2048 rows");
+    if (chunk.firstRow < plan.rows_) throw std::invalid_argument("the chunks' rows ascend and do not overlap");
+    for (uint32_t first = 0; first < chunk.tokens; first += ATTENTION_MAXIMUM_ROWS)
+      tiles.push_back({chunk.firstRow + first, std::min<uint32_t>(ATTENTION_MAXIMUM_ROWS, chunk.tokens - first), chunk.committed + first,
+                       chunk.tableFirst});
+    plan.rows_ = chunk.firstRow + chunk.tokens;
+  }
+  plan.tiles_ = uint32_t(tiles.size());
+  for (size_t first = 0; first < tiles.size(); first += ATTENTION_MAXIMUM_SEQUENCES)
+    plan.dispatches_.push_back(PagedAttention::plan(
+        geometry, {tiles.begin() + first, tiles.begin() + std::min(tiles.size(), first + ATTENTION_MAXIMUM_SEQUENCES)}));
+  return plan;
+}
+
+namespace {
+// Dispatch d's part of a chunk plan's workspace: its tiles' staged queries after those of the dispatches before it.
+AttentionWorkspace workspaceOf(const AttentionChunkPlan &plan, const AttentionWorkspace &all, size_t d) {
+  uint64_t queries = 0, sums = 0;
+  for (size_t i = 0; i < d; ++i) {
+    const AttentionWorkspaceSize before = plan.dispatches()[i].workspace();
+    queries += before.queries;
+    sums += before.querySums;
+  }
+  const AttentionWorkspaceSize mine = plan.dispatches()[d].workspace();
+  AttentionWorkspace w = all;
+  w.queries = all.queries.slice(queries, mine.queries);
+  w.querySums = all.querySums.slice(sums, mine.querySums);
+  return w;
+}
+void requireChunkWorkspace(const AttentionChunkPlan &plan, const AttentionWorkspace &w, bool attends) {
+  const AttentionWorkspaceSize need = plan.workspace();
+  requireBytes(w.queries, need.queries, "staged queries");
+  requireBytes(w.querySums, need.querySums, "staged query sums");
+  if (attends) {
+    requireBytes(w.partials, need.partials, "attention partials");
+    requireBytes(w.partialSums, need.partialSums, "attention partial sums");
+  }
+}
+} // namespace
+
+void PagedAttention::addChunkProjection(hip::CommandGraph &graph, const AttentionChunkPlan &plan, const AttentionProjectionBuffers &buffers,
+                                        const AttentionWorkspace &workspace, const KvPages &pages) {
+  requireChunkWorkspace(plan, workspace, false);
+  for (size_t d = 0; d < plan.dispatches().size(); ++d)
+    addProjection(graph, plan.dispatches()[d], buffers, workspaceOf(plan, workspace, d), pages);
+}
+
+void PagedAttention::addChunkAttention(hip::CommandGraph &graph, const AttentionChunkPlan &plan, const AttentionWorkspace &workspace,
+                                       const hip::Buffer &treeRows, const KvPages &pages, const hip::Buffer &output,
+                                       const hip::Buffer &outputTable, const hip::Buffer &packed) {
+  requireChunkWorkspace(plan, workspace, true);
+  // every dispatch writes its rows of the one table of all the rows
+  if (outputTable)
+    requireBytes(outputTable, gguf_tables_bytes(plan.geometry().qHeads * plan.geometry().headDimension, gguf_row_tiles(plan.rows())),
+                 "attention output table");
+  for (size_t d = 0; d < plan.dispatches().size(); ++d)
+    addAttention(graph, plan.dispatches()[d], workspaceOf(plan, workspace, d), treeRows, pages, output, outputTable, packed, plan.rows());
 }
 
 void PagedAttention::addPathCommit(hip::CommandGraph &graph, const AttentionPlan &plan, const hip::Buffer &retained,

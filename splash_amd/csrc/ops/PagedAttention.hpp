@@ -83,6 +83,37 @@ private:
   uint32_t splits_ = 1;
 };
 
+// A prompt chunk of one sequence (the reference's kv::ChunkedPrefillParams with its rows' place in the command,
+// PagedAttention.hpp:28-39): `tokens` rows at positions from `committed`, attending causally. It runs as tiles of
+// ATTENTION_MAXIMUM_ROWS rows (the reference's tiles of kAttentionTileRows, :42-50), tile t a block of the sequence
+// whose history ends where tile t - 1's rows end, ATTENTION_MAXIMUM_SEQUENCES tiles a dispatch.
+struct AttentionChunk final {
+  uint32_t firstRow = 0;    // first packed row
+  uint32_t tokens = 0;      // 1..kMaximumChunkRows
+  uint32_t committed = 0;   // tokens cached before the chunk
+  uint32_t tableFirst = 0;  // first page-table entry of the sequence
+};
+inline constexpr uint32_t kMaximumChunkRows = 2048;  // SPLASH_PREFILL_TOKEN_BUDGET, ExecutionGeometry.h:36
+
+// The dispatches of a command's chunks: each a plan of up to eight tiles. A tile's history splits follow its own
+// length alone (attentionSplits), so a row's result is, bit for bit, the one its tile gives as a verify block.
+class AttentionChunkPlan final {
+public:
+  [[nodiscard]] const AttentionGeometry &geometry() const noexcept { return geometry_; }
+  [[nodiscard]] const std::vector<AttentionPlan> &dispatches() const noexcept { return dispatches_; }
+  [[nodiscard]] uint32_t tiles() const noexcept { return tiles_; }
+  [[nodiscard]] uint32_t rows() const noexcept { return rows_; }
+  // Staged queries for every tile (a tile's survive from the projection pass to its attention), partials for the
+  // dispatch that needs the most (dispatches run one after the other).
+  [[nodiscard]] AttentionWorkspaceSize workspace() const noexcept;
+
+private:
+  friend class PagedAttention;
+  AttentionGeometry geometry_;
+  std::vector<AttentionPlan> dispatches_;
+  uint32_t tiles_ = 0, rows_ = 0;
+};
+
 struct AttentionProjectionBuffers final {
   hip::Buffer qkv;             // bf16 [packed rows][(q + 2 kv) heads * D]
   hip::Buffer queryNorm, keyNorm;  // bf16 [D]; used when geometry.normalize
@@ -112,10 +143,21 @@ public:
                                           const KvPages &pages);
   // Split + reduce (PagedAttention.cpp:466-607): output bf16 [packed rows][q heads * D].
   // outputTable (optional): the reduce also writes the rows as the activation table of the
-  // projection that follows (gguf_table_bytes(q heads * D, rows)), which then needs no table pass.
+  // projection that follows (gguf_table_bytes(q heads * D, rows)), which then needs no table pass; tableRows: the
+  // rows that table holds when they are more than this dispatch's (a chunk's dispatches share one table).
   static void addAttention(hip::CommandGraph &graph, const AttentionPlan &plan, const AttentionWorkspace &workspace,
                            const hip::Buffer &treeRows, const KvPages &pages, const hip::Buffer &output,
-                           const hip::Buffer &outputTable = {}, const hip::Buffer &packed = {});
+                           const hip::Buffer &outputTable = {}, const hip::Buffer &packed = {}, uint32_t tableRows = 0);
+  // Prompt chunks (the reference's plan over kv::ChunkedPrefillParams, PagedAttention.hpp:270-275, PagedAttention.cpp:351-389):
+  // throws for a chunk of no or more than kMaximumChunkRows rows. addChunkProjection runs the projection pass of every
+  // dispatch, so that every row's K and V are stored before any row attends; addChunkAttention then splits and merges
+  // dispatch by dispatch. Buffers as addProjection's and addAttention's, over all the chunks' rows.
+  [[nodiscard]] static AttentionChunkPlan planChunks(const AttentionGeometry &geometry, const std::vector<AttentionChunk> &chunks);
+  static void addChunkProjection(hip::CommandGraph &graph, const AttentionChunkPlan &plan, const AttentionProjectionBuffers &buffers,
+                                 const AttentionWorkspace &workspace, const KvPages &pages);
+  static void addChunkAttention(hip::CommandGraph &graph, const AttentionChunkPlan &plan, const AttentionWorkspace &workspace,
+                                const hip::Buffer &treeRows, const KvPages &pages, const hip::Buffer &output,
+                                const hip::Buffer &outputTable = {}, const hip::Buffer &packed = {});
   // Moves the retained path's slots to their depths (PagedAttention.cpp:647-667); retained is a
   // uint32 mask per sequence.
   // `layers` pools lie layerBytes apart from pages.pool (one dispatch commits them all, as the

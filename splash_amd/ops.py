@@ -297,6 +297,34 @@ class AttentionPlan:
             pass
 
 
+class AttentionChunkPlan:
+    """ops::AttentionChunkPlan: prompt chunks [(first_row, tokens, committed, table_first)] as dispatches of eight 16-row tiles."""
+
+    def __init__(self, q_heads, kv_heads, head_dim, chunks, rotary_pairs=0, normalize=False, gated=False, int8_queries=False):
+        g = nat.AttentionGeometry(q_heads, kv_heads, head_dim, rotary_pairs, int(normalize), int(gated), int(int8_queries))
+        rows = (nat.AttentionRows * len(chunks))(*[nat.AttentionRows(*c) for c in chunks])   # a chunk has a sequence's four fields
+        h = ctypes.c_void_p()
+        check(lib.spo_attention_chunk_plan_create(ctypes.byref(g), rows, len(chunks), ctypes.byref(h)))
+        self.handle = h
+        self.geometry = g
+        self.chunks = chunks
+
+    @property
+    def dispatches(self):
+        return lib.spo_attention_chunk_plan_dispatches(self.handle)
+
+    def workspace_sizes(self):
+        sizes = (ctypes.c_uint64 * 4)()
+        check(lib.spo_attention_chunk_workspace(self.handle, sizes))
+        return list(sizes)
+
+    def __del__(self):
+        try:
+            lib.spo_attention_chunk_plan_destroy(self.handle)
+        except Exception:
+            pass
+
+
 class AttentionWorkspace:
     def __init__(self, backend, plan):
         q, qs, po, ps = plan.workspace_sizes()
@@ -343,6 +371,23 @@ class PagedAttention:
                                               pages.table.handle, pages.pool.handle, pages.page_bytes, output.handle,
                                               output_table.handle if output_table is not None else None,
                                               packed_qkv.handle if packed_qkv is not None else None))
+        graph._keep.extend([plan, workspace, tree_rows, pages, output, output_table, packed_qkv])
+
+    @staticmethod
+    def add_chunk_projection(graph, plan, qkv, workspace, pages, query_norm=None, key_norm=None, rope_cos=None, rope_sin=None):
+        h = lambda b: b.handle if b is not None else None
+        check(lib.spo_attention_add_chunk_projection(graph.handle, plan.handle, qkv.handle, h(query_norm), h(key_norm), h(rope_cos),
+                                                     h(rope_sin), workspace.queries.handle, workspace.query_sums.handle,
+                                                     pages.table.handle, pages.pool.handle, pages.page_bytes))
+        graph._keep.extend([plan, qkv, workspace, pages, query_norm, key_norm, rope_cos, rope_sin])
+
+    @staticmethod
+    def add_chunk_attention(graph, plan, workspace, tree_rows, pages, output, output_table=None, packed_qkv=None):
+        check(lib.spo_attention_add_chunk_attention(graph.handle, plan.handle, workspace.queries.handle, workspace.query_sums.handle,
+                                                    workspace.partials.handle, workspace.partial_sums.handle, tree_rows.handle,
+                                                    pages.table.handle, pages.pool.handle, pages.page_bytes, output.handle,
+                                                    output_table.handle if output_table is not None else None,
+                                                    packed_qkv.handle if packed_qkv is not None else None))
         graph._keep.extend([plan, workspace, tree_rows, pages, output, output_table, packed_qkv])
 
     @staticmethod

@@ -26,14 +26,16 @@ class Lane:
 
 class DenseVerify:
     def __init__(self, backend, hidden, q_heads, kv_heads, head_dim, ffn, vocabulary, layers, rotary_pairs=None,
-                 normalize_heads=True, rope_theta=1e6, max_lanes=1, physical_pages=2, page_table_entries=None):
+                 normalize_heads=True, rope_theta=1e6, max_lanes=1, physical_pages=2, page_table_entries=None, prefill_rows=0):
+        """prefill_rows: the most rows of a prompt chunk (encode_prefill); 0: a step's most, 16 x max_lanes."""
         self.backend = backend
         pairs = head_dim // 2 if rotary_pairs is None else rotary_pairs
         self.dims = nat.DenseDimensions(hidden, q_heads, kv_heads, head_dim, ffn, vocabulary, layers, pairs, int(normalize_heads),
                                         rope_theta)
         h = ctypes.c_void_p()
         entries = page_table_entries if page_table_entries is not None else physical_pages
-        check(lib.spo_dense_verify_create(backend.handle, ctypes.byref(self.dims), max_lanes, physical_pages, entries, ctypes.byref(h)))
+        check(lib.spo_dense_verify_create_chunked(backend.handle, ctypes.byref(self.dims), max_lanes, physical_pages, entries, prefill_rows,
+                                                  ctypes.byref(h)))
         self.handle = h
         self.physical_pages = physical_pages
         self._keep = []

@@ -61,7 +61,7 @@ class DenseModel:
         pool.shutdown()
 
     # ------------------------------------------------------------------ GPU side
-    def build_gpu(self, backend, max_lanes, context_tokens):
+    def build_gpu(self, backend, max_lanes, context_tokens, prefill_rows=0):
         """context_tokens: the most tokens a lane's pages hold, one number for every lane or a list with one a lane;
         lane i's logical pages start at entry self.table_first[i] of the page table."""
         d = self.dims
@@ -72,7 +72,7 @@ class DenseModel:
         self.physical_pages = pages + 1
         gpu = verify.DenseVerify(backend, d["hidden"], d["q_heads"], d["kv_heads"], d["head_dim"], d["ffn"], d["vocabulary"],
                                  d["layers"], rope_theta=self.rope_theta, max_lanes=max_lanes, physical_pages=self.physical_pages,
-                                 page_table_entries=pages)
+                                 page_table_entries=pages, prefill_rows=prefill_rows)
         self.table = np.random.default_rng(99).permutation(self.physical_pages)[:pages].astype(np.uint64)
         gpu.buffer(verify.PAGE_TABLE).upload(self.table)
         D, H = d["head_dim"], d["hidden"]

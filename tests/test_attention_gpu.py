@@ -426,3 +426,91 @@ def test_attention_rejects_bad_arguments(backend):
     with pytest.raises(ValueError, match="page table"):
         ops.PagedAttention.add_attention(g, plan, ws, backend.allocate_buffer(16 * 8), kv, backend.allocate_buffer(16 * 8192 * 2))
     assert len(g) == 0
+
+
+class ChunkWorkspace:
+    """The workspace of a chunk plan: every tile's staged queries, the largest dispatch's partials."""
+
+    def __init__(self, backend, plan):
+        q, qs, po, ps = plan.workspace_sizes()
+        self.queries, self.query_sums = backend.allocate_buffer(q), backend.allocate_buffer(qs)
+        self.partials, self.partial_sums = backend.allocate_buffer(po), backend.allocate_buffer(ps)
+
+
+@pytest.mark.parametrize("geometry,tokens,committed,checked", [((16, 8, 64), 53, 0, None), ((32, 4, 128), 129, 250, None),
+                                                               ((64, 8, 128), 300, 1000, (0, 9, 18)),
+                                                               ((64, 8, 128), 2048, 4096, (0, 77, 127))])
+def test_a_prompt_chunk_attends_causally(backend, geometry, tokens, committed, checked):
+    """q8_chunked_prefill_metal_test.mm: a chunk of up to 2048 rows of one sequence, every row over the history and the
+    chunk's rows up to itself. Each checked tile of 16 rows against the oracle's page loop and its fp64 softmax under
+    the attention's gate, and bit for bit against the same tile run as a verify block of its own; the rows' activation
+    table, written by several dispatches, is the one the table pass would write."""
+    q_heads, kv_heads, D = geometry
+    print(f"case attention chunk geometry={geometry} tokens={tokens} committed={committed}", flush=True)
+    rng = np.random.default_rng(tokens + committed)
+    pairs = D // 4
+    kv, logical, table = build_context(rng, backend, q_heads, kv_heads, D, tokens, committed)
+    kc, ks, vc, vs = (a.copy() for a in logical)
+    width = (q_heads + 2 * kv_heads) * D
+    qkv = orc.f32_to_bf16(rng.standard_normal((tokens, width)).astype(np.float32))
+    qw = orc.f32_to_bf16((1 + 0.1 * rng.standard_normal(D)).astype(np.float32))
+    kw = orc.f32_to_bf16((1 + 0.1 * rng.standard_normal(D)).astype(np.float32))
+    angles = rng.uniform(0, 6.28, (tokens, pairs)).astype(np.float32)
+    cosv, sinv = np.cos(angles).astype(np.float32), np.sin(angles).astype(np.float32)
+    tiles = [(first, min(16, tokens - first)) for first in range(0, tokens, 16)]
+    tree = ops.chain_tree_rows([rows for _, rows in tiles])
+    plan = ops.AttentionChunkPlan(q_heads, kv_heads, D, [(0, tokens, committed, 0)], rotary_pairs=pairs, normalize=True)
+    assert plan.dispatches == (len(tiles) + 7) // 8
+    ws = ChunkWorkspace(backend, plan)
+    out = backend.allocate_buffer(tokens * q_heads * D * 2)
+    out_table = backend.allocate_buffer(ops.gguf_table_bytes(q_heads * D, tokens))
+    bufs = dict(qkv=backend.from_array(qkv), qn=backend.from_array(qw), kn=backend.from_array(kw), cos=backend.from_array(cosv),
+                sin=backend.from_array(sinv), tree=backend.from_array(tree))
+    graph = splash_amd.CommandGraph()
+    ops.PagedAttention.add_chunk_projection(graph, plan, bufs["qkv"], ws, kv, query_norm=bufs["qn"], key_norm=bufs["kn"],
+                                            rope_cos=bufs["cos"], rope_sin=bufs["sin"])
+    ops.PagedAttention.add_chunk_attention(graph, plan, ws, bufs["tree"], kv, out, output_table=out_table)
+    backend.run(graph)
+    got = out.download(np.uint16).reshape(tokens, q_heads, D)
+    orc.assert_table_holds(out_table.download(np.uint8), got.reshape(tokens, q_heads * D), lambda count: ops.gguf_table_bytes(q_heads * D, count))
+    # the oracle stores every row of the chunk, then each tile attends as a block that ends at its last row
+    q, kf, vf = orc.attention_prepare(q_heads, kv_heads, D, qkv, qw, kw, cosv, sinv, pairs)
+    kcod, kscl = orc.kv_quantize(kf)
+    vcod, vscl = orc.kv_quantize(vf)
+    for r in range(tokens):
+        t = committed + r
+        p, s = table[t // ops.PAGE_TOKENS], t % ops.PAGE_TOKENS
+        kc[p, :, s], ks[p, :, s], vc[p, :, s], vs[p, :, s] = kcod[r], kscl[r], vcod[r], vscl[r]
+    stored = kv.unpack_pages(kv.download())
+    for a, b in zip(stored, (kc, ks, vc, vs)):
+        assert np.array_equal(a[table], b[table])
+    for index in (range(len(tiles)) if checked is None else checked):
+        first, rows = tiles[index]
+        anc = tree["ancestors"][first:first + rows].astype(np.uint32)
+        want, want64 = orc.attention(np.ascontiguousarray(q[first:first + rows]), kc, ks, vc, vs, table, anc, committed + first)
+        cos, err = tolerance(got[first:first + rows], want64)
+        assert cos >= 0.9999 and err < 0.02, (index, cos, err)
+        cos2, err2 = tolerance(got[first:first + rows], orc.bf16_to_f32(want).astype(np.float64))
+        assert cos2 >= 0.9999 and err2 < 0.02, (index, cos2, err2)
+        # the tile as a verify block of the sequence: the same bits
+        single = ops.AttentionPlan(q_heads, kv_heads, D, [(0, rows, committed + first, 0)], rotary_pairs=pairs, normalize=True)
+        ws1 = ops.AttentionWorkspace(backend, single)
+        out1 = backend.allocate_buffer(rows * q_heads * D * 2)
+        graph = splash_amd.CommandGraph()
+        ops.PagedAttention.add_projection(graph, single, backend.from_array(qkv[first:first + rows]), ws1, kv, query_norm=bufs["qn"],
+                                          key_norm=bufs["kn"], rope_cos=backend.from_array(cosv[first:first + rows]),
+                                          rope_sin=backend.from_array(sinv[first:first + rows]))
+        ops.PagedAttention.add_attention(graph, single, ws1, backend.from_array(ops.chain_tree_rows([rows])), kv, out1)
+        backend.run(graph)
+        assert np.array_equal(out1.download(np.uint16).reshape(rows, q_heads, D), got[first:first + rows]), index
+
+
+def test_chunk_plans_reject_what_they_cannot_run(backend):
+    with pytest.raises(ValueError):
+        ops.AttentionChunkPlan(64, 8, 128, [(0, 0, 0, 0)])
+    with pytest.raises(ValueError):
+        ops.AttentionChunkPlan(64, 8, 128, [(0, 2049, 0, 0)])
+    with pytest.raises(ValueError):
+        ops.AttentionChunkPlan(64, 8, 128, [(0, 40, 0, 0), (32, 40, 0, 8)])   # overlapping rows
+    two = ops.AttentionChunkPlan(64, 8, 128, [(0, 40, 100, 0), (40, 200, 7, 8)])   # two sequences' chunks: 3 + 13 tiles
+    assert two.dispatches == 2

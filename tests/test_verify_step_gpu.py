@@ -329,6 +329,39 @@ def test_a_prompt_chunk_in_one_pass_equals_its_blocks_one_by_one(backend, prompt
     assert len(graph) < len(gpu.encode([verify.Lane(16, committed, table_first=first)], commit=False)) 
 
 
+@pytest.mark.parametrize("prompt_tokens", [300, 1000])
+def test_a_long_prompt_chunk_equals_its_blocks_one_by_one(backend, prompt_tokens):
+    """A chunk of more rows than a step's (a driver created with room for them): the projections run in windows of 256
+    rows around one chunked attention over all the rows, layer by layer. The pools and the hidden rows are those of
+    the sixteen-row blocks run one step after the other, bit for bit."""
+    print(f"case long prompt chunk tokens={prompt_tokens}", flush=True)
+    model = DenseModel(seed=23, hidden=1024, q_heads=16, kv_heads=8, head_dim=64, ffn=3072, vocabulary=32000, layers=3)
+    rng = np.random.default_rng(8)
+    gpu = model.build_gpu(backend, max_lanes=1, context_tokens=[prompt_tokens + 300], prefill_rows=1024)
+    model.seed_context(gpu, None, rng)
+    first, committed = model.table_first[0], 250
+    prompt = rng.integers(0, 32000, prompt_tokens).astype(np.uint32)
+    blocks = [(at, min(16, prompt_tokens - at)) for at in range(0, prompt_tokens, 16)]
+    pools = lambda: np.concatenate([gpu.buffer(verify.KV_POOL, layer).download(np.uint8) for layer in range(3)])
+    start = pools()
+    hidden = []
+    for at, rows in blocks:
+        lane = verify.Lane(rows, committed + at, table_first=first)
+        gpu.set_block([lane], prompt[at:at + rows])
+        backend.run(gpu.encode([lane], commit=False))
+        hidden.append(gpu.buffer(verify.HIDDEN, 0).download(np.uint16, rows * 1024).copy())
+    want_pools, want_hidden = pools(), np.concatenate(hidden)
+    for layer in range(3):
+        gpu.buffer(verify.KV_POOL, layer).upload(start.reshape(3, -1)[layer])
+    graph = gpu.encode_prefill(first, committed, prompt_tokens)
+    gpu.set_prefill_block(prompt)
+    backend.run(graph)
+    assert np.array_equal(pools(), want_pools)
+    assert np.array_equal(gpu.buffer(verify.HIDDEN, 0).download(np.uint16, prompt_tokens * 1024), want_hidden)
+    with pytest.raises(ValueError):
+        gpu.encode_prefill(first, committed, 1025)
+
+
 def test_eight_lanes_equal_each_lane_alone(backend):
     """The driver's most lanes: eight lanes of unequal blocks and histories in one step give, lane by lane, the logits,
     selections and acceptance each lane gives alone, bit for bit."""
