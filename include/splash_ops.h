@@ -240,6 +240,15 @@ sp_status spo_embedding_add(spo_graph *graph, uint32_t format, sp_buffer *native
 sp_status spo_row_copy_add(spo_graph *graph, sp_buffer *source, uint32_t from_row, uint32_t from_stride, uint32_t from_column,
                            sp_buffer *destination, uint32_t to_row, uint32_t to_stride, uint32_t to_column, uint32_t rows,
                            uint32_t width);
+/* The fp32 projection of weights kept as rows (addGgufFloat, LinearGguf.cpp:545-612; kernels/shared/gguf_float.metal): a
+ * MoE router, or the GDN alpha/beta gates of a GGUF that keeps them F32. weight_rows: [output_size][input_size] F32, or
+ * BF16 with bf16_weights; input: bf16 [rows][input_size], input_size a multiple of 8; output row r's columns
+ * [out_offset, out_offset + output_size) of out_stride values, fp32 with float32_output, else rounded to bf16. Every
+ * operand is exact in fp32; a sum's order is fixed (four chains by k mod 4, then (c0 + c1) + (c2 + c3)), so a row's
+ * result depends on no other row. */
+sp_status spo_float_projection_add(spo_graph *graph, sp_buffer *input, sp_buffer *weight_rows, uint32_t output_size,
+                                   uint32_t input_size, uint32_t bf16_weights, sp_buffer *output, uint32_t rows,
+                                   uint32_t out_stride, uint32_t out_offset, uint32_t float32_output);
 typedef struct spo_rope_sequence { uint32_t first_row, rows, anchor; } spo_rope_sequence;
 sp_status spo_rope_add_tree_tables(spo_graph *graph, sp_buffer *inverse_frequency, sp_buffer *depth, sp_buffer *cosines,
                                    sp_buffer *sines, uint32_t pairs, const spo_rope_sequence *sequences, uint32_t count);

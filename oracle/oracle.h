@@ -96,6 +96,11 @@ float orc_silu(float x);
 // ---- glue ----
 // bf16((x * rsqrt(sum x^2 / W + 1e-6)) * w) per row (normalization.metal:59-99).
 void orc_rms_norm(const uint16_t *x, const uint16_t *w, uint32_t rows, uint32_t width, uint16_t *out);
+// The fp32 projection of weights kept as rows (gguf_float.metal:1-8): x bf16 [rows][k], w F32 (or BF16) [n][k], out fp32
+// [rows][n]; four chains of fused multiply-adds by k mod 4, added (c0 + c1) + (c2 + c3). Pinned by the fp64 product
+// (it differs by fp32 accumulation only), by BF16 weights giving the bits of their F32 values, and by sums that only
+// this order gives exactly (tests/test_oracle_glue.py).
+void orc_float_projection(const uint16_t *x, const void *w, uint32_t bf16_weights, uint32_t rows, uint32_t n, uint32_t k, float *out);
 // Token gather from native rows: bf16(decode(table[token][dim])), token >= vocab -> 0 (embedding.metal:10-18).
 int orc_embed(uint32_t fmt, const uint8_t *table, uint32_t vocab, uint32_t hidden, const uint32_t *tokens,
               uint32_t rows, uint16_t *out);

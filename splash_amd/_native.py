@@ -281,6 +281,7 @@ _sig("spo_norm_add_rms", c_int, c_p, c_p, c_p, c_p, c_u32, c_u32)
 _sig("spo_norm_add_rms_table", c_int, c_p, c_p, c_p, c_p, c_p, c_u32, c_u32)
 _sig("spo_embedding_add", c_int, c_p, c_u32, c_p, c_u32, c_u32, c_p, c_p, c_u32)
 _sig("spo_rope_add_tree_tables", c_int, c_p, c_p, c_p, c_p, c_p, c_u32, P(RopeSequence), c_u32)
+_sig("spo_float_projection_add", c_int, c_p, c_p, c_p, c_u32, c_u32, c_u32, c_p, c_u32, c_u32, c_u32, c_u32)
 _sig("spo_gdn_layout", c_int, P(GdnShape), c_u32, P(GdnStateStrides), P(c_u64), P(c_u64))
 _sig("spo_gdn_add_decode", c_int, c_p, P(GdnDecodeBuffers), P(GdnShape), c_u32, P(GdnStateStrides), c_u32, P(GdnLane), c_u32)
 _sig("spo_gdn_add_prefill", c_int, c_p, P(GdnPrefillBuffers), P(GdnShape), c_u32, c_u32, P(GdnStateStrides), c_u32, P(GdnPrefillCapture), c_u32)

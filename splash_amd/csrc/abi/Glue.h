@@ -35,7 +35,23 @@ struct RowCopyParams {
   uint32_t to_row, to_stride, to_column;
 };
 
+// gguf_float_<f32|bf16>_<f32|bf16>: the fp32 projection of weights kept as rows (the reference's GgufFloatParams,
+// abi/Gguf.h:204, kernels/shared/gguf_float.metal): out[r][out_offset + n] = sum_k x[r][k] W[n][k], x the bf16 rows,
+// W F32 or BF16 rows as stored, every operand exact in fp32. A sum runs four chains of fused multiply-adds, chain j
+// over the inputs k = j mod 4 in ascending order, and adds them as (c0 + c1) + (c2 + c3): it depends neither on the
+// grid nor on the row count. Grid (ceil(output_size / 16), ceil(rows / 16)), 256 threads: a thread an output.
+#define GGUF_FLOAT_STEP 64u   // inputs a workgroup stages at a time
+struct GgufFloatParams {
+  uint32_t rows;
+  uint32_t input_size;   // K, a multiple of 8
+  uint32_t output_size;  // N
+  uint32_t out_stride;   // values of a destination row
+  uint32_t out_offset;   // the projection's first column in it
+  uint32_t reserved[3];
+};
+
 #ifdef __cplusplus
+static_assert(sizeof(GgufFloatParams) == 32, "float projection parameters are 32 bytes on both sides");
 static_assert(sizeof(RowCopyParams) == 32, "row copy parameters are 32 bytes on both sides");
 static_assert(sizeof(NormParams) == 16, "norm parameters are 16 bytes on both sides");
 static_assert(sizeof(RopeTreeParams) == 112, "RoPE tree parameters are 112 bytes on both sides");

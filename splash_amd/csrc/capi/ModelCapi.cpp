@@ -77,6 +77,16 @@ sp_status spo_rope_add_tree_tables(spo_graph *graph, sp_buffer *inverse_frequenc
   });
 }
 
+sp_status spo_float_projection_add(spo_graph *graph, sp_buffer *input, sp_buffer *weight_rows, uint32_t output_size, uint32_t input_size,
+                                   uint32_t bf16_weights, sp_buffer *output, uint32_t rows, uint32_t out_stride, uint32_t out_offset,
+                                   uint32_t float32_output) {
+  return capi::guard([&] {
+    capi::require(graph, "graph");
+    ops::FloatProjection::add(capi::graphOf(graph), B(input), ops::FloatRows{B(weight_rows), output_size, input_size, bf16_weights != 0},
+                              B(output), rows, out_stride, out_offset, float32_output ? ops::FloatOutput::Float32 : ops::FloatOutput::BFloat16);
+  });
+}
+
 sp_status spo_sampling_workspace(uint32_t rows, uint64_t sizes[5]) {
   return capi::guard([&] {
     capi::require(sizes, "result");

@@ -143,6 +143,56 @@ __global__ void rope_build_tree_tables(const float *__restrict__ inverse_frequen
 }
 SP_REGISTER_KERNEL("rope_build_tree_tables", &rope_build_tree_tables);
 
+// gguf_float_<weights>_<output>: the fp32 projection of weights kept as rows (abi/Glue.h; the reference's
+// kernels/shared/gguf_float.metal): a workgroup owns 16 rows x 16 columns and walks K in steps of 64 inputs staged in
+// LDS (the rows' bf16 values widened, the weights as stored or widened: every operand exact in fp32); thread (r, c)
+// runs the four chains of its output. The weights' rows are padded by one word in LDS so that the sixteen columns a
+// half-wave reads at one input fall in sixteen banks.
+template <bool kBf16Weights, bool kBf16Output>
+__global__ __launch_bounds__(256) void gguf_float(const uint16_t *__restrict__ input, const void *__restrict__ weights,
+                                                   void *__restrict__ output, GgufFloatParams p) {
+  constexpr uint32_t S = GGUF_FLOAT_STEP;
+  __shared__ float xs[16][S], ws[16][S + 1];
+  const uint32_t tid = threadIdx.x, c = tid & 15u, r = tid >> 4;
+  const uint32_t column0 = blockIdx.x * 16u, row0 = blockIdx.y * 16u, K = p.input_size;
+  float chain[4] = {0.f, 0.f, 0.f, 0.f};
+  for (uint32_t k0 = 0; k0 < K; k0 += S) {
+    // stage: thread t the four inputs 4 (t % 16) .. of row / column t / 16; zeros past the rows, the columns and K
+    {
+      const uint32_t line = tid >> 4, at = (tid & 15u) * 4u;
+#pragma unroll
+      for (uint32_t i = 0; i < 4; ++i) {
+        const uint32_t k = k0 + at + i;
+        const bool inside = k < K;
+        float x = 0.f, w = 0.f;
+        if (inside && row0 + line < p.rows) x = bf16_bits_to_float(input[size_t(row0 + line) * K + k]);
+        if (inside && column0 + line < p.output_size) {
+          if constexpr (kBf16Weights) w = bf16_bits_to_float(static_cast<const uint16_t *>(weights)[size_t(column0 + line) * K + k]);
+          else w = static_cast<const float *>(weights)[size_t(column0 + line) * K + k];
+        }
+        xs[line][at + i] = x;
+        ws[line][at + i] = w;
+      }
+    }
+    __syncthreads();
+#pragma unroll 4
+    for (uint32_t k = 0; k < S; k += 4) {
+#pragma unroll
+      for (uint32_t j = 0; j < 4; ++j) chain[j] = __builtin_fmaf(xs[r][k + j], ws[c][k + j], chain[j]);
+    }
+    __syncthreads();
+  }
+  const float sum = (chain[0] + chain[1]) + (chain[2] + chain[3]);
+  if (row0 + r >= p.rows || column0 + c >= p.output_size) return;
+  const size_t at = size_t(row0 + r) * p.out_stride + p.out_offset + column0 + c;
+  if constexpr (kBf16Output) static_cast<uint16_t *>(output)[at] = uint16_t(float_to_bf16_bits(sum));
+  else static_cast<float *>(output)[at] = sum;
+}
+SP_REGISTER_KERNEL("gguf_float_f32_f32", (&gguf_float<false, false>));
+SP_REGISTER_KERNEL("gguf_float_f32_bf16", (&gguf_float<false, true>));
+SP_REGISTER_KERNEL("gguf_float_bf16_f32", (&gguf_float<true, false>));
+SP_REGISTER_KERNEL("gguf_float_bf16_bf16", (&gguf_float<true, true>));
+
 // gguf_embed_<fmt>: out[r][:] = bf16(decode(native row tokens[r])); a token at or past the
 // vocabulary gives zeros (embedding.metal:10-18). Grid (rows, hidden / 256), 64 threads: a thread
 // decodes four values of a super-block.

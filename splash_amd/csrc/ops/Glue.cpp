@@ -45,6 +45,19 @@ void Embedding::add(hip::CommandGraph &graph, const EmbeddingTable &table, const
             GgufEmbedParams{rows, table.vocabulary, table.hidden}, {rows, table.hidden / GGUF_BLOCK, 1}, {64, 1, 1});
 }
 
+void FloatProjection::add(hip::CommandGraph &graph, const hip::Buffer &input, const FloatRows &w, const hip::Buffer &output, uint32_t rows,
+                          uint32_t outStride, uint32_t outOffset, FloatOutput type) {
+  if (!rows || !w.inputSize || w.inputSize % 8 || !w.outputSize || uint64_t{outOffset} + w.outputSize > outStride)
+    throw std::invalid_argument("invalid float projection");
+  requireBytes(w.rows, w.weightBytes(), "float projection weight");
+  requireBytes(input, uint64_t{rows} * w.inputSize * 2, "float projection input");
+  const uint64_t element = type == FloatOutput::Float32 ? 4 : 2;
+  requireBytes(output, (uint64_t{rows - 1} * outStride + outOffset + w.outputSize) * element, "float projection output");
+  graph.add(std::string("gguf_float_") + (w.bfloat16 ? "bf16" : "f32") + (type == FloatOutput::Float32 ? "_f32" : "_bf16"),
+            {input, w.rows, output}, GgufFloatParams{rows, w.inputSize, w.outputSize, outStride, outOffset, {}},
+            {(w.outputSize + 15) / 16, (rows + 15) / 16, 1}, {256, 1, 1});
+}
+
 void RoPE::addTreeTables(hip::CommandGraph &graph, const hip::Buffer &inverseFrequency, const hip::Buffer &depth,
                          const hip::Buffer &cosines, const hip::Buffer &sines, uint32_t pairs,
                          const std::vector<RopeSequence> &sequences) {

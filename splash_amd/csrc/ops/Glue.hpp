@@ -35,6 +35,14 @@ public:
                   uint32_t rows);
 };
 
+// The fp32 projection of weights kept as rows (the reference's addGgufFloat, LinearGguf.cpp:545-612): output row r's
+// columns [outOffset, outOffset + N) of outStride = sum_k x[r][k] W[n][k], fp32 or rounded to bf16.
+class FloatProjection final {
+public:
+  static void add(hip::CommandGraph &graph, const hip::Buffer &input, const FloatRows &weights, const hip::Buffer &output,
+                  uint32_t rows, uint32_t outStride, uint32_t outOffset, FloatOutput type);
+};
+
 struct RopeSequence final {
   uint32_t firstRow = 0, rows = 0, anchor = 0;
 };

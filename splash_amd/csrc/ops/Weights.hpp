@@ -36,6 +36,18 @@ struct QuantizedSegment final {
   [[nodiscard]] const char *name() const noexcept { return gguf_format_name(formatId); }
 };
 
+// Weights kept as rows of floats, [outputSize][inputSize] F32 or BF16 as their file stores them, which the fp32
+// projection reads (the reference's float segments, Weights.hpp:108-160 isFloat; a MoE router, the GDN alpha/beta
+// gates of a GGUF that keeps them F32).
+struct FloatRows final {
+  hip::Buffer rows;
+  uint32_t outputSize = 0;
+  uint32_t inputSize = 0;
+  bool bfloat16 = false;
+  [[nodiscard]] explicit operator bool() const noexcept { return static_cast<bool>(rows); }
+  [[nodiscard]] uint64_t weightBytes() const noexcept { return uint64_t{outputSize} * inputSize * (bfloat16 ? 2 : 4); }
+};
+
 struct BlockWeights final {
   std::vector<QuantizedSegment> segments;
 };

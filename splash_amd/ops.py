@@ -397,6 +397,17 @@ class PagedAttention:
         graph._keep.extend([plan, retained, pages])
 
 
+class FloatProjection:
+    """ops::FloatProjection: the fp32 projection of weights kept as F32 or BF16 rows."""
+
+    @staticmethod
+    def add(graph, input, weight_rows, output_size, input_size, output, rows, out_stride=None, out_offset=0, bf16_weights=False,
+            float32_output=True):
+        check(lib.spo_float_projection_add(graph.handle, input.handle, weight_rows.handle, output_size, input_size, int(bf16_weights),
+                                           output.handle, rows, out_stride or output_size, out_offset, int(float32_output)))
+        graph._keep.extend([input, weight_rows, output])
+
+
 class StateCodec:
     """ops::StateCodec: a running state's recurrent layers as int8 codes with a bf16 scale per block of 32 values."""
 

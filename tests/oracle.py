@@ -131,6 +131,21 @@ def gemv_column(fmt, native, x_bf16, N, threads=0):
     return out
 
 
+lib.orc_float_projection.restype = None
+lib.orc_float_projection.argtypes = [u16p, ctypes.c_void_p, c_u32, c_u32, c_u32, c_u32, f32p]
+
+
+def float_projection(x_bits, weights):
+    """fp32 [rows][n] = x (bf16 bits [rows][k]) times weights^T; weights float32 [n][k], or uint16 bf16 bits."""
+    x = np.ascontiguousarray(x_bits, np.uint16)
+    w = np.ascontiguousarray(weights)
+    assert w.dtype in (np.float32, np.uint16) and w.shape[1] == x.shape[1]
+    out = np.zeros((x.shape[0], w.shape[0]), np.float32)
+    lib.orc_float_projection(_p(x, u16p), w.ctypes.data_as(ctypes.c_void_p), int(w.dtype == np.uint16), x.shape[0], w.shape[0], w.shape[1],
+                             _p(out, f32p))
+    return out
+
+
 def rms_norm(x_bf16, w_bf16):
     x = np.ascontiguousarray(x_bf16, dtype=np.uint16)
     w = np.ascontiguousarray(w_bf16, dtype=np.uint16)

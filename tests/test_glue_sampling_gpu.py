@@ -39,6 +39,38 @@ def test_rms_norm_and_its_activation_table(backend, rows, width):
     assert np.array_equal(table.download(), table2.download())
 
 
+@pytest.mark.parametrize("rows,n,k,bf16_weights", [(130, 128, 2048, False), (1, 7, 8, False), (33, 64, 2048, True), (16, 250, 1000, False)])
+def test_float_projection_equals_the_oracle(backend, rows, n, k, bf16_weights):
+    """kernels/shared/gguf_float.metal: the fp32 projection of weights kept as rows, bit for bit the oracle's fixed
+    order; a row alone gives its bits of the batch; the bf16 destination is the fp32 result rounded once, written at
+    its columns of a wider row that it otherwise leaves alone (the GDN alpha/beta columns of a packed row)."""
+    print(f"case float projection rows={rows} n={n} k={k} bf16={bf16_weights}", flush=True)
+    rng = np.random.default_rng(rows + n)
+    x = orc.f32_to_bf16((rng.standard_normal((rows, k)) * 2).astype(np.float32))
+    w = (rng.standard_normal((n, k)) * 0.05).astype(np.float32)
+    weights = orc.f32_to_bf16(w) if bf16_weights else w
+    want = orc.float_projection(x, weights)
+    xb, wb = backend.from_array(x), backend.from_array(weights)
+    out = backend.allocate_buffer(rows * n * 4)
+    stride, offset = n + 24, 16
+    before = orc.f32_to_bf16(rng.standard_normal((rows, stride)).astype(np.float32))
+    packed = backend.from_array(before)
+    alone = backend.allocate_buffer(n * 4)
+    g = splash_amd.CommandGraph()
+    ops.FloatProjection.add(g, xb, wb, n, k, out, rows, bf16_weights=bf16_weights)
+    ops.FloatProjection.add(g, xb, wb, n, k, packed, rows, out_stride=stride, out_offset=offset, bf16_weights=bf16_weights, float32_output=False)
+    ops.FloatProjection.add(g, backend.from_array(x[rows - 1:]), wb, n, k, alone, 1, bf16_weights=bf16_weights)
+    backend.run(g)
+    got = out.download(np.float32).reshape(rows, n)
+    assert got.tobytes() == want.tobytes()
+    assert alone.download(np.float32).tobytes() == want[rows - 1].tobytes()
+    rows_out = packed.download(np.uint16).reshape(rows, stride)
+    assert np.array_equal(rows_out[:, offset:offset + n], orc.f32_to_bf16(want))
+    assert np.array_equal(rows_out[:, :offset], before[:, :offset]) and np.array_equal(rows_out[:, offset + n:], before[:, offset + n:])
+    with pytest.raises(ValueError):
+        ops.FloatProjection.add(splash_amd.CommandGraph(), xb, wb, n, k, packed, rows, out_stride=n, out_offset=8, float32_output=False)
+
+
 @pytest.mark.parametrize("fmt", ops.FORMATS)
 def test_embedding_gathers_native_rows(backend, fmt):
     """embedding.metal:10-18: bf16(decode(row)); a token past the vocabulary gives zeros."""

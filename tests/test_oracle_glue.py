@@ -246,3 +246,39 @@ def test_embedding_rows_are_the_golden_dequantization_rounded_to_bf16():
         for r, t in enumerate(tokens):
             want = orc.f32_to_bf16(values[t]) if t < vocab else np.zeros(hidden, np.uint16)   # a token past the table reads zeros
             assert np.array_equal(got[r], want), (fmt, r)
+
+
+# ------------------------------------------------------------------ float projection (gguf_float.metal:1-8)
+def test_float_projection_differs_from_the_fp64_product_by_fp32_accumulation_only():
+    rng = np.random.default_rng(17)
+    for rows, n, k in ((5, 24, 2048), (1, 7, 8), (33, 130, 200)):
+        x = _bits(rng.standard_normal((rows, k)) * 3)
+        w = (rng.standard_normal((n, k)) * 0.05).astype(np.float32)
+        got = orc.float_projection(x, w).astype(np.float64)
+        xf = orc.bf16_to_f32(x).astype(np.float64)
+        want = xf @ w.astype(np.float64).T
+        bound = 2.0 ** -24 * (k / 4 + 3) * (np.abs(xf) @ np.abs(w.astype(np.float64)).T)   # a chain of k / 4 sums, then two more
+        assert np.all(np.abs(got - want) <= bound + 1e-30), (rows, n, k)
+        # BF16 weights give the bits of the F32 tensor of their values
+        wb = _bits(w)
+        assert orc.float_projection(x, wb).tobytes() == orc.float_projection(x, orc.bf16_to_f32(wb)).tobytes()
+
+
+def test_float_projection_adds_in_four_chains_by_input_modulo_four():
+    """Sums only this order gives: 2^24 in chain 0 swallows the ones of chain 0 and not those of the other chains; a
+    sequential sum, or pairs of neighbours, would give other values."""
+    k = 16
+    x = _bits(np.ones((1, k)))
+    w = np.ones((1, k), np.float32)
+    w[0, 0] = 2.0 ** 24
+    # chain 0: 2^24 + 1 + 1 + 1 rounds to 2^24 each time; chains 1..3: 4 each; (2^24 + 4) + 8 = 2^24 + 12
+    assert orc.float_projection(x, w)[0, 0] == np.float32(2.0 ** 24 + 12)
+    w[0, 0], w[0, 13] = 1.0, 2.0 ** 24
+    # chain 1 now ends with 2^24: 3 + 2^24 is exact; (4 + (2^24 + 3)) -> 2^24 + 8 (ties to even), then + 8
+    assert orc.float_projection(x, w)[0, 0] == np.float32(np.float32(np.float32(4) + np.float32(2.0 ** 24 + 3)) + np.float32(8))
+    # fused multiply-adds: a product's low bits reach the sum
+    x2 = _bits(np.array([[1 + 2.0 ** -7, 1.0, 0, 0, 0, 0, 0, 0]]))
+    w2 = np.array([[1 + 2.0 ** -20, -1.0, 0, 0, 0, 0, 0, 0]], np.float32)
+    exact = (1 + 2.0 ** -7) * (1 + 2.0 ** -20) - 1.0
+    assert orc.float_projection(x2, w2)[0, 0] == np.float32(np.float32((1 + 2.0 ** -7) * (1 + 2.0 ** -20)) + np.float32(-1.0))
+    assert abs(float(orc.float_projection(x2, w2)[0, 0]) - exact) <= 2.0 ** -24
