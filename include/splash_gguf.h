@@ -69,6 +69,22 @@ sp_status spg_load_bf16(sp_backend *backend, const spg_file *file, uint64_t inde
 sp_status spg_dense_dimensions(const spg_file *file, spo_dense_dimensions *out);
 sp_status spo_dense_verify_load_gguf(spo_dense_verify *verify, const spg_file *file);
 
+/* A hybrid decoder from a file (the reference's HybridGguf family: architectures qwen35 and qwen35moe, GgufImage.cpp:474-520
+ * mixerImage and ffnImage, :541-557, :874-936). spg_hybrid_dimensions reads the geometry: the dense driver's keys, and
+ * full_attention_interval, ssm.group_count (key heads), ssm.time_step_rank (value heads), ssm.state_size (128),
+ * ssm.conv_kernel (4), ssm.inner_size, expert_count, expert_used_count, expert_feed_forward_length and
+ * expert_shared_feed_forward_length, or without experts feed_forward_length; block_count less nextn_predict_layers
+ * layers; gated attention when attn_q holds two rows a query dimension. spo_hybrid_verify_load_gguf loads a driver
+ * created with those dimensions: an attention layer's attn_q | attn_k | attn_v, head norms and attn_output; a Gated
+ * DeltaNet layer's attn_qkv | attn_gate with the value heads' rows regrouped by key head (llama.cpp stores them tiled,
+ * GgufImage.hpp:29-38), ssm_beta and ssm_alpha as rows of floats the fp32 projection runs, ssm_conv1d, ssm_a, ssm_dt.bias,
+ * ssm_norm (fp32) and ssm_out, whose input columns keep the file's order (the driver's GDN rows then leave tiled);
+ * ffn_gate_inp as rows of floats, the routed experts of ffn_gate_exps and ffn_up_exps (or the fused ffn_gate_up_exps)
+ * and ffn_down_exps an image an expert, the shared expert's slices after them, ffn_gate_inp_shexp; or a dense SwiGLU.
+ * Errors as the dense loader's. */
+sp_status spg_hybrid_dimensions(const spg_file *file, spo_hybrid_dimensions *out);
+sp_status spo_hybrid_verify_load_gguf(spo_hybrid_verify *verify, const spg_file *file);
+
 #ifdef __cplusplus
 }
 #endif

@@ -315,6 +315,8 @@ _sig("spo_dense_verify_set_fused_prepare", c_int, c_p, c_int)
 _sig("spo_dense_verify_results", c_int, c_p, P(VerifyLane), c_u32, P(c_u32), P(c_u32), P(c_u32), P(c_u32))
 _sig("spg_dense_dimensions", c_int, c_p, P(DenseDimensions))
 _sig("spo_dense_verify_load_gguf", c_int, c_p, c_p)
+_sig("spg_hybrid_dimensions", c_int, c_p, P(HybridDimensions))
+_sig("spo_hybrid_verify_load_gguf", c_int, c_p, c_p)
 _sig("spo_dense_verify_create", c_int, c_p, P(DenseDimensions), c_u32, c_u32, c_u32, P(c_p))
 _sig("spo_dense_verify_create_chunked", c_int, c_p, P(DenseDimensions), c_u32, c_u32, c_u32, c_u32, P(c_p))
 _sig("spo_dense_verify_destroy", None, c_p)

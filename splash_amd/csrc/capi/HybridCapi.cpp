@@ -2,7 +2,9 @@
 #include "splash_ops.h"
 #include "capi/Guard.hpp"
 #include "capi/Handles.hpp"
+#include "model/GgufTarget.hpp"
 #include "model/HybridVerify.hpp"
+#include "splash_gguf.h"
 #include "model/StepResults.hpp"
 
 #include <memory>
@@ -64,6 +66,40 @@ sp_status spo_hybrid_verify_create(sp_backend *backend, const spo_hybrid_dimensi
   });
 }
 void spo_hybrid_verify_destroy(spo_hybrid_verify *verify) { delete verify; }
+
+sp_status spg_hybrid_dimensions(const spg_file *file, spo_hybrid_dimensions *out) {
+  return capi::guard([&] {
+    capi::require(out, "result");
+    const model::HybridDimensions d = model::ggufHybridDimensions(capi::ggufOf(file));
+    *out = {};
+    out->hidden = d.hidden;
+    out->vocabulary = d.vocabulary;
+    out->layers = d.layers;
+    out->attention_interval = d.attentionInterval;
+    out->q_heads = d.qHeads;
+    out->kv_heads = d.kvHeads;
+    out->head_dim = d.headDimension;
+    out->rotary_pairs = d.rotaryPairs;
+    out->normalize_heads = d.normalizeHeads;
+    out->gated_attention = d.gatedAttention;
+    out->rope_theta = d.ropeTheta;
+    out->gdn_key_heads = d.gdnKeyHeads;
+    out->gdn_value_heads = d.gdnValueHeads;
+    out->gdn_packed_width = d.gdnPackedWidth;
+    out->experts = d.experts;
+    out->top_k = d.topK;
+    out->expert_ffn = d.expertFfn;
+    out->shared_slices = d.sharedSlices;
+    out->shared_gate = d.sharedGate;
+    out->dense_ffn = d.denseFfn;
+  });
+}
+sp_status spo_hybrid_verify_load_gguf(spo_hybrid_verify *verify, const spg_file *file) {
+  return capi::guard([&] {
+    capi::require(verify, "verify");
+    model::loadGgufHybridWeights(*verify->backend, capi::ggufOf(file), *verify->verify);
+  });
+}
 
 sp_status spo_hybrid_verify_set_layer(spo_hybrid_verify *verify, uint32_t layer, const spo_hybrid_layer *l) {
   return capi::guard([&] {

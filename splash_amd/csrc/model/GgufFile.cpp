@@ -266,6 +266,162 @@ LoadedImage loadImage(hip::Backend &backend, const GgufFile &file, const GgufTen
   return out;
 }
 
+RowRuns groupedHeadRows(uint64_t rows, uint64_t from, uint32_t headRows, uint32_t keyHeads, uint32_t valueHeadsPerKey) {
+  if (!headRows || !keyHeads || !valueHeadsPerKey || from > rows || (rows - from) != uint64_t{keyHeads} * valueHeadsPerKey * headRows)
+    throw std::invalid_argument("the rows past `from` are the value heads' rows");
+  RowRuns runs;
+  if (from) runs.push_back({0, from});
+  for (uint32_t h = 0; h < keyHeads; ++h)
+    for (uint32_t j = 0; j < valueHeadsPerKey; ++j) runs.push_back({from + (uint64_t{j} * keyHeads + h) * headRows, headRows});
+  return runs;
+}
+
+namespace {
+uint64_t runRows(const RowRuns &runs, uint64_t all) {
+  if (runs.empty()) return all;
+  uint64_t rows = 0;
+  for (const RowRun &run : runs) {
+    if (!run.rows || run.first > all || run.rows > all - run.first) throw std::invalid_argument("a run of rows lies past the tensor");
+    rows += run.rows;
+  }
+  return rows;
+}
+// The native rows of `runs`, columns [firstColumn, firstColumn + columns) of each, one after the other.
+std::vector<uint8_t> gatherNative(const GgufFile &file, const GgufTensor &tensor, uint32_t format, const RowRuns &runs, uint64_t firstColumn,
+                                  uint64_t columns) {
+  const uint64_t all = tensor.rows(), width = tensor.columns();
+  const uint64_t blockBytes = gguf_native_bytes(format), rowBytes = width / GGUF_BLOCK * blockBytes;
+  const uint64_t piece = columns / GGUF_BLOCK * blockBytes, skip = firstColumn / GGUF_BLOCK * blockBytes;
+  std::vector<uint8_t> native(runRows(runs, all) * piece);
+  const uint8_t *data = file.data(tensor);
+  uint64_t at = 0;
+  auto take = [&](uint64_t first, uint64_t rows) {
+    for (uint64_t r = 0; r < rows; ++r, at += piece) std::memcpy(native.data() + at, data + (first + r) * rowBytes + skip, piece);
+  };
+  if (runs.empty()) take(0, all);
+  for (const RowRun &run : runs) take(run.first, run.rows);
+  return native;
+}
+} // namespace
+
+PackedImages packImagesOfRows(const GgufFile &file, const GgufTensor &tensor, const std::vector<RowRuns> &images, uint64_t firstColumn,
+                              uint64_t columns) {
+  const std::optional<uint32_t> format = imageFormat(tensor.type);
+  if (!format) throw std::invalid_argument("tensor " + tensor.name + " is not of a projection format");
+  if (images.empty()) throw std::invalid_argument("no rows to load of " + tensor.name);
+  const uint64_t width = tensor.columns();
+  if (!columns) columns = width - std::min(width, firstColumn);
+  if (!columns || firstColumn % GGUF_BLOCK || columns % GGUF_BLOCK || firstColumn + columns > width || columns > UINT32_MAX)
+    throw std::invalid_argument("a weight image holds whole 256-input super-blocks: " + tensor.name);
+  const uint64_t rows = runRows(images.front(), tensor.rows());
+  if (!rows || rows % GGUF_TILE_COLUMNS || rows > UINT32_MAX) throw std::invalid_argument("a weight image holds whole 16-row tiles: " + tensor.name);
+  const uint64_t imageBytes = gguf_image_bytes(*format, uint32_t(rows), uint32_t(columns));
+  std::vector<uint8_t> packed(imageBytes * images.size());
+  for (size_t i = 0; i < images.size(); ++i) {
+    if (runRows(images[i], tensor.rows()) != rows) throw std::invalid_argument("the images of " + tensor.name + " hold the same rows each");
+    const std::vector<uint8_t> native = gatherNative(file, tensor, *format, images[i], firstColumn, columns);
+    ops::packGgufImage(*format, native.data(), uint32_t(rows), uint32_t(columns), packed.data() + i * imageBytes);
+  }
+  return {*format, uint32_t(rows), uint32_t(columns), std::move(packed)};
+}
+
+LoadedImage loadImagesOfRows(hip::Backend &backend, const GgufFile &file, const GgufTensor &tensor, const std::vector<RowRuns> &images,
+                             uint64_t firstColumn, uint64_t columns) {
+  const PackedImages packed = packImagesOfRows(file, tensor, images, firstColumn, columns);
+  LoadedImage out;
+  out.formatId = packed.formatId;
+  out.rows = packed.rows;
+  out.inputSize = packed.inputSize;
+  out.image = backend.allocateBuffer(packed.bytes.size(), hip::BufferStorage::Private, tensor.name.c_str());
+  out.image.upload(packed.bytes.data(), packed.bytes.size());
+  return out;
+}
+
+LoadedImage loadImageRows(hip::Backend &backend, const GgufFile &file, const GgufTensor &tensor, const RowRuns &runs, uint64_t firstColumn,
+                          uint64_t columns) {
+  return loadImagesOfRows(backend, file, tensor, {runs}, firstColumn, columns);
+}
+
+namespace {
+bool floatTensor(uint32_t type) { return type == ggml::kF32 || type == ggml::kF16 || type == ggml::kBF16; }
+uint32_t elementBytes(uint32_t type) { return type == ggml::kF32 ? 4 : 2; }
+float floatAt(const uint8_t *data, uint32_t type, uint64_t i) {
+  if (type == ggml::kF32) {
+    float f;
+    std::memcpy(&f, data + 4 * i, 4);
+    return f;
+  }
+  uint16_t h;
+  std::memcpy(&h, data + 2 * i, 2);
+  if (type == ggml::kF16) return halfToFloat(h);
+  const uint32_t bits = uint32_t{h} << 16;
+  float f;
+  std::memcpy(&f, &bits, 4);
+  return f;
+}
+// The fp32 values of `runs` of a float tensor.
+std::vector<float> gatherFloats(const GgufFile &file, const GgufTensor &tensor, const RowRuns &runs) {
+  if (!floatTensor(tensor.type)) throw std::invalid_argument("tensor " + tensor.name + " does not hold 16- or 32-bit floats");
+  // a vector's runs are runs of its values
+  const bool vector = tensor.dims.size() == 1;
+  const uint64_t all = vector ? tensor.columns() : tensor.rows(), width = vector ? 1 : tensor.columns();
+  std::vector<float> values;
+  values.reserve(runRows(runs, all) * width);
+  const uint8_t *data = file.data(tensor);
+  auto take = [&](uint64_t first, uint64_t rows) {
+    for (uint64_t i = first * width; i < (first + rows) * width; ++i) values.push_back(floatAt(data, tensor.type, i));
+  };
+  if (runs.empty()) take(0, all);
+  for (const RowRun &run : runs) take(run.first, run.rows);
+  return values;
+}
+} // namespace
+
+LoadedFloatRows loadFloatRows(hip::Backend &backend, const GgufFile &file, const std::vector<const GgufTensor *> &tensors, const RowRuns &runs) {
+  if (tensors.empty() || !tensors.front()) throw std::invalid_argument("no float rows to load");
+  const uint64_t width = tensors.front()->columns();
+  bool bfloat16 = true;
+  for (const GgufTensor *t : tensors) {
+    if (!t || !floatTensor(t->type) || t->columns() != width) throw std::invalid_argument("float rows of one width");
+    bfloat16 = bfloat16 && t->type == ggml::kBF16;
+  }
+  LoadedFloatRows out;
+  out.inputSize = uint32_t(width);
+  out.bfloat16 = bfloat16;
+  std::vector<uint8_t> bytes;
+  for (const GgufTensor *t : tensors) {
+    const std::vector<float> values = gatherFloats(file, *t, runs);
+    out.outputSize += uint32_t(values.size() / width);
+    for (float v : values) {
+      if (bfloat16) {
+        const uint16_t b = floatToBf16(v);  // exact: the value is a bf16's
+        bytes.insert(bytes.end(), reinterpret_cast<const uint8_t *>(&b), reinterpret_cast<const uint8_t *>(&b) + 2);
+      } else {
+        bytes.insert(bytes.end(), reinterpret_cast<const uint8_t *>(&v), reinterpret_cast<const uint8_t *>(&v) + 4);
+      }
+    }
+  }
+  out.rows = backend.allocateBuffer(std::max<uint64_t>(bytes.size(), 16), hip::BufferStorage::Private, tensors.front()->name.c_str());
+  out.rows.upload(bytes.data(), bytes.size());
+  return out;
+}
+
+hip::Buffer loadFloat32Values(hip::Backend &backend, const GgufFile &file, const GgufTensor &tensor, const RowRuns &runs) {
+  const std::vector<float> values = gatherFloats(file, tensor, runs);
+  hip::Buffer out = backend.allocateBuffer(std::max<uint64_t>(values.size() * 4, 16), hip::BufferStorage::Private, tensor.name.c_str());
+  out.upload(values.data(), values.size() * 4);
+  return out;
+}
+
+hip::Buffer loadBf16Values(hip::Backend &backend, const GgufFile &file, const GgufTensor &tensor, const RowRuns &runs) {
+  const std::vector<float> values = gatherFloats(file, tensor, runs);
+  std::vector<uint16_t> bits(values.size());
+  for (size_t i = 0; i < values.size(); ++i) bits[i] = floatToBf16(values[i]);
+  hip::Buffer out = backend.allocateBuffer(std::max<uint64_t>(bits.size() * 2, 16), hip::BufferStorage::Private, tensor.name.c_str());
+  out.upload(bits.data(), bits.size() * 2);
+  return out;
+}
+
 hip::Buffer loadBf16Vector(hip::Backend &backend, const GgufFile &file, const GgufTensor &tensor) {
   if (tensor.type != ggml::kF32 && tensor.type != ggml::kF16 && tensor.type != ggml::kBF16)
     throw std::invalid_argument("tensor " + tensor.name + " is not a 16- or 32-bit float vector");

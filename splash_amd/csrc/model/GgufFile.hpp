@@ -104,6 +104,43 @@ struct LoadedImage {
 // whole 256-input super-blocks) and uploads them; rows = 0 takes all.
 [[nodiscard]] LoadedImage loadImage(hip::Backend &backend, const GgufFile &file, const GgufTensor &tensor, uint32_t firstRow = 0,
                                     uint32_t rows = 0);
+// The rows of a tensor an image, a table of float rows or a vector takes, in the order it takes them: runs of source
+// rows one after the other (the reference's TensorRows with its RowOrder, GgufImage.hpp:29-38). All rows when empty.
+struct RowRun final {
+  uint64_t first = 0, rows = 0;
+};
+using RowRuns = std::vector<RowRun>;
+// Value heads of `headRows` rows from row `from` on, which llama.cpp stores tiled (value head j of key head h at
+// j * keyHeads + h) and these kernels group by key head (h * valueHeadsPerKey + j): the runs that put `rows` rows of a
+// tensor in grouped order (GgufImage.hpp:29-38, GgufImage.cpp:410-413); rows below `from` keep their order.
+[[nodiscard]] RowRuns groupedHeadRows(uint64_t rows, uint64_t from, uint32_t headRows, uint32_t keyHeads, uint32_t valueHeadsPerKey);
+// The weight image of `runs` of a tensor of an image format (any rank: its rows are those of all its outer
+// dimensions), columns [firstColumn, firstColumn + columns) of each (whole super-blocks; columns 0: all), the runs'
+// rows whole 16-row tiles in all.
+[[nodiscard]] LoadedImage loadImageRows(hip::Backend &backend, const GgufFile &file, const GgufTensor &tensor, const RowRuns &runs,
+                                        uint64_t firstColumn = 0, uint64_t columns = 0);
+// The same on the host: `images` images one after the other, image i of images[i]'s rows.
+struct PackedImages {
+  uint32_t formatId = 0, rows = 0, inputSize = 0;
+  std::vector<uint8_t> bytes;
+};
+[[nodiscard]] PackedImages packImagesOfRows(const GgufFile &file, const GgufTensor &tensor, const std::vector<RowRuns> &images,
+                                            uint64_t firstColumn = 0, uint64_t columns = 0);
+// `count` images one after the other in one buffer, image i of runs[i] (a layer's experts, each expert's rows an image).
+[[nodiscard]] LoadedImage loadImagesOfRows(hip::Backend &backend, const GgufFile &file, const GgufTensor &tensor,
+                                           const std::vector<RowRuns> &images, uint64_t firstColumn = 0, uint64_t columns = 0);
+// Rows of an F32, BF16 or F16 tensor as the fp32 projection reads them: F32 and BF16 as stored, F16 widened to F32
+// (GgufImage.cpp:353-366, :372-386). bfloat16: whether the rows are BF16.
+struct LoadedFloatRows {
+  hip::Buffer rows;
+  uint32_t outputSize = 0, inputSize = 0;
+  bool bfloat16 = false;
+};
+[[nodiscard]] LoadedFloatRows loadFloatRows(hip::Backend &backend, const GgufFile &file, const std::vector<const GgufTensor *> &tensors,
+                                            const RowRuns &runs = {});
+// The values of `runs` of an F32, F16 or BF16 tensor (rows of its first dimension) as fp32, or narrowed to bf16.
+[[nodiscard]] hip::Buffer loadFloat32Values(hip::Backend &backend, const GgufFile &file, const GgufTensor &tensor, const RowRuns &runs = {});
+[[nodiscard]] hip::Buffer loadBf16Values(hip::Backend &backend, const GgufFile &file, const GgufTensor &tensor, const RowRuns &runs = {});
 // A 1-D F32, F16 or BF16 tensor as bf16 in device memory (the norms' weights).
 [[nodiscard]] hip::Buffer loadBf16Vector(hip::Backend &backend, const GgufFile &file, const GgufTensor &tensor);
 

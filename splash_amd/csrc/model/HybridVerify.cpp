@@ -122,12 +122,12 @@ uint64_t HybridVerify::stepBytes(const std::vector<HybridLane> &lanes) const {
   const ops::MoeShape moe = dims_.moeShape();
   uint64_t bytes = weights_.head.weightBytes();
   for (const HybridLayer &l : weights_.layers) {
-    bytes += l.mixerInput.weightBytes() + l.mixerOutput.weightBytes();
+    bytes += l.mixerInput.weightBytes() + l.mixerOutput.weightBytes() + l.gateRows.weightBytes();
     if (dims_.dense()) {
       bytes += l.ffnGate.weightBytes() + l.ffnUp.weightBytes() + l.ffnDown.weightBytes();
       continue;
     }
-    bytes += l.router.weightBytes();
+    bytes += l.routerRows ? l.routerRows.weightBytes() : l.router.weightBytes();
     bytes += uint64_t{moe.allExperts()} * (2 * gguf_image_bytes(l.experts.format, moe.ffn, moe.hidden) +
                                            gguf_image_bytes(l.experts.downFormat, moe.hidden, moe.ffn));
   }
@@ -173,7 +173,8 @@ void HybridVerify::encodeLayer(hip::CommandGraph &graph, uint32_t layer, const s
     throw std::invalid_argument("the layer's projections do not fit the model");
   if (dims_.dense() ? (w.ffnGate.outputSize != dims_.denseFfn || w.ffnUp.outputSize != dims_.denseFfn || w.ffnDown.inputSize != dims_.denseFfn ||
                        w.ffnGate.inputSize != dims_.hidden || w.ffnUp.inputSize != dims_.hidden || w.ffnDown.outputSize != dims_.hidden)
-                    : (w.router.outputSize != dims_.experts || w.router.inputSize != dims_.hidden))
+                    : (w.routerRows ? (w.routerRows.outputSize != dims_.experts || w.routerRows.inputSize != dims_.hidden)
+                                    : (w.router.outputSize != dims_.experts || w.router.inputSize != dims_.hidden)))
     throw std::invalid_argument("the layer's FFN does not fit the model");
 
   // Mixer: hidden[1] = hidden[0] + out(mixer(in(norm(hidden[0])))). With one piece of rows the mixer's last kernel
@@ -190,6 +191,15 @@ void HybridVerify::encodeLayer(hip::CommandGraph &graph, uint32_t layer, const s
                              : ops::Normalization::addRmsTable(graph, rowsOf(residual, first, count, hiddenBytes), w.inputNorm, normalized,
                                                                scratch_, dims_.hidden, count);
     linear_.add(graph, in, w.mixerInput, linear_.plan(w.mixerInput, count));
+    if (!attends && w.gateRows) {
+      // beta | alpha from rows of floats: the packed row's columns after q, k, v and z
+      if (inputReady) throw std::invalid_argument("float gate rows read the normalized rows, which a deferred norm does not store");
+      const ops::GdnShape shape = dims_.gdnShape();
+      if (w.gateRows.outputSize != 2 * shape.valueHeads || w.gateRows.inputSize != dims_.hidden)
+        throw std::invalid_argument("a GDN layer's gate rows are beta then alpha, a row a value head each");
+      ops::FloatProjection::add(graph, normalized, w.gateRows, in.output, count, inputWidth,
+                                shape.convolutionDimension + shape.valueHeads * GDN_HEAD_DIMENSION, ops::FloatOutput::BFloat16);
+    }
   });
   if (attends) {
     const ops::AttentionPlan plan = planOf(lanes);
@@ -205,9 +215,10 @@ void HybridVerify::encodeLayer(hip::CommandGraph &graph, uint32_t layer, const s
                        tapeOffset(uint32_t(i), lane.parity, index), cellOffset(uint32_t(i), lane.parity), cellOffset(uint32_t(i), lane.parity ^ 1u)});
       firstRow += lane.block.rows;
     }
-    ops::GdnDecodeBuffers buffers{packed_, w.convolutionWeights, states_, tape_, w.decay, w.timeBias, w.mixerNorm, false, mixed_, treeRows_,
-                                  mixerTable ? mixedTable_ : hip::Buffer{}};
-    ops::GDN::addDecode(graph, buffers, dims_.gdnShape(), index, strides_, ops::GdnHeadOrder::Grouped, steps);
+    ops::GdnDecodeBuffers buffers{packed_, w.convolutionWeights, states_, tape_, w.decay, w.timeBias, w.mixerNorm, w.mixerNormFloat, mixed_,
+                                  treeRows_, mixerTable ? mixedTable_ : hip::Buffer{}};
+    ops::GDN::addDecode(graph, buffers, dims_.gdnShape(), index, strides_,
+                        tiledGdnHeads_ ? ops::GdnHeadOrder::Tiled : ops::GdnHeadOrder::Grouped, steps);
   }
   forRowPieces(rows, [&](uint32_t first, uint32_t count) {
     ops::LinearBuffers out;
@@ -247,7 +258,10 @@ void HybridVerify::encodeLayer(hip::CommandGraph &graph, uint32_t layer, const s
     router.scratch = scratch_;
     router.prepared = ops::Normalization::addRmsTable(graph, rowsOf(next, first, count, hiddenBytes), w.postNorm, normalized, scratch_,
                                                       dims_.hidden, count);
-    linear_.add(graph, router, w.router, linear_.plan(w.router, count));
+    if (w.routerRows)
+      ops::FloatProjection::add(graph, normalized, w.routerRows, router.output, count, dims_.experts, 0, ops::FloatOutput::Float32);
+    else
+      linear_.add(graph, router, w.router, linear_.plan(w.router, count));
   });
   const ops::MoeShape moe = dims_.moeShape();
   ops::MoE::addRouting(graph, scores_, dims_.experts, moeWorkspace_, moe, rows, normalized_, w.sharedScalarGate);
@@ -298,6 +312,8 @@ void HybridVerify::encode(hip::CommandGraph &graph, const std::vector<HybridLane
   bool feeds = rows <= kProjectionRows && dims_.hidden % GGUF_BLOCK == 0;
   if (dims_.dense())
     for (const HybridLayer &l : weights_.layers) feeds = feeds && linear_.normsRows(l.ffnDown, rows);
+  // float gate rows read the normalized rows themselves, which a layer fed by the combine before it never stores
+  for (const HybridLayer &l : weights_.layers) feeds = feeds && !l.gateRows;
   for (uint32_t layer = 0; layer < dims_.layers; ++layer) encodeLayer(graph, layer, lanes, feeds && layer > 0, feeds);
   encodeHead(graph, rows, feeds);
   ops::Sampling::addVerify(graph, sampling_, dims_.vocabulary, dims_.vocabulary, laneRows, policies);

@@ -76,6 +76,12 @@ struct HybridLayer final {
   ops::Projection router;                                           // hidden -> experts, fp32 scores
   ops::MoeExperts experts;                                          // the shared slices' images after the routed experts'
   hip::Buffer sharedScalarGate;                                     // fp32 [hidden], of a gated shared expert
+  // What a GGUF keeps as rows of floats (the reference's float segments, GgufImage.cpp:262-300, :353-366), each run by
+  // the fp32 projection in place of a quantized one:
+  ops::FloatRows routerRows;   // the router [experts][hidden], instead of `router`
+  ops::FloatRows gateRows;     // a GDN layer's beta rows then alpha rows [2 value heads][hidden]: the last columns of the
+                               // packed row, which mixerInput's segments then leave out
+  bool mixerNormFloat = false; // mixerNorm holds fp32 values
 };
 
 struct HybridWeights final {
@@ -131,6 +137,11 @@ public:
   // (read and written), the logits.
   [[nodiscard]] uint64_t stepBytes(const std::vector<HybridLane> &lanes) const;
 
+  // Value head h of a GDN layer's output rows leaves at (h % heads per key) * key heads + h / heads per key, the order
+  // llama.cpp's ssm_out reads them in (GgufImage.hpp:29-32): what a model loaded from a GGUF sets. Off by default.
+  void setTiledGdnHeads(bool tiled) noexcept { tiledGdnHeads_ = tiled; }
+  [[nodiscard]] bool tiledGdnHeads() const noexcept { return tiledGdnHeads_; }
+
   void encode(hip::CommandGraph &graph, const std::vector<HybridLane> &lanes, bool commit = true);
   void encodeEmbedding(hip::CommandGraph &graph, uint32_t rows);
   // A layer (or the head) whose predecessor in the same graph left the table of its input rows, less their inverse
@@ -151,6 +162,7 @@ private:
   HybridWeights weights_;
   ops::Linear linear_;
   uint32_t maxRows_ = 0, maxLanes_ = 0;
+  bool tiledGdnHeads_ = false;
   uint64_t pageBytes_ = 0, layerBytes_ = 0, cellBytes_ = 0, tapeLayerBytes_ = 0;
   ops::GdnStateStrides strides_;
   hip::Buffer kvAll_, states_, tape_;

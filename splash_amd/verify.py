@@ -209,6 +209,21 @@ class HybridVerify:
         except Exception:
             pass
 
+    @classmethod
+    def from_gguf(cls, backend, gguf_file, max_lanes=1, physical_pages=2, page_table_entries=None):
+        """A driver of the geometry the file's metadata names (architectures qwen35 and qwen35moe), every weight loaded
+        from the file (spg_hybrid_dimensions, spo_hybrid_verify_load_gguf)."""
+        d = nat.HybridDimensions()
+        check(lib.spg_hybrid_dimensions(gguf_file.handle, ctypes.byref(d)))
+        self = cls(backend, d.hidden, d.vocabulary, d.layers, d.q_heads, d.kv_heads, d.head_dim, d.gdn_key_heads, d.gdn_value_heads, d.experts,
+                   d.top_k, d.expert_ffn, attention_interval=d.attention_interval, rotary_pairs=d.rotary_pairs,
+                   normalize_heads=bool(d.normalize_heads), rope_theta=d.rope_theta, gdn_packed_width=d.gdn_packed_width, max_lanes=max_lanes,
+                   physical_pages=physical_pages, page_table_entries=page_table_entries, gated_attention=bool(d.gated_attention),
+                   shared_slices=d.shared_slices, shared_gate=bool(d.shared_gate), dense_ffn=d.dense_ffn)
+        check(lib.spo_hybrid_verify_load_gguf(self.handle, gguf_file.handle))
+        self._keep.append(gguf_file)
+        return self
+
     def attends(self, layer):
         return (layer + 1) % self.dims.attention_interval == 0
 

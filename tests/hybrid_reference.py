@@ -13,9 +13,12 @@ from tests.dense_reference import device_copy
 class HybridModel:
     def __init__(self, seed, hidden, vocabulary, layers, q_heads, kv_heads, head_dim, gdn_key_heads, gdn_value_heads, experts, top_k,
                  expert_ffn, attention_interval=4, rope_theta=1e6, gated_attention=False, shared_slices=0, shared_gate=False, dense_ffn=0,
-                 distinct_layers=None, threads=8):
+                 distinct_layers=None, threads=8, file_form=False):
         """`distinct_layers` weight sets are drawn (a multiple of the attention interval, so that a set's mixer is its
-        layers'), layer l holding set l % distinct_layers; all of them by default."""
+        layers'), layer l holding set l % distinct_layers; all of them by default. file_form: the model as a GGUF of the
+        hybrid targets holds it (hybrid_model_file) -- the router, the GDN beta and alpha gates and the GDN output norm as
+        fp32 values, run by the fp32 projection and read unrounded; a GDN layer's output rows in llama.cpp's tiled head
+        order, which its output projection's inputs are in; a packed row padded to whole 64-column groups."""
         self.dims = dict(hidden=hidden, vocabulary=vocabulary, layers=layers, q_heads=q_heads, kv_heads=kv_heads, head_dim=head_dim,
                          gdn_key_heads=gdn_key_heads, gdn_value_heads=gdn_value_heads, experts=experts, top_k=top_k, expert_ffn=expert_ffn,
                          attention_interval=attention_interval)
@@ -27,8 +30,10 @@ class HybridModel:
         self.rng = rng
         D = head_dim
         conv = (2 * gdn_key_heads + gdn_value_heads) * 128
-        self.packed_width = (conv + gdn_value_heads * 128 + 2 * gdn_value_heads + 15) // 16 * 16
-        self.gdn_shape = orc.gdn_shape(gdn_key_heads, gdn_value_heads, packed_width=self.packed_width)
+        self.file_form = file_form
+        self.packed_width = (conv + gdn_value_heads * 128 + 2 * gdn_value_heads + (63 if file_form else 15)) // (64 if file_form else 16) * (64 if file_form else 16)
+        # flags: 1 tiled output heads, 4 fp32 norm weights
+        self.gdn_shape = orc.gdn_shape(gdn_key_heads, gdn_value_heads, packed_width=self.packed_width, flags=5 if file_form else 0)
 
         pool = ThreadPoolExecutor(max(1, threads))
 
@@ -57,6 +62,8 @@ class HybridModel:
                          ffn_down=quant(hidden, dense_ffn, orc.FMT_Q6K))
             if shared_gate:
                 w["shared_scalar_gate"] = (rng.standard_normal(hidden) * 0.05).astype(np.float32)
+            if file_form and experts:
+                w["router"] = (rng.standard_normal((experts, hidden)) * 0.05).astype(np.float32)
             if self.attends(l):
                 w.update(q=quant(q_heads * D * (2 if self.gated else 1), hidden), k=quant(kv_heads * D, hidden), v=quant(kv_heads * D, hidden),
                          o=quant(hidden, q_heads * D), q_norm=norm(D), k_norm=norm(D))
@@ -66,6 +73,10 @@ class HybridModel:
                          conv_w=orc.f32_to_bf16((rng.standard_normal((conv, 4)) * 0.4).astype(np.float32)),
                          a_scale=(-np.exp(rng.uniform(-1.0, 1.0, gdn_value_heads))).astype(np.float32),
                          dt_bias=orc.f32_to_bf16(rng.uniform(-1.0, 1.0, gdn_value_heads).astype(np.float32)), mixer_norm=norm(128))
+                if file_form:
+                    w.update(mixer_in=quant(conv + gdn_value_heads * 128, hidden, scale=0.06),
+                             gate_rows=(rng.standard_normal((2 * gdn_value_heads, hidden)) * 0.06).astype(np.float32),
+                             mixer_norm=(1 + 0.1 * rng.standard_normal(128)).astype(np.float32))
             self.layers.append(w)
         self.layers = [self.layers[l % self.distinct] for l in range(layers)]
         pool.shutdown()
@@ -120,6 +131,19 @@ class HybridModel:
             gpu.set_layer(i, *args, **kwargs)
         gpu.set_head(orc.FMT_Q4K, backend.from_array(self.embedding), backend.from_array(self.final_norm),
                      P([(orc.FMT_Q6K, d["vocabulary"], self.head)], H, True))
+        self.gpu = gpu
+        return gpu
+
+    def build_gpu_from_file(self, backend, path, max_lanes, pages_per_lane):
+        """The driver of the model's GGUF (hybrid_model_file): geometry and weights as the loader reads them."""
+        from splash_amd import gguf
+        self.pages_per_lane = pages_per_lane
+        self.physical_pages = max_lanes * pages_per_lane + 1
+        gpu = verify.HybridVerify.from_gguf(backend, gguf.GgufFile(str(path)), max_lanes=max_lanes, physical_pages=self.physical_pages,
+                                            page_table_entries=max_lanes * pages_per_lane)
+        assert gpu.dims.gdn_packed_width == self.packed_width
+        self.table = np.random.default_rng(99).permutation(self.physical_pages)[:max_lanes * pages_per_lane].astype(np.uint64)
+        gpu.buffer(verify.PAGE_TABLE).upload(self.table)
         self.gpu = gpu
         return gpu
 
@@ -185,6 +209,11 @@ class HybridModel:
             D = d["head_dim"]
             out = np.concatenate([self._project(orc.FMT_Q4K, w[name], n, width) for name, width in
                                   (("q", d["q_heads"] * D * (2 if self.gated else 1)), ("k", d["kv_heads"] * D), ("v", d["kv_heads"] * D))], axis=1)
+        elif self.file_form:
+            # q | k | v | z from the quantized rows, beta | alpha from the rows of floats, the padding columns nobody reads
+            width = (2 * d["gdn_key_heads"] + 2 * d["gdn_value_heads"]) * 128
+            out = np.concatenate([self._project(orc.FMT_Q4K, w["mixer_in"], n, width), orc.float_projection(n, w["gate_rows"]),
+                                  np.zeros((n.shape[0], self.packed_width - width - 2 * d["gdn_value_heads"]))], axis=1)
         else:
             out = self._project(orc.FMT_Q4K, w["mixer_in"], n, self.packed_width)
         return orc.f32_to_bf16(out.astype(np.float32))
@@ -250,7 +279,7 @@ class HybridModel:
             mid = orc.swiglu(self._project(orc.FMT_Q4K, w["ffn_gate"], n, self.dense_ffn), self._project(orc.FMT_Q4K, w["ffn_up"], n, self.dense_ffn))
             down = self._project(orc.FMT_Q6K, w["ffn_down"], mid, d["hidden"])
             return None, orc.f32_to_bf16((down + orc.bf16_to_f32(hidden1)).astype(np.float32))
-        scores = self._project(orc.FMT_Q6K, w["router"], n, d["experts"]).astype(np.float32)
+        scores = orc.float_projection(n, w["router"]) if self.file_form else self._project(orc.FMT_Q6K, w["router"], n, d["experts"]).astype(np.float32)
         _, _, _, out = orc.moe_layer(n, hidden1, scores, d["top_k"], w["gate"], w["up"], w["down"], d["expert_ffn"],
                                      shared=self.shared_slices, shared_gate=w.get("shared_scalar_gate"))
         return scores, out
@@ -258,3 +287,83 @@ class HybridModel:
     def oracle_head(self, hidden):
         n = orc.rms_norm(hidden, self.final_norm)
         return self._project(orc.FMT_Q6K, self.head, n, self.dims["vocabulary"])
+
+
+def hybrid_model_file(path, model, router_kind="f32", fused_gate_up=False, skip=(), extra=(), more_metadata=()):
+    """A file_form HybridModel's GGUF as llama.cpp writes a qwen35moe (or, without experts, qwen35) model: the value heads of
+    attn_qkv, attn_gate, ssm_beta, ssm_alpha, ssm_conv1d, ssm_a and ssm_dt.bias in tiled order (value head j of key head
+    h at j * key heads + h), which the model holds grouped; the experts' tensors of three dimensions."""
+    from tests import gguf_writer as gw
+    assert model.file_form
+    d = model.dims
+    H, D, V, KH, VH = d["hidden"], d["head_dim"], d["vocabulary"], d["gdn_key_heads"], d["gdn_value_heads"]
+    E, F, S = d["experts"], d["expert_ffn"], model.shared_slices
+    per, conv_rows, value_rows = VH // KH, (2 * KH + VH) * 128, VH * 128
+    arch = "qwen35moe" if E else "qwen35"
+    f32 = lambda bits: orc.bf16_to_f32(bits).astype(np.float32)
+    # grouped head g = h * per + j  ->  tiled position j * KH + h
+    order = [h * per + j for j in range(per) for h in range(KH)]
+
+    def tiled(rows, head_rows, first=0):
+        """`rows` (an array of rows; natives as [rows][row bytes]) with the value heads from row `first` on in tiled order."""
+        rows = np.asarray(rows)
+        heads = rows[first:].reshape(VH, head_rows, *rows.shape[1:])
+        return np.concatenate([rows[:first], heads[order].reshape(VH * head_rows, *rows.shape[1:])])
+    native_rows = lambda native, n: np.asarray(native).reshape(n, -1)
+    tensors = [("token_embd.weight", gw.GGML_Q4_K, [H, V], model.embedding), ("output_norm.weight", gw.GGML_F32, [H], f32(model.final_norm)),
+               ("output.weight", gw.GGML_Q6_K, [H, V], model.head)]
+    for i, w in enumerate(model.layers):
+        p = f"blk.{i}."
+        tensors += [(p + "attn_norm.weight", gw.GGML_F32, [H], f32(w["input_norm"])),
+                    (p + "post_attention_norm.weight", gw.GGML_F32, [H], f32(w["post_norm"]))]
+        if model.attends(i):
+            q_rows = d["q_heads"] * D * (2 if model.gated else 1)
+            tensors += [(p + "attn_q.weight", gw.GGML_Q4_K, [H, q_rows], w["q"]), (p + "attn_k.weight", gw.GGML_Q4_K, [H, d["kv_heads"] * D], w["k"]),
+                        (p + "attn_v.weight", gw.GGML_Q4_K, [H, d["kv_heads"] * D], w["v"]),
+                        (p + "attn_q_norm.weight", gw.GGML_F32, [D], f32(w["q_norm"])), (p + "attn_k_norm.weight", gw.GGML_F32, [D], f32(w["k_norm"])),
+                        (p + "attn_output.weight", gw.GGML_Q4_K, [d["q_heads"] * D, H], w["o"])]
+        else:
+            rows = native_rows(w["mixer_in"], conv_rows + value_rows)
+            tensors += [(p + "attn_qkv.weight", gw.GGML_Q4_K, [H, conv_rows], tiled(rows[:conv_rows], 128, first=2 * KH * 128)),
+                        (p + "attn_gate.weight", gw.GGML_Q4_K, [H, value_rows], tiled(rows[conv_rows:], 128)),
+                        (p + "ssm_beta.weight", gw.GGML_F32, [H, VH], tiled(w["gate_rows"][:VH], 1)),
+                        (p + "ssm_alpha.weight", gw.GGML_F32, [H, VH], tiled(w["gate_rows"][VH:], 1)),
+                        (p + "ssm_conv1d.weight", gw.GGML_F32, [4, conv_rows], tiled(f32(w["conv_w"]), 128, first=2 * KH * 128)),
+                        (p + "ssm_a", gw.GGML_F32, [VH], tiled(w["a_scale"], 1)), (p + "ssm_dt.bias", gw.GGML_F32, [VH], tiled(f32(w["dt_bias"]), 1)),
+                        (p + "ssm_norm.weight", gw.GGML_F32, [128], w["mixer_norm"]),
+                        (p + "ssm_out.weight", gw.GGML_Q4_K, [value_rows, H], w["mixer_out"])]
+        if not E:
+            tensors += [(p + "ffn_gate.weight", gw.GGML_Q4_K, [H, model.dense_ffn], w["ffn_gate"]),
+                        (p + "ffn_up.weight", gw.GGML_Q4_K, [H, model.dense_ffn], w["ffn_up"]),
+                        (p + "ffn_down.weight", gw.GGML_Q6_K, [model.dense_ffn, H], w["ffn_down"])]
+            continue
+        router = {"f32": (gw.GGML_F32, w["router"]), "bf16": (gw.GGML_BF16, orc.f32_to_bf16(w["router"]))}[router_kind]
+        tensors.append((p + "ffn_gate_inp.weight", router[0], [H, E], router[1]))
+        cat = lambda natives: np.concatenate([np.asarray(x).ravel() for x in natives])
+        if fused_gate_up:    # expert e's gate rows, then its up rows
+            tensors.append((p + "ffn_gate_up_exps.weight", gw.GGML_Q4_K, [H, 2 * F, E], cat([x for e in range(E) for x in (w["gate"][e], w["up"][e])])))
+        else:
+            tensors += [(p + "ffn_gate_exps.weight", gw.GGML_Q4_K, [H, F, E], cat(w["gate"][:E])), (p + "ffn_up_exps.weight", gw.GGML_Q4_K, [H, F, E], cat(w["up"][:E]))]
+        tensors.append((p + "ffn_down_exps.weight", gw.GGML_Q4_K, [F, H, E], cat(w["down"][:E])))
+        if S:
+            tensors += [(p + "ffn_gate_shexp.weight", gw.GGML_Q4_K, [H, S * F], cat(w["gate"][E:])), (p + "ffn_up_shexp.weight", gw.GGML_Q4_K, [H, S * F], cat(w["up"][E:])),
+                        # a row of the shared down projection holds every slice's inputs, slice after slice
+                        (p + "ffn_down_shexp.weight", gw.GGML_Q4_K, [S * F, H], np.concatenate([native_rows(x, H) for x in w["down"][E:]], axis=1))]
+        if model.shared_gate:
+            tensors.append((p + "ffn_gate_inp_shexp.weight", gw.GGML_F32, [H], w["shared_scalar_gate"]))
+    tensors = [t for t in tensors if t[0] not in skip] + list(extra)
+    a = arch + "."
+    metadata = [("general.architecture", gw.STRING, arch), (a + "block_count", gw.U32, d["layers"]), (a + "embedding_length", gw.U32, H),
+                (a + "attention.head_count", gw.U32, d["q_heads"]), (a + "attention.head_count_kv", gw.U32, d["kv_heads"]),
+                (a + "attention.key_length", gw.U32, D), (a + "attention.value_length", gw.U32, D), (a + "rope.dimension_count", gw.U32, D),
+                (a + "attention.layer_norm_rms_epsilon", gw.F32, 1e-6), (a + "rope.freq_base", gw.F32, model.rope_theta),
+                (a + "full_attention_interval", gw.U32, d["attention_interval"]), (a + "ssm.conv_kernel", gw.U32, 4),
+                (a + "ssm.group_count", gw.U32, KH), (a + "ssm.time_step_rank", gw.U32, VH), (a + "ssm.state_size", gw.U32, 128),
+                (a + "ssm.inner_size", gw.U32, VH * 128)]
+    if E:
+        metadata += [(a + "expert_count", gw.U32, E), (a + "expert_used_count", gw.U32, d["top_k"]), (a + "expert_feed_forward_length", gw.U32, F),
+                     (a + "expert_shared_feed_forward_length", gw.U32, S * F)]
+    else:
+        metadata.append((a + "feed_forward_length", gw.U32, model.dense_ffn))
+    gw.write_gguf(path, metadata + list(more_metadata), tensors)
+    return path

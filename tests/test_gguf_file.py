@@ -319,3 +319,83 @@ def test_dense_geometry_from_metadata(tmp_path):
     g = gguf.GgufFile(both)
     with pytest.raises(splash_amd.SplashError, match="partial rotary.*rope.scaling.type yarn"):
         splash_amd.check(splash_amd.lib.spg_dense_dimensions(g.handle, ctypes.byref(d)))
+
+
+# ------------------------------------------------------------------ the hybrid targets' files (qwen35, qwen35moe)
+HYBRID = dict(hidden=256, vocabulary=1024, layers=4, q_heads=8, kv_heads=2, head_dim=128, gdn_key_heads=2, gdn_value_heads=4,
+              experts=16, top_k=2, expert_ffn=256)
+
+
+def test_hybrid_dimensions_come_from_the_metadata(tmp_path):
+    """GgufImage.cpp:874-936: the geometry of a qwen35moe file, the prediction blocks after the target's layers left out,
+    and the refusals: an architecture the hybrid driver does not compute, a state size the kernels do not hold."""
+    from splash_amd import _native as nat
+    from tests.dense_reference import DenseModel
+    from tests.hybrid_reference import HybridModel, hybrid_model_file
+    import ctypes
+    model = HybridModel(seed=3, **HYBRID, shared_slices=1, shared_gate=True, gated_attention=True, file_form=True)
+    path = hybrid_model_file(tmp_path / "hybrid.gguf", model, more_metadata=[("qwen35moe.nextn_predict_layers", gw.U32, 0)])
+    d = nat.HybridDimensions()
+    f = gguf.GgufFile(str(path))
+    nat.check(nat.lib.spg_hybrid_dimensions(f.handle, ctypes.byref(d)))
+    assert (d.hidden, d.vocabulary, d.layers, d.attention_interval, d.q_heads, d.kv_heads, d.head_dim, d.rotary_pairs) == (256, 1024, 4, 4, 8, 2, 128, 64)
+    assert (d.gdn_key_heads, d.gdn_value_heads, d.experts, d.top_k, d.expert_ffn, d.shared_slices, d.shared_gate, d.dense_ffn) == (2, 4, 16, 2, 256, 1, 1, 0)
+    assert d.gdn_packed_width == model.packed_width == 1600 and d.gated_attention == 1 and d.normalize_heads == 1
+    # a dense file is not a hybrid one
+    dense = DenseModel(seed=5, hidden=512, q_heads=8, kv_heads=2, head_dim=64, ffn=768, vocabulary=256, layers=1)
+    other = gguf.GgufFile(str(dense_model_file(tmp_path / "dense.gguf", dense, orc.FMT_Q6K, tied=True)))
+    with pytest.raises(splash_amd.SplashError, match="qwen35"):
+        nat.check(nat.lib.spg_hybrid_dimensions(other.handle, ctypes.byref(d)))
+    # the last block is a prediction block: one layer fewer
+    path = hybrid_model_file(tmp_path / "nextn.gguf", model, more_metadata=[("qwen35moe.nextn_predict_layers", gw.U32, 1)])
+    later = gguf.GgufFile(str(path))
+    nat.check(nat.lib.spg_hybrid_dimensions(later.handle, ctypes.byref(d)))
+    assert d.layers == 3
+    # a state size the kernels do not hold: the same file with the value patched
+    path = hybrid_model_file(tmp_path / "state.gguf", model)
+    raw = bytearray(open(path, "rb").read())
+    at = raw.index(b"qwen35moe.ssm.state_size") + len(b"qwen35moe.ssm.state_size") + 4
+    raw[at:at + 4] = (64).to_bytes(4, "little")
+    open(tmp_path / "state64.gguf", "wb").write(raw)
+    patched = gguf.GgufFile(str(tmp_path / "state64.gguf"))
+    with pytest.raises(splash_amd.SplashError, match="ssm.state_size"):
+        nat.check(nat.lib.spg_hybrid_dimensions(patched.handle, ctypes.byref(d)))
+
+
+@pytest.mark.gpu
+def test_a_hybrid_decoder_from_a_file_computes_the_oracles_step(backend, tmp_path):
+    """A qwen35moe file as llama.cpp lays it out (value heads tiled, F32 gates, router and norms, experts of three
+    dimensions, a gated shared expert, gated attention) through spg_hybrid_dimensions and spo_hybrid_verify_load_gguf:
+    the step, layer by layer, against the oracle over the model's own (grouped) tensors. The file with the fused
+    ffn_gate_up_exps gives the same logits bit for bit; refusals name what the loader cannot read."""
+    from splash_amd import verify
+    from tests.hybrid_reference import HybridModel, hybrid_model_file
+    from tests.test_hybrid_step_gpu import check_step
+    print("case hybrid gguf", flush=True)
+    model = HybridModel(seed=43, **HYBRID, shared_slices=1, shared_gate=True, gated_attention=True, file_form=True)
+    path = hybrid_model_file(tmp_path / "hybrid.gguf", model)
+    rng = np.random.default_rng(9)
+    lanes = [verify.HybridLane(6, 70, table_first=0), verify.HybridLane(16, 300, table_first=2)]
+    tokens = rng.integers(0, 1024, 22).astype(np.uint32)
+
+    def run(file_path):
+        gpu = model.build_gpu_from_file(backend, file_path, max_lanes=2, pages_per_lane=2)
+        seed = np.random.default_rng(10)
+        model.seed_context(seed)
+        model.seed_states(seed, lanes=2)
+        return gpu
+    check_step(backend, model, run(path), lanes, tokens)
+
+    def whole_step(gpu):
+        gpu.set_block(lanes, tokens)
+        backend.run(gpu.encode(lanes, commit=False))
+        return gpu.buffer(verify.LOGITS).download(np.float32, 22 * 1024).copy()
+    assert np.array_equal(whole_step(run(hybrid_model_file(tmp_path / "fused.gguf", model, fused_gate_up=True))), whole_step(run(path)))
+    # what the loader refuses: a quantized gate tensor, a tensor nobody reads, a missing one
+    w0 = model.layers[0]
+    quantized_beta = ("blk.0.ssm_beta.weight", gw.GGML_Q4_K, [256, 4], orc.quantize_rows(orc.FMT_Q4K, w0["gate_rows"][:4]))
+    for name, kwargs, needle in (("quantized", dict(skip=("blk.0.ssm_beta.weight",), extra=(quantized_beta,)), "ssm_beta.weight is not of 16- or 32-bit floats"),
+                                 ("bias", dict(extra=(("blk.1.ffn_gate_inp.bias", gw.GGML_F32, [16], np.zeros(16, np.float32)),)), "ffn_gate_inp.bias is not read"),
+                                 ("missing", dict(skip=("blk.2.ssm_out.weight",)), "blk.2.ssm_out.weight is missing")):
+        with pytest.raises(splash_amd.SplashError, match=needle):
+            model.build_gpu_from_file(backend, hybrid_model_file(tmp_path / f"{name}.gguf", model, **kwargs), max_lanes=1, pages_per_lane=2)
