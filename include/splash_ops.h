@@ -602,6 +602,11 @@ typedef struct spo_hybrid_layer {
 } spo_hybrid_layer;
 sp_status spo_hybrid_verify_create(sp_backend *backend, const spo_hybrid_dimensions *dimensions, uint32_t max_lanes,
                                    uint32_t physical_pages, uint32_t page_table_entries, spo_hybrid_verify **out);
+/* The same with room for prompt chunks of up to prefill_rows rows (spo_hybrid_verify_encode_prefill; 0: a step's most; at
+ * most 2048, SPLASH_PREFILL_TOKEN_BUDGET). */
+sp_status spo_hybrid_verify_create_chunked(sp_backend *backend, const spo_hybrid_dimensions *dimensions, uint32_t max_lanes,
+                                           uint32_t physical_pages, uint32_t page_table_entries, uint32_t prefill_rows,
+                                           spo_hybrid_verify **out);
 void spo_hybrid_verify_destroy(spo_hybrid_verify *verify);
 sp_status spo_hybrid_verify_set_layer(spo_hybrid_verify *verify, uint32_t layer, const spo_hybrid_layer *weights);
 sp_status spo_hybrid_verify_set_head(spo_hybrid_verify *verify, uint32_t embedding_format, sp_buffer *embedding_rows,
@@ -610,6 +615,15 @@ sp_status spo_hybrid_verify_set_head(spo_hybrid_verify *verify, uint32_t embeddi
 #define SPO_VERIFY_GDN_STATES 13
 #define SPO_VERIFY_GDN_TAPE 14
 sp_status spo_hybrid_verify_buffer(spo_hybrid_verify *verify, uint32_t which, uint32_t index, sp_buffer **out);
+/* HybridVerify::encodePrefill: a chunk of `tokens` prompt tokens of the sequence of lane `lane` (its pages from table_first,
+ * `committed` tokens cached; inputs as spo_dense_verify_encode_prefill's) through layers [first_layer, first_layer +
+ * layer_count) (layer_count 0: to the last; the embedding with first_layer 0), no head: the reference's chunked prefill over
+ * its hybrid target (QwenTarget.cpp:206-347 with GDN::addPrefill, GDN.cpp:132-222; PagedAttention.cpp:351-389). Attention
+ * layers store the chunk's keys and values and attend causally; Gated DeltaNet layers take every row into the state, from
+ * the lane's cell of `parity` to its other cell: the lane's next step has the other parity and no pending path. */
+sp_status spo_hybrid_verify_encode_prefill(spo_hybrid_verify *verify, spo_graph *graph, uint32_t lane, uint32_t table_first,
+                                           uint32_t committed, uint32_t tokens, uint32_t parity, uint32_t first_layer,
+                                           uint32_t layer_count);
 /* As spo_dense_verify_results. */
 sp_status spo_hybrid_verify_results(spo_hybrid_verify *verify, const spo_hybrid_lane *lanes, uint32_t count, uint32_t *tokens,
                                     uint32_t *retained, uint32_t *accepted, uint32_t *retained_rows);

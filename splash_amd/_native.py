@@ -328,6 +328,8 @@ _sig("spo_dense_verify_step_bytes", c_u64, c_p, P(VerifyLane), c_u32)
 _sig("spo_dense_verify_encode", c_int, c_p, c_p, P(VerifyLane), c_u32, c_int)
 _sig("spo_dense_verify_encode_part", c_int, c_p, c_p, c_u32, c_u32, P(VerifyLane), c_u32)
 _sig("spo_hybrid_verify_create", c_int, c_p, P(HybridDimensions), c_u32, c_u32, c_u32, P(c_p))
+_sig("spo_hybrid_verify_create_chunked", c_int, c_p, P(HybridDimensions), c_u32, c_u32, c_u32, c_u32, P(c_p))
+_sig("spo_hybrid_verify_encode_prefill", c_int, c_p, c_p, c_u32, c_u32, c_u32, c_u32, c_u32, c_u32, c_u32)
 _sig("spo_hybrid_verify_destroy", None, c_p)
 _sig("spo_hybrid_verify_set_layer", c_int, c_p, c_u32, P(HybridLayer))
 _sig("spo_hybrid_verify_set_head", c_int, c_p, c_u32, c_p, c_p, c_p)

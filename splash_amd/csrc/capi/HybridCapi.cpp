@@ -36,6 +36,10 @@ extern "C" {
 
 sp_status spo_hybrid_verify_create(sp_backend *backend, const spo_hybrid_dimensions *d, uint32_t max_lanes, uint32_t physical_pages,
                                    uint32_t page_table_entries, spo_hybrid_verify **out) {
+  return spo_hybrid_verify_create_chunked(backend, d, max_lanes, physical_pages, page_table_entries, 0, out);
+}
+sp_status spo_hybrid_verify_create_chunked(sp_backend *backend, const spo_hybrid_dimensions *d, uint32_t max_lanes, uint32_t physical_pages,
+                                           uint32_t page_table_entries, uint32_t prefill_rows, spo_hybrid_verify **out) {
   return capi::guard([&] {
     capi::require(backend && d && out, "backend, dimensions or result");
     auto holder = std::make_unique<spo_hybrid_verify>();
@@ -61,7 +65,7 @@ sp_status spo_hybrid_verify_create(sp_backend *backend, const spo_hybrid_dimensi
     dims.sharedSlices = d->shared_slices;
     dims.sharedGate = d->shared_gate != 0;
     dims.denseFfn = d->dense_ffn;
-    holder->verify = std::make_unique<model::HybridVerify>(*holder->backend, dims, max_lanes, physical_pages, page_table_entries);
+    holder->verify = std::make_unique<model::HybridVerify>(*holder->backend, dims, max_lanes, physical_pages, page_table_entries, prefill_rows);
     *out = holder.release();
   });
 }
@@ -216,6 +220,14 @@ sp_status spo_hybrid_verify_encode_part(spo_hybrid_verify *verify, spo_graph *gr
     else if (part == 1) verify->verify->encodeLayer(capi::graphOf(graph), index, list);
     else if (part == 2) verify->verify->encodeHead(capi::graphOf(graph), rows);
     else throw std::invalid_argument("no such part of the step");
+  });
+}
+
+sp_status spo_hybrid_verify_encode_prefill(spo_hybrid_verify *verify, spo_graph *graph, uint32_t lane, uint32_t table_first,
+                                           uint32_t committed, uint32_t tokens, uint32_t parity, uint32_t first_layer, uint32_t layer_count) {
+  return capi::guard([&] {
+    capi::require(verify && graph, "verify or graph");
+    verify->verify->encodePrefill(capi::graphOf(graph), lane, table_first, committed, tokens, parity, first_layer, layer_count);
   });
 }
 

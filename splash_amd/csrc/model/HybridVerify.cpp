@@ -17,8 +17,9 @@ template <class F> void forRowPieces(uint32_t rows, F &&piece) {
 } // namespace
 
 HybridVerify::HybridVerify(hip::Backend &backend, HybridDimensions d, uint32_t maxLanes, uint32_t physicalPages,
-                           uint32_t pageTableEntries)
+                           uint32_t pageTableEntries, uint32_t prefillRows)
     : backend_(backend), dims_(d), linear_(backend.deviceInfo()), maxLanes_(maxLanes) {
+  if (prefillRows > ops::kMaximumChunkRows) throw std::invalid_argument("a prompt chunk holds at most 2048 rows");
   if (!d.hidden || !d.layers || !d.vocabulary || !maxLanes || maxLanes > GDN_MAXIMUM_LANES)
     throw std::invalid_argument("a hybrid verify step takes a model and 1 to 8 lanes");
   if (!d.attentionInterval || d.layers % d.attentionInterval)
@@ -30,30 +31,33 @@ HybridVerify::HybridVerify(hip::Backend &backend, HybridDimensions d, uint32_t m
   if (d.dense() ? (!d.denseFfn || d.denseFfn % GGUF_BLOCK) : !d.moeShape().valid())
     throw std::invalid_argument(d.dense() ? "a dense FFN holds whole super-blocks" : "invalid MoE shape");
   maxRows_ = maxLanes * ATTENTION_MAXIMUM_ROWS;
+  rowCapacity_ = std::max(maxRows_, prefillRows);
+  // the most rows of one window of a chunk's projections and experts, or of a step
+  const uint32_t windowRows = std::min(rowCapacity_, std::max(maxRows_, kProjectionRows));
   weights_.layers.resize(d.layers);
   const ops::kv::Layout layout{d.kvHeads, d.headDimension};
   pageBytes_ = layout.bytesPerLayerPage();
   auto device = [&](uint64_t bytes, const char *label) { return backend.allocateBuffer(std::max<uint64_t>(bytes, 16), BufferStorage::Private, label); };
   auto shared = [&](uint64_t bytes, const char *label) { return backend.allocateBuffer(std::max<uint64_t>(bytes, 16), BufferStorage::Shared, label); };
-  const uint64_t R = maxRows_;
-  hidden_[0] = device(R * d.hidden * 2, "hidden 0");
-  hidden_[1] = device(R * d.hidden * 2, "hidden 1");
-  normalized_ = device(R * d.hidden * 2, "normalized");
-  packed_ = device(R * std::max(d.qkvWidth(), d.gdnPackedWidth) * 2, "mixer input rows");
-  mixed_ = device(R * std::max(d.attentionWidth(), d.gdnWidth()) * 2, "mixer output rows");
-  scores_ = device(R * d.experts * 4, "router scores");
+  const uint64_t R = maxRows_, C = rowCapacity_;
+  hidden_[0] = device(C * d.hidden * 2, "hidden 0");
+  hidden_[1] = device(C * d.hidden * 2, "hidden 1");
+  normalized_ = device(C * d.hidden * 2, "normalized");
+  packed_ = device(C * std::max(d.qkvWidth(), d.gdnPackedWidth) * 2, "mixer input rows");
+  mixed_ = device(C * std::max(d.attentionWidth(), d.gdnWidth()) * 2, "mixer output rows");
+  scores_ = device(uint64_t{windowRows} * d.experts * 4, "router scores");
   logits_ = device(R * d.vocabulary * 4, "logits");
-  ropeCos_ = device(R * std::max(1u, d.rotaryPairs) * 4, "rope cos");
-  ropeSin_ = device(R * std::max(1u, d.rotaryPairs) * 4, "rope sin");
+  ropeCos_ = device(C * std::max(1u, d.rotaryPairs) * 4, "rope cos");
+  ropeSin_ = device(C * std::max(1u, d.rotaryPairs) * 4, "rope sin");
   inverseFrequency_ = device(std::max(1u, d.rotaryPairs) * 4, "rope inverse frequency");
   if (d.rotaryPairs) {
     std::vector<float> inv(d.rotaryPairs);
     for (uint32_t i = 0; i < d.rotaryPairs; ++i) inv[i] = float(std::pow(double(d.ropeTheta), -double(i) / d.rotaryPairs));
     inverseFrequency_.upload(inv.data(), inv.size() * 4);
   }
-  inputTokens_ = shared(R * 4, "input tokens");
-  treeRows_ = shared(R * sizeof(AttentionTreeRow), "tree rows");
-  depths_ = shared(R * 4, "row depths");
+  inputTokens_ = shared(C * 4, "input tokens");
+  treeRows_ = shared(C * sizeof(AttentionTreeRow), "tree rows");
+  depths_ = shared(C * 4, "row depths");
   uniforms_ = shared(R * 8, "uniforms");
   tokens_ = shared(R * 4, "selected tokens");
   retained_ = shared(maxLanes * 4, "retained");
@@ -71,7 +75,7 @@ HybridVerify::HybridVerify(hip::Backend &backend, HybridDimensions d, uint32_t m
   states_ = device(cellBytes_ * 2 * maxLanes, "GDN state cells");
   tape_ = device(tapeLayerBytes_ * d.gdnLayers() * 2 * maxLanes, "GDN tapes");
   // Scratch of every dense projection at a piece's most rows.
-  const uint32_t pieceRows = std::min(maxRows_, kProjectionRows);
+  const uint32_t pieceRows = std::min(rowCapacity_, kProjectionRows);
   ops::LinearScratchSize size;
   for (ops::LinearMatrix m : {ops::LinearMatrix{d.qkvWidth(), d.hidden}, ops::LinearMatrix{d.hidden, d.attentionWidth()},
                               ops::LinearMatrix{d.gdnPackedWidth, d.hidden}, ops::LinearMatrix{d.hidden, d.gdnWidth()},
@@ -80,19 +84,22 @@ HybridVerify::HybridVerify(hip::Backend &backend, HybridDimensions d, uint32_t m
                               ops::LinearMatrix{d.vocabulary, d.hidden}})
     size.include(linear_.scratchSize(m, pieceRows));
   if (d.dense()) {
-    intermediate_ = device(R * d.denseFfn * 2, "SwiGLU rows");
+    intermediate_ = device(uint64_t{windowRows} * d.denseFfn * 2, "SwiGLU rows");
     ffnTable_ = device(gguf_tables_bytes(d.denseFfn, gguf_row_tiles(pieceRows)), "SwiGLU table");
   }
   scratch_.input = device(size.input, "linear table");
   scratch_.partials = device(size.partials, "linear partials");
   scratch_.counters = device(std::max<uint64_t>(size.counters, 4), "linear counters");
   mixedTable_ = device(gguf_tables_bytes(std::max(d.attentionWidth(), d.gdnWidth()), gguf_row_tiles(pieceRows)), "mixer output table");
-  const uint64_t fused = uint64_t{maxLanes} * d.kvHeads * (d.qHeads / std::max(1u, d.kvHeads)) * 16;
-  attentionWorkspace_.queries = device(fused * d.headDimension * 2, "staged queries");
-  attentionWorkspace_.querySums = device(fused * 4, "query sums");
+  // Staged queries for every tile of the longest chunk; partials for the tiles of one dispatch.
+  const uint64_t fusedTile = uint64_t{d.kvHeads} * (d.qHeads / std::max(1u, d.kvHeads)) * 16;
+  const uint64_t staged = fusedTile * std::max(maxLanes, gguf_row_tiles(rowCapacity_));
+  const uint64_t fused = fusedTile * (rowCapacity_ > maxRows_ ? ATTENTION_MAXIMUM_SEQUENCES : maxLanes);
+  attentionWorkspace_.queries = device(staged * d.headDimension * 2, "staged queries");
+  attentionWorkspace_.querySums = device(staged * 4, "query sums");
   attentionWorkspace_.partials = device(fused * ATTENTION_MAXIMUM_SPLITS * d.headDimension * 2, "attention partials");
   attentionWorkspace_.partialSums = device(fused * ATTENTION_MAXIMUM_SPLITS * 8, "attention partial sums");
-  const ops::MoeWorkspaceSize moe = d.dense() ? ops::MoeWorkspaceSize{} : ops::MoE::workspace(d.moeShape(), maxRows_);
+  const ops::MoeWorkspaceSize moe = d.dense() ? ops::MoeWorkspaceSize{} : ops::MoE::workspace(d.moeShape(), windowRows);
   moeWorkspace_ = {device(moe.selected, "moe selected"),    device(moe.weights, "moe weights"),     device(moe.routeSlot, "moe route slots"),
                    device(moe.slotRow, "moe slot rows"),    device(moe.tileExpert, "moe tile experts"), device(moe.tileRows, "moe tile rows"),
                    device(moe.tileTotal, "moe tile count"), device(moe.tables, "moe tables"),       device(moe.nextTables, "moe SwiGLU tables"),
@@ -108,6 +115,14 @@ HybridVerify::HybridVerify(hip::Backend &backend, HybridDimensions d, uint32_t m
   sampling_.uniforms = uniforms_;
   sampling_.inputTokens = inputTokens_;
   sampling_.treeRows = treeRows_;
+  // The rows a Gated DeltaNet layer's prefill passes hand each other, for the longest chunk.
+  const uint64_t keyWidth = uint64_t{d.gdnKeyHeads} * GDN_HEAD_DIMENSION;
+  gdnPrefill_.queries = device(C * keyWidth * 2, "GDN prefill queries");
+  gdnPrefill_.keys = device(C * keyWidth * 2, "GDN prefill keys");
+  gdnPrefill_.values = device(C * d.gdnWidth() * 2, "GDN prefill values");
+  gdnPrefill_.decay = device(C * d.gdnValueHeads * 4, "GDN prefill decay");
+  gdnPrefill_.beta = device(C * d.gdnValueHeads * 2, "GDN prefill beta");
+  gdnPrefill_.recurrentRows = device(C * d.gdnWidth() * 2, "GDN prefill rows");
 }
 
 const hip::Buffer &HybridVerify::draftProbabilities() {
@@ -323,6 +338,112 @@ void HybridVerify::encode(hip::CommandGraph &graph, const std::vector<HybridLane
   if (commit && dims_.attentionLayers())
     ops::PagedAttention::addPathCommit(graph, planOf(lanes), retainedRows_, {pageTable_, kvAll_, pageBytes_}, dims_.attentionLayers(),
                                        layerBytes_);
+}
+
+// A layer of a prompt chunk: every window's mixer input rows, the mixer over all the chunk's rows, then every window's
+// output projection and FFN. No projection defers its norm here: a window starts with a norm pass.
+void HybridVerify::encodePrefillLayer(hip::CommandGraph &graph, uint32_t layer, const ops::AttentionChunkPlan &plan, uint32_t tokens,
+                                      uint64_t currentCell, uint64_t nextCell) {
+  const HybridLayer &w = weights_.layers.at(layer);
+  const bool attends = dims_.attends(layer);
+  const uint32_t index = dims_.mixerIndex(layer);
+  const hip::Buffer &residual = hidden_[0], &next = hidden_[1];
+  const uint64_t hiddenBytes = uint64_t{dims_.hidden} * 2;
+  const uint32_t inputWidth = w.mixerInput.outputSize, mixedWidth = w.mixerOutput.inputSize;
+  if (inputWidth != (attends ? dims_.qkvWidth() : dims_.gdnPackedWidth) || mixedWidth != (attends ? dims_.attentionWidth() : dims_.gdnWidth()))
+    throw std::invalid_argument("the layer's projections do not fit the model");
+  forRowPieces(tokens, [&](uint32_t first, uint32_t count) {
+    const hip::Buffer normalized = rowsOf(normalized_, first, count, hiddenBytes);
+    ops::LinearBuffers in;
+    in.input = normalized;
+    in.output = rowsOf(packed_, first, count, uint64_t{inputWidth} * 2);
+    in.scratch = scratch_;
+    in.prepared = ops::Normalization::addRmsTable(graph, rowsOf(residual, first, count, hiddenBytes), w.inputNorm, normalized, scratch_,
+                                                  dims_.hidden, count);
+    linear_.add(graph, in, w.mixerInput, linear_.plan(w.mixerInput, count));
+    if (!attends && w.gateRows) {
+      const ops::GdnShape shape = dims_.gdnShape();
+      ops::FloatProjection::add(graph, normalized, w.gateRows, in.output, count, inputWidth,
+                                shape.convolutionDimension + shape.valueHeads * GDN_HEAD_DIMENSION, ops::FloatOutput::BFloat16);
+    }
+  });
+  if (attends) {
+    const ops::KvPages pages{pageTable_, kvPools_.at(index), pageBytes_};
+    ops::PagedAttention::addChunkProjection(graph, plan, {packed_, w.queryNorm, w.keyNorm, ropeCos_, ropeSin_}, attentionWorkspace_, pages);
+    ops::PagedAttention::addChunkAttention(graph, plan, attentionWorkspace_, treeRows_, pages, mixed_, {}, packed_);
+  } else {
+    ops::GdnPrefillBuffers buffers = gdnPrefill_;
+    buffers.packed = packed_;
+    buffers.convolutionWeights = w.convolutionWeights;
+    buffers.states = states_;
+    buffers.decayWeights = w.decay;
+    buffers.timeBias = w.timeBias;
+    buffers.mixerNorm = w.mixerNorm;
+    buffers.floatNorm = w.mixerNormFloat;
+    buffers.hidden = mixed_;
+    buffers.currentCell = currentCell;
+    buffers.nextCell = nextCell;
+    ops::GDN::addPrefill(graph, buffers, dims_.gdnShape(), index, tokens, strides_,
+                         tiledGdnHeads_ ? ops::GdnHeadOrder::Tiled : ops::GdnHeadOrder::Grouped);
+  }
+  const ops::MoeShape moe = dims_.moeShape();
+  forRowPieces(tokens, [&](uint32_t first, uint32_t count) {
+    const hip::Buffer nextRows = rowsOf(next, first, count, hiddenBytes), residualRows = rowsOf(residual, first, count, hiddenBytes);
+    const hip::Buffer normalized = rowsOf(normalized_, first, count, hiddenBytes);
+    ops::LinearBuffers out;
+    out.input = rowsOf(mixed_, first, count, uint64_t{mixedWidth} * 2);
+    out.output = nextRows;
+    out.residual = residualRows;
+    out.scratch = scratch_;
+    linear_.add(graph, out, w.mixerOutput, linear_.plan(w.mixerOutput, count, ops::LinearEpilogue::Residual));
+    const ops::PreparedInput prepared = ops::Normalization::addRmsTable(graph, nextRows, w.postNorm, normalized, scratch_, dims_.hidden, count);
+    if (dims_.dense()) {
+      const ops::FfnBuffers ffn{normalized, intermediate_, scratch_, ffnTable_};
+      linear_.addSwiGlu(graph, {&w.ffnGate, &w.ffnUp, &w.ffnDown}, ffn, nextRows, residualRows, count, prepared);
+      return;
+    }
+    if (w.routerRows) {
+      ops::FloatProjection::add(graph, normalized, w.routerRows, scores_, count, dims_.experts, 0, ops::FloatOutput::Float32);
+    } else {
+      ops::LinearBuffers router;
+      router.input = normalized;
+      router.output = scores_;
+      router.scratch = scratch_;
+      router.prepared = prepared;
+      linear_.add(graph, router, w.router, linear_.plan(w.router, count));
+    }
+    ops::MoE::addRouting(graph, scores_, dims_.experts, moeWorkspace_, moe, count, normalized, w.sharedScalarGate);
+    ops::MoE::addRouted(graph, normalized, nextRows, residualRows, w.experts, moeWorkspace_, moe, count, {});
+  });
+}
+
+void HybridVerify::encodePrefill(hip::CommandGraph &graph, uint32_t lane, uint32_t tableFirst, uint32_t committed, uint32_t tokens,
+                                 uint32_t parity, uint32_t firstLayer, uint32_t layerCount) {
+  if (!tokens || tokens > rowCapacity_) throw std::invalid_argument("a prompt chunk takes 1 to the driver's most prefill rows");
+  if (lane >= maxLanes_) throw std::invalid_argument("no such lane");
+  if (firstLayer >= dims_.layers || layerCount > dims_.layers - firstLayer) throw std::invalid_argument("no such layers");
+  const ops::AttentionChunkPlan plan = ops::PagedAttention::planChunks(
+      {dims_.qHeads, dims_.kvHeads, dims_.headDimension, dims_.rotaryPairs, dims_.normalizeHeads, dims_.gatedAttention},
+      {{0, tokens, committed, tableFirst}});
+  if (firstLayer == 0) {
+    if (dims_.rotaryPairs) {
+      // the RoPE tables eight blocks a dispatch, each dispatch over its own rows of the depths and tables
+      const uint32_t span = ATTENTION_MAXIMUM_SEQUENCES * ATTENTION_MAXIMUM_ROWS;
+      const uint64_t tableBytes = uint64_t{dims_.rotaryPairs} * 4;
+      for (uint32_t first = 0; first < tokens; first += span) {
+        const uint32_t count = std::min(span, tokens - first);
+        std::vector<ops::RopeSequence> rope;
+        for (uint32_t at = 0; at < count; at += ATTENTION_MAXIMUM_ROWS)
+          rope.push_back({at, std::min<uint32_t>(ATTENTION_MAXIMUM_ROWS, count - at), committed + first + at});
+        ops::RoPE::addTreeTables(graph, inverseFrequency_, rowsOf(depths_, first, count, 4), rowsOf(ropeCos_, first, count, tableBytes),
+                                 rowsOf(ropeSin_, first, count, tableBytes), dims_.rotaryPairs, rope);
+      }
+    }
+    encodeEmbedding(graph, tokens);
+  }
+  const uint32_t end = layerCount ? firstLayer + layerCount : dims_.layers;
+  for (uint32_t layer = firstLayer; layer < end; ++layer)
+    encodePrefillLayer(graph, layer, plan, tokens, cellOffset(lane, parity), cellOffset(lane, parity ^ 1u));
 }
 
 } // namespace splash::model

@@ -102,8 +102,10 @@ struct HybridLane final {
 
 class HybridVerify final {
 public:
+  // prefillRows: the most rows of a prompt chunk (encodePrefill), 0 for a step's most, up to ops::kMaximumChunkRows.
   HybridVerify(hip::Backend &backend, HybridDimensions dimensions, uint32_t maxLanes, uint32_t physicalPages,
-               uint32_t pageTableEntries);
+               uint32_t pageTableEntries, uint32_t prefillRows = 0);
+  [[nodiscard]] uint32_t prefillRows() const noexcept { return rowCapacity_; }
 
   [[nodiscard]] const HybridDimensions &dimensions() const noexcept { return dims_; }
   HybridWeights &weights() noexcept { return weights_; }
@@ -150,8 +152,21 @@ public:
   void encodeLayer(hip::CommandGraph &graph, uint32_t layer, const std::vector<HybridLane> &lanes, bool inputReady = false,
                    bool feedsNext = false);
   void encodeHead(hip::CommandGraph &graph, uint32_t rows, bool inputReady = false);
+  // A chunk of `tokens` prompt tokens (1 to prefillRows(); inputs where a step's are: tokens, a chain of tree rows a block
+  // of sixteen, each row's depth in its block) of the sequence of lane `lane`, `committed` tokens already cached, through
+  // layers [firstLayer, firstLayer + layerCount) (layerCount 0: to the last) and no head: the counterpart of the
+  // reference's chunked prefill over its hybrid target (QwenTarget.cpp:206-347 with GDN::addPrefill, GDN.cpp:132-222, and
+  // the plan over kv::ChunkedPrefillParams, PagedAttention.cpp:351-389). Attention layers store the chunk's keys and
+  // values and attend causally (ops::PagedAttention::planChunks); Gated DeltaNet layers take every row into the state
+  // (ops::GDN::addPrefill), from the lane's cell of `parity` to its other cell, so the lane's next step has the other
+  // parity and no pending path. The embedding runs with firstLayer 0. Projections and experts run in windows of
+  // ops::kMaximumDispatchRows rows.
+  void encodePrefill(hip::CommandGraph &graph, uint32_t lane, uint32_t tableFirst, uint32_t committed, uint32_t tokens, uint32_t parity,
+                     uint32_t firstLayer = 0, uint32_t layerCount = 0);
 
 private:
+  void encodePrefillLayer(hip::CommandGraph &graph, uint32_t layer, const ops::AttentionChunkPlan &plan, uint32_t tokens, uint64_t currentCell,
+                          uint64_t nextCell);
   [[nodiscard]] ops::AttentionPlan planOf(const std::vector<HybridLane> &lanes) const;
   [[nodiscard]] hip::Buffer rowsOf(const hip::Buffer &buffer, uint32_t first, uint32_t count, uint64_t rowBytes) const {
     return backend_.view(buffer, first * rowBytes, count * rowBytes);
@@ -161,8 +176,9 @@ private:
   HybridDimensions dims_;
   HybridWeights weights_;
   ops::Linear linear_;
-  uint32_t maxRows_ = 0, maxLanes_ = 0;
+  uint32_t maxRows_ = 0, maxLanes_ = 0, rowCapacity_ = 0;
   bool tiledGdnHeads_ = false;
+  ops::GdnPrefillBuffers gdnPrefill_;  // the rows a GDN layer's prefill passes hand each other (a long chunk's)
   uint64_t pageBytes_ = 0, layerBytes_ = 0, cellBytes_ = 0, tapeLayerBytes_ = 0;
   ops::GdnStateStrides strides_;
   hip::Buffer kvAll_, states_, tape_;

@@ -182,8 +182,10 @@ class HybridVerify:
 
     def __init__(self, backend, hidden, vocabulary, layers, q_heads, kv_heads, head_dim, gdn_key_heads, gdn_value_heads, experts, top_k,
                  expert_ffn, attention_interval=4, rotary_pairs=None, normalize_heads=True, rope_theta=1e6, gdn_packed_width=None,
-                 max_lanes=1, physical_pages=2, page_table_entries=None, gated_attention=False, shared_slices=0, shared_gate=False, dense_ffn=0):
-        """experts 0 and dense_ffn: every layer's FFN is a dense SwiGLU of that width instead of a mixture of experts."""
+                 max_lanes=1, physical_pages=2, page_table_entries=None, gated_attention=False, shared_slices=0, shared_gate=False, dense_ffn=0,
+                 prefill_rows=0):
+        """experts 0 and dense_ffn: every layer's FFN is a dense SwiGLU of that width instead of a mixture of experts.
+        prefill_rows: the most rows of a prompt chunk (encode_prefill); 0: a step's most."""
         self.backend = backend
         pairs = head_dim // 2 if rotary_pairs is None else rotary_pairs
         conv = (2 * gdn_key_heads + gdn_value_heads) * 128
@@ -193,7 +195,8 @@ class HybridVerify:
                                          shared_slices, int(shared_gate), dense_ffn)
         h = ctypes.c_void_p()
         entries = page_table_entries if page_table_entries is not None else physical_pages
-        check(lib.spo_hybrid_verify_create(backend.handle, ctypes.byref(self.dims), max_lanes, physical_pages, entries, ctypes.byref(h)))
+        check(lib.spo_hybrid_verify_create_chunked(backend.handle, ctypes.byref(self.dims), max_lanes, physical_pages, entries, prefill_rows,
+                                                   ctypes.byref(h)))
         self.handle = h
         self.physical_pages = physical_pages
         page, cell, tape = ctypes.c_uint64(), ctypes.c_uint64(), ctypes.c_uint64()
@@ -210,7 +213,7 @@ class HybridVerify:
             pass
 
     @classmethod
-    def from_gguf(cls, backend, gguf_file, max_lanes=1, physical_pages=2, page_table_entries=None):
+    def from_gguf(cls, backend, gguf_file, max_lanes=1, physical_pages=2, page_table_entries=None, prefill_rows=0):
         """A driver of the geometry the file's metadata names (architectures qwen35 and qwen35moe), every weight loaded
         from the file (spg_hybrid_dimensions, spo_hybrid_verify_load_gguf)."""
         d = nat.HybridDimensions()
@@ -219,7 +222,7 @@ class HybridVerify:
                    d.top_k, d.expert_ffn, attention_interval=d.attention_interval, rotary_pairs=d.rotary_pairs,
                    normalize_heads=bool(d.normalize_heads), rope_theta=d.rope_theta, gdn_packed_width=d.gdn_packed_width, max_lanes=max_lanes,
                    physical_pages=physical_pages, page_table_entries=page_table_entries, gated_attention=bool(d.gated_attention),
-                   shared_slices=d.shared_slices, shared_gate=bool(d.shared_gate), dense_ffn=d.dense_ffn)
+                   shared_slices=d.shared_slices, shared_gate=bool(d.shared_gate), dense_ffn=d.dense_ffn, prefill_rows=prefill_rows)
         check(lib.spo_hybrid_verify_load_gguf(self.handle, gguf_file.handle))
         self._keep.append(gguf_file)
         return self
@@ -277,7 +280,18 @@ class HybridVerify:
         graph._keep.append(self)
         return graph
 
+    def encode_prefill(self, lane, table_first, committed, tokens, parity=0, first_layer=0, layer_count=0, graph=None):
+        """A chunk of `tokens` prompt tokens of lane `lane`'s sequence through layers [first_layer, first_layer + layer_count)
+        (0: to the last; the embedding with first_layer 0), no head; the GDN layers go from the lane's cell of `parity` to
+        its other cell. Inputs as set_prefill_block writes them."""
+        graph = graph or CommandGraph()
+        check(lib.spo_hybrid_verify_encode_prefill(self.handle, graph.handle, lane, table_first, committed, tokens, parity, first_layer,
+                                                   layer_count))
+        graph._keep.append(self)
+        return graph
+
     set_block = DenseVerify.set_block
+    set_prefill_block = DenseVerify.set_prefill_block
     results = DenseVerify.results
     _results_call = "spo_hybrid_verify_results"
 

@@ -88,7 +88,7 @@ class HybridModel:
         return (layer + 1) % self.dims["attention_interval"] == 0
 
     # ------------------------------------------------------------------ GPU side
-    def build_gpu(self, backend, max_lanes, pages_per_lane):
+    def build_gpu(self, backend, max_lanes, pages_per_lane, prefill_rows=0):
         d = self.dims
         self.pages_per_lane = pages_per_lane
         self.physical_pages = max_lanes * pages_per_lane + 1
@@ -96,7 +96,7 @@ class HybridModel:
                                   d["gdn_key_heads"], d["gdn_value_heads"], d["experts"], d["top_k"], d["expert_ffn"],
                                   attention_interval=d["attention_interval"], rope_theta=self.rope_theta, max_lanes=max_lanes,
                                   gated_attention=self.gated, shared_slices=self.shared_slices, shared_gate=self.shared_gate,
-                                  dense_ffn=self.dense_ffn,
+                                  dense_ffn=self.dense_ffn, prefill_rows=prefill_rows,
                                   physical_pages=self.physical_pages, page_table_entries=max_lanes * pages_per_lane)
         assert gpu.dims.gdn_packed_width == self.packed_width
         self.table = np.random.default_rng(99).permutation(self.physical_pages)[:max_lanes * pages_per_lane].astype(np.uint64)
@@ -134,13 +134,13 @@ class HybridModel:
         self.gpu = gpu
         return gpu
 
-    def build_gpu_from_file(self, backend, path, max_lanes, pages_per_lane):
+    def build_gpu_from_file(self, backend, path, max_lanes, pages_per_lane, prefill_rows=0):
         """The driver of the model's GGUF (hybrid_model_file): geometry and weights as the loader reads them."""
         from splash_amd import gguf
         self.pages_per_lane = pages_per_lane
         self.physical_pages = max_lanes * pages_per_lane + 1
         gpu = verify.HybridVerify.from_gguf(backend, gguf.GgufFile(str(path)), max_lanes=max_lanes, physical_pages=self.physical_pages,
-                                            page_table_entries=max_lanes * pages_per_lane)
+                                            page_table_entries=max_lanes * pages_per_lane, prefill_rows=prefill_rows)
         assert gpu.dims.gdn_packed_width == self.packed_width
         self.table = np.random.default_rng(99).permutation(self.physical_pages)[:max_lanes * pages_per_lane].astype(np.uint64)
         gpu.buffer(verify.PAGE_TABLE).upload(self.table)
@@ -249,6 +249,40 @@ class HybridModel:
             first += rows
         out = np.concatenate(out)
         if self.gated:      # attention_gate.h:27-31: bf16(bf16(value) * sigmoid(gate))
+            sigmoid = np.float32(1) / (np.float32(1) + np.exp2(np.float32(-1.44269504089) * gates))
+            out = orc.f32_to_bf16((orc.bf16_to_f32(out) * sigmoid).astype(np.float32))
+        return out
+
+    def oracle_attention_chunk(self, packed, li, table_first, committed):
+        """A prompt chunk's attention rows: every row's K/V stored into the layer's context arrays, then each tile of
+        sixteen rows a block of the sequence that ends at its last row."""
+        d, w = self.dims, self.layers[li]
+        D, pairs, tokens = d["head_dim"], d["head_dim"] // 2, packed.shape[0]
+        kc, ks, vc, vs = self.context[li // d["attention_interval"]]
+        inv = np.array([self.rope_theta ** (-i / pairs) for i in range(pairs)]).astype(np.float32)
+        gates = None
+        if self.gated:
+            heads = packed[:, :d["q_heads"] * 2 * D].reshape(-1, d["q_heads"], 2, D)
+            gates = orc.bf16_to_f32(heads[:, :, 1]).reshape(-1, d["q_heads"] * D)
+            packed = np.concatenate([heads[:, :, 0].reshape(-1, d["q_heads"] * D), packed[:, d["q_heads"] * 2 * D:]], axis=1)
+        table = self.table[table_first:table_first + self.pages_per_lane].astype(np.uint32)
+        angle = ((committed + np.arange(tokens)).astype(np.float32)[:, None] * inv[None, :]).astype(np.float32)
+        cosv, sinv = np.cos(angle.astype(np.float64)).astype(np.float32), np.sin(angle.astype(np.float64)).astype(np.float32)
+        q, kf, vf = orc.attention_prepare(d["q_heads"], d["kv_heads"], D, packed, w["q_norm"], w["k_norm"], cosv, sinv, pairs)
+        kcod, kscl = orc.kv_quantize(kf)
+        vcod, vscl = orc.kv_quantize(vf)
+        for r in range(tokens):
+            t = committed + r
+            p, s = table[t // ops.PAGE_TOKENS], t % ops.PAGE_TOKENS
+            kc[p, :, s], ks[p, :, s], vc[p, :, s], vs[p, :, s] = kcod[r], kscl[r], vcod[r], vscl[r]
+        out = []
+        for first in range(0, tokens, 16):
+            rows = min(16, tokens - first)
+            anc = np.array([(2 << r) - 1 for r in range(rows)], dtype=np.uint32)
+            attn, _ = orc.attention(np.ascontiguousarray(q[first:first + rows]), kc, ks, vc, vs, table, anc, committed + first, want64=False)
+            out.append(attn.reshape(rows, d["q_heads"] * D))
+        out = np.concatenate(out)
+        if self.gated:
             sigmoid = np.float32(1) / (np.float32(1) + np.exp2(np.float32(-1.44269504089) * gates))
             out = orc.f32_to_bf16((orc.bf16_to_f32(out) * sigmoid).astype(np.float32))
         return out

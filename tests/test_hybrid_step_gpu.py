@@ -7,6 +7,7 @@ import pytest
 
 from splash_amd import ops, verify
 from tests import oracle as orc
+from tests.gdn_case import ulps
 from tests.hybrid_reference import HybridModel
 from tests.test_verify_step_gpu import close_bf16
 
@@ -188,3 +189,68 @@ def test_hybrid_rejects_bad_arguments(backend):
     gpu = verify.HybridVerify(backend, **SHAPE, max_lanes=1)
     with pytest.raises(ValueError):
         gpu.encode([verify.HybridLane(4, 0), verify.HybridLane(4, 0)])    # more lanes than it was built for
+
+
+@pytest.mark.parametrize("tokens,file_form", [(100, False), (300, True)])
+def test_a_prompt_chunk_through_the_hybrid_layers(backend, tmp_path, tokens, file_form):
+    """HybridVerify.encode_prefill: a prompt chunk of one lane, every layer against the oracle from the GPU's own layer
+    input -- an attention layer's rows from the history and the chunk's rows up to each (tile by tile as blocks of the
+    sequence), a Gated DeltaNet layer's rows and the cell it leaves from orc_gdn_prefill -- and then a verify step of the
+    lane from the cell and the pages the chunk left (the other parity, nothing pending), checked as any step is."""
+    from tests.hybrid_reference import hybrid_model_file
+    print(f"case hybrid prompt chunk tokens={tokens} file_form={file_form}", flush=True)
+    model = HybridModel(seed=47, **SHAPE, shared_slices=1, shared_gate=True, gated_attention=file_form, file_form=file_form)
+    if file_form:
+        gpu = model.build_gpu_from_file(backend, hybrid_model_file(tmp_path / "m.gguf", model), max_lanes=1, pages_per_lane=3, prefill_rows=320)
+    else:
+        gpu = model.build_gpu(backend, max_lanes=1, pages_per_lane=3, prefill_rows=128)
+    rng = np.random.default_rng(12)
+    model.seed_context(rng)
+    model.seed_states(rng, lanes=1)
+    d = model.dims
+    H, V, committed = d["hidden"], d["vocabulary"], 200
+    prompt = rng.integers(0, V, tokens).astype(np.uint32)
+    gpu.set_prefill_block(prompt)
+    hidden_of = lambda i=0: gpu.buffer(verify.HIDDEN, i).download(np.uint16, tokens * H).reshape(tokens, H)
+    before = model.oracle_embedding(prompt)
+    for layer in range(d["layers"]):
+        print(f"  layer {layer} ({'attention' if model.attends(layer) else 'GDN'})", flush=True)
+        g = gpu.mixer_index(layer)
+        if layer:
+            before = hidden_of()
+        if not model.attends(layer):
+            conv_in, state_in = model.read_cell(0, 0, g)
+        backend.run(gpu.encode_prefill(0, 0, committed, tokens, parity=0, first_layer=layer, layer_count=1))
+        packed = model.oracle_mixer_input(before, layer)
+        if model.attends(layer):
+            mixed = model.oracle_attention_chunk(packed, layer, 0, committed)
+        else:
+            w = model.layers[layer]
+            want = orc.gdn_prefill(model.gdn_shape, packed, w["conv_w"], w["a_scale"], w["dt_bias"], w["mixer_norm"], conv_in, state_in)
+            mixed = want["hidden"]
+            conv, state = model.read_cell(0, 1, g)
+            # the carry is the chunk's last packed rows, which the GPU's projection and the oracle's exact sums round apart
+            # now and then
+            ok, detail = close_bf16(conv, want["conv_out"])
+            assert ok and (ulps(conv, want["conv_out"]) > 0).mean() < 0.01, (layer, detail)
+            assert np.abs(state - want["state_out"]).max() <= 2e-3 * np.abs(want["state_out"]).max(), layer
+        ok, detail = close_bf16(hidden_of(1), model.oracle_mixer_output(mixed, before, layer))
+        assert ok, ("mixer", layer, detail)
+        scores, want = model.oracle_ffn(hidden_of(1), layer)
+        sure = sure_routes(scores, d["top_k"])
+        assert sure.mean() >= 0.9
+        ok, detail = close_bf16(hidden_of()[sure], want[sure])
+        assert ok, ("ffn", layer, detail)
+    if layer == 0:
+        assert np.array_equal(before, model.oracle_embedding(prompt))
+    # the chunk in one graph leaves the same pages, cells and rows as its layers one by one
+    pools = lambda: np.concatenate([gpu.buffer(verify.KV_POOL, a).download(np.uint8) for a in range(d["layers"] // d["attention_interval"])])
+    cells = lambda: gpu.buffer(verify.GDN_STATES).download(np.uint8).copy()
+    want_pools, want_cells, want_hidden = pools(), cells(), hidden_of().copy()
+    backend.run(gpu.encode_prefill(0, 0, committed, tokens, parity=0))
+    assert np.array_equal(pools(), want_pools) and np.array_equal(cells(), want_cells) and np.array_equal(hidden_of(), want_hidden)
+    # a verify step of the lane after the chunk
+    lanes = [verify.HybridLane(7, committed + tokens, table_first=0, pending_path=0, parity=1)]
+    check_step(backend, model, gpu, lanes, rng.integers(0, V, 7).astype(np.uint32))
+    with pytest.raises(ValueError):
+        gpu.encode_prefill(0, 0, committed, 321 if file_form else 129)
