@@ -468,6 +468,15 @@ sp_status spo_draft_add_verify_children(spo_graph *graph, sp_buffer *verify_sour
 sp_status spo_draft_add_verify_rows(spo_graph *graph, sp_buffer *tree_tokens, sp_buffer *trees, sp_buffer *tree_scores,
                                     sp_buffer *tree_sizes, sp_buffer *input_tokens, sp_buffer *tree_rows, sp_buffer *lane_rows,
                                     sp_buffer *verify_sources, uint32_t lanes, uint32_t rows, uint32_t lane_cap, float floor);
+/* The same layout in slots (no counterpart in the reference, whose kernels read each lane's rows from the device,
+ * SplashLaneRows, where a step's lanes here are fixed when its graph is recorded): lane l's rows are rows l * lane_cap on,
+ * its anchor and the best rows of its tree at or above the floor, up to lane_cap; the rest of its slot are inert rows
+ * (token 0xFFFFFFFF, whose embedding is zero and which no row selects; on no path but their own; a child of the anchor
+ * that never follows it; no source). A step recorded once for lane_cap rows a lane then takes trees of any size the
+ * device grows: lane_rows[l] is {l * lane_cap, the rows the lane took}. */
+sp_status spo_draft_add_verify_row_slots(spo_graph *graph, sp_buffer *tree_tokens, sp_buffer *trees, sp_buffer *tree_scores,
+                                         sp_buffer *tree_sizes, sp_buffer *input_tokens, sp_buffer *tree_rows, sp_buffer *lane_rows,
+                                         sp_buffer *verify_sources, uint32_t lanes, uint32_t lane_cap, float floor);
 
 /* ---- The dense verify step (the reference's model layer: QwenTarget.cpp:206-395, :457-496;
  *      Runtime.cpp:2677-2717, :2883-2892) ---- */

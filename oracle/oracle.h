@@ -164,6 +164,12 @@ uint32_t orc_accept_tree(const struct OrcTreeRow *tree, const uint32_t *tokens, 
 void orc_draft_verify_rows(const uint32_t *tree_tokens, const struct OrcTreeRow *trees, const float *scores, const uint32_t *sizes,
                            uint32_t lanes, uint32_t rows, uint32_t lane_cap, float floor, uint32_t *tokens, struct OrcTreeRow *tree,
                            uint32_t *lane_rows, uint32_t *sources);
+// The same rows in slots (a layout of this build; see abi/Sampling.h): lane l's rows from row l * lane_cap on, the rest of its
+// slot inert. Pinned by its relation to the packed layout above and by what makes a row inert to the step
+// (tests/test_oracle_sampling.py).
+void orc_draft_verify_row_slots(const uint32_t *tree_tokens, const struct OrcTreeRow *trees, const float *scores, const uint32_t *sizes,
+                                uint32_t lanes, uint32_t lane_cap, float floor, uint32_t *tokens, struct OrcTreeRow *tree,
+                                uint32_t *lane_rows, uint32_t *sources);
 // sampling.metal:1357-1766 draft_select_tree for one lane: candidates uint32 [7][16], unary fp32 [7][16], edges fp32
 // [7][16][16] ([position][predecessor][candidate]; position 0 reads predecessor 0 alone), the lane's host chain (15 tokens, a
 // rate for each of 4 agreements a token) and parameters (Sampling.h:242-252, one lane's). Outputs, 16 rows: tokens, tree

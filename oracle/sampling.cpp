@@ -254,6 +254,29 @@ void orc_draft_verify_rows(const uint32_t *tree_tokens, const struct OrcTreeRow 
   }
 }
 
+// The same rows in slots: lane l's from row l * lane_cap on (every lane may take its cap, so the step's rows never bind),
+// the rest of its slot inert rows -- no token, on no path but their own, a child of the anchor, no source.
+void orc_draft_verify_row_slots(const uint32_t *tree_tokens, const struct OrcTreeRow *trees, const float *scores, const uint32_t *sizes,
+                                uint32_t lanes, uint32_t lane_cap, float floor, uint32_t *tokens, struct OrcTreeRow *tree,
+                                uint32_t *lane_rows, uint32_t *sources) {
+  const uint32_t rows = lanes * lane_cap;
+  std::vector<uint32_t> packed_tokens(rows), packed_sources(rows), packed_lanes(2 * lanes);
+  std::vector<OrcTreeRow> packed_tree(rows);
+  orc_draft_verify_rows(tree_tokens, trees, scores, sizes, lanes, rows, lane_cap, floor, packed_tokens.data(), packed_tree.data(),
+                        packed_lanes.data(), packed_sources.data());
+  for (uint32_t lane = 0; lane < lanes; ++lane) {
+    const uint32_t from = packed_lanes[2 * lane], mine = packed_lanes[2 * lane + 1], first = lane * lane_cap;
+    for (uint32_t row = 0; row < lane_cap; ++row) {
+      const bool own = row < mine;
+      tokens[first + row] = own ? packed_tokens[from + row] : ORC_NO_TOKEN;
+      tree[first + row] = own ? packed_tree[from + row] : OrcTreeRow{1u << row, uint16_t(0), uint16_t(1)};
+      sources[first + row] = own ? packed_sources[from + row] : ORC_NO_TOKEN;
+    }
+    lane_rows[2 * lane] = first;
+    lane_rows[2 * lane + 1] = mine;
+  }
+}
+
 uint32_t orc_argmax(const float *logits, uint32_t vocab) {
   float best = -std::numeric_limits<float>::infinity();
   uint32_t index = ORC_NO_TOKEN;

@@ -304,6 +304,7 @@ class DraftTreeLane(ctypes.Structure):
 _sig("spo_draft_add_tree", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, P(DraftTreeLane), c_u32)
 _sig("spo_draft_add_verify_children", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_u32, c_u32)
 _sig("spo_draft_add_verify_rows", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_u32, c_u32, c_u32, ctypes.c_float)
+_sig("spo_draft_add_verify_row_slots", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_u32, c_u32, ctypes.c_float)
 _sig("spo_sampling_add_acceptance", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, P(LaneRows), P(c_u32), c_u32, P(c_u32))
 _sig("spo_sampling_greedy_rows_static", c_int, ctypes.c_void_p, c_u32, c_u32, c_u32, ctypes.c_void_p, ctypes.c_void_p)
 _sig("spo_verify_check_results", c_int, P(LaneRows), P(c_u32), c_u32, c_u32, c_u32, P(c_u32), P(c_u32), P(c_u32), P(c_u32))

@@ -60,11 +60,18 @@ struct TargetSamplingParams {
 // tree's other rows by estimate that the step's rows and the lanes' cap hold, none estimated below `floor`; the rows
 // past the lanes' belong to no lane.
 #define SAMPLING_TREE_ROOT 0xFFFFu  // the parent of a row without one (SPLASH_TREE_ROOT)
+// With `slots` the rows are not packed: lane l's rows are rows l * lane_cap on (rows == lanes * lane_cap), and the rows of
+// its slot past its own are inert -- token SAMPLING_NO_TOKEN (which no row selects, and whose embedding is zero), on no
+// path but their own, a child of the anchor that never follows it -- so that a step recorded for lane_cap rows a lane
+// takes trees of any size the device grows, with no word from the host. No counterpart in the reference, whose kernels
+// read each lane's rows from the device (SplashLaneRows) where these kernels' lanes are fixed when a step is recorded.
 struct VerifyRowsParams {
   uint32_t lanes;
   uint32_t rows;
   uint32_t lane_cap;
   float floor;
+  uint32_t slots;
+  uint32_t reserved[3];
 };
 
 // draft_select_top16_sharded, draft_select_edges (the reference's SelectorBatchParams, abi/Sampling.h:184-194, and
@@ -139,6 +146,6 @@ static_assert(sizeof(TargetSamplingParams) == 16 + 32 + 16 + 64 + 96 + 32, "targ
 static_assert(sizeof(DraftSelectParams) == 32 + 32, "draft selector parameters are 64 bytes on both sides");
 static_assert(sizeof(DraftTreeParams) == 4 * 32 + 16 + 32 + 224 + 32 + 64, "draft tree parameters are 496 bytes on both sides");
 static_assert(sizeof(VerifyChildrenParams) == 16, "verify children parameters are 16 bytes on both sides");
-static_assert(sizeof(VerifyRowsParams) == 16, "verify rows parameters are 16 bytes on both sides");
+static_assert(sizeof(VerifyRowsParams) == 32, "verify rows parameters are 32 bytes on both sides");
 static_assert(sizeof(AcceptBatchParams) == 16 + 32 + 16 + 64, "acceptance parameters are 128 bytes on both sides");
 #endif

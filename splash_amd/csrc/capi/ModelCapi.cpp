@@ -195,6 +195,18 @@ sp_status spo_draft_add_verify_rows(spo_graph *graph, sp_buffer *tree_tokens, sp
   });
 }
 
+sp_status spo_draft_add_verify_row_slots(spo_graph *graph, sp_buffer *tree_tokens, sp_buffer *trees, sp_buffer *tree_scores,
+                                         sp_buffer *tree_sizes, sp_buffer *input_tokens, sp_buffer *tree_rows, sp_buffer *lane_rows,
+                                         sp_buffer *verify_sources, uint32_t lanes, uint32_t lane_cap, float floor) {
+  return capi::guard([&] {
+    capi::require(graph, "graph");
+    ops::DraftSelector::addVerifyRows(capi::graphOf(graph),
+                                      {B(tree_tokens), B(trees), B(tree_scores), B(tree_sizes), B(input_tokens), B(tree_rows), B(lane_rows),
+                                       B(verify_sources)},
+                                      {lanes, lanes * lane_cap, lane_cap, true}, floor);
+  });
+}
+
 sp_status spo_dense_verify_create(sp_backend *backend, const spo_dense_dimensions *d, uint32_t max_lanes, uint32_t physical_pages,
                                   uint32_t page_table_entries, spo_dense_verify **out) {
   return spo_dense_verify_create_chunked(backend, d, max_lanes, physical_pages, page_table_entries, 0, out);

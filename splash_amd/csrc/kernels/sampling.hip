@@ -148,6 +148,7 @@ __global__ __launch_bounds__(128) void draft_verify_rows(const uint32_t *__restr
     first += l < lane ? takenOf[l] + 1u : 0u;
     total += takenOf[l] + 1u;
   }
+  if (p.slots) first = lane * p.lane_cap;
   const bool placed = row < mine;
   const AttentionTreeRow node = placed ? trees[t] : AttentionTreeRow{0u, 0u, 0u};
   pathOf[t] = placed ? node.ancestors : 0u;
@@ -175,6 +176,15 @@ __global__ __launch_bounds__(128) void draft_verify_rows(const uint32_t *__restr
     sources[first + place] = row;
   }
   if (lane < lanes && row == 0) lane_rows[lane] = SamplingLaneRows{first, mine};
+  if (p.slots) {
+    // the rows of a lane's slot past its own: inert
+    if (lane < lanes && row >= mine && row < p.lane_cap) {
+      tokens[first + row] = SAMPLING_NO_TOKEN;
+      tree[first + row] = AttentionTreeRow{1u << row, uint16_t(0), uint16_t(1)};
+      sources[first + row] = SAMPLING_NO_TOKEN;
+    }
+    return;
+  }
   for (uint32_t spare = total + t; spare < p.rows; spare += kAll) {
     tokens[spare] = tree_tokens[0];
     tree[spare] = AttentionTreeRow{0u, uint16_t(SAMPLING_TREE_ROOT), uint16_t(0)};

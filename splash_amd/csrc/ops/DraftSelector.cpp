@@ -104,6 +104,7 @@ void DraftSelector::addVerifyRows(hip::CommandGraph &graph, const DraftVerifyRow
   if (!step.lanes || step.lanes > SAMPLING_MAXIMUM_LANES || !step.laneCap || step.laneCap > SAMPLING_MAXIMUM_ROWS ||
       step.rows < step.lanes || step.rows > uint64_t{step.lanes} * step.laneCap)
     throw std::invalid_argument("invalid decode step rows");
+  if (step.slots && step.rows != step.lanes * step.laneCap) throw std::invalid_argument("rows in slots are a lane cap of rows a lane");
   if (!(floor >= 0.0f) || !std::isfinite(floor)) throw std::invalid_argument("invalid verify rows floor");
   const uint64_t treeRows = uint64_t{step.lanes} * SAMPLING_MAXIMUM_ROWS;
   requireBytes(b.treeTokens, treeRows * 4, "draft tree token");
@@ -115,7 +116,7 @@ void DraftSelector::addVerifyRows(hip::CommandGraph &graph, const DraftVerifyRow
   requireBytes(b.laneRows, uint64_t{step.lanes} * sizeof(SamplingLaneRows), "verify lane rows");
   requireBytes(b.verifySources, uint64_t{step.rows} * 4, "verify source");
   graph.add("draft_verify_rows", {b.treeTokens, b.trees, b.treeScores, b.treeSizes, b.inputTokens, b.treeRows, b.laneRows, b.verifySources},
-            VerifyRowsParams{step.lanes, step.rows, step.laneCap, floor}, {1, 1, 1}, {128, 1, 1});
+            VerifyRowsParams{step.lanes, step.rows, step.laneCap, floor, step.slots ? 1u : 0u, {}}, {1, 1, 1}, {128, 1, 1});
 }
 
 } // namespace splash::ops

@@ -18,6 +18,9 @@ struct StepRows final {
   uint32_t lanes = 0;
   uint32_t rows = 0;
   uint32_t laneCap = 0;
+  // Not packed: lane l's rows from row l * laneCap on (rows == lanes * laneCap), the rest of its slot inert rows, so that
+  // a step recorded for laneCap rows a lane takes trees of any size (abi/Sampling.h, VerifyRowsParams::slots).
+  bool slots = false;
 };
 
 struct DraftVerifyRowsBuffers final {

@@ -487,6 +487,15 @@ class DraftSelector:
         graph._keep.extend(buffers)
 
 
+    @staticmethod
+    def add_verify_row_slots(graph, tree_tokens, trees, tree_scores, tree_sizes, input_tokens, tree_rows, lane_rows, verify_sources, lanes,
+                             lane_cap, floor=0.0):
+        """The verify rows in slots: lane l's rows from row l * lane_cap on, the rest of its slot inert."""
+        buffers = [tree_tokens, trees, tree_scores, tree_sizes, input_tokens, tree_rows, lane_rows, verify_sources]
+        check(lib.spo_draft_add_verify_row_slots(graph.handle, *[b.handle for b in buffers], lanes, lane_cap, floor))
+        graph._keep.extend(buffers)
+
+
 def chain_tree_rows(rows_per_sequence):
     """SplashTreeRow of chains: ancestors (2 << r) - 1, parent r - 1, depth r, packed per sequence."""
     out = []

@@ -631,6 +631,23 @@ def draft_verify_rows(tree_tokens, trees, scores, sizes, rows, lane_cap, floor=0
     return tokens, tree, lane_rows, sources
 
 
+def draft_verify_row_slots(tree_tokens, trees, scores, sizes, lane_cap, floor=0.0):
+    """The verify rows in slots: lane l's rows from row l * lane_cap on, the rest of its slot inert."""
+    lanes = len(sizes)
+    rows = lanes * lane_cap
+    tree_tokens = np.ascontiguousarray(tree_tokens, dtype=np.uint32)
+    trees = np.ascontiguousarray(trees, dtype=TREE_DTYPE)
+    scores = np.ascontiguousarray(scores, dtype=np.float32)
+    sizes = np.ascontiguousarray(sizes, dtype=np.uint32)
+    tokens, tree = np.zeros(rows, np.uint32), np.zeros(rows, TREE_DTYPE)
+    lane_rows, sources = np.zeros((lanes, 2), np.uint32), np.zeros(rows, np.uint32)
+    lib.orc_draft_verify_row_slots.restype = None
+    lib.orc_draft_verify_row_slots(_p(tree_tokens, u32p), trees.ctypes.data_as(ctypes.c_void_p), _p(scores, f32p), _p(sizes, u32p), c_u32(lanes),
+                                   c_u32(lane_cap), c_f(floor), _p(tokens, u32p), tree.ctypes.data_as(ctypes.c_void_p),
+                                   _p(lane_rows, u32p), _p(sources, u32p))
+    return tokens, tree, lane_rows, sources
+
+
 class DraftTreeLane(ctypes.Structure):
     """One lane's DraftTreeParams (Sampling.h:242-252)."""
     _fields_ = [("anchor", c_u32), ("depth", c_u32), ("chain", c_u32), ("children", c_u32), ("slope", c_f), ("intercept", c_f * 7),

@@ -252,3 +252,67 @@ def test_a_tree_feeds_the_step_without_the_host(backend):
     assert np.array_equal(gpu.buffer(verify.LOGITS).download(np.float32, rows * V), device_logits)
     for got, want in zip(gpu.results([lane]), device_results):
         assert np.array_equal(got, want)
+
+
+def test_trees_of_any_size_feed_a_step_recorded_once(backend):
+    """Two greedy lanes whose drafts grow trees of different sizes on the device (sixteen rows and a chain of five): the
+    rows in slots (spo_draft_add_verify_row_slots) and their depths go straight into the dense driver's input buffers of a
+    step recorded, before any of it, for sixteen rows a lane. What each lane keeps, and its own rows' logits, are those
+    of the step a host records for the trees' exact sizes from the packed layout of the same trees."""
+    from splash_amd import verify
+    from tests.dense_reference import DenseModel
+    print("case trees of any size into one recorded step", flush=True)
+    V, cap, contexts = 32000, 16, (200, 300)
+    model = DenseModel(seed=22, hidden=1024, q_heads=16, kv_heads=8, head_dim=64, ffn=3072, vocabulary=V, layers=2)
+    rng = np.random.default_rng(33)
+    gpu = model.build_gpu(backend, max_lanes=2, context_tokens=[c + 16 for c in contexts])
+    model.seed_context(gpu, None, rng)
+    lanes = [verify.Lane(cap, c, table_first=f) for c, f in zip(contexts, model.table_first)]
+    gpu.set_block(lanes, np.zeros(2 * cap, np.uint32))
+    step = gpu.encode(lanes, commit=False)             # the step's shape: sixteen rows a lane, whatever the trees will be
+    rank = 256
+    up = backend.from_array
+    logits = rng.normal(0, 2.0, (16, V)).astype(np.float32)
+    hidden = orc.f32_to_bf16(rng.normal(0, 1, (16, rank)).astype(np.float32))
+    before = orc.f32_to_bf16(rng.normal(0, 0.08, (V, rank)).astype(np.float32))
+    after = orc.f32_to_bf16(rng.normal(0, 0.08, (V, rank)).astype(np.float32))
+    anchors = [777, 4242]
+    draft_lanes = [dict(anchor=anchors[0], depth=15, children=3, intercept=[0.3] * 7), dict(anchor=anchors[1], depth=4, children=1, intercept=[0.3] * 7)]
+    b = dict(candidates=backend.allocate_buffer(2 * 7 * 16 * 4), unary=backend.allocate_buffer(2 * 7 * 16 * 4), edges=backend.allocate_buffer(2 * 7 * 256 * 4),
+             scratch=backend.allocate_buffer(ops.DraftSelector.candidate_scratch_bytes(2, V)), tokens=backend.allocate_buffer(128),
+             trees=backend.allocate_buffer(256), scores=backend.allocate_buffer(256), sizes=backend.allocate_buffer(16), draws=backend.allocate_buffer(128),
+             next=backend.allocate_buffer(2048), caps=backend.allocate_buffer(128), lane_rows=backend.allocate_buffer(16), sources=backend.allocate_buffer(128),
+             ids=backend.allocate_buffer(32 * 16 * 4), q=backend.allocate_buffer(32 * 16 * 4), drawn=backend.allocate_buffer(32 * 4))
+    draft = splash_amd.CommandGraph()
+    ops.DraftSelector.add_candidates(draft, up(logits), up(hidden), b["scratch"], b["candidates"], b["unary"], b["edges"], up(before), up(after),
+                                     V, V, V, anchors)
+    ops.DraftSelector.add_tree(draft, b["candidates"], b["unary"], b["edges"], up(np.zeros((2, 15), np.uint32)), up(np.zeros((2, 15, 4), np.float32)),
+                               b["tokens"], b["trees"], b["scores"], b["sizes"], b["draws"], b["next"], b["caps"], draft_lanes)
+    ops.DraftSelector.add_verify_row_slots(draft, b["tokens"], b["trees"], b["scores"], b["sizes"], gpu.buffer(verify.INPUT_TOKENS),
+                                           gpu.buffer(verify.TREE_ROWS), b["lane_rows"], b["sources"], 2, cap)
+    ops.DraftSelector.add_verify_children(draft, b["sources"], b["lane_rows"], gpu.buffer(verify.TREE_ROWS), b["candidates"], b["next"], b["draws"],
+                                          b["ids"], b["q"], b["drawn"], gpu.buffer(verify.DEPTHS), 2, 2 * cap)
+    backend.run(draft)
+    backend.run(step)
+    sizes = b["sizes"].download(np.uint32)[:2]
+    assert list(sizes) == [16, 5]
+    lane_rows = b["lane_rows"].download(np.uint32)[:4].reshape(2, 2)
+    assert lane_rows.tolist() == [[0, 16], [16, 5]]
+    selected, retained, accepted, masks = (np.array(a).copy() for a in gpu.results(lanes))
+    slot_logits = gpu.buffer(verify.LOGITS).download(np.float32, 2 * cap * V).reshape(2 * cap, V).copy()
+    # the host's step for the trees' exact sizes, from the packed layout of the device's own trees
+    tokens = b["tokens"].download(np.uint32)[:32].reshape(2, 16)
+    trees = b["trees"].download(np.uint8)[:256].view(orc.TREE_DTYPE).reshape(2, 16)
+    scores = b["scores"].download(np.float32)[:64].reshape(2, 16, 2)
+    w_tokens, w_tree, w_lane_rows, _ = orc.draft_verify_rows(tokens, trees, scores, sizes, 21, cap)
+    assert w_lane_rows.tolist() == [[0, 16], [16, 5]]
+    exact = [verify.Lane(16, contexts[0], table_first=model.table_first[0]), verify.Lane(5, contexts[1], table_first=model.table_first[1])]
+    gpu.set_block(exact, w_tokens, tree_rows=w_tree)
+    backend.run(gpu.encode(exact, commit=False))
+    e_selected, e_retained, e_accepted, e_masks = gpu.results(exact)
+    exact_logits = gpu.buffer(verify.LOGITS).download(np.float32, 21 * V).reshape(21, V)
+    assert np.array_equal(slot_logits[:21], exact_logits)     # lane 1's five rows follow lane 0's sixteen in both
+    assert list(retained) == list(e_retained) and list(accepted) == list(e_accepted) and list(masks) == list(e_masks)
+    assert np.array_equal(selected[:retained[0]], np.asarray(e_selected)[:retained[0]])
+    assert np.array_equal(selected[cap:cap + retained[1]], np.asarray(e_selected)[16:16 + retained[1]])
+    assert all(m >> 5 == 0 for m in [masks[1]])               # nothing past the chain's five rows is ever kept

@@ -430,6 +430,43 @@ def test_verify_rows_are_laid_out_from_the_trees(backend):
                                           backend.from_array(sizes), *out, lanes, lanes * lane_cap + 1, lane_cap, 0.0)
 
 
+def test_verify_rows_in_slots(backend):
+    """The slots layout against the oracle, bit for bit, and what makes it useful: the acceptance walk over a lane's whole
+    slot (the shape a step is recorded for) keeps what the walk over the lane's own rows keeps."""
+    print("case draft verify row slots", flush=True)
+    from tests.draft_case import grown_trees
+    rng = np.random.default_rng(38)
+    for trial in range(30):
+        lanes = int(rng.integers(1, 9))
+        tokens, trees, scores, sizes = grown_trees(rng, lanes, ties=trial % 3 == 0)
+        cap = int(rng.integers(1, 17))
+        rows = lanes * cap
+        floor = float(rng.choice([0.0, 0.3, 0.7]))
+        out = [backend.from_array(np.full(rows, 0xA5A5A5A5, np.uint32)), backend.from_array(np.zeros(rows, dtype=orc.TREE_DTYPE)),
+               backend.from_array(np.zeros((lanes, 2), np.uint32)), backend.from_array(np.full(rows, 0xA5A5A5A5, np.uint32))]
+        graph = splash_amd.CommandGraph()
+        ops.DraftSelector.add_verify_row_slots(graph, backend.from_array(tokens), backend.from_array(trees), backend.from_array(scores),
+                                               backend.from_array(sizes), *out, lanes, cap, floor)
+        backend.run(graph)
+        want = orc.draft_verify_row_slots(tokens, trees, scores, sizes, cap, floor)
+        got = (out[0].download(np.uint32), out[1].download(np.uint8).view(orc.TREE_DTYPE), out[2].download(np.uint32).reshape(lanes, 2),
+               out[3].download(np.uint32))
+        for g, w in zip(got, want):
+            assert np.array_equal(g, w), (trial, lanes, cap, floor)
+        selected = rng.integers(0, 40, rows).astype(np.uint32)
+        tb, ret, acc, mask = (backend.from_array(selected), backend.allocate_buffer(lanes * 4), backend.allocate_buffer(lanes * 4),
+                              backend.allocate_buffer(lanes * 4))
+        graph = splash_amd.CommandGraph()
+        ops.Sampling.add_acceptance(graph, out[0], out[1], tb, ret, acc, mask, [(l * cap, cap) for l in range(lanes)], [0xFFFFFFFF] * lanes,
+                                    [0xFFFFFFFF] * 4)
+        backend.run(graph)
+        for lane in range(lanes):
+            first, mine = int(got[2][lane][0]), int(got[2][lane][1])
+            kept, a, m = orc.accept_tree(got[1][first:first + mine], got[0][first:first + mine], selected[first:first + mine])
+            assert ret.download(np.uint32)[lane] == len(kept) and acc.download(np.uint32)[lane] == a and mask.download(np.uint32)[lane] == m
+            assert np.array_equal(tb.download(np.uint32)[first:first + len(kept)], kept)
+
+
 def test_draft_candidates_and_edges(backend):
     """draft_select_top16_sharded and draft_select_edges (sampling.metal:1099-1356) against the oracle: candidates and
     their logits bit for bit (ties, signed zeros, short rows, rows of few finite columns, a draft vocabulary that skips a

@@ -225,6 +225,37 @@ def test_verify_rows_layout_against_a_sort_and_a_recursive_preorder():
         assert np.all(sources[used:] == orc.NO_TOKEN) and np.all(tree[used:]["ancestors"] == 0)
 
 
+def test_verify_rows_in_slots_are_the_packed_rows_moved_and_inert_rows():
+    """The slots layout against the packed one (pinned above) of the same trees with every lane free to take its cap:
+    a lane's rows moved to its slot as they are, and the rest of the slot rows that the step cannot mistake for drafted
+    ones -- the acceptance walk never follows them whatever the target selects, and they lie on no other row's path."""
+    from tests.draft_case import grown_trees
+    rng = np.random.default_rng(30)
+    for trial in range(100):
+        lanes = int(rng.integers(1, 9))
+        tokens, trees, scores, sizes = grown_trees(rng, lanes, ties=trial % 3 == 0)
+        cap = int(rng.integers(1, 17))
+        floor = float(rng.choice([0.0, 0.3, 0.7]))
+        got_tokens, got_tree, got_lanes, got_sources = orc.draft_verify_row_slots(tokens, trees, scores, sizes, cap, floor)
+        p_tokens, p_tree, p_lanes, p_sources = orc.draft_verify_rows(tokens, trees, scores, sizes, lanes * cap, cap, floor)
+        for lane in range(lanes):
+            first, mine = lane * cap, int(p_lanes[lane][1])
+            assert list(got_lanes[lane]) == [first, mine]
+            at = int(p_lanes[lane][0])
+            assert np.array_equal(got_tokens[first:first + mine], p_tokens[at:at + mine])
+            assert np.array_equal(got_tree[first:first + mine], p_tree[at:at + mine]) and np.array_equal(got_sources[first:first + mine], p_sources[at:at + mine])
+            pad = slice(first + mine, first + cap)
+            assert np.all(got_tokens[pad] == orc.NO_TOKEN) and np.all(got_sources[pad] == orc.NO_TOKEN)
+            assert np.all(got_tree[pad]["ancestors"] == (1 << np.arange(mine, cap)).astype(np.uint32))
+            # no drafted row's path names an inert row
+            assert not np.any(got_tree[first:first + mine]["ancestors"] >> mine)
+            # the walk over the whole slot keeps what the walk over the lane's own rows keeps, whatever is selected
+            selected = rng.integers(0, 50, cap).astype(np.uint32)
+            own = orc.accept_tree(got_tree[first:first + mine], got_tokens[first:first + mine], selected[:mine])
+            whole = orc.accept_tree(got_tree[first:first + cap], got_tokens[first:first + cap], selected)
+            assert np.array_equal(own[0], whole[0]) and own[1:] == whole[1:]
+
+
 def test_draft_candidates_are_the_sorted_heads_of_the_rows():
     """orc_draft_candidates against a lexicographic sort (logit descending, column ascending): plain rows, rows of few
     distinct values with signed zeros, rows with fewer finite columns than candidates, fewer columns than candidates, and a
