@@ -304,9 +304,68 @@ def time_prefill_ops(backend):
             log(f"  {name:5s} M={M:5d}: {us:9.1f} us a chunk ({gemm_us:9.1f} us the projection) {tflops:7.1f} TFLOP/s")
             del graph, x, out, table
         del projection
+    # The chunked prefill attention (ops.PagedAttention.add_chunk_*): a chunk of one sequence at the 27B geometry over a 32K
+    # history, the projection pass of every tile and then the tiles' split and merge, eight tiles a dispatch. Operations
+    # counted: 4 D per (row, head, visible token), the history and on average half the chunk.
+    from splash_amd import synthetic
+    QH, KVH, D, history = 64, 8, 128, 32768
+    attention = []
+    for M in (128, 512, 2048):
+        pages = (history + M + ops.PAGE_TOKENS - 1) // ops.PAGE_TOKENS
+        raw = synthetic.kv_pages(rng, KVH, D, 8)
+        pool = ops.KvPages(backend, KVH, D, pages, rng.permutation(pages).astype(np.uint64))
+        pool.upload(np.tile(raw, ((pages + 7) // 8, 1))[:pages])
+        plan = ops.AttentionChunkPlan(QH, KVH, D, [(0, M, history, 0)], rotary_pairs=D // 2, normalize=True)
+        sizes = plan.workspace_sizes()
+
+        class Workspace:
+            queries, query_sums, partials, partial_sums = (backend.allocate_buffer(b) for b in sizes)
+        qkv = backend.from_array(bf(rng.standard_normal((M, (QH + 2 * KVH) * D))))
+        norm = backend.from_array(bf(np.ones(D)))
+        angles = rng.uniform(0, 6.28, (M, D // 2)).astype(np.float32)
+        cos, sin = backend.from_array(np.cos(angles)), backend.from_array(np.sin(angles))
+        tree = backend.from_array(ops.chain_tree_rows([min(16, M - at) for at in range(0, M, 16)]))
+        out = backend.allocate_buffer(M * QH * D * 2)
+        graph = splash_amd.CommandGraph()
+        repeats = 4
+        for _ in range(repeats):
+            ops.PagedAttention.add_chunk_projection(graph, plan, qkv, Workspace, pool, query_norm=norm, key_norm=norm, rope_cos=cos, rope_sin=sin)
+            ops.PagedAttention.add_chunk_attention(graph, plan, Workspace, tree, pool, out)
+        backend.set_dispatch_profiling(True)
+        _, _, per = backend.run(graph, profiled=True)
+        backend.set_dispatch_profiling(False)
+        us = float(np.median(np.array(per).reshape(repeats, -1)[1:].sum(axis=1)) * 1e6)
+        flops = 4.0 * D * QH * M * (history + (M + 1) / 2)
+        attention.append({"M": M, "history": history, "dispatches": len(graph) // repeats, "us": round(us, 1), "tokens_per_s": round(M / us * 1e6),
+                          "TFLOP/s": round(flops / us / 1e6, 1), "frac": round(flops / us / 1e6 / peak, 4)})
+        log(f"  chunk attention M={M:5d} over {history}: {us:9.1f} us ({flops / us / 1e6:6.1f} TFLOP/s of the fp16 peak's {peak:.0f})")
+        del graph, pool, Workspace, qkv, out
+    # GDN::addPrefill at the 35B-A3B shape (16 key / 32 value heads): prepare, scan and gate of a chunk of one lane and layer.
+    gdn = ops.GDN(16, 32)
+    states = backend.allocate_buffer(gdn.cell_bytes * 2)
+    states.upload(np.zeros(gdn.cell_bytes * 2 // 4, np.float32))
+    weights = dict(convolution_weights=backend.from_array(bf(rng.standard_normal((gdn.shape.convolution_dimension, 4)) * 0.4)),
+                   decay_weights=backend.from_array((-np.exp(rng.uniform(-1, 1, 32))).astype(np.float32)),
+                   time_bias=backend.from_array(bf(rng.uniform(-1, 1, 32))), mixer_norm=backend.from_array(bf(np.ones(128))))
+    recurrent = []
+    for M in (128, 512, 2048):
+        work = gdn.prefill_workspace(backend, M)
+        packed = backend.from_array(bf(rng.standard_normal((M, gdn.shape.packed_width))))
+        graph = splash_amd.CommandGraph()
+        repeats = 4
+        for _ in range(repeats):
+            gdn.add_prefill(graph, dict(packed=packed, states=states, **weights, **work), 0, M, 0, gdn.cell_bytes)
+        backend.set_dispatch_profiling(True)
+        _, _, per = backend.run(graph, profiled=True)
+        backend.set_dispatch_profiling(False)
+        parts = np.median(np.array(per).reshape(repeats, 3)[1:], axis=0) * 1e6
+        recurrent.append({"M": M, "prepare_us": round(float(parts[0]), 1), "scan_us": round(float(parts[1]), 1), "gate_us": round(float(parts[2]), 1),
+                          "us": round(float(parts.sum()), 1), "scan_us_per_token": round(float(parts[1]) / M, 3)})
+        log(f"  GDN prefill M={M:5d}: prepare {parts[0]:7.1f} scan {parts[1]:8.1f} gate {parts[2]:6.1f} us ({parts[1] / M:.3f} us a token in the scan)")
+        del graph, work, packed
     print(json.dumps({"metric": "prefill projection us and TFLOP/s by rows", "unit": "us", "n_gpus": 1,
                       "data": "synthetic: random images, N(0, 1) rows", "roofline": {"bound": "mfma", "peak": peak, "unit": "TFLOP/s"},
-                      "results": results}), flush=True)
+                      "results": results, "chunk_attention": attention, "gdn_prefill": recurrent}), flush=True)
 
 
 def time_c3_ops(backend):
