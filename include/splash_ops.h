@@ -478,6 +478,60 @@ sp_status spo_draft_add_verify_row_slots(spo_graph *graph, sp_buffer *tree_token
                                          sp_buffer *tree_sizes, sp_buffer *input_tokens, sp_buffer *tree_rows, sp_buffer *lane_rows,
                                          sp_buffer *verify_sources, uint32_t lanes, uint32_t lane_cap, float floor);
 
+/* ---- ops::DraftAttention (runtime/ops/DraftAttention.hpp:12-152, DraftAttention.cpp:85-309; kernels/decode/draft.metal,
+ *      kernels/prefill/draft_context.metal): the attention block of the draft model that proposes a step's rows. The
+ *      compiled shape: 32 query heads over 8 KV heads of 128 dimensions (a q|k|v row 6144 values, an attention row 4096),
+ *      8 query rows a lane, up to 8 lanes, over a hidden state of `hidden` values (a whole number of 16-channel
+ *      convolution groups). A lane's ring of a layer: keys bf16 [8 KV heads][2048 slots][128], values bf16 [8][128][2048],
+ *      position p in slot p % 2048, each 4 MiB, `keys[l]` / `values[l]` bytes into the bound rings buffer (where the
+ *      reference binds a buffer a lane, DraftAttention.hpp:80-89). ---- */
+/* DraftAttentionPlan::workspace(): sizes[0..4] = convolution rows, q|k|v rows, grouped queries with the splits'
+ * partials behind them, query keys, query values. */
+sp_status spo_draft_attention_workspace(uint32_t hidden, uint32_t lanes, uint64_t sizes[5]);
+/* DraftAttention::addConvolution: a stage of a dynamic convolution over each lane's eight rows (finish: the stage
+ * after the attention or MLP, which adds the residual). dynamic bf16 [lanes * 8][4 * hidden / 16]: [stage][tap][group];
+ * weights bf16 [stage][tap][hidden]. out = in * (w[tap 0] + dyn[tap 0]) + in[row - 1] * (w[tap 1] + dyn[tap 1]) (+ residual). */
+sp_status spo_draft_attention_add_convolution(spo_graph *graph, sp_buffer *input, sp_buffer *dynamic, sp_buffer *weights, sp_buffer *residual,
+                                              sp_buffer *output, uint32_t hidden, uint32_t lanes, uint32_t finish);
+/* DraftAttention::addPrepare: head norms and RoPE of the rows' queries (grouped [lane][query head][8][128]) and keys
+ * (query_keys [lane][KV head][8][128]), values transposed (query_values [lane][KV head][128][8]). rope_cos / rope_sin
+ * fp32 [lane][16][64]: a lane's rows take the first eight of its sixteen RoPE rows. */
+sp_status spo_draft_attention_add_prepare(spo_graph *graph, sp_buffer *qkv, sp_buffer *grouped_queries, sp_buffer *query_norm,
+                                          sp_buffer *key_norm, sp_buffer *rope_cos, sp_buffer *rope_sin, sp_buffer *query_keys,
+                                          sp_buffer *query_values, uint32_t hidden, uint32_t lanes);
+/* DraftAttention::addDecode: each row r of a lane at position cache_lengths[l] + r attends to the ring's positions of
+ * its window of 2048 and to all eight current rows; the rows leave in the grouped queries' place as
+ * [lane][row][query head][128], the output projection's input. */
+sp_status spo_draft_attention_add_decode(spo_graph *graph, sp_buffer *grouped_queries, sp_buffer *rings, const uint64_t *keys,
+                                         const uint64_t *values, sp_buffer *query_keys, sp_buffer *query_values,
+                                         const uint32_t *cache_lengths, uint32_t hidden, uint32_t lanes);
+/* DraftAttention::addContextPrefill: `tokens` context rows (bf16 [tokens][1024 keys | 1024 values]) of one lane into
+ * the slots of positions start_position on: keys head-normalized, weighed by key_norm and turned by RoPE row r,
+ * values copied. */
+sp_status spo_draft_attention_add_context_prefill(spo_graph *graph, sp_buffer *context_kv, sp_buffer *key_norm, sp_buffer *rope_cos,
+                                                  sp_buffer *rope_sin, sp_buffer *rings, uint64_t keys, uint64_t values, uint32_t tokens,
+                                                  uint32_t start_position, uint32_t hidden);
+/* DraftAttention::addContextCommit: each lane's retained rows of a step (retained_rows uint32 [lanes], the masks
+ * acceptance wrote; lane_rows {first, rows} [lanes], which the step's proposer wrote) into its rings: the path's i-th
+ * row at position start_positions[l] + i, turned by the lane's RoPE row i. A step of `rows` rows, `lane_cap` a lane at most. */
+sp_status spo_draft_attention_add_context_commit(spo_graph *graph, sp_buffer *context_kv, sp_buffer *key_norm, sp_buffer *rope_cos,
+                                                 sp_buffer *rope_sin, sp_buffer *rings, const uint64_t *keys, const uint64_t *values,
+                                                 sp_buffer *retained_rows, sp_buffer *lane_rows, const uint32_t *start_positions,
+                                                 uint32_t lanes, uint32_t rows, uint32_t lane_cap, uint32_t hidden);
+/* The context window (DraftAttention.hpp:117-151): per ring slot the context row of `width` values in 4-bit codes over
+ * groups of 64 with an fp16 scale and minimum each: all slots' codes, then the (scale, minimum) pairs. Store, commit
+ * (the rows one lane retained, as the context commit picks them) and load. */
+sp_status spo_draft_context_window_bytes(uint32_t width, uint64_t *bytes);
+sp_status spo_draft_attention_add_window_store(spo_graph *graph, sp_buffer *context, sp_buffer *window, uint32_t rows, uint32_t start_position,
+                                               uint32_t width);
+sp_status spo_draft_attention_add_window_commit(spo_graph *graph, sp_buffer *context, sp_buffer *window, sp_buffer *retained,
+                                                sp_buffer *lane_rows, uint32_t context_rows, uint32_t rows, uint32_t start_position,
+                                                uint32_t width);
+sp_status spo_draft_attention_add_window_load(spo_graph *graph, sp_buffer *window, sp_buffer *context, uint32_t rows, uint32_t start_position,
+                                              uint32_t width);
+/* Embedding::addDraftMaskRows (runtime/ops/Embedding.cpp:49-58): rows 1..7 of each lane's eight input rows take the mask row. */
+sp_status spo_draft_attention_add_mask_rows(spo_graph *graph, sp_buffer *mask, sp_buffer *rows, uint32_t width, uint32_t lanes);
+
 /* ---- The dense verify step (the reference's model layer: QwenTarget.cpp:206-395, :457-496;
  *      Runtime.cpp:2677-2717, :2883-2892) ---- */
 typedef struct spo_dense_verify spo_dense_verify;

@@ -37,6 +37,13 @@
 //                                   reduces to when every expert is the same.
 //   orc_state_codes / _values       pinned: the compiled reference header (oracle/_ref, StateCodecReference.hpp) bit for
 //                                   bit, and the closed form (a value restores within half its block's step).
+//   orc_draft_conv / _prepare /     pinned by fp64 statements in numpy (the convolution exactly on dyadic inputs, as the
+//     _context_write                reference's test draws them; the head norm and rotation to a bf16 step; slots and
+//                                   untouched bytes by position).
+//   orc_draft_attention             pinned by a dense fp64 softmax in numpy over the rows' windows (short, wrapping and
+//                                   full rings) and by shift invariance: a ring rotated with its positions gives the same rows.
+//   orc_draft_window_*              pinned by the closed form (a value restores within half its group's step, extremes
+//                                   within an fp16 step of themselves) and numpy's codes.
 #pragma once
 #include <stddef.h>
 #include <stdint.h>
@@ -295,6 +302,21 @@ void orc_moe_combine(const uint16_t *y, const float *weights, const uint16_t *re
 uint64_t orc_state_codec_bytes(uint32_t rows, uint32_t columns);
 int orc_state_codes(const float *values, uint32_t rows, uint32_t columns, uint8_t *image);
 int orc_state_values(const uint8_t *image, uint32_t rows, uint32_t columns, float *values);
+
+// ---- the draft model's attention block (runtime/ops/DraftAttention.hpp, kernels/decode/draft.metal) ----
+// The compiled shape: 32 query heads over 8 KV heads of 128, eight query rows a lane, rings of 2048 slots.
+void orc_draft_conv(const uint16_t *input, const uint16_t *dynamic, const uint16_t *base, const uint16_t *residual, uint16_t *output,
+                    uint32_t hidden, uint32_t lanes, int finish);
+void orc_draft_prepare(const uint16_t *qkv, const uint16_t *query_norm, const uint16_t *key_norm, const float *cosines, const float *sines,
+                       uint32_t lanes, uint16_t *queries, uint16_t *keys, uint16_t *values);
+void orc_draft_context_write(const uint16_t *context_kv, const uint16_t *key_norm, const float *cosines, const float *sines,
+                             const uint32_t *source_rows, const uint32_t *positions, const uint32_t *rope_rows, uint32_t count,
+                             uint16_t *ring_keys, uint16_t *ring_values);
+void orc_draft_attention(const uint16_t *queries, const uint16_t *ring_keys, const uint16_t *ring_values, const uint16_t *query_keys,
+                         const uint16_t *query_values, uint32_t cache_length, double *output);
+uint64_t orc_draft_window_bytes(uint32_t width);
+void orc_draft_window_store(const uint16_t *context, const uint32_t *source_rows, uint32_t rows, uint32_t start, uint32_t width, uint8_t *window);
+void orc_draft_window_load(const uint8_t *window, uint32_t rows, uint32_t start, uint32_t width, uint16_t *context);
 
 #ifdef __cplusplus
 }

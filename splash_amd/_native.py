@@ -305,6 +305,18 @@ _sig("spo_draft_add_tree", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c
 _sig("spo_draft_add_verify_children", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_u32, c_u32)
 _sig("spo_draft_add_verify_rows", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_u32, c_u32, c_u32, ctypes.c_float)
 _sig("spo_draft_add_verify_row_slots", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_u32, c_u32, ctypes.c_float)
+_sig("spo_draft_attention_workspace", c_int, c_u32, c_u32, P(c_u64))
+_sig("spo_draft_attention_add_convolution", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_u32, c_u32, c_u32)
+_sig("spo_draft_attention_add_prepare", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_u32, c_u32)
+_sig("spo_draft_attention_add_decode", c_int, c_p, c_p, c_p, P(c_u64), P(c_u64), c_p, c_p, P(c_u32), c_u32, c_u32)
+_sig("spo_draft_attention_add_context_prefill", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_u64, c_u64, c_u32, c_u32, c_u32)
+_sig("spo_draft_attention_add_context_commit", c_int, c_p, c_p, c_p, c_p, c_p, c_p, P(c_u64), P(c_u64), c_p, c_p, P(c_u32), c_u32, c_u32,
+     c_u32, c_u32)
+_sig("spo_draft_context_window_bytes", c_int, c_u32, P(c_u64))
+_sig("spo_draft_attention_add_window_store", c_int, c_p, c_p, c_p, c_u32, c_u32, c_u32)
+_sig("spo_draft_attention_add_window_commit", c_int, c_p, c_p, c_p, c_p, c_p, c_u32, c_u32, c_u32, c_u32)
+_sig("spo_draft_attention_add_window_load", c_int, c_p, c_p, c_p, c_u32, c_u32, c_u32)
+_sig("spo_draft_attention_add_mask_rows", c_int, c_p, c_p, c_p, c_u32, c_u32)
 _sig("spo_sampling_add_acceptance", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, P(LaneRows), P(c_u32), c_u32, P(c_u32))
 _sig("spo_sampling_greedy_rows_static", c_int, ctypes.c_void_p, c_u32, c_u32, c_u32, ctypes.c_void_p, ctypes.c_void_p)
 _sig("spo_verify_check_results", c_int, P(LaneRows), P(c_u32), c_u32, c_u32, c_u32, P(c_u32), P(c_u32), P(c_u32), P(c_u32))

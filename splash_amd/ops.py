@@ -496,6 +496,86 @@ class DraftSelector:
         graph._keep.extend(buffers)
 
 
+DRAFT_QUERY_ROWS, DRAFT_WINDOW, DRAFT_QKV_WIDTH, DRAFT_ATTENTION_WIDTH, DRAFT_KV_WIDTH = 8, 2048, 6144, 4096, 1024
+DRAFT_RING_BYTES = 8 * DRAFT_WINDOW * 128 * 2
+
+
+class DraftAttention:
+    """ops::DraftAttention: the attention block of the draft model (32 query heads over 8 KV heads of 128, eight query rows
+    a lane, rings of 2048 slots) over a hidden state of `hidden` values, for `lanes` lanes."""
+
+    def __init__(self, hidden, lanes):
+        self.hidden, self.lanes = hidden, lanes
+        sizes = (ctypes.c_uint64 * 5)()
+        check(lib.spo_draft_attention_workspace(hidden, lanes, sizes))
+        self.convolution_bytes, self.qkv_bytes, self.grouped_queries_bytes, self.query_keys_bytes, self.query_values_bytes = list(sizes)
+
+    @staticmethod
+    def window_bytes(width):
+        out = ctypes.c_uint64()
+        check(lib.spo_draft_context_window_bytes(width, ctypes.byref(out)))
+        return out.value
+
+    def add_convolution(self, graph, input, dynamic, weights, residual, output, finish):
+        buffers = [input, dynamic, weights, residual if residual is not None else input, output]
+        check(lib.spo_draft_attention_add_convolution(graph.handle, *[b.handle for b in buffers], self.hidden, self.lanes, int(finish)))
+        graph._keep.extend(buffers)
+
+    def add_prepare(self, graph, qkv, grouped_queries, query_norm, key_norm, rope_cos, rope_sin, query_keys, query_values):
+        buffers = [qkv, grouped_queries, query_norm, key_norm, rope_cos, rope_sin, query_keys, query_values]
+        check(lib.spo_draft_attention_add_prepare(graph.handle, *[b.handle for b in buffers], self.hidden, self.lanes))
+        graph._keep.extend(buffers)
+
+    @staticmethod
+    def _offsets(values):
+        return (ctypes.c_uint64 * len(values))(*values)
+
+    def add_decode(self, graph, grouped_queries, rings, keys, values, query_keys, query_values, cache_lengths):
+        """rings: the buffer lane l's key ring starts keys[l] bytes into and its value ring values[l] bytes."""
+        if not len(keys) == len(values) == len(cache_lengths) == self.lanes:
+            raise nat.InvalidArgument(1, "a draft step binds a key ring, a value ring and a cache length a lane")
+        check(lib.spo_draft_attention_add_decode(graph.handle, grouped_queries.handle, rings.handle, self._offsets(keys), self._offsets(values),
+                                                 query_keys.handle, query_values.handle, (ctypes.c_uint32 * len(cache_lengths))(*cache_lengths),
+                                                 self.hidden, len(cache_lengths)))
+        graph._keep.extend([grouped_queries, rings, query_keys, query_values])
+
+    def add_context_prefill(self, graph, context_kv, key_norm, rope_cos, rope_sin, rings, keys, values, tokens, start_position):
+        check(lib.spo_draft_attention_add_context_prefill(graph.handle, context_kv.handle, key_norm.handle, rope_cos.handle, rope_sin.handle,
+                                                          rings.handle, keys, values, tokens, start_position, self.hidden))
+        graph._keep.extend([context_kv, key_norm, rope_cos, rope_sin, rings])
+
+    def add_context_commit(self, graph, context_kv, key_norm, rope_cos, rope_sin, rings, keys, values, retained_rows, lane_rows,
+                           start_positions, rows, lane_cap):
+        if not len(keys) == len(values) == len(start_positions):
+            raise nat.InvalidArgument(1, "a draft context commit binds a key ring, a value ring and a start position a lane")
+        check(lib.spo_draft_attention_add_context_commit(graph.handle, context_kv.handle, key_norm.handle, rope_cos.handle, rope_sin.handle,
+                                                         rings.handle, self._offsets(keys), self._offsets(values), retained_rows.handle,
+                                                         lane_rows.handle, (ctypes.c_uint32 * len(start_positions))(*start_positions),
+                                                         len(start_positions), rows, lane_cap, self.hidden))
+        graph._keep.extend([context_kv, key_norm, rope_cos, rope_sin, rings, retained_rows, lane_rows])
+
+    @staticmethod
+    def add_window_store(graph, context, window, rows, start_position, width):
+        check(lib.spo_draft_attention_add_window_store(graph.handle, context.handle, window.handle, rows, start_position, width))
+        graph._keep.extend([context, window])
+
+    @staticmethod
+    def add_window_commit(graph, context, window, retained, lane_rows, context_rows, rows, start_position, width):
+        check(lib.spo_draft_attention_add_window_commit(graph.handle, context.handle, window.handle, retained.handle, lane_rows.handle,
+                                                        context_rows, rows, start_position, width))
+        graph._keep.extend([context, window, retained, lane_rows])
+
+    @staticmethod
+    def add_window_load(graph, window, context, rows, start_position, width):
+        check(lib.spo_draft_attention_add_window_load(graph.handle, window.handle, context.handle, rows, start_position, width))
+        graph._keep.extend([window, context])
+
+    @staticmethod
+    def add_mask_rows(graph, mask, rows, width, lanes):
+        check(lib.spo_draft_attention_add_mask_rows(graph.handle, mask.handle, rows.handle, width, lanes))
+        graph._keep.extend([mask, rows])
+
+
 def chain_tree_rows(rows_per_sequence):
     """SplashTreeRow of chains: ancestors (2 << r) - 1, parent r - 1, depth r, packed per sequence."""
     out = []

@@ -734,3 +734,71 @@ def children_law(p_target, ids, q, n_draws):
     lib.orc_children_law.restype = None
     lib.orc_children_law(_p(p, f64p), c_u32(p.size), _p(ids, u32p), _p(q, f64p), c_u32(n_draws), _p(out, f64p))
     return out
+
+
+# ---- the draft model's attention block (oracle/draft_attention.cpp) ----
+DRAFT_ROWS, DRAFT_QUERY_HEADS, DRAFT_KV_HEADS, DRAFT_D, DRAFT_WINDOW = 8, 32, 8, 128, 2048
+
+
+def draft_conv(x, dynamic, base, residual, finish):
+    """bf16 bits [lanes * 8][hidden] through one stage of the dynamic convolution."""
+    x = np.ascontiguousarray(x, np.uint16)
+    lanes, hidden = x.shape[0] // DRAFT_ROWS, x.shape[1]
+    residual = np.ascontiguousarray(residual if residual is not None else x, np.uint16)
+    dynamic, base = np.ascontiguousarray(dynamic, np.uint16), np.ascontiguousarray(base, np.uint16)
+    out = np.empty_like(x)
+    lib.orc_draft_conv(_p(x, u16p), _p(dynamic, u16p), _p(base, u16p), _p(residual, u16p), _p(out, u16p), c_u32(hidden), c_u32(lanes),
+                       ctypes.c_int(int(finish)))
+    return out
+
+
+def draft_prepare(qkv, query_norm, key_norm, cosines, sines):
+    """qkv bf16 bits [lanes * 8][6144]; cosines / sines fp32 [lanes][16][64]. Returns the grouped queries
+    [lanes][32][8][128], the rows' keys [lanes][8][8][128] and their values [lanes][8][128][8]."""
+    qkv = np.ascontiguousarray(qkv, np.uint16)
+    lanes = qkv.shape[0] // DRAFT_ROWS
+    cosines, sines = np.ascontiguousarray(cosines, np.float32), np.ascontiguousarray(sines, np.float32)
+    q = np.empty((lanes, DRAFT_QUERY_HEADS, DRAFT_ROWS, DRAFT_D), np.uint16)
+    k = np.empty((lanes, DRAFT_KV_HEADS, DRAFT_ROWS, DRAFT_D), np.uint16)
+    v = np.empty((lanes, DRAFT_KV_HEADS, DRAFT_D, DRAFT_ROWS), np.uint16)
+    lib.orc_draft_prepare(_p(qkv, u16p), _p(np.ascontiguousarray(query_norm, np.uint16), u16p), _p(np.ascontiguousarray(key_norm, np.uint16), u16p),
+                          _p(cosines, f32p), _p(sines, f32p), c_u32(lanes), _p(q, u16p), _p(k, u16p), _p(v, u16p))
+    return q, k, v
+
+
+def draft_context_write(context_kv, key_norm, cosines, sines, source_rows, positions, rope_rows, ring_keys, ring_values):
+    """Writes context rows into one lane's rings in place: ring_keys [8][2048][128], ring_values [8][128][2048] (bf16 bits)."""
+    context_kv = np.ascontiguousarray(context_kv, np.uint16)
+    cosines, sines = np.ascontiguousarray(cosines, np.float32), np.ascontiguousarray(sines, np.float32)
+    src, pos, rope = (np.ascontiguousarray(a, np.uint32) for a in (source_rows, positions, rope_rows))
+    assert ring_keys.flags.c_contiguous and ring_values.flags.c_contiguous and ring_keys.dtype == np.uint16
+    lib.orc_draft_context_write(_p(context_kv, u16p), _p(np.ascontiguousarray(key_norm, np.uint16), u16p), _p(cosines, f32p), _p(sines, f32p),
+                                _p(src, u32p), _p(pos, u32p), _p(rope, u32p), c_u32(len(src)), _p(ring_keys, u16p), _p(ring_values, u16p))
+
+
+def draft_attention(queries, ring_keys, ring_values, query_keys, query_values, cache_length):
+    """One lane and KV head in fp64: queries [32][128], ring_keys [2048][128], ring_values [128][2048], query_keys
+    [8][128], query_values [128][8] (bf16 bits). Returns float64 [32][128]."""
+    args = [np.ascontiguousarray(a, np.uint16) for a in (queries, ring_keys, ring_values, query_keys, query_values)]
+    out = np.empty((4 * DRAFT_ROWS, DRAFT_D), np.float64)
+    lib.orc_draft_attention(*[_p(a, u16p) for a in args], c_u32(cache_length), _p(out, ctypes.POINTER(ctypes.c_double)))
+    return out
+
+
+def draft_window_bytes(width):
+    lib.orc_draft_window_bytes.restype = ctypes.c_uint64
+    return int(lib.orc_draft_window_bytes(c_u32(width)))
+
+
+def draft_window_store(context, source_rows, start, window):
+    """Stores rows source_rows of context (bf16 bits [.][width]) into the slots of positions start on, in place."""
+    context = np.ascontiguousarray(context, np.uint16)
+    src = np.ascontiguousarray(source_rows, np.uint32)
+    assert window.dtype == np.uint8 and window.flags.c_contiguous and window.size == draft_window_bytes(context.shape[1])
+    lib.orc_draft_window_store(_p(context, u16p), _p(src, u32p), c_u32(len(src)), c_u32(start), c_u32(context.shape[1]), _p(window, u8p))
+
+
+def draft_window_load(window, rows, start, width):
+    out = np.empty((rows, width), np.uint16)
+    lib.orc_draft_window_load(_p(np.ascontiguousarray(window, np.uint8), u8p), c_u32(rows), c_u32(start), c_u32(width), _p(out, u16p))
+    return out
