@@ -532,6 +532,57 @@ sp_status spo_draft_attention_add_window_load(spo_graph *graph, sp_buffer *windo
 /* Embedding::addDraftMaskRows (runtime/ops/Embedding.cpp:49-58): rows 1..7 of each lane's eight input rows take the mask row. */
 sp_status spo_draft_attention_add_mask_rows(spo_graph *graph, sp_buffer *mask, sp_buffer *rows, uint32_t width, uint32_t lanes);
 
+/* ---- model::DFlashDraft (runtime/model/DFlashDraft.hpp:66-356, DFlashDraft.cpp:184-430): the draft model that proposes a
+ *      step's rows. Per lane eight query rows (the anchor token's embedding in row 0, the mask embedding in rows 1..7)
+ *      through `layers` layers of norm -> dynamic convolution -> q|k|v -> attention over the lane's rings -> output ->
+ *      convolution with the residual -> norm -> dynamic convolution -> SwiGLU -> down -> convolution with the residual;
+ *      then the final norm, the target's vocabulary head (fp32 logits of the whole vocabulary; the reference may also run
+ *      a subset of the head's rows, DFlashDraft.cpp:44-52, which is the caller's choice of `head` here) and the selector's
+ *      projection, as spo_draft_add_candidates reads them. The context side turns the target's captured hidden rows
+ *      (target_layers layers' rows concatenated) into each layer's ring keys and values and the 4-bit window. The handle
+ *      owns the step's buffers and the state of max_lanes lanes (lane l of a call uses state l); projections may be of any
+ *      image format (the reference's draft quantizes in groups of 64 columns, a loader's concern). ---- */
+typedef struct spo_dflash_draft spo_dflash_draft;
+typedef struct spo_dflash_layout {
+  uint32_t layers, hidden, vocabulary, intermediate, target_layers;
+} spo_dflash_layout;
+typedef struct spo_dflash_layer {   /* DFlashDraftLayerWeights (DFlashDraft.hpp:195-209) */
+  const spo_projection *attention_dynamic, *qkv, *output, *mlp_dynamic, *gate, *up, *down;
+  sp_buffer *input_norm, *attention_convolution, *query_norm, *key_norm, *post_attention_norm, *mlp_convolution;
+} spo_dflash_layer;
+/* context_rows: the most rows a context call takes (at least a step's 16 a lane, at most 256). */
+sp_status spo_dflash_draft_create(sp_backend *backend, const spo_dflash_layout *layout, uint32_t max_lanes, uint32_t context_rows,
+                                  spo_dflash_draft **out);
+void spo_dflash_draft_destroy(spo_dflash_draft *draft);
+sp_status spo_dflash_draft_set_layer(spo_dflash_draft *draft, uint32_t layer, const spo_dflash_layer *weights);
+/* DFlashDraftWeights' model section (DFlashDraft.hpp:211-224) and the target's head; mask_embedding may be null. */
+sp_status spo_dflash_draft_set_model(spo_dflash_draft *draft, const spo_projection *context_projection, sp_buffer *hidden_norm,
+                                     sp_buffer *final_norm, const spo_projection *selector, sp_buffer *mask_embedding,
+                                     const spo_projection *head);
+/* The draft's buffers; each call returns a new reference (release it). SPO_DFLASH_HIDDEN index 0 holds the step's input
+ * rows [lanes * 8][hidden] (the caller writes row 0 of each lane); ROPE_COS / ROPE_SIN fp32 [lane][16][64], a lane's rows at
+ * positions cache length + r; RINGS lane l's rings from l * layers * 8 MiB on (layer i's keys, then its values);
+ * WINDOWS lane l's window; CAPTURED_TARGET_HIDDEN bf16 [rows][target_layers * hidden] and CONTEXT_ROPE_* fp32 [rows][64]
+ * (a prompt's rows one each; a step's [lane][16][64]) are the context calls' inputs. */
+typedef enum spo_dflash_buffer {
+  SPO_DFLASH_HIDDEN = 0, SPO_DFLASH_LOGITS, SPO_DFLASH_SELECTOR_HIDDEN, SPO_DFLASH_FINAL_HIDDEN, SPO_DFLASH_ROPE_COS, SPO_DFLASH_ROPE_SIN,
+  SPO_DFLASH_RINGS, SPO_DFLASH_WINDOWS, SPO_DFLASH_CAPTURED_TARGET_HIDDEN, SPO_DFLASH_CONTEXT_ROPE_COS, SPO_DFLASH_CONTEXT_ROPE_SIN,
+  SPO_DFLASH_CONTEXT_HIDDEN
+} spo_dflash_buffer;
+sp_status spo_dflash_draft_buffer(spo_dflash_draft *draft, spo_dflash_buffer which, uint32_t index, sp_buffer **out);
+/* DFlashDraft::addMaskRows and ::addDecode (DFlashDraft.cpp:274-380): the forward pass of `lanes` lanes, lane l's rows at
+ * positions cache_lengths[l] on. */
+sp_status spo_dflash_draft_encode_decode(spo_dflash_draft *draft, spo_graph *graph, const uint32_t *cache_lengths, uint32_t lanes);
+/* DFlashDraft::addContextPrefill (DFlashDraft.cpp:184-213): `rows` prompt rows of lane `lane` at positions start_position on
+ * into its window and rings; rebuild: ::addContextRebuild (:215-229), the rings from the window's rows instead. */
+sp_status spo_dflash_draft_encode_context_prefill(spo_dflash_draft *draft, spo_graph *graph, uint32_t lane, uint32_t rows,
+                                                  uint32_t start_position, int rebuild);
+/* DFlashDraft::addContextCommit (DFlashDraft.cpp:382-430): the rows each lane retained of a verify step of `rows` rows
+ * (retained_rows uint32 [lanes], lane_rows {first, rows} [lanes], both on the device), the path's i-th at
+ * start_positions[l] + i. */
+sp_status spo_dflash_draft_encode_context_commit(spo_dflash_draft *draft, spo_graph *graph, sp_buffer *retained_rows, sp_buffer *lane_rows,
+                                                 const uint32_t *start_positions, uint32_t lanes, uint32_t rows, uint32_t lane_cap);
+
 /* ---- The dense verify step (the reference's model layer: QwenTarget.cpp:206-395, :457-496;
  *      Runtime.cpp:2677-2717, :2883-2892) ---- */
 typedef struct spo_dense_verify spo_dense_verify;

@@ -185,6 +185,18 @@ class HybridLayer(ctypes.Structure):
                                                                     ("ffn_down", c_p)]
 
 
+class DFlashLayout(ctypes.Structure):
+    _fields_ = [(n, c_u32) for n in ("layers", "hidden", "vocabulary", "intermediate", "target_layers")]
+
+
+DFLASH_LAYER_FIELDS = ("attention_dynamic", "qkv", "output", "mlp_dynamic", "gate", "up", "down", "input_norm", "attention_convolution",
+                       "query_norm", "key_norm", "post_attention_norm", "mlp_convolution")
+
+
+class DFlashLayer(ctypes.Structure):
+    _fields_ = [(n, c_p) for n in DFLASH_LAYER_FIELDS]
+
+
 def _sig(name, restype, *argtypes):
     fn = getattr(lib, name)
     fn.restype = restype
@@ -317,6 +329,14 @@ _sig("spo_draft_attention_add_window_store", c_int, c_p, c_p, c_p, c_u32, c_u32,
 _sig("spo_draft_attention_add_window_commit", c_int, c_p, c_p, c_p, c_p, c_p, c_u32, c_u32, c_u32, c_u32)
 _sig("spo_draft_attention_add_window_load", c_int, c_p, c_p, c_p, c_u32, c_u32, c_u32)
 _sig("spo_draft_attention_add_mask_rows", c_int, c_p, c_p, c_p, c_u32, c_u32)
+_sig("spo_dflash_draft_create", c_int, c_p, P(DFlashLayout), c_u32, c_u32, P(c_p))
+_sig("spo_dflash_draft_destroy", None, c_p)
+_sig("spo_dflash_draft_set_layer", c_int, c_p, c_u32, P(DFlashLayer))
+_sig("spo_dflash_draft_set_model", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p)
+_sig("spo_dflash_draft_buffer", c_int, c_p, c_u32, c_u32, P(c_p))
+_sig("spo_dflash_draft_encode_decode", c_int, c_p, c_p, P(c_u32), c_u32)
+_sig("spo_dflash_draft_encode_context_prefill", c_int, c_p, c_p, c_u32, c_u32, c_u32, c_int)
+_sig("spo_dflash_draft_encode_context_commit", c_int, c_p, c_p, c_p, c_p, P(c_u32), c_u32, c_u32, c_u32)
 _sig("spo_sampling_add_acceptance", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, P(LaneRows), P(c_u32), c_u32, P(c_u32))
 _sig("spo_sampling_greedy_rows_static", c_int, ctypes.c_void_p, c_u32, c_u32, c_u32, ctypes.c_void_p, ctypes.c_void_p)
 _sig("spo_verify_check_results", c_int, P(LaneRows), P(c_u32), c_u32, c_u32, c_u32, P(c_u32), P(c_u32), P(c_u32), P(c_u32))

@@ -296,6 +296,72 @@ class HybridVerify:
     _results_call = "spo_hybrid_verify_results"
 
 
+(DFLASH_HIDDEN, DFLASH_LOGITS, DFLASH_SELECTOR_HIDDEN, DFLASH_FINAL_HIDDEN, DFLASH_ROPE_COS, DFLASH_ROPE_SIN, DFLASH_RINGS, DFLASH_WINDOWS,
+ DFLASH_CAPTURED_TARGET_HIDDEN, DFLASH_CONTEXT_ROPE_COS, DFLASH_CONTEXT_ROPE_SIN, DFLASH_CONTEXT_HIDDEN) = range(12)
+
+
+class DFlashDraft:
+    """model::DFlashDraft: the draft model that proposes a step's rows, and the writers of its context. The handle owns the
+    step's buffers and the rings and windows of max_lanes lanes."""
+
+    def __init__(self, backend, layers, hidden, vocabulary, intermediate, target_layers, max_lanes, context_rows=0):
+        self.backend = backend
+        self.layout = nat.DFlashLayout(layers, hidden, vocabulary, intermediate, target_layers)
+        self.max_lanes = max_lanes
+        out = ctypes.c_void_p()
+        check(lib.spo_dflash_draft_create(backend.handle, ctypes.byref(self.layout), max_lanes, context_rows, ctypes.byref(out)))
+        self.handle = out
+        self._keep = []
+
+    def close(self):
+        if self.handle:
+            lib.spo_dflash_draft_destroy(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def buffer(self, which, index=0):
+        out = ctypes.c_void_p()
+        check(lib.spo_dflash_draft_buffer(self.handle, which, index, ctypes.byref(out)))
+        return Buffer(out.value)
+
+    def set_layer(self, layer, **weights):
+        """weights: the projections and buffers of nat.DFLASH_LAYER_FIELDS by name."""
+        w = nat.DFlashLayer(*[weights[name].handle for name in nat.DFLASH_LAYER_FIELDS])
+        check(lib.spo_dflash_draft_set_layer(self.handle, layer, ctypes.byref(w)))
+        self._keep.extend(weights.values())
+
+    def set_model(self, context_projection, hidden_norm, final_norm, selector, mask_embedding, head):
+        check(lib.spo_dflash_draft_set_model(self.handle, context_projection.handle, hidden_norm.handle, final_norm.handle, selector.handle,
+                                             mask_embedding.handle if mask_embedding is not None else None, head.handle))
+        self._keep.extend([context_projection, hidden_norm, final_norm, selector, mask_embedding, head])
+
+    def encode_decode(self, cache_lengths, graph=None):
+        graph = graph or CommandGraph()
+        check(lib.spo_dflash_draft_encode_decode(self.handle, graph.handle, (ctypes.c_uint32 * len(cache_lengths))(*cache_lengths),
+                                                 len(cache_lengths)))
+        graph._keep.append(self)
+        return graph
+
+    def encode_context_prefill(self, lane, rows, start_position, rebuild=False, graph=None):
+        graph = graph or CommandGraph()
+        check(lib.spo_dflash_draft_encode_context_prefill(self.handle, graph.handle, lane, rows, start_position, int(rebuild)))
+        graph._keep.append(self)
+        return graph
+
+    def encode_context_commit(self, retained_rows, lane_rows, start_positions, rows, lane_cap, graph=None):
+        graph = graph or CommandGraph()
+        check(lib.spo_dflash_draft_encode_context_commit(self.handle, graph.handle, retained_rows.handle, lane_rows.handle,
+                                                         (ctypes.c_uint32 * len(start_positions))(*start_positions), len(start_positions),
+                                                         rows, lane_cap))
+        graph._keep.extend([self, retained_rows, lane_rows])
+        return graph
+
+
 def check_results(lanes, tokens, retained, accepted, retained_rows, vocabulary, remaining=None, step_rows=None):
     """spo_verify_check_results over host arrays: lanes [(first, rows)]."""
     arr = (nat.LaneRows * len(lanes))(*[nat.LaneRows(*l) for l in lanes])
