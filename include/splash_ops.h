@@ -613,6 +613,11 @@ sp_status spo_dense_verify_set_layer(spo_dense_verify *verify, uint32_t layer, c
                                      sp_buffer *query_norm, sp_buffer *key_norm);
 sp_status spo_dense_verify_set_head(spo_dense_verify *verify, uint32_t embedding_format, sp_buffer *embedding_rows,
                                     sp_buffer *final_norm, const spo_projection *head);
+/* The hidden rows a draft's context is computed from (QwenTarget's addCapture over RowCopy, runtime/ops/RowCopy.hpp:17-28):
+ * after layer layers[i] (ascending) every row's output goes to columns [i * hidden, (i + 1) * hidden) of its row of
+ * destination, bf16 [rows][count * hidden], in a step and in a prompt chunk alike; what spo_dflash_draft's context calls
+ * read (SPO_DFLASH_CAPTURED_TARGET_HIDDEN may be bound here directly). count 0 captures nothing. */
+sp_status spo_dense_verify_set_capture(spo_dense_verify *verify, const uint32_t *layers, uint32_t count, sp_buffer *destination);
 /* The step's buffers; each call returns a new reference (release it). `index` is the layer for KV pools and the
    stream (0 or 1) for the hidden rows. The last three hold what the layer that ran last left in them: its fused
    q|k|v rows before the head norms, its attention rows before the output projection, its SwiGLU rows before the

@@ -207,6 +207,13 @@ sp_status spo_draft_add_verify_row_slots(spo_graph *graph, sp_buffer *tree_token
   });
 }
 
+sp_status spo_dense_verify_set_capture(spo_dense_verify *verify, const uint32_t *layers, uint32_t count, sp_buffer *destination) {
+  return capi::guard([&] {
+    capi::require(verify && (layers || !count), "verify or layers");
+    verify->verify->setCapture(std::vector<uint32_t>(layers, layers + count), B(destination));
+  });
+}
+
 sp_status spo_dense_verify_create(sp_backend *backend, const spo_dense_dimensions *d, uint32_t max_lanes, uint32_t physical_pages,
                                   uint32_t page_table_entries, spo_dense_verify **out) {
   return spo_dense_verify_create_chunked(backend, d, max_lanes, physical_pages, page_table_entries, 0, out);

@@ -220,8 +220,24 @@ void DenseVerify::encodeLayer(hip::CommandGraph &graph, uint32_t layer, const op
   linear_.addSwiGlu(graph, {&w.gate, &w.up, &w.down}, ffn, next, residual, rows, prepared);
 }
 
+void DenseVerify::setCapture(std::vector<uint32_t> layers, hip::Buffer destination) {
+  for (size_t i = 0; i < layers.size(); ++i)
+    if (layers[i] >= dims_.layers || (i && layers[i] <= layers[i - 1])) throw std::invalid_argument("captured layers are the model's, ascending");
+  if (!layers.empty())
+    ops::requireBytes(destination, uint64_t{std::max(maxRows_, rowCapacity_)} * layers.size() * dims_.hidden * 2, "captured target hidden rows");
+  captureLayers_ = std::move(layers);
+  captured_ = std::move(destination);
+}
+
+void DenseVerify::encodeCapture(hip::CommandGraph &graph, uint32_t layer, uint32_t rows) const {
+  for (size_t slot = 0; slot < captureLayers_.size(); ++slot)
+    if (captureLayers_[slot] == layer)
+      ops::RowCopy::add(graph, hidden_[0], {0, dims_.hidden, 0}, captured_,
+                        {0, uint32_t(captureLayers_.size()) * dims_.hidden, uint32_t(slot) * dims_.hidden}, rows, dims_.hidden);
+}
+
 bool DenseVerify::chains(uint32_t rows) const noexcept {
-  if (!chained_ || rows > ops::kMaximumDecodeTileRows || !layersFeedNext(rows)) return false;
+  if (!chained_ || !captureLayers_.empty() || rows > ops::kMaximumDecodeTileRows || !layersFeedNext(rows)) return false;
   for (const DenseLayer &l : weights_.layers)
     if (!linear_.normsRows(l.output, rows)) return false;
   return true;
@@ -405,8 +421,10 @@ void DenseVerify::encodePrefill(hip::CommandGraph &graph, uint32_t tableFirst, u
     encodeEmbedding(graph, tokens);
     // every window is a step's worth of rows at most, so what holds for one holds for all
     const bool feeds = layersFeedNext(std::min(tokens, kWindowRows));
-    for (uint32_t layer = 0; layer < dims_.layers; ++layer)
+    for (uint32_t layer = 0; layer < dims_.layers; ++layer) {
       encodeChunkLayer(graph, layer, plan, tokens, feeds && layer > 0, feeds && layer + 1 < dims_.layers);
+      encodeCapture(graph, layer, tokens);
+    }
     return;
   }
   std::vector<ops::AttentionRows> sequences;
@@ -422,8 +440,10 @@ void DenseVerify::encodePrefill(hip::CommandGraph &graph, uint32_t tableFirst, u
     ops::RoPE::addTreeTables(graph, inverseFrequency_, depths_, ropeCos_, ropeSin_, dims_.rotaryPairs, rope);
   encodeEmbedding(graph, tokens);
   const bool feeds = layersFeedNext(tokens);
-  for (uint32_t layer = 0; layer < dims_.layers; ++layer)
+  for (uint32_t layer = 0; layer < dims_.layers; ++layer) {
     encodeLayer(graph, layer, plan, tokens, feeds && layer > 0, feeds && layer + 1 < dims_.layers);
+    encodeCapture(graph, layer, tokens);
+  }
 }
 
 void DenseVerify::encode(hip::CommandGraph &graph, const std::vector<VerifyLane> &lanes, bool commit) {
@@ -454,7 +474,10 @@ void DenseVerify::encode(hip::CommandGraph &graph, const std::vector<VerifyLane>
     encodeChainedLayers(graph, plan, rows);
   } else {
     const bool feeds = layersFeedNext(rows);
-    for (uint32_t layer = 0; layer < dims_.layers; ++layer) encodeLayer(graph, layer, plan, rows, feeds && layer > 0, feeds);
+    for (uint32_t layer = 0; layer < dims_.layers; ++layer) {
+      encodeLayer(graph, layer, plan, rows, feeds && layer > 0, feeds);
+      encodeCapture(graph, layer, rows);
+    }
     encodeHead(graph, rows, feeds);
   }
   // the sampled lanes' test is the step's choice (setTestChildren), not a property of which buffers were ever fetched

@@ -120,6 +120,11 @@ public:
   // that completes a head prepares its sixteen rows alone (four a wave, about 4 us of vector arithmetic), where the
   // prepare kernel spreads them over 1280 workgroups.
   void setFusedPrepare(bool fused) noexcept { fusedPrepare_ = fused; }
+  // The hidden rows a draft's context is computed from (the reference's QwenTarget addCapture over RowCopy,
+  // RowCopy.hpp:17-28): after layer layers[i] (ascending), every row's output goes to columns [i hidden, (i + 1) hidden)
+  // of its row of `destination`, bf16 [rows][layers.size() x hidden]; a step's rows and a prompt chunk's alike. A
+  // capturing driver chains no projections. An empty list captures nothing.
+  void setCapture(std::vector<uint32_t> layers, hip::Buffer destination);
   [[nodiscard]] bool fusedPrepare() const noexcept { return fusedPrepare_; }
   // Nonzero after a step in which a chained projection's wait for the one before it gave up: the step's results are
   // then not to be used. Reads the device's word (a copy of four bytes) and clears it.
@@ -144,6 +149,9 @@ private:
   hip::Buffer chainTables_[2], chainProgress_;
   ops::LinearScratch chainScratch_[GGUF_CHAIN_LINKS];
   bool chained_ = false, encodedChains_ = false, fusedPrepare_ = false, testChildren_ = false;
+  std::vector<uint32_t> captureLayers_;
+  hip::Buffer captured_;
+  void encodeCapture(hip::CommandGraph &graph, uint32_t layer, uint32_t rows) const;
   ops::SamplingBuffers children_;   // the four candidate-children buffers, bound into a step's sampling buffers when it tests them
   hip::Buffer chunkAttentionTable_;  // a long chunk's attention rows as the output projection's tables, every window's
   void encodeChunkLayer(hip::CommandGraph &graph, uint32_t layer, const ops::AttentionChunkPlan &plan, uint32_t tokens, bool first,

@@ -72,6 +72,12 @@ class DenseVerify:
                                              input_norm.handle, post_norm.handle, query_norm.handle, key_norm.handle))
         self._keep.extend([qkv, output, gate, up, down, input_norm, post_norm, query_norm, key_norm])
 
+    def set_capture(self, layers, destination):
+        """After each of `layers` (ascending) every row's output goes to its slot of `destination`, bf16 [rows][len(layers) x hidden]."""
+        check(lib.spo_dense_verify_set_capture(self.handle, (ctypes.c_uint32 * max(len(layers), 1))(*layers), len(layers),
+                                               destination.handle if destination is not None else None))
+        self._keep.append(destination)
+
     def set_head(self, embedding_format, embedding_rows, final_norm, head):
         check(lib.spo_dense_verify_set_head(self.handle, embedding_format, embedding_rows.handle, final_norm.handle, head.handle))
         self._keep.extend([embedding_rows, final_norm, head])
