@@ -562,6 +562,51 @@ def time_draft_candidates(backend):
         result[f"lanes_{lanes}"] = {"top16_us": round(top, 1), "top16_gbs": round(moved / top / 1e3, 1),
                                     "top16_frac": round(moved / top / 1e3 / HBM_PEAK_GBS, 4), "edges_us": round(edges, 1)}
         log(f"  {lanes} lane(s): top16 {top:6.1f} us {moved / top / 1e3:7.1f} GB/s, edges {edges:6.1f} us")
+        del logits, graph
+    # The draft model's forward pass (model::DFlashDraft) at a 27B target's widths: hidden 5120, the target's head of 151936
+    # tokens (Q6_K, fp32 logits), five layers of intermediate 13824 (a draft's config states its own layers and
+    # intermediate size; these stand in), every lane past its window of 2048 positions. One command a step, replayed.
+    from splash_amd import synthetic, verify
+    H, F, L = 5120, 13824, 5
+    bf = lambda a: (np.ascontiguousarray(a, np.float32).view(np.uint32) >> 16).astype(np.uint16)
+    image = lambda fmt, n, k: backend.from_array(ops.pack_gguf_image(fmt, synthetic.native(rng, fmt, n, k), n, k))
+    P = lambda n, k, fmt=ops.FMT_Q4K, f32=False: ops.Projection([(fmt, n, image(fmt, n, k))], k, f32)
+    norm = lambda n: backend.from_array(bf(1 + 0.05 * rng.standard_normal(n)))
+    draft = verify.DFlashDraft(backend, L, H, vocabulary, F, 5, max_lanes=8)
+    for layer in range(L):
+        draft.set_layer(layer, attention_dynamic=P(H // 4, H), qkv=P(6144, H), output=P(H, 4096), mlp_dynamic=P(H // 4, H), gate=P(F, H), up=P(F, H),
+                        down=P(H, F), input_norm=norm(H), attention_convolution=backend.from_array(bf(rng.standard_normal((4, H)) * 0.5)),
+                        query_norm=norm(128), key_norm=norm(128), post_attention_norm=norm(H),
+                        mlp_convolution=backend.from_array(bf(rng.standard_normal((4, H)) * 0.5)))
+    draft.set_model(P(H, 5 * H), norm(H), norm(H), P(256, H), norm(H), P(vocabulary, H, ops.FMT_Q6K, True))
+    draft.buffer(verify.DFLASH_RINGS).upload(bf(rng.standard_normal(8 * L * 2 * ops.DRAFT_RING_BYTES // 2) * 0.5))
+    angles = rng.uniform(0, 6.28, (8 * 16, 64))
+    draft.buffer(verify.DFLASH_ROPE_COS).upload(np.cos(angles).astype(np.float32))
+    draft.buffer(verify.DFLASH_ROPE_SIN).upload(np.sin(angles).astype(np.float32))
+    weights = L * (2 * ops.gguf_image_bytes(ops.FMT_Q4K, H // 4, H) + ops.gguf_image_bytes(ops.FMT_Q4K, 6144, H) + ops.gguf_image_bytes(ops.FMT_Q4K, H, 4096)
+                   + 3 * ops.gguf_image_bytes(ops.FMT_Q4K, F, H)) + ops.gguf_image_bytes(ops.FMT_Q6K, vocabulary, H) + ops.gguf_image_bytes(ops.FMT_Q4K, 256, H)
+    for lanes in (1, 8):
+        draft.buffer(verify.DFLASH_HIDDEN, 0).upload(bf(rng.standard_normal((lanes * 8, H))))
+        graph = draft.encode_decode([40000 + 100 * l for l in range(lanes)])
+        kernels = graph.kernels()
+        command = backend.record(graph)
+        for _ in range(3):
+            command.submit().wait()
+        step = float(np.median([command.submit().wait()[0] for _ in range(10)])) * 1e6
+        backend.set_dispatch_profiling(True)
+        _, _, per = backend.run(graph, profiled=True)
+        backend.set_dispatch_profiling(False)
+        by = {}
+        for name, seconds in zip(kernels, per):
+            by.setdefault(name, []).append(seconds * 1e6)
+        split, merge = float(np.median(by["draft_attention_split"])), float(np.median(by["draft_attention_merge"]))
+        ring = lanes * 2 * ops.DRAFT_RING_BYTES
+        result[f"draft_step_lanes_{lanes}"] = {"us": round(step, 1), "dispatches": len(kernels), "weights_gb": round(weights / 1e9, 3),
+                                               "weights_gbs": round(weights / step / 1e3, 1), "frac": round(weights / step / 1e3 / HBM_PEAK_GBS, 4),
+                                               "attention_split_us": round(split, 1), "attention_merge_us": round(merge, 1),
+                                               "attention_ring_gbs": round(ring / split / 1e3, 1)}
+        log(f"  draft step, {lanes} lane(s): {step:8.1f} us ({len(kernels)} dispatches, {weights / 1e9:.2f} GB of weights: {weights / step / 1e3:6.1f} GB/s); "
+            f"attention split {split:5.1f} us + merge {merge:4.1f} us over {ring / 1e6:.0f} MB of rings")
     print(json.dumps(result), flush=True)
 
 

@@ -307,20 +307,31 @@ __global__ __launch_bounds__(256) void draft_attention_split(const uint16_t *__r
 __global__ __launch_bounds__(256) void draft_attention_merge(const float *__restrict__ partials, uint16_t *__restrict__ output, DraftLanesParams) {
   const uint32_t head = blockIdx.x, batch = blockIdx.y, row = threadIdx.x / 8u, c = threadIdx.x % 8u;
   const float *from = partials + (size_t(batch) * kKvHeads + head) * DRAFT_ATTENTION_SPLITS * DRAFT_ATTENTION_PARTIAL_FLOATS;
-  float most = -INFINITY;
-  for (uint32_t split = 0; split < DRAFT_ATTENTION_SPLITS; ++split)
-    most = fmaxf(most, from[split * DRAFT_ATTENTION_PARTIAL_FLOATS + kM * kD + row]);
+  // Every split's maximum, sum and outputs are loaded whatever the split holds, so the loads do not wait for each other;
+  // a split with no visible key (a maximum of -inf) wrote no outputs, and what its place holds is set aside, not added.
+  float splitMax[DRAFT_ATTENTION_SPLITS], splitSum[DRAFT_ATTENTION_SPLITS], most = -INFINITY;
+#pragma unroll
+  for (uint32_t split = 0; split < DRAFT_ATTENTION_SPLITS; ++split) {
+    splitMax[split] = from[split * DRAFT_ATTENTION_PARTIAL_FLOATS + kM * kD + row];
+    splitSum[split] = from[split * DRAFT_ATTENTION_PARTIAL_FLOATS + kM * kD + kM + row];
+    most = fmaxf(most, splitMax[split]);
+  }
   float total = 0.f, acc[16];
 #pragma unroll
   for (int i = 0; i < 16; ++i) acc[i] = 0.f;
-  for (uint32_t split = 0; split < DRAFT_ATTENTION_SPLITS; ++split) {
-    const float *partial = from + split * DRAFT_ATTENTION_PARTIAL_FLOATS;
-    const float splitMax = partial[kM * kD + row];
-    if (splitMax == -INFINITY) continue;  // no visible key: nothing to add, and its outputs were never written
-    const float scale = __builtin_amdgcn_exp2f(splitMax - most);
-    total += scale * partial[kM * kD + kM + row];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) acc[i] += scale * partial[row * kD + 16u * c + i];
+  for (uint32_t split = 0; split < DRAFT_ATTENTION_SPLITS; ++split) {
+    const float4 *partial = reinterpret_cast<const float4 *>(from + split * DRAFT_ATTENTION_PARTIAL_FLOATS + row * kD + 16u * c);
+    const bool live = splitMax[split] != -INFINITY;
+    const float scale = __builtin_amdgcn_exp2f(splitMax[split] - most);
+    if (live) total += scale * splitSum[split];
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      const float4 four = partial[v];
+      const float values[4] = {four.x, four.y, four.z, four.w};
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[4 * v + i] += live ? scale * values[i] : 0.f;
+    }
   }
   const uint32_t queryRow = row % kRows, queryHead = head * (kM / kRows) + row / kRows;
   uint16_t *to = output + size_t(batch) * kRows * DRAFT_ATTENTION_WIDTH + (queryRow * kQueryHeads + queryHead) * kD + 16u * c;
