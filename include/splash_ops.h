@@ -48,6 +48,11 @@ sp_status spo_gguf_add_dequant(spo_graph *graph, uint32_t format, sp_buffer *ima
 sp_status spo_projection_create(uint32_t segments, const uint32_t *formats, const uint32_t *output_sizes,
                                 uint32_t input_size, sp_buffer *const *images, int float32_destination,
                                 spo_projection **out);
+/* Projection::rows (Weights.hpp:193-204): a view of a projection of one tensor over one or two ranges of its rows, whole
+ * 16-row tiles, which become its output columns in order; slices of the same image, no copy. The draft's vocabulary head
+ * over a subset of the tokens (DraftVocabulary::rows, DraftSelector.hpp:108-112: rows [0, leading) and [trailing, V)). */
+sp_status spo_projection_rows(const spo_projection *projection, const uint32_t *firsts, const uint32_t *counts, uint32_t ranges,
+                              spo_projection **out);
 void spo_projection_destroy(spo_projection *projection);
 uint64_t spo_projection_weight_bytes(const spo_projection *projection);
 
@@ -536,8 +541,9 @@ sp_status spo_draft_attention_add_mask_rows(spo_graph *graph, sp_buffer *mask, s
  *      step's rows. Per lane eight query rows (the anchor token's embedding in row 0, the mask embedding in rows 1..7)
  *      through `layers` layers of norm -> dynamic convolution -> q|k|v -> attention over the lane's rings -> output ->
  *      convolution with the residual -> norm -> dynamic convolution -> SwiGLU -> down -> convolution with the residual;
- *      then the final norm, the target's vocabulary head (fp32 logits of the whole vocabulary; the reference may also run
- *      a subset of the head's rows, DFlashDraft.cpp:44-52, which is the caller's choice of `head` here) and the selector's
+ *      then the final norm, the target's vocabulary head (fp32 logits; of the whole vocabulary, or of a subset of the
+ *      tokens when `head` is a view of the head's rows, spo_projection_rows: the reference's subsetRows, DFlashDraft.cpp:44-52,
+ *      the logits rows then holding the view's columns) and the selector's
  *      projection, as spo_draft_add_candidates reads them. The context side turns the target's captured hidden rows
  *      (target_layers layers' rows concatenated) into each layer's ring keys and values and the 4-bit window. The handle
  *      owns the step's buffers and the state of max_lanes lanes (lane l of a call uses state l); projections may be of any

@@ -125,6 +125,15 @@ sp_status spo_projection_create(uint32_t segments, const uint32_t *formats, cons
     *out = p;
   });
 }
+sp_status spo_projection_rows(const spo_projection *projection, const uint32_t *firsts, const uint32_t *counts, uint32_t ranges,
+                              spo_projection **out) {
+  return capi::guard([&] {
+    capi::require(projection && firsts && counts && out, "projection, ranges or result");
+    if (!ranges || ranges > 2) throw std::invalid_argument("a row view takes one or two ranges");
+    const ops::Projection &p = projection->projection;
+    *out = new spo_projection{ranges == 1 ? p.rows({{firsts[0], counts[0]}}) : p.rows({{firsts[0], counts[0]}, {firsts[1], counts[1]}})};
+  });
+}
 void spo_projection_destroy(spo_projection *projection) { delete projection; }
 uint64_t spo_projection_weight_bytes(const spo_projection *projection) {
   return projection ? projection->projection.weightBytes() : 0;

@@ -48,24 +48,16 @@ ops::DraftRings ringsOf(const hip::Buffer &rings, std::span<const DFlashLaneStat
 } // namespace
 
 ops::Projection projectionRowsFrom(const ops::Projection &projection, uint32_t first) {
-  const std::vector<ops::QuantizedSegment> &segments = projection.blocks().segments;
-  if (segments.size() != 1 || first % GGUF_TILE_COLUMNS || first >= projection.outputSize)
-    throw std::invalid_argument("a row range of a projection starts on a tile of one segment");
-  const ops::QuantizedSegment &whole = segments[0];
-  const uint64_t offset = gguf_image_bytes(whole.formatId, first, whole.inputSize);
-  const uint32_t rows = projection.outputSize - first;
-  ops::BlockWeights view;
-  view.segments.push_back(ops::QuantizedSegment::ofImage(whole.formatId, rows, whole.inputSize,
-                                                         whole.image.slice(offset, gguf_image_bytes(whole.formatId, rows, whole.inputSize))));
-  return ops::Projection(rows, projection.inputSize, std::move(view));
+  if (first >= projection.outputSize) throw std::invalid_argument("a row range of a projection starts inside it");
+  return projection.rows({{first, projection.outputSize - first}});
 }
 
 DFlashDraft::DFlashDraft(const DFlashDraftWeights &weights, const ops::Linear &linear, const ops::Projection &head)
     : weights_(weights), linear_(linear), head_(head) {
   requireWeights(weights);
-  if (head.outputSize != weights.layout.vocabularySize || head.inputSize != weights.layout.hiddenSize ||
+  if (!head.outputSize || head.outputSize > weights.layout.vocabularySize || head.inputSize != weights.layout.hiddenSize ||
       head.destination != ops::FloatOutput::Float32)
-    throw std::invalid_argument("the draft shares the target's vocabulary head, fp32 logits over its hidden size");
+    throw std::invalid_argument("the draft shares the target's vocabulary head (or a view of its rows), fp32 logits over its hidden size");
 }
 
 ops::LinearScratchSize DFlashDraft::scratchSize(uint32_t rows) const {

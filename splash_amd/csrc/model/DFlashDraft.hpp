@@ -94,7 +94,8 @@ struct DFlashContextBuffers final {
 
 class DFlashDraft final {
 public:
-  // `head`: the target's vocabulary head (fp32 logits), which the draft shares.
+  // `head`: the target's vocabulary head (fp32 logits), which the draft shares: whole, or a view of the rows of a subset
+  // of the tokens (ops::Projection::rows over DraftVocabulary's two ranges), whose columns the logits rows then hold.
   DFlashDraft(const DFlashDraftWeights &weights, const ops::Linear &linear, const ops::Projection &head);
 
   [[nodiscard]] const DFlashDraftLayout &layout() const noexcept { return weights_.layout; }

@@ -68,6 +68,34 @@ public:
     }
   }
   [[nodiscard]] const BlockWeights &blocks() const noexcept { return weights_; }
+  // Rows [first, first + count) of a projection's weights (Weights.hpp:193-204 in the reference).
+  struct RowRange final {
+    uint32_t first = 0;
+    uint32_t count = 0;
+  };
+  // A view of a projection of one tensor over the rows of `ranges`, whole 16-row tiles of them (an empty range holds
+  // none), which become its output columns in order: segments over slices of the same image (an image is rows of
+  // sixteen columns, so a range of whole tiles is contiguous in it), no copy. The draft's head over a subset of the
+  // vocabulary (DraftVocabulary::rows) and its context writers' key and value rows are such views.
+  [[nodiscard]] Projection rows(std::initializer_list<RowRange> ranges) const {
+    if (weights_.segments.size() != 1) throw std::invalid_argument("a row view is of a projection of one tensor");
+    const QuantizedSegment &whole = weights_.segments.front();
+    BlockWeights view;
+    uint32_t covered = 0;
+    for (const RowRange &range : ranges) {
+      if (range.first % GGUF_TILE_COLUMNS || range.count % GGUF_TILE_COLUMNS || range.first > outputSize || range.count > outputSize - range.first)
+        throw std::invalid_argument("a row view takes whole 16-row tiles inside the projection");
+      if (!range.count) continue;
+      view.segments.push_back(QuantizedSegment::ofImage(whole.formatId, range.count, inputSize,
+                                                        whole.image.slice(gguf_image_bytes(whole.formatId, range.first, inputSize),
+                                                                          gguf_image_bytes(whole.formatId, range.count, inputSize)),
+                                                        covered));
+      covered += range.count;
+    }
+    Projection result(covered, inputSize, std::move(view));
+    result.destination = destination;
+    return result;
+  }
   // Native bytes of its weights: what one pass over it streams from HBM.
   [[nodiscard]] uint64_t weightBytes() const noexcept {
     uint64_t bytes = 0;

@@ -60,6 +60,18 @@ class Projection:
         self.output_size = sum(s[1] for s in segments)
         self.float32 = float32
 
+    def rows(self, ranges):
+        """ops::Projection::rows: a view over one or two (first, count) ranges of this projection's rows, whole 16-row
+        tiles, which become its output columns in order; slices of the same image."""
+        firsts = (ctypes.c_uint32 * len(ranges))(*[r[0] for r in ranges])
+        counts = (ctypes.c_uint32 * len(ranges))(*[r[1] for r in ranges])
+        h = ctypes.c_void_p()
+        check(lib.spo_projection_rows(self.handle, firsts, counts, len(ranges), ctypes.byref(h)))
+        view = Projection.__new__(Projection)
+        view.handle, view.segments, view.input_size = h, self.segments, self.input_size    # the segments keep the image alive
+        view.output_size, view.float32 = sum(r[1] for r in ranges), self.float32
+        return view
+
     @classmethod
     def from_native(cls, backend, segments, input_size, float32=False):
         """segments: [(fmt, rows, native uint8 array)]; packs and uploads each image."""

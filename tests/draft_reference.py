@@ -43,7 +43,8 @@ class DraftModel:
         self.head = quant(vocabulary, hidden, orc.FMT_Q6K)
 
     # ------------------------------------------------------------------ GPU side
-    def build_gpu(self, backend, max_lanes, context_rows=0):
+    def build_gpu(self, backend, max_lanes, context_rows=0, head_ranges=None):
+        """head_ranges: [(first, count)] rows of the head the draft's logits cover (a vocabulary subset); all of them by default."""
         gpu = verify.DFlashDraft(backend, self.layer_count, self.hidden, self.vocabulary, self.intermediate, self.target_layers, max_lanes,
                                  context_rows)
         P = lambda native, n, k, fmt=orc.FMT_Q4K, f32=False: ops.Projection.from_native(backend, [(fmt, n, native)], k, float32=f32)
@@ -53,9 +54,10 @@ class DraftModel:
                           mlp_dynamic=P(w["mlp_dynamic"], H // 4, H), gate=P(w["gate"], F, H), up=P(w["up"], F, H), down=P(w["down"], H, F),
                           **{name: backend.from_array(w[name]) for name in ("input_norm", "attention_convolution", "query_norm", "key_norm",
                                                                              "post_attention_norm", "mlp_convolution")})
+        head = P(self.head, self.vocabulary, H, orc.FMT_Q6K, True)
         gpu.set_model(P(self.context_projection, H, self.target_layers * H), backend.from_array(self.hidden_norm),
                       backend.from_array(self.final_norm), P(self.selector, 256, H), backend.from_array(self.mask_embedding),
-                      P(self.head, self.vocabulary, H, orc.FMT_Q6K, True))
+                      head.rows(head_ranges) if head_ranges else head)
         return gpu
 
     # ------------------------------------------------------------------ oracle side

@@ -226,6 +226,43 @@ def test_rings_rebuilt_from_the_window(backend, draft):
         assert cosine(orc.bf16_to_f32(got_keys[:, slots]), orc.bf16_to_f32(old_keys[:, slots])) > 0.98
 
 
+def test_a_head_over_a_subset_of_the_vocabulary(backend):
+    """The draft's logits over the target's first 1024 tokens and those from 3072 on (the reference's DraftVocabulary): the
+    head is a view of the same image's rows, its logits those columns of the whole head's (inside the projection's fp64
+    interval, both), and the candidates name the tokens, not the columns."""
+    print("case draft model vocabulary subset", flush=True)
+    model = DraftModel(seed=33, hidden=1024, vocabulary=4096, intermediate=1024, layers=1, target_layers=1)
+    rng = np.random.default_rng(9)
+    hidden = bits(rng.standard_normal((ROWS, model.hidden)))
+    cosines, sines = rope_tables(np.arange(16))
+    logits = {}
+    for name, ranges in (("whole", None), ("subset", [(0, 1024), (3072, 1024)])):
+        gpu = model.build_gpu(backend, max_lanes=1, head_ranges=ranges)
+        gpu.buffer(verify.DFLASH_HIDDEN, 0).upload(hidden)
+        gpu.buffer(verify.DFLASH_ROPE_COS).upload(cosines)
+        gpu.buffer(verify.DFLASH_ROPE_SIN).upload(sines)
+        backend.run(gpu.encode_decode([0]))
+        columns = 2048 if ranges else 4096
+        logits[name] = gpu.buffer(verify.DFLASH_LOGITS).download(np.float32)[:ROWS * columns].reshape(ROWS, columns).copy()
+        final = gpu.buffer(verify.DFLASH_FINAL_HIDDEN).download(np.uint16)[:ROWS * model.hidden].reshape(ROWS, model.hidden).copy()
+        if ranges:
+            candidates, unary = backend.allocate_buffer(7 * 16 * 4), backend.allocate_buffer(7 * 16 * 4)
+            graph = splash_amd.CommandGraph()
+            ops.DraftSelector.add_candidates(graph, gpu.buffer(verify.DFLASH_LOGITS), gpu.buffer(verify.DFLASH_SELECTOR_HIDDEN),
+                                             backend.allocate_buffer(max(ops.DraftSelector.candidate_scratch_bytes(1, columns), 16)), candidates, unary,
+                                             backend.allocate_buffer(7 * 256 * 4), backend.from_array(bits(rng.standard_normal((4096, 256)) * 0.1)),
+                                             backend.from_array(bits(rng.standard_normal((4096, 256)) * 0.1)), 1024, 3072, 4096, [5])
+            backend.run(graph)
+            want_ids, want_logits = orc.draft_candidates(logits[name], 1, leading=1024, trailing=3072)
+            ids = candidates.download(np.uint32).reshape(7, 16)
+            assert np.array_equal(ids, want_ids) and np.all((ids < 1024) | (ids >= 3072)) and (ids >= 3072).any()
+        gpu.close()
+    exact = orc.gemm(orc.FMT_Q6K, model.head, final, model.vocabulary, want=("exact", "bound"))
+    keep = np.r_[0:1024, 3072:4096]
+    assert np.all(np.abs(logits["whole"] - exact["exact"]) <= exact["bound"] + 1e-6)
+    assert np.all(np.abs(logits["subset"] - exact["exact"][:, keep]) <= exact["bound"][:, keep] + 1e-6)
+
+
 def test_the_draft_refuses_what_it_cannot_run(backend, draft):
     print("case draft model refusals", flush=True)
     model, gpu = draft
