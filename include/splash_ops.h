@@ -736,6 +736,8 @@ void spo_hybrid_verify_destroy(spo_hybrid_verify *verify);
 sp_status spo_hybrid_verify_set_layer(spo_hybrid_verify *verify, uint32_t layer, const spo_hybrid_layer *weights);
 sp_status spo_hybrid_verify_set_head(spo_hybrid_verify *verify, uint32_t embedding_format, sp_buffer *embedding_rows,
                                      sp_buffer *final_norm, const spo_projection *head);
+/* As spo_dense_verify_set_capture: the hidden rows after the named layers, for a draft's context. */
+sp_status spo_hybrid_verify_set_capture(spo_hybrid_verify *verify, const uint32_t *layers, uint32_t count, sp_buffer *destination);
 /* The step's buffers, as spo_dense_verify_buffer; `index` is the attention layer for KV pools. */
 #define SPO_VERIFY_GDN_STATES 13
 #define SPO_VERIFY_GDN_TAPE 14

@@ -71,6 +71,13 @@ sp_status spo_hybrid_verify_create_chunked(sp_backend *backend, const spo_hybrid
 }
 void spo_hybrid_verify_destroy(spo_hybrid_verify *verify) { delete verify; }
 
+sp_status spo_hybrid_verify_set_capture(spo_hybrid_verify *verify, const uint32_t *layers, uint32_t count, sp_buffer *destination) {
+  return capi::guard([&] {
+    capi::require(verify && (layers || !count), "verify or layers");
+    verify->verify->setCapture(std::vector<uint32_t>(layers, layers + count), B(destination));
+  });
+}
+
 sp_status spg_hybrid_dimensions(const spg_file *file, spo_hybrid_dimensions *out) {
   return capi::guard([&] {
     capi::require(out, "result");

@@ -303,6 +303,22 @@ void HybridVerify::encodeHead(hip::CommandGraph &graph, uint32_t rows, bool inpu
   });
 }
 
+void HybridVerify::setCapture(std::vector<uint32_t> layers, hip::Buffer destination) {
+  for (size_t i = 0; i < layers.size(); ++i)
+    if (layers[i] >= dims_.layers || (i && layers[i] <= layers[i - 1])) throw std::invalid_argument("captured layers are the model's, ascending");
+  if (!layers.empty())
+    ops::requireBytes(destination, uint64_t{std::max(maxRows_, rowCapacity_)} * layers.size() * dims_.hidden * 2, "captured target hidden rows");
+  captureLayers_ = std::move(layers);
+  captured_ = std::move(destination);
+}
+
+void HybridVerify::encodeCapture(hip::CommandGraph &graph, uint32_t layer, uint32_t rows) const {
+  for (size_t slot = 0; slot < captureLayers_.size(); ++slot)
+    if (captureLayers_[slot] == layer)
+      ops::RowCopy::add(graph, hidden_[0], {0, dims_.hidden, 0}, captured_,
+                        {0, uint32_t(captureLayers_.size()) * dims_.hidden, uint32_t(slot) * dims_.hidden}, rows, dims_.hidden);
+}
+
 void HybridVerify::encode(hip::CommandGraph &graph, const std::vector<HybridLane> &lanes, bool commit) {
   if (lanes.empty() || lanes.size() > maxLanes_) throw std::invalid_argument("the step takes 1 to its most lanes");
   std::vector<ops::LaneRows> laneRows;
@@ -329,7 +345,10 @@ void HybridVerify::encode(hip::CommandGraph &graph, const std::vector<HybridLane
     for (const HybridLayer &l : weights_.layers) feeds = feeds && linear_.normsRows(l.ffnDown, rows);
   // float gate rows read the normalized rows themselves, which a layer fed by the combine before it never stores
   for (const HybridLayer &l : weights_.layers) feeds = feeds && !l.gateRows;
-  for (uint32_t layer = 0; layer < dims_.layers; ++layer) encodeLayer(graph, layer, lanes, feeds && layer > 0, feeds);
+  for (uint32_t layer = 0; layer < dims_.layers; ++layer) {
+    encodeLayer(graph, layer, lanes, feeds && layer > 0, feeds);
+    encodeCapture(graph, layer, rows);
+  }
   encodeHead(graph, rows, feeds);
   ops::Sampling::addVerify(graph, sampling_, dims_.vocabulary, dims_.vocabulary, laneRows, policies);
   const ops::AcceptanceBuffers acceptance{inputTokens_, treeRows_, tokens_, retained_, acceptedCount_, retainedRows_};
@@ -442,8 +461,10 @@ void HybridVerify::encodePrefill(hip::CommandGraph &graph, uint32_t lane, uint32
     encodeEmbedding(graph, tokens);
   }
   const uint32_t end = layerCount ? firstLayer + layerCount : dims_.layers;
-  for (uint32_t layer = firstLayer; layer < end; ++layer)
+  for (uint32_t layer = firstLayer; layer < end; ++layer) {
     encodePrefillLayer(graph, layer, plan, tokens, cellOffset(lane, parity), cellOffset(lane, parity ^ 1u));
+    encodeCapture(graph, layer, tokens);
+  }
 }
 
 } // namespace splash::model

@@ -142,6 +142,10 @@ public:
   // Value head h of a GDN layer's output rows leaves at (h % heads per key) * key heads + h / heads per key, the order
   // llama.cpp's ssm_out reads them in (GgufImage.hpp:29-32): what a model loaded from a GGUF sets. Off by default.
   void setTiledGdnHeads(bool tiled) noexcept { tiledGdnHeads_ = tiled; }
+  // The hidden rows a draft's context is computed from (the reference's QwenTarget addCapture over RowCopy): after
+  // layer layers[i] (ascending) every row's output goes to columns [i hidden, (i + 1) hidden) of its row of
+  // `destination`, bf16 [rows][layers.size() x hidden], in a step and in a prompt chunk alike. An empty list captures nothing.
+  void setCapture(std::vector<uint32_t> layers, hip::Buffer destination);
   [[nodiscard]] bool tiledGdnHeads() const noexcept { return tiledGdnHeads_; }
 
   void encode(hip::CommandGraph &graph, const std::vector<HybridLane> &lanes, bool commit = true);
@@ -178,6 +182,9 @@ private:
   ops::Linear linear_;
   uint32_t maxRows_ = 0, maxLanes_ = 0, rowCapacity_ = 0;
   bool tiledGdnHeads_ = false;
+  std::vector<uint32_t> captureLayers_;
+  hip::Buffer captured_;
+  void encodeCapture(hip::CommandGraph &graph, uint32_t layer, uint32_t rows) const;
   ops::GdnPrefillBuffers gdnPrefill_;  // the rows a GDN layer's prefill passes hand each other (a long chunk's)
   uint64_t pageBytes_ = 0, layerBytes_ = 0, cellBytes_ = 0, tapeLayerBytes_ = 0;
   ops::GdnStateStrides strides_;

@@ -264,6 +264,12 @@ class HybridVerify:
         self._keep.extend([mixer_input, mixer_output, input_norm, post_norm, router, gate_images, up_images, down_images, query_norm,
                            key_norm, convolution_weights, decay_weights, time_bias, mixer_norm, shared_scalar_gate, ffn])
 
+    def set_capture(self, layers, destination):
+        """After each of `layers` (ascending) every row's output goes to its slot of `destination`, bf16 [rows][len(layers) x hidden]."""
+        check(lib.spo_hybrid_verify_set_capture(self.handle, (ctypes.c_uint32 * max(len(layers), 1))(*layers), len(layers),
+                                                destination.handle if destination is not None else None))
+        self._keep.append(destination)
+
     def set_head(self, embedding_format, embedding_rows, final_norm, head):
         check(lib.spo_hybrid_verify_set_head(self.handle, embedding_format, embedding_rows.handle, final_norm.handle, head.handle))
         self._keep.extend([embedding_rows, final_norm, head])

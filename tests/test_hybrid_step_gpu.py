@@ -5,6 +5,8 @@ and the state rollback across two steps of two lanes (the accepted path of the f
 import numpy as np
 import pytest
 
+import splash_amd
+
 from splash_amd import ops, verify
 from tests import oracle as orc
 from tests.gdn_case import ulps
@@ -177,6 +179,43 @@ def test_dense_ffn_under_the_hybrid_mixers(backend):
     following = [verify.HybridLane(16, 33 + int(retained[0]), table_first=0, pending_path=int(masks[0]), parity=1),
                  verify.HybridLane(7, 90 + int(retained[1]), table_first=1, pending_path=int(masks[1]), parity=1)]
     check_step(backend, model, gpu, following, rng.integers(0, SHAPE["vocabulary"], 23).astype(np.uint32))
+
+
+def test_hidden_rows_are_captured_for_a_draft(backend):
+    """After the layers a draft reads, every row's output lies in its slot of the capture buffer: the rows the same layers
+    leave when the step runs part by part from the same cells and tapes."""
+    print("case hybrid capture", flush=True)
+    model = HybridModel(seed=43, **SHAPE)
+    gpu = model.build_gpu(backend, max_lanes=2, pages_per_lane=2)
+    rng = np.random.default_rng(6)
+    model.seed_context(rng)
+    model.seed_states(rng, lanes=2)
+    H, layers = SHAPE["hidden"], SHAPE["layers"]
+    lanes = [verify.HybridLane(5, 40, table_first=0), verify.HybridLane(16, 200, table_first=model.pages_per_lane)]
+    rows = 21
+    captured = backend.allocate_buffer(2 * 16 * 2 * H * 2)
+    picked = [1, layers - 1]
+    gpu.set_capture(picked, captured)
+    gpu.set_block(lanes, rng.integers(0, SHAPE["vocabulary"], rows).astype(np.uint32))
+    backend.run(gpu.encode(lanes, commit=False))
+    got = captured.download(np.uint16)[:rows * 2 * H].reshape(rows, 2, H).copy()
+    hidden_of = lambda: gpu.buffer(verify.HIDDEN, 0).download(np.uint16, rows * H).reshape(rows, H)
+    assert np.array_equal(got[:, 1], hidden_of())          # the last layer's rows are what the step left
+    alone = backend.allocate_buffer(2 * 16 * H * 2)
+    gpu.set_capture([1], alone)
+    backend.run(gpu.encode(lanes, commit=False))
+    assert np.array_equal(got[:, 0], alone.download(np.uint16)[:rows * H].reshape(rows, H))
+    # part by part a layer's norm is a pass of its own, where the whole step defers it into the projections: the same
+    # rows to that rounding
+    backend.run(gpu.encode_part(0, 0, lanes))
+    for layer in range(2):
+        backend.run(gpu.encode_part(1, layer, lanes))
+    ok, detail = close_bf16(got[:, 0], hidden_of())
+    assert ok, detail
+    with pytest.raises(splash_amd.SplashError):
+        gpu.set_capture([2, 1], captured)                 # ascending
+    with pytest.raises(splash_amd.SplashError):
+        gpu.set_capture([0, 1, 2], captured)              # a destination too small for three layers' rows
 
 
 def test_hybrid_rejects_bad_arguments(backend):
