@@ -58,7 +58,7 @@ struct DraftConvParams {
 };
 
 // draft_attention_qkv: grid (40, lanes) of 512 threads: a wave a (row, head) task of the 8 x (32 + 8) a lane, every
-// thread a share of the value rows' transpose. draft_attention_merge: grid (8 KV heads, lanes), 256 threads.
+// thread a share of the value rows' transpose. draft_attention_merge: grid (8 KV heads, lanes), 1024 threads.
 struct DraftLanesParams {
   uint32_t lanes;
 };

@@ -303,40 +303,37 @@ __global__ __launch_bounds__(256) void draft_attention_split(const uint16_t *__r
 }
 
 // The 17 partials of a (lane, KV head) in their order into the lane's rows, [query row][query head][dimension]: the
-// output projection's input, in the place of the grouped queries every split has read.
-__global__ __launch_bounds__(256) void draft_attention_merge(const float *__restrict__ partials, uint16_t *__restrict__ output, DraftLanesParams) {
-  const uint32_t head = blockIdx.x, batch = blockIdx.y, row = threadIdx.x / 8u, c = threadIdx.x % 8u;
+// output projection's input, in the place of the grouped queries every split has read. A thread holds four dimensions
+// of a row: its 17 splits' loads are in flight together, one round trip to memory.
+__global__ __launch_bounds__(1024) void draft_attention_merge(const float *__restrict__ partials, uint16_t *__restrict__ output, DraftLanesParams) {
+  const uint32_t head = blockIdx.x, batch = blockIdx.y, row = threadIdx.x / 32u, c = threadIdx.x % 32u;
   const float *from = partials + (size_t(batch) * kKvHeads + head) * DRAFT_ATTENTION_SPLITS * DRAFT_ATTENTION_PARTIAL_FLOATS;
   // Every split's maximum, sum and outputs are loaded whatever the split holds, so the loads do not wait for each other;
   // a split with no visible key (a maximum of -inf) wrote no outputs, and what its place holds is set aside, not added.
   float splitMax[DRAFT_ATTENTION_SPLITS], splitSum[DRAFT_ATTENTION_SPLITS], most = -INFINITY;
+  float4 four[DRAFT_ATTENTION_SPLITS];
 #pragma unroll
   for (uint32_t split = 0; split < DRAFT_ATTENTION_SPLITS; ++split) {
     splitMax[split] = from[split * DRAFT_ATTENTION_PARTIAL_FLOATS + kM * kD + row];
     splitSum[split] = from[split * DRAFT_ATTENTION_PARTIAL_FLOATS + kM * kD + kM + row];
+    four[split] = *reinterpret_cast<const float4 *>(from + split * DRAFT_ATTENTION_PARTIAL_FLOATS + row * kD + 4u * c);
     most = fmaxf(most, splitMax[split]);
   }
-  float total = 0.f, acc[16];
-#pragma unroll
-  for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+  float total = 0.f, acc[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
   for (uint32_t split = 0; split < DRAFT_ATTENTION_SPLITS; ++split) {
-    const float4 *partial = reinterpret_cast<const float4 *>(from + split * DRAFT_ATTENTION_PARTIAL_FLOATS + row * kD + 16u * c);
     const bool live = splitMax[split] != -INFINITY;
     const float scale = __builtin_amdgcn_exp2f(splitMax[split] - most);
     if (live) total += scale * splitSum[split];
+    const float values[4] = {four[split].x, four[split].y, four[split].z, four[split].w};
 #pragma unroll
-    for (int v = 0; v < 4; ++v) {
-      const float4 four = partial[v];
-      const float values[4] = {four.x, four.y, four.z, four.w};
-#pragma unroll
-      for (int i = 0; i < 4; ++i) acc[4 * v + i] += live ? scale * values[i] : 0.f;
-    }
+    for (int i = 0; i < 4; ++i) acc[i] += live ? scale * values[i] : 0.f;
   }
   const uint32_t queryRow = row % kRows, queryHead = head * (kM / kRows) + row / kRows;
-  uint16_t *to = output + size_t(batch) * kRows * DRAFT_ATTENTION_WIDTH + (queryRow * kQueryHeads + queryHead) * kD + 16u * c;
-#pragma unroll
-  for (int i = 0; i < 16; ++i) to[i] = uint16_t(float_to_bf16_bits(acc[i] / total));
+  uint16_t *to = output + size_t(batch) * kRows * DRAFT_ATTENTION_WIDTH + (queryRow * kQueryHeads + queryHead) * kD + 4u * c;
+  const uint32_t low = float_to_bf16_bits(acc[0] / total) | (float_to_bf16_bits(acc[1] / total) << 16);
+  const uint32_t high = float_to_bf16_bits(acc[2] / total) | (float_to_bf16_bits(acc[3] / total) << 16);
+  *reinterpret_cast<uint2 *>(to) = make_uint2(low, high);
 }
 
 // A wave a (row, group of 64 values): lane l holds value l; the code of x is round((x - minimum) / scale) with the scale

@@ -121,7 +121,8 @@ void DraftAttention::addDecode(hip::CommandGraph &graph, const DraftDecodeAttent
   const hip::Buffer partials = buffers.groupedQueries.slice(queryRowsBytes(plan), workspace.groupedQueriesBytes - queryRowsBytes(plan));
   graph.add("draft_attention_split", {buffers.groupedQueries, buffers.rings.buffer, buffers.queryKeys, buffers.queryValues, partials}, params,
             {DRAFT_ATTENTION_KV_HEADS, lanes, DRAFT_ATTENTION_SPLITS});
-  graph.add("draft_attention_merge", {partials, buffers.groupedQueries}, DraftLanesParams{lanes}, {DRAFT_ATTENTION_KV_HEADS, lanes, 1});
+  graph.add("draft_attention_merge", {partials, buffers.groupedQueries}, DraftLanesParams{lanes}, {DRAFT_ATTENTION_KV_HEADS, lanes, 1},
+            {1024, 1, 1});
 }
 
 void DraftAttention::addContextPrefill(hip::CommandGraph &graph, const hip::Buffer &contextKv, const hip::Buffer &keyNorm,
