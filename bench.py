@@ -728,6 +728,9 @@ def main():
     ap.add_argument("--prompt-chunk", type=int, default=0,
                     help="instead of the verify step: a chunk of this many prompt tokens (up to 2048) of one sequence "
                          "through every layer, no head (DenseVerify.encode_prefill)")
+    ap.add_argument("--staged-prefill", action="store_true",
+                    help="with --prompt-chunk above a step's rows: the chunk's projections through the prefill tile (the staged "
+                         "rule, as the reference's prompt chunks run) instead of windows of the step's kernels")
     ap.add_argument("--calibrate-traffic", action="store_true",
                     help="after the steps, run plain read and copy kernels of known size: the scale of the FETCH_SIZE / "
                          "WRITE_SIZE counters of a rocprofv3 --pmc run of this command")
@@ -772,6 +775,8 @@ def main():
     if args.prompt_chunk:
         # a prompt chunk that ends the context: every layer, no head
         tokens = args.prompt_chunk
+        if args.staged_prefill:
+            gpu.set_staged_prefill(True)
         gpu.set_prefill_block(rng.integers(0, w["vocabulary"], tokens).astype(np.uint32))
         command = backend.record(gpu.encode_prefill(0, w["context"] - tokens, tokens))
         for _ in range(args.warmup):
@@ -781,6 +786,7 @@ def main():
         print(json.dumps({"metric": "prompt chunk ms (every layer of the 27B shape, no head)", "value": round(seconds * 1e3, 4),
                           "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "tokens": tokens,
                           "tokens_per_s": round(tokens / seconds, 1), "higher_is_better": False, "data": "synthetic",
+                          "projections": "prefill tile, staged rule" if args.staged_prefill else "the step's kernels, register rule",
                           "config": {"workload": w["name"] if "name" in w else args.workload, "context_tokens": w["context"]}}), flush=True)
         return
     graph = gpu.encode(lanes, commit=True)

@@ -619,6 +619,11 @@ sp_status spo_dense_verify_set_layer(spo_dense_verify *verify, uint32_t layer, c
                                      sp_buffer *query_norm, sp_buffer *key_norm);
 sp_status spo_dense_verify_set_head(spo_dense_verify *verify, uint32_t embedding_format, sp_buffer *embedding_rows,
                                     sp_buffer *final_norm, const spo_projection *head);
+/* DenseVerify::setStagedPrefill: a prompt chunk of more rows than a step's runs its projections through the prefill tile
+ * (spo_linear_add_prefill: the staged rule, as the reference's prompt chunks do, LinearTile::GgufPrefill), its norms and
+ * SwiGLU as passes of their own; off by default (the chunk then equals its blocks run as steps bit for bit). Needs a
+ * driver created with prefill_rows and tensors of whole 128-column workgroups. */
+sp_status spo_dense_verify_set_staged_prefill(spo_dense_verify *verify, int on);
 /* The hidden rows a draft's context is computed from (QwenTarget's addCapture over RowCopy, runtime/ops/RowCopy.hpp:17-28):
  * after layer layers[i] (ascending) every row's output goes to columns [i * hidden, (i + 1) * hidden) of its row of
  * destination, bf16 [rows][count * hidden], in a step and in a prompt chunk alike; what spo_dflash_draft's context calls

@@ -342,6 +342,7 @@ _sig("spo_sampling_greedy_rows_static", c_int, ctypes.c_void_p, c_u32, c_u32, c_
 _sig("spo_verify_check_results", c_int, P(LaneRows), P(c_u32), c_u32, c_u32, c_u32, P(c_u32), P(c_u32), P(c_u32), P(c_u32))
 _sig("spo_projection_rows", c_int, c_p, P(c_u32), P(c_u32), c_u32, P(c_p))
 _sig("spo_hybrid_verify_set_capture", c_int, c_p, P(c_u32), c_u32, c_p)
+_sig("spo_dense_verify_set_staged_prefill", c_int, c_p, c_int)
 _sig("spo_dense_verify_set_capture", c_int, c_p, P(c_u32), c_u32, c_p)
 _sig("spo_dense_verify_set_chained", c_int, c_p, c_int)
 _sig("spo_dense_verify_chain_status", c_int, c_p, ctypes.POINTER(ctypes.c_uint32))

@@ -35,6 +35,12 @@ struct RowCopyParams {
   uint32_t to_row, to_stride, to_column;
 };
 
+// swiglu_rows: out = bf16(up * silu(gate)) over `count` bf16 values, eight a thread (the epilogue of the one-pass gate/up
+// projection, GGUF_EPILOGUE_GATE_UP, as a pass of its own for rows whose gate and up were projected apart).
+struct SwiGluRowsParams {
+  uint64_t count;
+};
+
 // gguf_float_<f32|bf16>_<f32|bf16>: the fp32 projection of weights kept as rows (the reference's GgufFloatParams,
 // abi/Gguf.h:204, kernels/shared/gguf_float.metal): out[r][out_offset + n] = sum_k x[r][k] W[n][k], x the bf16 rows,
 // W F32 or BF16 rows as stored, every operand exact in fp32. A sum runs four chains of fused multiply-adds, chain j

@@ -207,6 +207,13 @@ sp_status spo_draft_add_verify_row_slots(spo_graph *graph, sp_buffer *tree_token
   });
 }
 
+sp_status spo_dense_verify_set_staged_prefill(spo_dense_verify *verify, int on) {
+  return capi::guard([&] {
+    capi::require(verify, "verify");
+    verify->verify->setStagedPrefill(on != 0);
+  });
+}
+
 sp_status spo_dense_verify_set_capture(spo_dense_verify *verify, const uint32_t *layers, uint32_t count, sp_buffer *destination) {
   return capi::guard([&] {
     capi::require(verify && (layers || !count), "verify or layers");

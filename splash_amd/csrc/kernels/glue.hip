@@ -130,6 +130,28 @@ __global__ __launch_bounds__(256) void copy_rows_bf16(const uint16_t *__restrict
 }
 SP_REGISTER_KERNEL("copy_rows_bf16", &copy_rows_bf16);
 
+__global__ __launch_bounds__(256) void swiglu_rows(const uint16_t *__restrict__ gate, const uint16_t *__restrict__ up,
+                                                   uint16_t *__restrict__ output, SwiGluRowsParams p) {
+  const uint64_t first = (uint64_t(blockIdx.x) * 256u + threadIdx.x) * 8u;
+  if (first >= p.count) return;
+  if (first + 8u <= p.count) {
+    const uint4 g = *reinterpret_cast<const uint4 *>(gate + first), u = *reinterpret_cast<const uint4 *>(up + first);
+    const uint32_t gw[4] = {g.x, g.y, g.z, g.w}, uw[4] = {u.x, u.y, u.z, u.w};
+    uint32_t out[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t low = float_to_bf16_bits(bf16_bits_to_float(uw[i] & 0xFFFFu) * silu(bf16_bits_to_float(gw[i] & 0xFFFFu)));
+      const uint32_t high = float_to_bf16_bits(bf16_bits_to_float(uw[i] >> 16) * silu(bf16_bits_to_float(gw[i] >> 16)));
+      out[i] = low | (high << 16);
+    }
+    *reinterpret_cast<uint4 *>(output + first) = make_uint4(out[0], out[1], out[2], out[3]);
+  } else {
+    for (uint64_t i = first; i < p.count; ++i)
+      output[i] = uint16_t(float_to_bf16_bits(bf16_bits_to_float(up[i]) * silu(bf16_bits_to_float(gate[i]))));
+  }
+}
+SP_REGISTER_KERNEL("swiglu_rows", &swiglu_rows);
+
 __global__ void rope_build_tree_tables(const float *__restrict__ inverse_frequency, const uint32_t *__restrict__ depth,
                                        float *__restrict__ cosines, float *__restrict__ sines, RopeTreeParams p) {
   const uint32_t row = blockIdx.x, pair = threadIdx.x;

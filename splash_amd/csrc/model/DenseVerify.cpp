@@ -334,6 +334,36 @@ void DenseVerify::encodeHead(hip::CommandGraph &graph, uint32_t rows, bool input
   linear_.add(graph, head, weights_.head, linear_.plan(weights_.head, rows));
 }
 
+void DenseVerify::setStagedPrefill(bool staged) {
+  if (staged && !prefillTable_) {
+    if (rowCapacity_ <= maxRows_) throw std::invalid_argument("the driver was created without room for a long prompt chunk");
+    const uint32_t widest = std::max({dims_.hidden, dims_.attentionWidth(), dims_.ffn});
+    prefillTable_ = backend_.allocateBuffer(ops::Linear::prefillTableBytes(widest, rowCapacity_), BufferStorage::Private, "prefill tables");
+    const uint64_t ffnBytes = uint64_t{rowCapacity_} * dims_.ffn * 2;
+    gateRows_ = backend_.allocateBuffer(ffnBytes, BufferStorage::Private, "prefill gate rows");
+    upRows_ = backend_.allocateBuffer(ffnBytes, BufferStorage::Private, "prefill up rows");
+    swigluRows_ = backend_.allocateBuffer(ffnBytes, BufferStorage::Private, "prefill SwiGLU rows");
+  }
+  stagedPrefill_ = staged;
+}
+
+// A layer of a long chunk under the staged rule: each projection one pass of the prefill tile over all the rows.
+void DenseVerify::encodeStagedChunkLayer(hip::CommandGraph &graph, uint32_t layer, const ops::AttentionChunkPlan &plan, uint32_t tokens) {
+  const DenseLayer &w = weights_.layers.at(layer);
+  const hip::Buffer &residual = hidden_[0], &next = hidden_[1];
+  ops::Normalization::addRms(graph, residual, w.inputNorm, normalized_, dims_.hidden, tokens);
+  ops::Linear::addPrefill(graph, normalized_, w.qkv, qkv_, {}, prefillTable_, tokens);
+  const ops::KvPages pages{pageTable_, kvPools_.at(layer), pageBytes_};
+  ops::PagedAttention::addChunkProjection(graph, plan, {qkv_, w.queryNorm, w.keyNorm, ropeCos_, ropeSin_}, attentionWorkspace_, pages);
+  ops::PagedAttention::addChunkAttention(graph, plan, attentionWorkspace_, treeRows_, pages, attention_);
+  ops::Linear::addPrefill(graph, attention_, w.output, next, residual, prefillTable_, tokens);
+  ops::Normalization::addRms(graph, next, w.postNorm, normalized_, dims_.hidden, tokens);
+  ops::Linear::addPrefill(graph, normalized_, w.gate, gateRows_, {}, prefillTable_, tokens);
+  ops::Linear::addPrefill(graph, normalized_, w.up, upRows_, {}, prefillTable_, tokens);
+  ops::SwiGlu::add(graph, gateRows_, upRows_, swigluRows_, uint64_t{tokens} * dims_.ffn);
+  ops::Linear::addPrefill(graph, swigluRows_, w.down, residual, next, prefillTable_, tokens);
+}
+
 // A layer of a long chunk: every window's q|k|v rows, the chunked attention over all of them, then every window's output
 // projection and SwiGLU. Each window's projections and tables are the ones encodeLayer gives a step of its rows.
 void DenseVerify::encodeChunkLayer(hip::CommandGraph &graph, uint32_t layer, const ops::AttentionChunkPlan &plan, uint32_t tokens,
@@ -422,7 +452,8 @@ void DenseVerify::encodePrefill(hip::CommandGraph &graph, uint32_t tableFirst, u
     // every window is a step's worth of rows at most, so what holds for one holds for all
     const bool feeds = layersFeedNext(std::min(tokens, kWindowRows));
     for (uint32_t layer = 0; layer < dims_.layers; ++layer) {
-      encodeChunkLayer(graph, layer, plan, tokens, feeds && layer > 0, feeds && layer + 1 < dims_.layers);
+      if (stagedPrefill_) encodeStagedChunkLayer(graph, layer, plan, tokens);
+      else encodeChunkLayer(graph, layer, plan, tokens, feeds && layer > 0, feeds && layer + 1 < dims_.layers);
       encodeCapture(graph, layer, tokens);
     }
     return;

@@ -120,6 +120,14 @@ public:
   // that completes a head prepares its sixteen rows alone (four a wave, about 4 us of vector arithmetic), where the
   // prepare kernel spreads them over 1280 workgroups.
   void setFusedPrepare(bool fused) noexcept { fusedPrepare_ = fused; }
+  // A long prompt chunk (more rows than a step's) runs its projections through the prefill tile (ops::Linear::addPrefill:
+  // 128 rows x 128 columns a workgroup under the staged rule, every weight rounded once to half), as the reference's
+  // prompt chunks do (LinearTile::GgufPrefill, gguf_linear.metal:79-118): the norms and the SwiGLU are passes of their
+  // own, the attention the same chunked plan. Off by default: a chunk then equals its blocks run as steps bit for bit;
+  // on, it equals them to the staged rule's rounding and runs at the matrix cores' rate, not the step kernels'.
+  // Every tensor's columns must be whole 128-column workgroups.
+  void setStagedPrefill(bool staged);
+  [[nodiscard]] bool stagedPrefill() const noexcept { return stagedPrefill_; }
   // The hidden rows a draft's context is computed from (the reference's QwenTarget addCapture over RowCopy,
   // RowCopy.hpp:17-28): after layer layers[i] (ascending), every row's output goes to columns [i hidden, (i + 1) hidden)
   // of its row of `destination`, bf16 [rows][layers.size() x hidden]; a step's rows and a prompt chunk's alike. A
@@ -153,6 +161,9 @@ private:
   hip::Buffer captured_;
   void encodeCapture(hip::CommandGraph &graph, uint32_t layer, uint32_t rows) const;
   ops::SamplingBuffers children_;   // the four candidate-children buffers, bound into a step's sampling buffers when it tests them
+  bool stagedPrefill_ = false;
+  hip::Buffer prefillTable_, gateRows_, upRows_, swigluRows_;  // the staged prompt chunk's tables and SwiGLU rows
+  void encodeStagedChunkLayer(hip::CommandGraph &graph, uint32_t layer, const ops::AttentionChunkPlan &plan, uint32_t tokens);
   hip::Buffer chunkAttentionTable_;  // a long chunk's attention rows as the output projection's tables, every window's
   void encodeChunkLayer(hip::CommandGraph &graph, uint32_t layer, const ops::AttentionChunkPlan &plan, uint32_t tokens, bool first,
                         bool feedsNext);

@@ -79,6 +79,14 @@ void RoPE::addTreeTables(hip::CommandGraph &graph, const hip::Buffer &inverseFre
   graph.add("rope_build_tree_tables", {inverseFrequency, depth, cosines, sines}, params, {params.rows, 1, 1}, {pairs, 1, 1});
 }
 
+void SwiGlu::add(hip::CommandGraph &graph, const hip::Buffer &gate, const hip::Buffer &up, const hip::Buffer &output, uint64_t count) {
+  if (!count || count % 8) throw std::invalid_argument("a SwiGLU pass takes whole vectors of eight values");
+  requireBytes(gate, count * 2, "SwiGLU gate rows");
+  requireBytes(up, count * 2, "SwiGLU up rows");
+  requireBytes(output, count * 2, "SwiGLU rows");
+  graph.add("swiglu_rows", {gate, up, output}, SwiGluRowsParams{count}, {(count / 8 + 255) / 256, 1, 1}, {256, 1, 1});
+}
+
 void RowCopy::add(hip::CommandGraph &graph, const hip::Buffer &source, RowRegion from, const hip::Buffer &destination, RowRegion to,
                   uint32_t rows, uint32_t width) {
   if (!rows || !width || from.column + uint64_t{width} > from.stride || to.column + uint64_t{width} > to.stride)

@@ -43,6 +43,13 @@ public:
                   uint32_t rows, uint32_t outStride, uint32_t outOffset, FloatOutput type);
 };
 
+// output = bf16(up * silu(gate)) over rows of bf16 values: the SwiGLU of rows whose gate and up were projected apart
+// (a prompt chunk under the prefill tile, which has no gate/up epilogue); the arithmetic of LinearEpilogue::GateUp.
+class SwiGlu final {
+public:
+  static void add(hip::CommandGraph &graph, const hip::Buffer &gate, const hip::Buffer &up, const hip::Buffer &output, uint64_t count);
+};
+
 struct RopeSequence final {
   uint32_t firstRow = 0, rows = 0, anchor = 0;
 };

@@ -72,6 +72,10 @@ class DenseVerify:
                                              input_norm.handle, post_norm.handle, query_norm.handle, key_norm.handle))
         self._keep.extend([qkv, output, gate, up, down, input_norm, post_norm, query_norm, key_norm])
 
+    def set_staged_prefill(self, on):
+        """Long prompt chunks through the prefill tile (the staged rule) instead of the step's kernels; off by default."""
+        check(lib.spo_dense_verify_set_staged_prefill(self.handle, int(on)))
+
     def set_capture(self, layers, destination):
         """After each of `layers` (ascending) every row's output goes to its slot of `destination`, bf16 [rows][len(layers) x hidden]."""
         check(lib.spo_dense_verify_set_capture(self.handle, (ctypes.c_uint32 * max(len(layers), 1))(*layers), len(layers),

@@ -362,6 +362,65 @@ def test_a_long_prompt_chunk_equals_its_blocks_one_by_one(backend, prompt_tokens
         gpu.encode_prefill(first, committed, 1025)
 
 
+def test_a_staged_prompt_chunk_is_the_exact_one_to_the_staged_rules_rounding(backend):
+    """The same chunk through the prefill tile (DenseVerify::setStagedPrefill: every weight rounded once to half, as the
+    reference's prompt chunks run): the hidden rows agree with the exact chunk's as two bf16 tensors of several stages do,
+    the keys and values it stored are the exact chunk's codes but for a step here and there, and a verify step on top of
+    the context it built selects the tokens the exact context's step selects wherever the logits' margin exceeds their
+    difference."""
+    print("case staged prompt chunk", flush=True)
+    prompt_tokens, V = 600, 32000
+    model = DenseModel(seed=29, hidden=1024, q_heads=16, kv_heads=8, head_dim=64, ffn=3072, vocabulary=V, layers=3)
+    rng = np.random.default_rng(9)
+    gpu = model.build_gpu(backend, max_lanes=1, context_tokens=[prompt_tokens + 300], prefill_rows=1024)
+    model.seed_context(gpu, None, rng)
+    first, committed = model.table_first[0], 250
+    prompt = rng.integers(0, V, prompt_tokens).astype(np.uint32)
+    block = rng.integers(0, V, 16).astype(np.uint32)
+    pools = lambda: np.concatenate([gpu.buffer(verify.KV_POOL, layer).download(np.uint8) for layer in range(3)])
+    start = pools()
+    seen = {}
+    for staged in (False, True):
+        gpu.set_staged_prefill(staged)
+        for layer in range(3):
+            gpu.buffer(verify.KV_POOL, layer).upload(start.reshape(3, -1)[layer])
+        graph = gpu.encode_prefill(first, committed, prompt_tokens)
+        gpu.set_prefill_block(prompt)
+        backend.run(graph)
+        hidden = gpu.buffer(verify.HIDDEN, 0).download(np.uint16, prompt_tokens * 1024).copy()
+        stored = pools()
+        lane = verify.Lane(16, committed + prompt_tokens, table_first=first)
+        gpu.set_block([lane], block)
+        backend.run(gpu.encode([lane], commit=False))
+        logits = gpu.buffer(verify.LOGITS).download(np.float32, 16 * V).reshape(16, V).copy()
+        seen[staged] = (hidden, stored, logits, len(graph.kernels()))
+    gpu.set_staged_prefill(False)
+    (h0, p0, l0, d0), (h1, p1, l1, d1) = seen[False], seen[True]
+    print(f"  dispatches: {d0} in windows of the step's kernels, {d1} through the prefill tile", flush=True)
+    # Two rules, not two roundings of one: every weight is rounded to half before it multiplies, in every projection of
+    # every layer. The reference holds such rows to cosine 0.9999 and max-abs 2e-2 a stage; over three layers' stages:
+    a, b = orc.bf16_to_f32(h0).astype(np.float64), orc.bf16_to_f32(h1).astype(np.float64)
+    hidden_cosine, error = float((a * b).sum() / np.sqrt((a * a).sum() * (b * b).sum())), np.abs(a - b)
+    print(f"  hidden rows: cosine {hidden_cosine:.6f}, largest difference {error.max():.4f} of magnitudes up to {np.abs(a).max():.2f}, "
+          f"{(error > 2e-2).mean():.5f} of them past 2e-2", flush=True)
+    assert hidden_cosine >= 0.9999 and error.max() <= 6e-2 and (error > 2e-2).mean() <= 2e-3
+    # the keys and values the chunk stored: the same values to a couple of INT8 steps
+    helper = ops.KvPages.__new__(ops.KvPages)
+    helper.kv_heads, helper.head_dim, helper.page_bytes = 8, 64, gpu.page_bytes
+    assert (p0 != p1).any()
+    for layer in range(3):
+        kc0, ks0, vc0, vs0 = helper.unpack_pages(p0.reshape(3, -1, gpu.page_bytes)[layer])
+        kc1, ks1, vc1, vs1 = helper.unpack_pages(p1.reshape(3, -1, gpu.page_bytes)[layer])
+        for c0, s0, c1, s1 in ((kc0, ks0, kc1, ks1), (vc0, vs0, vc1, vs1)):
+            apart = np.abs(c0.astype(np.float64) * s0[..., None] - c1.astype(np.float64) * s1[..., None]) / np.maximum(s0[..., None], 1e-30)
+            assert np.percentile(apart, 99.9) <= 2.5 and apart.max() <= 8, (layer, float(np.percentile(apart, 99.9)), float(apart.max()))
+    cosine = float((l0.astype(np.float64) * l1).sum() / np.sqrt((l0.astype(np.float64) ** 2).sum() * (l1.astype(np.float64) ** 2).sum()))
+    top = np.sort(l0, axis=1)
+    clear = top[:, -1] - top[:, -2] > 2 * np.abs(l0 - l1).max()
+    print(f"  logits cosine {cosine:.6f}, largest difference {np.abs(l0 - l1).max():.4f}, rows with a clear margin {int(clear.sum())}/16", flush=True)
+    assert cosine >= 0.9999 and np.array_equal(l0.argmax(axis=1)[clear], l1.argmax(axis=1)[clear])
+
+
 def test_eight_lanes_equal_each_lane_alone(backend):
     """The driver's most lanes: eight lanes of unequal blocks and histories in one step give, lane by lane, the logits,
     selections and acceptance each lane gives alone, bit for bit."""
