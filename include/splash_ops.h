@@ -37,6 +37,10 @@ uint64_t spo_gguf_image_bytes(uint32_t format, uint32_t rows, uint32_t input_siz
 uint64_t spo_gguf_table_bytes(uint32_t input_size, uint32_t rows);
 sp_status spo_gguf_pack_image(uint32_t format, const uint8_t *native, uint32_t rows, uint32_t input_size, uint8_t *image);
 sp_status spo_gguf_unpack_image(uint32_t format, const uint8_t *image, uint32_t rows, uint32_t input_size, uint8_t *native);
+/* `blocks` Q3_K super-blocks (110 bytes each) as Q6_K blocks (210 bytes each) of the same values, which
+ * spo_gguf_pack_image then takes as format Q6_K: how a Q3_K tensor is read (the reference runs it through kernels of its
+ * own format: runtime/metal/abi/QuantFormat.h GGUF_FMT_Q3K; its values are GGML's dequantize_row_q3_K either way). */
+sp_status spo_gguf_transcode_q3k(const uint8_t *q3k, uint64_t blocks, uint8_t *q6k);
 /* The image's fp32 values [rows][input_size] (the reference's gguf_dequant_test.metal kernel). */
 sp_status spo_gguf_add_dequant(spo_graph *graph, uint32_t format, sp_buffer *image, sp_buffer *out, uint32_t rows,
                                uint32_t input_size);

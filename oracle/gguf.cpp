@@ -8,15 +8,16 @@ using namespace orc;
 
 namespace {
 
-constexpr uint32_t kQ4KBytes = 144, kQ5KBytes = 176, kQ6KBytes = 210, kQ80Bytes = 34, kIQ4XSBytes = 136, kIQ4NLBytes = 18, kBlock = 256;
+constexpr uint32_t kQ4KBytes = 144, kQ5KBytes = 176, kQ6KBytes = 210, kQ3KBytes = 110, kQ80Bytes = 34, kIQ4XSBytes = 136, kIQ4NLBytes = 18, kBlock = 256;
 // The 4-bit non-linear codebook of IQ4_NL and IQ4_XS (ggml's kvalues_iq4nl; GgufFormatReference.hpp:382-403 reads it).
 constexpr int8_t kIQ4Values[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
 constexpr uint32_t kQ6KScales = 128 + 64, kQ6KD = kQ6KScales + 16;  // GgufFormatReference.hpp:61
+constexpr uint32_t kQ3KScales = 32 + 64, kQ3KD = kQ3KScales + 12;    // GgufFormatReference.hpp:62
 
 // Bytes and elements of a native block: the K-quants' super-block of 256, Q8_0's group of 32.
 uint32_t blockBytes(uint32_t fmt) {
   return fmt == ORC_FMT_Q4K ? kQ4KBytes : fmt == ORC_FMT_Q5K ? kQ5KBytes : fmt == ORC_FMT_Q6K ? kQ6KBytes : fmt == ORC_FMT_Q80 ? kQ80Bytes
-         : fmt == ORC_FMT_IQ4XS ? kIQ4XSBytes : fmt == ORC_FMT_IQ4NL ? kIQ4NLBytes : 0;
+         : fmt == ORC_FMT_Q3K ? kQ3KBytes : fmt == ORC_FMT_IQ4XS ? kIQ4XSBytes : fmt == ORC_FMT_IQ4NL ? kIQ4NLBytes : 0;
 }
 uint32_t blockElements(uint32_t fmt) { return fmt == ORC_FMT_Q80 || fmt == ORC_FMT_IQ4NL ? 32 : kBlock; }
 
@@ -30,9 +31,9 @@ void scaleMinK4(const uint8_t *sc, int j, uint8_t &s, uint8_t &m) {
 // (quant_formats.h:105-137); Q6_K has a scale per 16 and code - 32 (quant_formats.h:153-168).
 struct Group {
   uint8_t code[32];
-  float s[2];  // Q4_K, Q5_K: s[0] = s[1] = d * sc; Q6_K: one per 16 elements; Q8_0, IQ4_NL: d; IQ4_XS: d * (ls - 32)
+  float s[2];  // Q4_K, Q5_K: s[0] = s[1] = d * sc; Q6_K, Q3_K: one per 16 elements; Q8_0, IQ4_NL: d; IQ4_XS: d * (ls - 32)
   float m;     // Q4_K, Q5_K: -dmin * mn; the others: 0
-  int bias;    // Q4_K, Q5_K: 0; Q6_K: 32; Q8_0, IQ4_NL, IQ4_XS: 128 (code = value or codebook value + 128)
+  int bias;    // Q4_K, Q5_K: 0; Q6_K: 32; Q3_K: 4; Q8_0, IQ4_NL, IQ4_XS: 128 (code = value or codebook value + 128)
 };
 void readGroup(uint32_t fmt, const uint8_t *row, uint32_t g, Group &out) {
   if (fmt == ORC_FMT_Q80) {   // GgufFormatReference.hpp:453-458: value = d * int8
@@ -63,6 +64,21 @@ void readGroup(uint32_t fmt, const uint8_t *row, uint32_t g, Group &out) {
     out.s[0] = out.s[1] = h2f(d16) * float(ls - 32);  // exact: 11 + 6 bits
     out.m = 0.f;
     out.bias = 128;
+    return;
+  }
+  if (fmt == ORC_FMT_Q3K) {   // GgufFormatReference.hpp:433-451: value = d * (scale - 32) * (two bits, less 4 where the mask bit is clear)
+    const uint8_t *mask = blk, *q = blk + 32 + 32 * (j / 4), *packed = blk + kQ3KScales;
+    uint16_t d16; std::memcpy(&d16, blk + kQ3KD, 2);
+    for (int k = 0; k < 32; ++k) out.code[k] = uint8_t(((q[k] >> (2 * (j % 4))) & 3) | (((mask[k] >> j) & 1) << 2));
+    // Sixteen 6-bit scales in twelve bytes: scale i has its low four bits in the low (i < 8) or high nibble of byte
+    // i % 8 and its high two bits at bit 2 (i / 4) of byte 8 + i % 4.
+    for (uint32_t h = 0; h < 2; ++h) {
+      const uint32_t i = 2 * j + h;
+      const int low = i < 8 ? packed[i] & 15 : packed[i - 8] >> 4, high = (packed[8 + i % 4] >> (2 * (i / 4))) & 3;
+      out.s[h] = h2f(d16) * float((low | (high << 4)) - 32);  // exact: 11 + 6 bits
+    }
+    out.m = 0.f;
+    out.bias = 4;
     return;
   }
   if (fmt == ORC_FMT_Q5K) {   // GgufFormatReference.hpp:405-416: the fifth bits in qh, bit j of byte k
@@ -100,7 +116,7 @@ void readGroup(uint32_t fmt, const uint8_t *row, uint32_t g, Group &out) {
 }
 
 // llama.cpp semantics (GgufFormatReference.hpp:370-381, :405-432, :453-458): Q4_K and Q5_K d*sc*code - dmin*mn
-// with one rounding (both products exact); Q6_K d*sc*(q-32), Q8_0 d*q and the IQ4 codebook formats' s*value, exact.
+// with one rounding (both products exact); Q6_K d*sc*(q-32), Q3_K d*(sc-32)*q (:433-451), Q8_0 d*q and the IQ4 codebook formats' s*value, exact.
 void groupValues(uint32_t fmt, const uint8_t *row, uint32_t g, float *vals) {
   Group grp; readGroup(fmt, row, g, grp);
   for (int k = 0; k < 32; ++k) {
@@ -243,7 +259,7 @@ template <class Scale>
 void makeNativeWith(uint32_t fmt, uint32_t rows, uint32_t K, std::mt19937 &rng, uint8_t *native, Scale scale) {
   const size_t bytes = size_t(rows) * orc_row_bytes(fmt, K), bb = blockBytes(fmt);
   for (size_t i = 0; i < bytes; ++i) native[i] = uint8_t(rng());
-  const uint32_t off = fmt == ORC_FMT_Q6K ? kQ6KD : 0;
+  const uint32_t off = fmt == ORC_FMT_Q6K ? kQ6KD : fmt == ORC_FMT_Q3K ? kQ3KD : 0;
   for (size_t b = 0; b < bytes / bb; ++b) {
     uint8_t *blk = native + b * bb;
     const uint16_t d = scale();

@@ -101,6 +101,7 @@ std::optional<uint32_t> imageFormat(uint32_t ggmlType) noexcept {
     case ggml::kQ4_K: return GGUF_FMT_Q4K;
     case ggml::kQ5_K: return GGUF_FMT_Q5K;
     case ggml::kQ6_K: return GGUF_FMT_Q6K;
+    case ggml::kQ3_K: return GGUF_FMT_Q6K;
     case ggml::kQ8_0: return GGUF_FMT_Q80;
     case ggml::kIQ4_XS: return GGUF_FMT_IQ4XS;
     case ggml::kIQ4_NL: return GGUF_FMT_IQ4NL;
@@ -253,8 +254,16 @@ LoadedImage loadImage(hip::Backend &backend, const GgufFile &file, const GgufTen
   if (!rows || uint64_t{firstRow} + rows > all || rows % GGUF_TILE_COLUMNS || firstRow % GGUF_TILE_COLUMNS || columns % GGUF_BLOCK ||
       columns > UINT32_MAX)
     throw std::invalid_argument("a weight image holds whole 16-row tiles of whole 256-input super-blocks: " + tensor.name);
-  const uint64_t rowBytes = columns / GGUF_BLOCK * gguf_native_bytes(*format);
-  const uint8_t *native = file.data(tensor) + uint64_t{firstRow} * rowBytes;
+  std::vector<uint8_t> rewritten;
+  const uint8_t *native;
+  if (tensor.type == ggml::kQ3_K) {
+    const uint64_t blocks = columns / GGUF_BLOCK * rows;
+    rewritten.resize(blocks * GGUF_Q6K_NATIVE);
+    ops::transcodeQ3KToQ6K(file.data(tensor) + uint64_t{firstRow} * (columns / GGUF_BLOCK * ops::kQ3KNativeBytes), blocks, rewritten.data());
+    native = rewritten.data();
+  } else {
+    native = file.data(tensor) + uint64_t{firstRow} * (columns / GGUF_BLOCK * gguf_native_bytes(*format));
+  }
   std::vector<uint8_t> image(gguf_image_bytes(*format, rows, uint32_t(columns)));
   ops::packGgufImage(*format, native, rows, uint32_t(columns), image.data());
   LoadedImage out;
@@ -264,6 +273,20 @@ LoadedImage loadImage(hip::Backend &backend, const GgufFile &file, const GgufTen
   out.image = backend.allocateBuffer(image.size(), hip::BufferStorage::Private, tensor.name.c_str());
   out.image.upload(image.data(), image.size());
   return out;
+}
+
+hip::Buffer loadNativeRows(hip::Backend &backend, const GgufFile &file, const GgufTensor &tensor, const char *label) {
+  if (tensor.type != ggml::kQ3_K) {
+    hip::Buffer rows = backend.allocateBuffer(tensor.bytes, hip::BufferStorage::Private, label);
+    rows.upload(file.data(tensor), tensor.bytes);
+    return rows;
+  }
+  const uint64_t blocks = tensor.bytes / ops::kQ3KNativeBytes;
+  std::vector<uint8_t> rewritten(blocks * GGUF_Q6K_NATIVE);
+  ops::transcodeQ3KToQ6K(file.data(tensor), blocks, rewritten.data());
+  hip::Buffer rows = backend.allocateBuffer(rewritten.size(), hip::BufferStorage::Private, label);
+  rows.upload(rewritten.data(), rewritten.size());
+  return rows;
 }
 
 RowRuns groupedHeadRows(uint64_t rows, uint64_t from, uint32_t headRows, uint32_t keyHeads, uint32_t valueHeadsPerKey) {
@@ -290,7 +313,8 @@ uint64_t runRows(const RowRuns &runs, uint64_t all) {
 std::vector<uint8_t> gatherNative(const GgufFile &file, const GgufTensor &tensor, uint32_t format, const RowRuns &runs, uint64_t firstColumn,
                                   uint64_t columns) {
   const uint64_t all = tensor.rows(), width = tensor.columns();
-  const uint64_t blockBytes = gguf_native_bytes(format), rowBytes = width / GGUF_BLOCK * blockBytes;
+  const bool q3k = tensor.type == ggml::kQ3_K;
+  const uint64_t blockBytes = q3k ? ops::kQ3KNativeBytes : gguf_native_bytes(format), rowBytes = width / GGUF_BLOCK * blockBytes;
   const uint64_t piece = columns / GGUF_BLOCK * blockBytes, skip = firstColumn / GGUF_BLOCK * blockBytes;
   std::vector<uint8_t> native(runRows(runs, all) * piece);
   const uint8_t *data = file.data(tensor);
@@ -300,6 +324,11 @@ std::vector<uint8_t> gatherNative(const GgufFile &file, const GgufTensor &tensor
   };
   if (runs.empty()) take(0, all);
   for (const RowRun &run : runs) take(run.first, run.rows);
+  if (q3k) {
+    std::vector<uint8_t> rewritten(native.size() / ops::kQ3KNativeBytes * GGUF_Q6K_NATIVE);
+    ops::transcodeQ3KToQ6K(native.data(), native.size() / ops::kQ3KNativeBytes, rewritten.data());
+    return rewritten;
+  }
   return native;
 }
 } // namespace

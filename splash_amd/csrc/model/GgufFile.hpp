@@ -23,7 +23,7 @@ public:
 
 // ggml type ids as GGUF tensor infos store them (ggml-common.h; GgufFile.hpp:35-66 in the reference).
 namespace ggml {
-inline constexpr uint32_t kF32 = 0, kF16 = 1, kQ8_0 = 8, kQ4_K = 12, kQ5_K = 13, kQ6_K = 14, kIQ4_NL = 20, kIQ4_XS = 23, kBF16 = 30;
+inline constexpr uint32_t kF32 = 0, kF16 = 1, kQ8_0 = 8, kQ3_K = 11, kQ4_K = 12, kQ5_K = 13, kQ6_K = 14, kIQ4_NL = 20, kIQ4_XS = 23, kBF16 = 30;
 }
 struct GgmlTypeTraits {
   const char *name;
@@ -32,7 +32,8 @@ struct GgmlTypeTraits {
 };
 // nullptr for a type this parser cannot size.
 [[nodiscard]] const GgmlTypeTraits *ggmlTypeTraits(uint32_t type) noexcept;
-// The weight-image format (abi/Gguf.h) of a ggml type, if the projections read it.
+// The weight-image format (abi/Gguf.h) of a ggml type, if the projections read it. Q3_K is read as Q6_K: the loader
+// rewrites its blocks as Q6_K blocks of the same values (ops::transcodeQ3KToQ6K).
 [[nodiscard]] std::optional<uint32_t> imageFormat(uint32_t ggmlType) noexcept;
 
 struct GgufTensor {
@@ -104,6 +105,8 @@ struct LoadedImage {
 // whole 256-input super-blocks) and uploads them; rows = 0 takes all.
 [[nodiscard]] LoadedImage loadImage(hip::Backend &backend, const GgufFile &file, const GgufTensor &tensor, uint32_t firstRow = 0,
                                     uint32_t rows = 0);
+// A projection tensor's native rows in device memory, in the format imageFormat names (what the token gather decodes).
+[[nodiscard]] hip::Buffer loadNativeRows(hip::Backend &backend, const GgufFile &file, const GgufTensor &tensor, const char *label);
 // The rows of a tensor an image, a table of float rows or a vector takes, in the order it takes them: runs of source
 // rows one after the other (the reference's TensorRows with its RowOrder, GgufImage.hpp:29-38). All rows when empty.
 struct RowRun final {

@@ -153,8 +153,7 @@ void loadGgufDenseWeights(hip::Backend &backend, const GgufFile &file, DenseVeri
     const std::optional<uint32_t> format = imageFormat(table->type);
     if (!format) problems.add("token_embd.weight is of a type the token gather does not read");
     else {
-      hip::Buffer rows = backend.allocateBuffer(table->bytes, hip::BufferStorage::Private, "token table");
-      rows.upload(file.data(*table), table->bytes);
+      hip::Buffer rows = loadNativeRows(backend, file, *table, "token table");
       w.embedding = {std::move(rows), *format, d.vocabulary, d.hidden};
     }
   }
@@ -428,8 +427,7 @@ void loadGgufHybridWeights(hip::Backend &backend, const GgufFile &file, HybridVe
     const std::optional<uint32_t> format = imageFormat(table->type);
     if (!format) problems.add("token_embd.weight is of a type the token gather does not read");
     else {
-      hip::Buffer rows = backend.allocateBuffer(table->bytes, hip::BufferStorage::Private, "token table");
-      rows.upload(file.data(*table), table->bytes);
+      hip::Buffer rows = loadNativeRows(backend, file, *table, "token table");
       w.embedding = {std::move(rows), *format, d.vocabulary, H};
     }
   }

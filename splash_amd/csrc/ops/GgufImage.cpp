@@ -217,4 +217,27 @@ void unpackGgufImage(uint32_t formatId, const uint8_t *image, uint32_t rows, uin
   });
 }
 
+void transcodeQ3KToQ6K(const uint8_t *q3k, uint64_t blocks, uint8_t *q6k) {
+  constexpr uint32_t kScales3 = 96, kD3 = 108, kHigh6 = 128, kScales6 = 192, kD6 = 208;
+  for (uint64_t b = 0; b < blocks; ++b, q3k += kQ3KNativeBytes, q6k += GGUF_Q6K_NATIVE) {
+    std::memset(q6k, 0, GGUF_Q6K_NATIVE);
+    const uint8_t *mask = q3k, *codes = q3k + 32, *packed = q3k + kScales3;
+    for (uint32_t i = 0; i < 16; ++i) {
+      const int low = i < 8 ? packed[i] & 15 : packed[i - 8] >> 4, high = (packed[8 + i % 4] >> (2 * (i / 4))) & 3;
+      q6k[kScales6 + i] = uint8_t(int8_t((low | (high << 4)) - 32));
+    }
+    // Value 32 j + k: Q3_K keeps its two bits at bit 2 (j % 4) of codes[32 (j / 4) + k] and its mask bit at bit j of
+    // mask[k]; Q6_K keeps the low nibble at nibble j % 4 / 2 of ql[64 (j / 4) + 32 (j % 2) + k] and the high two bits at
+    // bit 2 (j % 4) of qh[32 (j / 4) + k].
+    for (uint32_t j = 0; j < 8; ++j)
+      for (uint32_t k = 0; k < 32; ++k) {
+        const int two = (codes[32 * (j / 4) + k] >> (2 * (j % 4))) & 3, set = (mask[k] >> j) & 1;
+        const uint32_t q = uint32_t(two - (set ? 0 : 4) + 32), r = j % 4;
+        q6k[64 * (j / 4) + 32 * (r & 1) + k] |= uint8_t((q & 15) << (4 * (r >> 1)));
+        q6k[kHigh6 + 32 * (j / 4) + k] |= uint8_t((q >> 4) << (2 * r));
+      }
+    std::memcpy(q6k + kD6, q3k + kD3, 2);
+  }
+}
+
 } // namespace splash::ops

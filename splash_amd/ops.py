@@ -32,6 +32,17 @@ def pack_gguf_image(fmt, native, rows, input_size):
     return image
 
 
+def transcode_q3k(native):
+    """Q3_K super-blocks (110 bytes each) -> Q6_K blocks (210 bytes each) of the same values, which the images and the
+    token gather then read as Q6_K."""
+    native = np.ascontiguousarray(native, dtype=np.uint8)
+    if native.size % 110:
+        raise nat.InvalidArgument(1, "Q3_K rows are whole 110-byte blocks")
+    out = np.empty(native.size // 110 * 210, dtype=np.uint8)
+    check(lib.spo_gguf_transcode_q3k(native.ctypes.data, native.size // 110, out.ctypes.data))
+    return out
+
+
 def unpack_gguf_image(fmt, image, rows, input_size):
     image = np.ascontiguousarray(image, dtype=np.uint8)
     native = np.empty(image.size, dtype=np.uint8)

@@ -78,6 +78,76 @@ def test_malformed_files_are_refused(tmp_path):
         gguf.GgufFile(twice)
 
 
+def test_q3k_blocks_rewritten_as_q6k_keep_every_value():
+    """The loader's rewrite of Q3_K super-blocks as Q6_K blocks (spo_gguf_transcode_q3k): the Q6_K blocks' values are
+    GGML's dequantize_row_q3_K of the source bit for bit (the reference's golden hash, goldens.json:8), over every
+    6-bit scale and code the random fixture holds, and so are the oracle's projections of them."""
+    import hashlib
+    import json
+    import os
+    goldens = json.load(open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "gguf_dequantization.json")))
+    native = orc.fixture(orc.FMT_Q3K, 256, 1024, 7 + orc.FMT_Q3K)
+    rewritten = ops.transcode_q3k(native)
+    assert rewritten.size == native.size // 110 * 210
+    assert hashlib.sha256(orc.dequant_rows(orc.FMT_Q6K, rewritten, 256, 1024).tobytes()).hexdigest() == goldens["q3k"]
+    blocks = native.reshape(-1, 110)
+    scales = np.concatenate([blocks[:, 96:104] & 15, blocks[:, 96:104] >> 4], axis=1) | \
+        (((blocks[:, 104:108][:, np.arange(16) % 4] >> (2 * (np.arange(16) // 4))) & 3) << 4)
+    assert set(np.unique(scales)) == set(range(64))   # every scale value occurs
+    assert np.array_equal(rewritten.reshape(-1, 210)[:, 192:208].view(np.int8), scales.astype(np.int16) - 32)
+    realistic = orc.make_native(orc.FMT_Q3K, 64, 512, 3)
+    x_bits = orc.f32_to_bf16(np.random.default_rng(1).standard_normal((5, 512)).astype(np.float32))
+    a = orc.gemm(orc.FMT_Q3K, realistic, x_bits, 64, want=("exact", "bound"))
+    b = orc.gemm(orc.FMT_Q6K, ops.transcode_q3k(realistic), x_bits, 64, want=("exact", "bound"))
+    assert np.array_equal(a["exact"], b["exact"]) and np.array_equal(a["bound"], b["bound"])
+    with pytest.raises(splash_amd.SplashError):
+        ops.transcode_q3k(native[:109])
+
+
+@pytest.mark.gpu
+def test_a_q3k_tensor_loads_as_the_q6k_image_of_its_values(backend, tmp_path):
+    """A Q3_K tensor of a file: its image is the Q6_K image of the rewritten blocks, whole or a slice of rows or of
+    columns; the kernels' unpacking of it gives GGML's dequantize_row_q3_K values (the golden hash); and its projection
+    is the oracle's of the Q3_K rows."""
+    import hashlib
+    import json
+    import os
+    goldens = json.load(open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "gguf_dequantization.json")))
+    fixture = orc.fixture(orc.FMT_Q3K, 256, 1024, 7 + orc.FMT_Q3K)
+    realistic = orc.make_native(orc.FMT_Q3K, 64, 512, 3)
+    path = tmp_path / "q3k.gguf"
+    gw.write_gguf(path, [("general.architecture", gw.STRING, "qwen3")],
+                  [("fixture.weight", gw.GGML_Q3_K, [1024, 256], fixture), ("blk.0.attn_v.weight", gw.GGML_Q3_K, [512, 64], realistic)])
+    f = gguf.GgufFile(path)
+    print("case q3k golden through the file", flush=True)
+    fmt, rows, input_size, image = f.load_image(backend, f.find("fixture.weight"))
+    assert (fmt, rows, input_size) == (ops.FMT_Q6K, 256, 1024)
+    assert np.array_equal(image.download(np.uint8)[:ops.gguf_image_bytes(fmt, 256, 1024)],
+                          ops.pack_gguf_image(fmt, ops.transcode_q3k(fixture), 256, 1024))
+    out = backend.allocate_buffer(256 * 1024 * 4)
+    graph = splash_amd.CommandGraph()
+    ops.add_dequant(graph, fmt, image, out, 256, 1024)
+    backend.run(graph)
+    assert hashlib.sha256(out.download(np.float32, 256 * 1024).tobytes()).hexdigest() == goldens["q3k"]
+    print("case q3k rows 32..63", flush=True)
+    fmt, rows, _, image = f.load_image(backend, f.find("fixture.weight"), first_row=32, rows=32)
+    row_bytes = 1024 // 256 * 110
+    assert rows == 32 and np.array_equal(image.download(np.uint8)[:ops.gguf_image_bytes(fmt, 32, 1024)],
+                                         ops.pack_gguf_image(fmt, ops.transcode_q3k(fixture[32 * row_bytes:64 * row_bytes]), 32, 1024))
+    print("case q3k projection", flush=True)
+    fmt, rows, input_size, image = f.load_image(backend, f.find("blk.0.attn_v.weight"))
+    linear = ops.Linear(backend)
+    x_bits = orc.f32_to_bf16(np.random.default_rng(8).standard_normal((5, 512)).astype(np.float32))
+    projection = ops.Projection([(fmt, 64, image)], 512, float32=True)
+    plan = linear.plan(projection, 5)
+    out = backend.allocate_buffer(5 * 64 * 4)
+    graph = splash_amd.CommandGraph()
+    linear.add(graph, projection, plan, backend.from_array(x_bits), out, linear.scratch_for(backend, [plan]))
+    backend.run(graph)
+    want = orc.gemm(orc.FMT_Q3K, realistic, x_bits, 64, want=("exact", "bound"))
+    assert np.all(np.abs(out.download(np.float32).reshape(5, 64) - want["exact"]) <= want["bound"])
+
+
 @pytest.mark.gpu
 def test_projections_and_norms_load_from_a_file(backend, tmp_path):
     """A file's tensors become the operators' inputs: each projection format's rows give the result of the same
@@ -129,9 +199,10 @@ def dense_model_file(path, model, value_format, tied, extra=(), skip=(), more_me
     `value_format`, as a Q4_K_M file keeps them) ..., norms as F32, the token table, and the head unless tied."""
     d = model.dims
     H, D, F, V = d["hidden"], d["head_dim"], d["ffn"], d["vocabulary"]
-    kinds = {orc.FMT_Q4K: gw.GGML_Q4_K, orc.FMT_Q6K: gw.GGML_Q6_K, orc.FMT_Q5K: gw.GGML_Q5_K, orc.FMT_Q80: gw.GGML_Q8_0}
+    kinds = {orc.FMT_Q4K: gw.GGML_Q4_K, orc.FMT_Q6K: gw.GGML_Q6_K, orc.FMT_Q5K: gw.GGML_Q5_K, orc.FMT_Q80: gw.GGML_Q8_0,
+             orc.FMT_Q3K: gw.GGML_Q3_K}
     f32 = lambda bits: orc.bf16_to_f32(bits).astype(np.float32)
-    tensors = [("token_embd.weight", gw.GGML_Q4_K, [H, V], model.embedding)]
+    tensors = [("token_embd.weight", kinds[getattr(model, "table_format", orc.FMT_Q4K)], [H, V], model.embedding)]
     for i, w in enumerate(model.layers):
         p = f"blk.{i}."
         tensors += [(p + "attn_norm.weight", gw.GGML_F32, [H], f32(w["input_norm"])),
@@ -214,20 +285,31 @@ def test_a_split_file_reads_as_one(tmp_path):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("value_format,tied,parts", [(orc.FMT_Q6K, False, 1), (orc.FMT_Q4K, True, 1), (orc.FMT_Q6K, False, 3)])
+@pytest.mark.parametrize("value_format,tied,parts", [(orc.FMT_Q6K, False, 1), (orc.FMT_Q4K, True, 1), (orc.FMT_Q6K, False, 3),
+                                                     (orc.FMT_Q3K, True, 1)])
 def test_a_dense_decoder_loads_from_a_file(tmp_path, value_format, tied, parts):
     """spg_dense_dimensions and spo_dense_verify_load_gguf: the driver built from a file gives, bit for bit, the logits
     and the acceptance of the driver built by hand from the same tensors: q | k | v fused with the values in another
-    format than the queries and keys, a tied head, and the refusal of tensors the loader would ignore."""
+    format than the queries and keys, a tied head, and the refusal of tensors the loader would ignore. The Q3_K case
+    keeps the values and the tied token table as Q3_K, which the hand-built driver takes as the rewritten Q6_K blocks."""
     from splash_amd import verify
     from tests.dense_reference import DenseModel
     backend = splash_amd.Backend(0)
     model = DenseModel(seed=5, hidden=512, q_heads=16, kv_heads=8, head_dim=64, ffn=768, vocabulary=2048, layers=2, down_format=orc.FMT_Q6K)
-    if value_format != orc.FMT_Q4K:   # the values in the format a Q4_K_M file keeps them in
+    q3k = value_format == orc.FMT_Q3K
+    if q3k:
+        for i, w in enumerate(model.layers):
+            w["v"] = orc.make_native(orc.FMT_Q3K, 512, 512, 40 + i)
+        model.embedding = orc.make_native(orc.FMT_Q3K, 2048, 512, 50)
+        model.table_format = orc.FMT_Q3K
+    elif value_format != orc.FMT_Q4K:   # the values in the format a Q4_K_M file keeps them in
         for w in model.layers:
             w["v"] = orc.quantize_rows(value_format, orc.dequant_rows(orc.FMT_Q4K, w["v"], 512, 512))
     if tied:
         model.head = model.embedding
+    # what the kernels read: a Q3_K tensor as the Q6_K blocks of its values
+    seen = lambda fmt, native: (orc.FMT_Q6K, ops.transcode_q3k(native)) if fmt == orc.FMT_Q3K else (fmt, native)
+    table_format = orc.FMT_Q3K if q3k else orc.FMT_Q4K
     path = dense_model_file(tmp_path / "dense.gguf", model, value_format, tied, parts=parts)   # a path, or a split file's parts
     rows, context = 16, 200
     rng = np.random.default_rng(1)
@@ -244,12 +326,14 @@ def test_a_dense_decoder_loads_from_a_file(tmp_path, value_format, tied, parts):
         gpu = verify.DenseVerify(backend, 512, 16, 8, 64, 768, 2048, 2, rope_theta=model.rope_theta, max_lanes=1, physical_pages=pages + 1,
                                  page_table_entries=pages)
         for i, w in enumerate(model.layers):
-            gpu.set_layer(i, P([(orc.FMT_Q4K, 1024, w["q"]), (orc.FMT_Q4K, 512, w["k"]), (value_format, 512, w["v"])], 512),
+            value_seen, values = seen(value_format, w["v"])
+            gpu.set_layer(i, P([(orc.FMT_Q4K, 1024, w["q"]), (orc.FMT_Q4K, 512, w["k"]), (value_seen, 512, values)], 512),
                           P([(orc.FMT_Q4K, 512, w["o"])], 1024), P([(orc.FMT_Q4K, 768, w["gate"])], 512), P([(orc.FMT_Q4K, 768, w["up"])], 512),
                           P([(orc.FMT_Q6K, 512, w["down"])], 768), backend.from_array(w["input_norm"]), backend.from_array(w["post_norm"]),
                           backend.from_array(w["q_norm"]), backend.from_array(w["k_norm"]))
-        gpu.set_head(orc.FMT_Q4K, backend.from_array(model.embedding), backend.from_array(model.final_norm),
-                     P([(orc.FMT_Q4K if tied else orc.FMT_Q6K, 2048, model.head)], 512, True))
+        table_seen, table = seen(table_format, model.embedding)
+        head_seen, head = seen(table_format if tied else orc.FMT_Q6K, model.head)
+        gpu.set_head(table_seen, backend.from_array(table), backend.from_array(model.final_norm), P([(head_seen, 2048, head)], 512, True))
         return gpu
     outputs = []
     for gpu in (loaded, hand_built()):
