@@ -37,10 +37,13 @@ uint64_t spo_gguf_image_bytes(uint32_t format, uint32_t rows, uint32_t input_siz
 uint64_t spo_gguf_table_bytes(uint32_t input_size, uint32_t rows);
 sp_status spo_gguf_pack_image(uint32_t format, const uint8_t *native, uint32_t rows, uint32_t input_size, uint8_t *image);
 sp_status spo_gguf_unpack_image(uint32_t format, const uint8_t *image, uint32_t rows, uint32_t input_size, uint8_t *native);
-/* `blocks` Q3_K super-blocks (110 bytes each) as Q6_K blocks (210 bytes each) of the same values, which
- * spo_gguf_pack_image then takes as format Q6_K: how a Q3_K tensor is read (the reference runs it through kernels of its
- * own format: runtime/metal/abi/QuantFormat.h GGUF_FMT_Q3K; its values are GGML's dequantize_row_q3_K either way). */
-sp_status spo_gguf_transcode_q3k(const uint8_t *q3k, uint64_t blocks, uint8_t *q6k);
+/* ggml types read through another format's blocks of the same values, bit for bit: Q3_K (ggml type 11) as Q6_K, Q4_0
+ * (2) and Q5_0 (6) as Q8_0. spo_gguf_rewrite_format gives that format (0xFFFFFFFF for a type with no rewrite) and
+ * spo_gguf_rewrite writes `super_blocks` times 256 values of `source` as that format's native blocks, which
+ * spo_gguf_pack_image then takes; the GGUF loader does both by itself. (The reference runs these through kernels of their
+ * own formats: runtime/metal/abi/QuantFormat.h GGUF_FMT_Q3K, _Q40, _Q50; the values are GGML's dequantize_row_* either way.) */
+uint32_t spo_gguf_rewrite_format(uint32_t ggml_type);
+sp_status spo_gguf_rewrite(uint32_t ggml_type, const uint8_t *source, uint64_t super_blocks, uint8_t *out);
 /* The image's fp32 values [rows][input_size] (the reference's gguf_dequant_test.metal kernel). */
 sp_status spo_gguf_add_dequant(spo_graph *graph, uint32_t format, sp_buffer *image, sp_buffer *out, uint32_t rows,
                                uint32_t input_size);

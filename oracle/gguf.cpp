@@ -8,7 +8,7 @@ using namespace orc;
 
 namespace {
 
-constexpr uint32_t kQ4KBytes = 144, kQ5KBytes = 176, kQ6KBytes = 210, kQ3KBytes = 110, kQ80Bytes = 34, kIQ4XSBytes = 136, kIQ4NLBytes = 18, kBlock = 256;
+constexpr uint32_t kQ4KBytes = 144, kQ5KBytes = 176, kQ6KBytes = 210, kQ3KBytes = 110, kQ80Bytes = 34, kQ40Bytes = 18, kQ50Bytes = 22, kIQ4XSBytes = 136, kIQ4NLBytes = 18, kBlock = 256;
 // The 4-bit non-linear codebook of IQ4_NL and IQ4_XS (ggml's kvalues_iq4nl; GgufFormatReference.hpp:382-403 reads it).
 constexpr int8_t kIQ4Values[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
 constexpr uint32_t kQ6KScales = 128 + 64, kQ6KD = kQ6KScales + 16;  // GgufFormatReference.hpp:61
@@ -17,9 +17,9 @@ constexpr uint32_t kQ3KScales = 32 + 64, kQ3KD = kQ3KScales + 12;    // GgufForm
 // Bytes and elements of a native block: the K-quants' super-block of 256, Q8_0's group of 32.
 uint32_t blockBytes(uint32_t fmt) {
   return fmt == ORC_FMT_Q4K ? kQ4KBytes : fmt == ORC_FMT_Q5K ? kQ5KBytes : fmt == ORC_FMT_Q6K ? kQ6KBytes : fmt == ORC_FMT_Q80 ? kQ80Bytes
-         : fmt == ORC_FMT_Q3K ? kQ3KBytes : fmt == ORC_FMT_IQ4XS ? kIQ4XSBytes : fmt == ORC_FMT_IQ4NL ? kIQ4NLBytes : 0;
+         : fmt == ORC_FMT_Q3K ? kQ3KBytes : fmt == ORC_FMT_Q40 ? kQ40Bytes : fmt == ORC_FMT_Q50 ? kQ50Bytes : fmt == ORC_FMT_IQ4XS ? kIQ4XSBytes : fmt == ORC_FMT_IQ4NL ? kIQ4NLBytes : 0;
 }
-uint32_t blockElements(uint32_t fmt) { return fmt == ORC_FMT_Q80 || fmt == ORC_FMT_IQ4NL ? 32 : kBlock; }
+uint32_t blockElements(uint32_t fmt) { return fmt == ORC_FMT_Q80 || fmt == ORC_FMT_IQ4NL || fmt == ORC_FMT_Q40 || fmt == ORC_FMT_Q50 ? 32 : kBlock; }
 
 // GgufFormatReference.hpp:326-329
 void scaleMinK4(const uint8_t *sc, int j, uint8_t &s, uint8_t &m) {
@@ -33,7 +33,7 @@ struct Group {
   uint8_t code[32];
   float s[2];  // Q4_K, Q5_K: s[0] = s[1] = d * sc; Q6_K, Q3_K: one per 16 elements; Q8_0, IQ4_NL: d; IQ4_XS: d * (ls - 32)
   float m;     // Q4_K, Q5_K: -dmin * mn; the others: 0
-  int bias;    // Q4_K, Q5_K: 0; Q6_K: 32; Q3_K: 4; Q8_0, IQ4_NL, IQ4_XS: 128 (code = value or codebook value + 128)
+  int bias;    // Q4_K, Q5_K: 0; Q6_K: 32; Q3_K: 4; Q4_0: 8; Q5_0: 16; Q8_0, IQ4_NL, IQ4_XS: 128 (code = value or codebook value + 128)
 };
 void readGroup(uint32_t fmt, const uint8_t *row, uint32_t g, Group &out) {
   if (fmt == ORC_FMT_Q80) {   // GgufFormatReference.hpp:453-458: value = d * int8
@@ -43,6 +43,19 @@ void readGroup(uint32_t fmt, const uint8_t *row, uint32_t g, Group &out) {
     out.s[0] = out.s[1] = h2f(d16);
     out.m = 0.f;
     out.bias = 128;
+    return;
+  }
+  if (fmt == ORC_FMT_Q40 || fmt == ORC_FMT_Q50) {   // GgufFormatReference.hpp:529-551: value = d * (code - 8), d * (code - 16);
+    const bool five = fmt == ORC_FMT_Q50;           // byte k's low nibble is input k, its high nibble input 16 + k; Q5_0's fifth
+    const uint8_t *blk = row + size_t(g) * (five ? kQ50Bytes : kQ40Bytes), *qh = blk + 2, *qs = blk + (five ? 6 : 2);   // bits: bit k of qh
+    uint16_t d16; std::memcpy(&d16, blk, 2);
+    for (int k = 0; k < 32; ++k) {
+      const int low = k < 16 ? qs[k] & 15 : qs[k - 16] >> 4;
+      out.code[k] = uint8_t(five ? low | (((qh[k / 8] >> (k % 8)) & 1) << 4) : low);
+    }
+    out.s[0] = out.s[1] = h2f(d16);
+    out.m = 0.f;
+    out.bias = five ? 16 : 8;
     return;
   }
   if (fmt == ORC_FMT_IQ4NL) {   // GgufFormatReference.hpp:394-403: value = d * codebook[nibble]; byte k's low nibble is

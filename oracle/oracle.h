@@ -53,7 +53,8 @@ extern "C" {
 #endif
 
 // Format ids follow the reference's GGUF_FMT_* numbering (runtime/metal/abi/QuantFormat.h:138-154).
-enum { ORC_FMT_Q4K = 0, ORC_FMT_IQ4XS = 1, ORC_FMT_IQ4NL = 2, ORC_FMT_Q5K = 3, ORC_FMT_Q6K = 4, ORC_FMT_Q3K = 5, ORC_FMT_Q80 = 6 };
+enum { ORC_FMT_Q4K = 0, ORC_FMT_IQ4XS = 1, ORC_FMT_IQ4NL = 2, ORC_FMT_Q5K = 3, ORC_FMT_Q6K = 4, ORC_FMT_Q3K = 5, ORC_FMT_Q80 = 6, ORC_FMT_Q40 = 15,
+       ORC_FMT_Q50 = 39 };
 
 // ---- half / bfloat16 scalar conversions (round to nearest even) ----
 uint16_t orc_f2h(float f);

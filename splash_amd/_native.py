@@ -250,7 +250,8 @@ _sig("spo_graph_record", c_int, c_p, c_p, P(c_p))
 _sig("spo_gguf_image_bytes", c_u64, c_u32, c_u32, c_u32)
 _sig("spo_gguf_table_bytes", c_u64, c_u32, c_u32)
 _sig("spo_gguf_pack_image", c_int, c_u32, c_p, c_u32, c_u32, c_p)
-_sig("spo_gguf_transcode_q3k", c_int, c_p, ctypes.c_uint64, c_p)
+_sig("spo_gguf_rewrite_format", c_u32, c_u32)
+_sig("spo_gguf_rewrite", c_int, c_u32, c_p, ctypes.c_uint64, c_p)
 _sig("spo_gguf_unpack_image", c_int, c_u32, c_p, c_u32, c_u32, c_p)
 _sig("spo_gguf_add_dequant", c_int, c_p, c_u32, c_p, c_p, c_u32, c_u32)
 _sig("spo_projection_create", c_int, c_u32, P(c_u32), P(c_u32), c_u32, P(c_p), c_int, P(c_p))

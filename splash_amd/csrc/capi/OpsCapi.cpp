@@ -95,8 +95,12 @@ sp_status spo_gguf_pack_image(uint32_t format, const uint8_t *native, uint32_t r
 sp_status spo_gguf_unpack_image(uint32_t format, const uint8_t *image, uint32_t rows, uint32_t input_size, uint8_t *native) {
   return capi::guard([&] { capi::require(native && image, "rows or image"); ops::unpackGgufImage(format, image, rows, input_size, native); });
 }
-sp_status spo_gguf_transcode_q3k(const uint8_t *q3k, uint64_t blocks, uint8_t *q6k) {
-  return capi::guard([&] { capi::require(q3k && q6k, "blocks"); ops::transcodeQ3KToQ6K(q3k, blocks, q6k); });
+uint32_t spo_gguf_rewrite_format(uint32_t ggml_type) {
+  const ops::NativeRewrite *rewrite = ops::nativeRewriteOf(ggml_type);
+  return rewrite ? rewrite->imageFormat : 0xFFFFFFFFu;
+}
+sp_status spo_gguf_rewrite(uint32_t ggml_type, const uint8_t *source, uint64_t super_blocks, uint8_t *out) {
+  return capi::guard([&] { capi::require(source && out, "blocks"); ops::rewriteNative(ggml_type, source, super_blocks, out); });
 }
 sp_status spo_gguf_add_dequant(spo_graph *graph, uint32_t format, sp_buffer *image, sp_buffer *out, uint32_t rows,
                                uint32_t input_size) {

@@ -16,9 +16,9 @@ namespace splash::model {
 
 namespace {
 
-constexpr std::array<std::pair<uint32_t, GgmlTypeTraits>, 13> kTypes{{
+constexpr std::array<std::pair<uint32_t, GgmlTypeTraits>, 14> kTypes{{
     {0, {"F32", 1, 4}},        {1, {"F16", 1, 2}},        {2, {"Q4_0", 32, 18}},    {3, {"Q4_1", 32, 20}},
-    {8, {"Q8_0", 32, 34}},     {10, {"Q2_K", 256, 84}},   {11, {"Q3_K", 256, 110}}, {12, {"Q4_K", 256, 144}},
+    {6, {"Q5_0", 32, 22}},     {8, {"Q8_0", 32, 34}},     {10, {"Q2_K", 256, 84}},   {11, {"Q3_K", 256, 110}}, {12, {"Q4_K", 256, 144}},
     {13, {"Q5_K", 256, 176}},  {14, {"Q6_K", 256, 210}},  {20, {"IQ4_NL", 32, 18}},   {23, {"IQ4_XS", 256, 136}},
     {30, {"BF16", 1, 2}},
 }};
@@ -101,7 +101,7 @@ std::optional<uint32_t> imageFormat(uint32_t ggmlType) noexcept {
     case ggml::kQ4_K: return GGUF_FMT_Q4K;
     case ggml::kQ5_K: return GGUF_FMT_Q5K;
     case ggml::kQ6_K: return GGUF_FMT_Q6K;
-    case ggml::kQ3_K: return GGUF_FMT_Q6K;
+    case ggml::kQ3_K: case ggml::kQ4_0: case ggml::kQ5_0: return ops::nativeRewriteOf(ggmlType)->imageFormat;
     case ggml::kQ8_0: return GGUF_FMT_Q80;
     case ggml::kIQ4_XS: return GGUF_FMT_IQ4XS;
     case ggml::kIQ4_NL: return GGUF_FMT_IQ4NL;
@@ -256,10 +256,10 @@ LoadedImage loadImage(hip::Backend &backend, const GgufFile &file, const GgufTen
     throw std::invalid_argument("a weight image holds whole 16-row tiles of whole 256-input super-blocks: " + tensor.name);
   std::vector<uint8_t> rewritten;
   const uint8_t *native;
-  if (tensor.type == ggml::kQ3_K) {
+  if (const ops::NativeRewrite *rewrite = ops::nativeRewriteOf(tensor.type)) {
     const uint64_t blocks = columns / GGUF_BLOCK * rows;
-    rewritten.resize(blocks * GGUF_Q6K_NATIVE);
-    ops::transcodeQ3KToQ6K(file.data(tensor) + uint64_t{firstRow} * (columns / GGUF_BLOCK * ops::kQ3KNativeBytes), blocks, rewritten.data());
+    rewritten.resize(blocks * gguf_native_bytes(*format));
+    ops::rewriteNative(tensor.type, file.data(tensor) + uint64_t{firstRow} * (columns / GGUF_BLOCK * rewrite->sourceBytes), blocks, rewritten.data());
     native = rewritten.data();
   } else {
     native = file.data(tensor) + uint64_t{firstRow} * (columns / GGUF_BLOCK * gguf_native_bytes(*format));
@@ -276,14 +276,15 @@ LoadedImage loadImage(hip::Backend &backend, const GgufFile &file, const GgufTen
 }
 
 hip::Buffer loadNativeRows(hip::Backend &backend, const GgufFile &file, const GgufTensor &tensor, const char *label) {
-  if (tensor.type != ggml::kQ3_K) {
+  const ops::NativeRewrite *rewrite = ops::nativeRewriteOf(tensor.type);
+  if (!rewrite) {
     hip::Buffer rows = backend.allocateBuffer(tensor.bytes, hip::BufferStorage::Private, label);
     rows.upload(file.data(tensor), tensor.bytes);
     return rows;
   }
-  const uint64_t blocks = tensor.bytes / ops::kQ3KNativeBytes;
-  std::vector<uint8_t> rewritten(blocks * GGUF_Q6K_NATIVE);
-  ops::transcodeQ3KToQ6K(file.data(tensor), blocks, rewritten.data());
+  const uint64_t blocks = tensor.bytes / rewrite->sourceBytes;
+  std::vector<uint8_t> rewritten(blocks * gguf_native_bytes(rewrite->imageFormat));
+  ops::rewriteNative(tensor.type, file.data(tensor), blocks, rewritten.data());
   hip::Buffer rows = backend.allocateBuffer(rewritten.size(), hip::BufferStorage::Private, label);
   rows.upload(rewritten.data(), rewritten.size());
   return rows;
@@ -313,8 +314,8 @@ uint64_t runRows(const RowRuns &runs, uint64_t all) {
 std::vector<uint8_t> gatherNative(const GgufFile &file, const GgufTensor &tensor, uint32_t format, const RowRuns &runs, uint64_t firstColumn,
                                   uint64_t columns) {
   const uint64_t all = tensor.rows(), width = tensor.columns();
-  const bool q3k = tensor.type == ggml::kQ3_K;
-  const uint64_t blockBytes = q3k ? ops::kQ3KNativeBytes : gguf_native_bytes(format), rowBytes = width / GGUF_BLOCK * blockBytes;
+  const ops::NativeRewrite *rewrite = ops::nativeRewriteOf(tensor.type);
+  const uint64_t blockBytes = rewrite ? rewrite->sourceBytes : gguf_native_bytes(format), rowBytes = width / GGUF_BLOCK * blockBytes;
   const uint64_t piece = columns / GGUF_BLOCK * blockBytes, skip = firstColumn / GGUF_BLOCK * blockBytes;
   std::vector<uint8_t> native(runRows(runs, all) * piece);
   const uint8_t *data = file.data(tensor);
@@ -324,9 +325,9 @@ std::vector<uint8_t> gatherNative(const GgufFile &file, const GgufTensor &tensor
   };
   if (runs.empty()) take(0, all);
   for (const RowRun &run : runs) take(run.first, run.rows);
-  if (q3k) {
-    std::vector<uint8_t> rewritten(native.size() / ops::kQ3KNativeBytes * GGUF_Q6K_NATIVE);
-    ops::transcodeQ3KToQ6K(native.data(), native.size() / ops::kQ3KNativeBytes, rewritten.data());
+  if (rewrite) {
+    std::vector<uint8_t> rewritten(native.size() / rewrite->sourceBytes * gguf_native_bytes(format));
+    ops::rewriteNative(tensor.type, native.data(), native.size() / rewrite->sourceBytes, rewritten.data());
     return rewritten;
   }
   return native;

@@ -23,7 +23,7 @@ public:
 
 // ggml type ids as GGUF tensor infos store them (ggml-common.h; GgufFile.hpp:35-66 in the reference).
 namespace ggml {
-inline constexpr uint32_t kF32 = 0, kF16 = 1, kQ8_0 = 8, kQ3_K = 11, kQ4_K = 12, kQ5_K = 13, kQ6_K = 14, kIQ4_NL = 20, kIQ4_XS = 23, kBF16 = 30;
+inline constexpr uint32_t kF32 = 0, kF16 = 1, kQ4_0 = 2, kQ5_0 = 6, kQ8_0 = 8, kQ3_K = 11, kQ4_K = 12, kQ5_K = 13, kQ6_K = 14, kIQ4_NL = 20, kIQ4_XS = 23, kBF16 = 30;
 }
 struct GgmlTypeTraits {
   const char *name;
@@ -32,8 +32,8 @@ struct GgmlTypeTraits {
 };
 // nullptr for a type this parser cannot size.
 [[nodiscard]] const GgmlTypeTraits *ggmlTypeTraits(uint32_t type) noexcept;
-// The weight-image format (abi/Gguf.h) of a ggml type, if the projections read it. Q3_K is read as Q6_K: the loader
-// rewrites its blocks as Q6_K blocks of the same values (ops::transcodeQ3KToQ6K).
+// The weight-image format (abi/Gguf.h) of a ggml type, if the projections read it. Q3_K is read as Q6_K and Q4_0 and
+// Q5_0 as Q8_0: the loader rewrites their blocks as blocks of the same values (ops::rewriteNative).
 [[nodiscard]] std::optional<uint32_t> imageFormat(uint32_t ggmlType) noexcept;
 
 struct GgufTensor {

@@ -217,9 +217,14 @@ void unpackGgufImage(uint32_t formatId, const uint8_t *image, uint32_t rows, uin
   });
 }
 
-void transcodeQ3KToQ6K(const uint8_t *q3k, uint64_t blocks, uint8_t *q6k) {
+namespace {
+constexpr uint32_t kGgmlQ4_0 = 2, kGgmlQ5_0 = 6, kGgmlQ3_K = 11;
+constexpr uint32_t kQ3KBytes = 110, kQ40Bytes = 18, kQ50Bytes = 22, kQ80Bytes = 34;
+constexpr NativeRewrite kQ3KRewrite{GGUF_FMT_Q6K, kQ3KBytes}, kQ40Rewrite{GGUF_FMT_Q80, 8 * kQ40Bytes}, kQ50Rewrite{GGUF_FMT_Q80, 8 * kQ50Bytes};
+
+void q3kAsQ6K(const uint8_t *q3k, uint64_t blocks, uint8_t *q6k) {
   constexpr uint32_t kScales3 = 96, kD3 = 108, kHigh6 = 128, kScales6 = 192, kD6 = 208;
-  for (uint64_t b = 0; b < blocks; ++b, q3k += kQ3KNativeBytes, q6k += GGUF_Q6K_NATIVE) {
+  for (uint64_t b = 0; b < blocks; ++b, q3k += kQ3KBytes, q6k += GGUF_Q6K_NATIVE) {
     std::memset(q6k, 0, GGUF_Q6K_NATIVE);
     const uint8_t *mask = q3k, *codes = q3k + 32, *packed = q3k + kScales3;
     for (uint32_t i = 0; i < 16; ++i) {
@@ -238,6 +243,32 @@ void transcodeQ3KToQ6K(const uint8_t *q3k, uint64_t blocks, uint8_t *q6k) {
       }
     std::memcpy(q6k + kD6, q3k + kD3, 2);
   }
+}
+
+// Groups of 32 values: byte k of the sixteen holds value k in its low nibble and value 16 + k in its high one; Q5_0's
+// fifth bit of value k is bit k of the four bytes after d.
+void legacyAsQ80(bool five, const uint8_t *source, uint64_t groups, uint8_t *q80) {
+  const uint32_t bytes = five ? kQ50Bytes : kQ40Bytes;
+  for (uint64_t g = 0; g < groups; ++g, source += bytes, q80 += kQ80Bytes) {
+    const uint8_t *high = source + 2, *nibbles = source + (five ? 6 : 2);
+    std::memcpy(q80, source, 2);
+    for (uint32_t k = 0; k < 32; ++k) {
+      const int low = k < 16 ? nibbles[k] & 15 : nibbles[k - 16] >> 4;
+      const int q = five ? (low | (((high[k / 8] >> (k % 8)) & 1) << 4)) - 16 : low - 8;
+      q80[2 + k] = uint8_t(int8_t(q));
+    }
+  }
+}
+} // namespace
+
+const NativeRewrite *nativeRewriteOf(uint32_t ggmlType) noexcept {
+  return ggmlType == kGgmlQ3_K ? &kQ3KRewrite : ggmlType == kGgmlQ4_0 ? &kQ40Rewrite : ggmlType == kGgmlQ5_0 ? &kQ50Rewrite : nullptr;
+}
+
+void rewriteNative(uint32_t ggmlType, const uint8_t *source, uint64_t superBlocks, uint8_t *out) {
+  if (ggmlType == kGgmlQ3_K) return q3kAsQ6K(source, superBlocks, out);
+  if (ggmlType == kGgmlQ4_0 || ggmlType == kGgmlQ5_0) return legacyAsQ80(ggmlType == kGgmlQ5_0, source, superBlocks * 8, out);
+  throw std::invalid_argument("ggml type " + std::to_string(ggmlType) + " is not read through another format's blocks");
 }
 
 } // namespace splash::ops

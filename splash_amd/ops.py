@@ -32,15 +32,20 @@ def pack_gguf_image(fmt, native, rows, input_size):
     return image
 
 
-def transcode_q3k(native):
-    """Q3_K super-blocks (110 bytes each) -> Q6_K blocks (210 bytes each) of the same values, which the images and the
-    token gather then read as Q6_K."""
+GGML_Q4_0, GGML_Q5_0, GGML_Q3_K = 2, 6, 11
+_REWRITE_BYTES = {GGML_Q3_K: (110, 210), GGML_Q4_0: (8 * 18, 8 * 34), GGML_Q5_0: (8 * 22, 8 * 34)}   # of 256 values: source, written
+
+
+def rewrite_native(ggml_type, native):
+    """Rows of a ggml type with no kernels of its own as the blocks of the format that reads them, with the same values:
+    Q3_K as Q6_K, Q4_0 and Q5_0 as Q8_0. Returns (format, native rows of that format)."""
     native = np.ascontiguousarray(native, dtype=np.uint8)
-    if native.size % 110:
-        raise nat.InvalidArgument(1, "Q3_K rows are whole 110-byte blocks")
-    out = np.empty(native.size // 110 * 210, dtype=np.uint8)
-    check(lib.spo_gguf_transcode_q3k(native.ctypes.data, native.size // 110, out.ctypes.data))
-    return out
+    if ggml_type not in _REWRITE_BYTES or native.size % _REWRITE_BYTES[ggml_type][0]:
+        raise nat.InvalidArgument(1, "rows of whole 256-value blocks of Q3_K, Q4_0 or Q5_0")
+    source, written = _REWRITE_BYTES[ggml_type]
+    out = np.empty(native.size // source * written, dtype=np.uint8)
+    check(lib.spo_gguf_rewrite(ggml_type, native.ctypes.data, native.size // source, out.ctypes.data))
+    return lib.spo_gguf_rewrite_format(ggml_type), out
 
 
 def unpack_gguf_image(fmt, image, rows, input_size):

@@ -6,7 +6,7 @@ import numpy as np
 
 U8, I8, U16, I16, U32, I32, F32, BOOL, STRING, ARRAY, U64, I64, F64 = range(13)
 GGML_F32, GGML_F16, GGML_Q8_0, GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_IQ4_NL, GGML_IQ4_XS, GGML_BF16 = 0, 1, 8, 12, 13, 14, 20, 23, 30
-GGML_Q3_K = 11
+GGML_Q4_0, GGML_Q5_0, GGML_Q3_K = 2, 6, 11
 
 
 def _string(text):

@@ -7,7 +7,7 @@ import numpy as np
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 FMT_Q4K, FMT_IQ4XS, FMT_IQ4NL, FMT_Q5K, FMT_Q6K, FMT_Q80 = 0, 1, 2, 3, 4, 6
-FMT_Q3K = 5   # the oracle dequantizes it; the kernels read it rewritten as Q6_K blocks
+FMT_Q3K, FMT_Q40, FMT_Q50 = 5, 15, 39   # the oracle dequantizes them; the kernels read them rewritten as Q6_K / Q8_0 blocks
 ALL_FORMATS = [("q4k", FMT_Q4K), ("q6k", FMT_Q6K), ("q5k", FMT_Q5K), ("q80", FMT_Q80), ("iq4xs", FMT_IQ4XS), ("iq4nl", FMT_IQ4NL)]
 NO_TOKEN = 0xFFFFFFFF
 

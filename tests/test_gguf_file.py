@@ -1,4 +1,8 @@
 """The GGUF header parser (CPU) and the loading of a file's tensors as the operators' inputs (GPU)."""
+import hashlib
+import json
+import os
+
 import numpy as np
 import pytest
 
@@ -78,63 +82,69 @@ def test_malformed_files_are_refused(tmp_path):
         gguf.GgufFile(twice)
 
 
-def test_q3k_blocks_rewritten_as_q6k_keep_every_value():
-    """The loader's rewrite of Q3_K super-blocks as Q6_K blocks (spo_gguf_transcode_q3k): the Q6_K blocks' values are
-    GGML's dequantize_row_q3_K of the source bit for bit (the reference's golden hash, goldens.json:8), over every
-    6-bit scale and code the random fixture holds, and so are the oracle's projections of them."""
-    import hashlib
-    import json
-    import os
-    goldens = json.load(open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "gguf_dequantization.json")))
-    native = orc.fixture(orc.FMT_Q3K, 256, 1024, 7 + orc.FMT_Q3K)
-    rewritten = ops.transcode_q3k(native)
-    assert rewritten.size == native.size // 110 * 210
-    assert hashlib.sha256(orc.dequant_rows(orc.FMT_Q6K, rewritten, 256, 1024).tobytes()).hexdigest() == goldens["q3k"]
-    blocks = native.reshape(-1, 110)
-    scales = np.concatenate([blocks[:, 96:104] & 15, blocks[:, 96:104] >> 4], axis=1) | \
-        (((blocks[:, 104:108][:, np.arange(16) % 4] >> (2 * (np.arange(16) // 4))) & 3) << 4)
-    assert set(np.unique(scales)) == set(range(64))   # every scale value occurs
-    assert np.array_equal(rewritten.reshape(-1, 210)[:, 192:208].view(np.int8), scales.astype(np.int16) - 32)
-    realistic = orc.make_native(orc.FMT_Q3K, 64, 512, 3)
+GOLDENS = json.load(open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "gguf_dequantization.json")))
+# ggml types with no kernels of their own: (golden's name, the oracle's format, ggml type, the format they are read as)
+REWRITTEN = [("q3k", orc.FMT_Q3K, gw.GGML_Q3_K, orc.FMT_Q6K), ("q40", orc.FMT_Q40, gw.GGML_Q4_0, orc.FMT_Q80),
+             ("q50", orc.FMT_Q50, gw.GGML_Q5_0, orc.FMT_Q80)]
+
+
+@pytest.mark.parametrize("name,source,kind,read_as", REWRITTEN)
+def test_rewritten_blocks_keep_every_value(name, source, kind, read_as):
+    """The loader's rewrite of Q3_K blocks as Q6_K and of Q4_0 and Q5_0 blocks as Q8_0 (spo_gguf_rewrite): the written
+    blocks' values are GGML's dequantize_row_* of the source bit for bit (the reference's golden hashes,
+    goldens.json:8,18,22), over every scale and code the random fixture holds, and so are the oracle's projections."""
+    native = orc.fixture(source, 256, 1024, 7 + source)
+    fmt, rewritten = ops.rewrite_native(kind, native)
+    assert fmt == read_as and rewritten.size == orc.row_bytes(read_as, 1024) * 256
+    assert hashlib.sha256(orc.dequant_rows(read_as, rewritten, 256, 1024).tobytes()).hexdigest() == GOLDENS[name]
+    if source == orc.FMT_Q3K:
+        blocks = native.reshape(-1, 110)
+        scales = np.concatenate([blocks[:, 96:104] & 15, blocks[:, 96:104] >> 4], axis=1) | \
+            (((blocks[:, 104:108][:, np.arange(16) % 4] >> (2 * (np.arange(16) // 4))) & 3) << 4)
+        assert set(np.unique(scales)) == set(range(64))   # every scale value occurs
+        assert np.array_equal(rewritten.reshape(-1, 210)[:, 192:208].view(np.int8), scales.astype(np.int16) - 32)
+    else:
+        codes = rewritten.reshape(-1, 34)[:, 2:].view(np.int8)
+        assert (codes.min(), codes.max()) == ((-8, 7) if source == orc.FMT_Q40 else (-16, 15))
+    realistic = orc.make_native(source, 64, 512, 3)
     x_bits = orc.f32_to_bf16(np.random.default_rng(1).standard_normal((5, 512)).astype(np.float32))
-    a = orc.gemm(orc.FMT_Q3K, realistic, x_bits, 64, want=("exact", "bound"))
-    b = orc.gemm(orc.FMT_Q6K, ops.transcode_q3k(realistic), x_bits, 64, want=("exact", "bound"))
+    a = orc.gemm(source, realistic, x_bits, 64, want=("exact", "bound"))
+    b = orc.gemm(read_as, ops.rewrite_native(kind, realistic)[1], x_bits, 64, want=("exact", "bound"))
     assert np.array_equal(a["exact"], b["exact"]) and np.array_equal(a["bound"], b["bound"])
     with pytest.raises(splash_amd.SplashError):
-        ops.transcode_q3k(native[:109])
+        ops.rewrite_native(kind, native[:109])
+    with pytest.raises(splash_amd.SplashError):
+        ops.rewrite_native(gw.GGML_Q4_K, native)
 
 
 @pytest.mark.gpu
-def test_a_q3k_tensor_loads_as_the_q6k_image_of_its_values(backend, tmp_path):
-    """A Q3_K tensor of a file: its image is the Q6_K image of the rewritten blocks, whole or a slice of rows or of
-    columns; the kernels' unpacking of it gives GGML's dequantize_row_q3_K values (the golden hash); and its projection
-    is the oracle's of the Q3_K rows."""
-    import hashlib
-    import json
-    import os
-    goldens = json.load(open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "gguf_dequantization.json")))
-    fixture = orc.fixture(orc.FMT_Q3K, 256, 1024, 7 + orc.FMT_Q3K)
-    realistic = orc.make_native(orc.FMT_Q3K, 64, 512, 3)
-    path = tmp_path / "q3k.gguf"
+@pytest.mark.parametrize("name,source,kind,read_as", REWRITTEN)
+def test_a_rewritten_tensor_loads_as_the_image_of_its_values(backend, tmp_path, name, source, kind, read_as):
+    """A Q3_K, Q4_0 or Q5_0 tensor of a file: its image is the Q6_K or Q8_0 image of the rewritten blocks, whole or a
+    slice of rows; the kernels' unpacking of it gives GGML's dequantize_row_* values (the golden hash); and its projection
+    is the oracle's of the source rows."""
+    fixture = orc.fixture(source, 256, 1024, 7 + source)
+    realistic = orc.make_native(source, 64, 512, 3)
+    path = tmp_path / "rewritten.gguf"
     gw.write_gguf(path, [("general.architecture", gw.STRING, "qwen3")],
-                  [("fixture.weight", gw.GGML_Q3_K, [1024, 256], fixture), ("blk.0.attn_v.weight", gw.GGML_Q3_K, [512, 64], realistic)])
+                  [("fixture.weight", kind, [1024, 256], fixture), ("blk.0.attn_v.weight", kind, [512, 64], realistic)])
     f = gguf.GgufFile(path)
-    print("case q3k golden through the file", flush=True)
+    print(f"case {name} golden through the file", flush=True)
     fmt, rows, input_size, image = f.load_image(backend, f.find("fixture.weight"))
-    assert (fmt, rows, input_size) == (ops.FMT_Q6K, 256, 1024)
+    assert (fmt, rows, input_size) == (read_as, 256, 1024)
     assert np.array_equal(image.download(np.uint8)[:ops.gguf_image_bytes(fmt, 256, 1024)],
-                          ops.pack_gguf_image(fmt, ops.transcode_q3k(fixture), 256, 1024))
+                          ops.pack_gguf_image(fmt, ops.rewrite_native(kind, fixture)[1], 256, 1024))
     out = backend.allocate_buffer(256 * 1024 * 4)
     graph = splash_amd.CommandGraph()
     ops.add_dequant(graph, fmt, image, out, 256, 1024)
     backend.run(graph)
-    assert hashlib.sha256(out.download(np.float32, 256 * 1024).tobytes()).hexdigest() == goldens["q3k"]
-    print("case q3k rows 32..63", flush=True)
+    assert hashlib.sha256(out.download(np.float32, 256 * 1024).tobytes()).hexdigest() == GOLDENS[name]
+    print(f"case {name} rows 32..63", flush=True)
     fmt, rows, _, image = f.load_image(backend, f.find("fixture.weight"), first_row=32, rows=32)
-    row_bytes = 1024 // 256 * 110
+    row_bytes = orc.row_bytes(source, 1024)
     assert rows == 32 and np.array_equal(image.download(np.uint8)[:ops.gguf_image_bytes(fmt, 32, 1024)],
-                                         ops.pack_gguf_image(fmt, ops.transcode_q3k(fixture[32 * row_bytes:64 * row_bytes]), 32, 1024))
-    print("case q3k projection", flush=True)
+                                         ops.pack_gguf_image(fmt, ops.rewrite_native(kind, fixture[32 * row_bytes:64 * row_bytes])[1], 32, 1024))
+    print(f"case {name} projection", flush=True)
     fmt, rows, input_size, image = f.load_image(backend, f.find("blk.0.attn_v.weight"))
     linear = ops.Linear(backend)
     x_bits = orc.f32_to_bf16(np.random.default_rng(8).standard_normal((5, 512)).astype(np.float32))
@@ -144,7 +154,7 @@ def test_a_q3k_tensor_loads_as_the_q6k_image_of_its_values(backend, tmp_path):
     graph = splash_amd.CommandGraph()
     linear.add(graph, projection, plan, backend.from_array(x_bits), out, linear.scratch_for(backend, [plan]))
     backend.run(graph)
-    want = orc.gemm(orc.FMT_Q3K, realistic, x_bits, 64, want=("exact", "bound"))
+    want = orc.gemm(source, realistic, x_bits, 64, want=("exact", "bound"))
     assert np.all(np.abs(out.download(np.float32).reshape(5, 64) - want["exact"]) <= want["bound"])
 
 
@@ -200,7 +210,7 @@ def dense_model_file(path, model, value_format, tied, extra=(), skip=(), more_me
     d = model.dims
     H, D, F, V = d["hidden"], d["head_dim"], d["ffn"], d["vocabulary"]
     kinds = {orc.FMT_Q4K: gw.GGML_Q4_K, orc.FMT_Q6K: gw.GGML_Q6_K, orc.FMT_Q5K: gw.GGML_Q5_K, orc.FMT_Q80: gw.GGML_Q8_0,
-             orc.FMT_Q3K: gw.GGML_Q3_K}
+             orc.FMT_Q3K: gw.GGML_Q3_K, orc.FMT_Q40: gw.GGML_Q4_0, orc.FMT_Q50: gw.GGML_Q5_0}
     f32 = lambda bits: orc.bf16_to_f32(bits).astype(np.float32)
     tensors = [("token_embd.weight", kinds[getattr(model, "table_format", orc.FMT_Q4K)], [H, V], model.embedding)]
     for i, w in enumerate(model.layers):
@@ -286,30 +296,31 @@ def test_a_split_file_reads_as_one(tmp_path):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("value_format,tied,parts", [(orc.FMT_Q6K, False, 1), (orc.FMT_Q4K, True, 1), (orc.FMT_Q6K, False, 3),
-                                                     (orc.FMT_Q3K, True, 1)])
+                                                     (orc.FMT_Q3K, True, 1), (orc.FMT_Q40, True, 1), (orc.FMT_Q50, False, 1)])
 def test_a_dense_decoder_loads_from_a_file(tmp_path, value_format, tied, parts):
     """spg_dense_dimensions and spo_dense_verify_load_gguf: the driver built from a file gives, bit for bit, the logits
     and the acceptance of the driver built by hand from the same tensors: q | k | v fused with the values in another
-    format than the queries and keys, a tied head, and the refusal of tensors the loader would ignore. The Q3_K case
-    keeps the values and the tied token table as Q3_K, which the hand-built driver takes as the rewritten Q6_K blocks."""
+    format than the queries and keys, a tied head, and the refusal of tensors the loader would ignore. The Q3_K, Q4_0 and
+    Q5_0 cases keep the values and the token table in that format, which the hand-built driver takes as the rewritten
+    Q6_K or Q8_0 blocks."""
     from splash_amd import verify
     from tests.dense_reference import DenseModel
     backend = splash_amd.Backend(0)
     model = DenseModel(seed=5, hidden=512, q_heads=16, kv_heads=8, head_dim=64, ffn=768, vocabulary=2048, layers=2, down_format=orc.FMT_Q6K)
-    q3k = value_format == orc.FMT_Q3K
-    if q3k:
+    rewritten = {orc.FMT_Q3K: gw.GGML_Q3_K, orc.FMT_Q40: gw.GGML_Q4_0, orc.FMT_Q50: gw.GGML_Q5_0}
+    if value_format in rewritten:
         for i, w in enumerate(model.layers):
-            w["v"] = orc.make_native(orc.FMT_Q3K, 512, 512, 40 + i)
-        model.embedding = orc.make_native(orc.FMT_Q3K, 2048, 512, 50)
-        model.table_format = orc.FMT_Q3K
+            w["v"] = orc.make_native(value_format, 512, 512, 40 + i)
+        model.embedding = orc.make_native(value_format, 2048, 512, 50)
+        model.table_format = value_format
     elif value_format != orc.FMT_Q4K:   # the values in the format a Q4_K_M file keeps them in
         for w in model.layers:
             w["v"] = orc.quantize_rows(value_format, orc.dequant_rows(orc.FMT_Q4K, w["v"], 512, 512))
     if tied:
         model.head = model.embedding
     # what the kernels read: a Q3_K tensor as the Q6_K blocks of its values
-    seen = lambda fmt, native: (orc.FMT_Q6K, ops.transcode_q3k(native)) if fmt == orc.FMT_Q3K else (fmt, native)
-    table_format = orc.FMT_Q3K if q3k else orc.FMT_Q4K
+    seen = lambda fmt, native: ops.rewrite_native(rewritten[fmt], native) if fmt in rewritten else (fmt, native)
+    table_format = value_format if value_format in rewritten else orc.FMT_Q4K
     path = dense_model_file(tmp_path / "dense.gguf", model, value_format, tied, parts=parts)   # a path, or a split file's parts
     rows, context = 16, 200
     rng = np.random.default_rng(1)

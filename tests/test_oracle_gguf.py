@@ -21,15 +21,17 @@ def test_dequant_matches_ggml_golden_hash(name, fmt):
     assert hashlib.sha256(values.tobytes()).hexdigest() == GOLDENS[name]
 
 
-def test_q3k_dequant_matches_ggml_golden_hash():
-    """goldens.json:8 (dequantize_row_q3_K): the oracle's Q3_K, which the kernels read rewritten as Q6_K blocks."""
-    native = orc.fixture(orc.FMT_Q3K, ROWS, COLUMNS, SEED + orc.FMT_Q3K)
-    values = orc.dequant_rows(orc.FMT_Q3K, native, ROWS, COLUMNS)
-    assert hashlib.sha256(values.tobytes()).hexdigest() == GOLDENS["q3k"]
+@pytest.mark.parametrize("name,fmt", [("q3k", orc.FMT_Q3K), ("q40", orc.FMT_Q40), ("q50", orc.FMT_Q50)])
+def test_dequant_of_the_rewritten_formats_matches_ggml_golden_hash(name, fmt):
+    """goldens.json:8,18,22 (dequantize_row_q3_K, _q4_0, _q5_0): the oracle's Q3_K, Q4_0 and Q5_0, which the kernels read
+    rewritten as Q6_K and Q8_0 blocks."""
+    native = orc.fixture(fmt, ROWS, COLUMNS, SEED + fmt)
+    values = orc.dequant_rows(fmt, native, ROWS, COLUMNS)
+    assert hashlib.sha256(values.tobytes()).hexdigest() == GOLDENS[name]
 
 
 @pytest.mark.skipif(orc.ref is None, reason="oracle/_ref was not built (no reference tree)")
-@pytest.mark.parametrize("fmt", [f for _, f in orc.ALL_FORMATS] + [orc.FMT_Q3K])
+@pytest.mark.parametrize("fmt", [f for _, f in orc.ALL_FORMATS] + [orc.FMT_Q3K, orc.FMT_Q40, orc.FMT_Q50])
 def test_restatement_equals_compiled_reference(fmt):
     native = orc.fixture(fmt, 64, 1024, 99)
     assert np.array_equal(native, orc.fixture(fmt, 64, 1024, 99, library=orc.ref))
