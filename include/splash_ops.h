@@ -410,6 +410,33 @@ typedef struct spo_sampling_policy {
 sp_status spo_sampling_add_verify(spo_graph *graph, const spo_sampling_buffers *buffers, uint32_t vocabulary,
                                   uint32_t logits_stride, const spo_lane_rows *lanes, const spo_sampling_policy *policies,
                                   uint32_t count, const uint32_t *stop_tokens);
+/* The sampling penalties (ops::SamplingPenalties and PenaltyTable, Sampling.hpp:17-30, :85-91): repetition scales the
+ * logit of every token the prompt or the output holds (a positive logit is divided, another multiplied), presence and
+ * frequency lower that of every token the output holds by presence + frequency x count; 1, 0, 0 change nothing.
+ * table_row: the lane's row of the penalty table, `vocabulary` words a row in device memory: bit 31 marks a prompt
+ * token, the other bits count how often the target selected the token (abi/Sampling.h:120-125). */
+typedef struct spo_sampling_penalties {
+  float repetition, presence, frequency;
+  uint32_t table_row;
+} spo_sampling_penalties;
+/* Sampling::rebuildPenaltyWords (Sampling.cpp:91-114): a request's row of the table, in host memory (upload it to the
+ * row), from its history: the prompt, then the generated_tokens outputs it emitted; pending_token (0xFFFFFFFF: none) is
+ * counted too; mark_prompt sets the prompt bit of the prompt's tokens (only repetition reads it). SP_INVALID_ARGUMENT
+ * for a token past the vocabulary or a history with no prompt. */
+sp_status spo_sampling_rebuild_penalty_words(uint32_t *words, uint32_t vocabulary, const uint32_t *history, uint64_t history_tokens,
+                                             uint64_t generated_tokens, uint32_t pending_token, uint32_t mark_prompt);
+/* Sampling::addPenalties (Sampling.cpp:163-180; its addVerify runs it first): the logits rows of every lane whose
+ * penalties are active are rewritten in place, before spo_sampling_add_verify reads them. A row's context adds, to
+ * the table's counts, the block's draft tokens (input_tokens) on the row's path (tree_rows), the anchor's excepted.
+ * Dispatches nothing when no lane's penalties are active. */
+sp_status spo_sampling_add_penalties(spo_graph *graph, sp_buffer *logits, sp_buffer *words, sp_buffer *input_tokens, sp_buffer *tree_rows,
+                                     uint32_t vocabulary, uint32_t logits_stride, const spo_lane_rows *lanes,
+                                     const spo_sampling_penalties *penalties, uint32_t count);
+/* Sampling::countPenaltyTokens (Sampling.cpp:116-121), on the device: the tokens each penalized lane retained of the
+ * step (spo_sampling_add_acceptance's tokens and retained counts) are counted into its row of the table, so the
+ * next step's penalties see them without a host round trip. */
+sp_status spo_sampling_add_penalty_count(spo_graph *graph, sp_buffer *words, sp_buffer *tokens, sp_buffer *retained, uint32_t vocabulary,
+                                         const spo_lane_rows *lanes, const spo_sampling_penalties *penalties, uint32_t count);
 /* Sampling::addAcceptance (Sampling.cpp:330-357). */
 sp_status spo_sampling_add_acceptance(spo_graph *graph, sp_buffer *input_tokens, sp_buffer *tree_rows, sp_buffer *tokens,
                                       sp_buffer *retained, sp_buffer *accepted_count, sp_buffer *retained_rows,
@@ -648,9 +675,17 @@ typedef enum spo_verify_buffer {
   /* the sampled rows' candidate children (spo_sampling_buffers): index 0 ids, 1 probabilities, 2 drawn children, 3 child
      uniforms; host-visible, allocated by the first call. Fetching them changes no step: spo_dense_verify_set_test_children
      chooses which test the sampled lanes of later steps run */
-  SPO_VERIFY_CANDIDATE_CHILDREN = 18
+  SPO_VERIFY_CANDIDATE_CHILDREN = 18,
+  /* the penalty table: uint32 [max lanes][vocabulary] in device memory, lane l's row at words l x vocabulary on
+     (spo_sampling_rebuild_penalty_words makes a row); allocated, zeroed, by the first call or by set_penalties */
+  SPO_VERIFY_PENALTY_WORDS = 19
 } spo_verify_buffer;
 sp_status spo_dense_verify_buffer(spo_dense_verify *verify, spo_verify_buffer which, uint32_t index, sp_buffer **out);
+/* The sampling penalties of dispatch lane `lane` (SamplingPolicy::penalties, Sampling.hpp:71 in the reference) for the
+ * steps encoded after: its rows of the head's logits are rewritten from its row of SPO_VERIFY_PENALTY_WORDS before the
+ * step selects (spo_sampling_add_penalties), and a step that commits counts the tokens the lane keeps into that row
+ * (spo_sampling_add_penalty_count). 1, 0, 0 turns them off. */
+sp_status spo_dense_verify_set_penalties(spo_dense_verify *verify, uint32_t lane, float repetition, float presence, float frequency);
 uint64_t spo_dense_verify_page_bytes(const spo_dense_verify *verify);
 /* Algorithmic HBM bytes of one step: weights once, each lane's KV, logits written and read. */
 uint64_t spo_dense_verify_step_bytes(const spo_dense_verify *verify, const spo_verify_lane *lanes, uint32_t count);
@@ -754,6 +789,8 @@ sp_status spo_hybrid_verify_set_capture(spo_hybrid_verify *verify, const uint32_
 #define SPO_VERIFY_GDN_STATES 13
 #define SPO_VERIFY_GDN_TAPE 14
 sp_status spo_hybrid_verify_buffer(spo_hybrid_verify *verify, uint32_t which, uint32_t index, sp_buffer **out);
+/* As spo_dense_verify_set_penalties. */
+sp_status spo_hybrid_verify_set_penalties(spo_hybrid_verify *verify, uint32_t lane, float repetition, float presence, float frequency);
 /* HybridVerify::encodePrefill: a chunk of `tokens` prompt tokens of the sequence of lane `lane` (its pages from table_first,
  * `committed` tokens cached; inputs as spo_dense_verify_encode_prefill's) through layers [first_layer, first_layer +
  * layer_count) (layer_count 0: to the last; the embedding with first_layer 0), no head: the reference's chunked prefill over

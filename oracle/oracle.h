@@ -226,6 +226,13 @@ void orc_rejection_law_policy(const float *logits, uint32_t vocab, const struct 
 // The selection law of one sampled row in fp64, for the enumeration check
 // (target_sampling_metal_test.mm:2602-2631): out[t] = P(row selects t) when the draft proposes its
 // child from q and the row tests and redraws as above. It must equal softmax(logits / T).
+// The sampling penalties of one lane's verify rows, in place (PenaltyReference.hpp:27-40 for a logit; sampling.metal:1008-1050
+// for the draft tokens a row's context adds): logits fp32 [rows][stride], words uint32 [vocabulary] (bit 31: in the prompt;
+// the rest: times selected), the block's input tokens and ancestor masks. Pinned by closed forms on chosen cases
+// (tests/test_oracle_sampling.py): untouched tokens bitwise, a prompt token's one product, a count's one difference,
+// saturation, unselectable logits, and the rows of a chain and of a forked tree that count a drafted token.
+void orc_penalize(float *logits, uint32_t rows, uint32_t vocabulary, uint32_t stride, const uint32_t *words, const uint32_t *input_tokens,
+                  const uint32_t *ancestors, float repetition, float presence, float frequency);
 // sampling.metal:697-880: a verify row of a tree block: up to four drawn children among sixteen candidates (ids, their
 // draft probabilities q, the candidate indices drawn in order, 0xFF for none, one uniform a child), then the last
 // residual's draw at u_row. Returns the selected token.

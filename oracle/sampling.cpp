@@ -608,4 +608,28 @@ void orc_rejection_law_policy(const float *x, uint32_t V, const OrcSamplingPolic
     out[t] = std::min(double(q[t]), p[t]) + (Z > 0 ? (1.0 - acceptMass) * std::max(p[t] - double(q[t]), 0.0) / Z : 0.0);
 }
 
+// The sampling penalties of a lane's verify rows, in place. One logit (PenaltyReference.hpp:27-40, referencePenalty): a
+// token the output holds `count` times or the prompt holds has its logit divided by the repetition penalty when
+// positive and multiplied otherwise, then lowered by frequency * count + presence when count is not 0, and the result
+// saturates at the largest float; NaN and -infinity stay. Which rows count which tokens (sampling.metal:1008-1050): row
+// r's count is the table's (the word without its prompt bit) plus the block's rows 1.. on r's path (its ancestors mask,
+// itself included) whose input token is the token; row 0's input, the anchor, is in the table already.
+void orc_penalize(float *logits, uint32_t rows, uint32_t vocabulary, uint32_t stride, const uint32_t *words, const uint32_t *input_tokens,
+                  const uint32_t *ancestors, float repetition, float presence, float frequency) {
+  constexpr float kLargest = std::numeric_limits<float>::max();
+  const float inverse = std::min(1.0f / repetition, kLargest);
+  for (uint32_t r = 0; r < rows; ++r)
+    for (uint32_t t = 0; t < vocabulary; ++t) {
+      uint32_t count = words[t] & 0x7FFFFFFFu;
+      for (uint32_t j = 1; j < rows; ++j)
+        if (((ancestors[r] >> j) & 1u) && input_tokens[j] == t) ++count;
+      const bool prompt = words[t] >> 31;
+      float &x = logits[size_t(r) * stride + t];
+      if ((!count && !prompt) || unselectable(x)) continue;
+      float v = x * (x > 0.0f ? inverse : repetition);
+      if (count) v -= frequency * float(count) + presence;
+      x = std::clamp(v, -kLargest, kLargest);
+    }
+}
+
 } // extern "C"

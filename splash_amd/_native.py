@@ -166,6 +166,10 @@ class SamplingPolicy(ctypes.Structure):
                 ("constrained", c_u32), ("excludes_stop_tokens", c_u32)]
 
 
+class SamplingPenalties(ctypes.Structure):
+    _fields_ = [("repetition", ctypes.c_float), ("presence", ctypes.c_float), ("frequency", ctypes.c_float), ("table_row", c_u32)]
+
+
 class HybridDimensions(ctypes.Structure):
     _fields_ = [(n, c_u32) for n in ("hidden", "vocabulary", "layers", "attention_interval", "q_heads", "kv_heads", "head_dim",
                                      "rotary_pairs", "normalize_heads", "gated_attention")] + [("rope_theta", ctypes.c_float)] + [
@@ -340,6 +344,11 @@ _sig("spo_dflash_draft_encode_decode", c_int, c_p, c_p, P(c_u32), c_u32)
 _sig("spo_dflash_draft_encode_context_prefill", c_int, c_p, c_p, c_u32, c_u32, c_u32, c_int)
 _sig("spo_dflash_draft_encode_context_commit", c_int, c_p, c_p, c_p, c_p, P(c_u32), c_u32, c_u32, c_u32)
 _sig("spo_sampling_add_acceptance", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, P(LaneRows), P(c_u32), c_u32, P(c_u32))
+_sig("spo_dense_verify_set_penalties", c_int, c_p, c_u32, ctypes.c_float, ctypes.c_float, ctypes.c_float)
+_sig("spo_hybrid_verify_set_penalties", c_int, c_p, c_u32, ctypes.c_float, ctypes.c_float, ctypes.c_float)
+_sig("spo_sampling_rebuild_penalty_words", c_int, c_p, c_u32, c_p, ctypes.c_uint64, ctypes.c_uint64, c_u32, c_u32)
+_sig("spo_sampling_add_penalties", c_int, c_p, c_p, c_p, c_p, c_p, c_u32, c_u32, P(LaneRows), P(SamplingPenalties), c_u32)
+_sig("spo_sampling_add_penalty_count", c_int, c_p, c_p, c_p, c_p, c_u32, P(LaneRows), P(SamplingPenalties), c_u32)
 _sig("spo_sampling_greedy_rows_static", c_int, ctypes.c_void_p, c_u32, c_u32, c_u32, ctypes.c_void_p, ctypes.c_void_p)
 _sig("spo_verify_check_results", c_int, P(LaneRows), P(c_u32), c_u32, c_u32, c_u32, P(c_u32), P(c_u32), P(c_u32), P(c_u32))
 _sig("spo_projection_rows", c_int, c_p, P(c_u32), P(c_u32), c_u32, P(c_p))

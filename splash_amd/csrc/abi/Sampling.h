@@ -55,6 +55,35 @@ struct TargetSamplingParams {
   uint32_t reserved[2];
 };
 
+// A penalized request's word for each vocabulary token, in its row of the penalty table (the reference's
+// SPLASH_PENALTY_PROMPT_BIT / _COUNT_MASK, abi/Sampling.h:120-125): the top bit marks a token of the prompt, the others
+// count how often the target selected the token.
+#define SAMPLING_PENALTY_PROMPT 0x80000000u
+#define SAMPLING_PENALTY_COUNT 0x7FFFFFFFu
+// decode_sample_penalize (the reference's SamplingPenaltyParams, abi/Sampling.h:127-142): entry e rewrites the logits
+// rows of lane[e] from row table_row[e] of the penalty table. repetition_inverse is 1 / repetition, at most FLT_MAX.
+struct SamplingPenaltyParams {
+  uint32_t vocabulary;
+  uint32_t logits_stride;
+  uint32_t entries;
+  uint32_t reserved;
+  struct SamplingLaneRows lane[SAMPLING_MAXIMUM_LANES];
+  uint32_t table_row[SAMPLING_MAXIMUM_LANES];
+  float repetition[SAMPLING_MAXIMUM_LANES];
+  float repetition_inverse[SAMPLING_MAXIMUM_LANES];
+  float presence[SAMPLING_MAXIMUM_LANES];
+  float frequency[SAMPLING_MAXIMUM_LANES];
+};
+// decode_sample_count_tokens: entry e adds the tokens its lane retained of a step (the first retained[lane[e]] of the
+// lane's rows of the acceptance's tokens) to row table_row[e] of the penalty table.
+struct SamplingCountParams {
+  uint32_t vocabulary;
+  uint32_t entries;
+  uint32_t lane[SAMPLING_MAXIMUM_LANES];        // the entry's lane of the acceptance (its word of `retained`)
+  uint32_t first_row[SAMPLING_MAXIMUM_LANES];   // that lane's first packed row
+  uint32_t table_row[SAMPLING_MAXIMUM_LANES];
+};
+
 // draft_verify_rows: one workgroup lays out a decode step's rows from the trees a draft selector grew (the reference's
 // VerifyRowsParams, abi/Sampling.h:270-298): `rows` rows over `lanes` lanes, each lane its anchor and the best of its
 // tree's other rows by estimate that the step's rows and the lanes' cap hold, none estimated below `floor`; the rows

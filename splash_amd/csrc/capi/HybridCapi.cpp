@@ -78,6 +78,13 @@ sp_status spo_hybrid_verify_set_capture(spo_hybrid_verify *verify, const uint32_
   });
 }
 
+sp_status spo_hybrid_verify_set_penalties(spo_hybrid_verify *verify, uint32_t lane, float repetition, float presence, float frequency) {
+  return capi::guard([&] {
+    capi::require(verify, "verify");
+    verify->verify->setPenalties(lane, {repetition, presence, frequency});
+  });
+}
+
 sp_status spg_hybrid_dimensions(const spg_file *file, spo_hybrid_dimensions *out) {
   return capi::guard([&] {
     capi::require(out, "result");
@@ -186,6 +193,7 @@ sp_status spo_hybrid_verify_buffer(spo_hybrid_verify *verify, uint32_t which, ui
     case SPO_VERIFY_LOGITS: b = v.logits(); break;
     case SPO_VERIFY_DRAFT_PROBABILITIES: b = v.draftProbabilities(); break;
     case SPO_VERIFY_HIDDEN: b = v.hidden(index); break;
+    case SPO_VERIFY_PENALTY_WORDS: b = v.penaltyWords(); break;
     case SPO_VERIFY_GDN_STATES: b = v.gdnStates(); break;
     case SPO_VERIFY_GDN_TAPE: b = v.gdnTape(); break;
     default: throw std::invalid_argument("no such verify buffer");

@@ -111,6 +111,59 @@ sp_status spo_sampling_add_verify(spo_graph *graph, const spo_sampling_buffers *
     ops::Sampling::addVerify(capi::graphOf(graph), buffers, vocabulary, logits_stride, rows, policies, stops);
   });
 }
+namespace {
+struct PenalizedLanes {
+  std::vector<ops::LaneRows> rows;
+  std::vector<ops::SamplingPolicy> policies;
+  std::vector<uint32_t> tableRows;
+  std::vector<bool> active;
+};
+PenalizedLanes penalizedLanes(const spo_lane_rows *lanes, const spo_sampling_penalties *penalties, uint32_t count) {
+  PenalizedLanes out;
+  for (uint32_t i = 0; i < count; ++i) {
+    out.rows.push_back({lanes[i].first, lanes[i].rows});
+    ops::SamplingPolicy policy;
+    policy.penalties = {penalties[i].repetition, penalties[i].presence, penalties[i].frequency};
+    out.policies.push_back(policy);
+    out.tableRows.push_back(penalties[i].table_row);
+    out.active.push_back(policy.penalties.active());
+  }
+  return out;
+}
+} // namespace
+sp_status spo_sampling_rebuild_penalty_words(uint32_t *words, uint32_t vocabulary, const uint32_t *history, uint64_t history_tokens,
+                                             uint64_t generated_tokens, uint32_t pending_token, uint32_t mark_prompt) {
+  return capi::guard([&] {
+    capi::require(words && history, "words or history");
+    ops::Sampling::rebuildPenaltyWords({words, vocabulary}, {history, size_t(history_tokens)}, generated_tokens,
+                                       pending_token == SAMPLING_NO_TOKEN ? std::nullopt : std::optional<uint32_t>(pending_token),
+                                       mark_prompt != 0);
+  });
+}
+sp_status spo_sampling_add_penalties(spo_graph *graph, sp_buffer *logits, sp_buffer *words, sp_buffer *input_tokens, sp_buffer *tree_rows,
+                                     uint32_t vocabulary, uint32_t logits_stride, const spo_lane_rows *lanes,
+                                     const spo_sampling_penalties *penalties, uint32_t count) {
+  return capi::guard([&] {
+    capi::require(graph && lanes && penalties, "graph, lanes or penalties");
+    const PenalizedLanes p = penalizedLanes(lanes, penalties, count);
+    ops::SamplingBuffers buffers{};
+    buffers.logits = B(logits);
+    buffers.inputTokens = B(input_tokens);
+    buffers.treeRows = B(tree_rows);
+    ops::Sampling::addPenalties(capi::graphOf(graph), buffers, vocabulary, logits_stride, p.rows, p.policies, {B(words), p.tableRows});
+  });
+}
+sp_status spo_sampling_add_penalty_count(spo_graph *graph, sp_buffer *words, sp_buffer *tokens, sp_buffer *retained, uint32_t vocabulary,
+                                         const spo_lane_rows *lanes, const spo_sampling_penalties *penalties, uint32_t count) {
+  return capi::guard([&] {
+    capi::require(graph && lanes && penalties, "graph, lanes or penalties");
+    const PenalizedLanes p = penalizedLanes(lanes, penalties, count);
+    ops::AcceptanceBuffers buffers{};
+    buffers.tokens = B(tokens);
+    buffers.retained = B(retained);
+    ops::Sampling::addPenaltyCount(capi::graphOf(graph), buffers, vocabulary, p.rows, p.active, {B(words), p.tableRows});
+  });
+}
 sp_status spo_sampling_add_acceptance(spo_graph *graph, sp_buffer *input_tokens, sp_buffer *tree_rows, sp_buffer *tokens,
                                       sp_buffer *retained, sp_buffer *accepted_count, sp_buffer *retained_rows,
                                       const spo_lane_rows *lanes, const uint32_t *remaining, uint32_t count,
@@ -299,6 +352,7 @@ sp_status spo_dense_verify_buffer(spo_dense_verify *verify, spo_verify_buffer wh
     case SPO_VERIFY_ATTENTION_ROWS: b = v.attentionRows(); break;
     case SPO_VERIFY_FFN_ROWS: b = v.ffnRows(); break;
     case SPO_VERIFY_CANDIDATE_CHILDREN: b = v.candidateChildren(index); break;
+    case SPO_VERIFY_PENALTY_WORDS: b = v.penaltyWords(); break;
     default: throw std::invalid_argument("no such verify buffer");
     }
     sp_buffer_retain(b.handle());
@@ -338,6 +392,12 @@ sp_status spo_dense_verify_encode_prefill(spo_dense_verify *verify, spo_graph *g
   return capi::guard([&] {
     capi::require(verify && graph, "verify or graph");
     verify->verify->encodePrefill(capi::graphOf(graph), table_first, committed, tokens);
+  });
+}
+sp_status spo_dense_verify_set_penalties(spo_dense_verify *verify, uint32_t lane, float repetition, float presence, float frequency) {
+  return capi::guard([&] {
+    capi::require(verify, "verify");
+    verify->verify->setPenalties(lane, {repetition, presence, frequency});
   });
 }
 sp_status spo_dense_verify_set_test_children(spo_dense_verify *verify, int on) {

@@ -80,6 +80,70 @@ __global__ __launch_bounds__(256) void decode_sample_admit(float *__restrict__ l
 }
 SP_REGISTER_KERNEL("decode_sample_admit", &decode_sample_admit);
 
+// The sampling penalties of one logit (PenaltyReference.hpp:27-40, sampling.metal:991-1006 in the reference): the
+// repetition penalty divides a positive logit and multiplies another when the prompt or the output holds the token;
+// presence and frequency lower it by the output's count of the token; the result stays finite. NaN and -infinity, which
+// no selection takes, stay as they are. One product, one product and sum, one difference, each rounded once.
+__device__ __forceinline__ float penalized_logit(float value, uint32_t count, float repetition, float repetition_inverse, float presence,
+                                                 float frequency) {
+  const uint32_t bits = __float_as_uint(value);
+  if ((bits & 0x7FFFFFFFu) > 0x7F800000u || bits == 0xFF800000u) return value;
+  float v = value * (value > 0.0f ? repetition_inverse : repetition);
+  if (count) v = v - (frequency * float(count) + presence);
+  return fminf(fmaxf(v, -3.402823466e+38f), 3.402823466e+38f);
+}
+// decode_sample_penalize: grid (ceil(vocabulary / 1024), entries), 256 threads, four tokens a thread 256 apart. A token
+// that the entry's table row does not hold and no row of the block drafted is left alone (nearly every token). A row's
+// context adds, to the table's count, the block's draft tokens on its path: its ancestors' and its own input token, but
+// not the anchor's, which the table counted when the target selected it (sampling.metal:1008-1050).
+__global__ __launch_bounds__(256) void decode_sample_penalize(float *__restrict__ logits, const uint32_t *__restrict__ words,
+                                                              const uint32_t *__restrict__ input_tokens,
+                                                              const AttentionTreeRow *__restrict__ tree, SamplingPenaltyParams p) {
+  const uint32_t entry = blockIdx.y;
+  const SamplingLaneRows lane = p.lane[entry];
+  __shared__ uint32_t drafts[SAMPLING_MAXIMUM_ROWS], paths[SAMPLING_MAXIMUM_ROWS];
+  if (threadIdx.x < lane.rows) {
+    drafts[threadIdx.x] = input_tokens[lane.first + threadIdx.x];
+    paths[threadIdx.x] = tree[lane.first + threadIdx.x].ancestors & ~1u;
+  }
+  __syncthreads();
+  const float repetition = p.repetition[entry], inverse = p.repetition_inverse[entry], presence = p.presence[entry],
+              frequency = p.frequency[entry];
+  const uint32_t *row_words = words + size_t(p.table_row[entry]) * p.vocabulary;
+#pragma unroll
+  for (uint32_t i = 0; i < 4; ++i) {
+    const uint32_t token = (blockIdx.x * 4u + i) * 256u + threadIdx.x;
+    if (token >= p.vocabulary) continue;
+    const uint32_t word = row_words[token];
+    uint32_t drafted = 0;
+    for (uint32_t r = 1; r < lane.rows; ++r) drafted |= uint32_t(drafts[r] == token) << r;
+    if (!(word | drafted)) continue;
+    const uint32_t selected = word & SAMPLING_PENALTY_COUNT;
+    float *column = logits + size_t(lane.first) * p.logits_stride + token;
+    for (uint32_t r = 0; r < lane.rows; ++r) {
+      const uint32_t count = selected + uint32_t(__popc(drafted & paths[r]));
+      if (!count && !(word & SAMPLING_PENALTY_PROMPT)) continue;
+      float &x = column[size_t(r) * p.logits_stride];
+      x = penalized_logit(x, count, repetition, inverse, presence, frequency);
+    }
+  }
+}
+SP_REGISTER_KERNEL("decode_sample_penalize", &decode_sample_penalize);
+
+// decode_sample_count_tokens: grid (entries), 64 threads. The tokens a lane retained of a step (the acceptance's `tokens`
+// from the lane's first row, `retained` of them) are counted into its row of the penalty table on the device, where the
+// reference's engine counts them on the host into shared memory (Sampling::countPenaltyTokens, Sampling.cpp:116-121).
+// A token twice in one step is counted twice (atomic adds).
+__global__ __launch_bounds__(64) void decode_sample_count_tokens(uint32_t *__restrict__ words, const uint32_t *__restrict__ tokens,
+                                                                 const uint32_t *__restrict__ retained, SamplingCountParams p) {
+  const uint32_t entry = blockIdx.x;
+  const uint32_t count = min(retained[p.lane[entry]], uint32_t(SAMPLING_MAXIMUM_ROWS));
+  if (threadIdx.x >= count) return;
+  const uint32_t token = tokens[p.first_row[entry] + threadIdx.x];
+  if (token < p.vocabulary) atomicAdd(words + size_t(p.table_row[entry]) * p.vocabulary + token, 1u);
+}
+SP_REGISTER_KERNEL("decode_sample_count_tokens", &decode_sample_count_tokens);
+
 
 // draft_verify_rows (the layout the reference's sampling.metal:1799-1895 produces): lane l's tree holds sizes[l] rows
 // from row l * 16 of tree_tokens, trees and scores (a row's draft probability and its estimate, the chance that the

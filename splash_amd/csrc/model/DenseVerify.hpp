@@ -7,6 +7,7 @@
 // the step's buffers; the residual stream ping-pongs between two hidden buffers.
 #pragma once
 #include "hip/Backend.hpp"
+#include "model/LanePenalties.hpp"
 #include "ops/Glue.hpp"
 #include "ops/Linear.hpp"
 #include "ops/PagedAttention.hpp"
@@ -78,6 +79,12 @@ public:
   // Fetching them changes no step: setTestChildren chooses, for the steps encoded after it, whether sampled lanes
   // read them or the full-vocabulary draft probabilities (the default).
   [[nodiscard]] const hip::Buffer &candidateChildren(uint32_t which);
+  // The sampling penalties of dispatch lane `lane` for the steps encoded after (ops::SamplingPenalties; 1, 0, 0 turns them
+  // off) and the table they read: lane l's row is words [l vocabulary, (l + 1) vocabulary) of penaltyWords(), which a
+  // request that takes the lane uploads (ops::Sampling::rebuildPenaltyWords). A step that commits counts what a
+  // penalized lane keeps into its row.
+  void setPenalties(uint32_t lane, ops::SamplingPenalties penalties) { penalties_.set(lane, penalties); }
+  [[nodiscard]] const hip::Buffer &penaltyWords() { return penalties_.words(); }
   void setTestChildren(bool on) { testChildren_ = on; if (on) (void)candidateChildren(0); }
   [[nodiscard]] bool testChildren() const noexcept { return testChildren_; }
   [[nodiscard]] const hip::Buffer &hidden(uint32_t index) const noexcept { return hidden_[index & 1]; }
@@ -144,6 +151,7 @@ private:
   DenseWeights weights_;
   ops::Linear linear_;
   uint32_t maxRows_ = 0, maxLanes_ = 0, rowCapacity_ = 0;
+  LanePenalties penalties_;
   uint64_t pageBytes_ = 0, layerBytes_ = 0;
   hip::Buffer kvAll_;
   hip::Buffer hidden_[2], normalized_, qkv_, attention_, intermediate_, logits_, draft_;

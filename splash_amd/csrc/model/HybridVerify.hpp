@@ -14,6 +14,7 @@
 #pragma once
 #include "hip/Backend.hpp"
 #include "model/DenseVerify.hpp"
+#include "model/LanePenalties.hpp"
 #include "ops/Gdn.hpp"
 #include "ops/Glue.hpp"
 #include "ops/Linear.hpp"
@@ -142,6 +143,12 @@ public:
   // Value head h of a GDN layer's output rows leaves at (h % heads per key) * key heads + h / heads per key, the order
   // llama.cpp's ssm_out reads them in (GgufImage.hpp:29-32): what a model loaded from a GGUF sets. Off by default.
   void setTiledGdnHeads(bool tiled) noexcept { tiledGdnHeads_ = tiled; }
+  // The sampling penalties of dispatch lane `lane` for the steps encoded after (ops::SamplingPenalties; 1, 0, 0 turns them
+  // off) and the table they read: lane l's row is words [l vocabulary, (l + 1) vocabulary) of penaltyWords(), which a
+  // request that takes the lane uploads (ops::Sampling::rebuildPenaltyWords). A step that commits counts what a
+  // penalized lane keeps into its row.
+  void setPenalties(uint32_t lane, ops::SamplingPenalties penalties) { penalties_.set(lane, penalties); }
+  [[nodiscard]] const hip::Buffer &penaltyWords() { return penalties_.words(); }
   // The hidden rows a draft's context is computed from (the reference's QwenTarget addCapture over RowCopy): after
   // layer layers[i] (ascending) every row's output goes to columns [i hidden, (i + 1) hidden) of its row of
   // `destination`, bf16 [rows][layers.size() x hidden], in a step and in a prompt chunk alike. An empty list captures nothing.
@@ -181,6 +188,7 @@ private:
   HybridWeights weights_;
   ops::Linear linear_;
   uint32_t maxRows_ = 0, maxLanes_ = 0, rowCapacity_ = 0;
+  LanePenalties penalties_;
   bool tiledGdnHeads_ = false;
   std::vector<uint32_t> captureLayers_;
   hip::Buffer captured_;

@@ -6,6 +6,7 @@
 #include <cmath>
 #include <limits>
 #include <stdexcept>
+#include <string>
 
 namespace splash::ops {
 
@@ -108,6 +109,77 @@ void Sampling::addVerify(hip::CommandGraph &graph, const SamplingBuffers &b, uin
   else
     graph.add("decode_sample_draw", {b.logits, b.draftProbabilities, b.masses, b.uniforms, b.ranges, b.decisions, b.tokens}, params,
               {rows, 1, 1}, {64, 1, 1});
+}
+
+void Sampling::rebuildPenaltyWords(std::span<uint32_t> words, std::span<const uint32_t> history, uint64_t generatedTokens,
+                                   std::optional<uint32_t> pendingToken, bool markPrompt) {
+  if (history.size() <= generatedTokens) throw std::logic_error("a request's history holds a prompt");
+  const size_t promptTokens = history.size() - size_t(generatedTokens);
+  auto inside = [&](uint32_t token) {
+    if (token >= words.size()) throw std::invalid_argument("token " + std::to_string(token) + " lies past the vocabulary");
+  };
+  for (const uint32_t token : history) inside(token);
+  if (pendingToken) inside(*pendingToken);
+  std::fill(words.begin(), words.end(), 0u);
+  for (size_t i = 0; i < history.size(); ++i) {
+    if (i >= promptTokens) ++words[history[i]];
+    else if (markPrompt) words[history[i]] |= SAMPLING_PENALTY_PROMPT;
+  }
+  if (pendingToken) ++words[*pendingToken];
+}
+
+void Sampling::addPenalties(hip::CommandGraph &graph, const SamplingBuffers &b, uint32_t vocabulary, uint32_t logitsStride,
+                            const std::vector<LaneRows> &lanes, const std::vector<SamplingPolicy> &policies, const PenaltyTable &table) {
+  const uint32_t rows = packedRows(lanes);
+  if (policies.size() != lanes.size()) throw std::invalid_argument("the penalties take one policy per lane");
+  if (!vocabulary || logitsStride < vocabulary) throw std::invalid_argument("logits rows hold the vocabulary");
+  SamplingPenaltyParams params{};
+  params.vocabulary = vocabulary;
+  params.logits_stride = logitsStride;
+  for (size_t l = 0; l < lanes.size(); ++l) {
+    const SamplingPenalties &penalties = policies[l].penalties;
+    if (!penalties.active()) continue;
+    if (!(penalties.repetition > 0.0f) || !std::isfinite(penalties.repetition) || !std::isfinite(penalties.presence) ||
+        !std::isfinite(penalties.frequency))
+      throw std::invalid_argument("a repetition penalty is above 0 and every penalty finite");
+    if (l >= table.rows.size()) throw std::invalid_argument("a penalized lane names its row of the penalty table");
+    const uint32_t e = params.entries++;
+    params.lane[e] = {lanes[l].first, lanes[l].rows};
+    params.table_row[e] = table.rows[l];
+    params.repetition[e] = penalties.repetition;
+    params.repetition_inverse[e] = std::min(1.0f / penalties.repetition, std::numeric_limits<float>::max());
+    params.presence[e] = penalties.presence;
+    params.frequency[e] = penalties.frequency;
+    requireBytes(table.words, (uint64_t{table.rows[l]} + 1) * vocabulary * 4, "penalty words");
+  }
+  if (!params.entries) return;
+  requireBytes(b.logits, (uint64_t{rows - 1} * logitsStride + vocabulary) * 4, "logits");
+  requireBytes(b.inputTokens, uint64_t{rows} * 4, "input tokens");
+  requireBytes(b.treeRows, uint64_t{rows} * sizeof(AttentionTreeRow), "verify tree rows");
+  graph.add("decode_sample_penalize", {b.logits, table.words, b.inputTokens, b.treeRows}, params,
+            {(vocabulary + 1023) / 1024, params.entries, 1}, {256, 1, 1});
+}
+
+void Sampling::addPenaltyCount(hip::CommandGraph &graph, const AcceptanceBuffers &b, uint32_t vocabulary, const std::vector<LaneRows> &lanes,
+                               const std::vector<bool> &penalized, const PenaltyTable &table) {
+  const uint32_t rows = packedRows(lanes);
+  if (penalized.size() != lanes.size()) throw std::invalid_argument("the count takes one flag per lane");
+  if (!vocabulary) throw std::invalid_argument("a penalty table row holds the vocabulary");
+  SamplingCountParams params{};
+  params.vocabulary = vocabulary;
+  for (size_t l = 0; l < lanes.size(); ++l) {
+    if (!penalized[l]) continue;
+    if (l >= table.rows.size()) throw std::invalid_argument("a penalized lane names its row of the penalty table");
+    const uint32_t e = params.entries++;
+    params.lane[e] = uint32_t(l);
+    params.first_row[e] = lanes[l].first;
+    params.table_row[e] = table.rows[l];
+    requireBytes(table.words, (uint64_t{table.rows[l]} + 1) * vocabulary * 4, "penalty words");
+  }
+  if (!params.entries) return;
+  requireBytes(b.tokens, uint64_t{rows} * 4, "retained tokens");
+  requireBytes(b.retained, lanes.size() * 4, "retained counts");
+  graph.add("decode_sample_count_tokens", {table.words, b.tokens, b.retained}, params, {params.entries, 1, 1}, {64, 1, 1});
 }
 
 void Sampling::addAcceptance(hip::CommandGraph &graph, const AcceptanceBuffers &b, const std::vector<LaneRows> &lanes,

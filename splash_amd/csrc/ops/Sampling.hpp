@@ -14,8 +14,25 @@
 
 namespace splash::ops {
 
-// Sampling.hpp:56-83 in the reference; the sampling penalties and the thinking cutoff belong to the engine's request
-// handling, not to the verify step, and are not built.
+// The sampling penalties (Sampling.hpp:17-30 in the reference), which rewrite a lane's target logits before its policy
+// selects from them: repetition scales the logit of every token the prompt or the output holds, presence and frequency
+// lower that of every token the output holds. The defaults leave the logits unchanged.
+struct SamplingPenalties final {
+  float repetition = 1.0f;
+  float presence = 0.0f;
+  float frequency = 0.0f;
+  [[nodiscard]] bool active() const noexcept { return repetition != 1.0f || presence != 0.0f || frequency != 0.0f; }
+};
+
+// The penalty words of every state lane, one row of `vocabulary` words each, in device memory, and the row each lane of
+// a dispatch reads (PenaltyTable, Sampling.hpp:85-91 in the reference).
+struct PenaltyTable final {
+  hip::Buffer words;
+  std::span<const uint32_t> rows;
+};
+
+// Sampling.hpp:56-83 in the reference; the thinking cutoff belongs to the engine's request handling, not to the verify
+// step, and is not built.
 struct SamplingPolicy final {
   float temperature = 0.0f;
   // A sampling lane keeps the tokens minP leaves it (those that weigh at least minP of the
@@ -28,6 +45,8 @@ struct SamplingPolicy final {
   bool constrained = false;
   // The lane ignores end-of-sequence: it never selects a stop token (addVerify's stopTokens).
   bool excludesStopTokens = false;
+  // Greedy lanes take the argmax of the penalized logits, sampling lanes draw from them.
+  SamplingPenalties penalties{};
   // A lane samples unless it keeps only its most likely token (Sampling.hpp:79-82).
   [[nodiscard]] bool samples() const noexcept { return temperature > 0.0f && minP < 1.0f && topK != 1; }
   [[nodiscard]] bool truncates(uint32_t vocabulary) const noexcept {
@@ -82,6 +101,24 @@ public:
                                                                                        SAMPLING_NO_TOKEN, SAMPLING_NO_TOKEN});
   static void addAcceptance(hip::CommandGraph &graph, const AcceptanceBuffers &buffers, const std::vector<LaneRows> &lanes,
                             const std::vector<uint32_t> &remaining, const std::array<uint32_t, SAMPLING_STOP_TOKENS> &stopTokens);
+
+  // A penalized request's penalty words, rebuilt when it takes a state lane (Sampling::rebuildPenaltyWords,
+  // Sampling.cpp:91-114 in the reference): from its history, the prompt and then the `generatedTokens` outputs it
+  // emitted. Every prompt token gets the prompt bit when markPrompt (only repetition reads it); the counts are of the
+  // outputs and of the pending anchor. Host memory; the caller uploads the row. Throws std::logic_error for a history
+  // with no prompt and std::invalid_argument for a token past the vocabulary (words.size()).
+  static void rebuildPenaltyWords(std::span<uint32_t> words, std::span<const uint32_t> history, uint64_t generatedTokens,
+                                  std::optional<uint32_t> pendingToken, bool markPrompt);
+  // Each lane with active penalties has the logits rows of its block rewritten in place from its row of the table, a
+  // row's context adding the block's draft tokens on its path (Sampling::addPenalties, Sampling.cpp:163-180; addVerify
+  // runs it first). Nothing is dispatched when no lane's penalties are active. Runs before addVerify on the LM head's
+  // fresh rows; buffers.inputTokens and buffers.treeRows are read for every penalized lane.
+  static void addPenalties(hip::CommandGraph &graph, const SamplingBuffers &buffers, uint32_t vocabulary, uint32_t logitsStride,
+                           const std::vector<LaneRows> &lanes, const std::vector<SamplingPolicy> &policies, const PenaltyTable &table);
+  // The tokens each lane retained of the step are counted into its row of the table, on the device (the reference's
+  // engine calls Sampling::countPenaltyTokens on the host, Sampling.cpp:116-121). `penalized[l]` selects the lanes.
+  static void addPenaltyCount(hip::CommandGraph &graph, const AcceptanceBuffers &buffers, uint32_t vocabulary,
+                              const std::vector<LaneRows> &lanes, const std::vector<bool> &penalized, const PenaltyTable &table);
 };
 
 } // namespace splash::ops

@@ -767,6 +767,42 @@ class Sampling:
         check(lib.spo_sampling_add_verify(graph.handle, ctypes.byref(b), vocabulary, stride, arr, structs, len(lanes), stops))
         graph._keep.extend([v for k, v in buffers.items() if k != "mask_words"])
 
+    PENALTY_PROMPT = 0x80000000
+
+    @staticmethod
+    def rebuild_penalty_words(vocabulary, history, generated_tokens, pending_token=None, mark_prompt=True):
+        """Sampling::rebuildPenaltyWords: a request's row of the penalty table (uint32 [vocabulary], host memory) from its
+        history (the prompt, then `generated_tokens` outputs) and the pending anchor."""
+        history = np.ascontiguousarray(history, dtype=np.uint32)
+        words = np.empty(vocabulary, dtype=np.uint32)
+        check(lib.spo_sampling_rebuild_penalty_words(words.ctypes.data, vocabulary, history.ctypes.data, history.size, generated_tokens,
+                                                     NO_TOKEN if pending_token is None else int(pending_token), int(mark_prompt)))
+        return words
+
+    @staticmethod
+    def _penalized(lanes, penalties):
+        if len(penalties) != len(lanes):
+            raise nat.InvalidArgument(1, "one (repetition, presence, frequency, table row) per lane")
+        return ((nat.LaneRows * len(lanes))(*[nat.LaneRows(*l) for l in lanes]),
+                (nat.SamplingPenalties * len(lanes))(*[nat.SamplingPenalties(*p) for p in penalties]))
+
+    @staticmethod
+    def add_penalties(graph, logits, words, input_tokens, tree_rows, vocabulary, stride, lanes, penalties):
+        """Sampling::addPenalties: penalties: a lane's (repetition, presence, frequency, table row); (1, 0, 0, *) leaves
+        the lane alone. Runs before add_verify."""
+        rows, structs = Sampling._penalized(lanes, penalties)
+        check(lib.spo_sampling_add_penalties(graph.handle, logits.handle, words.handle, input_tokens.handle, tree_rows.handle, vocabulary,
+                                             stride, rows, structs, len(lanes)))
+        graph._keep.extend([logits, words, input_tokens, tree_rows])
+
+    @staticmethod
+    def add_penalty_count(graph, words, tokens, retained, vocabulary, lanes, penalties):
+        """The tokens each penalized lane retained of the step (add_acceptance's) counted into its row of the table."""
+        rows, structs = Sampling._penalized(lanes, penalties)
+        check(lib.spo_sampling_add_penalty_count(graph.handle, words.handle, tokens.handle, retained.handle, vocabulary, rows, structs,
+                                                 len(lanes)))
+        graph._keep.extend([words, tokens, retained])
+
     STATIC_MAXIMUM_ROWS = 256
 
     @staticmethod

@@ -11,7 +11,7 @@ from .backend import Buffer, CommandGraph, STORAGE_PRIVATE
 from . import ops
 
 (INPUT_TOKENS, TREE_ROWS, DEPTHS, UNIFORMS, TOKENS, RETAINED, ACCEPTED, RETAINED_ROWS, PAGE_TABLE, KV_POOL, LOGITS,
- DRAFT_PROBABILITIES, HIDDEN, GDN_STATES, GDN_TAPE, QKV_ROWS, ATTENTION_ROWS, FFN_ROWS, CANDIDATE_CHILDREN) = range(19)
+ DRAFT_PROBABILITIES, HIDDEN, GDN_STATES, GDN_TAPE, QKV_ROWS, ATTENTION_ROWS, FFN_ROWS, CANDIDATE_CHILDREN, PENALTY_WORDS) = range(20)
 
 
 class Lane:
@@ -75,6 +75,11 @@ class DenseVerify:
     def set_staged_prefill(self, on):
         """Long prompt chunks through the prefill tile (the staged rule) instead of the step's kernels; off by default."""
         check(lib.spo_dense_verify_set_staged_prefill(self.handle, int(on)))
+
+    def set_penalties(self, lane, repetition=1.0, presence=0.0, frequency=0.0):
+        """The sampling penalties of dispatch lane `lane` for the steps encoded after; its row of the PENALTY_WORDS buffer
+        (uint32 [lanes][vocabulary]; ops.Sampling.rebuild_penalty_words makes a row) holds what they read."""
+        check(lib.spo_dense_verify_set_penalties(self.handle, lane, repetition, presence, frequency))
 
     def set_capture(self, layers, destination):
         """After each of `layers` (ascending) every row's output goes to its slot of `destination`, bf16 [rows][len(layers) x hidden]."""
@@ -267,6 +272,11 @@ class HybridVerify:
         check(lib.spo_hybrid_verify_set_layer(self.handle, layer, ctypes.byref(w)))
         self._keep.extend([mixer_input, mixer_output, input_norm, post_norm, router, gate_images, up_images, down_images, query_norm,
                            key_norm, convolution_weights, decay_weights, time_bias, mixer_norm, shared_scalar_gate, ffn])
+
+    def set_penalties(self, lane, repetition=1.0, presence=0.0, frequency=0.0):
+        """The sampling penalties of dispatch lane `lane` for the steps encoded after; its row of the PENALTY_WORDS buffer
+        (uint32 [lanes][vocabulary]; ops.Sampling.rebuild_penalty_words makes a row) holds what they read."""
+        check(lib.spo_hybrid_verify_set_penalties(self.handle, lane, repetition, presence, frequency))
 
     def set_capture(self, layers, destination):
         """After each of `layers` (ascending) every row's output goes to its slot of `destination`, bf16 [rows][len(layers) x hidden]."""

@@ -249,6 +249,20 @@ def argmax(logits):
     return lib.orc_argmax(_p(x, f32p), c_u32(x.size))
 
 
+def penalize(logits, words, input_tokens, ancestors, repetition=1.0, presence=0.0, frequency=0.0):
+    """One lane's verify rows [rows][vocabulary] under the sampling penalties; returns the rewritten copy."""
+    x = np.array(logits, dtype=np.float32, order="C")
+    rows, vocabulary = x.shape
+    w = np.ascontiguousarray(words, dtype=np.uint32)
+    tokens = np.ascontiguousarray(input_tokens, dtype=np.uint32)
+    paths = np.ascontiguousarray(ancestors, dtype=np.uint32)
+    assert w.size == vocabulary and tokens.size == rows and paths.size == rows
+    lib.orc_penalize.restype = None
+    lib.orc_penalize(_p(x, f32p), c_u32(rows), c_u32(vocabulary), c_u32(vocabulary), _p(w, u32p), _p(tokens, u32p), _p(paths, u32p),
+                     c_f(repetition), c_f(presence), c_f(frequency))
+    return x
+
+
 def accept_tree(tree, tokens, selected, remaining=0xFFFFFFFF, stop_tokens=()):
     """tree: structured array (ancestors, parent, depth). Returns (kept tokens, accepted, retained_rows)."""
     rows = len(tree)

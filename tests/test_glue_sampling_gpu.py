@@ -391,6 +391,79 @@ def test_constraint_masks_and_stop_exclusion(backend):
         ops.Sampling.add_verify(splash_amd.CommandGraph(), {**b, "token_mask": None}, V, V, lanes, policies)
 
 
+def test_penalties_rewrite_the_rows_and_count_what_a_step_keeps(backend):
+    """Sampling::addPenalties and the device's count of a step's tokens: the logits rows of the penalized lanes are the
+    oracle's bit for bit (chain and tree blocks, a stride wider than the vocabulary, NaN and -infinity among the logits,
+    tokens drafted several times), the other lanes' rows are untouched, greedy rows then select the argmax of the
+    penalized rows, and the tokens each penalized lane retains are counted into its row of the table, twice if kept
+    twice, so that a second step's penalties see them."""
+    from tests.test_oracle_sampling import random_tree
+    print("case sampling penalties", flush=True)
+    rng = np.random.default_rng(77)
+    V, stride = 5003, 5008
+    lanes = [(0, 5), (5, 16), (21, 1), (22, 9)]
+    rows = 31
+    # lane 0: defaults (left alone); lane 1: a tree, all three penalties; lane 2: one row, repetition; lane 3: a chain, presence / frequency
+    penalties = [(1.0, 0.0, 0.0, 3), (1.25, 0.4, 0.15, 2), (0.8, 0.0, 0.0, 0), (1.0, 1.5, 0.3, 1)]
+    logits = np.zeros((rows, stride), np.float32)
+    logits[:, :V] = (rng.standard_normal((rows, V)) * 3).astype(np.float32)
+    logits[6, rng.integers(0, V, 40)] = -np.inf
+    logits[7, rng.integers(0, V, 40)] = np.nan
+    logits[:, V:] = 123.0                                            # the padding of a row is never touched
+    tree = np.concatenate([ops.chain_tree_rows([5]), random_tree(rng, 16), ops.chain_tree_rows([1]), ops.chain_tree_rows([9])])
+    tokens = rng.integers(0, 40, rows).astype(np.uint32)              # few distinct tokens: drafts repeat and hit the table
+    # a row whose best token its own context drafted and whose second best nothing penalizes: the selection moves
+    logits[24, tokens[23]], logits[24, 4000] = 20.0, 19.0
+    table = np.zeros((4, V), np.uint32)
+    for row in range(4):
+        hit = rng.integers(0, 60, 30)
+        table[row, hit] = rng.integers(0, 4, 30).astype(np.uint32) | (rng.integers(0, 2, 30).astype(np.uint32) << 31)
+    words = backend.from_array(table)
+    b = sampling_buffers(backend, rows, V, logits, tokens=tokens, tree=tree)
+    g = splash_amd.CommandGraph()
+    ops.Sampling.add_penalties(g, b["logits"], words, b["input_tokens"], b["tree_rows"], V, stride, lanes, penalties)
+    ops.Sampling.add_verify(g, b, V, stride, lanes, [0.0] * 4)
+    backend.run(g)
+    seen = b["logits"].download(np.float32).reshape(rows, stride)
+    selected = b["tokens"].download(np.uint32)
+    for (first, n), (repetition, presence, frequency, row) in zip(lanes, penalties):
+        want = orc.penalize(logits[first:first + n, :V], table[row], tokens[first:first + n], tree["ancestors"][first:first + n],
+                            repetition, presence, frequency)
+        assert seen[first:first + n, :V].tobytes() == want.tobytes(), first
+        assert np.all(seen[first:first + n, V:] == 123.0)
+        for r in range(n):
+            assert selected[first + r] == orc.argmax(want[r])
+    assert seen[:5].tobytes() == logits[:5].tobytes()
+    assert orc.argmax(logits[24, :V]) == tokens[23] and selected[24] == 4000
+    # the acceptance, then the count of what each penalized lane retained
+    print("case sampling penalty count", flush=True)
+    retained, accepted, mask = (backend.allocate_buffer(len(lanes) * 4) for _ in range(3))
+    kept_tokens = backend.from_array(selected.copy())
+    g = splash_amd.CommandGraph()
+    ops.Sampling.add_acceptance(g, b["input_tokens"], b["tree_rows"], kept_tokens, retained, accepted, mask, lanes, [16] * 4)
+    ops.Sampling.add_penalty_count(g, words, kept_tokens, retained, V, lanes, penalties)
+    backend.run(g)
+    counts, kept = retained.download(np.uint32), kept_tokens.download(np.uint32)
+    want_table = table.copy()
+    for (first, n), (_, _, _, row), count in zip(lanes[1:], penalties[1:], counts[1:]):
+        assert 1 <= count <= n
+        np.add.at(want_table[row], kept[first:first + count], 1)
+    assert np.array_equal(words.download(np.uint32).reshape(4, V), want_table)
+    assert np.array_equal(want_table[3], table[3])                    # the lane without penalties counts nothing
+    # a token kept twice in one step is counted twice
+    twice = backend.from_array(np.array([11, 11, 11], np.uint32))
+    g = splash_amd.CommandGraph()
+    ops.Sampling.add_penalty_count(g, words, twice, backend.from_array(np.array([3], np.uint32)), V, [(0, 3)], [(1.1, 0.0, 0.0, 3)])
+    backend.run(g)
+    assert words.download(np.uint32).reshape(4, V)[3, 11] == want_table[3, 11] + 3
+    with pytest.raises(ValueError, match="repetition"):
+        ops.Sampling.add_penalties(splash_amd.CommandGraph(), b["logits"], words, b["input_tokens"], b["tree_rows"], V, stride, lanes,
+                                   [(0.0, 0.0, 0.0, 0)] * 4)
+    with pytest.raises(ValueError, match="penalty words"):
+        ops.Sampling.add_penalties(splash_amd.CommandGraph(), b["logits"], words, b["input_tokens"], b["tree_rows"], V, stride, lanes,
+                                   [(1.5, 0.0, 0.0, 4)] * 4)
+
+
 def test_verify_rows_are_laid_out_from_the_trees(backend):
     """draft_verify_rows (sampling.metal:1799-1895) against the oracle, bit for bit: tokens, tree rows, lane rows and
     sources over random trees, caps, floors and tied estimates; and its outputs are what the acceptance walk reads."""

@@ -218,6 +218,52 @@ def test_hidden_rows_are_captured_for_a_draft(backend):
         gpu.set_capture([0, 1, 2], captured)              # a destination too small for three layers' rows
 
 
+def test_a_penalized_lane_of_a_hybrid_step(backend):
+    """The sampling penalties through the hybrid driver, as through the dense one: the penalized lane's rows of the
+    step's logits are the oracle's penalties of the rows the same step leaves without them, its selections their argmax;
+    the other lane is untouched; a committing step counts what the lane keeps."""
+    print("case hybrid penalized lane", flush=True)
+    from splash_amd import ops
+    model = HybridModel(seed=47, **SHAPE)
+    gpu = model.build_gpu(backend, max_lanes=2, pages_per_lane=2)
+    rng = np.random.default_rng(9)
+    model.seed_context(rng)
+    model.seed_states(rng, lanes=2)
+    V = SHAPE["vocabulary"]
+    make_lanes = lambda: [verify.HybridLane(7, 40, table_first=0), verify.HybridLane(12, 200, table_first=model.pages_per_lane)]
+    lanes, rows = make_lanes(), 19
+    tokens = rng.integers(0, V, rows).astype(np.uint32)
+    tokens[3] = tokens[2]
+    tree = ops.chain_tree_rows([7, 12])
+    logits_of = lambda: gpu.buffer(verify.LOGITS).download(np.float32, rows * V).reshape(rows, V)
+    gpu.set_block(lanes, tokens)
+    backend.run(gpu.encode(lanes, commit=False))
+    plain = logits_of()
+    favourites = np.argmax(plain[:7], axis=1).astype(np.uint32)
+    words = ops.Sampling.rebuild_penalty_words(V, np.concatenate([favourites, favourites[:3]]), 3, pending_token=int(tokens[0]))
+    table = gpu.buffer(verify.PENALTY_WORDS)
+    table.upload(words)                                          # lane 0's row
+    penalties = (1.3, 2.0, 0.5)
+    gpu.set_penalties(0, *penalties)
+    lanes = make_lanes()
+    gpu.set_block(lanes, tokens)
+    graph = gpu.encode(lanes, commit=True)
+    assert "decode_sample_penalize" in graph.kernels() and "decode_sample_count_tokens" in graph.kernels()
+    backend.run(graph)
+    seen = logits_of()
+    got_tokens, got_retained, _, _ = (np.array(a).copy() for a in gpu.results(lanes))
+    want = orc.penalize(plain[:7], words, tokens[:7], tree["ancestors"][:7], *penalties)
+    assert seen[:7].tobytes() == want.tobytes() and seen[7:].tobytes() == plain[7:].tobytes()
+    selected = np.array([orc.argmax(row) for row in want], np.uint32)
+    assert np.any(selected != favourites)
+    kept, _, _ = orc.accept_tree(tree[:7], tokens[:7], selected)
+    assert got_retained[0] == len(kept) and np.array_equal(got_tokens[:len(kept)], kept)
+    want_words = words.copy()
+    np.add.at(want_words, kept, 1)
+    counted = table.download(np.uint32, 2 * V).reshape(2, V)
+    assert np.array_equal(counted[0], want_words) and not counted[1].any()
+
+
 def test_hybrid_rejects_bad_arguments(backend):
     with pytest.raises(ValueError):
         verify.HybridVerify(backend, **{**SHAPE, "layers": 5})            # not whole groups of four layers

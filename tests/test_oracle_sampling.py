@@ -380,3 +380,73 @@ def test_children_row_decisions_at_their_thresholds():
     qz = np.zeros(16, np.float32); qz[0] = 1.0                                      # the drawn child has no target mass: rejected
     assert orc.children_row(only, policy, ids, qz, [0], [0.5], 0.25)[0] == ids[2]
     assert orc.children_row(only, policy, ids, qz, [0], [0.5], 0.75)[0] == ids[9]
+
+
+def test_penalties_closed_forms():
+    """orc_penalize against what the definition fixes (PenaltyReference.hpp:27-40; sampling.metal:1008-1050), case by
+    case in float32 arithmetic: untouched tokens bitwise, a prompt token's single product, a count's single difference,
+    saturation instead of infinity, unselectable logits, and which rows of a chain and of a forked tree count a draft
+    token. Each case would fail for a dropped term, a swapped multiply / divide, a row counting its siblings or the
+    anchor counted twice."""
+    f32 = np.float32
+    V = 64
+    rng = np.random.default_rng(31)
+    base = (rng.standard_normal((4, V)) * 3).astype(np.float32)
+    chain = np.array([(2 << r) - 1 for r in range(4)], np.uint32)
+    tokens = np.array([5, 9, 9, 12], np.uint32)            # the anchor 5, then drafts 9, 9, 12
+    words = np.zeros(V, np.uint32)
+    # defaults change nothing, whatever the table holds
+    words[[3, 5, 7]] = [0x80000000, 2, 0x80000001]
+    assert orc.penalize(base, words, tokens, chain).tobytes() == base.tobytes()
+    # repetition alone: prompt-only token 3, output token 5 (count 2), both (7), and drafted tokens by row
+    rep = f32(1.3)
+    out = orc.penalize(base, words, tokens, chain, repetition=rep)
+    scaled = lambda x: x * (f32(1.0) / rep) if x > 0 else x * rep
+    for r in range(4):
+        for t in (3, 5, 7):
+            assert out[r, t] == scaled(base[r, t])
+        # row r's context holds drafts 1..r: token 9 from row 1 on, token 12 at row 3 only
+        assert out[r, 9] == (scaled(base[r, 9]) if r >= 1 else base[r, 9])
+        assert out[r, 12] == (scaled(base[r, 12]) if r >= 3 else base[r, 12])
+        untouched = np.setdiff1d(np.arange(V), [3, 5, 7, 9, 12])
+        assert out[r, untouched].tobytes() == base[r, untouched].tobytes()
+    # the sign decides divide or multiply: a positive logit shrinks, a negative one grows in magnitude, zero stays zero
+    probe = np.zeros((1, V), np.float32); probe[0, 3] = 2.0; probe[0, 7] = -2.0
+    out = orc.penalize(probe, words, tokens[:1], chain[:1], repetition=2.0)
+    assert (out[0, 3], out[0, 7], out[0, 5]) == (1.0, -4.0, 0.0)
+    # presence and frequency: only counted tokens (the prompt-only token 3 is not), by presence + frequency * count
+    presence, frequency = f32(0.7), f32(0.25)
+    out = orc.penalize(base, words, tokens, chain, presence=presence, frequency=frequency)
+    for r in range(4):
+        assert out[r, 3] == base[r, 3]
+        assert out[r, 5] == base[r, 5] - (frequency * f32(2) + presence)       # the anchor is in the table, never added again
+        assert out[r, 7] == base[r, 7] - (frequency * f32(1) + presence)
+        drafted9 = min(r, 2)                                                   # rows 1 and 2 both hold token 9
+        assert out[r, 9] == (base[r, 9] - (frequency * f32(drafted9) + presence) if drafted9 else base[r, 9])
+    # all three at once: scale first, then subtract
+    out = orc.penalize(base, words, tokens, chain, repetition=rep, presence=presence, frequency=frequency)
+    assert out[2, 7] == scaled(base[2, 7]) - (frequency * f32(1) + presence)
+    # a forked tree: rows 1 and 2 are siblings under the anchor, row 3 under row 2: a row counts its own path only
+    tree = np.array([0b0001, 0b0011, 0b0101, 0b1101], np.uint32)
+    forked = np.array([5, 20, 21, 20], np.uint32)
+    out = orc.penalize(base, np.zeros(V, np.uint32), forked, tree, presence=1.0)
+    assert [out[r, 20] == base[r, 20] - f32(1) for r in range(4)] == [False, True, False, True]
+    assert [out[r, 21] == base[r, 21] - f32(1) for r in range(4)] == [False, False, True, True]
+    assert [out[r, 20] == base[r, 20] for r in range(4)] == [True, False, True, False]
+    # the anchor's own token drafted again further down counts there
+    again = np.array([5, 5], np.uint32)
+    out = orc.penalize(base[:2], np.zeros(V, np.uint32), again, chain[:2], presence=1.0)
+    assert out[0, 5] == base[0, 5] and out[1, 5] == base[1, 5] - f32(1)
+    # saturation and the unselectable
+    big = np.zeros((1, V), np.float32)
+    big[0, 3] = np.finfo(np.float32).max; big[0, 7] = -np.finfo(np.float32).max; big[0, 5] = np.inf
+    edge_words = np.zeros(V, np.uint32); edge_words[[3, 5, 7, 8, 9]] = [0x80000000, 1, 1, 1, 1]
+    big[0, 8] = -np.inf; big[0, 9] = np.nan
+    out = orc.penalize(big, edge_words, tokens[:1], chain[:1], repetition=0.5, presence=1.0)
+    assert out[0, 3] == np.finfo(np.float32).max          # max / 0.5 saturates
+    assert out[0, 7] == -np.finfo(np.float32).max * f32(0.5) - f32(1)
+    assert out[0, 5] == np.finfo(np.float32).max          # +infinity becomes the largest float: still selectable, never infinite
+    assert out[0, 8] == -np.inf and np.isnan(out[0, 9])
+    # a repetition so small that its inverse overflows: the inverse saturates, the product does too
+    out = orc.penalize(probe, words, tokens[:1], chain[:1], repetition=1e-39)
+    assert out[0, 3] == np.finfo(np.float32).max

@@ -55,3 +55,29 @@ def test_lanes_outside_the_step_and_missing_arrays():
         check([(0, 4), (6, 4)], tokens, [1, 1], [0, 0], [1, 1])
     with pytest.raises(splash_amd.SplashError, match="rows of the step"):
         check([(0, 17)], np.arange(17, dtype=np.uint32), [1], [0], [1])
+
+
+def test_penalty_words_are_rebuilt_from_a_history():
+    """Sampling::rebuildPenaltyWords (Sampling.cpp:91-114 in the reference): the prompt's tokens carry the prompt bit when
+    asked, the outputs and the pending anchor are counted, everything else is zero; a history without a prompt and a
+    token past the vocabulary are refused."""
+    from splash_amd import ops
+    V = 50
+    prompt, outputs = [3, 7, 7, 9], [7, 11, 11, 11]
+    words = ops.Sampling.rebuild_penalty_words(V, prompt + outputs, len(outputs), pending_token=9)
+    want = np.zeros(V, np.uint32)
+    want[[3, 7, 9]] = ops.Sampling.PENALTY_PROMPT
+    want[7] |= 1
+    want[11] = 3
+    want[9] |= 1
+    assert np.array_equal(words, want)
+    unmarked = ops.Sampling.rebuild_penalty_words(V, prompt + outputs, len(outputs), mark_prompt=False)
+    assert np.array_equal(unmarked, np.bincount(outputs, minlength=V).astype(np.uint32))
+    only_prompt = ops.Sampling.rebuild_penalty_words(V, prompt, 0)
+    assert np.array_equal(only_prompt, np.where(np.isin(np.arange(V), prompt), ops.Sampling.PENALTY_PROMPT, 0).astype(np.uint32))
+    with pytest.raises(splash_amd.SplashError):
+        ops.Sampling.rebuild_penalty_words(V, outputs, len(outputs))          # no prompt
+    with pytest.raises(ValueError):
+        ops.Sampling.rebuild_penalty_words(V, [3, V], 0)
+    with pytest.raises(ValueError):
+        ops.Sampling.rebuild_penalty_words(V, [3], 0, pending_token=V)

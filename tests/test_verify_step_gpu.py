@@ -224,6 +224,68 @@ def test_a_sampled_tree_block_tests_its_drawn_children(backend):
     assert 1 <= retained[0] <= rows and (not sure or accepted[0] >= 1)
 
 
+def test_a_penalized_lane_selects_from_its_penalized_rows(backend):
+    """SamplingPolicy::penalties through the driver (Sampling.hpp:71, Sampling.cpp:163-194 in the reference): of two lanes
+    one takes penalties. Its rows of the step's logits are the oracle's penalties of the rows the same step leaves without
+    them, bit for bit, its selections their argmax and its acceptance the walk over those; the other lane's rows and
+    results do not change. A step that commits counts the tokens the penalized lane keeps into its row of the table, which
+    the next step's penalties then read."""
+    print("case config 1 penalized lane", flush=True)
+    from splash_amd import ops
+    V = 4096
+    model = DenseModel(seed=21, hidden=512, q_heads=8, kv_heads=4, head_dim=64, ffn=1024, vocabulary=V, layers=2)
+    rng = np.random.default_rng(3)
+    context = 70
+    gpu = model.build_gpu(backend, max_lanes=2, context_tokens=context + 16)
+    make_lanes = lambda: [verify.Lane(6, context, table_first=model.table_first[0]), verify.Lane(9, context, table_first=model.table_first[1])]
+    lanes = make_lanes()
+    model.seed_context(gpu, None, rng)
+    tokens = rng.integers(0, V, 15).astype(np.uint32)
+    tokens[10] = tokens[11] = tokens[9]                               # the penalized lane drafts one token three times
+    tree = ops.chain_tree_rows([6, 9])
+    logits_of = lambda: gpu.buffer(verify.LOGITS).download(np.float32, 15 * V).reshape(15, V)
+    gpu.set_block(lanes, tokens, tree_rows=tree)
+    backend.run(gpu.encode(lanes, commit=False))
+    plain, plain_results = logits_of(), [np.array(a).copy() for a in gpu.results(lanes)]
+    # lane 1's history: a prompt that holds the plain step's favourite tokens, outputs that hold some of them again
+    favourites = np.argmax(plain[6:], axis=1).astype(np.uint32)
+    history = np.concatenate([favourites[:5], rng.integers(0, V, 20).astype(np.uint32), favourites[3:7], favourites[3:4]])
+    words = ops.Sampling.rebuild_penalty_words(V, history, 5, pending_token=int(tokens[6]))
+    table = gpu.buffer(verify.PENALTY_WORDS)
+    table.upload(words, offset_bytes=V * 4)
+    penalties = (1.4, 0.9, 0.35)
+    gpu.set_penalties(1, *penalties)
+    graph = gpu.encode(lanes, commit=False)
+    assert "decode_sample_penalize" in graph.kernels() and "decode_sample_count_tokens" not in graph.kernels()
+    backend.run(graph)
+    seen = logits_of()
+    got_tokens, got_retained, got_accepted, got_mask = (np.array(a).copy() for a in gpu.results(lanes))
+    want = orc.penalize(plain[6:], words, tokens[6:], tree["ancestors"][6:], *penalties)
+    assert seen[:6].tobytes() == plain[:6].tobytes() and seen[6:].tobytes() == want.tobytes()
+    assert (got_retained[0], got_accepted[0], got_mask[0]) == (plain_results[1][0], plain_results[2][0], plain_results[3][0])
+    assert np.array_equal(got_tokens[:got_retained[0]], plain_results[0][:got_retained[0]])
+    selected = np.array([orc.argmax(row) for row in want], np.uint32)
+    assert np.any(selected != favourites)                             # the penalties moved a selection
+    kept, accepted, mask = orc.accept_tree(tree[6:], tokens[6:], selected)
+    assert np.array_equal(got_tokens[6:6 + len(kept)], kept) and (got_retained[1], got_accepted[1], got_mask[1]) == (len(kept), accepted, mask)
+    # a committing step counts what the lane keeps; the lane without penalties counts nothing
+    graph = gpu.encode(lanes, commit=True)
+    assert "decode_sample_count_tokens" in graph.kernels()
+    backend.run(graph)
+    counted = table.download(np.uint32, 2 * V).reshape(2, V)
+    want_words = words.copy()
+    np.add.at(want_words, kept, 1)
+    assert np.array_equal(counted[1], want_words) and not counted[0].any()
+    # penalties off again: the step is the plain one
+    gpu.set_penalties(1)
+    lanes = make_lanes()
+    gpu.set_block(lanes, tokens, tree_rows=tree)
+    graph = gpu.encode(lanes, commit=False)
+    assert "decode_sample_penalize" not in graph.kernels()
+    backend.run(graph)
+    assert logits_of().tobytes() == plain.tobytes()
+
+
 @pytest.mark.parametrize("lanes_rows", [[16], [7, 16, 3]])
 def test_chained_projections_change_nothing(backend, lanes_rows):
     """A step whose layers dispatch their four projections after the attention as one chain (a layer's output, gate/up
