@@ -437,6 +437,21 @@ sp_status spo_sampling_add_penalties(spo_graph *graph, sp_buffer *logits, sp_buf
  * next step's penalties see them without a host round trip. */
 sp_status spo_sampling_add_penalty_count(spo_graph *graph, sp_buffer *words, sp_buffer *tokens, sp_buffer *retained, uint32_t vocabulary,
                                          const spo_lane_rows *lanes, const spo_sampling_penalties *penalties, uint32_t count);
+/* ops::ThinkingCutoff of a lane's policy (Sampling.hpp:30-55): the lane's selected rows of depth `row` on take the
+ * `count` tokens of `end` in order (as many as the block holds) unless a draft token on a row's path up to that depth is
+ * the last of `end` or `also_ends` (0xFFFFFFFF: none), which ended thinking first; with waits_for_mask the end starts,
+ * along each path, at the first row from depth `row` on whose constraint-mask row admits end[0]. active 0: no cutoff. */
+typedef struct spo_thinking_cutoff {
+  uint32_t active, row, count;
+  uint32_t end[16];
+  uint32_t also_ends, waits_for_mask;
+} spo_thinking_cutoff;
+/* The end of Sampling::addSelection (Sampling.cpp:314-327): rewrites the selections spo_sampling_add_verify left in
+ * `tokens`, before spo_sampling_add_acceptance walks them. token_mask (uint32 [rows][mask_words]) is read only for lanes
+ * whose end waits for their mask; NULL otherwise. Dispatches nothing when no lane's cutoff lies inside its block. */
+sp_status spo_sampling_add_thinking_cutoff(spo_graph *graph, sp_buffer *input_tokens, sp_buffer *tree_rows, sp_buffer *tokens,
+                                           sp_buffer *token_mask, uint32_t mask_words, uint32_t vocabulary,
+                                           const spo_lane_rows *lanes, const spo_thinking_cutoff *cutoffs, uint32_t count);
 /* Sampling::addAcceptance (Sampling.cpp:330-357). */
 sp_status spo_sampling_add_acceptance(spo_graph *graph, sp_buffer *input_tokens, sp_buffer *tree_rows, sp_buffer *tokens,
                                       sp_buffer *retained, sp_buffer *accepted_count, sp_buffer *retained_rows,
@@ -686,6 +701,10 @@ sp_status spo_dense_verify_buffer(spo_dense_verify *verify, spo_verify_buffer wh
  * step selects (spo_sampling_add_penalties), and a step that commits counts the tokens the lane keeps into that row
  * (spo_sampling_add_penalty_count). 1, 0, 0 turns them off. */
 sp_status spo_dense_verify_set_penalties(spo_dense_verify *verify, uint32_t lane, float repetition, float presence, float frequency);
+/* The thinking cutoff of dispatch lane `lane` (SamplingPolicy::thinkingCutoff, Sampling.hpp:76) for the steps encoded
+ * after; NULL, or active 0, clears it. The drivers' lanes are not constrained, so an end that waits for a mask is refused
+ * when the step is encoded. */
+sp_status spo_dense_verify_set_thinking_cutoff(spo_dense_verify *verify, uint32_t lane, const spo_thinking_cutoff *cutoff);
 uint64_t spo_dense_verify_page_bytes(const spo_dense_verify *verify);
 /* Algorithmic HBM bytes of one step: weights once, each lane's KV, logits written and read. */
 uint64_t spo_dense_verify_step_bytes(const spo_dense_verify *verify, const spo_verify_lane *lanes, uint32_t count);
@@ -791,6 +810,8 @@ sp_status spo_hybrid_verify_set_capture(spo_hybrid_verify *verify, const uint32_
 sp_status spo_hybrid_verify_buffer(spo_hybrid_verify *verify, uint32_t which, uint32_t index, sp_buffer **out);
 /* As spo_dense_verify_set_penalties. */
 sp_status spo_hybrid_verify_set_penalties(spo_hybrid_verify *verify, uint32_t lane, float repetition, float presence, float frequency);
+/* As spo_dense_verify_set_thinking_cutoff. */
+sp_status spo_hybrid_verify_set_thinking_cutoff(spo_hybrid_verify *verify, uint32_t lane, const spo_thinking_cutoff *cutoff);
 /* HybridVerify::encodePrefill: a chunk of `tokens` prompt tokens of the sequence of lane `lane` (its pages from table_first,
  * `committed` tokens cached; inputs as spo_dense_verify_encode_prefill's) through layers [first_layer, first_layer +
  * layer_count) (layer_count 0: to the last; the embedding with first_layer 0), no head: the reference's chunked prefill over

@@ -233,6 +233,15 @@ void orc_rejection_law_policy(const float *logits, uint32_t vocab, const struct 
 // saturation, unselectable logits, and the rows of a chain and of a forked tree that count a drafted token.
 void orc_penalize(float *logits, uint32_t rows, uint32_t vocabulary, uint32_t stride, const uint32_t *words, const uint32_t *input_tokens,
                   const uint32_t *ancestors, float repetition, float presence, float frequency);
+// The thinking cutoff of one lane's selections, in place (sampling.metal:1993-2039): tokens uint32 [rows] (the selections),
+// the block's input tokens and tree rows, the depth the end starts at, the end's first `count` tokens, the token that
+// closes thinking and the other that ends it, and, for an end that waits for its mask, whether each row's mask admits
+// end[0] (NULL: the end does not wait). Pinned by hand-worked chains and trees (tests/test_oracle_sampling.py): the rows
+// that take which end token, the rows past the end, an end already drafted on the path (and not on a sibling's), the
+// sentinel kept, and the waiting end's later start.
+void orc_thinking_cutoff(uint32_t *tokens, const uint32_t *input_tokens, const struct OrcTreeRow *tree, uint32_t rows, uint32_t vocabulary,
+                         uint32_t cutoff_row, const uint32_t *end, uint32_t count, uint32_t close, uint32_t also_ends,
+                         const uint8_t *admits);
 // sampling.metal:697-880: a verify row of a tree block: up to four drawn children among sixteen candidates (ids, their
 // draft probabilities q, the candidate indices drawn in order, 0xFF for none, one uniform a child), then the last
 // residual's draw at u_row. Returns the selected token.

@@ -632,4 +632,29 @@ void orc_penalize(float *logits, uint32_t rows, uint32_t vocabulary, uint32_t st
     }
 }
 
+// The thinking cutoff of one lane over its selections, in place (sampling.metal:1993-2039, ThinkingCutoffParams in
+// abi/Sampling.h:147-175): for every row, the cut is the depth of the first row of its path, from the anchor down, at
+// depth cutoff_row or deeper (and, when `admits` is given, an end that waits for its mask, whose admits[] is set); a
+// row `i` levels below its cut, i < count, selects end[i], unless a draft token of a path row other than the anchor at
+// depth <= cut is `close` or `also_ends`, or the row's selection is no token of the vocabulary.
+void orc_thinking_cutoff(uint32_t *tokens, const uint32_t *input_tokens, const struct OrcTreeRow *tree, uint32_t rows, uint32_t vocabulary,
+                         uint32_t cutoff_row, const uint32_t *end, uint32_t count, uint32_t close, uint32_t also_ends,
+                         const uint8_t *admits) {
+  for (uint32_t r = 0; r < rows; ++r) {
+    const uint32_t path = tree[r].ancestors, depth = tree[r].depth;
+    uint32_t cut = 0;
+    bool found = false;
+    for (uint32_t j = 0; j < rows && !found; ++j) {
+      if (!((path >> j) & 1u)) continue;
+      if (cut >= cutoff_row && (!admits || admits[j])) found = true;
+      else ++cut;
+    }
+    if (!found || cut > depth || depth - cut >= count) continue;
+    bool ended = false;
+    for (uint32_t j = 1; j < rows; ++j)
+      if (((path >> j) & 1u) && tree[j].depth <= cut && (input_tokens[j] == close || input_tokens[j] == also_ends)) ended = true;
+    if (!ended && tokens[r] < vocabulary) tokens[r] = end[depth - cut];
+  }
+}
+
 } // extern "C"

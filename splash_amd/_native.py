@@ -170,6 +170,10 @@ class SamplingPenalties(ctypes.Structure):
     _fields_ = [("repetition", ctypes.c_float), ("presence", ctypes.c_float), ("frequency", ctypes.c_float), ("table_row", c_u32)]
 
 
+class ThinkingCutoff(ctypes.Structure):
+    _fields_ = [("active", c_u32), ("row", c_u32), ("count", c_u32), ("end", c_u32 * 16), ("also_ends", c_u32), ("waits_for_mask", c_u32)]
+
+
 class HybridDimensions(ctypes.Structure):
     _fields_ = [(n, c_u32) for n in ("hidden", "vocabulary", "layers", "attention_interval", "q_heads", "kv_heads", "head_dim",
                                      "rotary_pairs", "normalize_heads", "gated_attention")] + [("rope_theta", ctypes.c_float)] + [
@@ -346,9 +350,12 @@ _sig("spo_dflash_draft_encode_context_commit", c_int, c_p, c_p, c_p, c_p, P(c_u3
 _sig("spo_sampling_add_acceptance", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, P(LaneRows), P(c_u32), c_u32, P(c_u32))
 _sig("spo_dense_verify_set_penalties", c_int, c_p, c_u32, ctypes.c_float, ctypes.c_float, ctypes.c_float)
 _sig("spo_hybrid_verify_set_penalties", c_int, c_p, c_u32, ctypes.c_float, ctypes.c_float, ctypes.c_float)
+_sig("spo_dense_verify_set_thinking_cutoff", c_int, c_p, c_u32, P(ThinkingCutoff))
+_sig("spo_hybrid_verify_set_thinking_cutoff", c_int, c_p, c_u32, P(ThinkingCutoff))
 _sig("spo_sampling_rebuild_penalty_words", c_int, c_p, c_u32, c_p, ctypes.c_uint64, ctypes.c_uint64, c_u32, c_u32)
 _sig("spo_sampling_add_penalties", c_int, c_p, c_p, c_p, c_p, c_p, c_u32, c_u32, P(LaneRows), P(SamplingPenalties), c_u32)
 _sig("spo_sampling_add_penalty_count", c_int, c_p, c_p, c_p, c_p, c_u32, P(LaneRows), P(SamplingPenalties), c_u32)
+_sig("spo_sampling_add_thinking_cutoff", c_int, c_p, c_p, c_p, c_p, c_p, c_u32, c_u32, P(LaneRows), P(ThinkingCutoff), c_u32)
 _sig("spo_sampling_greedy_rows_static", c_int, ctypes.c_void_p, c_u32, c_u32, c_u32, ctypes.c_void_p, ctypes.c_void_p)
 _sig("spo_verify_check_results", c_int, P(LaneRows), P(c_u32), c_u32, c_u32, c_u32, P(c_u32), P(c_u32), P(c_u32), P(c_u32))
 _sig("spo_projection_rows", c_int, c_p, P(c_u32), P(c_u32), c_u32, P(c_p))

@@ -84,6 +84,25 @@ struct SamplingCountParams {
   uint32_t table_row[SAMPLING_MAXIMUM_LANES];
 };
 
+// decode_sample_end_thinking (the reference's ThinkingCutoffParams, abi/Sampling.h:147-175): where a lane's thinking
+// budget runs out in a selection. Each row's path is cut at its row of depth row[lane] (for a lane of waiting_mask: at
+// its first row from that depth on whose constraint-mask row admits tokens[lane][0]); the path's row of depth cut + i
+// selects tokens[lane][i], for i below count[lane], unless a draft token on the path up to the cut, the anchor's
+// excepted, is close[lane] (the last token of the lane's end) or also_ends[lane]: thinking ended before. A row whose
+// selection is the sentinel keeps it. A lane without a cutoff has row SAMPLING_MAXIMUM_ROWS.
+struct ThinkingCutoffParams {
+  uint32_t vocabulary;
+  uint32_t lanes;
+  uint32_t waiting_mask;
+  uint32_t mask_words;   // words of a constraint-mask row, one a packed row (TargetSamplingParams::mask_words)
+  struct SamplingLaneRows lane[SAMPLING_MAXIMUM_LANES];
+  uint32_t row[SAMPLING_MAXIMUM_LANES];
+  uint32_t count[SAMPLING_MAXIMUM_LANES];
+  uint32_t close[SAMPLING_MAXIMUM_LANES];
+  uint32_t also_ends[SAMPLING_MAXIMUM_LANES];
+  uint32_t tokens[SAMPLING_MAXIMUM_LANES][SAMPLING_MAXIMUM_ROWS];
+};
+
 // draft_verify_rows: one workgroup lays out a decode step's rows from the trees a draft selector grew (the reference's
 // VerifyRowsParams, abi/Sampling.h:270-298): `rows` rows over `lanes` lanes, each lane its anchor and the best of its
 // tree's other rows by estimate that the step's rows and the lanes' cap hold, none estimated below `floor`; the rows

@@ -2,6 +2,7 @@
 #include "splash_ops.h"
 #include "capi/Guard.hpp"
 #include "capi/Handles.hpp"
+#include "capi/Policies.hpp"
 #include "model/GgufTarget.hpp"
 #include "model/HybridVerify.hpp"
 #include "splash_gguf.h"
@@ -82,6 +83,13 @@ sp_status spo_hybrid_verify_set_penalties(spo_hybrid_verify *verify, uint32_t la
   return capi::guard([&] {
     capi::require(verify, "verify");
     verify->verify->setPenalties(lane, {repetition, presence, frequency});
+  });
+}
+
+sp_status spo_hybrid_verify_set_thinking_cutoff(spo_hybrid_verify *verify, uint32_t lane, const spo_thinking_cutoff *cutoff) {
+  return capi::guard([&] {
+    capi::require(verify, "verify");
+    verify->verify->setThinkingCutoff(lane, capi::cutoffOf(cutoff));
   });
 }
 

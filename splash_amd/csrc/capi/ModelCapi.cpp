@@ -2,6 +2,7 @@
 #include "splash_ops.h"
 #include "capi/Guard.hpp"
 #include "capi/Handles.hpp"
+#include "capi/Policies.hpp"
 #include "model/DenseVerify.hpp"
 #include "model/StepResults.hpp"
 #include "model/GgufTarget.hpp"
@@ -162,6 +163,27 @@ sp_status spo_sampling_add_penalty_count(spo_graph *graph, sp_buffer *words, sp_
     buffers.tokens = B(tokens);
     buffers.retained = B(retained);
     ops::Sampling::addPenaltyCount(capi::graphOf(graph), buffers, vocabulary, p.rows, p.active, {B(words), p.tableRows});
+  });
+}
+sp_status spo_sampling_add_thinking_cutoff(spo_graph *graph, sp_buffer *input_tokens, sp_buffer *tree_rows, sp_buffer *tokens,
+                                           sp_buffer *token_mask, uint32_t mask_words, uint32_t vocabulary,
+                                           const spo_lane_rows *lanes, const spo_thinking_cutoff *cutoffs, uint32_t count) {
+  return capi::guard([&] {
+    capi::require(graph && lanes && cutoffs, "graph, lanes or cutoffs");
+    std::vector<ops::LaneRows> rows;
+    std::vector<ops::SamplingPolicy> policies(count);
+    for (uint32_t i = 0; i < count; ++i) {
+      rows.push_back({lanes[i].first, lanes[i].rows});
+      policies[i].thinkingCutoff = capi::cutoffOf(&cutoffs[i]);
+      policies[i].constrained = cutoffs[i].active && cutoffs[i].waits_for_mask;
+    }
+    ops::SamplingBuffers buffers{};
+    buffers.inputTokens = B(input_tokens);
+    buffers.treeRows = B(tree_rows);
+    buffers.tokens = B(tokens);
+    buffers.tokenMask = B(token_mask);
+    buffers.maskWords = mask_words;
+    ops::Sampling::addThinkingCutoff(capi::graphOf(graph), buffers, vocabulary, rows, policies);
   });
 }
 sp_status spo_sampling_add_acceptance(spo_graph *graph, sp_buffer *input_tokens, sp_buffer *tree_rows, sp_buffer *tokens,
@@ -398,6 +420,12 @@ sp_status spo_dense_verify_set_penalties(spo_dense_verify *verify, uint32_t lane
   return capi::guard([&] {
     capi::require(verify, "verify");
     verify->verify->setPenalties(lane, {repetition, presence, frequency});
+  });
+}
+sp_status spo_dense_verify_set_thinking_cutoff(spo_dense_verify *verify, uint32_t lane, const spo_thinking_cutoff *cutoff) {
+  return capi::guard([&] {
+    capi::require(verify, "verify");
+    verify->verify->setThinkingCutoff(lane, capi::cutoffOf(cutoff));
   });
 }
 sp_status spo_dense_verify_set_test_children(spo_dense_verify *verify, int on) {

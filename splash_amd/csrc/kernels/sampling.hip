@@ -144,6 +144,42 @@ __global__ __launch_bounds__(64) void decode_sample_count_tokens(uint32_t *__res
 }
 SP_REGISTER_KERNEL("decode_sample_count_tokens", &decode_sample_count_tokens);
 
+// decode_sample_end_thinking: grid (lanes), 64 threads, a thread a row of the lane's block (the reference walks a lane's
+// rows in one thread, sampling.metal:1993-2039; every row reads and writes its own selection only, so they go side by
+// side). The k-th row of a path, ascending, is its row of depth k.
+__global__ __launch_bounds__(64) void decode_sample_end_thinking(const uint32_t *__restrict__ input_tokens,
+                                                                 const uint32_t *__restrict__ token_mask,
+                                                                 const AttentionTreeRow *__restrict__ tree, uint32_t *__restrict__ tokens,
+                                                                 ThinkingCutoffParams p) {
+  const uint32_t lane = blockIdx.x;
+  const SamplingLaneRows block = p.lane[lane];
+  if (threadIdx.x >= block.rows || p.row[lane] >= SAMPLING_MAXIMUM_ROWS) return;
+  const uint32_t mine = block.first + threadIdx.x;
+  const uint32_t path = tree[mine].ancestors, depth = tree[mine].depth;
+  const bool waits = (p.waiting_mask >> lane) & 1u;
+  const uint32_t start = p.tokens[lane][0];
+  // the cut: the first depth from the lane's row on (whose row admits the end's first token, where the end waits)
+  uint32_t cut = 0, left = path;
+  bool found = false;
+  for (; left; left &= left - 1u, ++cut) {
+    if (cut < p.row[lane]) continue;
+    const uint32_t at = block.first + uint32_t(__ffs(int(left)) - 1);
+    if (!waits || ((token_mask[size_t(at) * p.mask_words + start / 32u] >> (start % 32u)) & 1u)) {
+      found = true;
+      break;
+    }
+  }
+  if (!found || cut > depth || depth - cut >= p.count[lane]) return;
+  // thinking that a draft token ended at or before the cut stays ended
+  for (uint32_t before = path & ~1u; before; before &= before - 1u) {
+    const uint32_t at = block.first + uint32_t(__ffs(int(before)) - 1);
+    const uint32_t draft = input_tokens[at];
+    if (tree[at].depth <= cut && (draft == p.close[lane] || draft == p.also_ends[lane])) return;
+  }
+  if (tokens[mine] < p.vocabulary) tokens[mine] = p.tokens[lane][depth - cut];
+}
+SP_REGISTER_KERNEL("decode_sample_end_thinking", &decode_sample_end_thinking);
+
 
 // draft_verify_rows (the layout the reference's sampling.metal:1799-1895 produces): lane l's tree holds sizes[l] rows
 // from row l * 16 of tree_tokens, trees and scores (a row's draft probability and its estimate, the chance that the

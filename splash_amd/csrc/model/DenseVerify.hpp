@@ -7,7 +7,7 @@
 // the step's buffers; the residual stream ping-pongs between two hidden buffers.
 #pragma once
 #include "hip/Backend.hpp"
-#include "model/LanePenalties.hpp"
+#include "model/LanePolicies.hpp"
 #include "ops/Glue.hpp"
 #include "ops/Linear.hpp"
 #include "ops/PagedAttention.hpp"
@@ -15,6 +15,7 @@
 
 #include <array>
 #include <cstdint>
+#include <optional>
 #include <vector>
 
 namespace splash::model {
@@ -85,6 +86,9 @@ public:
   // penalized lane keeps into its row.
   void setPenalties(uint32_t lane, ops::SamplingPenalties penalties) { penalties_.set(lane, penalties); }
   [[nodiscard]] const hip::Buffer &penaltyWords() { return penalties_.words(); }
+  // The thinking cutoff of dispatch lane `lane` for the steps encoded after (ops::ThinkingCutoff; none clears it): its
+  // rows from the cutoff's depth on select the end of thinking, between the step's selection and its acceptance.
+  void setThinkingCutoff(uint32_t lane, std::optional<ops::ThinkingCutoff> cutoff) { penalties_.setCutoff(lane, std::move(cutoff)); }
   void setTestChildren(bool on) { testChildren_ = on; if (on) (void)candidateChildren(0); }
   [[nodiscard]] bool testChildren() const noexcept { return testChildren_; }
   [[nodiscard]] const hip::Buffer &hidden(uint32_t index) const noexcept { return hidden_[index & 1]; }
@@ -151,7 +155,7 @@ private:
   DenseWeights weights_;
   ops::Linear linear_;
   uint32_t maxRows_ = 0, maxLanes_ = 0, rowCapacity_ = 0;
-  LanePenalties penalties_;
+  LanePolicies penalties_;
   uint64_t pageBytes_ = 0, layerBytes_ = 0;
   hip::Buffer kvAll_;
   hip::Buffer hidden_[2], normalized_, qkv_, attention_, intermediate_, logits_, draft_;

@@ -14,7 +14,7 @@
 #pragma once
 #include "hip/Backend.hpp"
 #include "model/DenseVerify.hpp"
-#include "model/LanePenalties.hpp"
+#include "model/LanePolicies.hpp"
 #include "ops/Gdn.hpp"
 #include "ops/Glue.hpp"
 #include "ops/Linear.hpp"
@@ -23,6 +23,7 @@
 #include "ops/Sampling.hpp"
 
 #include <cstdint>
+#include <optional>
 #include <vector>
 
 namespace splash::model {
@@ -149,6 +150,9 @@ public:
   // penalized lane keeps into its row.
   void setPenalties(uint32_t lane, ops::SamplingPenalties penalties) { penalties_.set(lane, penalties); }
   [[nodiscard]] const hip::Buffer &penaltyWords() { return penalties_.words(); }
+  // The thinking cutoff of dispatch lane `lane` for the steps encoded after (ops::ThinkingCutoff; none clears it): its
+  // rows from the cutoff's depth on select the end of thinking, between the step's selection and its acceptance.
+  void setThinkingCutoff(uint32_t lane, std::optional<ops::ThinkingCutoff> cutoff) { penalties_.setCutoff(lane, std::move(cutoff)); }
   // The hidden rows a draft's context is computed from (the reference's QwenTarget addCapture over RowCopy): after
   // layer layers[i] (ascending) every row's output goes to columns [i hidden, (i + 1) hidden) of its row of
   // `destination`, bf16 [rows][layers.size() x hidden], in a step and in a prompt chunk alike. An empty list captures nothing.
@@ -188,7 +192,7 @@ private:
   HybridWeights weights_;
   ops::Linear linear_;
   uint32_t maxRows_ = 0, maxLanes_ = 0, rowCapacity_ = 0;
-  LanePenalties penalties_;
+  LanePolicies penalties_;
   bool tiledGdnHeads_ = false;
   std::vector<uint32_t> captureLayers_;
   hip::Buffer captured_;

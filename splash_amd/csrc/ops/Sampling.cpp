@@ -93,7 +93,10 @@ void Sampling::addVerify(hip::CommandGraph &graph, const SamplingBuffers &b, uin
   graph.add("decode_sample_argmax_sharded", {b.logits, b.partialValues, b.partialIndices}, params, {rows * SAMPLING_SHARDS, 1, 1},
             {SAMPLING_THREADS, 1, 1});
   graph.add("decode_sample_argmax_reduce", {b.partialValues, b.partialIndices, b.tokens}, params, {rows, 1, 1}, {64, 1, 1});
-  if (!params.sampling_mask) return;
+  if (!params.sampling_mask) {
+    addThinkingCutoff(graph, b, vocabulary, lanes, policies);
+    return;
+  }
   graph.add("decode_sample_mass_sharded", {b.logits, b.masses}, params, {rows * SAMPLING_SHARDS, 1, 1}, {SAMPLING_THREADS, 1, 1});
   if (params.truncating_mask)
     graph.add("decode_sample_distribution_end", {b.logits, b.masses, b.decisions}, params, {rows, 1, 1}, {SAMPLING_THREADS, 1, 1});
@@ -109,6 +112,46 @@ void Sampling::addVerify(hip::CommandGraph &graph, const SamplingBuffers &b, uin
   else
     graph.add("decode_sample_draw", {b.logits, b.draftProbabilities, b.masses, b.uniforms, b.ranges, b.decisions, b.tokens}, params,
               {rows, 1, 1}, {64, 1, 1});
+  addThinkingCutoff(graph, b, vocabulary, lanes, policies);
+}
+
+void Sampling::addThinkingCutoff(hip::CommandGraph &graph, const SamplingBuffers &b, uint32_t vocabulary, const std::vector<LaneRows> &lanes,
+                                 const std::vector<SamplingPolicy> &policies) {
+  const uint32_t rows = packedRows(lanes);
+  if (policies.size() != lanes.size()) throw std::invalid_argument("the thinking cutoffs take one policy per lane");
+  ThinkingCutoffParams params{};
+  params.vocabulary = vocabulary;
+  params.lanes = uint32_t(lanes.size());
+  bool any = false;
+  for (size_t l = 0; l < lanes.size(); ++l) {
+    params.lane[l] = {lanes[l].first, lanes[l].rows};
+    const std::optional<ThinkingCutoff> &cutoff = policies[l].thinkingCutoff;
+    params.row[l] = cutoff ? std::min<uint32_t>(cutoff->row, SAMPLING_MAXIMUM_ROWS) : SAMPLING_MAXIMUM_ROWS;
+    if (params.row[l] >= lanes[l].rows) {   // no row of the block lies that deep
+      params.row[l] = SAMPLING_MAXIMUM_ROWS;
+      continue;
+    }
+    if (cutoff->end.empty()) throw std::invalid_argument("a thinking cutoff has an end");
+    if (cutoff->waitsForMask) {
+      if (!policies[l].constrained) throw std::invalid_argument("only a constrained lane's thinking end waits for its mask");
+      if (cutoff->end.front() >= vocabulary) throw std::invalid_argument("a thinking end that waits for a mask starts inside the vocabulary");
+      if (uint64_t{b.maskWords} * 32 < vocabulary) throw std::invalid_argument("a constraint-mask row holds a bit for every token");
+      requireBytes(b.tokenMask, uint64_t{rows} * b.maskWords * 4, "constraint masks");
+      params.waiting_mask |= 1u << l;
+      params.mask_words = b.maskWords;
+    }
+    params.count[l] = uint32_t(std::min<size_t>(cutoff->end.size(), SAMPLING_MAXIMUM_ROWS - params.row[l]));
+    std::copy_n(cutoff->end.begin(), params.count[l], params.tokens[l]);
+    params.close[l] = cutoff->end.back();
+    params.also_ends[l] = cutoff->alsoEnds;
+    any = true;
+  }
+  if (!any) return;
+  requireBytes(b.tokens, uint64_t{rows} * 4, "selected tokens");
+  requireBytes(b.inputTokens, uint64_t{rows} * 4, "input tokens");
+  requireBytes(b.treeRows, uint64_t{rows} * sizeof(AttentionTreeRow), "verify tree rows");
+  graph.add("decode_sample_end_thinking", {b.inputTokens, params.waiting_mask ? b.tokenMask : b.inputTokens, b.treeRows, b.tokens}, params,
+            {params.lanes, 1, 1}, {64, 1, 1});
 }
 
 void Sampling::rebuildPenaltyWords(std::span<uint32_t> words, std::span<const uint32_t> history, uint64_t generatedTokens,

@@ -7,6 +7,7 @@
 #include "abi/Sampling.h"
 #include "hip/Backend.hpp"
 
+#include <algorithm>
 #include <array>
 #include <optional>
 #include <span>
@@ -31,8 +32,24 @@ struct PenaltyTable final {
   std::span<const uint32_t> rows;
 };
 
-// Sampling.hpp:56-83 in the reference; the thinking cutoff belongs to the engine's request handling, not to the verify
-// step, and is not built.
+// Where a lane's thinking budget runs out in a selection (ThinkingCutoff, Sampling.hpp:30-55 in the reference): its
+// selected rows of depth `row` on take the `end` tokens in order, as many as the block holds, unless a draft token on a
+// row's path up to depth `row` is the last of `end`, which closes thinking, or `alsoEnds`: either ended thinking first.
+// An end that waits for the mask of a constrained lane starts instead, along each row's path, at the first of the
+// path's rows from depth `row` on whose mask admits its first token.
+struct ThinkingCutoff final {
+  uint32_t row = 0;
+  std::vector<uint32_t> end;
+  uint32_t alsoEnds = SAMPLING_NO_TOKEN;
+  bool waitsForMask = false;
+  // How many of the lane's proposals, from the first, the end makes (tokens the draft did not propose): the caller
+  // proposes them as a host chain of the lane's tree, so that acceptance keeps them.
+  [[nodiscard]] uint32_t replacedProposals() const noexcept {
+    return row || waitsForMask ? 0u : uint32_t(std::min<size_t>(end.size(), SAMPLING_MAXIMUM_ROWS - 1));
+  }
+};
+
+// Sampling.hpp:56-83 in the reference.
 struct SamplingPolicy final {
   float temperature = 0.0f;
   // A sampling lane keeps the tokens minP leaves it (those that weigh at least minP of the
@@ -47,6 +64,9 @@ struct SamplingPolicy final {
   bool excludesStopTokens = false;
   // Greedy lanes take the argmax of the penalized logits, sampling lanes draw from them.
   SamplingPenalties penalties{};
+  // While the lane thinks under a budget, where that budget runs out; the rows from there on select the end of
+  // thinking whatever their logits.
+  std::optional<ThinkingCutoff> thinkingCutoff{};
   // A lane samples unless it keeps only its most likely token (Sampling.hpp:79-82).
   [[nodiscard]] bool samples() const noexcept { return temperature > 0.0f && minP < 1.0f && topK != 1; }
   [[nodiscard]] bool truncates(uint32_t vocabulary) const noexcept {
@@ -101,6 +121,13 @@ public:
                                                                                        SAMPLING_NO_TOKEN, SAMPLING_NO_TOKEN});
   static void addAcceptance(hip::CommandGraph &graph, const AcceptanceBuffers &buffers, const std::vector<LaneRows> &lanes,
                             const std::vector<uint32_t> &remaining, const std::array<uint32_t, SAMPLING_STOP_TOKENS> &stopTokens);
+
+  // The thinking cutoff of each lane that has one, over the selections addVerify left in buffers.tokens and before
+  // addAcceptance walks them (the end of Sampling::addSelection, Sampling.cpp:314-327; addVerify runs it last). Reads
+  // buffers.inputTokens and buffers.treeRows, and buffers.tokenMask for a lane whose end waits for its mask. Nothing is
+  // dispatched when no lane's cutoff lies inside its block.
+  static void addThinkingCutoff(hip::CommandGraph &graph, const SamplingBuffers &buffers, uint32_t vocabulary,
+                                const std::vector<LaneRows> &lanes, const std::vector<SamplingPolicy> &policies);
 
   // A penalized request's penalty words, rebuilt when it takes a state lane (Sampling::rebuildPenaltyWords,
   // Sampling.cpp:91-114 in the reference): from its history, the prompt and then the `generatedTokens` outputs it

@@ -803,6 +803,23 @@ class Sampling:
                                                  len(lanes)))
         graph._keep.extend([words, tokens, retained])
 
+    @staticmethod
+    def thinking_cutoff(row, end, also_ends=NO_TOKEN, waits_for_mask=False):
+        """A lane's ops::ThinkingCutoff as the C struct; None stands for a lane without one."""
+        end = list(end)
+        return nat.ThinkingCutoff(1, row, len(end), (ctypes.c_uint32 * 16)(*end[:16]), also_ends, int(waits_for_mask))
+
+    @staticmethod
+    def add_thinking_cutoff(graph, input_tokens, tree_rows, tokens, vocabulary, lanes, cutoffs, token_mask=None, mask_words=0):
+        """The thinking cutoffs over add_verify's selections, before add_acceptance: cutoffs: one thinking_cutoff(...) or
+        None a lane."""
+        arr = (nat.LaneRows * len(lanes))(*[nat.LaneRows(*l) for l in lanes])
+        structs = (nat.ThinkingCutoff * len(lanes))(*[c if c is not None else nat.ThinkingCutoff() for c in cutoffs])
+        check(lib.spo_sampling_add_thinking_cutoff(graph.handle, input_tokens.handle, tree_rows.handle, tokens.handle,
+                                                   token_mask.handle if token_mask is not None else None, mask_words, vocabulary, arr,
+                                                   structs, len(lanes)))
+        graph._keep.extend([b for b in (input_tokens, tree_rows, tokens, token_mask) if b is not None])
+
     STATIC_MAXIMUM_ROWS = 256
 
     @staticmethod

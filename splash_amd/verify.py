@@ -81,6 +81,12 @@ class DenseVerify:
         (uint32 [lanes][vocabulary]; ops.Sampling.rebuild_penalty_words makes a row) holds what they read."""
         check(lib.spo_dense_verify_set_penalties(self.handle, lane, repetition, presence, frequency))
 
+    def set_thinking_cutoff(self, lane, row=None, end=(), also_ends=0xFFFFFFFF):
+        """The thinking cutoff of dispatch lane `lane` for the steps encoded after: its rows of depth `row` on select the
+        tokens of `end` in order; row None clears it."""
+        cutoff = None if row is None else ctypes.byref(ops.Sampling.thinking_cutoff(row, end, also_ends))
+        check(lib.spo_dense_verify_set_thinking_cutoff(self.handle, lane, cutoff))
+
     def set_capture(self, layers, destination):
         """After each of `layers` (ascending) every row's output goes to its slot of `destination`, bf16 [rows][len(layers) x hidden]."""
         check(lib.spo_dense_verify_set_capture(self.handle, (ctypes.c_uint32 * max(len(layers), 1))(*layers), len(layers),
@@ -277,6 +283,12 @@ class HybridVerify:
         """The sampling penalties of dispatch lane `lane` for the steps encoded after; its row of the PENALTY_WORDS buffer
         (uint32 [lanes][vocabulary]; ops.Sampling.rebuild_penalty_words makes a row) holds what they read."""
         check(lib.spo_hybrid_verify_set_penalties(self.handle, lane, repetition, presence, frequency))
+
+    def set_thinking_cutoff(self, lane, row=None, end=(), also_ends=0xFFFFFFFF):
+        """The thinking cutoff of dispatch lane `lane` for the steps encoded after: its rows of depth `row` on select the
+        tokens of `end` in order; row None clears it."""
+        cutoff = None if row is None else ctypes.byref(ops.Sampling.thinking_cutoff(row, end, also_ends))
+        check(lib.spo_hybrid_verify_set_thinking_cutoff(self.handle, lane, cutoff))
 
     def set_capture(self, layers, destination):
         """After each of `layers` (ascending) every row's output goes to its slot of `destination`, bf16 [rows][len(layers) x hidden]."""

@@ -263,6 +263,24 @@ def penalize(logits, words, input_tokens, ancestors, repetition=1.0, presence=0.
     return x
 
 
+def thinking_cutoff(selected, input_tokens, tree, vocabulary, row, end, also_ends=NO_TOKEN, admits=None):
+    """One lane's selections under its thinking cutoff; returns the rewritten copy. admits: per row, whether its
+    constraint mask admits end[0] (an end that waits for its mask), or None."""
+    rows = len(tree)
+    nodes = (OrcTreeRow * rows)(*[OrcTreeRow(int(t["ancestors"]), int(t["parent"]), int(t["depth"])) for t in tree])
+    out = np.array(selected, dtype=np.uint32)
+    if row >= rows:
+        return out
+    tok = np.ascontiguousarray(input_tokens, dtype=np.uint32)
+    ends = np.ascontiguousarray(end, dtype=np.uint32)
+    count = min(len(ends), 16 - row)
+    flags = None if admits is None else np.ascontiguousarray(admits, dtype=np.uint8)
+    lib.orc_thinking_cutoff.restype = None
+    lib.orc_thinking_cutoff(_p(out, u32p), _p(tok, u32p), nodes, c_u32(rows), c_u32(vocabulary), c_u32(row), _p(ends, u32p), c_u32(count),
+                            c_u32(int(ends[-1])), c_u32(also_ends), None if flags is None else flags.ctypes.data_as(ctypes.c_void_p))
+    return out
+
+
 def accept_tree(tree, tokens, selected, remaining=0xFFFFFFFF, stop_tokens=()):
     """tree: structured array (ancestors, parent, depth). Returns (kept tokens, accepted, retained_rows)."""
     rows = len(tree)

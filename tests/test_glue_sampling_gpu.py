@@ -464,6 +464,72 @@ def test_penalties_rewrite_the_rows_and_count_what_a_step_keeps(backend):
                                    [(1.5, 0.0, 0.0, 4)] * 4)
 
 
+def test_thinking_cutoffs_rewrite_the_selections(backend):
+    """decode_sample_end_thinking against the oracle over random chains and trees: lanes with and without a cutoff, ends
+    longer than the block, cutoffs below the block, close and also-ends tokens among the drafts (few distinct tokens, so
+    they occur), sentinels among the selections, and ends that wait for their masks. Then through add_verify, whose last
+    dispatch it is: greedy rows select the argmax, the cutoff's rows the end."""
+    from tests.test_oracle_sampling import random_tree
+    print("case sampling thinking cutoff", flush=True)
+    rng = np.random.default_rng(91)
+    V, words = 300, (300 + 31) // 32
+    for trial in range(30):
+        lanes, first, trees = [], 0, []
+        for _ in range(int(rng.integers(1, 9))):
+            n = int(rng.integers(1, 17))
+            lanes.append((first, n)); first += n
+            trees.append(random_tree(rng, n) if trial % 2 else ops.chain_tree_rows([n]))
+        rows = first
+        tree = np.concatenate(trees)
+        drafts = rng.integers(0, 6, rows).astype(np.uint32)
+        picked = rng.integers(100, 200, rows).astype(np.uint32)
+        picked[rng.random(rows) < 0.1] = ops.NO_TOKEN
+        allowed = rng.random((rows, V)) < 0.4
+        bits = np.zeros((rows, words * 32), dtype=np.uint8)
+        bits[:, :V] = allowed
+        mask = np.packbits(bits.reshape(rows, words, 32), axis=2, bitorder="little").view(np.uint32).reshape(rows, words)
+        cutoffs, specs = [], []
+        for f, n in lanes:
+            if rng.random() < 0.25:
+                cutoffs.append(None); specs.append(None)
+                continue
+            spec = dict(row=int(rng.integers(0, 18)), end=[int(t) for t in rng.integers(0, 8, int(rng.integers(1, 17)))],
+                        also_ends=int(rng.integers(0, 8)) if rng.random() < 0.5 else ops.NO_TOKEN, waits_for_mask=bool(rng.random() < 0.4))
+            specs.append(spec)
+            cutoffs.append(ops.Sampling.thinking_cutoff(**spec))
+        tokens = backend.from_array(picked.copy())
+        g = splash_amd.CommandGraph()
+        ops.Sampling.add_thinking_cutoff(g, backend.from_array(drafts), backend.from_array(tree), tokens, V, lanes, cutoffs,
+                                         token_mask=backend.from_array(mask), mask_words=words)
+        backend.run(g)
+        got = tokens.download(np.uint32)
+        for (f, n), spec in zip(lanes, specs):
+            want = picked[f:f + n]
+            if spec is not None:
+                admits = allowed[f:f + n, spec["end"][0]] if spec["waits_for_mask"] else None
+                want = orc.thinking_cutoff(picked[f:f + n], drafts[f:f + n], tree[f:f + n], V, spec["row"], spec["end"], spec["also_ends"],
+                                           admits=admits)
+            assert np.array_equal(got[f:f + n], want), (trial, f, spec)
+    # through add_verify: a greedy lane whose rows from depth 2 on end thinking
+    rows, V = 6, 5000
+    logits = (rng.standard_normal((rows, V)) * 2).astype(np.float32)
+    chain = ops.chain_tree_rows([rows])
+    b = sampling_buffers(backend, rows, V, logits, tokens=np.arange(rows, dtype=np.uint32) + 3000, tree=chain)
+    g = splash_amd.CommandGraph()
+    ops.Sampling.add_verify(g, b, V, V, [(0, rows)], [0.0])
+    ops.Sampling.add_thinking_cutoff(g, b["input_tokens"], b["tree_rows"], b["tokens"], V, [(0, rows)],
+                                     [ops.Sampling.thinking_cutoff(2, [11, 12])])
+    backend.run(g)
+    best = [orc.argmax(row) for row in logits]
+    assert list(b["tokens"].download(np.uint32)) == best[:2] + [11, 12] + best[4:]
+    with pytest.raises(ValueError, match="has an end"):
+        ops.Sampling.add_thinking_cutoff(splash_amd.CommandGraph(), b["input_tokens"], b["tree_rows"], b["tokens"], V, [(0, rows)],
+                                         [ops.Sampling.thinking_cutoff(2, [])])
+    with pytest.raises(ValueError, match="constraint"):
+        ops.Sampling.add_thinking_cutoff(splash_amd.CommandGraph(), b["input_tokens"], b["tree_rows"], b["tokens"], V, [(0, rows)],
+                                         [ops.Sampling.thinking_cutoff(2, [5], waits_for_mask=True)])
+
+
 def test_verify_rows_are_laid_out_from_the_trees(backend):
     """draft_verify_rows (sampling.metal:1799-1895) against the oracle, bit for bit: tokens, tree rows, lane rows and
     sources over random trees, caps, floors and tied estimates; and its outputs are what the acceptance walk reads."""

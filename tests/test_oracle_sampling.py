@@ -450,3 +450,63 @@ def test_penalties_closed_forms():
     # a repetition so small that its inverse overflows: the inverse saturates, the product does too
     out = orc.penalize(probe, words, tokens[:1], chain[:1], repetition=1e-39)
     assert out[0, 3] == np.finfo(np.float32).max
+
+
+def tree_of(parents):
+    tree = np.zeros(len(parents), dtype=orc.TREE_DTYPE)
+    for r, parent in enumerate(parents):
+        tree[r] = ((1 << r) | (0 if parent is None else int(tree[parent]["ancestors"])), 0xFFFF if parent is None else parent,
+                   0 if parent is None else int(tree[parent]["depth"]) + 1)
+    return tree
+
+
+def test_thinking_cutoff_hand_worked():
+    """orc_thinking_cutoff against cases worked by hand from its definition (ThinkingCutoffParams, abi/Sampling.h:147-175
+    in the reference): which rows take which end token, the rows past the end, an end that a draft token on the row's own
+    path already made (at or above the cut, never the anchor's, never a sibling's), the sentinel, and the later start of an
+    end that waits for its mask. Each would fail for an off-by-one in the cut, the depth or the count."""
+    V = 1000
+    chain = tree_of([None, 0, 1, 2, 3, 4])
+    drafts = np.array([50, 51, 52, 53, 54, 55], np.uint32)
+    picked = np.array([100, 101, 102, 103, 104, 105], np.uint32)
+    cut = lambda **kw: list(orc.thinking_cutoff(picked, kw.pop("drafts", drafts), kw.pop("tree", chain), V, **kw))
+    assert cut(row=2, end=[7, 8, 9]) == [100, 101, 7, 8, 9, 105]
+    assert cut(row=0, end=[7]) == [7, 101, 102, 103, 104, 105]
+    assert cut(row=4, end=[7, 8, 9, 10, 11, 12]) == [100, 101, 102, 103, 7, 8]           # as many as the block holds
+    assert cut(row=6, end=[7]) == list(picked) and cut(row=40, end=[7]) == list(picked)  # a cutoff below the block
+    # thinking that the draft ended at or above the cut stays ended: the close token (the end's last) or also_ends
+    with_close = lambda at: np.array([9 if i == at else d for i, d in enumerate(drafts)], np.uint32)
+    assert cut(row=2, end=[7, 8, 9], drafts=with_close(1)) == list(picked)
+    assert cut(row=2, end=[7, 8, 9], drafts=with_close(2)) == list(picked)               # at the cut counts
+    assert cut(row=2, end=[7, 8, 9], drafts=with_close(3)) == [100, 101, 7, 8, 9, 105]   # below the cut does not
+    assert cut(row=2, end=[7, 8, 9], drafts=with_close(0)) == [100, 101, 7, 8, 9, 105]   # the anchor is no draft token
+    assert cut(row=2, end=[7, 8, 9], also_ends=51) == list(picked)
+    assert cut(row=2, end=[7, 8, 9], also_ends=54) == [100, 101, 7, 8, 9, 105]
+    middle = np.array([50, 51, 8, 53, 54, 55], np.uint32)                                # the end's middle token closes nothing
+    assert cut(row=2, end=[7, 8, 9], drafts=middle) == [100, 101, 7, 8, 9, 105]
+    # a row with no selectable logit keeps its sentinel; a token outside the vocabulary likewise
+    holes = np.array([100, 101, 102, orc.NO_TOKEN, V, 105], np.uint32)
+    assert list(orc.thinking_cutoff(holes, drafts, chain, V, 2, [7, 8, 9])) == [100, 101, 7, orc.NO_TOKEN, V, 105]
+    # a tree: depths 0 1 1 2 2 2 3; every path is cut on its own
+    tree = tree_of([None, 0, 0, 1, 2, 2, 4])
+    seven = np.arange(100, 107).astype(np.uint32)
+    tdrafts = np.array([50, 51, 52, 53, 54, 55, 56], np.uint32)
+    assert list(orc.thinking_cutoff(seven, tdrafts, tree, V, 1, [7, 8])) == [100, 7, 7, 8, 8, 8, 106]
+    closed = tdrafts.copy(); closed[1] = 8                                               # row 1 drafted the close token
+    assert list(orc.thinking_cutoff(seven, closed, tree, V, 1, [7, 8])) == [100, 101, 7, 103, 8, 8, 106]
+    closed = tdrafts.copy(); closed[4] = 8                                               # depth 2 is below the cut at depth 1
+    assert list(orc.thinking_cutoff(seven, closed, tree, V, 1, [7, 8])) == [100, 7, 7, 8, 8, 8, 106]
+    assert list(orc.thinking_cutoff(seven, closed, tree, V, 2, [7, 8])) == [100, 101, 102, 7, 104, 7, 106]   # rows 4 and 6 hold it at the cut
+    # an end that waits for its mask starts at the first row from depth `row` on that admits end[0]
+    five, fdrafts = np.arange(100, 105).astype(np.uint32), np.arange(50, 55).astype(np.uint32)
+    short = tree_of([None, 0, 1, 2, 3])
+    waits = lambda admits, row=1: list(orc.thinking_cutoff(five, fdrafts, short, V, row, [7, 8, 9], admits=admits))
+    assert waits([0, 0, 0, 1, 1]) == [100, 101, 102, 7, 8]
+    assert waits([1, 0, 0, 1, 0]) == [100, 101, 102, 7, 8]                               # a row above `row` does not start it
+    assert waits([0, 1, 0, 0, 0]) == [100, 7, 8, 9, 104]
+    assert waits([0, 0, 0, 0, 0]) == list(five)
+    assert waits([1, 1, 1, 1, 1], row=0) == [7, 8, 9, 103, 104]
+    # a draft token ends thinking up to the later cut too
+    late = fdrafts.copy(); late[2] = 9
+    assert list(orc.thinking_cutoff(five, late, short, V, 1, [7, 8, 9], admits=[0, 0, 0, 1, 1])) == list(five)          # depth 2 <= cut 3
+    assert list(orc.thinking_cutoff(five, late, short, V, 1, [7, 8, 9], admits=[0, 1, 1, 1, 1])) == [100, 7, 8, 9, 104]  # depth 2 > cut 1

@@ -276,12 +276,26 @@ def test_a_penalized_lane_selects_from_its_penalized_rows(backend):
     want_words = words.copy()
     np.add.at(want_words, kept, 1)
     assert np.array_equal(counted[1], want_words) and not counted[0].any()
+    # a thinking cutoff on the other lane: its rows from depth 2 on select the end, whatever their logits; the acceptance
+    # walks those selections
+    gpu.set_thinking_cutoff(0, row=2, end=[17, 18, 19])
+    lanes = make_lanes()
+    gpu.set_block(lanes, tokens, tree_rows=tree)
+    graph = gpu.encode(lanes, commit=False)
+    assert "decode_sample_end_thinking" in graph.kernels()
+    backend.run(graph)
+    ended = np.array([orc.argmax(row) for row in plain[:6]], np.uint32)
+    ended[2:5] = [17, 18, 19]
+    kept0, accepted0, mask0 = orc.accept_tree(tree[:6], tokens[:6], ended)
+    got_tokens, got_retained, got_accepted, got_mask = (np.array(a).copy() for a in gpu.results(lanes))
+    assert np.array_equal(got_tokens[:len(kept0)], kept0) and (got_retained[0], got_accepted[0], got_mask[0]) == (len(kept0), accepted0, mask0)
+    gpu.set_thinking_cutoff(0)
     # penalties off again: the step is the plain one
     gpu.set_penalties(1)
     lanes = make_lanes()
     gpu.set_block(lanes, tokens, tree_rows=tree)
     graph = gpu.encode(lanes, commit=False)
-    assert "decode_sample_penalize" not in graph.kernels()
+    assert "decode_sample_penalize" not in graph.kernels() and "decode_sample_end_thinking" not in graph.kernels()
     backend.run(graph)
     assert logits_of().tobytes() == plain.tobytes()
 
