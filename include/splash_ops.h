@@ -693,7 +693,10 @@ typedef enum spo_verify_buffer {
   SPO_VERIFY_CANDIDATE_CHILDREN = 18,
   /* the penalty table: uint32 [max lanes][vocabulary] in device memory, lane l's row at words l x vocabulary on
      (spo_sampling_rebuild_penalty_words makes a row); allocated, zeroed, by the first call or by set_penalties */
-  SPO_VERIFY_PENALTY_WORDS = 19
+  SPO_VERIFY_PENALTY_WORDS = 19,
+  /* the constraint masks of constrained lanes: uint32 [max rows][ceil(vocabulary / 32)] in device memory, bit t % 32 of
+     word t / 32 of a packed row admits token t; allocated by the first call */
+  SPO_VERIFY_TOKEN_MASK = 20
 } spo_verify_buffer;
 sp_status spo_dense_verify_buffer(spo_dense_verify *verify, spo_verify_buffer which, uint32_t index, sp_buffer **out);
 /* The sampling penalties of dispatch lane `lane` (SamplingPolicy::penalties, Sampling.hpp:71 in the reference) for the
@@ -701,9 +704,15 @@ sp_status spo_dense_verify_buffer(spo_dense_verify *verify, spo_verify_buffer wh
  * step selects (spo_sampling_add_penalties), and a step that commits counts the tokens the lane keeps into that row
  * (spo_sampling_add_penalty_count). 1, 0, 0 turns them off. */
 sp_status spo_dense_verify_set_penalties(spo_dense_verify *verify, uint32_t lane, float repetition, float presence, float frequency);
+/* SamplingPolicy::constrained and ::excludesStopTokens of dispatch lane `lane` (Sampling.hpp:66-70) for the steps
+ * encoded after: a constrained lane's rows admit only the tokens of their rows of SPO_VERIFY_TOKEN_MASK; a lane that
+ * excludes stop tokens never selects one. */
+sp_status spo_dense_verify_set_admission(spo_dense_verify *verify, uint32_t lane, uint32_t constrained, uint32_t excludes_stop_tokens);
+/* The stop tokens of the steps encoded after (StopTokens of Sampling::addVerify / addAcceptance): four ids, 0xFFFFFFFF
+ * for none; NULL for none at all. Acceptance ends a lane's path at one. */
+sp_status spo_dense_verify_set_stop_tokens(spo_dense_verify *verify, const uint32_t *stop_tokens);
 /* The thinking cutoff of dispatch lane `lane` (SamplingPolicy::thinkingCutoff, Sampling.hpp:76) for the steps encoded
- * after; NULL, or active 0, clears it. The drivers' lanes are not constrained, so an end that waits for a mask is refused
- * when the step is encoded. */
+ * after; NULL, or active 0, clears it. An end that waits for its mask needs a constrained lane (set_admission). */
 sp_status spo_dense_verify_set_thinking_cutoff(spo_dense_verify *verify, uint32_t lane, const spo_thinking_cutoff *cutoff);
 uint64_t spo_dense_verify_page_bytes(const spo_dense_verify *verify);
 /* Algorithmic HBM bytes of one step: weights once, each lane's KV, logits written and read. */
@@ -810,7 +819,9 @@ sp_status spo_hybrid_verify_set_capture(spo_hybrid_verify *verify, const uint32_
 sp_status spo_hybrid_verify_buffer(spo_hybrid_verify *verify, uint32_t which, uint32_t index, sp_buffer **out);
 /* As spo_dense_verify_set_penalties. */
 sp_status spo_hybrid_verify_set_penalties(spo_hybrid_verify *verify, uint32_t lane, float repetition, float presence, float frequency);
-/* As spo_dense_verify_set_thinking_cutoff. */
+/* As spo_dense_verify_set_admission, _set_stop_tokens and _set_thinking_cutoff. */
+sp_status spo_hybrid_verify_set_admission(spo_hybrid_verify *verify, uint32_t lane, uint32_t constrained, uint32_t excludes_stop_tokens);
+sp_status spo_hybrid_verify_set_stop_tokens(spo_hybrid_verify *verify, const uint32_t *stop_tokens);
 sp_status spo_hybrid_verify_set_thinking_cutoff(spo_hybrid_verify *verify, uint32_t lane, const spo_thinking_cutoff *cutoff);
 /* HybridVerify::encodePrefill: a chunk of `tokens` prompt tokens of the sequence of lane `lane` (its pages from table_first,
  * `committed` tokens cached; inputs as spo_dense_verify_encode_prefill's) through layers [first_layer, first_layer +

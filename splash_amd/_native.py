@@ -350,6 +350,10 @@ _sig("spo_dflash_draft_encode_context_commit", c_int, c_p, c_p, c_p, c_p, P(c_u3
 _sig("spo_sampling_add_acceptance", c_int, c_p, c_p, c_p, c_p, c_p, c_p, c_p, P(LaneRows), P(c_u32), c_u32, P(c_u32))
 _sig("spo_dense_verify_set_penalties", c_int, c_p, c_u32, ctypes.c_float, ctypes.c_float, ctypes.c_float)
 _sig("spo_hybrid_verify_set_penalties", c_int, c_p, c_u32, ctypes.c_float, ctypes.c_float, ctypes.c_float)
+_sig("spo_dense_verify_set_admission", c_int, c_p, c_u32, c_u32, c_u32)
+_sig("spo_hybrid_verify_set_admission", c_int, c_p, c_u32, c_u32, c_u32)
+_sig("spo_dense_verify_set_stop_tokens", c_int, c_p, P(c_u32))
+_sig("spo_hybrid_verify_set_stop_tokens", c_int, c_p, P(c_u32))
 _sig("spo_dense_verify_set_thinking_cutoff", c_int, c_p, c_u32, P(ThinkingCutoff))
 _sig("spo_hybrid_verify_set_thinking_cutoff", c_int, c_p, c_u32, P(ThinkingCutoff))
 _sig("spo_sampling_rebuild_penalty_words", c_int, c_p, c_u32, c_p, ctypes.c_uint64, ctypes.c_uint64, c_u32, c_u32)

@@ -8,6 +8,7 @@
 #include "splash_gguf.h"
 #include "model/StepResults.hpp"
 
+#include <array>
 #include <memory>
 
 using namespace splash;
@@ -86,6 +87,20 @@ sp_status spo_hybrid_verify_set_penalties(spo_hybrid_verify *verify, uint32_t la
   });
 }
 
+sp_status spo_hybrid_verify_set_admission(spo_hybrid_verify *verify, uint32_t lane, uint32_t constrained, uint32_t excludes_stop_tokens) {
+  return capi::guard([&] {
+    capi::require(verify, "verify");
+    verify->verify->setAdmission(lane, constrained != 0, excludes_stop_tokens != 0);
+  });
+}
+sp_status spo_hybrid_verify_set_stop_tokens(spo_hybrid_verify *verify, const uint32_t *stop_tokens) {
+  return capi::guard([&] {
+    capi::require(verify, "verify");
+    std::array<uint32_t, SAMPLING_STOP_TOKENS> stops{SAMPLING_NO_TOKEN, SAMPLING_NO_TOKEN, SAMPLING_NO_TOKEN, SAMPLING_NO_TOKEN};
+    if (stop_tokens) for (size_t i = 0; i < stops.size(); ++i) stops[i] = stop_tokens[i];
+    verify->verify->setStopTokens(stops);
+  });
+}
 sp_status spo_hybrid_verify_set_thinking_cutoff(spo_hybrid_verify *verify, uint32_t lane, const spo_thinking_cutoff *cutoff) {
   return capi::guard([&] {
     capi::require(verify, "verify");
@@ -202,6 +217,7 @@ sp_status spo_hybrid_verify_buffer(spo_hybrid_verify *verify, uint32_t which, ui
     case SPO_VERIFY_DRAFT_PROBABILITIES: b = v.draftProbabilities(); break;
     case SPO_VERIFY_HIDDEN: b = v.hidden(index); break;
     case SPO_VERIFY_PENALTY_WORDS: b = v.penaltyWords(); break;
+    case SPO_VERIFY_TOKEN_MASK: b = v.tokenMask(); break;
     case SPO_VERIFY_GDN_STATES: b = v.gdnStates(); break;
     case SPO_VERIFY_GDN_TAPE: b = v.gdnTape(); break;
     default: throw std::invalid_argument("no such verify buffer");

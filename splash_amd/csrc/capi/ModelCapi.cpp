@@ -11,6 +11,7 @@
 #include "ops/Glue.hpp"
 #include "ops/Sampling.hpp"
 
+#include <array>
 #include <memory>
 
 using namespace splash;
@@ -375,6 +376,7 @@ sp_status spo_dense_verify_buffer(spo_dense_verify *verify, spo_verify_buffer wh
     case SPO_VERIFY_FFN_ROWS: b = v.ffnRows(); break;
     case SPO_VERIFY_CANDIDATE_CHILDREN: b = v.candidateChildren(index); break;
     case SPO_VERIFY_PENALTY_WORDS: b = v.penaltyWords(); break;
+    case SPO_VERIFY_TOKEN_MASK: b = v.tokenMask(); break;
     default: throw std::invalid_argument("no such verify buffer");
     }
     sp_buffer_retain(b.handle());
@@ -420,6 +422,20 @@ sp_status spo_dense_verify_set_penalties(spo_dense_verify *verify, uint32_t lane
   return capi::guard([&] {
     capi::require(verify, "verify");
     verify->verify->setPenalties(lane, {repetition, presence, frequency});
+  });
+}
+sp_status spo_dense_verify_set_admission(spo_dense_verify *verify, uint32_t lane, uint32_t constrained, uint32_t excludes_stop_tokens) {
+  return capi::guard([&] {
+    capi::require(verify, "verify");
+    verify->verify->setAdmission(lane, constrained != 0, excludes_stop_tokens != 0);
+  });
+}
+sp_status spo_dense_verify_set_stop_tokens(spo_dense_verify *verify, const uint32_t *stop_tokens) {
+  return capi::guard([&] {
+    capi::require(verify, "verify");
+    std::array<uint32_t, SAMPLING_STOP_TOKENS> stops{SAMPLING_NO_TOKEN, SAMPLING_NO_TOKEN, SAMPLING_NO_TOKEN, SAMPLING_NO_TOKEN};
+    if (stop_tokens) for (size_t i = 0; i < stops.size(); ++i) stops[i] = stop_tokens[i];
+    verify->verify->setStopTokens(stops);
   });
 }
 sp_status spo_dense_verify_set_thinking_cutoff(spo_dense_verify *verify, uint32_t lane, const spo_thinking_cutoff *cutoff) {

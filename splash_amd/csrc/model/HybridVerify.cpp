@@ -353,11 +353,15 @@ void HybridVerify::encode(hip::CommandGraph &graph, const std::vector<HybridLane
   encodeHead(graph, rows, feeds);
   // a lane's penalties rewrite its rows of the head's fresh logits before anything selects from them
   const bool penalized = penalties_.apply(policies);
-  if (penalized) ops::Sampling::addPenalties(graph, sampling_, dims_.vocabulary, dims_.vocabulary, laneRows, policies, penalties_.table());
-  ops::Sampling::addVerify(graph, sampling_, dims_.vocabulary, dims_.vocabulary, laneRows, policies);
+  ops::SamplingBuffers selection = sampling_;
+  if (penalties_.anyConstrained(lanes.size())) {
+    selection.tokenMask = penalties_.tokenMask(maxRows_);
+    selection.maskWords = penalties_.maskWords();
+  }
+  if (penalized) ops::Sampling::addPenalties(graph, selection, dims_.vocabulary, dims_.vocabulary, laneRows, policies, penalties_.table());
+  ops::Sampling::addVerify(graph, selection, dims_.vocabulary, dims_.vocabulary, laneRows, policies, penalties_.stopTokens());
   const ops::AcceptanceBuffers acceptance{inputTokens_, treeRows_, tokens_, retained_, acceptedCount_, retainedRows_};
-  ops::Sampling::addAcceptance(graph, acceptance, laneRows, remaining,
-                               {SAMPLING_NO_TOKEN, SAMPLING_NO_TOKEN, SAMPLING_NO_TOKEN, SAMPLING_NO_TOKEN});
+  ops::Sampling::addAcceptance(graph, acceptance, laneRows, remaining, penalties_.stopTokens());
   // a step that commits counts the tokens its penalized lanes keep, for the next step's penalties
   if (penalized && commit)
     ops::Sampling::addPenaltyCount(graph, acceptance, dims_.vocabulary, laneRows, penalties_.active(lanes.size()), penalties_.table());

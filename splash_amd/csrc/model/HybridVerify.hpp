@@ -22,6 +22,7 @@
 #include "ops/PagedAttention.hpp"
 #include "ops/Sampling.hpp"
 
+#include <array>
 #include <cstdint>
 #include <optional>
 #include <vector>
@@ -150,6 +151,12 @@ public:
   // penalized lane keeps into its row.
   void setPenalties(uint32_t lane, ops::SamplingPenalties penalties) { penalties_.set(lane, penalties); }
   [[nodiscard]] const hip::Buffer &penaltyWords() { return penalties_.words(); }
+  // Dispatch lane `lane` of the steps encoded after admits only the tokens of its rows of tokenMask() (constrained), never
+  // selects a stop token (excludesStopTokens); the step's stop tokens (SAMPLING_NO_TOKEN for none), at which acceptance
+  // ends a lane's path (SamplingPolicy::constrained / excludesStopTokens, StopTokens in the reference's Sampling.hpp).
+  void setAdmission(uint32_t lane, bool constrained, bool excludesStopTokens) { penalties_.setAdmission(lane, constrained, excludesStopTokens); }
+  void setStopTokens(const std::array<uint32_t, SAMPLING_STOP_TOKENS> &tokens) noexcept { penalties_.setStopTokens(tokens); }
+  [[nodiscard]] const hip::Buffer &tokenMask() { return penalties_.tokenMask(maxRows_); }
   // The thinking cutoff of dispatch lane `lane` for the steps encoded after (ops::ThinkingCutoff; none clears it): its
   // rows from the cutoff's depth on select the end of thinking, between the step's selection and its acceptance.
   void setThinkingCutoff(uint32_t lane, std::optional<ops::ThinkingCutoff> cutoff) { penalties_.setCutoff(lane, std::move(cutoff)); }

@@ -1,11 +1,13 @@
 // What a driver's lanes add to their sampling policies between steps: each dispatch lane's thinking cutoff
-// (ops::ThinkingCutoff), its penalties (ops::SamplingPenalties) and its row of the penalty table the driver owns, `vocabulary` words a lane in device memory, allocated (zeroed) when a lane first takes
-// active penalties. The reference's model keeps the table per state lane and the engine counts a step's tokens into it
+// (ops::ThinkingCutoff), whether it is constrained by its rows of the token mask and whether it ignores end-of-sequence,
+// the step's stop tokens, the lane's penalties (ops::SamplingPenalties) and its row of the penalty table the driver owns,
+// `vocabulary` words a lane in device memory, allocated (zeroed) when a lane first takes active penalties. The reference's model keeps the table per state lane and the engine counts a step's tokens into it
 // on the host (Sampling.hpp:85-91, Sampling::countPenaltyTokens); here a step that commits counts them on the device.
 #pragma once
 #include "hip/Backend.hpp"
 #include "ops/Sampling.hpp"
 
+#include <array>
 #include <numeric>
 #include <optional>
 #include <stdexcept>
@@ -15,9 +17,32 @@ namespace splash::model {
 
 class LanePolicies final {
 public:
+  using StopTokens = std::array<uint32_t, SAMPLING_STOP_TOKENS>;
   LanePolicies(hip::Backend &backend, uint32_t lanes, uint32_t vocabulary)
-      : backend_(backend), vocabulary_(vocabulary), penalties_(lanes), cutoffs_(lanes), rows_(lanes) {
+      : backend_(backend), vocabulary_(vocabulary), penalties_(lanes), cutoffs_(lanes), constrained_(lanes), excludesStop_(lanes),
+        rows_(lanes) {
     std::iota(rows_.begin(), rows_.end(), 0u);
+    stopTokens_.fill(SAMPLING_NO_TOKEN);
+  }
+  // The lane's rows admit only the tokens of their rows of tokenMask(); the lane never selects a stop token.
+  void setAdmission(uint32_t lane, bool constrained, bool excludesStopTokens) {
+    if (lane >= constrained_.size()) throw std::invalid_argument("the admission of a lane past the driver's");
+    constrained_[lane] = constrained;
+    excludesStop_[lane] = excludesStopTokens;
+  }
+  // The tokens that end a sequence: acceptance keeps nothing past one, and a lane that ignores them never selects one.
+  void setStopTokens(const StopTokens &tokens) noexcept { stopTokens_ = tokens; }
+  [[nodiscard]] const StopTokens &stopTokens() const noexcept { return stopTokens_; }
+  [[nodiscard]] uint32_t maskWords() const noexcept { return (vocabulary_ + 31) / 32; }
+  // The constraint masks: uint32 [rows][maskWords()], bit t % 32 of word t / 32 of a packed row admits token t.
+  const hip::Buffer &tokenMask(uint32_t rows) {
+    if (!tokenMask_) tokenMask_ = backend_.allocateBuffer(uint64_t{rows} * maskWords() * 4, hip::BufferStorage::Private, "token masks");
+    return tokenMask_;
+  }
+  [[nodiscard]] bool anyConstrained(size_t lanes) const {
+    for (size_t l = 0; l < lanes && l < constrained_.size(); ++l)
+      if (constrained_[l]) return true;
+    return false;
   }
   void set(uint32_t lane, ops::SamplingPenalties penalties) {
     if (lane >= penalties_.size()) throw std::invalid_argument("penalties of a lane past the driver's");
@@ -39,6 +64,8 @@ public:
     bool any = false;
     for (size_t l = 0; l < policies.size() && l < penalties_.size(); ++l) {
       policies[l].thinkingCutoff = cutoffs_[l];
+      policies[l].constrained = constrained_[l];
+      policies[l].excludesStopTokens = excludesStop_[l];
       policies[l].penalties = penalties_[l];
       any = any || penalties_[l].active();
     }
@@ -56,8 +83,10 @@ private:
   uint32_t vocabulary_;
   std::vector<ops::SamplingPenalties> penalties_;
   std::vector<std::optional<ops::ThinkingCutoff>> cutoffs_;
+  std::vector<bool> constrained_, excludesStop_;
+  StopTokens stopTokens_{};
   std::vector<uint32_t> rows_;
-  hip::Buffer words_;
+  hip::Buffer words_, tokenMask_;
 };
 
 } // namespace splash::model

@@ -11,7 +11,7 @@ from .backend import Buffer, CommandGraph, STORAGE_PRIVATE
 from . import ops
 
 (INPUT_TOKENS, TREE_ROWS, DEPTHS, UNIFORMS, TOKENS, RETAINED, ACCEPTED, RETAINED_ROWS, PAGE_TABLE, KV_POOL, LOGITS,
- DRAFT_PROBABILITIES, HIDDEN, GDN_STATES, GDN_TAPE, QKV_ROWS, ATTENTION_ROWS, FFN_ROWS, CANDIDATE_CHILDREN, PENALTY_WORDS) = range(20)
+ DRAFT_PROBABILITIES, HIDDEN, GDN_STATES, GDN_TAPE, QKV_ROWS, ATTENTION_ROWS, FFN_ROWS, CANDIDATE_CHILDREN, PENALTY_WORDS, TOKEN_MASK) = range(21)
 
 
 class Lane:
@@ -81,10 +81,20 @@ class DenseVerify:
         (uint32 [lanes][vocabulary]; ops.Sampling.rebuild_penalty_words makes a row) holds what they read."""
         check(lib.spo_dense_verify_set_penalties(self.handle, lane, repetition, presence, frequency))
 
-    def set_thinking_cutoff(self, lane, row=None, end=(), also_ends=0xFFFFFFFF):
+    def set_admission(self, lane, constrained=False, excludes_stop_tokens=False):
+        """Dispatch lane `lane` of the steps encoded after admits only the tokens of its rows of the TOKEN_MASK buffer
+        (uint32 [rows][ceil(vocabulary / 32)]) and / or never selects a stop token."""
+        check(lib.spo_dense_verify_set_admission(self.handle, lane, int(constrained), int(excludes_stop_tokens)))
+
+    def set_stop_tokens(self, stop_tokens=()):
+        """Up to four tokens that end a sequence, for the steps encoded after."""
+        stops = (ctypes.c_uint32 * 4)(*(list(stop_tokens) + [0xFFFFFFFF] * 4)[:4])
+        check(lib.spo_dense_verify_set_stop_tokens(self.handle, stops))
+
+    def set_thinking_cutoff(self, lane, row=None, end=(), also_ends=0xFFFFFFFF, waits_for_mask=False):
         """The thinking cutoff of dispatch lane `lane` for the steps encoded after: its rows of depth `row` on select the
         tokens of `end` in order; row None clears it."""
-        cutoff = None if row is None else ctypes.byref(ops.Sampling.thinking_cutoff(row, end, also_ends))
+        cutoff = None if row is None else ctypes.byref(ops.Sampling.thinking_cutoff(row, end, also_ends, waits_for_mask))
         check(lib.spo_dense_verify_set_thinking_cutoff(self.handle, lane, cutoff))
 
     def set_capture(self, layers, destination):
@@ -284,10 +294,20 @@ class HybridVerify:
         (uint32 [lanes][vocabulary]; ops.Sampling.rebuild_penalty_words makes a row) holds what they read."""
         check(lib.spo_hybrid_verify_set_penalties(self.handle, lane, repetition, presence, frequency))
 
-    def set_thinking_cutoff(self, lane, row=None, end=(), also_ends=0xFFFFFFFF):
+    def set_admission(self, lane, constrained=False, excludes_stop_tokens=False):
+        """Dispatch lane `lane` of the steps encoded after admits only the tokens of its rows of the TOKEN_MASK buffer
+        (uint32 [rows][ceil(vocabulary / 32)]) and / or never selects a stop token."""
+        check(lib.spo_hybrid_verify_set_admission(self.handle, lane, int(constrained), int(excludes_stop_tokens)))
+
+    def set_stop_tokens(self, stop_tokens=()):
+        """Up to four tokens that end a sequence, for the steps encoded after."""
+        stops = (ctypes.c_uint32 * 4)(*(list(stop_tokens) + [0xFFFFFFFF] * 4)[:4])
+        check(lib.spo_hybrid_verify_set_stop_tokens(self.handle, stops))
+
+    def set_thinking_cutoff(self, lane, row=None, end=(), also_ends=0xFFFFFFFF, waits_for_mask=False):
         """The thinking cutoff of dispatch lane `lane` for the steps encoded after: its rows of depth `row` on select the
         tokens of `end` in order; row None clears it."""
-        cutoff = None if row is None else ctypes.byref(ops.Sampling.thinking_cutoff(row, end, also_ends))
+        cutoff = None if row is None else ctypes.byref(ops.Sampling.thinking_cutoff(row, end, also_ends, waits_for_mask))
         check(lib.spo_hybrid_verify_set_thinking_cutoff(self.handle, lane, cutoff))
 
     def set_capture(self, layers, destination):

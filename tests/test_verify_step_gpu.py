@@ -300,6 +300,86 @@ def test_a_penalized_lane_selects_from_its_penalized_rows(backend):
     assert logits_of().tobytes() == plain.tobytes()
 
 
+def test_admission_and_stop_tokens_through_the_driver(backend):
+    """SamplingPolicy::constrained / excludesStopTokens and the step's stop tokens through the driver: a constrained lane
+    selects, row by row, the best token its mask row admits; a lane that ignores end-of-sequence never selects a stop
+    token; acceptance ends a path at a stop token it accepts; and a thinking end that waits for its mask starts at the
+    first row whose mask admits it. Against the oracle's argmax and walk over the plain step's logits."""
+    print("case config 1 admission and stop tokens", flush=True)
+    from splash_amd import ops
+    V = 4096
+    model = DenseModel(seed=23, hidden=512, q_heads=8, kv_heads=4, head_dim=64, ffn=1024, vocabulary=V, layers=2)
+    rng = np.random.default_rng(4)
+    context = 50
+    gpu = model.build_gpu(backend, max_lanes=2, context_tokens=context + 16)
+    make_lanes = lambda: [verify.Lane(5, context, table_first=model.table_first[0]), verify.Lane(8, context, table_first=model.table_first[1])]
+    lanes = make_lanes()
+    model.seed_context(gpu, None, rng)
+    tokens = rng.integers(0, V, 13).astype(np.uint32)
+    tree = ops.chain_tree_rows([5, 8])
+    gpu.set_block(lanes, tokens, tree_rows=tree)
+    backend.run(gpu.encode(lanes, commit=False))
+    plain = gpu.buffer(verify.LOGITS).download(np.float32, 13 * V).reshape(13, V)
+    best = np.argmax(plain, axis=1).astype(np.uint32)
+    # lane 0 constrained: its masks forbid each row's favourite; lane 1: its favourites of rows 0 and 2 are stop tokens
+    words = (V + 31) // 32
+    allowed = rng.random((13, V)) < 0.5
+    allowed[np.arange(13), best] = False
+    end_first = 777
+    allowed[:5, end_first] = [False, False, False, True, True]
+    mask = np.packbits(allowed.reshape(13, words, 32), axis=2, bitorder="little").view(np.uint32).reshape(13, words)
+    gpu.buffer(verify.TOKEN_MASK).upload(mask)
+    # lane 1's draft follows its own greedy continuation for three rows, so that the walk reaches a stop token
+    for r in range(3):
+        tokens[6 + r] = best[5 + r]
+        gpu.set_block(lanes, tokens, tree_rows=tree)
+        backend.run(gpu.encode(lanes, commit=False))
+        plain = gpu.buffer(verify.LOGITS).download(np.float32, 13 * V).reshape(13, V)
+        best = np.argmax(plain, axis=1).astype(np.uint32)
+    stops = [int(best[7]), 4095]
+    gpu.set_admission(0, constrained=True)
+    gpu.set_stop_tokens(stops)
+    lanes = make_lanes()
+    gpu.set_block(lanes, tokens, tree_rows=tree)
+    graph = gpu.encode(lanes, commit=False)
+    assert "decode_sample_admit" in graph.kernels()
+    backend.run(graph)
+    got_tokens, got_retained, got_accepted, got_mask = (np.array(a).copy() for a in gpu.results(lanes))
+    want0 = np.array([orc.argmax(np.where(allowed[r], plain[r], -np.inf)) for r in range(5)], np.uint32)
+    assert np.all(want0 != best[:5])
+    kept, accepted, path = orc.accept_tree(tree[:5], tokens[:5], want0, stop_tokens=stops)
+    assert np.array_equal(got_tokens[:len(kept)], kept) and (got_retained[0], got_accepted[0], got_mask[0]) == (len(kept), accepted, path)
+    # lane 1 does not exclude stop tokens: its walk accepts up to the stop token its row 2 selects and ends there
+    kept, accepted, path = orc.accept_tree(tree[5:], tokens[5:], best[5:], stop_tokens=stops)
+    assert len(kept) == 3 and kept[-1] == stops[0]
+    assert np.array_equal(got_tokens[5:5 + len(kept)], kept) and (got_retained[1], got_accepted[1], got_mask[1]) == (len(kept), accepted, path)
+    # excluding them, the lane selects its next best there and walks on
+    gpu.set_admission(1, excludes_stop_tokens=True)
+    lanes = make_lanes()
+    gpu.set_block(lanes, tokens, tree_rows=tree)
+    backend.run(gpu.encode(lanes, commit=False))
+    got_tokens, got_retained, got_accepted, got_mask = (np.array(a).copy() for a in gpu.results(lanes))
+    without = plain[5:].copy()
+    without[:, stops] = -np.inf
+    want1 = np.array([orc.argmax(row) for row in without], np.uint32)
+    kept, accepted, path = orc.accept_tree(tree[5:], tokens[5:], want1, stop_tokens=stops)
+    assert stops[0] not in kept
+    assert np.array_equal(got_tokens[5:5 + len(kept)], kept) and (got_retained[1], got_accepted[1], got_mask[1]) == (len(kept), accepted, path)
+    # the constrained lane's thinking end waits for its mask: rows 3 and 4 admit its first token
+    gpu.set_thinking_cutoff(0, row=1, end=[end_first, 778], waits_for_mask=True)
+    lanes = make_lanes()
+    gpu.set_block(lanes, tokens, tree_rows=tree)
+    backend.run(gpu.encode(lanes, commit=False))
+    ended = orc.thinking_cutoff(want0, tokens[:5], tree[:5], V, 1, [end_first, 778], admits=allowed[:5, end_first])
+    assert list(ended[3:]) == [end_first, 778] and np.array_equal(ended[:3], want0[:3])
+    kept, accepted, path = orc.accept_tree(tree[:5], tokens[:5], ended, stop_tokens=stops)
+    got_tokens, got_retained, got_accepted, got_mask = (np.array(a).copy() for a in gpu.results(lanes))
+    assert np.array_equal(got_tokens[:len(kept)], kept) and (got_retained[0], got_accepted[0], got_mask[0]) == (len(kept), accepted, path)
+    gpu.set_admission(0)
+    with pytest.raises(ValueError, match="constrained"):
+        gpu.encode(make_lanes(), commit=False)                        # an end that waits needs a constrained lane
+
+
 @pytest.mark.parametrize("lanes_rows", [[16], [7, 16, 3]])
 def test_chained_projections_change_nothing(backend, lanes_rows):
     """A step whose layers dispatch their four projections after the attention as one chain (a layer's output, gate/up
