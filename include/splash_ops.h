@@ -32,6 +32,22 @@ sp_status spo_graph_submit(sp_backend *backend, const spo_graph *graph, sp_ticke
 /* The graph recorded for replay (sp_command_create). */
 sp_status spo_graph_record(sp_backend *backend, const spo_graph *graph, sp_command **out);
 
+/* ---- prompt lookup (model::LookupIndex, runtime/model/LookupProposals.hpp:17-105): host code ----
+ * A request's tokens (its prompt, then every token its decode selects) and, after the latest, the match: the longest
+ * suffix, counted up to 64 tokens and none shorter than 3, that also ends at an earlier token, at its most recent such
+ * end. The tokens that followed it there are the lane's host chain (spo_draft_tree_lane.chain_tokens). */
+typedef struct spo_lookup_index spo_lookup_index;
+sp_status spo_lookup_index_create(spo_lookup_index **out);
+void spo_lookup_index_destroy(spo_lookup_index *index);
+sp_status spo_lookup_index_append(spo_lookup_index *index, const uint32_t *tokens, uint64_t count);
+/* length 0: no match; end: the index of the earlier occurrence's last token. */
+sp_status spo_lookup_index_match(const spo_lookup_index *index, uint32_t *length, uint32_t *end);
+/* Up to `count` tokens that followed the match, at most as far as the latest token, into `out`; returns how many. */
+uint32_t spo_lookup_index_proposals(const spo_lookup_index *index, uint32_t count, uint32_t *out);
+/* LookupAgreement of a lookup token `depth` positions past the anchor with the draft's candidates (per_position a
+ * position, most likely first, `positions` positions): 0 the most likely, 1 another candidate, 2 none, 3 not known. */
+uint32_t spo_lookup_agreement(uint32_t token, uint32_t depth, const uint32_t *candidates, uint32_t positions, uint32_t per_position);
+
 /* ---- weight image (load-time repack: runtime/model/GgufPreparation.cpp, gguf_repack.metal) ---- */
 uint64_t spo_gguf_image_bytes(uint32_t format, uint32_t rows, uint32_t input_size);
 uint64_t spo_gguf_table_bytes(uint32_t input_size, uint32_t rows);

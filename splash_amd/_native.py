@@ -360,6 +360,12 @@ _sig("spo_sampling_rebuild_penalty_words", c_int, c_p, c_u32, c_p, ctypes.c_uint
 _sig("spo_sampling_add_penalties", c_int, c_p, c_p, c_p, c_p, c_p, c_u32, c_u32, P(LaneRows), P(SamplingPenalties), c_u32)
 _sig("spo_sampling_add_penalty_count", c_int, c_p, c_p, c_p, c_p, c_u32, P(LaneRows), P(SamplingPenalties), c_u32)
 _sig("spo_sampling_add_thinking_cutoff", c_int, c_p, c_p, c_p, c_p, c_p, c_u32, c_u32, P(LaneRows), P(ThinkingCutoff), c_u32)
+_sig("spo_lookup_index_create", c_int, P(c_p))
+_sig("spo_lookup_index_destroy", None, c_p)
+_sig("spo_lookup_index_append", c_int, c_p, c_p, ctypes.c_uint64)
+_sig("spo_lookup_index_match", c_int, c_p, P(c_u32), P(c_u32))
+_sig("spo_lookup_index_proposals", c_u32, c_p, c_u32, c_p)
+_sig("spo_lookup_agreement", c_u32, c_u32, c_u32, c_p, c_u32, c_u32)
 _sig("spo_sampling_greedy_rows_static", c_int, ctypes.c_void_p, c_u32, c_u32, c_u32, ctypes.c_void_p, ctypes.c_void_p)
 _sig("spo_verify_check_results", c_int, P(LaneRows), P(c_u32), c_u32, c_u32, c_u32, P(c_u32), P(c_u32), P(c_u32), P(c_u32))
 _sig("spo_projection_rows", c_int, c_p, P(c_u32), P(c_u32), c_u32, P(c_p))

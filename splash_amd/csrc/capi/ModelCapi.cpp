@@ -6,6 +6,7 @@
 #include "model/DenseVerify.hpp"
 #include "model/StepResults.hpp"
 #include "model/GgufTarget.hpp"
+#include "model/LookupProposals.hpp"
 #include "splash_gguf.h"
 #include "ops/DraftSelector.hpp"
 #include "ops/Glue.hpp"
@@ -495,3 +496,38 @@ sp_status spo_dense_verify_encode_part(spo_dense_verify *verify, spo_graph *grap
 }
 
 } // extern "C"
+
+struct spo_lookup_index {
+  splash::model::LookupIndex index;
+};
+sp_status spo_lookup_index_create(spo_lookup_index **out) {
+  return capi::guard([&] {
+    capi::require(out, "result");
+    *out = new spo_lookup_index{};
+  });
+}
+void spo_lookup_index_destroy(spo_lookup_index *index) { delete index; }
+sp_status spo_lookup_index_append(spo_lookup_index *index, const uint32_t *tokens, uint64_t count) {
+  return capi::guard([&] {
+    capi::require(index && (tokens || !count), "index or tokens");
+    if (index->index.tokens().size() + count > UINT32_MAX / 2) throw std::invalid_argument("a lookup index holds fewer than 2^31 tokens");
+    index->index.append({tokens, size_t(count)});
+  });
+}
+sp_status spo_lookup_index_match(const spo_lookup_index *index, uint32_t *length, uint32_t *end) {
+  return capi::guard([&] {
+    capi::require(index && length && end, "index or results");
+    *length = index->index.match().length;
+    *end = index->index.match().end;
+  });
+}
+uint32_t spo_lookup_index_proposals(const spo_lookup_index *index, uint32_t count, uint32_t *out) {
+  if (!index || !out) return 0;
+  const std::span<const uint32_t> proposals = index->index.proposals(count);
+  std::copy(proposals.begin(), proposals.end(), out);
+  return uint32_t(proposals.size());
+}
+uint32_t spo_lookup_agreement(uint32_t token, uint32_t depth, const uint32_t *candidates, uint32_t positions, uint32_t per_position) {
+  if (!candidates) return uint32_t(splash::model::LookupAgreement::Unknown);
+  return uint32_t(splash::model::lookupAgreement(token, depth, {candidates, size_t{positions} * per_position}, per_position));
+}
