@@ -737,6 +737,9 @@ def main():
     ap.add_argument("--temperature", type=float, default=0.0,
                     help="above 0: rejection-sampling acceptance at this temperature against a full-vocabulary draft "
                          "distribution softmax(N(0, 2)) instead of greedy acceptance")
+    ap.add_argument("--penalties", action="store_true",
+                    help="every lane takes sampling penalties (repetition 1.1, presence 0.1, frequency 0.1) over a history of "
+                         "4096 tokens: the step then rewrites its logits rows before it selects and counts what it keeps")
     ap.add_argument("--ops", choices=["c2", "c3", "c5", "state", "draft", "prefill"],
                     help="instead of the dense step: c2 the projections alone by rows, c3 attention alone by context, "
                          "c5 the GDN step and the MoE layer of config 5, state the recurrent layers' cached form")
@@ -789,6 +792,13 @@ def main():
                           "projections": "prefill tile, staged rule" if args.staged_prefill else "the step's kernels, register rule",
                           "config": {"workload": w["name"] if "name" in w else args.workload, "context_tokens": w["context"]}}), flush=True)
         return
+    if args.penalties:
+        from splash_amd import ops as _ops
+        table = gpu.buffer(verify.PENALTY_WORDS)
+        for i in range(args.lanes):
+            history = rng.integers(0, w["vocabulary"], 4096).astype(np.uint32)
+            table.upload(_ops.Sampling.rebuild_penalty_words(w["vocabulary"], history, 2048), offset_bytes=i * w["vocabulary"] * 4)
+            gpu.set_penalties(i, 1.1, 0.1, 0.1)
     graph = gpu.encode(lanes, commit=True)
     if args.temperature > 0:
         # the draft model's distributions of the block's rows: softmax of N(0, 2) logits over the whole vocabulary
@@ -873,7 +883,8 @@ def main():
                 "uniform INT8 KV codes, uniform-random draft tokens, random page table",
         "config": {"workload": w["name"], "lanes": args.lanes, "rows_per_lane": w["rows"], "context_tokens": w["context"],
                    "layers": w["layers"], "dispatches": len(kernels),
-                   "acceptance": f"rejection sampling, T = {args.temperature}" if args.temperature > 0 else "greedy"},
+                   "acceptance": (f"rejection sampling, T = {args.temperature}" if args.temperature > 0 else "greedy") +
+                                 (", sampling penalties" if args.penalties else "")},
         "step_hbm": {"algorithmic_gb": round(step_bytes / 1e9, 3), "achieved_gbs": round(step_bytes / (ms * 1e-3) / 1e9, 1),
                      "frac_of_peak": round(step_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "wall_ms_per_step": round(wall_ms, 4)},
         "roofline": roofline,

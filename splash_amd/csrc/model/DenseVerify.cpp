@@ -25,7 +25,7 @@ hip::Buffer tablesOf(const hip::Buffer &tables, uint32_t k, uint32_t first, uint
 DenseVerify::DenseVerify(hip::Backend &backend, DenseDimensions d, uint32_t maxLanes, uint32_t physicalPages,
                          uint32_t pageTableEntries, uint32_t prefillRows)
     : backend_(backend), dims_(d), linear_(backend.deviceInfo()), maxLanes_(maxLanes),
-      penalties_(backend, maxLanes, d.vocabulary) {
+      lanePolicies_(backend, maxLanes, d.vocabulary) {
   if (prefillRows > ops::kMaximumChunkRows) throw std::invalid_argument("a prompt chunk holds at most 2048 rows");
   if (!d.hidden || !d.layers || !d.vocabulary || !d.ffn || !maxLanes || maxLanes > ATTENTION_MAXIMUM_SEQUENCES)
     throw std::invalid_argument("a dense verify step takes a model and 1 to 8 lanes");
@@ -521,18 +521,18 @@ void DenseVerify::encode(hip::CommandGraph &graph, const std::vector<VerifyLane>
     sampling.childUniforms = children_.childUniforms;
   }
   // a lane's penalties rewrite its rows of the head's fresh logits before anything selects from them
-  const bool penalized = penalties_.apply(policies);
-  if (penalties_.anyConstrained(lanes.size())) {
-    sampling.tokenMask = penalties_.tokenMask(maxRows_);
-    sampling.maskWords = penalties_.maskWords();
+  const bool penalized = lanePolicies_.apply(policies);
+  if (lanePolicies_.anyConstrained(lanes.size())) {
+    sampling.tokenMask = lanePolicies_.tokenMask(maxRows_);
+    sampling.maskWords = lanePolicies_.maskWords();
   }
-  if (penalized) ops::Sampling::addPenalties(graph, sampling, dims_.vocabulary, dims_.vocabulary, laneRows, policies, penalties_.table());
-  ops::Sampling::addVerify(graph, sampling, dims_.vocabulary, dims_.vocabulary, laneRows, policies, penalties_.stopTokens());
+  if (penalized) ops::Sampling::addPenalties(graph, sampling, dims_.vocabulary, dims_.vocabulary, laneRows, policies, lanePolicies_.table());
+  ops::Sampling::addVerify(graph, sampling, dims_.vocabulary, dims_.vocabulary, laneRows, policies, lanePolicies_.stopTokens());
   const ops::AcceptanceBuffers acceptance{inputTokens_, treeRows_, tokens_, retained_, acceptedCount_, retainedRows_};
-  ops::Sampling::addAcceptance(graph, acceptance, laneRows, remaining, penalties_.stopTokens());
+  ops::Sampling::addAcceptance(graph, acceptance, laneRows, remaining, lanePolicies_.stopTokens());
   // a step that commits counts the tokens its penalized lanes keep, for the next step's penalties
   if (penalized && commit)
-    ops::Sampling::addPenaltyCount(graph, acceptance, dims_.vocabulary, laneRows, penalties_.active(lanes.size()), penalties_.table());
+    ops::Sampling::addPenaltyCount(graph, acceptance, dims_.vocabulary, laneRows, lanePolicies_.penalized(lanes.size()), lanePolicies_.table());
   if (commit)
     ops::PagedAttention::addPathCommit(graph, plan, retainedRows_, {pageTable_, kvAll_, pageBytes_}, dims_.layers, layerBytes_);
 }

@@ -19,7 +19,7 @@ template <class F> void forRowPieces(uint32_t rows, F &&piece) {
 HybridVerify::HybridVerify(hip::Backend &backend, HybridDimensions d, uint32_t maxLanes, uint32_t physicalPages,
                            uint32_t pageTableEntries, uint32_t prefillRows)
     : backend_(backend), dims_(d), linear_(backend.deviceInfo()), maxLanes_(maxLanes),
-      penalties_(backend, maxLanes, d.vocabulary) {
+      lanePolicies_(backend, maxLanes, d.vocabulary) {
   if (prefillRows > ops::kMaximumChunkRows) throw std::invalid_argument("a prompt chunk holds at most 2048 rows");
   if (!d.hidden || !d.layers || !d.vocabulary || !maxLanes || maxLanes > GDN_MAXIMUM_LANES)
     throw std::invalid_argument("a hybrid verify step takes a model and 1 to 8 lanes");
@@ -352,19 +352,19 @@ void HybridVerify::encode(hip::CommandGraph &graph, const std::vector<HybridLane
   }
   encodeHead(graph, rows, feeds);
   // a lane's penalties rewrite its rows of the head's fresh logits before anything selects from them
-  const bool penalized = penalties_.apply(policies);
+  const bool penalized = lanePolicies_.apply(policies);
   ops::SamplingBuffers selection = sampling_;
-  if (penalties_.anyConstrained(lanes.size())) {
-    selection.tokenMask = penalties_.tokenMask(maxRows_);
-    selection.maskWords = penalties_.maskWords();
+  if (lanePolicies_.anyConstrained(lanes.size())) {
+    selection.tokenMask = lanePolicies_.tokenMask(maxRows_);
+    selection.maskWords = lanePolicies_.maskWords();
   }
-  if (penalized) ops::Sampling::addPenalties(graph, selection, dims_.vocabulary, dims_.vocabulary, laneRows, policies, penalties_.table());
-  ops::Sampling::addVerify(graph, selection, dims_.vocabulary, dims_.vocabulary, laneRows, policies, penalties_.stopTokens());
+  if (penalized) ops::Sampling::addPenalties(graph, selection, dims_.vocabulary, dims_.vocabulary, laneRows, policies, lanePolicies_.table());
+  ops::Sampling::addVerify(graph, selection, dims_.vocabulary, dims_.vocabulary, laneRows, policies, lanePolicies_.stopTokens());
   const ops::AcceptanceBuffers acceptance{inputTokens_, treeRows_, tokens_, retained_, acceptedCount_, retainedRows_};
-  ops::Sampling::addAcceptance(graph, acceptance, laneRows, remaining, penalties_.stopTokens());
+  ops::Sampling::addAcceptance(graph, acceptance, laneRows, remaining, lanePolicies_.stopTokens());
   // a step that commits counts the tokens its penalized lanes keep, for the next step's penalties
   if (penalized && commit)
-    ops::Sampling::addPenaltyCount(graph, acceptance, dims_.vocabulary, laneRows, penalties_.active(lanes.size()), penalties_.table());
+    ops::Sampling::addPenaltyCount(graph, acceptance, dims_.vocabulary, laneRows, lanePolicies_.penalized(lanes.size()), lanePolicies_.table());
   if (commit && dims_.attentionLayers())
     ops::PagedAttention::addPathCommit(graph, planOf(lanes), retainedRows_, {pageTable_, kvAll_, pageBytes_}, dims_.attentionLayers(),
                                        layerBytes_);

@@ -149,17 +149,17 @@ public:
   // off) and the table they read: lane l's row is words [l vocabulary, (l + 1) vocabulary) of penaltyWords(), which a
   // request that takes the lane uploads (ops::Sampling::rebuildPenaltyWords). A step that commits counts what a
   // penalized lane keeps into its row.
-  void setPenalties(uint32_t lane, ops::SamplingPenalties penalties) { penalties_.set(lane, penalties); }
-  [[nodiscard]] const hip::Buffer &penaltyWords() { return penalties_.words(); }
+  void setPenalties(uint32_t lane, ops::SamplingPenalties penalties) { lanePolicies_.setPenalties(lane, penalties); }
+  [[nodiscard]] const hip::Buffer &penaltyWords() { return lanePolicies_.words(); }
   // Dispatch lane `lane` of the steps encoded after admits only the tokens of its rows of tokenMask() (constrained), never
   // selects a stop token (excludesStopTokens); the step's stop tokens (SAMPLING_NO_TOKEN for none), at which acceptance
   // ends a lane's path (SamplingPolicy::constrained / excludesStopTokens, StopTokens in the reference's Sampling.hpp).
-  void setAdmission(uint32_t lane, bool constrained, bool excludesStopTokens) { penalties_.setAdmission(lane, constrained, excludesStopTokens); }
-  void setStopTokens(const std::array<uint32_t, SAMPLING_STOP_TOKENS> &tokens) noexcept { penalties_.setStopTokens(tokens); }
-  [[nodiscard]] const hip::Buffer &tokenMask() { return penalties_.tokenMask(maxRows_); }
+  void setAdmission(uint32_t lane, bool constrained, bool excludesStopTokens) { lanePolicies_.setAdmission(lane, constrained, excludesStopTokens); }
+  void setStopTokens(const std::array<uint32_t, SAMPLING_STOP_TOKENS> &tokens) noexcept { lanePolicies_.setStopTokens(tokens); }
+  [[nodiscard]] const hip::Buffer &tokenMask() { return lanePolicies_.tokenMask(maxRows_); }
   // The thinking cutoff of dispatch lane `lane` for the steps encoded after (ops::ThinkingCutoff; none clears it): its
   // rows from the cutoff's depth on select the end of thinking, between the step's selection and its acceptance.
-  void setThinkingCutoff(uint32_t lane, std::optional<ops::ThinkingCutoff> cutoff) { penalties_.setCutoff(lane, std::move(cutoff)); }
+  void setThinkingCutoff(uint32_t lane, std::optional<ops::ThinkingCutoff> cutoff) { lanePolicies_.setCutoff(lane, std::move(cutoff)); }
   // The hidden rows a draft's context is computed from (the reference's QwenTarget addCapture over RowCopy): after
   // layer layers[i] (ascending) every row's output goes to columns [i hidden, (i + 1) hidden) of its row of
   // `destination`, bf16 [rows][layers.size() x hidden], in a step and in a prompt chunk alike. An empty list captures nothing.
@@ -199,7 +199,7 @@ private:
   HybridWeights weights_;
   ops::Linear linear_;
   uint32_t maxRows_ = 0, maxLanes_ = 0, rowCapacity_ = 0;
-  LanePolicies penalties_;
+  LanePolicies lanePolicies_;
   bool tiledGdnHeads_ = false;
   std::vector<uint32_t> captureLayers_;
   hip::Buffer captured_;

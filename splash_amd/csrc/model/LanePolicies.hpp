@@ -44,7 +44,7 @@ public:
       if (constrained_[l]) return true;
     return false;
   }
-  void set(uint32_t lane, ops::SamplingPenalties penalties) {
+  void setPenalties(uint32_t lane, ops::SamplingPenalties penalties) {
     if (lane >= penalties_.size()) throw std::invalid_argument("penalties of a lane past the driver's");
     penalties_[lane] = penalties;
     if (penalties.active()) (void)words();
@@ -72,7 +72,7 @@ public:
     return any;
   }
   [[nodiscard]] ops::PenaltyTable table() { return {words(), rows_}; }
-  [[nodiscard]] std::vector<bool> active(size_t lanes) const {
+  [[nodiscard]] std::vector<bool> penalized(size_t lanes) const {
     std::vector<bool> out(lanes);
     for (size_t l = 0; l < lanes && l < penalties_.size(); ++l) out[l] = penalties_[l].active();
     return out;
