@@ -77,3 +77,48 @@ def test_linear_plans_without_a_device():
         linear.scratch_size(5120, 25600, 257)
     with pytest.raises(ValueError):
         linear.scratch_size(5121, 25600, 16)
+
+
+def test_headers_are_plain_c_and_a_c_caller_links(tmp_path):
+    """The boundary is a C ABI: every header compiles as C11 on its own, and a C program that calls host-side entry
+    points (a weight image's size, the rewrite of a Q4_0 block, a lookup index) links against the library and runs."""
+    import shutil
+    import subprocess
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("no C compiler here")
+    include = os.path.join(ROOT, "include")
+    for header in sorted(os.listdir(include)):
+        done = subprocess.run([gcc, "-x", "c", "-std=c11", "-Wall", "-Wextra", "-Werror", "-fsyntax-only", "-I", include, "-"],
+                              input=f'#include "{header}"\n', text=True, capture_output=True)
+        assert done.returncode == 0, (header, done.stderr[-800:])
+    source = tmp_path / "caller.c"
+    source.write_text(r'''
+#include "splash_ops.h"
+#include <stdio.h>
+#include <string.h>
+int main(void) {
+  if (spo_gguf_image_bytes(0, 16, 256) != 16u * 144u) return 1;
+  unsigned char q40[8 * 18], q80[8 * 34];
+  memset(q40, 0x21, sizeof q40);                       /* nibbles 1 and 2: codes - 8 = -7 and -6 */
+  if (spo_gguf_rewrite_format(2) != 6 || spo_gguf_rewrite(2, q40, 1, q80) != SP_OK) return 2;
+  if ((signed char)q80[2] != -7 || (signed char)q80[2 + 16] != -6 || q80[0] != 0x21) return 3;
+  spo_lookup_index *index = NULL;
+  const uint32_t tokens[] = {1, 2, 3, 4, 9, 1, 2, 3};
+  uint32_t length = 0, end = 0, next[2] = {0, 0};
+  if (spo_lookup_index_create(&index) != SP_OK || spo_lookup_index_append(index, tokens, 8) != SP_OK) return 4;
+  if (spo_lookup_index_match(index, &length, &end) != SP_OK || length != 3 || end != 2) return 5;
+  if (spo_lookup_index_proposals(index, 2, next) != 2 || next[0] != 4 || next[1] != 9) return 6;
+  spo_lookup_index_destroy(index);
+  puts("ok");
+  return 0;
+}
+''')
+    from splash_amd import _native as nat
+    library = nat.library_path()
+    binary = tmp_path / "caller"
+    done = subprocess.run([gcc, "-std=c11", "-Wall", "-Werror", "-I", include, str(source), "-o", str(binary), library,
+                           f"-Wl,-rpath,{os.path.dirname(library)}"], capture_output=True, text=True)
+    assert done.returncode == 0, done.stderr[-1500:]
+    ran = subprocess.run([str(binary)], capture_output=True, text=True, timeout=120)
+    assert ran.returncode == 0 and ran.stdout.strip() == "ok", (ran.returncode, ran.stdout, ran.stderr[-800:])
