@@ -81,12 +81,14 @@ sp_status spo_gdn_add_prefill(spo_graph *graph, const spo_gdn_prefill_buffers *b
 
 uint64_t spo_state_codec_layer_bytes(uint32_t rows, uint32_t columns) { return state_codec_layer_bytes(rows, columns); }
 
+extern "C++" {
 namespace {
 ops::StateCodecShape codecShapeOf(const spo_state_codec_shape &s) {
   return {s.layers, s.rows, s.columns, s.state_layer_bytes, s.codes_layer_bytes,
           s.bf16_state ? ops::GdnStateFormat::BFloat16 : ops::GdnStateFormat::Float32};
 }
 } // namespace
+} // extern "C++"
 
 sp_status spo_state_codec_add_quantize(spo_graph *graph, sp_buffer *state, sp_buffer *codes, const spo_state_codec_shape *shape) {
   return capi::guard([&] {

@@ -114,26 +114,6 @@ sp_status spo_sampling_add_verify(spo_graph *graph, const spo_sampling_buffers *
     ops::Sampling::addVerify(capi::graphOf(graph), buffers, vocabulary, logits_stride, rows, policies, stops);
   });
 }
-namespace {
-struct PenalizedLanes {
-  std::vector<ops::LaneRows> rows;
-  std::vector<ops::SamplingPolicy> policies;
-  std::vector<uint32_t> tableRows;
-  std::vector<bool> active;
-};
-PenalizedLanes penalizedLanes(const spo_lane_rows *lanes, const spo_sampling_penalties *penalties, uint32_t count) {
-  PenalizedLanes out;
-  for (uint32_t i = 0; i < count; ++i) {
-    out.rows.push_back({lanes[i].first, lanes[i].rows});
-    ops::SamplingPolicy policy;
-    policy.penalties = {penalties[i].repetition, penalties[i].presence, penalties[i].frequency};
-    out.policies.push_back(policy);
-    out.tableRows.push_back(penalties[i].table_row);
-    out.active.push_back(policy.penalties.active());
-  }
-  return out;
-}
-} // namespace
 sp_status spo_sampling_rebuild_penalty_words(uint32_t *words, uint32_t vocabulary, const uint32_t *history, uint64_t history_tokens,
                                              uint64_t generated_tokens, uint32_t pending_token, uint32_t mark_prompt) {
   return capi::guard([&] {
@@ -148,7 +128,7 @@ sp_status spo_sampling_add_penalties(spo_graph *graph, sp_buffer *logits, sp_buf
                                      const spo_sampling_penalties *penalties, uint32_t count) {
   return capi::guard([&] {
     capi::require(graph && lanes && penalties, "graph, lanes or penalties");
-    const PenalizedLanes p = penalizedLanes(lanes, penalties, count);
+    const capi::PenalizedLanes p = capi::penalizedLanes(lanes, penalties, count);
     ops::SamplingBuffers buffers{};
     buffers.logits = B(logits);
     buffers.inputTokens = B(input_tokens);
@@ -160,7 +140,7 @@ sp_status spo_sampling_add_penalty_count(spo_graph *graph, sp_buffer *words, sp_
                                          const spo_lane_rows *lanes, const spo_sampling_penalties *penalties, uint32_t count) {
   return capi::guard([&] {
     capi::require(graph && lanes && penalties, "graph, lanes or penalties");
-    const PenalizedLanes p = penalizedLanes(lanes, penalties, count);
+    const capi::PenalizedLanes p = capi::penalizedLanes(lanes, penalties, count);
     ops::AcceptanceBuffers buffers{};
     buffers.tokens = B(tokens);
     buffers.retained = B(retained);

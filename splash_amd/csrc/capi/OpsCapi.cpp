@@ -222,6 +222,7 @@ sp_status spo_linear_add_residual_norm(const spo_linear *linear, spo_graph *grap
     linear->linear.add(graph->graph, std::move(buffers), projection->projection, full);
   });
 }
+extern "C++" {
 namespace {
 ops::ChainedProjection linkOf(const spo_chain_link &l) {
   capi::require(l.projection, "a link's projection");
@@ -236,6 +237,7 @@ ops::ChainedProjection linkOf(const spo_chain_link &l) {
   return {std::move(buffers), &l.projection->projection, toPlan(l.projection->projection, l.plan), l.gate ? &l.gate->projection : nullptr};
 }
 } // namespace
+} // extern "C++"
 sp_status spo_linear_add_chain(const spo_linear *linear, spo_graph *graph, const spo_chain_link *links, uint32_t count,
                                sp_buffer *progress) {
   return capi::guard([&] {
