@@ -737,6 +737,8 @@ def main():
     ap.add_argument("--temperature", type=float, default=0.0,
                     help="above 0: rejection-sampling acceptance at this temperature against a full-vocabulary draft "
                          "distribution softmax(N(0, 2)) instead of greedy acceptance")
+    ap.add_argument("--direct-launch", action="store_true",
+                    help="launch the step's dispatches one by one on the command stream instead of replaying a recorded HIP graph")
     ap.add_argument("--penalties", action="store_true",
                     help="every lane takes sampling penalties (repetition 1.1, presence 0.1, frequency 0.1) over a history of "
                          "4096 tokens: the step then rewrites its logits rows before it selects and counts what it keeps")
@@ -816,7 +818,7 @@ def main():
     wall0 = time.time()
     gpu_seconds = 0.0
     for _ in range(args.steps):
-        gpu_seconds += command.submit().wait()[0]
+        gpu_seconds += (backend.run(graph) if args.direct_launch else command.submit().wait())[0]
     wall = time.time() - wall0
     ms = gpu_seconds / args.steps * 1e3
     wall_ms = wall / args.steps * 1e3
